@@ -1,0 +1,258 @@
+"""ctypes binding of oracle/liboracle.so (the C restatement in oracle.c). Test infrastructure only."""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+OR_F32, OR_Q4K, OR_W4A8, OR_W8A8 = 0, 1, 2, 3
+
+
+class Mat(C.Structure):
+    _fields_ = [("kind", C.c_int), ("N", C.c_int), ("K", C.c_int), ("data", C.c_void_p),
+                ("scales", C.c_void_p), ("act_group", C.c_int)]
+
+
+class Layer(C.Structure):
+    _fields_ = [(n, Mat) for n in ("q", "k", "v", "o", "gate", "up", "down")] + [
+        ("attn_norm", C.c_void_p), ("ffn_norm", C.c_void_p), ("q_norm", C.c_void_p), ("k_norm", C.c_void_p),
+        ("router", Mat), ("exp_gate", C.POINTER(Mat)), ("exp_up", C.POINTER(Mat)), ("exp_down", C.POINTER(Mat))]
+
+
+class Model(C.Structure):
+    _fields_ = [("n_layers", C.c_int), ("hidden", C.c_int), ("n_heads", C.c_int), ("n_kv", C.c_int),
+                ("head_dim", C.c_int), ("inter", C.c_int), ("vocab", C.c_int),
+                ("eps", C.c_double), ("attn_scale", C.c_double), ("softcap", C.c_double),
+                ("inv_freq", C.c_void_p),
+                ("n_experts", C.c_int), ("top_k", C.c_int), ("norm_topk", C.c_int), ("exp_inter", C.c_int),
+                ("kv_f16", C.c_int), ("layers", C.POINTER(Layer)), ("final_norm", C.c_void_p), ("head", Mat)]
+
+
+def build():
+    """Compile liboracle.so from the C sources beside this file."""
+    subprocess.check_call(["make", "-s", "-C", _HERE])
+
+
+def lib():
+    global _LIB
+    if _LIB is None:
+        path = os.path.join(_HERE, "liboracle.so")
+        if not os.path.exists(path):
+            build()
+        L = C.CDLL(path)
+        L.or_f32_to_f16.restype = C.c_uint16
+        L.or_f32_to_f16.argtypes = [C.c_float]
+        L.or_f16_to_f32.restype = C.c_float
+        L.or_f16_to_f32.argtypes = [C.c_uint16]
+        L.or_silu.restype = C.c_float
+        L.or_silu.argtypes = [C.c_float]
+        L.or_quantize_row_int8.restype = C.c_float
+        L.or_kprint_name.restype = C.c_char_p
+        L.or_cache_new.restype = C.c_void_p
+        L.or_cache_new.argtypes = [C.POINTER(Model), C.c_int]
+        L.or_cache_free.argtypes = [C.POINTER(Model), C.c_void_p]
+        _LIB = L
+    return _LIB
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def fingerprints():
+    L = lib()
+    out = {}
+    buf = C.create_string_buffer(80)
+    for i in range(L.or_kprint_count()):
+        L.or_kprint_run(i, buf)
+        out[L.or_kprint_name(i).decode()] = buf.value.decode()
+    return out
+
+
+def set_threads(n):
+    lib().or_set_threads(int(n))
+
+
+def dequant_q4k(blocks):
+    blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+    nb = blocks.size // 144
+    out = np.empty(nb * 256, np.float32)
+    lib().or_dequant_q4k(_p(blocks), C.c_size_t(nb), _p(out))
+    return out
+
+
+def quantize_act(a, group):
+    a = f32(a)
+    M, K = a.shape
+    nG = (K + group - 1) // group if group > 0 else 1
+    q = np.empty((M, K), np.int8)
+    S = np.empty((M, nG), np.float32)
+    lib().or_quantize_act(_p(a), M, K, group, _p(q), _p(S))
+    return q, S
+
+
+def quantize_rows_int8(w):
+    w = f32(w)
+    N, K = w.shape
+    q = np.empty((N, K), np.int8)
+    S = np.empty(N, np.float32)
+    lib().or_quantize_act(_p(w), N, K, 0, _p(q), _p(S))
+    return q, S
+
+
+def quantize_int4(w, group=32):
+    w = f32(w)
+    N, K = w.shape
+    q4 = np.empty((N, (K + 1) // 2), np.uint8)
+    s16 = np.empty((N, (K + group - 1) // group), np.uint16)
+    lib().or_quantize_int4_mat(_p(w), N, K, group, _p(q4), _p(s16))
+    return q4, s16
+
+
+class WMat:
+    """A weight matrix handed to the oracle; keeps its numpy buffers alive."""
+
+    def __init__(self, kind, N, K, data, scales=None, act_group=0):
+        self.kind, self.N, self.K, self.act_group = kind, N, K, act_group
+        self.data = np.ascontiguousarray(data)
+        self.scales = None if scales is None else np.ascontiguousarray(scales)
+
+    @staticmethod
+    def from_f32(w):
+        w = f32(w)
+        return WMat(OR_F32, w.shape[0], w.shape[1], w)
+
+    def c(self):
+        return Mat(self.kind, self.N, self.K, _p(self.data), _p(self.scales) if self.scales is not None else None,
+                   self.act_group)
+
+
+def matmul(w, a):
+    a = f32(a)
+    M = a.shape[0]
+    dst = np.empty((M, w.N), np.float32)
+    m = w.c()
+    lib().or_matmul(C.byref(m), _p(a), M, _p(dst))
+    return dst
+
+
+def matmul_f64ref(w, a):
+    a = f32(a)
+    M = a.shape[0]
+    dst = np.empty((M, w.N), np.float64)
+    m = w.c()
+    lib().or_matmul_f64ref(C.byref(m), _p(a), M, _p(dst))
+    return dst
+
+
+def rmsnorm(x, w, eps, add_one=False):
+    x = f32(x)
+    w = f32(w)
+    out = np.empty_like(x)
+    rows, dim = x.shape
+    lib().or_rmsnorm(_p(out), _p(x), _p(w), rows, dim, C.c_double(eps), int(add_one))
+    return out
+
+
+def rope(vec, heads, head_dim, pos, inv_freq, scale=1.0):
+    v = f32(vec).copy()
+    inv = np.ascontiguousarray(inv_freq, dtype=np.float64)
+    lib().or_rope(_p(v), heads, head_dim, int(pos), _p(inv), len(inv), C.c_double(scale))
+    return v
+
+
+def swiglu(gate, up):
+    g = f32(gate).copy()
+    u = f32(up)
+    lib().or_swiglu(_p(g), _p(u), g.size)
+    return g
+
+
+def route_experts(logits, k, norm, scale=0.0):
+    lg = f32(logits)
+    idx = np.empty(k, np.int32)
+    wts = np.empty(k, np.float32)
+    n = lib().or_route_experts(_p(lg), lg.size, k, int(norm), C.c_double(scale), _p(idx), _p(wts))
+    return idx[:n], wts[:n]
+
+
+def argmax(x):
+    x = f32(x)
+    return lib().or_argmax(_p(x), x.size)
+
+
+def attend(q, keys, vals, n_keys, nH, nKV, hd, scale, softcap=0.0, start=0):
+    q = f32(q)
+    keys = f32(keys)
+    vals = f32(vals)
+    ctx = np.empty(nH * hd, np.float32)
+    lib().or_attend(_p(q), _p(ctx), _p(keys), _p(vals), int(n_keys), int(start), nH, nKV, hd,
+                    C.c_double(scale), C.c_double(softcap))
+    return ctx
+
+
+class OracleModel:
+    """decodeMultiStep over numpy weights. layers: list of dicts with WMat entries q,k,v,o,(gate,up,down | router,
+    exp_gate[],exp_up[],exp_down[]) and f32 arrays attn_norm, ffn_norm, optional q_norm,k_norm."""
+
+    def __init__(self, cfg, layers, final_norm, head, inv_freq):
+        self.cfg = cfg
+        self._keep = []
+        nL = len(layers)
+        self._layers = (Layer * nL)()
+        nE = cfg.get("n_experts", 0)
+        for i, lw in enumerate(layers):
+            L = self._layers[i]
+            for n in ("q", "k", "v", "o"):
+                setattr(L, n, lw[n].c())
+            self._keep.append(lw)
+            for n in ("attn_norm", "ffn_norm", "q_norm", "k_norm"):
+                if lw.get(n) is not None:
+                    arr = f32(lw[n])
+                    self._keep.append(arr)
+                    setattr(L, n, _p(arr))
+            if nE == 0:
+                for n in ("gate", "up", "down"):
+                    setattr(L, n, lw[n].c())
+            else:
+                L.router = lw["router"].c()
+                for n in ("exp_gate", "exp_up", "exp_down"):
+                    arr = (Mat * nE)(*[m.c() for m in lw[n]])
+                    self._keep.append(arr)
+                    setattr(L, n, arr)
+        self._fn = f32(final_norm)
+        self._inv = np.ascontiguousarray(inv_freq, dtype=np.float64)
+        self._head = head
+        self.m = Model(nL, cfg["hidden"], cfg["n_heads"], cfg["n_kv"], cfg["head_dim"], cfg.get("inter", 0),
+                       cfg["vocab"], cfg["eps"], cfg["attn_scale"], cfg.get("softcap", 0.0), _p(self._inv),
+                       nE, cfg.get("top_k", 0), int(cfg.get("norm_topk", 0)), cfg.get("exp_inter", 0),
+                       int(cfg.get("kv_f16", 0)), self._layers, _p(self._fn), head.c())
+
+    def new_cache(self, cap):
+        return lib().or_cache_new(C.byref(self.m), cap)
+
+    def free_cache(self, c):
+        lib().or_cache_free(C.byref(self.m), C.c_void_p(c))
+
+    def step(self, emb, caches, want_moe=False):
+        emb = f32(emb)
+        B = emb.shape[0]
+        logits = np.empty((B, self.cfg["vocab"]), np.float32)
+        arr = (C.c_void_p * B)(*caches)
+        trace = None
+        if want_moe:
+            trace = np.full((B, self.cfg_layers(), self.cfg["top_k"]), -1, np.int32)
+        rc = lib().or_decode_multi_step(C.byref(self.m), B, _p(emb), arr, _p(logits), _p(trace) if want_moe else None)
+        if rc != 0:
+            raise RuntimeError("oracle: cache full")
+        return (logits, trace) if want_moe else logits
+
+    def cfg_layers(self):
+        return self.m.n_layers

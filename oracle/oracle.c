@@ -1,0 +1,687 @@
+/*
+ * oracle.c — CPU restatement of goinfer's ragged batched decode step. TEST INFRASTRUCTURE ONLY:
+ * see oracle.h for the contract, the reference citations and the pin status of every function.
+ * Build with -ffp-contract=off: the Go reference rounds every f32 operation (amd64 never fuses).
+ */
+#include "oracle.h"
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+static int g_threads = 1;
+void or_set_threads(int n) { g_threads = n < 1 ? 1 : n; }
+
+/* ------------------------------------------------------------------ f16 */
+/* internal/runtime/f16/f16.go:14-43 (Bits): round-half-up on the dropped mantissa bits. */
+uint16_t or_f32_to_f16(float f) {
+    uint32_t b;
+    memcpy(&b, &f, 4);
+    uint16_t sign = (uint16_t)((b >> 16) & 0x8000);
+    int32_t e = (int32_t)((b >> 23) & 0xFF) - 112;
+    uint32_t m = b & 0x7FFFFF;
+    if (((b >> 23) & 0xFF) == 0xFF) return m ? (sign | 0x7E00) : (sign | 0x7C00);
+    if (e >= 0x1F) return sign | 0x7C00;
+    if (e <= 0) {
+        if (e < -10) return sign;
+        m |= 0x800000;
+        uint32_t sh = (uint32_t)(14 - e);
+        return sign | (uint16_t)((m + (1u << (sh - 1))) >> sh);
+    }
+    uint16_t half = sign | (uint16_t)(e << 10) | (uint16_t)(m >> 13);
+    if (m & 0x1000) half++;
+    return half;
+}
+
+/* internal/runtime/f16/f16.go:46-63 (ToF32): exact widening. */
+float or_f16_to_f32(uint16_t h) {
+    uint32_t sign = (uint32_t)(h & 0x8000) << 16;
+    uint32_t exp = (h >> 10) & 0x1F, man = h & 0x3FF, u;
+    float f;
+    if (exp == 0) {
+        if (man == 0) {
+            u = sign;
+            memcpy(&f, &u, 4);
+            return f;
+        }
+        f = (float)man / 1024.0f * 6.103515625e-05f; /* 2^-14 */
+        return sign ? -f : f;
+    }
+    if (exp == 0x1F)
+        u = sign | 0x7F800000u | (man << 13);
+    else
+        u = sign | ((exp + 112) << 23) | (man << 13);
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+/* ------------------------------------------------------------------ Q4_K */
+/* ggml get_scale_min_k4: backend/cuda/actgroup.cu:64-75, backend/metal/kernels/gemm_kq_test.go:31-36. */
+void or_q4k_scale_min(int j, const uint8_t *q, int *sc, int *m) {
+    if (j < 4) {
+        *sc = q[j] & 63;
+        *m = q[j + 4] & 63;
+    } else {
+        *sc = (q[j + 4] & 15) | ((q[j - 4] >> 6) << 4);
+        *m = (q[j + 4] >> 4) | ((q[j] >> 6) << 4);
+    }
+}
+
+/* decoder/gguf.go:1508-1537 (q4kMat wraps the raw blocks) and gemm_kq_test.go:58-68: element e of a
+ * block, j=e/32, l=e%32, q=(qs[(j/2)*32+l]>>(4*(j&1)))&15, w = d*sc_j*q - dmin*m_j in f32 with the
+ * two products (d*sc), (dmin*m) formed first. */
+void or_dequant_q4k(const uint8_t *blocks, size_t n_blocks, float *out) {
+    for (size_t b = 0; b < n_blocks; b++) {
+        const uint8_t *blk = blocks + b * 144;
+        float d = or_f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+        float dmin = or_f16_to_f32((uint16_t)(blk[2] | (blk[3] << 8)));
+        const uint8_t *qs = blk + 16;
+        float *o = out + b * 256;
+        for (int j = 0; j < 8; j++) {
+            int sc, m;
+            or_q4k_scale_min(j, blk + 4, &sc, &m);
+            float d1 = d * (float)sc, m1 = dmin * (float)m;
+            for (int l = 0; l < 32; l++) {
+                int q = (qs[(j / 2) * 32 + l] >> (4 * (j & 1))) & 15;
+                o[j * 32 + l] = d1 * (float)q - m1;
+            }
+        }
+    }
+}
+
+/* ------------------------------------------------------------------ activation quantizers */
+static inline float round_half_away(float x) { return roundf(x); }
+
+/* backend/cuda/kv8_store.cu:3-5,27-35 (states aikit linalg.QuantizeRowInt8): scale = maxabs/127 in f32,
+ * q = round-half-away(x * (1/scale)) clamped to [-127,127]; an all-zero row gets scale 1 and zeros. */
+float or_quantize_row_int8(const float *row, int n, int8_t *q) {
+    float ma = 0.f;
+    for (int i = 0; i < n; i++) {
+        float a = fabsf(row[i]);
+        if (a > ma) ma = a;
+    }
+    if (ma == 0.f) {
+        memset(q, 0, (size_t)n);
+        return 1.f;
+    }
+    float sc = ma / 127.f, inv = 1.f / sc;
+    for (int i = 0; i < n; i++) {
+        float x = round_half_away(row[i] * inv);
+        if (x > 127.f) x = 127.f;
+        if (x < -127.f) x = -127.f;
+        q[i] = (int8_t)(int)x;
+    }
+    return sc;
+}
+
+/* aikit linalg.QuantizeActQ as called at decoder/cpu_gateup_fused.go:110-117 and weightmat.go:845-862:
+ * group 0 = QuantizeRowInt8 per row; group g = the same rule over every g consecutive elements
+ * (a ragged last group included), in-tree twin backend/cuda/actgroup.cu:32-54. */
+void or_quantize_act(const float *a, int M, int K, int group, int8_t *q, float *S) {
+    if (group <= 0) {
+        for (int m = 0; m < M; m++) S[m] = or_quantize_row_int8(a + (size_t)m * K, K, q + (size_t)m * K);
+        return;
+    }
+    int nG = (K + group - 1) / group;
+    for (int m = 0; m < M; m++)
+        for (int g = 0; g < nG; g++) {
+            int lo = g * group, n = K - lo < group ? K - lo : group;
+            S[(size_t)m * nG + g] = or_quantize_row_int8(a + (size_t)m * K + lo, n, q + (size_t)m * K + lo);
+        }
+}
+
+/* ------------------------------------------------------------------ int4 g32 */
+/* decoder/fakequant.go:52-56,99-131 ("sym", aikit's runtime int4): scale = maxabs/group... /7, zero group -> 1,
+ * code = clamp(round-half-away(v/s), -7, 7); canonical packing backend/cuda/internal/wpack/wpack.go:165-207
+ * and kernels/actgroup_kernel_test.go:252-261: element k in nibble k%2 (low first) of byte k/2, stored nib = code+8. */
+void or_quantize_int4_row(const float *row, int cols, int group, uint8_t *packed, float *scales) {
+    memset(packed, 0, (size_t)((cols + 1) / 2));
+    int nG = (cols + group - 1) / group;
+    for (int g = 0; g < nG; g++) {
+        int lo = g * group, hi = lo + group < cols ? lo + group : cols;
+        float mx = 0.f;
+        for (int k = lo; k < hi; k++) {
+            float a = fabsf(row[k]);
+            if (a > mx) mx = a;
+        }
+        float s = mx > 0.f ? mx / 7.f : 1.f;
+        float inv = 1.f / s;
+        scales[g] = s;
+        for (int k = lo; k < hi; k++) {
+            float c = round_half_away(row[k] * inv);
+            if (c > 7.f) c = 7.f;
+            if (c < -7.f) c = -7.f;
+            uint8_t nib = (uint8_t)((int)c + 8);
+            packed[k >> 1] |= (uint8_t)(nib << (4 * (k & 1)));
+        }
+    }
+}
+
+/* decoder/weightmat.go:166-178 (streamQuantizedRow4, quantInt4): per row QuantizeGroupInt4Row then the
+ * f32 group scales narrowed to binary16. */
+void or_quantize_int4_mat(const float *w, int rows, int cols, int group, uint8_t *q4, uint16_t *s16) {
+    int nG = (cols + group - 1) / group, bpr = (cols + 1) / 2;
+    float *sc = (float *)malloc(sizeof(float) * (size_t)nG);
+    for (int r = 0; r < rows; r++) {
+        or_quantize_int4_row(w + (size_t)r * cols, cols, group, q4 + (size_t)r * bpr, sc);
+        for (int g = 0; g < nG; g++) s16[(size_t)r * nG + g] = or_f32_to_f16(sc[g]);
+    }
+    free(sc);
+}
+
+/* ------------------------------------------------------------------ attention primitives */
+/* aikit linalg.MatmulQKAcc64 as called at decoder/forwardn.go:379-383: dst[i,s] = f32(sum_d f64(a[i,d])*f64(k[s,off+d])),
+ * d ascending (decoder/attention.go:335-352 dotsF64x8 states the same fold). */
+void or_qk_acc64(const float *a, const float *keys, float *dst, int M, int hd, int nKeys, int off, int kvDim) {
+    for (int i = 0; i < M; i++)
+        for (int s = 0; s < nKeys; s++) {
+            const float *k = keys + (size_t)s * kvDim + off;
+            double acc = 0;
+            for (int d = 0; d < hd; d++) acc += (double)a[i * hd + d] * (double)k[d];
+            dst[(size_t)i * nKeys + s] = (float)acc;
+        }
+}
+
+/* aikit linalg.MatmulAVAcc64 as called at decoder/forwardn.go:488-490: hd independent f64 accumulators,
+ * key-ascending adds, rounded to f32 once. */
+void or_av_acc64(const float *scores, const float *vals, float *dst, int M, int nKeys, int hd, int off, int kvDim) {
+    double *acc = (double *)malloc(sizeof(double) * (size_t)hd);
+    for (int i = 0; i < M; i++) {
+        for (int d = 0; d < hd; d++) acc[d] = 0;
+        for (int s = 0; s < nKeys; s++) {
+            double w = (double)scores[(size_t)i * nKeys + s];
+            const float *v = vals + (size_t)s * kvDim + off;
+            for (int d = 0; d < hd; d++) acc[d] += w * (double)v[d];
+        }
+        for (int d = 0; d < hd; d++) dst[i * hd + d] = (float)acc[d];
+    }
+    free(acc);
+}
+
+/* ------------------------------------------------------------------ glue */
+/* decoder/rmsnorm.go:29-92 (rmsNormInto): four f64 partial sums, (ss0+ss1)+(ss2+ss3)+tail. */
+void or_rmsnorm(float *dst, const float *src, const float *w, int rows, int dim, double eps, int add_one) {
+    for (int r = 0; r < rows; r++) {
+        const float *s = src + (size_t)r * dim;
+        float *o = dst + (size_t)r * dim;
+        double ss0 = 0, ss1 = 0, ss2 = 0, ss3 = 0, tail = 0;
+        int i = 0;
+        for (; i + 3 < dim; i += 4) {
+            double v0 = s[i], v1 = s[i + 1], v2 = s[i + 2], v3 = s[i + 3];
+            ss0 += v0 * v0;
+            ss1 += v1 * v1;
+            ss2 += v2 * v2;
+            ss3 += v3 * v3;
+        }
+        for (; i < dim; i++) tail += (double)s[i] * (double)s[i];
+        double ss = (ss0 + ss1) + (ss2 + ss3) + tail;
+        float inv = (float)(1.0 / sqrt(ss / (double)dim + eps));
+        for (i = 0; i < dim; i++) o[i] = add_one ? (s[i] * inv) * (1.f + w[i]) : (s[i] * inv) * w[i];
+    }
+}
+
+/* decoder/rope.go:28-64 (applyRoPE, NeoX rotate-half): theta, cos, sin and the rotation in f64. */
+void or_rope(float *vec, int heads, int head_dim, int pos, const double *inv_freq, int half, double scale) {
+    if (half == 0 || heads == 0) return;
+    double c[512], s[512];
+    for (int d = 0; d < half; d++) {
+        double theta = (double)pos * inv_freq[d];
+        c[d] = cos(theta) * scale;
+        s[d] = sin(theta) * scale;
+    }
+    for (int h = 0; h < heads; h++) {
+        float *v1 = vec + (size_t)h * head_dim, *v2 = v1 + half;
+        for (int d = 0; d < half; d++) {
+            double x1 = v1[d], x2 = v2[d];
+            v1[d] = (float)(x1 * c[d] - x2 * s[d]);
+            v2[d] = (float)(x2 * c[d] + x1 * s[d]);
+        }
+    }
+}
+
+/* decoder/rmsnorm.go:204-207 */
+float or_silu(float x) {
+    double x64 = x;
+    return (float)(x64 / (1 + exp(-x64)));
+}
+
+/* decoder/mlp.go:269-290 */
+void or_swiglu(float *gate, const float *up, int n) {
+    for (int i = 0; i < n; i++) gate[i] = or_silu(gate[i]) * up[i];
+}
+
+/* decoder/mlp.go:370-410 (softmaxF32): f32 max, e=exp(f64(x-max)) stored f32, f64 sum, out*=f32(1/sum). */
+void or_softmax_f32(const float *x, int n, float *out) {
+    if (n == 0) return;
+    float mx = x[0];
+    for (int i = 1; i < n; i++)
+        if (x[i] > mx) mx = x[i];
+    double sum = 0;
+    for (int i = 0; i < n; i++) {
+        double e = exp((double)(x[i] - mx));
+        out[i] = (float)e;
+        sum += e;
+    }
+    float inv = (float)(1.0 / sum);
+    for (int i = 0; i < n; i++) out[i] *= inv;
+}
+
+/* decoder/mlp.go:414-440 (topK): k passes of strict '>' — the lowest index wins a tie. */
+int or_topk(const float *x, int n, int k, int *idx, float *val) {
+    unsigned char *used = (unsigned char *)calloc((size_t)n, 1);
+    int cnt = 0;
+    for (; k > 0; k--) {
+        float best = -INFINITY;
+        int bi = -1;
+        for (int i = 0; i < n; i++)
+            if (!used[i] && x[i] > best) {
+                best = x[i];
+                bi = i;
+            }
+        if (bi < 0) break;
+        used[bi] = 1;
+        idx[cnt] = bi;
+        if (val) val[cnt] = best;
+        cnt++;
+    }
+    free(used);
+    return cnt;
+}
+
+/* decoder/mlp.go:130-184 (routeExperts), softmax scoring without bias or group limit: weights are the
+ * chosen scores, norm divides by their f32 sum taken in rank order, scale multiplies when not 0 or 1. */
+int or_route_experts(const float *logits, int nE, int k, int norm, double scale, int *idx, float *wts) {
+    float *scores = (float *)malloc(sizeof(float) * (size_t)nE);
+    or_softmax_f32(logits, nE, scores);
+    int n = or_topk(scores, nE, k, idx, NULL);
+    for (int j = 0; j < n; j++) wts[j] = scores[idx[j]];
+    if (norm) {
+        float s = 0.f;
+        for (int j = 0; j < n; j++) s += wts[j];
+        if (s > 0.f)
+            for (int j = 0; j < n; j++) wts[j] /= s;
+    }
+    if (scale != 0 && scale != 1)
+        for (int j = 0; j < n; j++) wts[j] *= (float)scale;
+    free(scores);
+    return n;
+}
+
+/* internal/runtime/sampling/sampler.go:485-520 (Argmax): strict '>' from index 0. */
+int or_argmax(const float *x, int n) {
+    int bi = 0;
+    float best = x[0];
+    for (int i = 1; i < n; i++)
+        if (x[i] > best) {
+            best = x[i];
+            bi = i;
+        }
+    return bi;
+}
+
+/* ------------------------------------------------------------------ matmul dispatch */
+/* decoder/weightmat.go:892-985 (matmulWS): the weight's kind picks the kernel. The int kinds quantize
+ * the activation first (group 32 in q4k mode, weightmat.go:33-38). Arithmetic of each row:
+ *   q4k   backend/cuda/actgroup.cu:298-355  facc += idot_g*((d*sc_g)*aS_g); facc += -(dmin*m_g)*asum_g
+ *   w4a8  backend/cuda/actgroup.cu:243-275  facc += idot_g*(f16(ws_g)*aS_g)      (per-row acts: *aS once at the end)
+ *   w8a8  backend/cuda/actgroup.cu:283-288,421-437  facc += idot_g*aS_g; dst = facc*wScale[n]
+ * groups ascending, one f32 accumulator per output. */
+static void matmul_q4k(const or_mat *w, const int8_t *aq, const float *aS, int M, float *dst) {
+    int N = w->N, K = w->K, nSB = K / 256, nG = K / 32;
+    const uint8_t *W = (const uint8_t *)w->data;
+    float *asum = (float *)malloc(sizeof(float) * (size_t)M * nG);
+    for (int m = 0; m < M; m++)
+        for (int g = 0; g < nG; g++) {
+            int s = 0;
+            for (int i = 0; i < 32; i++) s += aq[(size_t)m * K + g * 32 + i];
+            asum[(size_t)m * nG + g] = aS[(size_t)m * nG + g] * (float)s;
+        }
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+    for (int n = 0; n < N; n++) {
+        const uint8_t *row = W + (size_t)n * nSB * 144;
+        uint8_t qb[256];
+        for (int m = 0; m < M; m++) dst[(size_t)m * N + n] = 0.f;
+        for (int b = 0; b < nSB; b++) {
+            const uint8_t *blk = row + (size_t)b * 144;
+            float d = or_f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+            float dmin = or_f16_to_f32((uint16_t)(blk[2] | (blk[3] << 8)));
+            int sc[8], mn[8];
+            for (int j = 0; j < 8; j++) or_q4k_scale_min(j, blk + 4, &sc[j], &mn[j]);
+            for (int p = 0; p < 4; p++)
+                for (int l = 0; l < 32; l++) {
+                    uint8_t by = blk[16 + p * 32 + l];
+                    qb[(2 * p) * 32 + l] = by & 15;
+                    qb[(2 * p + 1) * 32 + l] = by >> 4;
+                }
+            for (int m = 0; m < M; m++) {
+                const int8_t *a = aq + (size_t)m * K + b * 256;
+                float facc = dst[(size_t)m * N + n];
+                for (int j = 0; j < 8; j++) {
+                    int32_t idot = 0;
+                    for (int l = 0; l < 32; l++) idot += (int32_t)qb[j * 32 + l] * (int32_t)a[j * 32 + l];
+                    int g = b * 8 + j;
+                    facc = fmaf((float)idot, (d * (float)sc[j]) * aS[(size_t)m * nG + g], facc);
+                    facc = fmaf(-(dmin * (float)mn[j]), asum[(size_t)m * nG + g], facc);
+                }
+                dst[(size_t)m * N + n] = facc;
+            }
+        }
+    }
+    free(asum);
+}
+
+static void matmul_w4a8(const or_mat *w, const int8_t *aq, const float *aS, int M, float *dst) {
+    int N = w->N, K = w->K, nG = (K + 31) / 32, bpr = (K + 1) / 2, ag = w->act_group;
+    const uint8_t *W = (const uint8_t *)w->data;
+    const uint16_t *S16 = (const uint16_t *)w->scales;
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+    for (int n = 0; n < N; n++) {
+        const uint8_t *row = W + (size_t)n * bpr;
+        for (int m = 0; m < M; m++) {
+            const int8_t *a = aq + (size_t)m * K;
+            float facc = 0.f;
+            for (int g = 0; g < nG; g++) {
+                int lo = g * 32, hi = lo + 32 < K ? lo + 32 : K;
+                int32_t idot = 0;
+                for (int k = lo; k < hi; k++) {
+                    int c = (int)((row[k >> 1] >> (4 * (k & 1))) & 15) - 8;
+                    idot += c * (int32_t)a[k];
+                }
+                float ws = or_f16_to_f32(S16[(size_t)n * nG + g]);
+                if (ag > 0)
+                    facc = fmaf((float)idot, ws * aS[(size_t)m * nG + g], facc);
+                else
+                    facc = fmaf((float)idot, ws, facc);
+            }
+            dst[(size_t)m * N + n] = ag > 0 ? facc : facc * aS[m];
+        }
+    }
+}
+
+static void matmul_w8a8(const or_mat *w, const int8_t *aq, const float *aS, int M, float *dst) {
+    int N = w->N, K = w->K, nG = (K + 31) / 32, ag = w->act_group;
+    const int8_t *W = (const int8_t *)w->data;
+    const float *wS = (const float *)w->scales;
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+    for (int n = 0; n < N; n++) {
+        const int8_t *row = W + (size_t)n * K;
+        for (int m = 0; m < M; m++) {
+            const int8_t *a = aq + (size_t)m * K;
+            if (ag > 0) {
+                float facc = 0.f;
+                for (int g = 0; g < nG; g++) {
+                    int lo = g * 32, hi = lo + 32 < K ? lo + 32 : K;
+                    int32_t idot = 0;
+                    for (int k = lo; k < hi; k++) idot += (int32_t)row[k] * (int32_t)a[k];
+                    facc = fmaf((float)idot, aS[(size_t)m * nG + g], facc);
+                }
+                dst[(size_t)m * N + n] = facc * wS[n];
+            } else {
+                int32_t idot = 0;
+                for (int k = 0; k < K; k++) idot += (int32_t)row[k] * (int32_t)a[k];
+                dst[(size_t)m * N + n] = ((float)idot * aS[m]) * wS[n];
+            }
+        }
+    }
+}
+
+void or_matmul(const or_mat *w, const float *a, int M, float *dst) {
+    int N = w->N, K = w->K;
+    if (w->kind == OR_F32) {
+        const float *W = (const float *)w->data;
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+        for (int n = 0; n < N; n++)
+            for (int m = 0; m < M; m++) {
+                double acc = 0;
+                for (int k = 0; k < K; k++) acc += (double)a[(size_t)m * K + k] * (double)W[(size_t)n * K + k];
+                dst[(size_t)m * N + n] = (float)acc;
+            }
+        return;
+    }
+    int group = w->act_group;
+    int nG = group > 0 ? (K + group - 1) / group : 1;
+    int8_t *aq = (int8_t *)malloc((size_t)M * K);
+    float *aS = (float *)malloc(sizeof(float) * (size_t)M * nG);
+    or_quantize_act(a, M, K, group, aq, aS);
+    if (w->kind == OR_Q4K)
+        matmul_q4k(w, aq, aS, M, dst);
+    else if (w->kind == OR_W4A8)
+        matmul_w4a8(w, aq, aS, M, dst);
+    else
+        matmul_w8a8(w, aq, aS, M, dst);
+    free(aq);
+    free(aS);
+}
+
+/* dequantized weight element (n,k) as a double */
+static double weight_at(const or_mat *w, int n, int k) {
+    switch (w->kind) {
+    case OR_F32: return ((const float *)w->data)[(size_t)n * w->K + k];
+    case OR_Q4K: {
+        const uint8_t *blk = (const uint8_t *)w->data + ((size_t)n * (w->K / 256) + k / 256) * 144;
+        int e = k % 256, j = e / 32, l = e % 32, sc, m;
+        or_q4k_scale_min(j, blk + 4, &sc, &m);
+        double d = or_f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+        double dmin = or_f16_to_f32((uint16_t)(blk[2] | (blk[3] << 8)));
+        int q = (blk[16 + (j / 2) * 32 + l] >> (4 * (j & 1))) & 15;
+        return d * sc * q - dmin * m;
+    }
+    case OR_W4A8: {
+        int nG = (w->K + 31) / 32, bpr = (w->K + 1) / 2;
+        int c = (int)((((const uint8_t *)w->data)[(size_t)n * bpr + (k >> 1)] >> (4 * (k & 1))) & 15) - 8;
+        return (double)c * (double)or_f16_to_f32(((const uint16_t *)w->scales)[(size_t)n * nG + k / 32]);
+    }
+    default: return (double)((const int8_t *)w->data)[(size_t)n * w->K + k] * (double)((const float *)w->scales)[n];
+    }
+}
+
+void or_matmul_f64ref(const or_mat *w, const float *a, int M, double *dst) {
+    int N = w->N, K = w->K;
+    double *ad = (double *)malloc(sizeof(double) * (size_t)M * K);
+    if (w->kind == OR_F32) {
+        for (size_t i = 0; i < (size_t)M * K; i++) ad[i] = a[i];
+    } else {
+        int group = w->act_group, nG = group > 0 ? (K + group - 1) / group : 1;
+        int8_t *aq = (int8_t *)malloc((size_t)M * K);
+        float *aS = (float *)malloc(sizeof(float) * (size_t)M * nG);
+        or_quantize_act(a, M, K, group, aq, aS);
+        for (int m = 0; m < M; m++)
+            for (int k = 0; k < K; k++)
+                ad[(size_t)m * K + k] = (double)aq[(size_t)m * K + k] * (double)aS[(size_t)m * nG + (group > 0 ? k / group : 0)];
+        free(aq);
+        free(aS);
+    }
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+    for (int n = 0; n < N; n++) {
+        double *wr = (double *)malloc(sizeof(double) * (size_t)K);
+        for (int k = 0; k < K; k++) wr[k] = weight_at(w, n, k);
+        for (int m = 0; m < M; m++) {
+            double acc = 0;
+            for (int k = 0; k < K; k++) acc += ad[(size_t)m * K + k] * wr[k];
+            dst[(size_t)m * N + n] = acc;
+        }
+        free(wr);
+    }
+    free(ad);
+}
+
+/* ------------------------------------------------------------------ attention */
+/* decoder/attention.go:287-295 */
+static double softcap_score(double s, double c) { return c == 0 ? s : c * tanh(s / c); }
+
+/* decoder/forwardn.go:295-500 with useAcc64 and K=1 (the form program_cpu_n.go:497-515 calls), no sinks,
+ * no tree mask: per query head, scores = f32(f64 dot) -> sc = softcap(f64(score)*scale) stored f32 ->
+ * max -> e = exp(f64(sc_f32) - max) stored f32, f64 sum -> w = f32(f64(e_f32) * (1/sum)) -> AV in f64. */
+void or_attend(const float *q, float *ctx, const float *keys, const float *vals, int n_keys, int start,
+               int nH, int nKV, int hd, double scale, double softcap) {
+    int kvDim = nKV * hd, group = nH / nKV;
+#pragma omp parallel for num_threads(g_threads) schedule(dynamic, 1)
+    for (int qh = 0; qh < nH; qh++) {
+        int kvh = qh / group;
+        float *scores = (float *)malloc(sizeof(float) * (size_t)n_keys);
+        or_qk_acc64(q + (size_t)qh * hd, keys, scores, 1, hd, n_keys, kvh * hd, kvDim);
+        int lo = start < 0 ? 0 : start, hi = n_keys - 1;
+        if (lo <= hi) {
+            double maxS = -INFINITY;
+            for (int s = lo; s <= hi; s++) {
+                double sc = softcap_score((double)scores[s] * scale, softcap);
+                scores[s] = (float)sc;
+                if (sc > maxS) maxS = sc;
+            }
+            double sum = 0;
+            for (int s = lo; s <= hi; s++) {
+                double e = exp((double)scores[s] - maxS);
+                scores[s] = (float)e;
+                sum += e;
+            }
+            double inv = 1.0 / sum;
+            for (int s = 0; s < lo; s++) scores[s] = 0.f;
+            for (int s = lo; s <= hi; s++) scores[s] = (float)((double)scores[s] * inv);
+        } else {
+            memset(scores, 0, sizeof(float) * (size_t)n_keys);
+        }
+        or_av_acc64(scores, vals, ctx + (size_t)qh * hd, 1, n_keys, hd, kvh * hd, kvDim);
+        free(scores);
+    }
+}
+
+/* ------------------------------------------------------------------ model */
+or_cache *or_cache_new(const or_model *m, int cap) {
+    or_cache *c = (or_cache *)calloc(1, sizeof(or_cache));
+    size_t kvDim = (size_t)m->n_kv * m->head_dim;
+    c->cap = cap;
+    c->k = (float **)calloc((size_t)m->n_layers, sizeof(float *));
+    c->v = (float **)calloc((size_t)m->n_layers, sizeof(float *));
+    for (int l = 0; l < m->n_layers; l++) {
+        c->k[l] = (float *)calloc((size_t)cap * kvDim, sizeof(float));
+        c->v[l] = (float *)calloc((size_t)cap * kvDim, sizeof(float));
+    }
+    return c;
+}
+
+void or_cache_free(const or_model *m, or_cache *c) {
+    if (!c) return;
+    for (int l = 0; l < m->n_layers; l++) {
+        free(c->k[l]);
+        free(c->v[l]);
+    }
+    free(c->k);
+    free(c->v);
+    free(c);
+}
+
+/* decoder/mlp.go:729-745 */
+static void add_scaled(float *dst, const float *src, float s, int n) {
+    for (int i = 0; i < n; i++) dst[i] += s * src[i];
+}
+
+/* decoder/program_cpu.go:351-364 (applyQKNorm): RMSNorm of each head with the shared [hd] weight. */
+static void qk_norm(float *x, int heads, int hd, const float *w, double eps) { or_rmsnorm(x, x, w, heads, hd, eps, 0); }
+
+/* decoder/mlp.go:36-120 (moeMLP) for one row: router matmul (M=1), routeExperts, experts in rank order,
+ * out += w_j * expert_j(h) (addScaled). mlp.go:630-726 (moeMLPBatchWith) folds each row in the same rank
+ * order and is bit-identical to this per-row form by its own contract. */
+static void moe_mlp(const or_model *m, const or_layer *lw, const float *h, float *out, int *idx_trace) {
+    int nE = m->n_experts, k = m->top_k, H = m->hidden, I = m->exp_inter;
+    float *logits = (float *)malloc(sizeof(float) * (size_t)nE);
+    int *idx = (int *)malloc(sizeof(int) * (size_t)k);
+    float *wts = (float *)malloc(sizeof(float) * (size_t)k);
+    float *g = (float *)malloc(sizeof(float) * (size_t)I), *u = (float *)malloc(sizeof(float) * (size_t)I);
+    float *eo = (float *)malloc(sizeof(float) * (size_t)H);
+    or_matmul(&lw->router, h, 1, logits);
+    int n = or_route_experts(logits, nE, k, m->norm_topk, 0, idx, wts);
+    memset(out, 0, sizeof(float) * (size_t)H);
+    for (int j = 0; j < n; j++) {
+        int e = idx[j];
+        if (idx_trace) idx_trace[j] = e;
+        or_matmul(&lw->exp_gate[e], h, 1, g);
+        or_matmul(&lw->exp_up[e], h, 1, u);
+        or_swiglu(g, u, I);
+        or_matmul(&lw->exp_down[e], g, 1, eo);
+        add_scaled(out, eo, wts[j], H);
+    }
+    free(logits);
+    free(idx);
+    free(wts);
+    free(g);
+    free(u);
+    free(eo);
+}
+
+/* decoder/cpu_batch.go:166-197 (decodeMultiStep) + program_cpu_n.go:406-563 (walkMulti) + forwardn.go:800-831 (lmHeadN).
+ * Pre-norm llama-style layer program: norm, q/k/v (M=B), optional QK-norm, RoPE at each row's own position,
+ * per-sequence append + attention, o-proj, residual, norm, gated FFN (dense at M=B, MoE per row), residual; final norm; head. */
+int or_decode_multi_step(const or_model *m, int B, const float *emb, or_cache **caches, float *logits, int *moe_idx_trace) {
+    int H = m->hidden, nH = m->n_heads, nKV = m->n_kv, hd = m->head_dim, I = m->inter;
+    int qDim = nH * hd, kvDim = nKV * hd;
+    for (int b = 0; b < B; b++)
+        if (caches[b]->pos >= caches[b]->cap) return -1;
+    float *h = (float *)malloc(sizeof(float) * (size_t)B * H);
+    float *norm = (float *)malloc(sizeof(float) * (size_t)B * H);
+    float *att = (float *)malloc(sizeof(float) * (size_t)B * H);
+    float *q = (float *)malloc(sizeof(float) * (size_t)B * qDim), *ctx = (float *)malloc(sizeof(float) * (size_t)B * qDim);
+    float *k = (float *)malloc(sizeof(float) * (size_t)B * kvDim), *v = (float *)malloc(sizeof(float) * (size_t)B * kvDim);
+    float *gate = NULL, *up = NULL;
+    if (m->n_experts == 0) {
+        gate = (float *)malloc(sizeof(float) * (size_t)B * I);
+        up = (float *)malloc(sizeof(float) * (size_t)B * I);
+    }
+    memcpy(h, emb, sizeof(float) * (size_t)B * H);
+    for (int l = 0; l < m->n_layers; l++) {
+        const or_layer *lw = &m->layers[l];
+        or_rmsnorm(norm, h, lw->attn_norm, B, H, m->eps, 0);
+        or_matmul(&lw->q, norm, B, q);
+        or_matmul(&lw->k, norm, B, k);
+        or_matmul(&lw->v, norm, B, v);
+        for (int b = 0; b < B; b++) {
+            float *qb = q + (size_t)b * qDim, *kb = k + (size_t)b * kvDim, *vb = v + (size_t)b * kvDim;
+            or_cache *c = caches[b];
+            if (lw->q_norm) {
+                qk_norm(qb, nH, hd, lw->q_norm, m->eps);
+                qk_norm(kb, nKV, hd, lw->k_norm, m->eps);
+            }
+            or_rope(qb, nH, hd, c->pos, m->inv_freq, hd / 2, 1.0);
+            or_rope(kb, nKV, hd, c->pos, m->inv_freq, hd / 2, 1.0);
+            float *kr = c->k[l] + (size_t)c->pos * kvDim, *vr = c->v[l] + (size_t)c->pos * kvDim;
+            if (m->kv_f16) { /* decoder/kvcache.go:21-40: stored as binary16 (round-half-up), widened on read */
+                for (int i = 0; i < kvDim; i++) {
+                    kr[i] = or_f16_to_f32(or_f32_to_f16(kb[i]));
+                    vr[i] = or_f16_to_f32(or_f32_to_f16(vb[i]));
+                }
+            } else {
+                memcpy(kr, kb, sizeof(float) * (size_t)kvDim);
+                memcpy(vr, vb, sizeof(float) * (size_t)kvDim);
+            }
+            or_attend(qb, ctx + (size_t)b * qDim, c->k[l], c->v[l], c->pos + 1, 0, nH, nKV, hd, m->attn_scale, m->softcap);
+        }
+        or_matmul(&lw->o, ctx, B, att);
+        for (size_t i = 0; i < (size_t)B * H; i++) h[i] += att[i];
+        or_rmsnorm(norm, h, lw->ffn_norm, B, H, m->eps, 0);
+        if (m->n_experts == 0) {
+            or_matmul(&lw->gate, norm, B, gate);
+            or_matmul(&lw->up, norm, B, up);
+            or_swiglu(gate, up, B * I);
+            or_matmul(&lw->down, gate, B, att);
+        } else {
+            for (int b = 0; b < B; b++)
+                moe_mlp(m, lw, norm + (size_t)b * H, att + (size_t)b * H,
+                        moe_idx_trace ? moe_idx_trace + ((size_t)b * m->n_layers + l) * m->top_k : NULL);
+        }
+        for (size_t i = 0; i < (size_t)B * H; i++) h[i] += att[i];
+    }
+    for (int b = 0; b < B; b++) caches[b]->pos++;
+    or_rmsnorm(h, h, m->final_norm, B, H, m->eps, 0);
+    or_matmul(&m->head, h, B, logits);
+    free(h);
+    free(norm);
+    free(att);
+    free(q);
+    free(ctx);
+    free(k);
+    free(v);
+    free(gate);
+    free(up);
+    return 0;
+}

@@ -1,0 +1,124 @@
+/*
+ * oracle.h — CPU restatement of goinfer's ragged batched decode step.
+ *
+ * TEST INFRASTRUCTURE ONLY. Nothing the product ships (the HIP kernels, the C-ABI host library, the
+ * benchmark's GPU leg) may call into this file; it exists so the GPU path has something to be checked
+ * against, and so the benchmark can time a CPU baseline beside the GPU number.
+ *
+ * Every function cites the reference file:line (relative to the goinfer tree) it restates. The
+ * arithmetic owned by the un-vendored module github.com/townsendmerino/aikit v1.78.0 (go.mod:8) is
+ * restated from its in-tree call sites and twins, and pinned by the SHA-256 fingerprints in
+ * testdata/kernel_fingerprints.json (see kprint.c).
+ *
+ * Pin status (checked by tests/test_oracle_fingerprints.py and tests/test_oracle_golden.py):
+ *   or_f32_to_f16 / or_f16_to_f32        pinned: linalg.F32ToF16, linalg.F16ToF32 fingerprints
+ *   or_dequant_q4k                       pinned: embed.GGUFFile(Q4_K).Tensor fingerprint
+ *   or_quantize_row_int8                 pinned: linalg.QuantizeRowInt8 fingerprint
+ *   or_quantize_act                      pinned: linalg.QuantizeActQ fingerprint (per-row and per-32)
+ *   or_quantize_int4_row / _mat          pinned: linalg.QuantizeGroupInt4Row, linalg.QuantizeInt4
+ *   or_qk_acc64 / or_av_acc64            pinned: linalg.MatmulQKAcc64, linalg.MatmulAVAcc64
+ *   or_rmsnorm, or_rope, or_swiglu, or_softmax_f32, or_topk, or_route_experts, or_argmax
+ *                                        plain Go in the reference, restated statement by statement;
+ *                                        pinned by closed forms + the HF goldens (llama-tiny, qwen3moe-tiny, mixtral-tiny)
+ *   or_matmul (f32 kind)                 parity unpinned at bit level (aikit's summation order is arch dependent);
+ *                                        pinned to tolerance by the HF goldens
+ *   or_matmul (q4k / w4a8 / w8a8 kinds)  parity unpinned at bit level: the reference's own result differs between
+ *                                        amd64 and arm64 (kernel_fingerprints.json). Restated in the mathematically
+ *                                        specified form (exact int32 dot per 32-group, f32 fold in ascending group
+ *                                        order, backend/cuda/actgroup.cu:298-355) and checked against an f64 sum.
+ */
+#ifndef GOINFER_ORACLE_H
+#define GOINFER_ORACLE_H
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- 16-bit conversions: internal/runtime/f16/f16.go:14-63 ---- */
+uint16_t or_f32_to_f16(float f);      /* round-half-up on the dropped bits */
+float or_f16_to_f32(uint16_t h);
+
+/* ---- Q4_K: decoder/gguf.go:1508-1537, backend/metal/kernels/gemm_kq_test.go:27-70 ---- */
+void or_q4k_scale_min(int j, const uint8_t *q12, int *sc, int *m);
+void or_dequant_q4k(const uint8_t *blocks, size_t n_blocks, float *out); /* 144 B -> 256 f32 each */
+
+/* ---- activation quantizers: backend/cuda/kv8_store.cu:3-35, actgroup.cu:26-54 ---- */
+float or_quantize_row_int8(const float *row, int n, int8_t *q);
+/* group==0: one scale per row (S[m]); group>0: S[m*nG+g], nG=ceil(K/group) */
+void or_quantize_act(const float *a, int M, int K, int group, int8_t *q, float *S);
+
+/* ---- int4 g32: decoder/fakequant.go:99-131, backend/cuda/internal/wpack/wpack.go:165-207 ---- */
+void or_quantize_int4_row(const float *row, int cols, int group, uint8_t *packed, float *scales);
+void or_quantize_int4_mat(const float *w, int rows, int cols, int group, uint8_t *q4, uint16_t *s16);
+
+/* ---- attention primitives: decoder/forwardn.go:379-383,488-490 (call sites of aikit MatmulQKAcc64/AVAcc64) ---- */
+void or_qk_acc64(const float *a, const float *keys, float *dst, int M, int hd, int nKeys, int off, int kvDim);
+void or_av_acc64(const float *scores, const float *vals, float *dst, int M, int nKeys, int hd, int off, int kvDim);
+
+/* ---- glue: decoder/rmsnorm.go:29-92,204-207; rope.go:28-64; mlp.go:269-290,370-440,130-184 ---- */
+void or_rmsnorm(float *dst, const float *src, const float *w, int rows, int dim, double eps, int add_one);
+void or_rope(float *vec, int heads, int head_dim, int pos, const double *inv_freq, int half, double scale);
+float or_silu(float x);
+void or_swiglu(float *gate, const float *up, int n);
+void or_softmax_f32(const float *x, int n, float *out);
+int or_topk(const float *x, int n, int k, int *idx, float *val);
+int or_route_experts(const float *logits, int nE, int k, int norm, double scale, int *idx, float *wts);
+int or_argmax(const float *x, int n); /* internal/runtime/sampling/sampler.go:485-520: first maximum wins */
+
+/* ---- weight matrices and the matmul dispatch: decoder/weightmat.go:845-985 ---- */
+enum { OR_F32 = 0, OR_Q4K = 1, OR_W4A8 = 2, OR_W8A8 = 3 };
+typedef struct {
+    int kind;           /* OR_* */
+    int N, K;           /* rows (outputs), cols (inputs) */
+    const void *data;   /* f32[N*K] | q4k blocks N*K/256*144 | nibbles N*((K+1)/2) | int8[N*K] */
+    const void *scales; /* w4a8: uint16 f16[N*ceil(K/32)] | w8a8: f32[N] */
+    int act_group;      /* activation quant group for int kinds: 32 (q4k mode) or 0 (per row) */
+} or_mat;
+void or_matmul(const or_mat *w, const float *a, int M, float *dst);
+/* the same product with f64 accumulation over dequantized weights and dequantized activations */
+void or_matmul_f64ref(const or_mat *w, const float *a, int M, double *dst);
+void or_set_threads(int n);
+
+/* ---- one sequence's decode attention over its own cache:
+ * decoder/program_cpu_n.go:497-515 + forwardn.go:295-500 (useAcc64, K=1) + kvcache.go:21-40 (f16 narrowing) ---- */
+void or_attend(const float *q, float *ctx, const float *keys, const float *vals, int n_keys, int start,
+               int nH, int nKV, int hd, double scale, double softcap);
+
+/* ---- the model and decodeMultiStep: decoder/cpu_batch.go:166-197, program_cpu_n.go:406-563, mlp.go:36-120 ---- */
+typedef struct {
+    or_mat q, k, v, o, gate, up, down; /* dense FFN when n_experts==0 */
+    const float *attn_norm, *ffn_norm; /* [hidden] */
+    const float *q_norm, *k_norm;      /* [hd] or NULL (Qwen3 QK-norm) */
+    or_mat router;                     /* [nE, hidden] */
+    or_mat *exp_gate, *exp_up, *exp_down; /* [nE] each */
+} or_layer;
+
+typedef struct {
+    int n_layers, hidden, n_heads, n_kv, head_dim, inter, vocab;
+    double eps, attn_scale, softcap;
+    const double *inv_freq; /* [head_dim/2] */
+    int n_experts, top_k, norm_topk, exp_inter;
+    int kv_f16;     /* 1: K/V rows narrowed to binary16 (round-half-up) on append */
+    or_layer *layers;
+    const float *final_norm;
+    or_mat head;
+} or_model;
+
+typedef struct {
+    int pos;       /* rows stored so far */
+    int cap;       /* allocated rows */
+    float **k, **v; /* per layer [cap][n_kv*head_dim] (values already narrowed when kv_f16) */
+} or_cache;
+
+or_cache *or_cache_new(const or_model *m, int cap);
+void or_cache_free(const or_model *m, or_cache *c);
+/* emb: [B][hidden] (embedding rows, already scaled); logits: [B][vocab]. Appends one position to every cache. */
+int or_decode_multi_step(const or_model *m, int B, const float *emb, or_cache **caches, float *logits,
+                         int *moe_idx_trace /* [B][layers][top_k] or NULL */);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
