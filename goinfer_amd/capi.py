@@ -1,0 +1,254 @@
+"""ctypes binding of librocmdecode.so (include/rocmdecode.h). numpy in, numpy out; no torch."""
+import ctypes as C
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "librocmdecode.so")
+HSACO_PATH = os.path.join(HERE, "lib", "rocmdecode_gfx950.hsaco")
+
+RD_OK, RD_DECLINED = 0, 1
+PROJ = dict(q=0, k=1, v=2, o=3, gate=4, up=5, down=6, head=7)
+VEC = dict(attn_norm=0, ffn_norm=1, q_norm=2, k_norm=3, final_norm=4, router=5)
+WANT_LOGITS, WANT_ARGMAX = 1, 2
+
+EXPORTS = [
+    "rd_device_open", "rd_device_open_image", "rd_device_close", "rd_last_error", "rd_backend_name", "rd_device_sync",
+    "rd_device_mem_info", "rd_matmul_bt", "rd_dequant_q4k", "rd_gemm_q4k", "rd_gemm_w8a8", "rd_gemm_w4a8",
+    "rd_attn_ragged", "rd_moe_route", "rd_rmsnorm", "rd_rope", "rd_model_create", "rd_model_destroy",
+    "rd_model_upload_q4k", "rd_model_upload_w8a8", "rd_model_upload_w4a8", "rd_model_upload_f32", "rd_model_finalize",
+    "rd_kv_configure", "rd_kv_upload", "rd_kv_truncate", "rd_kv_reset", "rd_step_batch", "rd_forward",
+    "rd_last_moe_indices", "rd_bench_steps", "rd_bench_kernel",
+]
+
+
+class RocmError(RuntimeError):
+    pass
+
+
+class ModelDesc(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("n_layers", "hidden", "n_heads", "n_kv_heads", "head_dim", "inter", "vocab")] + [
+        ("rms_eps", C.c_float), ("attn_scale", C.c_float), ("attn_softcap", C.c_float),
+        ("n_experts", C.c_int32), ("top_k", C.c_int32), ("norm_topk_prob", C.c_int32), ("expert_inter", C.c_int32),
+        ("qk_norm", C.c_int32), ("rope_inv_freq", C.c_void_p)]
+
+
+_lib = None
+
+
+def lib():
+    """The loaded C-ABI library. Raises when it has not been built: there is no fallback path."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RocmError("%s is missing: run `python -m goinfer_amd.build`" % LIB_PATH)
+        L = C.CDLL(LIB_PATH)
+        L.rd_last_error.restype = C.c_char_p
+        L.rd_backend_name.restype = C.c_char_p
+        for name in ("rd_device_close", "rd_model_destroy"):
+            getattr(L, name).restype = None
+        _lib = L
+    return _lib
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p) if a is not None else None
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def check(rc, what):
+    if rc != RD_OK:
+        kind = "declined" if rc == RD_DECLINED else "failed (%d)" % rc
+        raise RocmError("%s %s: %s" % (what, kind, lib().rd_last_error().decode()))
+
+
+class Device:
+    """rd_device: one MI355X, its code object and stream."""
+
+    def __init__(self, ordinal=0):
+        self.h = C.c_void_p()
+        check(lib().rd_device_open(ordinal, C.byref(self.h)), "rd_device_open")
+
+    def close(self):
+        if self.h:
+            lib().rd_device_close(self.h)
+            self.h = C.c_void_p()
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *a):
+        self.close()
+
+    def sync(self):
+        check(lib().rd_device_sync(self.h), "rd_device_sync")
+
+    def mem_info(self):
+        f, t = C.c_size_t(), C.c_size_t()
+        check(lib().rd_device_mem_info(self.h, C.byref(f), C.byref(t)), "rd_device_mem_info")
+        return f.value, t.value
+
+    def matmul_bt(self, a, b):
+        a, b = _f32(a), _f32(b)
+        M, K = a.shape
+        N = b.shape[0]
+        dst = np.empty((M, N), np.float32)
+        check(lib().rd_matmul_bt(self.h, _p(a), _p(b), _p(dst), M, K, N), "rd_matmul_bt")
+        return dst
+
+    def dequant_q4k(self, blocks, N, K):
+        blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+        out = np.empty((N, K), np.float32)
+        check(lib().rd_dequant_q4k(self.h, _p(blocks), N, K, _p(out)), "rd_dequant_q4k")
+        return out
+
+    def gemm_q4k(self, blocks, N, K, a, blocks2=None):
+        a = _f32(a)
+        blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+        b2 = None if blocks2 is None else np.ascontiguousarray(blocks2, dtype=np.uint8)
+        dst = np.empty((a.shape[0], N), np.float32)
+        check(lib().rd_gemm_q4k(self.h, _p(blocks), N, K, _p(a), a.shape[0], _p(dst), _p(b2)), "rd_gemm_q4k")
+        return dst
+
+    def gemm_w8a8(self, q, scales, a):
+        a = _f32(a)
+        q = np.ascontiguousarray(q, dtype=np.int8)
+        scales = _f32(scales)
+        N, K = q.shape
+        dst = np.empty((a.shape[0], N), np.float32)
+        check(lib().rd_gemm_w8a8(self.h, _p(q), _p(scales), N, K, _p(a), a.shape[0], _p(dst)), "rd_gemm_w8a8")
+        return dst
+
+    def gemm_w4a8(self, nib, s16, K, a):
+        a = _f32(a)
+        nib = np.ascontiguousarray(nib, dtype=np.uint8)
+        s16 = np.ascontiguousarray(s16, dtype=np.uint16)
+        N = nib.shape[0]
+        dst = np.empty((a.shape[0], N), np.float32)
+        check(lib().rd_gemm_w4a8(self.h, _p(nib), _p(s16), N, K, _p(a), a.shape[0], _p(dst)), "rd_gemm_w4a8")
+        return dst
+
+    def attn_ragged(self, lens, k, v, q, n_h, n_kv, hd, scale, softcap=0.0):
+        lens = np.ascontiguousarray(lens, dtype=np.int32)
+        off = np.zeros(len(lens), np.int64)
+        off[1:] = np.cumsum(lens[:-1])
+        k, v, q = _f32(k), _f32(v), _f32(q)
+        out = np.empty((len(lens), n_h * hd), np.float32)
+        check(lib().rd_attn_ragged(self.h, len(lens), _p(lens), _p(off), _p(k), _p(v), _p(q), n_h, n_kv, hd,
+                                   C.c_float(scale), C.c_float(softcap), _p(out)), "rd_attn_ragged")
+        return out
+
+    def moe_route(self, logits, k, norm):
+        logits = _f32(logits)
+        T, nE = logits.shape
+        idx = np.empty((T, k), np.int32)
+        wgt = np.empty((T, k), np.float32)
+        check(lib().rd_moe_route(self.h, _p(logits), T, nE, k, int(norm), _p(idx), _p(wgt)), "rd_moe_route")
+        return idx, wgt
+
+    def rmsnorm(self, x, w, eps):
+        x, w = _f32(x), _f32(w)
+        out = np.empty_like(x)
+        check(lib().rd_rmsnorm(self.h, _p(x), _p(w), x.shape[0], x.shape[1], C.c_float(eps), _p(out)), "rd_rmsnorm")
+        return out
+
+    def rope(self, vec, heads, head_dim, pos, inv_freq):
+        v = _f32(vec).copy()
+        pos = np.ascontiguousarray(pos, dtype=np.int32)
+        inv = np.ascontiguousarray(inv_freq, dtype=np.float64)
+        check(lib().rd_rope(self.h, _p(v), v.shape[0], heads, head_dim, _p(pos), _p(inv)), "rd_rope")
+        return v
+
+    def bench_kernel(self, name, args, warmup, iters):
+        a = np.ascontiguousarray(args, dtype=np.int64)
+        ms = np.empty(iters, np.float32)
+        check(lib().rd_bench_kernel(self.h, name.encode(), _p(a), len(a), warmup, iters, _p(ms)), "rd_bench_kernel")
+        return ms
+
+
+class Model:
+    """rd_model: the resident decoder (goinfer's resident.Forward + DecodeSubsystem for this backend)."""
+
+    def __init__(self, dev, cfg, inv_freq):
+        self.dev, self.cfg = dev, dict(cfg)
+        self._inv = np.ascontiguousarray(inv_freq, dtype=np.float64)
+        d = ModelDesc(cfg["n_layers"], cfg["hidden"], cfg["n_heads"], cfg["n_kv"], cfg["head_dim"], cfg.get("inter", 0),
+                      cfg["vocab"], cfg["eps"], cfg["attn_scale"], cfg.get("softcap", 0.0), cfg.get("n_experts", 0),
+                      cfg.get("top_k", 0), int(cfg.get("norm_topk", 0)), cfg.get("exp_inter", 0), int(cfg.get("qk_norm", 0)),
+                      _p(self._inv))
+        self.h = C.c_void_p()
+        check(lib().rd_model_create(dev.h, C.byref(d), C.byref(self.h)), "rd_model_create")
+
+    def close(self):
+        if self.h:
+            lib().rd_model_destroy(self.h)
+            self.h = C.c_void_p()
+
+    def upload_q4k(self, layer, proj, blocks, N, K):
+        blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+        check(lib().rd_model_upload_q4k(self.h, layer, PROJ[proj], _p(blocks), N, K), "rd_model_upload_q4k")
+
+    def upload_w8a8(self, layer, proj, q, scales):
+        q = np.ascontiguousarray(q, dtype=np.int8)
+        scales = _f32(scales)
+        check(lib().rd_model_upload_w8a8(self.h, layer, PROJ[proj], _p(q), _p(scales), q.shape[0], q.shape[1]),
+              "rd_model_upload_w8a8")
+
+    def upload_w4a8(self, layer, proj, expert, nib, s16, K):
+        nib = np.ascontiguousarray(nib, dtype=np.uint8)
+        s16 = np.ascontiguousarray(s16, dtype=np.uint16)
+        check(lib().rd_model_upload_w4a8(self.h, layer, PROJ[proj], expert, _p(nib), _p(s16), nib.shape[0], K),
+              "rd_model_upload_w4a8")
+
+    def upload_f32(self, layer, which, v):
+        v = _f32(v)
+        check(lib().rd_model_upload_f32(self.h, layer, VEC[which], _p(v), C.c_size_t(v.size)), "rd_model_upload_f32")
+
+    def finalize(self):
+        check(lib().rd_model_finalize(self.h), "rd_model_finalize")
+
+    def kv_configure(self, slots, ctx_cap):
+        check(lib().rd_kv_configure(self.h, slots, ctx_cap), "rd_kv_configure")
+
+    def kv_upload(self, slot, layer, base, keys, vals):
+        keys, vals = _f32(keys), _f32(vals)
+        check(lib().rd_kv_upload(self.h, slot, layer, base, keys.shape[0], _p(keys), _p(vals)), "rd_kv_upload")
+
+    def kv_reset(self, slot):
+        check(lib().rd_kv_reset(self.h, slot), "rd_kv_reset")
+
+    def kv_truncate(self, slot, pos):
+        check(lib().rd_kv_truncate(self.h, slot, pos), "rd_kv_truncate")
+
+    def step_batch(self, slots, pos, emb, want=WANT_LOGITS):
+        emb = _f32(emb)
+        B = emb.shape[0]
+        slots = np.ascontiguousarray(slots, dtype=np.int32)
+        pos = np.ascontiguousarray(pos, dtype=np.int32)
+        logits = np.empty((B, self.cfg["vocab"]), np.float32) if want & WANT_LOGITS else None
+        ids = np.empty(B, np.int32) if want & WANT_ARGMAX else None
+        check(lib().rd_step_batch(self.h, B, _p(slots), _p(pos), _p(emb), want, _p(logits), _p(ids)), "rd_step_batch")
+        return logits, ids
+
+    def forward(self, slot, pos, emb):
+        emb = _f32(emb)
+        logits = np.empty(self.cfg["vocab"], np.float32)
+        check(lib().rd_forward(self.h, slot, pos, _p(emb), _p(logits)), "rd_forward")
+        return logits
+
+    def last_moe_indices(self, B):
+        idx = np.empty((B, self.cfg["n_layers"], self.cfg["top_k"]), np.int32)
+        check(lib().rd_last_moe_indices(self.h, _p(idx)), "rd_last_moe_indices")
+        return idx
+
+    def bench_steps(self, slots, pos0, emb, warmup, steps):
+        emb = _f32(emb)
+        slots = np.ascontiguousarray(slots, dtype=np.int32)
+        pos0 = np.ascontiguousarray(pos0, dtype=np.int32)
+        ms = np.empty(steps, np.float32)
+        check(lib().rd_bench_steps(self.h, emb.shape[0], _p(slots), _p(pos0), _p(emb), warmup, steps, _p(ms)), "rd_bench_steps")
+        return ms

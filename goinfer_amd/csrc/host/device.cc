@@ -1,0 +1,259 @@
+// device.cc — device open/close, code-object loading, memory helpers, weight upload and the GEMM launcher.
+#include "device.h"
+#include <dlfcn.h>
+#include <mutex>
+#include <stdlib.h>
+#include <string.h>
+
+static thread_local char g_err[512] = "";
+
+void rd_set_error(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+}
+
+bool rd_hip_ok(const HipApi *hip, hipError_t e, const char *what) {
+    if (e == hipSuccess) return true;
+    rd_set_error("%s: %s", what, hip ? hip->GetErrorString(e) : "hip not loaded");
+    return false;
+}
+
+extern "C" const char *rd_last_error(void) { return g_err; }
+extern "C" const char *rd_backend_name(void) { return "rocm"; }
+
+int rd_device::alloc(void **p, size_t n) {
+    if (!rd_hip_ok(hip, hip->Malloc(p, n), "hipMalloc")) return RD_ERR_HIP;
+    return RD_OK;
+}
+void rd_device::release(void *p) {
+    if (p) (void)hip->Free(p);
+}
+int rd_device::h2d(void *dst, const void *src, size_t n) {
+    return rd_hip_ok(hip, hip->MemcpyAsync(dst, src, n, hipMemcpyHostToDevice, stream), "hipMemcpy H2D") ? RD_OK : RD_ERR_HIP;
+}
+int rd_device::d2h(void *dst, const void *src, size_t n) {
+    if (!rd_hip_ok(hip, hip->MemcpyAsync(dst, src, n, hipMemcpyDeviceToHost, stream), "hipMemcpy D2H")) return RD_ERR_HIP;
+    return sync();
+}
+int rd_device::sync() { return rd_hip_ok(hip, hip->StreamSynchronize(stream), "hipStreamSynchronize") ? RD_OK : RD_ERR_HIP; }
+
+static bool read_file(const std::string &path, std::vector<char> &out) {
+    FILE *f = fopen(path.c_str(), "rb");
+    if (!f) return false;
+    fseek(f, 0, SEEK_END);
+    long n = ftell(f);
+    fseek(f, 0, SEEK_SET);
+    out.resize((size_t)n);
+    bool ok = n > 0 && fread(out.data(), 1, (size_t)n, f) == (size_t)n;
+    fclose(f);
+    return ok;
+}
+
+// The code object sits beside this shared library unless ROCMDECODE_HSACO names it.
+static std::string default_hsaco_path() {
+    if (const char *e = getenv("ROCMDECODE_HSACO")) return e;
+    Dl_info info;
+    if (dladdr((void *)&rd_last_error, &info) && info.dli_fname) {
+        std::string p = info.dli_fname;
+        size_t s = p.find_last_of('/');
+        return (s == std::string::npos ? std::string(".") : p.substr(0, s)) + "/rocmdecode_gfx950.hsaco";
+    }
+    return "rocmdecode_gfx950.hsaco";
+}
+
+struct KName {
+    const char *name;
+    hipFunction_t Kernels::*slot;
+};
+static const KName kNames[] = {
+    {"rd_k_dequant_q4k", &Kernels::dequant_q4k},
+    {"rd_k_retile_q4k", &Kernels::retile_q4k},
+    {"rd_k_gemm_q4k_w4", &Kernels::gemm_q4k_w4},
+    {"rd_k_gemm_q4k_w2", &Kernels::gemm_q4k_w2},
+    {"rd_k_quant_act", &Kernels::quant_act},
+    {"rd_k_reduce_splits", &Kernels::reduce_splits},
+    {"rd_k_add_rmsnorm_quant", &Kernels::add_rmsnorm_quant},
+    {"rd_k_swiglu_quant", &Kernels::swiglu_quant},
+    {"rd_k_retile_w8a8", &Kernels::retile_w8a8},
+    {"rd_k_gemm_w8a8", &Kernels::gemm_w8a8},
+    {"rd_k_retile_w4a8", &Kernels::retile_w4a8},
+    {"rd_k_gemm_w4a8", &Kernels::gemm_w4a8},
+    {"rd_k_kv_store", &Kernels::kv_store},
+    {"rd_k_qkv_rope_store", &Kernels::qkv_rope_store},
+    {"rd_k_attn_partial", &Kernels::attn_partial},
+    {"rd_k_attn_combine", &Kernels::attn_combine},
+    {"rd_k_attn_combine_quant", &Kernels::attn_combine_quant},
+    {"rd_k_rmsnorm", &Kernels::rmsnorm},
+    {"rd_k_rope", &Kernels::rope},
+    {"rd_k_argmax_rows", &Kernels::argmax_rows},
+    {"rd_k_matmul_f32", &Kernels::matmul_f32},
+    {"rd_k_moe_route", &Kernels::moe_route},
+};
+
+static int open_common(int ordinal, const void *image, rd_device **out) {
+    const char *why = nullptr;
+    const HipApi *hip = hip_api(&why);
+    if (!hip) {
+        rd_set_error("%s", why);
+        return RD_DECLINED; // no ROCm runtime on this machine: the backend declines, the caller stays on its CPU path
+    }
+    if (!rd_hip_ok(hip, hip->Init(0), "hipInit")) return RD_DECLINED;
+    int n = 0;
+    if (!rd_hip_ok(hip, hip->GetDeviceCount(&n), "hipGetDeviceCount") || n <= ordinal) {
+        rd_set_error("no HIP device %d (count %d)", ordinal, n);
+        return RD_DECLINED;
+    }
+    rd_device *d = new rd_device();
+    d->hip = hip;
+    d->ordinal = ordinal;
+    if (!rd_hip_ok(hip, hip->SetDevice(ordinal), "hipSetDevice") || !rd_hip_ok(hip, hip->StreamCreate(&d->stream), "hipStreamCreate") ||
+        !rd_hip_ok(hip, hip->ModuleLoadData(&d->module, image), "hipModuleLoadData(gfx950 code object)")) {
+        delete d;
+        return RD_ERR_HIP;
+    }
+    for (const KName &kn : kNames) {
+        hipFunction_t f = nullptr;
+        if (hip->ModuleGetFunction(&f, d->module, kn.name) != hipSuccess) {
+            rd_set_error("code object lacks kernel %s", kn.name);
+            (void)hip->ModuleUnload(d->module);
+            (void)hip->StreamDestroy(d->stream);
+            delete d;
+            return RD_ERR_HIP;
+        }
+        d->k.*(kn.slot) = f;
+    }
+    *out = d;
+    return RD_OK;
+}
+
+extern "C" int rd_device_open_image(int ordinal, const void *hsaco, size_t len, rd_device **out) {
+    if (!hsaco || len == 0 || !out) {
+        rd_set_error("rd_device_open_image: null image");
+        return RD_ERR_ARG;
+    }
+    return open_common(ordinal, hsaco, out);
+}
+
+extern "C" int rd_device_open(int ordinal, rd_device **out) {
+    if (!out) return RD_ERR_ARG;
+    std::vector<char> img;
+    std::string path = default_hsaco_path();
+    if (!read_file(path, img)) {
+        rd_set_error("cannot read gfx950 code object %s (build it with goinfer_amd/build.py)", path.c_str());
+        return RD_ERR_STATE;
+    }
+    return open_common(ordinal, img.data(), out);
+}
+
+extern "C" void rd_device_close(rd_device *d) {
+    if (!d) return;
+    (void)d->hip->StreamSynchronize(d->stream);
+    for (void *p : d->owned) (void)d->hip->Free(p);
+    (void)d->hip->ModuleUnload(d->module);
+    (void)d->hip->StreamDestroy(d->stream);
+    delete d;
+}
+
+extern "C" int rd_device_sync(rd_device *d) { return d ? d->sync() : RD_ERR_ARG; }
+
+extern "C" int rd_device_mem_info(rd_device *d, size_t *free_b, size_t *total_b) {
+    if (!d) return RD_ERR_ARG;
+    HIPCHK(MemGetInfo(free_b, total_b));
+    return RD_OK;
+}
+
+// ---- GEMM planning: enough blocks to cover the 256 CUs, at least two K-blocks per split ----
+GemmPlan plan_gemm(int N, int nKB) {
+    GemmPlan p;
+    p.wpb = 4;
+    int groups = (N + 127) / 128;
+    int want = (512 + groups - 1) / groups; // ~2 blocks per CU
+    int maxSplits = nKB >= 2 ? nKB / 2 : 1;
+    int splits = want < 1 ? 1 : (want > maxSplits ? maxSplits : want);
+    if (const char *e = getenv("ROCMDECODE_SPLITS")) splits = atoi(e) > 0 ? atoi(e) : splits;
+    if (splits > nKB) splits = nKB;
+    p.kbPerSplit = (nKB + splits - 1) / splits;
+    p.splits = (nKB + p.kbPerSplit - 1) / p.kbPerSplit;
+    return p;
+}
+
+size_t panel_bytes_for(const DevWeight &w) { return w.kind == 0 ? (size_t)(w.K / 256) * Q4K_PANEL_BYTES : (size_t)(w.K / 128) * LIN_PANEL_BYTES; }
+int panel_kind_for(const DevWeight &w) { return w.kind == 0 ? PANEL_Q4K : (w.kind == 1 ? PANEL_LIN : PANEL_LIN4); }
+
+int upload_q4k(rd_device *d, const void *blocks, int N, int K, DevWeight *w) {
+    if (N <= 0 || K <= 0 || K % 256 || N % 32) {
+        rd_set_error("q4k upload: N=%d must be a multiple of 32 and K=%d of 256", N, K);
+        return RD_DECLINED;
+    }
+    size_t bytes = (size_t)N * (K / 256) * 144;
+    DevBuf raw(d);
+    int rc = raw.alloc(bytes);
+    if (rc) return rc;
+    if ((rc = d->alloc(&w->tiled, bytes))) return rc;
+    if ((rc = d->h2d(raw.p, blocks, bytes))) return rc;
+    int nSB = K / 256;
+    if ((rc = d->launch(d->k.retile_q4k, N / 32, nSB, 1, 320, (const void *)raw.p, w->tiled, N, nSB))) return rc;
+    if ((rc = d->sync())) return rc;
+    w->kind = 0, w->N = N, w->K = K;
+    return RD_OK;
+}
+
+int upload_w8a8(rd_device *d, const int8_t *q, const float *row_scale, int N, int K, DevWeight *w) {
+    if (N <= 0 || K <= 0 || K % 128 || N % 32) {
+        rd_set_error("w8a8 upload: N=%d must be a multiple of 32 and K=%d of 128", N, K);
+        return RD_DECLINED;
+    }
+    size_t bytes = (size_t)N * K;
+    DevBuf raw(d);
+    int rc = raw.alloc(bytes);
+    if (rc) return rc;
+    if ((rc = d->alloc(&w->tiled, bytes))) return rc;
+    if ((rc = d->alloc(&w->scales, sizeof(float) * (size_t)N))) return rc;
+    if ((rc = d->h2d(raw.p, q, bytes))) return rc;
+    if ((rc = d->h2d(w->scales, row_scale, sizeof(float) * (size_t)N))) return rc;
+    if ((rc = d->launch(d->k.retile_w8a8, N / 32, K / 128, 1, 256, (const void *)raw.p, w->tiled, N, K))) return rc;
+    if ((rc = d->sync())) return rc;
+    w->kind = 1, w->N = N, w->K = K;
+    return RD_OK;
+}
+
+int upload_w4a8(rd_device *d, const uint8_t *nib, const uint16_t *s16, int N, int K, DevWeight *w) {
+    if (N <= 0 || K <= 0 || K % 128 || N % 32) {
+        rd_set_error("w4a8 upload: N=%d must be a multiple of 32 and K=%d of 128", N, K);
+        return RD_DECLINED;
+    }
+    size_t nb = (size_t)N * K / 2, sb = (size_t)N * (K / 32) * 2;
+    DevBuf raw(d), rs(d);
+    int rc;
+    if ((rc = raw.alloc(nb)) || (rc = rs.alloc(sb))) return rc;
+    if ((rc = d->alloc(&w->tiled, nb + sb))) return rc;
+    if ((rc = d->h2d(raw.p, nib, nb)) || (rc = d->h2d(rs.p, s16, sb))) return rc;
+    if ((rc = d->launch(d->k.retile_w4a8, N / 32, K / 128, 1, 320, (const void *)raw.p, (const void *)rs.p, w->tiled, N, K))) return rc;
+    if ((rc = d->sync())) return rc;
+    w->kind = 2, w->N = N, w->K = K;
+    return RD_OK;
+}
+
+void free_weight(rd_device *d, DevWeight *w) {
+    d->release(w->tiled);
+    d->release(w->scales);
+    *w = DevWeight();
+}
+
+int launch_gemm(rd_device *d, const DevWeight &w, const void *Xp, float *P, int M, GemmPlan *plan_out) {
+    if (M < 1 || M > 32) {
+        rd_set_error("gemm: M=%d outside 1..32", M);
+        return RD_ERR_ARG;
+    }
+    int nKB = w.kind == 0 ? w.K / 256 : w.K / 128;
+    GemmPlan p = plan_gemm(w.N, nKB);
+    if (plan_out) *plan_out = p;
+    unsigned gx = (unsigned)((w.N + 32 * p.wpb - 1) / (32 * p.wpb));
+    if (w.kind == 0)
+        return d->launch(d->k.gemm_q4k_w4, gx, p.splits, 1, 256, (const void *)w.tiled, Xp, P, w.N, nKB, p.kbPerSplit, M);
+    if (w.kind == 1)
+        return d->launch(d->k.gemm_w8a8, gx, p.splits, 1, 256, (const void *)w.tiled, (const void *)w.scales, Xp, P, w.N, nKB, p.kbPerSplit, M);
+    return d->launch(d->k.gemm_w4a8, gx, p.splits, 1, 256, (const void *)w.tiled, Xp, P, w.N, nKB, p.kbPerSplit, M);
+}

@@ -1,0 +1,85 @@
+// device.h — the device object behind rd_device: the HIP module, its kernels, one stream, and small helpers.
+#pragma once
+#include "../../../include/rocmdecode.h"
+#include "hipdyn.h"
+#include <stdarg.h>
+#include <stdio.h>
+#include <string>
+#include <vector>
+
+void rd_set_error(const char *fmt, ...);
+bool rd_hip_ok(const HipApi *hip, hipError_t e, const char *what);
+#define HIPCHK(call)                                                      \
+    do {                                                                  \
+        if (!rd_hip_ok(d->hip, d->hip->call, #call)) return RD_ERR_HIP;   \
+    } while (0)
+
+// sizes shared with the kernels (goinfer_amd/csrc/kernels/common.h)
+constexpr size_t Q4K_PANEL_BYTES = 17 * 64 * 16;
+constexpr size_t LIN_PANEL_BYTES = 8 * 64 * 16;
+constexpr size_t Q4K_TILE_BYTES = 4608;
+enum { PANEL_Q4K = 0, PANEL_LIN = 1, PANEL_LIN4 = 2 };
+
+struct Kernels {
+    hipFunction_t dequant_q4k, retile_q4k, gemm_q4k_w4, gemm_q4k_w2, quant_act, reduce_splits, add_rmsnorm_quant, swiglu_quant;
+    hipFunction_t retile_w8a8, gemm_w8a8, retile_w4a8, gemm_w4a8;
+    hipFunction_t kv_store, qkv_rope_store, attn_partial, attn_combine, attn_combine_quant;
+    hipFunction_t rmsnorm, rope, argmax_rows, matmul_f32, moe_route;
+};
+
+struct rd_device {
+    const HipApi *hip = nullptr;
+    int ordinal = 0;
+    hipModule_t module = nullptr;
+    hipStream_t stream = nullptr;
+    Kernels k{};
+    std::vector<void *> owned; // device allocations freed at close
+
+    template <typename... A> int launch(hipFunction_t f, unsigned gx, unsigned gy, unsigned gz, unsigned bx, A... a) {
+        void *args[] = {(void *)&a...};
+        hipError_t e = hip->ModuleLaunchKernel(f, gx, gy, gz, bx, 1, 1, 0, stream, args, nullptr);
+        return rd_hip_ok(hip, e, "hipModuleLaunchKernel") ? RD_OK : RD_ERR_HIP;
+    }
+    int alloc(void **p, size_t n);
+    void release(void *p);
+    int h2d(void *dst, const void *src, size_t n);
+    int d2h(void *dst, const void *src, size_t n);
+    int sync();
+};
+
+// A device buffer that frees itself (for the call-scoped temporaries of the kernel-level entry points).
+struct DevBuf {
+    rd_device *d;
+    void *p = nullptr;
+    explicit DevBuf(rd_device *dev) : d(dev) {}
+    ~DevBuf() {
+        if (p) d->release(p);
+    }
+    int alloc(size_t n) { return d->alloc(&p, n ? n : 16); }
+    template <typename T> T *as() { return (T *)p; }
+};
+
+// split-K plan of one GEMM launch
+struct GemmPlan {
+    int wpb;        // waves per block: 4 (128 rows) or 2 (64 rows)
+    int splits;     // grid.y
+    int kbPerSplit; // K-blocks (super-blocks or 128-wide blocks) per split
+};
+GemmPlan plan_gemm(int N, int nKB);
+
+// Weight matrix resident on the device in its GEMM tiling.
+struct DevWeight {
+    int kind = -1; // 0 q4k, 1 w8a8, 2 w4a8
+    int N = 0, K = 0;
+    void *tiled = nullptr;  // re-tiled codes
+    void *scales = nullptr; // w8a8: f32[N]
+};
+
+int upload_q4k(rd_device *d, const void *blocks, int N, int K, DevWeight *w);
+int upload_w8a8(rd_device *d, const int8_t *q, const float *row_scale, int N, int K, DevWeight *w);
+int upload_w4a8(rd_device *d, const uint8_t *nib, const uint16_t *s16, int N, int K, DevWeight *w);
+void free_weight(rd_device *d, DevWeight *w);
+// P[splits][32][N] = panels(Xp) . W^T ; returns the plan used
+int launch_gemm(rd_device *d, const DevWeight &w, const void *Xp, float *P, int M, GemmPlan *plan);
+size_t panel_bytes_for(const DevWeight &w);
+int panel_kind_for(const DevWeight &w);

@@ -1,0 +1,168 @@
+// ops.cc — the kernel-level entry points (host pointers in, host pointers out): what the reference's kernel tests bind
+// (backend/cuda/kernels/actgroup_kernel_test.go, flash_decode_test.go, moe_route_test.go) and what the micro-benchmarks time.
+#include "device.h"
+#include <algorithm>
+#include <string.h>
+
+#define RC(x)                \
+    do {                     \
+        int rc_ = (x);       \
+        if (rc_) return rc_; \
+    } while (0)
+
+extern "C" int rd_dequant_q4k(rd_device *d, const void *blocks, int N, int K, float *out) {
+    if (!d || !blocks || !out || N <= 0 || K <= 0 || K % 256) {
+        rd_set_error("rd_dequant_q4k: bad arguments (K must be a multiple of 256)");
+        return RD_ERR_ARG;
+    }
+    size_t nb = (size_t)N * (K / 256);
+    DevBuf raw(d), o(d);
+    RC(raw.alloc(nb * 144));
+    RC(o.alloc(nb * 256 * sizeof(float)));
+    RC(d->h2d(raw.p, blocks, nb * 144));
+    RC(d->launch(d->k.dequant_q4k, (unsigned)nb, 1, 1, 256, (const void *)raw.p, o.as<float>(), (long)nb));
+    return d->d2h(out, o.p, nb * 256 * sizeof(float));
+}
+
+// a[M][K] host -> per-32 quantized f16 panels on the device, in chunks of 32 rows. Returns device buffers.
+static int quantize_rows(rd_device *d, const float *a_dev, int M, int K, int kind, size_t pbytes, void *Xp) {
+    (void)pbytes;
+    return d->launch(d->k.quant_act, (unsigned)((K + 255) / 256), (unsigned)M, 1, 256, a_dev, Xp, K, kind);
+}
+
+static int gemm_host(rd_device *d, DevWeight &w, DevWeight *w2, const float *a, int M, float *dst) {
+    int N = w.N, K = w.K;
+    size_t pbytes = panel_bytes_for(w);
+    int kind = panel_kind_for(w);
+    DevBuf A(d), Xp(d), P(d), O(d);
+    RC(A.alloc(sizeof(float) * (size_t)32 * K));
+    RC(Xp.alloc(pbytes));
+    int nKB = w.kind == 0 ? K / 256 : K / 128;
+    int Ntot = w2 ? 2 * N : N;
+    int maxSplits = plan_gemm(Ntot, nKB).splits;
+    RC(P.alloc(sizeof(float) * (size_t)maxSplits * 32 * Ntot));
+    RC(O.alloc(sizeof(float) * (size_t)32 * N));
+    for (int m0 = 0; m0 < M; m0 += 32) {
+        int mc = std::min(32, M - m0);
+        RC(d->h2d(A.p, a + (size_t)m0 * K, sizeof(float) * (size_t)mc * K));
+        RC(quantize_rows(d, A.as<float>(), mc, K, kind, pbytes, Xp.p));
+        GemmPlan plan;
+        if (!w2) {
+            RC(launch_gemm(d, w, Xp.p, P.as<float>(), mc, &plan));
+            RC(d->launch(d->k.reduce_splits, (unsigned)((N + 255) / 256), (unsigned)mc, 1, 256, (const float *)P.p, O.as<float>(), N, plan.splits));
+        } else {
+            // fused gate/up: w holds [gate; up] stacked (2N rows)
+            RC(launch_gemm(d, *w2, Xp.p, P.as<float>(), mc, &plan));
+            DevBuf X2(d);
+            RC(X2.alloc((size_t)((N + 255) / 256) * Q4K_PANEL_BYTES));
+            RC(d->launch(d->k.swiglu_quant, (unsigned)((N + 255) / 256), (unsigned)mc, 1, 256, (const float *)P.p, plan.splits, N, X2.p,
+                         (int)PANEL_Q4K, O.as<float>()));
+            RC(d->sync());
+        }
+        RC(d->d2h(dst + (size_t)m0 * N, O.p, sizeof(float) * (size_t)mc * N));
+    }
+    return RD_OK;
+}
+
+extern "C" int rd_gemm_q4k(rd_device *d, const void *W, int N, int K, const float *a, int M, float *dst, const void *W2) {
+    if (!d || !W || !a || !dst || M <= 0) {
+        rd_set_error("rd_gemm_q4k: bad arguments");
+        return RD_ERR_ARG;
+    }
+    DevWeight w, wcat;
+    int rc;
+    if (!W2) {
+        if ((rc = upload_q4k(d, W, N, K, &w))) return rc;
+        rc = gemm_host(d, w, nullptr, a, M, dst);
+        free_weight(d, &w);
+        return rc;
+    }
+    if (N % 256) { // the SwiGLU output feeds a Q4_K-style panel writer in chunks of 256
+        rd_set_error("rd_gemm_q4k fused: N=%d must be a multiple of 256", N);
+        return RD_DECLINED;
+    }
+    size_t bytes = (size_t)N * (K / 256) * 144;
+    std::vector<uint8_t> cat(2 * bytes);
+    memcpy(cat.data(), W, bytes);
+    memcpy(cat.data() + bytes, W2, bytes);
+    if ((rc = upload_q4k(d, cat.data(), 2 * N, K, &wcat))) return rc;
+    w.kind = 0, w.N = N, w.K = K;
+    rc = gemm_host(d, w, &wcat, a, M, dst);
+    free_weight(d, &wcat);
+    return rc;
+}
+
+extern "C" int rd_gemm_w8a8(rd_device *d, const int8_t *q, const float *row_scale, int N, int K, const float *a, int M, float *dst) {
+    if (!d || !q || !row_scale || !a || !dst || M <= 0) return RD_ERR_ARG;
+    DevWeight w;
+    int rc = upload_w8a8(d, q, row_scale, N, K, &w);
+    if (rc) return rc;
+    rc = gemm_host(d, w, nullptr, a, M, dst);
+    free_weight(d, &w);
+    return rc;
+}
+
+extern "C" int rd_gemm_w4a8(rd_device *d, const uint8_t *nib, const uint16_t *s16, int N, int K, const float *a, int M, float *dst) {
+    if (!d || !nib || !s16 || !a || !dst || M <= 0) return RD_ERR_ARG;
+    DevWeight w;
+    int rc = upload_w4a8(d, nib, s16, N, K, &w);
+    if (rc) return rc;
+    rc = gemm_host(d, w, nullptr, a, M, dst);
+    free_weight(d, &w);
+    return rc;
+}
+
+extern "C" int rd_matmul_bt(rd_device *d, const float *a, const float *b, float *dst, int M, int K, int N) {
+    if (!d || !a || !b || !dst || M <= 0 || K <= 0 || N <= 0) return RD_ERR_ARG;
+    DevBuf A(d), B(d), D(d);
+    RC(A.alloc(sizeof(float) * (size_t)M * K));
+    RC(B.alloc(sizeof(float) * (size_t)N * K));
+    RC(D.alloc(sizeof(float) * (size_t)M * N));
+    RC(d->h2d(A.p, a, sizeof(float) * (size_t)M * K));
+    RC(d->h2d(B.p, b, sizeof(float) * (size_t)N * K));
+    RC(d->launch(d->k.matmul_f32, (unsigned)((N + 63) / 64), (unsigned)M, 1, 64, (const float *)A.p, (const float *)B.p, D.as<float>(), M, K, N));
+    return d->d2h(dst, D.p, sizeof(float) * (size_t)M * N);
+}
+
+extern "C" int rd_rmsnorm(rd_device *d, const float *x, const float *w, int rows, int dim, float eps, float *out) {
+    if (!d || !x || !w || !out || rows <= 0 || dim <= 0) return RD_ERR_ARG;
+    DevBuf X(d), W(d), O(d);
+    RC(X.alloc(sizeof(float) * (size_t)rows * dim));
+    RC(W.alloc(sizeof(float) * (size_t)dim));
+    RC(O.alloc(sizeof(float) * (size_t)rows * dim));
+    RC(d->h2d(X.p, x, sizeof(float) * (size_t)rows * dim));
+    RC(d->h2d(W.p, w, sizeof(float) * (size_t)dim));
+    RC(d->launch(d->k.rmsnorm, (unsigned)rows, 1, 1, 256, (const float *)X.p, (const float *)W.p, O.as<float>(), dim, eps));
+    return d->d2h(out, O.p, sizeof(float) * (size_t)rows * dim);
+}
+
+extern "C" int rd_rope(rd_device *d, float *vec, int rows, int heads, int head_dim, const int *pos, const double *inv_freq) {
+    if (!d || !vec || !pos || !inv_freq || rows <= 0 || heads <= 0 || head_dim <= 0 || head_dim % 2 || head_dim > 2048) return RD_ERR_ARG;
+    size_t n = (size_t)rows * heads * head_dim;
+    DevBuf V(d), Pp(d), F(d);
+    RC(V.alloc(sizeof(float) * n));
+    RC(Pp.alloc(sizeof(int) * (size_t)rows));
+    RC(F.alloc(sizeof(double) * (size_t)(head_dim / 2)));
+    RC(d->h2d(V.p, vec, sizeof(float) * n));
+    RC(d->h2d(Pp.p, pos, sizeof(int) * (size_t)rows));
+    RC(d->h2d(F.p, inv_freq, sizeof(double) * (size_t)(head_dim / 2)));
+    RC(d->launch(d->k.rope, (unsigned)heads, (unsigned)rows, 1, (unsigned)(head_dim / 2), V.as<float>(), (const int *)Pp.p, (const double *)F.p, heads,
+                 head_dim));
+    return d->d2h(vec, V.p, sizeof(float) * n);
+}
+
+extern "C" int rd_moe_route(rd_device *d, const float *logits, int T, int nE, int k, int norm, int *idx, float *wgt) {
+    if (!d || !logits || !idx || !wgt || T <= 0 || nE <= 0 || nE > 256 || k <= 0 || k > nE) {
+        rd_set_error("rd_moe_route: bad arguments (nE <= 256)");
+        return RD_ERR_ARG;
+    }
+    DevBuf L(d), I(d), W(d);
+    RC(L.alloc(sizeof(float) * (size_t)T * nE));
+    RC(I.alloc(sizeof(int) * (size_t)T * k));
+    RC(W.alloc(sizeof(float) * (size_t)T * k));
+    RC(d->h2d(L.p, logits, sizeof(float) * (size_t)T * nE));
+    RC(d->launch(d->k.moe_route, (unsigned)((T + 63) / 64), 1, 1, 64, (const float *)L.p, T, nE, k, norm, I.as<int>(), W.as<float>(),
+                 (signed char *)nullptr));
+    RC(d->d2h(idx, I.p, sizeof(int) * (size_t)T * k));
+    return d->d2h(wgt, W.p, sizeof(float) * (size_t)T * k);
+}

@@ -1,0 +1,261 @@
+// attn.h — paged f16 KV cache and ragged flash-decode attention (goinfer decoder/forwardn.go:295-500 semantics; the CUDA
+// analogue is backend/cuda/decode_fa.cu + kvpage.cuh). One query position per sequence, every sequence its own length.
+//
+// KV pool, per layer: [block][kv head] regions of 64 positions. Inside a region the elements are stored in the order the
+// MFMA operand fragments are read, so every wave load is one contiguous 1 KB read:
+//   K region: [key tile of 16 (4)][d step c (HD/32)][lane = dq*16 + key][8 halves],   d = dq*(HD/4) + c*8 + i
+//   V region: [key tile of 32 (2)][d column tile ct (HD/16)][lane = kq*16 + dcol][8 halves], key = kq*8 + i, d = ct*16 + dcol
+// Values are binary16 narrowed with round-half-up, as goinfer's f16 KV cache narrows them (decoder/kvcache.go:21-40).
+#pragma once
+#include "common.h"
+
+template <int HD> __device__ __forceinline__ int k_elem_index(int p, int d) {
+    int kt = p >> 4, key = p & 15, dq = d / (HD / 4), rem = d % (HD / 4), c = rem >> 3, i = rem & 7;
+    return (((kt * (HD / 32) + c) * 64 + dq * 16 + key) << 3) + i;
+}
+template <int HD> __device__ __forceinline__ int v_elem_index(int p, int d) {
+    int kt = p >> 5, pk = p & 31, kq = pk >> 3, i = pk & 7, ct = d >> 4, dcol = d & 15;
+    return (((kt * (HD / 16) + ct) * 64 + kq * 16 + dcol) << 3) + i;
+}
+
+__device__ __forceinline__ void kv_store_elem(uint16_t *__restrict__ Kp, uint16_t *__restrict__ Vp, int HD, size_t region, int p, int d, float kv,
+                                              float vv) {
+    int ki = HD == 128 ? k_elem_index<128>(p, d) : k_elem_index<64>(p, d);
+    int vi = HD == 128 ? v_elem_index<128>(p, d) : v_elem_index<64>(p, d);
+    Kp[region + ki] = f32_to_f16_half_up(kv);
+    Vp[region + vi] = f32_to_f16_half_up(vv);
+}
+
+// Host-provided rows (UploadKV, decoder/resident/forward.go:20-26): k,v f32 [n][nKV*HD] -> positions base..base+n-1 of one sequence.
+// Grid (n), block nKV*HD threads (<= 1024).
+extern "C" __global__ void rd_k_kv_store(const float *__restrict__ k, const float *__restrict__ v, uint16_t *__restrict__ Kp,
+                                         uint16_t *__restrict__ Vp, const int *__restrict__ table, int base, int nKV, int HD) {
+    int i = blockIdx.x, t = threadIdx.x;
+    if (t >= nKV * HD) return;
+    int pos = base + i, blk = table[pos >> 6], p = pos & 63, kvh = t / HD, d = t % HD;
+    size_t region = ((size_t)blk * nKV + kvh) * 64 * HD;
+    kv_store_elem(Kp, Vp, HD, region, p, d, k[(size_t)i * nKV * HD + t], v[(size_t)i * nKV * HD + t]);
+}
+
+// After the q|k|v GEMM: reduce its split-K partials, optional per-head RMSNorm of q and k (Qwen3, decoder/program_cpu.go:351-364),
+// NeoX RoPE with f64 angles (decoder/rope.go:28-64), q -> f32 buffer, k,v -> this position of the row's sequence in the pool.
+// Grid (nH + 2*nKV, rows), block HD/2 threads... one thread per rotation pair.  P: [splits][32][(nH+2nKV)*HD].
+extern "C" __global__ void rd_k_qkv_rope_store(const float *__restrict__ P, int splits, float *__restrict__ q, uint16_t *__restrict__ Kp,
+                                               uint16_t *__restrict__ Vp, const int *__restrict__ tables, int tabStride,
+                                               const int *__restrict__ rowSlot, const int *__restrict__ rowPos, const double *__restrict__ invFreq,
+                                               const float *__restrict__ qnorm, const float *__restrict__ knorm, float eps, int nH, int nKV, int HD) {
+    int head = blockIdx.x, m = blockIdx.y, t = threadIdx.x, half = HD / 2; // one wave: half <= 64
+    int Ntot = (nH + 2 * nKV) * HD, pos = rowPos[m];
+    const float *src = P + (size_t)m * Ntot + (size_t)head * HD;
+    float x1 = src[t], x2 = src[t + half];
+    for (int s = 1; s < splits; s++) {
+        x1 = __fadd_rn(x1, src[(size_t)s * 32 * Ntot + t]);
+        x2 = __fadd_rn(x2, src[(size_t)s * 32 * Ntot + t + half]);
+    }
+    bool isQ = head < nH, isK = !isQ && head < nH + nKV;
+    const float *nw = isQ ? qnorm : (isK ? knorm : nullptr);
+    if (nw) { // RMSNorm over the head's HD values, f64 sum of squares
+        double ss = (double)x1 * x1 + (double)x2 * x2;
+        for (int o = half >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+        float inv = (float)(1.0 / sqrt(ss / (double)HD + (double)eps));
+        x1 = __fmul_rn(__fmul_rn(x1, inv), nw[t]);
+        x2 = __fmul_rn(__fmul_rn(x2, inv), nw[t + half]);
+    }
+    float o1 = x1, o2 = x2;
+    if (isQ || isK) {
+        double theta = (double)pos * invFreq[t];
+        double c = cos(theta), s = sin(theta);
+        o1 = (float)((double)x1 * c - (double)x2 * s);
+        o2 = (float)((double)x2 * c + (double)x1 * s);
+    }
+    if (isQ) {
+        float *dst = q + (size_t)m * nH * HD + (size_t)head * HD;
+        dst[t] = o1;
+        dst[t + half] = o2;
+        return;
+    }
+    int kvh = isK ? head - nH : head - nH - nKV;
+    int blk = tables[(size_t)rowSlot[m] * tabStride + (pos >> 6)], p = pos & 63;
+    size_t region = ((size_t)blk * nKV + kvh) * 64 * HD;
+    uint16_t *dstp = isK ? Kp : Vp;
+    for (int e = 0; e < 2; e++) {
+        int d = e ? t + half : t;
+        int idx = isK ? (HD == 128 ? k_elem_index<128>(p, d) : k_elem_index<64>(p, d)) : (HD == 128 ? v_elem_index<128>(p, d) : v_elem_index<64>(p, d));
+        dstp[region + idx] = f32_to_f16_half_up(e ? o2 : o1);
+    }
+}
+
+typedef float float4v __attribute__((ext_vector_type(4)));
+
+struct AttnItem {
+    int row, kvh, b0, b1; // sequence row, kv head, block range [b0,b1) of that sequence
+};
+
+// One wave per item: online-softmax attention of the G query heads of one kv head over blocks [b0,b1) of one sequence.
+// Scores: S = Q.K^T on 16x16x32 f16 MFMA with Q split into hi+lo halves (K is exactly f16), so dots carry f32 accuracy.
+// P.V likewise with P split hi+lo. Writes unnormalised (O, m, l) per head: part[item][G][HD+2].
+template <int HD>
+__device__ __forceinline__ void attn_partial_body(const AttnItem *__restrict__ items, const int *__restrict__ rowLen, const int *__restrict__ rowSlot,
+                                                  const int *__restrict__ tables, int tabStride, const uint16_t *__restrict__ Kp,
+                                                  const uint16_t *__restrict__ Vp, const float *__restrict__ q, float *__restrict__ part, int nH,
+                                                  int nKV, float scale, float softcap, half_t *pbuf) {
+    constexpr int NC = HD / 32, NCT = HD / 16;
+    const AttnItem it = items[blockIdx.x];
+    const int lane = threadIdx.x, l16 = lane & 15, lg = lane >> 4;
+    const int G = nH / nKV, len = rowLen[it.row];
+    const int *tab = tables + (size_t)rowSlot[it.row] * tabStride;
+
+    // Q fragments (A operand): lane (head row l16, d quarter lg)
+    half8_t qhi[NC], qlo[NC];
+#pragma unroll
+    for (int c = 0; c < NC; c++) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            float v = 0.f;
+            if (l16 < G) v = q[(size_t)it.row * nH * HD + (size_t)(it.kvh * G + l16) * HD + lg * (HD / 4) + c * 8 + i];
+            half_t hi = (half_t)v;
+            qhi[c][i] = hi;
+            qlo[c][i] = (half_t)(v - (float)hi);
+        }
+    }
+    float4v O[NCT];
+#pragma unroll
+    for (int ct = 0; ct < NCT; ct++) O[ct] = (float4v){0.f, 0.f, 0.f, 0.f};
+    float mrun[4], lrun[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) mrun[r] = -INFINITY, lrun[r] = 0.f;
+
+    const size_t regionHalves = (size_t)64 * HD;
+    for (int b = it.b0; b < it.b1; b++) {
+        const int blk = tab[b];
+        const uint4_t *Kr = (const uint4_t *)(Kp + ((size_t)blk * nKV + it.kvh) * regionHalves);
+        const uint4_t *Vr = (const uint4_t *)(Vp + ((size_t)blk * nKV + it.kvh) * regionHalves);
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            const int key0 = b * 64 + u * 32;
+            if (key0 >= len) break;
+            uint4_t kf[2][NC], vf[NCT];
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int c = 0; c < NC; c++) kf[t][c] = __builtin_nontemporal_load(Kr + ((u * 2 + t) * NC + c) * 64 + lane);
+#pragma unroll
+            for (int ct = 0; ct < NCT; ct++) vf[ct] = __builtin_nontemporal_load(Vr + (u * NCT + ct) * 64 + lane);
+            float4v S[2];
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                S[t] = (float4v){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int c = 0; c < NC; c++) {
+                    half8_t kb;
+                    __builtin_memcpy(&kb, &kf[t][c], 16);
+                    S[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(qhi[c], kb, S[t], 0, 0, 0);
+                    S[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(qlo[c], kb, S[t], 0, 0, 0);
+                }
+            }
+            // lane (key l16 of tile t, head rows 4*lg+r)
+            float mx[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                mx[r] = -INFINITY;
+#pragma unroll
+                for (int t = 0; t < 2; t++) {
+                    float s = S[t][r] * scale;
+                    if (softcap != 0.f) s = softcap * tanhf(s / softcap);
+                    if (key0 + t * 16 + l16 >= len) s = -INFINITY;
+                    S[t][r] = s;
+                    mx[r] = fmaxf(mx[r], s);
+                }
+                for (int o = 8; o > 0; o >>= 1) mx[r] = fmaxf(mx[r], __shfl_xor(mx[r], o, 64));
+            }
+            float alpha[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                float mn = fmaxf(mrun[r], mx[r]);
+                alpha[r] = __expf(mrun[r] - mn); // first unit: exp(-inf) = 0
+                mrun[r] = mn;
+                float ps = 0.f;
+#pragma unroll
+                for (int t = 0; t < 2; t++) {
+                    float p = __expf(S[t][r] - mn);
+                    ps += p;
+                    half_t hi = (half_t)p;
+                    int idx = (4 * lg + r) * 32 + t * 16 + l16;
+                    pbuf[idx] = hi;
+                    pbuf[512 + idx] = (half_t)(p - (float)hi);
+                }
+                lrun[r] = lrun[r] * alpha[r] + ps;
+            }
+#pragma unroll
+            for (int ct = 0; ct < NCT; ct++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) O[ct][r] *= alpha[r];
+            __syncthreads();
+            half8_t phi, plo;
+            {
+                uint4_t a = *(const uint4_t *)(pbuf + l16 * 32 + lg * 8), bq = *(const uint4_t *)(pbuf + 512 + l16 * 32 + lg * 8);
+                __builtin_memcpy(&phi, &a, 16);
+                __builtin_memcpy(&plo, &bq, 16);
+            }
+            __syncthreads();
+#pragma unroll
+            for (int ct = 0; ct < NCT; ct++) {
+                half8_t vb;
+                __builtin_memcpy(&vb, &vf[ct], 16);
+                O[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(phi, vb, O[ct], 0, 0, 0);
+                O[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(plo, vb, O[ct], 0, 0, 0);
+            }
+        }
+    }
+    // lane (d column l16 of tile ct, head rows 4*lg+r): O[ct][r]; l partial sums live per key lane -> reduce over the 16 lanes
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        for (int o = 8; o > 0; o >>= 1) lrun[r] += __shfl_xor(lrun[r], o, 64);
+        int g = 4 * lg + r;
+        if (g < G) {
+            float *dst = part + ((size_t)blockIdx.x * G + g) * (HD + 2);
+#pragma unroll
+            for (int ct = 0; ct < NCT; ct++) dst[ct * 16 + l16] = O[ct][r];
+            if (l16 == 0) {
+                dst[HD] = mrun[r];
+                dst[HD + 1] = lrun[r];
+            }
+        }
+    }
+}
+
+extern "C" __global__ __launch_bounds__(64) void rd_k_attn_partial(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
+                                                                   const int *__restrict__ rowSlot, const int *__restrict__ tables, int tabStride,
+                                                                   const uint16_t *__restrict__ Kp, const uint16_t *__restrict__ Vp,
+                                                                   const float *__restrict__ q, float *__restrict__ part, int nH, int nKV, int HD,
+                                                                   float scale, float softcap) {
+    __shared__ half_t pbuf[1024];
+    if (HD == 128)
+        attn_partial_body<128>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, q, part, nH, nKV, scale, softcap, pbuf);
+    else
+        attn_partial_body<64>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, q, part, nH, nKV, scale, softcap, pbuf);
+}
+
+// Merge the partials of one (row, query head) in ascending item order (deterministic): out = sum O_i e^(m_i-M) / sum l_i e^(m_i-M).
+// itemStart[row*nKV+kvh] .. itemStart[row*nKV+kvh+1] are that pair's items. Grid (nH, rows), block HD threads.
+__device__ __forceinline__ float attn_combine_value(const float *__restrict__ part, const int *__restrict__ itemStart, int nH, int nKV, int HD,
+                                                    int m, int head, int d) {
+    int G = nH / nKV, kvh = head / G, g = head % G;
+    int i0 = itemStart[m * nKV + kvh], i1 = itemStart[m * nKV + kvh + 1];
+    float M = -INFINITY;
+    for (int i = i0; i < i1; i++) M = fmaxf(M, part[((size_t)i * G + g) * (HD + 2) + HD]);
+    float num = 0.f, den = 0.f;
+    for (int i = i0; i < i1; i++) {
+        const float *p = part + ((size_t)i * G + g) * (HD + 2);
+        float w = __expf(p[HD] - M);
+        num = fmaf(p[d], w, num);
+        den = fmaf(p[HD + 1], w, den);
+    }
+    return num / den;
+}
+
+extern "C" __global__ void rd_k_attn_combine(const float *__restrict__ part, const int *__restrict__ itemStart, float *__restrict__ out, int nH,
+                                             int nKV, int HD) {
+    int head = blockIdx.x, m = blockIdx.y, d = threadIdx.x;
+    out[(size_t)m * nH * HD + (size_t)head * HD + d] = attn_combine_value(part, itemStart, nH, nKV, HD, m, head, d);
+}

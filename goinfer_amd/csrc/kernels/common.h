@@ -1,0 +1,107 @@
+// common.h — shared device helpers for the gfx950 decode kernels (wave64, CDNA4).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
+
+#define RD_WAVE 64
+
+// One activation "panel": the f16 operand of one K-block for all 32 batch rows, laid out exactly as the MFMA
+// A-operand fragments are read: [step][lane = half*32 + row][8 halves].
+//   Q4_K panels cover 256 k (one super-block): 16 data steps + 1 step holding the 8 group sums (for the -dmin*m term).
+//   Plain panels (int8 / int4-g32 weights) cover 128 k: 8 data steps in natural k order.
+#define RD_Q4K_PANEL_STEPS 17
+#define RD_Q4K_PANEL_BYTES (RD_Q4K_PANEL_STEPS * 64 * 16)
+#define RD_LIN_PANEL_STEPS 8
+#define RD_LIN_PANEL_BYTES (RD_LIN_PANEL_STEPS * 64 * 16)
+#define RD_Q4K_TILE_BYTES 4608 // 32 rows x 144 B, re-tiled: 512 B of headers + 4 x 1024 B of codes
+
+__device__ __forceinline__ float wave_max32(float v) {
+    // max over each aligned group of 32 lanes
+    for (int o = 16; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+__device__ __forceinline__ int wave_sum32_i(int v) {
+    for (int o = 16; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_sum64(float v) {
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ double wave_sum64_d(double v) {
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// binary16 <- f32 with round-half-up on the dropped bits: goinfer's KV narrowing (internal/runtime/f16/f16.go:14-43).
+__device__ __forceinline__ uint16_t f32_to_f16_half_up(float f) {
+    uint32_t b = __float_as_uint(f);
+    uint16_t sign = (uint16_t)((b >> 16) & 0x8000);
+    int32_t e = (int32_t)((b >> 23) & 0xFF) - 112;
+    uint32_t m = b & 0x7FFFFF;
+    if (((b >> 23) & 0xFF) == 0xFF) return m ? (sign | 0x7E00) : (sign | 0x7C00);
+    if (e >= 0x1F) return sign | 0x7C00;
+    if (e <= 0) {
+        if (e < -10) return sign;
+        m |= 0x800000;
+        uint32_t sh = (uint32_t)(14 - e);
+        return sign | (uint16_t)((m + (1u << (sh - 1))) >> sh);
+    }
+    uint16_t half = sign | (uint16_t)(e << 10) | (uint16_t)(m >> 13);
+    if (m & 0x1000) half++;
+    return half;
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
+    half_t x;
+    __builtin_memcpy(&x, &h, 2);
+    return (float)x;
+}
+__device__ __forceinline__ uint16_t f16_to_bits(half_t x) {
+    uint16_t h;
+    __builtin_memcpy(&h, &x, 2);
+    return h;
+}
+
+// Per-32 activation quantization of one element (goinfer: aikit QuantizeActQ group 32; backend/cuda/actgroup.cu:32-54,
+// with the CPU path's round-half-away): the 32 lanes of an aligned half-wave hold one group.
+// Returns the dequantized value code*scale; *gsum = scale * sum(codes) (the same on every lane of the group).
+__device__ __forceinline__ float quant_g32(float v, float *gsum) {
+    float ma = wave_max32(fabsf(v));
+    float sc = ma / 127.f;
+    float inv = sc > 0.f ? 1.f / sc : 0.f;
+    float r = roundf(__fmul_rn(v, inv));
+    r = fminf(127.f, fmaxf(-127.f, r));
+    int code = (int)r;
+    int s = wave_sum32_i(code);
+    *gsum = __fmul_rn(sc, (float)s);
+    return __fmul_rn((float)code, sc);
+}
+
+// Where element t (0..255) of a super-block goes inside a Q4_K activation panel, for batch row m.
+// Sub-block j=t/32 belongs to nibble pair p=j/2; lane half h=p/2 owns pairs 2h,2h+1; its 16 code words are the
+// 16 MFMA steps. Word s holds bytes e0..e0+3 (e0=4*(s%8)): the unpack yields
+// [lo e0, lo e0+2, hi e0, hi e0+2, lo e0+1, lo e0+3, hi e0+1, hi e0+3] (lo = sub-block 2p, hi = 2p+1).
+__device__ __forceinline__ int q4k_panel_index(int t, int m) {
+    int j = t >> 5, e = t & 31, p = j >> 1, h = p >> 1, pp = p & 1;
+    int s = pp * 8 + (e >> 2), b = e & 3;
+    int slot = ((b & 1) << 2) + (b >> 1) + ((j & 1) << 1);
+    return ((s * 64 + h * 32 + m) << 3) + slot;
+}
+// Group sum of sub-block j for batch row m: step 16, lane half j/4, slot j%4.
+__device__ __forceinline__ int q4k_panel_sum_index(int j, int m) { return (((16 * 64) + (j >> 2) * 32 + m) << 3) + (j & 3); }
+// Plain panels: element t (0..127) of a 128-wide block, natural order: step t/16, half (t/8)&1, slot t%8.
+__device__ __forceinline__ int lin_panel_index(int t, int m) { return ((((t >> 4) * 64) + ((t >> 3) & 1) * 32 + m) << 3) + (t & 7); }
+// int4-g32 panels: as plain panels, but the 8 slots of a lane hold offsets [0,4,1,5,2,6,3,7] (the nibble unpack order).
+__device__ __forceinline__ int lin4_panel_index(int t, int m) {
+    int o = t & 7;
+    return ((((t >> 4) * 64) + ((t >> 3) & 1) * 32 + m) << 3) + (((o & 3) << 1) | (o >> 2));
+}

@@ -1,0 +1,113 @@
+// misc.h — small row-wise kernels: plain RMSNorm and RoPE (kernel-level entry points), argmax, the f32 matmul behind
+// Backend.MatmulBT / the MoE router, and MoE routing.
+#pragma once
+#include "common.h"
+
+// decoder/rmsnorm.go:29-92. One block (256 threads) per row; H <= 8192.
+extern "C" __global__ __launch_bounds__(256) void rd_k_rmsnorm(const float *__restrict__ x, const float *__restrict__ w, float *__restrict__ out,
+                                                               int H, float eps) {
+    __shared__ double red[4];
+    int m = blockIdx.x, t = threadIdx.x;
+    double ss = 0;
+    for (int k = t; k < H; k += 256) {
+        double v = x[(size_t)m * H + k];
+        ss += v * v;
+    }
+    ss = wave_sum64_d(ss);
+    if ((t & 63) == 0) red[t >> 6] = ss;
+    __syncthreads();
+    ss = (red[0] + red[1]) + (red[2] + red[3]);
+    float inv = (float)(1.0 / sqrt(ss / (double)H + (double)eps));
+    for (int k = t; k < H; k += 256) out[(size_t)m * H + k] = __fmul_rn(__fmul_rn(x[(size_t)m * H + k], inv), w[k]);
+}
+
+// decoder/rope.go:28-64 (NeoX rotate-half, f64 angle and rotation). Grid (heads, rows), block HD/2.
+extern "C" __global__ void rd_k_rope(float *__restrict__ vec, const int *__restrict__ pos, const double *__restrict__ invFreq, int heads, int HD) {
+    int h = blockIdx.x, m = blockIdx.y, t = threadIdx.x, half = HD / 2;
+    float *v = vec + ((size_t)m * heads + h) * HD;
+    double theta = (double)pos[m] * invFreq[t], c = cos(theta), s = sin(theta);
+    double x1 = v[t], x2 = v[t + half];
+    v[t] = (float)(x1 * c - x2 * s);
+    v[t + half] = (float)(x2 * c + x1 * s);
+}
+
+// internal/runtime/sampling/sampler.go:485-520: the first maximum wins. One block per row, rows read from split-K partials.
+extern "C" __global__ __launch_bounds__(256) void rd_k_argmax_rows(const float *__restrict__ P, int splits, int N, int *__restrict__ ids,
+                                                                   float *__restrict__ logits_out) {
+    __shared__ float bv[256];
+    __shared__ int bi[256];
+    int m = blockIdx.x, t = threadIdx.x;
+    float best = -INFINITY;
+    int idx = 0x7fffffff;
+    for (int n = t; n < N; n += 256) {
+        float a = P[(size_t)m * N + n];
+        for (int s = 1; s < splits; s++) a = __fadd_rn(a, P[((size_t)s * 32 + m) * N + n]);
+        if (logits_out) logits_out[(size_t)m * N + n] = a;
+        if (a > best || (a == best && n < idx)) best = a, idx = n;
+    }
+    bv[t] = best, bi[t] = idx;
+    __syncthreads();
+    for (int o = 128; o > 0; o >>= 1) {
+        if (t < o) {
+            float v2 = bv[t + o];
+            int i2 = bi[t + o];
+            if (v2 > bv[t] || (v2 == bv[t] && i2 < bi[t])) bv[t] = v2, bi[t] = i2;
+        }
+        __syncthreads();
+    }
+    if (t == 0 && ids) ids[m] = bi[0] == 0x7fffffff ? 0 : bi[0];
+}
+
+// dst[M][N] = a[M][K] . b[N][K]^T with an ascending-k f64 accumulator rounded once: Backend.MatmulBT (decoder/backend.go:26-30)
+// and the f32 MoE router (decoder/mlp.go:55). One thread per output; exact products, so the result is order-stable.
+extern "C" __global__ void rd_k_matmul_f32(const float *__restrict__ a, const float *__restrict__ b, float *__restrict__ dst, int M, int K, int N) {
+    int n = blockIdx.x * blockDim.x + threadIdx.x, m = blockIdx.y;
+    if (n >= N || m >= M) return;
+    const float *ar = a + (size_t)m * K, *br = b + (size_t)n * K;
+    double acc = 0;
+    for (int k = 0; k < K; k++) acc += (double)ar[k] * (double)br[k];
+    dst[(size_t)m * N + n] = (float)acc;
+}
+
+// decoder/mlp.go:130-184 routeExperts (softmax scoring, no bias, no group limit) + mlp.go:370-440 softmaxF32/topK:
+// f32 max; e = f32(exp(f64(x - max))); f64 sum; scores *= f32(1/sum); k passes of strict '>' (lowest index wins);
+// weights = chosen scores, optionally divided by their f32 sum in rank order. One thread per token (nE <= 256).
+// Also fills rankOf[token][expert] = rank or -1 for the expert-major grouped GEMMs.
+extern "C" __global__ void rd_k_moe_route(const float *__restrict__ logits, int T, int nE, int k, int norm, int *__restrict__ idx,
+                                          float *__restrict__ wgt, signed char *__restrict__ rankOf) {
+    int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= T) return;
+    const float *x = logits + (size_t)t * nE;
+    float sc[256];
+    float mx = x[0];
+    for (int i = 1; i < nE; i++)
+        if (x[i] > mx) mx = x[i];
+    double sum = 0;
+    for (int i = 0; i < nE; i++) {
+        double e = exp((double)__fsub_rn(x[i], mx));
+        sc[i] = (float)e;
+        sum += e;
+    }
+    float inv = (float)(1.0 / sum);
+    for (int i = 0; i < nE; i++) sc[i] = __fmul_rn(sc[i], inv);
+    if (rankOf)
+        for (int i = 0; i < nE; i++) rankOf[(size_t)t * nE + i] = -1;
+    unsigned long long used[4] = {0, 0, 0, 0};
+    float s = 0.f;
+    int n = 0;
+    for (int j = 0; j < k; j++) {
+        float best = -INFINITY;
+        int bi = -1;
+        for (int i = 0; i < nE; i++)
+            if (!((used[i >> 6] >> (i & 63)) & 1ull) && sc[i] > best) best = sc[i], bi = i;
+        if (bi < 0) break;
+        used[bi >> 6] |= 1ull << (bi & 63);
+        idx[(size_t)t * k + j] = bi;
+        wgt[(size_t)t * k + j] = best;
+        if (rankOf) rankOf[(size_t)t * nE + bi] = (signed char)j;
+        s = __fadd_rn(s, best);
+        n++;
+    }
+    if (norm && s > 0.f)
+        for (int j = 0; j < n; j++) wgt[(size_t)t * k + j] = wgt[(size_t)t * k + j] / s;
+}

@@ -1,0 +1,146 @@
+// q4k.h — Q4_K kernels: bit-exact dequantization, re-tiling for coalesced loads, and the dequant-GEMM on f16 MFMA.
+//
+// Format (goinfer decoder/gguf.go:1508-1537, backend/cuda/actgroup.cu:56-75): a super-block is 256 weights in 144 bytes:
+// d f16 @0, dmin f16 @2, 12 bytes of packed 6-bit scales/mins @4, 128 bytes of nibbles @16; w = d*sc_j*q - dmin*m_j.
+#pragma once
+#include "common.h"
+#include "gemm.h"
+
+__device__ __forceinline__ void q4k_scale_min(int j, const uint8_t *q, int *sc, int *m) {
+    if (j < 4) {
+        *sc = q[j] & 63;
+        *m = q[j + 4] & 63;
+    } else {
+        *sc = (q[j + 4] & 15) | ((q[j - 4] >> 6) << 4);
+        *m = (q[j + 4] >> 4) | ((q[j] >> 6) << 4);
+    }
+}
+
+// One thread per weight. Bit-exact: (d*sc) and (dmin*m) are rounded products, then (d*sc)*q and the subtraction are
+// rounded separately (no fused multiply-add), as the CPU reference computes them.
+extern "C" __global__ void rd_k_dequant_q4k(const uint8_t *__restrict__ blocks, float *__restrict__ out, long n_blocks) {
+    long b = blockIdx.x;
+    int t = threadIdx.x; // 0..255
+    if (b >= n_blocks) return;
+    const uint8_t *blk = blocks + b * 144;
+    int j = t >> 5, l = t & 31, sc, m;
+    q4k_scale_min(j, blk + 4, &sc, &m);
+    float d = f16_bits_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+    float dmin = f16_bits_to_f32((uint16_t)(blk[2] | (blk[3] << 8)));
+    int q = (blk[16 + (j >> 1) * 32 + l] >> (4 * (j & 1))) & 15;
+    float d1 = __fmul_rn(d, (float)sc), m1 = __fmul_rn(dmin, (float)m);
+    out[b * 256 + t] = __fsub_rn(__fmul_rn(d1, (float)q), m1);
+}
+
+// Re-tile raw row-major super-blocks [N][nSB][144] into [N/32][nSB][4608]: per (row tile, super-block) the 32 headers
+// (16 B each), then 4 planes of 64 lanes x 16 B: lane (row r, half h) plane c holds raw code bytes [h*64+c*16, +16) of row r.
+// Same bytes, same size; every wave load of the GEMM becomes one contiguous 512 B or 1024 B read.
+extern "C" __global__ void rd_k_retile_q4k(const uint8_t *__restrict__ raw, uint8_t *__restrict__ tiled, int N, int nSB) {
+    int tile = blockIdx.x, sb = blockIdx.y;
+    int t = threadIdx.x; // 0..287: 288 x 16 B = 4608 B
+    if (t >= 288) return;
+    uint8_t *dst = tiled + ((size_t)tile * nSB + sb) * RD_Q4K_TILE_BYTES;
+    const uint4_t *src;
+    if (t < 32) {
+        src = (const uint4_t *)(raw + ((size_t)(tile * 32 + t) * nSB + sb) * 144);
+    } else {
+        int u = t - 32, c = u >> 6, lane = u & 63, r = lane & 31, h = lane >> 5;
+        src = (const uint4_t *)(raw + ((size_t)(tile * 32 + r) * nSB + sb) * 144 + 16 + h * 64 + c * 16);
+    }
+    *(uint4_t *)(dst + (size_t)t * 16) = *src;
+}
+
+struct Q4KTile {
+    uint4_t hdr, q[4];
+};
+
+__device__ __forceinline__ void q4k_tile_load(Q4KTile &w, const uint8_t *__restrict__ p, int lane) {
+    w.hdr = __builtin_nontemporal_load((const uint4_t *)(p + (lane & 31) * 16));
+#pragma unroll
+    for (int c = 0; c < 4; c++) w.q[c] = __builtin_nontemporal_load((const uint4_t *)(p + 512 + c * 1024 + lane * 16));
+}
+
+// acc += panel(32 batch rows x 256 k) . tile(32 weight rows x 256 k)^T, f16 MFMA with f32 accumulation.
+// Weights are dequantized in registers: nibble -> f16 via the exponent trick (0x6400|q = 1024+q, 0x5400|(q<<4) = 64+q),
+// then one packed fma per pair yields the centred weight (q-8)*dsc rounded once. The per-sub-block constants
+// 8*dsc - dmin*m ride a 17th MFMA step against the per-group activation sums.
+__device__ __forceinline__ void q4k_tile_mma(float16_t &acc, const Q4KTile &w, const uint4_t *__restrict__ panel, int lane) {
+    const int h = lane >> 5;
+    uint32_t y = w.hdr.y, z = w.hdr.z, x = w.hdr.w;
+    half2_t dd;
+    uint32_t hx = w.hdr.x;
+    __builtin_memcpy(&dd, &hx, 4);
+    float d = (float)dd.x, dmin = (float)dd.y;
+    // Centred form: w = (q-8)*dsc + (8*dsc - dmin*m). The fma constant c = f16(-(1024+8)*dsc) is inexact; its exact
+    // remainder delta = c + 1032*dsc is a per-sub-block constant and moves into the offset term, so each weight is
+    // rounded exactly once: fma(1024+q, dsc, c) = f16((q-8)*dsc + delta).
+    half2_t DSC[4], C0[4];
+    half_t off[4];
+#pragma unroll
+    for (int jj = 0; jj < 4; jj++) {
+        int sc_lo = (y >> (8 * jj)) & 63, m_lo = (z >> (8 * jj)) & 63;
+        int sc_hi = ((x >> (8 * jj)) & 15) | (((y >> (8 * jj + 6)) & 3) << 4);
+        int m_hi = ((x >> (8 * jj + 4)) & 15) | (((z >> (8 * jj + 6)) & 3) << 4);
+        int sc = h ? sc_hi : sc_lo, m = h ? m_hi : m_lo;
+        float dsc32 = d * (float)sc;
+        half_t dsc = (half_t)dsc32;
+        float dscf = (float)dsc;
+        const float bias = (jj & 1) ? 72.f : 1032.f; // odd sub-blocks decode as 64+q, even ones as 1024+q
+        half_t c = (half_t)(-bias * dscf);
+        float delta = (float)c + bias * dscf;
+        DSC[jj] = (half2_t){dsc, dsc};
+        C0[jj] = (half2_t){c, c};
+        off[jj] = (half_t)(8.f * dsc32 - delta - dmin * (float)m); // exact scale here keeps the scale rounding centred
+    }
+#pragma unroll
+    for (int s = 0; s < 16; s++) {
+        uint32_t wd = w.q[s >> 2][s & 3];
+        const int pp = s >> 3;
+        uint32_t t8 = wd >> 8;
+        uint32_t u0 = (wd & 0x000F000Fu) | 0x64006400u, u1 = (wd & 0x00F000F0u) | 0x54005400u;
+        uint32_t u2 = (t8 & 0x000F000Fu) | 0x64006400u, u3 = (t8 & 0x00F000F0u) | 0x54005400u;
+        half2_t v0, v1, v2, v3;
+        __builtin_memcpy(&v0, &u0, 4);
+        __builtin_memcpy(&v1, &u1, 4);
+        __builtin_memcpy(&v2, &u2, 4);
+        __builtin_memcpy(&v3, &u3, 4);
+        v0 = __builtin_elementwise_fma(v0, DSC[2 * pp], C0[2 * pp]);
+        v1 = __builtin_elementwise_fma(v1, DSC[2 * pp + 1], C0[2 * pp + 1]);
+        v2 = __builtin_elementwise_fma(v2, DSC[2 * pp], C0[2 * pp]);
+        v3 = __builtin_elementwise_fma(v3, DSC[2 * pp + 1], C0[2 * pp + 1]);
+        half8_t b = {v0.x, v0.y, v1.x, v1.y, v2.x, v2.y, v3.x, v3.y};
+        half8_t a;
+        uint4_t av = panel[s * 64 + lane];
+        __builtin_memcpy(&a, &av, 16);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc, 0, 0, 0);
+    }
+    {
+        half8_t b = {off[0], off[1], off[2], off[3], (half_t)0, (half_t)0, (half_t)0, (half_t)0};
+        half8_t a;
+        uint4_t av = panel[16 * 64 + lane];
+        __builtin_memcpy(&a, &av, 16);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc, 0, 0, 0);
+    }
+}
+
+struct Q4KTraits {
+    typedef Q4KTile Tile;
+    static constexpr int TILE_BYTES = RD_Q4K_TILE_BYTES;
+    static constexpr int PANEL_VECS = RD_Q4K_PANEL_BYTES / 16;
+    static __device__ __forceinline__ void load(Tile &w, const uint8_t *__restrict__ p, int lane) { q4k_tile_load(w, p, lane); }
+    static __device__ __forceinline__ void mma(float16_t &acc, const Tile &w, const uint4_t *__restrict__ panel, int lane) {
+        q4k_tile_mma(acc, w, panel, lane);
+    }
+    static __device__ __forceinline__ void finish(float16_t &, const void *, int, int) {}
+};
+
+extern "C" __global__ __launch_bounds__(256) void rd_k_gemm_q4k_w4(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ Xp,
+                                                                    float *__restrict__ P, int N, int nSB, int sbPerSplit, int M) {
+    __shared__ uint4_t lds[2 * RD_Q4K_PANEL_BYTES / 16];
+    gemm_body<Q4KTraits, 4>(Wt, nullptr, Xp, P, N, nSB, sbPerSplit, M, lds);
+}
+extern "C" __global__ __launch_bounds__(128) void rd_k_gemm_q4k_w2(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ Xp,
+                                                                    float *__restrict__ P, int N, int nSB, int sbPerSplit, int M) {
+    __shared__ uint4_t lds[2 * RD_Q4K_PANEL_BYTES / 16];
+    gemm_body<Q4KTraits, 2>(Wt, nullptr, Xp, P, N, nSB, sbPerSplit, M, lds);
+}

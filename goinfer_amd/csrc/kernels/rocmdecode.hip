@@ -1,0 +1,18 @@
+// rocmdecode.hip — the single translation unit of the gfx950 code object (rocmdecode_gfx950.hsaco).
+// Every entry point is an extern "C" __global__ so the host side (or a Go purego binding) finds it by name with
+// hipModuleGetFunction.
+#include "common.h"
+#include "q4k.h"
+#include "lin.h"
+#include "act.h"
+#include "attn.h"
+#include "misc.h"
+
+// Attention combine fused with the per-32 quantization that feeds the o-projection. Grid (nH, rows), block HD threads.
+extern "C" __global__ void rd_k_attn_combine_quant(const float *__restrict__ part, const int *__restrict__ itemStart, uint8_t *__restrict__ Xp,
+                                                   int kind, int nH, int nKV, int HD) {
+    int head = blockIdx.x, m = blockIdx.y, d = threadIdx.x;
+    float v = attn_combine_value(part, itemStart, nH, nKV, HD, m, head, d);
+    float gs, xh = quant_g32(v, &gs);
+    panel_store(Xp, kind, m, head * HD + d, xh, gs);
+}

@@ -1,0 +1,138 @@
+/*
+ * rocmdecode.h — C ABI of librocmdecode.so: the MI355X (gfx950) decode backend that sits behind goinfer's
+ * backend seam. A Go `backend/rocm` module binds these entry points with purego (cgo-free, the way
+ * backend/cuda/internal/gpudev binds libcuda); the library itself loads libamdhip64 at run time with
+ * dlopen and its gfx950 code object with hipModuleLoadData.
+ *
+ * Conventions: every call returns RD_OK (0), RD_DECLINED (1: this backend does not take the request —
+ * goinfer's DeclineResident, decoder/residency.go:240-255) or a negative failure; rd_last_error() holds the
+ * reason. All calls on one model come from one thread (goinfer's resident executor, backend/cuda/resident.go:2135).
+ * Host pointers are caller-owned and only read/written during the call.
+ *
+ * Reference interfaces replaced (paths relative to the goinfer tree):
+ *   decoder/backend.go:23-32        Backend{Name, MatmulBT, Close}
+ *   decoder/residency.go:208-210    ResidencyBackend.BuildResident
+ *   decoder/resident/forward.go:5-38   Forward{Forward, ForwardN, UploadKV, TruncateTo, Reset, Close}
+ *   decoder/resident/subsystems.go:102-117  DecodeSubsystem{StepBatch, ForwardArgmax}
+ *   decoder/resident/subsystems.go:236-251  KVSubsystem{KVSlots, UseKVSlot}
+ */
+#ifndef ROCMDECODE_H
+#define ROCMDECODE_H
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RD_OK 0
+#define RD_DECLINED 1
+#define RD_ERR_ARG (-1)
+#define RD_ERR_HIP (-2)
+#define RD_ERR_STATE (-3)
+#define RD_ERR_KV_FULL (-4) /* goinfer's ErrKVPoolFull (decoder/mc3_batch.go:492-499): the step wrote nothing */
+
+typedef struct rd_device rd_device;
+typedef struct rd_model rd_model;
+
+/* projection ids for the upload calls */
+enum { RD_PROJ_Q = 0, RD_PROJ_K, RD_PROJ_V, RD_PROJ_O, RD_PROJ_GATE, RD_PROJ_UP, RD_PROJ_DOWN, RD_PROJ_HEAD, RD_PROJ_COUNT };
+/* f32 vectors */
+enum { RD_VEC_ATTN_NORM = 0, RD_VEC_FFN_NORM, RD_VEC_Q_NORM, RD_VEC_K_NORM, RD_VEC_FINAL_NORM, RD_VEC_ROUTER };
+/* rd_step_batch `want` */
+enum { RD_WANT_LOGITS = 1, RD_WANT_ARGMAX = 2 };
+
+/* What BuildResident reads through Model.BackendView() (decoder/backend_view.go:17-108). */
+typedef struct {
+    int32_t n_layers, hidden, n_heads, n_kv_heads, head_dim, inter, vocab;
+    float rms_eps;
+    float attn_scale;        /* AttnScale(): 1/sqrt(head_dim) or query_pre_attn_scalar^-0.5 */
+    float attn_softcap;      /* AttnLogitSoftcap(): 0 = off */
+    int32_t n_experts;       /* 0 = dense FFN */
+    int32_t top_k, norm_topk_prob, expert_inter;
+    int32_t qk_norm;         /* per-head RMSNorm of q and k (Qwen3) */
+    const double *rope_inv_freq; /* Layer(i).RopeInvFreq: head_dim/2 float64 entries */
+} rd_model_desc;
+
+/* ---- device: replaces backend/cuda/internal/gpudev/cuda.go:65-83 (Device open/close) ---- */
+int rd_device_open(int ordinal, rd_device **out);
+/* the same, from a code-object image the caller embeds (Go's go:embed of the .hsaco) */
+int rd_device_open_image(int ordinal, const void *hsaco, size_t len, rd_device **out);
+void rd_device_close(rd_device *d);
+const char *rd_last_error(void);
+/* "rocm": Backend.Name(), decoder/backend.go:24 */
+const char *rd_backend_name(void);
+int rd_device_sync(rd_device *d);
+/* free and total device memory in bytes: decoder.RegisterMemoryProbe, backend/cuda/backend.go:20-25 */
+int rd_device_mem_info(rd_device *d, size_t *free_b, size_t *total_b);
+
+/* ---- Backend.MatmulBT (decoder/backend.go:26-30): dst[M,N] = a[M,K] . b[N,K]^T, f32, host pointers ---- */
+int rd_matmul_bt(rd_device *d, const float *a, const float *b, float *dst, int M, int K, int N);
+
+/* ---- kernel-level entry points (the reference's kernel tests bind these: backend/cuda/kernels tests) ---- */
+/* Q4_K super-blocks (144 B per 256 weights, decoder/gguf.go:1508-1537) -> f32, bit-exact d*sc*q - dmin*m.
+ * blocks: host, N*K/256*144 bytes; out: host f32[N*K]. */
+int rd_dequant_q4k(rd_device *d, const void *blocks, int N, int K, float *out);
+/* dst[M,N] = a[M,K] . W^T with W raw Q4_K blocks and per-32 int8 activation quantization
+ * (decoder/weightmat.go:961-971; backend/cuda/actgroup.cu:298-355 gemv_q4k_g32). If W2 != NULL the call is the
+ * fused gate/up SwiGLU: dst = silu(a.W^T) * (a.W2^T) (decoder/cpu_gateup_fused.go:83-148). Host pointers. */
+int rd_gemm_q4k(rd_device *d, const void *W, int N, int K, const float *a, int M, float *dst, const void *W2);
+/* int8 per-row weights x per-32 int8 activations (backend/cuda/actgroup.cu:421-437 gemv_w8a8_g32). */
+int rd_gemm_w8a8(rd_device *d, const int8_t *q, const float *row_scale, int N, int K, const float *a, int M, float *dst);
+/* int4 group-32 weights with f16 scales x per-32 int8 activations (backend/cuda/actgroup.cu:243-275). */
+int rd_gemm_w4a8(rd_device *d, const uint8_t *nib, const uint16_t *s16, int N, int K, const float *a, int M, float *dst);
+/* Ragged flash-decode attention (backend/cuda/decode_fa.cu fa_partial_ragged/fa_combine_ragged;
+ * decoder/forwardn.go:295-500): n_seq sequences, sequence i has len[i] keys; k,v: host f32 [sum len][n_kv*hd]
+ * (rows of sequence i start at row off[i]); they are narrowed to binary16 (round-half-up) into a paged pool
+ * as the cache does. q: host f32 [n_seq][n_h*hd]; out: host f32 [n_seq][n_h*hd]. softcap 0 = off. */
+int rd_attn_ragged(rd_device *d, int n_seq, const int *len, const int64_t *off, const float *k, const float *v,
+                   const float *q, int n_h, int n_kv, int hd, float scale, float softcap, float *out);
+/* MoE routing (decoder/mlp.go:130-184 routeExperts, softmax scoring; backend/cuda/moe.cu:49-104 moe_route):
+ * logits host f32 [T][nE]; idx int32 [T][k], wgt f32 [T][k], rank order. */
+int rd_moe_route(rd_device *d, const float *logits, int T, int nE, int k, int norm, int *idx, float *wgt);
+/* RMSNorm rows (decoder/rmsnorm.go:29-92) and NeoX RoPE (decoder/rope.go:28-64), host pointers. */
+int rd_rmsnorm(rd_device *d, const float *x, const float *w, int rows, int dim, float eps, float *out);
+int rd_rope(rd_device *d, float *vec, int rows, int heads, int head_dim, const int *pos, const double *inv_freq);
+
+/* ---- resident model: replaces backend/cuda/backend.go:138-259 (BuildResident) ---- */
+int rd_model_create(rd_device *d, const rd_model_desc *desc, rd_model **out);
+void rd_model_destroy(rd_model *m);
+/* raw 144-byte super-blocks, N rows of K/256 blocks (Model.OpenKQuant, decoder/kquant_native.go:198-273) */
+int rd_model_upload_q4k(rd_model *m, int layer, int proj, const void *blocks, int N, int K);
+/* int8 rows + per-row f32 scale (WeightMat.Int8, decoder/weightmat.go:931) */
+int rd_model_upload_w8a8(rd_model *m, int layer, int proj, const int8_t *q, const float *row_scale, int N, int K);
+/* canonical int4 nibbles + binary16 group-32 scales (WeightMat.Int4F16, decoder/weightmat.go:904); expert < 0 = dense */
+int rd_model_upload_w4a8(rd_model *m, int layer, int proj, int expert, const uint8_t *nib, const uint16_t *s16, int N, int K);
+/* norms, router */
+int rd_model_upload_f32(rd_model *m, int layer, int which, const float *v, size_t n);
+/* after the last upload: checks every tensor the step needs is present */
+int rd_model_finalize(rd_model *m);
+
+/* ---- KV: resident/subsystems.go:236-251 (KVSlots), resident/forward.go:20-30 (UploadKV, TruncateTo, Reset) ---- */
+int rd_kv_configure(rd_model *m, int slots, int ctx_cap);
+/* keys, vals: host f32 [n][n_kv*hd] for positions base..base+n-1 of `slot`, layer `layer` (already RoPE'd) */
+int rd_kv_upload(rd_model *m, int slot, int layer, int base, int n, const float *keys, const float *vals);
+int rd_kv_truncate(rd_model *m, int slot, int pos);
+int rd_kv_reset(rd_model *m, int slot);
+
+/* ---- the step: resident/subsystems.go:102-117 StepBatch; every row equals its own rd_forward bit for bit ---- */
+/* emb: host f32 [B][hidden] (embedding rows, already scaled: decoder/residency.go:1077-1123);
+ * logits: host f32 [B][vocab] when want&RD_WANT_LOGITS; ids: int32 [B] when want&RD_WANT_ARGMAX (lowest index wins). */
+int rd_step_batch(rd_model *m, int B, const int *slot, const int *pos, const float *emb, int want, float *logits, int *ids);
+/* Forward(embedding, pos) on one slot: the B=1 step through the same kernels */
+int rd_forward(rd_model *m, int slot, int pos, const float *emb, float *logits);
+/* expert indices the last step routed to: int32 [B][n_layers][top_k] (MoE models only; parity checks) */
+int rd_last_moe_indices(rd_model *m, int *idx);
+
+/* ---- measurement: HIP-event timing of steps with inputs already resident in HBM ---- */
+/* Runs `steps` decode steps for the given (slot,pos0) batch after `warmup` untimed ones; each step advances every
+ * row's position by one and feeds back a fixed embedding (no host transfer inside the timed region).
+ * ms_out[steps]: per-step milliseconds from HIP events on the stream the kernels are launched on. */
+int rd_bench_steps(rd_model *m, int B, const int *slot, const int *pos0, const float *emb, int warmup, int steps, float *ms_out);
+/* Times `iters` launches of one kernel class over resident synthetic operands; see rocmdecode_bench.h names. */
+int rd_bench_kernel(rd_device *d, const char *name, const int64_t *args, int n_args, int warmup, int iters, float *ms_out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,127 @@
+"""GPU parity of the kernel-level entry points against the CPU oracle, through the C ABI.
+
+Bars: Q4_K dequantization bit-exact; GEMMs within rel 2e-3 of the oracle's integer-exact result measured against the
+row's own scale (f16 operand rounding, fp32 accumulate) and far inside the north-star logit bar (2e-2 abs / 1e-2 rel).
+"""
+import numpy as np
+import pytest
+
+from goinfer_amd import capi, synth
+from oracle import binding as ob
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    d = capi.Device(0)
+    yield d
+    d.close()
+
+
+def rel_err(got, want):
+    """max |got-want| over the rms of want: error relative to the typical output magnitude."""
+    want = want.astype(np.float64)
+    return float(np.abs(got.astype(np.float64) - want).max() / (np.sqrt((want * want).mean()) + 1e-30))
+
+
+@pytest.mark.parametrize("N,K", [(32, 256), (96, 768), (200, 3072)])
+def test_dequant_q4k_bit_exact(dev, N, K):
+    rng = np.random.default_rng(N * K)
+    raw = rng.integers(0, 256, N * (K // 256) * 144, dtype=np.uint8).reshape(-1, 144)
+    # finite f16 d and dmin (exponent 5..11), as the reference's fixtures set them
+    for off in (0, 2):
+        h = (rng.integers(5, 12, len(raw)).astype(np.uint16) << 10) | rng.integers(0, 1024, len(raw)).astype(np.uint16)
+        raw[:, off] = h & 0xFF
+        raw[:, off + 1] = h >> 8
+    raw[::5, 4:16] = 0xFF  # saturated scales and mins
+    want = ob.dequant_q4k(raw).reshape(N, K)
+    got = dev.dequant_q4k(raw, N, K)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_dequant_q4k_synth_bit_exact(dev):
+    blocks = synth.q4k_normal(7, 128, 1024)
+    want = ob.dequant_q4k(blocks).reshape(128, 1024)
+    assert np.array_equal(dev.dequant_q4k(blocks, 128, 1024).view(np.uint32), want.view(np.uint32))
+    assert abs(float(want.std()) - 0.02) < 2e-3
+
+
+@pytest.mark.parametrize("M", [1, 4, 5, 32, 33, 64])
+@pytest.mark.parametrize("N,K", [(128, 256), (160, 1024), (512, 4096)])
+def test_gemm_q4k(dev, M, N, K):
+    blocks = synth.q4k_normal(11 + N, N, K)
+    a = synth.normal(100 + M, M * K).reshape(M, K)
+    w = ob.WMat(ob.OR_Q4K, N, K, blocks, act_group=32)
+    want = ob.matmul(w, a)
+    ref64 = ob.matmul_f64ref(w, a)
+    got = dev.gemm_q4k(blocks, N, K, a)
+    assert rel_err(want, ref64) < 1e-5  # the oracle itself, against the f64 sum (the reference's own kernel bar)
+    assert rel_err(got, ref64) < 2e-3
+    # batch invariance: a row computed in a batch equals the same row alone, bit for bit
+    solo = dev.gemm_q4k(blocks, N, K, a[:1])
+    assert np.array_equal(solo[0].view(np.uint32), got[0].view(np.uint32))
+
+
+def test_gemm_q4k_fused_gate_up(dev):
+    N, K, M = 512, 1024, 9
+    g, u = synth.q4k_normal(1, N, K, 0.05), synth.q4k_normal(2, N, K, 0.05)
+    a = synth.normal(3, M * K).reshape(M, K)
+    gate = ob.matmul(ob.WMat(ob.OR_Q4K, N, K, g, act_group=32), a)
+    up = ob.matmul(ob.WMat(ob.OR_Q4K, N, K, u, act_group=32), a)
+    want = ob.swiglu(gate, up)
+    got = dev.gemm_q4k(g, N, K, a, blocks2=u)
+    assert rel_err(got, want) < 8e-3  # a product of two GEMM outputs: both factors carry the f16 operand rounding
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 64, 128), (7, 256, 896), (32, 1024, 4096)])
+def test_gemm_w8a8(dev, M, N, K):
+    q, s = synth.w8a8_normal(5, N, K)
+    a = synth.normal(6, M * K).reshape(M, K)
+    w = ob.WMat(ob.OR_W8A8, N, K, q, s, act_group=32)
+    ref64 = ob.matmul_f64ref(w, a)
+    assert rel_err(dev.gemm_w8a8(q, s, a), ref64) < 2e-3
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 64, 128), (16, 768, 2048), (16, 2048, 768)])
+def test_gemm_w4a8(dev, M, N, K):
+    nib, s16 = synth.w4a8_normal(8, N, K)
+    a = synth.normal(9, M * K).reshape(M, K)
+    w = ob.WMat(ob.OR_W4A8, N, K, nib, s16, act_group=32)
+    ref64 = ob.matmul_f64ref(w, a)
+    assert rel_err(dev.gemm_w4a8(nib, s16, K, a), ref64) < 2e-3
+
+
+def test_synth_quantizers_follow_reference_rules():
+    """The synthetic int8/int4 weights obey the reference's quantization rule bit for bit (oracle pinned by fingerprints)."""
+    N, K = 8, 256
+    w = synth.normal(5, N * K, 0.02).reshape(N, K)
+    q, s = synth.w8a8_normal(5, N, K)
+    q2, s2 = ob.quantize_rows_int8(w)
+    assert np.array_equal(q, q2) and np.array_equal(s, s2)
+    w = synth.normal(8, N * K, 0.02).reshape(N, K)
+    nib, s16 = synth.w4a8_normal(8, N, K)
+    n2, t2 = ob.quantize_int4(w)
+    assert np.array_equal(nib, n2) and np.array_equal(s16, t2)
+
+
+def test_rmsnorm_rope_route(dev):
+    x = synth.normal(1, 5 * 4096).reshape(5, 4096)
+    w = synth.normal(2, 4096, 0.02, 1.0)
+    got, want = dev.rmsnorm(x, w, 1e-5), ob.rmsnorm(x, w, 1e-5)
+    assert np.abs(got - want).max() <= 1e-6 * np.abs(want).max()
+    inv = 1.0 / (5e5 ** (np.arange(0, 128, 2) / 128.0))
+    v = synth.normal(3, 3 * 4 * 128).reshape(3, 4 * 128)
+    pos = [0, 17, 4095]
+    got = dev.rope(v, 4, 128, pos, inv)
+    assert np.array_equal(got[0], v[0])  # position 0 is the identity
+    for r in range(3):
+        want = ob.rope(v[r], 4, 128, pos[r], inv)
+        assert np.abs(got[r] - want).max() <= 2e-6
+    logits = synth.normal(4, 16 * 128).reshape(16, 128)
+    logits[3, 7] = logits[3, 90]  # an exact tie: the lower index must win
+    idx, wgt = dev.moe_route(logits, 8, True)
+    for t in range(16):
+        wi, ww = ob.route_experts(logits[t], 8, True)
+        assert np.array_equal(idx[t], wi)
+        assert np.array_equal(wgt[t].view(np.uint32), ww.view(np.uint32))
