@@ -1,1 +1,140 @@
-#include "device.h"
+// bench.cc — measurement entry points: HIP-event timing on the stream the kernels are launched on, with every input
+// already resident in HBM when the timed region starts.
+#include "model.h"
+#include <algorithm>
+#include <string.h>
+#include <string>
+
+#define RC(x)                \
+    do {                     \
+        int rc_ = (x);       \
+        if (rc_) return rc_; \
+    } while (0)
+
+extern "C" int rd_bench_steps(rd_model *m, int B, const int *slot, const int *pos0, const float *emb, int warmup, int steps, float *ms_out) {
+    if (!m || !slot || !pos0 || !emb || !ms_out || steps <= 0 || warmup < 0 || B < 1 || B > 32) return RD_ERR_ARG;
+    rd_device *d = m->d;
+    RC(d->h2d(m->emb_dev, emb, sizeof(float) * (size_t)B * m->desc.hidden));
+    RC(d->sync());
+    hipEvent_t e0, e1;
+    HIPCHK(EventCreate(&e0));
+    HIPCHK(EventCreate(&e1));
+    std::vector<int> pos((size_t)B);
+    int rc = RD_OK;
+    for (int i = 0; i < warmup + steps && !rc; i++) {
+        for (int b = 0; b < B; b++) pos[(size_t)b] = pos0[b] + i;
+        (void)d->hip->EventRecord(e0, d->stream);
+        rc = model_step(m, B, slot, pos.data(), nullptr, m->emb_dev, RD_WANT_ARGMAX, nullptr, nullptr);
+        (void)d->hip->EventRecord(e1, d->stream);
+        if (!rd_hip_ok(d->hip, d->hip->EventSynchronize(e1), "hipEventSynchronize")) rc = RD_ERR_HIP;
+        float ms = 0.f;
+        (void)d->hip->EventElapsedTime(&ms, e0, e1);
+        if (i >= warmup) ms_out[i - warmup] = ms;
+    }
+    (void)d->hip->EventDestroy(e0);
+    (void)d->hip->EventDestroy(e1);
+    return rc;
+}
+
+// One step with an event pair around every kernel class: class_ms[KC_COUNT] total milliseconds, class_n[KC_COUNT] launches.
+extern "C" int rd_bench_profile(rd_model *m, int B, const int *slot, const int *pos, const float *emb, float *class_ms, int *class_n) {
+    if (!m || !slot || !pos || !emb || !class_ms || !class_n) return RD_ERR_ARG;
+    rd_device *d = m->d;
+    RC(d->h2d(m->emb_dev, emb, sizeof(float) * (size_t)B * m->desc.hidden));
+    RC(d->sync());
+    m->timer.on = true;
+    int rc = model_step(m, B, slot, pos, nullptr, m->emb_dev, RD_WANT_ARGMAX, nullptr, nullptr);
+    m->timer.on = false;
+    int rc2 = d->sync();
+    memset(class_ms, 0, sizeof(float) * KC_COUNT);
+    memset(class_n, 0, sizeof(int) * KC_COUNT);
+    for (size_t i = 0; i < m->timer.cls.size(); i++) {
+        float ms = 0.f;
+        if (!rc && !rc2) (void)d->hip->EventElapsedTime(&ms, m->timer.ev[2 * i], m->timer.ev[2 * i + 1]);
+        class_ms[m->timer.cls[i]] += ms;
+        class_n[m->timer.cls[i]]++;
+    }
+    for (hipEvent_t e : m->timer.ev) (void)d->hip->EventDestroy(e);
+    m->timer.ev.clear(), m->timer.cls.clear();
+    return rc ? rc : rc2;
+}
+
+extern "C" int rd_bench_class_count(void) { return KC_COUNT; }
+extern "C" const char *rd_bench_class_name(int c) {
+    static const char *names[KC_COUNT] = {"gemm_qkv", "rope_kvstore", "attn_partial", "attn_combine", "gemm_o", "add_rmsnorm_quant", "gemm_gateup",
+                                          "swiglu_quant", "gemm_down", "gemm_head", "argmax", "moe_router", "moe_gemm", "moe_glue"};
+    return c >= 0 && c < KC_COUNT ? names[c] : "";
+}
+
+// Kernel micro-benchmarks over resident synthetic operands.
+//   "gemm_q4k"  args {N, K, M, copies}: dst = a . W^T on `copies` distinct weight copies used round-robin (so the 256 MB
+//               Infinity Cache cannot hold the weights between launches); operands are random bytes with sane f16 scales.
+//   "copy"      args {bytes}: device-to-device copy kernel-free baseline (hipMemcpyAsync), for calibrating counters.
+// ms_out[iters]: per-launch milliseconds (HIP events on the launch stream).
+extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *args, int n_args, int warmup, int iters, float *ms_out) {
+    if (!d || !name || !args || iters <= 0 || !ms_out) return RD_ERR_ARG;
+    std::string nm(name);
+    std::vector<hipEvent_t> ev((size_t)iters * 2);
+    for (auto &e : ev) HIPCHK(EventCreate(&e));
+    int rc = RD_OK;
+    if (nm == "gemm_q4k" && n_args >= 4) {
+        int N = (int)args[0], K = (int)args[1], M = (int)args[2], copies = (int)std::max<int64_t>(1, args[3]);
+        if (N % 32 || K % 256 || M < 1 || M > 32) {
+            rd_set_error("gemm_q4k bench: bad shape");
+            return RD_ERR_ARG;
+        }
+        size_t bytes = (size_t)N * (K / 256) * 144;
+        std::vector<uint8_t> raw(bytes);
+        uint64_t s = 88172645463325252ULL;
+        for (size_t i = 0; i < bytes; i++) {
+            s ^= s << 13, s ^= s >> 7, s ^= s << 17;
+            raw[i] = (uint8_t)s;
+        }
+        for (size_t b = 0; b < bytes / 144; b++) raw[b * 144 + 1] = 0x10 | (raw[b * 144 + 1] & 3), raw[b * 144 + 3] = 0x10 | (raw[b * 144 + 3] & 3);
+        std::vector<DevWeight> ws((size_t)copies);
+        for (auto &w : ws)
+            if (!rc) rc = upload_q4k(d, raw.data(), N, K, &w);
+        DevBuf Xp(d), P(d);
+        size_t pb = (size_t)(K / 256) * Q4K_PANEL_BYTES;
+        if (!rc) rc = Xp.alloc(pb);
+        int nKB = K / 256;
+        GemmPlan plan = plan_gemm(N, nKB);
+        if (!rc) rc = P.alloc(sizeof(float) * (size_t)plan.splits * 32 * N);
+        if (!rc) {
+            std::vector<uint16_t> x(pb / 2);
+            for (size_t i = 0; i < x.size(); i++) x[i] = (uint16_t)(0x3000 + (i * 2654435761u >> 22 & 0x3ff)) | (uint16_t)((i & 1) << 15);
+            rc = d->h2d(Xp.p, x.data(), pb);
+        }
+        if (!rc) rc = d->sync();
+        for (int i = 0; i < warmup + iters && !rc; i++) {
+            const DevWeight &w = ws[(size_t)i % ws.size()];
+            if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup)], d->stream);
+            rc = launch_gemm(d, w, Xp.p, P.as<float>(), M, nullptr);
+            if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup) + 1], d->stream);
+        }
+        if (!rc) rc = d->sync();
+        for (auto &w : ws) free_weight(d, &w);
+    } else if (nm == "copy" && n_args >= 1) {
+        size_t bytes = (size_t)args[0];
+        DevBuf A(d), Bf(d);
+        rc = A.alloc(bytes);
+        if (!rc) rc = Bf.alloc(bytes);
+        if (!rc) rc = rd_hip_ok(d->hip, d->hip->MemsetAsync(A.p, 1, bytes, d->stream), "memset") ? RD_OK : RD_ERR_HIP;
+        for (int i = 0; i < warmup + iters && !rc; i++) {
+            if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup)], d->stream);
+            rc = rd_hip_ok(d->hip, d->hip->MemcpyAsync(Bf.p, A.p, bytes, hipMemcpyDeviceToDevice, d->stream), "copy") ? RD_OK : RD_ERR_HIP;
+            if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup) + 1], d->stream);
+        }
+        if (!rc) rc = d->sync();
+    } else {
+        rd_set_error("rd_bench_kernel: unknown kernel '%s'", name);
+        rc = RD_ERR_ARG;
+    }
+    for (int i = 0; i < iters; i++) {
+        float ms = 0.f;
+        if (!rc) (void)d->hip->EventElapsedTime(&ms, ev[2 * (size_t)i], ev[2 * (size_t)i + 1]);
+        ms_out[i] = ms;
+    }
+    for (auto &e : ev) (void)d->hip->EventDestroy(e);
+    return rc;
+}

@@ -90,6 +90,9 @@ static const KName kNames[] = {
     {"rd_k_argmax_rows", &Kernels::argmax_rows},
     {"rd_k_matmul_f32", &Kernels::matmul_f32},
     {"rd_k_moe_route", &Kernels::moe_route},
+    {"rd_k_gemm_w4a8_moe", &Kernels::gemm_w4a8_moe},
+    {"rd_k_moe_swiglu_quant", &Kernels::moe_swiglu_quant},
+    {"rd_k_moe_fold", &Kernels::moe_fold},
 };
 
 static int open_common(int ordinal, const void *image, rd_device **out) {

@@ -1,3 +1,640 @@
-// model.cc — placeholder until the resident model lands (next commit).
-#include "device.h"
-extern "C" void rd_model_destroy(rd_model *) {}
+// model.cc — the resident model: BuildResident's uploads (backend/cuda/backend.go:138-259), the paged KV pool
+// (backend/cuda/kvpool.go) and the ragged batched decode step (backend/cuda/batchstep.go:49-78 StepBatch).
+#include "model.h"
+#include <algorithm>
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define RC(x)                \
+    do {                     \
+        int rc_ = (x);       \
+        if (rc_) return rc_; \
+    } while (0)
+
+static int alloc_f32(rd_device *d, float **p, size_t n) { return d->alloc((void **)p, sizeof(float) * (n ? n : 1)); }
+
+extern "C" int rd_model_create(rd_device *d, const rd_model_desc *desc, rd_model **out) {
+    if (!d || !desc || !out) return RD_ERR_ARG;
+    const rd_model_desc &c = *desc;
+    // Admission (goinfer's Admit gates, decoder/admit.go:36-48): what these kernels are built for.
+    if (c.n_layers <= 0 || c.hidden <= 0 || c.hidden % 128 || c.hidden > 8192 || c.n_heads <= 0 || c.n_kv_heads <= 0 ||
+        c.n_heads % c.n_kv_heads || (c.head_dim != 64 && c.head_dim != 128) || c.n_heads / c.n_kv_heads > 16 || c.vocab <= 0 || c.vocab % 32 ||
+        !c.rope_inv_freq) {
+        rd_set_error("rocm resident declines: needs hidden%%128==0 (<=8192), head_dim 64 or 128, GQA group <=16, vocab%%32==0");
+        return RD_DECLINED;
+    }
+    if (c.n_experts > 0 && (c.n_experts > 256 || c.top_k <= 0 || c.top_k > c.n_experts || c.expert_inter % 128)) {
+        rd_set_error("rocm resident declines: MoE needs <=256 experts and expert width %%128==0");
+        return RD_DECLINED;
+    }
+    if (c.n_experts == 0 && (c.inter <= 0 || c.inter % 128)) {
+        rd_set_error("rocm resident declines: FFN width must be a multiple of 128");
+        return RD_DECLINED;
+    }
+    rd_model *m = new rd_model();
+    m->d = d;
+    m->desc = c;
+    m->inv_freq.assign(c.rope_inv_freq, c.rope_inv_freq + c.head_dim / 2);
+    m->desc.rope_inv_freq = nullptr;
+    m->layers.resize((size_t)c.n_layers);
+    for (auto &l : m->layers)
+        if (c.n_experts > 0) l.exp_have.assign((size_t)c.n_experts * 3, 0);
+    int rc = d->alloc((void **)&m->inv_freq_dev, sizeof(double) * m->inv_freq.size());
+    if (!rc) rc = d->h2d(m->inv_freq_dev, m->inv_freq.data(), sizeof(double) * m->inv_freq.size());
+    if (!rc) rc = d->sync();
+    if (rc) {
+        delete m;
+        return rc;
+    }
+    *out = m;
+    return RD_OK;
+}
+
+extern "C" void rd_model_destroy(rd_model *m) {
+    if (!m) return;
+    rd_device *d = m->d;
+    (void)d->sync();
+    for (auto &l : m->layers) {
+        free_weight(d, &l.qkv), free_weight(d, &l.o), free_weight(d, &l.gateup), free_weight(d, &l.down);
+        for (void *p : {(void *)l.attn_norm, (void *)l.ffn_norm, (void *)l.q_norm, (void *)l.k_norm, (void *)l.router, l.exp_gateup, l.exp_down,
+                        (void *)l.Kp, (void *)l.Vp})
+            d->release(p);
+    }
+    free_weight(d, &m->head);
+    for (void *p : {(void *)m->inv_freq_dev, (void *)m->final_norm, (void *)m->tables, (void *)m->h, (void *)m->normed, (void *)m->P, (void *)m->qbuf,
+                    (void *)m->part, (void *)m->logits, (void *)m->emb_dev, m->XpA, m->XpB, (void *)m->ids, (void *)m->rowSlot, (void *)m->rowPos,
+                    (void *)m->rowLen, (void *)m->itemStart, (void *)m->items, (void *)m->router_logits, (void *)m->moe_wgt, (void *)m->moe_gu,
+                    (void *)m->moe_dn, (void *)m->moe_out, (void *)m->moe_idx, (void *)m->moe_idx_all, (void *)m->moe_rank, m->XpE})
+        d->release(p);
+    if (m->host_stage) (void)d->hip->HostFree(m->host_stage);
+    for (hipEvent_t e : m->timer.ev) (void)d->hip->EventDestroy(e);
+    delete m;
+}
+
+// ---------------------------------------------------------------- uploads
+static bool layer_ok(rd_model *m, int layer, bool allow_head) {
+    if (allow_head && layer < 0) return true;
+    if (layer < 0 || layer >= m->desc.n_layers) {
+        rd_set_error("layer %d out of range", layer);
+        return false;
+    }
+    return true;
+}
+
+static int expect_shape(rd_model *m, int proj, int N, int K) {
+    const rd_model_desc &c = m->desc;
+    int qd = c.n_heads * c.head_dim, kvd = c.n_kv_heads * c.head_dim;
+    int wantN = 0, wantK = 0;
+    switch (proj) {
+    case RD_PROJ_Q: wantN = qd, wantK = c.hidden; break;
+    case RD_PROJ_K:
+    case RD_PROJ_V: wantN = kvd, wantK = c.hidden; break;
+    case RD_PROJ_O: wantN = c.hidden, wantK = qd; break;
+    case RD_PROJ_GATE:
+    case RD_PROJ_UP: wantN = c.inter, wantK = c.hidden; break;
+    case RD_PROJ_DOWN: wantN = c.hidden, wantK = c.inter; break;
+    case RD_PROJ_HEAD: wantN = c.vocab, wantK = c.hidden; break;
+    default: rd_set_error("unknown projection %d", proj); return RD_ERR_ARG;
+    }
+    if (N != wantN || K != wantK) {
+        rd_set_error("projection %d: got %dx%d, model wants %dx%d", proj, N, K, wantN, wantK);
+        return RD_ERR_ARG;
+    }
+    return RD_OK;
+}
+
+static int upload_pending(rd_device *d, const PendingMat &p, DevWeight *w) {
+    if (p.kind == 0) return upload_q4k(d, p.data.data(), p.N, p.K, w);
+    if (p.kind == 1) return upload_w8a8(d, (const int8_t *)p.data.data(), (const float *)p.scales.data(), p.N, p.K, w);
+    return upload_w4a8(d, p.data.data(), (const uint16_t *)p.scales.data(), p.N, p.K, w);
+}
+
+// Concatenate row-wise (all kinds are row-major with per-row side data) and upload as one weight.
+static int fuse_and_upload(rd_device *d, PendingMat *parts, int n, DevWeight *w) {
+    PendingMat cat;
+    cat.kind = parts[0].kind, cat.K = parts[0].K, cat.N = 0;
+    for (int i = 0; i < n; i++) {
+        if (parts[i].kind != cat.kind || parts[i].K != cat.K) {
+            rd_set_error("rocm resident declines: fused projections differ in kind or K");
+            return RD_DECLINED;
+        }
+        cat.N += parts[i].N;
+        cat.data.insert(cat.data.end(), parts[i].data.begin(), parts[i].data.end());
+        cat.scales.insert(cat.scales.end(), parts[i].scales.begin(), parts[i].scales.end());
+    }
+    int rc = upload_pending(d, cat, w);
+    if (!rc)
+        for (int i = 0; i < n; i++) parts[i] = PendingMat(), parts[i].kind = -2; // consumed
+    return rc;
+}
+
+static int accept(rd_model *m, int layer, int proj, PendingMat &&pm) {
+    if (m->finalized) {
+        rd_set_error("model already finalized");
+        return RD_ERR_STATE;
+    }
+    rd_device *d = m->d;
+    if (proj == RD_PROJ_HEAD) {
+        free_weight(d, &m->head);
+        return upload_pending(d, pm, &m->head);
+    }
+    LayerW &l = m->layers[(size_t)layer];
+    if (proj == RD_PROJ_O) {
+        free_weight(d, &l.o);
+        return upload_pending(d, pm, &l.o);
+    }
+    if (proj == RD_PROJ_DOWN) {
+        free_weight(d, &l.down);
+        return upload_pending(d, pm, &l.down);
+    }
+    l.pend[proj] = std::move(pm);
+    if (proj <= RD_PROJ_V) {
+        if (l.pend[RD_PROJ_Q].kind >= 0 && l.pend[RD_PROJ_K].kind >= 0 && l.pend[RD_PROJ_V].kind >= 0) {
+            free_weight(d, &l.qkv);
+            return fuse_and_upload(d, &l.pend[RD_PROJ_Q], 3, &l.qkv);
+        }
+    } else if (l.pend[RD_PROJ_GATE].kind >= 0 && l.pend[RD_PROJ_UP].kind >= 0) {
+        free_weight(d, &l.gateup);
+        return fuse_and_upload(d, &l.pend[RD_PROJ_GATE], 2, &l.gateup);
+    }
+    return RD_OK;
+}
+
+extern "C" int rd_model_upload_q4k(rd_model *m, int layer, int proj, const void *blocks, int N, int K) {
+    if (!m || !blocks) return RD_ERR_ARG;
+    if (!layer_ok(m, layer, proj == RD_PROJ_HEAD)) return RD_ERR_ARG;
+    RC(expect_shape(m, proj, N, K));
+    if (K % 256) {
+        rd_set_error("Q4_K needs K%%256==0 (goinfer kquant_native.go:88-90), got K=%d", K);
+        return RD_DECLINED;
+    }
+    PendingMat pm;
+    pm.kind = 0, pm.N = N, pm.K = K;
+    pm.data.assign((const uint8_t *)blocks, (const uint8_t *)blocks + (size_t)N * (K / 256) * 144);
+    return accept(m, layer, proj, std::move(pm));
+}
+
+extern "C" int rd_model_upload_w8a8(rd_model *m, int layer, int proj, const int8_t *q, const float *row_scale, int N, int K) {
+    if (!m || !q || !row_scale) return RD_ERR_ARG;
+    if (!layer_ok(m, layer, proj == RD_PROJ_HEAD)) return RD_ERR_ARG;
+    RC(expect_shape(m, proj, N, K));
+    PendingMat pm;
+    pm.kind = 1, pm.N = N, pm.K = K;
+    pm.data.assign((const uint8_t *)q, (const uint8_t *)q + (size_t)N * K);
+    pm.scales.assign((const uint8_t *)row_scale, (const uint8_t *)row_scale + sizeof(float) * (size_t)N);
+    return accept(m, layer, proj, std::move(pm));
+}
+
+extern "C" int rd_model_upload_w4a8(rd_model *m, int layer, int proj, int expert, const uint8_t *nib, const uint16_t *s16, int N, int K) {
+    if (!m || !nib || !s16) return RD_ERR_ARG;
+    if (!layer_ok(m, layer, proj == RD_PROJ_HEAD && expert < 0)) return RD_ERR_ARG;
+    rd_device *d = m->d;
+    const rd_model_desc &c = m->desc;
+    if (expert < 0) {
+        RC(expect_shape(m, proj, N, K));
+        PendingMat pm;
+        pm.kind = 2, pm.N = N, pm.K = K;
+        pm.data.assign(nib, nib + (size_t)N * K / 2);
+        pm.scales.assign((const uint8_t *)s16, (const uint8_t *)s16 + 2 * (size_t)N * (K / 32));
+        return accept(m, layer, proj, std::move(pm));
+    }
+    // expert tensors: gate and up are stacked [gate; up] per expert (one GEMM), down is its own stack
+    if (c.n_experts <= 0 || expert >= c.n_experts || (proj != RD_PROJ_GATE && proj != RD_PROJ_UP && proj != RD_PROJ_DOWN)) {
+        rd_set_error("bad expert upload (expert %d, proj %d)", expert, proj);
+        return RD_ERR_ARG;
+    }
+    int I = c.expert_inter, H = c.hidden;
+    bool isDown = proj == RD_PROJ_DOWN;
+    if ((isDown && (N != H || K != I)) || (!isDown && (N != I || K != H))) {
+        rd_set_error("expert projection %d: got %dx%d", proj, N, K);
+        return RD_ERR_ARG;
+    }
+    LayerW &l = m->layers[(size_t)layer];
+    size_t guBytes = (size_t)(2 * I / 32) * (H / 128) * 2304, dnBytes = (size_t)(H / 32) * (I / 128) * 2304;
+    if (!l.exp_gateup) {
+        RC(d->alloc(&l.exp_gateup, guBytes * c.n_experts));
+        RC(d->alloc(&l.exp_down, dnBytes * c.n_experts));
+    }
+    DevWeight tmp;
+    RC(upload_w4a8(d, nib, s16, N, K, &tmp));
+    size_t tb = (size_t)(N / 32) * (K / 128) * 2304;
+    uint8_t *dst = isDown ? (uint8_t *)l.exp_down + dnBytes * expert
+                          : (uint8_t *)l.exp_gateup + guBytes * expert + (proj == RD_PROJ_UP ? guBytes / 2 : 0);
+    int rc = rd_hip_ok(d->hip, d->hip->MemcpyAsync(dst, tmp.tiled, tb, hipMemcpyDeviceToDevice, d->stream), "expert copy") ? RD_OK : RD_ERR_HIP;
+    if (!rc) rc = d->sync();
+    free_weight(d, &tmp);
+    if (!rc) l.exp_have[(size_t)expert * 3 + (proj == RD_PROJ_GATE ? 0 : proj == RD_PROJ_UP ? 1 : 2)] = 1;
+    return rc;
+}
+
+extern "C" int rd_model_upload_f32(rd_model *m, int layer, int which, const float *v, size_t n) {
+    if (!m || !v) return RD_ERR_ARG;
+    rd_device *d = m->d;
+    const rd_model_desc &c = m->desc;
+    float **slot = nullptr;
+    size_t want = 0;
+    if (which == RD_VEC_FINAL_NORM) {
+        slot = &m->final_norm, want = (size_t)c.hidden;
+    } else {
+        if (!layer_ok(m, layer, false)) return RD_ERR_ARG;
+        LayerW &l = m->layers[(size_t)layer];
+        switch (which) {
+        case RD_VEC_ATTN_NORM: slot = &l.attn_norm, want = (size_t)c.hidden; break;
+        case RD_VEC_FFN_NORM: slot = &l.ffn_norm, want = (size_t)c.hidden; break;
+        case RD_VEC_Q_NORM: slot = &l.q_norm, want = (size_t)c.head_dim; break;
+        case RD_VEC_K_NORM: slot = &l.k_norm, want = (size_t)c.head_dim; break;
+        case RD_VEC_ROUTER: slot = &l.router, want = (size_t)c.n_experts * c.hidden; break;
+        default: rd_set_error("unknown vector %d", which); return RD_ERR_ARG;
+        }
+    }
+    if (n != want) {
+        rd_set_error("vector %d: got %zu values, want %zu", which, n, want);
+        return RD_ERR_ARG;
+    }
+    if (!*slot) RC(alloc_f32(d, slot, n));
+    RC(d->h2d(*slot, v, sizeof(float) * n));
+    return d->sync();
+}
+
+static size_t gemm_partial_floats(const DevWeight &w) {
+    if (w.kind < 0) return 0;
+    int nKB = w.kind == 0 ? w.K / 256 : w.K / 128;
+    return (size_t)plan_gemm(w.N, nKB).splits * 32 * w.N;
+}
+
+extern "C" int rd_model_finalize(rd_model *m) {
+    if (!m) return RD_ERR_ARG;
+    rd_device *d = m->d;
+    const rd_model_desc &c = m->desc;
+    size_t pf = 0;
+    for (int i = 0; i < c.n_layers; i++) {
+        LayerW &l = m->layers[(size_t)i];
+        bool ok = l.qkv.kind >= 0 && l.o.kind >= 0 && l.attn_norm && l.ffn_norm && (!c.qk_norm || (l.q_norm && l.k_norm));
+        if (c.n_experts == 0)
+            ok = ok && l.gateup.kind >= 0 && l.down.kind >= 0;
+        else {
+            ok = ok && l.router && l.exp_gateup;
+            for (char hv : l.exp_have) ok = ok && hv;
+        }
+        if (!ok) {
+            rd_set_error("layer %d is missing tensors", i);
+            return RD_ERR_STATE;
+        }
+        pf = std::max({pf, gemm_partial_floats(l.qkv), gemm_partial_floats(l.o), gemm_partial_floats(l.gateup), gemm_partial_floats(l.down)});
+    }
+    if (m->head.kind < 0 || !m->final_norm) {
+        rd_set_error("model is missing the head or the final norm");
+        return RD_ERR_STATE;
+    }
+    pf = std::max(pf, gemm_partial_floats(m->head));
+    int H = c.hidden, qd = c.n_heads * c.head_dim;
+    m->P_floats = pf;
+    RC(alloc_f32(d, &m->P, pf));
+    RC(alloc_f32(d, &m->h, (size_t)32 * H));
+    RC(alloc_f32(d, &m->emb_dev, (size_t)32 * H));
+    RC(alloc_f32(d, &m->normed, (size_t)32 * H));
+    RC(alloc_f32(d, &m->qbuf, (size_t)32 * qd));
+    RC(alloc_f32(d, &m->logits, (size_t)32 * c.vocab));
+    size_t kA = (size_t)H, kB = (size_t)std::max(qd, c.n_experts ? qd : c.inter);
+    RC(d->alloc(&m->XpA, (kA / 128) * LIN_PANEL_BYTES + Q4K_PANEL_BYTES)); // >= either panel kind for K=hidden
+    RC(d->alloc(&m->XpB, (kB / 128) * LIN_PANEL_BYTES + Q4K_PANEL_BYTES));
+    RC(d->alloc((void **)&m->ids, sizeof(int) * 32));
+    RC(d->alloc((void **)&m->rowSlot, sizeof(int) * 32));
+    RC(d->alloc((void **)&m->rowPos, sizeof(int) * 32));
+    RC(d->alloc((void **)&m->rowLen, sizeof(int) * 32));
+    if (c.n_experts > 0) {
+        int k = c.top_k, I = c.expert_inter;
+        RC(alloc_f32(d, &m->router_logits, (size_t)32 * c.n_experts));
+        RC(alloc_f32(d, &m->moe_wgt, (size_t)32 * k));
+        RC(alloc_f32(d, &m->moe_gu, (size_t)32 * k * 2 * I));
+        RC(alloc_f32(d, &m->moe_dn, (size_t)32 * k * H));
+        RC(alloc_f32(d, &m->moe_out, (size_t)32 * H));
+        RC(d->alloc((void **)&m->moe_idx, sizeof(int) * 32 * k));
+        RC(d->alloc((void **)&m->moe_idx_all, sizeof(int) * (size_t)c.n_layers * 32 * k));
+        RC(d->alloc((void **)&m->moe_rank, (size_t)32 * c.n_experts));
+        RC(d->alloc(&m->XpE, (size_t)c.n_experts * (I / 128) * LIN_PANEL_BYTES));
+        HIPCHK(MemsetAsync(m->XpE, 0, (size_t)c.n_experts * (I / 128) * LIN_PANEL_BYTES, d->stream));
+    }
+    m->host_stage_bytes = sizeof(float) * (size_t)32 * H + (1u << 20);
+    HIPCHK(HostMalloc(&m->host_stage, m->host_stage_bytes, 0));
+    m->finalized = true;
+    return d->sync();
+}
+
+// ---------------------------------------------------------------- KV
+extern "C" int rd_kv_configure(rd_model *m, int slots, int ctx_cap) {
+    if (!m || slots <= 0 || ctx_cap <= 0) return RD_ERR_ARG;
+    if (m->tables) {
+        rd_set_error("KV already configured");
+        return RD_ERR_STATE;
+    }
+    rd_device *d = m->d;
+    const rd_model_desc &c = m->desc;
+    m->slots = slots, m->ctx_cap = ctx_cap, m->blocks_per_slot = (ctx_cap + 63) / 64;
+    size_t nBlocks = (size_t)slots * m->blocks_per_slot + 1; // block 0 is the all-zero block no slot owns
+    size_t bytes = nBlocks * c.n_kv_heads * 64 * c.head_dim * 2;
+    size_t fr = 0, tot = 0;
+    HIPCHK(MemGetInfo(&fr, &tot));
+    if (bytes * 2 * c.n_layers > fr) {
+        rd_set_error("rocm resident declines: KV pool of %zu MiB exceeds free device memory (%zu MiB)", (bytes * 2 * c.n_layers) >> 20, fr >> 20);
+        return RD_DECLINED;
+    }
+    for (auto &l : m->layers) {
+        RC(d->alloc((void **)&l.Kp, bytes));
+        RC(d->alloc((void **)&l.Vp, bytes));
+        HIPCHK(MemsetAsync(l.Kp, 0, bytes, d->stream));
+        HIPCHK(MemsetAsync(l.Vp, 0, bytes, d->stream));
+    }
+    // Static ownership: slot s owns blocks 1+s*bps .. ; the table indirection stays so a pool allocator can replace it.
+    std::vector<int> tab((size_t)slots * m->blocks_per_slot);
+    for (size_t i = 0; i < tab.size(); i++) tab[i] = (int)(i + 1);
+    RC(d->alloc((void **)&m->tables, sizeof(int) * tab.size()));
+    RC(d->h2d(m->tables, tab.data(), sizeof(int) * tab.size()));
+    m->slot_len.assign((size_t)slots, 0);
+    // attention work list: ~4096 items plus one per (row, kv head) of rounding
+    m->max_items = 4096 + 32 * c.n_kv_heads * 2;
+    int G = c.n_heads / c.n_kv_heads;
+    RC(alloc_f32(d, &m->part, (size_t)m->max_items * G * (c.head_dim + 2)));
+    RC(d->alloc((void **)&m->items, sizeof(AttnItemH) * (size_t)m->max_items));
+    RC(d->alloc((void **)&m->itemStart, sizeof(int) * (size_t)(32 * c.n_kv_heads + 1)));
+    return d->sync();
+}
+
+static bool slot_ok(rd_model *m, int slot) {
+    if (!m->tables || slot < 0 || slot >= m->slots) {
+        rd_set_error("KV slot %d out of range (configured %d)", slot, m->slots);
+        return false;
+    }
+    return true;
+}
+
+extern "C" int rd_kv_upload(rd_model *m, int slot, int layer, int base, int n, const float *keys, const float *vals) {
+    if (!m || !keys || !vals || n <= 0 || base < 0) return RD_ERR_ARG;
+    if (!slot_ok(m, slot) || !layer_ok(m, layer, false)) return RD_ERR_ARG;
+    if (base + n > m->ctx_cap) {
+        rd_set_error("rd_kv_upload: positions %d..%d exceed the context cap %d", base, base + n - 1, m->ctx_cap);
+        return RD_ERR_KV_FULL;
+    }
+    rd_device *d = m->d;
+    const rd_model_desc &c = m->desc;
+    int kvd = c.n_kv_heads * c.head_dim;
+    DevBuf K(d), V(d);
+    RC(K.alloc(sizeof(float) * (size_t)n * kvd));
+    RC(V.alloc(sizeof(float) * (size_t)n * kvd));
+    RC(d->h2d(K.p, keys, sizeof(float) * (size_t)n * kvd));
+    RC(d->h2d(V.p, vals, sizeof(float) * (size_t)n * kvd));
+    LayerW &l = m->layers[(size_t)layer];
+    RC(d->launch(d->k.kv_store, (unsigned)n, 1, 1, (unsigned)kvd, (const float *)K.p, (const float *)V.p, l.Kp, l.Vp,
+                 (const int *)(m->tables + (size_t)slot * m->blocks_per_slot), base, c.n_kv_heads, c.head_dim));
+    RC(d->sync());
+    m->slot_len[(size_t)slot] = std::max(m->slot_len[(size_t)slot], base + n);
+    return RD_OK;
+}
+
+extern "C" int rd_kv_truncate(rd_model *m, int slot, int pos) {
+    if (!m || !slot_ok(m, slot) || pos < 0) return RD_ERR_ARG;
+    m->slot_len[(size_t)slot] = std::min(m->slot_len[(size_t)slot], pos);
+    return RD_OK;
+}
+
+extern "C" int rd_kv_reset(rd_model *m, int slot) { return rd_kv_truncate(m, slot, 0); }
+
+// ---------------------------------------------------------------- the step
+struct Scope { // times one kernel class when the model's timer is on
+    rd_model *m;
+    int cls;
+    Scope(rd_model *mm, int c) : m(mm), cls(c) {
+        if (!m->timer.on) return;
+        hipEvent_t a, b;
+        (void)m->d->hip->EventCreate(&a), (void)m->d->hip->EventCreate(&b);
+        m->timer.ev.push_back(a), m->timer.ev.push_back(b), m->timer.cls.push_back(cls);
+        (void)m->d->hip->EventRecord(a, m->d->stream);
+    }
+    ~Scope() {
+        if (m->timer.on) (void)m->d->hip->EventRecord(m->timer.ev.back(), m->d->stream);
+    }
+};
+
+static int build_attn_items(rd_model *m, int B, const int *pos, std::vector<AttnItemH> &items, std::vector<int> &start) {
+    const rd_model_desc &c = m->desc;
+    long total = 0;
+    for (int b = 0; b < B; b++) total += (long)((pos[b] + 1 + 63) / 64) * c.n_kv_heads;
+    int chunk = (int)std::max(1L, (total + 4095) / 4096);
+    if (const char *e = getenv("ROCMDECODE_ATTN_CHUNK")) chunk = std::max(1, atoi(e));
+    items.clear();
+    start.assign((size_t)B * c.n_kv_heads + 1, 0);
+    for (int b = 0; b < B; b++) {
+        int nb = (pos[b] + 1 + 63) / 64;
+        for (int h = 0; h < c.n_kv_heads; h++) {
+            start[(size_t)b * c.n_kv_heads + h] = (int)items.size();
+            for (int b0 = 0; b0 < nb; b0 += chunk) items.push_back({b, h, b0, std::min(nb, b0 + chunk)});
+        }
+    }
+    start[(size_t)B * c.n_kv_heads] = (int)items.size();
+    if ((int)items.size() > m->max_items) {
+        rd_set_error("attention work list overflow (%zu items)", items.size());
+        return RD_ERR_STATE;
+    }
+    return RD_OK;
+}
+
+static int add_norm_quant(rd_model *m, int B, const float *P, int splits, const float *w, const DevWeight &next, void *Xp, float *norm_out) {
+    rd_device *d = m->d;
+    Scope s(m, KC_ADD_NORM);
+    return d->launch(d->k.add_rmsnorm_quant, (unsigned)B, 1, 1, 256, m->h, P, splits, w, m->desc.rms_eps, m->desc.hidden, Xp, panel_kind_for(next),
+                     norm_out);
+}
+
+static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
+    rd_device *d = m->d;
+    const rd_model_desc &c = m->desc;
+    int H = c.hidden, I = c.expert_inter, k = c.top_k, nE = c.n_experts;
+    {
+        Scope s(m, KC_MOE_ROUTER);
+        RC(d->launch(d->k.matmul_f32, (unsigned)((nE + 63) / 64), (unsigned)B, 1, 64, (const float *)m->normed, (const float *)l.router,
+                     m->router_logits, B, H, nE));
+        RC(d->launch(d->k.moe_route, 1, 1, 1, 64, (const float *)m->router_logits, B, nE, k, c.norm_topk_prob, m->moe_idx, m->moe_wgt,
+                     m->moe_rank));
+        HIPCHK(MemcpyAsync(m->moe_idx_all + (size_t)layer * 32 * k, m->moe_idx, sizeof(int) * (size_t)B * k, hipMemcpyDeviceToDevice, d->stream));
+    }
+    size_t guStride = (size_t)(2 * I / 32) * (H / 128) * 2304, dnStride = (size_t)(H / 32) * (I / 128) * 2304;
+    size_t xpStride = (size_t)(I / 128) * LIN_PANEL_BYTES;
+    {
+        Scope s(m, KC_MOE_GEMM);
+        RC(d->launch(d->k.gemm_w4a8_moe, (unsigned)((2 * I + 127) / 128), (unsigned)nE, 1, 256, (const void *)l.exp_gateup, guStride,
+                     (const void *)m->XpA, (size_t)0, m->moe_gu, 2 * I, H / 128, B, k, (const signed char *)m->moe_rank, nE));
+    }
+    {
+        Scope s(m, KC_MOE_GLUE);
+        RC(d->launch(d->k.moe_swiglu_quant, (unsigned)((I + 255) / 256), (unsigned)(B * k), 1, 256, (const float *)m->moe_gu, (const int *)m->moe_idx,
+                     I, k, m->XpE, xpStride));
+    }
+    {
+        Scope s(m, KC_MOE_GEMM);
+        RC(d->launch(d->k.gemm_w4a8_moe, (unsigned)((H + 127) / 128), (unsigned)nE, 1, 256, (const void *)l.exp_down, dnStride, (const void *)m->XpE,
+                     xpStride, m->moe_dn, H, I / 128, B, k, (const signed char *)m->moe_rank, nE));
+    }
+    {
+        Scope s(m, KC_MOE_GLUE);
+        RC(d->launch(d->k.moe_fold, (unsigned)((H + 255) / 256), (unsigned)B, 1, 256, (const float *)m->moe_dn, (const float *)m->moe_wgt, m->moe_out,
+                     H, k));
+    }
+    return RD_OK;
+}
+
+// emb_host: [B][hidden] on the host, or emb_dev already on the device (benchmark loop). Logits/ids are host pointers.
+int model_step(rd_model *m, int B, const int *slot, const int *pos, const float *emb_host, const float *emb_dev, int want, float *logits,
+               int *ids) {
+    rd_device *d = m->d;
+    const rd_model_desc &c = m->desc;
+    if (!m->finalized || !m->tables) {
+        rd_set_error("step before rd_model_finalize / rd_kv_configure");
+        return RD_ERR_STATE;
+    }
+    if (B < 1 || B > 32) {
+        rd_set_error("rocm resident: batch %d outside the stepper range 1..32", B);
+        return RD_ERR_ARG;
+    }
+    for (int b = 0; b < B; b++) {
+        if (!slot_ok(m, slot[b])) return RD_ERR_ARG;
+        for (int a = 0; a < b; a++)
+            if (slot[a] == slot[b]) {
+                rd_set_error("slot %d appears twice in one step", slot[b]);
+                return RD_ERR_ARG;
+            }
+        if (pos[b] < 0 || pos[b] > m->slot_len[(size_t)slot[b]]) {
+            rd_set_error("row %d: position %d but slot %d holds %d rows", b, pos[b], slot[b], m->slot_len[(size_t)slot[b]]);
+            return RD_ERR_ARG;
+        }
+        if (pos[b] >= m->ctx_cap) { // ErrKVPoolFull: nothing has been written
+            rd_set_error("row %d: position %d reaches the context cap %d", b, pos[b], m->ctx_cap);
+            return RD_ERR_KV_FULL;
+        }
+    }
+    int H = c.hidden, nH = c.n_heads, nKV = c.n_kv_heads, HD = c.head_dim;
+    std::vector<AttnItemH> items;
+    std::vector<int> start;
+    RC(build_attn_items(m, B, pos, items, start));
+    // Stage the step's metadata in pinned memory and upload it asynchronously. The staging area is reused by the next
+    // step, which is safe because every step ends with a stream synchronisation (the read-back, or the caller's timing wait).
+    {
+        char *st = (char *)m->host_stage;
+        int *rs = (int *)st, *rp = rs + 32, *rl = rp + 32, *stt = rl + 32;
+        AttnItemH *it = (AttnItemH *)(st + 4096 + sizeof(int) * start.size());
+        float *eh = (float *)(st + (1u << 20));
+        for (int b = 0; b < B; b++) rs[b] = slot[b], rp[b] = pos[b], rl[b] = pos[b] + 1;
+        memcpy(stt, start.data(), sizeof(int) * start.size());
+        memcpy(it, items.data(), sizeof(AttnItemH) * items.size());
+        RC(d->h2d(m->rowSlot, rs, sizeof(int) * (size_t)B));
+        RC(d->h2d(m->rowPos, rp, sizeof(int) * (size_t)B));
+        RC(d->h2d(m->rowLen, rl, sizeof(int) * (size_t)B));
+        RC(d->h2d(m->itemStart, stt, sizeof(int) * start.size()));
+        RC(d->h2d(m->items, it, sizeof(AttnItemH) * items.size()));
+        if (emb_host) {
+            memcpy(eh, emb_host, sizeof(float) * (size_t)B * H);
+            RC(d->h2d(m->h, eh, sizeof(float) * (size_t)B * H));
+        } else {
+            HIPCHK(MemcpyAsync(m->h, emb_dev, sizeof(float) * (size_t)B * H, hipMemcpyDeviceToDevice, d->stream));
+        }
+    }
+    const float *resP = nullptr; // pending residual contribution (split-K partials of the previous block's last GEMM)
+    int resSplits = 0;
+    for (int li = 0; li < c.n_layers; li++) {
+        LayerW &l = m->layers[(size_t)li];
+        GemmPlan plan;
+        RC(add_norm_quant(m, B, resP, resSplits, l.attn_norm, l.qkv, m->XpA, nullptr));
+        {
+            Scope s(m, KC_GEMM_QKV);
+            RC(launch_gemm(d, l.qkv, m->XpA, m->P, B, &plan));
+        }
+        {
+            Scope s(m, KC_ROPE_STORE);
+            RC(d->launch(d->k.qkv_rope_store, (unsigned)(nH + 2 * nKV), (unsigned)B, 1, (unsigned)(HD / 2), (const float *)m->P, plan.splits, m->qbuf,
+                         l.Kp, l.Vp, (const int *)m->tables, m->blocks_per_slot, (const int *)m->rowSlot, (const int *)m->rowPos,
+                         (const double *)m->inv_freq_dev, (const float *)l.q_norm, (const float *)l.k_norm, c.rms_eps, nH, nKV, HD));
+        }
+        {
+            Scope s(m, KC_ATTN_PARTIAL);
+            RC(d->launch(d->k.attn_partial, (unsigned)items.size(), 1, 1, 64, (const void *)m->items, (const int *)m->rowLen, (const int *)m->rowSlot,
+                         (const int *)m->tables, m->blocks_per_slot, (const uint16_t *)l.Kp, (const uint16_t *)l.Vp, (const float *)m->qbuf, m->part,
+                         nH, nKV, HD, c.attn_scale, c.attn_softcap));
+        }
+        {
+            Scope s(m, KC_ATTN_COMBINE);
+            RC(d->launch(d->k.attn_combine_quant, (unsigned)nH, (unsigned)B, 1, (unsigned)HD, (const float *)m->part, (const int *)m->itemStart,
+                         m->XpB, panel_kind_for(l.o), nH, nKV, HD));
+        }
+        {
+            Scope s(m, KC_GEMM_O);
+            RC(launch_gemm(d, l.o, m->XpB, m->P, B, &plan));
+        }
+        if (c.n_experts == 0) {
+            RC(add_norm_quant(m, B, m->P, plan.splits, l.ffn_norm, l.gateup, m->XpA, nullptr));
+            {
+                Scope s(m, KC_GEMM_GATEUP);
+                RC(launch_gemm(d, l.gateup, m->XpA, m->P, B, &plan));
+            }
+            {
+                Scope s(m, KC_SWIGLU);
+                RC(d->launch(d->k.swiglu_quant, (unsigned)((c.inter + 255) / 256), (unsigned)B, 1, 256, (const float *)m->P, plan.splits, c.inter,
+                             m->XpB, panel_kind_for(l.down), (float *)nullptr));
+            }
+            {
+                Scope s(m, KC_GEMM_DOWN);
+                RC(launch_gemm(d, l.down, m->XpB, m->P, B, &plan));
+            }
+            resP = m->P, resSplits = plan.splits;
+        } else {
+            {
+                Scope s(m, KC_ADD_NORM);
+                RC(d->launch(d->k.add_rmsnorm_quant, (unsigned)B, 1, 1, 256, m->h, (const float *)m->P, plan.splits, (const float *)l.ffn_norm,
+                             c.rms_eps, H, m->XpA, (int)PANEL_LIN4, m->normed));
+            }
+            RC(moe_ffn(m, B, li, l));
+            resP = m->moe_out, resSplits = 1;
+        }
+    }
+    GemmPlan plan;
+    RC(add_norm_quant(m, B, resP, resSplits, m->final_norm, m->head, m->XpA, nullptr));
+    {
+        Scope s(m, KC_GEMM_HEAD);
+        RC(launch_gemm(d, m->head, m->XpA, m->P, B, &plan));
+    }
+    {
+        Scope s(m, KC_ARGMAX);
+        RC(d->launch(d->k.argmax_rows, (unsigned)B, 1, 1, 256, (const float *)m->P, plan.splits, c.vocab, (want & RD_WANT_ARGMAX) ? m->ids : (int *)nullptr,
+                     (want & RD_WANT_LOGITS) ? m->logits : (float *)nullptr));
+    }
+    for (int b = 0; b < B; b++) m->slot_len[(size_t)slot[b]] = pos[b] + 1;
+    m->last_B = B;
+    if ((want & RD_WANT_LOGITS) && logits) RC(d->d2h(logits, m->logits, sizeof(float) * (size_t)B * c.vocab));
+    if ((want & RD_WANT_ARGMAX) && ids) RC(d->d2h(ids, m->ids, sizeof(int) * (size_t)B));
+    return RD_OK;
+}
+
+extern "C" int rd_step_batch(rd_model *m, int B, const int *slot, const int *pos, const float *emb, int want, float *logits, int *ids) {
+    if (!m || !slot || !pos || !emb) return RD_ERR_ARG;
+    if (((want & RD_WANT_LOGITS) && !logits) || ((want & RD_WANT_ARGMAX) && !ids) || !(want & 3)) {
+        rd_set_error("rd_step_batch: want=%d needs its output buffer", want);
+        return RD_ERR_ARG;
+    }
+    return model_step(m, B, slot, pos, emb, nullptr, want, logits, ids);
+}
+
+extern "C" int rd_forward(rd_model *m, int slot, int pos, const float *emb, float *logits) {
+    if (!m || !emb || !logits) return RD_ERR_ARG;
+    return model_step(m, 1, &slot, &pos, emb, nullptr, RD_WANT_LOGITS, logits, nullptr);
+}
+
+extern "C" int rd_last_moe_indices(rd_model *m, int *idx) {
+    if (!m || !idx || m->desc.n_experts == 0 || m->last_B == 0) return RD_ERR_ARG;
+    rd_device *d = m->d;
+    int k = m->desc.top_k, B = m->last_B;
+    std::vector<int> all((size_t)m->desc.n_layers * 32 * k);
+    RC(d->d2h(all.data(), m->moe_idx_all, sizeof(int) * all.size()));
+    for (int b = 0; b < B; b++)
+        for (int l = 0; l < m->desc.n_layers; l++)
+            for (int j = 0; j < k; j++) idx[((size_t)b * m->desc.n_layers + l) * k + j] = all[((size_t)l * 32 + b) * k + j];
+    return RD_OK;
+}

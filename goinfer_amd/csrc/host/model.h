@@ -1,0 +1,78 @@
+// model.h — the resident decoder behind rd_model: weights in their GEMM tilings, the paged f16 KV pool, step scratch.
+#pragma once
+#include "device.h"
+#include <map>
+#include <vector>
+
+struct AttnItemH {
+    int row, kvh, b0, b1;
+};
+
+// kernel classes of one decode step, for per-class timing
+enum {
+    KC_GEMM_QKV = 0, KC_ROPE_STORE, KC_ATTN_PARTIAL, KC_ATTN_COMBINE, KC_GEMM_O, KC_ADD_NORM, KC_GEMM_GATEUP, KC_SWIGLU, KC_GEMM_DOWN,
+    KC_GEMM_HEAD, KC_ARGMAX, KC_MOE_ROUTER, KC_MOE_GEMM, KC_MOE_GLUE, KC_COUNT
+};
+
+struct PendingMat { // a projection uploaded but not yet fused with its siblings (q|k|v, gate|up)
+    int kind = -1, N = 0, K = 0;
+    std::vector<uint8_t> data;
+    std::vector<uint8_t> scales;
+};
+
+struct LayerW {
+    DevWeight qkv, o, gateup, down;
+    PendingMat pend[RD_PROJ_COUNT];
+    float *attn_norm = nullptr, *ffn_norm = nullptr, *q_norm = nullptr, *k_norm = nullptr;
+    // MoE
+    float *router = nullptr;           // [nE][hidden] f32
+    void *exp_gateup = nullptr;        // [nE] stacked tiled W4A8, each 2*expert_inter rows x hidden
+    void *exp_down = nullptr;          // [nE] stacked tiled W4A8, each hidden rows x expert_inter
+    std::vector<char> exp_have;        // [nE*3]
+    uint16_t *Kp = nullptr, *Vp = nullptr; // KV pool of this layer
+};
+
+struct StepTimer {
+    bool on = false;
+    std::vector<hipEvent_t> ev; // pairs
+    std::vector<int> cls;
+};
+
+struct rd_model {
+    rd_device *d = nullptr;
+    rd_model_desc desc{};
+    std::vector<double> inv_freq;
+    double *inv_freq_dev = nullptr;
+    std::vector<LayerW> layers;
+    DevWeight head;
+    PendingMat head_pend;
+    float *final_norm = nullptr;
+    bool finalized = false;
+
+    // KV
+    int slots = 0, ctx_cap = 0, blocks_per_slot = 0;
+    int *tables = nullptr; // [slots][blocks_per_slot]
+    std::vector<int> slot_len;
+
+    // step scratch (device)
+    float *h = nullptr, *normed = nullptr, *P = nullptr, *qbuf = nullptr, *part = nullptr, *logits = nullptr, *emb_dev = nullptr;
+    void *XpA = nullptr, *XpB = nullptr;
+    size_t P_floats = 0;
+    int *ids = nullptr, *rowSlot = nullptr, *rowPos = nullptr, *rowLen = nullptr, *itemStart = nullptr;
+    AttnItemH *items = nullptr;
+    int max_items = 0;
+    // MoE scratch
+    float *router_logits = nullptr, *moe_wgt = nullptr, *moe_gu = nullptr, *moe_dn = nullptr, *moe_out = nullptr;
+    int *moe_idx = nullptr, *moe_idx_all = nullptr; // [32][k], [layers][32][k]
+    signed char *moe_rank = nullptr;                 // [32][nE]
+    void *XpE = nullptr;                             // per-expert down panels
+    // pinned host staging
+    void *host_stage = nullptr;
+    size_t host_stage_bytes = 0;
+    int last_B = 0;
+
+    StepTimer timer;
+};
+
+int model_step(rd_model *m, int B, const int *slot, const int *pos, const float *emb_host, const float *emb_dev, int want, float *logits,
+               int *ids);

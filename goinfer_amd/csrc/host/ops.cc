@@ -2,6 +2,7 @@
 // (backend/cuda/kernels/actgroup_kernel_test.go, flash_decode_test.go, moe_route_test.go) and what the micro-benchmarks time.
 #include "device.h"
 #include <algorithm>
+#include <numeric>
 #include <string.h>
 
 #define RC(x)                \
@@ -165,4 +166,98 @@ extern "C" int rd_moe_route(rd_device *d, const float *logits, int T, int nE, in
                  (signed char *)nullptr));
     RC(d->d2h(idx, I.p, sizeof(int) * (size_t)T * k));
     return d->d2h(wgt, W.p, sizeof(float) * (size_t)T * k);
+}
+
+// ---- ragged attention over a temporary paged pool (kernel-level entry point) ----
+struct AttnItemO {
+    int row, kvh, b0, b1;
+};
+
+extern "C" int rd_attn_ragged(rd_device *d, int n_seq, const int *len, const int64_t *off, const float *k, const float *v, const float *q,
+                              int n_h, int n_kv, int hd, float scale, float softcap, float *out) {
+    if (!d || !len || !off || !k || !v || !q || !out || n_seq <= 0) return RD_ERR_ARG;
+    if (n_kv <= 0 || n_h % n_kv || n_h / n_kv > 16 || (hd != 64 && hd != 128)) {
+        rd_set_error("rd_attn_ragged declines: head_dim must be 64 or 128 and the GQA group <= 16");
+        return RD_DECLINED;
+    }
+    int kvd = n_kv * hd, qd = n_h * hd, G = n_h / n_kv;
+    int maxBlocks = 0;
+    long totalBlocks = 0;
+    for (int i = 0; i < n_seq; i++) {
+        if (len[i] <= 0) {
+            rd_set_error("sequence %d has no keys", i);
+            return RD_ERR_ARG;
+        }
+        int nb = (len[i] + 63) / 64;
+        maxBlocks = std::max(maxBlocks, nb), totalBlocks += nb;
+    }
+    // Scattered block table: physical blocks are handed out in a stride permutation, so paging is exercised.
+    std::vector<int> tab((size_t)n_seq * maxBlocks, 0);
+    {
+        long nb = totalBlocks, stride = std::max(1L, (long)(nb * 0.618));
+        while (stride < nb && std::gcd(stride, nb) != 1) stride++;
+        if (stride >= nb) stride = 1;
+        long idx = 0;
+        for (int i = 0; i < n_seq; i++)
+            for (int b = 0; b < (len[i] + 63) / 64; b++, idx++) tab[(size_t)i * maxBlocks + b] = 1 + (int)((idx * stride) % nb);
+    }
+    size_t poolBytes = (size_t)(totalBlocks + 1) * n_kv * 64 * hd * 2;
+    DevBuf Kp(d), Vp(d), T(d), Q(d), O(d), L(d), S(d), It(d), St(d), Part(d);
+    RC(Kp.alloc(poolBytes));
+    RC(Vp.alloc(poolBytes));
+    HIPCHK(MemsetAsync(Kp.p, 0, poolBytes, d->stream));
+    HIPCHK(MemsetAsync(Vp.p, 0, poolBytes, d->stream));
+    RC(T.alloc(sizeof(int) * tab.size()));
+    RC(d->h2d(T.p, tab.data(), sizeof(int) * tab.size()));
+    {
+        int chunkRows = 4096;
+        DevBuf Kc(d), Vc(d);
+        RC(Kc.alloc(sizeof(float) * (size_t)chunkRows * kvd));
+        RC(Vc.alloc(sizeof(float) * (size_t)chunkRows * kvd));
+        for (int i = 0; i < n_seq; i++)
+            for (int base = 0; base < len[i]; base += chunkRows) {
+                int n = std::min(chunkRows, len[i] - base);
+                RC(d->h2d(Kc.p, k + ((size_t)off[i] + base) * kvd, sizeof(float) * (size_t)n * kvd));
+                RC(d->h2d(Vc.p, v + ((size_t)off[i] + base) * kvd, sizeof(float) * (size_t)n * kvd));
+                RC(d->launch(d->k.kv_store, (unsigned)n, 1, 1, (unsigned)kvd, (const float *)Kc.p, (const float *)Vc.p, (uint16_t *)Kp.p,
+                             (uint16_t *)Vp.p, (const int *)((const int *)T.p + (size_t)i * maxBlocks), base, n_kv, hd));
+                RC(d->sync());
+            }
+    }
+    for (int r0 = 0; r0 < n_seq; r0 += 32) { // rows in groups of 32, as the step batches them
+        int rows = std::min(32, n_seq - r0);
+        std::vector<AttnItemO> items;
+        std::vector<int> start((size_t)rows * n_kv + 1), slots((size_t)rows), lens((size_t)rows);
+        long tb = 0;
+        for (int i = 0; i < rows; i++) tb += (long)((len[r0 + i] + 63) / 64) * n_kv;
+        int chunk = (int)std::max(1L, (tb + 4095) / 4096);
+        for (int i = 0; i < rows; i++) {
+            int nb = (len[r0 + i] + 63) / 64;
+            slots[(size_t)i] = r0 + i, lens[(size_t)i] = len[r0 + i];
+            for (int h = 0; h < n_kv; h++) {
+                start[(size_t)i * n_kv + h] = (int)items.size();
+                for (int b0 = 0; b0 < nb; b0 += chunk) items.push_back({i, h, b0, std::min(nb, b0 + chunk)});
+            }
+        }
+        start[(size_t)rows * n_kv] = (int)items.size();
+        DevBuf Q2(d), O2(d), L2(d), S2(d), I2(d), St2(d), P2(d);
+        RC(Q2.alloc(sizeof(float) * (size_t)rows * qd));
+        RC(O2.alloc(sizeof(float) * (size_t)rows * qd));
+        RC(L2.alloc(sizeof(int) * (size_t)rows));
+        RC(S2.alloc(sizeof(int) * (size_t)rows));
+        RC(I2.alloc(sizeof(AttnItemO) * items.size()));
+        RC(St2.alloc(sizeof(int) * start.size()));
+        RC(P2.alloc(sizeof(float) * items.size() * G * (hd + 2)));
+        RC(d->h2d(Q2.p, q + (size_t)r0 * qd, sizeof(float) * (size_t)rows * qd));
+        RC(d->h2d(L2.p, lens.data(), sizeof(int) * (size_t)rows));
+        RC(d->h2d(S2.p, slots.data(), sizeof(int) * (size_t)rows));
+        RC(d->h2d(I2.p, items.data(), sizeof(AttnItemO) * items.size()));
+        RC(d->h2d(St2.p, start.data(), sizeof(int) * start.size()));
+        RC(d->launch(d->k.attn_partial, (unsigned)items.size(), 1, 1, 64, (const void *)I2.p, (const int *)L2.p, (const int *)S2.p, (const int *)T.p,
+                     maxBlocks, (const uint16_t *)Kp.p, (const uint16_t *)Vp.p, (const float *)Q2.p, P2.as<float>(), n_h, n_kv, hd, scale, softcap));
+        RC(d->launch(d->k.attn_combine, (unsigned)n_h, (unsigned)rows, 1, (unsigned)hd, (const float *)P2.p, (const int *)St2.p, O2.as<float>(), n_h,
+                     n_kv, hd));
+        RC(d->d2h(out + (size_t)r0 * qd, O2.p, sizeof(float) * (size_t)rows * qd));
+    }
+    return RD_OK;
 }

@@ -8,19 +8,14 @@
 #pragma once
 #include "common.h"
 
+// acc += panels[kb0,kb1) . (the wave's tile stream at wbase)^T. Every wave of the block must call this (barriers inside).
 template <class T, int WPB>
-__device__ __forceinline__ void gemm_body(const uint8_t *__restrict__ Wt, const void *__restrict__ aux, const uint8_t *__restrict__ Xp,
-                                          float *__restrict__ P, int N, int nKB, int kbPerSplit, int M, uint4_t *lds) {
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const int tile = blockIdx.x * WPB + wave, split = blockIdx.y;
-    const int kb0 = split * kbPerSplit, kb1 = min(nKB, kb0 + kbPerSplit);
-    const bool active = tile * 32 < N;
+__device__ __forceinline__ void gemm_mainloop(float16_t &acc, const uint8_t *__restrict__ wbase, const uint8_t *__restrict__ Xp, int kb0, int kb1,
+                                              bool active, uint4_t *lds) {
+    const int tid = threadIdx.x, lane = tid & 63;
     constexpr int PV = T::PANEL_VECS;
     constexpr int NT = WPB * 64;
     constexpr int PER = (PV + NT - 1) / NT;
-    const uint8_t *wbase = Wt + (size_t)tile * nKB * T::TILE_BYTES;
-
-    float16_t acc;
 #pragma unroll
     for (int i = 0; i < 16; i++) acc[i] = 0.f;
     if (kb0 >= kb1) return;
@@ -66,7 +61,18 @@ __device__ __forceinline__ void gemm_body(const uint8_t *__restrict__ Wt, const 
         }
         __syncthreads();
     }
-    if (active) {
+}
+
+template <class T, int WPB>
+__device__ __forceinline__ void gemm_body(const uint8_t *__restrict__ Wt, const void *__restrict__ aux, const uint8_t *__restrict__ Xp,
+                                          float *__restrict__ P, int N, int nKB, int kbPerSplit, int M, uint4_t *lds) {
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int tile = blockIdx.x * WPB + wave, split = blockIdx.y;
+    const int kb0 = split * kbPerSplit, kb1 = min(nKB, kb0 + kbPerSplit);
+    const bool active = tile * 32 < N;
+    float16_t acc;
+    gemm_mainloop<T, WPB>(acc, Wt + (size_t)tile * nKB * T::TILE_BYTES, Xp, kb0, kb1, active, lds);
+    if (active && kb0 < kb1) {
         T::finish(acc, aux, tile, lane);
         float *out = P + (size_t)split * 32 * N + tile * 32 + (lane & 31);
 #pragma unroll

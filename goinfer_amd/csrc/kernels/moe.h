@@ -1,0 +1,56 @@
+// moe.h — expert-major MoE FFN (goinfer decoder/mlp.go:630-726 moeMLPBatchWith; CUDA analogue backend/cuda/moe_rows.cu).
+// A decode batch has at most 32 tokens, so one 32-row MFMA tile covers every token: each expert's GEMM runs over all
+// token rows at once and stores only the rows routed to it — the ragged token-to-expert grouping costs no gather and
+// every expert's weights are streamed exactly once per step. rankOf[token][expert] (from rd_k_moe_route) is the map.
+#pragma once
+#include "act.h"
+#include "lin.h"
+
+// out[(token*k + rank)][N] = panels . W_e^T for the experts that have at least one token. Grid (ceil(N/128), nE).
+// xpStride: bytes between the experts' panel sets (0 = all experts read the same panels: the gate/up projections).
+extern "C" __global__ __launch_bounds__(256) void rd_k_gemm_w4a8_moe(const uint8_t *__restrict__ Wt, size_t wStride, const uint8_t *__restrict__ Xp,
+                                                                      size_t xpStride, float *__restrict__ out, int N, int nKB, int T, int k,
+                                                                      const signed char *__restrict__ rankOf, int nE) {
+    __shared__ uint4_t lds[2 * RD_LIN_PANEL_BYTES / 16];
+    const int e = blockIdx.y, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    int mine = (tid < T && rankOf[(size_t)tid * nE + e] >= 0) ? 1 : 0;
+    if (!__syncthreads_or(mine)) return;
+    const int tile = blockIdx.x * 4 + wave;
+    const bool active = tile * 32 < N;
+    float16_t acc;
+    gemm_mainloop<W4Traits, 4>(acc, Wt + (size_t)e * wStride + (size_t)tile * nKB * W4Traits::TILE_BYTES, Xp + (size_t)e * xpStride, 0, nKB, active,
+                               lds);
+    if (!active) return;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        int m = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+        if (m < T) {
+            int rank = rankOf[(size_t)m * nE + e];
+            if (rank >= 0) out[((size_t)m * k + rank) * N + tile * 32 + (lane & 31)] = acc[r];
+        }
+    }
+}
+
+// gate/up rows [(token,rank)][2I] -> silu(gate)*up -> per-32 quantization -> the down-projection panels of that row's expert.
+// Grid (ceil(I/256), T*k).
+extern "C" __global__ __launch_bounds__(256) void rd_k_moe_swiglu_quant(const float *__restrict__ gu, const int *__restrict__ idx, int I, int k,
+                                                                        uint8_t *__restrict__ XpE, size_t xpStride) {
+    int row = blockIdx.y, n = blockIdx.x * 256 + threadIdx.x, t = row / k, e = idx[row];
+    float a = 0.f;
+    if (n < I) {
+        float g = gu[(size_t)row * 2 * I + n], u = gu[(size_t)row * 2 * I + I + n];
+        double g64 = (double)g;
+        a = __fmul_rn((float)(g64 / (1.0 + exp(-g64))), u);
+    }
+    float gs, xh = quant_g32(a, &gs);
+    if (n < I) panel_store(XpE + (size_t)e * xpStride, RD_PANEL_LIN4, t, n, xh, gs);
+}
+
+// out[t][:] = sum over ranks, in rank order, of wgt[t][rank] * down[(t,rank)][:]  (decoder/mlp.go:100-103, addScaled: mul then add).
+extern "C" __global__ void rd_k_moe_fold(const float *__restrict__ dn, const float *__restrict__ wgt, float *__restrict__ out, int H, int k) {
+    int t = blockIdx.y, n = blockIdx.x * 256 + threadIdx.x;
+    if (n >= H) return;
+    float acc = 0.f;
+    for (int r = 0; r < k; r++) acc = __fadd_rn(acc, __fmul_rn(wgt[t * k + r], dn[((size_t)t * k + r) * H + n]));
+    out[(size_t)t * H + n] = acc;
+}

@@ -7,6 +7,7 @@
 #include "act.h"
 #include "attn.h"
 #include "misc.h"
+#include "moe.h"
 
 // Attention combine fused with the per-32 quantization that feeds the o-projection. Grid (nH, rows), block HD threads.
 extern "C" __global__ void rd_k_attn_combine_quant(const float *__restrict__ part, const int *__restrict__ itemStart, uint8_t *__restrict__ Xp,

@@ -1,0 +1,92 @@
+"""Ragged flash-decode attention on the GPU against the oracle's f64-accumulated attention (goinfer forwardn.go:295-500),
+through rd_attn_ragged. Bar: the reference's own flash-decode bar, rel-err <= 1e-4 against the f64 oracle
+(backend/cuda/flash_decode_test.go:56-150), plus run-to-run bit determinism."""
+import numpy as np
+import pytest
+
+from goinfer_amd import capi, synth
+from oracle import binding as ob
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    d = capi.Device(0)
+    yield d
+    d.close()
+
+
+def f16_round_trip(x):
+    """What the cache stores: binary16 with round-half-up, widened back (the oracle's own conversion)."""
+    L = ob.lib()
+    flat = x.ravel()
+    out = np.empty_like(flat)
+    for i, v in enumerate(flat):
+        out[i] = L.or_f16_to_f32(L.or_f32_to_f16(float(v)))
+    return out.reshape(x.shape)
+
+
+def oracle_attn(lens, k, v, q, nH, nKV, hd, scale, softcap):
+    out = np.empty((len(lens), nH * hd), np.float32)
+    off = 0
+    for i, n in enumerate(lens):
+        out[i] = ob.attend(q[i], k[off:off + n], v[off:off + n], n, nH, nKV, hd, scale, softcap)
+        off += n
+    return out
+
+
+@pytest.mark.parametrize("hd", [64, 128])
+@pytest.mark.parametrize("nH,nKV", [(4, 1), (8, 8), (14, 2)])
+@pytest.mark.parametrize("softcap", [0.0, 50.0])
+def test_ragged_attention_small(dev, hd, nH, nKV, softcap):
+    lens = [1, 7, 8, 9, 63, 64, 65, 300]
+    tot, kvd = sum(lens), nKV * hd
+    k = synth.normal(1, tot * kvd).reshape(tot, kvd)
+    v = synth.normal(2, tot * kvd).reshape(tot, kvd)
+    q = synth.normal(3, len(lens) * nH * hd).reshape(len(lens), nH * hd)
+    scale = float(1.0 / np.sqrt(hd))
+    got = dev.attn_ragged(lens, k, v, q, nH, nKV, hd, scale, softcap)
+    want = oracle_attn(lens, f16_round_trip(k), f16_round_trip(v), q, nH, nKV, hd, scale, softcap)
+    err = np.abs(got - want).max() / np.abs(want).max()
+    assert err <= 1e-4, err
+    again = dev.attn_ragged(lens, k, v, q, nH, nKV, hd, scale, softcap)
+    assert np.array_equal(got.view(np.uint32), again.view(np.uint32))
+
+
+def test_ragged_attention_long_split(dev):
+    """Lengths past the split threshold (several work items per (sequence, kv head)), 32q/8kv hd128 as the benchmark shape."""
+    lens = [1000, 4097, 128, 2050]
+    nH, nKV, hd = 32, 8, 128
+    tot, kvd = sum(lens), nKV * hd
+    rng = np.random.default_rng(5)
+    k = rng.standard_normal((tot, kvd), dtype=np.float32).astype(np.float16).astype(np.float32)
+    v = rng.standard_normal((tot, kvd), dtype=np.float32).astype(np.float16).astype(np.float32)
+    q = rng.standard_normal((len(lens), nH * hd), dtype=np.float32)
+    scale = float(1.0 / np.sqrt(hd))
+    for softcap in (0.0, 50.0):
+        got = dev.attn_ragged(lens, k, v, q, nH, nKV, hd, scale, softcap)
+        want = oracle_attn(lens, k, v, q, nH, nKV, hd, scale, softcap)
+        err = np.abs(got - want).max() / np.abs(want).max()
+        assert err <= 1e-4, (softcap, err)
+
+
+def test_softcap_changes_result_and_matches_closed_form(dev):
+    """Large scores so the cap bites: out = softmax(cap*tanh(s/cap)) . V against numpy float64."""
+    n, nH, nKV, hd = 130, 4, 2, 64
+    rng = np.random.default_rng(9)
+    k = (4 * rng.standard_normal((n, nKV * hd))).astype(np.float16).astype(np.float32)
+    v = rng.standard_normal((n, nKV * hd)).astype(np.float16).astype(np.float32)
+    q = (4 * rng.standard_normal((1, nH * hd))).astype(np.float32)
+    cap, scale = 5.0, 0.125
+    got = dev.attn_ragged([n], k, v, q, nH, nKV, hd, scale, cap)[0]
+    plain = dev.attn_ragged([n], k, v, q, nH, nKV, hd, scale, 0.0)[0]
+    assert np.abs(got - plain).max() > 1e-2
+    for h in range(nH):
+        kv = h // (nH // nKV)
+        s = k[:, kv * hd:(kv + 1) * hd].astype(np.float64) @ q[0, h * hd:(h + 1) * hd].astype(np.float64) * scale
+        s = cap * np.tanh(s / cap)
+        p = np.exp(s - s.max())
+        p /= p.sum()
+        want = p @ v[:, kv * hd:(kv + 1) * hd].astype(np.float64)
+        assert np.abs(got[h * hd:(h + 1) * hd] - want).max() <= 2e-4 * max(1.0, np.abs(want).max())

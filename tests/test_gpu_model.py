@@ -1,0 +1,151 @@
+"""The resident ragged batched decode step on the GPU (rd_step_batch) against the oracle's decodeMultiStep on the same
+seeded weights, KV and token ids. Bars (the north-star's): logits max-abs <= 2e-2 and relative <= 1e-2; greedy tokens
+identical except near-ties (goinfer's 3 % rule); every batched row bit-identical to the same row stepped alone."""
+import numpy as np
+import pytest
+
+from goinfer_amd import capi
+from oracle import binding as ob
+from tests.models import Pair, dense_cfg, logits_close, moe_cfg, near_tie_ok, perturbed
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    d = capi.Device(0)
+    yield d
+    d.close()
+
+
+def prefill(pair, slot, toks):
+    for p, t in enumerate(toks):
+        g, _ = pair.gpu.step_batch([slot], [p], pair.emb[t][None, :])
+    return g[0]
+
+
+def oracle_run(pair, prompts, steps, eps=0.0, force=None):
+    """The oracle on the ragged batch: per-sequence prefill, then `steps` batched greedy steps. Returns the prefill's last
+    logits, the per-step logits, the tokens fed at each step and (MoE) the expert traces. eps perturbs every embedding."""
+    B = len(prompts)
+    caches = [pair.oracle.new_cache(pair.ctx_cap) for _ in range(B)]
+    emb = (lambda t, key: perturbed(pair.emb[t], eps, key)) if eps else (lambda t, key: pair.emb[t])
+    last = []
+    for b, toks in enumerate(prompts):
+        for p, t in enumerate(toks):
+            o = pair.oracle.step(emb([t], (b, p)), [caches[b]])
+        last.append(o[0].copy())
+    nxt = force[0] if force is not None else [ob.argmax(x) for x in last]
+    fed, outs, traces = [], [], []
+    moe = pair.cfg.get("n_experts", 0) > 0
+    for s in range(steps):
+        fed.append(list(nxt))
+        r = pair.oracle.step(emb(nxt, (99, s)), caches, want_moe=moe)
+        o, tr = r if moe else (r, None)
+        outs.append(o.copy())
+        traces.append(tr)
+        nxt = force[s + 1] if force is not None and s + 1 < steps else [ob.argmax(o[b]) for b in range(B)]
+    for c in caches:
+        pair.oracle.free_cache(c)
+    return last, outs, fed, traces
+
+
+def run_ragged(pair, prompts, steps):
+    """GPU vs oracle, teacher-forced on the oracle's greedy tokens. Returns the worst logit deviation and the noise floor."""
+    B = len(prompts)
+    last, outs, fed, traces = oracle_run(pair, prompts, steps)
+    last2, outs2, _, _ = oracle_run(pair, prompts, steps, eps=1e-6, force=fed)  # same tokens, perturbed embeddings
+    floor = max([float(np.abs(a - b).max()) for a, b in zip(last, last2)] + [float(np.abs(a - b).max()) for a, b in zip(outs, outs2)])
+    worst, agree, total = 0.0, 0, 0
+    diverged = [False] * B  # MoE rows whose routing has left the oracle's: a different expert is a different function
+    for b, toks in enumerate(prompts):
+        g = prefill(pair, b, toks)
+        prefill(pair, B + b, toks)  # a twin slot, stepped alone below
+        ok, d = logits_close(g, last[b], floor)
+        assert ok, ("prefill", b, d, floor)
+        worst = max(worst, d)
+    pos = [len(t) for t in prompts]
+    for s in range(steps):
+        emb = pair.emb[fed[s]]
+        g, ids = pair.gpu.step_batch(list(range(B)), pos, emb, capi.WANT_LOGITS | capi.WANT_ARGMAX)
+        o = outs[s]
+        if traces[s] is not None:
+            gi = pair.gpu.last_moe_indices(B)
+            agree += int((gi == traces[s]).sum())
+            total += traces[s].size
+            for b in range(B):
+                diverged[b] = diverged[b] or not np.array_equal(gi[b], traces[s][b])
+        for b in range(B):
+            if diverged[b]:
+                continue
+            ok, d = logits_close(g[b], o[b], floor)
+            assert ok, ("step", s, b, d, floor)
+            worst = max(worst, d)
+            assert near_tie_ok(o[b], int(ids[b])), ("greedy token", s, b)
+            assert ids[b] == int(np.argmax(g[b]))  # device argmax == argmax of the logits it returned (lowest index on ties)
+            solo = pair.gpu.forward(B + b, pos[b], emb[b])
+            assert np.array_equal(solo.view(np.uint32), g[b].view(np.uint32)), ("batched row != solo row", s, b)
+        pos = [p + 1 for p in pos]
+    return worst, floor, (agree, total, diverged)
+
+
+def check(pair, prompts, steps):
+    worst, floor, moe = run_ragged(pair, prompts, steps)
+    pair.close()
+    print("worst logit deviation %.4f, oracle noise floor %.4f" % (worst, floor))
+    return worst, floor, moe
+
+
+def test_dense_q4k_ragged_batch(dev):
+    rng = np.random.default_rng(0)
+    check(Pair(dense_cfg(), seed=1, dev=dev, slots=8), [list(rng.integers(0, 512, n)) for n in (3, 17, 64, 130)], steps=6)
+
+
+def test_dense_hd128_gqa4(dev):
+    cfg = dense_cfg(n_layers=2, hidden=512, n_heads=4, n_kv=1, head_dim=128, inter=768, vocab=1024)
+    rng = np.random.default_rng(1)
+    check(Pair(cfg, seed=2, dev=dev, slots=4), [list(rng.integers(0, 1024, n)) for n in (5, 66)], steps=4)
+
+
+def test_dense_int8_projections_when_k_not_256(dev):
+    """hidden 384 is not a multiple of 256: q/k/v/o/gate/up fall to int8 W8A8 per goinfer's q4k-mode policy, down stays Q4_K."""
+    cfg = dense_cfg(n_layers=2, hidden=384, n_heads=6, n_kv=2, head_dim=64, inter=512, vocab=512, theta=1e6, eps=1e-6)
+    rng = np.random.default_rng(2)
+    check(Pair(cfg, seed=3, dev=dev, slots=4), [list(rng.integers(0, 512, n)) for n in (9, 40)], steps=4)
+
+
+def test_softcap_model(dev):
+    rng = np.random.default_rng(3)
+    check(Pair(dense_cfg(softcap=50.0), seed=4, dev=dev, slots=4), [list(rng.integers(0, 512, n)) for n in (4, 70)], steps=3)
+
+
+def test_moe_ragged_batch(dev):
+    rng = np.random.default_rng(4)
+    _, _, (agree, total, diverged) = check(Pair(moe_cfg(), seed=5, dev=dev, slots=8),
+                                           [list(rng.integers(0, 512, n)) for n in (2, 33, 65)], steps=6)
+    # Expert choice is discrete: once the hidden state carries the oracle's own noise floor, a router near-tie can flip,
+    # and from then on that row computes a different function (goinfer's own tests replay the reference routing for this
+    # reason, decoder/mlp.go moeSelOverride). Rows are checked against the logit bar until their routing leaves the
+    # oracle's; bit-exact routing on identical logits is asserted at kernel level (test_gpu_kernels.py).
+    print("expert index agreement %d/%d, rows diverged %s" % (agree, total, diverged))
+    assert agree >= 0.9 * total, (agree, total)
+    assert not all(diverged)
+
+
+def test_step_errors(dev):
+    pair = Pair(dense_cfg(n_layers=1), seed=6, dev=dev, slots=2, ctx_cap=64)
+    e = pair.emb[:1]
+    with pytest.raises(capi.RocmError):
+        pair.gpu.step_batch([0], [5], e)  # position beyond what the slot holds
+    with pytest.raises(capi.RocmError):
+        pair.gpu.step_batch([7], [0], e)  # no such slot
+    with pytest.raises(capi.RocmError):
+        pair.gpu.step_batch([0, 0], [0, 0], pair.emb[:2])  # one slot twice in a step
+    for p in range(64):
+        pair.gpu.step_batch([0], [p], e)
+    with pytest.raises(capi.RocmError) as ei:
+        pair.gpu.step_batch([0], [64], e)  # the context cap: goinfer's ErrKVPoolFull
+    assert "(-4)" in str(ei.value)
+    pair.gpu.kv_reset(0)
+    pair.gpu.step_batch([0], [0], e)
+    pair.close()
