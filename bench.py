@@ -1,0 +1,186 @@
+#!/usr/bin/env python3
+"""Benchmark of the ragged batched decode step on one MI355X.
+
+A step is one pass of the hot path over one batch: the greedy decode step of 32 ragged sequences of a Llama-3-8B-shaped
+Q4_K model (BASELINE.json configs[3], the configuration its metric is quoted on). Inputs (weights, KV caches, embedding
+table) are resident in HBM before the timed region; the greedy chain runs on the device (argmax -> embedding gather).
+Prints ONE JSON line with the whole-job tok/s, the roofline of the dominant kernel and a CPU baseline (the oracle's
+restatement of goinfer's CPU path, timed on this box's host cores on a bounded sample of the same workload).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def log(msg):
+    print("[bench %6.1fs] %s" % (time.time() - T0, msg), file=sys.stderr, flush=True)
+
+
+def cpu_baseline(res, cfg, lens, kept_kv, threads):
+    """The oracle's decodeMultiStep on the first two layers of the same model, the same 32 ragged sequences and KV, one
+    step; scaled to the full depth. Returns (tok/s, description of the sample)."""
+    from oracle import binding as ob
+    ob.set_threads(threads)
+    nL = len(res.kept)
+    layers = []
+    for kp in res.kept:
+        lw = {p: ob.WMat(ob.OR_Q4K, kp[p][1], kp[p][2], kp[p][0], act_group=32) for p in ("q", "k", "v", "o", "gate", "up", "down")}
+        lw["attn_norm"], lw["ffn_norm"] = kp["attn_norm"], kp["ffn_norm"]
+        layers.append(lw)
+    c = dict(cfg)
+    c.update(n_layers=nL, kv_f16=1)
+    hq, hs = res.head
+    head = ob.WMat(ob.OR_W8A8, hq.shape[0], hq.shape[1], hq, hs, act_group=32)
+    from goinfer_amd.workloads import inv_freq
+    om = ob.OracleModel(c, layers, res.final_norm, head, inv_freq(cfg["head_dim"], cfg["theta"]))
+    B = len(lens)
+    caches = []
+    import ctypes as C
+    kvd = cfg["n_kv"] * cfg["head_dim"]
+    L = ob.lib()
+    for i, n in enumerate(lens):
+        cp = om.new_cache(int(n) + 2)
+        # fill the oracle cache rows directly (f16-narrowed as the cache stores them)
+        cs = C.cast(cp, C.POINTER(_OrCache)).contents
+        for l in range(nL):
+            k, v = kept_kv[l]
+            for arr, dst in ((k, cs.k[l]), (v, cs.v[l])):
+                h = arr[:n].astype(np.float16).astype(np.float32)  # values are N(0,1): RNE and half-up differ on ties only
+                C.memmove(dst, h.ctypes.data, h.nbytes)
+        cs.pos = int(n)
+        caches.append(cp)
+    ids = np.arange(B) * 977 % cfg["vocab"]
+    emb = res.embed_rows(ids)
+    t0 = time.time()
+    om.step(emb, caches)
+    t_step = time.time() - t0
+    # the head alone, to separate it from the per-layer cost
+    x = emb
+    t0 = time.time()
+    ob.matmul(head, x)
+    t_head = time.time() - t0
+    for cp in caches:
+        om.free_cache(cp)
+    per_layer = max(t_step - t_head, 1e-9) / nL
+    full = per_layer * cfg["n_layers"] + t_head
+    sample = ("oracle decodeMultiStep, %d of %d layers + int8 head, B=%d at the run's context lengths, 1 step (%.1f s), "
+              "scaled to %d layers" % (nL, cfg["n_layers"], B, t_step, cfg["n_layers"]))
+    return B / full, sample
+
+
+import ctypes as _C  # noqa: E402
+
+
+class _OrCache(_C.Structure):
+    _fields_ = [("pos", _C.c_int), ("cap", _C.c_int), ("k", _C.POINTER(_C.c_void_p)), ("v", _C.POINTER(_C.c_void_p))]
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=32, help="model depth (32 = the Llama-3-8B shape; fewer only for debugging)")
+    ap.add_argument("--batch", type=int, default=32)
+    ap.add_argument("--seed", type=int, default=1234)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this backend is single-GPU (goinfer has no collective path); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    from goinfer_amd import capi, workloads
+
+    cfg = workloads.llama3_8b_cfg(args.layers)
+    B = args.batch
+    rng = np.random.default_rng(args.seed)
+    lens = rng.integers(512, 4097, B).astype(np.int64)  # context lengths uniform in [512, 4096]
+    ids0 = rng.integers(0, cfg["vocab"], B).astype(np.int32)
+    cap = int(lens.max()) + args.steps + args.warmup + 8
+    dev = capi.Device(0)
+    log("building %s, %d layers" % (cfg["name"], cfg["n_layers"]))
+    res = workloads.Resident(dev, cfg, seed=args.seed, slots=B, ctx_cap=cap, keep_layers=0 if args.no_cpu else min(2, args.layers), progress=log)
+    kept_kv = res.prefill_kv(lens, progress=log)
+    slots = np.arange(B, dtype=np.int32)
+
+    # ---- timed region: K greedy decode steps after W warmup steps, HIP events per step on the launch stream ----
+    dev.sync()
+    t0 = time.time()
+    ms = res.model.bench_steps(slots, lens, ids0, args.warmup, args.steps)
+    dev.sync()
+    wall = time.time() - t0
+    total_ms = float(ms.sum())
+    tok_s = B * args.steps / (total_ms / 1e3)
+    log("steps: %.3f ms mean, %.3f ms median; wall for warmup+steps %.2f s" % (ms.mean(), float(np.median(ms)), wall))
+
+    # ---- algorithmic bytes of a step at the mid-run context lengths ----
+    mid = lens + args.warmup + args.steps // 2
+    kv_pos_bytes = workloads.kv_bytes_per_position(cfg)
+    kv_read = float((mid + 1).sum()) * kv_pos_bytes
+    w_bytes = workloads.weight_bytes(cfg)
+    step_bytes = w_bytes + kv_read + B * kv_pos_bytes
+    step_gbs = step_bytes / (ms.mean() / 1e3) / 1e9
+
+    # ---- roofline of the dominant kernel: the ragged flash-decode attention (KV is ~70 % of the step's bytes) ----
+    pos_prof = (lens + args.warmup + args.steps).astype(np.int32)
+    prof = {}
+    for rep in range(3):
+        p = res.model.bench_profile(slots, pos_prof + rep, ids0)
+        for k, (t, n) in p.items():
+            a = prof.setdefault(k, [0.0, 0])
+            a[0] += t
+            a[1] += n
+    kern = "attn_partial"
+    avg_ms = prof[kern][0] / prof[kern][1]
+    # per launch (one layer): every sequence's K and V rows once (f16), plus q in and partial results out
+    G = cfg["n_heads"] // cfg["n_kv"]
+    kv_launch = float((pos_prof + 2).sum()) * 2 * cfg["n_kv"] * cfg["head_dim"] * 2
+    q_launch = B * cfg["n_heads"] * cfg["head_dim"] * 4
+    achieved = (kv_launch + q_launch) / (avg_ms / 1e3) / 1e9
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        traffic = json.load(open(tpath)).get("%s/%s" % (kern, cfg["name"]))
+    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "traffic": traffic, "kernel": "rd_k_attn_partial", "avg_launch_ms": round(avg_ms, 5),
+                "algorithmic_bytes_per_launch": int(kv_launch + q_launch)}
+    classes = {k: {"ms_per_step": round(v[0] / 3, 4), "launches_per_step": v[1] // 3} for k, v in prof.items()}
+
+    cpu = None
+    if not args.no_cpu:
+        threads = min(16, len(os.sched_getaffinity(0)))
+        log("CPU baseline on %d threads" % threads)
+        v, sample = cpu_baseline(res, cfg, lens, kept_kv, threads)
+        cpu = {"value": round(v, 3), "unit": "tok/s", "cores": threads, "kind": "port", "sample": sample}
+    res.close()
+    dev.close()
+
+    out = {
+        "metric": "batch-32 decode tok/s, Llama-3-8B-shape Q4_K; achieved HBM GB/s vs peak",
+        "value": round(tok_s, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(float(ms.mean()), 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic: N(0,0.02) weights quantized to Q4_K (int8 head), N(0,1) KV, random token ids",
+        "config": {"workload": "configs[3]: %s, %d layers, B=%d ragged, ctx U[512,4096], greedy decode" % (cfg["name"], cfg["n_layers"], B),
+                   "batch": B, "ctx_min": int(lens.min()), "ctx_max": int(lens.max()), "ctx_mean": float(lens.mean()), "seed": args.seed},
+        "step_hbm": {"algorithmic_bytes_per_step": int(step_bytes), "achieved_GBs": round(step_gbs, 1), "frac_of_peak": round(step_gbs / HBM_PEAK_GBS, 4),
+                     "weights_bytes": int(w_bytes), "kv_read_bytes": int(kv_read)},
+        "roofline": roofline,
+        "kernel_classes": classes,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(out, default=float))
+
+
+if __name__ == "__main__":
+    T0 = time.time()
+    main()

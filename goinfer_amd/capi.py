@@ -19,7 +19,8 @@ EXPORTS = [
     "rd_attn_ragged", "rd_moe_route", "rd_rmsnorm", "rd_rope", "rd_model_create", "rd_model_destroy",
     "rd_model_upload_q4k", "rd_model_upload_w8a8", "rd_model_upload_w4a8", "rd_model_upload_f32", "rd_model_finalize",
     "rd_kv_configure", "rd_kv_upload", "rd_kv_truncate", "rd_kv_reset", "rd_step_batch", "rd_forward",
-    "rd_last_moe_indices", "rd_bench_steps", "rd_bench_kernel",
+    "rd_last_moe_indices", "rd_model_upload_embedding", "rd_bench_steps", "rd_bench_profile", "rd_bench_class_count",
+    "rd_bench_class_name", "rd_bench_kernel",
 ]
 
 
@@ -245,10 +246,29 @@ class Model:
         check(lib().rd_last_moe_indices(self.h, _p(idx)), "rd_last_moe_indices")
         return idx
 
-    def bench_steps(self, slots, pos0, emb, warmup, steps):
-        emb = _f32(emb)
+    def upload_embedding(self, q, scales):
+        q = np.ascontiguousarray(q, dtype=np.int8)
+        scales = _f32(scales)
+        assert q.shape == (self.cfg["vocab"], self.cfg["hidden"])
+        check(lib().rd_model_upload_embedding(self.h, _p(q), _p(scales)), "rd_model_upload_embedding")
+
+    def bench_steps(self, slots, pos0, ids0, warmup, steps, want_ids=False):
         slots = np.ascontiguousarray(slots, dtype=np.int32)
         pos0 = np.ascontiguousarray(pos0, dtype=np.int32)
+        ids0 = np.ascontiguousarray(ids0, dtype=np.int32)
         ms = np.empty(steps, np.float32)
-        check(lib().rd_bench_steps(self.h, emb.shape[0], _p(slots), _p(pos0), _p(emb), warmup, steps, _p(ms)), "rd_bench_steps")
-        return ms
+        ids = np.empty((steps, len(slots)), np.int32) if want_ids else None
+        check(lib().rd_bench_steps(self.h, len(slots), _p(slots), _p(pos0), _p(ids0), warmup, steps, _p(ms), _p(ids)), "rd_bench_steps")
+        return (ms, ids) if want_ids else ms
+
+    def bench_profile(self, slots, pos, ids0):
+        L = lib()
+        L.rd_bench_class_name.restype = C.c_char_p
+        n = L.rd_bench_class_count()
+        slots = np.ascontiguousarray(slots, dtype=np.int32)
+        pos = np.ascontiguousarray(pos, dtype=np.int32)
+        ids0 = np.ascontiguousarray(ids0, dtype=np.int32)
+        ms = np.zeros(n, np.float32)
+        cnt = np.zeros(n, np.int32)
+        check(L.rd_bench_profile(self.h, len(slots), _p(slots), _p(pos), _p(ids0), _p(ms), _p(cnt)), "rd_bench_profile")
+        return {L.rd_bench_class_name(i).decode(): (float(ms[i]), int(cnt[i])) for i in range(n) if cnt[i]}

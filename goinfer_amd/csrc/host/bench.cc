@@ -11,10 +11,14 @@
         if (rc_) return rc_; \
     } while (0)
 
-extern "C" int rd_bench_steps(rd_model *m, int B, const int *slot, const int *pos0, const float *emb, int warmup, int steps, float *ms_out) {
-    if (!m || !slot || !pos0 || !emb || !ms_out || steps <= 0 || warmup < 0 || B < 1 || B > 32) return RD_ERR_ARG;
+// Greedy decode chain entirely on the device: ids0 are the first tokens; every step embeds the previous step's argmax
+// (rd_model_upload_embedding), runs the ragged batched step and picks the next ids. ms_out[steps] are per-step
+// milliseconds; ids_out (optional) [steps][B] are the tokens picked.
+extern "C" int rd_bench_steps(rd_model *m, int B, const int *slot, const int *pos0, const int *ids0, int warmup, int steps, float *ms_out,
+                              int *ids_out) {
+    if (!m || !slot || !pos0 || !ids0 || !ms_out || steps <= 0 || warmup < 0 || B < 1 || B > 32) return RD_ERR_ARG;
     rd_device *d = m->d;
-    RC(d->h2d(m->emb_dev, emb, sizeof(float) * (size_t)B * m->desc.hidden));
+    RC(d->h2d(m->ids, ids0, sizeof(int) * (size_t)B));
     RC(d->sync());
     hipEvent_t e0, e1;
     HIPCHK(EventCreate(&e0));
@@ -24,12 +28,15 @@ extern "C" int rd_bench_steps(rd_model *m, int B, const int *slot, const int *po
     for (int i = 0; i < warmup + steps && !rc; i++) {
         for (int b = 0; b < B; b++) pos[(size_t)b] = pos0[b] + i;
         (void)d->hip->EventRecord(e0, d->stream);
-        rc = model_step(m, B, slot, pos.data(), nullptr, m->emb_dev, RD_WANT_ARGMAX, nullptr, nullptr);
+        rc = model_step(m, B, slot, pos.data(), nullptr, nullptr, RD_WANT_ARGMAX, nullptr, nullptr);
         (void)d->hip->EventRecord(e1, d->stream);
         if (!rd_hip_ok(d->hip, d->hip->EventSynchronize(e1), "hipEventSynchronize")) rc = RD_ERR_HIP;
         float ms = 0.f;
         (void)d->hip->EventElapsedTime(&ms, e0, e1);
-        if (i >= warmup) ms_out[i - warmup] = ms;
+        if (i >= warmup) {
+            ms_out[i - warmup] = ms;
+            if (ids_out && !rc) rc = d->d2h(ids_out + (size_t)(i - warmup) * B, m->ids, sizeof(int) * (size_t)B);
+        }
     }
     (void)d->hip->EventDestroy(e0);
     (void)d->hip->EventDestroy(e1);
@@ -37,13 +44,13 @@ extern "C" int rd_bench_steps(rd_model *m, int B, const int *slot, const int *po
 }
 
 // One step with an event pair around every kernel class: class_ms[KC_COUNT] total milliseconds, class_n[KC_COUNT] launches.
-extern "C" int rd_bench_profile(rd_model *m, int B, const int *slot, const int *pos, const float *emb, float *class_ms, int *class_n) {
-    if (!m || !slot || !pos || !emb || !class_ms || !class_n) return RD_ERR_ARG;
+extern "C" int rd_bench_profile(rd_model *m, int B, const int *slot, const int *pos, const int *ids0, float *class_ms, int *class_n) {
+    if (!m || !slot || !pos || !ids0 || !class_ms || !class_n) return RD_ERR_ARG;
     rd_device *d = m->d;
-    RC(d->h2d(m->emb_dev, emb, sizeof(float) * (size_t)B * m->desc.hidden));
+    RC(d->h2d(m->ids, ids0, sizeof(int) * (size_t)B));
     RC(d->sync());
     m->timer.on = true;
-    int rc = model_step(m, B, slot, pos, nullptr, m->emb_dev, RD_WANT_ARGMAX, nullptr, nullptr);
+    int rc = model_step(m, B, slot, pos, nullptr, nullptr, RD_WANT_ARGMAX, nullptr, nullptr);
     m->timer.on = false;
     int rc2 = d->sync();
     memset(class_ms, 0, sizeof(float) * KC_COUNT);

@@ -24,7 +24,7 @@ struct Kernels {
     hipFunction_t dequant_q4k, retile_q4k, gemm_q4k_w4, gemm_q4k_w2, quant_act, reduce_splits, add_rmsnorm_quant, swiglu_quant;
     hipFunction_t retile_w8a8, gemm_w8a8, retile_w4a8, gemm_w4a8;
     hipFunction_t kv_store, qkv_rope_store, attn_partial, attn_combine, attn_combine_quant;
-    hipFunction_t rmsnorm, rope, argmax_rows, matmul_f32, moe_route, gemm_w4a8_moe, moe_swiglu_quant, moe_fold;
+    hipFunction_t rmsnorm, rope, argmax_rows, argmax_final, matmul_f32, moe_route, gemm_w4a8_moe, moe_swiglu_quant, moe_fold, embed_rows;
 };
 
 struct rd_device {

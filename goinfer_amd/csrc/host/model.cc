@@ -62,8 +62,8 @@ extern "C" void rd_model_destroy(rd_model *m) {
             d->release(p);
     }
     free_weight(d, &m->head);
-    for (void *p : {(void *)m->inv_freq_dev, (void *)m->final_norm, (void *)m->tables, (void *)m->h, (void *)m->normed, (void *)m->P, (void *)m->qbuf,
-                    (void *)m->part, (void *)m->logits, (void *)m->emb_dev, m->XpA, m->XpB, (void *)m->ids, (void *)m->rowSlot, (void *)m->rowPos,
+    for (void *p : {(void *)m->embed_q, (void *)m->embed_scale, (void *)m->inv_freq_dev, (void *)m->final_norm, (void *)m->tables, (void *)m->h, (void *)m->normed, (void *)m->P, (void *)m->qbuf,
+                    (void *)m->part, (void *)m->cand_v, (void *)m->cand_i, (void *)m->logits, (void *)m->emb_dev, m->XpA, m->XpB, (void *)m->ids, (void *)m->rowSlot, (void *)m->rowPos,
                     (void *)m->rowLen, (void *)m->itemStart, (void *)m->items, (void *)m->router_logits, (void *)m->moe_wgt, (void *)m->moe_gu,
                     (void *)m->moe_dn, (void *)m->moe_out, (void *)m->moe_idx, (void *)m->moe_idx_all, (void *)m->moe_rank, m->XpE})
         d->release(p);
@@ -257,6 +257,21 @@ extern "C" int rd_model_upload_f32(rd_model *m, int layer, int which, const floa
     return d->sync();
 }
 
+// The int8 embedding table, resident so a greedy chain can run without the host (goinfer's GreedyChain*,
+// decoder/resident/subsystems.go:78-100); the ordinary step still takes host embedding rows.
+extern "C" int rd_model_upload_embedding(rd_model *m, const int8_t *q, const float *row_scale) {
+    if (!m || !q || !row_scale) return RD_ERR_ARG;
+    rd_device *d = m->d;
+    size_t V = (size_t)m->desc.vocab, H = (size_t)m->desc.hidden;
+    if (!m->embed_q) {
+        RC(d->alloc((void **)&m->embed_q, V * H));
+        RC(d->alloc((void **)&m->embed_scale, sizeof(float) * V));
+    }
+    RC(d->h2d(m->embed_q, q, V * H));
+    RC(d->h2d(m->embed_scale, row_scale, sizeof(float) * V));
+    return d->sync();
+}
+
 static size_t gemm_partial_floats(const DevWeight &w) {
     if (w.kind < 0) return 0;
     int nKB = w.kind == 0 ? w.K / 256 : w.K / 128;
@@ -300,6 +315,8 @@ extern "C" int rd_model_finalize(rd_model *m) {
     RC(d->alloc(&m->XpA, (kA / 128) * LIN_PANEL_BYTES + Q4K_PANEL_BYTES)); // >= either panel kind for K=hidden
     RC(d->alloc(&m->XpB, (kB / 128) * LIN_PANEL_BYTES + Q4K_PANEL_BYTES));
     RC(d->alloc((void **)&m->ids, sizeof(int) * 32));
+    RC(alloc_f32(d, &m->cand_v, (size_t)32 * ((c.vocab + 4095) / 4096)));
+    RC(d->alloc((void **)&m->cand_i, sizeof(int) * 32 * (size_t)((c.vocab + 4095) / 4096)));
     RC(d->alloc((void **)&m->rowSlot, sizeof(int) * 32));
     RC(d->alloc((void **)&m->rowPos, sizeof(int) * 32));
     RC(d->alloc((void **)&m->rowLen, sizeof(int) * 32));
@@ -442,7 +459,7 @@ static int build_attn_items(rd_model *m, int B, const int *pos, std::vector<Attn
 static int add_norm_quant(rd_model *m, int B, const float *P, int splits, const float *w, const DevWeight &next, void *Xp, float *norm_out) {
     rd_device *d = m->d;
     Scope s(m, KC_ADD_NORM);
-    return d->launch(d->k.add_rmsnorm_quant, (unsigned)B, 1, 1, 256, m->h, P, splits, w, m->desc.rms_eps, m->desc.hidden, Xp, panel_kind_for(next),
+    return d->launch(d->k.add_rmsnorm_quant, (unsigned)B, 1, 1, 1024, m->h, P, splits, w, m->desc.rms_eps, m->desc.hidden, Xp, panel_kind_for(next),
                      norm_out);
 }
 
@@ -534,8 +551,15 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
         if (emb_host) {
             memcpy(eh, emb_host, sizeof(float) * (size_t)B * H);
             RC(d->h2d(m->h, eh, sizeof(float) * (size_t)B * H));
-        } else {
+        } else if (emb_dev) {
             HIPCHK(MemcpyAsync(m->h, emb_dev, sizeof(float) * (size_t)B * H, hipMemcpyDeviceToDevice, d->stream));
+        } else { // greedy chain: the previous step's argmax ids, still on the device
+            if (!m->embed_q) {
+                rd_set_error("greedy chain needs rd_model_upload_embedding");
+                return RD_ERR_STATE;
+            }
+            RC(d->launch(d->k.embed_rows, (unsigned)B, 1, 1, 256, (const signed char *)m->embed_q, (const float *)m->embed_scale, (const int *)m->ids,
+                         m->h, H));
         }
     }
     const float *resP = nullptr; // pending residual contribution (split-K partials of the previous block's last GEMM)
@@ -562,7 +586,7 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
         }
         {
             Scope s(m, KC_ATTN_COMBINE);
-            RC(d->launch(d->k.attn_combine_quant, (unsigned)nH, (unsigned)B, 1, (unsigned)HD, (const float *)m->part, (const int *)m->itemStart,
+            RC(d->launch(d->k.attn_combine_quant, (unsigned)nH, (unsigned)B, 1, (unsigned)(HD / 4), (const float *)m->part, (const int *)m->itemStart,
                          m->XpB, panel_kind_for(l.o), nH, nKV, HD));
         }
         {
@@ -577,7 +601,7 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
             }
             {
                 Scope s(m, KC_SWIGLU);
-                RC(d->launch(d->k.swiglu_quant, (unsigned)((c.inter + 255) / 256), (unsigned)B, 1, 256, (const float *)m->P, plan.splits, c.inter,
+                RC(d->launch(d->k.swiglu_quant, (unsigned)((c.inter + 1023) / 1024), (unsigned)B, 1, 256, (const float *)m->P, plan.splits, c.inter,
                              m->XpB, panel_kind_for(l.down), (float *)nullptr));
             }
             {
@@ -588,7 +612,7 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
         } else {
             {
                 Scope s(m, KC_ADD_NORM);
-                RC(d->launch(d->k.add_rmsnorm_quant, (unsigned)B, 1, 1, 256, m->h, (const float *)m->P, plan.splits, (const float *)l.ffn_norm,
+                RC(d->launch(d->k.add_rmsnorm_quant, (unsigned)B, 1, 1, 1024, m->h, (const float *)m->P, plan.splits, (const float *)l.ffn_norm,
                              c.rms_eps, H, m->XpA, (int)PANEL_LIN4, m->normed));
             }
             RC(moe_ffn(m, B, li, l));
@@ -603,8 +627,10 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
     }
     {
         Scope s(m, KC_ARGMAX);
-        RC(d->launch(d->k.argmax_rows, (unsigned)B, 1, 1, 256, (const float *)m->P, plan.splits, c.vocab, (want & RD_WANT_ARGMAX) ? m->ids : (int *)nullptr,
+        int nChunks = (c.vocab + 4095) / 4096;
+        RC(d->launch(d->k.argmax_rows, (unsigned)nChunks, (unsigned)B, 1, 256, (const float *)m->P, plan.splits, c.vocab, m->cand_v, m->cand_i,
                      (want & RD_WANT_LOGITS) ? m->logits : (float *)nullptr));
+        if (want & RD_WANT_ARGMAX) RC(d->launch(d->k.argmax_final, (unsigned)B, 1, 1, 64, (const float *)m->cand_v, (const int *)m->cand_i, nChunks, m->ids));
     }
     for (int b = 0; b < B; b++) m->slot_len[(size_t)slot[b]] = pos[b] + 1;
     m->last_B = B;

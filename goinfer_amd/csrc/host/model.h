@@ -47,6 +47,8 @@ struct rd_model {
     DevWeight head;
     PendingMat head_pend;
     float *final_norm = nullptr;
+    signed char *embed_q = nullptr; // optional device copy of the int8 embedding table (device-side greedy chain)
+    float *embed_scale = nullptr;
     bool finalized = false;
 
     // KV
@@ -58,6 +60,8 @@ struct rd_model {
     float *h = nullptr, *normed = nullptr, *P = nullptr, *qbuf = nullptr, *part = nullptr, *logits = nullptr, *emb_dev = nullptr;
     void *XpA = nullptr, *XpB = nullptr;
     size_t P_floats = 0;
+    float *cand_v = nullptr;
+    int *cand_i = nullptr;
     int *ids = nullptr, *rowSlot = nullptr, *rowPos = nullptr, *rowLen = nullptr, *itemStart = nullptr;
     AttnItemH *items = nullptr;
     int max_items = 0;

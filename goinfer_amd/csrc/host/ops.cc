@@ -56,7 +56,7 @@ static int gemm_host(rd_device *d, DevWeight &w, DevWeight *w2, const float *a, 
             RC(launch_gemm(d, *w2, Xp.p, P.as<float>(), mc, &plan));
             DevBuf X2(d);
             RC(X2.alloc((size_t)((N + 255) / 256) * Q4K_PANEL_BYTES));
-            RC(d->launch(d->k.swiglu_quant, (unsigned)((N + 255) / 256), (unsigned)mc, 1, 256, (const float *)P.p, plan.splits, N, X2.p,
+            RC(d->launch(d->k.swiglu_quant, (unsigned)((N + 1023) / 1024), (unsigned)mc, 1, 256, (const float *)P.p, plan.splits, N, X2.p,
                          (int)PANEL_Q4K, O.as<float>()));
             RC(d->sync());
         }

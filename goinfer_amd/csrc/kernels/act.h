@@ -19,6 +19,45 @@ __device__ __forceinline__ void panel_store(uint8_t *__restrict__ Xp, int kind, 
     }
 }
 
+// Four consecutive elements k0..k0+3 (k0 % 4 == 0) of batch row m. In a Q4_K panel they are the four bytes of one code
+// word and land in slots {0,1} and {4,5} (+2 for an odd sub-block) of one lane row: two 4-byte stores.
+__device__ __forceinline__ void panel_store4(uint8_t *__restrict__ Xp, int kind, int m, int k0, float x0, float x1, float x2, float x3, float gsum) {
+    if (kind == RD_PANEL_Q4K) {
+        half_t *base = (half_t *)(Xp + (size_t)(k0 >> 8) * RD_Q4K_PANEL_BYTES);
+        int t = k0 & 255, j = t >> 5;
+        half_t *row = base + q4k_panel_index(t, m); // slot of byte 0
+        *(half2_t *)row = (half2_t){(half_t)x0, (half_t)x2};
+        *(half2_t *)(row + 4) = (half2_t){(half_t)x1, (half_t)x3};
+        if ((t & 31) == 0) {
+            half_t *sp = base + q4k_panel_sum_index(j, m);
+            sp[0] = (half_t)gsum;
+            sp[4] = (half_t)0.f; // slots 4..7 of the sum step stay zero
+        }
+    } else if (kind == RD_PANEL_LIN) {
+        half_t *row = (half_t *)(Xp + (size_t)(k0 >> 7) * RD_LIN_PANEL_BYTES) + lin_panel_index(k0 & 127, m);
+        *(half2_t *)row = (half2_t){(half_t)x0, (half_t)x1};
+        *(half2_t *)(row + 2) = (half2_t){(half_t)x2, (half_t)x3};
+    } else {
+        half_t *row = (half_t *)(Xp + (size_t)(k0 >> 7) * RD_LIN_PANEL_BYTES) + lin_panel_index((k0 & 127) & ~7, m);
+        int o = k0 & 4 ? 1 : 0; // offsets 0..3 -> slots 0,2,4,6; offsets 4..7 -> slots 1,3,5,7
+        row[o] = (half_t)x0, row[o + 2] = (half_t)x1, row[o + 4] = (half_t)x2, row[o + 6] = (half_t)x3;
+    }
+}
+
+// Per-32 quantization when each lane holds 4 consecutive elements: a group is 8 consecutive lanes.
+__device__ __forceinline__ void quant_g32x4(float v0, float v1, float v2, float v3, float *x0, float *x1, float *x2, float *x3, float *gsum) {
+    float ma = fmaxf(fmaxf(fabsf(v0), fabsf(v1)), fmaxf(fabsf(v2), fabsf(v3)));
+    for (int o = 4; o > 0; o >>= 1) ma = fmaxf(ma, __shfl_xor(ma, o, 64));
+    float sc = ma / 127.f;
+    float inv = sc > 0.f ? 1.f / sc : 0.f;
+    float r0 = fminf(127.f, fmaxf(-127.f, roundf(__fmul_rn(v0, inv)))), r1 = fminf(127.f, fmaxf(-127.f, roundf(__fmul_rn(v1, inv))));
+    float r2 = fminf(127.f, fmaxf(-127.f, roundf(__fmul_rn(v2, inv)))), r3 = fminf(127.f, fmaxf(-127.f, roundf(__fmul_rn(v3, inv))));
+    int s = (int)r0 + (int)r1 + (int)r2 + (int)r3;
+    for (int o = 4; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+    *gsum = __fmul_rn(sc, (float)s);
+    *x0 = __fmul_rn(r0, sc), *x1 = __fmul_rn(r1, sc), *x2 = __fmul_rn(r2, sc), *x3 = __fmul_rn(r3, sc);
+}
+
 // x f32 [M][K] -> panels. Grid (K/256, M), 256 threads: thread t is element t of the 256-wide chunk.
 extern "C" __global__ __launch_bounds__(256) void rd_k_quant_act(const float *__restrict__ x, uint8_t *__restrict__ Xp, int K, int kind) {
     int m = blockIdx.y, k = blockIdx.x * 256 + threadIdx.x;
@@ -36,68 +75,93 @@ extern "C" __global__ void rd_k_reduce_splits(const float *__restrict__ P, float
     out[(size_t)m * N + n] = a;
 }
 
-// One block per batch row:  h[m] (+)= sum_s P[s][m][:]   (residual add of a split-K GEMM result, when P != nullptr)
-//                           normed = (h*inv)*w with inv = f32(1/sqrt(ss/H+eps)), ss summed in f64   (decoder/rmsnorm.go:29-92)
-//                           panels <- per-32 quantization of normed                                  (weightmat.go:33-38)
-// Optionally writes normed f32 to norm_out (used by MoE routing, which reads the un-quantized row).
-extern "C" __global__ __launch_bounds__(256) void rd_k_add_rmsnorm_quant(float *__restrict__ h, const float *__restrict__ P, int splits,
-                                                                         const float *__restrict__ w, float eps, int H,
-                                                                         uint8_t *__restrict__ Xp, int kind, float *__restrict__ norm_out) {
-    __shared__ double red[4];
-    int m = blockIdx.x, t = threadIdx.x;
-    float *hr = h + (size_t)m * H;
-    float vals[32]; // H <= 8192
+// One block (1024 threads) per batch row, four consecutive elements per thread:
+//   h[m] (+)= sum_s P[s][m][:]   (residual add of a split-K GEMM result, when P != nullptr; ascending split order)
+//   normed = (h*inv)*w with inv = f32(1/sqrt(ss/H+eps)), ss summed in f64   (decoder/rmsnorm.go:29-92)
+//   panels <- per-32 quantization of normed                                  (weightmat.go:33-38)
+// Optionally writes normed f32 to norm_out (the MoE router reads the un-quantized row). H % 128 == 0, H <= 8192.
+extern "C" __global__ __launch_bounds__(1024) void rd_k_add_rmsnorm_quant(float *__restrict__ h, const float *__restrict__ P, int splits,
+                                                                          const float *__restrict__ w, float eps, int H,
+                                                                          uint8_t *__restrict__ Xp, int kind, float *__restrict__ norm_out) {
+    __shared__ double red[16];
+    const int m = blockIdx.x, t = threadIdx.x, nv = H >> 2;
+    float4_t v[2];
+    bool on[2];
     double ss = 0;
 #pragma unroll
-    for (int i = 0; i < 32; i++) {
-        int k = t + i * 256;
-        if (k < H) {
-            float v = hr[k];
-            if (P) {
-                float a = P[(size_t)m * H + k];
-                for (int s = 1; s < splits; s++) a = __fadd_rn(a, P[((size_t)s * 32 + m) * H + k]);
-                v = __fadd_rn(v, a);
-                hr[k] = v;
-            }
-            vals[i] = v;
-            ss += (double)v * (double)v;
-        }
+    for (int i = 0; i < 2; i++) {
+        int q = t + i * 1024;
+        on[i] = q < nv;
+        v[i] = (float4_t){0.f, 0.f, 0.f, 0.f};
+        if (on[i]) v[i] = *(const float4_t *)(h + (size_t)m * H + 4 * q);
     }
+    if (P) {
+        float4_t a[2];
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+            if (on[i]) a[i] = *(const float4_t *)(P + (size_t)m * H + 4 * (t + i * 1024));
+        for (int s = 1; s < splits; s++) {
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+                if (on[i]) {
+                    float4_t b = *(const float4_t *)(P + ((size_t)s * 32 + m) * H + 4 * (t + i * 1024));
+                    a[i].x = __fadd_rn(a[i].x, b.x), a[i].y = __fadd_rn(a[i].y, b.y), a[i].z = __fadd_rn(a[i].z, b.z), a[i].w = __fadd_rn(a[i].w, b.w);
+                }
+        }
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+            if (on[i]) {
+                v[i].x = __fadd_rn(v[i].x, a[i].x), v[i].y = __fadd_rn(v[i].y, a[i].y), v[i].z = __fadd_rn(v[i].z, a[i].z), v[i].w = __fadd_rn(v[i].w, a[i].w);
+                *(float4_t *)(h + (size_t)m * H + 4 * (t + i * 1024)) = v[i];
+            }
+    }
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+        ss += (double)v[i].x * v[i].x + (double)v[i].y * v[i].y + (double)v[i].z * v[i].z + (double)v[i].w * v[i].w;
     ss = wave_sum64_d(ss);
     if ((t & 63) == 0) red[t >> 6] = ss;
     __syncthreads();
-    ss = (red[0] + red[1]) + (red[2] + red[3]);
+    ss = 0;
+#pragma unroll
+    for (int i = 0; i < 16; i++) ss += red[i];
     float inv = (float)(1.0 / sqrt(ss / (double)H + (double)eps));
 #pragma unroll
-    for (int i = 0; i < 32; i++) {
-        int k = t + i * 256;
-        if (k < H) {
-            float nv = __fmul_rn(__fmul_rn(vals[i], inv), w[k]);
-            if (norm_out) norm_out[(size_t)m * H + k] = nv;
-            float gs, xh = quant_g32(nv, &gs);
-            panel_store(Xp, kind, m, k, xh, gs);
-        }
+    for (int i = 0; i < 2; i++) {
+        if (!on[i]) continue; // whole waves drop out together: nv is a multiple of 32
+        int k0 = 4 * (t + i * 1024);
+        float4_t wv = *(const float4_t *)(w + k0);
+        float n0 = __fmul_rn(__fmul_rn(v[i].x, inv), wv.x), n1 = __fmul_rn(__fmul_rn(v[i].y, inv), wv.y);
+        float n2 = __fmul_rn(__fmul_rn(v[i].z, inv), wv.z), n3 = __fmul_rn(__fmul_rn(v[i].w, inv), wv.w);
+        if (norm_out) *(float4_t *)(norm_out + (size_t)m * H + k0) = (float4_t){n0, n1, n2, n3};
+        float x0, x1, x2, x3, gs;
+        quant_g32x4(n0, n1, n2, n3, &x0, &x1, &x2, &x3, &gs);
+        panel_store4(Xp, kind, m, k0, x0, x1, x2, x3, gs);
     }
 }
 
 // gate/up partials P[s][32][2I] -> act = silu(gate)*up (decoder/rmsnorm.go:204-207: silu in f64) -> per-32 quant -> panels.
-// Grid (ceil(I/256), M).
+// Grid (ceil(I/1024), M), 256 threads, four consecutive columns per thread. I % 32 == 0.
 extern "C" __global__ __launch_bounds__(256) void rd_k_swiglu_quant(const float *__restrict__ P, int splits, int I, uint8_t *__restrict__ Xp,
                                                                     int kind, float *__restrict__ act_out) {
-    int m = blockIdx.y, n = blockIdx.x * 256 + threadIdx.x;
-    float a = 0.f;
-    if (n < I) {
+    int m = blockIdx.y, n0 = (blockIdx.x * 256 + threadIdx.x) * 4;
+    bool on = n0 < I; // groups of 8 lanes are on or off together
+    float a[4] = {0.f, 0.f, 0.f, 0.f};
+    if (on) {
         int N2 = 2 * I;
-        float g = P[(size_t)m * N2 + n], u = P[(size_t)m * N2 + I + n];
+        float4_t g = *(const float4_t *)(P + (size_t)m * N2 + n0), u = *(const float4_t *)(P + (size_t)m * N2 + I + n0);
         for (int s = 1; s < splits; s++) {
-            g = __fadd_rn(g, P[((size_t)s * 32 + m) * N2 + n]);
-            u = __fadd_rn(u, P[((size_t)s * 32 + m) * N2 + I + n]);
+            float4_t g2 = *(const float4_t *)(P + ((size_t)s * 32 + m) * N2 + n0), u2 = *(const float4_t *)(P + ((size_t)s * 32 + m) * N2 + I + n0);
+            g.x = __fadd_rn(g.x, g2.x), g.y = __fadd_rn(g.y, g2.y), g.z = __fadd_rn(g.z, g2.z), g.w = __fadd_rn(g.w, g2.w);
+            u.x = __fadd_rn(u.x, u2.x), u.y = __fadd_rn(u.y, u2.y), u.z = __fadd_rn(u.z, u2.z), u.w = __fadd_rn(u.w, u2.w);
         }
-        double g64 = (double)g;
-        float sl = (float)(g64 / (1.0 + exp(-g64)));
-        a = __fmul_rn(sl, u);
-        if (act_out) act_out[(size_t)m * I + n] = a;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            double g64 = (double)g[i];
+            a[i] = __fmul_rn((float)(g64 / (1.0 + exp(-g64))), u[i]);
+        }
+        if (act_out) *(float4_t *)(act_out + (size_t)m * I + n0) = (float4_t){a[0], a[1], a[2], a[3]};
     }
-    float gs, xh = quant_g32(a, &gs);
-    if (n < I) panel_store(Xp, kind, m, n, xh, gs);
+    float x0, x1, x2, x3, gs;
+    quant_g32x4(a[0], a[1], a[2], a[3], &x0, &x1, &x2, &x3, &gs);
+    if (on) panel_store4(Xp, kind, m, n0, x0, x1, x2, x3, gs);
 }

@@ -254,6 +254,24 @@ __device__ __forceinline__ float attn_combine_value(const float *__restrict__ pa
     return num / den;
 }
 
+__device__ __forceinline__ void attn_combine_value4(const float *__restrict__ part, const int *__restrict__ itemStart, int nH, int nKV, int HD,
+                                                    int m, int head, int d0, float *out) {
+    int G = nH / nKV, kvh = head / G, g = head % G;
+    int i0 = itemStart[m * nKV + kvh], i1 = itemStart[m * nKV + kvh + 1];
+    float M = -INFINITY;
+    for (int i = i0; i < i1; i++) M = fmaxf(M, part[((size_t)i * G + g) * (HD + 2) + HD]);
+    float num[4] = {0.f, 0.f, 0.f, 0.f}, den = 0.f;
+    for (int i = i0; i < i1; i++) {
+        const float *p = part + ((size_t)i * G + g) * (HD + 2);
+        float w = __expf(p[HD] - M);
+        float2 a = *(const float2 *)(p + d0), b = *(const float2 *)(p + d0 + 2); // rows are 8-byte aligned: (HD+2) is even
+        num[0] = fmaf(a.x, w, num[0]), num[1] = fmaf(a.y, w, num[1]), num[2] = fmaf(b.x, w, num[2]), num[3] = fmaf(b.y, w, num[3]);
+        den = fmaf(p[HD + 1], w, den);
+    }
+#pragma unroll
+    for (int e = 0; e < 4; e++) out[e] = num[e] / den;
+}
+
 extern "C" __global__ void rd_k_attn_combine(const float *__restrict__ part, const int *__restrict__ itemStart, float *__restrict__ out, int nH,
                                              int nKV, int HD) {
     int head = blockIdx.x, m = blockIdx.y, d = threadIdx.x;

@@ -31,31 +31,62 @@ extern "C" __global__ void rd_k_rope(float *__restrict__ vec, const int *__restr
     v[t + half] = (float)(x2 * c + x1 * s);
 }
 
-// internal/runtime/sampling/sampler.go:485-520: the first maximum wins. One block per row, rows read from split-K partials.
-extern "C" __global__ __launch_bounds__(256) void rd_k_argmax_rows(const float *__restrict__ P, int splits, int N, int *__restrict__ ids,
-                                                                   float *__restrict__ logits_out) {
-    __shared__ float bv[256];
-    __shared__ int bi[256];
-    int m = blockIdx.x, t = threadIdx.x;
+// internal/runtime/sampling/sampler.go:485-520: the first maximum wins. Two stages: per (row, 4096-column chunk) a block
+// reduces split-K partials, optionally writes the logits, and leaves its best (value, lowest index); a second kernel folds the
+// chunks of each row. N % 4 == 0.
+extern "C" __global__ __launch_bounds__(256) void rd_k_argmax_rows(const float *__restrict__ P, int splits, int N, float *__restrict__ cand_v,
+                                                                   int *__restrict__ cand_i, float *__restrict__ logits_out) {
+    __shared__ float bv[4];
+    __shared__ int bi[4];
+    const int m = blockIdx.y, t = threadIdx.x, nChunks = gridDim.x;
     float best = -INFINITY;
     int idx = 0x7fffffff;
-    for (int n = t; n < N; n += 256) {
-        float a = P[(size_t)m * N + n];
-        for (int s = 1; s < splits; s++) a = __fadd_rn(a, P[((size_t)s * 32 + m) * N + n]);
-        if (logits_out) logits_out[(size_t)m * N + n] = a;
-        if (a > best || (a == best && n < idx)) best = a, idx = n;
-    }
-    bv[t] = best, bi[t] = idx;
-    __syncthreads();
-    for (int o = 128; o > 0; o >>= 1) {
-        if (t < o) {
-            float v2 = bv[t + o];
-            int i2 = bi[t + o];
-            if (v2 > bv[t] || (v2 == bv[t] && i2 < bi[t])) bv[t] = v2, bi[t] = i2;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        int n0 = blockIdx.x * 4096 + (i * 256 + t) * 4;
+        if (n0 < N) {
+            float4_t a = *(const float4_t *)(P + (size_t)m * N + n0);
+            for (int s = 1; s < splits; s++) {
+                float4_t b = *(const float4_t *)(P + ((size_t)s * 32 + m) * N + n0);
+                a.x = __fadd_rn(a.x, b.x), a.y = __fadd_rn(a.y, b.y), a.z = __fadd_rn(a.z, b.z), a.w = __fadd_rn(a.w, b.w);
+            }
+            if (logits_out) *(float4_t *)(logits_out + (size_t)m * N + n0) = a;
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (a[e] > best) best = a[e], idx = n0 + e; // ascending n within a thread: strict '>' keeps the lowest index
         }
-        __syncthreads();
     }
-    if (t == 0 && ids) ids[m] = bi[0] == 0x7fffffff ? 0 : bi[0];
+    for (int o = 32; o > 0; o >>= 1) {
+        float v2 = __shfl_xor(best, o, 64);
+        int i2 = __shfl_xor(idx, o, 64);
+        if (v2 > best || (v2 == best && i2 < idx)) best = v2, idx = i2;
+    }
+    if ((t & 63) == 0) bv[t >> 6] = best, bi[t >> 6] = idx;
+    __syncthreads();
+    if (t == 0) {
+        for (int w = 1; w < 4; w++)
+            if (bv[w] > best || (bv[w] == best && bi[w] < idx)) best = bv[w], idx = bi[w];
+        cand_v[m * nChunks + blockIdx.x] = best;
+        cand_i[m * nChunks + blockIdx.x] = idx;
+    }
+}
+
+extern "C" __global__ __launch_bounds__(64) void rd_k_argmax_final(const float *__restrict__ cand_v, const int *__restrict__ cand_i, int nChunks,
+                                                                   int *__restrict__ ids) {
+    const int m = blockIdx.x, t = threadIdx.x;
+    float best = -INFINITY;
+    int idx = 0x7fffffff;
+    for (int c = t; c < nChunks; c += 64) {
+        float v = cand_v[m * nChunks + c];
+        int i = cand_i[m * nChunks + c];
+        if (v > best || (v == best && i < idx)) best = v, idx = i;
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+        float v2 = __shfl_xor(best, o, 64);
+        int i2 = __shfl_xor(idx, o, 64);
+        if (v2 > best || (v2 == best && i2 < idx)) best = v2, idx = i2;
+    }
+    if (t == 0) ids[m] = idx == 0x7fffffff ? 0 : idx;
 }
 
 // dst[M][N] = a[M][K] . b[N][K]^T with an ascending-k f64 accumulator rounded once: Backend.MatmulBT (decoder/backend.go:26-30)
@@ -110,4 +141,13 @@ extern "C" __global__ void rd_k_moe_route(const float *__restrict__ logits, int 
     }
     if (norm && s > 0.f)
         for (int j = 0; j < n; j++) wgt[(size_t)t * k + j] = wgt[(size_t)t * k + j] / s;
+}
+
+// Token embedding rows from an int8 table with one f32 scale per row (goinfer keeps the embedding table int8 in q4k mode,
+// decoder/weightmat.go:79-84; Embed.Row widens q*scale): h[m][k] = q[ids[m]][k] * scale[ids[m]]. Grid (rows), block 256.
+extern "C" __global__ void rd_k_embed_rows(const signed char *__restrict__ q, const float *__restrict__ scale, const int *__restrict__ ids,
+                                           float *__restrict__ h, int H) {
+    int m = blockIdx.x, id = ids[m];
+    float sc = scale[id];
+    for (int k = threadIdx.x; k < H; k += blockDim.x) h[(size_t)m * H + k] = __fmul_rn((float)q[(size_t)id * H + k], sc);
 }

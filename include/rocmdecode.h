@@ -124,12 +124,20 @@ int rd_forward(rd_model *m, int slot, int pos, const float *emb, float *logits);
 /* expert indices the last step routed to: int32 [B][n_layers][top_k] (MoE models only; parity checks) */
 int rd_last_moe_indices(rd_model *m, int *idx);
 
-/* ---- measurement: HIP-event timing of steps with inputs already resident in HBM ---- */
-/* Runs `steps` decode steps for the given (slot,pos0) batch after `warmup` untimed ones; each step advances every
- * row's position by one and feeds back a fixed embedding (no host transfer inside the timed region).
- * ms_out[steps]: per-step milliseconds from HIP events on the stream the kernels are launched on. */
-int rd_bench_steps(rd_model *m, int B, const int *slot, const int *pos0, const float *emb, int warmup, int steps, float *ms_out);
-/* Times `iters` launches of one kernel class over resident synthetic operands; see rocmdecode_bench.h names. */
+/* ---- measurement: HIP-event timing on the stream the kernels are launched on; inputs resident in HBM ---- */
+/* The int8 embedding table (vocab x hidden codes + one f32 scale per row), resident so a greedy chain needs no host
+ * round trip: goinfer's GreedyChain* (decoder/resident/subsystems.go:78-100). */
+int rd_model_upload_embedding(rd_model *m, const int8_t *q, const float *row_scale);
+/* Greedy decode chain on the device: step i runs rows (slot[b], pos0[b]+i) on the embedding of the previous step's
+ * argmax (ids0 for the first). ms_out[steps]: per-step milliseconds; ids_out: optional int32 [steps][B] picked tokens. */
+int rd_bench_steps(rd_model *m, int B, const int *slot, const int *pos0, const int *ids0, int warmup, int steps, float *ms_out,
+                   int *ids_out);
+/* One step with a HIP-event pair around every kernel class: class_ms[n] total milliseconds and class_n[n] launches,
+ * n = rd_bench_class_count(); names from rd_bench_class_name. */
+int rd_bench_profile(rd_model *m, int B, const int *slot, const int *pos, const int *ids0, float *class_ms, int *class_n);
+int rd_bench_class_count(void);
+const char *rd_bench_class_name(int c);
+/* Times `iters` launches of one kernel over resident synthetic operands: "gemm_q4k" args {N,K,M,copies}; "copy" args {bytes}. */
 int rd_bench_kernel(rd_device *d, const char *name, const int64_t *args, int n_args, int warmup, int iters, float *ms_out);
 
 #ifdef __cplusplus
