@@ -105,7 +105,7 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
         size_t pb = (size_t)(K / 256) * Q4K_PANEL_BYTES;
         if (!rc) rc = Xp.alloc(pb);
         int nKB = K / 256;
-        GemmPlan plan = plan_gemm(N, nKB);
+        GemmPlan plan = plan_gemm(0, N, nKB);
         if (!rc) rc = P.alloc(sizeof(float) * (size_t)plan.splits * 32 * N);
         if (!rc) {
             std::vector<uint16_t> x(pb / 2);

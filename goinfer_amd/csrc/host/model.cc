@@ -275,7 +275,7 @@ extern "C" int rd_model_upload_embedding(rd_model *m, const int8_t *q, const flo
 static size_t gemm_partial_floats(const DevWeight &w) {
     if (w.kind < 0) return 0;
     int nKB = w.kind == 0 ? w.K / 256 : w.K / 128;
-    return (size_t)plan_gemm(w.N, nKB).splits * 32 * w.N;
+    return (size_t)plan_gemm(w.kind, w.N, nKB).splits * 32 * w.N;
 }
 
 extern "C" int rd_model_finalize(rd_model *m) {
@@ -595,11 +595,15 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
         }
         if (c.n_experts == 0) {
             RC(add_norm_quant(m, B, m->P, plan.splits, l.ffn_norm, l.gateup, m->XpA, nullptr));
-            {
-                Scope s(m, KC_GEMM_GATEUP);
-                RC(launch_gemm(d, l.gateup, m->XpA, m->P, B, &plan));
-            }
-            {
+            if (l.gateup.kind == 0 && c.inter % 64 == 0 && !getenv("ROCMDECODE_NO_FUSED_GATEUP")) {
+                Scope s(m, KC_GEMM_GATEUP); // gate|up GEMM + SwiGLU + quantization in one launch
+                RC(d->launch(d->k.gemm_q4k_gateup, (unsigned)(c.inter / 64), 1, 1, 256, (const void *)l.gateup.tiled, (const void *)m->XpA, m->XpB,
+                             panel_kind_for(l.down), c.inter, H / 256, B));
+            } else {
+                {
+                    Scope s(m, KC_GEMM_GATEUP);
+                    RC(launch_gemm(d, l.gateup, m->XpA, m->P, B, &plan));
+                }
                 Scope s(m, KC_SWIGLU);
                 RC(d->launch(d->k.swiglu_quant, (unsigned)((c.inter + 1023) / 1024), (unsigned)B, 1, 256, (const float *)m->P, plan.splits, c.inter,
                              m->XpB, panel_kind_for(l.down), (float *)nullptr));

@@ -40,7 +40,7 @@ static int gemm_host(rd_device *d, DevWeight &w, DevWeight *w2, const float *a, 
     RC(Xp.alloc(pbytes));
     int nKB = w.kind == 0 ? K / 256 : K / 128;
     int Ntot = w2 ? 2 * N : N;
-    int maxSplits = plan_gemm(Ntot, nKB).splits;
+    int maxSplits = plan_gemm(w.kind, Ntot, nKB).splits;
     RC(P.alloc(sizeof(float) * (size_t)maxSplits * 32 * Ntot));
     RC(O.alloc(sizeof(float) * (size_t)32 * N));
     for (int m0 = 0; m0 < M; m0 += 32) {

@@ -87,6 +87,8 @@ extern "C" __global__ void rd_k_qkv_rope_store(const float *__restrict__ P, int 
 
 typedef float float4v __attribute__((ext_vector_type(4)));
 
+__device__ __forceinline__ float ld_part(const float *p) { return *p; }
+
 struct AttnItem {
     int row, kvh, b0, b1; // sequence row, kv head, block range [b0,b1) of that sequence
 };
@@ -216,10 +218,7 @@ __device__ __forceinline__ void attn_partial_body(const AttnItem *__restrict__ i
             float *dst = part + ((size_t)blockIdx.x * G + g) * (HD + 2);
 #pragma unroll
             for (int ct = 0; ct < NCT; ct++) dst[ct * 16 + l16] = O[ct][r];
-            if (l16 == 0) {
-                dst[HD] = mrun[r];
-                dst[HD + 1] = lrun[r];
-            }
+            if (l16 == 0) dst[HD] = mrun[r], dst[HD + 1] = lrun[r];
         }
     }
 }
@@ -254,19 +253,35 @@ __device__ __forceinline__ float attn_combine_value(const float *__restrict__ pa
     return num / den;
 }
 
+// Four consecutive d of one (row, head): the block's threads first fetch every item's running max in parallel (no
+// dependent-load chain), then fold the items in ascending order with independent loads.
 __device__ __forceinline__ void attn_combine_value4(const float *__restrict__ part, const int *__restrict__ itemStart, int nH, int nKV, int HD,
                                                     int m, int head, int d0, float *out) {
     int G = nH / nKV, kvh = head / G, g = head % G;
     int i0 = itemStart[m * nKV + kvh], i1 = itemStart[m * nKV + kvh + 1];
+    const float *base = part + ((size_t)i0 * G + g) * (HD + 2);
+    const size_t stride = (size_t)G * (HD + 2);
     float M = -INFINITY;
-    for (int i = i0; i < i1; i++) M = fmaxf(M, part[((size_t)i * G + g) * (HD + 2) + HD]);
+    for (int i = 0; i < i1 - i0; i += 4) {
+        float a = ld_part(base + (size_t)i * stride + HD);
+        float b = i + 1 < i1 - i0 ? ld_part(base + (size_t)(i + 1) * stride + HD) : -INFINITY;
+        float c = i + 2 < i1 - i0 ? ld_part(base + (size_t)(i + 2) * stride + HD) : -INFINITY;
+        float e = i + 3 < i1 - i0 ? ld_part(base + (size_t)(i + 3) * stride + HD) : -INFINITY;
+        M = fmaxf(fmaxf(M, fmaxf(a, b)), fmaxf(c, e));
+    }
     float num[4] = {0.f, 0.f, 0.f, 0.f}, den = 0.f;
-    for (int i = i0; i < i1; i++) {
-        const float *p = part + ((size_t)i * G + g) * (HD + 2);
-        float w = __expf(p[HD] - M);
-        float2 a = *(const float2 *)(p + d0), b = *(const float2 *)(p + d0 + 2); // rows are 8-byte aligned: (HD+2) is even
+    for (int i = 0; i < i1 - i0; i += 2) {
+        const float *p = base + (size_t)i * stride;
+        bool two = i + 1 < i1 - i0;
+        const float *p2 = two ? p + stride : p;
+        float2 a = {ld_part(p + d0), ld_part(p + d0 + 1)}, b = {ld_part(p + d0 + 2), ld_part(p + d0 + 3)};
+        float2 a2 = {ld_part(p2 + d0), ld_part(p2 + d0 + 1)}, b2 = {ld_part(p2 + d0 + 2), ld_part(p2 + d0 + 3)};
+        float w = __expf(ld_part(p + HD) - M), l = ld_part(p + HD + 1);
+        float w2 = two ? __expf(ld_part(p2 + HD) - M) : 0.f, l2 = ld_part(p2 + HD + 1);
         num[0] = fmaf(a.x, w, num[0]), num[1] = fmaf(a.y, w, num[1]), num[2] = fmaf(b.x, w, num[2]), num[3] = fmaf(b.y, w, num[3]);
-        den = fmaf(p[HD + 1], w, den);
+        den = fmaf(l, w, den);
+        num[0] = fmaf(a2.x, w2, num[0]), num[1] = fmaf(a2.y, w2, num[1]), num[2] = fmaf(b2.x, w2, num[2]), num[3] = fmaf(b2.y, w2, num[3]);
+        den = fmaf(l2, w2, den);
     }
 #pragma unroll
     for (int e = 0; e < 4; e++) out[e] = num[e] / den;

@@ -7,60 +7,70 @@
 // row computed in a batch is bit-identical to the same row computed alone.
 #pragma once
 #include "common.h"
+#include <type_traits>
 
 // acc += panels[kb0,kb1) . (the wave's tile stream at wbase)^T. Every wave of the block must call this (barriers inside).
-template <class T, int WPB>
+// Software pipeline: weight tiles are PF K-blocks ahead in registers; the activation panel of K-block it+2 is in flight
+// (global -> registers) while it is computed and is published to the LDS buffer vacated one barrier earlier.
+// Every load in the loop body is unconditional (indices are clamped to the last K-block, so the tail re-reads it):
+// with a fixed number of loads per iteration the compiler can wait for exactly the load it needs (s_waitcnt vmcnt(n))
+// and leave the prefetches in flight; conditional loads force it to drain the whole queue.
+template <class T, int WPB, int PF = 3>
 __device__ __forceinline__ void gemm_mainloop(float16_t &acc, const uint8_t *__restrict__ wbase, const uint8_t *__restrict__ Xp, int kb0, int kb1,
                                               bool active, uint4_t *lds) {
+    (void)active; // inactive waves run on a clamped tile (the caller clamps wbase) and simply do not store
     const int tid = threadIdx.x, lane = tid & 63;
     constexpr int PV = T::PANEL_VECS;
     constexpr int NT = WPB * 64;
     constexpr int PER = (PV + NT - 1) / NT;
 #pragma unroll
     for (int i = 0; i < 16; i++) acc[i] = 0.f;
-    if (kb0 >= kb1) return;
+    const int nk = kb1 - kb0;
+    if (nk <= 0) return;
+    const int last = nk - 1;
+    const uint8_t *wb = wbase + (size_t)kb0 * T::TILE_BYTES;
+    const uint4_t *src = (const uint4_t *)Xp + (size_t)kb0 * PV;
+    // vector index of this thread's PER panel slices (the last slice is clamped; its duplicate writes carry the same data)
+    int pv[PER];
+#pragma unroll
+    for (int i = 0; i < PER; i++) pv[i] = min(tid + i * NT, PV - 1);
 
-    typename T::Tile w0, w1;
-    if (active) {
-        T::load(w0, wbase + (size_t)kb0 * T::TILE_BYTES, lane);
-        if (kb0 + 1 < kb1) T::load(w1, wbase + (size_t)(kb0 + 1) * T::TILE_BYTES, lane);
-    }
-    {
-        const uint4_t *src = (const uint4_t *)Xp + (size_t)kb0 * PV;
+    typename T::Tile w[PF];
 #pragma unroll
-        for (int i = 0; i < PER; i++) {
-            int v = tid + i * NT;
-            if (v < PV) lds[v] = src[v];
-        }
-    }
+    for (int i = 0; i < PF; i++) T::load(w[i], wb + (size_t)min(i, last) * T::TILE_BYTES, lane);
+    uint4_t stage[PER];
+#pragma unroll
+    for (int i = 0; i < PER; i++) lds[pv[i]] = src[pv[i]];
+#pragma unroll
+    for (int i = 0; i < PER; i++) stage[i] = src[(size_t)min(1, last) * PV + pv[i]];
     __syncthreads();
-    for (int kb = kb0; kb < kb1; kb++) {
-        const int cur = (kb - kb0) & 1;
-        uint4_t stage[PER];
-        const bool more = kb + 1 < kb1;
-        if (more) {
-            const uint4_t *src = (const uint4_t *)Xp + (size_t)(kb + 1) * PV;
+
+    auto body = [&](int it, auto uc) {
+        constexpr int u = decltype(uc)::value;
+        const int cur = it & 1;
+        uint4_t *dst = lds + (cur ^ 1) * PV;
 #pragma unroll
-            for (int i = 0; i < PER; i++) {
-                int v = tid + i * NT;
-                if (v < PV) stage[i] = src[v];
-            }
-        }
-        if (active) {
-            T::mma(acc, w0, lds + cur * PV, lane);
-            w0 = w1;
-            if (kb + 2 < kb1) T::load(w1, wbase + (size_t)(kb + 2) * T::TILE_BYTES, lane);
-        }
-        if (more) {
-            uint4_t *dst = lds + (cur ^ 1) * PV;
+        for (int i = 0; i < PER; i++) dst[pv[i]] = stage[i]; // panel it+1 (or a harmless copy of the last one)
+        const uint4_t *s2 = src + (size_t)min(it + 2, last) * PV;
 #pragma unroll
-            for (int i = 0; i < PER; i++) {
-                int v = tid + i * NT;
-                if (v < PV) dst[v] = stage[i];
-            }
-        }
+        for (int i = 0; i < PER; i++) stage[i] = s2[pv[i]];
+        T::mma(acc, w[u], lds + cur * PV, lane);
+        T::load(w[u], wb + (size_t)min(it + PF, last) * T::TILE_BYTES, lane);
         __syncthreads();
+    };
+    int it = 0;
+    for (; it + PF <= nk; it += PF) {
+        if constexpr (PF > 0) body(it + 0, std::integral_constant<int, 0>{});
+        if constexpr (PF > 1) body(it + 1, std::integral_constant<int, 1>{});
+        if constexpr (PF > 2) body(it + 2, std::integral_constant<int, 2>{});
+        if constexpr (PF > 3) body(it + 3, std::integral_constant<int, 3>{});
     }
+    if constexpr (PF > 1)
+        if (it + 0 < nk) body(it + 0, std::integral_constant<int, 0>{});
+    if constexpr (PF > 2)
+        if (it + 1 < nk) body(it + 1, std::integral_constant<int, 1>{});
+    if constexpr (PF > 3)
+        if (it + 2 < nk) body(it + 2, std::integral_constant<int, 2>{});
 }
 
 template <class T, int WPB>
@@ -71,7 +81,11 @@ __device__ __forceinline__ void gemm_body(const uint8_t *__restrict__ Wt, const 
     const int kb0 = split * kbPerSplit, kb1 = min(nKB, kb0 + kbPerSplit);
     const bool active = tile * 32 < N;
     float16_t acc;
-    gemm_mainloop<T, WPB>(acc, Wt + (size_t)tile * nKB * T::TILE_BYTES, Xp, kb0, kb1, active, lds);
+#ifndef RD_STREAM_PF
+#define RD_STREAM_PF 3
+#endif
+    const int ltile = active ? tile : (N >> 5) - 1;
+    gemm_mainloop<T, WPB, RD_STREAM_PF>(acc, Wt + (size_t)ltile * nKB * T::TILE_BYTES, Xp, kb0, kb1, active, lds);
     if (active && kb0 < kb1) {
         T::finish(acc, aux, tile, lane);
         float *out = P + (size_t)split * 32 * N + tile * 32 + (lane & 31);
@@ -80,5 +94,60 @@ __device__ __forceinline__ void gemm_body(const uint8_t *__restrict__ Wt, const 
             int m = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
             if (m < M) out[(size_t)m * N] = acc[r];
         }
+    }
+}
+
+// The resident-panel variant: the block first brings the NP activation panels of its K range into LDS (one barrier), then
+// every wave streams its weight tiles with PF tiles in flight and no further synchronisation. It is the right shape when a
+// GEMM has too few blocks to hide a per-K-block barrier behind other blocks (the decode projections: a few MB each).
+// Same per-element reduction order as the streaming variant within a split.
+template <class T, int WPB, int NP, int PF>
+__device__ __forceinline__ void gemm_resident_body(const uint8_t *__restrict__ Wt, const void *__restrict__ aux, const uint8_t *__restrict__ Xp,
+                                                   float *__restrict__ P, int N, int nKB, int M, uint4_t *lds) {
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int tile = blockIdx.x * WPB + wave, split = blockIdx.y;
+    const int kb0 = split * NP, nk = min(NP, nKB - kb0);
+    const bool active = tile * 32 < N;
+    constexpr int PV = T::PANEL_VECS, NT = WPB * 64;
+    const uint8_t *wbase = Wt + ((size_t)tile * nKB + kb0) * T::TILE_BYTES;
+    typename T::Tile w[PF];
+#pragma unroll
+    for (int i = 0; i < PF; i++)
+        if (active && i < nk) T::load(w[i], wbase + (size_t)i * T::TILE_BYTES, lane);
+    {
+        const uint4_t *src = (const uint4_t *)Xp + (size_t)kb0 * PV;
+        const int total = nk * PV;
+        for (int base = 0; base < total; base += NT * 8) {
+            uint4_t r[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                int v = base + j * NT + tid;
+                if (v < total) r[j] = src[v];
+            }
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                int v = base + j * NT + tid;
+                if (v < total) lds[v] = r[j];
+            }
+        }
+    }
+    __syncthreads();
+    if (!active) return;
+    float16_t acc;
+#pragma unroll
+    for (int i = 0; i < 16; i++) acc[i] = 0.f;
+#pragma unroll
+    for (int i = 0; i < NP; i++) {
+        if (i < nk) {
+            T::mma(acc, w[i % PF], lds + i * PV, lane);
+            if (i + PF < nk) T::load(w[i % PF], wbase + (size_t)(i + PF) * T::TILE_BYTES, lane);
+        }
+    }
+    T::finish(acc, aux, tile, lane);
+    float *out = P + (size_t)split * 32 * N + tile * 32 + (lane & 31);
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        int m = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+        if (m < M) out[(size_t)m * N] = acc[r];
     }
 }

@@ -18,7 +18,8 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_gemm_w4a8_moe(const uint8
     const int tile = blockIdx.x * 4 + wave;
     const bool active = tile * 32 < N;
     float16_t acc;
-    gemm_mainloop<W4Traits, 4>(acc, Wt + (size_t)e * wStride + (size_t)tile * nKB * W4Traits::TILE_BYTES, Xp + (size_t)e * xpStride, 0, nKB, active,
+    const int ltile = active ? tile : (N >> 5) - 1;
+    gemm_mainloop<W4Traits, 4>(acc, Wt + (size_t)e * wStride + (size_t)ltile * nKB * W4Traits::TILE_BYTES, Xp + (size_t)e * xpStride, 0, nKB, active,
                                lds);
     if (!active) return;
 #pragma unroll

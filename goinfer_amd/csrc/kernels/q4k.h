@@ -50,6 +50,14 @@ extern "C" __global__ void rd_k_retile_q4k(const uint8_t *__restrict__ raw, uint
     *(uint4_t *)(dst + (size_t)t * 16) = *src;
 }
 
+// (a & b) | c in one VALU op. Both constants must sit in VGPRs: a VOP3 instruction on this ISA takes no literal and at
+// most one scalar operand, so the compiler otherwise emits v_and + v_or.
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t b, uint32_t c) {
+    uint32_t r;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
 struct Q4KTile {
     uint4_t hdr, q[4];
 };
@@ -65,7 +73,14 @@ __device__ __forceinline__ void q4k_tile_load(Q4KTile &w, const uint8_t *__restr
 // then one packed fma per pair yields the centred weight (q-8)*dsc rounded once. The per-sub-block constants
 // 8*dsc - dmin*m ride a 17th MFMA step against the per-group activation sums.
 __device__ __forceinline__ void q4k_tile_mma(float16_t &acc, const Q4KTile &w, const uint4_t *__restrict__ panel, int lane) {
+#ifdef RD_DBG_NO_MMA // measurement builds only: keep the loads alive, skip the arithmetic
+    uint32_t f = w.hdr.x ^ w.hdr.y ^ w.hdr.z ^ w.hdr.w;
+    for (int c = 0; c < 4; c++) f ^= w.q[c].x ^ w.q[c].y ^ w.q[c].z ^ w.q[c].w;
+    acc[0] += __uint_as_float(f & 0x3fffffffu) + __uint_as_float(panel[lane].x & 0x3fffffffu);
+    return;
+#endif
     const int h = lane >> 5;
+    const uint32_t mask_lo = 0x000F000Fu, mask_hi = 0x00F000F0u, magic_lo = 0x64006400u, magic_hi = 0x54005400u;
     uint32_t y = w.hdr.y, z = w.hdr.z, x = w.hdr.w;
     half2_t dd;
     uint32_t hx = w.hdr.x;
@@ -97,8 +112,8 @@ __device__ __forceinline__ void q4k_tile_mma(float16_t &acc, const Q4KTile &w, c
         uint32_t wd = w.q[s >> 2][s & 3];
         const int pp = s >> 3;
         uint32_t t8 = wd >> 8;
-        uint32_t u0 = (wd & 0x000F000Fu) | 0x64006400u, u1 = (wd & 0x00F000F0u) | 0x54005400u;
-        uint32_t u2 = (t8 & 0x000F000Fu) | 0x64006400u, u3 = (t8 & 0x00F000F0u) | 0x54005400u;
+        uint32_t u0 = and_or(wd, mask_lo, magic_lo), u1 = and_or(wd, mask_hi, magic_hi);
+        uint32_t u2 = and_or(t8, mask_lo, magic_lo), u3 = and_or(t8, mask_hi, magic_hi);
         half2_t v0, v1, v2, v3;
         __builtin_memcpy(&v0, &u0, 4);
         __builtin_memcpy(&v1, &u1, 4);
@@ -143,4 +158,62 @@ extern "C" __global__ __launch_bounds__(128) void rd_k_gemm_q4k_w2(const uint8_t
                                                                     float *__restrict__ P, int N, int nSB, int sbPerSplit, int M) {
     __shared__ uint4_t lds[2 * RD_Q4K_PANEL_BYTES / 16];
     gemm_body<Q4KTraits, 2>(Wt, nullptr, Xp, P, N, nSB, sbPerSplit, M, lds);
+}
+
+#define RD_Q4K_RESIDENT(NAME, WPB, NP, PF)                                                                                                     \
+    extern "C" __global__ __launch_bounds__(WPB * 64) void NAME(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ Xp,               \
+                                                                 float *__restrict__ P, int N, int nSB, int M) {                              \
+        __shared__ uint4_t lds[NP * RD_Q4K_PANEL_BYTES / 16];                                                                                  \
+        gemm_resident_body<Q4KTraits, WPB, NP, PF>(Wt, nullptr, Xp, P, N, nSB, M, lds);                                                        \
+    }
+RD_Q4K_RESIDENT(rd_k_gemm_q4k_r4x8, 4, 8, 4)
+RD_Q4K_RESIDENT(rd_k_gemm_q4k_r4x4, 4, 4, 4)
+RD_Q4K_RESIDENT(rd_k_gemm_q4k_r4x2, 4, 2, 2)
+RD_Q4K_RESIDENT(rd_k_gemm_q4k_r2x4, 2, 4, 4)
+RD_Q4K_RESIDENT(rd_k_gemm_q4k_r2x8, 2, 8, 4)
+RD_Q4K_RESIDENT(rd_k_gemm_q4k_r8x4, 8, 4, 3)
+
+// Fused gate/up projection + SwiGLU + per-32 quantization (goinfer decoder/cpu_gateup_fused.go:83-148, in one launch):
+// W holds [gate rows; up rows] (2*I rows). Block b: waves 0,1 own gate tiles 2b,2b+1, waves 2,3 the matching up tiles, all over
+// the full K (no split, so the sums are complete in registers). The up waves hand their sums over through LDS; the gate waves
+// compute silu(gate)*up (silu in f64, decoder/rmsnorm.go:204-207), quantize each row's 32 columns (one activation group) and write
+// the f16 panels the down projection reads. Grid (I/64), block 256.
+extern "C" __global__ __launch_bounds__(256) void rd_k_gemm_q4k_gateup(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ Xp,
+                                                                        uint8_t *__restrict__ XpOut, int outKind, int I, int nSB, int M) {
+    __shared__ uint4_t lds[2 * RD_Q4K_PANEL_BYTES / 16];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int isUp = wave >> 1, t = blockIdx.x * 2 + (wave & 1), nGate = I >> 5;
+    const int tile = isUp * nGate + t;
+    const bool active = t < nGate;
+    float16_t acc;
+    const int ltile = active ? tile : nGate - 1;
+    gemm_mainloop<Q4KTraits, 4, 3>(acc, Wt + (size_t)ltile * nSB * RD_Q4K_TILE_BYTES, Xp, 0, nSB, active, lds);
+    float *xch = (float *)lds; // [2 waves][16][64] floats = 8 KB, free after the main loop's last barrier
+    if (isUp) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) xch[((wave & 1) * 16 + r) * 64 + lane] = acc[r];
+    }
+    __syncthreads();
+    if (isUp || !active) return;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const int m = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+        float u = xch[((wave & 1) * 16 + r) * 64 + lane];
+        double g64 = (double)acc[r];
+        float a = __fmul_rn((float)(g64 / (1.0 + exp(-g64))), u);
+        float gs, xh = quant_g32(a, &gs);
+        if (m < M) {
+            int k = t * 32 + (lane & 31);
+            half_t *base = (half_t *)(XpOut + (size_t)(k >> 8) * RD_Q4K_PANEL_BYTES);
+            if (outKind == 0) {
+                int tt = k & 255, j = tt >> 5;
+                base[q4k_panel_index(tt, m)] = (half_t)xh;
+                if ((tt & 31) == 0) base[q4k_panel_sum_index(j, m)] = (half_t)gs;
+                if ((tt & 31) == 1) base[q4k_panel_sum_index(j, m) + 4] = (half_t)0.f;
+            } else {
+                half_t *b2 = (half_t *)(XpOut + (size_t)(k >> 7) * RD_LIN_PANEL_BYTES);
+                b2[outKind == 1 ? lin_panel_index(k & 127, m) : lin4_panel_index(k & 127, m)] = (half_t)xh;
+            }
+        }
+    }
 }

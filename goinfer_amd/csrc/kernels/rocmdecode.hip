@@ -20,3 +20,4 @@ extern "C" __global__ void rd_k_attn_combine_quant(const float *__restrict__ par
     quant_g32x4(v[0], v[1], v[2], v[3], &x0, &x1, &x2, &x3, &gs);
     panel_store4(Xp, kind, m, head * HD + d0, x0, x1, x2, x3, gs);
 }
+
