@@ -92,19 +92,6 @@ def test_gemm_w4a8(dev, M, N, K):
     assert rel_err(dev.gemm_w4a8(nib, s16, K, a), ref64) < 2e-3
 
 
-def test_synth_quantizers_follow_reference_rules():
-    """The synthetic int8/int4 weights obey the reference's quantization rule bit for bit (oracle pinned by fingerprints)."""
-    N, K = 8, 256
-    w = synth.normal(5, N * K, 0.02).reshape(N, K)
-    q, s = synth.w8a8_normal(5, N, K)
-    q2, s2 = ob.quantize_rows_int8(w)
-    assert np.array_equal(q, q2) and np.array_equal(s, s2)
-    w = synth.normal(8, N * K, 0.02).reshape(N, K)
-    nib, s16 = synth.w4a8_normal(8, N, K)
-    n2, t2 = ob.quantize_int4(w)
-    assert np.array_equal(nib, n2) and np.array_equal(s16, t2)
-
-
 def test_rmsnorm_rope_route(dev):
     x = synth.normal(1, 5 * 4096).reshape(5, 4096)
     w = synth.normal(2, 4096, 0.02, 1.0)
