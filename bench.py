@@ -155,6 +155,11 @@ def main():
                 "algorithmic_bytes_per_launch": int(kv_launch + q_launch)}
     classes = {k: {"ms_per_step": round(v[0] / 3, 4), "launches_per_step": v[1] // 3} for k, v in prof.items()}
 
+    # ---- a plain copy kernel of known size: the practical HBM rate, and the yardstick the traffic counters are scaled by ----
+    COPY_BYTES = 1 << 30
+    cms = dev.bench_kernel("copy", [COPY_BYTES], 2, 6)
+    copy_gbs = 2 * COPY_BYTES / (float(np.median(cms)) / 1e3) / 1e9
+
     cpu = None
     if not args.no_cpu:
         threads = min(16, len(os.sched_getaffinity(0)))
@@ -175,6 +180,7 @@ def main():
         "step_hbm": {"algorithmic_bytes_per_step": int(step_bytes), "achieved_GBs": round(step_gbs, 1), "frac_of_peak": round(step_gbs / HBM_PEAK_GBS, 4),
                      "weights_bytes": int(w_bytes), "kv_read_bytes": int(kv_read)},
         "roofline": roofline,
+        "copy_kernel": {"bytes_read": COPY_BYTES, "bytes_written": COPY_BYTES, "GBs": round(copy_gbs, 1)},
         "kernel_classes": classes,
         "cpu_baseline": cpu,
     }

@@ -76,20 +76,25 @@ extern "C" const char *rd_bench_class_name(int c) {
 // Kernel micro-benchmarks over resident synthetic operands.
 //   "gemm_q4k"  args {N, K, M, copies}: dst = a . W^T on `copies` distinct weight copies used round-robin (so the 256 MB
 //               Infinity Cache cannot hold the weights between launches); operands are random bytes with sane f16 scales.
-//   "copy"      args {bytes}: device-to-device copy kernel-free baseline (hipMemcpyAsync), for calibrating counters.
+//   "copy"      args {bytes}: a plain 16-byte-per-lane copy kernel over `bytes` (a multiple of 16), the yardstick for
+//               scaling hardware traffic counters and for the practical HBM rate.
 // ms_out[iters]: per-launch milliseconds (HIP events on the launch stream).
 extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *args, int n_args, int warmup, int iters, float *ms_out) {
     if (!d || !name || !args || iters <= 0 || !ms_out) return RD_ERR_ARG;
     std::string nm(name);
+    if (nm == "gemm_q4k" && n_args >= 4 && (args[0] % 32 || args[1] % 256 || args[0] <= 0 || args[1] <= 0 || args[2] < 1 || args[2] > 32)) {
+        rd_set_error("gemm_q4k bench: bad shape");
+        return RD_ERR_ARG;
+    }
+    if (nm == "copy" && n_args >= 1 && (args[0] <= 0 || args[0] % 16)) {
+        rd_set_error("copy bench: bytes must be a positive multiple of 16");
+        return RD_ERR_ARG;
+    }
     std::vector<hipEvent_t> ev((size_t)iters * 2);
     for (auto &e : ev) HIPCHK(EventCreate(&e));
     int rc = RD_OK;
     if (nm == "gemm_q4k" && n_args >= 4) {
         int N = (int)args[0], K = (int)args[1], M = (int)args[2], copies = (int)std::max<int64_t>(1, args[3]);
-        if (N % 32 || K % 256 || M < 1 || M > 32) {
-            rd_set_error("gemm_q4k bench: bad shape");
-            return RD_ERR_ARG;
-        }
         size_t bytes = (size_t)N * (K / 256) * 144;
         std::vector<uint8_t> raw(bytes);
         uint64_t s = 88172645463325252ULL;
@@ -129,7 +134,7 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
         if (!rc) rc = rd_hip_ok(d->hip, d->hip->MemsetAsync(A.p, 1, bytes, d->stream), "memset") ? RD_OK : RD_ERR_HIP;
         for (int i = 0; i < warmup + iters && !rc; i++) {
             if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup)], d->stream);
-            rc = rd_hip_ok(d->hip, d->hip->MemcpyAsync(Bf.p, A.p, bytes, hipMemcpyDeviceToDevice, d->stream), "copy") ? RD_OK : RD_ERR_HIP;
+            rc = d->launch(d->k.copy16, 4096, 1, 1, 256, (const void *)A.p, Bf.p, (size_t)(bytes / 16));
             if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup) + 1], d->stream);
         }
         if (!rc) rc = d->sync();

@@ -96,6 +96,7 @@ static const KName kNames[] = {
     {"rd_k_moe_swiglu_quant", &Kernels::moe_swiglu_quant},
     {"rd_k_moe_fold", &Kernels::moe_fold},
     {"rd_k_embed_rows", &Kernels::embed_rows},
+    {"rd_k_copy16", &Kernels::copy16},
 };
 
 int load_resident_variants(rd_device *d);

@@ -26,7 +26,7 @@ struct Kernels {
     hipFunction_t gemm_q4k_gateup;
     hipFunction_t gemm_q4k_r[6]; // resident-panel variants, see kResident in device.cc
     hipFunction_t kv_store, qkv_rope_store, attn_partial, attn_combine, attn_combine_quant;
-    hipFunction_t rmsnorm, rope, argmax_rows, argmax_final, matmul_f32, moe_route, gemm_w4a8_moe, moe_swiglu_quant, moe_fold, embed_rows;
+    hipFunction_t rmsnorm, rope, argmax_rows, argmax_final, matmul_f32, moe_route, gemm_w4a8_moe, moe_swiglu_quant, moe_fold, embed_rows, copy16;
 };
 
 struct rd_device {

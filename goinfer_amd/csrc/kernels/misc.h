@@ -151,3 +151,8 @@ extern "C" __global__ void rd_k_embed_rows(const signed char *__restrict__ q, co
     float sc = scale[id];
     for (int k = threadIdx.x; k < H; k += blockDim.x) h[(size_t)m * H + k] = __fmul_rn((float)q[(size_t)id * H + k], sc);
 }
+
+// Plain copy of n16 16-byte words (grid-stride). A traffic yardstick of known size: n16*16 bytes read, n16*16 written.
+extern "C" __global__ void rd_k_copy16(const uint4 *__restrict__ src, uint4 *__restrict__ dst, size_t n16) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x) dst[i] = src[i];
+}
