@@ -76,6 +76,8 @@ extern "C" const char *rd_bench_class_name(int c) {
 // Kernel micro-benchmarks over resident synthetic operands.
 //   "gemm_q4k"  args {N, K, M, copies}: dst = a . W^T on `copies` distinct weight copies used round-robin (so the 256 MB
 //               Infinity Cache cannot hold the weights between launches); operands are random bytes with sane f16 scales.
+//   "gateup"    args {I, K, M, copies}: the fused gate|up projection + SwiGLU + quantization kernel.
+//   "barrier"   args {blocks, words, rounds, shift}: the grid-wide barrier with a cross-block data hand-off per round.
 //   "copy"      args {bytes}: a plain 16-byte-per-lane copy kernel over `bytes` (a multiple of 16), the yardstick for
 //               scaling hardware traffic counters and for the practical HBM rate.
 // ms_out[iters]: per-launch milliseconds (HIP events on the launch stream).
@@ -84,6 +86,14 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
     std::string nm(name);
     if (nm == "gemm_q4k" && n_args >= 4 && (args[0] % 32 || args[1] % 256 || args[0] <= 0 || args[1] <= 0 || args[2] < 1 || args[2] > 32)) {
         rd_set_error("gemm_q4k bench: bad shape");
+        return RD_ERR_ARG;
+    }
+    if (nm == "gateup" && n_args >= 4 && (args[0] <= 0 || args[0] % 64 || args[1] <= 0 || args[1] % 256 || args[2] < 1 || args[2] > 32)) {
+        rd_set_error("gateup bench: bad shape");
+        return RD_ERR_ARG;
+    }
+    if (nm == "barrier" && n_args >= 4 && (args[0] < 1 || args[0] > 256 || args[1] < 1 || args[1] > (1 << 20) || args[2] < 1 || args[2] > 100000)) {
+        rd_set_error("barrier bench: blocks 1..256, words 1..2^20, rounds 1..100000");
         return RD_ERR_ARG;
     }
     if (nm == "copy" && n_args >= 1 && (args[0] <= 0 || args[0] % 16)) {
@@ -126,6 +136,69 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
         }
         if (!rc) rc = d->sync();
         for (auto &w : ws) free_weight(d, &w);
+    } else if (nm == "gateup" && n_args >= 4) {
+        // args {I, K, M, copies}: the fused gate|up + SwiGLU + quantization kernel on `copies` weight sets used round-robin
+        int I = (int)args[0], K = (int)args[1], M = (int)args[2], copies = (int)std::max<int64_t>(1, args[3]);
+        size_t bytes = (size_t)2 * I * (K / 256) * 144;
+        std::vector<uint8_t> raw(bytes);
+        uint64_t s = 88172645463325252ULL;
+        for (size_t i = 0; i < bytes; i++) {
+            s ^= s << 13, s ^= s >> 7, s ^= s << 17;
+            raw[i] = (uint8_t)s;
+        }
+        for (size_t b = 0; b < bytes / 144; b++) raw[b * 144 + 1] = 0x10 | (raw[b * 144 + 1] & 3), raw[b * 144 + 3] = 0x10 | (raw[b * 144 + 3] & 3);
+        std::vector<DevWeight> ws((size_t)copies);
+        for (auto &w : ws)
+            if (!rc) rc = upload_q4k(d, raw.data(), 2 * I, K, &w);
+        DevBuf Xp(d), Xo(d);
+        size_t pb = (size_t)(K / 256) * Q4K_PANEL_BYTES;
+        if (!rc) rc = Xp.alloc(pb);
+        if (!rc) rc = Xo.alloc((size_t)((I + 255) / 256) * Q4K_PANEL_BYTES);
+        if (!rc) {
+            std::vector<uint16_t> x(pb / 2);
+            for (size_t i = 0; i < x.size(); i++) x[i] = (uint16_t)(0x3000 + (i * 2654435761u >> 22 & 0x3ff)) | (uint16_t)((i & 1) << 15);
+            rc = d->h2d(Xp.p, x.data(), pb);
+        }
+        if (!rc) rc = d->sync();
+        for (int i = 0; i < warmup + iters && !rc; i++) {
+            const DevWeight &w = ws[(size_t)i % ws.size()];
+            if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup)], d->stream);
+            rc = d->launch(d->k.gemm_q4k_gateup, (unsigned)(I / 64), 1, 1, 512, (const void *)w.tiled, (const void *)Xp.p, Xo.as<uint8_t>(), (int)PANEL_Q4K,
+                           I, K / 256, M);
+            if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup) + 1], d->stream);
+        }
+        if (!rc) rc = d->sync();
+        for (auto &w : ws) free_weight(d, &w);
+    } else if (nm == "barrier" && n_args >= 4) {
+        // args {blocks, words, rounds, shift}: the grid barrier's cost and its cross-block hand-off; ms_out per launch, and the launch
+        // fails with RD_ERR_STATE if a hand-off delivered stale data or the barrier gave up
+        int blocks = (int)args[0], words = (int)args[1], rounds = (int)args[2], shift = (int)args[3];
+        DevBuf ctr(d), buf(d), out(d);
+        rc = ctr.alloc(256);
+        if (!rc) rc = buf.alloc(sizeof(float) * (size_t)blocks * words);
+        if (!rc) rc = out.alloc(sizeof(int) * (size_t)blocks);
+        for (int i = 0; i < warmup + iters && !rc; i++) {
+            rc = rd_hip_ok(d->hip, d->hip->MemsetAsync(ctr.p, 0, 256, d->stream), "memset") ? RD_OK : RD_ERR_HIP;
+            if (!rc) rc = rd_hip_ok(d->hip, d->hip->MemsetAsync(out.p, 0, sizeof(int) * (size_t)blocks, d->stream), "memset") ? RD_OK : RD_ERR_HIP;
+            if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup)], d->stream);
+            if (!rc)
+                rc = d->launch(d->k.barrier_probe, (unsigned)blocks, 1, 1, 256, ctr.as<unsigned>(), ctr.as<unsigned>() + 32, buf.as<float>(), words, rounds,
+                               shift, 200000u, out.as<int>());
+            if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup) + 1], d->stream);
+        }
+        if (!rc) rc = d->sync();
+        if (!rc) {
+            std::vector<int> h((size_t)blocks);
+            unsigned flag[64];
+            rc = d->d2h(h.data(), out.p, sizeof(int) * (size_t)blocks);
+            if (!rc) rc = d->d2h(flag, ctr.p, 256);
+            long bad = 0;
+            for (int v : h) bad += v;
+            if (!rc && (bad || flag[32])) {
+                rd_set_error("barrier probe: %ld stale hand-offs, abort flag %u", bad, flag[32]);
+                rc = RD_ERR_STATE;
+            }
+        }
     } else if (nm == "copy" && n_args >= 1) {
         size_t bytes = (size_t)args[0];
         DevBuf A(d), Bf(d);

@@ -72,6 +72,7 @@ static const KName kNames[] = {
     {"rd_k_retile_q4k", &Kernels::retile_q4k},
     {"rd_k_gemm_q4k_w4", &Kernels::gemm_q4k_w4},
     {"rd_k_gemm_q4k_w2", &Kernels::gemm_q4k_w2},
+    {"rd_k_gemm_q4k_k2", &Kernels::gemm_q4k_k2},
     {"rd_k_gemm_q4k_gateup", &Kernels::gemm_q4k_gateup},
     {"rd_k_quant_act", &Kernels::quant_act},
     {"rd_k_reduce_splits", &Kernels::reduce_splits},
@@ -97,6 +98,7 @@ static const KName kNames[] = {
     {"rd_k_moe_fold", &Kernels::moe_fold},
     {"rd_k_embed_rows", &Kernels::embed_rows},
     {"rd_k_copy16", &Kernels::copy16},
+    {"rd_k_barrier_probe", &Kernels::barrier_probe},
 };
 
 int load_resident_variants(rd_device *d);
@@ -216,6 +218,11 @@ static GemmPlan streaming_plan(int N, int nKB) {
 // one block per CU with the fewest K splits (each split costs a partial-sum round trip). Huge-N matrices (an LM head) have
 // thousands of blocks anyway and stream with the double-buffered kernel.
 GemmPlan plan_gemm(int kind, int N, int nKB) {
+    if (kind == 0 && getenv("ROCMDECODE_K2")) {
+        GemmPlan p = streaming_plan(N, nKB);
+        p.kgroups = 2;
+        return p;
+    }
     if (kind != 0 || getenv("ROCMDECODE_SPLITS")) return streaming_plan(N, nKB);
     int pick = -1;
     if (const char *e = getenv("ROCMDECODE_GEMM")) {
@@ -313,6 +320,8 @@ int launch_gemm(rd_device *d, const DevWeight &w, const void *Xp, float *P, int 
     unsigned gx = (unsigned)((w.N + 32 * p.wpb - 1) / (32 * p.wpb));
     if (p.variant >= 0)
         return d->launch(d->k.gemm_q4k_r[p.variant], gx, p.splits, 1, (unsigned)(64 * p.wpb), (const void *)w.tiled, Xp, P, w.N, nKB, M);
+    if (w.kind == 0 && p.kgroups == 2)
+        return d->launch(d->k.gemm_q4k_k2, gx, p.splits, 1, 512, (const void *)w.tiled, Xp, P, w.N, nKB, p.kbPerSplit, M);
     if (w.kind == 0)
         return d->launch(d->k.gemm_q4k_w4, gx, p.splits, 1, 256, (const void *)w.tiled, Xp, P, w.N, nKB, p.kbPerSplit, M);
     if (w.kind == 1)

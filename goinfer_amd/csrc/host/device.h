@@ -21,12 +21,12 @@ constexpr size_t Q4K_TILE_BYTES = 4608;
 enum { PANEL_Q4K = 0, PANEL_LIN = 1, PANEL_LIN4 = 2 };
 
 struct Kernels {
-    hipFunction_t dequant_q4k, retile_q4k, gemm_q4k_w4, gemm_q4k_w2, quant_act, reduce_splits, add_rmsnorm_quant, swiglu_quant;
+    hipFunction_t dequant_q4k, retile_q4k, gemm_q4k_w4, gemm_q4k_w2, gemm_q4k_k2, quant_act, reduce_splits, add_rmsnorm_quant, swiglu_quant;
     hipFunction_t retile_w8a8, gemm_w8a8, retile_w4a8, gemm_w4a8;
     hipFunction_t gemm_q4k_gateup;
     hipFunction_t gemm_q4k_r[6]; // resident-panel variants, see kResident in device.cc
     hipFunction_t kv_store, qkv_rope_store, attn_partial, attn_combine, attn_combine_quant;
-    hipFunction_t rmsnorm, rope, argmax_rows, argmax_final, matmul_f32, moe_route, gemm_w4a8_moe, moe_swiglu_quant, moe_fold, embed_rows, copy16;
+    hipFunction_t rmsnorm, rope, argmax_rows, argmax_final, matmul_f32, moe_route, gemm_w4a8_moe, moe_swiglu_quant, moe_fold, embed_rows, copy16, barrier_probe;
 };
 
 struct rd_device {
@@ -67,6 +67,7 @@ struct GemmPlan {
     int wpb;        // waves per block (32 weight rows each)
     int splits;     // grid.y
     int kbPerSplit; // K-blocks (super-blocks or 128-wide blocks) per split
+    int kgroups = 1; // waves sharing one tile's K range inside a block (Q4_K only)
 };
 GemmPlan plan_gemm(int kind, int N, int nKB);
 

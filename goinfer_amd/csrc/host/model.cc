@@ -597,7 +597,7 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
             RC(add_norm_quant(m, B, m->P, plan.splits, l.ffn_norm, l.gateup, m->XpA, nullptr));
             if (l.gateup.kind == 0 && c.inter % 64 == 0 && !getenv("ROCMDECODE_NO_FUSED_GATEUP")) {
                 Scope s(m, KC_GEMM_GATEUP); // gate|up GEMM + SwiGLU + quantization in one launch
-                RC(d->launch(d->k.gemm_q4k_gateup, (unsigned)(c.inter / 64), 1, 1, 256, (const void *)l.gateup.tiled, (const void *)m->XpA, m->XpB,
+                RC(d->launch(d->k.gemm_q4k_gateup, (unsigned)(c.inter / 64), 1, 1, 512, (const void *)l.gateup.tiled, (const void *)m->XpA, m->XpB,
                              panel_kind_for(l.down), c.inter, H / 256, B));
             } else {
                 {

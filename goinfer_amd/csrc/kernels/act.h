@@ -156,8 +156,7 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_swiglu_quant(const float 
         }
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            double g64 = (double)g[i];
-            a[i] = __fmul_rn((float)(g64 / (1.0 + exp(-g64))), u[i]);
+            a[i] = __fmul_rn(silu_f64(g[i]), u[i]);
         }
         if (act_out) *(float4_t *)(act_out + (size_t)m * I + n0) = (float4_t){a[0], a[1], a[2], a[3]};
     }

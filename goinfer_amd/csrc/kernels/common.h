@@ -86,6 +86,41 @@ __device__ __forceinline__ float quant_g32(float v, float *gsum) {
     return __fmul_rn((float)code, sc);
 }
 
+// silu(g) = f32(g64 / (1 + exp(-g64))), evaluated in f64 as goinfer does (decoder/rmsnorm.go:204-207). exp by range
+// reduction and a degree-13 Taylor polynomial on |r| <= ln2/2 (remainder < 1e-17), the quotient by a Newton-refined
+// reciprocal with one residual correction: the f64 value is within an ulp or two of the correctly rounded one, so the f32
+// result differs from a libm evaluation only if it lies within ~1e-15 (relative) of an f32 rounding boundary. An order of
+// magnitude fewer f64 instructions than exp() and an IEEE division. Huge magnitudes, inf and NaN take the library path.
+__device__ __forceinline__ float silu_f64(float g) {
+    const double g64 = (double)g;
+    if (!(fabsf(g) <= 80.f)) return (float)(g64 / (1.0 + exp(-g64)));
+    const double x = -g64;
+    const double n = rint(x * 1.44269504088896338700e+00);
+    double r = fma(n, -6.93147180369123816490e-01, x);
+    r = fma(n, -1.90821492927058770002e-10, r);
+    double p = 1.0 / 6227020800.0;
+    p = fma(p, r, 1.0 / 479001600.0);
+    p = fma(p, r, 1.0 / 39916800.0);
+    p = fma(p, r, 1.0 / 3628800.0);
+    p = fma(p, r, 1.0 / 362880.0);
+    p = fma(p, r, 1.0 / 40320.0);
+    p = fma(p, r, 1.0 / 5040.0);
+    p = fma(p, r, 1.0 / 720.0);
+    p = fma(p, r, 1.0 / 120.0);
+    p = fma(p, r, 1.0 / 24.0);
+    p = fma(p, r, 1.0 / 6.0);
+    p = fma(p, r, 0.5);
+    p = fma(p, r, 1.0);
+    p = fma(p, r, 1.0);
+    const double d = 1.0 + ldexp(p, (int)n);
+    double y = __builtin_amdgcn_rcp(d);
+    y = fma(fma(-d, y, 1.0), y, y);
+    y = fma(fma(-d, y, 1.0), y, y);
+    double q = g64 * y;
+    q = fma(fma(-d, q, g64), y, q);
+    return (float)q;
+}
+
 // Where element t (0..255) of a super-block goes inside a Q4_K activation panel, for batch row m.
 // Sub-block j=t/32 belongs to nibble pair p=j/2; lane half h=p/2 owns pairs 2h,2h+1; its 16 code words are the
 // 16 MFMA steps. Word s holds bytes e0..e0+3 (e0=4*(s%8)): the unpack yields

@@ -73,6 +73,120 @@ __device__ __forceinline__ void gemm_mainloop(float16_t &acc, const uint8_t *__r
         if (it + 2 < nk) body(it + 2, std::integral_constant<int, 2>{});
 }
 
+// The K-group main loop: a block of TPB*KG waves; wave w owns tile (w % TPB) and K-group (w / TPB). The block's K range
+// [kb0,kb1) is cut into KG contiguous runs of `per` K-blocks; each group streams its own run with its own double-buffered
+// panel in LDS (lds holds KG*2*PANEL_VECS vectors), all groups share the block barrier. Twice the waves per tile means
+// twice the weight bytes in flight per CU — what the HBM latency-bandwidth product asks for — at an unchanged grid.
+// A group whose run is shorter than `per` keeps loading (clamped) but skips the arithmetic. acc holds the group's partial
+// sum; the caller folds the groups in ascending order (gemm_fold_groups), so the order is fixed and independent of M.
+template <class T, int TPB, int KG, int PF = 3>
+__device__ __forceinline__ void gemm_mainloop_kg(float16_t &acc, const uint8_t *__restrict__ wbase, const uint8_t *__restrict__ Xp, int kb0, int kb1,
+                                                 uint4_t *lds_all) {
+    const int tid = threadIdx.x, lane = tid & 63, g = (tid >> 6) / TPB;
+    constexpr int PV = T::PANEL_VECS;
+    constexpr int NT = TPB * 64; // threads of one group
+    constexpr int PER = (PV + NT - 1) / NT;
+    const int gtid = tid - g * NT;
+    uint4_t *lds = lds_all + g * 2 * PV;
+#pragma unroll
+    for (int i = 0; i < 16; i++) acc[i] = 0.f;
+    const int nkAll = kb1 - kb0;
+    if (nkAll <= 0) return;
+    const int per = (nkAll + KG - 1) / KG; // block-uniform iteration count
+    const int s0 = min(kb0 + g * per, kb1 - 1);
+    const int nk = max(0, min(kb1, kb0 + g * per + per) - (kb0 + g * per));
+    const int last = max(nk - 1, 0);
+    const uint8_t *wb = wbase + (size_t)s0 * T::TILE_BYTES;
+    const uint4_t *src = (const uint4_t *)Xp + (size_t)s0 * PV;
+    int pv[PER];
+#pragma unroll
+    for (int i = 0; i < PER; i++) pv[i] = min(gtid + i * NT, PV - 1);
+
+    typename T::Tile w[PF];
+#pragma unroll
+    for (int i = 0; i < PF; i++) T::load(w[i], wb + (size_t)min(i, last) * T::TILE_BYTES, lane);
+    uint4_t stage[PER];
+#pragma unroll
+    for (int i = 0; i < PER; i++) lds[pv[i]] = src[pv[i]];
+#pragma unroll
+    for (int i = 0; i < PER; i++) stage[i] = src[(size_t)min(1, last) * PV + pv[i]];
+    __syncthreads();
+
+    auto body = [&](int it, auto uc) {
+        constexpr int u = decltype(uc)::value;
+        const int cur = it & 1;
+        uint4_t *dst = lds + (cur ^ 1) * PV;
+#ifndef RD_DBG_NO_PANEL
+#pragma unroll
+        for (int i = 0; i < PER; i++) dst[pv[i]] = stage[i];
+        const uint4_t *s2 = src + (size_t)min(it + 2, last) * PV;
+#pragma unroll
+        for (int i = 0; i < PER; i++) stage[i] = s2[pv[i]];
+#endif
+        if (it < nk) T::mma(acc, w[u], lds + cur * PV, lane);
+        T::load(w[u], wb + (size_t)min(it + PF, last) * T::TILE_BYTES, lane);
+#ifndef RD_DBG_NO_BARRIER
+        __syncthreads();
+#endif
+    };
+    int it = 0;
+    for (; it + PF <= per; it += PF) {
+        if constexpr (PF > 0) body(it + 0, std::integral_constant<int, 0>{});
+        if constexpr (PF > 1) body(it + 1, std::integral_constant<int, 1>{});
+        if constexpr (PF > 2) body(it + 2, std::integral_constant<int, 2>{});
+        if constexpr (PF > 3) body(it + 3, std::integral_constant<int, 3>{});
+    }
+    if constexpr (PF > 1)
+        if (it + 0 < per) body(it + 0, std::integral_constant<int, 0>{});
+    if constexpr (PF > 2)
+        if (it + 1 < per) body(it + 1, std::integral_constant<int, 1>{});
+    if constexpr (PF > 3)
+        if (it + 2 < per) body(it + 2, std::integral_constant<int, 2>{});
+}
+
+// Folds the K-groups' partial sums into group 0's registers in ascending group order through LDS (xch: (KG-1)*TPB*1024
+// floats, may alias the panel buffers: the main loop ends on a barrier). Every wave of the block must call it.
+template <int TPB, int KG>
+__device__ __forceinline__ void gemm_fold_groups(float16_t &acc, float *xch) {
+    if constexpr (KG > 1) {
+        const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = wave / TPB, t = wave % TPB;
+        if (g > 0) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) xch[(((g - 1) * TPB + t) * 16 + r) * 64 + lane] = acc[r];
+        }
+        __syncthreads();
+        if (g == 0) {
+#pragma unroll
+            for (int gg = 1; gg < KG; gg++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[r] += xch[(((gg - 1) * TPB + t) * 16 + r) * 64 + lane];
+        }
+    }
+}
+
+// gemm_body with K-groups: grid (ceil(N/(32*TPB)), splits), block TPB*KG*64 threads.
+template <class T, int TPB, int KG, int PF>
+__device__ __forceinline__ void gemm_body_kg(const uint8_t *__restrict__ Wt, const void *__restrict__ aux, const uint8_t *__restrict__ Xp,
+                                             float *__restrict__ P, int N, int nKB, int kbPerSplit, int M, uint4_t *lds) {
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int tile = blockIdx.x * TPB + wave % TPB, split = blockIdx.y;
+    const int kb0 = split * kbPerSplit, kb1 = min(nKB, kb0 + kbPerSplit);
+    const bool active = tile * 32 < N;
+    float16_t acc;
+    const int ltile = active ? tile : (N >> 5) - 1;
+    gemm_mainloop_kg<T, TPB, KG, PF>(acc, Wt + (size_t)ltile * nKB * T::TILE_BYTES, Xp, kb0, kb1, lds);
+    gemm_fold_groups<TPB, KG>(acc, (float *)lds);
+    if (active && kb0 < kb1 && wave < TPB) {
+        T::finish(acc, aux, tile, lane);
+        float *out = P + (size_t)split * 32 * N + tile * 32 + (lane & 31);
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            int m = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+            if (m < M) out[(size_t)m * N] = acc[r];
+        }
+    }
+}
+
 template <class T, int WPB>
 __device__ __forceinline__ void gemm_body(const uint8_t *__restrict__ Wt, const void *__restrict__ aux, const uint8_t *__restrict__ Xp,
                                           float *__restrict__ P, int N, int nKB, int kbPerSplit, int M, uint4_t *lds) {

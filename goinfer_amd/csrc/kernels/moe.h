@@ -40,8 +40,7 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_moe_swiglu_quant(const fl
     float a = 0.f;
     if (n < I) {
         float g = gu[(size_t)row * 2 * I + n], u = gu[(size_t)row * 2 * I + I + n];
-        double g64 = (double)g;
-        a = __fmul_rn((float)(g64 / (1.0 + exp(-g64))), u);
+        a = __fmul_rn(silu_f64(g), u);
     }
     float gs, xh = quant_g32(a, &gs);
     if (n < I) panel_store(XpE + (size_t)e * xpStride, RD_PANEL_LIN4, t, n, xh, gs);

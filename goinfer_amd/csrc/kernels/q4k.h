@@ -62,10 +62,15 @@ struct Q4KTile {
     uint4_t hdr, q[4];
 };
 
+#ifdef RD_DBG_NO_NT
+#define RD_WLOAD(p) (*(p))
+#else
+#define RD_WLOAD(p) __builtin_nontemporal_load(p)
+#endif
 __device__ __forceinline__ void q4k_tile_load(Q4KTile &w, const uint8_t *__restrict__ p, int lane) {
-    w.hdr = __builtin_nontemporal_load((const uint4_t *)(p + (lane & 31) * 16));
+    w.hdr = RD_WLOAD((const uint4_t *)(p + (lane & 31) * 16));
 #pragma unroll
-    for (int c = 0; c < 4; c++) w.q[c] = __builtin_nontemporal_load((const uint4_t *)(p + 512 + c * 1024 + lane * 16));
+    for (int c = 0; c < 4; c++) w.q[c] = RD_WLOAD((const uint4_t *)(p + 512 + c * 1024 + lane * 16));
 }
 
 // acc += panel(32 batch rows x 256 k) . tile(32 weight rows x 256 k)^T, f16 MFMA with f32 accumulation.
@@ -123,9 +128,19 @@ __device__ __forceinline__ void q4k_tile_mma(float16_t &acc, const Q4KTile &w, c
         v1 = __builtin_elementwise_fma(v1, DSC[2 * pp + 1], C0[2 * pp + 1]);
         v2 = __builtin_elementwise_fma(v2, DSC[2 * pp], C0[2 * pp]);
         v3 = __builtin_elementwise_fma(v3, DSC[2 * pp + 1], C0[2 * pp + 1]);
+#ifdef RD_DBG_NO_DEQUANT
+        uint4_t braw = {wd, t8, wd ^ x, t8 ^ y};
+        half8_t b;
+        __builtin_memcpy(&b, &braw, 16);
+#else
         half8_t b = {v0.x, v0.y, v1.x, v1.y, v2.x, v2.y, v3.x, v3.y};
+#endif
         half8_t a;
+#ifdef RD_DBG_NO_LDSREAD
+        uint4_t av = {wd, wd, wd, wd};
+#else
         uint4_t av = panel[s * 64 + lane];
+#endif
         __builtin_memcpy(&a, &av, 16);
         acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc, 0, 0, 0);
     }
@@ -177,43 +192,69 @@ RD_Q4K_RESIDENT(rd_k_gemm_q4k_r8x4, 8, 4, 3)
 // W holds [gate rows; up rows] (2*I rows). Block b: waves 0,1 own gate tiles 2b,2b+1, waves 2,3 the matching up tiles, all over
 // the full K (no split, so the sums are complete in registers). The up waves hand their sums over through LDS; the gate waves
 // compute silu(gate)*up (silu in f64, decoder/rmsnorm.go:204-207), quantize each row's 32 columns (one activation group) and write
-// the f16 panels the down projection reads. Grid (I/64), block 256.
-extern "C" __global__ __launch_bounds__(256) void rd_k_gemm_q4k_gateup(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ Xp,
-                                                                        uint8_t *__restrict__ XpOut, int outKind, int I, int nSB, int M) {
-    __shared__ uint4_t lds[2 * RD_Q4K_PANEL_BYTES / 16];
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const int isUp = wave >> 1, t = blockIdx.x * 2 + (wave & 1), nGate = I >> 5;
+// the f16 panels the down projection reads. Each tile's K range is shared by two waves (K-groups) whose partial sums are
+// folded in LDS first. Grid (I/64), block 512.
+template <int KG, int PF>
+__device__ __forceinline__ void q4k_gateup_body(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ Xp, uint8_t *__restrict__ XpOut,
+                                                int outKind, int I, int nSB, int M, uint4_t *lds) {
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, wt = wave & 3;
+    const int isUp = wt >> 1, t = blockIdx.x * 2 + (wt & 1), nGate = I >> 5;
     const int tile = isUp * nGate + t;
     const bool active = t < nGate;
     float16_t acc;
     const int ltile = active ? tile : nGate - 1;
-    gemm_mainloop<Q4KTraits, 4, 3>(acc, Wt + (size_t)ltile * nSB * RD_Q4K_TILE_BYTES, Xp, 0, nSB, active, lds);
-    float *xch = (float *)lds; // [2 waves][16][64] floats = 8 KB, free after the main loop's last barrier
-    if (isUp) {
+    gemm_mainloop_kg<Q4KTraits, 4, KG, PF>(acc, Wt + (size_t)ltile * nSB * RD_Q4K_TILE_BYTES, Xp, 0, nSB, lds);
+    gemm_fold_groups<4, KG>(acc, (float *)lds);
+#ifdef RD_DBG_NO_EPILOGUE
+    if (acc[3] == 1234.5f) XpOut[tid] = 1;
+    return;
+#endif
+    // Epilogue on all waves: the four complete tiles (gate t0,t1, up t0,t1) go to LDS as [tile][row m][column c]; then
+    // every thread takes elements (tile pair, m, c) with 32 consecutive lanes on one row's 32 columns = one activation group.
+    float *xe = (float *)lds + (KG - 1) * 4 * 1024; // 4 tiles x 32 x 32 floats past the fold area
+    if (wave < 4) {
 #pragma unroll
-        for (int r = 0; r < 16; r++) xch[((wave & 1) * 16 + r) * 64 + lane] = acc[r];
+        for (int r = 0; r < 16; r++) {
+            const int m = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+            xe[(wt * 32 + m) * 32 + (lane & 31)] = acc[r];
+        }
     }
     __syncthreads();
-    if (isUp || !active) return;
+    constexpr int NTHR = 4 * KG * 64;
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-        const int m = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-        float u = xch[((wave & 1) * 16 + r) * 64 + lane];
-        double g64 = (double)acc[r];
-        float a = __fmul_rn((float)(g64 / (1.0 + exp(-g64))), u);
+    for (int e = tid; e < 2048; e += NTHR) {
+        const int tl = e >> 10, m = (e >> 5) & 31, c = e & 31;
+        const int tt = blockIdx.x * 2 + tl;
+        float a = __fmul_rn(silu_f64(xe[(tl * 32 + m) * 32 + c]), xe[((2 + tl) * 32 + m) * 32 + c]);
         float gs, xh = quant_g32(a, &gs);
-        if (m < M) {
-            int k = t * 32 + (lane & 31);
+        if (m < M && tt < nGate) {
+            int k = tt * 32 + c;
             half_t *base = (half_t *)(XpOut + (size_t)(k >> 8) * RD_Q4K_PANEL_BYTES);
             if (outKind == 0) {
-                int tt = k & 255, j = tt >> 5;
-                base[q4k_panel_index(tt, m)] = (half_t)xh;
-                if ((tt & 31) == 0) base[q4k_panel_sum_index(j, m)] = (half_t)gs;
-                if ((tt & 31) == 1) base[q4k_panel_sum_index(j, m) + 4] = (half_t)0.f;
+                int t8 = k & 255, j = t8 >> 5;
+                base[q4k_panel_index(t8, m)] = (half_t)xh;
+                if (c == 0) base[q4k_panel_sum_index(j, m)] = (half_t)gs;
+                if (c == 1) base[q4k_panel_sum_index(j, m) + 4] = (half_t)0.f;
             } else {
                 half_t *b2 = (half_t *)(XpOut + (size_t)(k >> 7) * RD_LIN_PANEL_BYTES);
                 b2[outKind == 1 ? lin_panel_index(k & 127, m) : lin4_panel_index(k & 127, m)] = (half_t)xh;
             }
         }
     }
+}
+
+#ifndef RD_GATEUP_PF
+#define RD_GATEUP_PF 3
+#endif
+extern "C" __global__ __launch_bounds__(512) void rd_k_gemm_q4k_gateup(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ Xp,
+                                                                        uint8_t *__restrict__ XpOut, int outKind, int I, int nSB, int M) {
+    __shared__ uint4_t lds[2 * 2 * RD_Q4K_PANEL_BYTES / 16];
+    q4k_gateup_body<2, RD_GATEUP_PF>(Wt, Xp, XpOut, outKind, I, nSB, M, lds);
+}
+
+// The plain GEMM with two K-groups per block (8 waves): for launches whose grid cannot fill the chip with 4-wave blocks.
+extern "C" __global__ __launch_bounds__(512) void rd_k_gemm_q4k_k2(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ Xp,
+                                                                    float *__restrict__ P, int N, int nSB, int sbPerSplit, int M) {
+    __shared__ uint4_t lds[2 * 2 * RD_Q4K_PANEL_BYTES / 16];
+    gemm_body_kg<Q4KTraits, 4, 2, RD_GATEUP_PF>(Wt, nullptr, Xp, P, N, nSB, sbPerSplit, M, lds);
 }
