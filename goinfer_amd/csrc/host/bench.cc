@@ -163,7 +163,7 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
         for (int i = 0; i < warmup + iters && !rc; i++) {
             const DevWeight &w = ws[(size_t)i % ws.size()];
             if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup)], d->stream);
-            rc = d->launch(d->k.gemm_q4k_gateup, (unsigned)(I / 64), 1, 1, 512, (const void *)w.tiled, (const void *)Xp.p, Xo.as<uint8_t>(), (int)PANEL_Q4K,
+            rc = d->launch(d->k.gemm_q4k_gateup, (unsigned)(I / 64), 1, 1, GATEUP_THREADS, (const void *)w.tiled, (const void *)Xp.p, Xo.as<uint8_t>(), (int)PANEL_Q4K,
                            I, K / 256, M);
             if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup) + 1], d->stream);
         }

@@ -70,9 +70,7 @@ struct KName {
 static const KName kNames[] = {
     {"rd_k_dequant_q4k", &Kernels::dequant_q4k},
     {"rd_k_retile_q4k", &Kernels::retile_q4k},
-    {"rd_k_gemm_q4k_w4", &Kernels::gemm_q4k_w4},
-    {"rd_k_gemm_q4k_w2", &Kernels::gemm_q4k_w2},
-    {"rd_k_gemm_q4k_k2", &Kernels::gemm_q4k_k2},
+    {"rd_k_gemm_q4k", &Kernels::gemm_q4k},
     {"rd_k_gemm_q4k_gateup", &Kernels::gemm_q4k_gateup},
     {"rd_k_quant_act", &Kernels::quant_act},
     {"rd_k_reduce_splits", &Kernels::reduce_splits},
@@ -100,8 +98,6 @@ static const KName kNames[] = {
     {"rd_k_copy16", &Kernels::copy16},
     {"rd_k_barrier_probe", &Kernels::barrier_probe},
 };
-
-int load_resident_variants(rd_device *d);
 
 static int open_common(int ordinal, const void *image, rd_device **out) {
     const char *why = nullptr;
@@ -134,12 +130,6 @@ static int open_common(int ordinal, const void *image, rd_device **out) {
             return RD_ERR_HIP;
         }
         d->k.*(kn.slot) = f;
-    }
-    if (load_resident_variants(d) != RD_OK) {
-        (void)hip->ModuleUnload(d->module);
-        (void)hip->StreamDestroy(d->stream);
-        delete d;
-        return RD_ERR_HIP;
     }
     *out = d;
     return RD_OK;
@@ -182,66 +172,20 @@ extern "C" int rd_device_mem_info(rd_device *d, size_t *free_b, size_t *total_b)
 }
 
 // ---- GEMM planning ----
-struct ResidentVariant {
-    const char *name;
-    int wpb, np;
-};
-static const ResidentVariant kResident[6] = {{"rd_k_gemm_q4k_r4x8", 4, 8}, {"rd_k_gemm_q4k_r4x4", 4, 4}, {"rd_k_gemm_q4k_r4x2", 4, 2},
-                                             {"rd_k_gemm_q4k_r2x4", 2, 4}, {"rd_k_gemm_q4k_r2x8", 2, 8}, {"rd_k_gemm_q4k_r8x4", 8, 4}};
-
-int load_resident_variants(rd_device *d) {
-    for (int i = 0; i < 6; i++)
-        if (d->hip->ModuleGetFunction(&d->k.gemm_q4k_r[i], d->module, kResident[i].name) != hipSuccess) {
-            rd_set_error("code object lacks kernel %s", kResident[i].name);
-            return RD_ERR_HIP;
-        }
-    return RD_OK;
-}
-
-static GemmPlan streaming_plan(int N, int nKB) {
+// Split K so that about one block per CU is in flight: fewer blocks leave CUs (and their share of the memory system's
+// outstanding requests) idle, more splits only add partial-sum traffic. A split keeps at least two K-blocks.
+GemmPlan plan_gemm(int kind, int N, int nKB) {
+    (void)kind;
     GemmPlan p;
-    p.variant = -1, p.wpb = 4;
     int groups = (N + 127) / 128;
-    int target = 256; // blocks wanted: one per CU (more splits only add partial-sum traffic)
+    int target = 256;
     if (const char *e = getenv("ROCMDECODE_GEMM_BLOCKS")) target = atoi(e) > 0 ? atoi(e) : target;
-    int want = (target + groups - 1) / groups;
+    int want = target / groups; // rounded down: a few idle CUs cost less than another round of partial sums
     int maxSplits = nKB >= 2 ? nKB / 2 : 1;
     int splits = want < 1 ? 1 : (want > maxSplits ? maxSplits : want);
     if (const char *e = getenv("ROCMDECODE_SPLITS")) splits = atoi(e) > 0 ? atoi(e) : splits;
     if (splits > nKB) splits = nKB;
     p.kbPerSplit = (nKB + splits - 1) / splits;
-    p.splits = (nKB + p.kbPerSplit - 1) / p.kbPerSplit;
-    return p;
-}
-
-// Q4_K projections of a decode step are a few MB to a few tens of MB: pick the resident-panel variant that gives at least
-// one block per CU with the fewest K splits (each split costs a partial-sum round trip). Huge-N matrices (an LM head) have
-// thousands of blocks anyway and stream with the double-buffered kernel.
-GemmPlan plan_gemm(int kind, int N, int nKB) {
-    if (kind == 0 && getenv("ROCMDECODE_K2")) {
-        GemmPlan p = streaming_plan(N, nKB);
-        p.kgroups = 2;
-        return p;
-    }
-    if (kind != 0 || getenv("ROCMDECODE_SPLITS")) return streaming_plan(N, nKB);
-    int pick = -1;
-    if (const char *e = getenv("ROCMDECODE_GEMM")) {
-        for (int i = 0; i < 6; i++)
-            if (!strcmp(e, kResident[i].name + 14)) pick = i;
-        if (pick < 0) return streaming_plan(N, nKB);
-    } else {
-        if (!getenv("ROCMDECODE_RESIDENT")) return streaming_plan(N, nKB);
-        if ((long)N * nKB >= 64L * 1024 * 16) return streaming_plan(N, nKB); // >= 1M row-blocks: e.g. a Q4_K LM head
-        const int order[6] = {5, 0, 1, 4, 3, 2};                              // fewest splits first, wide blocks first
-        for (int oi = 0; oi < 6 && pick < 0; oi++) {
-            const ResidentVariant &v = kResident[order[oi]];
-            long blocks = (long)((N + 32 * v.wpb - 1) / (32 * v.wpb)) * ((nKB + v.np - 1) / v.np);
-            if (blocks >= 224) pick = order[oi];
-        }
-        if (pick < 0) pick = 2;
-    }
-    GemmPlan p;
-    p.variant = pick, p.wpb = kResident[pick].wpb, p.kbPerSplit = kResident[pick].np;
     p.splits = (nKB + p.kbPerSplit - 1) / p.kbPerSplit;
     return p;
 }
@@ -317,14 +261,10 @@ int launch_gemm(rd_device *d, const DevWeight &w, const void *Xp, float *P, int 
     int nKB = w.kind == 0 ? w.K / 256 : w.K / 128;
     GemmPlan p = plan_gemm(w.kind, w.N, nKB);
     if (plan_out) *plan_out = p;
-    unsigned gx = (unsigned)((w.N + 32 * p.wpb - 1) / (32 * p.wpb));
-    if (p.variant >= 0)
-        return d->launch(d->k.gemm_q4k_r[p.variant], gx, p.splits, 1, (unsigned)(64 * p.wpb), (const void *)w.tiled, Xp, P, w.N, nKB, M);
-    if (w.kind == 0 && p.kgroups == 2)
-        return d->launch(d->k.gemm_q4k_k2, gx, p.splits, 1, 512, (const void *)w.tiled, Xp, P, w.N, nKB, p.kbPerSplit, M);
+    unsigned gx = (unsigned)((w.N + 127) / 128);
     if (w.kind == 0)
-        return d->launch(d->k.gemm_q4k_w4, gx, p.splits, 1, 256, (const void *)w.tiled, Xp, P, w.N, nKB, p.kbPerSplit, M);
+        return d->launch(d->k.gemm_q4k, gx, p.splits, 1, GEMM_THREADS, (const void *)w.tiled, Xp, P, w.N, nKB, p.kbPerSplit, M);
     if (w.kind == 1)
-        return d->launch(d->k.gemm_w8a8, gx, p.splits, 1, 256, (const void *)w.tiled, (const void *)w.scales, Xp, P, w.N, nKB, p.kbPerSplit, M);
-    return d->launch(d->k.gemm_w4a8, gx, p.splits, 1, 256, (const void *)w.tiled, Xp, P, w.N, nKB, p.kbPerSplit, M);
+        return d->launch(d->k.gemm_w8a8, gx, p.splits, 1, GEMM_THREADS, (const void *)w.tiled, (const void *)w.scales, Xp, P, w.N, nKB, p.kbPerSplit, M);
+    return d->launch(d->k.gemm_w4a8, gx, p.splits, 1, GEMM_THREADS, (const void *)w.tiled, Xp, P, w.N, nKB, p.kbPerSplit, M);
 }

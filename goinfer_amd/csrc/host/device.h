@@ -21,10 +21,9 @@ constexpr size_t Q4K_TILE_BYTES = 4608;
 enum { PANEL_Q4K = 0, PANEL_LIN = 1, PANEL_LIN4 = 2 };
 
 struct Kernels {
-    hipFunction_t dequant_q4k, retile_q4k, gemm_q4k_w4, gemm_q4k_w2, gemm_q4k_k2, quant_act, reduce_splits, add_rmsnorm_quant, swiglu_quant;
+    hipFunction_t dequant_q4k, retile_q4k, gemm_q4k, quant_act, reduce_splits, add_rmsnorm_quant, swiglu_quant;
     hipFunction_t retile_w8a8, gemm_w8a8, retile_w4a8, gemm_w4a8;
     hipFunction_t gemm_q4k_gateup;
-    hipFunction_t gemm_q4k_r[6]; // resident-panel variants, see kResident in device.cc
     hipFunction_t kv_store, qkv_rope_store, attn_partial, attn_combine, attn_combine_quant;
     hipFunction_t rmsnorm, rope, argmax_rows, argmax_final, matmul_f32, moe_route, gemm_w4a8_moe, moe_swiglu_quant, moe_fold, embed_rows, copy16, barrier_probe;
 };
@@ -61,13 +60,13 @@ struct DevBuf {
     template <typename T> T *as() { return (T *)p; }
 };
 
+// block sizes of the GEMM kernels: (4 consumer + 1 producer waves) x K-groups; they match the code object's launch bounds
+constexpr unsigned GEMM_THREADS = 320, GATEUP_THREADS = 640;
+
 // split-K plan of one GEMM launch
 struct GemmPlan {
-    int variant;    // -1: streaming kernel (panel double-buffered per K-block); >=0: index into the resident-panel variants
-    int wpb;        // waves per block (32 weight rows each)
     int splits;     // grid.y
     int kbPerSplit; // K-blocks (super-blocks or 128-wide blocks) per split
-    int kgroups = 1; // waves sharing one tile's K range inside a block (Q4_K only)
 };
 GemmPlan plan_gemm(int kind, int N, int nKB);
 

@@ -479,7 +479,7 @@ static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
     size_t xpStride = (size_t)(I / 128) * LIN_PANEL_BYTES;
     {
         Scope s(m, KC_MOE_GEMM);
-        RC(d->launch(d->k.gemm_w4a8_moe, (unsigned)((2 * I + 127) / 128), (unsigned)nE, 1, 256, (const void *)l.exp_gateup, guStride,
+        RC(d->launch(d->k.gemm_w4a8_moe, (unsigned)((2 * I + 127) / 128), (unsigned)nE, 1, GEMM_THREADS, (const void *)l.exp_gateup, guStride,
                      (const void *)m->XpA, (size_t)0, m->moe_gu, 2 * I, H / 128, B, k, (const signed char *)m->moe_rank, nE));
     }
     {
@@ -489,7 +489,7 @@ static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
     }
     {
         Scope s(m, KC_MOE_GEMM);
-        RC(d->launch(d->k.gemm_w4a8_moe, (unsigned)((H + 127) / 128), (unsigned)nE, 1, 256, (const void *)l.exp_down, dnStride, (const void *)m->XpE,
+        RC(d->launch(d->k.gemm_w4a8_moe, (unsigned)((H + 127) / 128), (unsigned)nE, 1, GEMM_THREADS, (const void *)l.exp_down, dnStride, (const void *)m->XpE,
                      xpStride, m->moe_dn, H, I / 128, B, k, (const signed char *)m->moe_rank, nE));
     }
     {
@@ -597,7 +597,7 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
             RC(add_norm_quant(m, B, m->P, plan.splits, l.ffn_norm, l.gateup, m->XpA, nullptr));
             if (l.gateup.kind == 0 && c.inter % 64 == 0 && !getenv("ROCMDECODE_NO_FUSED_GATEUP")) {
                 Scope s(m, KC_GEMM_GATEUP); // gate|up GEMM + SwiGLU + quantization in one launch
-                RC(d->launch(d->k.gemm_q4k_gateup, (unsigned)(c.inter / 64), 1, 1, 512, (const void *)l.gateup.tiled, (const void *)m->XpA, m->XpB,
+                RC(d->launch(d->k.gemm_q4k_gateup, (unsigned)(c.inter / 64), 1, 1, GATEUP_THREADS, (const void *)l.gateup.tiled, (const void *)m->XpA, m->XpB,
                              panel_kind_for(l.down), c.inter, H / 256, B));
             } else {
                 {

@@ -24,6 +24,7 @@ struct W8Traits {
     typedef W8Tile Tile;
     static constexpr int TILE_BYTES = 4096;
     static constexpr int PANEL_VECS = RD_LIN_PANEL_BYTES / 16;
+    static constexpr int PRODUCER_DEPTH = 4; // 8 KB panels, short K-blocks: more of them in flight
     static __device__ __forceinline__ void load(Tile &w, const uint8_t *__restrict__ p, int lane) {
 #pragma unroll
         for (int c = 0; c < 4; c++) w.q[c] = __builtin_nontemporal_load((const uint4_t *)(p + c * 1024 + lane * 16));
@@ -57,11 +58,11 @@ struct W8Traits {
     }
 };
 
-extern "C" __global__ __launch_bounds__(256) void rd_k_gemm_w8a8(const uint8_t *__restrict__ Wt, const float *__restrict__ wscale,
+extern "C" __global__ __launch_bounds__(320) void rd_k_gemm_w8a8(const uint8_t *__restrict__ Wt, const float *__restrict__ wscale,
                                                                   const uint8_t *__restrict__ Xp, float *__restrict__ P, int N, int nKB,
                                                                   int kbPerSplit, int M) {
     __shared__ uint4_t lds[2 * RD_LIN_PANEL_BYTES / 16];
-    gemm_body<W8Traits, 4>(Wt, wscale, Xp, P, N, nKB, kbPerSplit, M, lds);
+    gemm_body<W8Traits, 4, 1, 3>(Wt, wscale, Xp, P, N, nKB, kbPerSplit, M, lds);
 }
 
 // ---------------- W4A8: canonical int4 nibbles (value nib-8), binary16 scale per 32 (decoder/weightmat.go:160-178) ----------------
@@ -94,6 +95,7 @@ struct W4Traits {
     typedef W4Tile Tile;
     static constexpr int TILE_BYTES = 2304;
     static constexpr int PANEL_VECS = RD_LIN_PANEL_BYTES / 16;
+    static constexpr int PRODUCER_DEPTH = 4; // 8 KB panels, short K-blocks: more of them in flight
     static __device__ __forceinline__ void load(Tile &w, const uint8_t *__restrict__ p, int lane) {
         w.sc = __builtin_nontemporal_load((const uint2_t *)(p + (lane & 31) * 8));
         w.q[0] = __builtin_nontemporal_load((const uint4_t *)(p + 256 + lane * 16));
@@ -128,8 +130,8 @@ struct W4Traits {
     static __device__ __forceinline__ void finish(float16_t &, const void *, int, int) {}
 };
 
-extern "C" __global__ __launch_bounds__(256) void rd_k_gemm_w4a8(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ Xp,
+extern "C" __global__ __launch_bounds__(320) void rd_k_gemm_w4a8(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ Xp,
                                                                   float *__restrict__ P, int N, int nKB, int kbPerSplit, int M) {
     __shared__ uint4_t lds[2 * RD_LIN_PANEL_BYTES / 16];
-    gemm_body<W4Traits, 4>(Wt, nullptr, Xp, P, N, nKB, kbPerSplit, M, lds);
+    gemm_body<W4Traits, 4, 1, 3>(Wt, nullptr, Xp, P, N, nKB, kbPerSplit, M, lds);
 }

@@ -6,22 +6,22 @@
 #include "act.h"
 #include "lin.h"
 
-// out[(token*k + rank)][N] = panels . W_e^T for the experts that have at least one token. Grid (ceil(N/128), nE).
+// out[(token*k + rank)][N] = panels . W_e^T for the experts that have at least one token. Grid (ceil(N/128), nE), block 320 (four consumer waves and a panel producer).
 // xpStride: bytes between the experts' panel sets (0 = all experts read the same panels: the gate/up projections).
-extern "C" __global__ __launch_bounds__(256) void rd_k_gemm_w4a8_moe(const uint8_t *__restrict__ Wt, size_t wStride, const uint8_t *__restrict__ Xp,
+extern "C" __global__ __launch_bounds__(320) void rd_k_gemm_w4a8_moe(const uint8_t *__restrict__ Wt, size_t wStride, const uint8_t *__restrict__ Xp,
                                                                       size_t xpStride, float *__restrict__ out, int N, int nKB, int T, int k,
                                                                       const signed char *__restrict__ rankOf, int nE) {
     __shared__ uint4_t lds[2 * RD_LIN_PANEL_BYTES / 16];
     const int e = blockIdx.y, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     int mine = (tid < T && rankOf[(size_t)tid * nE + e] >= 0) ? 1 : 0;
     if (!__syncthreads_or(mine)) return;
-    const int tile = blockIdx.x * 4 + wave;
+    const int tile = blockIdx.x * 4 + (wave & 3);
     const bool active = tile * 32 < N;
     float16_t acc;
     const int ltile = active ? tile : (N >> 5) - 1;
-    gemm_mainloop<W4Traits, 4>(acc, Wt + (size_t)e * wStride + (size_t)ltile * nKB * W4Traits::TILE_BYTES, Xp + (size_t)e * xpStride, 0, nKB, active,
-                               lds);
-    if (!active) return;
+    gemm_mainloop_pc<W4Traits, 4, 1, 3>(acc, Wt + (size_t)e * wStride + (size_t)ltile * nKB * W4Traits::TILE_BYTES, Xp + (size_t)e * xpStride, 0, nKB,
+                                        lds);
+    if (!active || wave >= 4) return;
 #pragma unroll
     for (int r = 0; r < 16; r++) {
         int m = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);

@@ -112,6 +112,11 @@ __device__ __forceinline__ void q4k_tile_mma(float16_t &acc, const Q4KTile &w, c
         C0[jj] = (half2_t){c, c};
         off[jj] = (half_t)(8.f * dsc32 - delta - dmin * (float)m); // exact scale here keeps the scale rounding centred
     }
+#ifdef RD_Q4K_ACC2
+    float16_t acc2;
+#pragma unroll
+    for (int i = 0; i < 16; i++) acc2[i] = 0.f;
+#endif
 #pragma unroll
     for (int s = 0; s < 16; s++) {
         uint32_t wd = w.q[s >> 2][s & 3];
@@ -142,7 +147,12 @@ __device__ __forceinline__ void q4k_tile_mma(float16_t &acc, const Q4KTile &w, c
         uint4_t av = panel[s * 64 + lane];
 #endif
         __builtin_memcpy(&a, &av, 16);
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc, 0, 0, 0);
+#ifdef RD_Q4K_ACC2
+        if (s & 1)
+            acc2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc2, 0, 0, 0);
+        else
+#endif
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc, 0, 0, 0);
     }
     {
         half8_t b = {off[0], off[1], off[2], off[3], (half_t)0, (half_t)0, (half_t)0, (half_t)0};
@@ -151,12 +161,17 @@ __device__ __forceinline__ void q4k_tile_mma(float16_t &acc, const Q4KTile &w, c
         __builtin_memcpy(&a, &av, 16);
         acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc, 0, 0, 0);
     }
+#ifdef RD_Q4K_ACC2
+#pragma unroll
+    for (int i = 0; i < 16; i++) acc[i] += acc2[i];
+#endif
 }
 
 struct Q4KTraits {
     typedef Q4KTile Tile;
     static constexpr int TILE_BYTES = RD_Q4K_TILE_BYTES;
     static constexpr int PANEL_VECS = RD_Q4K_PANEL_BYTES / 16;
+    static constexpr int PRODUCER_DEPTH = 2; // 17 KB panels: 68 registers each in the producer wave
     static __device__ __forceinline__ void load(Tile &w, const uint8_t *__restrict__ p, int lane) { q4k_tile_load(w, p, lane); }
     static __device__ __forceinline__ void mma(float16_t &acc, const Tile &w, const uint4_t *__restrict__ panel, int lane) {
         q4k_tile_mma(acc, w, panel, lane);
@@ -164,36 +179,19 @@ struct Q4KTraits {
     static __device__ __forceinline__ void finish(float16_t &, const void *, int, int) {}
 };
 
-extern "C" __global__ __launch_bounds__(256) void rd_k_gemm_q4k_w4(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ Xp,
-                                                                    float *__restrict__ P, int N, int nSB, int sbPerSplit, int M) {
+// Grid (ceil(N/128), splits), block 320: four consumer waves (one 32-row tile each) and one panel producer.
+extern "C" __global__ __launch_bounds__(320) void rd_k_gemm_q4k(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ Xp,
+                                                                 float *__restrict__ P, int N, int nSB, int sbPerSplit, int M) {
     __shared__ uint4_t lds[2 * RD_Q4K_PANEL_BYTES / 16];
-    gemm_body<Q4KTraits, 4>(Wt, nullptr, Xp, P, N, nSB, sbPerSplit, M, lds);
+    gemm_body<Q4KTraits, 4, 1, 3>(Wt, nullptr, Xp, P, N, nSB, sbPerSplit, M, lds);
 }
-extern "C" __global__ __launch_bounds__(128) void rd_k_gemm_q4k_w2(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ Xp,
-                                                                    float *__restrict__ P, int N, int nSB, int sbPerSplit, int M) {
-    __shared__ uint4_t lds[2 * RD_Q4K_PANEL_BYTES / 16];
-    gemm_body<Q4KTraits, 2>(Wt, nullptr, Xp, P, N, nSB, sbPerSplit, M, lds);
-}
-
-#define RD_Q4K_RESIDENT(NAME, WPB, NP, PF)                                                                                                     \
-    extern "C" __global__ __launch_bounds__(WPB * 64) void NAME(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ Xp,               \
-                                                                 float *__restrict__ P, int N, int nSB, int M) {                              \
-        __shared__ uint4_t lds[NP * RD_Q4K_PANEL_BYTES / 16];                                                                                  \
-        gemm_resident_body<Q4KTraits, WPB, NP, PF>(Wt, nullptr, Xp, P, N, nSB, M, lds);                                                        \
-    }
-RD_Q4K_RESIDENT(rd_k_gemm_q4k_r4x8, 4, 8, 4)
-RD_Q4K_RESIDENT(rd_k_gemm_q4k_r4x4, 4, 4, 4)
-RD_Q4K_RESIDENT(rd_k_gemm_q4k_r4x2, 4, 2, 2)
-RD_Q4K_RESIDENT(rd_k_gemm_q4k_r2x4, 2, 4, 4)
-RD_Q4K_RESIDENT(rd_k_gemm_q4k_r2x8, 2, 8, 4)
-RD_Q4K_RESIDENT(rd_k_gemm_q4k_r8x4, 8, 4, 3)
 
 // Fused gate/up projection + SwiGLU + per-32 quantization (goinfer decoder/cpu_gateup_fused.go:83-148, in one launch):
 // W holds [gate rows; up rows] (2*I rows). Block b: waves 0,1 own gate tiles 2b,2b+1, waves 2,3 the matching up tiles, all over
 // the full K (no split, so the sums are complete in registers). The up waves hand their sums over through LDS; the gate waves
 // compute silu(gate)*up (silu in f64, decoder/rmsnorm.go:204-207), quantize each row's 32 columns (one activation group) and write
 // the f16 panels the down projection reads. Each tile's K range is shared by two waves (K-groups) whose partial sums are
-// folded in LDS first. Grid (I/64), block 512.
+// folded in LDS first.
 template <int KG, int PF>
 __device__ __forceinline__ void q4k_gateup_body(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ Xp, uint8_t *__restrict__ XpOut,
                                                 int outKind, int I, int nSB, int M, uint4_t *lds) {
@@ -203,8 +201,16 @@ __device__ __forceinline__ void q4k_gateup_body(const uint8_t *__restrict__ Wt, 
     const bool active = t < nGate;
     float16_t acc;
     const int ltile = active ? tile : nGate - 1;
-    gemm_mainloop_kg<Q4KTraits, 4, KG, PF>(acc, Wt + (size_t)ltile * nSB * RD_Q4K_TILE_BYTES, Xp, 0, nSB, lds);
+#ifdef RD_DBG_TIMING
+#define RD_GSTAMP(k) if (tid == 0) rd_dbg_g[blockIdx.x * 8 + (k)] = __builtin_amdgcn_s_memrealtime();
+#else
+#define RD_GSTAMP(k)
+#endif
+    RD_GSTAMP(0)
+    gemm_mainloop_pc<Q4KTraits, 4, KG, PF>(acc, Wt + (size_t)ltile * nSB * RD_Q4K_TILE_BYTES, Xp, 0, nSB, lds);
+    RD_GSTAMP(1)
     gemm_fold_groups<4, KG>(acc, (float *)lds);
+    RD_GSTAMP(2)
 #ifdef RD_DBG_NO_EPILOGUE
     if (acc[3] == 1234.5f) XpOut[tid] = 1;
     return;
@@ -222,7 +228,7 @@ __device__ __forceinline__ void q4k_gateup_body(const uint8_t *__restrict__ Wt, 
     __syncthreads();
     constexpr int NTHR = 4 * KG * 64;
 #pragma unroll
-    for (int e = tid; e < 2048; e += NTHR) {
+    for (int e = tid; e < 2048 && tid < NTHR; e += NTHR) { // consumer waves only; whole waves drop out together
         const int tl = e >> 10, m = (e >> 5) & 31, c = e & 31;
         const int tt = blockIdx.x * 2 + tl;
         float a = __fmul_rn(silu_f64(xe[(tl * 32 + m) * 32 + c]), xe[((2 + tl) * 32 + m) * 32 + c]);
@@ -241,20 +247,12 @@ __device__ __forceinline__ void q4k_gateup_body(const uint8_t *__restrict__ Wt, 
             }
         }
     }
+    RD_GSTAMP(3)
 }
 
-#ifndef RD_GATEUP_PF
-#define RD_GATEUP_PF 3
-#endif
-extern "C" __global__ __launch_bounds__(512) void rd_k_gemm_q4k_gateup(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ Xp,
+// Grid (I/64), block 640: two K-groups of four consumer waves (gate t0,t1, up t0,t1) plus one producer each.
+extern "C" __global__ __launch_bounds__(640) void rd_k_gemm_q4k_gateup(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ Xp,
                                                                         uint8_t *__restrict__ XpOut, int outKind, int I, int nSB, int M) {
     __shared__ uint4_t lds[2 * 2 * RD_Q4K_PANEL_BYTES / 16];
-    q4k_gateup_body<2, RD_GATEUP_PF>(Wt, Xp, XpOut, outKind, I, nSB, M, lds);
-}
-
-// The plain GEMM with two K-groups per block (8 waves): for launches whose grid cannot fill the chip with 4-wave blocks.
-extern "C" __global__ __launch_bounds__(512) void rd_k_gemm_q4k_k2(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ Xp,
-                                                                    float *__restrict__ P, int N, int nSB, int sbPerSplit, int M) {
-    __shared__ uint4_t lds[2 * 2 * RD_Q4K_PANEL_BYTES / 16];
-    gemm_body_kg<Q4KTraits, 4, 2, RD_GATEUP_PF>(Wt, nullptr, Xp, P, N, nSB, sbPerSplit, M, lds);
+    q4k_gateup_body<2, 3>(Wt, Xp, XpOut, outKind, I, nSB, M, lds);
 }
