@@ -20,7 +20,7 @@ EXPORTS = [
     "rd_model_upload_q4k", "rd_model_upload_w8a8", "rd_model_upload_w4a8", "rd_model_upload_f32", "rd_model_finalize",
     "rd_kv_configure", "rd_kv_upload", "rd_kv_truncate", "rd_kv_reset", "rd_step_batch", "rd_forward",
     "rd_last_moe_indices", "rd_model_upload_embedding", "rd_bench_steps", "rd_bench_profile", "rd_bench_class_count",
-    "rd_bench_class_name", "rd_bench_kernel",
+    "rd_bench_class_name", "rd_bench_kernel", "rd_gateup_q4k_quant", "rd_moe_replay",
 ]
 
 
@@ -113,6 +113,14 @@ class Device:
         b2 = None if blocks2 is None else np.ascontiguousarray(blocks2, dtype=np.uint8)
         dst = np.empty((a.shape[0], N), np.float32)
         check(lib().rd_gemm_q4k(self.h, _p(blocks), N, K, _p(a), a.shape[0], _p(dst), _p(b2)), "rd_gemm_q4k")
+        return dst
+
+    def gateup_q4k_quant(self, gate, up, I, K, a):
+        a = _f32(a)
+        gate = np.ascontiguousarray(gate, dtype=np.uint8)
+        up = np.ascontiguousarray(up, dtype=np.uint8)
+        dst = np.empty((a.shape[0], I), np.float32)
+        check(lib().rd_gateup_q4k_quant(self.h, _p(gate), _p(up), I, K, _p(a), a.shape[0], _p(dst)), "rd_gateup_q4k_quant")
         return dst
 
     def gemm_w8a8(self, q, scales, a):
@@ -234,6 +242,12 @@ class Model:
         ids = np.empty(B, np.int32) if want & WANT_ARGMAX else None
         check(lib().rd_step_batch(self.h, B, _p(slots), _p(pos), _p(emb), want, _p(logits), _p(ids)), "rd_step_batch")
         return logits, ids
+
+    def moe_replay(self, idx, wgt):
+        """The next step replays this routing ([B][layers][k] indices and weights) instead of its own."""
+        idx = np.ascontiguousarray(idx, dtype=np.int32)
+        wgt = _f32(wgt)
+        check(lib().rd_moe_replay(self.h, idx.shape[0], _p(idx), _p(wgt)), "rd_moe_replay")
 
     def forward(self, slot, pos, emb):
         emb = _f32(emb)

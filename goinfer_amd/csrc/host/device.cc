@@ -97,6 +97,7 @@ static const KName kNames[] = {
     {"rd_k_embed_rows", &Kernels::embed_rows},
     {"rd_k_copy16", &Kernels::copy16},
     {"rd_k_barrier_probe", &Kernels::barrier_probe},
+    {"rd_k_unpanel_q4k", &Kernels::unpanel_q4k},
 };
 
 static int open_common(int ordinal, const void *image, rd_device **out) {

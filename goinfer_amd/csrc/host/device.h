@@ -25,7 +25,7 @@ struct Kernels {
     hipFunction_t retile_w8a8, gemm_w8a8, retile_w4a8, gemm_w4a8;
     hipFunction_t gemm_q4k_gateup;
     hipFunction_t kv_store, qkv_rope_store, attn_partial, attn_combine, attn_combine_quant;
-    hipFunction_t rmsnorm, rope, argmax_rows, argmax_final, matmul_f32, moe_route, gemm_w4a8_moe, moe_swiglu_quant, moe_fold, embed_rows, copy16, barrier_probe;
+    hipFunction_t rmsnorm, rope, argmax_rows, argmax_final, matmul_f32, moe_route, gemm_w4a8_moe, moe_swiglu_quant, moe_fold, embed_rows, copy16, barrier_probe, unpanel_q4k;
 };
 
 struct rd_device {
@@ -62,6 +62,13 @@ struct DevBuf {
 
 // block sizes of the GEMM kernels: (4 consumer + 1 producer waves) x K-groups; they match the code object's launch bounds
 constexpr unsigned GEMM_THREADS = 320, GATEUP_THREADS = 640;
+
+// How many 64-position KV blocks one attention work item covers for a sequence of nb blocks: every (sequence, kv head) is
+// cut into at most ATTN_PIECES pieces. The cut depends on the sequence's own length only, never on what else is in the
+// batch: the partial results are merged in piece order, so this is what keeps a row computed in a batch bit-identical to
+// the same row computed alone.
+constexpr int ATTN_PIECES = 16;
+inline int attn_chunk_blocks(int nb) { return (nb + ATTN_PIECES - 1) / ATTN_PIECES; }
 
 // split-K plan of one GEMM launch
 struct GemmPlan {

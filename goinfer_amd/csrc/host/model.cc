@@ -312,8 +312,10 @@ extern "C" int rd_model_finalize(rd_model *m) {
     RC(alloc_f32(d, &m->qbuf, (size_t)32 * qd));
     RC(alloc_f32(d, &m->logits, (size_t)32 * c.vocab));
     size_t kA = (size_t)H, kB = (size_t)std::max(qd, c.n_experts ? qd : c.inter);
-    RC(d->alloc(&m->XpA, (kA / 128) * LIN_PANEL_BYTES + Q4K_PANEL_BYTES)); // >= either panel kind for K=hidden
-    RC(d->alloc(&m->XpB, (kB / 128) * LIN_PANEL_BYTES + Q4K_PANEL_BYTES));
+    // room for either panel kind: 8 KB per 128 elements (int8/int4 consumers) or 17 KB per 256 (Q4_K consumers)
+    auto panel_room = [](size_t K) { return std::max(((K + 127) / 128) * (size_t)LIN_PANEL_BYTES, ((K + 255) / 256) * (size_t)Q4K_PANEL_BYTES); };
+    RC(d->alloc(&m->XpA, panel_room(kA)));
+    RC(d->alloc(&m->XpB, panel_room(kB)));
     RC(d->alloc((void **)&m->ids, sizeof(int) * 32));
     RC(alloc_f32(d, &m->cand_v, (size_t)32 * ((c.vocab + 4095) / 4096)));
     RC(d->alloc((void **)&m->cand_i, sizeof(int) * 32 * (size_t)((c.vocab + 4095) / 4096)));
@@ -370,7 +372,7 @@ extern "C" int rd_kv_configure(rd_model *m, int slots, int ctx_cap) {
     RC(d->h2d(m->tables, tab.data(), sizeof(int) * tab.size()));
     m->slot_len.assign((size_t)slots, 0);
     // attention work list: ~4096 items plus one per (row, kv head) of rounding
-    m->max_items = 4096 + 32 * c.n_kv_heads * 2;
+    m->max_items = 32 * c.n_kv_heads * ATTN_PIECES;
     int G = c.n_heads / c.n_kv_heads;
     RC(alloc_f32(d, &m->part, (size_t)m->max_items * G * (c.head_dim + 2)));
     RC(d->alloc((void **)&m->items, sizeof(AttnItemH) * (size_t)m->max_items));
@@ -435,14 +437,10 @@ struct Scope { // times one kernel class when the model's timer is on
 
 static int build_attn_items(rd_model *m, int B, const int *pos, std::vector<AttnItemH> &items, std::vector<int> &start) {
     const rd_model_desc &c = m->desc;
-    long total = 0;
-    for (int b = 0; b < B; b++) total += (long)((pos[b] + 1 + 63) / 64) * c.n_kv_heads;
-    int chunk = (int)std::max(1L, (total + 4095) / 4096);
-    if (const char *e = getenv("ROCMDECODE_ATTN_CHUNK")) chunk = std::max(1, atoi(e));
     items.clear();
     start.assign((size_t)B * c.n_kv_heads + 1, 0);
     for (int b = 0; b < B; b++) {
-        int nb = (pos[b] + 1 + 63) / 64;
+        const int nb = (pos[b] + 1 + 63) / 64, chunk = attn_chunk_blocks(nb);
         for (int h = 0; h < c.n_kv_heads; h++) {
             start[(size_t)b * c.n_kv_heads + h] = (int)items.size();
             for (int b0 = 0; b0 < nb; b0 += chunk) items.push_back({b, h, b0, std::min(nb, b0 + chunk)});
@@ -471,8 +469,14 @@ static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
         Scope s(m, KC_MOE_ROUTER);
         RC(d->launch(d->k.matmul_f32, (unsigned)((nE + 63) / 64), (unsigned)B, 1, 64, (const float *)m->normed, (const float *)l.router,
                      m->router_logits, B, H, nE));
-        RC(d->launch(d->k.moe_route, 1, 1, 1, 64, (const float *)m->router_logits, B, nE, k, c.norm_topk_prob, m->moe_idx, m->moe_wgt,
-                     m->moe_rank));
+        if (m->replay_B == B) { // replay a recorded routing (goinfer's moeSelOverride seam) instead of routing on these logits
+            RC(d->h2d(m->moe_idx, m->replay_idx[(size_t)layer].data(), sizeof(int) * (size_t)B * k));
+            RC(d->h2d(m->moe_wgt, m->replay_wgt[(size_t)layer].data(), sizeof(float) * (size_t)B * k));
+            RC(d->h2d(m->moe_rank, m->replay_rank[(size_t)layer].data(), (size_t)32 * nE));
+        } else {
+            RC(d->launch(d->k.moe_route, 1, 1, 1, 64, (const float *)m->router_logits, B, nE, k, c.norm_topk_prob, m->moe_idx, m->moe_wgt,
+                         m->moe_rank));
+        }
         HIPCHK(MemcpyAsync(m->moe_idx_all + (size_t)layer * 32 * k, m->moe_idx, sizeof(int) * (size_t)B * k, hipMemcpyDeviceToDevice, d->stream));
     }
     size_t guStride = (size_t)(2 * I / 32) * (H / 128) * 2304, dnStride = (size_t)(H / 32) * (I / 128) * 2304;
@@ -638,6 +642,9 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
     }
     for (int b = 0; b < B; b++) m->slot_len[(size_t)slot[b]] = pos[b] + 1;
     m->last_B = B;
+    const bool replayed = m->replay_B != 0;
+    m->replay_B = 0; // a routing override lasts one step
+    if (replayed) RC(d->sync()); // its host arrays were uploaded from pageable memory: let the copies finish before they can change
     if ((want & RD_WANT_LOGITS) && logits) RC(d->d2h(logits, m->logits, sizeof(float) * (size_t)B * c.vocab));
     if ((want & RD_WANT_ARGMAX) && ids) RC(d->d2h(ids, m->ids, sizeof(int) * (size_t)B));
     return RD_OK;
@@ -655,6 +662,32 @@ extern "C" int rd_step_batch(rd_model *m, int B, const int *slot, const int *pos
 extern "C" int rd_forward(rd_model *m, int slot, int pos, const float *emb, float *logits) {
     if (!m || !emb || !logits) return RD_ERR_ARG;
     return model_step(m, 1, &slot, &pos, emb, nullptr, RD_WANT_LOGITS, logits, nullptr);
+}
+
+extern "C" int rd_moe_replay(rd_model *m, int B, const int *idx, const float *wgt) {
+    if (!m || !idx || !wgt || m->desc.n_experts == 0 || B < 1 || B > 32) {
+        rd_set_error("rd_moe_replay: needs a MoE model, 1 <= B <= 32 and both arrays");
+        return RD_ERR_ARG;
+    }
+    const int L = m->desc.n_layers, k = m->desc.top_k, nE = m->desc.n_experts;
+    m->replay_idx.assign((size_t)L, std::vector<int>((size_t)B * k));
+    m->replay_wgt.assign((size_t)L, std::vector<float>((size_t)B * k));
+    m->replay_rank.assign((size_t)L, std::vector<signed char>((size_t)32 * nE, (signed char)-1));
+    for (int b = 0; b < B; b++)
+        for (int l = 0; l < L; l++)
+            for (int j = 0; j < k; j++) {
+                int e = idx[((size_t)b * L + l) * k + j];
+                if (e < 0 || e >= nE) {
+                    rd_set_error("rd_moe_replay: expert %d out of range at row %d layer %d", e, b, l);
+                    m->replay_B = 0;
+                    return RD_ERR_ARG;
+                }
+                m->replay_idx[(size_t)l][(size_t)b * k + j] = e;
+                m->replay_wgt[(size_t)l][(size_t)b * k + j] = wgt[((size_t)b * L + l) * k + j];
+                m->replay_rank[(size_t)l][(size_t)b * nE + e] = (signed char)j;
+            }
+    m->replay_B = B;
+    return RD_OK;
 }
 
 extern "C" int rd_last_moe_indices(rd_model *m, int *idx) {

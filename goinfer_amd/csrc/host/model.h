@@ -75,6 +75,12 @@ struct rd_model {
     size_t host_stage_bytes = 0;
     int last_B = 0;
 
+    // routing replay for the next step (rd_moe_replay): [layers] of host arrays the step uploads
+    int replay_B = 0;
+    std::vector<std::vector<int>> replay_idx;
+    std::vector<std::vector<float>> replay_wgt;
+    std::vector<std::vector<signed char>> replay_rank;
+
     StepTimer timer;
 };
 

@@ -52,7 +52,7 @@ static int gemm_host(rd_device *d, DevWeight &w, DevWeight *w2, const float *a, 
             RC(launch_gemm(d, w, Xp.p, P.as<float>(), mc, &plan));
             RC(d->launch(d->k.reduce_splits, (unsigned)((N + 255) / 256), (unsigned)mc, 1, 256, (const float *)P.p, O.as<float>(), N, plan.splits));
         } else {
-            // fused gate/up: w holds [gate; up] stacked (2N rows)
+            // gate|up stacked (2N rows): GEMM, then SwiGLU over the reduced partial sums
             RC(launch_gemm(d, *w2, Xp.p, P.as<float>(), mc, &plan));
             DevBuf X2(d);
             RC(X2.alloc((size_t)((N + 255) / 256) * Q4K_PANEL_BYTES));
@@ -90,6 +90,44 @@ extern "C" int rd_gemm_q4k(rd_device *d, const void *W, int N, int K, const floa
     w.kind = 0, w.N = N, w.K = K;
     rc = gemm_host(d, w, &wcat, a, M, dst);
     free_weight(d, &wcat);
+    return rc;
+}
+
+extern "C" int rd_gateup_q4k_quant(rd_device *d, const void *Wg, const void *Wu, int I, int K, const float *a, int M, float *dst) {
+    if (!d || !Wg || !Wu || !a || !dst || M <= 0) {
+        rd_set_error("rd_gateup_q4k_quant: bad arguments");
+        return RD_ERR_ARG;
+    }
+    if (I <= 0 || I % 256 || K <= 0 || K % 256) {
+        rd_set_error("rd_gateup_q4k_quant: I=%d and K=%d must be multiples of 256", I, K);
+        return RD_DECLINED;
+    }
+    size_t bytes = (size_t)I * (K / 256) * 144;
+    std::vector<uint8_t> cat(2 * bytes);
+    memcpy(cat.data(), Wg, bytes);
+    memcpy(cat.data() + bytes, Wu, bytes);
+    DevWeight w;
+    int rc = upload_q4k(d, cat.data(), 2 * I, K, &w);
+    if (rc) return rc;
+    DevBuf A(d), Xp(d), X2(d), O(d);
+    auto body = [&]() -> int {
+        RC(A.alloc(sizeof(float) * (size_t)32 * K));
+        RC(Xp.alloc((size_t)(K / 256) * Q4K_PANEL_BYTES));
+        RC(X2.alloc((size_t)(I / 256) * Q4K_PANEL_BYTES));
+        RC(O.alloc(sizeof(float) * (size_t)32 * I));
+        for (int m0 = 0; m0 < M; m0 += 32) {
+            int mc = std::min(32, M - m0);
+            RC(d->h2d(A.p, a + (size_t)m0 * K, sizeof(float) * (size_t)mc * K));
+            RC(quantize_rows(d, A.as<float>(), mc, K, PANEL_Q4K, 0, Xp.p));
+            RC(d->launch(d->k.gemm_q4k_gateup, (unsigned)(I / 64), 1, 1, GATEUP_THREADS, (const void *)w.tiled, (const void *)Xp.p, X2.as<uint8_t>(),
+                         (int)PANEL_Q4K, I, K / 256, mc));
+            RC(d->launch(d->k.unpanel_q4k, (unsigned)(I / 256), (unsigned)mc, 1, 256, (const void *)X2.p, O.as<float>(), I));
+            RC(d->d2h(dst + (size_t)m0 * I, O.p, sizeof(float) * (size_t)mc * I));
+        }
+        return RD_OK;
+    };
+    rc = body();
+    free_weight(d, &w);
     return rc;
 }
 
@@ -228,11 +266,8 @@ extern "C" int rd_attn_ragged(rd_device *d, int n_seq, const int *len, const int
         int rows = std::min(32, n_seq - r0);
         std::vector<AttnItemO> items;
         std::vector<int> start((size_t)rows * n_kv + 1), slots((size_t)rows), lens((size_t)rows);
-        long tb = 0;
-        for (int i = 0; i < rows; i++) tb += (long)((len[r0 + i] + 63) / 64) * n_kv;
-        int chunk = (int)std::max(1L, (tb + 4095) / 4096);
         for (int i = 0; i < rows; i++) {
-            int nb = (len[r0 + i] + 63) / 64;
+            const int nb = (len[r0 + i] + 63) / 64, chunk = attn_chunk_blocks(nb);
             slots[(size_t)i] = r0 + i, lens[(size_t)i] = len[r0 + i];
             for (int h = 0; h < n_kv; h++) {
                 start[(size_t)i * n_kv + h] = (int)items.size();

@@ -164,3 +164,12 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_swiglu_quant(const float 
     quant_g32x4(a[0], a[1], a[2], a[3], &x0, &x1, &x2, &x3, &gs);
     if (on) panel_store4(Xp, kind, m, n0, x0, x1, x2, x3, gs);
 }
+
+// A Q4_K-layout activation panel set back to rows: out[m][k] = the f16 value (code * scale) the GEMM reads for batch row m,
+// element k. Grid (ceil(K/256), M), block 256. The inverse of panel_store, for checking what a fused producer wrote.
+extern "C" __global__ void rd_k_unpanel_q4k(const uint8_t *__restrict__ Xp, float *__restrict__ out, int K) {
+    const int kb = blockIdx.x, m = blockIdx.y, t = threadIdx.x, k = kb * 256 + t;
+    if (k >= K) return;
+    const half_t *base = (const half_t *)(Xp + (size_t)kb * RD_Q4K_PANEL_BYTES);
+    out[(size_t)m * K + k] = (float)base[q4k_panel_index(t, m)];
+}

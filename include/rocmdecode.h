@@ -77,6 +77,10 @@ int rd_dequant_q4k(rd_device *d, const void *blocks, int N, int K, float *out);
  * (decoder/weightmat.go:961-971; backend/cuda/actgroup.cu:298-355 gemv_q4k_g32). If W2 != NULL the call is the
  * fused gate/up SwiGLU: dst = silu(a.W^T) * (a.W2^T) (decoder/cpu_gateup_fused.go:83-148). Host pointers. */
 int rd_gemm_q4k(rd_device *d, const void *W, int N, int K, const float *a, int M, float *dst, const void *W2);
+/* The decode step's own fused kernel on its own: gate|up projection + SwiGLU + per-32 quantization in one launch
+ * (decoder/cpu_gateup_fused.go:83-148 followed by linalg.QuantizeActQ at the down projection's input). dst[M][I] receives
+ * the quantized activations, code * scale, exactly as the down projection reads them. I and K multiples of 256. */
+int rd_gateup_q4k_quant(rd_device *d, const void *Wg, const void *Wu, int I, int K, const float *a, int M, float *dst);
 /* int8 per-row weights x per-32 int8 activations (backend/cuda/actgroup.cu:421-437 gemv_w8a8_g32). */
 int rd_gemm_w8a8(rd_device *d, const int8_t *q, const float *row_scale, int N, int K, const float *a, int M, float *dst);
 /* int4 group-32 weights with f16 scales x per-32 int8 activations (backend/cuda/actgroup.cu:243-275). */
@@ -123,6 +127,10 @@ int rd_step_batch(rd_model *m, int B, const int *slot, const int *pos, const flo
 int rd_forward(rd_model *m, int slot, int pos, const float *emb, float *logits);
 /* expert indices the last step routed to: int32 [B][n_layers][top_k] (MoE models only; parity checks) */
 int rd_last_moe_indices(rd_model *m, int *idx);
+/* Test seam, goinfer's moeSelOverride / moeWtsOverride (decoder/mlp.go:19-27,53-56): the NEXT step replays the given
+ * routing instead of routing on its own hidden state. idx, wgt: host [B][n_layers][top_k], the reference run's expert
+ * indices and weights; B must equal the next step's batch. The override is consumed by that step. */
+int rd_moe_replay(rd_model *m, int B, const int *idx, const float *wgt);
 
 /* ---- measurement: HIP-event timing on the stream the kernels are launched on; inputs resident in HBM ---- */
 /* The int8 embedding table (vocab x hidden codes + one f32 scale per row), resident so a greedy chain needs no host

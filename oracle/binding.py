@@ -31,6 +31,14 @@ class Model(C.Structure):
                 ("kv_f16", C.c_int), ("layers", C.POINTER(Layer)), ("final_norm", C.c_void_p), ("head", Mat)]
 
 
+def f16_round_trip(x):
+    """What an f16 cache holds of x (round-half-up narrowing, widened back)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty_like(x)
+    lib().or_f16_round_trip(x.ctypes.data, out.ctypes.data, x.size)
+    return out
+
+
 def build():
     """Compile liboracle.so from the C sources beside this file."""
     subprocess.check_call(["make", "-s", "-C", _HERE])
@@ -54,6 +62,9 @@ def lib():
         L.or_cache_new.restype = C.c_void_p
         L.or_cache_new.argtypes = [C.POINTER(Model), C.c_int]
         L.or_cache_free.argtypes = [C.POINTER(Model), C.c_void_p]
+        L.or_cache_upload.restype = C.c_int
+        L.or_cache_upload.argtypes = [C.POINTER(Model), C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+        L.or_f16_round_trip.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
         _LIB = L
     return _LIB
 
@@ -238,20 +249,36 @@ class OracleModel:
     def new_cache(self, cap):
         return lib().or_cache_new(C.byref(self.m), cap)
 
+    def cache_upload(self, c, layer, base, keys, vals):
+        """UploadKV: rows [n][kv dim] of one layer at positions base.., narrowed as the cache stores them."""
+        keys = np.ascontiguousarray(keys, dtype=np.float32)
+        vals = np.ascontiguousarray(vals, dtype=np.float32)
+        if lib().or_cache_upload(C.byref(self.m), C.c_void_p(c), layer, base, keys.shape[0], keys.ctypes.data, vals.ctypes.data):
+            raise RuntimeError("oracle: cache upload out of range")
+
     def free_cache(self, c):
         lib().or_cache_free(C.byref(self.m), C.c_void_p(c))
 
-    def step(self, emb, caches, want_moe=False):
+    def step(self, emb, caches, want_moe=False, want_weights=False, replay=None):
+        """One decodeMultiStep. want_moe: also the expert indices [B][layers][k]; want_weights: and the routing weights.
+        replay=(idx, wts): use this routing instead of the step's own."""
         emb = f32(emb)
         B = emb.shape[0]
         logits = np.empty((B, self.cfg["vocab"]), np.float32)
         arr = (C.c_void_p * B)(*caches)
-        trace = None
-        if want_moe:
+        trace = wts = None
+        if replay is not None:
+            trace = np.ascontiguousarray(replay[0], dtype=np.int32).copy()
+            wts = np.ascontiguousarray(replay[1], dtype=np.float32).copy()
+        elif want_moe or want_weights:
             trace = np.full((B, self.cfg_layers(), self.cfg["top_k"]), -1, np.int32)
-        rc = lib().or_decode_multi_step(C.byref(self.m), B, _p(emb), arr, _p(logits), _p(trace) if want_moe else None)
+            wts = np.zeros((B, self.cfg_layers(), self.cfg["top_k"]), np.float32)
+        rc = lib().or_decode_multi_step_traced(C.byref(self.m), B, _p(emb), arr, _p(logits), _p(trace) if trace is not None else None,
+                                               _p(wts) if wts is not None else None, 1 if replay is not None else 0)
         if rc != 0:
             raise RuntimeError("oracle: cache full")
+        if want_weights:
+            return logits, trace, wts
         return (logits, trace) if want_moe else logits
 
     def cfg_layers(self):

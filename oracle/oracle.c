@@ -572,6 +572,26 @@ void or_cache_free(const or_model *m, or_cache *c) {
     free(c);
 }
 
+void or_f16_round_trip(const float *src, float *dst, size_t n) {
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < n; i++) dst[i] = or_f16_to_f32(or_f32_to_f16(src[i]));
+}
+
+int or_cache_upload(const or_model *m, or_cache *c, int layer, int base, int n, const float *keys, const float *vals) {
+    size_t kvDim = (size_t)m->n_kv * m->head_dim;
+    if (layer < 0 || layer >= m->n_layers || base < 0 || n < 0 || base + n > c->cap) return -1;
+    float *kd = c->k[layer] + (size_t)base * kvDim, *vd = c->v[layer] + (size_t)base * kvDim;
+    if (m->kv_f16) {
+        or_f16_round_trip(keys, kd, (size_t)n * kvDim);
+        or_f16_round_trip(vals, vd, (size_t)n * kvDim);
+    } else {
+        memcpy(kd, keys, (size_t)n * kvDim * sizeof(float));
+        memcpy(vd, vals, (size_t)n * kvDim * sizeof(float));
+    }
+    if (base + n > c->pos) c->pos = base + n;
+    return 0;
+}
+
 /* decoder/mlp.go:729-745 */
 static void add_scaled(float *dst, const float *src, float s, int n) {
     for (int i = 0; i < n; i++) dst[i] += s * src[i];
@@ -583,7 +603,7 @@ static void qk_norm(float *x, int heads, int hd, const float *w, double eps) { o
 /* decoder/mlp.go:36-120 (moeMLP) for one row: router matmul (M=1), routeExperts, experts in rank order,
  * out += w_j * expert_j(h) (addScaled). mlp.go:630-726 (moeMLPBatchWith) folds each row in the same rank
  * order and is bit-identical to this per-row form by its own contract. */
-static void moe_mlp(const or_model *m, const or_layer *lw, const float *h, float *out, int *idx_trace) {
+static void moe_mlp(const or_model *m, const or_layer *lw, const float *h, float *out, int *idx_trace, float *wts_trace, int replay) {
     int nE = m->n_experts, k = m->top_k, H = m->hidden, I = m->exp_inter;
     float *logits = (float *)malloc(sizeof(float) * (size_t)nE);
     int *idx = (int *)malloc(sizeof(int) * (size_t)k);
@@ -592,10 +612,15 @@ static void moe_mlp(const or_model *m, const or_layer *lw, const float *h, float
     float *eo = (float *)malloc(sizeof(float) * (size_t)H);
     or_matmul(&lw->router, h, 1, logits);
     int n = or_route_experts(logits, nE, k, m->norm_topk, 0, idx, wts);
+    if (replay) { /* decoder/mlp.go:53-56: the recorded routing replaces this call's own */
+        n = k;
+        for (int j = 0; j < k; j++) idx[j] = idx_trace[j], wts[j] = wts_trace[j];
+    }
     memset(out, 0, sizeof(float) * (size_t)H);
     for (int j = 0; j < n; j++) {
         int e = idx[j];
-        if (idx_trace) idx_trace[j] = e;
+        if (idx_trace && !replay) idx_trace[j] = e;
+        if (wts_trace && !replay) wts_trace[j] = wts[j];
         or_matmul(&lw->exp_gate[e], h, 1, g);
         or_matmul(&lw->exp_up[e], h, 1, u);
         or_swiglu(g, u, I);
@@ -614,6 +639,12 @@ static void moe_mlp(const or_model *m, const or_layer *lw, const float *h, float
  * Pre-norm llama-style layer program: norm, q/k/v (M=B), optional QK-norm, RoPE at each row's own position,
  * per-sequence append + attention, o-proj, residual, norm, gated FFN (dense at M=B, MoE per row), residual; final norm; head. */
 int or_decode_multi_step(const or_model *m, int B, const float *emb, or_cache **caches, float *logits, int *moe_idx_trace) {
+    return or_decode_multi_step_traced(m, B, emb, caches, logits, moe_idx_trace, NULL, 0);
+}
+
+int or_decode_multi_step_traced(const or_model *m, int B, const float *emb, or_cache **caches, float *logits, int *moe_idx_trace,
+                                float *moe_wts_trace, int replay) {
+    if (replay && (!moe_idx_trace || !moe_wts_trace)) return -2;
     int H = m->hidden, nH = m->n_heads, nKV = m->n_kv, hd = m->head_dim, I = m->inter;
     int qDim = nH * hd, kvDim = nKV * hd;
     for (int b = 0; b < B; b++)
@@ -667,7 +698,8 @@ int or_decode_multi_step(const or_model *m, int B, const float *emb, or_cache **
         } else {
             for (int b = 0; b < B; b++)
                 moe_mlp(m, lw, norm + (size_t)b * H, att + (size_t)b * H,
-                        moe_idx_trace ? moe_idx_trace + ((size_t)b * m->n_layers + l) * m->top_k : NULL);
+                        moe_idx_trace ? moe_idx_trace + ((size_t)b * m->n_layers + l) * m->top_k : NULL,
+                        moe_wts_trace ? moe_wts_trace + ((size_t)b * m->n_layers + l) * m->top_k : NULL, replay);
         }
         for (size_t i = 0; i < (size_t)B * H; i++) h[i] += att[i];
     }

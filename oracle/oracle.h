@@ -114,9 +114,19 @@ typedef struct {
 
 or_cache *or_cache_new(const or_model *m, int cap);
 void or_cache_free(const or_model *m, or_cache *c);
+/* The prefill bridge, resident.Forward.UploadKV (decoder/resident/forward.go:17-22): writes post-RoPE K and raw V rows
+ * [n][n_kv*head_dim] of one layer at positions base..base+n-1, narrowed as the cache stores them; pos becomes
+ * max(pos, base+n) once the caller has uploaded every layer. Returns -1 when the rows do not fit. */
+int or_cache_upload(const or_model *m, or_cache *c, int layer, int base, int n, const float *keys, const float *vals);
+/* dst[i] = f16_to_f32(f32_to_f16(src[i])): what an f16 cache holds of src. */
+void or_f16_round_trip(const float *src, float *dst, size_t n);
 /* emb: [B][hidden] (embedding rows, already scaled); logits: [B][vocab]. Appends one position to every cache. */
 int or_decode_multi_step(const or_model *m, int B, const float *emb, or_cache **caches, float *logits,
                          int *moe_idx_trace /* [B][layers][top_k] or NULL */);
+/* The same, also recording the routing weights (decoder/mlp.go:17-27 moeSelTrace / moeWtsTrace) or, with replay != 0,
+ * reading both arrays as the routing to replay (moeSelOverride / moeWtsOverride, mlp.go:53-56). */
+int or_decode_multi_step_traced(const or_model *m, int B, const float *emb, or_cache **caches, float *logits, int *moe_idx_trace,
+                                float *moe_wts_trace /* [B][layers][top_k] or NULL */, int replay);
 
 #ifdef __cplusplus
 }

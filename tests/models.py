@@ -17,6 +17,21 @@ def moe_cfg(n_layers=2, hidden=256, n_heads=4, n_kv=2, head_dim=64, n_experts=8,
     return c
 
 
+class LazyEmbedding:
+    """Embedding rows generated on demand (row t from its own seed): a 128k x 4096 f32 table is 2 GB nobody needs whole."""
+
+    def __init__(self, seed, vocab, hidden, sigma):
+        self.seed, self.shape, self.sigma = seed, (vocab, hidden), sigma
+
+    def row(self, t):
+        return synth.normal(self.seed * 1000003 + int(t), self.shape[1], self.sigma)
+
+    def __getitem__(self, idx):
+        if np.ndim(idx) == 0:
+            return self.row(idx)
+        return np.stack([self.row(t) for t in idx])
+
+
 class Pair:
     """The same synthetic model as an oracle model and (when dev is given) a resident GPU model."""
 
@@ -27,7 +42,10 @@ class Pair:
         nE = cfg.get("n_experts", 0)
         inv = inv_freq(hd, cfg["theta"])
         self.gpu = capi.Model(dev, cfg, inv) if dev is not None else None
-        self.emb = synth.normal(seed * 1000 + 999, V * H, sigma).reshape(V, H)
+        if V * H > (1 << 26):
+            self.emb = LazyEmbedding(seed * 1000 + 999, V, H, sigma)
+        else:
+            self.emb = synth.normal(seed * 1000 + 999, V * H, sigma).reshape(V, H)
         s = [seed * 1000]
 
         def nxt():

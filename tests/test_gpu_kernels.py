@@ -74,6 +74,18 @@ def test_gemm_q4k_fused_gate_up(dev):
     assert rel_err(got, want) < 8e-3  # a product of two GEMM outputs: both factors carry the f16 operand rounding
 
 
+@pytest.mark.parametrize("M", [1, 9, 32, 40])
+def test_fused_gate_up_kernel(dev, M):
+    """The decode step's single-launch gate|up + SwiGLU + quantization kernel, on its own."""
+    from tests.test_gpu_baseline_shapes import check_fused
+    I, K = 512, 1024
+    g, u = synth.q4k_normal(1, I, K, 0.05), synth.q4k_normal(2, I, K, 0.05)
+    a = synth.normal(3, M * K).reshape(M, K)
+    gate = ob.matmul(ob.WMat(ob.OR_Q4K, I, K, g, act_group=32), a)
+    up = ob.matmul(ob.WMat(ob.OR_Q4K, I, K, u, act_group=32), a)
+    check_fused(dev.gateup_q4k_quant(g, u, I, K, a), gate, up)
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 64, 128), (7, 256, 896), (32, 1024, 4096)])
 def test_gemm_w8a8(dev, M, N, K):
     q, s = synth.w8a8_normal(5, N, K)
