@@ -6,6 +6,9 @@ Q4_K model (BASELINE.json configs[3], the configuration its metric is quoted on)
 table) are resident in HBM before the timed region; the greedy chain runs on the device (argmax -> embedding gather).
 Prints ONE JSON line with the whole-job tok/s, the roofline of the dominant kernel and a CPU baseline (the oracle's
 restatement of goinfer's CPU path, timed on this box's host cores on a bounded sample of the same workload).
+
+--workload c2 | c3 | c5 runs the other measurement configurations BASELINE.json names instead (the Q4_K GEMM microbench, the
+ragged attention microbench, the Qwen3-MoE-shaped step) and prints one line of the same form for that workload.
 """
 import argparse
 import json
@@ -47,19 +50,11 @@ def cpu_baseline(res, cfg, lens, kept_kv, threads):
     om = ob.OracleModel(c, layers, res.final_norm, head, inv_freq(cfg["head_dim"], cfg["theta"]))
     B = len(lens)
     caches = []
-    import ctypes as C
-    kvd = cfg["n_kv"] * cfg["head_dim"]
-    L = ob.lib()
     for i, n in enumerate(lens):
         cp = om.new_cache(int(n) + CPU_MAX_STEPS + 2)
-        # fill the oracle cache rows directly (f16-narrowed as the cache stores them)
-        cs = C.cast(cp, C.POINTER(_OrCache)).contents
         for l in range(nL):
             k, v = kept_kv[l]
-            for arr, dst in ((k, cs.k[l]), (v, cs.v[l])):
-                h = arr[:n].astype(np.float16).astype(np.float32)  # values are N(0,1): RNE and half-up differ on ties only
-                C.memmove(dst, h.ctypes.data, h.nbytes)
-        cs.pos = int(n)
+            om.cache_upload(cp, l, 0, k[:n], v[:n])  # UploadKV: narrowed to f16 as the cache stores it
         caches.append(cp)
     ids = np.arange(B) * 977 % cfg["vocab"]
     emb = res.embed_rows(ids)
@@ -86,14 +81,7 @@ def cpu_baseline(res, cfg, lens, kept_kv, threads):
     return B / full, sample
 
 
-import ctypes as _C  # noqa: E402
-
-
-class _OrCache(_C.Structure):
-    _fields_ = [("pos", _C.c_int), ("cap", _C.c_int), ("k", _C.POINTER(_C.c_void_p)), ("v", _C.POINTER(_C.c_void_p))]
-
-
-def main():
+def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=128)
@@ -102,10 +90,17 @@ def main():
     ap.add_argument("--batch", type=int, default=32)
     ap.add_argument("--seed", type=int, default=1234)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--workload", default="c4", choices=["c4", "c2", "c3", "c5"],
+                    help="c4 (default): the Llama-3-8B-shape step the metric is quoted on; c2: Q4_K GEMM microbench; c3: ragged "
+                         "attention microbench; c5: Qwen3-MoE-shape step")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this backend is single-GPU (goinfer has no collective path); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+    return args
+
+
+def run_c4(args):
 
     from goinfer_amd import capi, workloads
 
@@ -198,4 +193,10 @@ def main():
 
 if __name__ == "__main__":
     T0 = time.time()
-    main()
+    _args = parse_args()
+    if _args.workload == "c4":
+        run_c4(_args)
+    else:
+        import bench_micro
+        bench_micro.T0 = T0
+        {"c2": bench_micro.run_c2, "c3": bench_micro.run_c3, "c5": bench_micro.run_c5}[_args.workload](_args)

@@ -1,0 +1,259 @@
+"""The other measurement configurations of the decode path (bench.py --workload c2|c3|c5): one JSON line each, same form as
+the default workload's. Inputs are synthetic and resident in HBM before the timed region; times are HIP events on the launch
+stream; bytes are the algorithmic bytes of the call (every weight byte once, every KV byte once per sequence)."""
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+T0 = time.time()
+
+
+def log(msg):
+    print("[bench %6.1fs] %s" % (time.time() - T0, msg), file=sys.stderr, flush=True)
+
+
+def threads():
+    return min(16, len(os.sched_getaffinity(0)))
+
+
+def emit(out):
+    print(json.dumps(out, default=float))
+
+
+def base_line(metric, value, unit, steps, warmup, ms, workload, data, extra_cfg=None):
+    cfg = {"workload": workload}
+    cfg.update(extra_cfg or {})
+    return {"metric": metric, "value": round(value, 1), "unit": unit, "n_gpus": 1, "steps": steps, "warmup": warmup,
+            "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": data,
+            "config": cfg}
+
+
+# ------------------------------------------------------------------------------------------------------------ C2
+def run_c2(args):
+    """Q4_K dequant-GEMM: up 14336x4096, down 4096x14336, fused gate|up + SwiGLU + quantization; M in {1,4,16,32,64}.
+    A step is one GEMM call (M = 64 is two passes of 32 rows, as the step batches rows)."""
+    from goinfer_amd import capi
+    steps, warmup = (args.steps if args.steps != 128 else 100), (args.warmup if args.warmup != 8 else 20)
+    dev = capi.Device(0)
+    W = 14336 * (4096 // 256) * 144
+    cases = []
+    for name, kern, N, K, wbytes in (("up 14336x4096", "gemm_q4k", 14336, 4096, W), ("down 4096x14336", "gemm_q4k", 4096, 14336, W),
+                                     ("fused gate|up 2x14336x4096 + SwiGLU", "gateup", 14336, 4096, 2 * W)):
+        for M in (1, 4, 16, 32, 64):
+            ms = dev.bench_kernel(kern, [N, K, M, 8], warmup, steps)  # 8 weight copies round-robin: nothing stays in the 256 MB cache
+            t = float(np.median(ms))
+            nbytes = wbytes + 4 * M * K + (4 * M * N if kern == "gemm_q4k" else 2 * M * N)  # weights + activations in + result out
+            flops = 2.0 * M * N * K * (2 if kern == "gateup" else 1)
+            cases.append({"case": name, "M": M, "us": round(t * 1e3, 2), "GBs": round(nbytes / t / 1e6, 1), "TFLOPs": round(flops / t / 1e9, 1),
+                          "bytes": int(nbytes)})
+            log("%s M=%d: %.1f us, %.0f GB/s" % (name, M, t * 1e3, nbytes / t / 1e6))
+    head = next(c for c in cases if c["case"].startswith("fused") and c["M"] == 32)
+    out = base_line("Q4_K dequant-GEMM achieved HBM GB/s (fused gate|up SwiGLU at M=32; all cases listed)", head["GBs"], "GB/s", steps, warmup,
+                    head["us"] / 1e3, "configs[1]: Q4_K GEMM 14336x4096 / 4096x14336 / fused gate|up, M in {1,4,16,32,64}",
+                    "synthetic: random Q4_K super-blocks with sane f16 scales, 8 weight copies used round-robin", {"cases": cases})
+    out["roofline"] = {"bound": "hbm", "achieved": head["GBs"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(head["GBs"] / HBM_PEAK_GBS, 4),
+                       "traffic": None, "kernel": "rd_k_gemm_q4k_gateup", "avg_launch_ms": round(head["us"] / 1e3, 5),
+                       "algorithmic_bytes_per_launch": head["bytes"]}
+    cpu = None
+    if not args.no_cpu:
+        from goinfer_amd import synth
+        from oracle import binding as ob
+        ob.set_threads(threads())
+        g, u = synth.q4k_normal(1, 14336, 4096), synth.q4k_normal(2, 14336, 4096)
+        wg, wu = ob.WMat(ob.OR_Q4K, 14336, 4096, g, act_group=32), ob.WMat(ob.OR_Q4K, 14336, 4096, u, act_group=32)
+        a = synth.normal(3, 32 * 4096, 1.0).reshape(32, 4096)
+        ob.swiglu(ob.matmul(wg, a), ob.matmul(wu, a))
+        n, t = 0, 0.0
+        while t < 10.0 and n < 400:
+            t0 = time.time()
+            ob.swiglu(ob.matmul(wg, a), ob.matmul(wu, a))
+            t += time.time() - t0
+            n += 1
+        cpu = {"value": round(head["bytes"] / (t / n) / 1e9, 2), "unit": "GB/s", "cores": threads(), "kind": "port",
+               "sample": "oracle gate and up matmuls + SwiGLU at M=32, %d calls (%.1f s)" % (n, t)}
+    out["cpu_baseline"] = cpu
+    dev.close()
+    emit(out)
+
+
+# ------------------------------------------------------------------------------------------------------------ C3
+def run_c3(args):
+    """Ragged flash-decode attention: 64 sequences, KV lengths U[128,8192], 32 Q / 8 KV heads, head_dim 128, f16 KV; once without
+    softcap and once with softcap 50. A step is one ragged call (one layer)."""
+    from goinfer_amd import capi
+    steps, warmup = (args.steps if args.steps != 128 else 100), (args.warmup if args.warmup != 8 else 20)
+    nH, nKV, hd, nseq = 32, 8, 128, 64
+    lens = np.random.default_rng(args.seed).integers(128, 8193, nseq).astype(np.int32)
+    scale = float(1.0 / np.sqrt(hd))
+    kv_bytes = float(lens.sum()) * 2 * nKV * hd * 2
+    io_bytes = 2 * nseq * nH * hd * 4
+    dev = capi.Device(0)
+    res = {}
+    for cap in (0.0, 50.0):
+        tot, part = dev.bench_attn(lens, nH, nKV, hd, scale, cap, warmup, steps)
+        res[cap] = (float(np.median(tot)), float(np.median(part)))
+        log("softcap %g: call %.1f us (%.0f GB/s), partial kernels %.1f us (%.0f GB/s)" % (
+            cap, res[cap][0] * 1e3, (kv_bytes + io_bytes) / res[cap][0] / 1e6, res[cap][1] * 1e3, kv_bytes / res[cap][1] / 1e6))
+    t, tp = res[0.0]
+    gbs = (kv_bytes + io_bytes) / t / 1e6
+    out = base_line("ragged flash-decode attention achieved HBM GB/s (64 sequences, KV U[128,8192], 32/8 heads, head_dim 128)", gbs, "GB/s", steps,
+                    warmup, t, "configs[2]: ragged attention microbench", "synthetic: uniform [-2,2) f16 KV in a paged pool with a scattered block table, f32 q",
+                    {"n_seq": nseq, "kv_positions": int(lens.sum()), "kv_len_min": int(lens.min()), "kv_len_max": int(lens.max()), "seed": args.seed,
+                     "cases": [{"softcap": c, "call_us": round(v[0] * 1e3, 2), "call_GBs": round((kv_bytes + io_bytes) / v[0] / 1e6, 1),
+                                "partial_kernels_us": round(v[1] * 1e3, 2), "partial_kernels_GBs": round(kv_bytes / v[1] / 1e6, 1)} for c, v in res.items()]})
+    # the partial kernel is launched once per group of 32 rows: two launches per call here
+    per_launch = (kv_bytes + nseq * nH * hd * 4) / 2
+    out["roofline"] = {"bound": "hbm", "achieved": round(per_launch / (tp / 2) / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                       "frac": round(per_launch / (tp / 2) / 1e6 / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "rd_k_attn_partial",
+                       "avg_launch_ms": round(tp / 2, 5), "algorithmic_bytes_per_launch": int(per_launch)}
+    cpu = None
+    if not args.no_cpu:
+        from goinfer_amd import synth
+        from oracle import binding as ob
+        ob.set_threads(threads())
+        pick = list(range(0, nseq, 8))
+        kvd = nKV * hd
+        ops = []
+        for i in pick:
+            n = int(lens[i])
+            ops.append((synth.normal(990 + i, nH * hd, 1.0), ob.f16_round_trip(synth.normal(900 + i, n * kvd, 1.0).reshape(n, kvd)),
+                        ob.f16_round_trip(synth.normal(950 + i, n * kvd, 1.0).reshape(n, kvd)), n))
+        t_cpu, pos, reps = 0.0, 0, 0
+        while t_cpu < 10.0 and reps < 2000:
+            for q, k, v, n in ops:
+                t0 = time.time()
+                ob.attend(q, k, v, n, nH, nKV, hd, scale, 0.0)
+                t_cpu += time.time() - t0
+                pos += n
+            reps += 1
+        cpu = {"value": round(pos * 2 * kvd * 2 / t_cpu / 1e9, 3), "unit": "GB/s", "cores": threads(), "kind": "port",
+               "sample": "oracle attention (f64 accumulate, heads in parallel) on %d of the %d sequences, %d passes, %d positions (%.1f s)" % (
+                   len(pick), nseq, reps, pos, t_cpu)}
+    out["cpu_baseline"] = cpu
+    dev.close()
+    emit(out)
+
+
+# ------------------------------------------------------------------------------------------------------------ C5
+def run_c5(args):
+    """Qwen3-MoE-30B-A3B shape: 48 layers, 128 experts top-8 (int4-g32 experts, f32 router), Q4_K attention projections, int8 head;
+    16 ragged slots, ctx U[256,2048], greedy decode. A step is one decode step of the batch."""
+    from goinfer_amd import capi, workloads
+    layers = args.layers if args.layers != 32 else 48
+    B = args.batch if args.batch != 32 else 16
+    steps, warmup = (args.steps if args.steps != 128 else 64), (args.warmup if args.warmup != 8 else 4)
+    cfg = workloads.qwen3_moe_cfg(layers)
+    rng = np.random.default_rng(args.seed)
+    lens = rng.integers(256, 2049, B).astype(np.int64)
+    ids0 = rng.integers(0, cfg["vocab"], B).astype(np.int32)
+    cap = int(lens.max()) + steps + warmup + 8
+    dev = capi.Device(0)
+    log("building %s, %d layers" % (cfg["name"], layers))
+    res = workloads.Resident(dev, cfg, seed=args.seed, slots=B, ctx_cap=cap, keep_layers=0 if args.no_cpu else 1, progress=log)
+    kept_kv = res.prefill_kv(lens, progress=log)
+    slots = np.arange(B, dtype=np.int32)
+    dev.sync()
+    ms = res.model.bench_steps(slots, lens, ids0, warmup, steps)
+    dev.sync()
+    tok_s = B * steps / (float(ms.sum()) / 1e3)
+    log("steps: %.3f ms mean, %.3f ms median" % (ms.mean(), float(np.median(ms))))
+    # distinct experts per layer from the last step's recorded routing
+    idx = res.model.last_moe_indices(B)  # [B][layers][k]
+    distinct = [len(set(idx[:, l, :].ravel().tolist())) for l in range(layers)]
+    ebytes = workloads.expert_bytes(cfg)
+    mid = lens + warmup + steps // 2
+    kv_pos = workloads.kv_bytes_per_position(cfg)
+    kv_read = float((mid + 1).sum()) * kv_pos
+    w_bytes = workloads.weight_bytes(cfg)
+    exp_bytes = float(sum(distinct)) * ebytes
+    step_bytes = w_bytes + exp_bytes + kv_read + B * kv_pos
+    step_gbs = step_bytes / (ms.mean() / 1e3) / 1e9
+    pos_prof = (lens + warmup + steps).astype(np.int32)
+    prof = {}
+    for rep in range(3):
+        for k, (t, n) in res.model.bench_profile(slots, pos_prof + rep, ids0).items():
+            a = prof.setdefault(k, [0.0, 0])
+            a[0] += t
+            a[1] += n
+    classes = {k: {"ms_per_step": round(v[0] / 3, 4), "launches_per_step": v[1] // 3} for k, v in prof.items()}
+    # dominant kernel: the expert-major grouped GEMM (two launches per layer: gate|up of every touched expert, then down)
+    idx2 = res.model.last_moe_indices(B)
+    d2 = float(sum(len(set(idx2[:, l, :].ravel().tolist())) for l in range(layers)))
+    g_ms = prof["moe_gemm"][0] / prof["moe_gemm"][1]
+    per_launch = d2 * ebytes / (2 * layers)
+    out = base_line("batch-16 decode tok/s, Qwen3-MoE-30B-A3B shape (int4-g32 experts); achieved HBM GB/s vs peak", tok_s, "tok/s", steps, warmup,
+                    float(ms.mean()), "configs[4]: %s, %d layers, B=%d ragged, ctx U[256,2048], greedy decode" % (cfg["name"], layers, B),
+                    "synthetic: N(0,0.02) weights (Q4_K projections, int4-g32 experts, f32 router, int8 head), N(0,1) KV, random token ids",
+                    {"batch": B, "ctx_min": int(lens.min()), "ctx_max": int(lens.max()), "ctx_mean": float(lens.mean()), "seed": args.seed,
+                     "distinct_experts_per_layer_mean": round(float(np.mean(distinct)), 1)})
+    out["step_hbm"] = {"algorithmic_bytes_per_step": int(step_bytes), "achieved_GBs": round(step_gbs, 1), "frac_of_peak": round(step_gbs / HBM_PEAK_GBS, 4),
+                       "dense_weight_bytes": int(w_bytes), "expert_bytes": int(exp_bytes), "kv_read_bytes": int(kv_read)}
+    out["roofline"] = {"bound": "hbm", "achieved": round(per_launch / (g_ms / 1e3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                       "frac": round(per_launch / (g_ms / 1e3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "rd_k_gemm_w4a8_moe",
+                       "avg_launch_ms": round(g_ms, 5), "algorithmic_bytes_per_launch": int(per_launch)}
+    out["kernel_classes"] = classes
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline_moe(res, cfg, lens, kept_kv)
+    out["cpu_baseline"] = cpu
+    res.close()
+    dev.close()
+    emit(out)
+
+
+def cpu_baseline_moe(res, cfg, lens, kept_kv):
+    """The oracle's decodeMultiStep on the first layer of the same model (all 128 experts resident), the same ragged batch and KV,
+    greedy steps for about ten seconds; the per-layer cost scaled to the full depth."""
+    from goinfer_amd.workloads import inv_freq
+    from oracle import binding as ob
+    ob.set_threads(threads())
+    layers = []
+    for kp in res.kept:
+        lw = {p: ob.WMat(ob.OR_Q4K, kp[p][1], kp[p][2], kp[p][0], act_group=32) for p in ("q", "k", "v", "o")}
+        for n in ("attn_norm", "ffn_norm", "q_norm", "k_norm"):
+            lw[n] = kp[n]
+        lw["router"] = ob.WMat.from_f32(kp["router"])
+        for proj in ("gate", "up", "down"):
+            lw["exp_" + proj] = [ob.WMat(ob.OR_W4A8, ex[proj][2], ex[proj][3], ex[proj][0], ex[proj][1], act_group=32) for ex in kp["experts"]]
+        layers.append(lw)
+    nL = len(layers)
+    c = dict(cfg)
+    c.update(n_layers=nL, kv_f16=1)
+    hq, hs = res.head
+    head = ob.WMat(ob.OR_W8A8, hq.shape[0], hq.shape[1], hq, hs, act_group=32)
+    om = ob.OracleModel(c, layers, res.final_norm, head, inv_freq(cfg["head_dim"], cfg["theta"]))
+    B, MAXS = len(lens), 64
+    caches = []
+    for i, n in enumerate(lens):
+        cp = om.new_cache(int(n) + MAXS + 2)
+        for l in range(nL):
+            k, v = kept_kv[l]
+            om.cache_upload(cp, l, 0, k[:n], v[:n])
+        caches.append(cp)
+    emb = res.embed_rows(np.arange(B) * 977 % cfg["vocab"])
+    om.step(emb, caches)
+    n_steps, t_step = 0, 0.0
+    while n_steps < MAXS - 1 and t_step < 10.0:
+        t0 = time.time()
+        logits = om.step(emb, caches)
+        t_step += time.time() - t0
+        n_steps += 1
+        emb = res.embed_rows(np.array([ob.argmax(r) for r in logits]))
+    t0 = time.time()
+    for _ in range(3):
+        ob.matmul(head, emb)
+    t_head = (time.time() - t0) / 3
+    for cp in caches:
+        om.free_cache(cp)
+    per_layer = max(t_step / n_steps - t_head, 1e-9) / nL
+    full = per_layer * cfg["n_layers"] + t_head
+    return {"value": round(B / full, 3), "unit": "tok/s", "cores": threads(), "kind": "port",
+            "sample": "oracle decodeMultiStep, %d of %d layers + int8 head, B=%d at the run's context lengths, %d greedy steps (%.1f s), "
+                      "per-layer cost scaled to %d layers" % (nL, cfg["n_layers"], B, n_steps, t_step, cfg["n_layers"])}

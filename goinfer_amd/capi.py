@@ -20,7 +20,7 @@ EXPORTS = [
     "rd_model_upload_q4k", "rd_model_upload_w8a8", "rd_model_upload_w4a8", "rd_model_upload_f32", "rd_model_finalize",
     "rd_kv_configure", "rd_kv_upload", "rd_kv_truncate", "rd_kv_reset", "rd_step_batch", "rd_forward",
     "rd_last_moe_indices", "rd_model_upload_embedding", "rd_bench_steps", "rd_bench_profile", "rd_bench_class_count",
-    "rd_bench_class_name", "rd_bench_kernel", "rd_gateup_q4k_quant", "rd_moe_replay",
+    "rd_bench_class_name", "rd_bench_kernel", "rd_gateup_q4k_quant", "rd_moe_replay", "rd_bench_attn",
 ]
 
 
@@ -171,6 +171,13 @@ class Device:
         inv = np.ascontiguousarray(inv_freq, dtype=np.float64)
         check(lib().rd_rope(self.h, _p(v), v.shape[0], heads, head_dim, _p(pos), _p(inv)), "rd_rope")
         return v
+
+    def bench_attn(self, lens, n_h, n_kv, hd, scale, softcap, warmup, iters):
+        lens = np.ascontiguousarray(lens, dtype=np.int32)
+        tot, part = np.empty(iters, np.float32), np.empty(iters, np.float32)
+        check(lib().rd_bench_attn(self.h, len(lens), _p(lens), n_h, n_kv, hd, C.c_float(scale), C.c_float(softcap), warmup, iters,
+                                  _p(tot), _p(part)), "rd_bench_attn")
+        return tot, part
 
     def bench_kernel(self, name, args, warmup, iters):
         a = np.ascontiguousarray(args, dtype=np.int64)

@@ -2,6 +2,8 @@
 // already resident in HBM when the timed region starts.
 #include "model.h"
 #include <algorithm>
+#include <memory>
+#include <numeric>
 #include <string.h>
 #include <string>
 
@@ -84,11 +86,11 @@ extern "C" const char *rd_bench_class_name(int c) {
 extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *args, int n_args, int warmup, int iters, float *ms_out) {
     if (!d || !name || !args || iters <= 0 || !ms_out) return RD_ERR_ARG;
     std::string nm(name);
-    if (nm == "gemm_q4k" && n_args >= 4 && (args[0] % 32 || args[1] % 256 || args[0] <= 0 || args[1] <= 0 || args[2] < 1 || args[2] > 32)) {
+    if (nm == "gemm_q4k" && n_args >= 4 && (args[0] % 32 || args[1] % 256 || args[0] <= 0 || args[1] <= 0 || args[2] < 1 || args[2] > 64)) {
         rd_set_error("gemm_q4k bench: bad shape");
         return RD_ERR_ARG;
     }
-    if (nm == "gateup" && n_args >= 4 && (args[0] <= 0 || args[0] % 64 || args[1] <= 0 || args[1] % 256 || args[2] < 1 || args[2] > 32)) {
+    if (nm == "gateup" && n_args >= 4 && (args[0] <= 0 || args[0] % 64 || args[1] <= 0 || args[1] % 256 || args[2] < 1 || args[2] > 64)) {
         rd_set_error("gateup bench: bad shape");
         return RD_ERR_ARG;
     }
@@ -131,7 +133,7 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
         for (int i = 0; i < warmup + iters && !rc; i++) {
             const DevWeight &w = ws[(size_t)i % ws.size()];
             if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup)], d->stream);
-            rc = launch_gemm(d, w, Xp.p, P.as<float>(), M, nullptr);
+            for (int m0 = 0; m0 < M && !rc; m0 += 32) rc = launch_gemm(d, w, Xp.p, P.as<float>(), std::min(32, M - m0), nullptr); // rows in groups of 32
             if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup) + 1], d->stream);
         }
         if (!rc) rc = d->sync();
@@ -163,8 +165,9 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
         for (int i = 0; i < warmup + iters && !rc; i++) {
             const DevWeight &w = ws[(size_t)i % ws.size()];
             if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup)], d->stream);
-            rc = d->launch(d->k.gemm_q4k_gateup, (unsigned)(I / 64), 1, 1, GATEUP_THREADS, (const void *)w.tiled, (const void *)Xp.p, Xo.as<uint8_t>(), (int)PANEL_Q4K,
-                           I, K / 256, M);
+            for (int m0 = 0; m0 < M && !rc; m0 += 32)
+                rc = d->launch(d->k.gemm_q4k_gateup, (unsigned)(I / 64), 1, 1, GATEUP_THREADS, (const void *)w.tiled, (const void *)Xp.p, Xo.as<uint8_t>(),
+                               (int)PANEL_Q4K, I, K / 256, std::min(32, M - m0));
             if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup) + 1], d->stream);
         }
         if (!rc) rc = d->sync();
@@ -221,5 +224,120 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
         ms_out[i] = ms;
     }
     for (auto &e : ev) (void)d->hip->EventDestroy(e);
+    return rc;
+}
+
+// The ragged flash-decode attention of one layer over a synthetic paged f16 KV pool (uniform [-2,2) values, scattered
+// block table), rows in groups of 32 as the step batches them. ms_total[iters]: the whole call (partial + combine kernels
+// of every group); ms_partial[iters] (may be NULL): the partial kernels alone. HIP events on the launch stream.
+extern "C" int rd_bench_attn(rd_device *d, int n_seq, const int *len, int n_h, int n_kv, int hd, float scale, float softcap, int warmup, int iters,
+                             float *ms_total, float *ms_partial) {
+    if (!d || !len || n_seq <= 0 || iters <= 0 || !ms_total) return RD_ERR_ARG;
+    if (n_kv <= 0 || n_h % n_kv || n_h / n_kv > 16 || (hd != 64 && hd != 128)) {
+        rd_set_error("rd_bench_attn declines: head_dim must be 64 or 128 and the GQA group <= 16");
+        return RD_DECLINED;
+    }
+    struct Item {
+        int row, kvh, b0, b1;
+    };
+    const int qd = n_h * hd, G = n_h / n_kv;
+    int maxBlocks = 0;
+    long totalBlocks = 0;
+    for (int i = 0; i < n_seq; i++) {
+        if (len[i] <= 0) return RD_ERR_ARG;
+        int nb = (len[i] + 63) / 64;
+        maxBlocks = std::max(maxBlocks, nb), totalBlocks += nb;
+    }
+    std::vector<int> tab((size_t)n_seq * maxBlocks, 0);
+    {
+        long nb = totalBlocks, stride = std::max(1L, (long)(nb * 0.618));
+        while (stride < nb && std::gcd(stride, nb) != 1) stride++;
+        if (stride >= nb) stride = 1;
+        long idx = 0;
+        for (int i = 0; i < n_seq; i++)
+            for (int b = 0; b < (len[i] + 63) / 64; b++, idx++) tab[(size_t)i * maxBlocks + b] = 1 + (int)((idx * stride) % nb);
+    }
+    const size_t poolHalves = (size_t)(totalBlocks + 1) * n_kv * 64 * hd;
+    DevBuf Kp(d), Vp(d), T(d), Q(d), O(d);
+    RC(Kp.alloc(poolHalves * 2));
+    RC(Vp.alloc(poolHalves * 2));
+    RC(T.alloc(sizeof(int) * tab.size()));
+    RC(Q.alloc(sizeof(float) * (size_t)n_seq * qd));
+    RC(O.alloc(sizeof(float) * (size_t)n_seq * qd));
+    RC(d->h2d(T.p, tab.data(), sizeof(int) * tab.size()));
+    RC(d->launch(d->k.fill_f16, 2048, 1, 1, 256, Kp.as<uint16_t>(), poolHalves, 11u));
+    RC(d->launch(d->k.fill_f16, 2048, 1, 1, 256, Vp.as<uint16_t>(), poolHalves, 12u));
+    RC(d->launch(d->k.fill_f32, 256, 1, 1, 256, Q.as<float>(), (size_t)n_seq * qd, 13u));
+    struct Group {
+        int r0, rows, nItems;
+        DevBuf L, S, I, St, P;
+        Group(rd_device *dv) : r0(0), rows(0), nItems(0), L(dv), S(dv), I(dv), St(dv), P(dv) {}
+    };
+    std::vector<std::unique_ptr<Group>> groups;
+    for (int r0 = 0; r0 < n_seq; r0 += 32) {
+        auto g = std::make_unique<Group>(d);
+        g->r0 = r0, g->rows = std::min(32, n_seq - r0);
+        std::vector<Item> items;
+        std::vector<int> start((size_t)g->rows * n_kv + 1), slots((size_t)g->rows), lens((size_t)g->rows);
+        for (int i = 0; i < g->rows; i++) {
+            const int nb = (len[r0 + i] + 63) / 64, chunk = attn_chunk_blocks(nb);
+            slots[(size_t)i] = r0 + i, lens[(size_t)i] = len[r0 + i];
+            for (int h = 0; h < n_kv; h++) {
+                start[(size_t)i * n_kv + h] = (int)items.size();
+                for (int b0 = 0; b0 < nb; b0 += chunk) items.push_back({i, h, b0, std::min(nb, b0 + chunk)});
+            }
+        }
+        start[(size_t)g->rows * n_kv] = (int)items.size();
+        g->nItems = (int)items.size();
+        RC(g->L.alloc(sizeof(int) * lens.size()));
+        RC(g->S.alloc(sizeof(int) * slots.size()));
+        RC(g->I.alloc(sizeof(Item) * items.size()));
+        RC(g->St.alloc(sizeof(int) * start.size()));
+        RC(g->P.alloc(sizeof(float) * items.size() * G * (hd + 2)));
+        RC(d->h2d(g->L.p, lens.data(), sizeof(int) * lens.size()));
+        RC(d->h2d(g->S.p, slots.data(), sizeof(int) * slots.size()));
+        RC(d->h2d(g->I.p, items.data(), sizeof(Item) * items.size()));
+        RC(d->h2d(g->St.p, start.data(), sizeof(int) * start.size()));
+        groups.push_back(std::move(g));
+    }
+    RC(d->sync());
+    const size_t nG = groups.size();
+    std::vector<hipEvent_t> ev((size_t)iters * 2), evp((size_t)iters * nG * 2);
+    for (auto &e : ev) HIPCHK(EventCreate(&e));
+    for (auto &e : evp) HIPCHK(EventCreate(&e));
+    int rc = RD_OK;
+    for (int i = 0; i < warmup + iters && !rc; i++) {
+        const bool timed = i >= warmup;
+        const size_t t = (size_t)(i - warmup);
+        if (timed) (void)d->hip->EventRecord(ev[2 * t], d->stream);
+        for (size_t gi = 0; gi < nG && !rc; gi++) {
+            Group &g = *groups[gi];
+            if (timed) (void)d->hip->EventRecord(evp[(t * nG + gi) * 2], d->stream);
+            rc = d->launch(d->k.attn_partial, (unsigned)g.nItems, 1, 1, 64, (const void *)g.I.p, (const int *)g.L.p, (const int *)g.S.p, (const int *)T.p, maxBlocks,
+                           (const uint16_t *)Kp.p, (const uint16_t *)Vp.p, (const float *)((const float *)Q.p + (size_t)g.r0 * qd), g.P.as<float>(), n_h, n_kv, hd, scale,
+                           softcap);
+            if (timed) (void)d->hip->EventRecord(evp[(t * nG + gi) * 2 + 1], d->stream);
+            if (!rc)
+                rc = d->launch(d->k.attn_combine, (unsigned)n_h, (unsigned)g.rows, 1, (unsigned)(ATTN_PIECES * hd / 4), (const float *)g.P.p, (const int *)g.St.p,
+                               (float *)((float *)O.p + (size_t)g.r0 * qd), n_h, n_kv, hd);
+        }
+        if (timed) (void)d->hip->EventRecord(ev[2 * t + 1], d->stream);
+    }
+    if (!rc) rc = d->sync();
+    for (int i = 0; i < iters; i++) {
+        float ms = 0.f, mp = 0.f;
+        if (!rc) {
+            (void)d->hip->EventElapsedTime(&ms, ev[2 * (size_t)i], ev[2 * (size_t)i + 1]);
+            for (size_t gi = 0; gi < nG; gi++) {
+                float x = 0.f;
+                (void)d->hip->EventElapsedTime(&x, evp[((size_t)i * nG + gi) * 2], evp[((size_t)i * nG + gi) * 2 + 1]);
+                mp += x;
+            }
+        }
+        ms_total[i] = ms;
+        if (ms_partial) ms_partial[i] = mp;
+    }
+    for (auto &e : ev) (void)d->hip->EventDestroy(e);
+    for (auto &e : evp) (void)d->hip->EventDestroy(e);
     return rc;
 }

@@ -25,7 +25,7 @@ struct Kernels {
     hipFunction_t retile_w8a8, gemm_w8a8, retile_w4a8, gemm_w4a8;
     hipFunction_t gemm_q4k_gateup;
     hipFunction_t kv_store, qkv_rope_store, attn_partial, attn_combine, attn_combine_quant;
-    hipFunction_t rmsnorm, rope, argmax_rows, argmax_final, matmul_f32, moe_route, gemm_w4a8_moe, moe_swiglu_quant, moe_fold, embed_rows, copy16, barrier_probe, unpanel_q4k;
+    hipFunction_t rmsnorm, rope, argmax_rows, argmax_final, matmul_f32, moe_route, gemm_w4a8_moe, moe_swiglu_quant, moe_fold, embed_rows, copy16, barrier_probe, unpanel_q4k, fill_f16, fill_f32;
 };
 
 struct rd_device {
@@ -67,7 +67,7 @@ constexpr unsigned GEMM_THREADS = 320, GATEUP_THREADS = 640;
 // cut into at most ATTN_PIECES pieces. The cut depends on the sequence's own length only, never on what else is in the
 // batch: the partial results are merged in piece order, so this is what keeps a row computed in a batch bit-identical to
 // the same row computed alone.
-constexpr int ATTN_PIECES = 16;
+constexpr int ATTN_PIECES = 16; // = RD_ATTN_PIECES of the combine kernels
 inline int attn_chunk_blocks(int nb) { return (nb + ATTN_PIECES - 1) / ATTN_PIECES; }
 
 // split-K plan of one GEMM launch

@@ -24,7 +24,7 @@ extern "C" int rd_model_create(rd_device *d, const rd_model_desc *desc, rd_model
         rd_set_error("rocm resident declines: needs hidden%%128==0 (<=8192), head_dim 64 or 128, GQA group <=16, vocab%%32==0");
         return RD_DECLINED;
     }
-    if (c.n_experts > 0 && (c.n_experts > 256 || c.top_k <= 0 || c.top_k > c.n_experts || c.expert_inter % 128)) {
+    if (c.n_experts > 0 && (c.n_experts > 256 || c.top_k <= 0 || c.top_k > c.n_experts || c.top_k > 64 || c.expert_inter % 128)) {
         rd_set_error("rocm resident declines: MoE needs <=256 experts and expert width %%128==0");
         return RD_DECLINED;
     }
@@ -467,17 +467,18 @@ static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
     int H = c.hidden, I = c.expert_inter, k = c.top_k, nE = c.n_experts;
     {
         Scope s(m, KC_MOE_ROUTER);
-        RC(d->launch(d->k.matmul_f32, (unsigned)((nE + 63) / 64), (unsigned)B, 1, 64, (const float *)m->normed, (const float *)l.router,
-                     m->router_logits, B, H, nE));
-        if (m->replay_B == B) { // replay a recorded routing (goinfer's moeSelOverride seam) instead of routing on these logits
+        int *trace = m->moe_idx_all + (size_t)layer * 32 * k;
+        if (m->replay_B == B) { // replay a recorded routing (goinfer's moeSelOverride seam) instead of routing on this hidden state
             RC(d->h2d(m->moe_idx, m->replay_idx[(size_t)layer].data(), sizeof(int) * (size_t)B * k));
             RC(d->h2d(m->moe_wgt, m->replay_wgt[(size_t)layer].data(), sizeof(float) * (size_t)B * k));
             RC(d->h2d(m->moe_rank, m->replay_rank[(size_t)layer].data(), (size_t)32 * nE));
+            RC(d->h2d(trace, m->replay_idx[(size_t)layer].data(), sizeof(int) * (size_t)B * k));
         } else {
-            RC(d->launch(d->k.moe_route, 1, 1, 1, 64, (const float *)m->router_logits, B, nE, k, c.norm_topk_prob, m->moe_idx, m->moe_wgt,
-                         m->moe_rank));
+            RC(d->launch(d->k.matmul_f32, (unsigned)((nE + 3) / 4), (unsigned)B, 1, 256, (const float *)m->normed, (const float *)l.router,
+                         m->router_logits, B, H, nE));
+            RC(d->launch(d->k.moe_route, (unsigned)B, 1, 1, 64, (const float *)m->router_logits, B, nE, k, c.norm_topk_prob, m->moe_idx, m->moe_wgt,
+                         m->moe_rank, trace));
         }
-        HIPCHK(MemcpyAsync(m->moe_idx_all + (size_t)layer * 32 * k, m->moe_idx, sizeof(int) * (size_t)B * k, hipMemcpyDeviceToDevice, d->stream));
     }
     size_t guStride = (size_t)(2 * I / 32) * (H / 128) * 2304, dnStride = (size_t)(H / 32) * (I / 128) * 2304;
     size_t xpStride = (size_t)(I / 128) * LIN_PANEL_BYTES;
@@ -590,7 +591,7 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
         }
         {
             Scope s(m, KC_ATTN_COMBINE);
-            RC(d->launch(d->k.attn_combine_quant, (unsigned)nH, (unsigned)B, 1, (unsigned)(HD / 4), (const float *)m->part, (const int *)m->itemStart,
+            RC(d->launch(d->k.attn_combine_quant, (unsigned)nH, (unsigned)B, 1, (unsigned)(ATTN_PIECES * HD / 4), (const float *)m->part, (const int *)m->itemStart,
                          m->XpB, panel_kind_for(l.o), nH, nKV, HD));
         }
         {

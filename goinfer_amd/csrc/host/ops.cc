@@ -159,7 +159,7 @@ extern "C" int rd_matmul_bt(rd_device *d, const float *a, const float *b, float 
     RC(D.alloc(sizeof(float) * (size_t)M * N));
     RC(d->h2d(A.p, a, sizeof(float) * (size_t)M * K));
     RC(d->h2d(B.p, b, sizeof(float) * (size_t)N * K));
-    RC(d->launch(d->k.matmul_f32, (unsigned)((N + 63) / 64), (unsigned)M, 1, 64, (const float *)A.p, (const float *)B.p, D.as<float>(), M, K, N));
+    RC(d->launch(d->k.matmul_f32, (unsigned)((N + 3) / 4), (unsigned)M, 1, 256, (const float *)A.p, (const float *)B.p, D.as<float>(), M, K, N));
     return d->d2h(dst, D.p, sizeof(float) * (size_t)M * N);
 }
 
@@ -200,8 +200,8 @@ extern "C" int rd_moe_route(rd_device *d, const float *logits, int T, int nE, in
     RC(I.alloc(sizeof(int) * (size_t)T * k));
     RC(W.alloc(sizeof(float) * (size_t)T * k));
     RC(d->h2d(L.p, logits, sizeof(float) * (size_t)T * nE));
-    RC(d->launch(d->k.moe_route, (unsigned)((T + 63) / 64), 1, 1, 64, (const float *)L.p, T, nE, k, norm, I.as<int>(), W.as<float>(),
-                 (signed char *)nullptr));
+    RC(d->launch(d->k.moe_route, (unsigned)T, 1, 1, 64, (const float *)L.p, T, nE, k, norm, I.as<int>(), W.as<float>(),
+                 (signed char *)nullptr, (int *)nullptr));
     RC(d->d2h(idx, I.p, sizeof(int) * (size_t)T * k));
     return d->d2h(wgt, W.p, sizeof(float) * (size_t)T * k);
 }
@@ -290,7 +290,7 @@ extern "C" int rd_attn_ragged(rd_device *d, int n_seq, const int *len, const int
         RC(d->h2d(St2.p, start.data(), sizeof(int) * start.size()));
         RC(d->launch(d->k.attn_partial, (unsigned)items.size(), 1, 1, 64, (const void *)I2.p, (const int *)L2.p, (const int *)S2.p, (const int *)T.p,
                      maxBlocks, (const uint16_t *)Kp.p, (const uint16_t *)Vp.p, (const float *)Q2.p, P2.as<float>(), n_h, n_kv, hd, scale, softcap));
-        RC(d->launch(d->k.attn_combine, (unsigned)n_h, (unsigned)rows, 1, (unsigned)hd, (const float *)P2.p, (const int *)St2.p, O2.as<float>(), n_h,
+        RC(d->launch(d->k.attn_combine, (unsigned)n_h, (unsigned)rows, 1, (unsigned)(ATTN_PIECES * hd / 4), (const float *)P2.p, (const int *)St2.p, O2.as<float>(), n_h,
                      n_kv, hd));
         RC(d->d2h(out + (size_t)r0 * qd, O2.p, sizeof(float) * (size_t)rows * qd));
     }

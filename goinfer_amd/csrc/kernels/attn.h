@@ -235,60 +235,50 @@ extern "C" __global__ __launch_bounds__(64) void rd_k_attn_partial(const AttnIte
         attn_partial_body<64>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, q, part, nH, nKV, scale, softcap, pbuf);
 }
 
-// Merge the partials of one (row, query head) in ascending item order (deterministic): out = sum O_i e^(m_i-M) / sum l_i e^(m_i-M).
-// itemStart[row*nKV+kvh] .. itemStart[row*nKV+kvh+1] are that pair's items. Grid (nH, rows), block HD threads.
-__device__ __forceinline__ float attn_combine_value(const float *__restrict__ part, const int *__restrict__ itemStart, int nH, int nKV, int HD,
-                                                    int m, int head, int d) {
-    int G = nH / nKV, kvh = head / G, g = head % G;
-    int i0 = itemStart[m * nKV + kvh], i1 = itemStart[m * nKV + kvh + 1];
-    float M = -INFINITY;
-    for (int i = i0; i < i1; i++) M = fmaxf(M, part[((size_t)i * G + g) * (HD + 2) + HD]);
-    float num = 0.f, den = 0.f;
-    for (int i = i0; i < i1; i++) {
-        const float *p = part + ((size_t)i * G + g) * (HD + 2);
-        float w = __expf(p[HD] - M);
-        num = fmaf(p[d], w, num);
-        den = fmaf(p[HD + 1], w, den);
-    }
-    return num / den;
-}
-
-// Four consecutive d of one (row, head): the block's threads first fetch every item's running max in parallel (no
-// dependent-load chain), then fold the items in ascending order with independent loads.
-__device__ __forceinline__ void attn_combine_value4(const float *__restrict__ part, const int *__restrict__ itemStart, int nH, int nKV, int HD,
-                                                    int m, int head, int d0, float *out) {
-    int G = nH / nKV, kvh = head / G, g = head % G;
-    int i0 = itemStart[m * nKV + kvh], i1 = itemStart[m * nKV + kvh + 1];
-    const float *base = part + ((size_t)i0 * G + g) * (HD + 2);
+// Merge the partials of one (row, query head) in ascending item order (deterministic):
+// out = sum O_i e^(m_i-M) / sum l_i e^(m_i-M). itemStart[row*nKV+kvh] .. itemStart[row*nKV+kvh+1] are that pair's items; the
+// host cuts a sequence into at most RD_ATTN_PIECES of them. Block = RD_ATTN_PIECES * HD/4 threads: thread (item i, quarter
+// dq) brings four values of item i into LDS, so every item's load is in flight at once; the first HD/4 threads then fold
+// the items in order. lds: RD_ATTN_PIECES*(HD+2) floats. Returns true in the threads that hold a result (four consecutive d).
+#define RD_ATTN_PIECES 16
+__device__ __forceinline__ bool attn_combine_block(const float *__restrict__ part, const int *__restrict__ itemStart, int nH, int nKV, int HD,
+                                                   int m, int head, float *lds, float *out) {
+    const int Q = HD >> 2, ti = threadIdx.x / Q, dq = threadIdx.x - ti * Q;
+    const int G = nH / nKV, kvh = head / G, g = head % G;
+    const int i0 = itemStart[m * nKV + kvh], n = min(itemStart[m * nKV + kvh + 1] - i0, RD_ATTN_PIECES);
     const size_t stride = (size_t)G * (HD + 2);
-    float M = -INFINITY;
-    for (int i = 0; i < i1 - i0; i += 4) {
-        float a = ld_part(base + (size_t)i * stride + HD);
-        float b = i + 1 < i1 - i0 ? ld_part(base + (size_t)(i + 1) * stride + HD) : -INFINITY;
-        float c = i + 2 < i1 - i0 ? ld_part(base + (size_t)(i + 2) * stride + HD) : -INFINITY;
-        float e = i + 3 < i1 - i0 ? ld_part(base + (size_t)(i + 3) * stride + HD) : -INFINITY;
-        M = fmaxf(fmaxf(M, fmaxf(a, b)), fmaxf(c, e));
+    float *vals = lds, *mm = lds + RD_ATTN_PIECES * HD, *ll = mm + RD_ATTN_PIECES;
+    if (ti < n) {
+        const float *p = part + ((size_t)i0 * G + g) * (HD + 2) + (size_t)ti * stride;
+        const float2 a = *(const float2 *)(p + dq * 4), b = *(const float2 *)(p + dq * 4 + 2); // rows are 8-byte aligned (HD+2 is even)
+        float *v = vals + ti * HD + dq * 4;
+        v[0] = a.x, v[1] = a.y, v[2] = b.x, v[3] = b.y;
+        if (dq == 0) mm[ti] = p[HD], ll[ti] = p[HD + 1];
     }
+    __syncthreads();
+    if (ti != 0) return false;
+    float M = -INFINITY;
+    for (int i = 0; i < n; i++) M = fmaxf(M, mm[i]);
     float num[4] = {0.f, 0.f, 0.f, 0.f}, den = 0.f;
-    for (int i = 0; i < i1 - i0; i += 2) {
-        const float *p = base + (size_t)i * stride;
-        bool two = i + 1 < i1 - i0;
-        const float *p2 = two ? p + stride : p;
-        float2 a = {ld_part(p + d0), ld_part(p + d0 + 1)}, b = {ld_part(p + d0 + 2), ld_part(p + d0 + 3)};
-        float2 a2 = {ld_part(p2 + d0), ld_part(p2 + d0 + 1)}, b2 = {ld_part(p2 + d0 + 2), ld_part(p2 + d0 + 3)};
-        float w = __expf(ld_part(p + HD) - M), l = ld_part(p + HD + 1);
-        float w2 = two ? __expf(ld_part(p2 + HD) - M) : 0.f, l2 = ld_part(p2 + HD + 1);
-        num[0] = fmaf(a.x, w, num[0]), num[1] = fmaf(a.y, w, num[1]), num[2] = fmaf(b.x, w, num[2]), num[3] = fmaf(b.y, w, num[3]);
-        den = fmaf(l, w, den);
-        num[0] = fmaf(a2.x, w2, num[0]), num[1] = fmaf(a2.y, w2, num[1]), num[2] = fmaf(b2.x, w2, num[2]), num[3] = fmaf(b2.y, w2, num[3]);
-        den = fmaf(l2, w2, den);
+    for (int i = 0; i < n; i++) {
+        const float *v = vals + i * HD + dq * 4;
+        const float w = __expf(mm[i] - M);
+        num[0] = fmaf(v[0], w, num[0]), num[1] = fmaf(v[1], w, num[1]), num[2] = fmaf(v[2], w, num[2]), num[3] = fmaf(v[3], w, num[3]);
+        den = fmaf(ll[i], w, den);
     }
 #pragma unroll
     for (int e = 0; e < 4; e++) out[e] = num[e] / den;
+    return true;
 }
 
-extern "C" __global__ void rd_k_attn_combine(const float *__restrict__ part, const int *__restrict__ itemStart, float *__restrict__ out, int nH,
-                                             int nKV, int HD) {
-    int head = blockIdx.x, m = blockIdx.y, d = threadIdx.x;
-    out[(size_t)m * nH * HD + (size_t)head * HD + d] = attn_combine_value(part, itemStart, nH, nKV, HD, m, head, d);
+// Grid (nH, rows), block RD_ATTN_PIECES * HD/4.
+extern "C" __global__ __launch_bounds__(512) void rd_k_attn_combine(const float *__restrict__ part, const int *__restrict__ itemStart,
+                                                                     float *__restrict__ out, int nH, int nKV, int HD) {
+    __shared__ float lds[RD_ATTN_PIECES * (128 + 2)];
+    const int head = blockIdx.x, m = blockIdx.y;
+    float v[4];
+    if (attn_combine_block(part, itemStart, nH, nKV, HD, m, head, lds, v)) {
+        float *o = out + (size_t)m * nH * HD + (size_t)head * HD + threadIdx.x * 4;
+        o[0] = v[0], o[1] = v[1], o[2] = v[2], o[3] = v[3];
+    }
 }

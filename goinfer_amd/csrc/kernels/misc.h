@@ -89,58 +89,116 @@ extern "C" __global__ __launch_bounds__(64) void rd_k_argmax_final(const float *
     if (t == 0) ids[m] = idx == 0x7fffffff ? 0 : idx;
 }
 
-// dst[M][N] = a[M][K] . b[N][K]^T with an ascending-k f64 accumulator rounded once: Backend.MatmulBT (decoder/backend.go:26-30)
-// and the f32 MoE router (decoder/mlp.go:55). One thread per output; exact products, so the result is order-stable.
-extern "C" __global__ void rd_k_matmul_f32(const float *__restrict__ a, const float *__restrict__ b, float *__restrict__ dst, int M, int K, int N) {
-    int n = blockIdx.x * blockDim.x + threadIdx.x, m = blockIdx.y;
+// dst[M][N] = a[M][K] . b[N][K]^T accumulated in f64 and rounded once: Backend.MatmulBT (decoder/backend.go:26-30) and the
+// f32 MoE router (decoder/mlp.go:50). One wave per output: each lane sums its share of k in f64, then a fixed butterfly adds the
+// 64 lane sums. Products of two f32 are exact in f64 and the sum carries ~29 spare bits, so the f32 result matches an
+// ascending-k f64 sum except when that sum falls within ~1e-15 (relative) of an f32 rounding boundary.
+// Grid (ceil(N/4), M), block 256.
+extern "C" __global__ __launch_bounds__(256) void rd_k_matmul_f32(const float *__restrict__ a, const float *__restrict__ b, float *__restrict__ dst,
+                                                                   int M, int K, int N) {
+    const int lane = threadIdx.x & 63, n = blockIdx.x * 4 + (threadIdx.x >> 6), m = blockIdx.y;
     if (n >= N || m >= M) return;
     const float *ar = a + (size_t)m * K, *br = b + (size_t)n * K;
     double acc = 0;
-    for (int k = 0; k < K; k++) acc += (double)ar[k] * (double)br[k];
-    dst[(size_t)m * N + n] = (float)acc;
+    if ((K & 255) == 0) { // 16-byte loads, eight in flight per operand
+        const float4_t *a4 = (const float4_t *)ar + lane, *b4 = (const float4_t *)br + lane;
+        for (int c0 = 0; c0 < K / 256; c0 += 8) {
+            float4_t av[8], bv[8];
+#pragma unroll
+            for (int c = 0; c < 8; c++)
+                if (c0 + c < K / 256) av[c] = a4[(c0 + c) * 64], bv[c] = b4[(c0 + c) * 64];
+#pragma unroll
+            for (int c = 0; c < 8; c++)
+                if (c0 + c < K / 256) {
+                    acc = fma((double)av[c].x, (double)bv[c].x, acc);
+                    acc = fma((double)av[c].y, (double)bv[c].y, acc);
+                    acc = fma((double)av[c].z, (double)bv[c].z, acc);
+                    acc = fma((double)av[c].w, (double)bv[c].w, acc);
+                }
+        }
+    } else {
+        for (int k = lane; k < K; k += 64) acc = fma((double)ar[k], (double)br[k], acc);
+    }
+    for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+    if (lane == 0) dst[(size_t)m * N + n] = (float)acc;
 }
 
 // decoder/mlp.go:130-184 routeExperts (softmax scoring, no bias, no group limit) + mlp.go:370-440 softmaxF32/topK:
-// f32 max; e = f32(exp(f64(x - max))); f64 sum; scores *= f32(1/sum); k passes of strict '>' (lowest index wins);
-// weights = chosen scores, optionally divided by their f32 sum in rank order. One thread per token (nE <= 256).
-// Also fills rankOf[token][expert] = rank or -1 for the expert-major grouped GEMMs.
-extern "C" __global__ void rd_k_moe_route(const float *__restrict__ logits, int T, int nE, int k, int norm, int *__restrict__ idx,
-                                          float *__restrict__ wgt, signed char *__restrict__ rankOf) {
-    int t = blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= T) return;
-    const float *x = logits + (size_t)t * nE;
-    float sc[256];
-    float mx = x[0];
-    for (int i = 1; i < nE; i++)
-        if (x[i] > mx) mx = x[i];
-    double sum = 0;
-    for (int i = 0; i < nE; i++) {
-        double e = exp((double)__fsub_rn(x[i], mx));
-        sc[i] = (float)e;
-        sum += e;
+// f32 max; e = f32(exp(f64(x - max))); f64 sum in ascending expert order; scores *= f32(1/sum); k passes of strict '>'
+// (lowest index wins); weights = chosen scores, optionally divided by their f32 sum in rank order.
+// One wave per token (nE <= 256: up to four experts per lane). The f64 sum is taken by every lane over the same ascending
+// sequence (from LDS), so it is the reference's sum bit for bit. Also fills rankOf[token][expert] = rank or -1 for the
+// expert-major grouped GEMMs. Grid (T), block 64.
+// The routing of one token by one wave (see rd_k_moe_route); x: the token's nE logits (global or LDS).
+__device__ __forceinline__ void moe_route_wave(const float *x, int t, int nE, int k, int norm, int *__restrict__ idx, float *__restrict__ wgt,
+                                               signed char *__restrict__ rankOf, double *e64, int *__restrict__ idx_copy) {
+    const int lane = threadIdx.x & 63;
+    float xv[4], sc[4];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        int i = lane + 64 * j;
+        xv[j] = i < nE ? x[i] : -INFINITY;
+        mx = fmaxf(mx, xv[j]);
     }
-    float inv = (float)(1.0 / sum);
-    for (int i = 0; i < nE; i++) sc[i] = __fmul_rn(sc[i], inv);
-    if (rankOf)
-        for (int i = 0; i < nE; i++) rankOf[(size_t)t * nE + i] = -1;
-    unsigned long long used[4] = {0, 0, 0, 0};
-    float s = 0.f;
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        int i = lane + 64 * j;
+        double e = i < nE ? exp((double)__fsub_rn(xv[j], mx)) : 0.0;
+        sc[j] = (float)e;
+        if (i < nE) e64[i] = e;
+    }
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0): this wave's LDS writes have landed before its lanes read them back
+    double sum = 0;
+    for (int i = 0; i < nE; i++) sum += e64[i];
+    const float inv = (float)(1.0 / sum);
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        int i = lane + 64 * j;
+        sc[j] = i < nE ? __fmul_rn(sc[j], inv) : -INFINITY;
+        if (rankOf && i < nE) rankOf[(size_t)t * nE + i] = -1;
+    }
+    float s = 0.f, mine = 0.f; // lane j keeps the rank-j weight
     int n = 0;
-    for (int j = 0; j < k; j++) {
+    for (int r = 0; r < k; r++) {
         float best = -INFINITY;
-        int bi = -1;
-        for (int i = 0; i < nE; i++)
-            if (!((used[i >> 6] >> (i & 63)) & 1ull) && sc[i] > best) best = sc[i], bi = i;
-        if (bi < 0) break;
-        used[bi >> 6] |= 1ull << (bi & 63);
-        idx[(size_t)t * k + j] = bi;
-        wgt[(size_t)t * k + j] = best;
-        if (rankOf) rankOf[(size_t)t * nE + bi] = (signed char)j;
+        int bi = 0x7fffffff;
+#pragma unroll
+        for (int j = 0; j < 4; j++) // ascending index within the lane: strict '>' keeps the lowest
+            if (sc[j] > best) best = sc[j], bi = lane + 64 * j;
+        for (int o = 32; o > 0; o >>= 1) {
+            float v2 = __shfl_xor(best, o, 64);
+            int i2 = __shfl_xor(bi, o, 64);
+            if (v2 > best || (v2 == best && i2 < bi)) best = v2, bi = i2;
+        }
+        if (bi == 0x7fffffff) break; // nothing left (k > nE)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            if (bi == lane + 64 * j) {
+                sc[j] = -INFINITY; // used
+                if (rankOf) rankOf[(size_t)t * nE + bi] = (signed char)r;
+            }
+        if (lane == r) mine = best;
+        if (lane == 0) {
+            idx[(size_t)t * k + r] = bi;
+            if (idx_copy) idx_copy[(size_t)t * k + r] = bi;
+        }
         s = __fadd_rn(s, best);
         n++;
     }
-    if (norm && s > 0.f)
-        for (int j = 0; j < n; j++) wgt[(size_t)t * k + j] = wgt[(size_t)t * k + j] / s;
+    if (lane < n) wgt[(size_t)t * k + lane] = (norm && s > 0.f) ? mine / s : mine;
+}
+
+// idx_copy (may be NULL) receives a second copy of the indices: the step's per-layer routing trace.
+extern "C" __global__ __launch_bounds__(64) void rd_k_moe_route(const float *__restrict__ logits, int T, int nE, int k, int norm,
+                                                                 int *__restrict__ idx, float *__restrict__ wgt, signed char *__restrict__ rankOf,
+                                                                 int *__restrict__ idx_copy) {
+    __shared__ double e64[256];
+    const int t = blockIdx.x;
+    if (t >= T) return;
+    moe_route_wave(logits + (size_t)t * nE, t, nE, k, norm, idx, wgt, rankOf, e64, idx_copy);
 }
 
 // Token embedding rows from an int8 table with one f32 scale per row (goinfer keeps the embedding table int8 in q4k mode,
@@ -155,6 +213,26 @@ extern "C" __global__ void rd_k_embed_rows(const signed char *__restrict__ q, co
 // Plain copy of n16 16-byte words (grid-stride). A traffic yardstick of known size: n16*16 bytes read, n16*16 written.
 extern "C" __global__ void rd_k_copy16(const uint4 *__restrict__ src, uint4 *__restrict__ dst, size_t n16) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x) dst[i] = src[i];
+}
+
+// Synthetic operand fills for the micro-benchmarks: element i = uniform in [-2, 2) from a counter hash of (seed, i).
+__device__ __forceinline__ float fill_value(size_t i, unsigned seed) {
+    unsigned long long z = (unsigned long long)i * 0x9E3779B97F4A7C15ull + (unsigned long long)seed * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z ^= z >> 31;
+    return (float)(unsigned)(z >> 40) * (4.0f / 16777216.0f) - 2.0f;
+}
+extern "C" __global__ void rd_k_fill_f16(uint16_t *__restrict__ dst, size_t n, unsigned seed) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        half_t h = (half_t)fill_value(i, seed);
+        uint16_t u;
+        __builtin_memcpy(&u, &h, 2);
+        dst[i] = u;
+    }
+}
+extern "C" __global__ void rd_k_fill_f32(float *__restrict__ dst, size_t n, unsigned seed) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) dst[i] = fill_value(i, seed);
 }
 
 // ---- grid-wide barrier for kernels whose blocks are all resident at once (grid <= CUs, one block per CU) ----
