@@ -237,9 +237,6 @@ extern "C" int rd_bench_attn(rd_device *d, int n_seq, const int *len, int n_h, i
         rd_set_error("rd_bench_attn declines: head_dim must be 64 or 128 and the GQA group <= 16");
         return RD_DECLINED;
     }
-    struct Item {
-        int row, kvh, b0, b1;
-    };
     const int qd = n_h * hd, G = n_h / n_kv;
     int maxBlocks = 0;
     long totalBlocks = 0;
@@ -277,26 +274,19 @@ extern "C" int rd_bench_attn(rd_device *d, int n_seq, const int *len, int n_h, i
     for (int r0 = 0; r0 < n_seq; r0 += 32) {
         auto g = std::make_unique<Group>(d);
         g->r0 = r0, g->rows = std::min(32, n_seq - r0);
-        std::vector<Item> items;
-        std::vector<int> start((size_t)g->rows * n_kv + 1), slots((size_t)g->rows), lens((size_t)g->rows);
-        for (int i = 0; i < g->rows; i++) {
-            const int nb = (len[r0 + i] + 63) / 64, chunk = attn_chunk_blocks(nb);
-            slots[(size_t)i] = r0 + i, lens[(size_t)i] = len[r0 + i];
-            for (int h = 0; h < n_kv; h++) {
-                start[(size_t)i * n_kv + h] = (int)items.size();
-                for (int b0 = 0; b0 < nb; b0 += chunk) items.push_back({i, h, b0, std::min(nb, b0 + chunk)});
-            }
-        }
-        start[(size_t)g->rows * n_kv] = (int)items.size();
+        std::vector<AttnItemH> items;
+        std::vector<int> start, slots((size_t)g->rows), lens((size_t)g->rows);
+        for (int i = 0; i < g->rows; i++) slots[(size_t)i] = r0 + i, lens[(size_t)i] = len[r0 + i];
+        build_attn_worklist(lens.data(), g->rows, n_kv, items, start);
         g->nItems = (int)items.size();
         RC(g->L.alloc(sizeof(int) * lens.size()));
         RC(g->S.alloc(sizeof(int) * slots.size()));
-        RC(g->I.alloc(sizeof(Item) * items.size()));
+        RC(g->I.alloc(sizeof(AttnItemH) * items.size()));
         RC(g->St.alloc(sizeof(int) * start.size()));
         RC(g->P.alloc(sizeof(float) * items.size() * G * (hd + 2)));
         RC(d->h2d(g->L.p, lens.data(), sizeof(int) * lens.size()));
         RC(d->h2d(g->S.p, slots.data(), sizeof(int) * slots.size()));
-        RC(d->h2d(g->I.p, items.data(), sizeof(Item) * items.size()));
+        RC(d->h2d(g->I.p, items.data(), sizeof(AttnItemH) * items.size()));
         RC(d->h2d(g->St.p, start.data(), sizeof(int) * start.size()));
         groups.push_back(std::move(g));
     }

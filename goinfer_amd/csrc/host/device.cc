@@ -1,4 +1,5 @@
 // device.cc — device open/close, code-object loading, memory helpers, weight upload and the GEMM launcher.
+#include <algorithm>
 #include "device.h"
 #include <dlfcn.h>
 #include <mutex>
@@ -172,6 +173,22 @@ extern "C" int rd_device_mem_info(rd_device *d, size_t *free_b, size_t *total_b)
     if (!d) return RD_ERR_ARG;
     HIPCHK(MemGetInfo(free_b, total_b));
     return RD_OK;
+}
+
+void build_attn_worklist(const int *len, int rows, int n_kv, std::vector<AttnItemH> &items, std::vector<int> &ranges) {
+    std::vector<int> order((size_t)rows);
+    for (int i = 0; i < rows; i++) order[(size_t)i] = i;
+    std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return len[a] > len[b]; });
+    items.clear();
+    ranges.assign((size_t)rows * n_kv * 2, 0);
+    for (int r : order) {
+        const int nb = (len[r] + 63) / 64, chunk = attn_chunk_blocks(nb);
+        for (int h = 0; h < n_kv; h++) {
+            ranges[((size_t)r * n_kv + h) * 2] = (int)items.size();
+            for (int b0 = 0; b0 < nb; b0 += chunk) items.push_back({r, h, b0, std::min(nb, b0 + chunk)});
+            ranges[((size_t)r * n_kv + h) * 2 + 1] = (int)items.size();
+        }
+    }
 }
 
 // ---- GEMM planning ----

@@ -70,6 +70,14 @@ constexpr unsigned GEMM_THREADS = 320, GATEUP_THREADS = 640;
 constexpr int ATTN_PIECES = 16; // = RD_ATTN_PIECES of the combine kernels
 inline int attn_chunk_blocks(int nb) { return (nb + ATTN_PIECES - 1) / ATTN_PIECES; }
 
+// One attention work item: blocks [b0,b1) of one (sequence row, kv head); one wave each.
+struct AttnItemH {
+    int row, kvh, b0, b1;
+};
+// The attention work list of a step: items of the longest sequences first (the grid is dispatched in index order, so the
+// short items fill the tail), and ranges[2*(row*n_kv+kvh)], ranges[..+1] = that pair's first item and one past its last.
+void build_attn_worklist(const int *len, int rows, int n_kv, std::vector<AttnItemH> &items, std::vector<int> &ranges);
+
 // split-K plan of one GEMM launch
 struct GemmPlan {
     int splits;     // grid.y

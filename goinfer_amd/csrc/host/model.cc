@@ -376,7 +376,7 @@ extern "C" int rd_kv_configure(rd_model *m, int slots, int ctx_cap) {
     int G = c.n_heads / c.n_kv_heads;
     RC(alloc_f32(d, &m->part, (size_t)m->max_items * G * (c.head_dim + 2)));
     RC(d->alloc((void **)&m->items, sizeof(AttnItemH) * (size_t)m->max_items));
-    RC(d->alloc((void **)&m->itemStart, sizeof(int) * (size_t)(32 * c.n_kv_heads + 1)));
+    RC(d->alloc((void **)&m->itemStart, sizeof(int) * (size_t)(32 * c.n_kv_heads * 2)));
     return d->sync();
 }
 
@@ -435,18 +435,10 @@ struct Scope { // times one kernel class when the model's timer is on
     }
 };
 
-static int build_attn_items(rd_model *m, int B, const int *pos, std::vector<AttnItemH> &items, std::vector<int> &start) {
-    const rd_model_desc &c = m->desc;
-    items.clear();
-    start.assign((size_t)B * c.n_kv_heads + 1, 0);
-    for (int b = 0; b < B; b++) {
-        const int nb = (pos[b] + 1 + 63) / 64, chunk = attn_chunk_blocks(nb);
-        for (int h = 0; h < c.n_kv_heads; h++) {
-            start[(size_t)b * c.n_kv_heads + h] = (int)items.size();
-            for (int b0 = 0; b0 < nb; b0 += chunk) items.push_back({b, h, b0, std::min(nb, b0 + chunk)});
-        }
-    }
-    start[(size_t)B * c.n_kv_heads] = (int)items.size();
+static int build_attn_items(rd_model *m, int B, const int *pos, std::vector<AttnItemH> &items, std::vector<int> &ranges) {
+    int len[32];
+    for (int b = 0; b < B; b++) len[b] = pos[b] + 1;
+    build_attn_worklist(len, B, m->desc.n_kv_heads, items, ranges);
     if ((int)items.size() > m->max_items) {
         rd_set_error("attention work list overflow (%zu items)", items.size());
         return RD_ERR_STATE;

@@ -4,10 +4,6 @@
 #include <map>
 #include <vector>
 
-struct AttnItemH {
-    int row, kvh, b0, b1;
-};
-
 // kernel classes of one decode step, for per-class timing
 enum {
     KC_GEMM_QKV = 0, KC_ROPE_STORE, KC_ATTN_PARTIAL, KC_ATTN_COMBINE, KC_GEMM_O, KC_ADD_NORM, KC_GEMM_GATEUP, KC_SWIGLU, KC_GEMM_DOWN,

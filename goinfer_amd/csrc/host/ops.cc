@@ -207,10 +207,6 @@ extern "C" int rd_moe_route(rd_device *d, const float *logits, int T, int nE, in
 }
 
 // ---- ragged attention over a temporary paged pool (kernel-level entry point) ----
-struct AttnItemO {
-    int row, kvh, b0, b1;
-};
-
 extern "C" int rd_attn_ragged(rd_device *d, int n_seq, const int *len, const int64_t *off, const float *k, const float *v, const float *q,
                               int n_h, int n_kv, int hd, float scale, float softcap, float *out) {
     if (!d || !len || !off || !k || !v || !q || !out || n_seq <= 0) return RD_ERR_ARG;
@@ -264,29 +260,22 @@ extern "C" int rd_attn_ragged(rd_device *d, int n_seq, const int *len, const int
     }
     for (int r0 = 0; r0 < n_seq; r0 += 32) { // rows in groups of 32, as the step batches them
         int rows = std::min(32, n_seq - r0);
-        std::vector<AttnItemO> items;
-        std::vector<int> start((size_t)rows * n_kv + 1), slots((size_t)rows), lens((size_t)rows);
-        for (int i = 0; i < rows; i++) {
-            const int nb = (len[r0 + i] + 63) / 64, chunk = attn_chunk_blocks(nb);
-            slots[(size_t)i] = r0 + i, lens[(size_t)i] = len[r0 + i];
-            for (int h = 0; h < n_kv; h++) {
-                start[(size_t)i * n_kv + h] = (int)items.size();
-                for (int b0 = 0; b0 < nb; b0 += chunk) items.push_back({i, h, b0, std::min(nb, b0 + chunk)});
-            }
-        }
-        start[(size_t)rows * n_kv] = (int)items.size();
+        std::vector<AttnItemH> items;
+        std::vector<int> start, slots((size_t)rows), lens((size_t)rows);
+        for (int i = 0; i < rows; i++) slots[(size_t)i] = r0 + i, lens[(size_t)i] = len[r0 + i];
+        build_attn_worklist(lens.data(), rows, n_kv, items, start);
         DevBuf Q2(d), O2(d), L2(d), S2(d), I2(d), St2(d), P2(d);
         RC(Q2.alloc(sizeof(float) * (size_t)rows * qd));
         RC(O2.alloc(sizeof(float) * (size_t)rows * qd));
         RC(L2.alloc(sizeof(int) * (size_t)rows));
         RC(S2.alloc(sizeof(int) * (size_t)rows));
-        RC(I2.alloc(sizeof(AttnItemO) * items.size()));
+        RC(I2.alloc(sizeof(AttnItemH) * items.size()));
         RC(St2.alloc(sizeof(int) * start.size()));
         RC(P2.alloc(sizeof(float) * items.size() * G * (hd + 2)));
         RC(d->h2d(Q2.p, q + (size_t)r0 * qd, sizeof(float) * (size_t)rows * qd));
         RC(d->h2d(L2.p, lens.data(), sizeof(int) * (size_t)rows));
         RC(d->h2d(S2.p, slots.data(), sizeof(int) * (size_t)rows));
-        RC(d->h2d(I2.p, items.data(), sizeof(AttnItemO) * items.size()));
+        RC(d->h2d(I2.p, items.data(), sizeof(AttnItemH) * items.size()));
         RC(d->h2d(St2.p, start.data(), sizeof(int) * start.size()));
         RC(d->launch(d->k.attn_partial, (unsigned)items.size(), 1, 1, 64, (const void *)I2.p, (const int *)L2.p, (const int *)S2.p, (const int *)T.p,
                      maxBlocks, (const uint16_t *)Kp.p, (const uint16_t *)Vp.p, (const float *)Q2.p, P2.as<float>(), n_h, n_kv, hd, scale, softcap));

@@ -236,7 +236,7 @@ extern "C" __global__ __launch_bounds__(64) void rd_k_attn_partial(const AttnIte
 }
 
 // Merge the partials of one (row, query head) in ascending item order (deterministic):
-// out = sum O_i e^(m_i-M) / sum l_i e^(m_i-M). itemStart[row*nKV+kvh] .. itemStart[row*nKV+kvh+1] are that pair's items; the
+// out = sum O_i e^(m_i-M) / sum l_i e^(m_i-M). itemStart[2*(row*nKV+kvh)] and the entry after it bound that pair's items; the
 // host cuts a sequence into at most RD_ATTN_PIECES of them. Block = RD_ATTN_PIECES * HD/4 threads: thread (item i, quarter
 // dq) brings four values of item i into LDS, so every item's load is in flight at once; the first HD/4 threads then fold
 // the items in order. lds: RD_ATTN_PIECES*(HD+2) floats. Returns true in the threads that hold a result (four consecutive d).
@@ -245,7 +245,7 @@ __device__ __forceinline__ bool attn_combine_block(const float *__restrict__ par
                                                    int m, int head, float *lds, float *out) {
     const int Q = HD >> 2, ti = threadIdx.x / Q, dq = threadIdx.x - ti * Q;
     const int G = nH / nKV, kvh = head / G, g = head % G;
-    const int i0 = itemStart[m * nKV + kvh], n = min(itemStart[m * nKV + kvh + 1] - i0, RD_ATTN_PIECES);
+    const int i0 = itemStart[(m * nKV + kvh) * 2], n = min(itemStart[(m * nKV + kvh) * 2 + 1] - i0, RD_ATTN_PIECES);
     const size_t stride = (size_t)G * (HD + 2);
     float *vals = lds, *mm = lds + RD_ATTN_PIECES * HD, *ll = mm + RD_ATTN_PIECES;
     if (ti < n) {
