@@ -47,13 +47,13 @@ __device__ __forceinline__ void panel_store4(uint8_t *__restrict__ Xp, int kind,
 // Per-32 quantization when each lane holds 4 consecutive elements: a group is 8 consecutive lanes.
 __device__ __forceinline__ void quant_g32x4(float v0, float v1, float v2, float v3, float *x0, float *x1, float *x2, float *x3, float *gsum) {
     float ma = fmaxf(fmaxf(fabsf(v0), fabsf(v1)), fmaxf(fabsf(v2), fabsf(v3)));
-    for (int o = 4; o > 0; o >>= 1) ma = fmaxf(ma, __shfl_xor(ma, o, 64));
+    ma = group_max8(ma);
     float sc = ma / 127.f;
     float inv = sc > 0.f ? 1.f / sc : 0.f;
     float r0 = fminf(127.f, fmaxf(-127.f, roundf(__fmul_rn(v0, inv)))), r1 = fminf(127.f, fmaxf(-127.f, roundf(__fmul_rn(v1, inv))));
     float r2 = fminf(127.f, fmaxf(-127.f, roundf(__fmul_rn(v2, inv)))), r3 = fminf(127.f, fmaxf(-127.f, roundf(__fmul_rn(v3, inv))));
     int s = (int)r0 + (int)r1 + (int)r2 + (int)r3;
-    for (int o = 4; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+    s = group_sum8_i(s);
     *gsum = __fmul_rn(sc, (float)s);
     *x0 = __fmul_rn(r0, sc), *x1 = __fmul_rn(r1, sc), *x2 = __fmul_rn(r2, sc), *x3 = __fmul_rn(r3, sc);
 }
@@ -96,17 +96,27 @@ extern "C" __global__ __launch_bounds__(1024) void rd_k_add_rmsnorm_quant(float 
         if (on[i]) v[i] = *(const float4_t *)(h + (size_t)m * H + 4 * q);
     }
     if (P) {
+        // the split-K partials in ascending split order; eight splits' loads are issued together (a runtime-trip loop of
+        // dependent adds would expose one memory latency per split)
         float4_t a[2];
 #pragma unroll
         for (int i = 0; i < 2; i++)
             if (on[i]) a[i] = *(const float4_t *)(P + (size_t)m * H + 4 * (t + i * 1024));
-        for (int s = 1; s < splits; s++) {
+        for (int s0 = 1; s0 < splits; s0 += 8) {
+            float4_t b[2][8];
 #pragma unroll
-            for (int i = 0; i < 2; i++)
-                if (on[i]) {
-                    float4_t b = *(const float4_t *)(P + ((size_t)s * 32 + m) * H + 4 * (t + i * 1024));
-                    a[i].x = __fadd_rn(a[i].x, b.x), a[i].y = __fadd_rn(a[i].y, b.y), a[i].z = __fadd_rn(a[i].z, b.z), a[i].w = __fadd_rn(a[i].w, b.w);
-                }
+            for (int j = 0; j < 8; j++)
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+                    if (on[i] && s0 + j < splits) b[i][j] = *(const float4_t *)(P + ((size_t)(s0 + j) * 32 + m) * H + 4 * (t + i * 1024));
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+                    if (on[i] && s0 + j < splits) {
+                        a[i].x = __fadd_rn(a[i].x, b[i][j].x), a[i].y = __fadd_rn(a[i].y, b[i][j].y);
+                        a[i].z = __fadd_rn(a[i].z, b[i][j].z), a[i].w = __fadd_rn(a[i].w, b[i][j].w);
+                    }
         }
 #pragma unroll
         for (int i = 0; i < 2; i++)

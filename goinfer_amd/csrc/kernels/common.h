@@ -23,14 +23,42 @@ typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
 #define RD_LIN_PANEL_BYTES (RD_LIN_PANEL_STEPS * 64 * 16)
 #define RD_Q4K_TILE_BYTES 4608 // 32 rows x 144 B, re-tiled: 512 B of headers + 4 x 1024 B of codes
 
+// Cross-lane exchanges on the VALU's data-parallel path (DPP) instead of the LDS crossbar: a few cycles each instead of
+// an LDS round trip. Each returns, for every lane, the value of its partner lane: XOR1/XOR2 inside a quad, then the
+// half-row and row mirrors (lane i <-> 7-i of its 8, lane i <-> 15-i of its 16) — partners in the other half, which is all
+// a reduction needs once the lower levels are uniform — and lane i <-> i^16 through ds_swizzle.
+#define RD_DPP_QUAD_XOR1 0xB1   // quad_perm:[1,0,3,2]
+#define RD_DPP_QUAD_XOR2 0x4E   // quad_perm:[2,3,0,1]
+#define RD_DPP_HALF_MIRROR 0x141 // row_half_mirror
+#define RD_DPP_ROW_MIRROR 0x140  // row_mirror
+template <int CTRL> __device__ __forceinline__ int dpp_i(int v) { return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true); }
+template <int CTRL> __device__ __forceinline__ float dpp_f(float v) { return __int_as_float(dpp_i<CTRL>(__float_as_int(v))); }
+__device__ __forceinline__ int swz_xor16_i(int v) { return __builtin_amdgcn_ds_swizzle(v, 0x401F); } // bit mode: and 0x1F, xor 0x10
+__device__ __forceinline__ float swz_xor16_f(float v) { return __int_as_float(swz_xor16_i(__float_as_int(v))); }
+
+// max / sum over each aligned group of 8, 16 or 32 lanes, delivered to every lane of the group
+__device__ __forceinline__ float group_max8(float v) {
+    v = fmaxf(v, dpp_f<RD_DPP_QUAD_XOR1>(v));
+    v = fmaxf(v, dpp_f<RD_DPP_QUAD_XOR2>(v));
+    return fmaxf(v, dpp_f<RD_DPP_HALF_MIRROR>(v));
+}
+__device__ __forceinline__ int group_sum8_i(int v) {
+    v += dpp_i<RD_DPP_QUAD_XOR1>(v);
+    v += dpp_i<RD_DPP_QUAD_XOR2>(v);
+    return v + dpp_i<RD_DPP_HALF_MIRROR>(v);
+}
+__device__ __forceinline__ float group_max16(float v) {
+    v = group_max8(v);
+    return fmaxf(v, dpp_f<RD_DPP_ROW_MIRROR>(v));
+}
 __device__ __forceinline__ float wave_max32(float v) {
-    // max over each aligned group of 32 lanes
-    for (int o = 16; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-    return v;
+    v = group_max16(v);
+    return fmaxf(v, swz_xor16_f(v));
 }
 __device__ __forceinline__ int wave_sum32_i(int v) {
-    for (int o = 16; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-    return v;
+    v = group_sum8_i(v);
+    v += dpp_i<RD_DPP_ROW_MIRROR>(v);
+    return v + swz_xor16_i(v);
 }
 __device__ __forceinline__ float wave_sum64(float v) {
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
