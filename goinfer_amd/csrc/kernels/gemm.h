@@ -8,10 +8,6 @@
 #pragma once
 #include "common.h"
 #include <type_traits>
-#ifdef RD_DBG_TIMING
-__device__ unsigned long long rd_dbg_t[256];
-__device__ unsigned long long rd_dbg_g[8 * 1024];
-#endif
 
 // The producer/consumer main loop. Loads return in issue order as far as a wave's wait counter is concerned, so a wave that
 // both streams weights and stages activation panels must, when it waits for a panel, also wait for every weight tile it
@@ -57,10 +53,6 @@ __device__ __forceinline__ void gemm_mainloop_pc(float16_t &acc, const uint8_t *
         __syncthreads();
         auto pbody = [&](int it, auto sc) {
             constexpr int slot = decltype(sc)::value;
-#ifdef RD_DBG_NO_PANEL
-            __syncthreads();
-            return;
-#endif
             uint4_t *dst = lds + ((it + 1) & 1) * PV + lane;
 #pragma unroll
             for (int j = 0; j < PVL; j++) dst[j * 64] = ring[slot][j]; // panel it+1 (a copy of the last one at the tail)
@@ -89,21 +81,11 @@ __device__ __forceinline__ void gemm_mainloop_pc(float16_t &acc, const uint8_t *
 #pragma unroll
     for (int i = 0; i < PF; i++) T::load(w[i], wb + (size_t)min(i, last) * T::TILE_BYTES, lane);
     __syncthreads();
-#ifdef RD_DBG_TIMING
-#define RD_STAMP(k)                                                                                              \
-    if (blockIdx.x == RD_DBG_TIMING && blockIdx.y == 0 && wave == 0 && lane == 0 && it < 64) rd_dbg_t[it * 4 + (k)] = __builtin_amdgcn_s_memtime();
-#else
-#define RD_STAMP(k)
-#endif
     auto body = [&](int it, auto uc) {
         constexpr int u = decltype(uc)::value;
-        RD_STAMP(0)
         if (it < nk) T::mma(acc, w[u], lds + (it & 1) * PV, lane);
-        RD_STAMP(1)
         T::load(w[u], wb + (size_t)min(it + PF, last) * T::TILE_BYTES, lane);
-        RD_STAMP(2)
         __syncthreads();
-        RD_STAMP(3)
     };
     int it = 0;
     for (; it + PF <= per; it += PF) {

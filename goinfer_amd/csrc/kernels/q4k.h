@@ -62,15 +62,10 @@ struct Q4KTile {
     uint4_t hdr, q[4];
 };
 
-#ifdef RD_DBG_NO_NT
-#define RD_WLOAD(p) (*(p))
-#else
-#define RD_WLOAD(p) __builtin_nontemporal_load(p)
-#endif
 __device__ __forceinline__ void q4k_tile_load(Q4KTile &w, const uint8_t *__restrict__ p, int lane) {
-    w.hdr = RD_WLOAD((const uint4_t *)(p + (lane & 31) * 16));
+    w.hdr = __builtin_nontemporal_load((const uint4_t *)(p + (lane & 31) * 16));
 #pragma unroll
-    for (int c = 0; c < 4; c++) w.q[c] = RD_WLOAD((const uint4_t *)(p + 512 + c * 1024 + lane * 16));
+    for (int c = 0; c < 4; c++) w.q[c] = __builtin_nontemporal_load((const uint4_t *)(p + 512 + c * 1024 + lane * 16));
 }
 
 // acc += panel(32 batch rows x 256 k) . tile(32 weight rows x 256 k)^T, f16 MFMA with f32 accumulation.
@@ -78,12 +73,6 @@ __device__ __forceinline__ void q4k_tile_load(Q4KTile &w, const uint8_t *__restr
 // then one packed fma per pair yields the centred weight (q-8)*dsc rounded once. The per-sub-block constants
 // 8*dsc - dmin*m ride a 17th MFMA step against the per-group activation sums.
 __device__ __forceinline__ void q4k_tile_mma(float16_t &acc, const Q4KTile &w, const uint4_t *__restrict__ panel, int lane) {
-#ifdef RD_DBG_NO_MMA // measurement builds only: keep the loads alive, skip the arithmetic
-    uint32_t f = w.hdr.x ^ w.hdr.y ^ w.hdr.z ^ w.hdr.w;
-    for (int c = 0; c < 4; c++) f ^= w.q[c].x ^ w.q[c].y ^ w.q[c].z ^ w.q[c].w;
-    acc[0] += __uint_as_float(f & 0x3fffffffu) + __uint_as_float(panel[lane].x & 0x3fffffffu);
-    return;
-#endif
     const int h = lane >> 5;
     const uint32_t mask_lo = 0x000F000Fu, mask_hi = 0x00F000F0u, magic_lo = 0x64006400u, magic_hi = 0x54005400u;
     uint32_t y = w.hdr.y, z = w.hdr.z, x = w.hdr.w;
@@ -112,11 +101,6 @@ __device__ __forceinline__ void q4k_tile_mma(float16_t &acc, const Q4KTile &w, c
         C0[jj] = (half2_t){c, c};
         off[jj] = (half_t)(8.f * dsc32 - delta - dmin * (float)m); // exact scale here keeps the scale rounding centred
     }
-#ifdef RD_Q4K_ACC2
-    float16_t acc2;
-#pragma unroll
-    for (int i = 0; i < 16; i++) acc2[i] = 0.f;
-#endif
 #pragma unroll
     for (int s = 0; s < 16; s++) {
         uint32_t wd = w.q[s >> 2][s & 3];
@@ -133,25 +117,10 @@ __device__ __forceinline__ void q4k_tile_mma(float16_t &acc, const Q4KTile &w, c
         v1 = __builtin_elementwise_fma(v1, DSC[2 * pp + 1], C0[2 * pp + 1]);
         v2 = __builtin_elementwise_fma(v2, DSC[2 * pp], C0[2 * pp]);
         v3 = __builtin_elementwise_fma(v3, DSC[2 * pp + 1], C0[2 * pp + 1]);
-#ifdef RD_DBG_NO_DEQUANT
-        uint4_t braw = {wd, t8, wd ^ x, t8 ^ y};
-        half8_t b;
-        __builtin_memcpy(&b, &braw, 16);
-#else
         half8_t b = {v0.x, v0.y, v1.x, v1.y, v2.x, v2.y, v3.x, v3.y};
-#endif
         half8_t a;
-#ifdef RD_DBG_NO_LDSREAD
-        uint4_t av = {wd, wd, wd, wd};
-#else
         uint4_t av = panel[s * 64 + lane];
-#endif
         __builtin_memcpy(&a, &av, 16);
-#ifdef RD_Q4K_ACC2
-        if (s & 1)
-            acc2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc2, 0, 0, 0);
-        else
-#endif
             acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc, 0, 0, 0);
     }
     {
@@ -161,10 +130,6 @@ __device__ __forceinline__ void q4k_tile_mma(float16_t &acc, const Q4KTile &w, c
         __builtin_memcpy(&a, &av, 16);
         acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc, 0, 0, 0);
     }
-#ifdef RD_Q4K_ACC2
-#pragma unroll
-    for (int i = 0; i < 16; i++) acc[i] += acc2[i];
-#endif
 }
 
 struct Q4KTraits {
@@ -201,20 +166,8 @@ __device__ __forceinline__ void q4k_gateup_body(const uint8_t *__restrict__ Wt, 
     const bool active = t < nGate;
     float16_t acc;
     const int ltile = active ? tile : nGate - 1;
-#ifdef RD_DBG_TIMING
-#define RD_GSTAMP(k) if (tid == 0) rd_dbg_g[blockIdx.x * 8 + (k)] = __builtin_amdgcn_s_memrealtime();
-#else
-#define RD_GSTAMP(k)
-#endif
-    RD_GSTAMP(0)
     gemm_mainloop_pc<Q4KTraits, 4, KG, PF>(acc, Wt + (size_t)ltile * nSB * RD_Q4K_TILE_BYTES, Xp, 0, nSB, lds);
-    RD_GSTAMP(1)
     gemm_fold_groups<4, KG>(acc, (float *)lds);
-    RD_GSTAMP(2)
-#ifdef RD_DBG_NO_EPILOGUE
-    if (acc[3] == 1234.5f) XpOut[tid] = 1;
-    return;
-#endif
     // Epilogue on all waves: the four complete tiles (gate t0,t1, up t0,t1) go to LDS as [tile][row m][column c]; then
     // every thread takes elements (tile pair, m, c) with 32 consecutive lanes on one row's 32 columns = one activation group.
     float *xe = (float *)lds + (KG - 1) * 4 * 1024; // 4 tiles x 32 x 32 floats past the fold area
@@ -247,7 +200,6 @@ __device__ __forceinline__ void q4k_gateup_body(const uint8_t *__restrict__ Wt, 
             }
         }
     }
-    RD_GSTAMP(3)
 }
 
 // Grid (I/64), block 640: two K-groups of four consumer waves (gate t0,t1, up t0,t1) plus one producer each.
