@@ -147,7 +147,7 @@ int rd_bench_class_count(void);
 const char *rd_bench_class_name(int c);
 /* Times `iters` launches of one kernel over resident synthetic operands: "gemm_q4k" args {N,K,M,copies}; "copy" args {bytes}. */
 int rd_bench_kernel(rd_device *d, const char *name, const int64_t *args, int n_args, int warmup, int iters, float *ms_out);
-/* The ragged attention of one layer (C3 of the measurement plan) over a synthetic paged f16 pool built on the device:
+/* The ragged attention of one layer over a synthetic paged f16 pool built on the device (the attention micro-benchmark):
  * n_seq sequences of len[i] keys, rows in groups of 32. ms_total[iters]: partial + combine kernels of every group;
  * ms_partial[iters] (may be NULL): the flash-decode partial kernels alone. */
 int rd_bench_attn(rd_device *d, int n_seq, const int *len, int n_h, int n_kv, int hd, float scale, float softcap, int warmup, int iters,
