@@ -95,6 +95,10 @@ extern "C" __global__ __launch_bounds__(1024) void rd_k_add_rmsnorm_quant(float 
         v[i] = (float4_t){0.f, 0.f, 0.f, 0.f};
         if (on[i]) v[i] = *(const float4_t *)(h + (size_t)m * H + 4 * q);
     }
+    float4_t wv[2]; // the norm weights are needed last: ask for them first
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+        if (on[i]) wv[i] = *(const float4_t *)(w + 4 * (t + i * 1024));
     if (P) {
         // the split-K partials in ascending split order; eight splits' loads are issued together (a runtime-trip loop of
         // dependent adds would expose one memory latency per split)
@@ -139,9 +143,8 @@ extern "C" __global__ __launch_bounds__(1024) void rd_k_add_rmsnorm_quant(float 
     for (int i = 0; i < 2; i++) {
         if (!on[i]) continue; // whole waves drop out together: nv is a multiple of 32
         int k0 = 4 * (t + i * 1024);
-        float4_t wv = *(const float4_t *)(w + k0);
-        float n0 = __fmul_rn(__fmul_rn(v[i].x, inv), wv.x), n1 = __fmul_rn(__fmul_rn(v[i].y, inv), wv.y);
-        float n2 = __fmul_rn(__fmul_rn(v[i].z, inv), wv.z), n3 = __fmul_rn(__fmul_rn(v[i].w, inv), wv.w);
+        float n0 = __fmul_rn(__fmul_rn(v[i].x, inv), wv[i].x), n1 = __fmul_rn(__fmul_rn(v[i].y, inv), wv[i].y);
+        float n2 = __fmul_rn(__fmul_rn(v[i].z, inv), wv[i].z), n3 = __fmul_rn(__fmul_rn(v[i].w, inv), wv[i].w);
         if (norm_out) *(float4_t *)(norm_out + (size_t)m * H + k0) = (float4_t){n0, n1, n2, n3};
         float x0, x1, x2, x3, gs;
         quant_g32x4(n0, n1, n2, n3, &x0, &x1, &x2, &x3, &gs);

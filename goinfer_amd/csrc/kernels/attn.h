@@ -46,12 +46,21 @@ extern "C" __global__ void rd_k_qkv_rope_store(const float *__restrict__ P, int 
                                                const float *__restrict__ qnorm, const float *__restrict__ knorm, float eps, int nH, int nKV, int HD) {
     int head = blockIdx.x, m = blockIdx.y, t = threadIdx.x, half = HD / 2; // one wave: half <= 64
     int Ntot = (nH + 2 * nKV) * HD, pos = rowPos[m];
+    // everything this thread will need from memory is requested up front: one latency instead of a chain of them
+    const int slotRow = rowSlot[m];
+    const double invf = invFreq[t];
     const float *src = P + (size_t)m * Ntot + (size_t)head * HD;
     float x1 = src[t], x2 = src[t + half];
-    for (int s = 1; s < splits; s++) {
-        x1 = __fadd_rn(x1, src[(size_t)s * 32 * Ntot + t]);
-        x2 = __fadd_rn(x2, src[(size_t)s * 32 * Ntot + t + half]);
+    for (int s0 = 1; s0 < splits; s0 += 8) { // ascending split order; eight splits' loads in flight together
+        float a1[8], a2[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            if (s0 + j < splits) a1[j] = src[(size_t)(s0 + j) * 32 * Ntot + t], a2[j] = src[(size_t)(s0 + j) * 32 * Ntot + t + half];
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            if (s0 + j < splits) x1 = __fadd_rn(x1, a1[j]), x2 = __fadd_rn(x2, a2[j]);
     }
+    const int blkPre = tables[(size_t)slotRow * tabStride + (pos >> 6)];
     bool isQ = head < nH, isK = !isQ && head < nH + nKV;
     const float *nw = isQ ? qnorm : (isK ? knorm : nullptr);
     if (nw) { // RMSNorm over the head's HD values, f64 sum of squares
@@ -63,7 +72,7 @@ extern "C" __global__ void rd_k_qkv_rope_store(const float *__restrict__ P, int 
     }
     float o1 = x1, o2 = x2;
     if (isQ || isK) {
-        double theta = (double)pos * invFreq[t];
+        double theta = (double)pos * invf;
         double c = cos(theta), s = sin(theta);
         o1 = (float)((double)x1 * c - (double)x2 * s);
         o2 = (float)((double)x2 * c + (double)x1 * s);
@@ -75,7 +84,7 @@ extern "C" __global__ void rd_k_qkv_rope_store(const float *__restrict__ P, int 
         return;
     }
     int kvh = isK ? head - nH : head - nH - nKV;
-    int blk = tables[(size_t)rowSlot[m] * tabStride + (pos >> 6)], p = pos & 63;
+    int blk = blkPre, p = pos & 63;
     size_t region = ((size_t)blk * nKV + kvh) * 64 * HD;
     uint16_t *dstp = isK ? Kp : Vp;
     for (int e = 0; e < 2; e++) {
