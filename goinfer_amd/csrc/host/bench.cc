@@ -22,26 +22,27 @@ extern "C" int rd_bench_steps(rd_model *m, int B, const int *slot, const int *po
     rd_device *d = m->d;
     RC(d->h2d(m->ids, ids0, sizeof(int) * (size_t)B));
     RC(d->sync());
-    hipEvent_t e0, e1;
-    HIPCHK(EventCreate(&e0));
-    HIPCHK(EventCreate(&e1));
+    // One event per step boundary; nothing is waited for until the last step is enqueued, so the host runs ahead of the
+    // GPU as a serving loop chaining greedy steps on the device would (ids_out asks for a read-back per step instead).
+    const int total = warmup + steps;
+    std::vector<hipEvent_t> ev((size_t)total + 1);
+    for (auto &e : ev) HIPCHK(EventCreate(&e));
     std::vector<int> pos((size_t)B);
     int rc = RD_OK;
-    for (int i = 0; i < warmup + steps && !rc; i++) {
+    (void)d->hip->EventRecord(ev[0], d->stream);
+    for (int i = 0; i < total && !rc; i++) {
         for (int b = 0; b < B; b++) pos[(size_t)b] = pos0[b] + i;
-        (void)d->hip->EventRecord(e0, d->stream);
         rc = model_step(m, B, slot, pos.data(), nullptr, nullptr, RD_WANT_ARGMAX, nullptr, nullptr);
-        (void)d->hip->EventRecord(e1, d->stream);
-        if (!rd_hip_ok(d->hip, d->hip->EventSynchronize(e1), "hipEventSynchronize")) rc = RD_ERR_HIP;
-        float ms = 0.f;
-        (void)d->hip->EventElapsedTime(&ms, e0, e1);
-        if (i >= warmup) {
-            ms_out[i - warmup] = ms;
-            if (ids_out && !rc) rc = d->d2h(ids_out + (size_t)(i - warmup) * B, m->ids, sizeof(int) * (size_t)B);
-        }
+        (void)d->hip->EventRecord(ev[(size_t)i + 1], d->stream);
+        if (i >= warmup && ids_out && !rc) rc = d->d2h(ids_out + (size_t)(i - warmup) * B, m->ids, sizeof(int) * (size_t)B);
     }
-    (void)d->hip->EventDestroy(e0);
-    (void)d->hip->EventDestroy(e1);
+    if (!rc) rc = d->sync();
+    for (int i = warmup; i < total; i++) {
+        float ms = 0.f;
+        if (!rc) (void)d->hip->EventElapsedTime(&ms, ev[(size_t)i], ev[(size_t)i + 1]);
+        ms_out[i - warmup] = ms;
+    }
+    for (auto &e : ev) (void)d->hip->EventDestroy(e);
     return rc;
 }
 

@@ -63,11 +63,12 @@ extern "C" void rd_model_destroy(rd_model *m) {
     }
     free_weight(d, &m->head);
     for (void *p : {(void *)m->embed_q, (void *)m->embed_scale, (void *)m->inv_freq_dev, (void *)m->final_norm, (void *)m->tables, (void *)m->h, (void *)m->normed, (void *)m->P, (void *)m->qbuf,
-                    (void *)m->part, (void *)m->cand_v, (void *)m->cand_i, (void *)m->logits, (void *)m->emb_dev, m->XpA, m->XpB, (void *)m->ids, (void *)m->rowSlot, (void *)m->rowPos,
-                    (void *)m->rowLen, (void *)m->itemStart, (void *)m->items, (void *)m->router_logits, (void *)m->moe_wgt, (void *)m->moe_gu,
+                    (void *)m->part, (void *)m->cand_v, (void *)m->cand_i, (void *)m->logits, (void *)m->emb_dev, m->XpA, m->XpB, (void *)m->ids, (void *)m->meta, (void *)m->router_logits, (void *)m->moe_wgt, (void *)m->moe_gu,
                     (void *)m->moe_dn, (void *)m->moe_out, (void *)m->moe_idx, (void *)m->moe_idx_all, (void *)m->moe_rank, m->XpE})
         d->release(p);
     if (m->host_stage) (void)d->hip->HostFree(m->host_stage);
+    for (hipEvent_t e : m->stage_ev)
+        if (e) (void)d->hip->EventDestroy(e);
     for (hipEvent_t e : m->timer.ev) (void)d->hip->EventDestroy(e);
     delete m;
 }
@@ -319,9 +320,6 @@ extern "C" int rd_model_finalize(rd_model *m) {
     RC(d->alloc((void **)&m->ids, sizeof(int) * 32));
     RC(alloc_f32(d, &m->cand_v, (size_t)32 * ((c.vocab + 4095) / 4096)));
     RC(d->alloc((void **)&m->cand_i, sizeof(int) * 32 * (size_t)((c.vocab + 4095) / 4096)));
-    RC(d->alloc((void **)&m->rowSlot, sizeof(int) * 32));
-    RC(d->alloc((void **)&m->rowPos, sizeof(int) * 32));
-    RC(d->alloc((void **)&m->rowLen, sizeof(int) * 32));
     if (c.n_experts > 0) {
         int k = c.top_k, I = c.expert_inter;
         RC(alloc_f32(d, &m->router_logits, (size_t)32 * c.n_experts));
@@ -336,7 +334,8 @@ extern "C" int rd_model_finalize(rd_model *m) {
         HIPCHK(MemsetAsync(m->XpE, 0, (size_t)c.n_experts * (I / 128) * LIN_PANEL_BYTES, d->stream));
     }
     m->host_stage_bytes = sizeof(float) * (size_t)32 * H + (1u << 20);
-    HIPCHK(HostMalloc(&m->host_stage, m->host_stage_bytes, 0));
+    HIPCHK(HostMalloc(&m->host_stage, m->host_stage_bytes * rd_model::STAGE_SLOTS, 0));
+    for (auto &e : m->stage_ev) HIPCHK(EventCreate(&e));
     m->finalized = true;
     return d->sync();
 }
@@ -375,8 +374,13 @@ extern "C" int rd_kv_configure(rd_model *m, int slots, int ctx_cap) {
     m->max_items = 32 * c.n_kv_heads * ATTN_PIECES;
     int G = c.n_heads / c.n_kv_heads;
     RC(alloc_f32(d, &m->part, (size_t)m->max_items * G * (c.head_dim + 2)));
-    RC(d->alloc((void **)&m->items, sizeof(AttnItemH) * (size_t)m->max_items));
-    RC(d->alloc((void **)&m->itemStart, sizeof(int) * (size_t)(32 * c.n_kv_heads * 2)));
+    // The step's metadata lives in one device block so a step uploads it with one copy:
+    // [row slot 32][row position 32][row length 32][item ranges 32*nKV*2][items max_items x 4] ints
+    const size_t rangeInts = (size_t)32 * c.n_kv_heads * 2;
+    m->meta_ints = 96 + rangeInts + (size_t)m->max_items * 4;
+    RC(d->alloc((void **)&m->meta, sizeof(int) * m->meta_ints));
+    m->rowSlot = m->meta, m->rowPos = m->meta + 32, m->rowLen = m->meta + 64, m->itemStart = m->meta + 96;
+    m->items = (AttnItemH *)(m->meta + 96 + rangeInts);
     return d->sync();
 }
 
@@ -530,24 +534,26 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
     std::vector<AttnItemH> items;
     std::vector<int> start;
     RC(build_attn_items(m, B, pos, items, start));
-    // Stage the step's metadata in pinned memory and upload it asynchronously. The staging area is reused by the next
-    // step, which is safe because every step ends with a stream synchronisation (the read-back, or the caller's timing wait).
+    // Stage the step's metadata (and host embeddings) in pinned memory and upload it asynchronously. A slot is reused only
+    // once the upload it last fed has completed, which its event tells.
+    const unsigned stage_slot = m->stage_next++ % rd_model::STAGE_SLOTS;
+    if (m->stage_busy[stage_slot]) HIPCHK(EventSynchronize(m->stage_ev[stage_slot]));
     {
-        char *st = (char *)m->host_stage;
-        int *rs = (int *)st, *rp = rs + 32, *rl = rp + 32, *stt = rl + 32;
-        AttnItemH *it = (AttnItemH *)(st + 4096 + sizeof(int) * start.size());
+        char *st = (char *)m->host_stage + (size_t)stage_slot * m->host_stage_bytes;
+        int *hm = (int *)st; // the metadata block, laid out as on the device
+        const size_t rangeInts = (size_t)32 * nKV * 2;
         float *eh = (float *)(st + (1u << 20));
-        for (int b = 0; b < B; b++) rs[b] = slot[b], rp[b] = pos[b], rl[b] = pos[b] + 1;
-        memcpy(stt, start.data(), sizeof(int) * start.size());
-        memcpy(it, items.data(), sizeof(AttnItemH) * items.size());
-        RC(d->h2d(m->rowSlot, rs, sizeof(int) * (size_t)B));
-        RC(d->h2d(m->rowPos, rp, sizeof(int) * (size_t)B));
-        RC(d->h2d(m->rowLen, rl, sizeof(int) * (size_t)B));
-        RC(d->h2d(m->itemStart, stt, sizeof(int) * start.size()));
-        RC(d->h2d(m->items, it, sizeof(AttnItemH) * items.size()));
+        for (int b = 0; b < B; b++) hm[b] = slot[b], hm[32 + b] = pos[b], hm[64 + b] = pos[b] + 1;
+        memcpy(hm + 96, start.data(), sizeof(int) * start.size());
+        memcpy(hm + 96 + rangeInts, items.data(), sizeof(AttnItemH) * items.size());
+        RC(d->h2d(m->meta, hm, sizeof(int) * (96 + rangeInts + items.size() * 4)));
         if (emb_host) {
             memcpy(eh, emb_host, sizeof(float) * (size_t)B * H);
             RC(d->h2d(m->h, eh, sizeof(float) * (size_t)B * H));
+        }
+        HIPCHK(EventRecord(m->stage_ev[stage_slot], d->stream));
+        m->stage_busy[stage_slot] = true;
+        if (emb_host) {
         } else if (emb_dev) {
             HIPCHK(MemcpyAsync(m->h, emb_dev, sizeof(float) * (size_t)B * H, hipMemcpyDeviceToDevice, d->stream));
         } else { // greedy chain: the previous step's argmax ids, still on the device

@@ -60,6 +60,8 @@ struct rd_model {
     int *cand_i = nullptr;
     int *ids = nullptr, *rowSlot = nullptr, *rowPos = nullptr, *rowLen = nullptr, *itemStart = nullptr;
     AttnItemH *items = nullptr;
+    int *meta = nullptr; // one device block holding rowSlot, rowPos, rowLen, itemStart and items (one upload per step)
+    size_t meta_ints = 0;
     int max_items = 0;
     // MoE scratch
     float *router_logits = nullptr, *moe_wgt = nullptr, *moe_gu = nullptr, *moe_dn = nullptr, *moe_out = nullptr;
@@ -67,8 +69,14 @@ struct rd_model {
     signed char *moe_rank = nullptr;                 // [32][nE]
     void *XpE = nullptr;                             // per-expert down panels
     // pinned host staging
+    // STAGE_SLOTS slots used round-robin, so a caller that chains steps without reading anything back (the device greedy
+    // chain) can enqueue several steps ahead of the GPU; a slot is rewritten only after its own upload has completed
+    static constexpr int STAGE_SLOTS = 4;
     void *host_stage = nullptr;
-    size_t host_stage_bytes = 0;
+    size_t host_stage_bytes = 0; // per slot
+    hipEvent_t stage_ev[STAGE_SLOTS] = {};
+    bool stage_busy[STAGE_SLOTS] = {};
+    unsigned stage_next = 0;
     int last_B = 0;
 
     // routing replay for the next step (rd_moe_replay): [layers] of host arrays the step uploads
