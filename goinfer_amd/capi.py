@@ -20,7 +20,7 @@ EXPORTS = [
     "rd_model_upload_q4k", "rd_model_upload_w8a8", "rd_model_upload_w4a8", "rd_model_upload_f32", "rd_model_finalize",
     "rd_kv_configure", "rd_kv_upload", "rd_kv_truncate", "rd_kv_reset", "rd_step_batch", "rd_forward",
     "rd_last_moe_indices", "rd_model_upload_embedding", "rd_bench_steps", "rd_bench_profile", "rd_bench_class_count",
-    "rd_bench_class_name", "rd_bench_kernel", "rd_gateup_q4k_quant", "rd_moe_replay", "rd_bench_attn",
+    "rd_bench_class_name", "rd_bench_kernel", "rd_gateup_q4k_quant", "rd_moe_replay", "rd_bench_attn", "rd_step_ragged", "rd_prefill_last",
 ]
 
 
@@ -249,6 +249,24 @@ class Model:
         ids = np.empty(B, np.int32) if want & WANT_ARGMAX else None
         check(lib().rd_step_batch(self.h, B, _p(slots), _p(pos), _p(emb), want, _p(logits), _p(ids)), "rd_step_batch")
         return logits, ids
+
+    def step_ragged(self, slots, pos, embs, want=WANT_LOGITS):
+        """embs: one [rows_i][hidden] array per sequence. Returns (logits [sum rows][vocab] or None, ids [sum rows] or None)."""
+        n_rows = np.ascontiguousarray([len(e) for e in embs], dtype=np.int32)
+        emb = _f32(np.concatenate([np.asarray(e, dtype=np.float32).reshape(len(e), -1) for e in embs], axis=0))
+        slots = np.ascontiguousarray(slots, dtype=np.int32)
+        pos = np.ascontiguousarray(pos, dtype=np.int32)
+        R = int(n_rows.sum())
+        logits = np.empty((R, self.cfg["vocab"]), np.float32) if want & WANT_LOGITS else None
+        ids = np.empty(R, np.int32) if want & WANT_ARGMAX else None
+        check(lib().rd_step_ragged(self.h, len(slots), _p(slots), _p(pos), _p(n_rows), _p(emb), want, _p(logits), _p(ids)), "rd_step_ragged")
+        return logits, ids
+
+    def prefill_last(self, slot, start_pos, emb):
+        emb = _f32(emb)
+        logits = np.empty(self.cfg["vocab"], np.float32)
+        check(lib().rd_prefill_last(self.h, slot, start_pos, emb.shape[0], _p(emb), _p(logits)), "rd_prefill_last")
+        return logits
 
     def moe_replay(self, idx, wgt):
         """The next step replays this routing ([B][layers][k] indices and weights) instead of its own."""

@@ -503,7 +503,7 @@ static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
 
 // emb_host: [B][hidden] on the host, or emb_dev already on the device (benchmark loop). Logits/ids are host pointers.
 int model_step(rd_model *m, int B, const int *slot, const int *pos, const float *emb_host, const float *emb_dev, int want, float *logits,
-               int *ids) {
+               int *ids, bool multirow) {
     rd_device *d = m->d;
     const rd_model_desc &c = m->desc;
     if (!m->finalized || !m->tables) {
@@ -514,14 +514,20 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
         rd_set_error("rocm resident: batch %d outside the stepper range 1..32", B);
         return RD_ERR_ARG;
     }
+    // A slot may carry several rows in one step if they sit at consecutive positions (a ragged step's verify or prefill
+    // rows): all their K/V is written before any row attends, and row j reads keys [0, pos_j], so each row is the row its own
+    // single-token step would compute. Anything else naming a slot twice is refused before a byte is written.
     for (int b = 0; b < B; b++) {
         if (!slot_ok(m, slot[b])) return RD_ERR_ARG;
+        int prev = -1;
         for (int a = 0; a < b; a++)
-            if (slot[a] == slot[b]) {
+            if (slot[a] == slot[b]) prev = a;
+        if (prev >= 0) {
+            if (!multirow || pos[b] != pos[prev] + 1) {
                 rd_set_error("slot %d appears twice in one step", slot[b]);
                 return RD_ERR_ARG;
             }
-        if (pos[b] < 0 || pos[b] > m->slot_len[(size_t)slot[b]]) {
+        } else if (pos[b] < 0 || pos[b] > m->slot_len[(size_t)slot[b]]) {
             rd_set_error("row %d: position %d but slot %d holds %d rows", b, pos[b], slot[b], m->slot_len[(size_t)slot[b]]);
             return RD_ERR_ARG;
         }
@@ -639,7 +645,7 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
                      (want & RD_WANT_LOGITS) ? m->logits : (float *)nullptr));
         if (want & RD_WANT_ARGMAX) RC(d->launch(d->k.argmax_final, (unsigned)B, 1, 1, 64, (const float *)m->cand_v, (const int *)m->cand_i, nChunks, m->ids));
     }
-    for (int b = 0; b < B; b++) m->slot_len[(size_t)slot[b]] = pos[b] + 1;
+    for (int b = 0; b < B; b++) m->slot_len[(size_t)slot[b]] = std::max(m->slot_len[(size_t)slot[b]], pos[b] + 1);
     m->last_B = B;
     const bool replayed = m->replay_B != 0;
     m->replay_B = 0; // a routing override lasts one step
@@ -655,12 +661,90 @@ extern "C" int rd_step_batch(rd_model *m, int B, const int *slot, const int *pos
         rd_set_error("rd_step_batch: want=%d needs its output buffer", want);
         return RD_ERR_ARG;
     }
-    return model_step(m, B, slot, pos, emb, nullptr, want, logits, ids);
+    return model_step(m, B, slot, pos, emb, nullptr, want, logits, ids, false);
+}
+
+// resident/subsystems.go:112-117 StepRagged, forward.go:9-16 ForwardN, subsystems.go:124 PrefillLast: sequences of one or more
+// rows at consecutive positions. Rows go through the step's kernels in passes of at most 32 (the GEMMs' row tile), in the
+// order given; a sequence longer than a pass simply continues in the next one.
+extern "C" int rd_step_ragged(rd_model *m, int n_seq, const int *slot, const int *pos, const int *n_rows, const float *emb, int want, float *logits,
+                              int *ids) {
+    if (!m || !slot || !pos || !n_rows || !emb || n_seq <= 0) return RD_ERR_ARG;
+    if (((want & RD_WANT_LOGITS) && !logits) || ((want & RD_WANT_ARGMAX) && !ids) || !(want & 3)) {
+        rd_set_error("rd_step_ragged: want=%d needs its output buffer", want);
+        return RD_ERR_ARG;
+    }
+    if (!m->finalized || !m->tables) {
+        rd_set_error("step before rd_model_finalize / rd_kv_configure");
+        return RD_ERR_STATE;
+    }
+    // validate the whole call first: a refused call writes nothing
+    std::vector<int> rslot, rpos;
+    for (int i = 0; i < n_seq; i++) {
+        if (!slot_ok(m, slot[i])) return RD_ERR_ARG;
+        for (int a = 0; a < i; a++)
+            if (slot[a] == slot[i]) {
+                rd_set_error("KV slot %d is named by two sequences", slot[i]);
+                return RD_ERR_ARG;
+            }
+        if (n_rows[i] <= 0) {
+            rd_set_error("sequence %d has no rows", i);
+            return RD_ERR_ARG;
+        }
+        if (pos[i] < 0 || pos[i] > m->slot_len[(size_t)slot[i]]) {
+            rd_set_error("sequence %d: position %d but slot %d holds %d rows", i, pos[i], slot[i], m->slot_len[(size_t)slot[i]]);
+            return RD_ERR_ARG;
+        }
+        if (pos[i] + n_rows[i] > m->ctx_cap) {
+            rd_set_error("sequence %d: rows %d..%d reach the context cap %d", i, pos[i], pos[i] + n_rows[i] - 1, m->ctx_cap);
+            return RD_ERR_KV_FULL;
+        }
+        for (int j = 0; j < n_rows[i]; j++) rslot.push_back(slot[i]), rpos.push_back(pos[i] + j);
+    }
+    const size_t H = (size_t)m->desc.hidden, V = (size_t)m->desc.vocab;
+    for (size_t r0 = 0; r0 < rslot.size(); r0 += 32) {
+        const int rows = (int)std::min<size_t>(32, rslot.size() - r0);
+        RC(model_step(m, rows, rslot.data() + r0, rpos.data() + r0, emb + r0 * H, nullptr, want, logits ? logits + r0 * V : nullptr,
+                      ids ? ids + r0 : nullptr, true));
+    }
+    return RD_OK;
+}
+
+// PrefillLast: n rows of one sequence from start_pos; only the last row's logits come back.
+extern "C" int rd_prefill_last(rd_model *m, int slot, int start_pos, int n, const float *emb, float *logits) {
+    if (!m || !emb || !logits || n <= 0) return RD_ERR_ARG;
+    if (!m->finalized || !m->tables) {
+        rd_set_error("prefill before rd_model_finalize / rd_kv_configure");
+        return RD_ERR_STATE;
+    }
+    if (!slot_ok(m, slot)) return RD_ERR_ARG;
+    if (start_pos < 0 || start_pos > m->slot_len[(size_t)slot]) {
+        rd_set_error("prefill at position %d but slot %d holds %d rows", start_pos, slot, m->slot_len[(size_t)slot]);
+        return RD_ERR_ARG;
+    }
+    if (start_pos + n > m->ctx_cap) {
+        rd_set_error("prefill rows %d..%d reach the context cap %d", start_pos, start_pos + n - 1, m->ctx_cap);
+        return RD_ERR_KV_FULL;
+    }
+    const size_t H = (size_t)m->desc.hidden;
+    std::vector<int> rslot(32, slot), rpos(32);
+    std::vector<float> tail; // the last pass returns its rows' logits; only the final row is handed on
+    std::vector<int> idsink(32);
+    for (int r0 = 0; r0 < n; r0 += 32) {
+        const int rows = std::min(32, n - r0);
+        const bool last = r0 + rows == n;
+        for (int j = 0; j < rows; j++) rpos[(size_t)j] = start_pos + r0 + j;
+        if (last) tail.resize((size_t)rows * m->desc.vocab);
+        RC(model_step(m, rows, rslot.data(), rpos.data(), emb + (size_t)r0 * H, nullptr, last ? RD_WANT_LOGITS : RD_WANT_ARGMAX, last ? tail.data() : nullptr,
+                      last ? nullptr : idsink.data(), true));
+        if (last) memcpy(logits, tail.data() + (size_t)(rows - 1) * m->desc.vocab, sizeof(float) * (size_t)m->desc.vocab);
+    }
+    return RD_OK;
 }
 
 extern "C" int rd_forward(rd_model *m, int slot, int pos, const float *emb, float *logits) {
     if (!m || !emb || !logits) return RD_ERR_ARG;
-    return model_step(m, 1, &slot, &pos, emb, nullptr, RD_WANT_LOGITS, logits, nullptr);
+    return model_step(m, 1, &slot, &pos, emb, nullptr, RD_WANT_LOGITS, logits, nullptr, false);
 }
 
 extern "C" int rd_moe_replay(rd_model *m, int B, const int *idx, const float *wgt) {

@@ -88,5 +88,6 @@ struct rd_model {
     StepTimer timer;
 };
 
+// multirow: a slot may carry several rows at consecutive positions (ragged verify / prefill rows)
 int model_step(rd_model *m, int B, const int *slot, const int *pos, const float *emb_host, const float *emb_dev, int want, float *logits,
-               int *ids);
+               int *ids, bool multirow = false);

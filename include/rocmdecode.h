@@ -123,6 +123,16 @@ int rd_kv_reset(rd_model *m, int slot);
 /* emb: host f32 [B][hidden] (embedding rows, already scaled: decoder/residency.go:1077-1123);
  * logits: host f32 [B][vocab] when want&RD_WANT_LOGITS; ids: int32 [B] when want&RD_WANT_ARGMAX (lowest index wins). */
 int rd_step_batch(rd_model *m, int B, const int *slot, const int *pos, const float *emb, int want, float *logits, int *ids);
+/* resident/subsystems.go:112-117 StepRagged (and resident/forward.go:9-16 ForwardN as its one-sequence case): n_seq sequences
+ * on distinct slots, sequence i with n_rows[i] >= 1 rows at positions pos[i], pos[i]+1, ... Rows are laid out sequence after
+ * sequence: emb host f32 [sum n_rows][hidden]; logits [sum n_rows][vocab] / ids [sum n_rows] as in rd_step_batch. Row j of a
+ * sequence equals that sequence's own rd_forward at pos+j bit for bit. A refused call (RD_ERR_ARG, RD_ERR_KV_FULL) writes nothing. */
+int rd_step_ragged(rd_model *m, int n_seq, const int *slot, const int *pos, const int *n_rows, const float *emb, int want, float *logits,
+                   int *ids);
+/* resident/subsystems.go:124 PrefillLast: n prompt rows of one slot from start_pos into the same paged KV the decode step reads;
+ * logits: host f32 [vocab] of the last row. The rows run through the decode step's kernels 32 at a time (every pass re-streams
+ * the weights: correct and bit-identical to token-by-token, not yet a prefill-rate kernel). */
+int rd_prefill_last(rd_model *m, int slot, int start_pos, int n, const float *emb, float *logits);
 /* Forward(embedding, pos) on one slot: the B=1 step through the same kernels */
 int rd_forward(rd_model *m, int slot, int pos, const float *emb, float *logits);
 /* expert indices the last step routed to: int32 [B][n_layers][top_k] (MoE models only; parity checks) */

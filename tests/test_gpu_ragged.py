@@ -1,0 +1,107 @@
+"""The ragged step and the prefill bridge (rd_step_ragged, rd_prefill_last) against the single-token path and the oracle.
+
+goinfer's contract for StepRagged / ForwardN (resident/forward.go:9-16, resident/subsystems.go:112-117): row j of a sequence
+equals that sequence's own Forward at Pos+j bit for bit, and the K/V a prefill pass leaves behind are those the token-by-token
+path would have left. Both are asserted with array_equal; the oracle comparison carries the usual noise-floor bar."""
+import numpy as np
+import pytest
+
+from goinfer_amd import capi
+from oracle import binding as ob
+from tests.models import Pair, dense_cfg, logits_close, moe_cfg, perturbed
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    d = capi.Device(0)
+    yield d
+    d.close()
+
+
+def bits(x):
+    return np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+
+
+def forward_tokens(pair, slot, toks, start=0):
+    """Token by token on one slot; returns every position's logits."""
+    return np.stack([pair.gpu.forward(slot, start + p, pair.emb[t]) for p, t in enumerate(toks)])
+
+
+@pytest.mark.parametrize("cfg", [dense_cfg(), moe_cfg()], ids=["dense", "moe"])
+def test_ragged_rows_equal_single_token_steps(dev, cfg):
+    pair = Pair(cfg, seed=51, dev=dev, slots=8, ctx_cap=256)
+    rng = np.random.default_rng(5)
+    a, b, c = (list(rng.integers(0, cfg["vocab"], n)) for n in (5, 1, 40))
+    want = [forward_tokens(pair, 4 + i, t) for i, t in enumerate((a, b, c))]  # twins on slots 4..6
+    # one call: 5 + 1 + 40 rows = two passes of the step; the 40-row sequence straddles them
+    got, ids = pair.gpu.step_ragged([0, 1, 2], [0, 0, 0], [pair.emb[a], pair.emb[b], pair.emb[c]], capi.WANT_LOGITS | capi.WANT_ARGMAX)
+    off = 0
+    for w in want:
+        assert np.array_equal(bits(got[off:off + len(w)]), bits(w))
+        assert np.array_equal(ids[off:off + len(w)], np.argmax(w, axis=1))
+        off += len(w)
+    # the KV left behind is the token-by-token KV: the next single-token step agrees bit for bit
+    nxt = int(rng.integers(0, cfg["vocab"]))
+    for s, n in ((0, 5), (1, 1), (2, 40)):
+        assert np.array_equal(bits(pair.gpu.forward(s, n, pair.emb[nxt])), bits(pair.gpu.forward(4 + s, n, pair.emb[nxt])))
+    # a second ragged call continues where the first stopped (decode row + verify rows)
+    more = list(rng.integers(0, cfg["vocab"], 3))
+    g2, _ = pair.gpu.step_ragged([2, 0], [41, 6], [pair.emb[more], pair.emb[more[:1]]])
+    w2 = forward_tokens(pair, 6, more, start=41)
+    assert np.array_equal(bits(g2[:3]), bits(w2))
+    pair.close()
+
+
+def test_prefill_last_matches_token_by_token_and_oracle(dev):
+    cfg = dense_cfg()
+    pair = Pair(cfg, seed=52, dev=dev, slots=4, ctx_cap=256)
+    rng = np.random.default_rng(6)
+    toks = list(rng.integers(0, cfg["vocab"], 97))  # four passes: 32 + 32 + 32 + 1
+    got = pair.gpu.prefill_last(0, 0, pair.emb[toks])
+    want = forward_tokens(pair, 1, toks)[-1]
+    assert np.array_equal(bits(got), bits(want))
+    # a prefix prefilled, then the rest: the same bits (PrefillTailExact, resident/forward.go:105-109)
+    pair.gpu.prefill_last(2, 0, pair.emb[toks[:40]])
+    tail = pair.gpu.prefill_last(2, 40, pair.emb[toks[40:]])
+    assert np.array_equal(bits(tail), bits(want))
+    # against the oracle
+    c1, c2 = pair.oracle.new_cache(256), pair.oracle.new_cache(256)
+    floor = 0.0
+    for p, t in enumerate(toks):
+        o = pair.oracle.step(pair.emb[t][None, :], [c1])
+        o2 = pair.oracle.step(perturbed(pair.emb[t][None, :], 1e-6, (7, p)), [c2])
+        floor = max(floor, float(np.abs(o - o2).max()))
+    ok, d = logits_close(got, o[0], floor)
+    assert ok, (d, floor)
+    # and decode continues from the prefilled slot
+    t = ob.argmax(o[0])
+    g, _ = pair.gpu.step_batch([0], [97], pair.emb[t][None, :])
+    o = pair.oracle.step(pair.emb[t][None, :], [c1])
+    o2 = pair.oracle.step(perturbed(pair.emb[t][None, :], 1e-6, (7, 97)), [c2])
+    ok, d = logits_close(g[0], o[0], max(floor, float(np.abs(o - o2).max())))
+    assert ok, (d, floor)
+    pair.close()
+
+
+def test_ragged_refusals_write_nothing(dev):
+    cfg = dense_cfg()
+    pair = Pair(cfg, seed=53, dev=dev, slots=4, ctx_cap=64)
+    e = pair.emb[[1, 2, 3]]
+    with pytest.raises(capi.RocmError, match="two sequences"):
+        pair.gpu.step_ragged([0, 0], [0, 0], [e, e])
+    with pytest.raises(capi.RocmError, match="holds 0 rows"):
+        pair.gpu.step_ragged([0], [2], [e])
+    with pytest.raises(capi.RocmError, match=r"\(-4\)"):  # RD_ERR_KV_FULL: 70 rows do not fit a 64-row slot
+        pair.gpu.step_ragged([1], [0], [pair.emb[list(range(70))]])
+    with pytest.raises(capi.RocmError, match=r"\(-4\)"):
+        pair.gpu.prefill_last(1, 0, pair.emb[list(range(70))])
+    # nothing was written: slot 1 still starts at position 0, and its first token equals a fresh slot's
+    a = pair.gpu.forward(1, 0, pair.emb[5])
+    b = pair.gpu.forward(2, 0, pair.emb[5])
+    assert np.array_equal(bits(a), bits(b))
+    # a step that names a slot twice without consecutive positions is still refused by the plain batch step
+    with pytest.raises(capi.RocmError, match="appears twice"):
+        pair.gpu.step_batch([3, 3], [0, 1], pair.emb[[1, 2]])
+    pair.close()
