@@ -174,32 +174,33 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
         if (!rc) rc = d->sync();
         for (auto &w : ws) free_weight(d, &w);
     } else if (nm == "barrier" && n_args >= 4) {
-        // args {blocks, words, rounds, shift}: the grid barrier's cost and its cross-block hand-off; ms_out per launch, and the launch
+        // args {blocks, words, rounds, shift[, mode]}: the grid barrier's cost and its cross-block hand-off; ms_out per launch, and the launch
         // fails with RD_ERR_STATE if a hand-off delivered stale data or the barrier gave up
-        int blocks = (int)args[0], words = (int)args[1], rounds = (int)args[2], shift = (int)args[3];
+        int blocks = (int)args[0], words = (int)args[1], rounds = (int)args[2], shift = (int)args[3], mode = n_args > 4 ? (int)args[4] : 0;
+        const size_t ctrBytes = 128 * 12; // flag, eight group counters, top counter, abort flag: one 128-byte line each
         DevBuf ctr(d), buf(d), out(d);
-        rc = ctr.alloc(256);
+        rc = ctr.alloc(ctrBytes);
         if (!rc) rc = buf.alloc(sizeof(float) * (size_t)blocks * words);
         if (!rc) rc = out.alloc(sizeof(int) * (size_t)blocks);
         for (int i = 0; i < warmup + iters && !rc; i++) {
-            rc = rd_hip_ok(d->hip, d->hip->MemsetAsync(ctr.p, 0, 256, d->stream), "memset") ? RD_OK : RD_ERR_HIP;
+            rc = rd_hip_ok(d->hip, d->hip->MemsetAsync(ctr.p, 0, ctrBytes, d->stream), "memset") ? RD_OK : RD_ERR_HIP;
             if (!rc) rc = rd_hip_ok(d->hip, d->hip->MemsetAsync(out.p, 0, sizeof(int) * (size_t)blocks, d->stream), "memset") ? RD_OK : RD_ERR_HIP;
             if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup)], d->stream);
             if (!rc)
-                rc = d->launch(d->k.barrier_probe, (unsigned)blocks, 1, 1, 256, ctr.as<unsigned>(), ctr.as<unsigned>() + 32, buf.as<float>(), words, rounds,
-                               shift, 200000u, out.as<int>());
+                rc = d->launch(d->k.barrier_probe, (unsigned)blocks, 1, 1, 256, ctr.as<unsigned>(), ctr.as<unsigned>() + 32 * 11, buf.as<float>(), words, rounds,
+                               shift, 200000u, out.as<int>(), mode);
             if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup) + 1], d->stream);
         }
         if (!rc) rc = d->sync();
         if (!rc) {
             std::vector<int> h((size_t)blocks);
-            unsigned flag[64];
+            unsigned flag[32 * 12];
             rc = d->d2h(h.data(), out.p, sizeof(int) * (size_t)blocks);
-            if (!rc) rc = d->d2h(flag, ctr.p, 256);
+            if (!rc) rc = d->d2h(flag, ctr.p, ctrBytes);
             long bad = 0;
             for (int v : h) bad += v;
-            if (!rc && (bad || flag[32])) {
-                rd_set_error("barrier probe: %ld stale hand-offs, abort flag %u", bad, flag[32]);
+            if (!rc && (bad || flag[32 * 11])) {
+                rd_set_error("barrier probe: %ld stale hand-offs, abort flag %u", bad, flag[32 * 11]);
                 rc = RD_ERR_STATE;
             }
         }
