@@ -8,7 +8,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB = None
 
-OR_F32, OR_Q4K, OR_W4A8, OR_W8A8 = 0, 1, 2, 3
+OR_F32, OR_Q4K, OR_W4A8, OR_W8A8, OR_Q5K, OR_Q6K = 0, 1, 2, 3, 4, 5
 
 
 class Mat(C.Structure):
@@ -96,6 +96,22 @@ def dequant_q4k(blocks):
     nb = blocks.size // 144
     out = np.empty(nb * 256, np.float32)
     lib().or_dequant_q4k(_p(blocks), C.c_size_t(nb), _p(out))
+    return out
+
+
+def dequant_q5k(blocks):
+    blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+    nb = blocks.size // 176
+    out = np.empty(nb * 256, np.float32)
+    lib().or_dequant_q5k(_p(blocks), C.c_size_t(nb), _p(out))
+    return out
+
+
+def dequant_q6k(blocks):
+    blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+    nb = blocks.size // 210
+    out = np.empty(nb * 256, np.float32)
+    lib().or_dequant_q6k(_p(blocks), C.c_size_t(nb), _p(out))
     return out
 
 

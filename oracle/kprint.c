@@ -152,6 +152,17 @@ static uint8_t *g_blocks_q4k(gen *g, int n_blocks) {
         }
     return raw;
 }
+/* the same for any block format: size bytes per block, n16 binary16 fields at the given offsets */
+static uint8_t *g_blocks_fmt(gen *g, int n_blocks, int size, const int *f16_at, int n16) {
+    uint8_t *raw = g_bytes(g, n_blocks * size);
+    for (int b = 0; b < n_blocks; b++)
+        for (int f = 0; f < n16; f++) {
+            uint16_t h = g_half16_one(g, 5, 11) & 0x7fff;
+            raw[b * size + f16_at[f]] = (uint8_t)h;
+            raw[b * size + f16_at[f] + 1] = (uint8_t)(h >> 8);
+        }
+    return raw;
+}
 static float *g_probs(gen *g, int rows, int nKeys) {
     float *p = (float *)malloc(sizeof(float) * (size_t)rows * nKeys);
     for (int i = 0; i < rows * nKeys; i++) p[i] = (float)(g_unit(g) + 1) * (1.0f / 512);
@@ -214,6 +225,31 @@ static void k_f16_to_f32(sha256 *s, gen *g) {
     for (int h = 0; h < 65536; h++) out[h] = or_f16_to_f32((uint16_t)h);
     s_f32(s, out, 65536);
     free(out);
+}
+
+/* kernelprint.go:888-918 (ggufTensor1) for Q5_K (ggml type 13) and Q6_K (type 14); formats.go:30-31 give the block shapes */
+static void k_gguf_fmt(sha256 *s, gen *g, int size, const int *f16_at, int n16, void (*deq)(const uint8_t *, size_t, float *)) {
+    static const int nbs[] = {1, 3}, rws[] = {1, 3};
+    for (int a = 0; a < 2; a++)
+        for (int b = 0; b < 2; b++) {
+            int nb = nbs[a], rows = rws[b], cols = nb * 256, nblk = rows * cols / 256;
+            uint8_t *data = g_blocks_fmt(g, nblk, size, f16_at, n16);
+            float *out = (float *)malloc(sizeof(float) * (size_t)rows * cols);
+            deq(data, (size_t)nblk, out);
+            long t[3] = {nb, rows, 2};
+            s_tag(s, "t", 3, t);
+            s_f32(s, out, (size_t)rows * cols);
+            free(out);
+            free(data);
+        }
+}
+static void k_gguf_q5k(sha256 *s, gen *g) {
+    static const int at[] = {0, 2};
+    k_gguf_fmt(s, g, 176, at, 2, or_dequant_q5k);
+}
+static void k_gguf_q6k(sha256 *s, gen *g) {
+    static const int at[] = {208};
+    k_gguf_fmt(s, g, 210, at, 1, or_dequant_q6k);
 }
 
 /* kernelprint.go:888-918 (ggufTensor1) for Q4_K */
@@ -417,6 +453,8 @@ static const kernel suite[] = {
     {"linalg.F32ToF16", k_f32_to_f16},
     {"linalg.F16ToF32", k_f16_to_f32},
     {"embed.GGUFFile(Q4_K).Tensor", k_gguf_q4k},
+    {"embed.GGUFFile(Q5_K).Tensor", k_gguf_q5k},
+    {"embed.GGUFFile(Q6_K).Tensor", k_gguf_q6k},
     {"linalg.QuantizeRowInt8", k_quantize_row_int8},
     {"linalg.QuantizeActQ", k_quantize_act},
     {"linalg.QuantizeGroupInt4Row", k_quantize_group_int4_row},

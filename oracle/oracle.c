@@ -91,6 +91,51 @@ void or_dequant_q4k(const uint8_t *blocks, size_t n_blocks, float *out) {
     }
 }
 
+/* The public ggml Q5_K layout (ggml-quants dequantize_row_q5_K; the reference's kernels state it at
+ * backend/cuda/actgroup.cu:77-137): 64 elements per pass, low nibbles then high nibbles of qs[32*pass..], fifth bits from
+ * bits 2*pass and 2*pass+1 of qh[l]. Products d*sc and dmin*m formed first, as for Q4_K. */
+static inline int q5k_code(const uint8_t *blk, int e) {
+    int j = e / 32, l = e % 32;
+    int nib = (blk[48 + (j / 2) * 32 + l] >> (4 * (j & 1))) & 15;
+    return nib | (((blk[16 + l] >> j) & 1) << 4);
+}
+void or_dequant_q5k(const uint8_t *blocks, size_t n_blocks, float *out) {
+    for (size_t b = 0; b < n_blocks; b++) {
+        const uint8_t *blk = blocks + b * 176;
+        float d = or_f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+        float dmin = or_f16_to_f32((uint16_t)(blk[2] | (blk[3] << 8)));
+        float *o = out + b * 256;
+        for (int j = 0; j < 8; j++) {
+            int sc, m;
+            or_q4k_scale_min(j, blk + 4, &sc, &m);
+            float d1 = d * (float)sc, m1 = dmin * (float)m;
+            for (int l = 0; l < 32; l++) o[j * 32 + l] = d1 * (float)q5k_code(blk, j * 32 + l) - m1;
+        }
+    }
+}
+
+/* The public ggml Q6_K layout (dequantize_row_q6_K; backend/cuda/actgroup.cu:139-205): two halves of 128 elements; in a
+ * half, element 32*g + l (g = 0..3) takes its nibble from ql[64*half + 32*(g&1) + l] (low for g < 2, high above) and its two
+ * high bits from bits 2g, 2g+1 of qh[32*half + l]; its sub-block scale is sc[8*half + 2*g + l/16]. w = (d*sc) * (q-32). */
+static inline int q6k_code(const uint8_t *blk, int e) {
+    int half = e / 128, r = e % 128, g = r / 32, l = r % 32;
+    int nib = (blk[64 * half + 32 * (g & 1) + l] >> (4 * (g >> 1))) & 15;
+    int hi = (blk[128 + 32 * half + l] >> (2 * g)) & 3;
+    return (nib | (hi << 4)) - 32;
+}
+static inline int q6k_scale(const uint8_t *blk, int e) {
+    int half = e / 128, r = e % 128, g = r / 32, l = r % 32;
+    return (int)(int8_t)blk[192 + 8 * half + 2 * g + l / 16];
+}
+void or_dequant_q6k(const uint8_t *blocks, size_t n_blocks, float *out) {
+    for (size_t b = 0; b < n_blocks; b++) {
+        const uint8_t *blk = blocks + b * 210;
+        float d = or_f16_to_f32((uint16_t)(blk[208] | (blk[209] << 8)));
+        float *o = out + b * 256;
+        for (int e = 0; e < 256; e++) o[e] = (d * (float)q6k_scale(blk, e)) * (float)q6k_code(blk, e);
+    }
+}
+
 /* ------------------------------------------------------------------ activation quantizers */
 static inline float round_half_away(float x) { return roundf(x); }
 
@@ -372,6 +417,73 @@ static void matmul_q4k(const or_mat *w, const int8_t *aq, const float *aS, int M
     free(asum);
 }
 
+/* Q5_K x per-32 int8 activations, backend/cuda/actgroup.cu:85-137 (rowsQ5K): per 32-group
+ * facc = fma(idot, (d*sc)*aS, facc); facc = fma(-(dmin*m), asum, facc), groups ascending. */
+static void matmul_q5k(const or_mat *w, const int8_t *aq, const float *aS, int M, float *dst) {
+    int N = w->N, K = w->K, nSB = K / 256, nG = K / 32;
+    const uint8_t *W = (const uint8_t *)w->data;
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+    for (int n = 0; n < N; n++) {
+        const uint8_t *row = W + (size_t)n * nSB * 176;
+        for (int m = 0; m < M; m++) {
+            const int8_t *a = aq + (size_t)m * K;
+            float facc = 0.f;
+            for (int b = 0; b < nSB; b++) {
+                const uint8_t *blk = row + (size_t)b * 176;
+                float d = or_f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+                float dmin = or_f16_to_f32((uint16_t)(blk[2] | (blk[3] << 8)));
+                for (int j = 0; j < 8; j++) {
+                    int sc, mn;
+                    or_q4k_scale_min(j, blk + 4, &sc, &mn);
+                    int32_t idot = 0, asum = 0;
+                    for (int l = 0; l < 32; l++) {
+                        idot += (int32_t)q5k_code(blk, j * 32 + l) * (int32_t)a[b * 256 + j * 32 + l];
+                        asum += a[b * 256 + j * 32 + l];
+                    }
+                    int g = b * 8 + j;
+                    float as = aS[(size_t)m * nG + g];
+                    facc = fmaf((float)idot, (d * (float)sc) * as, facc);
+                    facc = fmaf(-(dmin * (float)mn), as * (float)asum, facc);
+                }
+            }
+            dst[(size_t)m * N + n] = facc;
+        }
+    }
+}
+
+/* Q6_K x per-32 int8 activations, backend/cuda/actgroup.cu:139-205 (rowsQ6K): an activation group of 32 spans two 16-element
+ * sub-blocks; facc = fma((float)(sc_lo*idot_lo + sc_hi*idot_hi), d*aS, facc) in the mathematically specified form (the CUDA
+ * lanes fold sc*idot per 8 elements; the integer part is exact either way), groups ascending. */
+static void matmul_q6k(const or_mat *w, const int8_t *aq, const float *aS, int M, float *dst) {
+    int N = w->N, K = w->K, nSB = K / 256, nG = K / 32;
+    const uint8_t *W = (const uint8_t *)w->data;
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+    for (int n = 0; n < N; n++) {
+        const uint8_t *row = W + (size_t)n * nSB * 210;
+        for (int m = 0; m < M; m++) {
+            const int8_t *a = aq + (size_t)m * K;
+            float facc = 0.f;
+            for (int b = 0; b < nSB; b++) {
+                const uint8_t *blk = row + (size_t)b * 210;
+                float d = or_f16_to_f32((uint16_t)(blk[208] | (blk[209] << 8)));
+                for (int j = 0; j < 8; j++) {
+                    int32_t acc = 0;
+                    for (int h = 0; h < 2; h++) {
+                        int32_t idot = 0;
+                        for (int l = 0; l < 16; l++) {
+                            int e = j * 32 + h * 16 + l;
+                            idot += (int32_t)q6k_code(blk, e) * (int32_t)a[b * 256 + e];
+                        }
+                        acc += (int32_t)q6k_scale(blk, j * 32 + h * 16) * idot;
+                    }
+                    facc = fmaf((float)acc, d * aS[(size_t)m * nG + b * 8 + j], facc);
+                }
+            }
+            dst[(size_t)m * N + n] = facc;
+        }
+    }
+}
+
 static void matmul_w4a8(const or_mat *w, const int8_t *aq, const float *aS, int M, float *dst) {
     int N = w->N, K = w->K, nG = (K + 31) / 32, bpr = (K + 1) / 2, ag = w->act_group;
     const uint8_t *W = (const uint8_t *)w->data;
@@ -447,6 +559,10 @@ void or_matmul(const or_mat *w, const float *a, int M, float *dst) {
     or_quantize_act(a, M, K, group, aq, aS);
     if (w->kind == OR_Q4K)
         matmul_q4k(w, aq, aS, M, dst);
+    else if (w->kind == OR_Q5K)
+        matmul_q5k(w, aq, aS, M, dst);
+    else if (w->kind == OR_Q6K)
+        matmul_q6k(w, aq, aS, M, dst);
     else if (w->kind == OR_W4A8)
         matmul_w4a8(w, aq, aS, M, dst);
     else
@@ -467,6 +583,19 @@ static double weight_at(const or_mat *w, int n, int k) {
         double dmin = or_f16_to_f32((uint16_t)(blk[2] | (blk[3] << 8)));
         int q = (blk[16 + (j / 2) * 32 + l] >> (4 * (j & 1))) & 15;
         return d * sc * q - dmin * m;
+    }
+    case OR_Q5K: {
+        const uint8_t *blk = (const uint8_t *)w->data + ((size_t)n * (w->K / 256) + k / 256) * 176;
+        int e = k % 256, sc, m;
+        or_q4k_scale_min(e / 32, blk + 4, &sc, &m);
+        double d = or_f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+        double dmin = or_f16_to_f32((uint16_t)(blk[2] | (blk[3] << 8)));
+        return d * sc * q5k_code(blk, e) - dmin * m;
+    }
+    case OR_Q6K: {
+        const uint8_t *blk = (const uint8_t *)w->data + ((size_t)n * (w->K / 256) + k / 256) * 210;
+        int e = k % 256;
+        return (double)or_f16_to_f32((uint16_t)(blk[208] | (blk[209] << 8))) * q6k_scale(blk, e) * q6k_code(blk, e);
     }
     case OR_W4A8: {
         int nG = (w->K + 31) / 32, bpr = (w->K + 1) / 2;

@@ -42,7 +42,13 @@ float or_f16_to_f32(uint16_t h);
 
 /* ---- Q4_K: decoder/gguf.go:1508-1537, backend/metal/kernels/gemm_kq_test.go:27-70 ---- */
 void or_q4k_scale_min(int j, const uint8_t *q12, int *sc, int *m);
-void or_dequant_q4k(const uint8_t *blocks, size_t n_blocks, float *out); /* 144 B -> 256 f32 each */
+void or_dequant_q4k(const uint8_t *blocks, size_t n_blocks, float *out);
+/* GGUF Q5_K (176-byte super-blocks: d, dmin f16; 12 bytes of 6-bit scales and mins as Q4_K; qh[32] fifth bits; qs[128] nibbles):
+ * w = d*sc_j*q - dmin*m_j with q = nibble | fifth bit << 4. Pinned bit-exact by fingerprint embed.GGUFFile(Q5_K).Tensor. */
+void or_dequant_q5k(const uint8_t *blocks, size_t n_blocks, float *out);
+/* GGUF Q6_K (210-byte super-blocks: ql[128] low nibbles, qh[64] two high bits each, 16 int8 sub-block scales, d f16):
+ * w = d*sc_s*(q-32), 16 sub-blocks of 16. Pinned bit-exact by fingerprint embed.GGUFFile(Q6_K).Tensor. */
+void or_dequant_q6k(const uint8_t *blocks, size_t n_blocks, float *out); /* 144 B -> 256 f32 each */
 
 /* ---- activation quantizers: backend/cuda/kv8_store.cu:3-35, actgroup.cu:26-54 ---- */
 float or_quantize_row_int8(const float *row, int n, int8_t *q);
@@ -68,7 +74,7 @@ int or_route_experts(const float *logits, int nE, int k, int norm, double scale,
 int or_argmax(const float *x, int n); /* internal/runtime/sampling/sampler.go:485-520: first maximum wins */
 
 /* ---- weight matrices and the matmul dispatch: decoder/weightmat.go:845-985 ---- */
-enum { OR_F32 = 0, OR_Q4K = 1, OR_W4A8 = 2, OR_W8A8 = 3 };
+enum { OR_F32 = 0, OR_Q4K = 1, OR_W4A8 = 2, OR_W8A8 = 3, OR_Q5K = 4, OR_Q6K = 5 };
 typedef struct {
     int kind;           /* OR_* */
     int N, K;           /* rows (outputs), cols (inputs) */

@@ -17,6 +17,8 @@ PINS = {
     "linalg.F32ToF16": ALL,
     "linalg.F16ToF32": ALL,
     "embed.GGUFFile(Q4_K).Tensor": ALL,
+    "embed.GGUFFile(Q5_K).Tensor": ALL,
+    "embed.GGUFFile(Q6_K).Tensor": ALL,
     "linalg.QuantizeRowInt8": ALL,
     "linalg.QuantizeActQ": ALL,
     "linalg.QuantizeGroupInt4Row": ALL,
