@@ -21,6 +21,7 @@ EXPORTS = [
     "rd_kv_configure", "rd_kv_upload", "rd_kv_truncate", "rd_kv_reset", "rd_step_batch", "rd_forward",
     "rd_last_moe_indices", "rd_model_upload_embedding", "rd_bench_steps", "rd_bench_profile", "rd_bench_class_count",
     "rd_bench_class_name", "rd_bench_kernel", "rd_gateup_q4k_quant", "rd_moe_replay", "rd_bench_attn", "rd_step_ragged", "rd_prefill_last",
+    "rd_dequant_q5k", "rd_dequant_q6k", "rd_gemm_q5k", "rd_gemm_q6k", "rd_model_upload_q5k", "rd_model_upload_q6k",
 ]
 
 
@@ -106,6 +107,22 @@ class Device:
         out = np.empty((N, K), np.float32)
         check(lib().rd_dequant_q4k(self.h, _p(blocks), N, K, _p(out)), "rd_dequant_q4k")
         return out
+
+    def dequant_kquant(self, fmt, blocks, N, K):
+        """fmt 'q5k' or 'q6k': raw super-blocks -> f32 [N][K]."""
+        blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+        out = np.empty((N, K), np.float32)
+        name = "rd_dequant_" + fmt
+        check(getattr(lib(), name)(self.h, _p(blocks), N, K, _p(out)), name)
+        return out
+
+    def gemm_kquant(self, fmt, blocks, N, K, a):
+        a = _f32(a)
+        blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+        dst = np.empty((a.shape[0], N), np.float32)
+        name = "rd_gemm_" + fmt
+        check(getattr(lib(), name)(self.h, _p(blocks), N, K, _p(a), a.shape[0], _p(dst)), name)
+        return dst
 
     def gemm_q4k(self, blocks, N, K, a, blocks2=None):
         a = _f32(a)
@@ -207,6 +224,11 @@ class Model:
     def upload_q4k(self, layer, proj, blocks, N, K):
         blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
         check(lib().rd_model_upload_q4k(self.h, layer, PROJ[proj], _p(blocks), N, K), "rd_model_upload_q4k")
+
+    def upload_kquant(self, fmt, layer, proj, blocks, N, K):
+        blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+        name = "rd_model_upload_" + fmt
+        check(getattr(lib(), name)(self.h, layer, PROJ[proj], _p(blocks), N, K), name)
 
     def upload_w8a8(self, layer, proj, q, scales):
         q = np.ascontiguousarray(q, dtype=np.int8)

@@ -81,6 +81,12 @@ static const KName kNames[] = {
     {"rd_k_gemm_w8a8", &Kernels::gemm_w8a8},
     {"rd_k_retile_w4a8", &Kernels::retile_w4a8},
     {"rd_k_gemm_w4a8", &Kernels::gemm_w4a8},
+    {"rd_k_dequant_q5k", &Kernels::dequant_q5k},
+    {"rd_k_retile_q5k", &Kernels::retile_q5k},
+    {"rd_k_gemm_q5k", &Kernels::gemm_q5k},
+    {"rd_k_dequant_q6k", &Kernels::dequant_q6k},
+    {"rd_k_retile_q6k", &Kernels::retile_q6k},
+    {"rd_k_gemm_q6k", &Kernels::gemm_q6k},
     {"rd_k_kv_store", &Kernels::kv_store},
     {"rd_k_qkv_rope_store", &Kernels::qkv_rope_store},
     {"rd_k_attn_partial", &Kernels::attn_partial},
@@ -210,8 +216,8 @@ GemmPlan plan_gemm(int kind, int N, int nKB) {
     return p;
 }
 
-size_t panel_bytes_for(const DevWeight &w) { return w.kind == 0 ? (size_t)(w.K / 256) * Q4K_PANEL_BYTES : (size_t)(w.K / 128) * LIN_PANEL_BYTES; }
-int panel_kind_for(const DevWeight &w) { return w.kind == 0 ? PANEL_Q4K : (w.kind == 1 ? PANEL_LIN : PANEL_LIN4); }
+size_t panel_bytes_for(const DevWeight &w) { return kblock_of(w.kind) == 256 ? (size_t)(w.K / 256) * Q4K_PANEL_BYTES : (size_t)(w.K / 128) * LIN_PANEL_BYTES; }
+int panel_kind_for(const DevWeight &w) { return kblock_of(w.kind) == 256 ? PANEL_Q4K : (w.kind == 2 ? PANEL_LIN4 : PANEL_LIN); }
 
 int upload_q4k(rd_device *d, const void *blocks, int N, int K, DevWeight *w) {
     if (N <= 0 || K <= 0 || K % 256 || N % 32) {
@@ -228,6 +234,44 @@ int upload_q4k(rd_device *d, const void *blocks, int N, int K, DevWeight *w) {
     if ((rc = d->launch(d->k.retile_q4k, N / 32, nSB, 1, 320, (const void *)raw.p, w->tiled, N, nSB))) return rc;
     if ((rc = d->sync())) return rc;
     w->kind = 0, w->N = N, w->K = K;
+    return RD_OK;
+}
+
+// Q5_K: 176 B super-blocks re-tiled to 5632 B per (32 rows, super-block). Q6_K: 210 B super-blocks re-tiled to two
+// 3456 B tiles per (32 rows, super-block), one per half; the tiled form is 6.75 bits per weight against 6.5625 raw.
+int upload_q5k(rd_device *d, const void *blocks, int N, int K, DevWeight *w) {
+    if (N <= 0 || K <= 0 || K % 256 || N % 32) {
+        rd_set_error("q5k upload: N=%d must be a multiple of 32 and K=%d of 256", N, K);
+        return RD_DECLINED;
+    }
+    int nSB = K / 256;
+    size_t bytes = (size_t)N * nSB * 176;
+    DevBuf raw(d);
+    int rc = raw.alloc(bytes);
+    if (rc) return rc;
+    if ((rc = d->alloc(&w->tiled, (size_t)(N / 32) * nSB * 5632))) return rc;
+    if ((rc = d->h2d(raw.p, blocks, bytes))) return rc;
+    if ((rc = d->launch(d->k.retile_q5k, N / 32, nSB, 1, 384, (const void *)raw.p, w->tiled, N, nSB))) return rc;
+    if ((rc = d->sync())) return rc;
+    w->kind = 3, w->N = N, w->K = K;
+    return RD_OK;
+}
+
+int upload_q6k(rd_device *d, const void *blocks, int N, int K, DevWeight *w) {
+    if (N <= 0 || K <= 0 || K % 256 || N % 32) {
+        rd_set_error("q6k upload: N=%d must be a multiple of 32 and K=%d of 256", N, K);
+        return RD_DECLINED;
+    }
+    int nSB = K / 256;
+    size_t bytes = (size_t)N * nSB * 210;
+    DevBuf raw(d);
+    int rc = raw.alloc(bytes);
+    if (rc) return rc;
+    if ((rc = d->alloc(&w->tiled, (size_t)(N / 32) * nSB * 2 * 3456))) return rc;
+    if ((rc = d->h2d(raw.p, blocks, bytes))) return rc;
+    if ((rc = d->launch(d->k.retile_q6k, N / 32, 2 * nSB, 1, 256, (const void *)raw.p, w->tiled, N, nSB))) return rc;
+    if ((rc = d->sync())) return rc;
+    w->kind = 4, w->N = N, w->K = K;
     return RD_OK;
 }
 
@@ -278,12 +322,14 @@ int launch_gemm(rd_device *d, const DevWeight &w, const void *Xp, float *P, int 
         rd_set_error("gemm: M=%d outside 1..32", M);
         return RD_ERR_ARG;
     }
-    int nKB = w.kind == 0 ? w.K / 256 : w.K / 128;
+    int nKB = kblocks_for(w);
     GemmPlan p = plan_gemm(w.kind, w.N, nKB);
     if (plan_out) *plan_out = p;
     unsigned gx = (unsigned)((w.N + 127) / 128);
     if (w.kind == 0)
         return d->launch(d->k.gemm_q4k, gx, p.splits, 1, GEMM_THREADS, (const void *)w.tiled, Xp, P, w.N, nKB, p.kbPerSplit, M);
+    if (w.kind == 3 || w.kind == 4)
+        return d->launch(w.kind == 3 ? d->k.gemm_q5k : d->k.gemm_q6k, gx, p.splits, 1, GEMM_THREADS, (const void *)w.tiled, Xp, P, w.N, nKB, p.kbPerSplit, M);
     if (w.kind == 1)
         return d->launch(d->k.gemm_w8a8, gx, p.splits, 1, GEMM_THREADS, (const void *)w.tiled, (const void *)w.scales, Xp, P, w.N, nKB, p.kbPerSplit, M);
     return d->launch(d->k.gemm_w4a8, gx, p.splits, 1, GEMM_THREADS, (const void *)w.tiled, Xp, P, w.N, nKB, p.kbPerSplit, M);

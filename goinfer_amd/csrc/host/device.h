@@ -23,6 +23,7 @@ enum { PANEL_Q4K = 0, PANEL_LIN = 1, PANEL_LIN4 = 2 };
 struct Kernels {
     hipFunction_t dequant_q4k, retile_q4k, gemm_q4k, quant_act, reduce_splits, add_rmsnorm_quant, swiglu_quant;
     hipFunction_t retile_w8a8, gemm_w8a8, retile_w4a8, gemm_w4a8;
+    hipFunction_t dequant_q5k, retile_q5k, gemm_q5k, dequant_q6k, retile_q6k, gemm_q6k;
     hipFunction_t gemm_q4k_gateup;
     hipFunction_t kv_store, qkv_rope_store, attn_partial, attn_combine, attn_combine_quant;
     hipFunction_t rmsnorm, rope, argmax_rows, argmax_final, matmul_f32, moe_route, gemm_w4a8_moe, moe_swiglu_quant, moe_fold, embed_rows, copy16, barrier_probe, unpanel_q4k, fill_f16, fill_f32;
@@ -87,13 +88,15 @@ GemmPlan plan_gemm(int kind, int N, int nKB);
 
 // Weight matrix resident on the device in its GEMM tiling.
 struct DevWeight {
-    int kind = -1; // 0 q4k, 1 w8a8, 2 w4a8
+    int kind = -1; // 0 q4k, 1 w8a8, 2 w4a8, 3 q5k, 4 q6k
     int N = 0, K = 0;
     void *tiled = nullptr;  // re-tiled codes
     void *scales = nullptr; // w8a8: f32[N]
 };
 
 int upload_q4k(rd_device *d, const void *blocks, int N, int K, DevWeight *w);
+int upload_q5k(rd_device *d, const void *blocks, int N, int K, DevWeight *w);
+int upload_q6k(rd_device *d, const void *blocks, int N, int K, DevWeight *w);
 int upload_w8a8(rd_device *d, const int8_t *q, const float *row_scale, int N, int K, DevWeight *w);
 int upload_w4a8(rd_device *d, const uint8_t *nib, const uint16_t *s16, int N, int K, DevWeight *w);
 void free_weight(rd_device *d, DevWeight *w);
@@ -101,3 +104,6 @@ void free_weight(rd_device *d, DevWeight *w);
 int launch_gemm(rd_device *d, const DevWeight &w, const void *Xp, float *P, int M, GemmPlan *plan);
 size_t panel_bytes_for(const DevWeight &w);
 int panel_kind_for(const DevWeight &w);
+// K-blocks of a weight: super-blocks of 256 for the kinds on Q4_K-style panels (q4k, q5k), 128 otherwise
+inline int kblock_of(int kind) { return (kind == 0 || kind == 3) ? 256 : 128; }
+inline int kblocks_for(const DevWeight &w) { return w.K / kblock_of(w.kind); }

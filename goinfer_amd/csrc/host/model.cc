@@ -107,6 +107,8 @@ static int expect_shape(rd_model *m, int proj, int N, int K) {
 
 static int upload_pending(rd_device *d, const PendingMat &p, DevWeight *w) {
     if (p.kind == 0) return upload_q4k(d, p.data.data(), p.N, p.K, w);
+    if (p.kind == 3) return upload_q5k(d, p.data.data(), p.N, p.K, w);
+    if (p.kind == 4) return upload_q6k(d, p.data.data(), p.N, p.K, w);
     if (p.kind == 1) return upload_w8a8(d, (const int8_t *)p.data.data(), (const float *)p.scales.data(), p.N, p.K, w);
     return upload_w4a8(d, p.data.data(), (const uint16_t *)p.scales.data(), p.N, p.K, w);
 }
@@ -174,6 +176,26 @@ extern "C" int rd_model_upload_q4k(rd_model *m, int layer, int proj, const void 
     pm.kind = 0, pm.N = N, pm.K = K;
     pm.data.assign((const uint8_t *)blocks, (const uint8_t *)blocks + (size_t)N * (K / 256) * 144);
     return accept(m, layer, proj, std::move(pm));
+}
+
+static int upload_kquant(rd_model *m, int layer, int proj, const void *blocks, int N, int K, int kind, int bb, const char *name) {
+    if (!m || !blocks) return RD_ERR_ARG;
+    if (!layer_ok(m, layer, proj == RD_PROJ_HEAD)) return RD_ERR_ARG;
+    RC(expect_shape(m, proj, N, K));
+    if (K % 256) {
+        rd_set_error("%s needs K%%256==0 (goinfer kquant_native.go:88-90), got K=%d", name, K);
+        return RD_DECLINED;
+    }
+    PendingMat pm;
+    pm.kind = kind, pm.N = N, pm.K = K;
+    pm.data.assign((const uint8_t *)blocks, (const uint8_t *)blocks + (size_t)N * (K / 256) * bb);
+    return accept(m, layer, proj, std::move(pm));
+}
+extern "C" int rd_model_upload_q5k(rd_model *m, int layer, int proj, const void *blocks, int N, int K) {
+    return upload_kquant(m, layer, proj, blocks, N, K, 3, 176, "Q5_K");
+}
+extern "C" int rd_model_upload_q6k(rd_model *m, int layer, int proj, const void *blocks, int N, int K) {
+    return upload_kquant(m, layer, proj, blocks, N, K, 4, 210, "Q6_K");
 }
 
 extern "C" int rd_model_upload_w8a8(rd_model *m, int layer, int proj, const int8_t *q, const float *row_scale, int N, int K) {
@@ -275,7 +297,7 @@ extern "C" int rd_model_upload_embedding(rd_model *m, const int8_t *q, const flo
 
 static size_t gemm_partial_floats(const DevWeight &w) {
     if (w.kind < 0) return 0;
-    int nKB = w.kind == 0 ? w.K / 256 : w.K / 128;
+    int nKB = kblocks_for(w);
     return (size_t)plan_gemm(w.kind, w.N, nKB).splits * 32 * w.N;
 }
 

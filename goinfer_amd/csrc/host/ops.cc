@@ -38,7 +38,7 @@ static int gemm_host(rd_device *d, DevWeight &w, DevWeight *w2, const float *a, 
     DevBuf A(d), Xp(d), P(d), O(d);
     RC(A.alloc(sizeof(float) * (size_t)32 * K));
     RC(Xp.alloc(pbytes));
-    int nKB = w.kind == 0 ? K / 256 : K / 128;
+    int nKB = kblocks_for(w);
     int Ntot = w2 ? 2 * N : N;
     int maxSplits = plan_gemm(w.kind, Ntot, nKB).splits;
     RC(P.alloc(sizeof(float) * (size_t)maxSplits * 32 * Ntot));
@@ -127,6 +127,51 @@ extern "C" int rd_gateup_q4k_quant(rd_device *d, const void *Wg, const void *Wu,
         return RD_OK;
     };
     rc = body();
+    free_weight(d, &w);
+    return rc;
+}
+
+// Q5_K / Q6_K: the file's own super-blocks (176 B / 210 B per 256 weights) dequantized or multiplied natively.
+static int dequant_kquant(rd_device *d, hipFunction_t k, int bb, const void *blocks, int N, int K, float *out, const char *who) {
+    if (!d || !blocks || !out || N <= 0 || K <= 0 || K % 256) {
+        rd_set_error("%s: bad arguments (K must be a multiple of 256)", who);
+        return RD_ERR_ARG;
+    }
+    size_t nb = (size_t)N * (K / 256);
+    DevBuf raw(d), o(d);
+    RC(raw.alloc(nb * bb));
+    RC(o.alloc(nb * 256 * sizeof(float)));
+    RC(d->h2d(raw.p, blocks, nb * bb));
+    RC(d->launch(k, (unsigned)nb, 1, 1, 256, (const void *)raw.p, o.as<float>(), (long)nb));
+    return d->d2h(out, o.p, nb * 256 * sizeof(float));
+}
+extern "C" int rd_dequant_q5k(rd_device *d, const void *blocks, int N, int K, float *out) {
+    return dequant_kquant(d, d ? d->k.dequant_q5k : nullptr, 176, blocks, N, K, out, "rd_dequant_q5k");
+}
+extern "C" int rd_dequant_q6k(rd_device *d, const void *blocks, int N, int K, float *out) {
+    return dequant_kquant(d, d ? d->k.dequant_q6k : nullptr, 210, blocks, N, K, out, "rd_dequant_q6k");
+}
+extern "C" int rd_gemm_q5k(rd_device *d, const void *W, int N, int K, const float *a, int M, float *dst) {
+    if (!d || !W || !a || !dst || M <= 0) {
+        rd_set_error("rd_gemm_q5k: bad arguments");
+        return RD_ERR_ARG;
+    }
+    DevWeight w;
+    int rc = upload_q5k(d, W, N, K, &w);
+    if (rc) return rc;
+    rc = gemm_host(d, w, nullptr, a, M, dst);
+    free_weight(d, &w);
+    return rc;
+}
+extern "C" int rd_gemm_q6k(rd_device *d, const void *W, int N, int K, const float *a, int M, float *dst) {
+    if (!d || !W || !a || !dst || M <= 0) {
+        rd_set_error("rd_gemm_q6k: bad arguments");
+        return RD_ERR_ARG;
+    }
+    DevWeight w;
+    int rc = upload_q6k(d, W, N, K, &w);
+    if (rc) return rc;
+    rc = gemm_host(d, w, nullptr, a, M, dst);
     free_weight(d, &w);
     return rc;
 }

@@ -147,6 +147,101 @@ extern "C" void synth_q4k_normal(uint64_t seed, int N, int K, float sigma, uint8
     }
 }
 
+// One super-block: 256 f32 -> 176 bytes of Q5_K (ggml layout): the Q4_K header, 32 levels per sub-block.
+static void quantize_block_q5k(const float *x, uint8_t *blk) {
+    float scales[8], mins[8];
+    float max_scale = 0.f, max_min = 0.f;
+    for (int j = 0; j < 8; j++) {
+        float mn = x[j * 32], mx = x[j * 32];
+        for (int l = 1; l < 32; l++) {
+            float v = x[j * 32 + l];
+            if (v < mn) mn = v;
+            if (v > mx) mx = v;
+        }
+        if (mn > 0.f) mn = 0.f;
+        scales[j] = (mx - mn) / 31.f;
+        mins[j] = -mn;
+        if (scales[j] > max_scale) max_scale = scales[j];
+        if (mins[j] > max_min) max_min = mins[j];
+    }
+    uint16_t dh = f32_to_f16_rne(max_scale / 63.f), mh = f32_to_f16_rne(max_min / 63.f);
+    float d = f16_to_f32(dh), dmin = f16_to_f32(mh);
+    uint8_t ls[8], lm[8];
+    for (int j = 0; j < 8; j++) {
+        int s = d > 0.f ? (int)lrintf(scales[j] / d) : 0, m = dmin > 0.f ? (int)lrintf(mins[j] / dmin) : 0;
+        ls[j] = (uint8_t)(s < 0 ? 0 : (s > 63 ? 63 : s));
+        lm[j] = (uint8_t)(m < 0 ? 0 : (m > 63 ? 63 : m));
+    }
+    memset(blk, 0, 176);
+    blk[0] = (uint8_t)dh, blk[1] = (uint8_t)(dh >> 8), blk[2] = (uint8_t)mh, blk[3] = (uint8_t)(mh >> 8);
+    uint8_t *q = blk + 4;
+    for (int j = 0; j < 8; j++) {
+        if (j < 4) {
+            q[j] |= ls[j];
+            q[j + 4] |= lm[j];
+        } else {
+            q[j + 4] = (uint8_t)((ls[j] & 0xF) | ((lm[j] & 0xF) << 4));
+            q[j - 4] |= (uint8_t)((ls[j] >> 4) << 6);
+            q[j] |= (uint8_t)((lm[j] >> 4) << 6);
+        }
+    }
+    uint8_t *qh = blk + 16, *qs = blk + 48;
+    for (int j = 0; j < 8; j++) {
+        float dl = d * (float)ls[j], ml = dmin * (float)lm[j];
+        for (int l = 0; l < 32; l++) {
+            int v = dl > 0.f ? (int)lrintf((x[j * 32 + l] + ml) / dl) : 0;
+            v = v < 0 ? 0 : (v > 31 ? 31 : v);
+            qs[(j / 2) * 32 + l] |= (uint8_t)((v & 15) << (4 * (j & 1)));
+            qh[l] |= (uint8_t)((v >> 4) << j);
+        }
+    }
+}
+
+// One super-block: 256 f32 -> 210 bytes of Q6_K (ggml layout): 16 sub-blocks of 16, symmetric codes in [-32, 31].
+static void quantize_block_q6k(const float *x, uint8_t *blk) {
+    float scales[16], max_abs_scale = 0.f;
+    for (int j = 0; j < 16; j++) {
+        float am = 0.f, sv = 0.f;
+        for (int l = 0; l < 16; l++) {
+            float v = x[j * 16 + l];
+            if (fabsf(v) > am) am = fabsf(v), sv = v;
+        }
+        scales[j] = -sv / 32.f; // the largest magnitude lands on code -32, as ggml's make_qx_quants does
+        if (fabsf(scales[j]) > max_abs_scale) max_abs_scale = fabsf(scales[j]);
+    }
+    memset(blk, 0, 210);
+    uint16_t dh = f32_to_f16_rne(max_abs_scale / 127.f);
+    float d = f16_to_f32(dh);
+    blk[208] = (uint8_t)dh, blk[209] = (uint8_t)(dh >> 8);
+    for (int j = 0; j < 16; j++) {
+        int s = d > 0.f ? (int)lrintf(scales[j] / d) : 0;
+        s = s < -128 ? -128 : (s > 127 ? 127 : s);
+        blk[192 + j] = (uint8_t)(int8_t)s;
+    }
+    for (int e = 0; e < 256; e++) {
+        int half = e / 128, r = e % 128, g = r / 32, l = r % 32;
+        float dl = d * (float)(int8_t)blk[192 + e / 16];
+        int v = dl != 0.f ? (int)lrintf(x[e] / dl) : 0;
+        v = (v < -32 ? -32 : (v > 31 ? 31 : v)) + 32;
+        blk[64 * half + 32 * (g & 1) + l] |= (uint8_t)((v & 15) << (4 * (g >> 1)));
+        blk[128 + 32 * half + l] |= (uint8_t)((v >> 4) << (2 * g));
+    }
+}
+
+// N x K weights ~ N(0, sigma), element (n,k) = normal_at(seed, n*K+k), as Q5_K (fmt 5) or Q6_K (fmt 6) super-blocks.
+extern "C" void synth_kquant_normal(int fmt, uint64_t seed, int N, int K, float sigma, uint8_t *blocks) {
+    size_t nb = (size_t)N * (K / 256);
+#pragma omp parallel for schedule(static)
+    for (size_t b = 0; b < nb; b++) {
+        float x[256];
+        for (int i = 0; i < 256; i++) x[i] = sigma * normal_at(seed, b * 256 + i);
+        if (fmt == 5)
+            quantize_block_q5k(x, blocks + b * 176);
+        else
+            quantize_block_q6k(x, blocks + b * 210);
+    }
+}
+
 // int8 rows with the reference's rule (aikit QuantizeRowInt8: scale maxabs/127, round half away, zero row -> scale 1).
 extern "C" void synth_w8a8_normal(uint64_t seed, int N, int K, float sigma, int8_t *q, float *scales) {
 #pragma omp parallel for schedule(static)

@@ -4,6 +4,7 @@
 #include "common.h"
 #include "q4k.h"
 #include "lin.h"
+#include "kquant.h"
 #include "act.h"
 #include "attn.h"
 #include "misc.h"

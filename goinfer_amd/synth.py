@@ -34,6 +34,14 @@ def q4k_normal(seed, N, K, sigma=0.02):
     return out
 
 
+def kquant_normal(fmt, seed, N, K, sigma=0.02):
+    """N x K weights ~ N(0, sigma) as raw Q5_K ('q5k', 176 B) or Q6_K ('q6k', 210 B) super-blocks."""
+    bb, code = {"q5k": (176, 5), "q6k": (210, 6)}[fmt]
+    out = np.empty(N * (K // 256) * bb, np.uint8)
+    lib().synth_kquant_normal(code, C.c_uint64(seed), N, K, C.c_float(sigma), _p(out))
+    return out
+
+
 def quantize_q4k(w):
     w = np.ascontiguousarray(w, dtype=np.float32)
     N, K = w.shape

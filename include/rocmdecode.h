@@ -81,6 +81,14 @@ int rd_gemm_q4k(rd_device *d, const void *W, int N, int K, const float *a, int M
  * (decoder/cpu_gateup_fused.go:83-148 followed by linalg.QuantizeActQ at the down projection's input). dst[M][I] receives
  * the quantized activations, code * scale, exactly as the down projection reads them. I and K multiples of 256. */
 int rd_gateup_q4k_quant(rd_device *d, const void *Wg, const void *Wu, int I, int K, const float *a, int M, float *dst);
+/* Q5_K (176 B) and Q6_K (210 B) super-blocks, the file's own bytes as decoder.KQuantReader.RowSource hands them out
+ * (decoder/kquant_native.go:240-265): -> f32 bit-exactly as (d*sc)*q - dmin*m and (d*sc)*(q-32), and
+ * dst[M,N] = a[M,K] . W^T against per-32 int8 activations (backend/cuda/actgroup.cu:457-530 gemv_q5k_g32 / gemv_q6k_g32,
+ * arithmetic at :77-205). Host pointers; K a multiple of 256, N of 32. */
+int rd_dequant_q5k(rd_device *d, const void *blocks, int N, int K, float *out);
+int rd_dequant_q6k(rd_device *d, const void *blocks, int N, int K, float *out);
+int rd_gemm_q5k(rd_device *d, const void *W, int N, int K, const float *a, int M, float *dst);
+int rd_gemm_q6k(rd_device *d, const void *W, int N, int K, const float *a, int M, float *dst);
 /* int8 per-row weights x per-32 int8 activations (backend/cuda/actgroup.cu:421-437 gemv_w8a8_g32). */
 int rd_gemm_w8a8(rd_device *d, const int8_t *q, const float *row_scale, int N, int K, const float *a, int M, float *dst);
 /* int4 group-32 weights with f16 scales x per-32 int8 activations (backend/cuda/actgroup.cu:243-275). */
@@ -103,6 +111,11 @@ int rd_model_create(rd_device *d, const rd_model_desc *desc, rd_model **out);
 void rd_model_destroy(rd_model *m);
 /* raw 144-byte super-blocks, N rows of K/256 blocks (Model.OpenKQuant, decoder/kquant_native.go:198-273) */
 int rd_model_upload_q4k(rd_model *m, int layer, int proj, const void *blocks, int N, int K);
+/* raw Q5_K / Q6_K super-blocks of a tensor the file stores that way (decoder/kquant_native.go:49-80 noteKQuant records the
+ * source, :240-265 serves the rows; backend/cuda/resident_build.go:1030 binds the native lanes). Projections that are
+ * fused into one GEMM (q|k|v, gate|up) must share one kind; otherwise the upload is declined. */
+int rd_model_upload_q5k(rd_model *m, int layer, int proj, const void *blocks, int N, int K);
+int rd_model_upload_q6k(rd_model *m, int layer, int proj, const void *blocks, int N, int K);
 /* int8 rows + per-row f32 scale (WeightMat.Int8, decoder/weightmat.go:931) */
 int rd_model_upload_w8a8(rd_model *m, int layer, int proj, const int8_t *q, const float *row_scale, int N, int K);
 /* canonical int4 nibbles + binary16 group-32 scales (WeightMat.Int4F16, decoder/weightmat.go:904); expert < 0 = dense */

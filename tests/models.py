@@ -35,8 +35,10 @@ class LazyEmbedding:
 class Pair:
     """The same synthetic model as an oracle model and (when dev is given) a resident GPU model."""
 
-    def __init__(self, cfg, seed, dev=None, slots=8, ctx_cap=512, sigma=0.02):
+    def __init__(self, cfg, seed, dev=None, slots=8, ctx_cap=512, sigma=0.02, kinds=None):
+        """kinds: optional {projection: 'q5k' | 'q6k'} for dense projections stored as those super-blocks."""
         self.cfg = cfg
+        kinds = kinds or {}
         H, nH, nKV, hd = cfg["hidden"], cfg["n_heads"], cfg["n_kv"], cfg["head_dim"]
         qd, kvd, I, V = nH * hd, nKV * hd, cfg["inter"], cfg["vocab"]
         nE = cfg.get("n_experts", 0)
@@ -59,6 +61,12 @@ class Pair:
                 if self.gpu:
                     self.gpu.upload_w4a8(layer, proj, expert, nib, s16, K)
                 return ob.WMat(ob.OR_W4A8, N, K, nib, s16, act_group=32)
+            if proj in kinds:
+                fmt = kinds[proj]
+                blocks = synth.kquant_normal(fmt, nxt(), N, K, sigma)
+                if self.gpu:
+                    self.gpu.upload_kquant(fmt, layer, proj, blocks, N, K)
+                return ob.WMat(ob.OR_Q5K if fmt == "q5k" else ob.OR_Q6K, N, K, blocks, act_group=32)
             if K % 256 == 0 and proj != "head":
                 blocks = synth.q4k_normal(nxt(), N, K, sigma)
                 if self.gpu:

@@ -1,0 +1,102 @@
+"""GPU parity of the Q5_K and Q6_K lanes against the CPU oracle, through the C ABI.
+
+Bars as for Q4_K: dequantization bit-exact; GEMMs within rel 2e-3 of the f64 sum over the dequantized weights and the
+quantized activations; a row computed in a batch bit-identical to the row alone; a model whose projections mix Q4_K with
+Q5_K / Q6_K tensors within the decode bar against the oracle.
+"""
+import numpy as np
+import pytest
+
+from goinfer_amd import capi, synth
+from oracle import binding as ob
+
+from tests.models import Pair, dense_cfg
+from tests.test_gpu_model import check
+
+pytestmark = pytest.mark.gpu
+
+FMT = {"q5k": (176, ob.OR_Q5K, ob.dequant_q5k), "q6k": (210, ob.OR_Q6K, ob.dequant_q6k)}
+
+
+@pytest.fixture(scope="module")
+def dev():
+    d = capi.Device(0)
+    yield d
+    d.close()
+
+
+def rel_err(got, want):
+    want = want.astype(np.float64)
+    return float(np.abs(got.astype(np.float64) - want).max() / (np.sqrt((want * want).mean()) + 1e-30))
+
+
+def random_blocks(fmt, rng, n):
+    """Random bytes with finite f16 super-scales, some blocks with saturated sub-block scales."""
+    bb = FMT[fmt][0]
+    raw = rng.integers(0, 256, n * bb, dtype=np.uint8).reshape(n, bb)
+    for off in ((0, 2) if fmt == "q5k" else (208,)):
+        h = (rng.integers(5, 12, n).astype(np.uint16) << 10) | rng.integers(0, 1024, n).astype(np.uint16)
+        h |= (rng.integers(0, 2, n).astype(np.uint16) << 15) if fmt == "q6k" else 0
+        raw[:, off] = h & 0xFF
+        raw[:, off + 1] = h >> 8
+    if fmt == "q5k":
+        raw[::5, 4:16] = 0xFF
+    else:
+        raw[::5, 192:208] = 0x80  # scale -128
+        raw[1::5, 192:208] = 0x7F
+    return raw
+
+
+@pytest.mark.parametrize("fmt", ["q5k", "q6k"])
+@pytest.mark.parametrize("N,K", [(32, 256), (96, 768), (200, 3072)])
+def test_dequant_bit_exact(dev, fmt, N, K):
+    raw = random_blocks(fmt, np.random.default_rng(N * K), N * (K // 256))
+    want = FMT[fmt][2](raw).reshape(N, K)
+    got = dev.dequant_kquant(fmt, raw, N, K)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("fmt", ["q5k", "q6k"])
+@pytest.mark.parametrize("M", [1, 5, 32, 33])
+@pytest.mark.parametrize("N,K", [(128, 256), (160, 1024), (512, 4096)])
+def test_gemm(dev, fmt, M, N, K):
+    blocks = synth.kquant_normal(fmt, 11 + N, N, K)
+    a = synth.normal(100 + M, M * K).reshape(M, K)
+    w = ob.WMat(FMT[fmt][1], N, K, blocks, act_group=32)
+    want = ob.matmul(w, a)
+    ref64 = ob.matmul_f64ref(w, a)
+    got = dev.gemm_kquant(fmt, blocks, N, K, a)
+    assert rel_err(want, ref64) < 1e-5
+    assert rel_err(got, ref64) < 2e-3
+    solo = dev.gemm_kquant(fmt, blocks, N, K, a[:1])
+    assert np.array_equal(solo[0].view(np.uint32), got[0].view(np.uint32))
+
+
+@pytest.mark.parametrize("fmt", ["q5k", "q6k"])
+def test_gemm_random_blocks(dev, fmt):
+    """Every code, sign and scale value: random blocks rather than quantized normals."""
+    N, K, M = 64, 512, 8
+    raw = random_blocks(fmt, np.random.default_rng(5), N * (K // 256))
+    a = synth.normal(77, M * K).reshape(M, K)
+    w = ob.WMat(FMT[fmt][1], N, K, raw, act_group=32)
+    ref64 = ob.matmul_f64ref(w, a)
+    got = dev.gemm_kquant(fmt, raw, N, K, a)
+    assert rel_err(got, ref64) < 2e-3
+
+
+@pytest.mark.parametrize("kinds", [
+    dict(o="q6k", down="q6k", head="q6k"),
+    dict(q="q5k", k="q5k", v="q5k", gate="q5k", up="q5k", down="q5k"),
+    dict(q="q6k", k="q6k", v="q6k", gate="q6k", up="q6k", o="q5k", head="q5k"),
+], ids=["q6k-o-down-head", "q5k-fused", "q6k-fused-q5k-head"])
+def test_model_mixed_kinds(dev, kinds):
+    """Ragged batched decode, teacher-forced, against the oracle on the same blocks; batched rows == solo rows."""
+    rng = np.random.default_rng(9)
+    cfg = dense_cfg(n_layers=2, hidden=256, inter=512, vocab=512)
+    check(Pair(cfg, seed=31, dev=dev, slots=8, kinds=kinds), [list(rng.integers(0, 512, n)) for n in (3, 40, 70)], steps=4)
+
+
+def test_mixed_kind_fusion_declined(dev):
+    cfg = dense_cfg(n_layers=1, hidden=256, inter=512, vocab=512)
+    with pytest.raises(capi.RocmError, match="differ in kind"):
+        Pair(cfg, 32, dev, slots=2, ctx_cap=32, kinds=dict(v="q6k"))
