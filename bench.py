@@ -8,7 +8,7 @@ Prints ONE JSON line with the whole-job tok/s, the roofline of the dominant kern
 restatement of goinfer's CPU path, timed on this box's host cores on a bounded sample of the same workload).
 
 --workload c2 | c3 | c5 runs the other measurement configurations BASELINE.json names instead (the Q4_K GEMM microbench, the
-ragged attention microbench, the Qwen3-MoE-shaped step) and prints one line of the same form for that workload.
+ragged attention microbench, the Qwen3-MoE-shaped step; kquant: the Q5_K / Q6_K GEMMs beside Q4_K) and prints one line of the same form for that workload.
 """
 import argparse
 import json
@@ -90,9 +90,9 @@ def parse_args():
     ap.add_argument("--batch", type=int, default=32)
     ap.add_argument("--seed", type=int, default=1234)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--workload", default="c4", choices=["c4", "c2", "c3", "c5"],
+    ap.add_argument("--workload", default="c4", choices=["c4", "c2", "c3", "c5", "kquant"],
                     help="c4 (default): the Llama-3-8B-shape step the metric is quoted on; c2: Q4_K GEMM microbench; c3: ragged "
-                         "attention microbench; c5: Qwen3-MoE-shape step")
+                         "attention microbench; c5: Qwen3-MoE-shape step; kquant: Q4_K / Q5_K / Q6_K GEMMs at the FFN and head shapes")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this backend is single-GPU (goinfer has no collective path); run with --gpus 1", file=sys.stderr)
@@ -199,4 +199,4 @@ if __name__ == "__main__":
     else:
         import bench_micro
         bench_micro.T0 = T0
-        {"c2": bench_micro.run_c2, "c3": bench_micro.run_c3, "c5": bench_micro.run_c5}[_args.workload](_args)
+        {"c2": bench_micro.run_c2, "c3": bench_micro.run_c3, "c5": bench_micro.run_c5, "kquant": bench_micro.run_kquant}[_args.workload](_args)

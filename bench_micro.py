@@ -1,4 +1,4 @@
-"""The other measurement configurations of the decode path (bench.py --workload c2|c3|c5): one JSON line each, same form as
+"""The other measurement configurations of the decode path (bench.py --workload c2|c3|c5|kquant): one JSON line each, same form as
 the default workload's. Inputs are synthetic and resident in HBM before the timed region; times are HIP events on the launch
 stream; bytes are the algorithmic bytes of the call (every weight byte once, every KV byte once per sequence)."""
 import json
@@ -78,6 +78,50 @@ def run_c2(args):
             n += 1
         cpu = {"value": round(head["bytes"] / (t / n) / 1e9, 2), "unit": "GB/s", "cores": threads(), "kind": "port",
                "sample": "oracle gate and up matmuls + SwiGLU at M=32, %d calls (%.1f s)" % (n, t)}
+    out["cpu_baseline"] = cpu
+    dev.close()
+    emit(out)
+
+
+def run_kquant(args):
+    """The Q5_K and Q6_K lanes beside Q4_K: dequant-GEMMs at the FFN shapes and at the 128256 x 4096 head (the tensor GGUF
+    Q4_K_M files most often store as Q6_K), M = 1 and 32. Bytes are the file's own super-blocks + activations in + result out."""
+    from goinfer_amd import capi
+    steps, warmup = (args.steps if args.steps != 128 else 60), (args.warmup if args.warmup != 8 else 10)
+    dev = capi.Device(0)
+    cases = []
+    for kern, bb in (("gemm_q4k", 144), ("gemm_q5k", 176), ("gemm_q6k", 210)):
+        for N, K in ((14336, 4096), (4096, 14336), (128256, 4096)):
+            for M in (1, 32):
+                ms = dev.bench_kernel(kern, [N, K, M, 4 if N > 100000 else 8], warmup, steps)
+                t = float(np.median(ms))
+                nbytes = N * (K // 256) * bb + 4 * M * K + 4 * M * N
+                cases.append({"kernel": "rd_k_" + kern, "N": N, "K": K, "M": M, "us": round(t * 1e3, 2), "GBs": round(nbytes / t / 1e6, 1), "bytes": int(nbytes)})
+                log("%s %dx%d M=%d: %.1f us, %.0f GB/s" % (kern, N, K, M, t * 1e3, nbytes / t / 1e6))
+    head = next(c for c in cases if c["kernel"] == "rd_k_gemm_q6k" and c["N"] == 128256 and c["M"] == 32)
+    out = base_line("Q6_K dequant-GEMM achieved HBM GB/s (head 128256x4096 at M=32; all cases listed)", head["GBs"], "GB/s", steps, warmup,
+                    head["us"] / 1e3, "Q4_K / Q5_K / Q6_K GEMM at 14336x4096, 4096x14336, 128256x4096, M in {1,32}",
+                    "synthetic: random super-blocks with sane f16 scales, 4-8 weight copies used round-robin", {"cases": cases})
+    out["roofline"] = {"bound": "hbm", "achieved": head["GBs"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(head["GBs"] / HBM_PEAK_GBS, 4),
+                       "traffic": None, "kernel": "rd_k_gemm_q6k", "avg_launch_ms": round(head["us"] / 1e3, 5),
+                       "algorithmic_bytes_per_launch": head["bytes"]}
+    cpu = None
+    if not args.no_cpu:
+        from goinfer_amd import synth
+        from oracle import binding as ob
+        ob.set_threads(threads())
+        N, K = 16384, 4096  # a bounded slice of the head's rows
+        w = ob.WMat(ob.OR_Q6K, N, K, synth.kquant_normal("q6k", 1, N, K), act_group=32)
+        a = synth.normal(3, 32 * K, 1.0).reshape(32, K)
+        ob.matmul(w, a)
+        n, t = 0, 0.0
+        while t < 10.0 and n < 400:
+            t0 = time.time()
+            ob.matmul(w, a)
+            t += time.time() - t0
+            n += 1
+        cpu = {"value": round((N * (K // 256) * 210 + 4 * 32 * (K + N)) / (t / n) / 1e9, 2), "unit": "GB/s", "cores": threads(), "kind": "port",
+               "sample": "oracle Q6_K matmul, %d x %d rows of the head at M=32, %d calls (%.1f s)" % (N, K, n, t)}
     out["cpu_baseline"] = cpu
     dev.close()
     emit(out)

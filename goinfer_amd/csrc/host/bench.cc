@@ -77,7 +77,7 @@ extern "C" const char *rd_bench_class_name(int c) {
 }
 
 // Kernel micro-benchmarks over resident synthetic operands.
-//   "gemm_q4k"  args {N, K, M, copies}: dst = a . W^T on `copies` distinct weight copies used round-robin (so the 256 MB
+//   "gemm_q4k", "gemm_q5k", "gemm_q6k"  args {N, K, M, copies}: dst = a . W^T on `copies` distinct weight copies used round-robin (so the 256 MB
 //               Infinity Cache cannot hold the weights between launches); operands are random bytes with sane f16 scales.
 //   "gateup"    args {I, K, M, copies}: the fused gate|up projection + SwiGLU + quantization kernel.
 //   "barrier"   args {blocks, words, rounds, shift}: the grid-wide barrier with a cross-block data hand-off per round.
@@ -87,8 +87,9 @@ extern "C" const char *rd_bench_class_name(int c) {
 extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *args, int n_args, int warmup, int iters, float *ms_out) {
     if (!d || !name || !args || iters <= 0 || !ms_out) return RD_ERR_ARG;
     std::string nm(name);
-    if (nm == "gemm_q4k" && n_args >= 4 && (args[0] % 32 || args[1] % 256 || args[0] <= 0 || args[1] <= 0 || args[2] < 1 || args[2] > 64)) {
-        rd_set_error("gemm_q4k bench: bad shape");
+    const bool isGemm = nm == "gemm_q4k" || nm == "gemm_q5k" || nm == "gemm_q6k";
+    if (isGemm && n_args >= 4 && (args[0] % 32 || args[1] % 256 || args[0] <= 0 || args[1] <= 0 || args[2] < 1 || args[2] > 64)) {
+        rd_set_error("%s bench: bad shape", name);
         return RD_ERR_ARG;
     }
     if (nm == "gateup" && n_args >= 4 && (args[0] <= 0 || args[0] % 64 || args[1] <= 0 || args[1] % 256 || args[2] < 1 || args[2] > 64)) {
@@ -106,24 +107,31 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
     std::vector<hipEvent_t> ev((size_t)iters * 2);
     for (auto &e : ev) HIPCHK(EventCreate(&e));
     int rc = RD_OK;
-    if (nm == "gemm_q4k" && n_args >= 4) {
+    if (isGemm && n_args >= 4) {
         int N = (int)args[0], K = (int)args[1], M = (int)args[2], copies = (int)std::max<int64_t>(1, args[3]);
-        size_t bytes = (size_t)N * (K / 256) * 144;
+        const int kind = nm == "gemm_q4k" ? 0 : (nm == "gemm_q5k" ? 3 : 4), bb = kind == 0 ? 144 : (kind == 3 ? 176 : 210);
+        size_t bytes = (size_t)N * (K / 256) * bb;
         std::vector<uint8_t> raw(bytes);
         uint64_t s = 88172645463325252ULL;
         for (size_t i = 0; i < bytes; i++) {
             s ^= s << 13, s ^= s >> 7, s ^= s << 17;
             raw[i] = (uint8_t)s;
         }
-        for (size_t b = 0; b < bytes / 144; b++) raw[b * 144 + 1] = 0x10 | (raw[b * 144 + 1] & 3), raw[b * 144 + 3] = 0x10 | (raw[b * 144 + 3] & 3);
+        for (size_t b = 0; b < bytes / bb; b++) { // small finite f16 super-scales
+            uint8_t *blk = raw.data() + b * bb;
+            if (kind == 4)
+                blk[209] = 0x10 | (blk[209] & 3);
+            else
+                blk[1] = 0x10 | (blk[1] & 3), blk[3] = 0x10 | (blk[3] & 3);
+        }
         std::vector<DevWeight> ws((size_t)copies);
         for (auto &w : ws)
-            if (!rc) rc = upload_q4k(d, raw.data(), N, K, &w);
+            if (!rc) rc = kind == 0 ? upload_q4k(d, raw.data(), N, K, &w) : (kind == 3 ? upload_q5k(d, raw.data(), N, K, &w) : upload_q6k(d, raw.data(), N, K, &w));
         DevBuf Xp(d), P(d);
-        size_t pb = (size_t)(K / 256) * Q4K_PANEL_BYTES;
+        size_t pb = kind == 4 ? (size_t)(K / 128) * LIN_PANEL_BYTES : (size_t)(K / 256) * Q4K_PANEL_BYTES;
         if (!rc) rc = Xp.alloc(pb);
-        int nKB = K / 256;
-        GemmPlan plan = plan_gemm(0, N, nKB);
+        int nKB = K / kblock_of(kind);
+        GemmPlan plan = plan_gemm(kind, N, nKB);
         if (!rc) rc = P.alloc(sizeof(float) * (size_t)plan.splits * 32 * N);
         if (!rc) {
             std::vector<uint16_t> x(pb / 2);

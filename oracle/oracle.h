@@ -13,6 +13,7 @@
  * Pin status (checked by tests/test_oracle_fingerprints.py and tests/test_oracle_golden.py):
  *   or_f32_to_f16 / or_f16_to_f32        pinned: linalg.F32ToF16, linalg.F16ToF32 fingerprints
  *   or_dequant_q4k                       pinned: embed.GGUFFile(Q4_K).Tensor fingerprint
+ *   or_dequant_q5k / or_dequant_q6k      pinned: embed.GGUFFile(Q5_K).Tensor, embed.GGUFFile(Q6_K).Tensor fingerprints
  *   or_quantize_row_int8                 pinned: linalg.QuantizeRowInt8 fingerprint
  *   or_quantize_act                      pinned: linalg.QuantizeActQ fingerprint (per-row and per-32)
  *   or_quantize_int4_row / _mat          pinned: linalg.QuantizeGroupInt4Row, linalg.QuantizeInt4
@@ -26,6 +27,11 @@
  *                                        amd64 and arm64 (kernel_fingerprints.json). Restated in the mathematically
  *                                        specified form (exact int32 dot per 32-group, f32 fold in ascending group
  *                                        order, backend/cuda/actgroup.cu:298-355) and checked against an f64 sum.
+ *   or_matmul (q5k / q6k kinds)          parity unpinned at bit level: the reference holds no digest or golden for its
+ *                                        native Q5_K / Q6_K lanes (they exist only as CUDA / Metal kernels). Restated in
+ *                                        the specified form (backend/cuda/actgroup.cu:77-205) and held to 1e-5 of the f64
+ *                                        sum over the fingerprint-pinned dequantizer and activation quantizer
+ *                                        (tests/test_oracle_matmul.py).
  */
 #ifndef GOINFER_ORACLE_H
 #define GOINFER_ORACLE_H
@@ -42,13 +48,13 @@ float or_f16_to_f32(uint16_t h);
 
 /* ---- Q4_K: decoder/gguf.go:1508-1537, backend/metal/kernels/gemm_kq_test.go:27-70 ---- */
 void or_q4k_scale_min(int j, const uint8_t *q12, int *sc, int *m);
-void or_dequant_q4k(const uint8_t *blocks, size_t n_blocks, float *out);
+void or_dequant_q4k(const uint8_t *blocks, size_t n_blocks, float *out); /* 144 B -> 256 f32 each */
 /* GGUF Q5_K (176-byte super-blocks: d, dmin f16; 12 bytes of 6-bit scales and mins as Q4_K; qh[32] fifth bits; qs[128] nibbles):
  * w = d*sc_j*q - dmin*m_j with q = nibble | fifth bit << 4. Pinned bit-exact by fingerprint embed.GGUFFile(Q5_K).Tensor. */
 void or_dequant_q5k(const uint8_t *blocks, size_t n_blocks, float *out);
 /* GGUF Q6_K (210-byte super-blocks: ql[128] low nibbles, qh[64] two high bits each, 16 int8 sub-block scales, d f16):
  * w = d*sc_s*(q-32), 16 sub-blocks of 16. Pinned bit-exact by fingerprint embed.GGUFFile(Q6_K).Tensor. */
-void or_dequant_q6k(const uint8_t *blocks, size_t n_blocks, float *out); /* 144 B -> 256 f32 each */
+void or_dequant_q6k(const uint8_t *blocks, size_t n_blocks, float *out);
 
 /* ---- activation quantizers: backend/cuda/kv8_store.cu:3-35, actgroup.cu:26-54 ---- */
 float or_quantize_row_int8(const float *row, int n, int8_t *q);
