@@ -312,25 +312,28 @@ int upload_w4a8(rd_device *d, const uint8_t *nib, const uint16_t *s16, int N, in
 }
 
 void free_weight(rd_device *d, DevWeight *w) {
+    for (auto &p : w->parts) free_weight(d, &p);
     d->release(w->tiled);
     d->release(w->scales);
     *w = DevWeight();
 }
 
-int launch_gemm(rd_device *d, const DevWeight &w, const void *Xp, float *P, int M, GemmPlan *plan_out) {
+int launch_gemm(rd_device *d, const DevWeight &w, const void *Xp, float *P, int M, GemmPlan *plan_out, int ldP, int splits) {
     if (M < 1 || M > 32) {
         rd_set_error("gemm: M=%d outside 1..32", M);
         return RD_ERR_ARG;
     }
     int nKB = kblocks_for(w);
     GemmPlan p = plan_gemm(w.kind, w.N, nKB);
+    if (splits > 0) p.kbPerSplit = (nKB + splits - 1) / splits, p.splits = splits;
     if (plan_out) *plan_out = p;
+    if (ldP <= 0) ldP = w.N;
     unsigned gx = (unsigned)((w.N + 127) / 128);
     if (w.kind == 0)
-        return d->launch(d->k.gemm_q4k, gx, p.splits, 1, GEMM_THREADS, (const void *)w.tiled, Xp, P, w.N, nKB, p.kbPerSplit, M);
+        return d->launch(d->k.gemm_q4k, gx, p.splits, 1, GEMM_THREADS, (const void *)w.tiled, Xp, P, w.N, nKB, p.kbPerSplit, M, ldP);
     if (w.kind == 3 || w.kind == 4)
-        return d->launch(w.kind == 3 ? d->k.gemm_q5k : d->k.gemm_q6k, gx, p.splits, 1, GEMM_THREADS, (const void *)w.tiled, Xp, P, w.N, nKB, p.kbPerSplit, M);
+        return d->launch(w.kind == 3 ? d->k.gemm_q5k : d->k.gemm_q6k, gx, p.splits, 1, GEMM_THREADS, (const void *)w.tiled, Xp, P, w.N, nKB, p.kbPerSplit, M, ldP);
     if (w.kind == 1)
-        return d->launch(d->k.gemm_w8a8, gx, p.splits, 1, GEMM_THREADS, (const void *)w.tiled, (const void *)w.scales, Xp, P, w.N, nKB, p.kbPerSplit, M);
-    return d->launch(d->k.gemm_w4a8, gx, p.splits, 1, GEMM_THREADS, (const void *)w.tiled, Xp, P, w.N, nKB, p.kbPerSplit, M);
+        return d->launch(d->k.gemm_w8a8, gx, p.splits, 1, GEMM_THREADS, (const void *)w.tiled, (const void *)w.scales, Xp, P, w.N, nKB, p.kbPerSplit, M, ldP);
+    return d->launch(d->k.gemm_w4a8, gx, p.splits, 1, GEMM_THREADS, (const void *)w.tiled, Xp, P, w.N, nKB, p.kbPerSplit, M, ldP);
 }

@@ -88,11 +88,14 @@ GemmPlan plan_gemm(int kind, int N, int nKB);
 
 // Weight matrix resident on the device in its GEMM tiling.
 struct DevWeight {
-    int kind = -1; // 0 q4k, 1 w8a8, 2 w4a8, 3 q5k, 4 q6k
+    int kind = -1; // 0 q4k, 1 w8a8, 2 w4a8, 3 q5k, 4 q6k, 5 a group of weights of different kinds stacked row-wise (parts)
     int N = 0, K = 0;
     void *tiled = nullptr;  // re-tiled codes
     void *scales = nullptr; // w8a8: f32[N]
+    std::vector<DevWeight> parts; // kind 5: the members, each of one kind, rows [col0[i], col0[i] + parts[i].N) of the group
+    std::vector<int> col0;
 };
+enum { WKIND_GROUP = 5 };
 
 int upload_q4k(rd_device *d, const void *blocks, int N, int K, DevWeight *w);
 int upload_q5k(rd_device *d, const void *blocks, int N, int K, DevWeight *w);
@@ -101,7 +104,9 @@ int upload_w8a8(rd_device *d, const int8_t *q, const float *row_scale, int N, in
 int upload_w4a8(rd_device *d, const uint8_t *nib, const uint16_t *s16, int N, int K, DevWeight *w);
 void free_weight(rd_device *d, DevWeight *w);
 // P[splits][32][N] = panels(Xp) . W^T ; returns the plan used
-int launch_gemm(rd_device *d, const DevWeight &w, const void *Xp, float *P, int M, GemmPlan *plan);
+// ldP: floats between rows of P (0 = w.N); splits > 0 forces the split count (trailing splits that get no K-block store zeros),
+// which lets weights of different kinds write side by side into one partial-sum buffer.
+int launch_gemm(rd_device *d, const DevWeight &w, const void *Xp, float *P, int M, GemmPlan *plan, int ldP = 0, int splits = 0);
 size_t panel_bytes_for(const DevWeight &w);
 int panel_kind_for(const DevWeight &w);
 // K-blocks of a weight: super-blocks of 256 for the kinds on Q4_K-style panels (q4k, q5k), 128 otherwise

@@ -63,7 +63,7 @@ extern "C" void rd_model_destroy(rd_model *m) {
     }
     free_weight(d, &m->head);
     for (void *p : {(void *)m->embed_q, (void *)m->embed_scale, (void *)m->inv_freq_dev, (void *)m->final_norm, (void *)m->tables, (void *)m->h, (void *)m->normed, (void *)m->P, (void *)m->qbuf,
-                    (void *)m->part, (void *)m->cand_v, (void *)m->cand_i, (void *)m->logits, (void *)m->emb_dev, m->XpA, m->XpB, (void *)m->ids, (void *)m->meta, (void *)m->router_logits, (void *)m->moe_wgt, (void *)m->moe_gu,
+                    (void *)m->part, (void *)m->cand_v, (void *)m->cand_i, (void *)m->logits, (void *)m->emb_dev, m->XpA, m->XpA2, m->XpB, (void *)m->ids, (void *)m->meta, (void *)m->router_logits, (void *)m->moe_wgt, (void *)m->moe_gu,
                     (void *)m->moe_dn, (void *)m->moe_out, (void *)m->moe_idx, (void *)m->moe_idx_all, (void *)m->moe_rank, m->XpE})
         d->release(p);
     if (m->host_stage) (void)d->hip->HostFree(m->host_stage);
@@ -113,20 +113,50 @@ static int upload_pending(rd_device *d, const PendingMat &p, DevWeight *w) {
     return upload_w4a8(d, p.data.data(), (const uint16_t *)p.scales.data(), p.N, p.K, w);
 }
 
-// Concatenate row-wise (all kinds are row-major with per-row side data) and upload as one weight.
+// Concatenate row-wise (all kinds are row-major with per-row side data) and upload as one weight. Members of different
+// kinds (a GGUF Q4_K_M file stores some attn_v as Q6_K, and goinfer's q4k mode turns those into int8 copies) become a group:
+// each run of one kind is its own weight, multiplied by its own kernel into the group's shared partial-sum buffer.
 static int fuse_and_upload(rd_device *d, PendingMat *parts, int n, DevWeight *w) {
-    PendingMat cat;
-    cat.kind = parts[0].kind, cat.K = parts[0].K, cat.N = 0;
-    for (int i = 0; i < n; i++) {
-        if (parts[i].kind != cat.kind || parts[i].K != cat.K) {
-            rd_set_error("rocm resident declines: fused projections differ in kind or K");
+    for (int i = 1; i < n; i++)
+        if (parts[i].K != parts[0].K) {
+            rd_set_error("rocm resident declines: fused projections differ in K");
             return RD_DECLINED;
         }
+    std::vector<PendingMat> runs;
+    for (int i = 0; i < n; i++) {
+        if (runs.empty() || runs.back().kind != parts[i].kind) {
+            runs.emplace_back();
+            runs.back().kind = parts[i].kind, runs.back().K = parts[i].K, runs.back().N = 0;
+        }
+        PendingMat &cat = runs.back();
         cat.N += parts[i].N;
         cat.data.insert(cat.data.end(), parts[i].data.begin(), parts[i].data.end());
         cat.scales.insert(cat.scales.end(), parts[i].scales.begin(), parts[i].scales.end());
     }
-    int rc = upload_pending(d, cat, w);
+    int rc = RD_OK;
+    if (runs.size() == 1) {
+        rc = upload_pending(d, runs[0], w);
+    } else {
+        std::vector<int> pk;
+        DevWeight g;
+        g.kind = WKIND_GROUP, g.K = parts[0].K, g.N = 0;
+        for (auto &r : runs) {
+            g.parts.emplace_back();
+            g.col0.push_back(g.N);
+            if ((rc = upload_pending(d, r, &g.parts.back()))) break;
+            g.N += r.N;
+            int k = panel_kind_for(g.parts.back());
+            if (std::find(pk.begin(), pk.end(), k) == pk.end()) pk.push_back(k);
+        }
+        if (!rc && pk.size() > 2) {
+            rd_set_error("rocm resident declines: fused projections need more than two activation layouts");
+            rc = RD_DECLINED;
+        }
+        if (rc)
+            free_weight(d, &g);
+        else
+            *w = std::move(g);
+    }
     if (!rc)
         for (int i = 0; i < n; i++) parts[i] = PendingMat(), parts[i].kind = -2; // consumed
     return rc;
@@ -297,6 +327,7 @@ extern "C" int rd_model_upload_embedding(rd_model *m, const int8_t *q, const flo
 
 static size_t gemm_partial_floats(const DevWeight &w) {
     if (w.kind < 0) return 0;
+    if (w.kind == WKIND_GROUP) return (size_t)plan_gemm(0, w.N, w.K / 256 > 0 ? w.K / 256 : 1).splits * 32 * w.N;
     int nKB = kblocks_for(w);
     return (size_t)plan_gemm(w.kind, w.N, nKB).splits * 32 * w.N;
 }
@@ -338,6 +369,7 @@ extern "C" int rd_model_finalize(rd_model *m) {
     // room for either panel kind: 8 KB per 128 elements (int8/int4 consumers) or 17 KB per 256 (Q4_K consumers)
     auto panel_room = [](size_t K) { return std::max(((K + 127) / 128) * (size_t)LIN_PANEL_BYTES, ((K + 255) / 256) * (size_t)Q4K_PANEL_BYTES); };
     RC(d->alloc(&m->XpA, panel_room(kA)));
+    RC(d->alloc(&m->XpA2, panel_room(kA)));
     RC(d->alloc(&m->XpB, panel_room(kB)));
     RC(d->alloc((void **)&m->ids, sizeof(int) * 32));
     RC(alloc_f32(d, &m->cand_v, (size_t)32 * ((c.vocab + 4095) / 4096)));
@@ -472,11 +504,43 @@ static int build_attn_items(rd_model *m, int B, const int *pos, std::vector<Attn
     return RD_OK;
 }
 
+// The panel layouts a weight's GEMMs read: one, or two for a group whose members differ.
+static void panel_kinds_of(const DevWeight &w, int *kA, int *kB) {
+    *kB = -1;
+    if (w.kind != WKIND_GROUP) {
+        *kA = panel_kind_for(w);
+        return;
+    }
+    *kA = panel_kind_for(w.parts[0]);
+    for (const auto &p : w.parts)
+        if (panel_kind_for(p) != *kA) *kB = panel_kind_for(p);
+}
+
 static int add_norm_quant(rd_model *m, int B, const float *P, int splits, const float *w, const DevWeight &next, void *Xp, float *norm_out) {
     rd_device *d = m->d;
     Scope s(m, KC_ADD_NORM);
-    return d->launch(d->k.add_rmsnorm_quant, (unsigned)B, 1, 1, 1024, m->h, P, splits, w, m->desc.rms_eps, m->desc.hidden, Xp, panel_kind_for(next),
-                     norm_out);
+    int kA, kB;
+    panel_kinds_of(next, &kA, &kB);
+    return d->launch(d->k.add_rmsnorm_quant, (unsigned)B, 1, 1, 1024, m->h, P, splits, w, m->desc.rms_eps, m->desc.hidden, Xp, kA, norm_out,
+                     kB >= 0 ? m->XpA2 : (void *)nullptr, kB);
+}
+
+// One GEMM, or for a group one GEMM per member into column ranges of the same P[split][32][N], all with the group's split
+// count so that the consumer sums the same number of partials for every column.
+static int launch_proj(rd_model *m, const DevWeight &w, const void *Xp, int B, GemmPlan *plan) {
+    rd_device *d = m->d;
+    if (w.kind != WKIND_GROUP) return launch_gemm(d, w, Xp, m->P, B, plan);
+    int kA, kB;
+    panel_kinds_of(w, &kA, &kB);
+    GemmPlan g = plan_gemm(0, w.N, w.K / 256 > 0 ? w.K / 256 : 1);
+    for (const auto &p : w.parts) g.splits = std::min(g.splits, std::max(1, kblocks_for(p))); // no member gets more splits than K-blocks
+    for (size_t i = 0; i < w.parts.size(); i++) {
+        const DevWeight &p = w.parts[i];
+        RC(launch_gemm(d, p, panel_kind_for(p) == kA ? Xp : m->XpA2, m->P + w.col0[i], B, nullptr, w.N, g.splits));
+    }
+    g.kbPerSplit = 0;
+    if (plan) *plan = g;
+    return RD_OK;
 }
 
 static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
@@ -601,7 +665,7 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
         RC(add_norm_quant(m, B, resP, resSplits, l.attn_norm, l.qkv, m->XpA, nullptr));
         {
             Scope s(m, KC_GEMM_QKV);
-            RC(launch_gemm(d, l.qkv, m->XpA, m->P, B, &plan));
+            RC(launch_proj(m, l.qkv, m->XpA, B, &plan));
         }
         {
             Scope s(m, KC_ROPE_STORE);
@@ -633,7 +697,7 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
             } else {
                 {
                     Scope s(m, KC_GEMM_GATEUP);
-                    RC(launch_gemm(d, l.gateup, m->XpA, m->P, B, &plan));
+                    RC(launch_proj(m, l.gateup, m->XpA, B, &plan));
                 }
                 Scope s(m, KC_SWIGLU);
                 RC(d->launch(d->k.swiglu_quant, (unsigned)((c.inter + 1023) / 1024), (unsigned)B, 1, 256, (const float *)m->P, plan.splits, c.inter,
@@ -648,7 +712,7 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
             {
                 Scope s(m, KC_ADD_NORM);
                 RC(d->launch(d->k.add_rmsnorm_quant, (unsigned)B, 1, 1, 1024, m->h, (const float *)m->P, plan.splits, (const float *)l.ffn_norm,
-                             c.rms_eps, H, m->XpA, (int)PANEL_LIN4, m->normed));
+                             c.rms_eps, H, m->XpA, (int)PANEL_LIN4, m->normed, (void *)nullptr, -1));
             }
             RC(moe_ffn(m, B, li, l));
             resP = m->moe_out, resSplits = 1;

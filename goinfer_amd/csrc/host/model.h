@@ -55,6 +55,7 @@ struct rd_model {
     // step scratch (device)
     float *h = nullptr, *normed = nullptr, *P = nullptr, *qbuf = nullptr, *part = nullptr, *logits = nullptr, *emb_dev = nullptr;
     void *XpA = nullptr, *XpB = nullptr;
+    void *XpA2 = nullptr; // the normed row in a second panel layout, for a q|k|v or gate|up group whose members differ in kind
     size_t P_floats = 0;
     float *cand_v = nullptr;
     int *cand_i = nullptr;

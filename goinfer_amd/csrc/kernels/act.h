@@ -79,10 +79,12 @@ extern "C" __global__ void rd_k_reduce_splits(const float *__restrict__ P, float
 //   h[m] (+)= sum_s P[s][m][:]   (residual add of a split-K GEMM result, when P != nullptr; ascending split order)
 //   normed = (h*inv)*w with inv = f32(1/sqrt(ss/H+eps)), ss summed in f64   (decoder/rmsnorm.go:29-92)
 //   panels <- per-32 quantization of normed                                  (weightmat.go:33-38)
-// Optionally writes normed f32 to norm_out (the MoE router reads the un-quantized row). H % 128 == 0, H <= 8192.
+// Optionally writes normed f32 to norm_out (the MoE router reads the un-quantized row) and the same quantized values in a
+// second panel layout (Xp2, kind2) when the consuming projections differ in kind. H % 128 == 0, H <= 8192.
 extern "C" __global__ __launch_bounds__(1024) void rd_k_add_rmsnorm_quant(float *__restrict__ h, const float *__restrict__ P, int splits,
                                                                           const float *__restrict__ w, float eps, int H,
-                                                                          uint8_t *__restrict__ Xp, int kind, float *__restrict__ norm_out) {
+                                                                          uint8_t *__restrict__ Xp, int kind, float *__restrict__ norm_out,
+                                                                          uint8_t *__restrict__ Xp2, int kind2) {
     __shared__ double red[16];
     const int m = blockIdx.x, t = threadIdx.x, nv = H >> 2;
     float4_t v[2];
@@ -149,6 +151,7 @@ extern "C" __global__ __launch_bounds__(1024) void rd_k_add_rmsnorm_quant(float 
         float x0, x1, x2, x3, gs;
         quant_g32x4(n0, n1, n2, n3, &x0, &x1, &x2, &x3, &gs);
         panel_store4(Xp, kind, m, k0, x0, x1, x2, x3, gs);
+        if (Xp2) panel_store4(Xp2, kind2, m, k0, x0, x1, x2, x3, gs); // a second consumer that reads another panel layout
     }
 }
 

@@ -128,10 +128,12 @@ __device__ __forceinline__ void gemm_fold_groups(float16_t &acc, float *xch) {
     }
 }
 
-// gemm_body on the producer/consumer loop: grid (ceil(N/(32*TPB)), splits), block (TPB+1)*KG*64 threads.
+// gemm_body on the producer/consumer loop: grid (ceil(N/(32*TPB)), splits), block (TPB+1)*KG*64 threads. P rows are ldP floats
+// apart (ldP > N when several weights of different kinds write side by side into one partial-sum buffer); a split past the
+// end of K stores zeros, so that every weight of such a group can be launched with the group's split count.
 template <class T, int TPB, int KG, int PF>
 __device__ __forceinline__ void gemm_body(const uint8_t *__restrict__ Wt, const void *__restrict__ aux, const uint8_t *__restrict__ Xp,
-                                             float *__restrict__ P, int N, int nKB, int kbPerSplit, int M, uint4_t *lds) {
+                                             float *__restrict__ P, int N, int nKB, int kbPerSplit, int M, int ldP, uint4_t *lds) {
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int tile = blockIdx.x * TPB + wave % TPB, split = blockIdx.y;
     const int kb0 = split * kbPerSplit, kb1 = min(nKB, kb0 + kbPerSplit);
@@ -140,13 +142,13 @@ __device__ __forceinline__ void gemm_body(const uint8_t *__restrict__ Wt, const 
     const int ltile = active ? tile : (N >> 5) - 1;
     gemm_mainloop_pc<T, TPB, KG, PF>(acc, Wt + (size_t)ltile * nKB * T::TILE_BYTES, Xp, kb0, kb1, lds);
     gemm_fold_groups<TPB, KG>(acc, (float *)lds);
-    if (active && kb0 < kb1 && wave < TPB) {
+    if (active && wave < TPB) {
         T::finish(acc, aux, tile, lane);
-        float *out = P + (size_t)split * 32 * N + tile * 32 + (lane & 31);
+        float *out = P + (size_t)split * 32 * ldP + tile * 32 + (lane & 31);
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             int m = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-            if (m < M) out[(size_t)m * N] = acc[r];
+            if (m < M) out[(size_t)m * ldP] = acc[r];
         }
     }
 }

@@ -166,9 +166,9 @@ struct Q5KTraits {
 };
 
 extern "C" __global__ __launch_bounds__(320) void rd_k_gemm_q5k(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ Xp,
-                                                                 float *__restrict__ P, int N, int nSB, int sbPerSplit, int M) {
+                                                                 float *__restrict__ P, int N, int nSB, int sbPerSplit, int M, int ldP) {
     __shared__ uint4_t lds[2 * RD_Q4K_PANEL_BYTES / 16];
-    gemm_body<Q5KTraits, 4, 1, 3>(Wt, nullptr, Xp, P, N, nSB, sbPerSplit, M, lds);
+    gemm_body<Q5KTraits, 4, 1, 3>(Wt, nullptr, Xp, P, N, nSB, sbPerSplit, M, ldP, lds);
 }
 
 // ---------------- Q6_K ----------------
@@ -274,7 +274,7 @@ struct Q6KTraits {
 };
 
 extern "C" __global__ __launch_bounds__(320) void rd_k_gemm_q6k(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ Xp,
-                                                                 float *__restrict__ P, int N, int nKB, int kbPerSplit, int M) {
+                                                                 float *__restrict__ P, int N, int nKB, int kbPerSplit, int M, int ldP) {
     __shared__ uint4_t lds[2 * RD_LIN_PANEL_BYTES / 16];
-    gemm_body<Q6KTraits, 4, 1, 3>(Wt, nullptr, Xp, P, N, nKB, kbPerSplit, M, lds);
+    gemm_body<Q6KTraits, 4, 1, 3>(Wt, nullptr, Xp, P, N, nKB, kbPerSplit, M, ldP, lds);
 }

@@ -60,9 +60,9 @@ struct W8Traits {
 
 extern "C" __global__ __launch_bounds__(320) void rd_k_gemm_w8a8(const uint8_t *__restrict__ Wt, const float *__restrict__ wscale,
                                                                   const uint8_t *__restrict__ Xp, float *__restrict__ P, int N, int nKB,
-                                                                  int kbPerSplit, int M) {
+                                                                  int kbPerSplit, int M, int ldP) {
     __shared__ uint4_t lds[2 * RD_LIN_PANEL_BYTES / 16];
-    gemm_body<W8Traits, 4, 1, 3>(Wt, wscale, Xp, P, N, nKB, kbPerSplit, M, lds);
+    gemm_body<W8Traits, 4, 1, 3>(Wt, wscale, Xp, P, N, nKB, kbPerSplit, M, ldP, lds);
 }
 
 // ---------------- W4A8: canonical int4 nibbles (value nib-8), binary16 scale per 32 (decoder/weightmat.go:160-178) ----------------
@@ -131,7 +131,7 @@ struct W4Traits {
 };
 
 extern "C" __global__ __launch_bounds__(320) void rd_k_gemm_w4a8(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ Xp,
-                                                                  float *__restrict__ P, int N, int nKB, int kbPerSplit, int M) {
+                                                                  float *__restrict__ P, int N, int nKB, int kbPerSplit, int M, int ldP) {
     __shared__ uint4_t lds[2 * RD_LIN_PANEL_BYTES / 16];
-    gemm_body<W4Traits, 4, 1, 3>(Wt, nullptr, Xp, P, N, nKB, kbPerSplit, M, lds);
+    gemm_body<W4Traits, 4, 1, 3>(Wt, nullptr, Xp, P, N, nKB, kbPerSplit, M, ldP, lds);
 }

@@ -146,9 +146,9 @@ struct Q4KTraits {
 
 // Grid (ceil(N/128), splits), block 320: four consumer waves (one 32-row tile each) and one panel producer.
 extern "C" __global__ __launch_bounds__(320) void rd_k_gemm_q4k(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ Xp,
-                                                                 float *__restrict__ P, int N, int nSB, int sbPerSplit, int M) {
+                                                                 float *__restrict__ P, int N, int nSB, int sbPerSplit, int M, int ldP) {
     __shared__ uint4_t lds[2 * RD_Q4K_PANEL_BYTES / 16];
-    gemm_body<Q4KTraits, 4, 1, 3>(Wt, nullptr, Xp, P, N, nSB, sbPerSplit, M, lds);
+    gemm_body<Q4KTraits, 4, 1, 3>(Wt, nullptr, Xp, P, N, nSB, sbPerSplit, M, ldP, lds);
 }
 
 // Fused gate/up projection + SwiGLU + per-32 quantization (goinfer decoder/cpu_gateup_fused.go:83-148, in one launch):

@@ -112,8 +112,9 @@ void rd_model_destroy(rd_model *m);
 /* raw 144-byte super-blocks, N rows of K/256 blocks (Model.OpenKQuant, decoder/kquant_native.go:198-273) */
 int rd_model_upload_q4k(rd_model *m, int layer, int proj, const void *blocks, int N, int K);
 /* raw Q5_K / Q6_K super-blocks of a tensor the file stores that way (decoder/kquant_native.go:49-80 noteKQuant records the
- * source, :240-265 serves the rows; backend/cuda/resident_build.go:1030 binds the native lanes). Projections that are
- * fused into one GEMM (q|k|v, gate|up) must share one kind; otherwise the upload is declined. */
+ * source, :240-265 serves the rows; backend/cuda/resident_build.go:1030 binds the native lanes). Projections that feed one
+ * consumer (q|k|v, gate|up) may differ in kind, as a Q4_K_M file's attn_v does: each run of one kind is multiplied by its
+ * own kernel into the shared partial sums. */
 int rd_model_upload_q5k(rd_model *m, int layer, int proj, const void *blocks, int N, int K);
 int rd_model_upload_q6k(rd_model *m, int layer, int proj, const void *blocks, int N, int K);
 /* int8 rows + per-row f32 scale (WeightMat.Int8, decoder/weightmat.go:931) */

@@ -36,7 +36,7 @@ class Pair:
     """The same synthetic model as an oracle model and (when dev is given) a resident GPU model."""
 
     def __init__(self, cfg, seed, dev=None, slots=8, ctx_cap=512, sigma=0.02, kinds=None):
-        """kinds: optional {projection: 'q5k' | 'q6k'} for dense projections stored as those super-blocks."""
+        """kinds: optional {projection: 'q5k' | 'q6k' | 'w8a8'} for dense projections stored as those super-blocks or int8 rows."""
         self.cfg = cfg
         kinds = kinds or {}
         H, nH, nKV, hd = cfg["hidden"], cfg["n_heads"], cfg["n_kv"], cfg["head_dim"]
@@ -61,6 +61,11 @@ class Pair:
                 if self.gpu:
                     self.gpu.upload_w4a8(layer, proj, expert, nib, s16, K)
                 return ob.WMat(ob.OR_W4A8, N, K, nib, s16, act_group=32)
+            if kinds.get(proj) == "w8a8":
+                q, sc = synth.w8a8_normal(nxt(), N, K, sigma)
+                if self.gpu:
+                    self.gpu.upload_w8a8(layer, proj, q, sc)
+                return ob.WMat(ob.OR_W8A8, N, K, q, sc, act_group=32)
             if proj in kinds:
                 fmt = kinds[proj]
                 blocks = synth.kquant_normal(fmt, nxt(), N, K, sigma)

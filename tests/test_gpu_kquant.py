@@ -2,7 +2,7 @@
 
 Bars as for Q4_K: dequantization bit-exact; GEMMs within rel 2e-3 of the f64 sum over the dequantized weights and the
 quantized activations; a row computed in a batch bit-identical to the row alone; a model whose projections mix Q4_K with
-Q5_K / Q6_K tensors within the decode bar against the oracle.
+Q5_K / Q6_K tensors — also inside one fused q|k|v or gate|up group — within the decode bar against the oracle.
 """
 import numpy as np
 import pytest
@@ -88,15 +88,12 @@ def test_gemm_random_blocks(dev, fmt):
     dict(o="q6k", down="q6k", head="q6k"),
     dict(q="q5k", k="q5k", v="q5k", gate="q5k", up="q5k", down="q5k"),
     dict(q="q6k", k="q6k", v="q6k", gate="q6k", up="q6k", o="q5k", head="q5k"),
-], ids=["q6k-o-down-head", "q5k-fused", "q6k-fused-q5k-head"])
+    dict(v="q6k", down="q6k", head="q6k"),      # the GGUF Q4_K_M pattern: q, k, gate, up Q4_K; v, down, head Q6_K
+    dict(v="w8a8", down="w8a8"),                # the same file as goinfer's q4k mode loads it: int8 copies of the Q6_K tensors
+    dict(q="q5k", k="q5k", v="q6k", up="q6k"),  # Q5_K_M-like, and a gate|up pair that differs
+], ids=["q6k-o-down-head", "q5k-fused", "q6k-fused-q5k-head", "q4km-mixed-qkv", "q4k-int8-mixed-qkv", "q5km-mixed-qkv-gateup"])
 def test_model_mixed_kinds(dev, kinds):
     """Ragged batched decode, teacher-forced, against the oracle on the same blocks; batched rows == solo rows."""
     rng = np.random.default_rng(9)
     cfg = dense_cfg(n_layers=2, hidden=256, inter=512, vocab=512)
     check(Pair(cfg, seed=31, dev=dev, slots=8, kinds=kinds), [list(rng.integers(0, 512, n)) for n in (3, 40, 70)], steps=4)
-
-
-def test_mixed_kind_fusion_declined(dev):
-    cfg = dense_cfg(n_layers=1, hidden=256, inter=512, vocab=512)
-    with pytest.raises(capi.RocmError, match="differ in kind"):
-        Pair(cfg, 32, dev, slots=2, ctx_cap=32, kinds=dict(v="q6k"))
