@@ -21,12 +21,34 @@ EXPORTS = [
     "rd_kv_configure", "rd_kv_upload", "rd_kv_truncate", "rd_kv_reset", "rd_step_batch", "rd_forward",
     "rd_last_moe_indices", "rd_model_upload_embedding", "rd_bench_steps", "rd_bench_profile", "rd_bench_class_count",
     "rd_bench_class_name", "rd_bench_kernel", "rd_gateup_q4k_quant", "rd_moe_replay", "rd_bench_attn", "rd_step_ragged", "rd_prefill_last",
+    "rd_step_batch_draw", "rd_sample_rows", "rd_greedy_chain_start", "rd_greedy_chain_next", "rd_sample_chain_start",
+    "rd_sample_chain_next", "rd_greedy_chain_stop",
     "rd_dequant_q5k", "rd_dequant_q6k", "rd_gemm_q5k", "rd_gemm_q6k", "rd_model_upload_q5k", "rd_model_upload_q6k",
 ]
 
 
 class RocmError(RuntimeError):
     pass
+
+
+class Draw(C.Structure):
+    _fields_ = [("temperature", C.c_double), ("seed", C.c_uint64), ("draw", C.c_uint64), ("mode", C.c_int32), ("reserved", C.c_int32)]
+
+
+DRAW_NONE, DRAW_GREEDY, DRAW_GUMBEL = 0, 1, 2
+
+
+def make_draws(draws):
+    """per row None, "greedy" or (temperature, seed, draw) -> a ctypes array of rd_draw"""
+    arr = (Draw * len(draws))()
+    for i, dw in enumerate(draws):
+        if dw is None:
+            arr[i].mode = DRAW_NONE
+        elif isinstance(dw, str):
+            arr[i].mode = DRAW_GREEDY
+        else:
+            arr[i].mode, arr[i].temperature, arr[i].seed, arr[i].draw = DRAW_GUMBEL, dw[0], dw[1], dw[2]
+    return arr
 
 
 class ModelDesc(C.Structure):
@@ -48,7 +70,7 @@ def lib():
         L = C.CDLL(LIB_PATH)
         L.rd_last_error.restype = C.c_char_p
         L.rd_backend_name.restype = C.c_char_p
-        for name in ("rd_device_close", "rd_model_destroy"):
+        for name in ("rd_device_close", "rd_model_destroy", "rd_greedy_chain_stop"):
             getattr(L, name).restype = None
         _lib = L
     return _lib
@@ -123,6 +145,15 @@ class Device:
         name = "rd_gemm_" + fmt
         check(getattr(lib(), name)(self.h, _p(blocks), N, K, _p(a), a.shape[0], _p(dst)), name)
         return dst
+
+    def sample_rows(self, logits, draws):
+        """draws: per row "greedy" or (temperature, seed, draw). Returns int32 ids."""
+        logits = _f32(logits)
+        rows, V = logits.shape
+        arr = make_draws(draws)
+        ids = np.empty(rows, np.int32)
+        check(lib().rd_sample_rows(self.h, _p(logits), rows, V, arr, _p(ids)), "rd_sample_rows")
+        return ids
 
     def gemm_q4k(self, blocks, N, K, a, blocks2=None):
         a = _f32(a)
@@ -271,6 +302,38 @@ class Model:
         ids = np.empty(B, np.int32) if want & WANT_ARGMAX else None
         check(lib().rd_step_batch(self.h, B, _p(slots), _p(pos), _p(emb), want, _p(logits), _p(ids)), "rd_step_batch")
         return logits, ids
+
+    def step_batch_draw(self, slots, pos, emb, draws, want=0):
+        """draws: per row None, "greedy" or (temperature, seed, draw). Returns (logits or None, ids with -1 for rows without a draw)."""
+        emb = _f32(emb)
+        B = emb.shape[0]
+        slots = np.ascontiguousarray(slots, dtype=np.int32)
+        pos = np.ascontiguousarray(pos, dtype=np.int32)
+        arr = make_draws(draws)
+        logits = np.empty((B, self.cfg["vocab"]), np.float32) if want & WANT_LOGITS else None
+        ids = np.empty(B, np.int32)
+        check(lib().rd_step_batch_draw(self.h, B, _p(slots), _p(pos), _p(emb), arr, want, _p(logits), _p(ids)), "rd_step_batch_draw")
+        return logits, ids
+
+    def greedy_chain_start(self, slot, tok, pos):
+        check(lib().rd_greedy_chain_start(self.h, slot, int(tok), pos), "rd_greedy_chain_start")
+
+    def greedy_chain_next(self):
+        out = C.c_int(-1)
+        check(lib().rd_greedy_chain_next(self.h, C.byref(out)), "rd_greedy_chain_next")
+        return out.value
+
+    def sample_chain_start(self, slot, tok, pos, temperature, seed, draw):
+        check(lib().rd_sample_chain_start(self.h, slot, int(tok), pos, C.c_double(temperature), C.c_uint64(seed), C.c_uint64(draw)),
+              "rd_sample_chain_start")
+
+    def sample_chain_next(self, seed, draw):
+        out = C.c_int(-1)
+        check(lib().rd_sample_chain_next(self.h, C.c_uint64(seed), C.c_uint64(draw), C.byref(out)), "rd_sample_chain_next")
+        return out.value
+
+    def chain_stop(self):
+        lib().rd_greedy_chain_stop(self.h)
 
     def step_ragged(self, slots, pos, embs, want=WANT_LOGITS):
         """embs: one [rows_i][hidden] array per sequence. Returns (logits [sum rows][vocab] or None, ids [sum rows] or None)."""

@@ -9,8 +9,8 @@
 
 #define RC(x)                \
     do {                     \
-        int rc_ = (x);       \
-        if (rc_) return rc_; \
+        int rd_rc_macro_ = (x); \
+        if (rd_rc_macro_) return rd_rc_macro_; \
     } while (0)
 
 // Greedy decode chain entirely on the device: ids0 are the first tokens; every step embeds the previous step's argmax

@@ -2,14 +2,15 @@
 // (backend/cuda/kvpool.go) and the ragged batched decode step (backend/cuda/batchstep.go:49-78 StepBatch).
 #include "model.h"
 #include <algorithm>
+#include <cmath>
 #include <math.h>
 #include <stdlib.h>
 #include <string.h>
 
 #define RC(x)                \
     do {                     \
-        int rc_ = (x);       \
-        if (rc_) return rc_; \
+        int rd_rc_macro_ = (x); \
+        if (rd_rc_macro_) return rd_rc_macro_; \
     } while (0)
 
 static int alloc_f32(rd_device *d, float **p, size_t n) { return d->alloc((void **)p, sizeof(float) * (n ? n : 1)); }
@@ -67,6 +68,9 @@ extern "C" void rd_model_destroy(rd_model *m) {
                     (void *)m->moe_dn, (void *)m->moe_out, (void *)m->moe_idx, (void *)m->moe_idx_all, (void *)m->moe_rank, m->XpE})
         d->release(p);
     if (m->host_stage) (void)d->hip->HostFree(m->host_stage);
+    if (m->chain.host_ids) (void)d->hip->HostFree(m->chain.host_ids);
+    for (hipEvent_t e : m->chain.ev)
+        if (e) (void)d->hip->EventDestroy(e);
     for (hipEvent_t e : m->stage_ev)
         if (e) (void)d->hip->EventDestroy(e);
     for (hipEvent_t e : m->timer.ev) (void)d->hip->EventDestroy(e);
@@ -429,12 +433,13 @@ extern "C" int rd_kv_configure(rd_model *m, int slots, int ctx_cap) {
     int G = c.n_heads / c.n_kv_heads;
     RC(alloc_f32(d, &m->part, (size_t)m->max_items * G * (c.head_dim + 2)));
     // The step's metadata lives in one device block so a step uploads it with one copy:
-    // [row slot 32][row position 32][row length 32][item ranges 32*nKV*2][items max_items x 4] ints
+    // [row slot 32][row position 32][row length 32][row draw records 32 x 6][item ranges 32*nKV*2][items max_items x 4] ints
     const size_t rangeInts = (size_t)32 * c.n_kv_heads * 2;
-    m->meta_ints = 96 + rangeInts + (size_t)m->max_items * 4;
+    m->meta_ints = rd_model::META_HDR + rangeInts + (size_t)m->max_items * 4;
     RC(d->alloc((void **)&m->meta, sizeof(int) * m->meta_ints));
-    m->rowSlot = m->meta, m->rowPos = m->meta + 32, m->rowLen = m->meta + 64, m->itemStart = m->meta + 96;
-    m->items = (AttnItemH *)(m->meta + 96 + rangeInts);
+    m->rowSlot = m->meta, m->rowPos = m->meta + 32, m->rowLen = m->meta + 64, m->rowDraw = m->meta + 96;
+    m->itemStart = m->meta + rd_model::META_HDR;
+    m->items = (AttnItemH *)(m->meta + rd_model::META_HDR + rangeInts);
     return d->sync();
 }
 
@@ -596,6 +601,10 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
         rd_set_error("step before rd_model_finalize / rd_kv_configure");
         return RD_ERR_STATE;
     }
+    if (m->chain.open && !m->chain.in_call) {
+        rd_set_error("a chain is open: between its start and stop the resident takes no other step");
+        return RD_ERR_STATE;
+    }
     if (B < 1 || B > 32) {
         rd_set_error("rocm resident: batch %d outside the stepper range 1..32", B);
         return RD_ERR_ARG;
@@ -636,9 +645,30 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
         const size_t rangeInts = (size_t)32 * nKV * 2;
         float *eh = (float *)(st + (1u << 20));
         for (int b = 0; b < B; b++) hm[b] = slot[b], hm[32 + b] = pos[b], hm[64 + b] = pos[b] + 1;
-        memcpy(hm + 96, start.data(), sizeof(int) * start.size());
-        memcpy(hm + 96 + rangeInts, items.data(), sizeof(AttnItemH) * items.size());
-        RC(d->h2d(m->meta, hm, sizeof(int) * (96 + rangeInts + items.size() * 4)));
+        // Draw records (resident/forward.go:43-52 BatchDraw) with Sampler.gumbelDraw's guards applied here
+        // (internal/runtime/sampling/sampler_gumbel.go:80-88): a temperature <= 0 means 1, and one so small that 1/T
+        // overflows f32 is the plain argmax.
+        for (int b = 0; b < 32; b++) {
+            int *r = hm + 96 + b * 6;
+            memset(r, 0, sizeof(int) * 6);
+            if (b >= B || !m->step_draws) continue;
+            const rd_draw &dw = m->step_draws[b];
+            r[0] = dw.mode;
+            if (dw.mode == RD_DRAW_GUMBEL) {
+                float invT = (float)(1.0 / (dw.temperature <= 0 ? 1.0 : dw.temperature));
+                if (std::isinf(invT)) {
+                    r[0] = RD_DRAW_GREEDY;
+                    continue;
+                }
+                memcpy(&r[1], &invT, 4);
+                r[2] = (int)(uint32_t)dw.seed, r[3] = (int)(uint32_t)(dw.seed >> 32);
+                r[4] = (int)(uint32_t)dw.draw, r[5] = (int)(uint32_t)(dw.draw >> 32);
+            }
+        }
+        constexpr int HDR = rd_model::META_HDR;
+        memcpy(hm + HDR, start.data(), sizeof(int) * start.size());
+        memcpy(hm + HDR + rangeInts, items.data(), sizeof(AttnItemH) * items.size());
+        RC(d->h2d(m->meta, hm, sizeof(int) * (HDR + rangeInts + items.size() * 4)));
         if (emb_host) {
             memcpy(eh, emb_host, sizeof(float) * (size_t)B * H);
             RC(d->h2d(m->h, eh, sizeof(float) * (size_t)B * H));
@@ -728,7 +758,7 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
         Scope s(m, KC_ARGMAX);
         int nChunks = (c.vocab + 4095) / 4096;
         RC(d->launch(d->k.argmax_rows, (unsigned)nChunks, (unsigned)B, 1, 256, (const float *)m->P, plan.splits, c.vocab, m->cand_v, m->cand_i,
-                     (want & RD_WANT_LOGITS) ? m->logits : (float *)nullptr));
+                     (want & RD_WANT_LOGITS) ? m->logits : (float *)nullptr, (const int *)(m->step_draws ? m->rowDraw : nullptr)));
         if (want & RD_WANT_ARGMAX) RC(d->launch(d->k.argmax_final, (unsigned)B, 1, 1, 64, (const float *)m->cand_v, (const int *)m->cand_i, nChunks, m->ids));
     }
     for (int b = 0; b < B; b++) m->slot_len[(size_t)slot[b]] = std::max(m->slot_len[(size_t)slot[b]], pos[b] + 1);
@@ -748,6 +778,145 @@ extern "C" int rd_step_batch(rd_model *m, int B, const int *slot, const int *pos
         return RD_ERR_ARG;
     }
     return model_step(m, B, slot, pos, emb, nullptr, want, logits, ids, false);
+}
+
+// ---------------------------------------------------------------- device-chained decode
+// decoder/resident/subsystems.go:78-100: GreedyChainStart / GreedyChainNext / GreedyChainStop and their temperature-only
+// siblings SampleChainStart / SampleChainNext. Each forward takes its input row from the embedding table at the id the previous
+// forward picked, all on the device; the host reads four bytes per token and the next forward is already queued when it does.
+static int chain_queue(rd_model *m) {
+    rd_model::Chain &ch = m->chain;
+    rd_device *d = m->d;
+    rd_draw dw{};
+    dw.mode = ch.sample ? RD_DRAW_GUMBEL : RD_DRAW_GREEDY;
+    dw.temperature = ch.temperature, dw.seed = ch.seed, dw.draw = ch.draw_next;
+    m->step_draws = &dw;
+    ch.in_call = true;
+    int rc = model_step(m, 1, &ch.slot, &ch.next_pos, nullptr, nullptr, RD_WANT_ARGMAX, nullptr, nullptr, false);
+    ch.in_call = false;
+    m->step_draws = nullptr;
+    if (rc) return rc;
+    unsigned s = ch.tail % rd_model::Chain::DEPTH;
+    HIPCHK(MemcpyAsync(ch.host_ids + s, m->ids, sizeof(int), hipMemcpyDeviceToHost, d->stream));
+    HIPCHK(EventRecord(ch.ev[s], d->stream));
+    ch.tail++, ch.next_pos++, ch.draw_next++;
+    return RD_OK;
+}
+
+// Queue ahead; a look-ahead forward that cannot run (the context cap) is not an error until its token is asked for.
+static void chain_look_ahead(rd_model *m) {
+    rd_model::Chain &ch = m->chain;
+    while (!ch.exhausted && ch.tail - ch.head < (unsigned)rd_model::Chain::DEPTH) {
+        int rc = chain_queue(m);
+        if (rc) ch.exhausted = true, ch.exhausted_rc = rc;
+    }
+}
+
+static int chain_start(rd_model *m, int slot, int id, int pos, bool sample, double temperature, uint64_t seed, uint64_t draw) {
+    if (!m) return RD_ERR_ARG;
+    rd_model::Chain &ch = m->chain;
+    if (ch.open) {
+        rd_set_error("a chain is already open");
+        return RD_ERR_STATE;
+    }
+    if (!m->finalized || !m->tables || !m->embed_q) {
+        rd_set_error("a chain needs rd_model_finalize, rd_kv_configure and rd_model_upload_embedding");
+        return RD_ERR_STATE;
+    }
+    if (id < 0 || id >= m->desc.vocab || !slot_ok(m, slot)) {
+        rd_set_error("chain start: token %d or slot %d out of range", id, slot);
+        return RD_ERR_ARG;
+    }
+    rd_device *d = m->d;
+    if (!ch.host_ids) {
+        HIPCHK(HostMalloc((void **)&ch.host_ids, sizeof(int) * rd_model::Chain::DEPTH, 0));
+        for (auto &e : ch.ev) HIPCHK(EventCreate(&e));
+    }
+    RC(d->h2d(m->ids, &id, sizeof(int)));
+    ch.slot = slot, ch.next_pos = pos, ch.sample = sample, ch.temperature = temperature, ch.seed = seed;
+    ch.draw_next = ch.draw_head = draw, ch.head = ch.tail = 0, ch.exhausted = false, ch.exhausted_rc = 0;
+    int rc = chain_queue(m); // the first forward's own failure (bad position, context cap) is the caller's
+    if (rc) return rc;
+    ch.open = true;
+    chain_look_ahead(m);
+    return RD_OK;
+}
+
+static int chain_next(rd_model *m, int *id) {
+    if (!m || !id) return RD_ERR_ARG;
+    rd_model::Chain &ch = m->chain;
+    if (!ch.open) {
+        rd_set_error("no chain is open");
+        return RD_ERR_STATE;
+    }
+    if (ch.head == ch.tail) { // nothing queued: the look-ahead had failed
+        rd_set_error("chain: the forward at position %d could not be queued (%d)", ch.next_pos, ch.exhausted_rc);
+        return ch.exhausted_rc ? ch.exhausted_rc : RD_ERR_STATE;
+    }
+    unsigned s = ch.head % rd_model::Chain::DEPTH;
+    rd_device *d = m->d;
+    HIPCHK(EventSynchronize(ch.ev[s]));
+    *id = ch.host_ids[s];
+    ch.head++, ch.draw_head++;
+    chain_look_ahead(m);
+    return RD_OK;
+}
+
+extern "C" int rd_greedy_chain_start(rd_model *m, int slot, int id, int pos) { return chain_start(m, slot, id, pos, false, 1.0, 0, 0); }
+extern "C" int rd_greedy_chain_next(rd_model *m, int *id) {
+    if (m && m->chain.open && m->chain.sample) {
+        rd_set_error("the open chain is a sample chain");
+        return RD_ERR_STATE;
+    }
+    return chain_next(m, id);
+}
+extern "C" int rd_sample_chain_start(rd_model *m, int slot, int id, int pos, double temperature, uint64_t seed, uint64_t draw) {
+    if (std::isnan(temperature)) return RD_ERR_ARG;
+    return chain_start(m, slot, id, pos, true, temperature, seed, draw);
+}
+extern "C" int rd_sample_chain_next(rd_model *m, uint64_t seed, uint64_t draw, int *id) {
+    if (!m) return RD_ERR_ARG;
+    rd_model::Chain &ch = m->chain;
+    if (!ch.open || !ch.sample) {
+        rd_set_error("no sample chain is open");
+        return RD_ERR_STATE;
+    }
+    if (seed != ch.seed || draw != ch.draw_head) { // the caller's sampler and the chain must agree on the draw of this forward
+        rd_set_error("sample chain: the forward was drawn with (seed %llu, draw %llu), not (%llu, %llu)", (unsigned long long)ch.seed,
+                     (unsigned long long)ch.draw_head, (unsigned long long)seed, (unsigned long long)draw);
+        return RD_ERR_ARG;
+    }
+    return chain_next(m, id);
+}
+// Waits out any forward queued past the last token taken. Those forwards have written their K/V rows (the rows of tokens the
+// chain itself picked); positions at or past the one the caller continues from are simply written again.
+extern "C" void rd_greedy_chain_stop(rd_model *m) {
+    if (!m || !m->chain.open) return;
+    (void)m->d->sync();
+    m->chain.open = false;
+}
+
+// StepBatch with per-row draws (resident/forward.go:37-58): a row with a draw returns the id drawn on the device — the argmax
+// for a greedy draw, the Gumbel-max token for a temperature draw — and a row without one returns -1 in ids.
+extern "C" int rd_step_batch_draw(rd_model *m, int B, const int *slot, const int *pos, const float *emb, const rd_draw *draws, int want,
+                                  float *logits, int *ids) {
+    if (!m || !slot || !pos || !emb || !draws || !ids) return RD_ERR_ARG;
+    if ((want & RD_WANT_LOGITS) && !logits) {
+        rd_set_error("rd_step_batch_draw: want=%d needs its output buffer", want);
+        return RD_ERR_ARG;
+    }
+    for (int b = 0; b < B && b < 32; b++)
+        if (draws[b].mode < RD_DRAW_NONE || draws[b].mode > RD_DRAW_GUMBEL || (draws[b].mode == RD_DRAW_GUMBEL && std::isnan(draws[b].temperature))) {
+            rd_set_error("rd_step_batch_draw: row %d has draw mode %d, temperature %g", b, draws[b].mode, draws[b].temperature);
+            return RD_ERR_ARG;
+        }
+    m->step_draws = draws;
+    int rc = model_step(m, B, slot, pos, emb, nullptr, want | RD_WANT_ARGMAX, logits, ids, false);
+    m->step_draws = nullptr;
+    if (!rc)
+        for (int b = 0; b < B; b++)
+            if (draws[b].mode == RD_DRAW_NONE) ids[b] = -1;
+    return rc;
 }
 
 // resident/subsystems.go:112-117 StepRagged, forward.go:9-16 ForwardN, subsystems.go:124 PrefillLast: sequences of one or more

@@ -54,6 +54,20 @@ struct rd_model {
 
     // step scratch (device)
     float *h = nullptr, *normed = nullptr, *P = nullptr, *qbuf = nullptr, *part = nullptr, *logits = nullptr, *emb_dev = nullptr;
+    // A device-chained decode (GreedyChain* / SampleChain*): forwards queued ahead of the host, one token id coming back per forward
+    struct Chain {
+        static constexpr int DEPTH = 2; // forwards in flight: the one whose token is read next and one queued past it
+        bool open = false, sample = false, in_call = false, exhausted = false;
+        int slot = 0, next_pos = 0, exhausted_rc = 0;
+        double temperature = 1;
+        uint64_t seed = 0, draw_next = 0, draw_head = 0;
+        unsigned head = 0, tail = 0; // forwards taken / queued
+        int *host_ids = nullptr;     // pinned [DEPTH]
+        hipEvent_t ev[DEPTH] = {};
+    } chain;
+    static constexpr int META_HDR = 96 + 32 * 6; // row slot, position, length (32 each) and the rows' draw records (6 ints each)
+    int *rowDraw = nullptr;               // inside meta
+    const rd_draw *step_draws = nullptr;  // set by the entry point for the one step it runs; null = plain argmax for every row
     void *XpA = nullptr, *XpB = nullptr;
     void *XpA2 = nullptr; // the normed row in a second panel layout, for a q|k|v or gate|up group whose members differ in kind
     size_t P_floats = 0;

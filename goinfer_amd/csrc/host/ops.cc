@@ -2,13 +2,15 @@
 // (backend/cuda/kernels/actgroup_kernel_test.go, flash_decode_test.go, moe_route_test.go) and what the micro-benchmarks time.
 #include "device.h"
 #include <algorithm>
+#include <vector>
+#include <cmath>
 #include <numeric>
 #include <string.h>
 
 #define RC(x)                \
     do {                     \
-        int rc_ = (x);       \
-        if (rc_) return rc_; \
+        int rd_rc_macro_ = (x); \
+        if (rd_rc_macro_) return rd_rc_macro_; \
     } while (0)
 
 extern "C" int rd_dequant_q4k(rd_device *d, const void *blocks, int N, int K, float *out) {
@@ -194,6 +196,50 @@ extern "C" int rd_gemm_w4a8(rd_device *d, const uint8_t *nib, const uint16_t *s1
     rc = gemm_host(d, w, nullptr, a, M, dst);
     free_weight(d, &w);
     return rc;
+}
+
+// Device-side draws over explicit logit rows: the kernels the step ends with, on their own (what the reference's
+// backend/cuda/kernels/gumbel_test.go binds). Rows are padded to a multiple of four columns with -Inf, which is never drawn.
+extern "C" int rd_sample_rows(rd_device *d, const float *logits, int rows, int V, const rd_draw *draws, int *ids) {
+    if (!d || !logits || !draws || !ids || rows <= 0 || V <= 0) {
+        rd_set_error("rd_sample_rows: bad arguments");
+        return RD_ERR_ARG;
+    }
+    const int Vp = (V + 3) & ~3, nChunks = (Vp + 4095) / 4096;
+    DevBuf L(d), cv(d), ci(d), rec(d), out(d);
+    RC(L.alloc(sizeof(float) * (size_t)32 * Vp));
+    RC(cv.alloc(sizeof(float) * (size_t)32 * nChunks));
+    RC(ci.alloc(sizeof(int) * (size_t)32 * nChunks));
+    RC(rec.alloc(sizeof(int) * 32 * 6));
+    RC(out.alloc(sizeof(int) * 32));
+    std::vector<float> pad((size_t)32 * Vp);
+    for (int r0 = 0; r0 < rows; r0 += 32) {
+        int nr = std::min(32, rows - r0);
+        int recs[32 * 6] = {0};
+        for (int r = 0; r < nr; r++) {
+            const rd_draw &dw = draws[r0 + r];
+            int *q = recs + r * 6;
+            q[0] = dw.mode == RD_DRAW_NONE ? RD_DRAW_GREEDY : dw.mode;
+            if (dw.mode == RD_DRAW_GUMBEL) {
+                float invT = (float)(1.0 / (dw.temperature <= 0 ? 1.0 : dw.temperature));
+                if (std::isinf(invT)) {
+                    q[0] = RD_DRAW_GREEDY;
+                } else {
+                    memcpy(&q[1], &invT, 4);
+                    q[2] = (int)(uint32_t)dw.seed, q[3] = (int)(uint32_t)(dw.seed >> 32), q[4] = (int)(uint32_t)dw.draw, q[5] = (int)(uint32_t)(dw.draw >> 32);
+                }
+            }
+            memcpy(pad.data() + (size_t)r * Vp, logits + (size_t)(r0 + r) * V, sizeof(float) * (size_t)V);
+            for (int c = V; c < Vp; c++) pad[(size_t)r * Vp + c] = -INFINITY;
+        }
+        RC(d->h2d(L.p, pad.data(), sizeof(float) * (size_t)nr * Vp));
+        RC(d->h2d(rec.p, recs, sizeof(recs)));
+        RC(d->launch(d->k.argmax_rows, (unsigned)nChunks, (unsigned)nr, 1, 256, (const float *)L.p, 1, Vp, cv.as<float>(), ci.as<int>(), (float *)nullptr,
+                     (const int *)rec.p));
+        RC(d->launch(d->k.argmax_final, (unsigned)nr, 1, 1, 64, (const float *)cv.p, (const int *)ci.p, nChunks, out.as<int>()));
+        RC(d->d2h(ids + r0, out.p, sizeof(int) * (size_t)nr));
+    }
+    return RD_OK;
 }
 
 extern "C" int rd_matmul_bt(rd_device *d, const float *a, const float *b, float *dst, int M, int K, int N) {

@@ -31,14 +31,42 @@ extern "C" __global__ void rd_k_rope(float *__restrict__ vec, const int *__restr
     v[t + half] = (float)(x2 * c + x1 * s);
 }
 
+// Philox4x32-10 (internal/runtime/sampling/philox.go:13-40): integer only, the key bumped between rounds.
+__device__ __forceinline__ void philox4x32(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1, uint32_t *out) {
+#pragma unroll
+    for (int r = 0; r < 10; r++) {
+        if (r > 0) k0 += 0x9E3779B9u, k1 += 0xBB67AE85u;
+        const uint32_t hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
+        const uint32_t hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+        const uint32_t n0 = hi1 ^ c1 ^ k0, n2 = hi0 ^ c3 ^ k1;
+        c0 = n0, c1 = lo1, c2 = n2, c3 = lo0;
+    }
+    out[0] = c0, out[1] = c1, out[2] = c2, out[3] = c3;
+}
+// Standard Gumbel variate from 32 random bits, in f64 and rounded once, as the host computes it
+// (internal/runtime/sampling/sampler_gumbel.go:33-37): w = (h + 0.5) / 2^32, G = -ln(-ln1p(-w)).
+__device__ __forceinline__ float gumbel_noise(uint32_t h) {
+    double w = ((double)h + 0.5) * (1.0 / 4294967296.0);
+    return (float)(-log(-log1p(-w)));
+}
+
+// Per-row draw record, six ints: mode (0 none, 1 greedy, 2 Gumbel-max), 1/T as f32 bits, Philox key (seed lo, hi), draw lo, hi.
+#define RD_DRAW_INTS 6
+
 // internal/runtime/sampling/sampler.go:485-520: the first maximum wins. Two stages: per (row, 4096-column chunk) a block
 // reduces split-K partials, optionally writes the logits, and leaves its best (value, lowest index); a second kernel folds the
-// chunks of each row. N % 4 == 0.
+// chunks of each row. N % 4 == 0. A row whose draw record says Gumbel-max competes with key = f32(logit * 1/T) + G_i instead of
+// the logit (sampler_gumbel.go:41-66; backend/cuda/gumbel.cu:72-101): entry i takes word i&3 of Philox(counter (i>>2, draw lo,
+// draw hi, 0), key seed), and a thread's four consecutive entries are exactly one Philox call.
 extern "C" __global__ __launch_bounds__(256) void rd_k_argmax_rows(const float *__restrict__ P, int splits, int N, float *__restrict__ cand_v,
-                                                                   int *__restrict__ cand_i, float *__restrict__ logits_out) {
+                                                                   int *__restrict__ cand_i, float *__restrict__ logits_out,
+                                                                   const int *__restrict__ rowDraw) {
     __shared__ float bv[4];
     __shared__ int bi[4];
     const int m = blockIdx.y, t = threadIdx.x, nChunks = gridDim.x;
+    const int *dr = rowDraw ? rowDraw + m * RD_DRAW_INTS : nullptr;
+    const bool gumbel = dr && dr[0] == 2;
+    const float invT = gumbel ? __int_as_float(dr[1]) : 1.f;
     float best = -INFINITY;
     int idx = 0x7fffffff;
 #pragma unroll
@@ -51,6 +79,12 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_argmax_rows(const float *
                 a.x = __fadd_rn(a.x, b.x), a.y = __fadd_rn(a.y, b.y), a.z = __fadd_rn(a.z, b.z), a.w = __fadd_rn(a.w, b.w);
             }
             if (logits_out) *(float4_t *)(logits_out + (size_t)m * N + n0) = a;
+            if (gumbel) {
+                uint32_t r[4];
+                philox4x32((uint32_t)(n0 >> 2), (uint32_t)dr[4], (uint32_t)dr[5], 0u, (uint32_t)dr[2], (uint32_t)dr[3], r);
+#pragma unroll
+                for (int e = 0; e < 4; e++) a[e] = __fadd_rn(__fmul_rn(a[e], invT), gumbel_noise(r[e]));
+            }
 #pragma unroll
             for (int e = 0; e < 4; e++)
                 if (a[e] > best) best = a[e], idx = n0 + e; // ascending n within a thread: strict '>' keeps the lowest index
@@ -71,6 +105,8 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_argmax_rows(const float *
     }
 }
 
+// Folds a row's chunk candidates. No comparable candidate (every key -Inf or NaN: a fully masked row) gives index 0, which
+// is what the plain argmax the host falls back to returns for such a row (sampler_gumbel.go:104-107).
 extern "C" __global__ __launch_bounds__(64) void rd_k_argmax_final(const float *__restrict__ cand_v, const int *__restrict__ cand_i, int nChunks,
                                                                    int *__restrict__ ids) {
     const int m = blockIdx.x, t = threadIdx.x;

@@ -137,6 +137,35 @@ int rd_kv_reset(rd_model *m, int slot);
 /* emb: host f32 [B][hidden] (embedding rows, already scaled: decoder/residency.go:1077-1123);
  * logits: host f32 [B][vocab] when want&RD_WANT_LOGITS; ids: int32 [B] when want&RD_WANT_ARGMAX (lowest index wins). */
 int rd_step_batch(rd_model *m, int B, const int *slot, const int *pos, const float *emb, int want, float *logits, int *ids);
+/* A row's on-device draw: resident/forward.go:43-52 BatchDraw with the (seed, draw) of Sampler.NextDraw
+ * (internal/runtime/sampling/sampler_gumbel.go:68-76). RD_DRAW_GUMBEL is the temperature-only draw
+ * argmax_i(f32(l_i * 1/T) + G_i) with Philox4x32-10 noise, the function of sampler_gumbel.go:41-66,117-123 and
+ * backend/cuda/gumbel.cu; the noise transform is evaluated in f64 as on the host. */
+enum { RD_DRAW_NONE = 0, RD_DRAW_GREEDY = 1, RD_DRAW_GUMBEL = 2 };
+typedef struct rd_draw {
+    double temperature; /* <= 0 means 1; so small that 1/T overflows f32: the argmax */
+    uint64_t seed, draw;
+    int32_t mode;       /* RD_DRAW_* */
+    int32_t reserved;
+} rd_draw;
+/* rd_step_batch with draws[B] (resident/subsystems.go:102-110 StepBatch, BatchSeq.Draw): ids[i] is the drawn token of a row
+ * that carries a draw and -1 for a row that does not; logits as in rd_step_batch when want & RD_WANT_LOGITS. */
+int rd_step_batch_draw(rd_model *m, int B, const int *slot, const int *pos, const float *emb, const rd_draw *draws, int want,
+                       float *logits, int *ids);
+/* The same draws over explicit logit rows (host f32 [rows][V]), the kernels on their own as the reference's
+ * backend/cuda/kernels/gumbel_test.go binds them; RD_DRAW_NONE is taken as greedy. */
+int rd_sample_rows(rd_device *d, const float *logits, int rows, int V, const rd_draw *draws, int *ids);
+/* Decode chained on the device (decoder/resident/subsystems.go:78-100 GreedyChainStart / GreedyChainNext / GreedyChainStop and
+ * SampleChainStart / SampleChainNext): the chain's first input is token `id` at position `pos` of `slot`; each _next returns the
+ * token the forward at the chain's next position picked (the argmax, or the Gumbel-max draw with draw index draw, draw+1, ...),
+ * which is also the next forward's input, taken from the table of rd_model_upload_embedding without a host round trip. One
+ * forward is queued past the token last returned. rd_sample_chain_next refuses a (seed, draw) that is not the draw the
+ * forward was made with. Between start and stop no other step may run on the model; stop waits out what is queued. */
+int rd_greedy_chain_start(rd_model *m, int slot, int id, int pos);
+int rd_greedy_chain_next(rd_model *m, int *id);
+int rd_sample_chain_start(rd_model *m, int slot, int id, int pos, double temperature, uint64_t seed, uint64_t draw);
+int rd_sample_chain_next(rd_model *m, uint64_t seed, uint64_t draw, int *id);
+void rd_greedy_chain_stop(rd_model *m);
 /* resident/subsystems.go:112-117 StepRagged (and resident/forward.go:9-16 ForwardN as its one-sequence case): n_seq sequences
  * on distinct slots, sequence i with n_rows[i] >= 1 rows at positions pos[i], pos[i]+1, ... Rows are laid out sequence after
  * sequence: emb host f32 [sum n_rows][hidden]; logits [sum n_rows][vocab] / ids [sum n_rows] as in rd_step_batch. Row j of a
@@ -157,8 +186,9 @@ int rd_last_moe_indices(rd_model *m, int *idx);
 int rd_moe_replay(rd_model *m, int B, const int *idx, const float *wgt);
 
 /* ---- measurement: HIP-event timing on the stream the kernels are launched on; inputs resident in HBM ---- */
-/* The int8 embedding table (vocab x hidden codes + one f32 scale per row), resident so a greedy chain needs no host
- * round trip: goinfer's GreedyChain* (decoder/resident/subsystems.go:78-100). */
+/* The int8 embedding table (vocab x hidden codes + one f32 scale per row), resident so a chain needs no host
+ * round trip: goinfer's GreedyChain* (decoder/resident/subsystems.go:78-100). Row id is code * scale, the row the host's
+ * embedding lookup sends for the same table. */
 int rd_model_upload_embedding(rd_model *m, const int8_t *q, const float *row_scale);
 /* Greedy decode chain on the device: step i runs rows (slot[b], pos0[b]+i) on the embedding of the previous step's
  * argmax (ids0 for the first). ms_out[steps]: per-step milliseconds; ids_out: optional int32 [steps][B] picked tokens. */

@@ -299,3 +299,38 @@ class OracleModel:
 
     def cfg_layers(self):
         return self.m.n_layers
+
+
+def philox4x32(ctr, key):
+    c = (C.c_uint32 * 4)(*ctr)
+    k = (C.c_uint32 * 2)(*key)
+    out = (C.c_uint32 * 4)()
+    lib().or_philox4x32(c, k, out)
+    return tuple(out)
+
+
+def gumbel_noise(h):
+    f = lib().or_gumbel_noise
+    f.restype = C.c_float
+    return float(f(C.c_uint32(int(h))))
+
+
+def gumbel_draw(logits, temperature, seed, draw, guarded=False):
+    """GumbelDraw(logits, temperature, seed, draw); guarded=True adds Sampler.gumbelDraw's temperature guards."""
+    x = f32(logits)
+    f = lib().or_sampler_gumbel_draw if guarded else lib().or_gumbel_draw
+    return int(f(_p(x), x.size, C.c_double(temperature), C.c_uint64(seed), C.c_uint64(draw)))
+
+
+def gumbel_draw_many(logits, temperature, seed, draw0, count):
+    x = f32(logits)
+    out = np.empty(count, np.int32)
+    lib().or_gumbel_draw_many(_p(x), x.size, C.c_double(temperature), C.c_uint64(seed), C.c_uint64(draw0), count, _p(out))
+    return out
+
+
+def gumbel_noise_many(h):
+    h = np.ascontiguousarray(h, dtype=np.uint32)
+    out = np.empty(h.size, np.float32)
+    lib().or_gumbel_noise_many(_p(h), C.c_size_t(h.size), _p(out))
+    return out

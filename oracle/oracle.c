@@ -366,6 +366,71 @@ int or_argmax(const float *x, int n) {
     return bi;
 }
 
+/* ------------------------------------------------------------------ temperature-only sampling (Gumbel-max) */
+/* internal/runtime/sampling/philox.go:13-40 (Philox4x32): Philox4x32-10; the key is bumped between rounds, not before the first. */
+void or_philox4x32(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]) {
+    uint32_t c0 = ctr[0], c1 = ctr[1], c2 = ctr[2], c3 = ctr[3], k0 = key[0], k1 = key[1];
+    for (int r = 0; r < 10; r++) {
+        if (r > 0) k0 += 0x9E3779B9u, k1 += 0xBB67AE85u;
+        uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+        uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+        c0 = n0, c1 = (uint32_t)p1, c2 = n2, c3 = (uint32_t)p0;
+    }
+    out[0] = c0, out[1] = c1, out[2] = c2, out[3] = c3;
+}
+
+/* sampler_gumbel.go:33-37 (gumbelNoise): w = (h + 0.5) / 2^32 in f64, E = -log1p(-w), G = f32(-log(E)). */
+float or_gumbel_noise(uint32_t h) {
+    double w = ((double)h + 0.5) * (1.0 / 4294967296.0);
+    double e = -log1p(-w);
+    return (float)(-log(e));
+}
+
+/* sampler_gumbel.go:41-43 (GumbelKey): the product is rounded to f32 before the add (no fused multiply-add). */
+float or_gumbel_key(float logit, float invT, uint32_t h) {
+    volatile float prod = logit * invT;
+    return prod + or_gumbel_noise(h);
+}
+
+/* sampler_gumbel.go:47-66 (GumbelArgmaxRange over the whole row) and :117-123 (GumbelDraw): counter (i>>2, draw, draw>>32, 0),
+ * key (seed, seed>>32), lane i&3; strict '>' from -Inf in ascending index order, so the lowest index wins a tie and a NaN or
+ * -Inf key is never chosen; no comparable entry -> the plain argmax. */
+int or_gumbel_draw(const float *logits, int n, double temperature, uint64_t seed, uint64_t draw) {
+    float invT = (float)(1.0 / temperature);
+    uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+    float best = -INFINITY;
+    int idx = -1;
+    for (int b = 0; (b << 2) < n; b++) {
+        uint32_t ctr[4] = {(uint32_t)b, (uint32_t)draw, (uint32_t)(draw >> 32), 0}, r[4];
+        or_philox4x32(ctr, key, r);
+        for (int lane = 0; lane < 4; lane++) {
+            int i = (b << 2) + lane;
+            if (i >= n) continue;
+            float k = or_gumbel_key(logits[i], invT, r[lane]);
+            if (k > best) best = k, idx = i;
+        }
+    }
+    return idx < 0 ? or_argmax(logits, n) : idx;
+}
+
+/* sampler_gumbel.go:79-109 (Sampler.gumbelDraw): the guards in front of the draw — a temperature <= 0 means 1, and a
+ * temperature so small that 1/T overflows f32 is the argmax, as greedy. */
+int or_sampler_gumbel_draw(const float *logits, int n, double temperature, uint64_t seed, uint64_t draw) {
+    if (temperature <= 0) temperature = 1;
+    float invT = (float)(1.0 / temperature);
+    if (isinf(invT)) return or_argmax(logits, n);
+    return or_gumbel_draw(logits, n, temperature, seed, draw);
+}
+
+/* Test conveniences: `count` consecutive draws of one row (draw0, draw0+1, ...), and the noise of many words. */
+void or_gumbel_draw_many(const float *logits, int n, double temperature, uint64_t seed, uint64_t draw0, int count, int *out) {
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+    for (int i = 0; i < count; i++) out[i] = or_gumbel_draw(logits, n, temperature, seed, draw0 + (uint64_t)i);
+}
+void or_gumbel_noise_many(const uint32_t *h, size_t n, float *out) {
+    for (size_t i = 0; i < n; i++) out[i] = or_gumbel_noise(h[i]);
+}
+
 /* ------------------------------------------------------------------ matmul dispatch */
 /* decoder/weightmat.go:892-985 (matmulWS): the weight's kind picks the kernel. The int kinds quantize
  * the activation first (group 32 in q4k mode, weightmat.go:33-38). Arithmetic of each row:

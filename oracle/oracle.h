@@ -21,6 +21,12 @@
  *   or_rmsnorm, or_rope, or_swiglu, or_softmax_f32, or_topk, or_route_experts, or_argmax
  *                                        plain Go in the reference, restated statement by statement;
  *                                        pinned by closed forms + the HF goldens (llama-tiny, qwen3moe-tiny, mixtral-tiny)
+ *   or_philox4x32                        pinned: the Random123 known-answer vectors the reference's philox_test.go holds
+ *   or_gumbel_noise / _key / _draw       pinned by the closed form the reference's tests state (f64 -log(-log1p(-w)), range,
+ *                                        monotone), by chi-square fit of the draw to softmax(l/T) under the reference's own
+ *                                        pre-registered rule, and by its edge rows (-Inf never drawn, masked row -> argmax).
+ *                                        The reference holds no golden token stream, so the counter layout (i>>2, draw,
+ *                                        draw>>32, 0; lane i&3) is "parity unpinned" beyond its statement in the source.
  *   or_matmul (f32 kind)                 parity unpinned at bit level (aikit's summation order is arch dependent);
  *                                        pinned to tolerance by the HF goldens
  *   or_matmul (q4k / w4a8 / w8a8 kinds)  parity unpinned at bit level: the reference's own result differs between
@@ -78,6 +84,15 @@ void or_softmax_f32(const float *x, int n, float *out);
 int or_topk(const float *x, int n, int k, int *idx, float *val);
 int or_route_experts(const float *logits, int nE, int k, int norm, double scale, int *idx, float *wts);
 int or_argmax(const float *x, int n); /* internal/runtime/sampling/sampler.go:485-520: first maximum wins */
+
+/* ---- temperature-only sampling by Gumbel-max: internal/runtime/sampling/philox.go, sampler_gumbel.go ---- */
+void or_philox4x32(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]);
+float or_gumbel_noise(uint32_t h);
+float or_gumbel_key(float logit, float invT, uint32_t h);
+int or_gumbel_draw(const float *logits, int n, double temperature, uint64_t seed, uint64_t draw);         /* GumbelDraw */
+int or_sampler_gumbel_draw(const float *logits, int n, double temperature, uint64_t seed, uint64_t draw); /* Sampler.gumbelDraw's guards */
+void or_gumbel_draw_many(const float *logits, int n, double temperature, uint64_t seed, uint64_t draw0, int count, int *out);
+void or_gumbel_noise_many(const uint32_t *h, size_t n, float *out);
 
 /* ---- weight matrices and the matmul dispatch: decoder/weightmat.go:845-985 ---- */
 enum { OR_F32 = 0, OR_Q4K = 1, OR_W4A8 = 2, OR_W8A8 = 3, OR_Q5K = 4, OR_Q6K = 5 };
