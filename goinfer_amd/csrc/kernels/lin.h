@@ -3,6 +3,7 @@
 #pragma once
 #include "common.h"
 #include "gemm.h"
+#include "q4k.h"
 
 // ---------------- W8A8: int8 codes, one f32 scale per row (goinfer WeightMat.Int8, decoder/weightmat.go:931) ----------------
 // Tile of 32 rows x 128 k = 4096 B as 4 planes [64 lanes][16 B]; lane (row r, half h) plane c holds codes
@@ -103,6 +104,7 @@ struct W4Traits {
     }
     static __device__ __forceinline__ void mma(float16_t &acc, const Tile &w, const uint4_t *__restrict__ panel, int lane) {
         const half2_t o_lo = {(half_t)(-1032.f), (half_t)(-1032.f)}, o_hi = {(half_t)(-72.f), (half_t)(-72.f)};
+        const uint32_t mask_lo = 0x000F000Fu, mask_hi = 0x00F000F0u, magic_lo = 0x64006400u, magic_hi = 0x54005400u;
         half2_t s01, s23;
         uint32_t a0 = w.sc.x, a1 = w.sc.y;
         __builtin_memcpy(&s01, &a0, 4);
@@ -112,8 +114,8 @@ struct W4Traits {
         for (int s = 0; s < 8; s++) {
             uint32_t wd = w.q[s >> 2][s & 3], t8 = wd >> 8;
             half2_t sc = {gs[s >> 1], gs[s >> 1]};
-            uint32_t u0 = (wd & 0x000F000Fu) | 0x64006400u, u1 = (wd & 0x00F000F0u) | 0x54005400u;
-            uint32_t u2 = (t8 & 0x000F000Fu) | 0x64006400u, u3 = (t8 & 0x00F000F0u) | 0x54005400u;
+            uint32_t u0 = and_or(wd, mask_lo, magic_lo), u1 = and_or(wd, mask_hi, magic_hi);
+            uint32_t u2 = and_or(t8, mask_lo, magic_lo), u3 = and_or(t8, mask_hi, magic_hi);
             half2_t v0, v1, v2, v3;
             __builtin_memcpy(&v0, &u0, 4);
             __builtin_memcpy(&v1, &u1, 4);
@@ -128,6 +130,12 @@ struct W4Traits {
         }
     }
     static __device__ __forceinline__ void finish(float16_t &, const void *, int, int) {}
+};
+
+// The expert GEMM's K loops are short (6 to 16 blocks) and its grid large: a shallower producer ring keeps the block under
+// 128 registers, so three blocks instead of two share a CU.
+struct W4MoeTraits : W4Traits {
+    static constexpr int PRODUCER_DEPTH = 2;
 };
 
 extern "C" __global__ __launch_bounds__(320) void rd_k_gemm_w4a8(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ Xp,

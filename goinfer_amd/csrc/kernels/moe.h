@@ -19,7 +19,7 @@ extern "C" __global__ __launch_bounds__(320) void rd_k_gemm_w4a8_moe(const uint8
     const bool active = tile * 32 < N;
     float16_t acc;
     const int ltile = active ? tile : (N >> 5) - 1;
-    gemm_mainloop_pc<W4Traits, 4, 1, 3>(acc, Wt + (size_t)e * wStride + (size_t)ltile * nKB * W4Traits::TILE_BYTES, Xp + (size_t)e * xpStride, 0, nKB,
+    gemm_mainloop_pc<W4MoeTraits, 4, 1, 3>(acc, Wt + (size_t)e * wStride + (size_t)ltile * nKB * W4Traits::TILE_BYTES, Xp + (size_t)e * xpStride, 0, nKB,
                                         lds);
     if (!active || wave >= 4) return;
 #pragma unroll
