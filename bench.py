@@ -31,7 +31,7 @@ def log(msg):
     print("[bench %6.1fs] %s" % (time.time() - T0, msg), file=sys.stderr, flush=True)
 
 
-def cpu_baseline(res, cfg, lens, kept_kv, threads):
+def cpu_baseline(res, cfg, lens, kept_kv, threads, kv="f16"):
     """The oracle's decodeMultiStep on the first layers of the same model, the same 32 ragged sequences and KV, greedy
     steps for about ten seconds; the per-layer cost scaled to the full depth. Returns (tok/s, description of the sample)."""
     from oracle import binding as ob
@@ -43,7 +43,7 @@ def cpu_baseline(res, cfg, lens, kept_kv, threads):
         lw["attn_norm"], lw["ffn_norm"] = kp["attn_norm"], kp["ffn_norm"]
         layers.append(lw)
     c = dict(cfg)
-    c.update(n_layers=nL, kv_f16=1)
+    c.update(n_layers=nL, kv_f16=1 if kv == "f16" else 2)
     hq, hs = res.head
     head = ob.WMat(ob.OR_W8A8, hq.shape[0], hq.shape[1], hq, hs, act_group=32)
     from goinfer_amd.workloads import inv_freq
@@ -90,6 +90,8 @@ def parse_args():
     ap.add_argument("--batch", type=int, default=32)
     ap.add_argument("--seed", type=int, default=1234)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--kv", default="f16", choices=["f16", "i8"],
+                    help="KV cache element (c4 and c3): f16 as the metric is quoted, or goinfer's int8 cache (KVQuant i8), a variant of the workload")
     ap.add_argument("--workload", default="c4", choices=["c4", "c2", "c3", "c5", "kquant"],
                     help="c4 (default): the Llama-3-8B-shape step the metric is quoted on; c2: Q4_K GEMM microbench; c3: ragged "
                          "attention microbench; c5: Qwen3-MoE-shape step; kquant: Q4_K / Q5_K / Q6_K GEMMs at the FFN and head shapes")
@@ -112,7 +114,7 @@ def run_c4(args):
     cap = int(lens.max()) + args.steps + args.warmup + 8
     dev = capi.Device(0)
     log("building %s, %d layers" % (cfg["name"], cfg["n_layers"]))
-    res = workloads.Resident(dev, cfg, seed=args.seed, slots=B, ctx_cap=cap, keep_layers=0 if args.no_cpu else min(CPU_LAYERS, args.layers), progress=log)
+    res = workloads.Resident(dev, cfg, seed=args.seed, slots=B, ctx_cap=cap, keep_layers=0 if args.no_cpu else min(CPU_LAYERS, args.layers), progress=log, kv=args.kv)
     kept_kv = res.prefill_kv(lens, progress=log)
     slots = np.arange(B, dtype=np.int32)
 
@@ -128,7 +130,7 @@ def run_c4(args):
 
     # ---- algorithmic bytes of a step at the mid-run context lengths ----
     mid = lens + args.warmup + args.steps // 2
-    kv_pos_bytes = workloads.kv_bytes_per_position(cfg)
+    kv_pos_bytes = workloads.kv_bytes_per_position(cfg, args.kv)
     kv_read = float((mid + 1).sum()) * kv_pos_bytes
     w_bytes = workloads.weight_bytes(cfg)
     step_bytes = w_bytes + kv_read + B * kv_pos_bytes
@@ -145,9 +147,9 @@ def run_c4(args):
             a[1] += n
     kern = "attn_partial"
     avg_ms = prof[kern][0] / prof[kern][1]
-    # per launch (one layer): every sequence's K and V rows once (f16), plus q in and partial results out
+    # per launch (one layer): every sequence's K and V rows once (f16, or int8 and their scales), plus q in and partial results out
     G = cfg["n_heads"] // cfg["n_kv"]
-    kv_launch = float((pos_prof + 2).sum()) * 2 * cfg["n_kv"] * cfg["head_dim"] * 2
+    kv_launch = float((pos_prof + 2).sum()) * kv_pos_bytes / cfg["n_layers"]
     q_launch = B * cfg["n_heads"] * cfg["head_dim"] * 4
     achieved = (kv_launch + q_launch) / (avg_ms / 1e3) / 1e9
     traffic = None
@@ -155,7 +157,7 @@ def run_c4(args):
     if os.path.exists(tpath):
         traffic = json.load(open(tpath)).get("%s/%s" % (kern, cfg["name"]))
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "traffic": traffic, "kernel": "rd_k_attn_partial", "avg_launch_ms": round(avg_ms, 5),
+                "traffic": traffic if args.kv == "f16" else None, "kernel": "rd_k_attn_partial" if args.kv == "f16" else "rd_k_attn_partial_i8", "avg_launch_ms": round(avg_ms, 5),
                 "algorithmic_bytes_per_launch": int(kv_launch + q_launch)}
     classes = {k: {"ms_per_step": round(v[0] / 3, 4), "launches_per_step": v[1] // 3} for k, v in prof.items()}
 
@@ -168,7 +170,7 @@ def run_c4(args):
     if not args.no_cpu:
         threads = min(16, len(os.sched_getaffinity(0)))
         log("CPU baseline on %d threads" % threads)
-        v, sample = cpu_baseline(res, cfg, lens, kept_kv, threads)
+        v, sample = cpu_baseline(res, cfg, lens, kept_kv, threads, args.kv)
         cpu = {"value": round(v, 3), "unit": "tok/s", "cores": threads, "kind": "port", "sample": sample}
     res.close()
     dev.close()
@@ -179,7 +181,8 @@ def run_c4(args):
         "ms_per_step": round(float(ms.mean()), 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16",
         "data": "synthetic: N(0,0.02) weights quantized to Q4_K (int8 head), N(0,1) KV, random token ids",
-        "config": {"workload": "configs[3]: %s, %d layers, B=%d ragged, ctx U[512,4096], greedy decode" % (cfg["name"], cfg["n_layers"], B),
+        "config": {"workload": "configs[3]: %s, %d layers, B=%d ragged, ctx U[512,4096], greedy decode%s"
+                               % (cfg["name"], cfg["n_layers"], B, "" if args.kv == "f16" else " (variant: int8 KV cache)"), "kv": args.kv,
                    "batch": B, "ctx_min": int(lens.min()), "ctx_max": int(lens.max()), "ctx_mean": float(lens.mean()), "seed": args.seed},
         "step_hbm": {"algorithmic_bytes_per_step": int(step_bytes), "achieved_GBs": round(step_gbs, 1), "frac_of_peak": round(step_gbs / HBM_PEAK_GBS, 4),
                      "weights_bytes": int(w_bytes), "kv_read_bytes": int(kv_read)},

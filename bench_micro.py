@@ -136,26 +136,28 @@ def run_c3(args):
     nH, nKV, hd, nseq = 32, 8, 128, 64
     lens = np.random.default_rng(args.seed).integers(128, 8193, nseq).astype(np.int32)
     scale = float(1.0 / np.sqrt(hd))
-    kv_bytes = float(lens.sum()) * 2 * nKV * hd * 2
+    kv = getattr(args, "kv", "f16")
+    kv_bytes = float(lens.sum()) * 2 * nKV * (hd * 2 if kv == "f16" else hd + 4)  # int8: the codes and one f32 scale per (position, kv head)
     io_bytes = 2 * nseq * nH * hd * 4
     dev = capi.Device(0)
     res = {}
     for cap in (0.0, 50.0):
-        tot, part = dev.bench_attn(lens, nH, nKV, hd, scale, cap, warmup, steps)
+        tot, part = dev.bench_attn(lens, nH, nKV, hd, scale, cap, warmup, steps, kv=kv)
         res[cap] = (float(np.median(tot)), float(np.median(part)))
         log("softcap %g: call %.1f us (%.0f GB/s), partial kernels %.1f us (%.0f GB/s)" % (
             cap, res[cap][0] * 1e3, (kv_bytes + io_bytes) / res[cap][0] / 1e6, res[cap][1] * 1e3, kv_bytes / res[cap][1] / 1e6))
     t, tp = res[0.0]
     gbs = (kv_bytes + io_bytes) / t / 1e6
     out = base_line("ragged flash-decode attention achieved HBM GB/s (64 sequences, KV U[128,8192], 32/8 heads, head_dim 128)", gbs, "GB/s", steps,
-                    warmup, t, "configs[2]: ragged attention microbench", "synthetic: uniform [-2,2) f16 KV in a paged pool with a scattered block table, f32 q",
-                    {"n_seq": nseq, "kv_positions": int(lens.sum()), "kv_len_min": int(lens.min()), "kv_len_max": int(lens.max()), "seed": args.seed,
+                    warmup, t, "configs[2]: ragged attention microbench" + ("" if kv == "f16" else " (variant: int8 KV cache)"),
+                    "synthetic: uniform [-2,2) f16 KV (or random int8 codes and scales) in a paged pool with a scattered block table, f32 q",
+                    {"kv": kv, "n_seq": nseq, "kv_positions": int(lens.sum()), "kv_len_min": int(lens.min()), "kv_len_max": int(lens.max()), "seed": args.seed,
                      "cases": [{"softcap": c, "call_us": round(v[0] * 1e3, 2), "call_GBs": round((kv_bytes + io_bytes) / v[0] / 1e6, 1),
                                 "partial_kernels_us": round(v[1] * 1e3, 2), "partial_kernels_GBs": round(kv_bytes / v[1] / 1e6, 1)} for c, v in res.items()]})
     # the partial kernel is launched once per group of 32 rows: two launches per call here
     per_launch = (kv_bytes + nseq * nH * hd * 4) / 2
     out["roofline"] = {"bound": "hbm", "achieved": round(per_launch / (tp / 2) / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                       "frac": round(per_launch / (tp / 2) / 1e6 / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "rd_k_attn_partial",
+                       "frac": round(per_launch / (tp / 2) / 1e6 / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "rd_k_attn_partial" if kv == "f16" else "rd_k_attn_partial_i8",
                        "avg_launch_ms": round(tp / 2, 5), "algorithmic_bytes_per_launch": int(per_launch)}
     cpu = None
     if not args.no_cpu:

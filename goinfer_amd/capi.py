@@ -21,6 +21,7 @@ EXPORTS = [
     "rd_kv_configure", "rd_kv_upload", "rd_kv_truncate", "rd_kv_reset", "rd_step_batch", "rd_forward",
     "rd_last_moe_indices", "rd_model_upload_embedding", "rd_bench_steps", "rd_bench_profile", "rd_bench_class_count",
     "rd_bench_class_name", "rd_bench_kernel", "rd_gateup_q4k_quant", "rd_moe_replay", "rd_bench_attn", "rd_step_ragged", "rd_prefill_last",
+    "rd_kv_configure_typed", "rd_attn_ragged_i8", "rd_bench_attn_i8",
     "rd_step_batch_draw", "rd_sample_rows", "rd_greedy_chain_start", "rd_greedy_chain_next", "rd_sample_chain_start",
     "rd_sample_chain_next", "rd_greedy_chain_stop",
     "rd_dequant_q5k", "rd_dequant_q6k", "rd_gemm_q5k", "rd_gemm_q6k", "rd_model_upload_q5k", "rd_model_upload_q6k",
@@ -189,14 +190,16 @@ class Device:
         check(lib().rd_gemm_w4a8(self.h, _p(nib), _p(s16), N, K, _p(a), a.shape[0], _p(dst)), "rd_gemm_w4a8")
         return dst
 
-    def attn_ragged(self, lens, k, v, q, n_h, n_kv, hd, scale, softcap=0.0):
+    def attn_ragged(self, lens, k, v, q, n_h, n_kv, hd, scale, softcap=0.0, kv="f16"):
+        """kv: "f16" (the binary16 cache) or "i8" (the int8 cache with one scale per position and kv head)."""
         lens = np.ascontiguousarray(lens, dtype=np.int32)
         off = np.zeros(len(lens), np.int64)
         off[1:] = np.cumsum(lens[:-1])
         k, v, q = _f32(k), _f32(v), _f32(q)
         out = np.empty((len(lens), n_h * hd), np.float32)
-        check(lib().rd_attn_ragged(self.h, len(lens), _p(lens), _p(off), _p(k), _p(v), _p(q), n_h, n_kv, hd,
-                                   C.c_float(scale), C.c_float(softcap), _p(out)), "rd_attn_ragged")
+        name = "rd_attn_ragged" if kv == "f16" else "rd_attn_ragged_i8"
+        check(getattr(lib(), name)(self.h, len(lens), _p(lens), _p(off), _p(k), _p(v), _p(q), n_h, n_kv, hd,
+                                   C.c_float(scale), C.c_float(softcap), _p(out)), name)
         return out
 
     def moe_route(self, logits, k, norm):
@@ -220,11 +223,12 @@ class Device:
         check(lib().rd_rope(self.h, _p(v), v.shape[0], heads, head_dim, _p(pos), _p(inv)), "rd_rope")
         return v
 
-    def bench_attn(self, lens, n_h, n_kv, hd, scale, softcap, warmup, iters):
+    def bench_attn(self, lens, n_h, n_kv, hd, scale, softcap, warmup, iters, kv="f16"):
         lens = np.ascontiguousarray(lens, dtype=np.int32)
         tot, part = np.empty(iters, np.float32), np.empty(iters, np.float32)
-        check(lib().rd_bench_attn(self.h, len(lens), _p(lens), n_h, n_kv, hd, C.c_float(scale), C.c_float(softcap), warmup, iters,
-                                  _p(tot), _p(part)), "rd_bench_attn")
+        name = "rd_bench_attn" if kv == "f16" else "rd_bench_attn_i8"
+        check(getattr(lib(), name)(self.h, len(lens), _p(lens), n_h, n_kv, hd, C.c_float(scale), C.c_float(softcap), warmup, iters,
+                                   _p(tot), _p(part)), name)
         return tot, part
 
     def bench_kernel(self, name, args, warmup, iters):
@@ -280,8 +284,11 @@ class Model:
     def finalize(self):
         check(lib().rd_model_finalize(self.h), "rd_model_finalize")
 
-    def kv_configure(self, slots, ctx_cap):
-        check(lib().rd_kv_configure(self.h, slots, ctx_cap), "rd_kv_configure")
+    def kv_configure(self, slots, ctx_cap, kv="f16"):
+        if kv == "f16":
+            check(lib().rd_kv_configure(self.h, slots, ctx_cap), "rd_kv_configure")
+        else:
+            check(lib().rd_kv_configure_typed(self.h, slots, ctx_cap, {"i8": 1}[kv]), "rd_kv_configure_typed")
 
     def kv_upload(self, slot, layer, base, keys, vals):
         keys, vals = _f32(keys), _f32(vals)

@@ -240,8 +240,8 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
 // The ragged flash-decode attention of one layer over a synthetic paged f16 KV pool (uniform [-2,2) values, scattered
 // block table), rows in groups of 32 as the step batches them. ms_total[iters]: the whole call (partial + combine kernels
 // of every group); ms_partial[iters] (may be NULL): the partial kernels alone. HIP events on the launch stream.
-extern "C" int rd_bench_attn(rd_device *d, int n_seq, const int *len, int n_h, int n_kv, int hd, float scale, float softcap, int warmup, int iters,
-                             float *ms_total, float *ms_partial) {
+static int bench_attn_typed(rd_device *d, int kv_type, int n_seq, const int *len, int n_h, int n_kv, int hd, float scale, float softcap, int warmup,
+                            int iters, float *ms_total, float *ms_partial) {
     if (!d || !len || n_seq <= 0 || iters <= 0 || !ms_total) return RD_ERR_ARG;
     if (n_kv <= 0 || n_h % n_kv || n_h / n_kv > 16 || (hd != 64 && hd != 128)) {
         rd_set_error("rd_bench_attn declines: head_dim must be 64 or 128 and the GQA group <= 16");
@@ -264,10 +264,18 @@ extern "C" int rd_bench_attn(rd_device *d, int n_seq, const int *len, int n_h, i
         for (int i = 0; i < n_seq; i++)
             for (int b = 0; b < (len[i] + 63) / 64; b++, idx++) tab[(size_t)i * maxBlocks + b] = 1 + (int)((idx * stride) % nb);
     }
-    const size_t poolHalves = (size_t)(totalBlocks + 1) * n_kv * 64 * hd;
-    DevBuf Kp(d), Vp(d), T(d), Q(d), O(d);
+    const bool i8 = kv_type == RD_KV_I8;
+    // the int8 pool is filled as binary16 values over half as many elements: every byte pattern is a valid code
+    const size_t poolHalves = (size_t)(totalBlocks + 1) * n_kv * 64 * hd / (i8 ? 2 : 1), scFloats = (size_t)(totalBlocks + 1) * n_kv * 64;
+    DevBuf Kp(d), Vp(d), Ksc(d), Vsc(d), T(d), Q(d), O(d);
     RC(Kp.alloc(poolHalves * 2));
     RC(Vp.alloc(poolHalves * 2));
+    if (i8) {
+        RC(Ksc.alloc(scFloats * sizeof(float)));
+        RC(Vsc.alloc(scFloats * sizeof(float)));
+        RC(d->launch(d->k.fill_f32, 256, 1, 1, 256, Ksc.as<float>(), scFloats, 14u));
+        RC(d->launch(d->k.fill_f32, 256, 1, 1, 256, Vsc.as<float>(), scFloats, 15u));
+    }
     RC(T.alloc(sizeof(int) * tab.size()));
     RC(Q.alloc(sizeof(float) * (size_t)n_seq * qd));
     RC(O.alloc(sizeof(float) * (size_t)n_seq * qd));
@@ -313,9 +321,14 @@ extern "C" int rd_bench_attn(rd_device *d, int n_seq, const int *len, int n_h, i
         for (size_t gi = 0; gi < nG && !rc; gi++) {
             Group &g = *groups[gi];
             if (timed) (void)d->hip->EventRecord(evp[(t * nG + gi) * 2], d->stream);
-            rc = d->launch(d->k.attn_partial, (unsigned)g.nItems, 1, 1, 64, (const void *)g.I.p, (const int *)g.L.p, (const int *)g.S.p, (const int *)T.p, maxBlocks,
-                           (const uint16_t *)Kp.p, (const uint16_t *)Vp.p, (const float *)((const float *)Q.p + (size_t)g.r0 * qd), g.P.as<float>(), n_h, n_kv, hd, scale,
-                           softcap);
+            if (i8)
+                rc = d->launch(d->k.attn_partial_i8, (unsigned)g.nItems, 1, 1, 64, (const void *)g.I.p, (const int *)g.L.p, (const int *)g.S.p, (const int *)T.p,
+                               maxBlocks, (const signed char *)Kp.p, (const signed char *)Vp.p, (const float *)Ksc.p, (const float *)Vsc.p,
+                               (const float *)((const float *)Q.p + (size_t)g.r0 * qd), g.P.as<float>(), n_h, n_kv, hd, scale, softcap);
+            else
+                rc = d->launch(d->k.attn_partial, (unsigned)g.nItems, 1, 1, 64, (const void *)g.I.p, (const int *)g.L.p, (const int *)g.S.p, (const int *)T.p, maxBlocks,
+                               (const uint16_t *)Kp.p, (const uint16_t *)Vp.p, (const float *)((const float *)Q.p + (size_t)g.r0 * qd), g.P.as<float>(), n_h, n_kv, hd,
+                               scale, softcap);
             if (timed) (void)d->hip->EventRecord(evp[(t * nG + gi) * 2 + 1], d->stream);
             if (!rc)
                 rc = d->launch(d->k.attn_combine, (unsigned)n_h, (unsigned)g.rows, 1, (unsigned)(ATTN_PIECES * hd / 4), (const float *)g.P.p, (const int *)g.St.p,
@@ -340,4 +353,12 @@ extern "C" int rd_bench_attn(rd_device *d, int n_seq, const int *len, int n_h, i
     for (auto &e : ev) (void)d->hip->EventDestroy(e);
     for (auto &e : evp) (void)d->hip->EventDestroy(e);
     return rc;
+}
+extern "C" int rd_bench_attn(rd_device *d, int n_seq, const int *len, int n_h, int n_kv, int hd, float scale, float softcap, int warmup, int iters,
+                             float *ms_total, float *ms_partial) {
+    return bench_attn_typed(d, RD_KV_F16, n_seq, len, n_h, n_kv, hd, scale, softcap, warmup, iters, ms_total, ms_partial);
+}
+extern "C" int rd_bench_attn_i8(rd_device *d, int n_seq, const int *len, int n_h, int n_kv, int hd, float scale, float softcap, int warmup, int iters,
+                                float *ms_total, float *ms_partial) {
+    return bench_attn_typed(d, RD_KV_I8, n_seq, len, n_h, n_kv, hd, scale, softcap, warmup, iters, ms_total, ms_partial);
 }

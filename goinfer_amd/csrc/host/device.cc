@@ -90,6 +90,9 @@ static const KName kNames[] = {
     {"rd_k_kv_store", &Kernels::kv_store},
     {"rd_k_qkv_rope_store", &Kernels::qkv_rope_store},
     {"rd_k_attn_partial", &Kernels::attn_partial},
+    {"rd_k_kv_store_i8", &Kernels::kv_store_i8},
+    {"rd_k_qkv_rope_store_i8", &Kernels::qkv_rope_store_i8},
+    {"rd_k_attn_partial_i8", &Kernels::attn_partial_i8},
     {"rd_k_attn_combine", &Kernels::attn_combine},
     {"rd_k_attn_combine_quant", &Kernels::attn_combine_quant},
     {"rd_k_rmsnorm", &Kernels::rmsnorm},

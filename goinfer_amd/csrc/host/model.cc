@@ -59,7 +59,7 @@ extern "C" void rd_model_destroy(rd_model *m) {
     for (auto &l : m->layers) {
         free_weight(d, &l.qkv), free_weight(d, &l.o), free_weight(d, &l.gateup), free_weight(d, &l.down);
         for (void *p : {(void *)l.attn_norm, (void *)l.ffn_norm, (void *)l.q_norm, (void *)l.k_norm, (void *)l.router, l.exp_gateup, l.exp_down,
-                        (void *)l.Kp, (void *)l.Vp})
+                        (void *)l.Kp, (void *)l.Vp, (void *)l.Ksc, (void *)l.Vsc})
             d->release(p);
     }
     free_weight(d, &m->head);
@@ -399,8 +399,14 @@ extern "C" int rd_model_finalize(rd_model *m) {
 }
 
 // ---------------------------------------------------------------- KV
-extern "C" int rd_kv_configure(rd_model *m, int slots, int ctx_cap) {
+extern "C" int rd_kv_configure(rd_model *m, int slots, int ctx_cap) { return rd_kv_configure_typed(m, slots, ctx_cap, RD_KV_F16); }
+
+extern "C" int rd_kv_configure_typed(rd_model *m, int slots, int ctx_cap, int kv_type) {
     if (!m || slots <= 0 || ctx_cap <= 0) return RD_ERR_ARG;
+    if (kv_type != RD_KV_F16 && kv_type != RD_KV_I8) {
+        rd_set_error("rd_kv_configure_typed: unknown KV type %d", kv_type);
+        return RD_ERR_ARG;
+    }
     if (m->tables) {
         rd_set_error("KV already configured");
         return RD_ERR_STATE;
@@ -409,11 +415,14 @@ extern "C" int rd_kv_configure(rd_model *m, int slots, int ctx_cap) {
     const rd_model_desc &c = m->desc;
     m->slots = slots, m->ctx_cap = ctx_cap, m->blocks_per_slot = (ctx_cap + 63) / 64;
     size_t nBlocks = (size_t)slots * m->blocks_per_slot + 1; // block 0 is the all-zero block no slot owns
-    size_t bytes = nBlocks * c.n_kv_heads * 64 * c.head_dim * 2;
+    const bool i8 = kv_type == RD_KV_I8;
+    size_t bytes = nBlocks * c.n_kv_heads * 64 * c.head_dim * (i8 ? 1 : 2);
+    size_t scBytes = i8 ? nBlocks * c.n_kv_heads * 64 * sizeof(float) : 0;
+    m->kv_type = kv_type;
     size_t fr = 0, tot = 0;
     HIPCHK(MemGetInfo(&fr, &tot));
-    if (bytes * 2 * c.n_layers > fr) {
-        rd_set_error("rocm resident declines: KV pool of %zu MiB exceeds free device memory (%zu MiB)", (bytes * 2 * c.n_layers) >> 20, fr >> 20);
+    if ((bytes + scBytes) * 2 * c.n_layers > fr) {
+        rd_set_error("rocm resident declines: KV pool of %zu MiB exceeds free device memory (%zu MiB)", ((bytes + scBytes) * 2 * c.n_layers) >> 20, fr >> 20);
         return RD_DECLINED;
     }
     for (auto &l : m->layers) {
@@ -421,6 +430,12 @@ extern "C" int rd_kv_configure(rd_model *m, int slots, int ctx_cap) {
         RC(d->alloc((void **)&l.Vp, bytes));
         HIPCHK(MemsetAsync(l.Kp, 0, bytes, d->stream));
         HIPCHK(MemsetAsync(l.Vp, 0, bytes, d->stream));
+        if (i8) {
+            RC(d->alloc((void **)&l.Ksc, scBytes));
+            RC(d->alloc((void **)&l.Vsc, scBytes));
+            HIPCHK(MemsetAsync(l.Ksc, 0, scBytes, d->stream));
+            HIPCHK(MemsetAsync(l.Vsc, 0, scBytes, d->stream));
+        }
     }
     // Static ownership: slot s owns blocks 1+s*bps .. ; the table indirection stays so a pool allocator can replace it.
     std::vector<int> tab((size_t)slots * m->blocks_per_slot);
@@ -467,8 +482,12 @@ extern "C" int rd_kv_upload(rd_model *m, int slot, int layer, int base, int n, c
     RC(d->h2d(K.p, keys, sizeof(float) * (size_t)n * kvd));
     RC(d->h2d(V.p, vals, sizeof(float) * (size_t)n * kvd));
     LayerW &l = m->layers[(size_t)layer];
-    RC(d->launch(d->k.kv_store, (unsigned)n, 1, 1, (unsigned)kvd, (const float *)K.p, (const float *)V.p, l.Kp, l.Vp,
-                 (const int *)(m->tables + (size_t)slot * m->blocks_per_slot), base, c.n_kv_heads, c.head_dim));
+    if (m->kv_type == RD_KV_I8)
+        RC(d->launch(d->k.kv_store_i8, (unsigned)n, (unsigned)c.n_kv_heads, 1, 64, (const float *)K.p, (const float *)V.p, (signed char *)l.Kp,
+                     (signed char *)l.Vp, l.Ksc, l.Vsc, (const int *)(m->tables + (size_t)slot * m->blocks_per_slot), base, c.n_kv_heads, c.head_dim));
+    else
+        RC(d->launch(d->k.kv_store, (unsigned)n, 1, 1, (unsigned)kvd, (const float *)K.p, (const float *)V.p, l.Kp, l.Vp,
+                     (const int *)(m->tables + (size_t)slot * m->blocks_per_slot), base, c.n_kv_heads, c.head_dim));
     RC(d->sync());
     m->slot_len[(size_t)slot] = std::max(m->slot_len[(size_t)slot], base + n);
     return RD_OK;
@@ -699,13 +718,24 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
         }
         {
             Scope s(m, KC_ROPE_STORE);
-            RC(d->launch(d->k.qkv_rope_store, (unsigned)(nH + 2 * nKV), (unsigned)B, 1, (unsigned)(HD / 2), (const float *)m->P, plan.splits, m->qbuf,
+            if (m->kv_type == RD_KV_I8)
+                RC(d->launch(d->k.qkv_rope_store_i8, (unsigned)(nH + 2 * nKV), (unsigned)B, 1, (unsigned)(HD / 2), (const float *)m->P, plan.splits, m->qbuf,
+                             (signed char *)l.Kp, (signed char *)l.Vp, l.Ksc, l.Vsc, (const int *)m->tables, m->blocks_per_slot, (const int *)m->rowSlot,
+                             (const int *)m->rowPos, (const double *)m->inv_freq_dev, (const float *)l.q_norm, (const float *)l.k_norm, c.rms_eps, nH, nKV,
+                             HD));
+            else
+                RC(d->launch(d->k.qkv_rope_store, (unsigned)(nH + 2 * nKV), (unsigned)B, 1, (unsigned)(HD / 2), (const float *)m->P, plan.splits, m->qbuf,
                          l.Kp, l.Vp, (const int *)m->tables, m->blocks_per_slot, (const int *)m->rowSlot, (const int *)m->rowPos,
                          (const double *)m->inv_freq_dev, (const float *)l.q_norm, (const float *)l.k_norm, c.rms_eps, nH, nKV, HD));
         }
         {
             Scope s(m, KC_ATTN_PARTIAL);
-            RC(d->launch(d->k.attn_partial, (unsigned)items.size(), 1, 1, 64, (const void *)m->items, (const int *)m->rowLen, (const int *)m->rowSlot,
+            if (m->kv_type == RD_KV_I8)
+                RC(d->launch(d->k.attn_partial_i8, (unsigned)items.size(), 1, 1, 64, (const void *)m->items, (const int *)m->rowLen, (const int *)m->rowSlot,
+                             (const int *)m->tables, m->blocks_per_slot, (const signed char *)l.Kp, (const signed char *)l.Vp, (const float *)l.Ksc,
+                             (const float *)l.Vsc, (const float *)m->qbuf, m->part, nH, nKV, HD, c.attn_scale, c.attn_softcap));
+            else
+                RC(d->launch(d->k.attn_partial, (unsigned)items.size(), 1, 1, 64, (const void *)m->items, (const int *)m->rowLen, (const int *)m->rowSlot,
                          (const int *)m->tables, m->blocks_per_slot, (const uint16_t *)l.Kp, (const uint16_t *)l.Vp, (const float *)m->qbuf, m->part,
                          nH, nKV, HD, c.attn_scale, c.attn_softcap));
         }

@@ -25,7 +25,8 @@ struct LayerW {
     void *exp_gateup = nullptr;        // [nE] stacked tiled W4A8, each 2*expert_inter rows x hidden
     void *exp_down = nullptr;          // [nE] stacked tiled W4A8, each hidden rows x expert_inter
     std::vector<char> exp_have;        // [nE*3]
-    uint16_t *Kp = nullptr, *Vp = nullptr; // KV pool of this layer
+    uint16_t *Kp = nullptr, *Vp = nullptr; // KV pool of this layer (binary16, or int8 codes when the model's kv_type says so)
+    float *Ksc = nullptr, *Vsc = nullptr;  // int8 pool: one scale per (block, kv head, position)
 };
 
 struct StepTimer {
@@ -65,6 +66,7 @@ struct rd_model {
         int *host_ids = nullptr;     // pinned [DEPTH]
         hipEvent_t ev[DEPTH] = {};
     } chain;
+    int kv_type = 0; // RD_KV_F16 or RD_KV_I8
     static constexpr int META_HDR = 96 + 32 * 6; // row slot, position, length (32 each) and the rows' draw records (6 ints each)
     int *rowDraw = nullptr;               // inside meta
     const rd_draw *step_draws = nullptr;  // set by the entry point for the one step it runs; null = plain argmax for every row

@@ -298,8 +298,8 @@ extern "C" int rd_moe_route(rd_device *d, const float *logits, int T, int nE, in
 }
 
 // ---- ragged attention over a temporary paged pool (kernel-level entry point) ----
-extern "C" int rd_attn_ragged(rd_device *d, int n_seq, const int *len, const int64_t *off, const float *k, const float *v, const float *q,
-                              int n_h, int n_kv, int hd, float scale, float softcap, float *out) {
+static int attn_ragged_typed(rd_device *d, int kv_type, int n_seq, const int *len, const int64_t *off, const float *k, const float *v, const float *q,
+                             int n_h, int n_kv, int hd, float scale, float softcap, float *out) {
     if (!d || !len || !off || !k || !v || !q || !out || n_seq <= 0) return RD_ERR_ARG;
     if (n_kv <= 0 || n_h % n_kv || n_h / n_kv > 16 || (hd != 64 && hd != 128)) {
         rd_set_error("rd_attn_ragged declines: head_dim must be 64 or 128 and the GQA group <= 16");
@@ -326,12 +326,19 @@ extern "C" int rd_attn_ragged(rd_device *d, int n_seq, const int *len, const int
         for (int i = 0; i < n_seq; i++)
             for (int b = 0; b < (len[i] + 63) / 64; b++, idx++) tab[(size_t)i * maxBlocks + b] = 1 + (int)((idx * stride) % nb);
     }
-    size_t poolBytes = (size_t)(totalBlocks + 1) * n_kv * 64 * hd * 2;
-    DevBuf Kp(d), Vp(d), T(d), Q(d), O(d), L(d), S(d), It(d), St(d), Part(d);
+    const bool i8 = kv_type == RD_KV_I8;
+    size_t poolBytes = (size_t)(totalBlocks + 1) * n_kv * 64 * hd * (i8 ? 1 : 2), scBytes = (size_t)(totalBlocks + 1) * n_kv * 64 * sizeof(float);
+    DevBuf Kp(d), Vp(d), Ksc(d), Vsc(d), T(d), Q(d), O(d), L(d), S(d), It(d), St(d), Part(d);
     RC(Kp.alloc(poolBytes));
     RC(Vp.alloc(poolBytes));
     HIPCHK(MemsetAsync(Kp.p, 0, poolBytes, d->stream));
     HIPCHK(MemsetAsync(Vp.p, 0, poolBytes, d->stream));
+    if (i8) {
+        RC(Ksc.alloc(scBytes));
+        RC(Vsc.alloc(scBytes));
+        HIPCHK(MemsetAsync(Ksc.p, 0, scBytes, d->stream));
+        HIPCHK(MemsetAsync(Vsc.p, 0, scBytes, d->stream));
+    }
     RC(T.alloc(sizeof(int) * tab.size()));
     RC(d->h2d(T.p, tab.data(), sizeof(int) * tab.size()));
     {
@@ -344,8 +351,12 @@ extern "C" int rd_attn_ragged(rd_device *d, int n_seq, const int *len, const int
                 int n = std::min(chunkRows, len[i] - base);
                 RC(d->h2d(Kc.p, k + ((size_t)off[i] + base) * kvd, sizeof(float) * (size_t)n * kvd));
                 RC(d->h2d(Vc.p, v + ((size_t)off[i] + base) * kvd, sizeof(float) * (size_t)n * kvd));
-                RC(d->launch(d->k.kv_store, (unsigned)n, 1, 1, (unsigned)kvd, (const float *)Kc.p, (const float *)Vc.p, (uint16_t *)Kp.p,
-                             (uint16_t *)Vp.p, (const int *)((const int *)T.p + (size_t)i * maxBlocks), base, n_kv, hd));
+                if (i8)
+                    RC(d->launch(d->k.kv_store_i8, (unsigned)n, (unsigned)n_kv, 1, 64, (const float *)Kc.p, (const float *)Vc.p, (signed char *)Kp.p,
+                                 (signed char *)Vp.p, Ksc.as<float>(), Vsc.as<float>(), (const int *)((const int *)T.p + (size_t)i * maxBlocks), base, n_kv, hd));
+                else
+                    RC(d->launch(d->k.kv_store, (unsigned)n, 1, 1, (unsigned)kvd, (const float *)Kc.p, (const float *)Vc.p, (uint16_t *)Kp.p,
+                                 (uint16_t *)Vp.p, (const int *)((const int *)T.p + (size_t)i * maxBlocks), base, n_kv, hd));
                 RC(d->sync());
             }
     }
@@ -368,11 +379,24 @@ extern "C" int rd_attn_ragged(rd_device *d, int n_seq, const int *len, const int
         RC(d->h2d(S2.p, slots.data(), sizeof(int) * (size_t)rows));
         RC(d->h2d(I2.p, items.data(), sizeof(AttnItemH) * items.size()));
         RC(d->h2d(St2.p, start.data(), sizeof(int) * start.size()));
-        RC(d->launch(d->k.attn_partial, (unsigned)items.size(), 1, 1, 64, (const void *)I2.p, (const int *)L2.p, (const int *)S2.p, (const int *)T.p,
-                     maxBlocks, (const uint16_t *)Kp.p, (const uint16_t *)Vp.p, (const float *)Q2.p, P2.as<float>(), n_h, n_kv, hd, scale, softcap));
+        if (i8)
+            RC(d->launch(d->k.attn_partial_i8, (unsigned)items.size(), 1, 1, 64, (const void *)I2.p, (const int *)L2.p, (const int *)S2.p, (const int *)T.p,
+                         maxBlocks, (const signed char *)Kp.p, (const signed char *)Vp.p, (const float *)Ksc.p, (const float *)Vsc.p, (const float *)Q2.p,
+                         P2.as<float>(), n_h, n_kv, hd, scale, softcap));
+        else
+            RC(d->launch(d->k.attn_partial, (unsigned)items.size(), 1, 1, 64, (const void *)I2.p, (const int *)L2.p, (const int *)S2.p, (const int *)T.p,
+                         maxBlocks, (const uint16_t *)Kp.p, (const uint16_t *)Vp.p, (const float *)Q2.p, P2.as<float>(), n_h, n_kv, hd, scale, softcap));
         RC(d->launch(d->k.attn_combine, (unsigned)n_h, (unsigned)rows, 1, (unsigned)(ATTN_PIECES * hd / 4), (const float *)P2.p, (const int *)St2.p, O2.as<float>(), n_h,
                      n_kv, hd));
         RC(d->d2h(out + (size_t)r0 * qd, O2.p, sizeof(float) * (size_t)rows * qd));
     }
     return RD_OK;
+}
+extern "C" int rd_attn_ragged(rd_device *d, int n_seq, const int *len, const int64_t *off, const float *k, const float *v, const float *q,
+                              int n_h, int n_kv, int hd, float scale, float softcap, float *out) {
+    return attn_ragged_typed(d, RD_KV_F16, n_seq, len, off, k, v, q, n_h, n_kv, hd, scale, softcap, out);
+}
+extern "C" int rd_attn_ragged_i8(rd_device *d, int n_seq, const int *len, const int64_t *off, const float *k, const float *v, const float *q,
+                                 int n_h, int n_kv, int hd, float scale, float softcap, float *out) {
+    return attn_ragged_typed(d, RD_KV_I8, n_seq, len, off, k, v, q, n_h, n_kv, hd, scale, softcap, out);
 }

@@ -6,6 +6,14 @@
 //   K region: [key tile of 16 (4)][d step c (HD/32)][lane = dq*16 + key][8 halves],   d = dq*(HD/4) + c*8 + i
 //   V region: [key tile of 32 (2)][d column tile ct (HD/16)][lane = kq*16 + dcol][8 halves], key = kq*8 + i, d = ct*16 + dcol
 // Values are binary16 narrowed with round-half-up, as goinfer's f16 KV cache narrows them (decoder/kvcache.go:21-40).
+//
+// The int8 cache (goinfer's kvI8: decoder/kvcache.go:43-52 quantizeHeads, backend/cuda/kv8_store.cu, kvtype.cuh:48-73) holds per
+// (position, kv head) HD codes and one f32 scale for K and one for V: scale = maxabs/127, code = round-half-away(x/scale)
+// clamped to +-127, an all-zero head scale 1; a reader takes code * scale. The pool stores code + 128 as an unsigned byte. Its regions are the same fragment orders in bytes,
+// two 8-byte fragments per 16-byte lane slot so that a wave load stays 1 KB:
+//   K region: [key tile of 16 (4)][d step pair (HD/64)][lane = dq*16 + key][2 x 8 bytes]   (steps 2cp, 2cp+1)
+//   V region: [key tile of 32 (2)][d column tile pair (HD/32)][lane = kq*16 + dcol][2 x 8 bytes]   (tiles 2cp, 2cp+1)
+// and the scales sit beside them as [block][kv head][64 positions] f32.
 #pragma once
 #include "common.h"
 
@@ -16,6 +24,52 @@ template <int HD> __device__ __forceinline__ int k_elem_index(int p, int d) {
 template <int HD> __device__ __forceinline__ int v_elem_index(int p, int d) {
     int kt = p >> 5, pk = p & 31, kq = pk >> 3, i = pk & 7, ct = d >> 4, dcol = d & 15;
     return (((kt * (HD / 16) + ct) * 64 + kq * 16 + dcol) << 3) + i;
+}
+
+template <int HD> __device__ __forceinline__ int k8_elem_index(int p, int d) {
+    int kt = p >> 4, key = p & 15, dq = d / (HD / 4), rem = d % (HD / 4), c = rem >> 3, i = rem & 7;
+    return (((kt * (HD / 64) + (c >> 1)) * 64 + dq * 16 + key) << 4) + (c & 1) * 8 + i;
+}
+template <int HD> __device__ __forceinline__ int v8_elem_index(int p, int d) {
+    int kt = p >> 5, pk = p & 31, kq = pk >> 3, i = pk & 7, ct = d >> 4, dcol = d & 15;
+    return (((kt * (HD / 32) + (ct >> 1)) * 64 + kq * 16 + dcol) << 4) + (ct & 1) * 8 + i;
+}
+__device__ __forceinline__ int k8_index(int HD, int p, int d) { return HD == 128 ? k8_elem_index<128>(p, d) : k8_elem_index<64>(p, d); }
+__device__ __forceinline__ int v8_index(int HD, int p, int d) { return HD == 128 ? v8_elem_index<128>(p, d) : v8_elem_index<64>(p, d); }
+
+// linalg.QuantizeRowInt8's rule for one value, given the head's scale (backend/cuda/kv8_store.cu:27-35)
+// The pool keeps code + 128 as an unsigned byte: under a 0x64 high byte that is the f16 value 1024 + 128 + code with no further work.
+__device__ __forceinline__ unsigned char kv8_code(float x, float inv) {
+    float r = roundf(__fmul_rn(x, inv)); // round half away from zero
+    r = fminf(127.f, fmaxf(-127.f, r));
+    return (unsigned char)((int)r + 128);
+}
+// scale and its reciprocal from the head's largest magnitude: maxabs/127, or 1 for an all-zero head (then every code is 0)
+__device__ __forceinline__ float kv8_scale(float maxabs, float *inv) {
+    float sc = 1.f;
+    *inv = 0.f;
+    if (maxabs != 0.f) sc = __fdiv_rn(maxabs, 127.f), *inv = __fdiv_rn(1.f, sc);
+    return sc;
+}
+
+// Host-provided rows into the int8 cache: grid (n, nKV), block 64; lane l quantizes elements l, l+64 of the head.
+extern "C" __global__ __launch_bounds__(64) void rd_k_kv_store_i8(const float *__restrict__ k, const float *__restrict__ v, signed char *__restrict__ Kp,
+                                                                  signed char *__restrict__ Vp, float *__restrict__ Ksc, float *__restrict__ Vsc,
+                                                                  const int *__restrict__ table, int base, int nKV, int HD) {
+    const int i = blockIdx.x, kvh = blockIdx.y, lane = threadIdx.x;
+    const int pos = base + i, blk = table[pos >> 6], p = pos & 63;
+    const size_t region = ((size_t)blk * nKV + kvh) * 64 * HD, srow = ((size_t)blk * nKV + kvh) * 64 + p;
+    for (int which = 0; which < 2; which++) {
+        const float *src = (which ? v : k) + (size_t)i * nKV * HD + (size_t)kvh * HD;
+        float x0 = lane < HD ? src[lane] : 0.f, x1 = lane + 64 < HD ? src[lane + 64] : 0.f;
+        float ma = fmaxf(fabsf(x0), fabsf(x1));
+        for (int o = 32; o > 0; o >>= 1) ma = fmaxf(ma, __shfl_xor(ma, o, 64));
+        float inv, sc = kv8_scale(ma, &inv);
+        unsigned char *dst = (unsigned char *)(which ? Vp : Kp) + region;
+        if (lane < HD) dst[which ? v8_index(HD, p, lane) : k8_index(HD, p, lane)] = kv8_code(x0, inv);
+        if (lane + 64 < HD) dst[which ? v8_index(HD, p, lane + 64) : k8_index(HD, p, lane + 64)] = kv8_code(x1, inv);
+        if (lane == 0) (which ? Vsc : Ksc)[srow] = sc;
+    }
 }
 
 __device__ __forceinline__ void kv_store_elem(uint16_t *__restrict__ Kp, uint16_t *__restrict__ Vp, int HD, size_t region, int p, int d, float kv,
@@ -40,8 +94,10 @@ extern "C" __global__ void rd_k_kv_store(const float *__restrict__ k, const floa
 // After the q|k|v GEMM: reduce its split-K partials, optional per-head RMSNorm of q and k (Qwen3, decoder/program_cpu.go:351-364),
 // NeoX RoPE with f64 angles (decoder/rope.go:28-64), q -> f32 buffer, k,v -> this position of the row's sequence in the pool.
 // Grid (nH + 2*nKV, rows), block HD/2 threads... one thread per rotation pair.  P: [splits][32][(nH+2nKV)*HD].
-extern "C" __global__ void rd_k_qkv_rope_store(const float *__restrict__ P, int splits, float *__restrict__ q, uint16_t *__restrict__ Kp,
-                                               uint16_t *__restrict__ Vp, const int *__restrict__ tables, int tabStride,
+template <bool I8>
+__device__ __forceinline__ void qkv_rope_store_body(const float *__restrict__ P, int splits, float *__restrict__ q, void *__restrict__ KpV,
+                                               void *__restrict__ VpV, float *__restrict__ Ksc, float *__restrict__ Vsc,
+                                               const int *__restrict__ tables, int tabStride,
                                                const int *__restrict__ rowSlot, const int *__restrict__ rowPos, const double *__restrict__ invFreq,
                                                const float *__restrict__ qnorm, const float *__restrict__ knorm, float eps, int nH, int nKV, int HD) {
     int head = blockIdx.x, m = blockIdx.y, t = threadIdx.x, half = HD / 2; // one wave: half <= 64
@@ -86,7 +142,18 @@ extern "C" __global__ void rd_k_qkv_rope_store(const float *__restrict__ P, int 
     int kvh = isK ? head - nH : head - nH - nKV;
     int blk = blkPre, p = pos & 63;
     size_t region = ((size_t)blk * nKV + kvh) * 64 * HD;
-    uint16_t *dstp = isK ? Kp : Vp;
+    if constexpr (I8) {
+        // one scale per (position, kv head): the head's largest magnitude over all its rotation pairs (block = one head)
+        float ma = fmaxf(fabsf(o1), fabsf(o2));
+        for (int o = half >> 1; o > 0; o >>= 1) ma = fmaxf(ma, __shfl_xor(ma, o, 64));
+        float inv, sc = kv8_scale(ma, &inv);
+        unsigned char *dst8 = (unsigned char *)(isK ? KpV : VpV) + region;
+        dst8[isK ? k8_index(HD, p, t) : v8_index(HD, p, t)] = kv8_code(o1, inv);
+        dst8[isK ? k8_index(HD, p, t + half) : v8_index(HD, p, t + half)] = kv8_code(o2, inv);
+        if (t == 0) (isK ? Ksc : Vsc)[((size_t)blk * nKV + kvh) * 64 + p] = sc;
+        return;
+    }
+    uint16_t *dstp = (uint16_t *)(isK ? KpV : VpV);
     for (int e = 0; e < 2; e++) {
         int d = e ? t + half : t;
         int idx = isK ? (HD == 128 ? k_elem_index<128>(p, d) : k_elem_index<64>(p, d)) : (HD == 128 ? v_elem_index<128>(p, d) : v_elem_index<64>(p, d));
@@ -94,7 +161,30 @@ extern "C" __global__ void rd_k_qkv_rope_store(const float *__restrict__ P, int 
     }
 }
 
+extern "C" __global__ void rd_k_qkv_rope_store(const float *__restrict__ P, int splits, float *__restrict__ q, uint16_t *__restrict__ Kp,
+                                               uint16_t *__restrict__ Vp, const int *__restrict__ tables, int tabStride,
+                                               const int *__restrict__ rowSlot, const int *__restrict__ rowPos, const double *__restrict__ invFreq,
+                                               const float *__restrict__ qnorm, const float *__restrict__ knorm, float eps, int nH, int nKV, int HD) {
+    qkv_rope_store_body<false>(P, splits, q, Kp, Vp, nullptr, nullptr, tables, tabStride, rowSlot, rowPos, invFreq, qnorm, knorm, eps, nH, nKV, HD);
+}
+// The same into the int8 cache: the K or V head is quantized with its own scale after RoPE (backend/cuda/kv8_store.cu).
+extern "C" __global__ void rd_k_qkv_rope_store_i8(const float *__restrict__ P, int splits, float *__restrict__ q, signed char *__restrict__ Kp,
+                                                  signed char *__restrict__ Vp, float *__restrict__ Ksc, float *__restrict__ Vsc,
+                                                  const int *__restrict__ tables, int tabStride, const int *__restrict__ rowSlot,
+                                                  const int *__restrict__ rowPos, const double *__restrict__ invFreq, const float *__restrict__ qnorm,
+                                                  const float *__restrict__ knorm, float eps, int nH, int nKV, int HD) {
+    qkv_rope_store_body<true>(P, splits, q, Kp, Vp, Ksc, Vsc, tables, tabStride, rowSlot, rowPos, invFreq, qnorm, knorm, eps, nH, nKV, HD);
+}
+
 typedef float float4v __attribute__((ext_vector_type(4)));
+
+// tanh(x) = 1 - 2 / (e^(2x) + 1), with the hardware exponential and reciprocal: absolute error below 1e-6 over the whole
+// range (the argument is clamped where the result is 1 to the last bit anyway), far inside the attention bar.
+__device__ __forceinline__ float fast_tanh(float x) {
+    x = fminf(12.f, fmaxf(-12.f, x));
+    float t = __expf(2.f * x);
+    return 1.f - 2.f * __frcp_rn(t + 1.f);
+}
 
 __device__ __forceinline__ float ld_part(const float *p) { return *p; }
 
@@ -105,12 +195,32 @@ struct AttnItem {
 // One wave per item: online-softmax attention of the G query heads of one kv head over blocks [b0,b1) of one sequence.
 // Scores: S = Q.K^T on 16x16x32 f16 MFMA with Q split into hi+lo halves (K is exactly f16), so dots carry f32 accuracy.
 // P.V likewise with P split hi+lo. Writes unnormalised (O, m, l) per head: part[item][G][HD+2].
-template <int HD>
+// I8: K and V are int8 codes with one f32 scale per (key, kv head). A code is exactly an f16, so the same MFMAs run on the
+// codes; the key's K scale multiplies its finished scores and its V scale multiplies its probabilities before the P.V product:
+// sum_d q_d (c_d s) = s sum_d q_d c_d and sum_key p (c s) = sum_key (p s) c, which is the dequantized arithmetic up to f32 rounding.
+// eight stored bytes (code + 128) -> eight f16 codes, exactly: under a 0x64 high byte a byte u is 1024 + u; minus 1152.
+__device__ __forceinline__ half8_t kv8_to_half8(uint32_t w0, uint32_t w1) {
+    const half2_t off = {(half_t)(-1152.f), (half_t)(-1152.f)};
+    uint32_t u0 = __builtin_amdgcn_perm(0x64646464u, w0, 0x04010400u), u1 = __builtin_amdgcn_perm(0x64646464u, w0, 0x04030402u);
+    uint32_t u2 = __builtin_amdgcn_perm(0x64646464u, w1, 0x04010400u), u3 = __builtin_amdgcn_perm(0x64646464u, w1, 0x04030402u);
+    half2_t v0, v1, v2, v3;
+    __builtin_memcpy(&v0, &u0, 4);
+    __builtin_memcpy(&v1, &u1, 4);
+    __builtin_memcpy(&v2, &u2, 4);
+    __builtin_memcpy(&v3, &u3, 4);
+    v0 += off, v1 += off, v2 += off, v3 += off;
+    return (half8_t){v0.x, v0.y, v1.x, v1.y, v2.x, v2.y, v3.x, v3.y};
+}
+
+template <int HD, bool I8>
 __device__ __forceinline__ void attn_partial_body(const AttnItem *__restrict__ items, const int *__restrict__ rowLen, const int *__restrict__ rowSlot,
-                                                  const int *__restrict__ tables, int tabStride, const uint16_t *__restrict__ Kp,
-                                                  const uint16_t *__restrict__ Vp, const float *__restrict__ q, float *__restrict__ part, int nH,
-                                                  int nKV, float scale, float softcap, half_t *pbuf) {
+                                                  const int *__restrict__ tables, int tabStride, const void *__restrict__ KpV,
+                                                  const void *__restrict__ VpV, const float *__restrict__ Ksc, const float *__restrict__ Vsc,
+                                                  const float *__restrict__ q, float *__restrict__ part, int nH, int nKV, float scale,
+                                                  float softcap, half_t *pbuf) {
     constexpr int NC = HD / 32, NCT = HD / 16;
+    constexpr int KL = I8 ? NC / 2 : NC, VL = I8 ? NCT / 2 : NCT; // 16-byte loads per key tile of K, per 32 keys of V
+    constexpr int ELEM = I8 ? 1 : 2;
     const AttnItem it = items[blockIdx.x];
     const int lane = threadIdx.x, l16 = lane & 15, lg = lane >> 4;
     const int G = nH / nKV, len = rowLen[it.row];
@@ -135,23 +245,30 @@ __device__ __forceinline__ void attn_partial_body(const AttnItem *__restrict__ i
     float mrun[4], lrun[4];
 #pragma unroll
     for (int r = 0; r < 4; r++) mrun[r] = -INFINITY, lrun[r] = 0.f;
+    const float rcap = softcap != 0.f ? 1.f / softcap : 0.f;
 
-    const size_t regionHalves = (size_t)64 * HD;
+    const size_t regionBytes = (size_t)64 * HD * ELEM;
     for (int b = it.b0; b < it.b1; b++) {
         const int blk = tab[b];
-        const uint4_t *Kr = (const uint4_t *)(Kp + ((size_t)blk * nKV + it.kvh) * regionHalves);
-        const uint4_t *Vr = (const uint4_t *)(Vp + ((size_t)blk * nKV + it.kvh) * regionHalves);
+        const uint4_t *Kr = (const uint4_t *)((const char *)KpV + ((size_t)blk * nKV + it.kvh) * regionBytes);
+        const uint4_t *Vr = (const uint4_t *)((const char *)VpV + ((size_t)blk * nKV + it.kvh) * regionBytes);
+        const size_t srow = ((size_t)blk * nKV + it.kvh) * 64;
 #pragma unroll
         for (int u = 0; u < 2; u++) {
             const int key0 = b * 64 + u * 32;
             if (key0 >= len) break;
-            uint4_t kf[2][NC], vf[NCT];
+            uint4_t kf[2][KL], vf[VL];
 #pragma unroll
             for (int t = 0; t < 2; t++)
 #pragma unroll
-                for (int c = 0; c < NC; c++) kf[t][c] = __builtin_nontemporal_load(Kr + ((u * 2 + t) * NC + c) * 64 + lane);
+                for (int c = 0; c < KL; c++) kf[t][c] = __builtin_nontemporal_load(Kr + ((u * 2 + t) * KL + c) * 64 + lane);
 #pragma unroll
-            for (int ct = 0; ct < NCT; ct++) vf[ct] = __builtin_nontemporal_load(Vr + (u * NCT + ct) * 64 + lane);
+            for (int ct = 0; ct < VL; ct++) vf[ct] = __builtin_nontemporal_load(Vr + (u * VL + ct) * 64 + lane);
+            float ks[2] = {1.f, 1.f}, vs[2] = {1.f, 1.f}; // this lane's keys t*16 + l16
+            if constexpr (I8) {
+#pragma unroll
+                for (int t = 0; t < 2; t++) ks[t] = Ksc[srow + u * 32 + t * 16 + l16], vs[t] = Vsc[srow + u * 32 + t * 16 + l16];
+            }
             float4v S[2];
 #pragma unroll
             for (int t = 0; t < 2; t++) {
@@ -159,7 +276,10 @@ __device__ __forceinline__ void attn_partial_body(const AttnItem *__restrict__ i
 #pragma unroll
                 for (int c = 0; c < NC; c++) {
                     half8_t kb;
-                    __builtin_memcpy(&kb, &kf[t][c], 16);
+                    if constexpr (I8)
+                        kb = kv8_to_half8(kf[t][c >> 1][(c & 1) * 2], kf[t][c >> 1][(c & 1) * 2 + 1]);
+                    else
+                        __builtin_memcpy(&kb, &kf[t][c], 16);
                     S[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(qhi[c], kb, S[t], 0, 0, 0);
                     S[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(qlo[c], kb, S[t], 0, 0, 0);
                 }
@@ -172,12 +292,13 @@ __device__ __forceinline__ void attn_partial_body(const AttnItem *__restrict__ i
 #pragma unroll
                 for (int t = 0; t < 2; t++) {
                     float s = S[t][r] * scale;
-                    if (softcap != 0.f) s = softcap * tanhf(s / softcap);
+                    if constexpr (I8) s = S[t][r] * ks[t] * scale;
+                    if (softcap != 0.f) s = softcap * fast_tanh(s * rcap);
                     if (key0 + t * 16 + l16 >= len) s = -INFINITY;
                     S[t][r] = s;
                     mx[r] = fmaxf(mx[r], s);
                 }
-                for (int o = 8; o > 0; o >>= 1) mx[r] = fmaxf(mx[r], __shfl_xor(mx[r], o, 64));
+                mx[r] = group_max16(mx[r]); // the 16 key lanes of this head row are one DPP row
             }
             float alpha[4];
 #pragma unroll
@@ -190,6 +311,7 @@ __device__ __forceinline__ void attn_partial_body(const AttnItem *__restrict__ i
                 for (int t = 0; t < 2; t++) {
                     float p = __expf(S[t][r] - mn);
                     ps += p;
+                    if constexpr (I8) p = (key0 + t * 16 + l16 < len) ? p * vs[t] : 0.f; // a key past the end has no scale to trust
                     half_t hi = (half_t)p;
                     int idx = (4 * lg + r) * 32 + t * 16 + l16;
                     pbuf[idx] = hi;
@@ -197,10 +319,14 @@ __device__ __forceinline__ void attn_partial_body(const AttnItem *__restrict__ i
                 }
                 lrun[r] = lrun[r] * alpha[r] + ps;
             }
+            // Rescale the running output only when some row's maximum moved: past the first keys of a sequence it rarely does,
+            // and a factor of exactly 1 changes nothing.
+            if (__builtin_amdgcn_ballot_w64(alpha[0] != 1.f || alpha[1] != 1.f || alpha[2] != 1.f || alpha[3] != 1.f) != 0) {
 #pragma unroll
-            for (int ct = 0; ct < NCT; ct++)
+                for (int ct = 0; ct < NCT; ct++)
 #pragma unroll
-                for (int r = 0; r < 4; r++) O[ct][r] *= alpha[r];
+                    for (int r = 0; r < 4; r++) O[ct][r] *= alpha[r];
+            }
             __syncthreads();
             half8_t phi, plo;
             {
@@ -212,7 +338,10 @@ __device__ __forceinline__ void attn_partial_body(const AttnItem *__restrict__ i
 #pragma unroll
             for (int ct = 0; ct < NCT; ct++) {
                 half8_t vb;
-                __builtin_memcpy(&vb, &vf[ct], 16);
+                if constexpr (I8)
+                    vb = kv8_to_half8(vf[ct >> 1][(ct & 1) * 2], vf[ct >> 1][(ct & 1) * 2 + 1]);
+                else
+                    __builtin_memcpy(&vb, &vf[ct], 16);
                 O[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(phi, vb, O[ct], 0, 0, 0);
                 O[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(plo, vb, O[ct], 0, 0, 0);
             }
@@ -239,9 +368,23 @@ extern "C" __global__ __launch_bounds__(64) void rd_k_attn_partial(const AttnIte
                                                                    float scale, float softcap) {
     __shared__ half_t pbuf[1024];
     if (HD == 128)
-        attn_partial_body<128>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, q, part, nH, nKV, scale, softcap, pbuf);
+        attn_partial_body<128, false>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, pbuf);
     else
-        attn_partial_body<64>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, q, part, nH, nKV, scale, softcap, pbuf);
+        attn_partial_body<64, false>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, pbuf);
+}
+
+// The same over the int8 cache: half the key/value bytes per launch.
+extern "C" __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void rd_k_attn_partial_i8(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
+                                                                      const int *__restrict__ rowSlot, const int *__restrict__ tables, int tabStride,
+                                                                      const signed char *__restrict__ Kp, const signed char *__restrict__ Vp,
+                                                                      const float *__restrict__ Ksc, const float *__restrict__ Vsc,
+                                                                      const float *__restrict__ q, float *__restrict__ part, int nH, int nKV, int HD,
+                                                                      float scale, float softcap) {
+    __shared__ half_t pbuf[1024];
+    if (HD == 128)
+        attn_partial_body<128, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, Ksc, Vsc, q, part, nH, nKV, scale, softcap, pbuf);
+    else
+        attn_partial_body<64, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, Ksc, Vsc, q, part, nH, nKV, scale, softcap, pbuf);
 }
 
 // Merge the partials of one (row, query head) in ascending item order (deterministic):

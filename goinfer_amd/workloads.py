@@ -47,15 +47,16 @@ def expert_bytes(cfg):
     return 3 * cfg["exp_inter"] * cfg["hidden"] * 0.5625
 
 
-def kv_bytes_per_position(cfg):
-    """f16 K and V of one position over all layers."""
-    return cfg["n_layers"] * 2 * cfg["n_kv"] * cfg["head_dim"] * 2
+def kv_bytes_per_position(cfg, kv="f16"):
+    """K and V of one position over all layers: binary16, or int8 codes plus one f32 scale per kv head."""
+    per_head = cfg["head_dim"] * 2 if kv == "f16" else cfg["head_dim"] + 4
+    return cfg["n_layers"] * 2 * cfg["n_kv"] * per_head
 
 
 class Resident:
     """A synthetic model resident on the device, with its KV slots pre-filled."""
 
-    def __init__(self, dev, cfg, seed=1234, slots=32, ctx_cap=4352, keep_layers=0, progress=None):
+    def __init__(self, dev, cfg, seed=1234, slots=32, ctx_cap=4352, keep_layers=0, progress=None, kv="f16"):
         self.dev, self.cfg = dev, cfg
         H, hd = cfg["hidden"], cfg["head_dim"]
         qd, kvd, V = cfg["n_heads"] * hd, cfg["n_kv"] * hd, cfg["vocab"]
@@ -120,7 +121,7 @@ class Resident:
         self.embed = synth.w8a8_normal(nxt(), V, H, SIGMA)
         m.upload_embedding(*self.embed)
         m.finalize()
-        m.kv_configure(slots, ctx_cap)
+        m.kv_configure(slots, ctx_cap, kv)
         if progress:
             progress("model resident")
 

@@ -99,6 +99,9 @@ int rd_gemm_w4a8(rd_device *d, const uint8_t *nib, const uint16_t *s16, int N, i
  * as the cache does. q: host f32 [n_seq][n_h*hd]; out: host f32 [n_seq][n_h*hd]. softcap 0 = off. */
 int rd_attn_ragged(rd_device *d, int n_seq, const int *len, const int64_t *off, const float *k, const float *v,
                    const float *q, int n_h, int n_kv, int hd, float scale, float softcap, float *out);
+/* The same through the int8 cache (RD_KV_I8 below): k and v are quantized per (position, kv head) as the cache stores them. */
+int rd_attn_ragged_i8(rd_device *d, int n_seq, const int *len, const int64_t *off, const float *k, const float *v,
+                      const float *q, int n_h, int n_kv, int hd, float scale, float softcap, float *out);
 /* MoE routing (decoder/mlp.go:130-184 routeExperts, softmax scoring; backend/cuda/moe.cu:49-104 moe_route):
  * logits host f32 [T][nE]; idx int32 [T][k], wgt f32 [T][k], rank order. */
 int rd_moe_route(rd_device *d, const float *logits, int T, int nE, int k, int norm, int *idx, float *wgt);
@@ -128,6 +131,12 @@ int rd_model_finalize(rd_model *m);
 
 /* ---- KV: resident/subsystems.go:236-251 (KVSlots), resident/forward.go:20-30 (UploadKV, TruncateTo, Reset) ---- */
 int rd_kv_configure(rd_model *m, int slots, int ctx_cap);
+/* The same with the cache's element type: RD_KV_F16 (rd_kv_configure's), or RD_KV_I8 = goinfer's int8 cache (KVQuant "i8":
+ * decoder/kvcache.go:13-20,43-52 quantizeHeads; backend/cuda/kv8_store.cu, kvtype.cuh:48-73): per (position, kv head) head_dim
+ * signed bytes and one f32 scale for K and one for V, scale = maxabs/127, code = round-half-away(x/scale) in [-127, 127], an
+ * all-zero head scale 1; readers take code * scale. Half the KV bytes of the f16 cache per step. */
+enum { RD_KV_F16 = 0, RD_KV_I8 = 1 };
+int rd_kv_configure_typed(rd_model *m, int slots, int ctx_cap, int kv_type);
 /* keys, vals: host f32 [n][n_kv*hd] for positions base..base+n-1 of `slot`, layer `layer` (already RoPE'd) */
 int rd_kv_upload(rd_model *m, int slot, int layer, int base, int n, const float *keys, const float *vals);
 int rd_kv_truncate(rd_model *m, int slot, int pos);
@@ -206,6 +215,8 @@ int rd_bench_kernel(rd_device *d, const char *name, const int64_t *args, int n_a
  * ms_partial[iters] (may be NULL): the flash-decode partial kernels alone. */
 int rd_bench_attn(rd_device *d, int n_seq, const int *len, int n_h, int n_kv, int hd, float scale, float softcap, int warmup, int iters,
                   float *ms_total, float *ms_partial);
+int rd_bench_attn_i8(rd_device *d, int n_seq, const int *len, int n_h, int n_kv, int hd, float scale, float softcap, int warmup, int iters,
+                     float *ms_total, float *ms_partial);
 
 #ifdef __cplusplus
 }

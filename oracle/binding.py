@@ -334,3 +334,12 @@ def gumbel_noise_many(h):
     out = np.empty(h.size, np.float32)
     lib().or_gumbel_noise_many(_p(h), C.c_size_t(h.size), _p(out))
     return out
+
+
+def dequantize_rows_int8(q, scales):
+    q = np.ascontiguousarray(q, dtype=np.int8)
+    scales = f32(scales)
+    rows, cols = q.shape
+    out = np.empty((rows, cols), np.float32)
+    lib().or_dequantize_rows_int8(_p(out), _p(q), _p(scales), rows, cols)
+    return out

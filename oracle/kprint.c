@@ -287,6 +287,30 @@ static void k_quantize_row_int8(sha256 *s, gen *g) {
     }
 }
 
+/* kernelprint.go:1005-1016 (int8Rows): rows x cols random codes, then positive per-row scales */
+static int8_t *int8_rows(gen *g, int rows, int cols, float **sc_out) {
+    int8_t *q = (int8_t *)g_bytes(g, rows * cols);
+    float *sc = (float *)malloc(sizeof(float) * (size_t)rows);
+    for (int i = 0; i < rows; i++) sc[i] = (float)(g_unit(g) * (1.0 / 64)) + (1.0f / 32);
+    *sc_out = sc;
+    return q;
+}
+/* kernelprint.go:366-377 */
+static void k_dequantize_rows_int8(sha256 *s, gen *g) {
+    static const int rowsList[] = {1, 3, 4};
+    for (int ri = 0; ri < 3; ri++)
+        for (int c = 0; c < LEN(quantCols); c++) {
+            int rows = rowsList[ri], cols = quantCols[c];
+            float *sc, *dst = (float *)malloc(sizeof(float) * (size_t)rows * cols);
+            int8_t *q = int8_rows(g, rows, cols, &sc);
+            or_dequantize_rows_int8(dst, q, sc, rows, cols);
+            long t[2] = {rows, cols};
+            s_tag(s, "dq", 2, t);
+            s_f32(s, dst, (size_t)rows * cols);
+            free(q), free(sc), free(dst);
+        }
+}
+
 /* kernelprint.go:495-515 */
 static void k_quantize_act(sha256 *s, gen *g) {
     static const int groups[] = {0, 32}, ks0[] = {1, 7, 17, 33, 100, 256};
@@ -456,6 +480,7 @@ static const kernel suite[] = {
     {"embed.GGUFFile(Q5_K).Tensor", k_gguf_q5k},
     {"embed.GGUFFile(Q6_K).Tensor", k_gguf_q6k},
     {"linalg.QuantizeRowInt8", k_quantize_row_int8},
+    {"linalg.DequantizeRowsInt8Into", k_dequantize_rows_int8},
     {"linalg.QuantizeActQ", k_quantize_act},
     {"linalg.QuantizeGroupInt4Row", k_quantize_group_int4_row},
     {"linalg.QuantizeInt4", k_quantize_int4},

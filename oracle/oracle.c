@@ -136,6 +136,14 @@ void or_dequant_q6k(const uint8_t *blocks, size_t n_blocks, float *out) {
     }
 }
 
+/* ------------------------------------------------------------------ int8 rows back to f32 */
+/* decoder/kvcache.go:54-59 (dequantHeads -> linalg.DequantizeRowsInt8Into), backend/cuda/kvtype.cuh:48-52 (KV_LDS):
+ * dst[r][c] = (float)q[r][c] * scales[r], one f32 product per element. */
+void or_dequantize_rows_int8(float *dst, const int8_t *q, const float *scales, int rows, int cols) {
+    for (int r = 0; r < rows; r++)
+        for (int c = 0; c < cols; c++) dst[(size_t)r * cols + c] = (float)q[(size_t)r * cols + c] * scales[r];
+}
+
 /* ------------------------------------------------------------------ activation quantizers */
 static inline float round_half_away(float x) { return roundf(x); }
 
@@ -766,6 +774,24 @@ void or_cache_free(const or_model *m, or_cache *c) {
     free(c);
 }
 
+/* What the cache holds of one position's K or V row [n_kv][hd]: the row itself (f32 cache), its binary16 narrowing
+ * (decoder/kvcache.go:21-40), or per head the int8 codes times their scale (kvcache.go:43-59 quantizeHeads / dequantHeads;
+ * backend/cuda/kv8_store.cu, kvtype.cuh:48-52). */
+static void kv_narrow_row(const or_model *m, const float *src, float *dst) {
+    int kvDim = m->n_kv * m->head_dim;
+    if (m->kv_f16 == 1) {
+        for (int i = 0; i < kvDim; i++) dst[i] = or_f16_to_f32(or_f32_to_f16(src[i]));
+    } else if (m->kv_f16 == 2) {
+        int8_t q[1024];
+        for (int h = 0; h < m->n_kv; h++) {
+            float sc = or_quantize_row_int8(src + (size_t)h * m->head_dim, m->head_dim, q);
+            or_dequantize_rows_int8(dst + (size_t)h * m->head_dim, q, &sc, 1, m->head_dim);
+        }
+    } else {
+        memcpy(dst, src, sizeof(float) * (size_t)kvDim);
+    }
+}
+
 void or_f16_round_trip(const float *src, float *dst, size_t n) {
 #pragma omp parallel for schedule(static)
     for (size_t i = 0; i < n; i++) dst[i] = or_f16_to_f32(or_f32_to_f16(src[i]));
@@ -775,12 +801,10 @@ int or_cache_upload(const or_model *m, or_cache *c, int layer, int base, int n, 
     size_t kvDim = (size_t)m->n_kv * m->head_dim;
     if (layer < 0 || layer >= m->n_layers || base < 0 || n < 0 || base + n > c->cap) return -1;
     float *kd = c->k[layer] + (size_t)base * kvDim, *vd = c->v[layer] + (size_t)base * kvDim;
-    if (m->kv_f16) {
-        or_f16_round_trip(keys, kd, (size_t)n * kvDim);
-        or_f16_round_trip(vals, vd, (size_t)n * kvDim);
-    } else {
-        memcpy(kd, keys, (size_t)n * kvDim * sizeof(float));
-        memcpy(vd, vals, (size_t)n * kvDim * sizeof(float));
+#pragma omp parallel for schedule(static)
+    for (int i = 0; i < n; i++) {
+        kv_narrow_row(m, keys + (size_t)i * kvDim, kd + (size_t)i * kvDim);
+        kv_narrow_row(m, vals + (size_t)i * kvDim, vd + (size_t)i * kvDim);
     }
     if (base + n > c->pos) c->pos = base + n;
     return 0;
@@ -870,15 +894,8 @@ int or_decode_multi_step_traced(const or_model *m, int B, const float *emb, or_c
             or_rope(qb, nH, hd, c->pos, m->inv_freq, hd / 2, 1.0);
             or_rope(kb, nKV, hd, c->pos, m->inv_freq, hd / 2, 1.0);
             float *kr = c->k[l] + (size_t)c->pos * kvDim, *vr = c->v[l] + (size_t)c->pos * kvDim;
-            if (m->kv_f16) { /* decoder/kvcache.go:21-40: stored as binary16 (round-half-up), widened on read */
-                for (int i = 0; i < kvDim; i++) {
-                    kr[i] = or_f16_to_f32(or_f32_to_f16(kb[i]));
-                    vr[i] = or_f16_to_f32(or_f32_to_f16(vb[i]));
-                }
-            } else {
-                memcpy(kr, kb, sizeof(float) * (size_t)kvDim);
-                memcpy(vr, vb, sizeof(float) * (size_t)kvDim);
-            }
+            kv_narrow_row(m, kb, kr); /* as the cache stores it: f32, binary16 or int8 per head */
+            kv_narrow_row(m, vb, vr);
             or_attend(qb, ctx + (size_t)b * qDim, c->k[l], c->v[l], c->pos + 1, 0, nH, nKV, hd, m->attn_scale, m->softcap);
         }
         or_matmul(&lw->o, ctx, B, att);

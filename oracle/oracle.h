@@ -16,6 +16,8 @@
  *   or_dequant_q5k / or_dequant_q6k      pinned: embed.GGUFFile(Q5_K).Tensor, embed.GGUFFile(Q6_K).Tensor fingerprints
  *   or_quantize_row_int8                 pinned: linalg.QuantizeRowInt8 fingerprint
  *   or_quantize_act                      pinned: linalg.QuantizeActQ fingerprint (per-row and per-32)
+ *   or_dequantize_rows_int8              pinned: linalg.DequantizeRowsInt8Into fingerprint (with or_quantize_row_int8 the
+ *                                        whole of the int8 KV cache's store and read)
  *   or_quantize_int4_row / _mat          pinned: linalg.QuantizeGroupInt4Row, linalg.QuantizeInt4
  *   or_qk_acc64 / or_av_acc64            pinned: linalg.MatmulQKAcc64, linalg.MatmulAVAcc64
  *   or_rmsnorm, or_rope, or_swiglu, or_softmax_f32, or_topk, or_route_experts, or_argmax
@@ -61,6 +63,9 @@ void or_dequant_q5k(const uint8_t *blocks, size_t n_blocks, float *out);
 /* GGUF Q6_K (210-byte super-blocks: ql[128] low nibbles, qh[64] two high bits each, 16 int8 sub-block scales, d f16):
  * w = d*sc_s*(q-32), 16 sub-blocks of 16. Pinned bit-exact by fingerprint embed.GGUFFile(Q6_K).Tensor. */
 void or_dequant_q6k(const uint8_t *blocks, size_t n_blocks, float *out);
+
+/* ---- int8 rows back to f32: decoder/kvcache.go:54-59, backend/cuda/kvtype.cuh:48-52 ---- */
+void or_dequantize_rows_int8(float *dst, const int8_t *q, const float *scales, int rows, int cols);
 
 /* ---- activation quantizers: backend/cuda/kv8_store.cu:3-35, actgroup.cu:26-54 ---- */
 float or_quantize_row_int8(const float *row, int n, int8_t *q);
@@ -127,7 +132,7 @@ typedef struct {
     double eps, attn_scale, softcap;
     const double *inv_freq; /* [head_dim/2] */
     int n_experts, top_k, norm_topk, exp_inter;
-    int kv_f16;     /* 1: K/V rows narrowed to binary16 (round-half-up) on append */
+    int kv_f16;     /* KV cache element: 0 f32, 1 binary16 (round-half-up on append), 2 int8 per (position, kv head) with an f32 scale */
     or_layer *layers;
     const float *final_norm;
     or_mat head;

@@ -35,8 +35,10 @@ class LazyEmbedding:
 class Pair:
     """The same synthetic model as an oracle model and (when dev is given) a resident GPU model."""
 
-    def __init__(self, cfg, seed, dev=None, slots=8, ctx_cap=512, sigma=0.02, kinds=None):
+    def __init__(self, cfg, seed, dev=None, slots=8, ctx_cap=512, sigma=0.02, kinds=None, kv="f16"):
         """kinds: optional {projection: 'q5k' | 'q6k' | 'w8a8'} for dense projections stored as those super-blocks or int8 rows."""
+        if kv == "i8":  # the int8 KV cache on both sides
+            cfg = dict(cfg, kv_f16=2)
         self.cfg = cfg
         kinds = kinds or {}
         H, nH, nKV, hd = cfg["hidden"], cfg["n_heads"], cfg["n_kv"], cfg["head_dim"]
@@ -113,7 +115,7 @@ class Pair:
         self.oracle = ob.OracleModel(cfg, layers, fn, head, inv)
         if self.gpu:
             self.gpu.finalize()
-            self.gpu.kv_configure(slots, ctx_cap)
+            self.gpu.kv_configure(slots, ctx_cap, kv)
         self.ctx_cap = ctx_cap
 
     def close(self):

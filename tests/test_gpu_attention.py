@@ -90,3 +90,50 @@ def test_softcap_changes_result_and_matches_closed_form(dev):
         p /= p.sum()
         want = p @ v[:, kv * hd:(kv + 1) * hd].astype(np.float64)
         assert np.abs(got[h * hd:(h + 1) * hd] - want).max() <= 2e-4 * max(1.0, np.abs(want).max())
+
+
+def i8_round_trip(x, nKV, hd):
+    """What the int8 cache holds of K or V rows [n][nKV*hd]: per head the codes times their scale (the oracle's own functions,
+    both pinned by the reference's fingerprints)."""
+    heads = x.reshape(-1, hd)
+    q, sc = ob.quantize_rows_int8(heads)
+    return ob.dequantize_rows_int8(q, sc).reshape(x.shape)
+
+
+@pytest.mark.parametrize("hd", [64, 128])
+@pytest.mark.parametrize("nH,nKV", [(4, 1), (8, 8), (14, 2)])
+@pytest.mark.parametrize("softcap", [0.0, 50.0])
+def test_ragged_attention_i8_small(dev, hd, nH, nKV, softcap):
+    """The int8 cache: the same bar against the oracle's attention over the dequantized rows."""
+    lens = [1, 7, 8, 9, 63, 64, 65, 300]
+    tot, kvd = sum(lens), nKV * hd
+    k = synth.normal(1, tot * kvd).reshape(tot, kvd)
+    v = synth.normal(2, tot * kvd).reshape(tot, kvd)
+    k[5] = 0.0  # an all-zero row: scale 1, codes 0
+    q = synth.normal(3, len(lens) * nH * hd).reshape(len(lens), nH * hd)
+    scale = float(1.0 / np.sqrt(hd))
+    got = dev.attn_ragged(lens, k, v, q, nH, nKV, hd, scale, softcap, kv="i8")
+    want = oracle_attn(lens, i8_round_trip(k, nKV, hd), i8_round_trip(v, nKV, hd), q, nH, nKV, hd, scale, softcap)
+    err = np.abs(got - want).max() / np.abs(want).max()
+    assert err <= 1e-4, err
+    again = dev.attn_ragged(lens, k, v, q, nH, nKV, hd, scale, softcap, kv="i8")
+    assert np.array_equal(got.view(np.uint32), again.view(np.uint32))
+    # and it is a different cache from the f16 one: the quantization is visible
+    f16 = dev.attn_ragged(lens, k, v, q, nH, nKV, hd, scale, softcap)
+    assert np.abs(got - f16).max() > 1e-4
+
+
+def test_ragged_attention_i8_long_split(dev):
+    lens = [1000, 4097, 128, 2050]
+    nH, nKV, hd = 32, 8, 128
+    tot, kvd = sum(lens), nKV * hd
+    rng = np.random.default_rng(5)
+    k = rng.standard_normal((tot, kvd), dtype=np.float32) * np.exp(rng.standard_normal((tot, 1), dtype=np.float32))  # rows of very different scale
+    v = rng.standard_normal((tot, kvd), dtype=np.float32)
+    q = rng.standard_normal((len(lens), nH * hd), dtype=np.float32)
+    scale = float(1.0 / np.sqrt(hd))
+    for softcap in (0.0, 50.0):
+        got = dev.attn_ragged(lens, k, v, q, nH, nKV, hd, scale, softcap, kv="i8")
+        want = oracle_attn(lens, i8_round_trip(k, nKV, hd), i8_round_trip(v, nKV, hd), q, nH, nKV, hd, scale, softcap)
+        err = np.abs(got - want).max() / np.abs(want).max()
+        assert err <= 1e-4, (softcap, err)

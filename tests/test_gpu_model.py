@@ -149,3 +149,49 @@ def test_step_errors(dev):
     pair.gpu.kv_reset(0)
     pair.gpu.step_batch([0], [0], e)
     pair.close()
+
+
+def test_dense_i8_kv_cache(dev):
+    """The int8 KV cache (goinfer's KVQuant "i8") on both sides: prefill through the step, ragged batched decode, batched == solo."""
+    rng = np.random.default_rng(7)
+    check(Pair(dense_cfg(), seed=8, dev=dev, slots=8, kv="i8"), [list(rng.integers(0, 512, n)) for n in (3, 17, 64, 130)], steps=6)
+
+
+def test_dense_i8_kv_hd128(dev):
+    cfg = dense_cfg(n_layers=2, hidden=512, n_heads=4, n_kv=1, head_dim=128, inter=768, vocab=1024)
+    rng = np.random.default_rng(1)
+    check(Pair(cfg, seed=2, dev=dev, slots=4, kv="i8"), [list(rng.integers(0, 1024, n)) for n in (5, 66)], steps=4)
+
+
+def uploaded_prefix_deviation(dev, kv):
+    """A 70-row prefix that arrives through rd_kv_upload (the prefill bridge), then three steps: worst deviation from the oracle."""
+    cfg = dense_cfg(n_layers=2, hidden=512, n_heads=4, n_kv=1, head_dim=128, inter=768, vocab=1024)
+    pair = Pair(cfg, seed=9, dev=dev, slots=2, ctx_cap=128, kv=kv)
+    try:
+        rng = np.random.default_rng(3)
+        n, kvd = 70, cfg["n_kv"] * cfg["head_dim"]
+        cache = pair.oracle.new_cache(128)
+        for l in range(cfg["n_layers"]):
+            k = rng.standard_normal((n, kvd)).astype(np.float32)
+            v = rng.standard_normal((n, kvd)).astype(np.float32)
+            pair.oracle.cache_upload(cache, l, 0, k, v)
+            pair.gpu.kv_upload(0, l, 0, k, v)
+        worst = 0.0
+        for step in range(3):
+            tok = int(rng.integers(0, 1024))
+            want = pair.oracle.step(pair.emb[[tok]], [cache])
+            got, _ = pair.gpu.step_batch([0], [n + step], pair.emb[[tok]])
+            worst = max(worst, float(np.abs(got[0] - want[0]).max()))
+        pair.oracle.free_cache(cache)
+        return worst
+    finally:
+        pair.close()
+
+
+def test_i8_kv_uploaded_prefix(dev):
+    """rd_kv_upload into the int8 cache. What the GPU's f16 GEMM operands cost against the oracle's integer-exact ones is the
+    same whatever the cache holds, so the int8 cache may not sit further from its oracle than the f16 cache sits from its own
+    (the kernel-level bar, 1e-4 against the oracle's attention over the dequantized rows, is in test_gpu_attention.py)."""
+    d_f16, d_i8 = uploaded_prefix_deviation(dev, "f16"), uploaded_prefix_deviation(dev, "i8")
+    print("uploaded prefix: deviation f16 %.4f, i8 %.4f" % (d_f16, d_i8))
+    assert d_i8 <= max(2e-2, 1.5 * d_f16), (d_i8, d_f16)

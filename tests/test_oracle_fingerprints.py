@@ -20,6 +20,7 @@ PINS = {
     "embed.GGUFFile(Q5_K).Tensor": ALL,
     "embed.GGUFFile(Q6_K).Tensor": ALL,
     "linalg.QuantizeRowInt8": ALL,
+    "linalg.DequantizeRowsInt8Into": ALL,  # with QuantizeRowInt8: the int8 KV cache's store and read
     "linalg.QuantizeActQ": ALL,
     "linalg.QuantizeGroupInt4Row": ALL,
     "linalg.QuantizeInt4": ALL,
