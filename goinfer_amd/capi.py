@@ -21,7 +21,7 @@ EXPORTS = [
     "rd_kv_configure", "rd_kv_upload", "rd_kv_truncate", "rd_kv_reset", "rd_step_batch", "rd_forward",
     "rd_last_moe_indices", "rd_model_upload_embedding", "rd_bench_steps", "rd_bench_profile", "rd_bench_class_count",
     "rd_bench_class_name", "rd_bench_kernel", "rd_gateup_q4k_quant", "rd_moe_replay", "rd_bench_attn", "rd_step_ragged", "rd_prefill_last",
-    "rd_kv_configure_typed", "rd_attn_ragged_i8", "rd_bench_attn_i8",
+    "rd_kv_configure_typed", "rd_attn_ragged_i8", "rd_bench_attn_i8", "rd_step_ragged_draw", "rd_forward_no_logits",
     "rd_step_batch_draw", "rd_sample_rows", "rd_greedy_chain_start", "rd_greedy_chain_next", "rd_sample_chain_start",
     "rd_sample_chain_next", "rd_greedy_chain_stop",
     "rd_dequant_q5k", "rd_dequant_q6k", "rd_gemm_q5k", "rd_gemm_q6k", "rd_model_upload_q5k", "rd_model_upload_q6k",
@@ -353,6 +353,23 @@ class Model:
         ids = np.empty(R, np.int32) if want & WANT_ARGMAX else None
         check(lib().rd_step_ragged(self.h, len(slots), _p(slots), _p(pos), _p(n_rows), _p(emb), want, _p(logits), _p(ids)), "rd_step_ragged")
         return logits, ids
+
+    def step_ragged_draw(self, slots, pos, embs, draws, want=0):
+        """draws: per sequence None, "greedy" or (temperature, seed, draw), for its last row. Returns (logits or None, ids per row)."""
+        n_rows = np.ascontiguousarray([len(e) for e in embs], dtype=np.int32)
+        emb = _f32(np.concatenate([np.asarray(e, dtype=np.float32).reshape(len(e), -1) for e in embs], axis=0))
+        slots = np.ascontiguousarray(slots, dtype=np.int32)
+        pos = np.ascontiguousarray(pos, dtype=np.int32)
+        R = int(n_rows.sum())
+        logits = np.empty((R, self.cfg["vocab"]), np.float32) if want & WANT_LOGITS else None
+        ids = np.empty(R, np.int32)
+        check(lib().rd_step_ragged_draw(self.h, len(slots), _p(slots), _p(pos), _p(n_rows), _p(emb), make_draws(draws), want, _p(logits), _p(ids)),
+              "rd_step_ragged_draw")
+        return logits, ids
+
+    def forward_no_logits(self, slot, pos, emb):
+        emb = _f32(emb)
+        check(lib().rd_forward_no_logits(self.h, slot, pos, _p(emb)), "rd_forward_no_logits")
 
     def prefill_last(self, slot, start_pos, emb):
         emb = _f32(emb)

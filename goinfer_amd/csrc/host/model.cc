@@ -778,19 +778,24 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
             resP = m->moe_out, resSplits = 1;
         }
     }
-    GemmPlan plan;
-    RC(add_norm_quant(m, B, resP, resSplits, m->final_norm, m->head, m->XpA, nullptr));
-    {
-        Scope s(m, KC_GEMM_HEAD);
-        RC(launch_gemm(d, m->head, m->XpA, m->P, B, &plan));
+    if (want & (RD_WANT_LOGITS | RD_WANT_ARGMAX)) {
+        GemmPlan plan;
+        RC(add_norm_quant(m, B, resP, resSplits, m->final_norm, m->head, m->XpA, nullptr));
+        {
+            Scope s(m, KC_GEMM_HEAD);
+            RC(launch_gemm(d, m->head, m->XpA, m->P, B, &plan));
+        }
+        {
+            Scope s(m, KC_ARGMAX);
+            int nChunks = (c.vocab + 4095) / 4096;
+            RC(d->launch(d->k.argmax_rows, (unsigned)nChunks, (unsigned)B, 1, 256, (const float *)m->P, plan.splits, c.vocab, m->cand_v, m->cand_i,
+                         (want & RD_WANT_LOGITS) ? m->logits : (float *)nullptr, (const int *)(m->step_draws ? m->rowDraw : nullptr)));
+            if (want & RD_WANT_ARGMAX) RC(d->launch(d->k.argmax_final, (unsigned)B, 1, 1, 64, (const float *)m->cand_v, (const int *)m->cand_i, nChunks, m->ids));
+        }
     }
-    {
-        Scope s(m, KC_ARGMAX);
-        int nChunks = (c.vocab + 4095) / 4096;
-        RC(d->launch(d->k.argmax_rows, (unsigned)nChunks, (unsigned)B, 1, 256, (const float *)m->P, plan.splits, c.vocab, m->cand_v, m->cand_i,
-                     (want & RD_WANT_LOGITS) ? m->logits : (float *)nullptr, (const int *)(m->step_draws ? m->rowDraw : nullptr)));
-        if (want & RD_WANT_ARGMAX) RC(d->launch(d->k.argmax_final, (unsigned)B, 1, 1, 64, (const float *)m->cand_v, (const int *)m->cand_i, nChunks, m->ids));
-    }
+    // else: no logits asked for (resident.Forward's ForwardNoLogits, decoder/resident/subsystems.go:68-77: a prompt token that only
+    // builds its K/V): the final norm, the head GEMM and the argmax are skipped, and the last block's pending residual
+    // contribution stays unadded, since nothing reads the hidden state after it.
     for (int b = 0; b < B; b++) m->slot_len[(size_t)slot[b]] = std::max(m->slot_len[(size_t)slot[b]], pos[b] + 1);
     m->last_B = B;
     const bool replayed = m->replay_B != 0;
@@ -995,6 +1000,68 @@ extern "C" int rd_step_ragged(rd_model *m, int n_seq, const int *slot, const int
     return RD_OK;
 }
 
+// StepRagged with a draw per sequence (decoder/resident/forward.go:60-75 RaggedSeq.Draw): the last row of a sequence that carries a
+// draw returns the token drawn on the device in ids; every other row returns -1 there.
+extern "C" int rd_step_ragged_draw(rd_model *m, int n_seq, const int *slot, const int *pos, const int *n_rows, const float *emb, const rd_draw *draws,
+                                   int want, float *logits, int *ids) {
+    if (!m || !slot || !pos || !n_rows || !emb || !draws || !ids || n_seq <= 0) return RD_ERR_ARG;
+    if ((want & RD_WANT_LOGITS) && !logits) {
+        rd_set_error("rd_step_ragged_draw: want=%d needs its output buffer", want);
+        return RD_ERR_ARG;
+    }
+    if (!m->finalized || !m->tables) {
+        rd_set_error("step before rd_model_finalize / rd_kv_configure");
+        return RD_ERR_STATE;
+    }
+    std::vector<int> rslot, rpos;
+    std::vector<rd_draw> rdraw;
+    for (int i = 0; i < n_seq; i++) {
+        if (!slot_ok(m, slot[i])) return RD_ERR_ARG;
+        for (int a = 0; a < i; a++)
+            if (slot[a] == slot[i]) {
+                rd_set_error("KV slot %d is named by two sequences", slot[i]);
+                return RD_ERR_ARG;
+            }
+        if (n_rows[i] <= 0 || pos[i] < 0 || pos[i] > m->slot_len[(size_t)slot[i]]) {
+            rd_set_error("sequence %d: %d rows at position %d, slot %d holds %d rows", i, n_rows[i], pos[i], slot[i], m->slot_len[(size_t)slot[i]]);
+            return RD_ERR_ARG;
+        }
+        if (pos[i] + n_rows[i] > m->ctx_cap) {
+            rd_set_error("sequence %d: rows %d..%d reach the context cap %d", i, pos[i], pos[i] + n_rows[i] - 1, m->ctx_cap);
+            return RD_ERR_KV_FULL;
+        }
+        if (draws[i].mode < RD_DRAW_NONE || draws[i].mode > RD_DRAW_GUMBEL || (draws[i].mode == RD_DRAW_GUMBEL && std::isnan(draws[i].temperature))) {
+            rd_set_error("rd_step_ragged_draw: sequence %d has draw mode %d, temperature %g", i, draws[i].mode, draws[i].temperature);
+            return RD_ERR_ARG;
+        }
+        for (int j = 0; j < n_rows[i]; j++) {
+            rslot.push_back(slot[i]), rpos.push_back(pos[i] + j);
+            rd_draw none{};
+            rdraw.push_back(j == n_rows[i] - 1 ? draws[i] : none);
+        }
+    }
+    const size_t H = (size_t)m->desc.hidden, V = (size_t)m->desc.vocab;
+    int rc = RD_OK;
+    for (size_t r0 = 0; r0 < rslot.size() && !rc; r0 += 32) {
+        const int rows = (int)std::min<size_t>(32, rslot.size() - r0);
+        m->step_draws = rdraw.data() + r0;
+        rc = model_step(m, rows, rslot.data() + r0, rpos.data() + r0, emb + r0 * H, nullptr, want | RD_WANT_ARGMAX, logits ? logits + r0 * V : nullptr,
+                        ids + r0, true);
+        m->step_draws = nullptr;
+    }
+    if (!rc)
+        for (size_t r = 0; r < rslot.size(); r++)
+            if (rdraw[r].mode == RD_DRAW_NONE) ids[r] = -1;
+    return rc;
+}
+
+// ForwardNoLogits (decoder/resident/subsystems.go:68-77): one token's forward that only builds its K/V; the layer chain, hence the
+// K/V written, is the one rd_forward runs.
+extern "C" int rd_forward_no_logits(rd_model *m, int slot, int pos, const float *emb) {
+    if (!m || !emb) return RD_ERR_ARG;
+    return model_step(m, 1, &slot, &pos, emb, nullptr, 0, nullptr, nullptr, false);
+}
+
 // PrefillLast: n rows of one sequence from start_pos; only the last row's logits come back.
 extern "C" int rd_prefill_last(rd_model *m, int slot, int start_pos, int n, const float *emb, float *logits) {
     if (!m || !emb || !logits || n <= 0) return RD_ERR_ARG;
@@ -1014,14 +1081,12 @@ extern "C" int rd_prefill_last(rd_model *m, int slot, int start_pos, int n, cons
     const size_t H = (size_t)m->desc.hidden;
     std::vector<int> rslot(32, slot), rpos(32);
     std::vector<float> tail; // the last pass returns its rows' logits; only the final row is handed on
-    std::vector<int> idsink(32);
     for (int r0 = 0; r0 < n; r0 += 32) {
         const int rows = std::min(32, n - r0);
         const bool last = r0 + rows == n;
         for (int j = 0; j < rows; j++) rpos[(size_t)j] = start_pos + r0 + j;
         if (last) tail.resize((size_t)rows * m->desc.vocab);
-        RC(model_step(m, rows, rslot.data(), rpos.data(), emb + (size_t)r0 * H, nullptr, last ? RD_WANT_LOGITS : RD_WANT_ARGMAX, last ? tail.data() : nullptr,
-                      last ? nullptr : idsink.data(), true));
+        RC(model_step(m, rows, rslot.data(), rpos.data(), emb + (size_t)r0 * H, nullptr, last ? RD_WANT_LOGITS : 0, last ? tail.data() : nullptr, nullptr, true));
         if (last) memcpy(logits, tail.data() + (size_t)(rows - 1) * m->desc.vocab, sizeof(float) * (size_t)m->desc.vocab);
     }
     return RD_OK;

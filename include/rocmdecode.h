@@ -185,6 +185,14 @@ int rd_step_ragged(rd_model *m, int n_seq, const int *slot, const int *pos, cons
  * logits: host f32 [vocab] of the last row. The rows run through the decode step's kernels 32 at a time (every pass re-streams
  * the weights: correct and bit-identical to token-by-token, not yet a prefill-rate kernel). */
 int rd_prefill_last(rd_model *m, int slot, int start_pos, int n, const float *emb, float *logits);
+/* rd_step_ragged with one draw per sequence (decoder/resident/forward.go:60-75 RaggedSeq.Draw): ids [sum n_rows] holds the token
+ * drawn on the device for the last row of a sequence that carries a draw and -1 for every other row. */
+int rd_step_ragged_draw(rd_model *m, int n_seq, const int *slot, const int *pos, const int *n_rows, const float *emb, const rd_draw *draws,
+                        int want, float *logits, int *ids);
+/* resident.Forward's optional ForwardNoLogits (decoder/resident/subsystems.go:68-77): the token's forward builds only its K/V; the
+ * final norm, the head matmul and the logits readback are skipped. rd_prefill_last uses the same short cut for every pass but
+ * its last. */
+int rd_forward_no_logits(rd_model *m, int slot, int pos, const float *emb);
 /* Forward(embedding, pos) on one slot: the B=1 step through the same kernels */
 int rd_forward(rd_model *m, int slot, int pos, const float *emb, float *logits);
 /* expert indices the last step routed to: int32 [B][n_layers][top_k] (MoE models only; parity checks) */

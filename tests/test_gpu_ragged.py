@@ -105,3 +105,42 @@ def test_ragged_refusals_write_nothing(dev):
     with pytest.raises(capi.RocmError, match="appears twice"):
         pair.gpu.step_batch([3, 3], [0, 1], pair.emb[[1, 2]])
     pair.close()
+
+
+def test_forward_no_logits_builds_the_same_kv(dev):
+    """ForwardNoLogits skips the head; the K/V it leaves is rd_forward's, so the next token's logits are bit-identical."""
+    pair = Pair(dense_cfg(), seed=54, dev=dev, slots=4, ctx_cap=64)
+    toks = [5, 77, 300, 12]
+    for p, t in enumerate(toks):
+        pair.gpu.forward(0, p, pair.emb[t])
+        pair.gpu.forward_no_logits(1, p, pair.emb[t])
+    a = pair.gpu.forward(0, len(toks), pair.emb[9])
+    b = pair.gpu.forward(1, len(toks), pair.emb[9])
+    assert np.array_equal(bits(a), bits(b))
+    pair.close()
+
+
+def test_ragged_step_with_draws(dev):
+    """A sequence's draw applies to its last row: the argmax, or the host's Gumbel-max token on that row's logits; other rows -1."""
+    cfg = dense_cfg(vocab=8192)
+    pair = Pair(cfg, seed=55, dev=dev, slots=4, ctx_cap=64)
+    rng = np.random.default_rng(4)
+    embs = [pair.emb[rng.integers(0, cfg["vocab"], n)] for n in (1, 3, 5, 2)]
+    draws = ["greedy", (0.8, 77, 3), None, (1.4, 5 + (9 << 32), 1 << 33)]
+    logits, ids = pair.gpu.step_ragged_draw([0, 1, 2, 3], [0, 0, 0, 0], embs, draws, want=capi.WANT_LOGITS)
+    last = np.cumsum([len(e) for e in embs]) - 1
+    for i, r in enumerate(last):
+        if draws[i] is None:
+            assert ids[r] == -1
+        elif draws[i] == "greedy":
+            assert ids[r] == int(np.argmax(logits[r]))
+        else:
+            assert ids[r] == ob.gumbel_draw(logits[r], *draws[i], guarded=True)
+    others = sorted(set(range(len(ids))) - set(int(r) for r in last))
+    assert all(ids[r] == -1 for r in others)
+    # the logits are those of the plain ragged step on twin state
+    pair2 = Pair(cfg, seed=55, dev=dev, slots=4, ctx_cap=64)
+    plain, _ = pair2.gpu.step_ragged([0, 1, 2, 3], [0, 0, 0, 0], embs)
+    assert np.array_equal(bits(plain), bits(logits))
+    pair.close()
+    pair2.close()
