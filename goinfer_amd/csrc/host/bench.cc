@@ -88,7 +88,7 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
     if (!d || !name || !args || iters <= 0 || !ms_out) return RD_ERR_ARG;
     std::string nm(name);
     const bool isGemm = nm == "gemm_q4k" || nm == "gemm_q5k" || nm == "gemm_q6k";
-    if (isGemm && n_args >= 4 && (args[0] % 32 || args[1] % 256 || args[0] <= 0 || args[1] <= 0 || args[2] < 1 || args[2] > 64)) {
+    if (isGemm && n_args >= 4 && (args[0] % 32 || args[1] % 256 || args[0] <= 0 || args[1] <= 0 || args[2] < 1 || args[2] > 128)) {
         rd_set_error("%s bench: bad shape", name);
         return RD_ERR_ARG;
     }
@@ -129,20 +129,22 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
             if (!rc) rc = kind == 0 ? upload_q4k(d, raw.data(), N, K, &w) : (kind == 3 ? upload_q5k(d, raw.data(), N, K, &w) : upload_q6k(d, raw.data(), N, K, &w));
         DevBuf Xp(d), P(d);
         size_t pb = kind == 4 ? (size_t)(K / 128) * LIN_PANEL_BYTES : (size_t)(K / 256) * Q4K_PANEL_BYTES;
-        if (!rc) rc = Xp.alloc(pb);
+        const int tiles = (M + 31) / 32; // rows beyond 32 are further M-tiles, each with its own panels and partial sums
+        if (!rc) rc = Xp.alloc(pb * tiles);
         int nKB = K / kblock_of(kind);
         GemmPlan plan = plan_gemm(kind, N, nKB);
-        if (!rc) rc = P.alloc(sizeof(float) * (size_t)plan.splits * 32 * N);
+        const size_t pStride = (size_t)plan.splits * 32 * N;
+        if (!rc) rc = P.alloc(sizeof(float) * pStride * tiles);
         if (!rc) {
-            std::vector<uint16_t> x(pb / 2);
+            std::vector<uint16_t> x(pb * tiles / 2);
             for (size_t i = 0; i < x.size(); i++) x[i] = (uint16_t)(0x3000 + (i * 2654435761u >> 22 & 0x3ff)) | (uint16_t)((i & 1) << 15);
-            rc = d->h2d(Xp.p, x.data(), pb);
+            rc = d->h2d(Xp.p, x.data(), pb * tiles);
         }
         if (!rc) rc = d->sync();
         for (int i = 0; i < warmup + iters && !rc; i++) {
             const DevWeight &w = ws[(size_t)i % ws.size()];
             if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup)], d->stream);
-            for (int m0 = 0; m0 < M && !rc; m0 += 32) rc = launch_gemm(d, w, Xp.p, P.as<float>(), std::min(32, M - m0), nullptr); // rows in groups of 32
+            rc = launch_gemm_wide(d, w, Xp.p, pb, P.as<float>(), pStride, M, nullptr); // M-tiles of 32 rows; Q4_K reads its weights once for all of them
             if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup) + 1], d->stream);
         }
         if (!rc) rc = d->sync();

@@ -81,6 +81,7 @@ static const KName kNames[] = {
     {"rd_k_gemm_w8a8", &Kernels::gemm_w8a8},
     {"rd_k_retile_w4a8", &Kernels::retile_w4a8},
     {"rd_k_gemm_w4a8", &Kernels::gemm_w4a8},
+    {"rd_k_gemm_q4k_wide", &Kernels::gemm_q4k_wide},
     {"rd_k_dequant_q5k", &Kernels::dequant_q5k},
     {"rd_k_retile_q5k", &Kernels::retile_q5k},
     {"rd_k_gemm_q5k", &Kernels::gemm_q5k},
@@ -339,4 +340,26 @@ int launch_gemm(rd_device *d, const DevWeight &w, const void *Xp, float *P, int 
     if (w.kind == 1)
         return d->launch(d->k.gemm_w8a8, gx, p.splits, 1, GEMM_THREADS, (const void *)w.tiled, (const void *)w.scales, Xp, P, w.N, nKB, p.kbPerSplit, M, ldP);
     return d->launch(d->k.gemm_w4a8, gx, p.splits, 1, GEMM_THREADS, (const void *)w.tiled, Xp, P, w.N, nKB, p.kbPerSplit, M, ldP);
+}
+
+int launch_gemm_wide(rd_device *d, const DevWeight &w, const void *Xp, size_t xpStride, float *P, size_t pStride, int M, GemmPlan *plan_out, int ldP,
+                     int splits) {
+    if (M < 1 || M > GEMM_WIDE_ROWS) {
+        rd_set_error("wide gemm: M=%d outside 1..%d", M, GEMM_WIDE_ROWS);
+        return RD_ERR_ARG;
+    }
+    if (w.kind != 0 || M <= 32 || getenv("ROCMDECODE_NO_WIDE_GEMM")) {
+        for (int m0 = 0, mt = 0; m0 < M; m0 += 32, mt++) {
+            int rc = launch_gemm(d, w, (const char *)Xp + (size_t)mt * xpStride, P + (size_t)mt * pStride, std::min(32, M - m0), plan_out, ldP, splits);
+            if (rc) return rc;
+        }
+        return RD_OK;
+    }
+    int nKB = kblocks_for(w);
+    GemmPlan p = plan_gemm(w.kind, w.N, nKB);
+    if (splits > 0) p.kbPerSplit = (nKB + splits - 1) / splits, p.splits = splits;
+    if (plan_out) *plan_out = p;
+    if (ldP <= 0) ldP = w.N;
+    return d->launch(d->k.gemm_q4k_wide, (unsigned)((w.N + 127) / 128), p.splits, 1, GEMM_WIDE_THREADS, (const void *)w.tiled, Xp, xpStride, P, pStride, w.N, nKB,
+                     p.kbPerSplit, M, ldP);
 }

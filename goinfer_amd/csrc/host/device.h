@@ -23,6 +23,7 @@ enum { PANEL_Q4K = 0, PANEL_LIN = 1, PANEL_LIN4 = 2 };
 struct Kernels {
     hipFunction_t dequant_q4k, retile_q4k, gemm_q4k, quant_act, reduce_splits, add_rmsnorm_quant, swiglu_quant;
     hipFunction_t retile_w8a8, gemm_w8a8, retile_w4a8, gemm_w4a8;
+    hipFunction_t gemm_q4k_wide;
     hipFunction_t dequant_q5k, retile_q5k, gemm_q5k, dequant_q6k, retile_q6k, gemm_q6k;
     hipFunction_t gemm_q4k_gateup;
     hipFunction_t kv_store, qkv_rope_store, attn_partial, attn_combine, attn_combine_quant;
@@ -108,6 +109,13 @@ void free_weight(rd_device *d, DevWeight *w);
 // ldP: floats between rows of P (0 = w.N); splits > 0 forces the split count (trailing splits that get no K-block store zeros),
 // which lets weights of different kinds write side by side into one partial-sum buffer.
 int launch_gemm(rd_device *d, const DevWeight &w, const void *Xp, float *P, int M, GemmPlan *plan, int ldP = 0, int splits = 0);
+// Up to 128 rows as M-tiles of 32: M-tile mt reads its panels at Xp + mt*xpStride (bytes) and writes its partial sums at
+// P + mt*pStride (floats), each laid out as launch_gemm's. Q4_K weights go through the wide kernel (weights read once for
+// all rows); the other kinds run launch_gemm per M-tile. Rows come out identical to launch_gemm's either way.
+constexpr int GEMM_WIDE_ROWS = 128;
+constexpr unsigned GEMM_WIDE_THREADS = 512;
+int launch_gemm_wide(rd_device *d, const DevWeight &w, const void *Xp, size_t xpStride, float *P, size_t pStride, int M, GemmPlan *plan, int ldP = 0,
+                     int splits = 0);
 size_t panel_bytes_for(const DevWeight &w);
 int panel_kind_for(const DevWeight &w);
 // K-blocks of a weight: super-blocks of 256 for the kinds on Q4_K-style panels (q4k, q5k), 128 otherwise

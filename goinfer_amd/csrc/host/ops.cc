@@ -37,22 +37,27 @@ static int gemm_host(rd_device *d, DevWeight &w, DevWeight *w2, const float *a, 
     int N = w.N, K = w.K;
     size_t pbytes = panel_bytes_for(w);
     int kind = panel_kind_for(w);
+    const int chunk = w2 ? 32 : GEMM_WIDE_ROWS, tiles = chunk / 32; // rows per pass: M-tiles of 32 side by side
     DevBuf A(d), Xp(d), P(d), O(d);
-    RC(A.alloc(sizeof(float) * (size_t)32 * K));
-    RC(Xp.alloc(pbytes));
+    RC(A.alloc(sizeof(float) * (size_t)chunk * K));
+    RC(Xp.alloc(pbytes * tiles));
     int nKB = kblocks_for(w);
     int Ntot = w2 ? 2 * N : N;
     int maxSplits = plan_gemm(w.kind, Ntot, nKB).splits;
-    RC(P.alloc(sizeof(float) * (size_t)maxSplits * 32 * Ntot));
-    RC(O.alloc(sizeof(float) * (size_t)32 * N));
-    for (int m0 = 0; m0 < M; m0 += 32) {
-        int mc = std::min(32, M - m0);
+    const size_t pStride = (size_t)maxSplits * 32 * Ntot;
+    RC(P.alloc(sizeof(float) * pStride * tiles));
+    RC(O.alloc(sizeof(float) * (size_t)chunk * N));
+    for (int m0 = 0; m0 < M; m0 += chunk) {
+        int mc = std::min(chunk, M - m0);
         RC(d->h2d(A.p, a + (size_t)m0 * K, sizeof(float) * (size_t)mc * K));
-        RC(quantize_rows(d, A.as<float>(), mc, K, kind, pbytes, Xp.p));
+        for (int t = 0; t * 32 < mc; t++)
+            RC(quantize_rows(d, A.as<float>() + (size_t)t * 32 * K, std::min(32, mc - t * 32), K, kind, pbytes, (char *)Xp.p + (size_t)t * pbytes));
         GemmPlan plan;
         if (!w2) {
-            RC(launch_gemm(d, w, Xp.p, P.as<float>(), mc, &plan));
-            RC(d->launch(d->k.reduce_splits, (unsigned)((N + 255) / 256), (unsigned)mc, 1, 256, (const float *)P.p, O.as<float>(), N, plan.splits));
+            RC(launch_gemm_wide(d, w, Xp.p, pbytes, P.as<float>(), pStride, mc, &plan));
+            for (int t = 0; t * 32 < mc; t++)
+                RC(d->launch(d->k.reduce_splits, (unsigned)((N + 255) / 256), (unsigned)std::min(32, mc - t * 32), 1, 256,
+                             (const float *)(P.as<float>() + (size_t)t * pStride), O.as<float>() + (size_t)t * 32 * N, N, plan.splits));
         } else {
             // gate|up stacked (2N rows): GEMM, then SwiGLU over the reduced partial sums
             RC(launch_gemm(d, *w2, Xp.p, P.as<float>(), mc, &plan));

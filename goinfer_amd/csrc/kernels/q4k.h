@@ -132,6 +132,78 @@ __device__ __forceinline__ void q4k_tile_mma(float16_t &acc, const Q4KTile &w, c
     }
 }
 
+// The tile product against MT panels (M-tiles of 32 batch rows): each step's weights are dequantized once and multiplied
+// against every M-tile in use. Per M-tile the MFMA sequence is q4k_tile_mma's. mtStride: vectors between the M-tiles' buffers.
+template <int MT>
+__device__ __forceinline__ void q4k_tile_mma_wide(float16_t (&acc)[MT], const Q4KTile &w, const uint4_t *__restrict__ panel, int mtStride, int nMT,
+                                                  int lane) {
+    const int h = lane >> 5;
+    const uint32_t mask_lo = 0x000F000Fu, mask_hi = 0x00F000F0u, magic_lo = 0x64006400u, magic_hi = 0x54005400u;
+    uint32_t y = w.hdr.y, z = w.hdr.z, x = w.hdr.w;
+    half2_t dd;
+    uint32_t hx = w.hdr.x;
+    __builtin_memcpy(&dd, &hx, 4);
+    float d = (float)dd.x, dmin = (float)dd.y;
+    half2_t DSC[4], C0[4];
+    half_t off[4];
+#pragma unroll
+    for (int jj = 0; jj < 4; jj++) {
+        int sc_lo = (y >> (8 * jj)) & 63, m_lo = (z >> (8 * jj)) & 63;
+        int sc_hi = ((x >> (8 * jj)) & 15) | (((y >> (8 * jj + 6)) & 3) << 4);
+        int m_hi = ((x >> (8 * jj + 4)) & 15) | (((z >> (8 * jj + 6)) & 3) << 4);
+        int sc = h ? sc_hi : sc_lo, m = h ? m_hi : m_lo;
+        float dsc32 = d * (float)sc;
+        half_t dsc = (half_t)dsc32;
+        float dscf = (float)dsc;
+        const float bias = (jj & 1) ? 72.f : 1032.f;
+        half_t c = (half_t)(-bias * dscf);
+        float delta = (float)c + bias * dscf;
+        DSC[jj] = (half2_t){dsc, dsc};
+        C0[jj] = (half2_t){c, c};
+        off[jj] = (half_t)(8.f * dsc32 - delta - dmin * (float)m);
+    }
+    // Every M-tile is multiplied, in use or not (an unused one reads whatever its LDS buffer holds and its sums are never
+    // stored): no branch stands between the LDS reads and the MFMAs, so the reads of a step go out together. The loop is bound by
+    // those reads (one 1 KB LDS read per MFMA and wave): reading a step further ahead changes nothing.
+#pragma unroll
+    for (int s = 0; s < 16; s++) {
+        uint32_t wd = w.q[s >> 2][s & 3];
+        const int pp = s >> 3;
+        uint32_t t8 = wd >> 8;
+        uint32_t u0 = and_or(wd, mask_lo, magic_lo), u1 = and_or(wd, mask_hi, magic_hi);
+        uint32_t u2 = and_or(t8, mask_lo, magic_lo), u3 = and_or(t8, mask_hi, magic_hi);
+        half2_t v0, v1, v2, v3;
+        __builtin_memcpy(&v0, &u0, 4);
+        __builtin_memcpy(&v1, &u1, 4);
+        __builtin_memcpy(&v2, &u2, 4);
+        __builtin_memcpy(&v3, &u3, 4);
+        v0 = __builtin_elementwise_fma(v0, DSC[2 * pp], C0[2 * pp]);
+        v1 = __builtin_elementwise_fma(v1, DSC[2 * pp + 1], C0[2 * pp + 1]);
+        v2 = __builtin_elementwise_fma(v2, DSC[2 * pp], C0[2 * pp]);
+        v3 = __builtin_elementwise_fma(v3, DSC[2 * pp + 1], C0[2 * pp + 1]);
+        half8_t b = {v0.x, v0.y, v1.x, v1.y, v2.x, v2.y, v3.x, v3.y};
+        uint4_t av[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) av[mt] = panel[(size_t)mt * mtStride + s * 64 + lane];
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) {
+            half8_t a;
+            __builtin_memcpy(&a, &av[mt], 16);
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[mt], 0, 0, 0);
+        }
+    }
+    {
+        half8_t b = {off[0], off[1], off[2], off[3], (half_t)0, (half_t)0, (half_t)0, (half_t)0};
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) {
+            half8_t a;
+            uint4_t av = panel[(size_t)mt * mtStride + 16 * 64 + lane];
+            __builtin_memcpy(&a, &av, 16);
+            acc[mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[mt], 0, 0, 0);
+        }
+    }
+}
+
 struct Q4KTraits {
     typedef Q4KTile Tile;
     static constexpr int TILE_BYTES = RD_Q4K_TILE_BYTES;
@@ -141,6 +213,11 @@ struct Q4KTraits {
     static __device__ __forceinline__ void mma(float16_t &acc, const Tile &w, const uint4_t *__restrict__ panel, int lane) {
         q4k_tile_mma(acc, w, panel, lane);
     }
+    template <int MT>
+    static __device__ __forceinline__ void mma_wide(float16_t (&acc)[MT], const Tile &w, const uint4_t *__restrict__ panel, int mtStride, int nMT,
+                                                    int lane) {
+        q4k_tile_mma_wide<MT>(acc, w, panel, mtStride, nMT, lane);
+    }
     static __device__ __forceinline__ void finish(float16_t &, const void *, int, int) {}
 };
 
@@ -149,6 +226,16 @@ extern "C" __global__ __launch_bounds__(320) void rd_k_gemm_q4k(const uint8_t *_
                                                                  float *__restrict__ P, int N, int nSB, int sbPerSplit, int M, int ldP) {
     __shared__ uint4_t lds[2 * RD_Q4K_PANEL_BYTES / 16];
     gemm_body<Q4KTraits, 4, 1, 3>(Wt, nullptr, Xp, P, N, nSB, sbPerSplit, M, ldP, lds);
+}
+
+// Up to 128 batch rows per launch (prefill and verify rows): grid (ceil(N/128), splits), block 512 = four consumer waves and
+// one panel producer per M-tile of 32 rows; 136 KB of LDS, one block per CU.
+#define RD_GEMM_WIDE_MT 4
+extern "C" __global__ __launch_bounds__(512) void rd_k_gemm_q4k_wide(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ Xp, size_t xpStride,
+                                                                      float *__restrict__ P, size_t pStride, int N, int nSB, int sbPerSplit, int M,
+                                                                      int ldP) {
+    __shared__ uint4_t lds[RD_GEMM_WIDE_MT * 2 * RD_Q4K_PANEL_BYTES / 16];
+    gemm_body_wide<Q4KTraits, 4, RD_GEMM_WIDE_MT, 3>(Wt, nullptr, Xp, xpStride, P, pStride, N, nSB, sbPerSplit, M, ldP, lds);
 }
 
 // Fused gate/up projection + SwiGLU + per-32 quantization (goinfer decoder/cpu_gateup_fused.go:83-148, in one launch):

@@ -47,7 +47,7 @@ def test_dequant_q4k_synth_bit_exact(dev):
     assert abs(float(want.std()) - 0.02) < 2e-3
 
 
-@pytest.mark.parametrize("M", [1, 4, 5, 32, 33, 64])
+@pytest.mark.parametrize("M", [1, 4, 5, 32, 33, 64, 100, 128, 131])
 @pytest.mark.parametrize("N,K", [(128, 256), (160, 1024), (512, 4096)])
 def test_gemm_q4k(dev, M, N, K):
     blocks = synth.q4k_normal(11 + N, N, K)
@@ -61,6 +61,20 @@ def test_gemm_q4k(dev, M, N, K):
     # batch invariance: a row computed in a batch equals the same row alone, bit for bit
     solo = dev.gemm_q4k(blocks, N, K, a[:1])
     assert np.array_equal(solo[0].view(np.uint32), got[0].view(np.uint32))
+
+
+def test_gemm_q4k_wide_rows_equal_narrow_rows(dev, monkeypatch):
+    """More than 32 rows go through the kernel that reads the weights once for up to 128 rows; every row must come out as the
+    32-row kernel computes it, bit for bit."""
+    N, K, M = 416, 2048, 131
+    blocks = synth.q4k_normal(21, N, K)
+    a = synth.normal(22, M * K).reshape(M, K)
+    wide = dev.gemm_q4k(blocks, N, K, a)
+    monkeypatch.setenv("ROCMDECODE_NO_WIDE_GEMM", "1")
+    narrow = dev.gemm_q4k(blocks, N, K, a)
+    assert np.array_equal(wide.view(np.uint32), narrow.view(np.uint32))
+    solo = dev.gemm_q4k(blocks, N, K, a[77:78])
+    assert np.array_equal(solo[0].view(np.uint32), wide[77].view(np.uint32))
 
 
 def test_gemm_q4k_fused_gate_up(dev):
