@@ -82,6 +82,7 @@ static const KName kNames[] = {
     {"rd_k_retile_w4a8", &Kernels::retile_w4a8},
     {"rd_k_gemm_w4a8", &Kernels::gemm_w4a8},
     {"rd_k_gemm_q4k_wide", &Kernels::gemm_q4k_wide},
+    {"rd_k_gemm_q4k_wide2", &Kernels::gemm_q4k_wide2},
     {"rd_k_dequant_q5k", &Kernels::dequant_q5k},
     {"rd_k_retile_q5k", &Kernels::retile_q5k},
     {"rd_k_gemm_q5k", &Kernels::gemm_q5k},
@@ -360,6 +361,9 @@ int launch_gemm_wide(rd_device *d, const DevWeight &w, const void *Xp, size_t xp
     if (splits > 0) p.kbPerSplit = (nKB + splits - 1) / splits, p.splits = splits;
     if (plan_out) *plan_out = p;
     if (ldP <= 0) ldP = w.N;
+    if (M <= 64)
+        return d->launch(d->k.gemm_q4k_wide2, (unsigned)((w.N + 127) / 128), p.splits, 1, 384u, (const void *)w.tiled, Xp, xpStride, P, pStride, w.N, nKB,
+                         p.kbPerSplit, M, ldP);
     return d->launch(d->k.gemm_q4k_wide, (unsigned)((w.N + 127) / 128), p.splits, 1, GEMM_WIDE_THREADS, (const void *)w.tiled, Xp, xpStride, P, pStride, w.N, nKB,
                      p.kbPerSplit, M, ldP);
 }

@@ -23,7 +23,7 @@ enum { PANEL_Q4K = 0, PANEL_LIN = 1, PANEL_LIN4 = 2 };
 struct Kernels {
     hipFunction_t dequant_q4k, retile_q4k, gemm_q4k, quant_act, reduce_splits, add_rmsnorm_quant, swiglu_quant;
     hipFunction_t retile_w8a8, gemm_w8a8, retile_w4a8, gemm_w4a8;
-    hipFunction_t gemm_q4k_wide;
+    hipFunction_t gemm_q4k_wide, gemm_q4k_wide2;
     hipFunction_t dequant_q5k, retile_q5k, gemm_q5k, dequant_q6k, retile_q6k, gemm_q6k;
     hipFunction_t gemm_q4k_gateup;
     hipFunction_t kv_store, qkv_rope_store, attn_partial, attn_combine, attn_combine_quant;

@@ -362,22 +362,26 @@ extern "C" int rd_model_finalize(rd_model *m) {
     }
     pf = std::max(pf, gemm_partial_floats(m->head));
     int H = c.hidden, qd = c.n_heads * c.head_dim;
+    m->max_rows = c.n_experts > 0 ? 32 : rd_model::ROWS_MAX;
+    const size_t R = (size_t)m->max_rows, tiles = R / 32;
     m->P_floats = pf;
-    RC(alloc_f32(d, &m->P, pf));
-    RC(alloc_f32(d, &m->h, (size_t)32 * H));
-    RC(alloc_f32(d, &m->emb_dev, (size_t)32 * H));
+    m->pStride = pf;
+    RC(alloc_f32(d, &m->P, pf * tiles));
+    RC(alloc_f32(d, &m->h, R * H));
+    RC(alloc_f32(d, &m->emb_dev, R * H));
     RC(alloc_f32(d, &m->normed, (size_t)32 * H));
-    RC(alloc_f32(d, &m->qbuf, (size_t)32 * qd));
-    RC(alloc_f32(d, &m->logits, (size_t)32 * c.vocab));
+    RC(alloc_f32(d, &m->qbuf, R * qd));
+    RC(alloc_f32(d, &m->logits, R * c.vocab));
     size_t kA = (size_t)H, kB = (size_t)std::max(qd, c.n_experts ? qd : c.inter);
     // room for either panel kind: 8 KB per 128 elements (int8/int4 consumers) or 17 KB per 256 (Q4_K consumers)
     auto panel_room = [](size_t K) { return std::max(((K + 127) / 128) * (size_t)LIN_PANEL_BYTES, ((K + 255) / 256) * (size_t)Q4K_PANEL_BYTES); };
-    RC(d->alloc(&m->XpA, panel_room(kA)));
-    RC(d->alloc(&m->XpA2, panel_room(kA)));
-    RC(d->alloc(&m->XpB, panel_room(kB)));
-    RC(d->alloc((void **)&m->ids, sizeof(int) * 32));
-    RC(alloc_f32(d, &m->cand_v, (size_t)32 * ((c.vocab + 4095) / 4096)));
-    RC(d->alloc((void **)&m->cand_i, sizeof(int) * 32 * (size_t)((c.vocab + 4095) / 4096)));
+    m->xpAStride = panel_room(kA), m->xpBStride = panel_room(kB);
+    RC(d->alloc(&m->XpA, m->xpAStride * tiles));
+    RC(d->alloc(&m->XpA2, m->xpAStride * tiles));
+    RC(d->alloc(&m->XpB, m->xpBStride * tiles));
+    RC(d->alloc((void **)&m->ids, sizeof(int) * R));
+    RC(alloc_f32(d, &m->cand_v, R * ((c.vocab + 4095) / 4096)));
+    RC(d->alloc((void **)&m->cand_i, sizeof(int) * R * (size_t)((c.vocab + 4095) / 4096)));
     if (c.n_experts > 0) {
         int k = c.top_k, I = c.expert_inter;
         RC(alloc_f32(d, &m->router_logits, (size_t)32 * c.n_experts));
@@ -391,7 +395,7 @@ extern "C" int rd_model_finalize(rd_model *m) {
         RC(d->alloc(&m->XpE, (size_t)c.n_experts * (I / 128) * LIN_PANEL_BYTES));
         HIPCHK(MemsetAsync(m->XpE, 0, (size_t)c.n_experts * (I / 128) * LIN_PANEL_BYTES, d->stream));
     }
-    m->host_stage_bytes = sizeof(float) * (size_t)32 * H + (1u << 20);
+    m->host_stage_bytes = sizeof(float) * R * H + (1u << 20);
     HIPCHK(HostMalloc(&m->host_stage, m->host_stage_bytes * rd_model::STAGE_SLOTS, 0));
     for (auto &e : m->stage_ev) HIPCHK(EventCreate(&e));
     m->finalized = true;
@@ -444,15 +448,16 @@ extern "C" int rd_kv_configure_typed(rd_model *m, int slots, int ctx_cap, int kv
     RC(d->h2d(m->tables, tab.data(), sizeof(int) * tab.size()));
     m->slot_len.assign((size_t)slots, 0);
     // attention work list: ~4096 items plus one per (row, kv head) of rounding
-    m->max_items = 32 * c.n_kv_heads * ATTN_PIECES;
+    m->max_items = m->max_rows * c.n_kv_heads * ATTN_PIECES;
     int G = c.n_heads / c.n_kv_heads;
     RC(alloc_f32(d, &m->part, (size_t)m->max_items * G * (c.head_dim + 2)));
     // The step's metadata lives in one device block so a step uploads it with one copy:
-    // [row slot 32][row position 32][row length 32][row draw records 32 x 6][item ranges 32*nKV*2][items max_items x 4] ints
-    const size_t rangeInts = (size_t)32 * c.n_kv_heads * 2;
+    // [row slot R][row position R][row length R][row draw records R x 6][item ranges max_rows*nKV*2][items max_items x 4] ints, R = ROWS_MAX
+    const size_t rangeInts = (size_t)m->max_rows * c.n_kv_heads * 2;
     m->meta_ints = rd_model::META_HDR + rangeInts + (size_t)m->max_items * 4;
     RC(d->alloc((void **)&m->meta, sizeof(int) * m->meta_ints));
-    m->rowSlot = m->meta, m->rowPos = m->meta + 32, m->rowLen = m->meta + 64, m->rowDraw = m->meta + 96;
+    constexpr int RM = rd_model::ROWS_MAX;
+    m->rowSlot = m->meta, m->rowPos = m->meta + RM, m->rowLen = m->meta + 2 * RM, m->rowDraw = m->meta + 3 * RM;
     m->itemStart = m->meta + rd_model::META_HDR;
     m->items = (AttnItemH *)(m->meta + rd_model::META_HDR + rangeInts);
     return d->sync();
@@ -518,7 +523,7 @@ struct Scope { // times one kernel class when the model's timer is on
 };
 
 static int build_attn_items(rd_model *m, int B, const int *pos, std::vector<AttnItemH> &items, std::vector<int> &ranges) {
-    int len[32];
+    int len[rd_model::ROWS_MAX];
     for (int b = 0; b < B; b++) len[b] = pos[b] + 1;
     build_attn_worklist(len, B, m->desc.n_kv_heads, items, ranges);
     if ((int)items.size() > m->max_items) {
@@ -546,21 +551,21 @@ static int add_norm_quant(rd_model *m, int B, const float *P, int splits, const 
     int kA, kB;
     panel_kinds_of(next, &kA, &kB);
     return d->launch(d->k.add_rmsnorm_quant, (unsigned)B, 1, 1, 1024, m->h, P, splits, w, m->desc.rms_eps, m->desc.hidden, Xp, kA, norm_out,
-                     kB >= 0 ? m->XpA2 : (void *)nullptr, kB);
+                     kB >= 0 ? m->XpA2 : (void *)nullptr, kB, m->pStride, m->xpAStride, m->xpAStride);
 }
 
 // One GEMM, or for a group one GEMM per member into column ranges of the same P[split][32][N], all with the group's split
 // count so that the consumer sums the same number of partials for every column.
-static int launch_proj(rd_model *m, const DevWeight &w, const void *Xp, int B, GemmPlan *plan) {
+static int launch_proj(rd_model *m, const DevWeight &w, const void *Xp, size_t xpStride, int B, GemmPlan *plan) {
     rd_device *d = m->d;
-    if (w.kind != WKIND_GROUP) return launch_gemm(d, w, Xp, m->P, B, plan);
+    if (w.kind != WKIND_GROUP) return launch_gemm_wide(d, w, Xp, xpStride, m->P, m->pStride, B, plan);
     int kA, kB;
     panel_kinds_of(w, &kA, &kB);
     GemmPlan g = plan_gemm(0, w.N, w.K / 256 > 0 ? w.K / 256 : 1);
     for (const auto &p : w.parts) g.splits = std::min(g.splits, std::max(1, kblocks_for(p))); // no member gets more splits than K-blocks
     for (size_t i = 0; i < w.parts.size(); i++) {
         const DevWeight &p = w.parts[i];
-        RC(launch_gemm(d, p, panel_kind_for(p) == kA ? Xp : m->XpA2, m->P + w.col0[i], B, nullptr, w.N, g.splits));
+        RC(launch_gemm_wide(d, p, panel_kind_for(p) == kA ? Xp : m->XpA2, xpStride, m->P + w.col0[i], m->pStride, B, nullptr, w.N, g.splits));
     }
     g.kbPerSplit = 0;
     if (plan) *plan = g;
@@ -624,8 +629,8 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
         rd_set_error("a chain is open: between its start and stop the resident takes no other step");
         return RD_ERR_STATE;
     }
-    if (B < 1 || B > 32) {
-        rd_set_error("rocm resident: batch %d outside the stepper range 1..32", B);
+    if (B < 1 || B > m->max_rows) {
+        rd_set_error("rocm resident: batch %d outside the stepper range 1..%d", B, m->max_rows);
         return RD_ERR_ARG;
     }
     // A slot may carry several rows in one step if they sit at consecutive positions (a ragged step's verify or prefill
@@ -661,14 +666,15 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
     {
         char *st = (char *)m->host_stage + (size_t)stage_slot * m->host_stage_bytes;
         int *hm = (int *)st; // the metadata block, laid out as on the device
-        const size_t rangeInts = (size_t)32 * nKV * 2;
+        const size_t rangeInts = (size_t)m->max_rows * nKV * 2;
+        constexpr int RM = rd_model::ROWS_MAX;
         float *eh = (float *)(st + (1u << 20));
-        for (int b = 0; b < B; b++) hm[b] = slot[b], hm[32 + b] = pos[b], hm[64 + b] = pos[b] + 1;
+        for (int b = 0; b < B; b++) hm[b] = slot[b], hm[RM + b] = pos[b], hm[2 * RM + b] = pos[b] + 1;
         // Draw records (resident/forward.go:43-52 BatchDraw) with Sampler.gumbelDraw's guards applied here
         // (internal/runtime/sampling/sampler_gumbel.go:80-88): a temperature <= 0 means 1, and one so small that 1/T
         // overflows f32 is the plain argmax.
-        for (int b = 0; b < 32; b++) {
-            int *r = hm + 96 + b * 6;
+        for (int b = 0; b < RM; b++) {
+            int *r = hm + 3 * RM + b * 6;
             memset(r, 0, sizeof(int) * 6);
             if (b >= B || !m->step_draws) continue;
             const rd_draw &dw = m->step_draws[b];
@@ -714,7 +720,7 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
         RC(add_norm_quant(m, B, resP, resSplits, l.attn_norm, l.qkv, m->XpA, nullptr));
         {
             Scope s(m, KC_GEMM_QKV);
-            RC(launch_proj(m, l.qkv, m->XpA, B, &plan));
+            RC(launch_proj(m, l.qkv, m->XpA, m->xpAStride, B, &plan));
         }
         {
             Scope s(m, KC_ROPE_STORE);
@@ -722,11 +728,11 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
                 RC(d->launch(d->k.qkv_rope_store_i8, (unsigned)(nH + 2 * nKV), (unsigned)B, 1, (unsigned)(HD / 2), (const float *)m->P, plan.splits, m->qbuf,
                              (signed char *)l.Kp, (signed char *)l.Vp, l.Ksc, l.Vsc, (const int *)m->tables, m->blocks_per_slot, (const int *)m->rowSlot,
                              (const int *)m->rowPos, (const double *)m->inv_freq_dev, (const float *)l.q_norm, (const float *)l.k_norm, c.rms_eps, nH, nKV,
-                             HD));
+                             HD, m->pStride));
             else
                 RC(d->launch(d->k.qkv_rope_store, (unsigned)(nH + 2 * nKV), (unsigned)B, 1, (unsigned)(HD / 2), (const float *)m->P, plan.splits, m->qbuf,
                          l.Kp, l.Vp, (const int *)m->tables, m->blocks_per_slot, (const int *)m->rowSlot, (const int *)m->rowPos,
-                         (const double *)m->inv_freq_dev, (const float *)l.q_norm, (const float *)l.k_norm, c.rms_eps, nH, nKV, HD));
+                         (const double *)m->inv_freq_dev, (const float *)l.q_norm, (const float *)l.k_norm, c.rms_eps, nH, nKV, HD, m->pStride));
         }
         {
             Scope s(m, KC_ATTN_PARTIAL);
@@ -742,37 +748,37 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
         {
             Scope s(m, KC_ATTN_COMBINE);
             RC(d->launch(d->k.attn_combine_quant, (unsigned)nH, (unsigned)B, 1, (unsigned)(ATTN_PIECES * HD / 4), (const float *)m->part, (const int *)m->itemStart,
-                         m->XpB, panel_kind_for(l.o), nH, nKV, HD));
+                         m->XpB, panel_kind_for(l.o), nH, nKV, HD, m->xpBStride));
         }
         {
             Scope s(m, KC_GEMM_O);
-            RC(launch_gemm(d, l.o, m->XpB, m->P, B, &plan));
+            RC(launch_gemm_wide(d, l.o, m->XpB, m->xpBStride, m->P, m->pStride, B, &plan));
         }
         if (c.n_experts == 0) {
             RC(add_norm_quant(m, B, m->P, plan.splits, l.ffn_norm, l.gateup, m->XpA, nullptr));
-            if (l.gateup.kind == 0 && c.inter % 64 == 0 && !getenv("ROCMDECODE_NO_FUSED_GATEUP")) {
+            if (B <= 32 && l.gateup.kind == 0 && c.inter % 64 == 0 && !getenv("ROCMDECODE_NO_FUSED_GATEUP")) {
                 Scope s(m, KC_GEMM_GATEUP); // gate|up GEMM + SwiGLU + quantization in one launch
                 RC(d->launch(d->k.gemm_q4k_gateup, (unsigned)(c.inter / 64), 1, 1, GATEUP_THREADS, (const void *)l.gateup.tiled, (const void *)m->XpA, m->XpB,
                              panel_kind_for(l.down), c.inter, H / 256, B));
             } else {
                 {
                     Scope s(m, KC_GEMM_GATEUP);
-                    RC(launch_proj(m, l.gateup, m->XpA, B, &plan));
+                    RC(launch_proj(m, l.gateup, m->XpA, m->xpAStride, B, &plan));
                 }
                 Scope s(m, KC_SWIGLU);
                 RC(d->launch(d->k.swiglu_quant, (unsigned)((c.inter + 1023) / 1024), (unsigned)B, 1, 256, (const float *)m->P, plan.splits, c.inter,
-                             m->XpB, panel_kind_for(l.down), (float *)nullptr));
+                             m->XpB, panel_kind_for(l.down), (float *)nullptr, m->pStride, m->xpBStride));
             }
             {
                 Scope s(m, KC_GEMM_DOWN);
-                RC(launch_gemm(d, l.down, m->XpB, m->P, B, &plan));
+                RC(launch_gemm_wide(d, l.down, m->XpB, m->xpBStride, m->P, m->pStride, B, &plan));
             }
             resP = m->P, resSplits = plan.splits;
         } else {
             {
                 Scope s(m, KC_ADD_NORM);
                 RC(d->launch(d->k.add_rmsnorm_quant, (unsigned)B, 1, 1, 1024, m->h, (const float *)m->P, plan.splits, (const float *)l.ffn_norm,
-                             c.rms_eps, H, m->XpA, (int)PANEL_LIN4, m->normed, (void *)nullptr, -1));
+                             c.rms_eps, H, m->XpA, (int)PANEL_LIN4, m->normed, (void *)nullptr, -1, m->pStride, m->xpAStride, m->xpAStride));
             }
             RC(moe_ffn(m, B, li, l));
             resP = m->moe_out, resSplits = 1;
@@ -783,13 +789,13 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
         RC(add_norm_quant(m, B, resP, resSplits, m->final_norm, m->head, m->XpA, nullptr));
         {
             Scope s(m, KC_GEMM_HEAD);
-            RC(launch_gemm(d, m->head, m->XpA, m->P, B, &plan));
+            RC(launch_gemm_wide(d, m->head, m->XpA, m->xpAStride, m->P, m->pStride, B, &plan));
         }
         {
             Scope s(m, KC_ARGMAX);
             int nChunks = (c.vocab + 4095) / 4096;
             RC(d->launch(d->k.argmax_rows, (unsigned)nChunks, (unsigned)B, 1, 256, (const float *)m->P, plan.splits, c.vocab, m->cand_v, m->cand_i,
-                         (want & RD_WANT_LOGITS) ? m->logits : (float *)nullptr, (const int *)(m->step_draws ? m->rowDraw : nullptr)));
+                         (want & RD_WANT_LOGITS) ? m->logits : (float *)nullptr, (const int *)(m->step_draws ? m->rowDraw : nullptr), m->pStride));
             if (want & RD_WANT_ARGMAX) RC(d->launch(d->k.argmax_final, (unsigned)B, 1, 1, 64, (const float *)m->cand_v, (const int *)m->cand_i, nChunks, m->ids));
         }
     }
@@ -940,7 +946,7 @@ extern "C" int rd_step_batch_draw(rd_model *m, int B, const int *slot, const int
         rd_set_error("rd_step_batch_draw: want=%d needs its output buffer", want);
         return RD_ERR_ARG;
     }
-    for (int b = 0; b < B && b < 32; b++)
+    for (int b = 0; b < B && b < m->max_rows; b++)
         if (draws[b].mode < RD_DRAW_NONE || draws[b].mode > RD_DRAW_GUMBEL || (draws[b].mode == RD_DRAW_GUMBEL && std::isnan(draws[b].temperature))) {
             rd_set_error("rd_step_batch_draw: row %d has draw mode %d, temperature %g", b, draws[b].mode, draws[b].temperature);
             return RD_ERR_ARG;
@@ -955,7 +961,7 @@ extern "C" int rd_step_batch_draw(rd_model *m, int B, const int *slot, const int
 }
 
 // resident/subsystems.go:112-117 StepRagged, forward.go:9-16 ForwardN, subsystems.go:124 PrefillLast: sequences of one or more
-// rows at consecutive positions. Rows go through the step's kernels in passes of at most 32 (the GEMMs' row tile), in the
+// rows at consecutive positions. Rows go through the step's kernels in passes of at most 128 (four GEMM row tiles; 32 for a MoE model), in the
 // order given; a sequence longer than a pass simply continues in the next one.
 extern "C" int rd_step_ragged(rd_model *m, int n_seq, const int *slot, const int *pos, const int *n_rows, const float *emb, int want, float *logits,
                               int *ids) {
@@ -992,8 +998,9 @@ extern "C" int rd_step_ragged(rd_model *m, int n_seq, const int *slot, const int
         for (int j = 0; j < n_rows[i]; j++) rslot.push_back(slot[i]), rpos.push_back(pos[i] + j);
     }
     const size_t H = (size_t)m->desc.hidden, V = (size_t)m->desc.vocab;
-    for (size_t r0 = 0; r0 < rslot.size(); r0 += 32) {
-        const int rows = (int)std::min<size_t>(32, rslot.size() - r0);
+    const size_t pass = (size_t)m->max_rows; // rows per pass: the step's widest batch
+    for (size_t r0 = 0; r0 < rslot.size(); r0 += pass) {
+        const int rows = (int)std::min<size_t>(pass, rslot.size() - r0);
         RC(model_step(m, rows, rslot.data() + r0, rpos.data() + r0, emb + r0 * H, nullptr, want, logits ? logits + r0 * V : nullptr,
                       ids ? ids + r0 : nullptr, true));
     }
@@ -1042,8 +1049,9 @@ extern "C" int rd_step_ragged_draw(rd_model *m, int n_seq, const int *slot, cons
     }
     const size_t H = (size_t)m->desc.hidden, V = (size_t)m->desc.vocab;
     int rc = RD_OK;
-    for (size_t r0 = 0; r0 < rslot.size() && !rc; r0 += 32) {
-        const int rows = (int)std::min<size_t>(32, rslot.size() - r0);
+    const size_t pass = (size_t)m->max_rows;
+    for (size_t r0 = 0; r0 < rslot.size() && !rc; r0 += pass) {
+        const int rows = (int)std::min<size_t>(pass, rslot.size() - r0);
         m->step_draws = rdraw.data() + r0;
         rc = model_step(m, rows, rslot.data() + r0, rpos.data() + r0, emb + r0 * H, nullptr, want | RD_WANT_ARGMAX, logits ? logits + r0 * V : nullptr,
                         ids + r0, true);
@@ -1079,16 +1087,18 @@ extern "C" int rd_prefill_last(rd_model *m, int slot, int start_pos, int n, cons
         return RD_ERR_KV_FULL;
     }
     const size_t H = (size_t)m->desc.hidden;
-    std::vector<int> rslot(32, slot), rpos(32);
-    std::vector<float> tail; // the last pass returns its rows' logits; only the final row is handed on
-    for (int r0 = 0; r0 < n; r0 += 32) {
-        const int rows = std::min(32, n - r0);
-        const bool last = r0 + rows == n;
+    // All rows but the last only build their K/V (no final norm, no head, nothing read back), in passes as wide as the step
+    // takes; the last row is an ordinary one-row step whose logits are the answer. Each row is the row its own single-token
+    // forward computes, whatever pass it rides in.
+    const int pass = m->max_rows;
+    std::vector<int> rslot((size_t)pass, slot), rpos((size_t)pass);
+    for (int r0 = 0; r0 < n - 1; r0 += pass) {
+        const int rows = std::min(pass, n - 1 - r0);
         for (int j = 0; j < rows; j++) rpos[(size_t)j] = start_pos + r0 + j;
-        if (last) tail.resize((size_t)rows * m->desc.vocab);
-        RC(model_step(m, rows, rslot.data(), rpos.data(), emb + (size_t)r0 * H, nullptr, last ? RD_WANT_LOGITS : 0, last ? tail.data() : nullptr, nullptr, true));
-        if (last) memcpy(logits, tail.data() + (size_t)(rows - 1) * m->desc.vocab, sizeof(float) * (size_t)m->desc.vocab);
+        RC(model_step(m, rows, rslot.data(), rpos.data(), emb + (size_t)r0 * H, nullptr, 0, nullptr, nullptr, true));
     }
+    const int lastPos = start_pos + n - 1;
+    RC(model_step(m, 1, &slot, &lastPos, emb + (size_t)(n - 1) * H, nullptr, RD_WANT_LOGITS, logits, nullptr, false));
     return RD_OK;
 }
 

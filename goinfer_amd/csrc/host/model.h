@@ -67,7 +67,12 @@ struct rd_model {
         hipEvent_t ev[DEPTH] = {};
     } chain;
     int kv_type = 0; // RD_KV_F16 or RD_KV_I8
-    static constexpr int META_HDR = 96 + 32 * 6; // row slot, position, length (32 each) and the rows' draw records (6 ints each)
+    // Rows per step: up to ROWS_MAX as M-tiles of 32 (a dense model; MoE steps keep to one M-tile). The step's buffers hold
+    // max_rows rows; partial sums and panels are per M-tile, pStride floats / xpStride bytes apart.
+    static constexpr int ROWS_MAX = 128;
+    int max_rows = 32;
+    size_t pStride = 0, xpAStride = 0, xpBStride = 0;
+    static constexpr int META_HDR = 3 * ROWS_MAX + ROWS_MAX * 6; // row slot, position, length and the rows' draw records (6 ints each)
     int *rowDraw = nullptr;               // inside meta
     const rd_draw *step_draws = nullptr;  // set by the entry point for the one step it runs; null = plain argmax for every row
     void *XpA = nullptr, *XpB = nullptr;

@@ -84,9 +84,15 @@ extern "C" __global__ void rd_k_reduce_splits(const float *__restrict__ P, float
 extern "C" __global__ __launch_bounds__(1024) void rd_k_add_rmsnorm_quant(float *__restrict__ h, const float *__restrict__ P, int splits,
                                                                           const float *__restrict__ w, float eps, int H,
                                                                           uint8_t *__restrict__ Xp, int kind, float *__restrict__ norm_out,
-                                                                          uint8_t *__restrict__ Xp2, int kind2) {
+                                                                          uint8_t *__restrict__ Xp2, int kind2, size_t pStride, size_t xpStride,
+                                                                          size_t xp2Stride) {
     __shared__ double red[16];
     const int m = blockIdx.x, t = threadIdx.x, nv = H >> 2;
+    // rows beyond 32 are further M-tiles: their partial sums and panels sit pStride floats / xpStride bytes further on
+    const int mt = m >> 5, mr = m & 31;
+    if (P) P += (size_t)mt * pStride;
+    Xp += (size_t)mt * xpStride;
+    if (Xp2) Xp2 += (size_t)mt * xp2Stride;
     float4_t v[2];
     bool on[2];
     double ss = 0;
@@ -107,14 +113,14 @@ extern "C" __global__ __launch_bounds__(1024) void rd_k_add_rmsnorm_quant(float 
         float4_t a[2];
 #pragma unroll
         for (int i = 0; i < 2; i++)
-            if (on[i]) a[i] = *(const float4_t *)(P + (size_t)m * H + 4 * (t + i * 1024));
+            if (on[i]) a[i] = *(const float4_t *)(P + (size_t)mr * H + 4 * (t + i * 1024));
         for (int s0 = 1; s0 < splits; s0 += 8) {
             float4_t b[2][8];
 #pragma unroll
             for (int j = 0; j < 8; j++)
 #pragma unroll
                 for (int i = 0; i < 2; i++)
-                    if (on[i] && s0 + j < splits) b[i][j] = *(const float4_t *)(P + ((size_t)(s0 + j) * 32 + m) * H + 4 * (t + i * 1024));
+                    if (on[i] && s0 + j < splits) b[i][j] = *(const float4_t *)(P + ((size_t)(s0 + j) * 32 + mr) * H + 4 * (t + i * 1024));
 #pragma unroll
             for (int j = 0; j < 8; j++)
 #pragma unroll
@@ -150,16 +156,18 @@ extern "C" __global__ __launch_bounds__(1024) void rd_k_add_rmsnorm_quant(float 
         if (norm_out) *(float4_t *)(norm_out + (size_t)m * H + k0) = (float4_t){n0, n1, n2, n3};
         float x0, x1, x2, x3, gs;
         quant_g32x4(n0, n1, n2, n3, &x0, &x1, &x2, &x3, &gs);
-        panel_store4(Xp, kind, m, k0, x0, x1, x2, x3, gs);
-        if (Xp2) panel_store4(Xp2, kind2, m, k0, x0, x1, x2, x3, gs); // a second consumer that reads another panel layout
+        panel_store4(Xp, kind, mr, k0, x0, x1, x2, x3, gs);
+        if (Xp2) panel_store4(Xp2, kind2, mr, k0, x0, x1, x2, x3, gs); // a second consumer that reads another panel layout
     }
 }
 
 // gate/up partials P[s][32][2I] -> act = silu(gate)*up (decoder/rmsnorm.go:204-207: silu in f64) -> per-32 quant -> panels.
 // Grid (ceil(I/1024), M), 256 threads, four consecutive columns per thread. I % 32 == 0.
 extern "C" __global__ __launch_bounds__(256) void rd_k_swiglu_quant(const float *__restrict__ P, int splits, int I, uint8_t *__restrict__ Xp,
-                                                                    int kind, float *__restrict__ act_out) {
-    int m = blockIdx.y, n0 = (blockIdx.x * 256 + threadIdx.x) * 4;
+                                                                    int kind, float *__restrict__ act_out, size_t pStride, size_t xpStride) {
+    const int row = blockIdx.y, m = row & 31, n0 = (blockIdx.x * 256 + threadIdx.x) * 4;
+    P += (size_t)(row >> 5) * pStride; // M-tile of this row
+    Xp += (size_t)(row >> 5) * xpStride;
     bool on = n0 < I; // groups of 8 lanes are on or off together
     float a[4] = {0.f, 0.f, 0.f, 0.f};
     if (on) {
@@ -174,7 +182,7 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_swiglu_quant(const float 
         for (int i = 0; i < 4; i++) {
             a[i] = __fmul_rn(silu_f64(g[i]), u[i]);
         }
-        if (act_out) *(float4_t *)(act_out + (size_t)m * I + n0) = (float4_t){a[0], a[1], a[2], a[3]};
+        if (act_out) *(float4_t *)(act_out + (size_t)row * I + n0) = (float4_t){a[0], a[1], a[2], a[3]};
     }
     float x0, x1, x2, x3, gs;
     quant_g32x4(a[0], a[1], a[2], a[3], &x0, &x1, &x2, &x3, &gs);

@@ -99,13 +99,14 @@ __device__ __forceinline__ void qkv_rope_store_body(const float *__restrict__ P,
                                                void *__restrict__ VpV, float *__restrict__ Ksc, float *__restrict__ Vsc,
                                                const int *__restrict__ tables, int tabStride,
                                                const int *__restrict__ rowSlot, const int *__restrict__ rowPos, const double *__restrict__ invFreq,
-                                               const float *__restrict__ qnorm, const float *__restrict__ knorm, float eps, int nH, int nKV, int HD) {
+                                               const float *__restrict__ qnorm, const float *__restrict__ knorm, float eps, int nH, int nKV, int HD,
+                                               size_t pStride) {
     int head = blockIdx.x, m = blockIdx.y, t = threadIdx.x, half = HD / 2; // one wave: half <= 64
     int Ntot = (nH + 2 * nKV) * HD, pos = rowPos[m];
     // everything this thread will need from memory is requested up front: one latency instead of a chain of them
     const int slotRow = rowSlot[m];
     const double invf = invFreq[t];
-    const float *src = P + (size_t)m * Ntot + (size_t)head * HD;
+    const float *src = P + (size_t)(m >> 5) * pStride + (size_t)(m & 31) * Ntot + (size_t)head * HD; // M-tile m/32, row m%32
     float x1 = src[t], x2 = src[t + half];
     for (int s0 = 1; s0 < splits; s0 += 8) { // ascending split order; eight splits' loads in flight together
         float a1[8], a2[8];
@@ -164,16 +165,17 @@ __device__ __forceinline__ void qkv_rope_store_body(const float *__restrict__ P,
 extern "C" __global__ void rd_k_qkv_rope_store(const float *__restrict__ P, int splits, float *__restrict__ q, uint16_t *__restrict__ Kp,
                                                uint16_t *__restrict__ Vp, const int *__restrict__ tables, int tabStride,
                                                const int *__restrict__ rowSlot, const int *__restrict__ rowPos, const double *__restrict__ invFreq,
-                                               const float *__restrict__ qnorm, const float *__restrict__ knorm, float eps, int nH, int nKV, int HD) {
-    qkv_rope_store_body<false>(P, splits, q, Kp, Vp, nullptr, nullptr, tables, tabStride, rowSlot, rowPos, invFreq, qnorm, knorm, eps, nH, nKV, HD);
+                                               const float *__restrict__ qnorm, const float *__restrict__ knorm, float eps, int nH, int nKV, int HD,
+                                               size_t pStride) {
+    qkv_rope_store_body<false>(P, splits, q, Kp, Vp, nullptr, nullptr, tables, tabStride, rowSlot, rowPos, invFreq, qnorm, knorm, eps, nH, nKV, HD, pStride);
 }
 // The same into the int8 cache: the K or V head is quantized with its own scale after RoPE (backend/cuda/kv8_store.cu).
 extern "C" __global__ void rd_k_qkv_rope_store_i8(const float *__restrict__ P, int splits, float *__restrict__ q, signed char *__restrict__ Kp,
                                                   signed char *__restrict__ Vp, float *__restrict__ Ksc, float *__restrict__ Vsc,
                                                   const int *__restrict__ tables, int tabStride, const int *__restrict__ rowSlot,
                                                   const int *__restrict__ rowPos, const double *__restrict__ invFreq, const float *__restrict__ qnorm,
-                                                  const float *__restrict__ knorm, float eps, int nH, int nKV, int HD) {
-    qkv_rope_store_body<true>(P, splits, q, Kp, Vp, Ksc, Vsc, tables, tabStride, rowSlot, rowPos, invFreq, qnorm, knorm, eps, nH, nKV, HD);
+                                                  const float *__restrict__ knorm, float eps, int nH, int nKV, int HD, size_t pStride) {
+    qkv_rope_store_body<true>(P, splits, q, Kp, Vp, Ksc, Vsc, tables, tabStride, rowSlot, rowPos, invFreq, qnorm, knorm, eps, nH, nKV, HD, pStride);
 }
 
 typedef float float4v __attribute__((ext_vector_type(4)));

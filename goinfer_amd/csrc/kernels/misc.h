@@ -60,10 +60,11 @@ __device__ __forceinline__ float gumbel_noise(uint32_t h) {
 // draw hi, 0), key seed), and a thread's four consecutive entries are exactly one Philox call.
 extern "C" __global__ __launch_bounds__(256) void rd_k_argmax_rows(const float *__restrict__ P, int splits, int N, float *__restrict__ cand_v,
                                                                    int *__restrict__ cand_i, float *__restrict__ logits_out,
-                                                                   const int *__restrict__ rowDraw) {
+                                                                   const int *__restrict__ rowDraw, size_t pStride) {
     __shared__ float bv[4];
     __shared__ int bi[4];
-    const int m = blockIdx.y, t = threadIdx.x, nChunks = gridDim.x;
+    const int m = blockIdx.y, t = threadIdx.x, nChunks = gridDim.x, mr = m & 31;
+    P += (size_t)(m >> 5) * pStride; // rows beyond 32 are further M-tiles of partial sums
     const int *dr = rowDraw ? rowDraw + m * RD_DRAW_INTS : nullptr;
     const bool gumbel = dr && dr[0] == 2;
     const float invT = gumbel ? __int_as_float(dr[1]) : 1.f;
@@ -73,9 +74,9 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_argmax_rows(const float *
     for (int i = 0; i < 4; i++) {
         int n0 = blockIdx.x * 4096 + (i * 256 + t) * 4;
         if (n0 < N) {
-            float4_t a = *(const float4_t *)(P + (size_t)m * N + n0);
+            float4_t a = *(const float4_t *)(P + (size_t)mr * N + n0);
             for (int s = 1; s < splits; s++) {
-                float4_t b = *(const float4_t *)(P + ((size_t)s * 32 + m) * N + n0);
+                float4_t b = *(const float4_t *)(P + ((size_t)s * 32 + mr) * N + n0);
                 a.x = __fadd_rn(a.x, b.x), a.y = __fadd_rn(a.y, b.y), a.z = __fadd_rn(a.z, b.z), a.w = __fadd_rn(a.w, b.w);
             }
             if (logits_out) *(float4_t *)(logits_out + (size_t)m * N + n0) = a;

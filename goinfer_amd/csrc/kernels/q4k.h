@@ -238,6 +238,14 @@ extern "C" __global__ __launch_bounds__(512) void rd_k_gemm_q4k_wide(const uint8
     gemm_body_wide<Q4KTraits, 4, RD_GEMM_WIDE_MT, 3>(Wt, nullptr, Xp, xpStride, P, pStride, N, nSB, sbPerSplit, M, ldP, lds);
 }
 
+// 33 to 64 rows: two M-tiles, block 384, 68 KB of LDS (two blocks per CU).
+extern "C" __global__ __launch_bounds__(384) void rd_k_gemm_q4k_wide2(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ Xp, size_t xpStride,
+                                                                       float *__restrict__ P, size_t pStride, int N, int nSB, int sbPerSplit, int M,
+                                                                       int ldP) {
+    __shared__ uint4_t lds[2 * 2 * RD_Q4K_PANEL_BYTES / 16];
+    gemm_body_wide<Q4KTraits, 4, 2, 3>(Wt, nullptr, Xp, xpStride, P, pStride, N, nSB, sbPerSplit, M, ldP, lds);
+}
+
 // Fused gate/up projection + SwiGLU + per-32 quantization (goinfer decoder/cpu_gateup_fused.go:83-148, in one launch):
 // W holds [gate rows; up rows] (2*I rows). Block b: waves 0,1 own gate tiles 2b,2b+1, waves 2,3 the matching up tiles, all over
 // the full K (no split, so the sums are complete in registers). The up waves hand their sums over through LDS; the gate waves

@@ -195,3 +195,27 @@ def test_i8_kv_uploaded_prefix(dev):
     d_f16, d_i8 = uploaded_prefix_deviation(dev, "f16"), uploaded_prefix_deviation(dev, "i8")
     print("uploaded prefix: deviation f16 %.4f, i8 %.4f" % (d_f16, d_i8))
     assert d_i8 <= max(2e-2, 1.5 * d_f16), (d_i8, d_f16)
+
+
+def test_wide_batch_rows_equal_solo_rows(dev):
+    """A dense model steps up to 128 rows at once (four GEMM row tiles): every row is still the row its own one-row step computes,
+    bit for bit, whatever tile it rides in; a batch past the range is refused."""
+    cfg = dense_cfg(n_layers=2)
+    B = 70
+    pair = Pair(cfg, seed=61, dev=dev, slots=2 * B, ctx_cap=32)
+    try:
+        rng = np.random.default_rng(6)
+        pos = [0] * B
+        for step in range(3):
+            toks = rng.integers(0, cfg["vocab"], B)
+            emb = pair.emb[toks]
+            got, ids = pair.gpu.step_batch(list(range(B)), pos, emb, capi.WANT_LOGITS | capi.WANT_ARGMAX)
+            for b in (0, 31, 32, 33, 63, 64, 69):
+                solo = pair.gpu.forward(B + b, pos[b], emb[b])
+                assert np.array_equal(solo.view(np.uint32), got[b].view(np.uint32)), (step, b)
+                assert ids[b] == int(np.argmax(got[b]))
+            pos = [p + 1 for p in pos]  # the twin slots of the checked rows advance with them; the other twins are never read
+        with pytest.raises(capi.RocmError, match="stepper range"):
+            pair.gpu.step_batch(list(range(129)), [0] * 129, pair.emb[:129])
+    finally:
+        pair.close()
