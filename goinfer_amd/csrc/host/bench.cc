@@ -18,7 +18,7 @@
 // milliseconds; ids_out (optional) [steps][B] are the tokens picked.
 extern "C" int rd_bench_steps(rd_model *m, int B, const int *slot, const int *pos0, const int *ids0, int warmup, int steps, float *ms_out,
                               int *ids_out) {
-    if (!m || !slot || !pos0 || !ids0 || !ms_out || steps <= 0 || warmup < 0 || B < 1 || B > 32) return RD_ERR_ARG;
+    if (!m || !slot || !pos0 || !ids0 || !ms_out || steps <= 0 || warmup < 0 || B < 1 || B > m->max_rows) return RD_ERR_ARG;
     rd_device *d = m->d;
     RC(d->h2d(m->ids, ids0, sizeof(int) * (size_t)B));
     RC(d->sync());
