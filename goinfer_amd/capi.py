@@ -21,7 +21,7 @@ EXPORTS = [
     "rd_kv_configure", "rd_kv_upload", "rd_kv_truncate", "rd_kv_reset", "rd_step_batch", "rd_forward",
     "rd_last_moe_indices", "rd_model_upload_embedding", "rd_bench_steps", "rd_bench_profile", "rd_bench_class_count",
     "rd_bench_class_name", "rd_bench_kernel", "rd_gateup_q4k_quant", "rd_moe_replay", "rd_bench_attn", "rd_step_ragged", "rd_prefill_last",
-    "rd_kv_configure_typed", "rd_attn_ragged_i8", "rd_bench_attn_i8", "rd_step_ragged_draw", "rd_forward_no_logits",
+    "rd_kv_configure_typed", "rd_attn_ragged_i8", "rd_attn_ragged_rows", "rd_bench_attn_i8", "rd_step_ragged_draw", "rd_forward_no_logits",
     "rd_step_batch_draw", "rd_sample_rows", "rd_greedy_chain_start", "rd_greedy_chain_next", "rd_sample_chain_start",
     "rd_sample_chain_next", "rd_greedy_chain_stop",
     "rd_dequant_q5k", "rd_dequant_q6k", "rd_gemm_q5k", "rd_gemm_q6k", "rd_model_upload_q5k", "rd_model_upload_q6k",
@@ -200,6 +200,18 @@ class Device:
         name = "rd_attn_ragged" if kv == "f16" else "rd_attn_ragged_i8"
         check(getattr(lib(), name)(self.h, len(lens), _p(lens), _p(off), _p(k), _p(v), _p(q), n_h, n_kv, hd,
                                    C.c_float(scale), C.c_float(softcap), _p(out)), name)
+        return out
+
+    def attn_ragged_rows(self, lens, nq, k, v, q, n_h, n_kv, hd, scale, softcap=0.0, kv="f16"):
+        """Sequence i brings nq[i] query rows (its last nq[i] positions); q, out: [sum nq][n_h*hd]."""
+        lens = np.ascontiguousarray(lens, dtype=np.int32)
+        nq = np.ascontiguousarray(nq, dtype=np.int32)
+        off = np.zeros(len(lens), np.int64)
+        off[1:] = np.cumsum(lens[:-1])
+        k, v, q = _f32(k), _f32(v), _f32(q)
+        out = np.empty((int(nq.sum()), n_h * hd), np.float32)
+        check(lib().rd_attn_ragged_rows(self.h, 0 if kv == "f16" else 1, len(lens), _p(lens), _p(nq), _p(off), _p(k), _p(v), _p(q), n_h, n_kv,
+                                        hd, C.c_float(scale), C.c_float(softcap), _p(out)), "rd_attn_ragged_rows")
         return out
 
     def moe_route(self, logits, k, norm):

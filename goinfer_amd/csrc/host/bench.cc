@@ -297,7 +297,7 @@ static int bench_attn_typed(rd_device *d, int kv_type, int n_seq, const int *len
         std::vector<AttnItemH> items;
         std::vector<int> start, slots((size_t)g->rows), lens((size_t)g->rows);
         for (int i = 0; i < g->rows; i++) slots[(size_t)i] = r0 + i, lens[(size_t)i] = len[r0 + i];
-        build_attn_worklist(lens.data(), g->rows, n_kv, items, start);
+        build_attn_worklist(lens.data(), nullptr, G, g->rows, n_kv, items, start);
         g->nItems = (int)items.size();
         RC(g->L.alloc(sizeof(int) * lens.size()));
         RC(g->S.alloc(sizeof(int) * slots.size()));
@@ -333,7 +333,7 @@ static int bench_attn_typed(rd_device *d, int kv_type, int n_seq, const int *len
                                scale, softcap);
             if (timed) (void)d->hip->EventRecord(evp[(t * nG + gi) * 2 + 1], d->stream);
             if (!rc)
-                rc = d->launch(d->k.attn_combine, (unsigned)n_h, (unsigned)g.rows, 1, (unsigned)(ATTN_PIECES * hd / 4), (const float *)g.P.p, (const int *)g.St.p,
+                rc = d->launch(d->k.attn_combine, (unsigned)n_h, (unsigned)g.rows, 1, (unsigned)(ATTN_PIECES * hd / 4), (const float *)g.P.p, (const int *)g.St.p, G,
                                (float *)((float *)O.p + (size_t)g.r0 * qd), n_h, n_kv, hd);
         }
         if (timed) (void)d->hip->EventRecord(ev[2 * t + 1], d->stream);

@@ -95,6 +95,8 @@ static const KName kNames[] = {
     {"rd_k_kv_store_i8", &Kernels::kv_store_i8},
     {"rd_k_qkv_rope_store_i8", &Kernels::qkv_rope_store_i8},
     {"rd_k_attn_partial_i8", &Kernels::attn_partial_i8},
+    {"rd_k_attn_partial_rows", &Kernels::attn_partial_rows},
+    {"rd_k_attn_partial_rows_i8", &Kernels::attn_partial_rows_i8},
     {"rd_k_attn_combine", &Kernels::attn_combine},
     {"rd_k_attn_combine_quant", &Kernels::attn_combine_quant},
     {"rd_k_rmsnorm", &Kernels::rmsnorm},
@@ -186,20 +188,38 @@ extern "C" int rd_device_mem_info(rd_device *d, size_t *free_b, size_t *total_b)
     return RD_OK;
 }
 
-void build_attn_worklist(const int *len, int rows, int n_kv, std::vector<AttnItemH> &items, std::vector<int> &ranges) {
-    std::vector<int> order((size_t)rows);
-    for (int i = 0; i < rows; i++) order[(size_t)i] = i;
-    std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return len[a] > len[b]; });
+bool build_attn_worklist(const int *len, const int *slot, int G, int rows, int n_kv, std::vector<AttnItemH> &items, std::vector<int> &ranges) {
+    static const bool no_groups = getenv("ROCMDECODE_NO_ATTN_GROUPS") != nullptr;
+    const int maxGroup = (slot && !no_groups && G <= ATTN_TILE_ROWS) ? ATTN_TILE_ROWS / G : 1;
+    struct Group {
+        int row, n;
+    };
+    std::vector<Group> groups;
+    for (int r = 0; r < rows;) {
+        int n = 1;
+        while (n < maxGroup && r + n < rows && slot[r + n] == slot[r] && len[r + n] == len[r] + n && (len[r + n] + 63) / 64 == (len[r] + 63) / 64) n++;
+        groups.push_back({r, n});
+        r += n;
+    }
+    std::stable_sort(groups.begin(), groups.end(), [&](const Group &a, const Group &b) { return len[a.row] > len[b.row]; });
     items.clear();
-    ranges.assign((size_t)rows * n_kv * 2, 0);
-    for (int r : order) {
-        const int nb = (len[r] + 63) / 64, chunk = attn_chunk_blocks(nb);
+    ranges.assign((size_t)rows * n_kv * ATTN_RANGE_INTS, 0);
+    bool grouped = false;
+    for (const Group &g : groups) {
+        const int nb = (len[g.row] + 63) / 64, chunk = attn_chunk_blocks(nb);
+        grouped = grouped || g.n > 1;
         for (int h = 0; h < n_kv; h++) {
-            ranges[((size_t)r * n_kv + h) * 2] = (int)items.size();
-            for (int b0 = 0; b0 < nb; b0 += chunk) items.push_back({r, h, b0, std::min(nb, b0 + chunk)});
-            ranges[((size_t)r * n_kv + h) * 2 + 1] = (int)items.size();
+            const int first = (int)items.size();
+            for (int b0 = 0; b0 < nb; b0 += chunk) items.push_back({g.row, h | (g.n << 16), b0, std::min(nb, b0 + chunk)});
+            for (int j = 0; j < g.n; j++) {
+                int *rg = &ranges[((size_t)(g.row + j) * n_kv + h) * ATTN_RANGE_INTS];
+                rg[0] = first, rg[1] = (int)items.size(), rg[2] = j;
+            }
         }
     }
+    if (!grouped)
+        for (auto &it : items) it.kvh &= 0xffff;
+    return grouped;
 }
 
 // ---- GEMM planning ----

@@ -27,7 +27,7 @@ struct Kernels {
     hipFunction_t dequant_q5k, retile_q5k, gemm_q5k, dequant_q6k, retile_q6k, gemm_q6k;
     hipFunction_t gemm_q4k_gateup;
     hipFunction_t kv_store, qkv_rope_store, attn_partial, attn_combine, attn_combine_quant;
-    hipFunction_t kv_store_i8, qkv_rope_store_i8, attn_partial_i8;
+    hipFunction_t kv_store_i8, qkv_rope_store_i8, attn_partial_i8, attn_partial_rows, attn_partial_rows_i8;
     hipFunction_t rmsnorm, rope, argmax_rows, argmax_final, matmul_f32, moe_route, gemm_w4a8_moe, moe_swiglu_quant, moe_fold, embed_rows, copy16, barrier_probe, unpanel_q4k, fill_f16, fill_f32;
 };
 
@@ -73,13 +73,19 @@ constexpr unsigned GEMM_THREADS = 320, GATEUP_THREADS = 640;
 constexpr int ATTN_PIECES = 16; // = RD_ATTN_PIECES of the combine kernels
 inline int attn_chunk_blocks(int nb) { return (nb + ATTN_PIECES - 1) / ATTN_PIECES; }
 
-// One attention work item: blocks [b0,b1) of one (sequence row, kv head); one wave each.
+// One attention work item: blocks [b0,b1) of one kv head of one sequence, for the step's row `row` — or, from the grouping
+// builder, for rows row..row+n-1 with n in the high 16 bits of kvh; one wave each.
 struct AttnItemH {
     int row, kvh, b0, b1;
 };
+constexpr int ATTN_RANGE_INTS = 3; // per (row, kv head): first item, one past the last, the row's place among its items' positions
+constexpr int ATTN_TILE_ROWS = 16; // head rows of the attention MFMA tile: an item holds at most 16 / (heads per kv head) positions
 // The attention work list of a step: items of the longest sequences first (the grid is dispatched in index order, so the
-// short items fill the tail), and ranges[2*(row*n_kv+kvh)], ranges[..+1] = that pair's first item and one past its last.
-void build_attn_worklist(const int *len, int rows, int n_kv, std::vector<AttnItemH> &items, std::vector<int> &ranges);
+// short items fill the tail), and ranges[3*(row*n_kv+kvh)..] as above.
+// slot == nullptr: one position per item. Otherwise consecutive rows of one slot whose lengths ascend by one and need the same
+// number of blocks (so their cuts coincide) share items, up to 16/G of them; returns true if any item holds more than one
+// position, in which case the step runs the kernels that read the high bits of kvh and write 16 head rows per item.
+bool build_attn_worklist(const int *len, const int *slot, int G, int rows, int n_kv, std::vector<AttnItemH> &items, std::vector<int> &ranges);
 
 // split-K plan of one GEMM launch
 struct GemmPlan {

@@ -449,11 +449,11 @@ extern "C" int rd_kv_configure_typed(rd_model *m, int slots, int ctx_cap, int kv
     m->slot_len.assign((size_t)slots, 0);
     // attention work list: ~4096 items plus one per (row, kv head) of rounding
     m->max_items = m->max_rows * c.n_kv_heads * ATTN_PIECES;
-    int G = c.n_heads / c.n_kv_heads;
-    RC(alloc_f32(d, &m->part, (size_t)m->max_items * G * (c.head_dim + 2)));
+    // an item writes one head row per query head of its kv head, or a whole tile of 16 when it covers several positions
+    RC(alloc_f32(d, &m->part, (size_t)m->max_items * ATTN_TILE_ROWS * (c.head_dim + 2)));
     // The step's metadata lives in one device block so a step uploads it with one copy:
-    // [row slot R][row position R][row length R][row draw records R x 6][item ranges max_rows*nKV*2][items max_items x 4] ints, R = ROWS_MAX
-    const size_t rangeInts = (size_t)m->max_rows * c.n_kv_heads * 2;
+    // [row slot R][row position R][row length R][row draw records R x 6][item ranges max_rows*nKV*3][items max_items x 4] ints, R = ROWS_MAX
+    const size_t rangeInts = (size_t)m->max_rows * c.n_kv_heads * ATTN_RANGE_INTS;
     m->meta_ints = rd_model::META_HDR + rangeInts + (size_t)m->max_items * 4;
     RC(d->alloc((void **)&m->meta, sizeof(int) * m->meta_ints));
     constexpr int RM = rd_model::ROWS_MAX;
@@ -522,10 +522,11 @@ struct Scope { // times one kernel class when the model's timer is on
     }
 };
 
-static int build_attn_items(rd_model *m, int B, const int *pos, std::vector<AttnItemH> &items, std::vector<int> &ranges) {
+// *grouped: some item covers several positions of one sequence (the step then runs the attention kernels for such items).
+static int build_attn_items(rd_model *m, int B, const int *slot, const int *pos, std::vector<AttnItemH> &items, std::vector<int> &ranges, bool *grouped) {
     int len[rd_model::ROWS_MAX];
     for (int b = 0; b < B; b++) len[b] = pos[b] + 1;
-    build_attn_worklist(len, B, m->desc.n_kv_heads, items, ranges);
+    *grouped = build_attn_worklist(len, slot, m->desc.n_heads / m->desc.n_kv_heads, B, m->desc.n_kv_heads, items, ranges);
     if ((int)items.size() > m->max_items) {
         rd_set_error("attention work list overflow (%zu items)", items.size());
         return RD_ERR_STATE;
@@ -658,7 +659,9 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
     int H = c.hidden, nH = c.n_heads, nKV = c.n_kv_heads, HD = c.head_dim;
     std::vector<AttnItemH> items;
     std::vector<int> start;
-    RC(build_attn_items(m, B, pos, items, start));
+    bool grouped = false;
+    RC(build_attn_items(m, B, slot, pos, items, start, &grouped));
+    const int partRows = grouped ? ATTN_TILE_ROWS : nH / nKV;
     // Stage the step's metadata (and host embeddings) in pinned memory and upload it asynchronously. A slot is reused only
     // once the upload it last fed has completed, which its event tells.
     const unsigned stage_slot = m->stage_next++ % rd_model::STAGE_SLOTS;
@@ -666,7 +669,7 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
     {
         char *st = (char *)m->host_stage + (size_t)stage_slot * m->host_stage_bytes;
         int *hm = (int *)st; // the metadata block, laid out as on the device
-        const size_t rangeInts = (size_t)m->max_rows * nKV * 2;
+        const size_t rangeInts = (size_t)m->max_rows * nKV * ATTN_RANGE_INTS;
         constexpr int RM = rd_model::ROWS_MAX;
         float *eh = (float *)(st + (1u << 20));
         for (int b = 0; b < B; b++) hm[b] = slot[b], hm[RM + b] = pos[b], hm[2 * RM + b] = pos[b] + 1;
@@ -737,18 +740,18 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
         {
             Scope s(m, KC_ATTN_PARTIAL);
             if (m->kv_type == RD_KV_I8)
-                RC(d->launch(d->k.attn_partial_i8, (unsigned)items.size(), 1, 1, 64, (const void *)m->items, (const int *)m->rowLen, (const int *)m->rowSlot,
+                RC(d->launch(grouped ? d->k.attn_partial_rows_i8 : d->k.attn_partial_i8, (unsigned)items.size(), 1, 1, 64, (const void *)m->items, (const int *)m->rowLen, (const int *)m->rowSlot,
                              (const int *)m->tables, m->blocks_per_slot, (const signed char *)l.Kp, (const signed char *)l.Vp, (const float *)l.Ksc,
                              (const float *)l.Vsc, (const float *)m->qbuf, m->part, nH, nKV, HD, c.attn_scale, c.attn_softcap));
             else
-                RC(d->launch(d->k.attn_partial, (unsigned)items.size(), 1, 1, 64, (const void *)m->items, (const int *)m->rowLen, (const int *)m->rowSlot,
+                RC(d->launch(grouped ? d->k.attn_partial_rows : d->k.attn_partial, (unsigned)items.size(), 1, 1, 64, (const void *)m->items, (const int *)m->rowLen, (const int *)m->rowSlot,
                          (const int *)m->tables, m->blocks_per_slot, (const uint16_t *)l.Kp, (const uint16_t *)l.Vp, (const float *)m->qbuf, m->part,
                          nH, nKV, HD, c.attn_scale, c.attn_softcap));
         }
         {
             Scope s(m, KC_ATTN_COMBINE);
             RC(d->launch(d->k.attn_combine_quant, (unsigned)nH, (unsigned)B, 1, (unsigned)(ATTN_PIECES * HD / 4), (const float *)m->part, (const int *)m->itemStart,
-                         m->XpB, panel_kind_for(l.o), nH, nKV, HD, m->xpBStride));
+                         partRows, m->XpB, panel_kind_for(l.o), nH, nKV, HD, m->xpBStride));
         }
         {
             Scope s(m, KC_GEMM_O);

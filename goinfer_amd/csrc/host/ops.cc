@@ -303,8 +303,9 @@ extern "C" int rd_moe_route(rd_device *d, const float *logits, int T, int nE, in
 }
 
 // ---- ragged attention over a temporary paged pool (kernel-level entry point) ----
-static int attn_ragged_typed(rd_device *d, int kv_type, int n_seq, const int *len, const int64_t *off, const float *k, const float *v, const float *q,
-                             int n_h, int n_kv, int hd, float scale, float softcap, float *out) {
+// nq (optional): sequence i brings nq[i] query rows, its last nq[i] positions; row j of them sees keys 0..len[i]-nq[i]+j.
+static int attn_ragged_typed(rd_device *d, int kv_type, int n_seq, const int *len, const int *nq, const int64_t *off, const float *k, const float *v,
+                             const float *q, int n_h, int n_kv, int hd, float scale, float softcap, float *out) {
     if (!d || !len || !off || !k || !v || !q || !out || n_seq <= 0) return RD_ERR_ARG;
     if (n_kv <= 0 || n_h % n_kv || n_h / n_kv > 16 || (hd != 64 && hd != 128)) {
         rd_set_error("rd_attn_ragged declines: head_dim must be 64 or 128 and the GQA group <= 16");
@@ -316,6 +317,10 @@ static int attn_ragged_typed(rd_device *d, int kv_type, int n_seq, const int *le
     for (int i = 0; i < n_seq; i++) {
         if (len[i] <= 0) {
             rd_set_error("sequence %d has no keys", i);
+            return RD_ERR_ARG;
+        }
+        if (nq && (nq[i] <= 0 || nq[i] > len[i])) {
+            rd_set_error("sequence %d: %d query rows over %d keys", i, nq[i], len[i]);
             return RD_ERR_ARG;
         }
         int nb = (len[i] + 63) / 64;
@@ -365,12 +370,16 @@ static int attn_ragged_typed(rd_device *d, int kv_type, int n_seq, const int *le
                 RC(d->sync());
             }
     }
-    for (int r0 = 0; r0 < n_seq; r0 += 32) { // rows in groups of 32, as the step batches them
-        int rows = std::min(32, n_seq - r0);
+    std::vector<int> rowSeq, rowLens; // the query rows in order: sequence, keys visible
+    for (int i = 0; i < n_seq; i++)
+        for (int j = 0, n = nq ? nq[i] : 1; j < n; j++) rowSeq.push_back(i), rowLens.push_back(len[i] - n + 1 + j);
+    const int n_rows = (int)rowSeq.size();
+    for (int r0 = 0; r0 < n_rows; r0 += 32) { // rows in groups of 32, as the step batches them
+        int rows = std::min(32, n_rows - r0);
         std::vector<AttnItemH> items;
-        std::vector<int> start, slots((size_t)rows), lens((size_t)rows);
-        for (int i = 0; i < rows; i++) slots[(size_t)i] = r0 + i, lens[(size_t)i] = len[r0 + i];
-        build_attn_worklist(lens.data(), rows, n_kv, items, start);
+        std::vector<int> start, slots(rowSeq.begin() + r0, rowSeq.begin() + r0 + rows), lens(rowLens.begin() + r0, rowLens.begin() + r0 + rows);
+        const bool grouped = build_attn_worklist(lens.data(), nq ? slots.data() : nullptr, G, rows, n_kv, items, start);
+        const int partRows = grouped ? ATTN_TILE_ROWS : G;
         DevBuf Q2(d), O2(d), L2(d), S2(d), I2(d), St2(d), P2(d);
         RC(Q2.alloc(sizeof(float) * (size_t)rows * qd));
         RC(O2.alloc(sizeof(float) * (size_t)rows * qd));
@@ -378,30 +387,36 @@ static int attn_ragged_typed(rd_device *d, int kv_type, int n_seq, const int *le
         RC(S2.alloc(sizeof(int) * (size_t)rows));
         RC(I2.alloc(sizeof(AttnItemH) * items.size()));
         RC(St2.alloc(sizeof(int) * start.size()));
-        RC(P2.alloc(sizeof(float) * items.size() * G * (hd + 2)));
+        RC(P2.alloc(sizeof(float) * items.size() * partRows * (hd + 2)));
         RC(d->h2d(Q2.p, q + (size_t)r0 * qd, sizeof(float) * (size_t)rows * qd));
         RC(d->h2d(L2.p, lens.data(), sizeof(int) * (size_t)rows));
         RC(d->h2d(S2.p, slots.data(), sizeof(int) * (size_t)rows));
         RC(d->h2d(I2.p, items.data(), sizeof(AttnItemH) * items.size()));
         RC(d->h2d(St2.p, start.data(), sizeof(int) * start.size()));
         if (i8)
-            RC(d->launch(d->k.attn_partial_i8, (unsigned)items.size(), 1, 1, 64, (const void *)I2.p, (const int *)L2.p, (const int *)S2.p, (const int *)T.p,
-                         maxBlocks, (const signed char *)Kp.p, (const signed char *)Vp.p, (const float *)Ksc.p, (const float *)Vsc.p, (const float *)Q2.p,
-                         P2.as<float>(), n_h, n_kv, hd, scale, softcap));
+            RC(d->launch(grouped ? d->k.attn_partial_rows_i8 : d->k.attn_partial_i8, (unsigned)items.size(), 1, 1, 64, (const void *)I2.p, (const int *)L2.p,
+                         (const int *)S2.p, (const int *)T.p, maxBlocks, (const signed char *)Kp.p, (const signed char *)Vp.p, (const float *)Ksc.p,
+                         (const float *)Vsc.p, (const float *)Q2.p, P2.as<float>(), n_h, n_kv, hd, scale, softcap));
         else
-            RC(d->launch(d->k.attn_partial, (unsigned)items.size(), 1, 1, 64, (const void *)I2.p, (const int *)L2.p, (const int *)S2.p, (const int *)T.p,
-                         maxBlocks, (const uint16_t *)Kp.p, (const uint16_t *)Vp.p, (const float *)Q2.p, P2.as<float>(), n_h, n_kv, hd, scale, softcap));
-        RC(d->launch(d->k.attn_combine, (unsigned)n_h, (unsigned)rows, 1, (unsigned)(ATTN_PIECES * hd / 4), (const float *)P2.p, (const int *)St2.p, O2.as<float>(), n_h,
-                     n_kv, hd));
+            RC(d->launch(grouped ? d->k.attn_partial_rows : d->k.attn_partial, (unsigned)items.size(), 1, 1, 64, (const void *)I2.p, (const int *)L2.p,
+                         (const int *)S2.p, (const int *)T.p, maxBlocks, (const uint16_t *)Kp.p, (const uint16_t *)Vp.p, (const float *)Q2.p, P2.as<float>(), n_h,
+                         n_kv, hd, scale, softcap));
+        RC(d->launch(d->k.attn_combine, (unsigned)n_h, (unsigned)rows, 1, (unsigned)(ATTN_PIECES * hd / 4), (const float *)P2.p, (const int *)St2.p, partRows,
+                     O2.as<float>(), n_h, n_kv, hd));
         RC(d->d2h(out + (size_t)r0 * qd, O2.p, sizeof(float) * (size_t)rows * qd));
     }
     return RD_OK;
 }
 extern "C" int rd_attn_ragged(rd_device *d, int n_seq, const int *len, const int64_t *off, const float *k, const float *v, const float *q,
                               int n_h, int n_kv, int hd, float scale, float softcap, float *out) {
-    return attn_ragged_typed(d, RD_KV_F16, n_seq, len, off, k, v, q, n_h, n_kv, hd, scale, softcap, out);
+    return attn_ragged_typed(d, RD_KV_F16, n_seq, len, nullptr, off, k, v, q, n_h, n_kv, hd, scale, softcap, out);
 }
 extern "C" int rd_attn_ragged_i8(rd_device *d, int n_seq, const int *len, const int64_t *off, const float *k, const float *v, const float *q,
                                  int n_h, int n_kv, int hd, float scale, float softcap, float *out) {
-    return attn_ragged_typed(d, RD_KV_I8, n_seq, len, off, k, v, q, n_h, n_kv, hd, scale, softcap, out);
+    return attn_ragged_typed(d, RD_KV_I8, n_seq, len, nullptr, off, k, v, q, n_h, n_kv, hd, scale, softcap, out);
+}
+extern "C" int rd_attn_ragged_rows(rd_device *d, int kv_type, int n_seq, const int *len, const int *nq, const int64_t *off, const float *k, const float *v,
+                                   const float *q, int n_h, int n_kv, int hd, float scale, float softcap, float *out) {
+    if (!nq || (kv_type != RD_KV_F16 && kv_type != RD_KV_I8)) return RD_ERR_ARG;
+    return attn_ragged_typed(d, kv_type, n_seq, len, nq, off, k, v, q, n_h, n_kv, hd, scale, softcap, out);
 }

@@ -191,7 +191,7 @@ __device__ __forceinline__ float fast_tanh(float x) {
 __device__ __forceinline__ float ld_part(const float *p) { return *p; }
 
 struct AttnItem {
-    int row, kvh, b0, b1; // sequence row, kv head, block range [b0,b1) of that sequence
+    int row, kvh, b0, b1; // first row, kv head (low 16 bits) and number of rows (high 16 bits), block range [b0,b1) of the sequence
 };
 
 // One wave per item: online-softmax attention of the G query heads of one kv head over blocks [b0,b1) of one sequence.
@@ -200,6 +200,11 @@ struct AttnItem {
 // I8: K and V are int8 codes with one f32 scale per (key, kv head). A code is exactly an f16, so the same MFMAs run on the
 // codes; the key's K scale multiplies its finished scores and its V scale multiplies its probabilities before the P.V product:
 // sum_d q_d (c_d s) = s sum_d q_d c_d and sum_key p (c s) = sum_key (p s) c, which is the dequantized arithmetic up to f32 rounding.
+// ROWS: an item covers up to 16/G consecutive positions of one sequence (rows row..row+n-1 of the step, lengths len..len+n-1, all
+// with the same number of blocks): the 16 rows of the A operand hold (position j, head g) at j*G + g, every K and V fragment
+// is read once for all of them, and each row masks the keys past its own length. A row's arithmetic is what it would be in
+// an item of its own: a unit in which all of its keys are masked leaves its maximum, sum and output untouched (factor 1, p = 0).
+// Partials: part[item][16][HD+2] instead of part[item][G][HD+2].
 // eight stored bytes (code + 128) -> eight f16 codes, exactly: under a 0x64 high byte a byte u is 1024 + u; minus 1152.
 __device__ __forceinline__ half8_t kv8_to_half8(uint32_t w0, uint32_t w1) {
     const half2_t off = {(half_t)(-1152.f), (half_t)(-1152.f)};
@@ -214,7 +219,7 @@ __device__ __forceinline__ half8_t kv8_to_half8(uint32_t w0, uint32_t w1) {
     return (half8_t){v0.x, v0.y, v1.x, v1.y, v2.x, v2.y, v3.x, v3.y};
 }
 
-template <int HD, bool I8>
+template <int HD, bool I8, bool ROWS = false>
 __device__ __forceinline__ void attn_partial_body(const AttnItem *__restrict__ items, const int *__restrict__ rowLen, const int *__restrict__ rowSlot,
                                                   const int *__restrict__ tables, int tabStride, const void *__restrict__ KpV,
                                                   const void *__restrict__ VpV, const float *__restrict__ Ksc, const float *__restrict__ Vsc,
@@ -223,10 +228,18 @@ __device__ __forceinline__ void attn_partial_body(const AttnItem *__restrict__ i
     constexpr int NC = HD / 32, NCT = HD / 16;
     constexpr int KL = I8 ? NC / 2 : NC, VL = I8 ? NCT / 2 : NCT; // 16-byte loads per key tile of K, per 32 keys of V
     constexpr int ELEM = I8 ? 1 : 2;
-    const AttnItem it = items[blockIdx.x];
+    AttnItem it = items[blockIdx.x];
+    const int nrows = ROWS ? it.kvh >> 16 : 1;
+    it.kvh &= 0xffff;
     const int lane = threadIdx.x, l16 = lane & 15, lg = lane >> 4;
-    const int G = nH / nKV, len = rowLen[it.row];
+    const int G = nH / nKV, len0 = rowLen[it.row];
+    const int len = len0 + nrows - 1; // the longest row's: the unit loop runs to it
     const int *tab = tables + (size_t)rowSlot[it.row] * tabStride;
+    // head row a of the tile = (position a / G, head a % G); this lane loads Q for row l16 and owns score rows 4*lg + r
+    const int qj = ROWS ? l16 / G : 0, qg = ROWS ? l16 - qj * G : l16;
+    int lenr[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) lenr[r] = ROWS ? len0 + min((4 * lg + r) / G, nrows - 1) : len;
 
     // Q fragments (A operand): lane (head row l16, d quarter lg)
     half8_t qhi[NC], qlo[NC];
@@ -235,7 +248,7 @@ __device__ __forceinline__ void attn_partial_body(const AttnItem *__restrict__ i
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             float v = 0.f;
-            if (l16 < G) v = q[(size_t)it.row * nH * HD + (size_t)(it.kvh * G + l16) * HD + lg * (HD / 4) + c * 8 + i];
+            if (ROWS ? qj < nrows : l16 < G) v = q[(size_t)(it.row + qj) * nH * HD + (size_t)(it.kvh * G + qg) * HD + lg * (HD / 4) + c * 8 + i];
             half_t hi = (half_t)v;
             qhi[c][i] = hi;
             qlo[c][i] = (half_t)(v - (float)hi);
@@ -296,7 +309,7 @@ __device__ __forceinline__ void attn_partial_body(const AttnItem *__restrict__ i
                     float s = S[t][r] * scale;
                     if constexpr (I8) s = S[t][r] * ks[t] * scale;
                     if (softcap != 0.f) s = softcap * fast_tanh(s * rcap);
-                    if (key0 + t * 16 + l16 >= len) s = -INFINITY;
+                    if (key0 + t * 16 + l16 >= lenr[r]) s = -INFINITY;
                     S[t][r] = s;
                     mx[r] = fmaxf(mx[r], s);
                 }
@@ -313,7 +326,7 @@ __device__ __forceinline__ void attn_partial_body(const AttnItem *__restrict__ i
                 for (int t = 0; t < 2; t++) {
                     float p = __expf(S[t][r] - mn);
                     ps += p;
-                    if constexpr (I8) p = (key0 + t * 16 + l16 < len) ? p * vs[t] : 0.f; // a key past the end has no scale to trust
+                    if constexpr (I8) p = (key0 + t * 16 + l16 < lenr[r]) ? p * vs[t] : 0.f; // a key past the end has no scale to trust
                     half_t hi = (half_t)p;
                     int idx = (4 * lg + r) * 32 + t * 16 + l16;
                     pbuf[idx] = hi;
@@ -354,8 +367,8 @@ __device__ __forceinline__ void attn_partial_body(const AttnItem *__restrict__ i
     for (int r = 0; r < 4; r++) {
         for (int o = 8; o > 0; o >>= 1) lrun[r] += __shfl_xor(lrun[r], o, 64);
         int g = 4 * lg + r;
-        if (g < G) {
-            float *dst = part + ((size_t)blockIdx.x * G + g) * (HD + 2);
+        if (ROWS ? g < nrows * G : g < G) {
+            float *dst = part + ((size_t)blockIdx.x * (ROWS ? 16 : G) + g) * (HD + 2);
 #pragma unroll
             for (int ct = 0; ct < NCT; ct++) dst[ct * 16 + l16] = O[ct][r];
             if (l16 == 0) dst[HD] = mrun[r], dst[HD + 1] = lrun[r];
@@ -389,21 +402,50 @@ extern "C" __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3
         attn_partial_body<64, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, Ksc, Vsc, q, part, nH, nKV, scale, softcap, pbuf);
 }
 
+// Items of several positions each (see ROWS above): steps that carry more than one row of a sequence — prompt passes, verification.
+extern "C" __global__ __launch_bounds__(64) void rd_k_attn_partial_rows(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
+                                                                        const int *__restrict__ rowSlot, const int *__restrict__ tables, int tabStride,
+                                                                        const uint16_t *__restrict__ Kp, const uint16_t *__restrict__ Vp,
+                                                                        const float *__restrict__ q, float *__restrict__ part, int nH, int nKV, int HD,
+                                                                        float scale, float softcap) {
+    __shared__ half_t pbuf[1024];
+    if (HD == 128)
+        attn_partial_body<128, false, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, pbuf);
+    else
+        attn_partial_body<64, false, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, pbuf);
+}
+
+extern "C" __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void rd_k_attn_partial_rows_i8(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
+                                                                      const int *__restrict__ rowSlot, const int *__restrict__ tables, int tabStride,
+                                                                      const signed char *__restrict__ Kp, const signed char *__restrict__ Vp,
+                                                                      const float *__restrict__ Ksc, const float *__restrict__ Vsc,
+                                                                      const float *__restrict__ q, float *__restrict__ part, int nH, int nKV, int HD,
+                                                                      float scale, float softcap) {
+    __shared__ half_t pbuf[1024];
+    if (HD == 128)
+        attn_partial_body<128, true, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, Ksc, Vsc, q, part, nH, nKV, scale, softcap, pbuf);
+    else
+        attn_partial_body<64, true, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, Ksc, Vsc, q, part, nH, nKV, scale, softcap, pbuf);
+}
+
 // Merge the partials of one (row, query head) in ascending item order (deterministic):
-// out = sum O_i e^(m_i-M) / sum l_i e^(m_i-M). itemStart[2*(row*nKV+kvh)] and the entry after it bound that pair's items; the
-// host cuts a sequence into at most RD_ATTN_PIECES of them. Block = RD_ATTN_PIECES * HD/4 threads: thread (item i, quarter
+// out = sum O_i e^(m_i-M) / sum l_i e^(m_i-M). itemStart[3*(row*nKV+kvh)] and the entry after it bound that pair's items, the
+// third entry is the row's place among the positions its items cover (0 where an item is one position); partRows is the
+// number of head rows an item writes (G, or 16 from the kernels whose items cover several positions). The
+// host cuts a sequence into at most RD_ATTN_PIECES items. Block = RD_ATTN_PIECES * HD/4 threads: thread (item i, quarter
 // dq) brings four values of item i into LDS, so every item's load is in flight at once; the first HD/4 threads then fold
 // the items in order. lds: RD_ATTN_PIECES*(HD+2) floats. Returns true in the threads that hold a result (four consecutive d).
 #define RD_ATTN_PIECES 16
-__device__ __forceinline__ bool attn_combine_block(const float *__restrict__ part, const int *__restrict__ itemStart, int nH, int nKV, int HD,
-                                                   int m, int head, float *lds, float *out) {
+__device__ __forceinline__ bool attn_combine_block(const float *__restrict__ part, const int *__restrict__ itemStart, int partRows, int nH, int nKV,
+                                                   int HD, int m, int head, float *lds, float *out) {
     const int Q = HD >> 2, ti = threadIdx.x / Q, dq = threadIdx.x - ti * Q;
     const int G = nH / nKV, kvh = head / G, g = head % G;
-    const int i0 = itemStart[(m * nKV + kvh) * 2], n = min(itemStart[(m * nKV + kvh) * 2 + 1] - i0, RD_ATTN_PIECES);
-    const size_t stride = (size_t)G * (HD + 2);
+    const int *rg = itemStart + (m * nKV + kvh) * 3;
+    const int i0 = rg[0], n = min(rg[1] - i0, RD_ATTN_PIECES), sub = rg[2];
+    const size_t stride = (size_t)partRows * (HD + 2);
     float *vals = lds, *mm = lds + RD_ATTN_PIECES * HD, *ll = mm + RD_ATTN_PIECES;
     if (ti < n) {
-        const float *p = part + ((size_t)i0 * G + g) * (HD + 2) + (size_t)ti * stride;
+        const float *p = part + ((size_t)i0 * partRows + sub * G + g) * (HD + 2) + (size_t)ti * stride;
         const float2 a = *(const float2 *)(p + dq * 4), b = *(const float2 *)(p + dq * 4 + 2); // rows are 8-byte aligned (HD+2 is even)
         float *v = vals + ti * HD + dq * 4;
         v[0] = a.x, v[1] = a.y, v[2] = b.x, v[3] = b.y;
@@ -426,12 +468,12 @@ __device__ __forceinline__ bool attn_combine_block(const float *__restrict__ par
 }
 
 // Grid (nH, rows), block RD_ATTN_PIECES * HD/4.
-extern "C" __global__ __launch_bounds__(512) void rd_k_attn_combine(const float *__restrict__ part, const int *__restrict__ itemStart,
+extern "C" __global__ __launch_bounds__(512) void rd_k_attn_combine(const float *__restrict__ part, const int *__restrict__ itemStart, int partRows,
                                                                      float *__restrict__ out, int nH, int nKV, int HD) {
     __shared__ float lds[RD_ATTN_PIECES * (128 + 2)];
     const int head = blockIdx.x, m = blockIdx.y;
     float v[4];
-    if (attn_combine_block(part, itemStart, nH, nKV, HD, m, head, lds, v)) {
+    if (attn_combine_block(part, itemStart, partRows, nH, nKV, HD, m, head, lds, v)) {
         float *o = out + (size_t)m * nH * HD + (size_t)head * HD + threadIdx.x * 4;
         o[0] = v[0], o[1] = v[1], o[2] = v[2], o[3] = v[3];
     }

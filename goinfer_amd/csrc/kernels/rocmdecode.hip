@@ -12,13 +12,13 @@
 
 // Attention combine fused with the per-32 quantization that feeds the o-projection. Grid (nH, rows), block
 // RD_ATTN_PIECES * HD/4; the first HD/4 threads (whole 8-lane quantization groups) finish the row.
-extern "C" __global__ __launch_bounds__(512) void rd_k_attn_combine_quant(const float *__restrict__ part, const int *__restrict__ itemStart,
+extern "C" __global__ __launch_bounds__(512) void rd_k_attn_combine_quant(const float *__restrict__ part, const int *__restrict__ itemStart, int partRows,
                                                                            uint8_t *__restrict__ Xp, int kind, int nH, int nKV, int HD,
                                                                            size_t xpStride) {
     __shared__ float lds[RD_ATTN_PIECES * (128 + 2)];
     const int head = blockIdx.x, m = blockIdx.y;
     float v[4];
-    if (!attn_combine_block(part, itemStart, nH, nKV, HD, m, head, lds, v)) return;
+    if (!attn_combine_block(part, itemStart, partRows, nH, nKV, HD, m, head, lds, v)) return;
     float x0, x1, x2, x3, gs;
     quant_g32x4(v[0], v[1], v[2], v[3], &x0, &x1, &x2, &x3, &gs);
     panel_store4(Xp + (size_t)(m >> 5) * xpStride, kind, m & 31, head * HD + threadIdx.x * 4, x0, x1, x2, x3, gs); // M-tile m/32, row m%32

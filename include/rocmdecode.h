@@ -102,6 +102,13 @@ int rd_attn_ragged(rd_device *d, int n_seq, const int *len, const int64_t *off, 
 /* The same through the int8 cache (RD_KV_I8 below): k and v are quantized per (position, kv head) as the cache stores them. */
 int rd_attn_ragged_i8(rd_device *d, int n_seq, const int *len, const int64_t *off, const float *k, const float *v,
                       const float *q, int n_h, int n_kv, int hd, float scale, float softcap, float *out);
+/* Several query rows per sequence, as a prompt pass or a verification step brings them (decoder/forwardn.go:295-500: row j of
+ * a sequence's n rows attends to the keys up to its own position): sequence i has nq[i] <= len[i] query rows, its last
+ * nq[i] positions, and row j sees keys 0..len[i]-nq[i]+j. q, out: host f32 [sum nq][n_h*hd] in sequence order. kv_type
+ * RD_KV_F16 or RD_KV_I8. Consecutive rows of a sequence share one pass over its keys and values; each row's result is
+ * bit-identical to the row computed alone. */
+int rd_attn_ragged_rows(rd_device *d, int kv_type, int n_seq, const int *len, const int *nq, const int64_t *off, const float *k,
+                        const float *v, const float *q, int n_h, int n_kv, int hd, float scale, float softcap, float *out);
 /* MoE routing (decoder/mlp.go:130-184 routeExperts, softmax scoring; backend/cuda/moe.cu:49-104 moe_route):
  * logits host f32 [T][nE]; idx int32 [T][k], wgt f32 [T][k], rank order. */
 int rd_moe_route(rd_device *d, const float *logits, int T, int nE, int k, int norm, int *idx, float *wgt);

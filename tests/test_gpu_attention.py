@@ -137,3 +137,39 @@ def test_ragged_attention_i8_long_split(dev):
         want = oracle_attn(lens, i8_round_trip(k, nKV, hd), i8_round_trip(v, nKV, hd), q, nH, nKV, hd, scale, softcap)
         err = np.abs(got - want).max() / np.abs(want).max()
         assert err <= 1e-4, (softcap, err)
+
+
+def rows_as_sequences(lens, nq, k, v):
+    """The query rows of rd_attn_ragged_rows restated as one-row sequences: row j of sequence i sees keys 0..len-nq+j."""
+    rl, ks, vs = [], [], []
+    off = 0
+    for n, m in zip(lens, nq):
+        for j in range(m):
+            see = n - m + 1 + j
+            rl.append(see), ks.append(k[off:off + see]), vs.append(v[off:off + see])
+        off += n
+    return rl, np.concatenate(ks), np.concatenate(vs)
+
+
+@pytest.mark.parametrize("kv", ["f16", "i8"])
+@pytest.mark.parametrize("nH,nKV,hd", [(4, 1, 64), (8, 8, 128), (14, 2, 64), (32, 8, 128), (16, 2, 128)])
+def test_rows_of_a_sequence_share_items_and_equal_solo_rows(dev, nH, nKV, hd, kv):
+    """Several positions of one sequence in one item (they share every K and V read): each row against the oracle and
+    bit-identical to the same row as a sequence of its own. The lengths put groups across a block boundary (where the rows
+    part, their cuts differing), at a block's last key, and past the split threshold."""
+    lens = [5, 64, 67, 130, 300, 1100, 1]
+    nq = [5, 3, 6, 9, 2, 7, 1]
+    tot, kvd = sum(lens), nKV * hd
+    k = synth.normal(11, tot * kvd).reshape(tot, kvd).astype(np.float16).astype(np.float32)  # exactly what the f16 cache holds
+    v = synth.normal(12, tot * kvd).reshape(tot, kvd).astype(np.float16).astype(np.float32)
+    q = synth.normal(13, sum(nq) * nH * hd).reshape(sum(nq), nH * hd)
+    scale = float(1.0 / np.sqrt(hd))
+    for softcap in (0.0, 30.0):
+        got = dev.attn_ragged_rows(lens, nq, k, v, q, nH, nKV, hd, scale, softcap, kv=kv)
+        rl, k1, v1 = rows_as_sequences(lens, nq, k, v)
+        solo = dev.attn_ragged(rl, k1, v1, q, nH, nKV, hd, scale, softcap, kv=kv)
+        assert np.array_equal(got.view(np.uint32), solo.view(np.uint32)), np.abs(got - solo).max()
+        rt = (lambda x: x) if kv == "f16" else (lambda x: i8_round_trip(x, nKV, hd))
+        want = oracle_attn(rl, rt(k1), rt(v1), q, nH, nKV, hd, scale, softcap)
+        err = np.abs(got - want).max() / np.abs(want).max()
+        assert err <= 1e-4, (softcap, err)
