@@ -21,7 +21,7 @@ EXPORTS = [
     "rd_kv_configure", "rd_kv_upload", "rd_kv_truncate", "rd_kv_reset", "rd_step_batch", "rd_forward",
     "rd_last_moe_indices", "rd_model_upload_embedding", "rd_bench_steps", "rd_bench_profile", "rd_bench_class_count",
     "rd_bench_class_name", "rd_bench_kernel", "rd_gateup_q4k_quant", "rd_moe_replay", "rd_bench_attn", "rd_step_ragged", "rd_prefill_last",
-    "rd_kv_configure_typed", "rd_attn_ragged_i8", "rd_attn_ragged_rows", "rd_bench_attn_i8", "rd_step_ragged_draw", "rd_forward_no_logits",
+    "rd_kv_configure_typed", "rd_attn_ragged_i8", "rd_attn_ragged_rows", "rd_plan_attention", "rd_plan_gemm", "rd_bench_attn_i8", "rd_step_ragged_draw", "rd_forward_no_logits",
     "rd_step_batch_draw", "rd_sample_rows", "rd_greedy_chain_start", "rd_greedy_chain_next", "rd_sample_chain_start",
     "rd_sample_chain_next", "rd_greedy_chain_stop",
     "rd_dequant_q5k", "rd_dequant_q6k", "rd_gemm_q5k", "rd_gemm_q6k", "rd_model_upload_q5k", "rd_model_upload_q6k",
@@ -30,6 +30,24 @@ EXPORTS = [
 
 class RocmError(RuntimeError):
     pass
+
+
+def plan_attention(lens, slots, heads_per_kv, n_kv, max_items=1 << 16):
+    """The step's attention work list (host planning, no device): (items [n][4], ranges [rows][n_kv][3], grouped)."""
+    lens = np.ascontiguousarray(lens, dtype=np.int32)
+    sl = None if slots is None else np.ascontiguousarray(slots, dtype=np.int32)
+    items = np.zeros((max_items, 4), np.int32)
+    ranges = np.zeros((len(lens), n_kv, 3), np.int32)
+    n, g = C.c_int(0), C.c_int(0)
+    check(lib().rd_plan_attention(len(lens), _p(lens), None if sl is None else _p(sl), heads_per_kv, n_kv, _p(items), max_items, _p(ranges),
+                                  C.byref(n), C.byref(g)), "rd_plan_attention")
+    return items[:n.value].copy(), ranges, bool(g.value)
+
+
+def plan_gemm(N, n_kblocks):
+    s, k = C.c_int(0), C.c_int(0)
+    check(lib().rd_plan_gemm(N, n_kblocks, C.byref(s), C.byref(k)), "rd_plan_gemm")
+    return s.value, k.value
 
 
 class Draw(C.Structure):

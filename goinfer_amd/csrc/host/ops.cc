@@ -420,3 +420,32 @@ extern "C" int rd_attn_ragged_rows(rd_device *d, int kv_type, int n_seq, const i
     if (!nq || (kv_type != RD_KV_F16 && kv_type != RD_KV_I8)) return RD_ERR_ARG;
     return attn_ragged_typed(d, kv_type, n_seq, len, nq, off, k, v, q, n_h, n_kv, hd, scale, softcap, out);
 }
+
+// ---- host planning without a device ----
+extern "C" int rd_plan_attention(int rows, const int *len, const int *slot, int heads_per_kv, int n_kv, int *items_out, int max_items, int *ranges_out,
+                                 int *n_items, int *grouped) {
+    if (rows <= 0 || !len || heads_per_kv <= 0 || n_kv <= 0 || !items_out || !ranges_out || !n_items || !grouped) return RD_ERR_ARG;
+    for (int r = 0; r < rows; r++)
+        if (len[r] <= 0) {
+            rd_set_error("row %d has no keys", r);
+            return RD_ERR_ARG;
+        }
+    std::vector<AttnItemH> items;
+    std::vector<int> ranges;
+    *grouped = build_attn_worklist(len, slot, heads_per_kv, rows, n_kv, items, ranges) ? 1 : 0;
+    *n_items = (int)items.size();
+    if ((int)items.size() > max_items) {
+        rd_set_error("attention work list of %zu items exceeds %d", items.size(), max_items);
+        return RD_ERR_ARG;
+    }
+    memcpy(items_out, items.data(), sizeof(AttnItemH) * items.size());
+    memcpy(ranges_out, ranges.data(), sizeof(int) * ranges.size());
+    return RD_OK;
+}
+
+extern "C" int rd_plan_gemm(int N, int n_kblocks, int *splits, int *kblocks_per_split) {
+    if (N <= 0 || n_kblocks <= 0 || !splits || !kblocks_per_split) return RD_ERR_ARG;
+    GemmPlan p = plan_gemm(0, N, n_kblocks);
+    *splits = p.splits, *kblocks_per_split = p.kbPerSplit;
+    return RD_OK;
+}

@@ -209,6 +209,18 @@ int rd_last_moe_indices(rd_model *m, int *idx);
  * indices and weights; B must equal the next step's batch. The override is consumed by that step. */
 int rd_moe_replay(rd_model *m, int B, const int *idx, const float *wgt);
 
+/* ---- host planning, callable without a GPU (no counterpart in the reference: its CUDA module plans inside its launch code,
+ * backend/cuda/resident.go; exposed so the plans can be checked on a machine with no device) ---- */
+/* The attention work list of one step: rows of len[r] visible keys on KV slot slot[r] (slot may be NULL: every row its own
+ * sequence), heads_per_kv query heads per kv head, n_kv kv heads. items_out: int32 [max_items][4] = (first row, kv head |
+ * rows << 16 (rows is 0 in a list where every item is one row), first block, one past the last block); ranges_out: int32
+ * [rows][n_kv][3] = (first item, one past the last item, the row's place among its items' rows). *n_items, *grouped (1 if
+ * some item covers several rows) are written. Fails with RD_ERR_ARG if the list needs more than max_items. */
+int rd_plan_attention(int rows, const int *len, const int *slot, int heads_per_kv, int n_kv, int *items_out, int max_items,
+                      int *ranges_out, int *n_items, int *grouped);
+/* The split-K plan of a GEMM launch over N output rows and n_kblocks K-blocks: *splits partial sums of *kblocks_per_split. */
+int rd_plan_gemm(int N, int n_kblocks, int *splits, int *kblocks_per_split);
+
 /* ---- measurement: HIP-event timing on the stream the kernels are launched on; inputs resident in HBM ---- */
 /* The int8 embedding table (vocab x hidden codes + one f32 scale per row), resident so a chain needs no host
  * round trip: goinfer's GreedyChain* (decoder/resident/subsystems.go:78-100). Row id is code * scale, the row the host's
