@@ -355,6 +355,7 @@ extern "C" int rd_model_finalize(rd_model *m) {
             return RD_ERR_STATE;
         }
         pf = std::max({pf, gemm_partial_floats(l.qkv), gemm_partial_floats(l.o), gemm_partial_floats(l.gateup), gemm_partial_floats(l.down)});
+        if (c.n_experts == 0) pf = std::max(pf, (size_t)2 * 32 * l.gateup.N); // the unfused gate|up launch with two splits
     }
     if (m->head.kind < 0 || !m->final_norm) {
         rd_set_error("model is missing the head or the final norm");
@@ -573,6 +574,11 @@ static int launch_proj(rd_model *m, const DevWeight &w, const void *Xp, size_t x
     return RD_OK;
 }
 
+// Where the fused gate|up kernel can run it sums K in two halves (its two K-groups, folded once). The unfused path — steps of
+// more than 32 rows, or the fused kernel switched off — is launched with exactly those two splits, so both produce the same
+// bits and a row is the same row in a batch of any size.
+static bool gateup_fusable(const rd_model_desc &c, const DevWeight &w) { return w.kind == 0 && c.inter % 64 == 0; }
+
 static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
     rd_device *d = m->d;
     const rd_model_desc &c = m->desc;
@@ -759,14 +765,17 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
         }
         if (c.n_experts == 0) {
             RC(add_norm_quant(m, B, m->P, plan.splits, l.ffn_norm, l.gateup, m->XpA, nullptr));
-            if (B <= 32 && l.gateup.kind == 0 && c.inter % 64 == 0 && !getenv("ROCMDECODE_NO_FUSED_GATEUP")) {
+            if (B <= 32 && gateup_fusable(c, l.gateup) && !getenv("ROCMDECODE_NO_FUSED_GATEUP")) {
                 Scope s(m, KC_GEMM_GATEUP); // gate|up GEMM + SwiGLU + quantization in one launch
                 RC(d->launch(d->k.gemm_q4k_gateup, (unsigned)(c.inter / 64), 1, 1, GATEUP_THREADS, (const void *)l.gateup.tiled, (const void *)m->XpA, m->XpB,
                              panel_kind_for(l.down), c.inter, H / 256, B));
             } else {
                 {
                     Scope s(m, KC_GEMM_GATEUP);
-                    RC(launch_proj(m, l.gateup, m->XpA, m->xpAStride, B, &plan));
+                    if (gateup_fusable(c, l.gateup))
+                        RC(launch_gemm_wide(d, l.gateup, m->XpA, m->xpAStride, m->P, m->pStride, B, &plan, 0, 2));
+                    else
+                        RC(launch_proj(m, l.gateup, m->XpA, m->xpAStride, B, &plan));
                 }
                 Scope s(m, KC_SWIGLU);
                 RC(d->launch(d->k.swiglu_quant, (unsigned)((c.inter + 1023) / 1024), (unsigned)B, 1, 256, (const float *)m->P, plan.splits, c.inter,

@@ -197,6 +197,34 @@ def test_i8_kv_uploaded_prefix(dev):
     assert d_i8 <= max(2e-2, 1.5 * d_f16), (d_i8, d_f16)
 
 
+def test_wide_batch_rows_equal_solo_rows_deep_k(dev):
+    """The same identity where K spans six super-blocks (hidden 1536; the split-K planner on its own would cut this gate|up in
+    three): a one-row step runs the fused gate|up kernel, which sums K in two halves, a step of more than 32 rows runs the GEMM
+    with split K and the SwiGLU kernel — with those same two halves, so the bits agree. Switching the fused kernel off changes
+    nothing either."""
+    import os
+    cfg = dense_cfg(n_layers=2, hidden=1536, n_heads=12, n_kv=2, head_dim=128, inter=1536, vocab=512)
+    assert capi.plan_gemm(2 * cfg["inter"], cfg["hidden"] // 256)[0] == 3
+    B = 40
+    pair = Pair(cfg, seed=62, dev=dev, slots=2 * B + 1, ctx_cap=32)
+    try:
+        rng = np.random.default_rng(7)
+        toks = rng.integers(0, cfg["vocab"], B)
+        emb = pair.emb[toks]
+        got, _ = pair.gpu.step_batch(list(range(B)), [0] * B, emb, capi.WANT_LOGITS)
+        for b in (0, 31, 32, 39):
+            solo = pair.gpu.forward(B + b, 0, emb[b])
+            assert np.array_equal(solo.view(np.uint32), got[b].view(np.uint32)), b
+        os.environ["ROCMDECODE_NO_FUSED_GATEUP"] = "1"
+        try:
+            unfused = pair.gpu.forward(2 * B, 0, emb[0])
+        finally:
+            del os.environ["ROCMDECODE_NO_FUSED_GATEUP"]
+        assert np.array_equal(unfused.view(np.uint32), got[0].view(np.uint32))
+    finally:
+        pair.close()
+
+
 def test_wide_batch_rows_equal_solo_rows(dev):
     """A dense model steps up to 128 rows at once (four GEMM row tiles): every row is still the row its own one-row step computes,
     bit for bit, whatever tile it rides in; a batch past the range is refused."""
