@@ -226,6 +226,46 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
             if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup) + 1], d->stream);
         }
         if (!rc) rc = d->sync();
+    } else if (nm == "moe_gemm" && n_args >= 7) {
+        // args {N, K, nE, active, T, per_expert_panels, copies[, first[, bitmap]]}: the grouped expert GEMM over nE experts of which `active`
+        // have a token (spread evenly, or the first `active` ones when `first` is set: then every block with work precedes every
+        // block without in dispatch order; `bitmap`: the kernel gets the active-expert bitmap and orders the grid itself); int4 group-32 weights of arbitrary bits, `copies` weight sets used round-robin.
+        int N = (int)args[0], K = (int)args[1], nE = (int)args[2], active = (int)args[3], T = (int)args[4], perE = (int)args[5];
+        int copies = (int)std::max<int64_t>(1, args[6]);
+        if (N <= 0 || N % 32 || K <= 0 || K % 128 || nE < 1 || nE > 256 || active < 0 || active > nE || T < 1 || T > 32) {
+            rd_set_error("moe_gemm bench: bad shape");
+            rc = RD_ERR_ARG;
+        }
+        const size_t wStride = (size_t)(N / 32) * (K / 128) * 2304, wBytes = wStride * nE;
+        const size_t xpStride = (size_t)(K / 128) * LIN_PANEL_BYTES;
+        DevBuf W(d), Xp(d), R(d), O(d), Bits(d);
+        if (!rc) rc = W.alloc(wBytes * copies);
+        if (!rc) rc = Xp.alloc(xpStride * (perE ? nE : 1));
+        if (!rc) rc = R.alloc((size_t)32 * nE);
+        if (!rc) rc = O.alloc(sizeof(float) * (size_t)T * N);
+        if (!rc) rc = d->launch(d->k.fill_f16, 2048, 1, 1, 256, W.as<uint16_t>(), wBytes * copies / 2, 21u);
+        if (!rc) rc = d->launch(d->k.fill_f16, 256, 1, 1, 256, Xp.as<uint16_t>(), xpStride * (perE ? nE : 1) / 2, 22u);
+        if (!rc) {
+            std::vector<signed char> rk((size_t)32 * nE, -1);
+            for (int e = 0; e < nE; e++)
+                if (n_args >= 8 && args[7] ? e < active : (long)(e + 1) * active / nE > (long)e * active / nE) rk[(size_t)(e % T) * nE + e] = 0;
+            rc = d->h2d(R.p, rk.data(), rk.size());
+            unsigned bits[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            for (int e = 0; e < nE; e++)
+                if (rk[(size_t)(e % T) * nE + e] == 0) bits[e >> 5] |= 1u << (e & 31);
+            if (!rc) rc = Bits.alloc(sizeof(bits));
+            if (!rc) rc = d->h2d(Bits.p, bits, sizeof(bits));
+        }
+        if (!rc) rc = d->sync();
+        for (int i = 0; i < warmup + iters && !rc; i++) {
+            const uint8_t *w = (const uint8_t *)W.p + (size_t)(i % copies) * wBytes;
+            if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup)], d->stream);
+            rc = d->launch(d->k.gemm_w4a8_moe, (unsigned)((N + 127) / 128), (unsigned)nE, 1, GEMM_THREADS, (const void *)w, wStride, (const void *)Xp.p,
+                           perE ? xpStride : (size_t)0, O.as<float>(), N, K / 128, T, 1, (const signed char *)R.p, nE,
+                           (n_args >= 9 && args[8]) ? (const unsigned *)Bits.p : (const unsigned *)nullptr);
+            if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup) + 1], d->stream);
+        }
+        if (!rc) rc = d->sync();
     } else {
         rd_set_error("rd_bench_kernel: unknown kernel '%s'", name);
         rc = RD_ERR_ARG;

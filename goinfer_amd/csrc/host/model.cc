@@ -65,7 +65,7 @@ extern "C" void rd_model_destroy(rd_model *m) {
     free_weight(d, &m->head);
     for (void *p : {(void *)m->embed_q, (void *)m->embed_scale, (void *)m->inv_freq_dev, (void *)m->final_norm, (void *)m->tables, (void *)m->h, (void *)m->normed, (void *)m->P, (void *)m->qbuf,
                     (void *)m->part, (void *)m->cand_v, (void *)m->cand_i, (void *)m->logits, (void *)m->emb_dev, m->XpA, m->XpA2, m->XpB, (void *)m->ids, (void *)m->meta, (void *)m->router_logits, (void *)m->moe_wgt, (void *)m->moe_gu,
-                    (void *)m->moe_dn, (void *)m->moe_out, (void *)m->moe_idx, (void *)m->moe_idx_all, (void *)m->moe_rank, m->XpE})
+                    (void *)m->moe_dn, (void *)m->moe_out, (void *)m->moe_idx, (void *)m->moe_idx_all, (void *)m->moe_rank, (void *)m->moe_bits, m->XpE})
         d->release(p);
     if (m->host_stage) (void)d->hip->HostFree(m->host_stage);
     if (m->chain.host_ids) (void)d->hip->HostFree(m->chain.host_ids);
@@ -393,6 +393,8 @@ extern "C" int rd_model_finalize(rd_model *m) {
         RC(d->alloc((void **)&m->moe_idx, sizeof(int) * 32 * k));
         RC(d->alloc((void **)&m->moe_idx_all, sizeof(int) * (size_t)c.n_layers * 32 * k));
         RC(d->alloc((void **)&m->moe_rank, (size_t)32 * c.n_experts));
+        RC(d->alloc((void **)&m->moe_bits, sizeof(unsigned) * 8));
+        HIPCHK(MemsetAsync(m->moe_bits, 0, sizeof(unsigned) * 8, d->stream));
         RC(d->alloc(&m->XpE, (size_t)c.n_experts * (I / 128) * LIN_PANEL_BYTES));
         HIPCHK(MemsetAsync(m->XpE, 0, (size_t)c.n_experts * (I / 128) * LIN_PANEL_BYTES, d->stream));
     }
@@ -547,13 +549,15 @@ static void panel_kinds_of(const DevWeight &w, int *kA, int *kB) {
         if (panel_kind_for(p) != *kA) *kB = panel_kind_for(p);
 }
 
-static int add_norm_quant(rd_model *m, int B, const float *P, int splits, const float *w, const DevWeight &next, void *Xp, float *norm_out) {
+// foldW: P holds an MoE layer's down-projection rows and foldW their weights (see the kernel); else split-K partial sums.
+static int add_norm_quant(rd_model *m, int B, const float *P, int splits, const float *w, const DevWeight &next, void *Xp, float *norm_out,
+                          const float *foldW = nullptr) {
     rd_device *d = m->d;
     Scope s(m, KC_ADD_NORM);
     int kA, kB;
     panel_kinds_of(next, &kA, &kB);
     return d->launch(d->k.add_rmsnorm_quant, (unsigned)B, 1, 1, 1024, m->h, P, splits, w, m->desc.rms_eps, m->desc.hidden, Xp, kA, norm_out,
-                     kB >= 0 ? m->XpA2 : (void *)nullptr, kB, m->pStride, m->xpAStride, m->xpAStride);
+                     kB >= 0 ? m->XpA2 : (void *)nullptr, kB, m->pStride, m->xpAStride, m->xpAStride, foldW);
 }
 
 // One GEMM, or for a group one GEMM per member into column ranges of the same P[split][32][N], all with the group's split
@@ -579,6 +583,8 @@ static int launch_proj(rd_model *m, const DevWeight &w, const void *Xp, size_t x
 // bits and a row is the same row in a batch of any size.
 static bool gateup_fusable(const rd_model_desc &c, const DevWeight &w) { return w.kind == 0 && c.inter % 64 == 0; }
 
+constexpr int MOE_FOLD_FUSED_MAX = 8; // ranks rd_k_add_rmsnorm_quant folds in registers
+
 static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
     rd_device *d = m->d;
     const rd_model_desc &c = m->desc;
@@ -591,11 +597,17 @@ static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
             RC(d->h2d(m->moe_wgt, m->replay_wgt[(size_t)layer].data(), sizeof(float) * (size_t)B * k));
             RC(d->h2d(m->moe_rank, m->replay_rank[(size_t)layer].data(), (size_t)32 * nE));
             RC(d->h2d(trace, m->replay_idx[(size_t)layer].data(), sizeof(int) * (size_t)B * k));
+            unsigned bits[8] = {0, 0, 0, 0, 0, 0, 0, 0}; // the experts the replayed routing uses
+            for (int i = 0; i < B * k; i++) {
+                int e = m->replay_idx[(size_t)layer][(size_t)i];
+                bits[e >> 5] |= 1u << (e & 31);
+            }
+            RC(d->h2d(m->moe_bits, bits, sizeof(bits)));
         } else {
             RC(d->launch(d->k.matmul_f32, (unsigned)((nE + 3) / 4), (unsigned)B, 1, 256, (const float *)m->normed, (const float *)l.router,
-                         m->router_logits, B, H, nE));
+                         m->router_logits, B, H, nE, m->moe_bits));
             RC(d->launch(d->k.moe_route, (unsigned)B, 1, 1, 64, (const float *)m->router_logits, B, nE, k, c.norm_topk_prob, m->moe_idx, m->moe_wgt,
-                         m->moe_rank, trace));
+                         m->moe_rank, trace, m->moe_bits));
         }
     }
     size_t guStride = (size_t)(2 * I / 32) * (H / 128) * 2304, dnStride = (size_t)(H / 32) * (I / 128) * 2304;
@@ -603,7 +615,7 @@ static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
     {
         Scope s(m, KC_MOE_GEMM);
         RC(d->launch(d->k.gemm_w4a8_moe, (unsigned)((2 * I + 127) / 128), (unsigned)nE, 1, GEMM_THREADS, (const void *)l.exp_gateup, guStride,
-                     (const void *)m->XpA, (size_t)0, m->moe_gu, 2 * I, H / 128, B, k, (const signed char *)m->moe_rank, nE));
+                     (const void *)m->XpA, (size_t)0, m->moe_gu, 2 * I, H / 128, B, k, (const signed char *)m->moe_rank, nE, (const unsigned *)m->moe_bits));
     }
     {
         Scope s(m, KC_MOE_GLUE);
@@ -613,9 +625,9 @@ static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
     {
         Scope s(m, KC_MOE_GEMM);
         RC(d->launch(d->k.gemm_w4a8_moe, (unsigned)((H + 127) / 128), (unsigned)nE, 1, GEMM_THREADS, (const void *)l.exp_down, dnStride, (const void *)m->XpE,
-                     xpStride, m->moe_dn, H, I / 128, B, k, (const signed char *)m->moe_rank, nE));
+                     xpStride, m->moe_dn, H, I / 128, B, k, (const signed char *)m->moe_rank, nE, (const unsigned *)m->moe_bits));
     }
-    {
+    if (k > MOE_FOLD_FUSED_MAX) { // else the next norm kernel folds the ranks itself as it adds them to the residual
         Scope s(m, KC_MOE_GLUE);
         RC(d->launch(d->k.moe_fold, (unsigned)((H + 255) / 256), (unsigned)B, 1, 256, (const float *)m->moe_dn, (const float *)m->moe_wgt, m->moe_out,
                      H, k));
@@ -721,12 +733,14 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
                          m->h, H));
         }
     }
-    const float *resP = nullptr; // pending residual contribution (split-K partials of the previous block's last GEMM)
+    // pending residual contribution: split-K partials of the previous block's last GEMM, or (resW set) an MoE layer's
+    // down-projection rows and their weights, folded by the kernel that adds them
+    const float *resP = nullptr, *resW = nullptr;
     int resSplits = 0;
     for (int li = 0; li < c.n_layers; li++) {
         LayerW &l = m->layers[(size_t)li];
         GemmPlan plan;
-        RC(add_norm_quant(m, B, resP, resSplits, l.attn_norm, l.qkv, m->XpA, nullptr));
+        RC(add_norm_quant(m, B, resP, resSplits, l.attn_norm, l.qkv, m->XpA, nullptr, resW));
         {
             Scope s(m, KC_GEMM_QKV);
             RC(launch_proj(m, l.qkv, m->XpA, m->xpAStride, B, &plan));
@@ -785,20 +799,24 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
                 Scope s(m, KC_GEMM_DOWN);
                 RC(launch_gemm_wide(d, l.down, m->XpB, m->xpBStride, m->P, m->pStride, B, &plan));
             }
-            resP = m->P, resSplits = plan.splits;
+            resP = m->P, resSplits = plan.splits, resW = nullptr;
         } else {
             {
                 Scope s(m, KC_ADD_NORM);
                 RC(d->launch(d->k.add_rmsnorm_quant, (unsigned)B, 1, 1, 1024, m->h, (const float *)m->P, plan.splits, (const float *)l.ffn_norm,
-                             c.rms_eps, H, m->XpA, (int)PANEL_LIN4, m->normed, (void *)nullptr, -1, m->pStride, m->xpAStride, m->xpAStride));
+                             c.rms_eps, H, m->XpA, (int)PANEL_LIN4, m->normed, (void *)nullptr, -1, m->pStride, m->xpAStride, m->xpAStride,
+                             (const float *)nullptr));
             }
             RC(moe_ffn(m, B, li, l));
-            resP = m->moe_out, resSplits = 1;
+            if (c.top_k <= MOE_FOLD_FUSED_MAX)
+                resP = m->moe_dn, resSplits = c.top_k, resW = m->moe_wgt;
+            else
+                resP = m->moe_out, resSplits = 1, resW = nullptr;
         }
     }
     if (want & (RD_WANT_LOGITS | RD_WANT_ARGMAX)) {
         GemmPlan plan;
-        RC(add_norm_quant(m, B, resP, resSplits, m->final_norm, m->head, m->XpA, nullptr));
+        RC(add_norm_quant(m, B, resP, resSplits, m->final_norm, m->head, m->XpA, nullptr, resW));
         {
             Scope s(m, KC_GEMM_HEAD);
             RC(launch_gemm_wide(d, m->head, m->XpA, m->xpAStride, m->P, m->pStride, B, &plan));

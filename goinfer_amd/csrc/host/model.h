@@ -89,6 +89,7 @@ struct rd_model {
     float *router_logits = nullptr, *moe_wgt = nullptr, *moe_gu = nullptr, *moe_dn = nullptr, *moe_out = nullptr;
     int *moe_idx = nullptr, *moe_idx_all = nullptr; // [32][k], [layers][32][k]
     signed char *moe_rank = nullptr;                 // [32][nE]
+    unsigned *moe_bits = nullptr;                    // bitmap of the experts the current layer's routing chose (8 words)
     void *XpE = nullptr;                             // per-expert down panels
     // pinned host staging
     // STAGE_SLOTS slots used round-robin, so a caller that chains steps without reading anything back (the device greedy

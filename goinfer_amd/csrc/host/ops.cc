@@ -255,7 +255,7 @@ extern "C" int rd_matmul_bt(rd_device *d, const float *a, const float *b, float 
     RC(D.alloc(sizeof(float) * (size_t)M * N));
     RC(d->h2d(A.p, a, sizeof(float) * (size_t)M * K));
     RC(d->h2d(B.p, b, sizeof(float) * (size_t)N * K));
-    RC(d->launch(d->k.matmul_f32, (unsigned)((N + 3) / 4), (unsigned)M, 1, 256, (const float *)A.p, (const float *)B.p, D.as<float>(), M, K, N));
+    RC(d->launch(d->k.matmul_f32, (unsigned)((N + 3) / 4), (unsigned)M, 1, 256, (const float *)A.p, (const float *)B.p, D.as<float>(), M, K, N, (unsigned *)nullptr));
     return d->d2h(dst, D.p, sizeof(float) * (size_t)M * N);
 }
 
@@ -297,7 +297,7 @@ extern "C" int rd_moe_route(rd_device *d, const float *logits, int T, int nE, in
     RC(W.alloc(sizeof(float) * (size_t)T * k));
     RC(d->h2d(L.p, logits, sizeof(float) * (size_t)T * nE));
     RC(d->launch(d->k.moe_route, (unsigned)T, 1, 1, 64, (const float *)L.p, T, nE, k, norm, I.as<int>(), W.as<float>(),
-                 (signed char *)nullptr, (int *)nullptr));
+                 (signed char *)nullptr, (int *)nullptr, (unsigned *)nullptr));
     RC(d->d2h(idx, I.p, sizeof(int) * (size_t)T * k));
     return d->d2h(wgt, W.p, sizeof(float) * (size_t)T * k);
 }

@@ -81,11 +81,14 @@ extern "C" __global__ void rd_k_reduce_splits(const float *__restrict__ P, float
 //   panels <- per-32 quantization of normed                                  (weightmat.go:33-38)
 // Optionally writes normed f32 to norm_out (the MoE router reads the un-quantized row) and the same quantized values in a
 // second panel layout (Xp2, kind2) when the consuming projections differ in kind. H % 128 == 0, H <= 8192.
+// foldW != NULL: the pending contribution is an MoE layer's output instead, folded here from the experts' down-projection rows:
+// P is [(row*k + rank)][H] with k = splits (<= 8), foldW is [row][k], and the row's contribution is the sum over ranks, in rank
+// order from zero, of foldW * P (multiply, then add: decoder/mlp.go:100-103 addScaled).
 extern "C" __global__ __launch_bounds__(1024) void rd_k_add_rmsnorm_quant(float *__restrict__ h, const float *__restrict__ P, int splits,
                                                                           const float *__restrict__ w, float eps, int H,
                                                                           uint8_t *__restrict__ Xp, int kind, float *__restrict__ norm_out,
                                                                           uint8_t *__restrict__ Xp2, int kind2, size_t pStride, size_t xpStride,
-                                                                          size_t xp2Stride) {
+                                                                          size_t xp2Stride, const float *__restrict__ foldW) {
     __shared__ double red[16];
     const int m = blockIdx.x, t = threadIdx.x, nv = H >> 2;
     // rows beyond 32 are further M-tiles: their partial sums and panels sit pStride floats / xpStride bytes further on
@@ -107,7 +110,31 @@ extern "C" __global__ __launch_bounds__(1024) void rd_k_add_rmsnorm_quant(float 
 #pragma unroll
     for (int i = 0; i < 2; i++)
         if (on[i]) wv[i] = *(const float4_t *)(w + 4 * (t + i * 1024));
-    if (P) {
+    if (P && foldW) {
+        float4_t b[2][8];
+        float wr[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            if (j < splits) {
+                wr[j] = foldW[m * splits + j];
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+                    if (on[i]) b[i][j] = *(const float4_t *)(P + ((size_t)m * splits + j) * H + 4 * (t + i * 1024));
+            }
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            if (!on[i]) continue;
+            float4_t a = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                if (j < splits) {
+                    a.x = __fadd_rn(a.x, __fmul_rn(wr[j], b[i][j].x)), a.y = __fadd_rn(a.y, __fmul_rn(wr[j], b[i][j].y));
+                    a.z = __fadd_rn(a.z, __fmul_rn(wr[j], b[i][j].z)), a.w = __fadd_rn(a.w, __fmul_rn(wr[j], b[i][j].w));
+                }
+            v[i].x = __fadd_rn(v[i].x, a.x), v[i].y = __fadd_rn(v[i].y, a.y), v[i].z = __fadd_rn(v[i].z, a.z), v[i].w = __fadd_rn(v[i].w, a.w);
+            *(float4_t *)(h + (size_t)m * H + 4 * (t + i * 1024)) = v[i];
+        }
+    } else if (P) {
         // the split-K partials in ascending split order; eight splits' loads are issued together (a runtime-trip loop of
         // dependent adds would expose one memory latency per split)
         float4_t a[2];

@@ -130,9 +130,11 @@ extern "C" __global__ __launch_bounds__(64) void rd_k_argmax_final(const float *
 // f32 MoE router (decoder/mlp.go:50). One wave per output: each lane sums its share of k in f64, then a fixed butterfly adds the
 // 64 lane sums. Products of two f32 are exact in f64 and the sum carries ~29 spare bits, so the f32 result matches an
 // ascending-k f64 sum except when that sum falls within ~1e-15 (relative) of an f32 rounding boundary.
-// Grid (ceil(N/4), M), block 256.
+// Grid (ceil(N/4), M), block 256. clear8 (may be NULL): eight words this launch sets to zero on the side — the router's launch
+// clears the active-expert bitmap that the routing kernel, next in the stream, fills.
 extern "C" __global__ __launch_bounds__(256) void rd_k_matmul_f32(const float *__restrict__ a, const float *__restrict__ b, float *__restrict__ dst,
-                                                                   int M, int K, int N) {
+                                                                   int M, int K, int N, unsigned *__restrict__ clear8) {
+    if (clear8 && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x < 8) clear8[threadIdx.x] = 0u;
     const int lane = threadIdx.x & 63, n = blockIdx.x * 4 + (threadIdx.x >> 6), m = blockIdx.y;
     if (n >= N || m >= M) return;
     const float *ar = a + (size_t)m * K, *br = b + (size_t)n * K;
@@ -168,7 +170,8 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_matmul_f32(const float *_
 // expert-major grouped GEMMs. Grid (T), block 64.
 // The routing of one token by one wave (see rd_k_moe_route); x: the token's nE logits (global or LDS).
 __device__ __forceinline__ void moe_route_wave(const float *x, int t, int nE, int k, int norm, int *__restrict__ idx, float *__restrict__ wgt,
-                                               signed char *__restrict__ rankOf, double *e64, int *__restrict__ idx_copy) {
+                                               signed char *__restrict__ rankOf, double *e64, int *__restrict__ idx_copy,
+                                               unsigned *__restrict__ activeBits) {
     const int lane = threadIdx.x & 63;
     float xv[4], sc[4];
     float mx = -INFINITY;
@@ -184,12 +187,18 @@ __device__ __forceinline__ void moe_route_wave(const float *x, int t, int nE, in
         int i = lane + 64 * j;
         double e = i < nE ? exp((double)__fsub_rn(xv[j], mx)) : 0.0;
         sc[j] = (float)e;
-        if (i < nE) e64[i] = e;
+        e64[i] = e; // all 256 entries: zeros past nE, which leave the sum as it is
     }
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0): this wave's LDS writes have landed before its lanes read them back
     double sum = 0;
-    for (int i = 0; i < nE; i++) sum += e64[i];
+    for (int i = 0; i < nE; i += 8) { // eight reads in flight, then the adds in ascending order
+        double v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = e64[i + u];
+#pragma unroll
+        for (int u = 0; u < 8; u++) sum += v[u];
+    }
     const float inv = (float)(1.0 / sum);
 #pragma unroll
     for (int j = 0; j < 4; j++) {
@@ -221,6 +230,7 @@ __device__ __forceinline__ void moe_route_wave(const float *x, int t, int nE, in
         if (lane == 0) {
             idx[(size_t)t * k + r] = bi;
             if (idx_copy) idx_copy[(size_t)t * k + r] = bi;
+            if (activeBits) atomicOr(activeBits + (bi >> 5), 1u << (bi & 31));
         }
         s = __fadd_rn(s, best);
         n++;
@@ -228,14 +238,15 @@ __device__ __forceinline__ void moe_route_wave(const float *x, int t, int nE, in
     if (lane < n) wgt[(size_t)t * k + lane] = (norm && s > 0.f) ? mine / s : mine;
 }
 
-// idx_copy (may be NULL) receives a second copy of the indices: the step's per-layer routing trace.
+// idx_copy (may be NULL) receives a second copy of the indices: the step's per-layer routing trace. activeBits (may be NULL):
+// a bitmap of nE bits, zero on entry, in which every chosen expert's bit is set.
 extern "C" __global__ __launch_bounds__(64) void rd_k_moe_route(const float *__restrict__ logits, int T, int nE, int k, int norm,
                                                                  int *__restrict__ idx, float *__restrict__ wgt, signed char *__restrict__ rankOf,
-                                                                 int *__restrict__ idx_copy) {
+                                                                 int *__restrict__ idx_copy, unsigned *__restrict__ activeBits) {
     __shared__ double e64[256];
     const int t = blockIdx.x;
     if (t >= T) return;
-    moe_route_wave(logits + (size_t)t * nE, t, nE, k, norm, idx, wgt, rankOf, e64, idx_copy);
+    moe_route_wave(logits + (size_t)t * nE, t, nE, k, norm, idx, wgt, rankOf, e64, idx_copy, activeBits);
 }
 
 // Token embedding rows from an int8 table with one f32 scale per row (goinfer keeps the embedding table int8 in q4k mode,

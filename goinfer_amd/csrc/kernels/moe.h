@@ -8,20 +8,41 @@
 
 // out[(token*k + rank)][N] = panels . W_e^T for the experts that have at least one token. Grid (ceil(N/128), nE), block 320 (four consumer waves and a panel producer).
 // xpStride: bytes between the experts' panel sets (0 = all experts read the same panels: the gate/up projections).
-extern "C" __global__ __launch_bounds__(320) void rd_k_gemm_w4a8_moe(const uint8_t *__restrict__ Wt, size_t wStride, const uint8_t *__restrict__ Xp,
-                                                                      size_t xpStride, float *__restrict__ out, int N, int nKB, int T, int k,
-                                                                      const signed char *__restrict__ rankOf, int nE) {
-    __shared__ uint4_t lds[2 * RD_LIN_PANEL_BYTES / 16];
-    const int e = blockIdx.y, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    int mine = (tid < T && rankOf[(size_t)tid * nE + e] >= 0) ? 1 : 0;
-    if (!__syncthreads_or(mine)) return;
-    const int tile = blockIdx.x * 4 + (wave & 3);
+// activeBits (may be NULL): the bitmap of experts with a token. Row y of the grid then works on the y-th expert whose bit is set,
+// and the rows past the last one exit: the blocks with work are the first in dispatch order, which spreads them evenly over
+// the XCDs and CUs (blocks are handed out round-robin; idle ones scattered among them skew that). Without the bitmap row y is
+// expert y, and exits when no token chose it.
+template <int TPB, int PF>
+__device__ __forceinline__ void moe_gemm_body(const uint8_t *__restrict__ Wt, size_t wStride, const uint8_t *__restrict__ Xp, size_t xpStride,
+                                              float *__restrict__ out, int N, int nKB, int T, int k, const signed char *__restrict__ rankOf, int nE,
+                                              const unsigned *__restrict__ activeBits, uint4_t *lds) {
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    int e = blockIdx.y;
+    if (activeBits) {
+        int y = blockIdx.y;
+        e = -1;
+        for (int w = 0; w < (nE + 31) >> 5; w++) {
+            unsigned b = activeBits[w];
+            const int c = __popc(b);
+            if (y < c) {
+                for (int i = 0; i < y; i++) b &= b - 1; // drop the y lowest set bits
+                e = w * 32 + __ffs((int)b) - 1;
+                break;
+            }
+            y -= c;
+        }
+        if (e < 0) return;
+    } else {
+        int mine = (tid < T && rankOf[(size_t)tid * nE + e] >= 0) ? 1 : 0;
+        if (!__syncthreads_or(mine)) return;
+    }
+    const int tile = blockIdx.x * TPB + (wave % TPB);
     const bool active = tile * 32 < N;
     float16_t acc;
     const int ltile = active ? tile : (N >> 5) - 1;
-    gemm_mainloop_pc<W4MoeTraits, 4, 1, 3>(acc, Wt + (size_t)e * wStride + (size_t)ltile * nKB * W4Traits::TILE_BYTES, Xp + (size_t)e * xpStride, 0, nKB,
-                                        lds);
-    if (!active || wave >= 4) return;
+    gemm_mainloop_pc<W4MoeTraits, TPB, 1, PF>(acc, Wt + (size_t)e * wStride + (size_t)ltile * nKB * W4Traits::TILE_BYTES, Xp + (size_t)e * xpStride, 0,
+                                              nKB, lds);
+    if (!active || wave >= TPB) return;
 #pragma unroll
     for (int r = 0; r < 16; r++) {
         int m = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
@@ -32,6 +53,13 @@ extern "C" __global__ __launch_bounds__(320) void rd_k_gemm_w4a8_moe(const uint8
     }
 }
 
+extern "C" __global__ __launch_bounds__(320) void rd_k_gemm_w4a8_moe(const uint8_t *__restrict__ Wt, size_t wStride, const uint8_t *__restrict__ Xp,
+                                                                      size_t xpStride, float *__restrict__ out, int N, int nKB, int T, int k,
+                                                                      const signed char *__restrict__ rankOf, int nE,
+                                                                      const unsigned *__restrict__ activeBits) {
+    __shared__ uint4_t lds[2 * RD_LIN_PANEL_BYTES / 16];
+    moe_gemm_body<4, 3>(Wt, wStride, Xp, xpStride, out, N, nKB, T, k, rankOf, nE, activeBits, lds);
+}
 // gate/up rows [(token,rank)][2I] -> silu(gate)*up -> per-32 quantization -> the down-projection panels of that row's expert.
 // Grid (ceil(I/256), T*k).
 extern "C" __global__ __launch_bounds__(256) void rd_k_moe_swiglu_quant(const float *__restrict__ gu, const int *__restrict__ idx, int I, int k,
