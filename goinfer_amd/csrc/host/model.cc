@@ -612,12 +612,17 @@ static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
     }
     size_t guStride = (size_t)(2 * I / 32) * (H / 128) * 2304, dnStride = (size_t)(H / 32) * (I / 128) * 2304;
     size_t xpStride = (size_t)(I / 128) * LIN_PANEL_BYTES;
-    {
-        Scope s(m, KC_MOE_GEMM);
-        RC(d->launch(d->k.gemm_w4a8_moe, (unsigned)((2 * I + 127) / 128), (unsigned)nE, 1, GEMM_THREADS, (const void *)l.exp_gateup, guStride,
-                     (const void *)m->XpA, (size_t)0, m->moe_gu, 2 * I, H / 128, B, k, (const signed char *)m->moe_rank, nE, (const unsigned *)m->moe_bits));
-    }
-    {
+    if (I % 64 == 0 && !getenv("ROCMDECODE_NO_FUSED_MOE_GATEUP")) {
+        Scope s(m, KC_MOE_GEMM); // gate|up of every touched expert + SwiGLU + quantization into the experts' down panels
+        RC(d->launch(d->k.gemm_w4a8_moe_gateup, (unsigned)(I / 64), (unsigned)nE, 1, GEMM_THREADS, (const void *)l.exp_gateup, guStride,
+                     (const void *)m->XpA, m->XpE, xpStride, I, H / 128, B, (const signed char *)m->moe_rank, nE, (const unsigned *)m->moe_bits));
+    } else {
+        {
+            Scope s(m, KC_MOE_GEMM);
+            RC(d->launch(d->k.gemm_w4a8_moe, (unsigned)((2 * I + 127) / 128), (unsigned)nE, 1, GEMM_THREADS, (const void *)l.exp_gateup, guStride,
+                         (const void *)m->XpA, (size_t)0, m->moe_gu, 2 * I, H / 128, B, k, (const signed char *)m->moe_rank, nE,
+                         (const unsigned *)m->moe_bits));
+        }
         Scope s(m, KC_MOE_GLUE);
         RC(d->launch(d->k.moe_swiglu_quant, (unsigned)((I + 255) / 256), (unsigned)(B * k), 1, 256, (const float *)m->moe_gu, (const int *)m->moe_idx,
                      I, k, m->XpE, xpStride));

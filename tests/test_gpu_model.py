@@ -132,6 +132,30 @@ def test_moe_ragged_batch(dev):
     assert not all(diverged)
 
 
+def test_moe_fused_expert_gateup_equals_two_launches(dev):
+    """The expert gate|up GEMM with SwiGLU and quantization in its epilogue against the same step run as GEMM + SwiGLU kernel:
+    identical logits and routing, bit for bit."""
+    import os
+    cfg = moe_cfg(n_layers=2, hidden=512, n_heads=4, n_kv=2, head_dim=64, n_experts=16, top_k=4, exp_inter=256)
+    pair = Pair(cfg, seed=71, dev=dev, slots=12, ctx_cap=32)
+    try:
+        rng = np.random.default_rng(8)
+        B = 5
+        for step in range(2):
+            emb = pair.emb[rng.integers(0, cfg["vocab"], B)]
+            fused, _ = pair.gpu.step_batch(list(range(B)), [step] * B, emb, capi.WANT_LOGITS)
+            idx_fused = pair.gpu.last_moe_indices(B).copy()
+            os.environ["ROCMDECODE_NO_FUSED_MOE_GATEUP"] = "1"
+            try:
+                plain, _ = pair.gpu.step_batch(list(range(B, 2 * B)), [step] * B, emb, capi.WANT_LOGITS)
+            finally:
+                del os.environ["ROCMDECODE_NO_FUSED_MOE_GATEUP"]
+            assert np.array_equal(idx_fused, pair.gpu.last_moe_indices(B))
+            assert np.array_equal(fused.view(np.uint32), plain.view(np.uint32)), step
+    finally:
+        pair.close()
+
+
 def test_step_errors(dev):
     pair = Pair(dense_cfg(n_layers=1), seed=6, dev=dev, slots=2, ctx_cap=64)
     e = pair.emb[:1]
