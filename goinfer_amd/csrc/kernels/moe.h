@@ -12,11 +12,11 @@
 // and the rows past the last one exit: the blocks with work are the first in dispatch order, which spreads them evenly over
 // the XCDs and CUs (blocks are handed out round-robin; idle ones scattered among them skew that). Without the bitmap row y is
 // expert y, and exits when no token chose it.
-// The expert grid row blockIdx.y works on, or -1 (uniform over the block; every thread must call it).
-__device__ __forceinline__ int moe_block_expert(const unsigned *__restrict__ activeBits, const signed char *__restrict__ rankOf, int nE, int T) {
-    int e = blockIdx.y;
+// The expert grid row `row` works on, or -1 (uniform over the block; every thread must call it).
+__device__ __forceinline__ int moe_block_expert(const unsigned *__restrict__ activeBits, const signed char *__restrict__ rankOf, int nE, int T, int row) {
+    int e = row;
     if (activeBits) {
-        int y = blockIdx.y;
+        int y = row;
         for (int w = 0; w < (nE + 31) >> 5; w++) {
             unsigned b = activeBits[w];
             const int c = __popc(b);
@@ -37,9 +37,16 @@ __device__ __forceinline__ void moe_gemm_body(const uint8_t *__restrict__ Wt, si
                                               float *__restrict__ out, int N, int nKB, int T, int k, const signed char *__restrict__ rankOf, int nE,
                                               const unsigned *__restrict__ activeBits, uint4_t *lds) {
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const int e = moe_block_expert(activeBits, rankOf, nE, T);
+    // perExpertPanels: every expert reads panels of its own, so all blocks of an expert are placed on one XCD (blocks go to the
+    // eight XCDs round-robin in linear order) and its panels are pulled into one L2 instead of eight.
+    int bx = blockIdx.x, row = blockIdx.y;
+    if (xpStride != 0 && (gridDim.y & 7) == 0) {
+        const int gx = gridDim.x, L = row * gx + bx, j = L >> 3;
+        row = (j / gx) * 8 + (L & 7), bx = j % gx;
+    }
+    const int e = moe_block_expert(activeBits, rankOf, nE, T, row);
     if (e < 0) return;
-    const int tile = blockIdx.x * TPB + (wave % TPB);
+    const int tile = bx * TPB + (wave % TPB);
     const bool active = tile * 32 < N;
     float16_t acc;
     const int ltile = active ? tile : (N >> 5) - 1;
@@ -56,7 +63,7 @@ __device__ __forceinline__ void moe_gemm_body(const uint8_t *__restrict__ Wt, si
     }
 }
 
-extern "C" __global__ __launch_bounds__(320) void rd_k_gemm_w4a8_moe(const uint8_t *__restrict__ Wt, size_t wStride, const uint8_t *__restrict__ Xp,
+extern "C" __global__ __launch_bounds__(320) __attribute__((amdgpu_waves_per_eu(7, 7))) void rd_k_gemm_w4a8_moe(const uint8_t *__restrict__ Wt, size_t wStride, const uint8_t *__restrict__ Xp,
                                                                       size_t xpStride, float *__restrict__ out, int N, int nKB, int T, int k,
                                                                       const signed char *__restrict__ rankOf, int nE,
                                                                       const unsigned *__restrict__ activeBits) {
@@ -76,7 +83,7 @@ extern "C" __global__ __launch_bounds__(320) void rd_k_gemm_w4a8_moe_gateup(cons
     __shared__ uint4_t lds[2 * RD_LIN_PANEL_BYTES / 16];
     static_assert(2 * RD_LIN_PANEL_BYTES >= 4 * 32 * 32 * 4, "the four finished tiles are exchanged through the panel buffers");
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, wt = wave & 3;
-    const int e = moe_block_expert(activeBits, rankOf, nE, T);
+    const int e = moe_block_expert(activeBits, rankOf, nE, T, blockIdx.y);
     if (e < 0) return;
     const int nGate = I >> 5, tile = (wt >> 1) * nGate + blockIdx.x * 2 + (wt & 1);
     float16_t acc;
