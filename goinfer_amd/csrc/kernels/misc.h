@@ -209,17 +209,27 @@ __device__ __forceinline__ void moe_route_wave(const float *x, int t, int nE, in
     float s = 0.f, mine = 0.f; // lane j keeps the rank-j weight
     int n = 0;
     for (int r = 0; r < k; r++) {
-        float best = -INFINITY;
-        int bi = 0x7fffffff;
+        // The pass's pick as the maximum of a 64-bit key per lane: (score bits + 1, ~index), 0 for nothing left. Scores are >= 0,
+        // so their bit patterns order as the values do; of equal scores the lower index has the larger key, which is the
+        // strict '>' scan's choice. The maximum over the wave: within rows of 16 lanes on the DPP path, across the rows by swizzle
+        // and one permute.
+        unsigned kh = 0u, kl = 0u;
 #pragma unroll
-        for (int j = 0; j < 4; j++) // ascending index within the lane: strict '>' keeps the lowest
-            if (sc[j] > best) best = sc[j], bi = lane + 64 * j;
-        for (int o = 32; o > 0; o >>= 1) {
-            float v2 = __shfl_xor(best, o, 64);
-            int i2 = __shfl_xor(bi, o, 64);
-            if (v2 > best || (v2 == best && i2 < bi)) best = v2, bi = i2;
-        }
-        if (bi == 0x7fffffff) break; // nothing left (k > nE)
+        for (int j = 3; j >= 0; j--) // descending, '>=' on the score: the lowest index among this lane's equals survives
+            if (sc[j] >= 0.f && __float_as_uint(sc[j]) + 1u >= kh) kh = __float_as_uint(sc[j]) + 1u, kl = ~(unsigned)(lane + 64 * j);
+        auto take = [&](unsigned oh, unsigned ol) {
+            const bool gt = oh > kh || (oh == kh && ol > kl);
+            kh = gt ? oh : kh, kl = gt ? ol : kl;
+        };
+        take((unsigned)dpp_i<RD_DPP_QUAD_XOR1>((int)kh), (unsigned)dpp_i<RD_DPP_QUAD_XOR1>((int)kl));
+        take((unsigned)dpp_i<RD_DPP_QUAD_XOR2>((int)kh), (unsigned)dpp_i<RD_DPP_QUAD_XOR2>((int)kl));
+        take((unsigned)dpp_i<RD_DPP_HALF_MIRROR>((int)kh), (unsigned)dpp_i<RD_DPP_HALF_MIRROR>((int)kl));
+        take((unsigned)dpp_i<RD_DPP_ROW_MIRROR>((int)kh), (unsigned)dpp_i<RD_DPP_ROW_MIRROR>((int)kl));
+        take((unsigned)swz_xor16_i((int)kh), (unsigned)swz_xor16_i((int)kl));
+        take((unsigned)__shfl_xor((int)kh, 32, 64), (unsigned)__shfl_xor((int)kl, 32, 64));
+        if (kh == 0u) break; // nothing left (k > nE)
+        const int bi = (int)~kl;
+        const float best = __uint_as_float(kh - 1u);
 #pragma unroll
         for (int j = 0; j < 4; j++)
             if (bi == lane + 64 * j) {
