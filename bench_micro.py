@@ -229,11 +229,15 @@ def run_c5(args):
             a[0] += t
             a[1] += n
     classes = {k: {"ms_per_step": round(v[0] / 3, 4), "launches_per_step": v[1] // 3} for k, v in prof.items()}
-    # dominant kernel: the expert-major grouped GEMM (two launches per layer: gate|up of every touched expert, then down)
+    # dominant kernel: the experts' gate|up GEMM (one launch per layer over every touched expert; two thirds of an expert's bytes)
     idx2 = res.model.last_moe_indices(B)
     d2 = float(sum(len(set(idx2[:, l, :].ravel().tolist())) for l in range(layers)))
-    g_ms = prof["moe_gemm"][0] / prof["moe_gemm"][1]
-    per_launch = d2 * ebytes / (2 * layers)
+    g_ms = prof["moe_gemm_gateup"][0] / prof["moe_gemm_gateup"][1]
+    per_launch = d2 * ebytes * (2.0 / 3.0) / layers
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        traffic = json.load(open(tpath)).get("gemm_w4a8_moe_gateup/%s" % cfg["name"])
     out = base_line("batch-16 decode tok/s, Qwen3-MoE-30B-A3B shape (int4-g32 experts); achieved HBM GB/s vs peak", tok_s, "tok/s", steps, warmup,
                     float(ms.mean()), "configs[4]: %s, %d layers, B=%d ragged, ctx U[256,2048], greedy decode" % (cfg["name"], layers, B),
                     "synthetic: N(0,0.02) weights (Q4_K projections, int4-g32 experts, f32 router, int8 head), N(0,1) KV, random token ids",
@@ -242,7 +246,7 @@ def run_c5(args):
     out["step_hbm"] = {"algorithmic_bytes_per_step": int(step_bytes), "achieved_GBs": round(step_gbs, 1), "frac_of_peak": round(step_gbs / HBM_PEAK_GBS, 4),
                        "dense_weight_bytes": int(w_bytes), "expert_bytes": int(exp_bytes), "kv_read_bytes": int(kv_read)}
     out["roofline"] = {"bound": "hbm", "achieved": round(per_launch / (g_ms / 1e3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                       "frac": round(per_launch / (g_ms / 1e3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "rd_k_gemm_w4a8_moe",
+                       "frac": round(per_launch / (g_ms / 1e3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": traffic, "kernel": "rd_k_gemm_w4a8_moe_gateup",
                        "avg_launch_ms": round(g_ms, 5), "algorithmic_bytes_per_launch": int(per_launch)}
     out["kernel_classes"] = classes
     cpu = None

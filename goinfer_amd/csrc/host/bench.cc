@@ -72,7 +72,7 @@ extern "C" int rd_bench_profile(rd_model *m, int B, const int *slot, const int *
 extern "C" int rd_bench_class_count(void) { return KC_COUNT; }
 extern "C" const char *rd_bench_class_name(int c) {
     static const char *names[KC_COUNT] = {"gemm_qkv", "rope_kvstore", "attn_partial", "attn_combine", "gemm_o", "add_rmsnorm_quant", "gemm_gateup",
-                                          "swiglu_quant", "gemm_down", "gemm_head", "argmax", "moe_router", "moe_gemm", "moe_glue"};
+                                          "swiglu_quant", "gemm_down", "gemm_head", "argmax", "moe_router", "moe_gemm_gateup", "moe_gemm_down", "moe_glue"};
     return c >= 0 && c < KC_COUNT ? names[c] : "";
 }
 

@@ -628,7 +628,7 @@ static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
                      I, k, m->XpE, xpStride));
     }
     {
-        Scope s(m, KC_MOE_GEMM);
+        Scope s(m, KC_MOE_GEMM_DOWN);
         RC(d->launch(d->k.gemm_w4a8_moe, (unsigned)((H + 127) / 128), (unsigned)nE, 1, GEMM_THREADS, (const void *)l.exp_down, dnStride, (const void *)m->XpE,
                      xpStride, m->moe_dn, H, I / 128, B, k, (const signed char *)m->moe_rank, nE, (const unsigned *)m->moe_bits));
     }

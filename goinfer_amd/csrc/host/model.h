@@ -7,7 +7,7 @@
 // kernel classes of one decode step, for per-class timing
 enum {
     KC_GEMM_QKV = 0, KC_ROPE_STORE, KC_ATTN_PARTIAL, KC_ATTN_COMBINE, KC_GEMM_O, KC_ADD_NORM, KC_GEMM_GATEUP, KC_SWIGLU, KC_GEMM_DOWN,
-    KC_GEMM_HEAD, KC_ARGMAX, KC_MOE_ROUTER, KC_MOE_GEMM, KC_MOE_GLUE, KC_COUNT
+    KC_GEMM_HEAD, KC_ARGMAX, KC_MOE_ROUTER, KC_MOE_GEMM, KC_MOE_GEMM_DOWN, KC_MOE_GLUE, KC_COUNT
 };
 
 struct PendingMat { // a projection uploaded but not yet fused with its siblings (q|k|v, gate|up)
