@@ -95,6 +95,8 @@ static const KName kNames[] = {
     {"rd_k_kv_store_i8", &Kernels::kv_store_i8},
     {"rd_k_qkv_rope_store_i8", &Kernels::qkv_rope_store_i8},
     {"rd_k_attn_partial_i8", &Kernels::attn_partial_i8},
+    {"rd_k_attn_partial_deep", &Kernels::attn_partial_deep},
+    {"rd_k_attn_partial_deep_i8", &Kernels::attn_partial_deep_i8},
     {"rd_k_attn_partial_rows", &Kernels::attn_partial_rows},
     {"rd_k_attn_partial_rows_i8", &Kernels::attn_partial_rows_i8},
     {"rd_k_attn_combine", &Kernels::attn_combine},
@@ -187,6 +189,12 @@ extern "C" int rd_device_mem_info(rd_device *d, size_t *free_b, size_t *total_b)
     if (!d) return RD_ERR_ARG;
     HIPCHK(MemGetInfo(free_b, total_b));
     return RD_OK;
+}
+
+hipFunction_t attn_partial_kernel(const rd_device *d, bool i8, bool grouped, size_t n_items) {
+    if (grouped) return i8 ? d->k.attn_partial_rows_i8 : d->k.attn_partial_rows;
+    if (n_items <= (size_t)ATTN_DEEP_MAX_ITEMS && !getenv("ROCMDECODE_NO_DEEP_ATTN")) return i8 ? d->k.attn_partial_deep_i8 : d->k.attn_partial_deep;
+    return i8 ? d->k.attn_partial_i8 : d->k.attn_partial;
 }
 
 bool build_attn_worklist(const int *len, const int *slot, int G, int rows, int n_kv, std::vector<AttnItemH> &items, std::vector<int> &ranges) {

@@ -765,11 +765,11 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
         {
             Scope s(m, KC_ATTN_PARTIAL);
             if (m->kv_type == RD_KV_I8)
-                RC(d->launch(grouped ? d->k.attn_partial_rows_i8 : d->k.attn_partial_i8, (unsigned)items.size(), 1, 1, 64, (const void *)m->items, (const int *)m->rowLen, (const int *)m->rowSlot,
+                RC(d->launch(attn_partial_kernel(d, true, grouped, items.size()), (unsigned)items.size(), 1, 1, 64, (const void *)m->items, (const int *)m->rowLen, (const int *)m->rowSlot,
                              (const int *)m->tables, m->blocks_per_slot, (const signed char *)l.Kp, (const signed char *)l.Vp, (const float *)l.Ksc,
                              (const float *)l.Vsc, (const float *)m->qbuf, m->part, nH, nKV, HD, c.attn_scale, c.attn_softcap));
             else
-                RC(d->launch(grouped ? d->k.attn_partial_rows : d->k.attn_partial, (unsigned)items.size(), 1, 1, 64, (const void *)m->items, (const int *)m->rowLen, (const int *)m->rowSlot,
+                RC(d->launch(attn_partial_kernel(d, false, grouped, items.size()), (unsigned)items.size(), 1, 1, 64, (const void *)m->items, (const int *)m->rowLen, (const int *)m->rowSlot,
                          (const int *)m->tables, m->blocks_per_slot, (const uint16_t *)l.Kp, (const uint16_t *)l.Vp, (const float *)m->qbuf, m->part,
                          nH, nKV, HD, c.attn_scale, c.attn_softcap));
         }

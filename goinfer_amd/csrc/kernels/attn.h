@@ -219,7 +219,88 @@ __device__ __forceinline__ half8_t kv8_to_half8(uint32_t w0, uint32_t w1) {
     return (half8_t){v0.x, v0.y, v1.x, v1.y, v2.x, v2.y, v3.x, v3.y};
 }
 
-template <int HD, bool I8, bool ROWS = false>
+// The work on one unit of 32 keys whose K and V fragments (KF, VF) and int8 scales (KS, VS) are in registers: scores, online softmax
+// with a lazy rescale of the running output (only when some row's maximum moved: a factor of exactly 1 changes nothing; a key
+// past a row's end has no scale to trust, so its probability is zeroed rather than scaled), P.V. A macro, not a function, so
+// that the unit loops below expand to the same statements wherever they use it. Uses the enclosing kernel body's names.
+#define RD_ATTN_UNIT(KF, VF, KS, VS, KEY0) \
+    { \
+        float4v S[2];                                                                                                                                  \
+        _Pragma("unroll")                                                                                                                              \
+        for (int t = 0; t < 2; t++) {                                                                                                                  \
+            S[t] = (float4v){0.f, 0.f, 0.f, 0.f};                                                                                                      \
+        _Pragma("unroll")                                                                                                                              \
+            for (int c = 0; c < NC; c++) {                                                                                                             \
+                half8_t kb;                                                                                                                            \
+                if constexpr (I8)                                                                                                                      \
+                    kb = kv8_to_half8(KF[t][c >> 1][(c & 1) * 2], KF[t][c >> 1][(c & 1) * 2 + 1]);                                                     \
+                else                                                                                                                                   \
+                    __builtin_memcpy(&kb, &KF[t][c], 16);                                                                                              \
+                S[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(qhi[c], kb, S[t], 0, 0, 0);                                                              \
+                S[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(qlo[c], kb, S[t], 0, 0, 0);                                                              \
+            }                                                                                                                                          \
+        }                                                                                                                                              \
+        float mx[4];                                                                                                                                   \
+        _Pragma("unroll")                                                                                                                              \
+        for (int r = 0; r < 4; r++) {                                                                                                                  \
+            mx[r] = -INFINITY;                                                                                                                         \
+        _Pragma("unroll")                                                                                                                              \
+            for (int t = 0; t < 2; t++) {                                                                                                              \
+                float s = S[t][r] * scale;                                                                                                             \
+                if constexpr (I8) s = S[t][r] * KS[t] * scale;                                                                                         \
+                if (softcap != 0.f) s = softcap * fast_tanh(s * rcap);                                                                                 \
+                if ((KEY0) + t * 16 + l16 >= lenr[r]) s = -INFINITY;                                                                                   \
+                S[t][r] = s;                                                                                                                           \
+                mx[r] = fmaxf(mx[r], s);                                                                                                               \
+            }                                                                                                                                          \
+            mx[r] = group_max16(mx[r]);                                                                                                                \
+        }                                                                                                                                              \
+        float alpha[4];                                                                                                                                \
+        _Pragma("unroll")                                                                                                                              \
+        for (int r = 0; r < 4; r++) {                                                                                                                  \
+            float mn = fmaxf(mrun[r], mx[r]);                                                                                                          \
+            alpha[r] = __expf(mrun[r] - mn);                                                                                                           \
+            mrun[r] = mn;                                                                                                                              \
+            float ps = 0.f;                                                                                                                            \
+        _Pragma("unroll")                                                                                                                              \
+            for (int t = 0; t < 2; t++) {                                                                                                              \
+                float p = __expf(S[t][r] - mn);                                                                                                        \
+                ps += p;                                                                                                                               \
+                if constexpr (I8) p = ((KEY0) + t * 16 + l16 < lenr[r]) ? p * VS[t] : 0.f;                                                             \
+                half_t hi = (half_t)p;                                                                                                                 \
+                int idx = (4 * lg + r) * 32 + t * 16 + l16;                                                                                            \
+                pbuf[idx] = hi;                                                                                                                        \
+                pbuf[512 + idx] = (half_t)(p - (float)hi);                                                                                             \
+            }                                                                                                                                          \
+            lrun[r] = lrun[r] * alpha[r] + ps;                                                                                                         \
+        }                                                                                                                                              \
+        if (__builtin_amdgcn_ballot_w64(alpha[0] != 1.f || alpha[1] != 1.f || alpha[2] != 1.f || alpha[3] != 1.f) != 0) {                              \
+        _Pragma("unroll")                                                                                                                              \
+            for (int ct = 0; ct < NCT; ct++)                                                                                                           \
+        _Pragma("unroll")                                                                                                                              \
+                for (int r = 0; r < 4; r++) O[ct][r] *= alpha[r];                                                                                      \
+        }                                                                                                                                              \
+        __syncthreads();                                                                                                                               \
+        half8_t phi, plo;                                                                                                                              \
+        {                                                                                                                                              \
+            uint4_t a = *(const uint4_t *)(pbuf + l16 * 32 + lg * 8), bq = *(const uint4_t *)(pbuf + 512 + l16 * 32 + lg * 8);                         \
+            __builtin_memcpy(&phi, &a, 16);                                                                                                            \
+            __builtin_memcpy(&plo, &bq, 16);                                                                                                           \
+        }                                                                                                                                              \
+        __syncthreads();                                                                                                                               \
+        _Pragma("unroll")                                                                                                                              \
+        for (int ct = 0; ct < NCT; ct++) {                                                                                                             \
+            half8_t vb;                                                                                                                                \
+            if constexpr (I8)                                                                                                                          \
+                vb = kv8_to_half8(VF[ct >> 1][(ct & 1) * 2], VF[ct >> 1][(ct & 1) * 2 + 1]);                                                           \
+            else                                                                                                                                       \
+                __builtin_memcpy(&vb, &VF[ct], 16);                                                                                                    \
+            O[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(phi, vb, O[ct], 0, 0, 0);                                                                   \
+            O[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(plo, vb, O[ct], 0, 0, 0);                                                                   \
+        }                                                                                                                                              \
+    }
+
+template <int HD, bool I8, bool ROWS = false, bool DEEP = false, int DEEP_UNITS = 2>
 __device__ __forceinline__ void attn_partial_body(const AttnItem *__restrict__ items, const int *__restrict__ rowLen, const int *__restrict__ rowSlot,
                                                   const int *__restrict__ tables, int tabStride, const void *__restrict__ KpV,
                                                   const void *__restrict__ VpV, const float *__restrict__ Ksc, const float *__restrict__ Vsc,
@@ -263,6 +344,48 @@ __device__ __forceinline__ void attn_partial_body(const AttnItem *__restrict__ i
     const float rcap = softcap != 0.f ? 1.f / softcap : 0.f;
 
     const size_t regionBytes = (size_t)64 * HD * ELEM;
+    if constexpr (DEEP) {
+        // DEEP_UNITS units in flight per wave: unit i+DEEP_UNITS is requested as soon as unit i has been worked on, so a wave that has the SIMD
+        // to itself overlaps its memory latency with its own arithmetic. For steps whose work list leaves most SIMDs one wave
+        // (few or short sequences); the units are worked on in the same order, so the results are the plain loop's bit for bit.
+        struct Unit {
+            uint4_t kf[2][KL], vf[VL];
+            float ks[2], vs[2];
+        };
+        const int nU = min(2 * (it.b1 - it.b0), (len - it.b0 * 64 + 31) >> 5); // units with a key of the longest row
+        auto load_unit = [&](Unit &un, int i) {
+            const int blk = tab[it.b0 + (i >> 1)], u = i & 1;
+            const uint4_t *Kr = (const uint4_t *)((const char *)KpV + ((size_t)blk * nKV + it.kvh) * regionBytes);
+            const uint4_t *Vr = (const uint4_t *)((const char *)VpV + ((size_t)blk * nKV + it.kvh) * regionBytes);
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int c = 0; c < KL; c++) un.kf[t][c] = __builtin_nontemporal_load(Kr + ((u * 2 + t) * KL + c) * 64 + lane);
+#pragma unroll
+            for (int ct = 0; ct < VL; ct++) un.vf[ct] = __builtin_nontemporal_load(Vr + (u * VL + ct) * 64 + lane);
+            un.ks[0] = un.ks[1] = un.vs[0] = un.vs[1] = 1.f;
+            if constexpr (I8) {
+                const size_t srow = ((size_t)blk * nKV + it.kvh) * 64;
+#pragma unroll
+                for (int t = 0; t < 2; t++) un.ks[t] = Ksc[srow + u * 32 + t * 16 + l16], un.vs[t] = Vsc[srow + u * 32 + t * 16 + l16];
+            }
+        };
+        Unit un[DEEP_UNITS];
+#pragma unroll
+        for (int j = 0; j < DEEP_UNITS; j++)
+            if (j < nU) load_unit(un[j], j);
+        for (int i0 = 0; i0 < nU; i0 += DEEP_UNITS) {
+#pragma unroll
+            for (int j = 0; j < DEEP_UNITS; j++) {
+                const int i = i0 + j;
+                if (i < nU) {
+                    const int key0 = (it.b0 + (i >> 1)) * 64 + (i & 1) * 32;
+                    RD_ATTN_UNIT(un[j].kf, un[j].vf, un[j].ks, un[j].vs, key0)
+                    if (i + DEEP_UNITS < nU) load_unit(un[j], i + DEEP_UNITS);
+                }
+            }
+        }
+    } else
     for (int b = it.b0; b < it.b1; b++) {
         const int blk = tab[b];
         const uint4_t *Kr = (const uint4_t *)((const char *)KpV + ((size_t)blk * nKV + it.kvh) * regionBytes);
@@ -284,82 +407,7 @@ __device__ __forceinline__ void attn_partial_body(const AttnItem *__restrict__ i
 #pragma unroll
                 for (int t = 0; t < 2; t++) ks[t] = Ksc[srow + u * 32 + t * 16 + l16], vs[t] = Vsc[srow + u * 32 + t * 16 + l16];
             }
-            float4v S[2];
-#pragma unroll
-            for (int t = 0; t < 2; t++) {
-                S[t] = (float4v){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int c = 0; c < NC; c++) {
-                    half8_t kb;
-                    if constexpr (I8)
-                        kb = kv8_to_half8(kf[t][c >> 1][(c & 1) * 2], kf[t][c >> 1][(c & 1) * 2 + 1]);
-                    else
-                        __builtin_memcpy(&kb, &kf[t][c], 16);
-                    S[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(qhi[c], kb, S[t], 0, 0, 0);
-                    S[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(qlo[c], kb, S[t], 0, 0, 0);
-                }
-            }
-            // lane (key l16 of tile t, head rows 4*lg+r)
-            float mx[4];
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                mx[r] = -INFINITY;
-#pragma unroll
-                for (int t = 0; t < 2; t++) {
-                    float s = S[t][r] * scale;
-                    if constexpr (I8) s = S[t][r] * ks[t] * scale;
-                    if (softcap != 0.f) s = softcap * fast_tanh(s * rcap);
-                    if (key0 + t * 16 + l16 >= lenr[r]) s = -INFINITY;
-                    S[t][r] = s;
-                    mx[r] = fmaxf(mx[r], s);
-                }
-                mx[r] = group_max16(mx[r]); // the 16 key lanes of this head row are one DPP row
-            }
-            float alpha[4];
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                float mn = fmaxf(mrun[r], mx[r]);
-                alpha[r] = __expf(mrun[r] - mn); // first unit: exp(-inf) = 0
-                mrun[r] = mn;
-                float ps = 0.f;
-#pragma unroll
-                for (int t = 0; t < 2; t++) {
-                    float p = __expf(S[t][r] - mn);
-                    ps += p;
-                    if constexpr (I8) p = (key0 + t * 16 + l16 < lenr[r]) ? p * vs[t] : 0.f; // a key past the end has no scale to trust
-                    half_t hi = (half_t)p;
-                    int idx = (4 * lg + r) * 32 + t * 16 + l16;
-                    pbuf[idx] = hi;
-                    pbuf[512 + idx] = (half_t)(p - (float)hi);
-                }
-                lrun[r] = lrun[r] * alpha[r] + ps;
-            }
-            // Rescale the running output only when some row's maximum moved: past the first keys of a sequence it rarely does,
-            // and a factor of exactly 1 changes nothing.
-            if (__builtin_amdgcn_ballot_w64(alpha[0] != 1.f || alpha[1] != 1.f || alpha[2] != 1.f || alpha[3] != 1.f) != 0) {
-#pragma unroll
-                for (int ct = 0; ct < NCT; ct++)
-#pragma unroll
-                    for (int r = 0; r < 4; r++) O[ct][r] *= alpha[r];
-            }
-            __syncthreads();
-            half8_t phi, plo;
-            {
-                uint4_t a = *(const uint4_t *)(pbuf + l16 * 32 + lg * 8), bq = *(const uint4_t *)(pbuf + 512 + l16 * 32 + lg * 8);
-                __builtin_memcpy(&phi, &a, 16);
-                __builtin_memcpy(&plo, &bq, 16);
-            }
-            __syncthreads();
-#pragma unroll
-            for (int ct = 0; ct < NCT; ct++) {
-                half8_t vb;
-                if constexpr (I8)
-                    vb = kv8_to_half8(vf[ct >> 1][(ct & 1) * 2], vf[ct >> 1][(ct & 1) * 2 + 1]);
-                else
-                    __builtin_memcpy(&vb, &vf[ct], 16);
-                O[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(phi, vb, O[ct], 0, 0, 0);
-                O[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(plo, vb, O[ct], 0, 0, 0);
-            }
+            RD_ATTN_UNIT(kf, vf, ks, vs, key0)
         }
     }
     // lane (d column l16 of tile ct, head rows 4*lg+r): O[ct][r]; l partial sums live per key lane -> reduce over the 16 lanes
@@ -400,6 +448,32 @@ extern "C" __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3
         attn_partial_body<128, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, Ksc, Vsc, q, part, nH, nKV, scale, softcap, pbuf);
     else
         attn_partial_body<64, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, Ksc, Vsc, q, part, nH, nKV, scale, softcap, pbuf);
+}
+
+// The same two kernels with two units in flight per wave (see DEEP above), one wave per SIMD.
+extern "C" __global__ __launch_bounds__(64) void rd_k_attn_partial_deep(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
+                                                                        const int *__restrict__ rowSlot, const int *__restrict__ tables, int tabStride,
+                                                                        const uint16_t *__restrict__ Kp, const uint16_t *__restrict__ Vp,
+                                                                        const float *__restrict__ q, float *__restrict__ part, int nH, int nKV, int HD,
+                                                                        float scale, float softcap) {
+    __shared__ half_t pbuf[1024];
+    if (HD == 128)
+        attn_partial_body<128, false, false, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, pbuf);
+    else
+        attn_partial_body<64, false, false, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, pbuf);
+}
+
+extern "C" __global__ __launch_bounds__(64) void rd_k_attn_partial_deep_i8(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
+                                                                      const int *__restrict__ rowSlot, const int *__restrict__ tables, int tabStride,
+                                                                      const signed char *__restrict__ Kp, const signed char *__restrict__ Vp,
+                                                                      const float *__restrict__ Ksc, const float *__restrict__ Vsc,
+                                                                      const float *__restrict__ q, float *__restrict__ part, int nH, int nKV, int HD,
+                                                                      float scale, float softcap) {
+    __shared__ half_t pbuf[1024];
+    if (HD == 128)
+        attn_partial_body<128, true, false, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, Ksc, Vsc, q, part, nH, nKV, scale, softcap, pbuf);
+    else
+        attn_partial_body<64, true, false, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, Ksc, Vsc, q, part, nH, nKV, scale, softcap, pbuf);
 }
 
 // Items of several positions each (see ROWS above): steps that carry more than one row of a sequence — prompt passes, verification.

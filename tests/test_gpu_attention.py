@@ -173,3 +173,25 @@ def test_rows_of_a_sequence_share_items_and_equal_solo_rows(dev, nH, nKV, hd, kv
         want = oracle_attn(rl, rt(k1), rt(v1), q, nH, nKV, hd, scale, softcap)
         err = np.abs(got - want).max() / np.abs(want).max()
         assert err <= 1e-4, (softcap, err)
+
+
+@pytest.mark.parametrize("kv", ["f16", "i8"])
+def test_short_work_lists_run_two_units_in_flight_with_the_same_bits(dev, kv):
+    """A work list of at most one item per SIMD runs the kernel that keeps two units of 32 keys in flight per wave; with the
+    switch that turns it off the plain kernel runs. Same units in the same order: identical output bits."""
+    import os
+    lens = [1, 31, 32, 33, 64, 97, 700, 2049]
+    nH, nKV, hd = 8, 2, 128
+    tot, kvd = sum(lens), nKV * hd
+    k = synth.normal(21, tot * kvd).reshape(tot, kvd)
+    v = synth.normal(22, tot * kvd).reshape(tot, kvd)
+    q = synth.normal(23, len(lens) * nH * hd).reshape(len(lens), nH * hd)
+    scale = float(1.0 / np.sqrt(hd))
+    for softcap in (0.0, 20.0):
+        deep = dev.attn_ragged(lens, k, v, q, nH, nKV, hd, scale, softcap, kv=kv)
+        os.environ["ROCMDECODE_NO_DEEP_ATTN"] = "1"
+        try:
+            plain = dev.attn_ragged(lens, k, v, q, nH, nKV, hd, scale, softcap, kv=kv)
+        finally:
+            del os.environ["ROCMDECODE_NO_DEEP_ATTN"]
+        assert np.array_equal(deep.view(np.uint32), plain.view(np.uint32)), softcap
