@@ -89,6 +89,8 @@ def parse_args():
     ap.add_argument("--layers", type=int, default=32, help="model depth (32 = the Llama-3-8B shape; fewer only for debugging)")
     ap.add_argument("--batch", type=int, default=32)
     ap.add_argument("--seed", type=int, default=1234)
+    ap.add_argument("--ctx-min", type=int, default=512, help="c4: shortest context (the configuration's own range is 512..4096)")
+    ap.add_argument("--ctx-max", type=int, default=4096, help="c4: longest context")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--kv", default="f16", choices=["f16", "i8"],
                     help="KV cache element (c4 and c3): f16 as the metric is quoted, or goinfer's int8 cache (KVQuant i8), a variant of the workload")
@@ -109,7 +111,7 @@ def run_c4(args):
     cfg = workloads.llama3_8b_cfg(args.layers)
     B = args.batch
     rng = np.random.default_rng(args.seed)
-    lens = rng.integers(512, 4097, B).astype(np.int64)  # context lengths uniform in [512, 4096]
+    lens = rng.integers(args.ctx_min, args.ctx_max + 1, B).astype(np.int64)  # context lengths uniform in [512, 4096] unless asked otherwise
     ids0 = rng.integers(0, cfg["vocab"], B).astype(np.int32)
     cap = int(lens.max()) + args.steps + args.warmup + 8
     dev = capi.Device(0)
@@ -181,8 +183,8 @@ def run_c4(args):
         "ms_per_step": round(float(ms.mean()), 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16",
         "data": "synthetic: N(0,0.02) weights quantized to Q4_K (int8 head), N(0,1) KV, random token ids",
-        "config": {"workload": "configs[3]: %s, %d layers, B=%d ragged, ctx U[512,4096], greedy decode%s"
-                               % (cfg["name"], cfg["n_layers"], B, "" if args.kv == "f16" else " (variant: int8 KV cache)"), "kv": args.kv,
+        "config": {"workload": "configs[3]: %s, %d layers, B=%d ragged, ctx U[%d,%d], greedy decode%s"
+                               % (cfg["name"], cfg["n_layers"], B, args.ctx_min, args.ctx_max, "" if args.kv == "f16" else " (variant: int8 KV cache)"), "kv": args.kv,
                    "batch": B, "ctx_min": int(lens.min()), "ctx_max": int(lens.max()), "ctx_mean": float(lens.mean()), "seed": args.seed},
         "step_hbm": {"algorithmic_bytes_per_step": int(step_bytes), "achieved_GBs": round(step_gbs, 1), "frac_of_peak": round(step_gbs / HBM_PEAK_GBS, 4),
                      "weights_bytes": int(w_bytes), "kv_read_bytes": int(kv_read)},

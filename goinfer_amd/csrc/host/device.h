@@ -4,6 +4,7 @@
 #include "hipdyn.h"
 #include <stdarg.h>
 #include <stdio.h>
+#include <algorithm>
 #include <string>
 #include <vector>
 
@@ -67,11 +68,17 @@ struct DevBuf {
 constexpr unsigned GEMM_THREADS = 320, GATEUP_THREADS = 640;
 
 // How many 64-position KV blocks one attention work item covers for a sequence of nb blocks: every (sequence, kv head) is
-// cut into at most ATTN_PIECES pieces. The cut depends on the sequence's own length only, never on what else is in the
+// cut into pieces. The cut depends on the sequence's own length only, never on what else is in the
 // batch: the partial results are merged in piece order, so this is what keeps a row computed in a batch bit-identical to
 // the same row computed alone.
-constexpr int ATTN_PIECES = 16; // = RD_ATTN_PIECES of the combine kernels
-inline int attn_chunk_blocks(int nb) { return (nb + ATTN_PIECES - 1) / ATTN_PIECES; }
+constexpr int ATTN_PIECES = 16; // = RD_ATTN_PIECES of the combine kernels: pieces they fold per round
+// Blocks per item: a sixteenth of the sequence, but at most ATTN_MAX_CHUNK blocks (512 keys), so that a sequence of more than 128
+// blocks is cut into more than 16 items and even a lone long sequence spreads over the chip. (A cap of four blocks serves a
+// lone 8k-token sequence better, 18 against 29 us per layer, but costs the 64-sequence attention benchmark 5 %.)
+constexpr int ATTN_MAX_CHUNK = 8;
+inline int attn_chunk_blocks(int nb) { return std::min((nb + ATTN_PIECES - 1) / ATTN_PIECES, ATTN_MAX_CHUNK); }
+// the most items one (row, kv head) of a sequence of up to nb blocks is cut into
+inline int attn_max_pieces(int nb) { return std::max(ATTN_PIECES, (nb + ATTN_MAX_CHUNK - 1) / ATTN_MAX_CHUNK); }
 
 // One attention work item: blocks [b0,b1) of one kv head of one sequence, for the step's row `row` — or, from the grouping
 // builder, for rows row..row+n-1 with n in the high 16 bits of kvh; one wave each.

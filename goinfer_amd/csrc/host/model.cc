@@ -398,8 +398,6 @@ extern "C" int rd_model_finalize(rd_model *m) {
         RC(d->alloc(&m->XpE, (size_t)c.n_experts * (I / 128) * LIN_PANEL_BYTES));
         HIPCHK(MemsetAsync(m->XpE, 0, (size_t)c.n_experts * (I / 128) * LIN_PANEL_BYTES, d->stream));
     }
-    m->host_stage_bytes = sizeof(float) * R * H + (1u << 20);
-    HIPCHK(HostMalloc(&m->host_stage, m->host_stage_bytes * rd_model::STAGE_SLOTS, 0));
     for (auto &e : m->stage_ev) HIPCHK(EventCreate(&e));
     m->finalized = true;
     return d->sync();
@@ -450,9 +448,8 @@ extern "C" int rd_kv_configure_typed(rd_model *m, int slots, int ctx_cap, int kv
     RC(d->alloc((void **)&m->tables, sizeof(int) * tab.size()));
     RC(d->h2d(m->tables, tab.data(), sizeof(int) * tab.size()));
     m->slot_len.assign((size_t)slots, 0);
-    // attention work list: ~4096 items plus one per (row, kv head) of rounding
-    m->max_items = m->max_rows * c.n_kv_heads * ATTN_PIECES;
-    // an item writes one head row per query head of its kv head, or a whole tile of 16 when it covers several positions
+    // attention work list: every (row, kv head) of a step is cut into at most attn_max_pieces items
+    m->max_items = m->max_rows * c.n_kv_heads * attn_max_pieces(m->blocks_per_slot);
     RC(alloc_f32(d, &m->part, (size_t)m->max_items * ATTN_TILE_ROWS * (c.head_dim + 2)));
     // The step's metadata lives in one device block so a step uploads it with one copy:
     // [row slot R][row position R][row length R][row draw records R x 6][item ranges max_rows*nKV*3][items max_items x 4] ints, R = ROWS_MAX
@@ -463,6 +460,10 @@ extern "C" int rd_kv_configure_typed(rd_model *m, int slots, int ctx_cap, int kv
     m->rowSlot = m->meta, m->rowPos = m->meta + RM, m->rowLen = m->meta + 2 * RM, m->rowDraw = m->meta + 3 * RM;
     m->itemStart = m->meta + rd_model::META_HDR;
     m->items = (AttnItemH *)(m->meta + rd_model::META_HDR + rangeInts);
+    // pinned staging, STAGE_SLOTS slots: the step's metadata block as on the device, then the embeddings
+    m->stage_meta_bytes = (sizeof(int) * m->meta_ints + 4095) & ~(size_t)4095;
+    m->host_stage_bytes = m->stage_meta_bytes + sizeof(float) * (size_t)m->max_rows * c.hidden;
+    HIPCHK(HostMalloc(&m->host_stage, m->host_stage_bytes * rd_model::STAGE_SLOTS, 0));
     return d->sync();
 }
 
@@ -694,7 +695,7 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
         int *hm = (int *)st; // the metadata block, laid out as on the device
         const size_t rangeInts = (size_t)m->max_rows * nKV * ATTN_RANGE_INTS;
         constexpr int RM = rd_model::ROWS_MAX;
-        float *eh = (float *)(st + (1u << 20));
+        float *eh = (float *)(st + m->stage_meta_bytes);
         for (int b = 0; b < B; b++) hm[b] = slot[b], hm[RM + b] = pos[b], hm[2 * RM + b] = pos[b] + 1;
         // Draw records (resident/forward.go:43-52 BatchDraw) with Sampler.gumbelDraw's guards applied here
         // (internal/runtime/sampling/sampler_gumbel.go:80-88): a temperature <= 0 means 1, and one so small that 1/T

@@ -97,6 +97,7 @@ struct rd_model {
     static constexpr int STAGE_SLOTS = 4;
     void *host_stage = nullptr;
     size_t host_stage_bytes = 0; // per slot
+    size_t stage_meta_bytes = 0; // of which the metadata block (the embeddings follow)
     hipEvent_t stage_ev[STAGE_SLOTS] = {};
     bool stage_busy[STAGE_SLOTS] = {};
     unsigned stage_next = 0;

@@ -505,8 +505,7 @@ extern "C" __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3
 // Merge the partials of one (row, query head) in ascending item order (deterministic):
 // out = sum O_i e^(m_i-M) / sum l_i e^(m_i-M). itemStart[3*(row*nKV+kvh)] and the entry after it bound that pair's items, the
 // third entry is the row's place among the positions its items cover (0 where an item is one position); partRows is the
-// number of head rows an item writes (G, or 16 from the kernels whose items cover several positions). The
-// host cuts a sequence into at most RD_ATTN_PIECES items. Block = RD_ATTN_PIECES * HD/4 threads: thread (item i, quarter
+// number of head rows an item writes (G, or 16 from the kernels whose items cover several positions). Block = RD_ATTN_PIECES * HD/4 threads: thread (item i, quarter
 // dq) brings four values of item i into LDS, so every item's load is in flight at once; the first HD/4 threads then fold
 // the items in order. lds: RD_ATTN_PIECES*(HD+2) floats. Returns true in the threads that hold a result (four consecutive d).
 #define RD_ATTN_PIECES 16
@@ -515,27 +514,47 @@ __device__ __forceinline__ bool attn_combine_block(const float *__restrict__ par
     const int Q = HD >> 2, ti = threadIdx.x / Q, dq = threadIdx.x - ti * Q;
     const int G = nH / nKV, kvh = head / G, g = head % G;
     const int *rg = itemStart + (m * nKV + kvh) * 3;
-    const int i0 = rg[0], n = min(rg[1] - i0, RD_ATTN_PIECES), sub = rg[2];
+    const int i0 = rg[0], n = rg[1] - i0, sub = rg[2];
     const size_t stride = (size_t)partRows * (HD + 2);
+    const float *p0 = part + ((size_t)i0 * partRows + sub * G + g) * (HD + 2);
     float *vals = lds, *mm = lds + RD_ATTN_PIECES * HD, *ll = mm + RD_ATTN_PIECES;
-    if (ti < n) {
-        const float *p = part + ((size_t)i0 * partRows + sub * G + g) * (HD + 2) + (size_t)ti * stride;
-        const float2 a = *(const float2 *)(p + dq * 4), b = *(const float2 *)(p + dq * 4 + 2); // rows are 8-byte aligned (HD+2 is even)
-        float *v = vals + ti * HD + dq * 4;
-        v[0] = a.x, v[1] = a.y, v[2] = b.x, v[3] = b.y;
-        if (dq == 0) mm[ti] = p[HD], ll[ti] = p[HD + 1];
-    }
-    __syncthreads();
-    if (ti != 0) return false;
+    // A sequence of up to 128 blocks has at most RD_ATTN_PIECES items: one round. A longer one has more (its items stay short so
+    // that even a lone long sequence spreads over the chip): the maximum over all of them first, then rounds of RD_ATTN_PIECES
+    // folded in the same ascending order with the same arithmetic.
     float M = -INFINITY;
-    for (int i = 0; i < n; i++) M = fmaxf(M, mm[i]);
-    float num[4] = {0.f, 0.f, 0.f, 0.f}, den = 0.f;
-    for (int i = 0; i < n; i++) {
-        const float *v = vals + i * HD + dq * 4;
-        const float w = __expf(mm[i] - M);
-        num[0] = fmaf(v[0], w, num[0]), num[1] = fmaf(v[1], w, num[1]), num[2] = fmaf(v[2], w, num[2]), num[3] = fmaf(v[3], w, num[3]);
-        den = fmaf(ll[i], w, den);
+    if (n > RD_ATTN_PIECES) {
+        for (int i = threadIdx.x; i < n; i += blockDim.x) M = fmaxf(M, p0[(size_t)i * stride + HD]);
+        for (int o = 32; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o, 64));
+        if ((threadIdx.x & 63) == 0) mm[threadIdx.x >> 6] = M; // at most 8 waves: fits the 16 floats of mm
+        __syncthreads();
+        M = -INFINITY;
+        for (int w = 0; w < (int)(blockDim.x >> 6); w++) M = fmaxf(M, mm[w]);
+        __syncthreads(); // mm is reused by the rounds
     }
+    float num[4] = {0.f, 0.f, 0.f, 0.f}, den = 0.f;
+    for (int base = 0; base < n; base += RD_ATTN_PIECES) {
+        const int nb = min(n - base, RD_ATTN_PIECES);
+        if (ti < nb) {
+            const float *p = p0 + (size_t)(base + ti) * stride;
+            const float2 a = *(const float2 *)(p + dq * 4), b = *(const float2 *)(p + dq * 4 + 2); // rows are 8-byte aligned (HD+2 is even)
+            float *v = vals + ti * HD + dq * 4;
+            v[0] = a.x, v[1] = a.y, v[2] = b.x, v[3] = b.y;
+            if (dq == 0) mm[ti] = p[HD], ll[ti] = p[HD + 1];
+        }
+        __syncthreads();
+        if (ti == 0) {
+            if (n <= RD_ATTN_PIECES)
+                for (int i = 0; i < nb; i++) M = fmaxf(M, mm[i]);
+            for (int i = 0; i < nb; i++) {
+                const float *v = vals + i * HD + dq * 4;
+                const float w = __expf(mm[i] - M);
+                num[0] = fmaf(v[0], w, num[0]), num[1] = fmaf(v[1], w, num[1]), num[2] = fmaf(v[2], w, num[2]), num[3] = fmaf(v[3], w, num[3]);
+                den = fmaf(ll[i], w, den);
+            }
+        }
+        if (base + RD_ATTN_PIECES < n) __syncthreads(); // the next round overwrites what the folding threads read
+    }
+    if (ti != 0) return false;
 #pragma unroll
     for (int e = 0; e < 4; e++) out[e] = num[e] / den;
     return true;

@@ -195,3 +195,24 @@ def test_short_work_lists_run_two_units_in_flight_with_the_same_bits(dev, kv):
         finally:
             del os.environ["ROCMDECODE_NO_DEEP_ATTN"]
         assert np.array_equal(deep.view(np.uint32), plain.view(np.uint32)), softcap
+
+
+@pytest.mark.parametrize("kv", ["f16", "i8"])
+def test_long_sequences_are_cut_into_more_than_sixteen_items(dev, kv):
+    """Beyond 128 blocks an item stays at eight blocks, so the items of a (sequence, kv head) outnumber what the combine folds in
+    one round: 8193 keys (17 items), 9000 (18) and 20000 (40) beside a short sequence, against the oracle."""
+    lens = [8193, 9000, 300, 20000]
+    nH, nKV, hd = 8, 2, 128
+    tot, kvd = sum(lens), nKV * hd
+    rng = np.random.default_rng(31)
+    k = rng.standard_normal((tot, kvd), dtype=np.float32).astype(np.float16).astype(np.float32)
+    v = rng.standard_normal((tot, kvd), dtype=np.float32).astype(np.float16).astype(np.float32)
+    q = rng.standard_normal((len(lens), nH * hd), dtype=np.float32)
+    scale = float(1.0 / np.sqrt(hd))
+    got = dev.attn_ragged(lens, k, v, q, nH, nKV, hd, scale, 0.0, kv=kv)
+    rt = (lambda x: x) if kv == "f16" else (lambda x: i8_round_trip(x, nKV, hd))
+    want = oracle_attn(lens, rt(k), rt(v), q, nH, nKV, hd, scale, 0.0)
+    err = np.abs(got - want).max() / np.abs(want).max()
+    assert err <= 1e-4, err
+    again = dev.attn_ragged(lens, k, v, q, nH, nKV, hd, scale, 0.0, kv=kv)
+    assert np.array_equal(got.view(np.uint32), again.view(np.uint32))

@@ -212,6 +212,39 @@ def uploaded_prefix_deviation(dev, kv):
         pair.close()
 
 
+def test_long_context_row_in_a_batch(dev):
+    """A sequence of more than 128 blocks is cut into more than 16 attention items (the combine then folds them in rounds): an
+    8400-row uploaded prefix beside a short sequence, two steps against the oracle, batched rows == solo rows bit for bit."""
+    cfg = dense_cfg(n_layers=2, hidden=256, n_heads=4, n_kv=2, head_dim=64, inter=512, vocab=512)
+    pair = Pair(cfg, seed=12, dev=dev, slots=4, ctx_cap=8448)
+    try:
+        rng = np.random.default_rng(13)
+        kvd = cfg["n_kv"] * cfg["head_dim"]
+        lens = [8400, 37]
+        caches = [pair.oracle.new_cache(8448) for _ in lens]
+        for s, n in enumerate(lens):
+            for l in range(cfg["n_layers"]):
+                k = rng.standard_normal((n, kvd)).astype(np.float32)
+                v = rng.standard_normal((n, kvd)).astype(np.float32)
+                pair.oracle.cache_upload(caches[s], l, 0, k, v)
+                pair.gpu.kv_upload(s, l, 0, k, v)
+                pair.gpu.kv_upload(2 + s, l, 0, k, v)  # twin slots, stepped alone
+        for step in range(2):
+            toks = rng.integers(0, cfg["vocab"], 2)
+            emb = pair.emb[toks]
+            want = pair.oracle.step(emb, caches)
+            got, _ = pair.gpu.step_batch([0, 1], [n + step for n in lens], emb)
+            for b in range(2):
+                ok, d = logits_close(got[b], want[b], floor=1e-2)
+                assert ok, (step, b, d)
+                solo = pair.gpu.forward(2 + b, lens[b] + step, emb[b])
+                assert np.array_equal(solo.view(np.uint32), got[b].view(np.uint32)), (step, b)
+        for c in caches:
+            pair.oracle.free_cache(c)
+    finally:
+        pair.close()
+
+
 def test_i8_kv_uploaded_prefix(dev):
     """rd_kv_upload into the int8 cache. What the GPU's f16 GEMM operands cost against the oracle's integer-exact ones is the
     same whatever the cache holds, so the int8 cache may not sit further from its oracle than the f16 cache sits from its own

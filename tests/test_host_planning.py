@@ -1,6 +1,7 @@
 """Host planning of a step, checked without a GPU through the C ABI (rd_plan_attention, rd_plan_gemm).
 
-What the plans must guarantee: every (row, kv head) has its blocks covered once, in order, by at most 16 items; a row's cut
+What the plans must guarantee: every (row, kv head) has its blocks covered once, in order, by items of a sixteenth of the
+sequence but at most eight blocks (so a sequence of up to 128 blocks has at most 16 items, a longer one more); a row's cut
 depends on its own length only (the partial results are merged in item order, so this is what keeps a row in a batch
 bit-identical to the row alone, goinfer's StepBatch contract, decoder/resident/subsystems.go:102-110); rows share items only
 when they are consecutive positions of one sequence with the same number of blocks."""
@@ -9,7 +10,7 @@ import pytest
 
 from goinfer_amd import capi
 
-PIECES = 16
+PIECES, MAX_CHUNK = 16, 8
 
 
 def rows_of(item):
@@ -26,7 +27,9 @@ def check_cover(items, ranges, lens, n_kv):
         nb = (n + 63) // 64
         for h in range(n_kv):
             c = cuts(items, ranges, r, h)
-            assert 1 <= len(c) <= PIECES
+            chunk = min(-(-nb // PIECES), MAX_CHUNK)
+            assert len(c) == -(-nb // chunk) and all(b1 - b0 <= chunk for b0, b1 in c)
+            assert len(c) <= PIECES or nb > PIECES * MAX_CHUNK
             assert c[0][0] == 0 and c[-1][1] == nb
             assert all(a[1] == b[0] for a, b in zip(c, c[1:])) and all(b0 < b1 for b0, b1 in c)
             i0, i1, sub = ranges[r, h]
@@ -38,7 +41,7 @@ def check_cover(items, ranges, lens, n_kv):
 @pytest.mark.parametrize("n_kv,G", [(8, 4), (2, 7), (4, 8), (1, 1), (1, 16)])
 def test_one_row_per_sequence(n_kv, G):
     rng = np.random.default_rng(3)
-    lens = [1, 63, 64, 65, 1024, 1025, 8192, 4097] + list(rng.integers(1, 9000, 24))
+    lens = [1, 63, 64, 65, 1024, 1025, 8192, 8193, 40000] + list(rng.integers(1, 9000, 23))
     items, ranges, grouped = capi.plan_attention(lens, None, G, n_kv)
     assert not grouped and all(int(it[1]) >> 16 == 0 for it in items)
     check_cover(items, ranges, lens, n_kv)
