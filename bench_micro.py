@@ -36,6 +36,12 @@ def base_line(metric, value, unit, steps, warmup, ms, workload, data, extra_cfg=
 
 
 # ------------------------------------------------------------------------------------------------------------ C2
+def counter_traffic(key):
+    """HBM bytes per launch of a kernel on a workload as the rocprofv3 counter runs measured them (profiles/traffic.json), or None."""
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    return json.load(open(tpath)).get(key) if os.path.exists(tpath) else None
+
+
 def run_c2(args):
     """Q4_K dequant-GEMM: up 14336x4096, down 4096x14336, fused gate|up + SwiGLU + quantization; M in {1,4,16,32,64}.
     A step is one GEMM call (M = 64 is two passes of 32 rows, as the step batches rows)."""
@@ -59,7 +65,8 @@ def run_c2(args):
                     head["us"] / 1e3, "configs[1]: Q4_K GEMM 14336x4096 / 4096x14336 / fused gate|up, M in {1,4,16,32,64}",
                     "synthetic: random Q4_K super-blocks with sane f16 scales, 8 weight copies used round-robin", {"cases": cases})
     out["roofline"] = {"bound": "hbm", "achieved": head["GBs"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(head["GBs"] / HBM_PEAK_GBS, 4),
-                       "traffic": None, "kernel": "rd_k_gemm_q4k_gateup", "avg_launch_ms": round(head["us"] / 1e3, 5),
+                       "traffic": counter_traffic("gemm_q4k_gateup/ffn-14336x4096-m32"), "kernel": "rd_k_gemm_q4k_gateup",
+                       "avg_launch_ms": round(head["us"] / 1e3, 5),
                        "algorithmic_bytes_per_launch": head["bytes"]}
     cpu = None
     if not args.no_cpu:
@@ -157,7 +164,9 @@ def run_c3(args):
     # the partial kernel is launched once per group of 32 rows: two launches per call here
     per_launch = (kv_bytes + nseq * nH * hd * 4) / 2
     out["roofline"] = {"bound": "hbm", "achieved": round(per_launch / (tp / 2) / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                       "frac": round(per_launch / (tp / 2) / 1e6 / HBM_PEAK_GBS, 4), "traffic": None, "kernel": "rd_k_attn_partial" if kv == "f16" else "rd_k_attn_partial_i8",
+                       "frac": round(per_launch / (tp / 2) / 1e6 / HBM_PEAK_GBS, 4),
+                       "traffic": counter_traffic("attn_partial/64seq-u128-8192") if kv == "f16" and args.seed == 1234 else None,
+                       "kernel": "rd_k_attn_partial" if kv == "f16" else "rd_k_attn_partial_i8",
                        "avg_launch_ms": round(tp / 2, 5), "algorithmic_bytes_per_launch": int(per_launch)}
     cpu = None
     if not args.no_cpu:
@@ -234,10 +243,7 @@ def run_c5(args):
     d2 = float(sum(len(set(idx2[:, l, :].ravel().tolist())) for l in range(layers)))
     g_ms = prof["moe_gemm_gateup"][0] / prof["moe_gemm_gateup"][1]
     per_launch = d2 * ebytes * (2.0 / 3.0) / layers
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "traffic.json")
-    if os.path.exists(tpath):
-        traffic = json.load(open(tpath)).get("gemm_w4a8_moe_gateup/%s" % cfg["name"])
+    traffic = counter_traffic("gemm_w4a8_moe_gateup/%s" % cfg["name"])
     out = base_line("batch-16 decode tok/s, Qwen3-MoE-30B-A3B shape (int4-g32 experts); achieved HBM GB/s vs peak", tok_s, "tok/s", steps, warmup,
                     float(ms.mean()), "configs[4]: %s, %d layers, B=%d ragged, ctx U[256,2048], greedy decode" % (cfg["name"], layers, B),
                     "synthetic: N(0,0.02) weights (Q4_K projections, int4-g32 experts, f32 router, int8 head), N(0,1) KV, random token ids",
