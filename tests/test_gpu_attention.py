@@ -156,9 +156,9 @@ def rows_as_sequences(lens, nq, k, v):
 def test_rows_of_a_sequence_share_items_and_equal_solo_rows(dev, nH, nKV, hd, kv):
     """Several positions of one sequence in one item (they share every K and V read): each row against the oracle and
     bit-identical to the same row as a sequence of its own. The lengths put groups across a block boundary (where the rows
-    part, their cuts differing), at a block's last key, and past the split threshold."""
-    lens = [5, 64, 67, 130, 300, 1100, 1]
-    nq = [5, 3, 6, 9, 2, 7, 1]
+    part, their cuts differing), at a block's last key, past the split threshold, and past 128 blocks."""
+    lens = [5, 64, 67, 130, 300, 1100, 1, 8300]
+    nq = [5, 3, 6, 9, 2, 7, 1, 5]  # the last sequence is cut into more than 16 items: the combine folds them in rounds
     tot, kvd = sum(lens), nKV * hd
     k = synth.normal(11, tot * kvd).reshape(tot, kvd).astype(np.float16).astype(np.float32)  # exactly what the f16 cache holds
     v = synth.normal(12, tot * kvd).reshape(tot, kvd).astype(np.float16).astype(np.float32)
