@@ -1,0 +1,119 @@
+"""A random walk over the resident's entry points (batched steps, ragged steps with several rows per slot, prompt passes,
+truncation, reset, uploaded prefixes) on a few KV slots, checked by replay: whatever order the calls came in, the logits a slot
+last returned are, bit for bit, those of its token history stepped one token at a time on a fresh slot.
+
+This is goinfer's resident contract read as a whole (resident/forward.go:5-38: ForwardN == K x Forward, TruncateTo and Reset
+leave a prefix that behaves as if nothing else had been there; resident/subsystems.go:102-117: a row in a batch == the row
+alone), exercised for what single-feature tests miss: stale state between calls."""
+import numpy as np
+import pytest
+
+from goinfer_amd import capi
+from tests.models import Pair, dense_cfg, moe_cfg
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    d = capi.Device(0)
+    yield d
+    d.close()
+
+
+def bits(x):
+    return np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+
+
+def walk(pair, vocab, slots, cap, seed, n_ops, max_batch, kv_dim=None):
+    """Returns (history per slot, last logits per slot). Slot `slots` (one past the last) is left for the replay."""
+    rng = np.random.default_rng(seed)
+    hist = [[] for _ in range(slots)]  # what each slot holds: a list of ("tok", id) or ("kv", layer arrays)
+    last = [None] * slots
+    g = pair.gpu
+    for _ in range(n_ops):
+        op = rng.choice(["batch", "batch", "ragged", "prefill", "truncate", "reset", "nologits"])
+        if op == "batch":
+            k = int(rng.integers(1, min(slots, max_batch) + 1))
+            chosen = [int(s) for s in rng.permutation(slots)[:k] if len(hist[s]) < cap - 1]
+            if not chosen:
+                continue
+            toks = rng.integers(0, vocab, len(chosen))
+            out, ids = g.step_batch(chosen, [len(hist[s]) for s in chosen], pair.emb[toks], capi.WANT_LOGITS | capi.WANT_ARGMAX)
+            for i, s in enumerate(chosen):
+                hist[s].append(int(toks[i]))
+                last[s] = out[i].copy()
+                assert ids[i] == int(np.argmax(out[i]))
+        elif op == "ragged":
+            k = int(rng.integers(1, min(3, slots) + 1))
+            chosen = [int(s) for s in rng.permutation(slots)[:k]]
+            rows = [int(rng.integers(1, 7)) for _ in chosen]
+            keep = [(s, r) for s, r in zip(chosen, rows) if len(hist[s]) + r < cap]
+            if not keep or sum(r for _, r in keep) > max_batch:
+                continue
+            toks = [rng.integers(0, vocab, r) for _, r in keep]
+            out, _ = g.step_ragged([s for s, _ in keep], [len(hist[s]) for s, _ in keep], [pair.emb[t] for t in toks])
+            off = 0
+            for (s, r), t in zip(keep, toks):
+                hist[s].extend(int(x) for x in t)
+                last[s] = out[off + r - 1].copy()
+                off += r
+        elif op == "prefill":
+            s = int(rng.integers(0, slots))
+            n = int(rng.integers(1, 50))
+            if len(hist[s]) + n >= cap:
+                continue
+            toks = rng.integers(0, vocab, n)
+            last[s] = g.prefill_last(s, len(hist[s]), pair.emb[toks]).copy()
+            hist[s].extend(int(x) for x in toks)
+        elif op == "nologits":
+            s = int(rng.integers(0, slots))
+            if len(hist[s]) >= cap - 1:
+                continue
+            t = int(rng.integers(0, vocab))
+            g.forward_no_logits(s, len(hist[s]), pair.emb[t])
+            hist[s].append(t)
+            last[s] = None  # this call returns nothing to compare; the tokens after it will
+        elif op == "truncate":
+            s = int(rng.integers(0, slots))
+            if len(hist[s]) < 2:
+                continue
+            n = int(rng.integers(1, len(hist[s])))
+            g.kv_truncate(s, n)
+            del hist[s][n:]
+            last[s] = None
+        else:
+            s = int(rng.integers(0, slots))
+            g.kv_reset(s)
+            hist[s] = []
+            last[s] = None
+    return hist, last
+
+
+@pytest.mark.parametrize("seed", [82, 83, 84])
+@pytest.mark.parametrize("kind,kv", [("dense", "f16"), ("dense", "i8"), ("moe", "f16")])
+def test_random_walk_replays_bit_identically(dev, kind, kv, seed):
+    cfg = dense_cfg(n_layers=2) if kind == "dense" else moe_cfg(n_layers=2)
+    slots, cap = 5, 160
+    pair = Pair(cfg, seed=81, dev=dev, slots=slots + 1, ctx_cap=cap, kv=kv)
+    try:
+        hist, last = walk(pair, cfg["vocab"], slots, cap, seed=seed, n_ops=300, max_batch=32 if kind == "moe" else 128)
+        checked = 0
+        for s in range(slots):
+            if not hist[s]:
+                continue
+            # the slot's state, not only its last answer: one more token on the slot and on the replay must agree too
+            pair.gpu.kv_reset(slots)
+            replay = None
+            for p, t in enumerate(hist[s]):
+                replay = pair.gpu.forward(slots, p, pair.emb[t])
+            if last[s] is not None:
+                assert np.array_equal(bits(last[s]), bits(replay)), ("last logits", s, len(hist[s]))
+                checked += 1
+            nxt = 7
+            a = pair.gpu.forward(s, len(hist[s]), pair.emb[nxt])
+            b = pair.gpu.forward(slots, len(hist[s]), pair.emb[nxt])
+            assert np.array_equal(bits(a), bits(b)), ("next token", s, len(hist[s]))
+        assert checked >= 1
+    finally:
+        pair.close()
