@@ -25,21 +25,22 @@ def bits(x):
     return np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
 
 
-def walk(pair, vocab, slots, cap, seed, n_ops, max_batch, kv_dim=None):
-    """Returns (history per slot, last logits per slot). Slot `slots` (one past the last) is left for the replay."""
+def walk(pair, emb, vocab, slots, cap, seed, n_ops, max_batch, chains=False):
+    """emb: the embedding rows by token id. Returns (history per slot, last logits per slot). Slot `slots` (one past the last) is
+    left for the replay. chains: the device-side greedy chain is one of the moves (emb must then be the resident table's rows)."""
     rng = np.random.default_rng(seed)
     hist = [[] for _ in range(slots)]  # what each slot holds: a list of ("tok", id) or ("kv", layer arrays)
     last = [None] * slots
     g = pair.gpu
     for _ in range(n_ops):
-        op = rng.choice(["batch", "batch", "ragged", "prefill", "truncate", "reset", "nologits"])
+        op = rng.choice(["batch", "batch", "ragged", "prefill", "truncate", "reset", "nologits"] + (["chain"] if chains else []))
         if op == "batch":
             k = int(rng.integers(1, min(slots, max_batch) + 1))
             chosen = [int(s) for s in rng.permutation(slots)[:k] if len(hist[s]) < cap - 1]
             if not chosen:
                 continue
             toks = rng.integers(0, vocab, len(chosen))
-            out, ids = g.step_batch(chosen, [len(hist[s]) for s in chosen], pair.emb[toks], capi.WANT_LOGITS | capi.WANT_ARGMAX)
+            out, ids = g.step_batch(chosen, [len(hist[s]) for s in chosen], emb[toks], capi.WANT_LOGITS | capi.WANT_ARGMAX)
             for i, s in enumerate(chosen):
                 hist[s].append(int(toks[i]))
                 last[s] = out[i].copy()
@@ -52,7 +53,7 @@ def walk(pair, vocab, slots, cap, seed, n_ops, max_batch, kv_dim=None):
             if not keep or sum(r for _, r in keep) > max_batch:
                 continue
             toks = [rng.integers(0, vocab, r) for _, r in keep]
-            out, _ = g.step_ragged([s for s, _ in keep], [len(hist[s]) for s, _ in keep], [pair.emb[t] for t in toks])
+            out, _ = g.step_ragged([s for s, _ in keep], [len(hist[s]) for s, _ in keep], [emb[t] for t in toks])
             off = 0
             for (s, r), t in zip(keep, toks):
                 hist[s].extend(int(x) for x in t)
@@ -64,16 +65,27 @@ def walk(pair, vocab, slots, cap, seed, n_ops, max_batch, kv_dim=None):
             if len(hist[s]) + n >= cap:
                 continue
             toks = rng.integers(0, vocab, n)
-            last[s] = g.prefill_last(s, len(hist[s]), pair.emb[toks]).copy()
+            last[s] = g.prefill_last(s, len(hist[s]), emb[toks]).copy()
             hist[s].extend(int(x) for x in toks)
         elif op == "nologits":
             s = int(rng.integers(0, slots))
             if len(hist[s]) >= cap - 1:
                 continue
             t = int(rng.integers(0, vocab))
-            g.forward_no_logits(s, len(hist[s]), pair.emb[t])
+            g.forward_no_logits(s, len(hist[s]), emb[t])
             hist[s].append(t)
             last[s] = None  # this call returns nothing to compare; the tokens after it will
+        elif op == "chain":
+            s = int(rng.integers(0, slots))
+            n = int(rng.integers(1, 9))
+            if len(hist[s]) + n >= cap - 1:
+                continue
+            t = int(rng.integers(0, vocab))
+            g.greedy_chain_start(s, t, len(hist[s]))
+            ids = [g.greedy_chain_next() for _ in range(n)]
+            g.chain_stop()
+            hist[s].extend([t] + ids[:-1])  # the chain fed its first token and every pick but the last
+            last[s] = None
         elif op == "truncate":
             s = int(rng.integers(0, slots))
             if len(hist[s]) < 2:
@@ -91,13 +103,20 @@ def walk(pair, vocab, slots, cap, seed, n_ops, max_batch, kv_dim=None):
 
 
 @pytest.mark.parametrize("seed", [82, 83, 84])
-@pytest.mark.parametrize("kind,kv", [("dense", "f16"), ("dense", "i8"), ("moe", "f16")])
+@pytest.mark.parametrize("kind,kv", [("dense", "f16"), ("dense", "i8"), ("moe", "f16"), ("dense-chains", "f16")])
 def test_random_walk_replays_bit_identically(dev, kind, kv, seed):
-    cfg = dense_cfg(n_layers=2) if kind == "dense" else moe_cfg(n_layers=2)
+    cfg = moe_cfg(n_layers=2) if kind == "moe" else dense_cfg(n_layers=2)
     slots, cap = 5, 160
     pair = Pair(cfg, seed=81, dev=dev, slots=slots + 1, ctx_cap=cap, kv=kv)
     try:
-        hist, last = walk(pair, cfg["vocab"], slots, cap, seed=seed, n_ops=300, max_batch=32 if kind == "moe" else 128)
+        emb = pair.emb
+        if kind == "dense-chains":  # the chain looks its tokens up in the resident int8 table: every move uses that table's rows
+            from goinfer_amd import synth
+            q, sc = synth.w8a8_normal(85, cfg["vocab"], cfg["hidden"], 0.02)
+            pair.gpu.upload_embedding(q, sc)
+            emb = q.astype(np.float32) * sc[:, None]
+        hist, last = walk(pair, emb, cfg["vocab"], slots, cap, seed=seed, n_ops=300, max_batch=32 if kind == "moe" else 128,
+                          chains=kind == "dense-chains")
         checked = 0
         for s in range(slots):
             if not hist[s]:
@@ -106,13 +125,13 @@ def test_random_walk_replays_bit_identically(dev, kind, kv, seed):
             pair.gpu.kv_reset(slots)
             replay = None
             for p, t in enumerate(hist[s]):
-                replay = pair.gpu.forward(slots, p, pair.emb[t])
+                replay = pair.gpu.forward(slots, p, emb[t])
             if last[s] is not None:
                 assert np.array_equal(bits(last[s]), bits(replay)), ("last logits", s, len(hist[s]))
                 checked += 1
             nxt = 7
-            a = pair.gpu.forward(s, len(hist[s]), pair.emb[nxt])
-            b = pair.gpu.forward(slots, len(hist[s]), pair.emb[nxt])
+            a = pair.gpu.forward(s, len(hist[s]), emb[nxt])
+            b = pair.gpu.forward(slots, len(hist[s]), emb[nxt])
             assert np.array_equal(bits(a), bits(b)), ("next token", s, len(hist[s]))
         assert checked >= 1
     finally:
