@@ -21,7 +21,7 @@ EXPORTS = [
     "rd_kv_configure", "rd_kv_upload", "rd_kv_truncate", "rd_kv_reset", "rd_step_batch", "rd_forward",
     "rd_last_moe_indices", "rd_model_upload_embedding", "rd_bench_steps", "rd_bench_profile", "rd_bench_class_count",
     "rd_bench_class_name", "rd_bench_kernel", "rd_gateup_q4k_quant", "rd_moe_replay", "rd_bench_attn", "rd_step_ragged", "rd_prefill_last",
-    "rd_kv_configure_typed", "rd_attn_ragged_i8", "rd_attn_ragged_rows", "rd_plan_attention", "rd_plan_gemm", "rd_bench_attn_i8", "rd_step_ragged_draw", "rd_forward_no_logits",
+    "rd_kv_configure_typed", "rd_attn_ragged_i8", "rd_attn_ragged_rows", "rd_plan_attention", "rd_plan_gemm", "rd_step_batch_topk", "rd_last_logits", "rd_topk_rows", "rd_bench_attn_i8", "rd_step_ragged_draw", "rd_forward_no_logits",
     "rd_step_batch_draw", "rd_sample_rows", "rd_greedy_chain_start", "rd_greedy_chain_next", "rd_sample_chain_start",
     "rd_sample_chain_next", "rd_greedy_chain_stop",
     "rd_dequant_q5k", "rd_dequant_q6k", "rd_gemm_q5k", "rd_gemm_q6k", "rd_model_upload_q5k", "rd_model_upload_q6k",
@@ -207,6 +207,17 @@ class Device:
         dst = np.empty((a.shape[0], N), np.float32)
         check(lib().rd_gemm_w4a8(self.h, _p(nib), _p(s16), N, K, _p(a), a.shape[0], _p(dst)), "rd_gemm_w4a8")
         return dst
+
+    def topk_rows(self, logits, k, temperature=1.0, want_z=True):
+        """Each row's k best entries in (logit descending, id ascending) order: (ids [rows][k'], vals [rows][k'], z [rows] or None)."""
+        logits = _f32(logits)
+        rows, V = logits.shape
+        kk = min(k, V)
+        ids = np.empty((rows, kk), np.int32)
+        vals = np.empty((rows, kk), np.float32)
+        z = np.empty(rows, np.float64) if want_z else None
+        check(lib().rd_topk_rows(self.h, _p(logits), rows, V, k, C.c_double(temperature), int(want_z), _p(ids), _p(vals), _p(z)), "rd_topk_rows")
+        return ids, vals, z
 
     def attn_ragged(self, lens, k, v, q, n_h, n_kv, hd, scale, softcap=0.0, kv="f16"):
         """kv: "f16" (the binary16 cache) or "i8" (the int8 cache with one scale per position and kv head)."""
@@ -396,6 +407,26 @@ class Model:
         check(lib().rd_step_ragged_draw(self.h, len(slots), _p(slots), _p(pos), _p(n_rows), _p(emb), make_draws(draws), want, _p(logits), _p(ids)),
               "rd_step_ragged_draw")
         return logits, ids
+
+    def step_batch_topk(self, slots, pos, emb, k, temperature=None):
+        """The step with each row's logits reduced to its k best entries: (ids [B][k'], vals [B][k'], z [B] or None)."""
+        emb = _f32(emb)
+        B = emb.shape[0]
+        slots = np.ascontiguousarray(slots, dtype=np.int32)
+        pos = np.ascontiguousarray(pos, dtype=np.int32)
+        kk = min(k, self.cfg["vocab"])
+        ids = np.empty((B, kk), np.int32)
+        vals = np.empty((B, kk), np.float32)
+        t = None if temperature is None else np.ascontiguousarray(np.broadcast_to(temperature, (B,)), dtype=np.float64)
+        z = None if t is None else np.empty(B, np.float64)
+        check(lib().rd_step_batch_topk(self.h, B, _p(slots), _p(pos), _p(emb), k, _p(t), int(t is not None), _p(ids), _p(vals), _p(z)),
+              "rd_step_batch_topk")
+        return ids, vals, z
+
+    def last_logits(self, row):
+        out = np.empty(self.cfg["vocab"], np.float32)
+        check(lib().rd_last_logits(self.h, row, _p(out)), "rd_last_logits")
+        return out
 
     def forward_no_logits(self, slot, pos, emb):
         emb = _f32(emb)

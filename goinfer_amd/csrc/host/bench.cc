@@ -226,6 +226,26 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
             if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup) + 1], d->stream);
         }
         if (!rc) rc = d->sync();
+    } else if (nm == "topk" && n_args >= 3) {
+        // args {rows, V, k}: the top-K reduction (with Z) of `rows` logits rows of uniform values
+        int rows = (int)args[0], V = (int)args[1], k = (int)args[2];
+        if (rows < 1 || rows > 4096 || V < 1 || k < 1 || k > TOPK_MAX || k > V) {
+            rd_set_error("topk bench: bad shape");
+            rc = RD_ERR_ARG;
+        }
+        DevBuf L(d), I(d), Vv(d), Z(d);
+        if (!rc) rc = L.alloc(sizeof(float) * (size_t)rows * V);
+        if (!rc) rc = I.alloc(sizeof(int) * (size_t)rows * k);
+        if (!rc) rc = Vv.alloc(sizeof(float) * (size_t)rows * k);
+        if (!rc) rc = Z.alloc(sizeof(double) * (size_t)rows);
+        if (!rc) rc = d->launch(d->k.fill_f32, 1024, 1, 1, 256, L.as<float>(), (size_t)rows * V, 31u);
+        for (int i = 0; i < warmup + iters && !rc; i++) {
+            if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup)], d->stream);
+            rc = d->launch(d->k.topk_rows, (unsigned)rows, 1, 1, 1024u, (const float *)L.p, V, k, 1.f, (const float *)nullptr, I.as<int>(), Vv.as<float>(),
+                           Z.as<double>());
+            if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup) + 1], d->stream);
+        }
+        if (!rc) rc = d->sync();
     } else if (nm == "moe_gemm" && n_args >= 7) {
         // args {N, K, nE, active, T, per_expert_panels, copies[, first[, bitmap]]}: the grouped expert GEMM over nE experts of which `active`
         // have a token (spread evenly, or the first `active` ones when `first` is set: then every block with work precedes every

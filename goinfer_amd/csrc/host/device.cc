@@ -107,6 +107,7 @@ static const KName kNames[] = {
     {"rd_k_argmax_final", &Kernels::argmax_final},
     {"rd_k_matmul_f32", &Kernels::matmul_f32},
     {"rd_k_moe_route", &Kernels::moe_route},
+    {"rd_k_topk_rows", &Kernels::topk_rows},
     {"rd_k_gemm_w4a8_moe", &Kernels::gemm_w4a8_moe},
     {"rd_k_gemm_w4a8_moe_gateup", &Kernels::gemm_w4a8_moe_gateup},
     {"rd_k_moe_swiglu_quant", &Kernels::moe_swiglu_quant},

@@ -28,7 +28,7 @@ struct Kernels {
     hipFunction_t dequant_q5k, retile_q5k, gemm_q5k, dequant_q6k, retile_q6k, gemm_q6k;
     hipFunction_t gemm_q4k_gateup;
     hipFunction_t kv_store, qkv_rope_store, attn_partial, attn_combine, attn_combine_quant;
-    hipFunction_t kv_store_i8, qkv_rope_store_i8, attn_partial_i8, attn_partial_rows, attn_partial_rows_i8, attn_partial_deep, attn_partial_deep_i8;
+    hipFunction_t kv_store_i8, qkv_rope_store_i8, attn_partial_i8, attn_partial_rows, attn_partial_rows_i8, attn_partial_deep, attn_partial_deep_i8, topk_rows;
     hipFunction_t rmsnorm, rope, argmax_rows, argmax_final, matmul_f32, moe_route, gemm_w4a8_moe, gemm_w4a8_moe_gateup, moe_swiglu_quant, moe_fold, embed_rows, copy16, barrier_probe, unpanel_q4k, fill_f16, fill_f32;
 };
 
@@ -90,6 +90,7 @@ constexpr int ATTN_RANGE_INTS = 3; // per (row, kv head): first item, one past t
 // per wave: with so few waves nothing else hides a wave's memory latency. Same results bit for bit.
 constexpr int ATTN_DEEP_MAX_ITEMS = 1024;
 hipFunction_t attn_partial_kernel(const struct rd_device *d, bool i8, bool grouped, size_t n_items);
+constexpr int TOPK_MAX = 1024; // = RD_TOPK_MAX of the top-K kernel
 constexpr int ATTN_TILE_ROWS = 16; // head rows of the attention MFMA tile: an item holds at most 16 / (heads per kv head) positions
 // The attention work list of a step: items of the longest sequences first (the grid is dispatched in index order, so the
 // short items fill the tail), and ranges[3*(row*n_kv+kvh)..] as above.

@@ -65,7 +65,7 @@ extern "C" void rd_model_destroy(rd_model *m) {
     free_weight(d, &m->head);
     for (void *p : {(void *)m->embed_q, (void *)m->embed_scale, (void *)m->inv_freq_dev, (void *)m->final_norm, (void *)m->tables, (void *)m->h, (void *)m->normed, (void *)m->P, (void *)m->qbuf,
                     (void *)m->part, (void *)m->cand_v, (void *)m->cand_i, (void *)m->logits, (void *)m->emb_dev, m->XpA, m->XpA2, m->XpB, (void *)m->ids, (void *)m->meta, (void *)m->router_logits, (void *)m->moe_wgt, (void *)m->moe_gu,
-                    (void *)m->moe_dn, (void *)m->moe_out, (void *)m->moe_idx, (void *)m->moe_idx_all, (void *)m->moe_rank, (void *)m->moe_bits, m->XpE})
+                    (void *)m->moe_dn, (void *)m->moe_out, (void *)m->moe_idx, (void *)m->moe_idx_all, (void *)m->moe_rank, (void *)m->moe_bits, (void *)m->topk_ids, (void *)m->topk_vals, (void *)m->topk_invT, (void *)m->topk_z, m->XpE})
         d->release(p);
     if (m->host_stage) (void)d->hip->HostFree(m->host_stage);
     if (m->chain.host_ids) (void)d->hip->HostFree(m->chain.host_ids);
@@ -398,6 +398,10 @@ extern "C" int rd_model_finalize(rd_model *m) {
         RC(d->alloc(&m->XpE, (size_t)c.n_experts * (I / 128) * LIN_PANEL_BYTES));
         HIPCHK(MemsetAsync(m->XpE, 0, (size_t)c.n_experts * (I / 128) * LIN_PANEL_BYTES, d->stream));
     }
+    RC(d->alloc((void **)&m->topk_ids, sizeof(int) * R * TOPK_MAX));
+    RC(alloc_f32(d, &m->topk_vals, R * TOPK_MAX));
+    RC(alloc_f32(d, &m->topk_invT, R));
+    RC(d->alloc((void **)&m->topk_z, sizeof(double) * R));
     for (auto &e : m->stage_ev) HIPCHK(EventCreate(&e));
     m->finalized = true;
     return d->sync();
@@ -840,6 +844,7 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
     // contribution stays unadded, since nothing reads the hidden state after it.
     for (int b = 0; b < B; b++) m->slot_len[(size_t)slot[b]] = std::max(m->slot_len[(size_t)slot[b]], pos[b] + 1);
     m->last_B = B;
+    m->last_logits_valid = (want & RD_WANT_LOGITS) != 0;
     const bool replayed = m->replay_B != 0;
     m->replay_B = 0; // a routing override lasts one step
     if (replayed) RC(d->sync()); // its host arrays were uploaded from pageable memory: let the copies finish before they can change
@@ -1141,6 +1146,46 @@ extern "C" int rd_prefill_last(rd_model *m, int slot, int start_pos, int n, cons
 extern "C" int rd_forward(rd_model *m, int slot, int pos, const float *emb, float *logits) {
     if (!m || !emb || !logits) return RD_ERR_ARG;
     return model_step(m, 1, &slot, &pos, emb, nullptr, RD_WANT_LOGITS, logits, nullptr, false);
+}
+
+// resident.TopKRow (decoder/resident/forward.go:86-96; ForwardTopK, backend/cuda/topk.go:30-67): the step's kernel chain, then
+// each row's logits reduced on the device to its k best entries; k*8 bytes (+8 for Z) per row come back instead of vocab*4.
+extern "C" int rd_step_batch_topk(rd_model *m, int B, const int *slot, const int *pos, const float *emb, int k, const double *temperature,
+                                  int want_z, int *ids, float *vals, double *z) {
+    if (!m || !slot || !pos || !emb || !ids || !vals || (want_z && (!z || !temperature))) return RD_ERR_ARG;
+    if (k < 1 || k > TOPK_MAX) {
+        rd_set_error("rd_step_batch_topk: k=%d outside [1,%d]", k, TOPK_MAX);
+        return RD_ERR_ARG;
+    }
+    rd_device *d = m->d;
+    const int V = m->desc.vocab;
+    if (k > V) k = V;
+    RC(model_step(m, B, slot, pos, emb, nullptr, RD_WANT_LOGITS, nullptr, nullptr, false)); // the logits stay on the device
+    if (want_z) {
+        float invT[rd_model::ROWS_MAX];
+        for (int b = 0; b < B; b++) invT[b] = temperature[b] > 0 ? (float)(1.0 / temperature[b]) : 1.f; // backend/cuda/topk.go:74-77
+        RC(d->h2d(m->topk_invT, invT, sizeof(float) * (size_t)B));
+    }
+    RC(d->launch(d->k.topk_rows, (unsigned)B, 1, 1, 1024u, (const float *)m->logits, V, k, 1.f, (const float *)(want_z ? m->topk_invT : nullptr),
+                 m->topk_ids, m->topk_vals, want_z ? m->topk_z : (double *)nullptr));
+    RC(d->d2h(ids, m->topk_ids, sizeof(int) * (size_t)B * k));
+    RC(d->d2h(vals, m->topk_vals, sizeof(float) * (size_t)B * k));
+    if (want_z) RC(d->d2h(z, m->topk_z, sizeof(double) * (size_t)B));
+    return RD_OK;
+}
+
+// TopKRow.Full: the whole logits row of the last step's row `row`, for the token where k entries were not enough. Valid until
+// the next step.
+extern "C" int rd_last_logits(rd_model *m, int row, float *logits) {
+    if (!m || !logits || row < 0 || row >= m->last_B) {
+        if (m) rd_set_error("rd_last_logits: row %d of a step of %d", row, m->last_B);
+        return RD_ERR_ARG;
+    }
+    if (!m->last_logits_valid) {
+        rd_set_error("rd_last_logits: the last step kept no logits");
+        return RD_ERR_STATE;
+    }
+    return m->d->d2h(logits, m->logits + (size_t)row * m->desc.vocab, sizeof(float) * (size_t)m->desc.vocab);
 }
 
 extern "C" int rd_moe_replay(rd_model *m, int B, const int *idx, const float *wgt) {

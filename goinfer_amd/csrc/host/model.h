@@ -89,6 +89,10 @@ struct rd_model {
     float *router_logits = nullptr, *moe_wgt = nullptr, *moe_gu = nullptr, *moe_dn = nullptr, *moe_out = nullptr;
     int *moe_idx = nullptr, *moe_idx_all = nullptr; // [32][k], [layers][32][k]
     signed char *moe_rank = nullptr;                 // [32][nE]
+    bool last_logits_valid = false; // the last step wrote its rows' logits to `logits`
+    int *topk_ids = nullptr;      // [max_rows][TOPK_MAX], the top-K of the last step's logits rows
+    float *topk_vals = nullptr, *topk_invT = nullptr;
+    double *topk_z = nullptr;
     unsigned *moe_bits = nullptr;                    // bitmap of the experts the current layer's routing chose (8 words)
     void *XpE = nullptr;                             // per-expert down panels
     // pinned host staging

@@ -421,6 +421,32 @@ extern "C" int rd_attn_ragged_rows(rd_device *d, int kv_type, int n_seq, const i
     return attn_ragged_typed(d, kv_type, n_seq, len, nq, off, k, v, q, n_h, n_kv, hd, scale, softcap, out);
 }
 
+// ---- top-K of logits rows (kernel-level entry point) ----
+// 1/T as the sampler's device paths take it (backend/cuda/topk.go:74-77): f32(1/T), 1 for T <= 0
+static float topk_inv_t(double temperature) { return temperature > 0 ? (float)(1.0 / temperature) : 1.f; }
+
+extern "C" int rd_topk_rows(rd_device *d, const float *logits, int rows, int V, int k, double temperature, int want_z, int *ids, float *vals,
+                            double *z) {
+    if (!d || !logits || !ids || !vals || (want_z && !z) || rows <= 0 || V <= 0) return RD_ERR_ARG;
+    if (k < 1 || k > TOPK_MAX) {
+        rd_set_error("rd_topk_rows: k=%d outside [1,%d]", k, TOPK_MAX);
+        return RD_ERR_ARG;
+    }
+    if (k > V) k = V;
+    DevBuf L(d), I(d), Vv(d), Z(d);
+    RC(L.alloc(sizeof(float) * (size_t)rows * V));
+    RC(I.alloc(sizeof(int) * (size_t)rows * k));
+    RC(Vv.alloc(sizeof(float) * (size_t)rows * k));
+    RC(Z.alloc(sizeof(double) * (size_t)rows));
+    RC(d->h2d(L.p, logits, sizeof(float) * (size_t)rows * V));
+    RC(d->launch(d->k.topk_rows, (unsigned)rows, 1, 1, 1024u, (const float *)L.p, V, k, topk_inv_t(temperature), (const float *)nullptr, I.as<int>(),
+                 Vv.as<float>(), want_z ? Z.as<double>() : (double *)nullptr));
+    RC(d->d2h(ids, I.p, sizeof(int) * (size_t)rows * k));
+    RC(d->d2h(vals, Vv.p, sizeof(float) * (size_t)rows * k));
+    if (want_z) RC(d->d2h(z, Z.p, sizeof(double) * (size_t)rows));
+    return RD_OK;
+}
+
 // ---- host planning without a device ----
 extern "C" int rd_plan_attention(int rows, const int *len, const int *slot, int heads_per_kv, int n_kv, int *items_out, int max_items, int *ranges_out,
                                  int *n_items, int *grouped) {

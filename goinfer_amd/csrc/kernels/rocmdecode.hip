@@ -9,6 +9,7 @@
 #include "attn.h"
 #include "misc.h"
 #include "moe.h"
+#include "topk.h"
 
 // Attention combine fused with the per-32 quantization that feeds the o-projection. Grid (nH, rows), block
 // RD_ATTN_PIECES * HD/4; the first HD/4 threads (whole 8-lane quantization groups) finish the row.

@@ -171,6 +171,19 @@ int rd_step_batch_draw(rd_model *m, int B, const int *slot, const int *pos, cons
 /* The same draws over explicit logit rows (host f32 [rows][V]), the kernels on their own as the reference's
  * backend/cuda/kernels/gumbel_test.go binds them; RD_DRAW_NONE is taken as greedy. */
 int rd_sample_rows(rd_device *d, const float *logits, int rows, int V, const rd_draw *draws, int *ids);
+/* resident.TopKRow for every row of a step (decoder/resident/forward.go:86-96; ForwardTopK, backend/cuda/topk.go:30-67, is the
+ * B = 1 case): the step's kernel chain, then each logits row reduced on the device to its k best entries, ordered (logit
+ * descending, token id ascending) — the tie order of the host's topKByLogit (internal/runtime/sampling/sampler.go:726-745), -0
+ * and +0 equal. ids, vals: [B][min(k, vocab)]; 1 <= k <= 1024. want_z: z[b] = sum over the row of exp((l - max) / T_b) with
+ * temperature[b] = T_b (<= 0 taken as 1), exp in f32 summed in f64 (the reference's own device sum is held to 1e-6 of the f64
+ * sum, backend/cuda/topk_test.go:118); temperature and z may be NULL otherwise. */
+int rd_step_batch_topk(rd_model *m, int B, const int *slot, const int *pos, const float *emb, int k, const double *temperature, int want_z,
+                       int *ids, float *vals, double *z);
+/* TopKRow.Full: the whole logits row of row `row` of the last step, if that step produced logits; valid until the next step. */
+int rd_last_logits(rd_model *m, int row, float *logits);
+/* The same reduction over explicit logit rows (host f32 [rows][V]), the kernel on its own as the reference's
+ * backend/cuda/topk_test.go binds it; one temperature for all rows. */
+int rd_topk_rows(rd_device *d, const float *logits, int rows, int V, int k, double temperature, int want_z, int *ids, float *vals, double *z);
 /* Decode chained on the device (decoder/resident/subsystems.go:78-100 GreedyChainStart / GreedyChainNext / GreedyChainStop and
  * SampleChainStart / SampleChainNext): the chain's first input is token `id` at position `pos` of `slot`; each _next returns the
  * token the forward at the chain's next position picked (the argmax, or the Gumbel-max draw with draw index draw, draw+1, ...),

@@ -59,6 +59,7 @@ def lib():
         L.or_silu.argtypes = [C.c_float]
         L.or_quantize_row_int8.restype = C.c_float
         L.or_kprint_name.restype = C.c_char_p
+        L.or_softmax_z.restype = C.c_double
         L.or_cache_new.restype = C.c_void_p
         L.or_cache_new.argtypes = [C.POINTER(Model), C.c_int]
         L.or_cache_free.argtypes = [C.POINTER(Model), C.c_void_p]
@@ -208,6 +209,19 @@ def route_experts(logits, k, norm, scale=0.0):
     wts = np.empty(k, np.float32)
     n = lib().or_route_experts(_p(lg), lg.size, k, int(norm), C.c_double(scale), _p(idx), _p(wts))
     return idx[:n], wts[:n]
+
+
+def topk_by_logit(x, k):
+    x = f32(x)
+    ids = np.empty(min(k, x.size), np.int32)
+    vals = np.empty(min(k, x.size), np.float32)
+    n = lib().or_topk_by_logit(_p(x), x.size, k, _p(ids), _p(vals))
+    return ids[:n], vals[:n]
+
+
+def softmax_z(x, temperature):
+    x = f32(x)
+    return lib().or_softmax_z(_p(x), x.size, C.c_double(temperature))
 
 
 def argmax(x):

@@ -374,6 +374,59 @@ int or_argmax(const float *x, int n) {
     return bi;
 }
 
+/* ------------------------------------------------------------------ the K best logits of a row */
+/* internal/runtime/sampling/sampler.go:726-782 (topKByLogit): a k-bounded min-heap whose root is the worst kept entry, "worse" being
+ * the lower logit or, on a tie, the LARGER id; then the order its callers give the result, (logit descending, id ascending)
+ * (sampler_topk.go:10-15, decoder/resident/forward.go:86-90). ids, vals: min(k, n) entries. Returns that count. */
+static int topk_worse(const float *x, int a, int b) { return x[a] != x[b] ? x[a] < x[b] : a > b; }
+int or_topk_by_logit(const float *x, int n, int k, int *ids, float *vals) {
+    if (k > n) k = n;
+    if (k <= 0) return 0;
+    int *h = (int *)malloc(sizeof(int) * (size_t)k), len = 0;
+    for (int id = 0; id < n; id++) {
+        if (len < k) {
+            int i = len;
+            h[len++] = id;
+            while (i > 0) { /* siftUp: a child worse than its parent moves toward the root */
+                int p = (i - 1) / 2;
+                if (!topk_worse(x, h[i], h[p])) break;
+                int t = h[p];
+                h[p] = h[i], h[i] = t, i = p;
+            }
+        } else if (topk_worse(x, h[0], id)) { /* the candidate is better than the worst kept */
+            h[0] = id;
+            for (int i = 0;;) { /* siftDownRoot */
+                int l = 2 * i + 1, r = 2 * i + 2, m = i;
+                if (l < len && topk_worse(x, h[l], h[m])) m = l;
+                if (r < len && topk_worse(x, h[r], h[m])) m = r;
+                if (m == i) break;
+                int t = h[i];
+                h[i] = h[m], h[m] = t, i = m;
+            }
+        }
+    }
+    /* (logit desc, id asc): insertion sort, k <= 1024 */
+    for (int i = 1; i < len; i++) {
+        int v = h[i], j = i - 1;
+        while (j >= 0 && topk_worse(x, h[j], v)) h[j + 1] = h[j], j--;
+        h[j + 1] = v;
+    }
+    for (int i = 0; i < len; i++) ids[i] = h[i], vals[i] = x[h[i]];
+    free(h);
+    return len;
+}
+
+/* The top-p denominator as the host forms every probability (sampler.go:784-800 topPCandidates, sampler_chunked.go:136-141 chunkedZ):
+ * sum over the row of exp((f64(l) - max) / T), here in plain ascending order (the host's fixed chunking regroups the same f64
+ * terms; the difference is a few ulp of f64). */
+double or_softmax_z(const float *x, int n, double temperature) {
+    double mx = x[0], z = 0;
+    for (int i = 1; i < n; i++)
+        if (x[i] > mx) mx = x[i];
+    for (int i = 0; i < n; i++) z += exp(((double)x[i] - mx) / temperature);
+    return z;
+}
+
 /* ------------------------------------------------------------------ temperature-only sampling (Gumbel-max) */
 /* internal/runtime/sampling/philox.go:13-40 (Philox4x32): Philox4x32-10; the key is bumped between rounds, not before the first. */
 void or_philox4x32(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]) {

@@ -23,6 +23,10 @@
  *   or_rmsnorm, or_rope, or_swiglu, or_softmax_f32, or_topk, or_route_experts, or_argmax
  *                                        plain Go in the reference, restated statement by statement;
  *                                        pinned by closed forms + the HF goldens (llama-tiny, qwen3moe-tiny, mixtral-tiny)
+ *   or_topk_by_logit, or_softmax_z       pinned by what the definition fixes: the first K of the row sorted by (logit desc, id asc) is
+ *                                        unique, so the heap restatement is checked against an independent full sort (numpy
+ *                                        lexsort) on normal, heavily tied and signed-zero rows, K from 1 to the row (the shapes of
+ *                                        the reference's own topk_test.go); Z against numpy's f64 sum
  *   or_philox4x32                        pinned: the Random123 known-answer vectors the reference's philox_test.go holds
  *   or_gumbel_noise / _key / _draw       pinned by the closed form the reference's tests state (f64 -log(-log1p(-w)), range,
  *                                        monotone), by chi-square fit of the draw to softmax(l/T) under the reference's own
@@ -89,6 +93,8 @@ void or_softmax_f32(const float *x, int n, float *out);
 int or_topk(const float *x, int n, int k, int *idx, float *val);
 int or_route_experts(const float *logits, int nE, int k, int norm, double scale, int *idx, float *wts);
 int or_argmax(const float *x, int n); /* internal/runtime/sampling/sampler.go:485-520: first maximum wins */
+int or_topk_by_logit(const float *x, int n, int k, int *ids, float *vals); /* sampler.go:726-782 + the (logit desc, id asc) order of TopKRow */
+double or_softmax_z(const float *x, int n, double temperature);            /* the top-p denominator, f64 */
 
 /* ---- temperature-only sampling by Gumbel-max: internal/runtime/sampling/philox.go, sampler_gumbel.go ---- */
 void or_philox4x32(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]);
