@@ -227,7 +227,8 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
         }
         if (!rc) rc = d->sync();
     } else if (nm == "topk" && n_args >= 3) {
-        // args {rows, V, k}: the top-K reduction (with Z) of `rows` logits rows of uniform values
+        // args {rows, V, k[, bell]}: the top-K reduction (with Z) of `rows` logits rows of uniform values, or (bell) of sums of
+        // twelve uniforms, the shape of real logits: a thin upper tail
         int rows = (int)args[0], V = (int)args[1], k = (int)args[2];
         if (rows < 1 || rows > 4096 || V < 1 || k < 1 || k > TOPK_MAX || k > V) {
             rd_set_error("topk bench: bad shape");
@@ -238,14 +239,32 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
         if (!rc) rc = I.alloc(sizeof(int) * (size_t)rows * k);
         if (!rc) rc = Vv.alloc(sizeof(float) * (size_t)rows * k);
         if (!rc) rc = Z.alloc(sizeof(double) * (size_t)rows);
-        if (!rc) rc = d->launch(d->k.fill_f32, 1024, 1, 1, 256, L.as<float>(), (size_t)rows * V, 31u);
+        if (!rc && n_args >= 4 && args[3]) {
+            std::vector<float> h((size_t)rows * V);
+            uint64_t s = 0x9E3779B97F4A7C15ULL;
+            for (auto &x : h) {
+                float a = -6.f;
+                for (int j = 0; j < 12; j++) {
+                    s ^= s << 13, s ^= s >> 7, s ^= s << 17;
+                    a += (float)(s >> 40) * (1.0f / 16777216.0f);
+                }
+                x = 3.f * a;
+            }
+            rc = d->h2d(L.p, h.data(), sizeof(float) * h.size());
+            if (!rc) rc = d->sync();
+        } else if (!rc) {
+            rc = d->launch(d->k.fill_f32, 1024, 1, 1, 256, L.as<float>(), (size_t)rows * V, 31u);
+        }
+        TopkScratch sc;
+        if (!rc) rc = topk_scratch_alloc(d, rows, V, &sc);
         for (int i = 0; i < warmup + iters && !rc; i++) {
             if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup)], d->stream);
-            rc = d->launch(d->k.topk_rows, (unsigned)rows, 1, 1, 1024u, (const float *)L.p, V, k, 1.f, (const float *)nullptr, I.as<int>(), Vv.as<float>(),
-                           Z.as<double>());
+            rc = launch_topk(d, (const float *)L.p, rows, V, k, 1.f, false, sc, I.as<int>(), Vv.as<float>(), Z.as<double>());
             if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup) + 1], d->stream);
         }
         if (!rc) rc = d->sync();
+        for (void *p : {(void *)sc.ghist, (void *)sc.ccount, (void *)sc.gmax, (void *)sc.cand_i, (void *)sc.cand_v, (void *)sc.invT, (void *)sc.zpart})
+            if (p) d->release(p);
     } else if (nm == "moe_gemm" && n_args >= 7) {
         // args {N, K, nE, active, T, per_expert_panels, copies[, first[, bitmap]]}: the grouped expert GEMM over nE experts of which `active`
         // have a token (spread evenly, or the first `active` ones when `first` is set: then every block with work precedes every

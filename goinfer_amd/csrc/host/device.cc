@@ -108,6 +108,9 @@ static const KName kNames[] = {
     {"rd_k_matmul_f32", &Kernels::matmul_f32},
     {"rd_k_moe_route", &Kernels::moe_route},
     {"rd_k_topk_rows", &Kernels::topk_rows},
+    {"rd_k_topk_hist", &Kernels::topk_hist},
+    {"rd_k_topk_pick", &Kernels::topk_pick},
+    {"rd_k_topk_finish", &Kernels::topk_finish},
     {"rd_k_gemm_w4a8_moe", &Kernels::gemm_w4a8_moe},
     {"rd_k_gemm_w4a8_moe_gateup", &Kernels::gemm_w4a8_moe_gateup},
     {"rd_k_moe_swiglu_quant", &Kernels::moe_swiglu_quant},
@@ -190,6 +193,36 @@ extern "C" int rd_device_mem_info(rd_device *d, size_t *free_b, size_t *total_b)
     if (!d) return RD_ERR_ARG;
     HIPCHK(MemGetInfo(free_b, total_b));
     return RD_OK;
+}
+
+int topk_scratch_alloc(rd_device *d, int rows, int V, TopkScratch *s) {
+    const size_t R = (size_t)rows, chunks = (size_t)(V + TOPK_CHUNK - 1) / TOPK_CHUNK;
+    int rc = d->alloc((void **)&s->ghist, sizeof(int) * R * chunks * TOPK_BINS);
+    if (!rc) rc = d->alloc((void **)&s->ccount, sizeof(int) * R);
+    if (!rc) rc = d->alloc((void **)&s->gmax, sizeof(unsigned) * R * chunks);
+    if (!rc) rc = d->alloc((void **)&s->cand_i, sizeof(int) * R * TOPK_CAP);
+    if (!rc) rc = d->alloc((void **)&s->cand_v, sizeof(float) * R * TOPK_CAP);
+    if (!rc) rc = d->alloc((void **)&s->invT, sizeof(float) * R);
+    if (!rc) rc = d->alloc((void **)&s->zpart, sizeof(double) * R * chunks);
+    if (rc) return rc;
+    if (!rd_hip_ok(d->hip, d->hip->MemsetAsync(s->ccount, 0, sizeof(int) * R, d->stream), "memset")) return RD_ERR_HIP;
+    return RD_OK;
+}
+
+int launch_topk(rd_device *d, const float *logits, int rows, int V, int k, float invT, bool rowsInvT, const TopkScratch &s, int *ids, float *vals,
+                double *z) {
+    const float *it = rowsInvT ? s.invT : nullptr;
+    if (V < 2 * TOPK_CHUNK) // a narrow row: one block reads it a few times
+        return d->launch(d->k.topk_rows, (unsigned)rows, 1, 1, 1024u, logits, V, k, invT, it, ids, vals, z);
+    const unsigned chunks = (unsigned)((V + TOPK_CHUNK - 1) / TOPK_CHUNK);
+    int rc = d->launch(d->k.topk_hist, chunks, (unsigned)rows, 1, 1024u, logits, V, s.ghist, s.gmax);
+    if (!rc)
+        rc = d->launch(d->k.topk_pick, chunks, (unsigned)rows, 1, 1024u, logits, V, k, invT, it, (const int *)s.ghist, (const unsigned *)s.gmax, s.cand_v,
+                       s.cand_i, s.ccount, z ? s.zpart : (double *)nullptr);
+    if (!rc)
+        rc = d->launch(d->k.topk_finish, (unsigned)rows, 1, 1, 1024u, logits, V, k, (int)chunks, (const float *)s.cand_v,
+                       (const int *)s.cand_i, s.ccount, (const double *)s.zpart, ids, vals, z);
+    return rc;
 }
 
 hipFunction_t attn_partial_kernel(const rd_device *d, bool i8, bool grouped, size_t n_items) {

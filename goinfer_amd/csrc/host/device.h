@@ -28,7 +28,7 @@ struct Kernels {
     hipFunction_t dequant_q5k, retile_q5k, gemm_q5k, dequant_q6k, retile_q6k, gemm_q6k;
     hipFunction_t gemm_q4k_gateup;
     hipFunction_t kv_store, qkv_rope_store, attn_partial, attn_combine, attn_combine_quant;
-    hipFunction_t kv_store_i8, qkv_rope_store_i8, attn_partial_i8, attn_partial_rows, attn_partial_rows_i8, attn_partial_deep, attn_partial_deep_i8, topk_rows;
+    hipFunction_t kv_store_i8, qkv_rope_store_i8, attn_partial_i8, attn_partial_rows, attn_partial_rows_i8, attn_partial_deep, attn_partial_deep_i8, topk_rows, topk_hist, topk_pick, topk_finish;
     hipFunction_t rmsnorm, rope, argmax_rows, argmax_final, matmul_f32, moe_route, gemm_w4a8_moe, gemm_w4a8_moe_gateup, moe_swiglu_quant, moe_fold, embed_rows, copy16, barrier_probe, unpanel_q4k, fill_f16, fill_f32;
 };
 
@@ -90,7 +90,21 @@ constexpr int ATTN_RANGE_INTS = 3; // per (row, kv head): first item, one past t
 // per wave: with so few waves nothing else hides a wave's memory latency. Same results bit for bit.
 constexpr int ATTN_DEEP_MAX_ITEMS = 1024;
 hipFunction_t attn_partial_kernel(const struct rd_device *d, bool i8, bool grouped, size_t n_items);
-constexpr int TOPK_MAX = 1024; // = RD_TOPK_MAX of the top-K kernel
+constexpr int TOPK_MAX = 1024; // = RD_TOPK_MAX of the top-K kernels
+constexpr int TOPK_CAP = 4096, TOPK_BINS = 2048, TOPK_CHUNK = 16384; // = RD_TOPK_CAP, RD_TOPK_BINS, RD_TOPK_CHUNK
+// Scratch of the top-K over `rows` rows of width V (device memory the caller owns): per-chunk histograms and maxima, candidate
+// counts (zero between calls), candidate lists, per-chunk shares of Z, and 1/T per row.
+struct TopkScratch {
+    int *ghist = nullptr, *ccount = nullptr, *cand_i = nullptr;
+    unsigned *gmax = nullptr;
+    float *cand_v = nullptr, *invT = nullptr;
+    double *zpart = nullptr;
+};
+int topk_scratch_alloc(struct rd_device *d, int rows, int V, TopkScratch *s); // allocates and zeroes; the caller releases the seven buffers
+// Rows of logits (device, [rows][V]) to ids, vals ([rows][k]) and z ([rows], may be null) on the device. invT: scalar used when
+// rowsInvT is false, else s.invT holds one per row. Wide rows go over the chip in three launches, narrow ones take one block each.
+int launch_topk(struct rd_device *d, const float *logits, int rows, int V, int k, float invT, bool rowsInvT, const TopkScratch &s, int *ids,
+                float *vals, double *z);
 constexpr int ATTN_TILE_ROWS = 16; // head rows of the attention MFMA tile: an item holds at most 16 / (heads per kv head) positions
 // The attention work list of a step: items of the longest sequences first (the grid is dispatched in index order, so the
 // short items fill the tail), and ranges[3*(row*n_kv+kvh)..] as above.

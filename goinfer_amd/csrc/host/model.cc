@@ -65,7 +65,7 @@ extern "C" void rd_model_destroy(rd_model *m) {
     free_weight(d, &m->head);
     for (void *p : {(void *)m->embed_q, (void *)m->embed_scale, (void *)m->inv_freq_dev, (void *)m->final_norm, (void *)m->tables, (void *)m->h, (void *)m->normed, (void *)m->P, (void *)m->qbuf,
                     (void *)m->part, (void *)m->cand_v, (void *)m->cand_i, (void *)m->logits, (void *)m->emb_dev, m->XpA, m->XpA2, m->XpB, (void *)m->ids, (void *)m->meta, (void *)m->router_logits, (void *)m->moe_wgt, (void *)m->moe_gu,
-                    (void *)m->moe_dn, (void *)m->moe_out, (void *)m->moe_idx, (void *)m->moe_idx_all, (void *)m->moe_rank, (void *)m->moe_bits, (void *)m->topk_ids, (void *)m->topk_vals, (void *)m->topk_invT, (void *)m->topk_z, m->XpE})
+                    (void *)m->moe_dn, (void *)m->moe_out, (void *)m->moe_idx, (void *)m->moe_idx_all, (void *)m->moe_rank, (void *)m->moe_bits, (void *)m->topk_ids, (void *)m->topk_vals, (void *)m->topk_z, (void *)m->topk_scratch.ghist, (void *)m->topk_scratch.ccount, (void *)m->topk_scratch.gmax, (void *)m->topk_scratch.cand_i, (void *)m->topk_scratch.cand_v, (void *)m->topk_scratch.invT, (void *)m->topk_scratch.zpart, m->XpE})
         d->release(p);
     if (m->host_stage) (void)d->hip->HostFree(m->host_stage);
     if (m->chain.host_ids) (void)d->hip->HostFree(m->chain.host_ids);
@@ -400,7 +400,7 @@ extern "C" int rd_model_finalize(rd_model *m) {
     }
     RC(d->alloc((void **)&m->topk_ids, sizeof(int) * R * TOPK_MAX));
     RC(alloc_f32(d, &m->topk_vals, R * TOPK_MAX));
-    RC(alloc_f32(d, &m->topk_invT, R));
+    RC(topk_scratch_alloc(d, (int)R, c.vocab, &m->topk_scratch));
     RC(d->alloc((void **)&m->topk_z, sizeof(double) * R));
     for (auto &e : m->stage_ev) HIPCHK(EventCreate(&e));
     m->finalized = true;
@@ -1164,10 +1164,10 @@ extern "C" int rd_step_batch_topk(rd_model *m, int B, const int *slot, const int
     if (want_z) {
         float invT[rd_model::ROWS_MAX];
         for (int b = 0; b < B; b++) invT[b] = temperature[b] > 0 ? (float)(1.0 / temperature[b]) : 1.f; // backend/cuda/topk.go:74-77
-        RC(d->h2d(m->topk_invT, invT, sizeof(float) * (size_t)B));
+        RC(d->h2d(m->topk_scratch.invT, invT, sizeof(float) * (size_t)B));
     }
-    RC(d->launch(d->k.topk_rows, (unsigned)B, 1, 1, 1024u, (const float *)m->logits, V, k, 1.f, (const float *)(want_z ? m->topk_invT : nullptr),
-                 m->topk_ids, m->topk_vals, want_z ? m->topk_z : (double *)nullptr));
+    RC(launch_topk(d, (const float *)m->logits, B, V, k, 1.f, want_z != 0, m->topk_scratch, m->topk_ids, m->topk_vals,
+                   want_z ? m->topk_z : (double *)nullptr));
     RC(d->d2h(ids, m->topk_ids, sizeof(int) * (size_t)B * k));
     RC(d->d2h(vals, m->topk_vals, sizeof(float) * (size_t)B * k));
     if (want_z) RC(d->d2h(z, m->topk_z, sizeof(double) * (size_t)B));

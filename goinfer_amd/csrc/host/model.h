@@ -91,8 +91,9 @@ struct rd_model {
     signed char *moe_rank = nullptr;                 // [32][nE]
     bool last_logits_valid = false; // the last step wrote its rows' logits to `logits`
     int *topk_ids = nullptr;      // [max_rows][TOPK_MAX], the top-K of the last step's logits rows
-    float *topk_vals = nullptr, *topk_invT = nullptr;
+    float *topk_vals = nullptr;
     double *topk_z = nullptr;
+    TopkScratch topk_scratch;
     unsigned *moe_bits = nullptr;                    // bitmap of the experts the current layer's routing chose (8 words)
     void *XpE = nullptr;                             // per-expert down panels
     // pinned host staging

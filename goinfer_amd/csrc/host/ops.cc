@@ -439,8 +439,13 @@ extern "C" int rd_topk_rows(rd_device *d, const float *logits, int rows, int V, 
     RC(Vv.alloc(sizeof(float) * (size_t)rows * k));
     RC(Z.alloc(sizeof(double) * (size_t)rows));
     RC(d->h2d(L.p, logits, sizeof(float) * (size_t)rows * V));
-    RC(d->launch(d->k.topk_rows, (unsigned)rows, 1, 1, 1024u, (const float *)L.p, V, k, topk_inv_t(temperature), (const float *)nullptr, I.as<int>(),
-                 Vv.as<float>(), want_z ? Z.as<double>() : (double *)nullptr));
+    TopkScratch sc;
+    RC(topk_scratch_alloc(d, rows, V, &sc));
+    int rc = launch_topk(d, (const float *)L.p, rows, V, k, topk_inv_t(temperature), false, sc, I.as<int>(), Vv.as<float>(),
+                         want_z ? Z.as<double>() : (double *)nullptr);
+    if (!rc) rc = d->sync();
+    for (void *p : {(void *)sc.ghist, (void *)sc.ccount, (void *)sc.gmax, (void *)sc.cand_i, (void *)sc.cand_v, (void *)sc.invT, (void *)sc.zpart}) d->release(p);
+    RC(rc);
     RC(d->d2h(ids, I.p, sizeof(int) * (size_t)rows * k));
     RC(d->d2h(vals, Vv.p, sizeof(float) * (size_t)rows * k));
     if (want_z) RC(d->d2h(z, Z.p, sizeof(double) * (size_t)rows));
