@@ -10,7 +10,7 @@ HSACO_PATH = os.path.join(HERE, "lib", "rocmdecode_gfx950.hsaco")
 
 RD_OK, RD_DECLINED = 0, 1
 PROJ = dict(q=0, k=1, v=2, o=3, gate=4, up=5, down=6, head=7)
-VEC = dict(attn_norm=0, ffn_norm=1, q_norm=2, k_norm=3, final_norm=4, router=5)
+VEC = dict(attn_norm=0, ffn_norm=1, q_norm=2, k_norm=3, final_norm=4, router=5, qkv_bias=6)
 WANT_LOGITS, WANT_ARGMAX = 1, 2
 
 EXPORTS = [

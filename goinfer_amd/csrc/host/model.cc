@@ -58,7 +58,7 @@ extern "C" void rd_model_destroy(rd_model *m) {
     (void)d->sync();
     for (auto &l : m->layers) {
         free_weight(d, &l.qkv), free_weight(d, &l.o), free_weight(d, &l.gateup), free_weight(d, &l.down);
-        for (void *p : {(void *)l.attn_norm, (void *)l.ffn_norm, (void *)l.q_norm, (void *)l.k_norm, (void *)l.router, l.exp_gateup, l.exp_down,
+        for (void *p : {(void *)l.attn_norm, (void *)l.ffn_norm, (void *)l.q_norm, (void *)l.k_norm, (void *)l.qkv_bias, (void *)l.router, l.exp_gateup, l.exp_down,
                         (void *)l.Kp, (void *)l.Vp, (void *)l.Ksc, (void *)l.Vsc})
             d->release(p);
     }
@@ -301,6 +301,7 @@ extern "C" int rd_model_upload_f32(rd_model *m, int layer, int which, const floa
         case RD_VEC_FFN_NORM: slot = &l.ffn_norm, want = (size_t)c.hidden; break;
         case RD_VEC_Q_NORM: slot = &l.q_norm, want = (size_t)c.head_dim; break;
         case RD_VEC_K_NORM: slot = &l.k_norm, want = (size_t)c.head_dim; break;
+        case RD_VEC_QKV_BIAS: slot = &l.qkv_bias, want = (size_t)(c.n_heads + 2 * c.n_kv_heads) * c.head_dim; break;
         case RD_VEC_ROUTER: slot = &l.router, want = (size_t)c.n_experts * c.hidden; break;
         default: rd_set_error("unknown vector %d", which); return RD_ERR_ARG;
         }
@@ -761,11 +762,12 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
                 RC(d->launch(d->k.qkv_rope_store_i8, (unsigned)(nH + 2 * nKV), (unsigned)B, 1, (unsigned)(HD / 2), (const float *)m->P, plan.splits, m->qbuf,
                              (signed char *)l.Kp, (signed char *)l.Vp, l.Ksc, l.Vsc, (const int *)m->tables, m->blocks_per_slot, (const int *)m->rowSlot,
                              (const int *)m->rowPos, (const double *)m->inv_freq_dev, (const float *)l.q_norm, (const float *)l.k_norm, c.rms_eps, nH, nKV,
-                             HD, m->pStride));
+                             HD, m->pStride, (const float *)l.qkv_bias));
             else
                 RC(d->launch(d->k.qkv_rope_store, (unsigned)(nH + 2 * nKV), (unsigned)B, 1, (unsigned)(HD / 2), (const float *)m->P, plan.splits, m->qbuf,
                          l.Kp, l.Vp, (const int *)m->tables, m->blocks_per_slot, (const int *)m->rowSlot, (const int *)m->rowPos,
-                         (const double *)m->inv_freq_dev, (const float *)l.q_norm, (const float *)l.k_norm, c.rms_eps, nH, nKV, HD, m->pStride));
+                         (const double *)m->inv_freq_dev, (const float *)l.q_norm, (const float *)l.k_norm, c.rms_eps, nH, nKV, HD, m->pStride,
+                         (const float *)l.qkv_bias));
         }
         {
             Scope s(m, KC_ATTN_PARTIAL);

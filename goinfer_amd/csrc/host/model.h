@@ -20,6 +20,7 @@ struct LayerW {
     DevWeight qkv, o, gateup, down;
     PendingMat pend[RD_PROJ_COUNT];
     float *attn_norm = nullptr, *ffn_norm = nullptr, *q_norm = nullptr, *k_norm = nullptr;
+    float *qkv_bias = nullptr; // optional: q bias, k bias, v bias end to end
     // MoE
     float *router = nullptr;           // [nE][hidden] f32
     void *exp_gateup = nullptr;        // [nE] stacked tiled W4A8, each 2*expert_inter rows x hidden

@@ -91,7 +91,8 @@ extern "C" __global__ void rd_k_kv_store(const float *__restrict__ k, const floa
     kv_store_elem(Kp, Vp, HD, region, p, d, k[(size_t)i * nKV * HD + t], v[(size_t)i * nKV * HD + t]);
 }
 
-// After the q|k|v GEMM: reduce its split-K partials, optional per-head RMSNorm of q and k (Qwen3, decoder/program_cpu.go:351-364),
+// After the q|k|v GEMM: reduce its split-K partials, optional q|k|v bias (Qwen2; decoder/attention.go:12-34 addBias, applied right
+// after the projections, program_cpu_n.go:470-476), optional per-head RMSNorm of q and k (Qwen3, decoder/program_cpu.go:351-364),
 // NeoX RoPE with f64 angles (decoder/rope.go:28-64), q -> f32 buffer, k,v -> this position of the row's sequence in the pool.
 // Grid (nH + 2*nKV, rows), block HD/2 threads... one thread per rotation pair.  P: [splits][32][(nH+2nKV)*HD].
 template <bool I8>
@@ -100,7 +101,7 @@ __device__ __forceinline__ void qkv_rope_store_body(const float *__restrict__ P,
                                                const int *__restrict__ tables, int tabStride,
                                                const int *__restrict__ rowSlot, const int *__restrict__ rowPos, const double *__restrict__ invFreq,
                                                const float *__restrict__ qnorm, const float *__restrict__ knorm, float eps, int nH, int nKV, int HD,
-                                               size_t pStride) {
+                                               size_t pStride, const float *__restrict__ bias) {
     int head = blockIdx.x, m = blockIdx.y, t = threadIdx.x, half = HD / 2; // one wave: half <= 64
     int Ntot = (nH + 2 * nKV) * HD, pos = rowPos[m];
     // everything this thread will need from memory is requested up front: one latency instead of a chain of them
@@ -108,6 +109,8 @@ __device__ __forceinline__ void qkv_rope_store_body(const float *__restrict__ P,
     const double invf = invFreq[t];
     const float *src = P + (size_t)(m >> 5) * pStride + (size_t)(m & 31) * Ntot + (size_t)head * HD; // M-tile m/32, row m%32
     float x1 = src[t], x2 = src[t + half];
+    float b1 = 0.f, b2 = 0.f;
+    if (bias) b1 = bias[head * HD + t], b2 = bias[head * HD + t + half];
     for (int s0 = 1; s0 < splits; s0 += 8) { // ascending split order; eight splits' loads in flight together
         float a1[8], a2[8];
 #pragma unroll
@@ -117,6 +120,7 @@ __device__ __forceinline__ void qkv_rope_store_body(const float *__restrict__ P,
         for (int j = 0; j < 8; j++)
             if (s0 + j < splits) x1 = __fadd_rn(x1, a1[j]), x2 = __fadd_rn(x2, a2[j]);
     }
+    if (bias) x1 = __fadd_rn(x1, b1), x2 = __fadd_rn(x2, b2);
     const int blkPre = tables[(size_t)slotRow * tabStride + (pos >> 6)];
     bool isQ = head < nH, isK = !isQ && head < nH + nKV;
     const float *nw = isQ ? qnorm : (isK ? knorm : nullptr);
@@ -166,16 +170,16 @@ extern "C" __global__ void rd_k_qkv_rope_store(const float *__restrict__ P, int 
                                                uint16_t *__restrict__ Vp, const int *__restrict__ tables, int tabStride,
                                                const int *__restrict__ rowSlot, const int *__restrict__ rowPos, const double *__restrict__ invFreq,
                                                const float *__restrict__ qnorm, const float *__restrict__ knorm, float eps, int nH, int nKV, int HD,
-                                               size_t pStride) {
-    qkv_rope_store_body<false>(P, splits, q, Kp, Vp, nullptr, nullptr, tables, tabStride, rowSlot, rowPos, invFreq, qnorm, knorm, eps, nH, nKV, HD, pStride);
+                                               size_t pStride, const float *__restrict__ bias) {
+    qkv_rope_store_body<false>(P, splits, q, Kp, Vp, nullptr, nullptr, tables, tabStride, rowSlot, rowPos, invFreq, qnorm, knorm, eps, nH, nKV, HD, pStride, bias);
 }
 // The same into the int8 cache: the K or V head is quantized with its own scale after RoPE (backend/cuda/kv8_store.cu).
 extern "C" __global__ void rd_k_qkv_rope_store_i8(const float *__restrict__ P, int splits, float *__restrict__ q, signed char *__restrict__ Kp,
                                                   signed char *__restrict__ Vp, float *__restrict__ Ksc, float *__restrict__ Vsc,
                                                   const int *__restrict__ tables, int tabStride, const int *__restrict__ rowSlot,
                                                   const int *__restrict__ rowPos, const double *__restrict__ invFreq, const float *__restrict__ qnorm,
-                                                  const float *__restrict__ knorm, float eps, int nH, int nKV, int HD, size_t pStride) {
-    qkv_rope_store_body<true>(P, splits, q, Kp, Vp, Ksc, Vsc, tables, tabStride, rowSlot, rowPos, invFreq, qnorm, knorm, eps, nH, nKV, HD, pStride);
+                                                  const float *__restrict__ knorm, float eps, int nH, int nKV, int HD, size_t pStride, const float *__restrict__ bias) {
+    qkv_rope_store_body<true>(P, splits, q, Kp, Vp, Ksc, Vsc, tables, tabStride, rowSlot, rowPos, invFreq, qnorm, knorm, eps, nH, nKV, HD, pStride, bias);
 }
 
 typedef float float4v __attribute__((ext_vector_type(4)));

@@ -37,8 +37,9 @@ typedef struct rd_model rd_model;
 
 /* projection ids for the upload calls */
 enum { RD_PROJ_Q = 0, RD_PROJ_K, RD_PROJ_V, RD_PROJ_O, RD_PROJ_GATE, RD_PROJ_UP, RD_PROJ_DOWN, RD_PROJ_HEAD, RD_PROJ_COUNT };
-/* f32 vectors */
-enum { RD_VEC_ATTN_NORM = 0, RD_VEC_FFN_NORM, RD_VEC_Q_NORM, RD_VEC_K_NORM, RD_VEC_FINAL_NORM, RD_VEC_ROUTER };
+/* f32 vectors. RD_VEC_QKV_BIAS (optional): the q, k and v projection biases end to end, (n_heads + 2 n_kv_heads) * head_dim values,
+ * added right after the projections (Qwen2; decoder/attention.go:12-34 addBias, program_cpu_n.go:470-476). */
+enum { RD_VEC_ATTN_NORM = 0, RD_VEC_FFN_NORM, RD_VEC_Q_NORM, RD_VEC_K_NORM, RD_VEC_FINAL_NORM, RD_VEC_ROUTER, RD_VEC_QKV_BIAS };
 /* rd_step_batch `want` */
 enum { RD_WANT_LOGITS = 1, RD_WANT_ARGMAX = 2 };
 

@@ -19,6 +19,7 @@ class Mat(C.Structure):
 class Layer(C.Structure):
     _fields_ = [(n, Mat) for n in ("q", "k", "v", "o", "gate", "up", "down")] + [
         ("attn_norm", C.c_void_p), ("ffn_norm", C.c_void_p), ("q_norm", C.c_void_p), ("k_norm", C.c_void_p),
+        ("q_bias", C.c_void_p), ("k_bias", C.c_void_p), ("v_bias", C.c_void_p),
         ("router", Mat), ("exp_gate", C.POINTER(Mat)), ("exp_up", C.POINTER(Mat)), ("exp_down", C.POINTER(Mat))]
 
 
@@ -241,7 +242,7 @@ def attend(q, keys, vals, n_keys, nH, nKV, hd, scale, softcap=0.0, start=0):
 
 class OracleModel:
     """decodeMultiStep over numpy weights. layers: list of dicts with WMat entries q,k,v,o,(gate,up,down | router,
-    exp_gate[],exp_up[],exp_down[]) and f32 arrays attn_norm, ffn_norm, optional q_norm,k_norm."""
+    exp_gate[],exp_up[],exp_down[]) and f32 arrays attn_norm, ffn_norm, optional q_norm,k_norm and q_bias,k_bias,v_bias."""
 
     def __init__(self, cfg, layers, final_norm, head, inv_freq):
         self.cfg = cfg
@@ -254,7 +255,7 @@ class OracleModel:
             for n in ("q", "k", "v", "o"):
                 setattr(L, n, lw[n].c())
             self._keep.append(lw)
-            for n in ("attn_norm", "ffn_norm", "q_norm", "k_norm"):
+            for n in ("attn_norm", "ffn_norm", "q_norm", "k_norm", "q_bias", "k_bias", "v_bias"):
                 if lw.get(n) is not None:
                     arr = f32(lw[n])
                     self._keep.append(arr)

@@ -940,6 +940,11 @@ int or_decode_multi_step_traced(const or_model *m, int B, const float *emb, or_c
         for (int b = 0; b < B; b++) {
             float *qb = q + (size_t)b * qDim, *kb = k + (size_t)b * kvDim, *vb = v + (size_t)b * kvDim;
             or_cache *c = caches[b];
+            if (lw->q_bias) { /* program_cpu_n.go:470-476: addBias (attention.go:12-34) right after the projections */
+                for (int i = 0; i < qDim; i++) qb[i] += lw->q_bias[i];
+                for (int i = 0; i < kvDim; i++) kb[i] += lw->k_bias[i];
+                for (int i = 0; i < kvDim; i++) vb[i] += lw->v_bias[i];
+            }
             if (lw->q_norm) {
                 qk_norm(qb, nH, hd, lw->q_norm, m->eps);
                 qk_norm(kb, nKV, hd, lw->k_norm, m->eps);

@@ -129,6 +129,7 @@ typedef struct {
     or_mat q, k, v, o, gate, up, down; /* dense FFN when n_experts==0 */
     const float *attn_norm, *ffn_norm; /* [hidden] */
     const float *q_norm, *k_norm;      /* [hd] or NULL (Qwen3 QK-norm) */
+    const float *q_bias, *k_bias, *v_bias; /* [nH*hd], [nKV*hd], [nKV*hd] or NULL (Qwen2 projection biases) */
     or_mat router;                     /* [nE, hidden] */
     or_mat *exp_gate, *exp_up, *exp_down; /* [nE] each */
 } or_layer;

@@ -96,6 +96,11 @@ class Pair:
             lw["attn_norm"], lw["ffn_norm"] = vec(l, "attn_norm", H), vec(l, "ffn_norm", H)
             if cfg.get("qk_norm"):
                 lw["q_norm"], lw["k_norm"] = vec(l, "q_norm", hd), vec(l, "k_norm", hd)
+            if cfg.get("qkv_bias"):  # Qwen2: biases on the q, k and v projections, sent to the GPU as one vector
+                b = synth.normal(nxt(), qd + 2 * kvd, 0.5)
+                lw["q_bias"], lw["k_bias"], lw["v_bias"] = b[:qd].copy(), b[qd:qd + kvd].copy(), b[qd + kvd:].copy()
+                if self.gpu:
+                    self.gpu.upload_f32(l, "qkv_bias", b)
             if nE == 0:
                 lw["gate"], lw["up"], lw["down"] = mat(l, "gate", I, H), mat(l, "up", I, H), mat(l, "down", H, I)
             else:

@@ -114,6 +114,25 @@ def test_dense_int8_projections_when_k_not_256(dev):
     check(Pair(cfg, seed=3, dev=dev, slots=4), [list(rng.integers(0, 512, n)) for n in (9, 40)], steps=4)
 
 
+def test_qwen2_projection_biases(dev):
+    """q, k and v biases (Qwen2), added after the projections and before RoPE: hidden 384 also puts the projections on the int8 lane,
+    as the Qwen2-0.5B shape's 896 does."""
+    cfg = dense_cfg(n_layers=2, hidden=384, n_heads=6, n_kv=2, head_dim=64, inter=512, vocab=512, theta=1e6, eps=1e-6)
+    cfg["qkv_bias"] = 1
+    rng = np.random.default_rng(12)
+    check(Pair(cfg, seed=13, dev=dev, slots=4), [list(rng.integers(0, 512, n)) for n in (6, 70)], steps=4)
+    # and the biases are not ignored: the same model without them answers differently
+    with_b, without = Pair(cfg, seed=13, dev=dev, slots=2), Pair(dict(cfg, qkv_bias=0), seed=13, dev=dev, slots=2)
+    try:
+        e = with_b.emb[[5]]
+        a, _ = with_b.gpu.step_batch([0], [0], e)
+        b, _ = without.gpu.step_batch([0], [0], e)
+        assert np.abs(a - b).max() > 1e-3
+    finally:
+        with_b.close()
+        without.close()
+
+
 def test_softcap_model(dev):
     rng = np.random.default_rng(3)
     check(Pair(dense_cfg(softcap=50.0), seed=4, dev=dev, slots=4), [list(rng.integers(0, 512, n)) for n in (4, 70)], steps=3)
