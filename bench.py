@@ -94,9 +94,10 @@ def parse_args():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--kv", default="f16", choices=["f16", "i8"],
                     help="KV cache element (c4 and c3): f16 as the metric is quoted, or goinfer's int8 cache (KVQuant i8), a variant of the workload")
-    ap.add_argument("--workload", default="c4", choices=["c4", "c2", "c3", "c5", "kquant"],
+    ap.add_argument("--workload", default="c4", choices=["c4", "c2", "c3", "c5", "kquant", "topk"],
                     help="c4 (default): the Llama-3-8B-shape step the metric is quoted on; c2: Q4_K GEMM microbench; c3: ragged "
-                         "attention microbench; c5: Qwen3-MoE-shape step; kquant: Q4_K / Q5_K / Q6_K GEMMs at the FFN and head shapes")
+                         "attention microbench; c5: Qwen3-MoE-shape step; kquant: Q4_K / Q5_K / Q6_K GEMMs at the FFN and head shapes; topk: "
+                         "the device-side top-K of logits rows")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this backend is single-GPU (goinfer has no collective path); run with --gpus 1", file=sys.stderr)
@@ -204,4 +205,5 @@ if __name__ == "__main__":
     else:
         import bench_micro
         bench_micro.T0 = T0
-        {"c2": bench_micro.run_c2, "c3": bench_micro.run_c3, "c5": bench_micro.run_c5, "kquant": bench_micro.run_kquant}[_args.workload](_args)
+        {"c2": bench_micro.run_c2, "c3": bench_micro.run_c3, "c5": bench_micro.run_c5, "kquant": bench_micro.run_kquant,
+         "topk": bench_micro.run_topk}[_args.workload](_args)

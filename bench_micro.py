@@ -134,6 +134,47 @@ def run_kquant(args):
     emit(out)
 
 
+def run_topk(args):
+    """The device-side top-K of logits rows (goinfer's TopKRow): rows of bell-shaped values, as logits are, and of uniform ones,
+    whose crowded threshold bin sends them down the exact one-block route. A step is one reduction of all the rows, Z included."""
+    from goinfer_amd import capi
+    steps, warmup = (args.steps if args.steps != 128 else 50), (args.warmup if args.warmup != 8 else 10)
+    dev = capi.Device(0)
+    cases = []
+    for rows, V, k in ((1, 128256, 256), (32, 128256, 256), (32, 128256, 1024), (128, 128256, 256), (32, 151936, 256), (32, 262144, 1024)):
+        for bell in (1, 0):
+            ms = dev.bench_kernel("topk", [rows, V, k, bell], warmup, steps)
+            t = float(np.median(ms))
+            cases.append({"rows": rows, "V": V, "k": k, "values": "bell" if bell else "uniform", "us": round(t * 1e3, 1),
+                          "GBs": round(rows * V * 4 / t / 1e6, 1), "bytes": rows * V * 4})
+            log("%d rows x %d, k=%d, %s: %.1f us" % (rows, V, k, "bell" if bell else "uniform", t * 1e3))
+    head = next(c for c in cases if c["rows"] == 32 and c["V"] == 128256 and c["k"] == 256 and c["values"] == "bell")
+    out = base_line("device-side top-K of logits rows, achieved GB/s over one read of the rows (32 rows of 128256, K=256; all cases listed)",
+                    head["GBs"], "GB/s", steps, warmup, head["us"] / 1e3, "top-K of logits rows (TopKRow): ids, logits and Z",
+                    "synthetic: sums of twelve uniforms (bell) or uniform values", {"cases": cases})
+    out["roofline"] = {"bound": "hbm", "achieved": head["GBs"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(head["GBs"] / HBM_PEAK_GBS, 4),
+                       "traffic": None, "kernel": "rd_k_topk_hist + rd_k_topk_pick + rd_k_topk_finish", "avg_launch_ms": round(head["us"] / 1e3, 5),
+                       "algorithmic_bytes_per_launch": head["bytes"]}
+    cpu = None
+    if not args.no_cpu:
+        from oracle import binding as ob
+        rng = np.random.default_rng(1)
+        x = (rng.standard_normal((32, 128256)) * 3).astype(np.float32)
+        n, t = 0, 0.0
+        while t < 5.0 and n < 200:
+            t0 = time.time()
+            for r in range(32):
+                ob.topk_by_logit(x[r], 256)
+                ob.softmax_z(x[r], 0.7)
+            t += time.time() - t0
+            n += 1
+        cpu = {"value": round(32 * 128256 * 4 / (t / n) / 1e9, 2), "unit": "GB/s", "cores": 1, "kind": "port",
+               "sample": "oracle topKByLogit + Z over 32 rows of 128256, K=256, %d passes (%.1f s)" % (n, t)}
+    out["cpu_baseline"] = cpu
+    dev.close()
+    emit(out)
+
+
 # ------------------------------------------------------------------------------------------------------------ C3
 def run_c3(args):
     """Ragged flash-decode attention: 64 sequences, KV lengths U[128,8192], 32 Q / 8 KV heads, head_dim 128, f16 KV; once without
