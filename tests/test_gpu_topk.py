@@ -43,6 +43,25 @@ def test_topk_rows_match_the_reference_order(dev, V):
     assert np.array_equal(again[0], first[0]) and np.array_equal(again[2].view(np.uint64), first[2].view(np.uint64))
 
 
+@pytest.mark.parametrize("V", [3000, 70000])
+def test_topk_rows_with_masked_entries(dev, V):
+    """Rows a logit processor has masked: most entries -Inf (never in the top while finite ones remain, tied among themselves by
+    id when K reaches into them) and Z counts them as zero."""
+    rng = np.random.default_rng(V)
+    x = np.full((2, V), -np.inf, np.float32)
+    keep = rng.choice(V, 300, replace=False)
+    x[0, keep] = rng.standard_normal(300).astype(np.float32) * 2
+    x[1, keep[:5]] = np.float32(1.25)  # five equal finite entries, the rest masked
+    for k in (1, 5, 200, 512):
+        ids, vals, z = dev.topk_rows(x, k, 0.9)
+        for r in range(2):
+            wi, wv = ob.topk_by_logit(x[r], k)
+            assert np.array_equal(ids[r], wi), (V, k, r)
+            assert np.array_equal(vals[r].view(np.uint32), wv.view(np.uint32))
+            zw = ob.softmax_z(x[r], 0.9)
+            assert abs(z[r] - zw) <= 1e-6 * zw
+
+
 def test_topk_rows_arguments(dev):
     x = np.zeros((1, 100), np.float32)
     with pytest.raises(capi.RocmError):
