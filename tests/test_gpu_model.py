@@ -301,11 +301,11 @@ def test_wide_batch_rows_equal_solo_rows_deep_k(dev):
         pair.close()
 
 
-def test_wide_batch_rows_equal_solo_rows(dev):
+@pytest.mark.parametrize("B", [70, 128])
+def test_wide_batch_rows_equal_solo_rows(dev, B):
     """A dense model steps up to 128 rows at once (four GEMM row tiles): every row is still the row its own one-row step computes,
     bit for bit, whatever tile it rides in; a batch past the range is refused."""
     cfg = dense_cfg(n_layers=2)
-    B = 70
     pair = Pair(cfg, seed=61, dev=dev, slots=2 * B, ctx_cap=32)
     try:
         rng = np.random.default_rng(6)
@@ -314,7 +314,7 @@ def test_wide_batch_rows_equal_solo_rows(dev):
             toks = rng.integers(0, cfg["vocab"], B)
             emb = pair.emb[toks]
             got, ids = pair.gpu.step_batch(list(range(B)), pos, emb, capi.WANT_LOGITS | capi.WANT_ARGMAX)
-            for b in (0, 31, 32, 33, 63, 64, 69):
+            for b in (0, 31, 32, 33, 63, 64, 69, B - 1):
                 solo = pair.gpu.forward(B + b, pos[b], emb[b])
                 assert np.array_equal(solo.view(np.uint32), got[b].view(np.uint32)), (step, b)
                 assert ids[b] == int(np.argmax(got[b]))
