@@ -24,7 +24,9 @@ bool rd_hip_ok(const HipApi *hip, hipError_t e, const char *what) {
 extern "C" const char *rd_last_error(void) { return g_err; }
 extern "C" const char *rd_backend_name(void) { return "rocm"; }
 
+int rd_device::use() { return rd_hip_ok(hip, hip->SetDevice(ordinal), "hipSetDevice") ? RD_OK : RD_ERR_HIP; }
 int rd_device::alloc(void **p, size_t n) {
+    if (use()) return RD_ERR_HIP;
     if (!rd_hip_ok(hip, hip->Malloc(p, n), "hipMalloc")) return RD_ERR_HIP;
     return RD_OK;
 }
@@ -32,6 +34,7 @@ void rd_device::release(void *p) {
     if (p) (void)hip->Free(p);
 }
 int rd_device::h2d(void *dst, const void *src, size_t n) {
+    if (use()) return RD_ERR_HIP;
     return rd_hip_ok(hip, hip->MemcpyAsync(dst, src, n, hipMemcpyHostToDevice, stream), "hipMemcpy H2D") ? RD_OK : RD_ERR_HIP;
 }
 int rd_device::d2h(void *dst, const void *src, size_t n) {
@@ -180,6 +183,7 @@ extern "C" int rd_device_open(int ordinal, rd_device **out) {
 
 extern "C" void rd_device_close(rd_device *d) {
     if (!d) return;
+    (void)d->use();
     (void)d->hip->StreamSynchronize(d->stream);
     for (void *p : d->owned) (void)d->hip->Free(p);
     (void)d->hip->ModuleUnload(d->module);

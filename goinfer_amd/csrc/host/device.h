@@ -45,6 +45,9 @@ struct rd_device {
         hipError_t e = hip->ModuleLaunchKernel(f, gx, gy, gz, bx, 1, 1, 0, stream, args, nullptr);
         return rd_hip_ok(hip, e, "hipModuleLaunchKernel") ? RD_OK : RD_ERR_HIP;
     }
+    // HIP's current device belongs to the calling thread, and a caller's threads come and go (a Go program's goroutines move
+    // between OS threads): every call that allocates, copies or starts a step makes this device current first.
+    int use();
     int alloc(void **p, size_t n);
     void release(void *p);
     int h2d(void *dst, const void *src, size_t n);

@@ -422,6 +422,7 @@ extern "C" int rd_kv_configure_typed(rd_model *m, int slots, int ctx_cap, int kv
         return RD_ERR_STATE;
     }
     rd_device *d = m->d;
+    RC(d->use());
     const rd_model_desc &c = m->desc;
     m->slots = slots, m->ctx_cap = ctx_cap, m->blocks_per_slot = (ctx_cap + 63) / 64;
     size_t nBlocks = (size_t)slots * m->blocks_per_slot + 1; // block 0 is the all-zero block no slot owns
@@ -663,6 +664,7 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
         rd_set_error("rocm resident: batch %d outside the stepper range 1..%d", B, m->max_rows);
         return RD_ERR_ARG;
     }
+    RC(d->use());
     // A slot may carry several rows in one step if they sit at consecutive positions (a ragged step's verify or prefill
     // rows): all their K/V is written before any row attends, and row j reads keys [0, pos_j], so each row is the row its own
     // single-token step would compute. Anything else naming a slot twice is refused before a byte is written.
@@ -912,6 +914,7 @@ static int chain_start(rd_model *m, int slot, int id, int pos, bool sample, doub
         return RD_ERR_ARG;
     }
     rd_device *d = m->d;
+    RC(d->use());
     if (!ch.host_ids) {
         HIPCHK(HostMalloc((void **)&ch.host_ids, sizeof(int) * rd_model::Chain::DEPTH, 0));
         for (auto &e : ch.ev) HIPCHK(EventCreate(&e));
