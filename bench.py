@@ -8,7 +8,8 @@ Prints ONE JSON line with the whole-job tok/s, the roofline of the dominant kern
 restatement of goinfer's CPU path, timed on this box's host cores on a bounded sample of the same workload).
 
 --workload c2 | c3 | c5 runs the other measurement configurations BASELINE.json names instead (the Q4_K GEMM microbench, the
-ragged attention microbench, the Qwen3-MoE-shaped step; kquant: the Q5_K / Q6_K GEMMs beside Q4_K) and prints one line of the same form for that workload.
+ragged attention microbench, the Qwen3-MoE-shaped step; kquant: the Q5_K / Q6_K GEMMs beside Q4_K), topk (the device-side top-K of logits rows) or prefill (a 2048-token prompt
+pass into the same paged KV) and prints one line of the same form for that workload.
 """
 import argparse
 import json
@@ -94,10 +95,10 @@ def parse_args():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--kv", default="f16", choices=["f16", "i8"],
                     help="KV cache element (c4 and c3): f16 as the metric is quoted, or goinfer's int8 cache (KVQuant i8), a variant of the workload")
-    ap.add_argument("--workload", default="c4", choices=["c4", "c2", "c3", "c5", "kquant", "topk"],
+    ap.add_argument("--workload", default="c4", choices=["c4", "c2", "c3", "c5", "kquant", "topk", "prefill"],
                     help="c4 (default): the Llama-3-8B-shape step the metric is quoted on; c2: Q4_K GEMM microbench; c3: ragged "
                          "attention microbench; c5: Qwen3-MoE-shape step; kquant: Q4_K / Q5_K / Q6_K GEMMs at the FFN and head shapes; topk: "
-                         "the device-side top-K of logits rows")
+                         "the device-side top-K of logits rows; prefill: a 2048-token prompt pass into the same paged KV")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this backend is single-GPU (goinfer has no collective path); run with --gpus 1", file=sys.stderr)
@@ -206,4 +207,4 @@ if __name__ == "__main__":
         import bench_micro
         bench_micro.T0 = T0
         {"c2": bench_micro.run_c2, "c3": bench_micro.run_c3, "c5": bench_micro.run_c5, "kquant": bench_micro.run_kquant,
-         "topk": bench_micro.run_topk}[_args.workload](_args)
+         "topk": bench_micro.run_topk, "prefill": bench_micro.run_prefill}[_args.workload](_args)

@@ -354,3 +354,94 @@ def cpu_baseline_moe(res, cfg, lens, kept_kv):
     return {"value": round(B / full, 3), "unit": "tok/s", "cores": threads(), "kind": "port",
             "sample": "oracle decodeMultiStep, %d of %d layers + int8 head, B=%d at the run's context lengths, %d greedy steps (%.1f s), "
                       "per-layer cost scaled to %d layers" % (nL, cfg["n_layers"], B, n_steps, t_step, cfg["n_layers"])}
+
+
+# ------------------------------------------------------------------------------------------------------------ prefill
+MFMA_F16_PEAK_TFLOPS = 2500.0
+
+
+def run_prefill(args):
+    """A prompt pass into the decode step's own paged KV (PrefillLast): Llama-3-8B shape, one sequence, 2048 prompt tokens from
+    position 0, in passes of 128 rows; token ids through the embedding table, so nothing crosses PCIe inside the timed region.
+    A step is one whole prompt."""
+    from goinfer_amd import capi, workloads
+    n_tok = 2048
+    steps, warmup = (args.steps if args.steps != 128 else 5), (args.warmup if args.warmup != 8 else 1)
+    cfg = workloads.llama3_8b_cfg(args.layers)
+    dev = capi.Device(0)
+    log("building %s, %d layers" % (cfg["name"], args.layers))
+    res = workloads.Resident(dev, cfg, seed=args.seed, slots=1, ctx_cap=n_tok + 64, keep_layers=0 if args.no_cpu else min(4, args.layers), progress=log)
+    rng = np.random.default_rng(args.seed)
+    ids = rng.integers(0, cfg["vocab"], n_tok).astype(np.int32)
+    ms = []
+    for i in range(warmup + steps):
+        t = res.model.bench_prefill(0, ids)
+        if i >= warmup:
+            ms.append(t)
+        log("prompt %d: %.2f ms" % (i, t))
+    ms = np.array(ms)
+    tok_s = n_tok / (float(ms.mean()) / 1e3)
+    _, prof = res.model.bench_prefill(0, ids, profile=True)
+    classes = {k: {"ms_per_step": round(v[0], 4), "launches_per_step": v[1]} for k, v in prof.items()}
+    # dominant kernel: the Q4_K GEMM over 128 rows (every weight tile read and dequantized once for four row tiles of 32); the
+    # four projections of a layer are one launch each per pass. Flops over all rows of the prompt, milliseconds over all four classes
+    # (the last row's one-row step rides in the same classes: 1 row of 2048).
+    H, hd = cfg["hidden"], cfg["head_dim"]
+    qd, kvd, I = cfg["n_heads"] * hd, cfg["n_kv"] * hd, cfg["inter"]
+    w_elems = (qd + 2 * kvd) * H + H * qd + 2 * I * H + H * I
+    flops = 2.0 * n_tok * w_elems * cfg["n_layers"]
+    g_ms = sum(prof[k][0] for k in ("gemm_qkv", "gemm_o", "gemm_gateup", "gemm_down"))
+    g_n = sum(prof[k][1] for k in ("gemm_qkv", "gemm_o", "gemm_gateup", "gemm_down"))
+    tfl = flops / (g_ms / 1e3) / 1e12
+    out = base_line("prompt tok/s into the paged KV, Llama-3-8B-shape Q4_K, 2048-token prompt; achieved MFMA TFLOP/s vs peak", tok_s, "tok/s", steps, warmup,
+                    float(ms.mean()), "prefill: %s, %d layers, one sequence, %d prompt tokens from position 0 (PrefillLast), passes of 128 rows"
+                    % (cfg["name"], args.layers, n_tok),
+                    "synthetic: N(0,0.02) weights quantized to Q4_K (int8 head and embedding), random token ids", {"prompt_tokens": n_tok, "seed": args.seed})
+    out["roofline"] = {"bound": "mfma", "achieved": round(tfl, 1), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tfl / MFMA_F16_PEAK_TFLOPS, 4),
+                       "traffic": None, "kernel": "rd_k_gemm_q4k_wide", "avg_launch_ms": round(g_ms / g_n, 5), "algorithmic_flops_per_launch": int(flops / g_n)}
+    out["kernel_classes"] = classes
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline_prefill(res, cfg, ids)
+    out["cpu_baseline"] = cpu
+    res.close()
+    dev.close()
+    emit(out)
+
+
+def cpu_baseline_prefill(res, cfg, ids):
+    """The oracle walking the first tokens of the same prompt one at a time through the first layers of the same model (the reference's CPU
+    prompt pass computes the same rows), about ten seconds; the per-layer cost scaled to the full depth, the head left out as in a prompt pass."""
+    from goinfer_amd.workloads import inv_freq
+    from oracle import binding as ob
+    ob.set_threads(threads())
+    layers = []
+    for kp in res.kept:
+        lw = {p: ob.WMat(ob.OR_Q4K, kp[p][1], kp[p][2], kp[p][0], act_group=32) for p in ("q", "k", "v", "o", "gate", "up", "down")}
+        lw["attn_norm"], lw["ffn_norm"] = kp["attn_norm"], kp["ffn_norm"]
+        layers.append(lw)
+    nL = len(layers)
+    c = dict(cfg)
+    c.update(n_layers=nL, kv_f16=1)
+    hq, hs = res.head
+    head = ob.WMat(ob.OR_W8A8, hq.shape[0], hq.shape[1], hq, hs, act_group=32)
+    om = ob.OracleModel(c, layers, res.final_norm, head, inv_freq(cfg["head_dim"], cfg["theta"]))
+    MAXT = 1024
+    cp = om.new_cache(MAXT + 2)
+    emb = res.embed_rows(ids[:MAXT])
+    om.step(emb[0:1], [cp])
+    t0 = time.time()
+    for _ in range(3):
+        ob.matmul(head, emb[0:1])
+    t_head = (time.time() - t0) / 3
+    n, t = 0, 0.0
+    while n < MAXT - 1 and t < 10.0:
+        t0 = time.time()
+        om.step(emb[n + 1:n + 2], [cp])
+        t += time.time() - t0
+        n += 1
+    om.free_cache(cp)
+    per_layer = max(t / n - t_head, 1e-9) / nL
+    return {"value": round(1.0 / (per_layer * cfg["n_layers"]), 3), "unit": "tok/s", "cores": threads(), "kind": "port",
+            "sample": "oracle, %d of %d layers, the prompt's first %d tokens one at a time (%.1f s), head time taken out, per-layer cost scaled to %d layers"
+                      % (nL, cfg["n_layers"], n, t, cfg["n_layers"])}

@@ -69,6 +69,59 @@ extern "C" int rd_bench_profile(rd_model *m, int B, const int *slot, const int *
     return rc ? rc : rc2;
 }
 
+// A prompt pass with every input on the device: rows 0..n-1 of `slot` from token ids through the embedding table, in the passes
+// rd_prefill_last makes (all rows but the last build only their K/V, as wide as the step goes; the last is a one-row step with
+// the head). ms_total: the whole prompt, HIP events on the launch stream. profile != 0: an event pair around every kernel class
+// as in rd_bench_profile (the pairs stretch the run; take ms_total from a call without them).
+extern "C" int rd_bench_prefill(rd_model *m, int slot, int n, const int *ids, int profile, float *ms_total, float *class_ms, int *class_n) {
+    if (!m || !ids || !ms_total || n < 1 || (profile && (!class_ms || !class_n))) return RD_ERR_ARG;
+    if (!m->embed_q || !m->tables || slot < 0 || slot >= m->slots || n > m->ctx_cap) {
+        rd_set_error("rd_bench_prefill: needs the embedding table, a configured KV pool, a slot in range and n within the context cap");
+        return RD_ERR_STATE;
+    }
+    rd_device *d = m->d;
+    RC(rd_kv_reset(m, slot));
+    int *ids_dev = nullptr;
+    RC(d->alloc((void **)&ids_dev, sizeof(int) * (size_t)n));
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    int rc = d->h2d(ids_dev, ids, sizeof(int) * (size_t)n);
+    if (!rc) rc = d->sync();
+    if (!rc && (d->hip->EventCreate(&e0) != hipSuccess || d->hip->EventCreate(&e1) != hipSuccess)) rc = RD_ERR_HIP;
+    const int pass = m->max_rows;
+    std::vector<int> rslot((size_t)pass, slot), rpos((size_t)pass);
+    m->timer.on = profile != 0;
+    if (!rc) (void)d->hip->EventRecord(e0, d->stream);
+    auto run = [&](int r0, int rows, int want) {
+        for (int j = 0; j < rows; j++) rpos[(size_t)j] = r0 + j;
+        if (!rd_hip_ok(d->hip, d->hip->MemcpyAsync(m->ids, ids_dev + r0, sizeof(int) * (size_t)rows, hipMemcpyDeviceToDevice, d->stream), "hipMemcpy D2D"))
+            return (int)RD_ERR_HIP;
+        return model_step(m, rows, rslot.data(), rpos.data(), nullptr, nullptr, want, nullptr, nullptr, true);
+    };
+    for (int r0 = 0; r0 < n - 1 && !rc; r0 += pass) rc = run(r0, std::min(pass, n - 1 - r0), 0);
+    if (!rc) rc = run(n - 1, 1, RD_WANT_ARGMAX);
+    m->timer.on = false;
+    if (!rc) (void)d->hip->EventRecord(e1, d->stream);
+    int rc2 = d->sync();
+    *ms_total = 0.f;
+    if (!rc && !rc2) (void)d->hip->EventElapsedTime(ms_total, e0, e1);
+    if (profile) {
+        memset(class_ms, 0, sizeof(float) * KC_COUNT);
+        memset(class_n, 0, sizeof(int) * KC_COUNT);
+        for (size_t i = 0; i < m->timer.cls.size(); i++) {
+            float ms = 0.f;
+            if (!rc && !rc2) (void)d->hip->EventElapsedTime(&ms, m->timer.ev[2 * i], m->timer.ev[2 * i + 1]);
+            class_ms[m->timer.cls[i]] += ms;
+            class_n[m->timer.cls[i]]++;
+        }
+    }
+    for (hipEvent_t e : m->timer.ev) (void)d->hip->EventDestroy(e);
+    m->timer.ev.clear(), m->timer.cls.clear();
+    if (e0) (void)d->hip->EventDestroy(e0);
+    if (e1) (void)d->hip->EventDestroy(e1);
+    d->release(ids_dev);
+    return rc ? rc : rc2;
+}
+
 extern "C" int rd_bench_class_count(void) { return KC_COUNT; }
 extern "C" const char *rd_bench_class_name(int c) {
     static const char *names[KC_COUNT] = {"gemm_qkv", "rope_kvstore", "attn_partial", "attn_combine", "gemm_o", "add_rmsnorm_quant", "gemm_gateup",

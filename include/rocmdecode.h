@@ -247,6 +247,10 @@ int rd_bench_steps(rd_model *m, int B, const int *slot, const int *pos0, const i
 /* One step with a HIP-event pair around every kernel class: class_ms[n] total milliseconds and class_n[n] launches,
  * n = rd_bench_class_count(); names from rd_bench_class_name. */
 int rd_bench_profile(rd_model *m, int B, const int *slot, const int *pos, const int *ids0, float *class_ms, int *class_n);
+/* A whole prompt pass timed on the device: rows 0..n-1 of `slot` (reset first) from token ids through the embedding table, in
+ * rd_prefill_last's passes. ms_total: milliseconds for the prompt; profile != 0 also fills class_ms / class_n as
+ * rd_bench_profile does. */
+int rd_bench_prefill(rd_model *m, int slot, int n, const int *ids, int profile, float *ms_total, float *class_ms, int *class_n);
 int rd_bench_class_count(void);
 const char *rd_bench_class_name(int c);
 /* Times `iters` launches of one kernel over resident synthetic operands: "gemm_q4k" args {N,K,M,copies}; "copy" args {bytes}. */
