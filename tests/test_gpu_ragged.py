@@ -144,3 +144,26 @@ def test_ragged_step_with_draws(dev):
     assert np.array_equal(bits(plain), bits(logits))
     pair.close()
     pair2.close()
+
+
+def test_timed_prompt_pass_leaves_the_prefill_state(dev):
+    """rd_bench_prefill (what `bench.py --workload prefill` times) runs rd_prefill_last's passes with the rows looked up on the
+    device: the slot it fills continues with the same bits as a slot filled through rd_prefill_last from host rows."""
+    from goinfer_amd import synth
+    cfg = dense_cfg(n_layers=2, hidden=256, inter=512, vocab=4096)
+    pair = Pair(cfg, 47, dev, slots=2, ctx_cap=320)
+    try:
+        q, sc = synth.w8a8_normal(78, cfg["vocab"], cfg["hidden"], 0.02)
+        rows = q.astype(np.float32) * sc[:, None]
+        pair.gpu.upload_embedding(q, sc)
+        rng = np.random.default_rng(9)
+        toks = rng.integers(0, cfg["vocab"], 283)  # two full passes of 128, one of 26, the last row alone
+        pair.gpu.prefill_last(0, 0, rows[toks])
+        ms, classes = pair.gpu.bench_prefill(1, toks, profile=True)
+        assert ms > 0 and classes["gemm_qkv"][1] == 4 * cfg["n_layers"]
+        nxt = rows[17][None, :]
+        a, _ = pair.gpu.step_batch([0], [len(toks)], nxt)
+        b, _ = pair.gpu.step_batch([1], [len(toks)], nxt)
+        assert np.array_equal(bits(a), bits(b))
+    finally:
+        pair.close()
