@@ -35,7 +35,10 @@
  *                                        draw>>32, 0; lane i&3) is "parity unpinned" beyond its statement in the source.
  *   or_matmul (f32 kind)                 parity unpinned at bit level (aikit's summation order is arch dependent);
  *                                        pinned to tolerance by the HF goldens
- *   or_matmul (q4k / w4a8 / w8a8 kinds)  parity unpinned at bit level: the reference's own result differs between
+ *   or_matmul (w8a8 kind)                pinned: linalg.MatmulBTW8A8 fingerprint (per-row activations, every reference
+ *                                        configuration); per-32 activations: linalg.MatmulBTW8A8Into, bit-exact to the
+ *                                        arm64[dotprod] entry (the reference's own amd64 and arm64 digests differ)
+ *   or_matmul (q4k / w4a8 kinds)         parity unpinned at bit level: the reference's own result differs between
  *                                        amd64 and arm64 (kernel_fingerprints.json). Restated in the mathematically
  *                                        specified form (exact int32 dot per 32-group, f32 fold in ascending group
  *                                        order, backend/cuda/actgroup.cu:298-355) and checked against an f64 sum.
