@@ -25,7 +25,7 @@ def bits(x):
     return np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
 
 
-def walk(pair, emb, vocab, slots, cap, seed, n_ops, max_batch, chains=False):
+def walk(pair, emb, vocab, slots, cap, seed, n_ops, max_batch, chains=False, max_prefill=50, max_ragged=7, moves=None):
     """emb: the embedding rows by token id. Returns (history per slot, last logits per slot). Slot `slots` (one past the last) is
     left for the replay. chains: the device-side greedy chain is one of the moves (emb must then be the resident table's rows)."""
     rng = np.random.default_rng(seed)
@@ -33,7 +33,7 @@ def walk(pair, emb, vocab, slots, cap, seed, n_ops, max_batch, chains=False):
     last = [None] * slots
     g = pair.gpu
     for _ in range(n_ops):
-        op = rng.choice(["batch", "batch", "ragged", "prefill", "truncate", "reset", "nologits"] + (["chain"] if chains else []))
+        op = rng.choice(moves or (["batch", "batch", "ragged", "prefill", "truncate", "reset", "nologits"] + (["chain"] if chains else [])))
         if op == "batch":
             k = int(rng.integers(1, min(slots, max_batch) + 1))
             chosen = [int(s) for s in rng.permutation(slots)[:k] if len(hist[s]) < cap - 1]
@@ -48,7 +48,7 @@ def walk(pair, emb, vocab, slots, cap, seed, n_ops, max_batch, chains=False):
         elif op == "ragged":
             k = int(rng.integers(1, min(3, slots) + 1))
             chosen = [int(s) for s in rng.permutation(slots)[:k]]
-            rows = [int(rng.integers(1, 7)) for _ in chosen]
+            rows = [int(rng.integers(1, max_ragged)) for _ in chosen]
             keep = [(s, r) for s, r in zip(chosen, rows) if len(hist[s]) + r < cap]
             if not keep or sum(r for _, r in keep) > max_batch:
                 continue
@@ -61,7 +61,7 @@ def walk(pair, emb, vocab, slots, cap, seed, n_ops, max_batch, chains=False):
                 off += r
         elif op == "prefill":
             s = int(rng.integers(0, slots))
-            n = int(rng.integers(1, 50))
+            n = int(rng.integers(1, max_prefill))
             if len(hist[s]) + n >= cap:
                 continue
             toks = rng.integers(0, vocab, n)
@@ -102,11 +102,15 @@ def walk(pair, emb, vocab, slots, cap, seed, n_ops, max_batch, chains=False):
     return hist, last
 
 
-@pytest.mark.parametrize("seed", [82, 83, 84])
+@pytest.mark.parametrize("seed", [82, 83, 84, "long"])
 @pytest.mark.parametrize("kind,kv", [("dense", "f16"), ("dense", "i8"), ("moe", "f16"), ("dense-chains", "f16")])
 def test_random_walk_replays_bit_identically(dev, kind, kv, seed):
     cfg = moe_cfg(n_layers=2) if kind == "moe" else dense_cfg(n_layers=2)
     slots, cap = 5, 160
+    grow = {}
+    if seed == "long":  # moves that mostly add rows, many at a time: the slots pass 1024 positions, where a sequence's attention is cut in pieces of several blocks
+        slots, cap, seed = 4, 2600, 86
+        grow = dict(max_prefill=500, max_ragged=41, moves=["batch"] * 8 + ["ragged"] * 6 + ["prefill"] * 6 + ["nologits", "truncate"] + (["chain"] if kind == "dense-chains" else []))
     pair = Pair(cfg, seed=81, dev=dev, slots=slots + 1, ctx_cap=cap, kv=kv)
     try:
         emb = pair.emb
@@ -115,8 +119,10 @@ def test_random_walk_replays_bit_identically(dev, kind, kv, seed):
             q, sc = synth.w8a8_normal(85, cfg["vocab"], cfg["hidden"], 0.02)
             pair.gpu.upload_embedding(q, sc)
             emb = q.astype(np.float32) * sc[:, None]
-        hist, last = walk(pair, emb, cfg["vocab"], slots, cap, seed=seed, n_ops=300, max_batch=32 if kind == "moe" else 128,
-                          chains=kind == "dense-chains")
+        hist, last = walk(pair, emb, cfg["vocab"], slots, cap, seed=seed, n_ops=120 if grow else 300, max_batch=32 if kind == "moe" else 128,
+                          chains=kind == "dense-chains", **grow)
+        if grow:
+            assert max(len(h) for h in hist) > 1024
         checked = 0
         for s in range(slots):
             if not hist[s]:
