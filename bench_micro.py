@@ -398,7 +398,7 @@ def run_prefill(args):
                     % (cfg["name"], args.layers, n_tok),
                     "synthetic: N(0,0.02) weights quantized to Q4_K (int8 head and embedding), random token ids", {"prompt_tokens": n_tok, "seed": args.seed})
     out["roofline"] = {"bound": "mfma", "achieved": round(tfl, 1), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tfl / MFMA_F16_PEAK_TFLOPS, 4),
-                       "traffic": None, "kernel": "rd_k_gemm_q4k_wide", "avg_launch_ms": round(g_ms / g_n, 5), "algorithmic_flops_per_launch": int(flops / g_n)}
+                       "traffic": counter_traffic("gemm_q4k_wide/%s/prefill%d" % (cfg["name"], n_tok)), "kernel": "rd_k_gemm_q4k_wide", "avg_launch_ms": round(g_ms / g_n, 5), "algorithmic_flops_per_launch": int(flops / g_n)}
     out["kernel_classes"] = classes
     cpu = None
     if not args.no_cpu:
