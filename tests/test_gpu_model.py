@@ -18,22 +18,35 @@ def dev():
     d.close()
 
 
-def prefill(pair, slot, toks):
+def prefill(pair, slot, toks, traces=None):
+    """Token by token; returns the last logits and, given the oracle's expert traces of the same prompt, whether the GPU's
+    routing stayed on them at every position."""
+    on_trace = True
     for p, t in enumerate(toks):
         g, _ = pair.gpu.step_batch([slot], [p], pair.emb[t][None, :])
-    return g[0]
+        if traces is not None and on_trace:
+            on_trace = np.array_equal(pair.gpu.last_moe_indices(1)[0], traces[p][0])
+    return (g[0], on_trace) if traces is not None else g[0]
 
 
-def oracle_run(pair, prompts, steps, eps=0.0, force=None):
+def oracle_run(pair, prompts, steps, eps=0.0, force=None, prompt_traces=None):
     """The oracle on the ragged batch: per-sequence prefill, then `steps` batched greedy steps. Returns the prefill's last
-    logits, the per-step logits, the tokens fed at each step and (MoE) the expert traces. eps perturbs every embedding."""
+    logits, the per-step logits, the tokens fed at each step and (MoE) the expert traces. eps perturbs every embedding.
+    prompt_traces: a list that receives, per prompt, the expert trace of every prompt position (MoE)."""
     B = len(prompts)
     caches = [pair.oracle.new_cache(pair.ctx_cap) for _ in range(B)]
     emb = (lambda t, key: perturbed(pair.emb[t], eps, key)) if eps else (lambda t, key: pair.emb[t])
     last = []
+    want_pt = prompt_traces is not None and pair.cfg.get("n_experts", 0) > 0
     for b, toks in enumerate(prompts):
+        pt = []
         for p, t in enumerate(toks):
-            o = pair.oracle.step(emb([t], (b, p)), [caches[b]])
+            o = pair.oracle.step(emb([t], (b, p)), [caches[b]], want_moe=want_pt)
+            if want_pt:
+                o, tr = o
+                pt.append(np.asarray(tr).copy())
+        if want_pt:
+            prompt_traces.append(pt)
         last.append(o[0].copy())
     nxt = force[0] if force is not None else [ob.argmax(x) for x in last]
     fed, outs, traces = [], [], []
@@ -53,15 +66,24 @@ def oracle_run(pair, prompts, steps, eps=0.0, force=None):
 def run_ragged(pair, prompts, steps):
     """GPU vs oracle, teacher-forced on the oracle's greedy tokens. Returns the worst logit deviation and the noise floor."""
     B = len(prompts)
-    last, outs, fed, traces = oracle_run(pair, prompts, steps)
+    ptraces = []
+    last, outs, fed, traces = oracle_run(pair, prompts, steps, prompt_traces=ptraces)
     last2, outs2, _, _ = oracle_run(pair, prompts, steps, eps=1e-6, force=fed)  # same tokens, perturbed embeddings
     floor = max([float(np.abs(a - b).max()) for a, b in zip(last, last2)] + [float(np.abs(a - b).max()) for a, b in zip(outs, outs2)])
     worst, agree, total = 0.0, 0, 0
     diverged = [False] * B  # MoE rows whose routing has left the oracle's: a different expert is a different function
+    off_prompt = [False] * B  # MoE rows with such a position inside their prompt
     for b, toks in enumerate(prompts):
-        g = prefill(pair, b, toks)
+        if ptraces:  # MoE: a prompt position routed to another expert than the oracle's has written different K/V for that position
+            g, on_trace = prefill(pair, b, toks, ptraces[b])
+            off_prompt[b] = not on_trace
+        else:
+            g = prefill(pair, b, toks)
         prefill(pair, B + b, toks)  # a twin slot, stepped alone below
         ok, d = logits_close(g, last[b], floor)
+        if not ok and off_prompt[b]:  # held to the bar all the same; only a miss is put down to the other expert
+            diverged[b] = True
+            continue
         assert ok, ("prefill", b, d, floor)
         worst = max(worst, d)
     pos = [len(t) for t in prompts]
@@ -79,6 +101,9 @@ def run_ragged(pair, prompts, steps):
             if diverged[b]:
                 continue
             ok, d = logits_close(g[b], o[b], floor)
+            if not ok and off_prompt[b]:
+                diverged[b] = True
+                continue
             assert ok, ("step", s, b, d, floor)
             worst = max(worst, d)
             assert near_tie_ok(o[b], int(ids[b])), ("greedy token", s, b)
