@@ -128,8 +128,8 @@ extern "C" __global__ __launch_bounds__(1024) void rd_k_add_rmsnorm_quant(float 
 #pragma unroll
             for (int j = 0; j < 8; j++)
                 if (j < splits) {
-                    a.x = __fadd_rn(a.x, __fmul_rn(wr[j], b[i][j].x)), a.y = __fadd_rn(a.y, __fmul_rn(wr[j], b[i][j].y));
-                    a.z = __fadd_rn(a.z, __fmul_rn(wr[j], b[i][j].z)), a.w = __fadd_rn(a.w, __fmul_rn(wr[j], b[i][j].w));
+                    a.x = __fadd_rn(a.x, mul_rounded(wr[j], b[i][j].x)), a.y = __fadd_rn(a.y, mul_rounded(wr[j], b[i][j].y));
+                    a.z = __fadd_rn(a.z, mul_rounded(wr[j], b[i][j].z)), a.w = __fadd_rn(a.w, mul_rounded(wr[j], b[i][j].w));
                 }
             v[i].x = __fadd_rn(v[i].x, a.x), v[i].y = __fadd_rn(v[i].y, a.y), v[i].z = __fadd_rn(v[i].z, a.z), v[i].w = __fadd_rn(v[i].w, a.w);
             *(float4_t *)(h + (size_t)m * H + 4 * (t + i * 1024)) = v[i];

@@ -31,6 +31,14 @@ typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
 #define RD_DPP_QUAD_XOR2 0x4E   // quad_perm:[2,3,0,1]
 #define RD_DPP_HALF_MIRROR 0x141 // row_half_mirror
 #define RD_DPP_ROW_MIRROR 0x140  // row_mirror
+// a*b rounded to f32 on its own. HIP's __fmul_rn is a plain product, which the compiler is free to contract with a following add
+// into one FMA (one rounding instead of two); where the reference's arithmetic rounds the product first and an add follows, the
+// product goes through here.
+__device__ __forceinline__ float mul_rounded(float a, float b) {
+#pragma clang fp contract(off)
+    return a * b;
+}
+
 template <int CTRL> __device__ __forceinline__ int dpp_i(int v) { return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true); }
 template <int CTRL> __device__ __forceinline__ float dpp_f(float v) { return __int_as_float(dpp_i<CTRL>(__float_as_int(v))); }
 __device__ __forceinline__ int swz_xor16_i(int v) { return __builtin_amdgcn_ds_swizzle(v, 0x401F); } // bit mode: and 0x1F, xor 0x10

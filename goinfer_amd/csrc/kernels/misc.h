@@ -84,7 +84,7 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_argmax_rows(const float *
                 uint32_t r[4];
                 philox4x32((uint32_t)(n0 >> 2), (uint32_t)dr[4], (uint32_t)dr[5], 0u, (uint32_t)dr[2], (uint32_t)dr[3], r);
 #pragma unroll
-                for (int e = 0; e < 4; e++) a[e] = __fadd_rn(__fmul_rn(a[e], invT), gumbel_noise(r[e]));
+                for (int e = 0; e < 4; e++) a[e] = __fadd_rn(mul_rounded(a[e], invT), gumbel_noise(r[e]));
             }
 #pragma unroll
             for (int e = 0; e < 4; e++)

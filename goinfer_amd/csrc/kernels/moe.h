@@ -130,6 +130,6 @@ extern "C" __global__ void rd_k_moe_fold(const float *__restrict__ dn, const flo
     int t = blockIdx.y, n = blockIdx.x * 256 + threadIdx.x;
     if (n >= H) return;
     float acc = 0.f;
-    for (int r = 0; r < k; r++) acc = __fadd_rn(acc, __fmul_rn(wgt[t * k + r], dn[((size_t)t * k + r) * H + n]));
+    for (int r = 0; r < k; r++) acc = __fadd_rn(acc, mul_rounded(wgt[t * k + r], dn[((size_t)t * k + r) * H + n]));
     out[(size_t)t * H + n] = acc;
 }

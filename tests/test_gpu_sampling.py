@@ -155,3 +155,22 @@ def test_chain_runs_into_the_context_cap(dev):
         pair.gpu.step_batch([0], [0], rows[:1])
     finally:
         pair.close()
+
+
+def test_tied_keys_at_tiny_temperatures_keep_the_host_order(dev):
+    """Two equal largest logits at a temperature so small that the noise vanishes in the f32 key: the keys tie and the lowest
+    index wins, as on the host. The product logit * 1/T must be rounded before the noise is added (sampler_gumbel.go:41-66): a
+    fused multiply-add lets the noise's sign decide the rounding of a product that falls halfway between two f32 values, and
+    the tie breaks the other way."""
+    seed, draw = 4648040972980819852, 2410598768476298352
+    V = 211
+    row = np.full(V, -3.0, np.float32)
+    row[107] = row[115] = 6.0
+    for T in (1e-30, 1e-25, 1e-20, 1e-10, 1e-6, 1e-3, 1.0):
+        got = dev.sample_rows(row[None, :], [(T, seed, draw)])
+        assert int(got[0]) == ob.gumbel_draw(row, T, seed, draw, guarded=True), T
+    rng = np.random.default_rng(5)
+    rows = np.round(rng.standard_normal((64, 300)) * 2).astype(np.float32)  # heavily tied rows
+    draws = [((1e-30, 1e-10, 1e-8, 3e-7)[r % 4], int(rng.integers(0, 1 << 62)), r) for r in range(64)]
+    got = dev.sample_rows(rows, draws)
+    assert list(got) == [ob.gumbel_draw(rows[r], *draws[r], guarded=True) for r in range(64)]
