@@ -421,6 +421,12 @@ extern "C" int rd_kv_configure_typed(rd_model *m, int slots, int ctx_cap, int kv
         rd_set_error("KV already configured");
         return RD_ERR_STATE;
     }
+    // The work list, the partial-sum area, the metadata block and the pinned staging slots are sized from the widest step the
+    // model takes, which rd_model_finalize settles: configuring first would size them for a narrower step than the model runs.
+    if (!m->finalized) {
+        rd_set_error("rd_kv_configure before rd_model_finalize");
+        return RD_ERR_STATE;
+    }
     rd_device *d = m->d;
     RC(d->use());
     const rd_model_desc &c = m->desc;
@@ -501,7 +507,7 @@ extern "C" int rd_kv_upload(rd_model *m, int slot, int layer, int base, int n, c
         RC(d->launch(d->k.kv_store_i8, (unsigned)n, (unsigned)c.n_kv_heads, 1, 64, (const float *)K.p, (const float *)V.p, (signed char *)l.Kp,
                      (signed char *)l.Vp, l.Ksc, l.Vsc, (const int *)(m->tables + (size_t)slot * m->blocks_per_slot), base, c.n_kv_heads, c.head_dim));
     else
-        RC(d->launch(d->k.kv_store, (unsigned)n, 1, 1, (unsigned)kvd, (const float *)K.p, (const float *)V.p, l.Kp, l.Vp,
+        RC(d->launch(d->k.kv_store, (unsigned)n, (unsigned)c.n_kv_heads, 1, (unsigned)c.head_dim, (const float *)K.p, (const float *)V.p, l.Kp, l.Vp,
                      (const int *)(m->tables + (size_t)slot * m->blocks_per_slot), base, c.n_kv_heads, c.head_dim));
     RC(d->sync());
     m->slot_len[(size_t)slot] = std::max(m->slot_len[(size_t)slot], base + n);

@@ -365,7 +365,7 @@ static int attn_ragged_typed(rd_device *d, int kv_type, int n_seq, const int *le
                     RC(d->launch(d->k.kv_store_i8, (unsigned)n, (unsigned)n_kv, 1, 64, (const float *)Kc.p, (const float *)Vc.p, (signed char *)Kp.p,
                                  (signed char *)Vp.p, Ksc.as<float>(), Vsc.as<float>(), (const int *)((const int *)T.p + (size_t)i * maxBlocks), base, n_kv, hd));
                 else
-                    RC(d->launch(d->k.kv_store, (unsigned)n, 1, 1, (unsigned)kvd, (const float *)Kc.p, (const float *)Vc.p, (uint16_t *)Kp.p,
+                    RC(d->launch(d->k.kv_store, (unsigned)n, (unsigned)n_kv, 1, (unsigned)hd, (const float *)Kc.p, (const float *)Vc.p, (uint16_t *)Kp.p,
                                  (uint16_t *)Vp.p, (const int *)((const int *)T.p + (size_t)i * maxBlocks), base, n_kv, hd));
                 RC(d->sync());
             }

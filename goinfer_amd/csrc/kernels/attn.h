@@ -81,14 +81,14 @@ __device__ __forceinline__ void kv_store_elem(uint16_t *__restrict__ Kp, uint16_
 }
 
 // Host-provided rows (UploadKV, decoder/resident/forward.go:20-26): k,v f32 [n][nKV*HD] -> positions base..base+n-1 of one sequence.
-// Grid (n), block nKV*HD threads (<= 1024).
+// Grid (n, nKV), block HD threads: one block per (position, kv head), whatever the number of kv heads.
 extern "C" __global__ void rd_k_kv_store(const float *__restrict__ k, const float *__restrict__ v, uint16_t *__restrict__ Kp,
                                          uint16_t *__restrict__ Vp, const int *__restrict__ table, int base, int nKV, int HD) {
-    int i = blockIdx.x, t = threadIdx.x;
-    if (t >= nKV * HD) return;
-    int pos = base + i, blk = table[pos >> 6], p = pos & 63, kvh = t / HD, d = t % HD;
-    size_t region = ((size_t)blk * nKV + kvh) * 64 * HD;
-    kv_store_elem(Kp, Vp, HD, region, p, d, k[(size_t)i * nKV * HD + t], v[(size_t)i * nKV * HD + t]);
+    int i = blockIdx.x, kvh = blockIdx.y, d = threadIdx.x;
+    if (d >= HD) return;
+    int pos = base + i, blk = table[pos >> 6], p = pos & 63;
+    size_t region = ((size_t)blk * nKV + kvh) * 64 * HD, src = ((size_t)i * nKV + kvh) * HD + d;
+    kv_store_elem(Kp, Vp, HD, region, p, d, k[src], v[src]);
 }
 
 // After the q|k|v GEMM: reduce its split-K partials, optional q|k|v bias (Qwen2; decoder/attention.go:12-34 addBias, applied right

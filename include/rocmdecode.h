@@ -138,6 +138,8 @@ int rd_model_upload_f32(rd_model *m, int layer, int which, const float *v, size_
 int rd_model_finalize(rd_model *m);
 
 /* ---- KV: resident/subsystems.go:236-251 (KVSlots), resident/forward.go:20-30 (UploadKV, TruncateTo, Reset) ---- */
+/* Order: rd_model_create, the uploads, rd_model_finalize, then rd_kv_configure(_typed), once. The pool's work list and staging
+ * are sized for the widest step the finalized model takes; before rd_model_finalize the call returns RD_ERR_STATE. */
 int rd_kv_configure(rd_model *m, int slots, int ctx_cap);
 /* The same with the cache's element type: RD_KV_F16 (rd_kv_configure's), or RD_KV_I8 = goinfer's int8 cache (KVQuant "i8":
  * decoder/kvcache.go:13-20,43-52 quantizeHeads; backend/cuda/kv8_store.cu, kvtype.cuh:48-73): per (position, kv head) head_dim

@@ -53,3 +53,70 @@ def test_kquant_matmul_random_blocks(fmt):
     q, S = ob.quantize_act(a, 32)
     want = (q.astype(np.float64) * np.repeat(S.astype(np.float64), 32, axis=1)) @ w.T
     assert np.abs(got - want).max() / np.sqrt((want * want).mean()) < 1e-5
+
+
+def f16_bits_to_f64(bits):
+    """binary16 bit patterns widened by numpy's own IEEE conversion (no oracle code involved)."""
+    return np.asarray(bits, dtype=np.uint16).view(np.float16).astype(np.float64)
+
+
+def int4_weights_f64(nib, s16, N, K):
+    """Canonical int4 rows as the reference states them (backend/cuda/kernels/actgroup_kernel_test.go:252-261: element k sits in
+    nibble k%2 of byte k/2, low nibble first, value nib-8; backend/cuda/internal/wpack/wpack.go:165-207 is the permuted device
+    form of the same words), times the binary16 group scale of k/32."""
+    nib = np.asarray(nib, dtype=np.uint8).reshape(N, (K + 1) // 2)
+    codes = np.empty((N, K), np.float64)
+    codes[:, 0::2] = (nib & 15).astype(np.float64)[:, :(K + 1) // 2]
+    codes[:, 1::2] = (nib >> 4).astype(np.float64)[:, :K // 2]
+    scales = f16_bits_to_f64(np.asarray(s16).reshape(N, -1))
+    return (codes - 8.0) * np.repeat(scales, 32, axis=1)[:, :K]
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 32, 128), (5, 96, 768), (16, 64, 2048), (3, 40, 96)])
+def test_w4a8_matmul_is_the_sum_of_pinned_pieces(M, N, K):
+    """The int4 lane (the MoE experts' kind) from pieces pinned on their own: quantize_int4's nibbles and binary16 scales
+    (fingerprints QuantizeGroupInt4Row / QuantizeInt4 / F32ToF16) and quantize_act's codes and scales (QuantizeActQ). A wrong
+    nibble order, a missing -8, a scale taken from the wrong group or widened wrongly fails by orders of magnitude."""
+    w = synth.normal(31 + N, N * K, 0.02).reshape(N, K)
+    nib, s16 = ob.quantize_int4(w)
+    a = synth.normal(7 + M, M * K).reshape(M, K)
+    mat = ob.WMat(ob.OR_W4A8, N, K, nib, s16, act_group=32)
+    got = ob.matmul(mat, a)
+    wd = int4_weights_f64(nib, s16, N, K)
+    assert np.abs(wd - w).max() < 0.02 * 4.5 / 7 * 0.6  # and the pieces are a quantization of w at all
+    q, S = ob.quantize_act(a, 32)
+    want = (q.astype(np.float64) * np.repeat(S.astype(np.float64), 32, axis=1)) @ wd.T
+    rms = np.sqrt((want * want).mean())
+    assert np.abs(got - want).max() / rms < 1e-5
+    assert np.abs(ob.matmul_f64ref(mat, a) - want).max() / rms < 1e-6
+
+
+def test_w4a8_matmul_random_nibbles_and_scales():
+    """Random bytes reach every nibble value and the scales' whole exponent range in use, which quantized normals do not."""
+    N, K, M = 32, 512, 3
+    rng = np.random.default_rng(5)
+    nib = rng.integers(0, 256, N * K // 2, dtype=np.uint8).reshape(N, K // 2)
+    s16 = ((rng.integers(1, 20, N * (K // 32)).astype(np.uint16) << 10) | rng.integers(0, 1024, N * (K // 32)).astype(np.uint16)).reshape(N, K // 32)
+    a = synth.normal(9, M * K).reshape(M, K)
+    mat = ob.WMat(ob.OR_W4A8, N, K, nib, s16, act_group=32)
+    q, S = ob.quantize_act(a, 32)
+    want = (q.astype(np.float64) * np.repeat(S.astype(np.float64), 32, axis=1)) @ int4_weights_f64(nib, s16, N, K).T
+    rms = np.sqrt((want * want).mean())
+    assert np.abs(ob.matmul(mat, a) - want).max() / rms < 1e-5
+    assert np.abs(ob.matmul_f64ref(mat, a) - want).max() / rms < 1e-6
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 32, 128), (7, 64, 896), (32, 96, 4096)])
+def test_w8a8_per32_matmul_is_the_sum_of_pinned_pieces(M, N, K):
+    """The int8 lane with per-32 activations (LM head and the projections whose K is no multiple of 256), against the same sum:
+    quantize_rows_int8's codes and per-row scales are pinned by QuantizeRowInt8, the activations by QuantizeActQ."""
+    w = synth.normal(41 + N, N * K, 0.02).reshape(N, K)
+    wq, ws = ob.quantize_rows_int8(w)
+    a = synth.normal(3 + M, M * K).reshape(M, K)
+    mat = ob.WMat(ob.OR_W8A8, N, K, wq, ws, act_group=32)
+    q, S = ob.quantize_act(a, 32)
+    wd = wq.astype(np.float64) * ws.astype(np.float64)[:, None]
+    want = (q.astype(np.float64) * np.repeat(S.astype(np.float64), 32, axis=1)) @ wd.T
+    rms = np.sqrt((want * want).mean())
+    assert np.abs(ob.matmul(mat, a) - want).max() / rms < 1e-5
+    assert np.abs(ob.matmul_f64ref(mat, a) - want).max() / rms < 1e-6
