@@ -25,6 +25,7 @@ EXPORTS = [
     "rd_step_batch_draw", "rd_sample_rows", "rd_greedy_chain_start", "rd_greedy_chain_next", "rd_sample_chain_start",
     "rd_sample_chain_next", "rd_greedy_chain_stop",
     "rd_dequant_q5k", "rd_dequant_q6k", "rd_gemm_q5k", "rd_gemm_q6k", "rd_model_upload_q5k", "rd_model_upload_q6k",
+    "rd_kv_download", "rd_qkv_rope_store",
 ]
 
 
@@ -243,6 +244,22 @@ class Device:
                                         hd, C.c_float(scale), C.c_float(softcap), _p(out)), "rd_attn_ragged_rows")
         return out
 
+    def qkv_rope_store(self, x, pos, n_h, n_kv, hd, inv_freq, q_norm=None, k_norm=None, eps=1e-6, bias=None, kv="f16"):
+        """The step's q|k|v epilogue on rows x [rows][(n_h+2n_kv)*hd]: (q, k as stored, v as stored)."""
+        x = _f32(x)
+        rows = x.shape[0]
+        pos = np.ascontiguousarray(pos, dtype=np.int32)
+        inv = np.ascontiguousarray(inv_freq, dtype=np.float64)
+        qn = None if q_norm is None else _f32(q_norm)
+        kn = None if k_norm is None else _f32(k_norm)
+        bi = None if bias is None else _f32(bias)
+        q = np.empty((rows, n_h * hd), np.float32)
+        k = np.empty((rows, n_kv * hd), np.float32)
+        v = np.empty((rows, n_kv * hd), np.float32)
+        check(lib().rd_qkv_rope_store(self.h, 0 if kv == "f16" else 1, rows, _p(x), _p(pos), n_h, n_kv, hd, _p(inv), _p(qn), _p(kn), C.c_float(eps),
+                                      _p(bi), _p(q), _p(k), _p(v)), "rd_qkv_rope_store")
+        return q, k, v
+
     def moe_route(self, logits, k, norm):
         logits = _f32(logits)
         T, nE = logits.shape
@@ -334,6 +351,13 @@ class Model:
     def kv_upload(self, slot, layer, base, keys, vals):
         keys, vals = _f32(keys), _f32(vals)
         check(lib().rd_kv_upload(self.h, slot, layer, base, keys.shape[0], _p(keys), _p(vals)), "rd_kv_upload")
+
+    def kv_download(self, slot, layer, base, n):
+        """Rows base..base+n-1 of a slot as the cache holds them, widened to f32: (keys, vals), each [n][n_kv*hd]."""
+        kvd = self.cfg["n_kv"] * self.cfg["head_dim"]
+        keys, vals = np.empty((n, kvd), np.float32), np.empty((n, kvd), np.float32)
+        check(lib().rd_kv_download(self.h, slot, layer, base, n, _p(keys), _p(vals)), "rd_kv_download")
+        return keys, vals
 
     def kv_reset(self, slot):
         check(lib().rd_kv_reset(self.h, slot), "rd_kv_reset")

@@ -93,6 +93,7 @@ static const KName kNames[] = {
     {"rd_k_retile_q6k", &Kernels::retile_q6k},
     {"rd_k_gemm_q6k", &Kernels::gemm_q6k},
     {"rd_k_kv_store", &Kernels::kv_store},
+    {"rd_k_kv_read", &Kernels::kv_read},
     {"rd_k_qkv_rope_store", &Kernels::qkv_rope_store},
     {"rd_k_attn_partial", &Kernels::attn_partial},
     {"rd_k_kv_store_i8", &Kernels::kv_store_i8},

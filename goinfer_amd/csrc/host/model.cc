@@ -514,6 +514,30 @@ extern "C" int rd_kv_upload(rd_model *m, int slot, int layer, int base, int n, c
     return RD_OK;
 }
 
+// The host copy of rows a slot holds (decoder/resident/subsystems.go:280-287 SnapshotKV takes one per layer): what the cache
+// stores, widened to f32 the way an attention read sees it.
+extern "C" int rd_kv_download(rd_model *m, int slot, int layer, int base, int n, float *keys, float *vals) {
+    if (!m || !keys || !vals || n <= 0 || base < 0) return RD_ERR_ARG;
+    if (!slot_ok(m, slot) || !layer_ok(m, layer, false)) return RD_ERR_ARG;
+    if (base + n > m->slot_len[(size_t)slot]) {
+        rd_set_error("rd_kv_download: rows %d..%d, slot %d holds %d", base, base + n - 1, slot, m->slot_len[(size_t)slot]);
+        return RD_ERR_ARG;
+    }
+    rd_device *d = m->d;
+    RC(d->use());
+    const rd_model_desc &c = m->desc;
+    const size_t bytes = sizeof(float) * (size_t)n * c.n_kv_heads * c.head_dim;
+    DevBuf K(d), V(d);
+    RC(K.alloc(bytes));
+    RC(V.alloc(bytes));
+    LayerW &l = m->layers[(size_t)layer];
+    RC(d->launch(d->k.kv_read, (unsigned)n, (unsigned)c.n_kv_heads, 1, (unsigned)c.head_dim, (const void *)l.Kp, (const void *)l.Vp, (const float *)l.Ksc,
+                 (const float *)l.Vsc, K.as<float>(), V.as<float>(), (const int *)(m->tables + (size_t)slot * m->blocks_per_slot), base, c.n_kv_heads,
+                 c.head_dim, m->kv_type == RD_KV_I8 ? 1 : 0));
+    RC(d->d2h(keys, K.p, bytes));
+    return d->d2h(vals, V.p, bytes);
+}
+
 extern "C" int rd_kv_truncate(rd_model *m, int slot, int pos) {
     if (!m || !slot_ok(m, slot) || pos < 0) return RD_ERR_ARG;
     m->slot_len[(size_t)slot] = std::min(m->slot_len[(size_t)slot], pos);

@@ -302,6 +302,84 @@ extern "C" int rd_moe_route(rd_device *d, const float *logits, int T, int nE, in
     return d->d2h(wgt, W.p, sizeof(float) * (size_t)T * k);
 }
 
+// ---- the step's q|k|v epilogue on its own: bias, QK-norm, RoPE, and the K/V rows as the cache then holds them ----
+// x: f32 [rows][(n_h + 2 n_kv) * hd], the q|k|v projection outputs of `rows` sequences, row r at position pos[r] of its own
+// one-sequence cache. q_out: f32 [rows][n_h*hd]; k_out, v_out: f32 [rows][n_kv*hd], read back from the cache (f16 widened, or
+// code * scale for the int8 cache). q_norm, k_norm, bias may be null.
+extern "C" int rd_qkv_rope_store(rd_device *d, int kv_type, int rows, const float *x, const int *pos, int n_h, int n_kv, int hd, const double *inv_freq,
+                                 const float *q_norm, const float *k_norm, float eps, const float *bias, float *q_out, float *k_out, float *v_out) {
+    if (!d || !x || !pos || !inv_freq || !q_out || !k_out || !v_out || rows <= 0 || rows > 32) {
+        rd_set_error("rd_qkv_rope_store: bad arguments (1 <= rows <= 32)");
+        return RD_ERR_ARG;
+    }
+    if (n_h <= 0 || n_kv <= 0 || (hd != 64 && hd != 128) || (kv_type != RD_KV_F16 && kv_type != RD_KV_I8)) {
+        rd_set_error("rd_qkv_rope_store declines: head_dim must be 64 or 128");
+        return RD_DECLINED;
+    }
+    int maxPos = 0;
+    for (int r = 0; r < rows; r++) {
+        if (pos[r] < 0) return RD_ERR_ARG;
+        maxPos = std::max(maxPos, pos[r]);
+    }
+    const bool i8 = kv_type == RD_KV_I8;
+    const int bps = maxPos / 64 + 1, Ntot = (n_h + 2 * n_kv) * hd, kvd = n_kv * hd;
+    const size_t nBlocks = (size_t)rows * bps + 1;
+    const size_t poolBytes = nBlocks * n_kv * 64 * hd * (i8 ? 1 : 2), scBytes = nBlocks * n_kv * 64 * sizeof(float);
+    std::vector<int> tab((size_t)rows * bps), slots((size_t)rows);
+    for (size_t i = 0; i < tab.size(); i++) tab[i] = (int)i + 1;
+    for (int r = 0; r < rows; r++) slots[(size_t)r] = r;
+    DevBuf X(d), Q(d), Kp(d), Vp(d), Ksc(d), Vsc(d), T(d), S(d), Pp(d), F(d), QN(d), KN(d), Bi(d), Ko(d), Vo(d);
+    RC(X.alloc(sizeof(float) * (size_t)32 * Ntot));
+    RC(Q.alloc(sizeof(float) * (size_t)rows * n_h * hd));
+    RC(Kp.alloc(poolBytes));
+    RC(Vp.alloc(poolBytes));
+    HIPCHK(MemsetAsync(Kp.p, 0, poolBytes, d->stream));
+    HIPCHK(MemsetAsync(Vp.p, 0, poolBytes, d->stream));
+    RC(Ksc.alloc(scBytes));
+    RC(Vsc.alloc(scBytes));
+    HIPCHK(MemsetAsync(Ksc.p, 0, scBytes, d->stream));
+    HIPCHK(MemsetAsync(Vsc.p, 0, scBytes, d->stream));
+    RC(T.alloc(sizeof(int) * tab.size()));
+    RC(S.alloc(sizeof(int) * (size_t)rows));
+    RC(Pp.alloc(sizeof(int) * (size_t)rows));
+    RC(F.alloc(sizeof(double) * (size_t)(hd / 2)));
+    RC(Ko.alloc(sizeof(float) * (size_t)kvd));
+    RC(Vo.alloc(sizeof(float) * (size_t)kvd));
+    RC(d->h2d(X.p, x, sizeof(float) * (size_t)rows * Ntot));
+    RC(d->h2d(T.p, tab.data(), sizeof(int) * tab.size()));
+    RC(d->h2d(S.p, slots.data(), sizeof(int) * (size_t)rows));
+    RC(d->h2d(Pp.p, pos, sizeof(int) * (size_t)rows));
+    RC(d->h2d(F.p, inv_freq, sizeof(double) * (size_t)(hd / 2)));
+    if (q_norm) {
+        RC(QN.alloc(sizeof(float) * (size_t)hd));
+        RC(d->h2d(QN.p, q_norm, sizeof(float) * (size_t)hd));
+    }
+    if (k_norm) {
+        RC(KN.alloc(sizeof(float) * (size_t)hd));
+        RC(d->h2d(KN.p, k_norm, sizeof(float) * (size_t)hd));
+    }
+    if (bias) {
+        RC(Bi.alloc(sizeof(float) * (size_t)Ntot));
+        RC(d->h2d(Bi.p, bias, sizeof(float) * (size_t)Ntot));
+    }
+    if (i8)
+        RC(d->launch(d->k.qkv_rope_store_i8, (unsigned)(n_h + 2 * n_kv), (unsigned)rows, 1, (unsigned)(hd / 2), (const float *)X.p, 1, Q.as<float>(),
+                     (signed char *)Kp.p, (signed char *)Vp.p, Ksc.as<float>(), Vsc.as<float>(), (const int *)T.p, bps, (const int *)S.p, (const int *)Pp.p,
+                     (const double *)F.p, (const float *)QN.p, (const float *)KN.p, eps, n_h, n_kv, hd, (size_t)0, (const float *)Bi.p));
+    else
+        RC(d->launch(d->k.qkv_rope_store, (unsigned)(n_h + 2 * n_kv), (unsigned)rows, 1, (unsigned)(hd / 2), (const float *)X.p, 1, Q.as<float>(),
+                     (uint16_t *)Kp.p, (uint16_t *)Vp.p, (const int *)T.p, bps, (const int *)S.p, (const int *)Pp.p, (const double *)F.p, (const float *)QN.p,
+                     (const float *)KN.p, eps, n_h, n_kv, hd, (size_t)0, (const float *)Bi.p));
+    RC(d->d2h(q_out, Q.p, sizeof(float) * (size_t)rows * n_h * hd));
+    for (int r = 0; r < rows; r++) {
+        RC(d->launch(d->k.kv_read, 1u, (unsigned)n_kv, 1, (unsigned)hd, (const void *)Kp.p, (const void *)Vp.p, (const float *)Ksc.p, (const float *)Vsc.p,
+                     Ko.as<float>(), Vo.as<float>(), (const int *)((const int *)T.p + (size_t)r * bps), pos[r], n_kv, hd, i8 ? 1 : 0));
+        RC(d->d2h(k_out + (size_t)r * kvd, Ko.p, sizeof(float) * (size_t)kvd));
+        RC(d->d2h(v_out + (size_t)r * kvd, Vo.p, sizeof(float) * (size_t)kvd));
+    }
+    return RD_OK;
+}
+
 // ---- ragged attention over a temporary paged pool (kernel-level entry point) ----
 // nq (optional): sequence i brings nq[i] query rows, its last nq[i] positions; row j of them sees keys 0..len[i]-nq[i]+j.
 static int attn_ragged_typed(rd_device *d, int kv_type, int n_seq, const int *len, const int *nq, const int64_t *off, const float *k, const float *v,

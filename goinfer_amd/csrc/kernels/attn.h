@@ -91,6 +91,29 @@ extern "C" __global__ void rd_k_kv_store(const float *__restrict__ k, const floa
     kv_store_elem(Kp, Vp, HD, region, p, d, k[src], v[src]);
 }
 
+// Rows back out of the cache, widened to f32 exactly as an attention read sees them (the host copy a KV snapshot takes,
+// decoder/resident/subsystems.go:280-287 SnapshotKV): positions base..base+n-1 of one sequence into k,v f32 [n][nKV*HD].
+// f16 cache: the stored binary16 widened; int8 cache: code * scale (linalg.DequantizeRowsInt8Into). Grid (n, nKV), block HD.
+extern "C" __global__ void rd_k_kv_read(const void *__restrict__ KpV, const void *__restrict__ VpV, const float *__restrict__ Ksc,
+                                        const float *__restrict__ Vsc, float *__restrict__ k, float *__restrict__ v, const int *__restrict__ table,
+                                        int base, int nKV, int HD, int i8) {
+    int i = blockIdx.x, kvh = blockIdx.y, d = threadIdx.x;
+    if (d >= HD) return;
+    int pos = base + i, blk = table[pos >> 6], p = pos & 63;
+    size_t region = ((size_t)blk * nKV + kvh) * 64 * HD, dst = ((size_t)i * nKV + kvh) * HD + d;
+    if (i8) {
+        size_t srow = ((size_t)blk * nKV + kvh) * 64 + p;
+        int kc = (int)((const unsigned char *)KpV)[region + k8_index(HD, p, d)] - 128, vc = (int)((const unsigned char *)VpV)[region + v8_index(HD, p, d)] - 128;
+        k[dst] = __fmul_rn((float)kc, Ksc[srow]);
+        v[dst] = __fmul_rn((float)vc, Vsc[srow]);
+    } else {
+        int ki = HD == 128 ? k_elem_index<128>(p, d) : k_elem_index<64>(p, d);
+        int vi = HD == 128 ? v_elem_index<128>(p, d) : v_elem_index<64>(p, d);
+        k[dst] = f16_bits_to_f32(((const uint16_t *)KpV)[region + ki]);
+        v[dst] = f16_bits_to_f32(((const uint16_t *)VpV)[region + vi]);
+    }
+}
+
 // After the q|k|v GEMM: reduce its split-K partials, optional q|k|v bias (Qwen2; decoder/attention.go:12-34 addBias, applied right
 // after the projections, program_cpu_n.go:470-476), optional per-head RMSNorm of q and k (Qwen3, decoder/program_cpu.go:351-364),
 // NeoX RoPE with f64 angles (decoder/rope.go:28-64), q -> f32 buffer, k,v -> this position of the row's sequence in the pool.

@@ -94,6 +94,14 @@ int rd_gemm_q6k(rd_device *d, const void *W, int N, int K, const float *a, int M
 int rd_gemm_w8a8(rd_device *d, const int8_t *q, const float *row_scale, int N, int K, const float *a, int M, float *dst);
 /* int4 group-32 weights with f16 scales x per-32 int8 activations (backend/cuda/actgroup.cu:243-275). */
 int rd_gemm_w4a8(rd_device *d, const uint8_t *nib, const uint16_t *s16, int N, int K, const float *a, int M, float *dst);
+/* The step's q|k|v epilogue on its own (backend/cuda/gemv_fwd.cu:51-101 rope_kv, prefill_batched.cu rope_kv_ragged; CPU:
+ * decoder/attention.go:12-34 addBias, program_cpu.go:351-375 applyQKNorm / applyRope, kvcache.go:21-40,43-52 Append's narrowing):
+ * x: host f32 [rows][(n_h+2*n_kv)*hd], the projections of `rows` (<= 32) sequences, row r at position pos[r] of its own cache.
+ * Adds bias, applies the per-head RMSNorm of q and k (either may be NULL) and NeoX RoPE with f64 angles, and stores k and v into
+ * a cache of kv_type. q_out: f32 [rows][n_h*hd]; k_out, v_out: f32 [rows][n_kv*hd], the stored row read back from the cache
+ * (binary16 narrowed half-up and widened, or code * scale of the int8 cache). */
+int rd_qkv_rope_store(rd_device *d, int kv_type, int rows, const float *x, const int *pos, int n_h, int n_kv, int hd, const double *inv_freq,
+                      const float *q_norm, const float *k_norm, float eps, const float *bias, float *q_out, float *k_out, float *v_out);
 /* Ragged flash-decode attention (backend/cuda/decode_fa.cu fa_partial_ragged/fa_combine_ragged;
  * decoder/forwardn.go:295-500): n_seq sequences, sequence i has len[i] keys; k,v: host f32 [sum len][n_kv*hd]
  * (rows of sequence i start at row off[i]); they are narrowed to binary16 (round-half-up) into a paged pool
@@ -149,6 +157,10 @@ enum { RD_KV_F16 = 0, RD_KV_I8 = 1 };
 int rd_kv_configure_typed(rd_model *m, int slots, int ctx_cap, int kv_type);
 /* keys, vals: host f32 [n][n_kv*hd] for positions base..base+n-1 of `slot`, layer `layer` (already RoPE'd) */
 int rd_kv_upload(rd_model *m, int slot, int layer, int base, int n, const float *keys, const float *vals);
+/* The rows a slot holds, widened to f32 as an attention read sees them (the host copy decoder/resident/subsystems.go:280-287
+ * SnapshotKV takes): positions base..base+n-1 (all below the slot's length) of `layer` into keys, vals: host f32 [n][n_kv*hd].
+ * f16 cache: the stored binary16 values; int8 cache: code * scale. */
+int rd_kv_download(rd_model *m, int slot, int layer, int base, int n, float *keys, float *vals);
 int rd_kv_truncate(rd_model *m, int slot, int pos);
 int rd_kv_reset(rd_model *m, int slot);
 
