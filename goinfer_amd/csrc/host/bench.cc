@@ -133,7 +133,6 @@ extern "C" const char *rd_bench_class_name(int c) {
 //   "gemm_q4k", "gemm_q5k", "gemm_q6k"  args {N, K, M, copies}: dst = a . W^T on `copies` distinct weight copies used round-robin (so the 256 MB
 //               Infinity Cache cannot hold the weights between launches); operands are random bytes with sane f16 scales.
 //   "gateup"    args {I, K, M, copies}: the fused gate|up projection + SwiGLU + quantization kernel.
-//   "barrier"   args {blocks, words, rounds, shift}: the grid-wide barrier with a cross-block data hand-off per round.
 //   "copy"      args {bytes}: a plain 16-byte-per-lane copy kernel over `bytes` (a multiple of 16), the yardstick for
 //               scaling hardware traffic counters and for the practical HBM rate.
 // ms_out[iters]: per-launch milliseconds (HIP events on the launch stream).
@@ -147,10 +146,6 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
     }
     if (nm == "gateup" && n_args >= 4 && (args[0] <= 0 || args[0] % 64 || args[1] <= 0 || args[1] % 256 || args[2] < 1 || args[2] > 64)) {
         rd_set_error("gateup bench: bad shape");
-        return RD_ERR_ARG;
-    }
-    if (nm == "barrier" && n_args >= 4 && (args[0] < 1 || args[0] > 256 || args[1] < 1 || args[1] > (1 << 20) || args[2] < 1 || args[2] > 100000)) {
-        rd_set_error("barrier bench: blocks 1..256, words 1..2^20, rounds 1..100000");
         return RD_ERR_ARG;
     }
     if (nm == "copy" && n_args >= 1 && (args[0] <= 0 || args[0] % 16)) {
@@ -236,37 +231,6 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
         }
         if (!rc) rc = d->sync();
         for (auto &w : ws) free_weight(d, &w);
-    } else if (nm == "barrier" && n_args >= 4) {
-        // args {blocks, words, rounds, shift[, mode]}: the grid barrier's cost and its cross-block hand-off; ms_out per launch, and the launch
-        // fails with RD_ERR_STATE if a hand-off delivered stale data or the barrier gave up
-        int blocks = (int)args[0], words = (int)args[1], rounds = (int)args[2], shift = (int)args[3], mode = n_args > 4 ? (int)args[4] : 0;
-        const size_t ctrBytes = 128 * 12; // flag, eight group counters, top counter, abort flag: one 128-byte line each
-        DevBuf ctr(d), buf(d), out(d);
-        rc = ctr.alloc(ctrBytes);
-        if (!rc) rc = buf.alloc(sizeof(float) * (size_t)blocks * words);
-        if (!rc) rc = out.alloc(sizeof(int) * (size_t)blocks);
-        for (int i = 0; i < warmup + iters && !rc; i++) {
-            rc = rd_hip_ok(d->hip, d->hip->MemsetAsync(ctr.p, 0, ctrBytes, d->stream), "memset") ? RD_OK : RD_ERR_HIP;
-            if (!rc) rc = rd_hip_ok(d->hip, d->hip->MemsetAsync(out.p, 0, sizeof(int) * (size_t)blocks, d->stream), "memset") ? RD_OK : RD_ERR_HIP;
-            if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup)], d->stream);
-            if (!rc)
-                rc = d->launch(d->k.barrier_probe, (unsigned)blocks, 1, 1, 256, ctr.as<unsigned>(), ctr.as<unsigned>() + 32 * 11, buf.as<float>(), words, rounds,
-                               shift, 200000u, out.as<int>(), mode);
-            if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup) + 1], d->stream);
-        }
-        if (!rc) rc = d->sync();
-        if (!rc) {
-            std::vector<int> h((size_t)blocks);
-            unsigned flag[32 * 12];
-            rc = d->d2h(h.data(), out.p, sizeof(int) * (size_t)blocks);
-            if (!rc) rc = d->d2h(flag, ctr.p, ctrBytes);
-            long bad = 0;
-            for (int v : h) bad += v;
-            if (!rc && (bad || flag[32 * 11])) {
-                rd_set_error("barrier probe: %ld stale hand-offs, abort flag %u", bad, flag[32 * 11]);
-                rc = RD_ERR_STATE;
-            }
-        }
     } else if (nm == "copy" && n_args >= 1) {
         size_t bytes = (size_t)args[0];
         DevBuf A(d), Bf(d);

@@ -121,7 +121,6 @@ static const KName kNames[] = {
     {"rd_k_moe_fold", &Kernels::moe_fold},
     {"rd_k_embed_rows", &Kernels::embed_rows},
     {"rd_k_copy16", &Kernels::copy16},
-    {"rd_k_barrier_probe", &Kernels::barrier_probe},
     {"rd_k_unpanel_q4k", &Kernels::unpanel_q4k},
     {"rd_k_fill_f16", &Kernels::fill_f16},
     {"rd_k_fill_f32", &Kernels::fill_f32},

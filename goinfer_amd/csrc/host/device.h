@@ -29,7 +29,7 @@ struct Kernels {
     hipFunction_t gemm_q4k_gateup;
     hipFunction_t kv_store, kv_read, qkv_rope_store, attn_partial, attn_combine, attn_combine_quant;
     hipFunction_t kv_store_i8, qkv_rope_store_i8, attn_partial_i8, attn_partial_rows, attn_partial_rows_i8, attn_partial_deep, attn_partial_deep_i8, topk_rows, topk_hist, topk_pick, topk_finish;
-    hipFunction_t rmsnorm, rope, argmax_rows, argmax_final, matmul_f32, moe_route, gemm_w4a8_moe, gemm_w4a8_moe_gateup, moe_swiglu_quant, moe_fold, embed_rows, copy16, barrier_probe, unpanel_q4k, fill_f16, fill_f32;
+    hipFunction_t rmsnorm, rope, argmax_rows, argmax_final, matmul_f32, moe_route, gemm_w4a8_moe, gemm_w4a8_moe_gateup, moe_swiglu_quant, moe_fold, embed_rows, copy16, unpanel_q4k, fill_f16, fill_f32;
 };
 
 struct rd_device {

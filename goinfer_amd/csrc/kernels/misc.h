@@ -292,86 +292,3 @@ extern "C" __global__ void rd_k_fill_f16(uint16_t *__restrict__ dst, size_t n, u
 extern "C" __global__ void rd_k_fill_f32(float *__restrict__ dst, size_t n, unsigned seed) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) dst[i] = fill_value(i, seed);
 }
-
-// ---- grid-wide barrier for kernels whose blocks are all resident at once (grid <= CUs, one block per CU) ----
-// Arrive with an agent-scope release (the compiler writes this XCD's dirty L2 lines back), wait on the shared counter with
-// relaxed agent-scope polls and one acquire fence at the end (which invalidates this XCD's stale lines): data written before the barrier by any block is
-// visible after it to every block, whatever XCD it runs on. The wait is bounded: after `spin_limit` polls the block sets
-// *abort_flag and gives up, and every later barrier call returns at once, so a block that can never be joined (a grid that
-// is not co-resident, a fault elsewhere) still lets every wave reach its end. Returns false once aborted.
-// `target` is the counter value that means "everyone arrived": the caller adds gridDim.x per barrier.
-__device__ __forceinline__ bool grid_barrier(unsigned *counter, unsigned target, unsigned *abort_flag, unsigned spin_limit) {
-    __shared__ unsigned s_ok;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        unsigned ok = 1;
-        __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-        unsigned spins = 0;
-        while ((int)(__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - target) < 0) {
-            if (++spins > spin_limit || __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) {
-                __hip_atomic_store(abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                ok = 0;
-                break;
-            }
-            __builtin_amdgcn_s_sleep(2);
-        }
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-        s_ok = ok;
-    }
-    __syncthreads();
-    return s_ok != 0;
-}
-
-// The same barrier with two-level arrival: blocks arrive on one of eight counters (by block index modulo 8, each on its own
-// 128-byte line), the last arrival of a group arrives on a top counter, the last group publishes the generation in a flag
-// that everyone polls. Arrivals on one address serialise at the memory side (about 40 ns each), so eight short queues and
-// one of eight beat one queue of 256. ctr: [0] flag, [32*(1+g)] group g, [32*9] top; gen counts barriers from 0.
-__device__ __forceinline__ bool grid_barrier2(unsigned *ctr, unsigned gen, unsigned *abort_flag, unsigned spin_limit) {
-    __shared__ unsigned s_ok2;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        const unsigned nb = gridDim.x, g = blockIdx.x & 7u, gsize = (nb - g + 7u) >> 3, ngroups = nb < 8u ? nb : 8u;
-        unsigned ok = 1;
-        unsigned old = __hip_atomic_fetch_add(ctr + 32 * (1 + g), 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-        if (old + 1 == gsize * (gen + 1)) {
-            unsigned o2 = __hip_atomic_fetch_add(ctr + 32 * 9, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-            if (o2 + 1 == ngroups * (gen + 1)) __hip_atomic_store(ctr, gen + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        unsigned spins = 0;
-        while ((int)(__hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) - (gen + 1)) < 0) {
-            if (++spins > spin_limit || __hip_atomic_load(abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) {
-                __hip_atomic_store(abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                ok = 0;
-                break;
-            }
-            __builtin_amdgcn_s_sleep(4);
-        }
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-        s_ok2 = ok;
-    }
-    __syncthreads();
-    return s_ok2 != 0;
-}
-
-// Measures the barrier: `iters` rounds in which every block writes `words` floats of its own slice of buf, crosses the
-// barrier, and sums the slice of the block `shift` places on (written by someone else, usually on another XCD). out[block]
-// receives the number of wrong sums (0 when the hand-off works). Grid <= number of CUs, block 256.
-// mode 0: the one-counter barrier; mode 1: the two-level one (counter then points at its ten-line block).
-extern "C" __global__ __launch_bounds__(256) void rd_k_barrier_probe(unsigned *counter, unsigned *abort_flag, float *buf, int words, int iters,
-                                                                      int shift, unsigned spin_limit, int *out, int mode) {
-    const int nb = gridDim.x, b = blockIdx.x, peer = (b + shift) % nb;
-    int wrong = 0;
-    unsigned target = 0;
-    for (int it = 0; it < iters; it++) {
-        for (int i = threadIdx.x; i < words; i += blockDim.x) buf[(size_t)b * words + i] = (float)(it + b + (i & 7));
-        target += nb;
-        if (!(mode ? grid_barrier2(counter, (unsigned)(2 * it), abort_flag, spin_limit) : grid_barrier(counter, target, abort_flag, spin_limit))) break;
-        float sum = 0.f;
-        for (int i = threadIdx.x; i < words; i += blockDim.x) sum += buf[(size_t)peer * words + i] - (float)(it + peer + (i & 7));
-        if (sum != 0.f) wrong++;
-        target += nb;
-        if (!(mode ? grid_barrier2(counter, (unsigned)(2 * it + 1), abort_flag, spin_limit) : grid_barrier(counter, target, abort_flag, spin_limit)))
-            break; // readers done before the next round overwrites
-    }
-    if (wrong) atomicAdd(&out[b], wrong);
-}
