@@ -2,6 +2,7 @@
 
   rocmdecode_gfx950.hsaco   the gfx950 code object (hipcc --genco, cross-compiles without a GPU)
   librocmdecode.so          the C-ABI host library (g++; binds libamdhip64 at run time with dlopen)
+  librocmdecode_static.so   the allocation-free top-K entry point (hipcc; links the HIP runtime; opened by the library above)
 """
 import os
 import subprocess
@@ -37,6 +38,21 @@ def build_host(verbose=False):
     return SO
 
 
+STATIC_SO = os.path.join(LIB, "librocmdecode_static.so")
+
+
+def build_static(verbose=False):
+    """The allocation-free entry point's library: one hipcc translation unit (host and gfx950 device code) that links the HIP runtime."""
+    os.makedirs(LIB, exist_ok=True)
+    src = os.path.join(HERE, "csrc", "static", "topk_static.hip")
+    cmd = [os.path.join(ROCM, "bin", "hipcc"), "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-o", STATIC_SO, src]
+    if verbose:
+        print(" ".join(cmd))
+    subprocess.check_call(cmd)
+    return STATIC_SO
+
+
 SYNTH = os.path.join(LIB, "libgoinfer_synth.so")
 
 
@@ -51,7 +67,7 @@ def build_synth(verbose=False):
 
 
 def build_all(verbose=False):
-    return build_kernels(verbose), build_host(verbose), build_synth(verbose)
+    return build_kernels(verbose), build_host(verbose), build_static(verbose), build_synth(verbose)
 
 
 if __name__ == "__main__":

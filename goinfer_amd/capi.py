@@ -25,7 +25,7 @@ EXPORTS = [
     "rd_step_batch_draw", "rd_sample_rows", "rd_greedy_chain_start", "rd_greedy_chain_next", "rd_sample_chain_start",
     "rd_sample_chain_next", "rd_greedy_chain_stop",
     "rd_dequant_q5k", "rd_dequant_q6k", "rd_gemm_q5k", "rd_gemm_q6k", "rd_model_upload_q5k", "rd_model_upload_q6k",
-    "rd_kv_download", "rd_qkv_rope_store",
+    "rd_kv_download", "rd_qkv_rope_store", "rd_topk_rows_static",
 ]
 
 

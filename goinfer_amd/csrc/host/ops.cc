@@ -6,6 +6,7 @@
 #include <cmath>
 #include <numeric>
 #include <string.h>
+#include <string>
 
 #define RC(x)                \
     do {                     \
@@ -528,6 +529,52 @@ extern "C" int rd_topk_rows(rd_device *d, const float *logits, int rows, int V, 
     RC(d->d2h(vals, Vv.p, sizeof(float) * (size_t)rows * k));
     if (want_z) RC(d->d2h(z, Z.p, sizeof(double) * (size_t)rows));
     return RD_OK;
+}
+
+// ---- the same reduction with nothing allocated: forwards to librocmdecode_static.so ----
+// That library (csrc/static/topk_static.hip, built by hipcc) keeps the scratch between the launches in a file-scope device array
+// and links the HIP runtime; it sits beside this one and is opened on the first call, so this library itself still binds
+// libamdhip64 only at run time.
+#include <dlfcn.h>
+#include <mutex>
+typedef int (*topk_static_fn)(int, void *, const float *, int, int, int, double, int, int *, float *, double *, char *, size_t);
+static topk_static_fn load_topk_static(std::string *why) {
+    static std::once_flag once;
+    static topk_static_fn fn = nullptr;
+    static std::string err;
+    std::call_once(once, [] {
+        std::string path = "librocmdecode_static.so";
+        Dl_info info;
+        if (dladdr((void *)&rd_plan_gemm, &info) && info.dli_fname) {
+            std::string p = info.dli_fname;
+            size_t s = p.find_last_of('/');
+            path = (s == std::string::npos ? std::string(".") : p.substr(0, s)) + "/librocmdecode_static.so";
+        }
+        if (const char *e = getenv("ROCMDECODE_STATIC_LIB")) path = e;
+        void *h = dlopen(path.c_str(), RTLD_NOW | RTLD_LOCAL);
+        if (!h) {
+            err = std::string("cannot load ") + path + ": " + dlerror();
+            return;
+        }
+        fn = (topk_static_fn)dlsym(h, "rd_topk_rows_static_impl");
+        if (!fn) err = path + " lacks rd_topk_rows_static_impl";
+    });
+    if (!fn && why) *why = err;
+    return fn;
+}
+
+extern "C" int rd_topk_rows_static(int device, void *stream, const float *logits_dev, int rows, int V, int k, double temperature, int want_z,
+                                   int *ids_dev, float *vals_dev, double *z_dev) {
+    std::string why;
+    topk_static_fn fn = load_topk_static(&why);
+    if (!fn) {
+        rd_set_error("rd_topk_rows_static: %s", why.c_str());
+        return RD_ERR_STATE;
+    }
+    char msg[400] = "";
+    int rc = fn(device, stream, logits_dev, rows, V, k, temperature, want_z, ids_dev, vals_dev, z_dev, msg, sizeof msg);
+    if (rc) rd_set_error("%s", msg);
+    return rc;
 }
 
 // ---- host planning without a device ----
