@@ -20,7 +20,9 @@ def build_kernels(verbose=False):
     os.makedirs(LIB, exist_ok=True)
     src = os.path.join(HERE, "csrc", "kernels", "rocmdecode.hip")
     cmd = [os.path.join(ROCM, "bin", "hipcc"), "--genco", "--offload-arch=gfx950", "-O3", "-std=c++17",
-           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-o", HSACO, src]
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           # MFMA results that the VALU reads next (the int8 dots before their f32 fold) stay in ordinary VGPRs
+           "-mllvm", "-amdgpu-mfma-vgpr-form=1", "-o", HSACO, src]
     if verbose:
         print(" ".join(cmd))
     subprocess.check_call(cmd)

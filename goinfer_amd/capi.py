@@ -25,7 +25,7 @@ EXPORTS = [
     "rd_step_batch_draw", "rd_sample_rows", "rd_greedy_chain_start", "rd_greedy_chain_next", "rd_sample_chain_start",
     "rd_sample_chain_next", "rd_greedy_chain_stop",
     "rd_dequant_q5k", "rd_dequant_q6k", "rd_gemm_q5k", "rd_gemm_q6k", "rd_model_upload_q5k", "rd_model_upload_q6k",
-    "rd_kv_download", "rd_qkv_rope_store", "rd_topk_rows_static",
+    "rd_kv_download", "rd_qkv_rope_store", "rd_topk_rows_static", "rd_quant_act",
 ]
 
 
@@ -259,6 +259,16 @@ class Device:
         check(lib().rd_qkv_rope_store(self.h, 0 if kv == "f16" else 1, rows, _p(x), _p(pos), n_h, n_kv, hd, _p(inv), _p(qn), _p(kn), C.c_float(eps),
                                       _p(bi), _p(q), _p(k), _p(v)), "rd_qkv_rope_store")
         return q, k, v
+
+    def quant_act(self, a):
+        """Per-32 int8 quantization of rows a [M][K]: (codes int8 [M][K], scales f32 [M][K/32], sums f32 [M][K/32])."""
+        a = _f32(a)
+        M, K = a.shape
+        codes = np.empty((M, K), np.int8)
+        scales = np.empty((M, K // 32), np.float32)
+        sums = np.empty((M, K // 32), np.float32)
+        check(lib().rd_quant_act(self.h, _p(a), M, K, _p(codes), _p(scales), _p(sums)), "rd_quant_act")
+        return codes, scales, sums
 
     def moe_route(self, logits, k, norm):
         logits = _f32(logits)

@@ -175,24 +175,24 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
         std::vector<DevWeight> ws((size_t)copies);
         for (auto &w : ws)
             if (!rc) rc = kind == 0 ? upload_q4k(d, raw.data(), N, K, &w) : (kind == 3 ? upload_q5k(d, raw.data(), N, K, &w) : upload_q6k(d, raw.data(), N, K, &w));
-        DevBuf Xp(d), P(d);
-        size_t pb = kind == 4 ? (size_t)(K / 128) * LIN_PANEL_BYTES : (size_t)(K / 256) * Q4K_PANEL_BYTES;
+        DevBuf Xp(d), P(d), X(d);
+        const int pkind = kind == 0 ? PANEL_A8 : (kind == 3 ? PANEL_Q4K : PANEL_LIN);
+        size_t pb = kind == 0 ? a8_bytes(K) : (kind == 4 ? (size_t)(K / 128) * LIN_PANEL_BYTES : (size_t)(K / 256) * Q4K_PANEL_BYTES);
         const int tiles = (M + 31) / 32; // rows beyond 32 are further M-tiles, each with its own panels and partial sums
         if (!rc) rc = Xp.alloc(pb * tiles);
         int nKB = K / kblock_of(kind);
         GemmPlan plan = plan_gemm(kind, N, nKB);
         const size_t pStride = (size_t)plan.splits * 32 * N;
         if (!rc) rc = P.alloc(sizeof(float) * pStride * tiles);
-        if (!rc) {
-            std::vector<uint16_t> x(pb * tiles / 2);
-            for (size_t i = 0; i < x.size(); i++) x[i] = (uint16_t)(0x3000 + (i * 2654435761u >> 22 & 0x3ff)) | (uint16_t)((i & 1) << 15);
-            rc = d->h2d(Xp.p, x.data(), pb * tiles);
-        }
+        if (!rc) rc = X.alloc(sizeof(float) * (size_t)32 * K);
+        if (!rc) rc = d->launch(d->k.fill_f32, 256, 1, 1, 256, X.as<float>(), (size_t)32 * K, 7u); // the same 32 rows for every M-tile
+        for (int t = 0; t < tiles && !rc; t++)
+            rc = d->launch(d->k.quant_act, (unsigned)((K + 255) / 256), 32u, 1, 256, (const float *)X.p, (uint8_t *)Xp.p + (size_t)t * pb, K, pkind);
         if (!rc) rc = d->sync();
         for (int i = 0; i < warmup + iters && !rc; i++) {
             const DevWeight &w = ws[(size_t)i % ws.size()];
             if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup)], d->stream);
-            rc = launch_gemm_wide(d, w, Xp.p, pb, P.as<float>(), pStride, M, nullptr); // M-tiles of 32 rows; Q4_K reads its weights once for all of them
+            rc = launch_gemm_wide(d, w, Xp.p, pb, P.as<float>(), pStride, M, nullptr); // M-tiles of 32 rows
             if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup) + 1], d->stream);
         }
         if (!rc) rc = d->sync();
@@ -211,22 +211,19 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
         std::vector<DevWeight> ws((size_t)copies);
         for (auto &w : ws)
             if (!rc) rc = upload_q4k(d, raw.data(), 2 * I, K, &w);
-        DevBuf Xp(d), Xo(d);
-        size_t pb = (size_t)(K / 256) * Q4K_PANEL_BYTES;
-        if (!rc) rc = Xp.alloc(pb);
-        if (!rc) rc = Xo.alloc((size_t)((I + 255) / 256) * Q4K_PANEL_BYTES);
-        if (!rc) {
-            std::vector<uint16_t> x(pb / 2);
-            for (size_t i = 0; i < x.size(); i++) x[i] = (uint16_t)(0x3000 + (i * 2654435761u >> 22 & 0x3ff)) | (uint16_t)((i & 1) << 15);
-            rc = d->h2d(Xp.p, x.data(), pb);
-        }
+        DevBuf Xp(d), Xo(d), X(d);
+        if (!rc) rc = Xp.alloc(a8_bytes(K));
+        if (!rc) rc = Xo.alloc(a8_bytes(I));
+        if (!rc) rc = X.alloc(sizeof(float) * (size_t)32 * K);
+        if (!rc) rc = d->launch(d->k.fill_f32, 256, 1, 1, 256, X.as<float>(), (size_t)32 * K, 7u);
+        if (!rc) rc = d->launch(d->k.quant_act, (unsigned)((K + 255) / 256), 32u, 1, 256, (const float *)X.p, (uint8_t *)Xp.p, K, (int)PANEL_A8);
         if (!rc) rc = d->sync();
         for (int i = 0; i < warmup + iters && !rc; i++) {
             const DevWeight &w = ws[(size_t)i % ws.size()];
             if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup)], d->stream);
             for (int m0 = 0; m0 < M && !rc; m0 += 32)
-                rc = d->launch(d->k.gemm_q4k_gateup, (unsigned)(I / 64), 1, 1, GATEUP_THREADS, (const void *)w.tiled, (const void *)Xp.p, Xo.as<uint8_t>(),
-                               (int)PANEL_Q4K, I, K / 256, std::min(32, M - m0));
+                rc = d->launch(d->k.gemm8_q4k_gateup, (unsigned)(I / 32), 1, 1, GATEUP_THREADS, (const void *)w.tiled, (const void *)Xp.p, Xo.as<uint8_t>(),
+                               (int)PANEL_A8, I, K / 256, std::min(32, M - m0));
             if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup) + 1], d->stream);
         }
         if (!rc) rc = d->sync();
@@ -288,12 +285,13 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
         // block without in dispatch order; `bitmap`: the kernel gets the active-expert bitmap and orders the grid itself); int4 group-32 weights of arbitrary bits, `copies` weight sets used round-robin.
         int N = (int)args[0], K = (int)args[1], nE = (int)args[2], active = (int)args[3], T = (int)args[4], perE = (int)args[5];
         int copies = (int)std::max<int64_t>(1, args[6]);
-        if (N <= 0 || N % 32 || K <= 0 || K % 128 || nE < 1 || nE > 256 || active < 0 || active > nE || T < 1 || T > 32) {
+        if (N <= 0 || N % 32 || K <= 0 || K % 32 || nE < 1 || nE > 256 || active < 0 || active > nE || T < 1 || T > 32) {
             rd_set_error("moe_gemm bench: bad shape");
             rc = RD_ERR_ARG;
         }
-        const size_t wStride = (size_t)(N / 32) * (K / 128) * 2304, wBytes = wStride * nE;
-        const size_t xpStride = (size_t)(K / 128) * LIN_PANEL_BYTES;
+        const int nKB = (K + 255) / 256;
+        const size_t wStride = (size_t)(N / 32) * nKB * 4608, wBytes = wStride * nE;
+        const size_t xpStride = a8_bytes(K);
         DevBuf W(d), Xp(d), R(d), O(d), Bits(d);
         if (!rc) rc = W.alloc(wBytes * copies);
         if (!rc) rc = Xp.alloc(xpStride * (perE ? nE : 1));
@@ -316,8 +314,8 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
         for (int i = 0; i < warmup + iters && !rc; i++) {
             const uint8_t *w = (const uint8_t *)W.p + (size_t)(i % copies) * wBytes;
             if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup)], d->stream);
-            rc = d->launch(d->k.gemm_w4a8_moe, (unsigned)((N + 127) / 128), (unsigned)nE, 1, GEMM_THREADS, (const void *)w, wStride, (const void *)Xp.p,
-                           perE ? xpStride : (size_t)0, O.as<float>(), N, K / 128, T, 1, (const signed char *)R.p, nE,
+            rc = d->launch(d->k.gemm8_w4a8_moe, (unsigned)((N + 63) / 64), (unsigned)nE, 1, MOE_THREADS, (const void *)w, wStride, (const void *)Xp.p,
+                           perE ? xpStride : (size_t)0, O.as<float>(), N, nKB, T, 1, (const signed char *)R.p, nE,
                            (n_args >= 9 && args[8]) ? (const unsigned *)Bits.p : (const unsigned *)nullptr);
             if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup) + 1], d->stream);
         }

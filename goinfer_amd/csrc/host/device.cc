@@ -73,19 +73,18 @@ struct KName {
 };
 static const KName kNames[] = {
     {"rd_k_dequant_q4k", &Kernels::dequant_q4k},
-    {"rd_k_retile_q4k", &Kernels::retile_q4k},
-    {"rd_k_gemm_q4k", &Kernels::gemm_q4k},
-    {"rd_k_gemm_q4k_gateup", &Kernels::gemm_q4k_gateup},
     {"rd_k_quant_act", &Kernels::quant_act},
     {"rd_k_reduce_splits", &Kernels::reduce_splits},
     {"rd_k_add_rmsnorm_quant", &Kernels::add_rmsnorm_quant},
     {"rd_k_swiglu_quant", &Kernels::swiglu_quant},
-    {"rd_k_retile_w8a8", &Kernels::retile_w8a8},
-    {"rd_k_gemm_w8a8", &Kernels::gemm_w8a8},
-    {"rd_k_retile_w4a8", &Kernels::retile_w4a8},
-    {"rd_k_gemm_w4a8", &Kernels::gemm_w4a8},
-    {"rd_k_gemm_q4k_wide", &Kernels::gemm_q4k_wide},
-    {"rd_k_gemm_q4k_wide2", &Kernels::gemm_q4k_wide2},
+    {"rd_k_unpack_act8", &Kernels::unpack_act8},
+    {"rd_k_unpanel_a8", &Kernels::unpanel_a8},
+    {"rd_k_retile_w8a8_8", &Kernels::retile_w8a8_8},
+    {"rd_k_retile_w4a8_8", &Kernels::retile_w4a8_8},
+    {"rd_k_gemm8_q4k_gateup", &Kernels::gemm8_q4k_gateup},
+    {"rd_k_gemm8_w4a8_moe", &Kernels::gemm8_w4a8_moe},
+    {"rd_k_gemm8_w4a8_moe_gateup", &Kernels::gemm8_w4a8_moe_gateup},
+    {"rd_k_retile_q4k8", &Kernels::retile_q4k8},
     {"rd_k_dequant_q5k", &Kernels::dequant_q5k},
     {"rd_k_retile_q5k", &Kernels::retile_q5k},
     {"rd_k_gemm_q5k", &Kernels::gemm_q5k},
@@ -115,8 +114,6 @@ static const KName kNames[] = {
     {"rd_k_topk_hist", &Kernels::topk_hist},
     {"rd_k_topk_pick", &Kernels::topk_pick},
     {"rd_k_topk_finish", &Kernels::topk_finish},
-    {"rd_k_gemm_w4a8_moe", &Kernels::gemm_w4a8_moe},
-    {"rd_k_gemm_w4a8_moe_gateup", &Kernels::gemm_w4a8_moe_gateup},
     {"rd_k_moe_swiglu_quant", &Kernels::moe_swiglu_quant},
     {"rd_k_moe_fold", &Kernels::moe_fold},
     {"rd_k_embed_rows", &Kernels::embed_rows},
@@ -158,6 +155,20 @@ static int open_common(int ordinal, const void *image, rd_device **out) {
         }
         d->k.*(kn.slot) = f;
     }
+    static const char *kindName[3] = {"q4k", "w8a8", "w4a8"};
+    static const int kwOf[3] = {2, 4, 8};
+    for (int kind = 0; kind < 3; kind++)
+        for (int i = 0; i < 3; i++) {
+            char name[64];
+            snprintf(name, sizeof name, "rd_k_gemm8_%s_kw%d", kindName[kind], kwOf[i]);
+            if (hip->ModuleGetFunction(&d->k.gemm8[kind][i], d->module, name) != hipSuccess) {
+                rd_set_error("code object lacks kernel %s", name);
+                (void)hip->ModuleUnload(d->module);
+                (void)hip->StreamDestroy(d->stream);
+                delete d;
+                return RD_ERR_HIP;
+            }
+        }
     *out = d;
     return RD_OK;
 }
@@ -270,11 +281,25 @@ bool build_attn_worklist(const int *len, const int *slot, int G, int rows, int n
 }
 
 // ---- GEMM planning ----
-// Split K so that about one block per CU is in flight: fewer blocks leave CUs (and their share of the memory system's
-// outstanding requests) idle, more splits only add partial-sum traffic. A split keeps at least two K-blocks.
+// f16-MFMA kinds (Q5_K, Q6_K): split K so that about one block per CU is in flight; a split keeps at least two K-blocks.
+// int8-MFMA kinds: enough waves to give every SIMD about two; K is cut inside the block first (KW waves per tile, their partial
+// sums folded in LDS, nothing through memory) and across blocks only when eight waves per tile still leave SIMDs idle.
+// The plan depends on the weight's shape only, never on the number of rows: a row is summed in the same order in any batch.
 GemmPlan plan_gemm(int kind, int N, int nKB) {
-    (void)kind;
     GemmPlan p;
+    if (is_gemm8_kind(kind)) {
+        const int tiles = (N + 31) / 32;
+        int want = (2048 + tiles - 1) / tiles; // waves per tile for two per SIMD
+        want = std::min(want, std::max(1, nKB));
+        p.kw = want >= 8 ? 8 : (want >= 4 ? 4 : 2);
+        p.splits = 1;
+        if (p.kw == 8) p.splits = std::max(1, std::min(want / 8, nKB / 8)); // every wave keeps at least one K-block
+        if (const char *e = getenv("ROCMDECODE_GEMM8_KW")) p.kw = atoi(e) == 8 ? 8 : (atoi(e) == 2 ? 2 : 4);
+        if (const char *e = getenv("ROCMDECODE_GEMM8_SPLITS")) p.splits = std::max(1, std::min(atoi(e), nKB));
+        p.kbPerSplit = (nKB + p.splits - 1) / p.splits;
+        p.splits = (nKB + p.kbPerSplit - 1) / p.kbPerSplit;
+        return p;
+    }
     int groups = (N + 127) / 128;
     int target = 256;
     if (const char *e = getenv("ROCMDECODE_GEMM_BLOCKS")) target = atoi(e) > 0 ? atoi(e) : target;
@@ -288,8 +313,11 @@ GemmPlan plan_gemm(int kind, int N, int nKB) {
     return p;
 }
 
-size_t panel_bytes_for(const DevWeight &w) { return kblock_of(w.kind) == 256 ? (size_t)(w.K / 256) * Q4K_PANEL_BYTES : (size_t)(w.K / 128) * LIN_PANEL_BYTES; }
-int panel_kind_for(const DevWeight &w) { return kblock_of(w.kind) == 256 ? PANEL_Q4K : (w.kind == 2 ? PANEL_LIN4 : PANEL_LIN); }
+size_t panel_bytes_for(const DevWeight &w) {
+    if (is_gemm8_kind(w.kind)) return a8_bytes(w.K);
+    return w.kind == 3 ? (size_t)(w.K / 256) * Q4K_PANEL_BYTES : (size_t)(w.K / 128) * LIN_PANEL_BYTES;
+}
+int panel_kind_for(const DevWeight &w) { return is_gemm8_kind(w.kind) ? PANEL_A8 : (w.kind == 3 ? PANEL_Q4K : PANEL_LIN); }
 
 int upload_q4k(rd_device *d, const void *blocks, int N, int K, DevWeight *w) {
     if (N <= 0 || K <= 0 || K % 256 || N % 32) {
@@ -303,7 +331,7 @@ int upload_q4k(rd_device *d, const void *blocks, int N, int K, DevWeight *w) {
     if ((rc = d->alloc(&w->tiled, bytes))) return rc;
     if ((rc = d->h2d(raw.p, blocks, bytes))) return rc;
     int nSB = K / 256;
-    if ((rc = d->launch(d->k.retile_q4k, N / 32, nSB, 1, 320, (const void *)raw.p, w->tiled, N, nSB))) return rc;
+    if ((rc = d->launch(d->k.retile_q4k8, N / 32, nSB, 1, 320, (const void *)raw.p, w->tiled, N, nSB))) return rc;
     if ((rc = d->sync())) return rc;
     w->kind = 0, w->N = N, w->K = K;
     return RD_OK;
@@ -348,36 +376,38 @@ int upload_q6k(rd_device *d, const void *blocks, int N, int K, DevWeight *w) {
 }
 
 int upload_w8a8(rd_device *d, const int8_t *q, const float *row_scale, int N, int K, DevWeight *w) {
-    if (N <= 0 || K <= 0 || K % 128 || N % 32) {
-        rd_set_error("w8a8 upload: N=%d must be a multiple of 32 and K=%d of 128", N, K);
+    if (N <= 0 || K <= 0 || K % 32 || N % 32) {
+        rd_set_error("w8a8 upload: N=%d and K=%d must be multiples of 32", N, K);
         return RD_DECLINED;
     }
     size_t bytes = (size_t)N * K;
+    const int nKB = (K + 255) / 256;
     DevBuf raw(d);
     int rc = raw.alloc(bytes);
     if (rc) return rc;
-    if ((rc = d->alloc(&w->tiled, bytes))) return rc;
+    if ((rc = d->alloc(&w->tiled, (size_t)(N / 32) * nKB * 8192))) return rc;
     if ((rc = d->alloc(&w->scales, sizeof(float) * (size_t)N))) return rc;
     if ((rc = d->h2d(raw.p, q, bytes))) return rc;
     if ((rc = d->h2d(w->scales, row_scale, sizeof(float) * (size_t)N))) return rc;
-    if ((rc = d->launch(d->k.retile_w8a8, N / 32, K / 128, 1, 256, (const void *)raw.p, w->tiled, N, K))) return rc;
+    if ((rc = d->launch(d->k.retile_w8a8_8, N / 32, nKB, 1, 512, (const void *)raw.p, w->tiled, N, K))) return rc;
     if ((rc = d->sync())) return rc;
     w->kind = 1, w->N = N, w->K = K;
     return RD_OK;
 }
 
 int upload_w4a8(rd_device *d, const uint8_t *nib, const uint16_t *s16, int N, int K, DevWeight *w) {
-    if (N <= 0 || K <= 0 || K % 128 || N % 32) {
-        rd_set_error("w4a8 upload: N=%d must be a multiple of 32 and K=%d of 128", N, K);
+    if (N <= 0 || K <= 0 || K % 32 || N % 32) {
+        rd_set_error("w4a8 upload: N=%d and K=%d must be multiples of 32", N, K);
         return RD_DECLINED;
     }
     size_t nb = (size_t)N * K / 2, sb = (size_t)N * (K / 32) * 2;
+    const int nKB = (K + 255) / 256;
     DevBuf raw(d), rs(d);
     int rc;
     if ((rc = raw.alloc(nb)) || (rc = rs.alloc(sb))) return rc;
-    if ((rc = d->alloc(&w->tiled, nb + sb))) return rc;
+    if ((rc = d->alloc(&w->tiled, (size_t)(N / 32) * nKB * 4608))) return rc;
     if ((rc = d->h2d(raw.p, nib, nb)) || (rc = d->h2d(rs.p, s16, sb))) return rc;
-    if ((rc = d->launch(d->k.retile_w4a8, N / 32, K / 128, 1, 320, (const void *)raw.p, (const void *)rs.p, w->tiled, N, K))) return rc;
+    if ((rc = d->launch(d->k.retile_w4a8_8, N / 32, nKB, 1, 320, (const void *)raw.p, (const void *)rs.p, w->tiled, N, K))) return rc;
     if ((rc = d->sync())) return rc;
     w->kind = 2, w->N = N, w->K = K;
     return RD_OK;
@@ -390,47 +420,41 @@ void free_weight(rd_device *d, DevWeight *w) {
     *w = DevWeight();
 }
 
-int launch_gemm(rd_device *d, const DevWeight &w, const void *Xp, float *P, int M, GemmPlan *plan_out, int ldP, int splits) {
+int launch_gemm(rd_device *d, const DevWeight &w, const void *Xp, float *P, int M, GemmPlan *plan_out, int ldP, int splits, int kw, float *resid) {
     if (M < 1 || M > 32) {
         rd_set_error("gemm: M=%d outside 1..32", M);
         return RD_ERR_ARG;
     }
     int nKB = kblocks_for(w);
     GemmPlan p = plan_gemm(w.kind, w.N, nKB);
+    if (resid) splits = 1;
     if (splits > 0) p.kbPerSplit = (nKB + splits - 1) / splits, p.splits = splits;
+    if (kw > 0) p.kw = kw;
     if (plan_out) *plan_out = p;
     if (ldP <= 0) ldP = w.N;
+    if (is_gemm8_kind(w.kind)) {
+        const int tiles = w.N / 32, tpb = p.kw == 2 ? 2 : 1;
+        hipFunction_t f = d->k.gemm8[w.kind][p.kw == 8 ? 2 : (p.kw == 4 ? 1 : 0)];
+        return d->launch(f, (unsigned)((tiles + tpb - 1) / tpb), (unsigned)p.splits, 1, (unsigned)(64 * p.kw * tpb), (const void *)w.tiled, (const void *)w.scales, Xp, P,
+                         w.N, nKB, p.kbPerSplit, M, ldP, resid);
+    }
+    if (resid) {
+        rd_set_error("gemm: weight kind %d has no residual epilogue", w.kind);
+        return RD_ERR_STATE;
+    }
     unsigned gx = (unsigned)((w.N + 127) / 128);
-    if (w.kind == 0)
-        return d->launch(d->k.gemm_q4k, gx, p.splits, 1, GEMM_THREADS, (const void *)w.tiled, Xp, P, w.N, nKB, p.kbPerSplit, M, ldP);
-    if (w.kind == 3 || w.kind == 4)
-        return d->launch(w.kind == 3 ? d->k.gemm_q5k : d->k.gemm_q6k, gx, p.splits, 1, GEMM_THREADS, (const void *)w.tiled, Xp, P, w.N, nKB, p.kbPerSplit, M, ldP);
-    if (w.kind == 1)
-        return d->launch(d->k.gemm_w8a8, gx, p.splits, 1, GEMM_THREADS, (const void *)w.tiled, (const void *)w.scales, Xp, P, w.N, nKB, p.kbPerSplit, M, ldP);
-    return d->launch(d->k.gemm_w4a8, gx, p.splits, 1, GEMM_THREADS, (const void *)w.tiled, Xp, P, w.N, nKB, p.kbPerSplit, M, ldP);
+    return d->launch(w.kind == 3 ? d->k.gemm_q5k : d->k.gemm_q6k, gx, p.splits, 1, GEMM_THREADS, (const void *)w.tiled, Xp, P, w.N, nKB, p.kbPerSplit, M, ldP);
 }
 
 int launch_gemm_wide(rd_device *d, const DevWeight &w, const void *Xp, size_t xpStride, float *P, size_t pStride, int M, GemmPlan *plan_out, int ldP,
-                     int splits) {
+                     int splits, int kw) {
     if (M < 1 || M > GEMM_WIDE_ROWS) {
         rd_set_error("wide gemm: M=%d outside 1..%d", M, GEMM_WIDE_ROWS);
         return RD_ERR_ARG;
     }
-    if (w.kind != 0 || M <= 32 || getenv("ROCMDECODE_NO_WIDE_GEMM")) {
-        for (int m0 = 0, mt = 0; m0 < M; m0 += 32, mt++) {
-            int rc = launch_gemm(d, w, (const char *)Xp + (size_t)mt * xpStride, P + (size_t)mt * pStride, std::min(32, M - m0), plan_out, ldP, splits);
-            if (rc) return rc;
-        }
-        return RD_OK;
+    for (int m0 = 0, mt = 0; m0 < M; m0 += 32, mt++) {
+        int rc = launch_gemm(d, w, (const char *)Xp + (size_t)mt * xpStride, P + (size_t)mt * pStride, std::min(32, M - m0), plan_out, ldP, splits, kw);
+        if (rc) return rc;
     }
-    int nKB = kblocks_for(w);
-    GemmPlan p = plan_gemm(w.kind, w.N, nKB);
-    if (splits > 0) p.kbPerSplit = (nKB + splits - 1) / splits, p.splits = splits;
-    if (plan_out) *plan_out = p;
-    if (ldP <= 0) ldP = w.N;
-    if (M <= 64)
-        return d->launch(d->k.gemm_q4k_wide2, (unsigned)((w.N + 127) / 128), p.splits, 1, 384u, (const void *)w.tiled, Xp, xpStride, P, pStride, w.N, nKB,
-                         p.kbPerSplit, M, ldP);
-    return d->launch(d->k.gemm_q4k_wide, (unsigned)((w.N + 127) / 128), p.splits, 1, GEMM_WIDE_THREADS, (const void *)w.tiled, Xp, xpStride, P, pStride, w.N, nKB,
-                     p.kbPerSplit, M, ldP);
+    return RD_OK;
 }

@@ -19,17 +19,19 @@ bool rd_hip_ok(const HipApi *hip, hipError_t e, const char *what);
 constexpr size_t Q4K_PANEL_BYTES = 17 * 64 * 16;
 constexpr size_t LIN_PANEL_BYTES = 8 * 64 * 16;
 constexpr size_t Q4K_TILE_BYTES = 4608;
-enum { PANEL_Q4K = 0, PANEL_LIN = 1, PANEL_LIN4 = 2 };
+constexpr size_t A8_BLOCK_BYTES = 10240; // one A8 activation block: 256 elements x 32 rows (gemm8.h)
+inline size_t a8_bytes(int K) { return (size_t)((K + 255) / 256) * A8_BLOCK_BYTES; }
+enum { PANEL_Q4K = 0, PANEL_LIN = 1, PANEL_LIN4 = 2, PANEL_A8 = 3 };
 
 struct Kernels {
-    hipFunction_t dequant_q4k, retile_q4k, gemm_q4k, quant_act, reduce_splits, add_rmsnorm_quant, swiglu_quant;
-    hipFunction_t retile_w8a8, gemm_w8a8, retile_w4a8, gemm_w4a8;
-    hipFunction_t gemm_q4k_wide, gemm_q4k_wide2;
+    hipFunction_t dequant_q4k, quant_act, reduce_splits, add_rmsnorm_quant, swiglu_quant;
+    hipFunction_t unpack_act8, unpanel_a8, retile_q4k8, retile_w8a8_8, retile_w4a8_8;
+    hipFunction_t gemm8[3][3]; // [weight kind 0 q4k, 1 w8a8, 2 w4a8][waves per tile 2, 4, 8]
+    hipFunction_t gemm8_q4k_gateup, gemm8_w4a8_moe, gemm8_w4a8_moe_gateup;
     hipFunction_t dequant_q5k, retile_q5k, gemm_q5k, dequant_q6k, retile_q6k, gemm_q6k;
-    hipFunction_t gemm_q4k_gateup;
     hipFunction_t kv_store, kv_read, qkv_rope_store, attn_partial, attn_combine, attn_combine_quant;
     hipFunction_t kv_store_i8, qkv_rope_store_i8, attn_partial_i8, attn_partial_rows, attn_partial_rows_i8, attn_partial_deep, attn_partial_deep_i8, topk_rows, topk_hist, topk_pick, topk_finish;
-    hipFunction_t rmsnorm, rope, argmax_rows, argmax_final, matmul_f32, moe_route, gemm_w4a8_moe, gemm_w4a8_moe_gateup, moe_swiglu_quant, moe_fold, embed_rows, copy16, unpanel_q4k, fill_f16, fill_f32;
+    hipFunction_t rmsnorm, rope, argmax_rows, argmax_final, matmul_f32, moe_route, moe_swiglu_quant, moe_fold, embed_rows, copy16, unpanel_q4k, fill_f16, fill_f32;
 };
 
 struct rd_device {
@@ -67,8 +69,9 @@ struct DevBuf {
     template <typename T> T *as() { return (T *)p; }
 };
 
-// block sizes of the GEMM kernels: (4 consumer + 1 producer waves) x K-groups; they match the code object's launch bounds
-constexpr unsigned GEMM_THREADS = 320, GATEUP_THREADS = 640;
+// block sizes that match the code object's launch bounds: the f16-MFMA k-quant GEMMs (4 consumer + 1 producer waves), the fused
+// gate|up kernel (two tiles x four waves), the expert kernels (two tiles x two waves)
+constexpr unsigned GEMM_THREADS = 320, GATEUP_THREADS = 512, MOE_THREADS = 256;
 
 // How many 64-position KV blocks one attention work item covers for a sequence of nb blocks: every (sequence, kv head) is
 // cut into pieces. The cut depends on the sequence's own length only, never on what else is in the
@@ -119,7 +122,8 @@ bool build_attn_worklist(const int *len, const int *slot, int G, int rows, int n
 // split-K plan of one GEMM launch
 struct GemmPlan {
     int splits;     // grid.y
-    int kbPerSplit; // K-blocks (super-blocks or 128-wide blocks) per split
+    int kbPerSplit; // K-blocks (blocks of 256, or 128 for Q6_K) per split
+    int kw = 0;     // int8-MFMA kinds: waves per weight tile inside a block, each on its own K range (2, 4 or 8)
 };
 GemmPlan plan_gemm(int kind, int N, int nKB);
 
@@ -143,16 +147,19 @@ void free_weight(rd_device *d, DevWeight *w);
 // P[splits][32][N] = panels(Xp) . W^T ; returns the plan used
 // ldP: floats between rows of P (0 = w.N); splits > 0 forces the split count (trailing splits that get no K-block store zeros),
 // which lets weights of different kinds write side by side into one partial-sum buffer.
-int launch_gemm(rd_device *d, const DevWeight &w, const void *Xp, float *P, int M, GemmPlan *plan, int ldP = 0, int splits = 0);
+// Q4_K, int8 and int4-g32 weights go through the int8-MFMA kernels over A8 activation blocks (gemm8.h), Q5_K and Q6_K through
+// the f16-MFMA kernels over f16 panels (kquant.h). kw > 0 forces the waves per tile of the int8-MFMA kinds.
+// resid != NULL (int8-MFMA kinds, one split): the sums are added to resid[m][n] (row stride ldP) in place and nothing goes to P.
+int launch_gemm(rd_device *d, const DevWeight &w, const void *Xp, float *P, int M, GemmPlan *plan, int ldP = 0, int splits = 0, int kw = 0,
+                float *resid = nullptr);
+inline bool is_gemm8_kind(int kind) { return kind >= 0 && kind <= 2; }
 // Up to 128 rows as M-tiles of 32: M-tile mt reads its panels at Xp + mt*xpStride (bytes) and writes its partial sums at
-// P + mt*pStride (floats), each laid out as launch_gemm's. Q4_K weights go through the wide kernel (weights read once for
-// all rows); the other kinds run launch_gemm per M-tile. Rows come out identical to launch_gemm's either way.
+// P + mt*pStride (floats), each laid out as launch_gemm's: one launch_gemm per M-tile, so a row is the same row whatever pass it rides in.
 constexpr int GEMM_WIDE_ROWS = 128;
-constexpr unsigned GEMM_WIDE_THREADS = 512;
 int launch_gemm_wide(rd_device *d, const DevWeight &w, const void *Xp, size_t xpStride, float *P, size_t pStride, int M, GemmPlan *plan, int ldP = 0,
-                     int splits = 0);
+                     int splits = 0, int kw = 0);
 size_t panel_bytes_for(const DevWeight &w);
 int panel_kind_for(const DevWeight &w);
-// K-blocks of a weight: super-blocks of 256 for the kinds on Q4_K-style panels (q4k, q5k), 128 otherwise
-inline int kblock_of(int kind) { return (kind == 0 || kind == 3) ? 256 : 128; }
-inline int kblocks_for(const DevWeight &w) { return w.K / kblock_of(w.kind); }
+// K-blocks of a weight: 256 elements (an A8 block, a Q5_K super-block), 128 for Q6_K's half super-blocks. The int8-MFMA kinds pad K up to whole blocks with zeros.
+inline int kblock_of(int kind) { return kind == 4 ? 128 : 256; }
+inline int kblocks_for(const DevWeight &w) { return (w.K + kblock_of(w.kind) - 1) / kblock_of(w.kind); }

@@ -268,14 +268,14 @@ extern "C" int rd_model_upload_w4a8(rd_model *m, int layer, int proj, int expert
         return RD_ERR_ARG;
     }
     LayerW &l = m->layers[(size_t)layer];
-    size_t guBytes = (size_t)(2 * I / 32) * (H / 128) * 2304, dnBytes = (size_t)(H / 32) * (I / 128) * 2304;
+    size_t guBytes = (size_t)(2 * I / 32) * ((H + 255) / 256) * 4608, dnBytes = (size_t)(H / 32) * ((I + 255) / 256) * 4608;
     if (!l.exp_gateup) {
         RC(d->alloc(&l.exp_gateup, guBytes * c.n_experts));
         RC(d->alloc(&l.exp_down, dnBytes * c.n_experts));
     }
     DevWeight tmp;
     RC(upload_w4a8(d, nib, s16, N, K, &tmp));
-    size_t tb = (size_t)(N / 32) * (K / 128) * 2304;
+    size_t tb = (size_t)(N / 32) * ((K + 255) / 256) * 4608;
     uint8_t *dst = isDown ? (uint8_t *)l.exp_down + dnBytes * expert
                           : (uint8_t *)l.exp_gateup + guBytes * expert + (proj == RD_PROJ_UP ? guBytes / 2 : 0);
     int rc = rd_hip_ok(d->hip, d->hip->MemcpyAsync(dst, tmp.tiled, tb, hipMemcpyDeviceToDevice, d->stream), "expert copy") ? RD_OK : RD_ERR_HIP;
@@ -330,9 +330,17 @@ extern "C" int rd_model_upload_embedding(rd_model *m, const int8_t *q, const flo
     return d->sync();
 }
 
+// A group's members all run with one split count, so that the consumer sums the same number of partials for every column: the
+// fewest any member's own plan asks for (no member then gets more splits than it has K-blocks).
+static GemmPlan group_plan(const DevWeight &w) {
+    GemmPlan g{1 << 30, 0, 0};
+    for (const auto &p : w.parts) g.splits = std::min(g.splits, plan_gemm(p.kind, p.N, kblocks_for(p)).splits);
+    return g;
+}
+
 static size_t gemm_partial_floats(const DevWeight &w) {
     if (w.kind < 0) return 0;
-    if (w.kind == WKIND_GROUP) return (size_t)plan_gemm(0, w.N, w.K / 256 > 0 ? w.K / 256 : 1).splits * 32 * w.N;
+    if (w.kind == WKIND_GROUP) return (size_t)group_plan(w).splits * 32 * w.N;
     int nKB = kblocks_for(w);
     return (size_t)plan_gemm(w.kind, w.N, nKB).splits * 32 * w.N;
 }
@@ -356,7 +364,6 @@ extern "C" int rd_model_finalize(rd_model *m) {
             return RD_ERR_STATE;
         }
         pf = std::max({pf, gemm_partial_floats(l.qkv), gemm_partial_floats(l.o), gemm_partial_floats(l.gateup), gemm_partial_floats(l.down)});
-        if (c.n_experts == 0) pf = std::max(pf, (size_t)2 * 32 * l.gateup.N); // the unfused gate|up launch with two splits
     }
     if (m->head.kind < 0 || !m->final_norm) {
         rd_set_error("model is missing the head or the final norm");
@@ -376,7 +383,7 @@ extern "C" int rd_model_finalize(rd_model *m) {
     RC(alloc_f32(d, &m->logits, R * c.vocab));
     size_t kA = (size_t)H, kB = (size_t)std::max(qd, c.n_experts ? qd : c.inter);
     // room for either panel kind: 8 KB per 128 elements (int8/int4 consumers) or 17 KB per 256 (Q4_K consumers)
-    auto panel_room = [](size_t K) { return std::max(((K + 127) / 128) * (size_t)LIN_PANEL_BYTES, ((K + 255) / 256) * (size_t)Q4K_PANEL_BYTES); };
+    auto panel_room = [](size_t K) { return std::max({((K + 127) / 128) * (size_t)LIN_PANEL_BYTES, ((K + 255) / 256) * (size_t)Q4K_PANEL_BYTES, a8_bytes((int)K)}); };
     m->xpAStride = panel_room(kA), m->xpBStride = panel_room(kB);
     RC(d->alloc(&m->XpA, m->xpAStride * tiles));
     RC(d->alloc(&m->XpA2, m->xpAStride * tiles));
@@ -396,8 +403,8 @@ extern "C" int rd_model_finalize(rd_model *m) {
         RC(d->alloc((void **)&m->moe_rank, (size_t)32 * c.n_experts));
         RC(d->alloc((void **)&m->moe_bits, sizeof(unsigned) * 8));
         HIPCHK(MemsetAsync(m->moe_bits, 0, sizeof(unsigned) * 8, d->stream));
-        RC(d->alloc(&m->XpE, (size_t)c.n_experts * (I / 128) * LIN_PANEL_BYTES));
-        HIPCHK(MemsetAsync(m->XpE, 0, (size_t)c.n_experts * (I / 128) * LIN_PANEL_BYTES, d->stream));
+        RC(d->alloc(&m->XpE, (size_t)c.n_experts * a8_bytes(I)));
+        HIPCHK(MemsetAsync(m->XpE, 0, (size_t)c.n_experts * a8_bytes(I), d->stream));
     }
     RC(d->alloc((void **)&m->topk_ids, sizeof(int) * R * TOPK_MAX));
     RC(alloc_f32(d, &m->topk_vals, R * TOPK_MAX));
@@ -604,8 +611,7 @@ static int launch_proj(rd_model *m, const DevWeight &w, const void *Xp, size_t x
     if (w.kind != WKIND_GROUP) return launch_gemm_wide(d, w, Xp, xpStride, m->P, m->pStride, B, plan);
     int kA, kB;
     panel_kinds_of(w, &kA, &kB);
-    GemmPlan g = plan_gemm(0, w.N, w.K / 256 > 0 ? w.K / 256 : 1);
-    for (const auto &p : w.parts) g.splits = std::min(g.splits, std::max(1, kblocks_for(p))); // no member gets more splits than K-blocks
+    GemmPlan g = group_plan(w);
     for (size_t i = 0; i < w.parts.size(); i++) {
         const DevWeight &p = w.parts[i];
         RC(launch_gemm_wide(d, p, panel_kind_for(p) == kA ? Xp : m->XpA2, xpStride, m->P + w.col0[i], m->pStride, B, nullptr, w.N, g.splits));
@@ -615,10 +621,11 @@ static int launch_proj(rd_model *m, const DevWeight &w, const void *Xp, size_t x
     return RD_OK;
 }
 
-// Where the fused gate|up kernel can run it sums K in two halves (its two K-groups, folded once). The unfused path — steps of
-// more than 32 rows, or the fused kernel switched off — is launched with exactly those two splits, so both produce the same
-// bits and a row is the same row in a batch of any size.
-static bool gateup_fusable(const rd_model_desc &c, const DevWeight &w) { return w.kind == 0 && c.inter % 64 == 0; }
+// Where the fused gate|up kernel can run it sums K over four waves per tile, folded in LDS. The unfused path — steps of more than
+// 32 rows, or the fused kernel switched off — is launched with the same four waves and one split, so both produce the same bits
+// and a row is the same row in a batch of any size.
+static bool gateup_fusable(const rd_model_desc &c, const DevWeight &w) { return w.kind == 0 && c.inter % 32 == 0; }
+constexpr int GATEUP_KW = 4; // waves per tile of the fused gate|up kernel
 
 constexpr int MOE_FOLD_FUSED_MAX = 8; // ranks rd_k_add_rmsnorm_quant folds in registers
 
@@ -647,17 +654,18 @@ static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
                          m->moe_rank, trace, m->moe_bits));
         }
     }
-    size_t guStride = (size_t)(2 * I / 32) * (H / 128) * 2304, dnStride = (size_t)(H / 32) * (I / 128) * 2304;
-    size_t xpStride = (size_t)(I / 128) * LIN_PANEL_BYTES;
-    if (I % 64 == 0 && !getenv("ROCMDECODE_NO_FUSED_MOE_GATEUP")) {
-        Scope s(m, KC_MOE_GEMM); // gate|up of every touched expert + SwiGLU + quantization into the experts' down panels
-        RC(d->launch(d->k.gemm_w4a8_moe_gateup, (unsigned)(I / 64), (unsigned)nE, 1, GEMM_THREADS, (const void *)l.exp_gateup, guStride,
-                     (const void *)m->XpA, m->XpE, xpStride, I, H / 128, B, (const signed char *)m->moe_rank, nE, (const unsigned *)m->moe_bits));
+    const int nKBh = (H + 255) / 256, nKBi = (I + 255) / 256;
+    size_t guStride = (size_t)(2 * I / 32) * nKBh * 4608, dnStride = (size_t)(H / 32) * nKBi * 4608;
+    size_t xpStride = a8_bytes(I);
+    if (I % 32 == 0 && !getenv("ROCMDECODE_NO_FUSED_MOE_GATEUP")) {
+        Scope s(m, KC_MOE_GEMM); // gate|up of every touched expert + SwiGLU + quantization into the experts' down activations
+        RC(d->launch(d->k.gemm8_w4a8_moe_gateup, (unsigned)(I / 32), (unsigned)nE, 1, MOE_THREADS, (const void *)l.exp_gateup, guStride,
+                     (const void *)m->XpA, m->XpE, xpStride, I, nKBh, B, (const signed char *)m->moe_rank, nE, (const unsigned *)m->moe_bits));
     } else {
         {
             Scope s(m, KC_MOE_GEMM);
-            RC(d->launch(d->k.gemm_w4a8_moe, (unsigned)((2 * I + 127) / 128), (unsigned)nE, 1, GEMM_THREADS, (const void *)l.exp_gateup, guStride,
-                         (const void *)m->XpA, (size_t)0, m->moe_gu, 2 * I, H / 128, B, k, (const signed char *)m->moe_rank, nE,
+            RC(d->launch(d->k.gemm8_w4a8_moe, (unsigned)((2 * I + 63) / 64), (unsigned)nE, 1, MOE_THREADS, (const void *)l.exp_gateup, guStride,
+                         (const void *)m->XpA, (size_t)0, m->moe_gu, 2 * I, nKBh, B, k, (const signed char *)m->moe_rank, nE,
                          (const unsigned *)m->moe_bits));
         }
         Scope s(m, KC_MOE_GLUE);
@@ -666,8 +674,8 @@ static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
     }
     {
         Scope s(m, KC_MOE_GEMM_DOWN);
-        RC(d->launch(d->k.gemm_w4a8_moe, (unsigned)((H + 127) / 128), (unsigned)nE, 1, GEMM_THREADS, (const void *)l.exp_down, dnStride, (const void *)m->XpE,
-                     xpStride, m->moe_dn, H, I / 128, B, k, (const signed char *)m->moe_rank, nE, (const unsigned *)m->moe_bits));
+        RC(d->launch(d->k.gemm8_w4a8_moe, (unsigned)((H + 63) / 64), (unsigned)nE, 1, MOE_THREADS, (const void *)l.exp_down, dnStride, (const void *)m->XpE,
+                     xpStride, m->moe_dn, H, nKBi, B, k, (const signed char *)m->moe_rank, nE, (const unsigned *)m->moe_bits));
     }
     if (k > MOE_FOLD_FUSED_MAX) { // else the next norm kernel folds the ranks itself as it adds them to the residual
         Scope s(m, KC_MOE_GLUE);
@@ -825,13 +833,13 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
             RC(add_norm_quant(m, B, m->P, plan.splits, l.ffn_norm, l.gateup, m->XpA, nullptr));
             if (B <= 32 && gateup_fusable(c, l.gateup) && !getenv("ROCMDECODE_NO_FUSED_GATEUP")) {
                 Scope s(m, KC_GEMM_GATEUP); // gate|up GEMM + SwiGLU + quantization in one launch
-                RC(d->launch(d->k.gemm_q4k_gateup, (unsigned)(c.inter / 64), 1, 1, GATEUP_THREADS, (const void *)l.gateup.tiled, (const void *)m->XpA, m->XpB,
+                RC(d->launch(d->k.gemm8_q4k_gateup, (unsigned)(c.inter / 32), 1, 1, GATEUP_THREADS, (const void *)l.gateup.tiled, (const void *)m->XpA, m->XpB,
                              panel_kind_for(l.down), c.inter, H / 256, B));
             } else {
                 {
                     Scope s(m, KC_GEMM_GATEUP);
                     if (gateup_fusable(c, l.gateup))
-                        RC(launch_gemm_wide(d, l.gateup, m->XpA, m->xpAStride, m->P, m->pStride, B, &plan, 0, 2));
+                        RC(launch_gemm_wide(d, l.gateup, m->XpA, m->xpAStride, m->P, m->pStride, B, &plan, 0, 1, GATEUP_KW));
                     else
                         RC(launch_proj(m, l.gateup, m->XpA, m->xpAStride, B, &plan));
                 }
@@ -848,7 +856,7 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
             {
                 Scope s(m, KC_ADD_NORM);
                 RC(d->launch(d->k.add_rmsnorm_quant, (unsigned)B, 1, 1, 1024, m->h, (const float *)m->P, plan.splits, (const float *)l.ffn_norm,
-                             c.rms_eps, H, m->XpA, (int)PANEL_LIN4, m->normed, (void *)nullptr, -1, m->pStride, m->xpAStride, m->xpAStride,
+                             c.rms_eps, H, m->XpA, (int)PANEL_A8, m->normed, (void *)nullptr, -1, m->pStride, m->xpAStride, m->xpAStride,
                              (const float *)nullptr));
             }
             RC(moe_ffn(m, B, li, l));

@@ -63,9 +63,9 @@ static int gemm_host(rd_device *d, DevWeight &w, DevWeight *w2, const float *a, 
             // gate|up stacked (2N rows): GEMM, then SwiGLU over the reduced partial sums
             RC(launch_gemm(d, *w2, Xp.p, P.as<float>(), mc, &plan));
             DevBuf X2(d);
-            RC(X2.alloc((size_t)((N + 255) / 256) * Q4K_PANEL_BYTES));
+            RC(X2.alloc(a8_bytes(N)));
             RC(d->launch(d->k.swiglu_quant, (unsigned)((N + 1023) / 1024), (unsigned)mc, 1, 256, (const float *)P.p, plan.splits, N, X2.p,
-                         (int)PANEL_Q4K, O.as<float>(), (size_t)0, (size_t)0));
+                         (int)PANEL_A8, O.as<float>(), (size_t)0, (size_t)0));
             RC(d->sync());
         }
         RC(d->d2h(dst + (size_t)m0 * N, O.p, sizeof(float) * (size_t)mc * N));
@@ -120,16 +120,16 @@ extern "C" int rd_gateup_q4k_quant(rd_device *d, const void *Wg, const void *Wu,
     DevBuf A(d), Xp(d), X2(d), O(d);
     auto body = [&]() -> int {
         RC(A.alloc(sizeof(float) * (size_t)32 * K));
-        RC(Xp.alloc((size_t)(K / 256) * Q4K_PANEL_BYTES));
-        RC(X2.alloc((size_t)(I / 256) * Q4K_PANEL_BYTES));
+        RC(Xp.alloc(a8_bytes(K)));
+        RC(X2.alloc(a8_bytes(I)));
         RC(O.alloc(sizeof(float) * (size_t)32 * I));
         for (int m0 = 0; m0 < M; m0 += 32) {
             int mc = std::min(32, M - m0);
             RC(d->h2d(A.p, a + (size_t)m0 * K, sizeof(float) * (size_t)mc * K));
-            RC(quantize_rows(d, A.as<float>(), mc, K, PANEL_Q4K, 0, Xp.p));
-            RC(d->launch(d->k.gemm_q4k_gateup, (unsigned)(I / 64), 1, 1, GATEUP_THREADS, (const void *)w.tiled, (const void *)Xp.p, X2.as<uint8_t>(),
-                         (int)PANEL_Q4K, I, K / 256, mc));
-            RC(d->launch(d->k.unpanel_q4k, (unsigned)(I / 256), (unsigned)mc, 1, 256, (const void *)X2.p, O.as<float>(), I));
+            RC(quantize_rows(d, A.as<float>(), mc, K, PANEL_A8, 0, Xp.p));
+            RC(d->launch(d->k.gemm8_q4k_gateup, (unsigned)(I / 32), 1, 1, GATEUP_THREADS, (const void *)w.tiled, (const void *)Xp.p, X2.as<uint8_t>(),
+                         (int)PANEL_A8, I, K / 256, mc));
+            RC(d->launch(d->k.unpanel_a8, (unsigned)(I / 256), (unsigned)mc, 1, 256, (const void *)X2.p, O.as<float>(), I));
             RC(d->d2h(dst + (size_t)m0 * I, O.p, sizeof(float) * (size_t)mc * I));
         }
         return RD_OK;
@@ -137,6 +137,33 @@ extern "C" int rd_gateup_q4k_quant(rd_device *d, const void *Wg, const void *Wu,
     rc = body();
     free_weight(d, &w);
     return rc;
+}
+
+// The activation quantizer on its own (goinfer: aikit QuantizeActQ group 32, call sites decoder/weightmat.go:845-862;
+// backend/cuda/actgroup.cu:32-54 quantG32): a f32 [M][K] -> int8 codes [M][K], f32 scales and sums (scale * sum of codes) [M][K/32],
+// as the GEMMs consume them. K % 32 == 0.
+extern "C" int rd_quant_act(rd_device *d, const float *a, int M, int K, int8_t *codes, float *scales, float *sums) {
+    if (!d || !a || !codes || !scales || !sums || M <= 0 || K <= 0 || K % 32) {
+        rd_set_error("rd_quant_act: bad arguments (K must be a multiple of 32)");
+        return RD_ERR_ARG;
+    }
+    const int nG = K / 32;
+    DevBuf A(d), A8(d), C(d), S(d), U(d);
+    RC(A.alloc(sizeof(float) * (size_t)32 * K));
+    RC(A8.alloc(a8_bytes(K)));
+    RC(C.alloc((size_t)32 * K));
+    RC(S.alloc(sizeof(float) * (size_t)32 * nG));
+    RC(U.alloc(sizeof(float) * (size_t)32 * nG));
+    for (int m0 = 0; m0 < M; m0 += 32) {
+        const int mc = std::min(32, M - m0);
+        RC(d->h2d(A.p, a + (size_t)m0 * K, sizeof(float) * (size_t)mc * K));
+        RC(quantize_rows(d, A.as<float>(), mc, K, PANEL_A8, 0, A8.p));
+        RC(d->launch(d->k.unpack_act8, (unsigned)((K + 255) / 256), (unsigned)mc, 1, 256, (const void *)A8.p, (signed char *)C.p, S.as<float>(), U.as<float>(), K));
+        RC(d->d2h(codes + (size_t)m0 * K, C.p, (size_t)mc * K));
+        RC(d->d2h(scales + (size_t)m0 * nG, S.p, sizeof(float) * (size_t)mc * nG));
+        RC(d->d2h(sums + (size_t)m0 * nG, U.p, sizeof(float) * (size_t)mc * nG));
+    }
+    return RD_OK;
 }
 
 // Q5_K / Q6_K: the file's own super-blocks (176 B / 210 B per 256 weights) dequantized or multiplied natively.

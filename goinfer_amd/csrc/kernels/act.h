@@ -1,69 +1,90 @@
 // act.h — the row-wise glue between GEMMs: split-K reduction, residual add, RMSNorm, SwiGLU, and the per-32 int8
 // activation quantization whose dequantized values are written as f16 MFMA panels for the next GEMM.
 #pragma once
+#include "a8.h"
 #include "common.h"
 
-enum { RD_PANEL_Q4K = 0, RD_PANEL_LIN = 1, RD_PANEL_LIN4 = 2 };
+enum { RD_PANEL_Q4K = 0, RD_PANEL_LIN = 1, RD_PANEL_LIN4 = 2, RD_PANEL_A8 = 3 };
 
-// Store one quantized-then-dequantized activation (element k of batch row m) into its panel.
-__device__ __forceinline__ void panel_store(uint8_t *__restrict__ Xp, int kind, int m, int k, float xhat, float gsum) {
-    if (kind == RD_PANEL_Q4K) {
+// One quantized element: its int8 code, the group's scale and scaled code sum, and the dequantized value code * scale that
+// the f16 panel kinds store.
+struct Quant1 {
+    int code;
+    float sc, gsum, xhat;
+};
+__device__ __forceinline__ Quant1 quant_one(float v) { // an aligned half-wave holds one group of 32
+    Quant1 q;
+    q.code = quant8_g32(v, &q.sc, &q.gsum);
+    q.xhat = __fmul_rn((float)q.code, q.sc);
+    return q;
+}
+// Four consecutive elements per lane (a group is 8 consecutive lanes).
+struct Quant4 {
+    uint32_t codes; // packed, low byte first
+    float sc, gsum, x[4];
+};
+__device__ __forceinline__ Quant4 quant_four(float v0, float v1, float v2, float v3) {
+    Quant4 q;
+    q.codes = quant8_g32x4(v0, v1, v2, v3, &q.sc, &q.gsum);
+#pragma unroll
+    for (int i = 0; i < 4; i++) q.x[i] = __fmul_rn((float)(int)(signed char)(q.codes >> (8 * i)), q.sc);
+    return q;
+}
+
+// Store one quantized activation (element k of batch row m) in the layout the consuming GEMM reads.
+__device__ __forceinline__ void panel_store(uint8_t *__restrict__ Xp, int kind, int m, int k, const Quant1 &q) {
+    if (kind == RD_PANEL_A8) {
+        Xp[a8_code_offset(m, k)] = (uint8_t)q.code;
+        if ((k & 31) == 0) {
+            uint8_t *p = Xp + a8_scale_offset(m, k >> 5);
+            *(float *)p = q.sc;
+            *(float *)(p + (RD_A8_SUMS - RD_A8_SCALES)) = q.gsum;
+        }
+    } else if (kind == RD_PANEL_Q4K) {
         half_t *base = (half_t *)(Xp + (size_t)(k >> 8) * RD_Q4K_PANEL_BYTES);
         int t = k & 255, j = t >> 5;
-        base[q4k_panel_index(t, m)] = (half_t)xhat;
-        if ((t & 31) == 0) base[q4k_panel_sum_index(j, m)] = (half_t)gsum;
-        if ((t & 31) == 1) base[q4k_panel_sum_index(j, m) - (j & 3) + 4 + (j & 3)] = (half_t)0.f;
+        base[q4k_panel_index(t, m)] = (half_t)q.xhat;
+        if ((t & 31) == 0) base[q4k_panel_sum_index(j, m)] = (half_t)q.gsum;
+        if ((t & 31) == 1) base[q4k_panel_sum_index(j, m) + 4] = (half_t)0.f;
     } else {
         half_t *base = (half_t *)(Xp + (size_t)(k >> 7) * RD_LIN_PANEL_BYTES);
-        base[kind == RD_PANEL_LIN ? lin_panel_index(k & 127, m) : lin4_panel_index(k & 127, m)] = (half_t)xhat;
+        base[kind == RD_PANEL_LIN ? lin_panel_index(k & 127, m) : lin4_panel_index(k & 127, m)] = (half_t)q.xhat;
     }
 }
 
 // Four consecutive elements k0..k0+3 (k0 % 4 == 0) of batch row m. In a Q4_K panel they are the four bytes of one code
 // word and land in slots {0,1} and {4,5} (+2 for an odd sub-block) of one lane row: two 4-byte stores.
-__device__ __forceinline__ void panel_store4(uint8_t *__restrict__ Xp, int kind, int m, int k0, float x0, float x1, float x2, float x3, float gsum) {
-    if (kind == RD_PANEL_Q4K) {
+__device__ __forceinline__ void panel_store4(uint8_t *__restrict__ Xp, int kind, int m, int k0, const Quant4 &q) {
+    if (kind == RD_PANEL_A8) {
+        a8_store4(Xp, m, k0, q.codes, q.sc, q.gsum);
+    } else if (kind == RD_PANEL_Q4K) {
         half_t *base = (half_t *)(Xp + (size_t)(k0 >> 8) * RD_Q4K_PANEL_BYTES);
         int t = k0 & 255, j = t >> 5;
         half_t *row = base + q4k_panel_index(t, m); // slot of byte 0
-        *(half2_t *)row = (half2_t){(half_t)x0, (half_t)x2};
-        *(half2_t *)(row + 4) = (half2_t){(half_t)x1, (half_t)x3};
+        *(half2_t *)row = (half2_t){(half_t)q.x[0], (half_t)q.x[2]};
+        *(half2_t *)(row + 4) = (half2_t){(half_t)q.x[1], (half_t)q.x[3]};
         if ((t & 31) == 0) {
             half_t *sp = base + q4k_panel_sum_index(j, m);
-            sp[0] = (half_t)gsum;
+            sp[0] = (half_t)q.gsum;
             sp[4] = (half_t)0.f; // slots 4..7 of the sum step stay zero
         }
     } else if (kind == RD_PANEL_LIN) {
         half_t *row = (half_t *)(Xp + (size_t)(k0 >> 7) * RD_LIN_PANEL_BYTES) + lin_panel_index(k0 & 127, m);
-        *(half2_t *)row = (half2_t){(half_t)x0, (half_t)x1};
-        *(half2_t *)(row + 2) = (half2_t){(half_t)x2, (half_t)x3};
+        *(half2_t *)row = (half2_t){(half_t)q.x[0], (half_t)q.x[1]};
+        *(half2_t *)(row + 2) = (half2_t){(half_t)q.x[2], (half_t)q.x[3]};
     } else {
         half_t *row = (half_t *)(Xp + (size_t)(k0 >> 7) * RD_LIN_PANEL_BYTES) + lin_panel_index((k0 & 127) & ~7, m);
         int o = k0 & 4 ? 1 : 0; // offsets 0..3 -> slots 0,2,4,6; offsets 4..7 -> slots 1,3,5,7
-        row[o] = (half_t)x0, row[o + 2] = (half_t)x1, row[o + 4] = (half_t)x2, row[o + 6] = (half_t)x3;
+        row[o] = (half_t)q.x[0], row[o + 2] = (half_t)q.x[1], row[o + 4] = (half_t)q.x[2], row[o + 6] = (half_t)q.x[3];
     }
-}
-
-// Per-32 quantization when each lane holds 4 consecutive elements: a group is 8 consecutive lanes.
-__device__ __forceinline__ void quant_g32x4(float v0, float v1, float v2, float v3, float *x0, float *x1, float *x2, float *x3, float *gsum) {
-    float ma = fmaxf(fmaxf(fabsf(v0), fabsf(v1)), fmaxf(fabsf(v2), fabsf(v3)));
-    ma = group_max8(ma);
-    float sc = ma / 127.f;
-    float inv = sc > 0.f ? 1.f / sc : 0.f;
-    float r0 = fminf(127.f, fmaxf(-127.f, roundf(__fmul_rn(v0, inv)))), r1 = fminf(127.f, fmaxf(-127.f, roundf(__fmul_rn(v1, inv))));
-    float r2 = fminf(127.f, fmaxf(-127.f, roundf(__fmul_rn(v2, inv)))), r3 = fminf(127.f, fmaxf(-127.f, roundf(__fmul_rn(v3, inv))));
-    int s = (int)r0 + (int)r1 + (int)r2 + (int)r3;
-    s = group_sum8_i(s);
-    *gsum = __fmul_rn(sc, (float)s);
-    *x0 = __fmul_rn(r0, sc), *x1 = __fmul_rn(r1, sc), *x2 = __fmul_rn(r2, sc), *x3 = __fmul_rn(r3, sc);
 }
 
 // x f32 [M][K] -> panels. Grid (K/256, M), 256 threads: thread t is element t of the 256-wide chunk.
 extern "C" __global__ __launch_bounds__(256) void rd_k_quant_act(const float *__restrict__ x, uint8_t *__restrict__ Xp, int K, int kind) {
     int m = blockIdx.y, k = blockIdx.x * 256 + threadIdx.x;
     float v = k < K ? x[(size_t)m * K + k] : 0.f;
-    float gs, xh = quant_g32(v, &gs);
-    if (k < K) panel_store(Xp, kind, m, k, xh, gs);
+    const Quant1 q = quant_one(v);
+    if (k < K || kind == RD_PANEL_A8) panel_store(Xp, kind, m, k, q); // A8: the tail of the last block is written as zero groups
 }
 
 // out[m][n] = sum_s P[s][m][n] in ascending split order (deterministic).
@@ -181,10 +202,9 @@ extern "C" __global__ __launch_bounds__(1024) void rd_k_add_rmsnorm_quant(float 
         float n0 = __fmul_rn(__fmul_rn(v[i].x, inv), wv[i].x), n1 = __fmul_rn(__fmul_rn(v[i].y, inv), wv[i].y);
         float n2 = __fmul_rn(__fmul_rn(v[i].z, inv), wv[i].z), n3 = __fmul_rn(__fmul_rn(v[i].w, inv), wv[i].w);
         if (norm_out) *(float4_t *)(norm_out + (size_t)m * H + k0) = (float4_t){n0, n1, n2, n3};
-        float x0, x1, x2, x3, gs;
-        quant_g32x4(n0, n1, n2, n3, &x0, &x1, &x2, &x3, &gs);
-        panel_store4(Xp, kind, mr, k0, x0, x1, x2, x3, gs);
-        if (Xp2) panel_store4(Xp2, kind2, mr, k0, x0, x1, x2, x3, gs); // a second consumer that reads another panel layout
+        const Quant4 q = quant_four(n0, n1, n2, n3);
+        panel_store4(Xp, kind, mr, k0, q);
+        if (Xp2) panel_store4(Xp2, kind2, mr, k0, q); // a second consumer that reads another panel layout
     }
 }
 
@@ -211,9 +231,8 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_swiglu_quant(const float 
         }
         if (act_out) *(float4_t *)(act_out + (size_t)row * I + n0) = (float4_t){a[0], a[1], a[2], a[3]};
     }
-    float x0, x1, x2, x3, gs;
-    quant_g32x4(a[0], a[1], a[2], a[3], &x0, &x1, &x2, &x3, &gs);
-    if (on) panel_store4(Xp, kind, m, n0, x0, x1, x2, x3, gs);
+    const Quant4 q = quant_four(a[0], a[1], a[2], a[3]);
+    if (on) panel_store4(Xp, kind, m, n0, q);
 }
 
 // A Q4_K-layout activation panel set back to rows: out[m][k] = the f16 value (code * scale) the GEMM reads for batch row m,

@@ -1,4 +1,4 @@
-// gemm.h — the dequant-GEMM skeleton shared by the Q4_K, int8 and int4-g32 weight kinds.
+// gemm.h — the f16-MFMA dequant-GEMM skeleton of the Q5_K and Q6_K weight kinds (kquant.h).
 //
 // P[split][32][N] = panels . tiles^T for M <= 32 batch rows. Grid (ceil(N/(32*TPB)), splits), block (TPB+1)*KG waves.
 // Each consumer wave owns one 32-row weight tile and streams its K-blocks from HBM with PF tiles in flight; producer waves
@@ -149,122 +149,6 @@ __device__ __forceinline__ void gemm_body(const uint8_t *__restrict__ Wt, const 
         for (int r = 0; r < 16; r++) {
             int m = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
             if (m < M) out[(size_t)m * ldP] = acc[r];
-        }
-    }
-}
-
-// ---- wide rows (prefill, verify): MT M-tiles of 32 batch rows share every weight tile ----
-// Block = TPB consumer waves + MT producer waves; producer p stages the panels of M-tile p (its own double buffer in LDS, its
-// own ring of T::PRODUCER_DEPTH panels in registers), consumer t streams weight tile t as in the narrow loop and multiplies
-// each K-block against the MT panels before it moves on: the weights are read and dequantized once for up to 32*MT rows.
-// For every M-tile the MFMA sequence and its operands are those of the narrow loop, so a row's result does not depend on
-// which loop computed it. LDS: MT*2*PANEL_VECS vectors. nMT: M-tiles in use (the others' producers only keep the barriers).
-template <class T, int TPB, int MT, int PF>
-__device__ __forceinline__ void gemm_mainloop_wide(float16_t (&acc)[MT], const uint8_t *__restrict__ wbase, const uint8_t *__restrict__ Xp,
-                                                   size_t xpStride, int kb0, int kb1, int nMT, uint4_t *lds_all) {
-    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    constexpr int PV = T::PANEL_VECS, PVL = PV / 64;
-    const bool producer = wave >= TPB;
-#pragma unroll
-    for (int m = 0; m < MT; m++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) acc[m][i] = 0.f;
-    const int per = kb1 - kb0;
-    if (per <= 0) return;
-    const int last = per - 1;
-    if (producer) {
-        const int pm = wave - TPB;
-        if (pm >= nMT) { // an M-tile with no rows: nothing to stage
-            for (int it = 0; it <= per; it++) __syncthreads();
-            return;
-        }
-        constexpr int PD = T::PRODUCER_DEPTH;
-        uint4_t *lds = lds_all + pm * 2 * PV;
-        const uint4_t *src = (const uint4_t *)(Xp + (size_t)pm * xpStride) + (size_t)kb0 * PV + lane;
-        uint4_t ring[PD][PVL];
-#pragma unroll
-        for (int d = 0; d < PD; d++)
-#pragma unroll
-            for (int j = 0; j < PVL; j++) ring[d][j] = src[(size_t)min(d, last) * PV + j * 64];
-        auto move = [&](int jp, auto sc) {
-            constexpr int slot = decltype(sc)::value;
-            uint4_t *dst = lds + (jp & 1) * PV + lane;
-#pragma unroll
-            for (int j = 0; j < PVL; j++) dst[j * 64] = ring[slot][j];
-            const uint4_t *s2 = src + (size_t)min(jp + PD, last) * PV;
-#pragma unroll
-            for (int j = 0; j < PVL; j++) ring[slot][j] = s2[j * 64];
-        };
-        using S0 = std::integral_constant<int, 0>;
-        using S1 = std::integral_constant<int, 1 % PD>;
-        using S2 = std::integral_constant<int, 2 % PD>;
-        using S3 = std::integral_constant<int, 3 % PD>;
-        move(0, S0{});
-        __syncthreads();
-        int it = 0;
-        for (; it + PD <= per; it += PD) {
-            if constexpr (PD > 1) move(it + 1, S1{}), __syncthreads();
-            if constexpr (PD > 2) move(it + 2, S2{}), __syncthreads();
-            if constexpr (PD > 3) move(it + 3, S3{}), __syncthreads();
-            move(it + PD, S0{}), __syncthreads();
-        }
-        if constexpr (PD > 1)
-            if (it + 0 < per) move(it + 1, S1{}), __syncthreads();
-        if constexpr (PD > 2)
-            if (it + 1 < per) move(it + 2, S2{}), __syncthreads();
-        if constexpr (PD > 3)
-            if (it + 2 < per) move(it + 3, S3{}), __syncthreads();
-        return;
-    }
-    const uint8_t *wb = wbase + (size_t)kb0 * T::TILE_BYTES;
-    typename T::Tile w[PF];
-#pragma unroll
-    for (int i = 0; i < PF; i++) T::load(w[i], wb + (size_t)min(i, last) * T::TILE_BYTES, lane);
-    __syncthreads();
-    auto body = [&](int it, auto uc) {
-        constexpr int u = decltype(uc)::value;
-        T::template mma_wide<MT>(acc, w[u], lds_all + (it & 1) * PV, 2 * PV, nMT, lane);
-        T::load(w[u], wb + (size_t)min(it + PF, last) * T::TILE_BYTES, lane);
-        __syncthreads();
-    };
-    int it = 0;
-    for (; it + PF <= per; it += PF) {
-        if constexpr (PF > 0) body(it + 0, std::integral_constant<int, 0>{});
-        if constexpr (PF > 1) body(it + 1, std::integral_constant<int, 1>{});
-        if constexpr (PF > 2) body(it + 2, std::integral_constant<int, 2>{});
-    }
-    if constexpr (PF > 1)
-        if (it + 0 < per) body(it + 0, std::integral_constant<int, 0>{});
-    if constexpr (PF > 2)
-        if (it + 1 < per) body(it + 1, std::integral_constant<int, 1>{});
-}
-
-// Grid (ceil(N/(32*TPB)), splits), block (TPB+MT)*64 threads. M-tile mt's rows go to P + mt*pStride (floats), laid out as the
-// narrow kernel lays out its 32 rows; its panels are read at Xp + mt*xpStride (bytes). M: rows in all (<= 32*MT).
-template <class T, int TPB, int MT, int PF>
-__device__ __forceinline__ void gemm_body_wide(const uint8_t *__restrict__ Wt, const void *__restrict__ aux, const uint8_t *__restrict__ Xp, size_t xpStride,
-                                               float *__restrict__ P, size_t pStride, int N, int nKB, int kbPerSplit, int M, int ldP, uint4_t *lds) {
-    static_assert(PF <= 3, "the wide loop unrolls up to three tiles in flight");
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const int tile = blockIdx.x * TPB + wave % TPB, split = blockIdx.y;
-    const int kb0 = split * kbPerSplit, kb1 = min(nKB, kb0 + kbPerSplit);
-    const bool active = tile * 32 < N;
-    const int nMT = (M + 31) >> 5;
-    float16_t acc[MT];
-    const int ltile = active ? tile : (N >> 5) - 1;
-    gemm_mainloop_wide<T, TPB, MT, PF>(acc, Wt + (size_t)ltile * nKB * T::TILE_BYTES, Xp, xpStride, kb0, kb1, nMT, lds);
-    if (active && wave < TPB) {
-#pragma unroll
-        for (int mt = 0; mt < MT; mt++) {
-            if (mt >= nMT) break;
-            T::finish(acc[mt], aux, tile, lane);
-            float *out = P + (size_t)mt * pStride + (size_t)split * 32 * ldP + tile * 32 + (lane & 31);
-            const int rows = min(32, M - 32 * mt);
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                int m = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-                if (m < rows) out[(size_t)m * ldP] = acc[mt][r];
-            }
         }
     }
 }

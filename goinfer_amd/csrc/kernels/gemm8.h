@@ -1,0 +1,413 @@
+// gemm8.h — the decode GEMMs in the reference's own arithmetic: int8 activation codes x integer weight codes on the int8
+// matrix cores, an exact int32 dot per group of 32, folded in f32 by the group's two scales
+// (goinfer backend/cuda/actgroup.cu:298-355 rowQ4K: facc += idot_g * ((d*sc_g) * aS_g); facc += -(dmin*m_g) * asum_g).
+//
+// Activations arrive as A8 blocks (a8.h): int8 codes in MFMA operand order, a scale and a scaled code sum per group of 32.
+//
+// One MFMA gives the 32x32 int32 dots of one group (32 batch rows x 32 weight rows). The products of the two scales, one per
+// (batch row, weight row, group), are an outer product: v_mfma_f32_32x32x1_2b_f32 forms them for two groups at once in the
+// accumulator layout, so the fold costs a convert and an fma per output and group. The -dmin*m term is a small f32 matrix
+// product over the groups and rides v_mfma_f32_32x32x2_f32 into the same accumulators.
+//
+// A block is KW waves per 32-row weight tile, each on its own K range with its own operands straight from global memory (no
+// LDS staging, no barrier in the loop); their partial sums are folded through LDS in ascending wave order. The order of every
+// output's sum is fixed by (split, wave, super-block, group) and independent of M: a row in a batch is the row alone, bit for bit.
+#pragma once
+#include "act.h"
+
+typedef int i32x4_t __attribute__((ext_vector_type(4)));
+typedef int i32x16_t __attribute__((ext_vector_type(16)));
+typedef float f32x32_t __attribute__((ext_vector_type(32)));
+
+// A8 blocks back to rows, for checking what a producer wrote: codes int8 [M][K], scales and sums f32 [M][K/32].
+// Grid (ceil(K/256), M), block 256.
+extern "C" __global__ void rd_k_unpack_act8(const uint8_t *__restrict__ A8, signed char *__restrict__ codes, float *__restrict__ scales,
+                                            float *__restrict__ sums, int K) {
+    const int m = blockIdx.y, k = blockIdx.x * 256 + threadIdx.x;
+    if (k >= K) return;
+    codes[(size_t)m * K + k] = (signed char)A8[a8_code_offset(m, k)];
+    if ((k & 31) == 0) {
+        const uint8_t *p = A8 + a8_scale_offset(m, k >> 5);
+        scales[(size_t)m * (K >> 5) + (k >> 5)] = *(const float *)p;
+        sums[(size_t)m * (K >> 5) + (k >> 5)] = *(const float *)(p + (RD_A8_SUMS - RD_A8_SCALES));
+    }
+}
+
+// A8 blocks as the values a consumer multiplies: out[m][k] = code * scale (f32). Grid (ceil(K/256), M), block 256.
+extern "C" __global__ void rd_k_unpanel_a8(const uint8_t *__restrict__ A8, float *__restrict__ out, int K) {
+    const int m = blockIdx.y, k = blockIdx.x * 256 + threadIdx.x;
+    if (k >= K) return;
+    out[(size_t)m * K + k] = __fmul_rn((float)(signed char)A8[a8_code_offset(m, k)], *(const float *)(A8 + a8_scale_offset(m, k >> 5)));
+}
+
+// Operands are read through buffer descriptors that cover exactly the K range of the wave: a prefetch past the end of the range
+// is answered with zeros by the address check and touches no memory, so the loop issues every load unconditionally and the
+// compiler's count of loads in flight stays exact (a branch around a load makes it wait for everything).
+typedef __amdgpu_buffer_rsrc_t rd_rsrc_t;
+__device__ __forceinline__ rd_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ uint4_t buf_load16(rd_rsrc_t r, int voff, int imm) {
+    return __builtin_amdgcn_raw_buffer_load_b128(r, voff + imm, 0, 0);
+}
+__device__ __forceinline__ uint4_t buf_load16_nt(rd_rsrc_t r, int voff, int imm) { // streamed once: weights
+    return __builtin_amdgcn_raw_buffer_load_b128(r, voff + imm, 0, 2);
+}
+
+struct A8Regs {
+    uint4_t c[8];
+    float4_t as, asum;
+};
+// voff: byte offset of the block inside the descriptor's range plus lane * 16
+__device__ __forceinline__ void a8_load(A8Regs &a, rd_rsrc_t r, int voff) {
+#pragma unroll
+    for (int g = 0; g < 8; g++) a.c[g] = buf_load16(r, voff, g * 1024);
+    uint4_t s = buf_load16(r, voff, RD_A8_SCALES), u = buf_load16(r, voff, RD_A8_SUMS);
+    __builtin_memcpy(&a.as, &s, 16);
+    __builtin_memcpy(&a.asum, &u, 16);
+}
+
+__device__ __forceinline__ i32x4_t as_i32x4(uint4_t v) {
+    i32x4_t r;
+    __builtin_memcpy(&r, &v, 16);
+    return r;
+}
+
+// acc += fold of one group's dots: a convert and an fma per output (the scale products come from the matrix core)
+#define RD_FOLD16(ACC, DOT, S, OFF)                                                    \
+    _Pragma("unroll") for (int r_ = 0; r_ < 16; r_++) ACC[r_] = __builtin_fmaf((float)DOT[r_], S[(OFF) + r_], ACC[r_]);
+
+// ---------------- Q4_K ----------------
+// Tile of 32 rows x one super-block, 4608 B: the 32 headers (16 B: d, dmin, 12 scale bytes), then four planes [64 lanes][16 B]:
+// plane p, lane (row r, half h) holds raw code bytes [32p + 16h, +16) of row r, i.e. elements 16h..16h+15 of sub-block 2p in
+// the low nibbles and of sub-block 2p+1 in the high nibbles. Same bytes as the file, same 4.5 bits per weight.
+extern "C" __global__ void rd_k_retile_q4k8(const uint8_t *__restrict__ raw, uint8_t *__restrict__ tiled, int N, int nSB) {
+    const int tile = blockIdx.x, sb = blockIdx.y, t = threadIdx.x; // 288 x 16 B
+    if (t >= 288) return;
+    uint8_t *dst = tiled + ((size_t)tile * nSB + sb) * 4608;
+    const uint4_t *src;
+    if (t < 32) {
+        src = (const uint4_t *)(raw + ((size_t)(tile * 32 + t) * nSB + sb) * 144);
+    } else {
+        const int u = t - 32, p = u >> 6, lane = u & 63, r = lane & 31, h = lane >> 5;
+        src = (const uint4_t *)(raw + ((size_t)(tile * 32 + r) * nSB + sb) * 144 + 16 + p * 32 + h * 16);
+    }
+    *(uint4_t *)(dst + (size_t)t * 16) = *src;
+}
+
+struct Q4K8Tile {
+    uint4_t hdr, q[4];
+};
+
+struct Q4K8Traits {
+    typedef Q4K8Tile Tile;
+    static constexpr int TILE_BYTES = 4608;
+    // off: byte offset of the tile inside the descriptor's range
+    static __device__ __forceinline__ void load(Tile &w, rd_rsrc_t r, int off, int lane) {
+        w.hdr = buf_load16_nt(r, off + (lane & 31) * 16, 0);
+#pragma unroll
+        for (int c = 0; c < 4; c++) w.q[c] = buf_load16_nt(r, off + lane * 16, 512 + c * 1024);
+    }
+    // acc[m][n] += sum over the super-block's 8 groups. Lane (n, h) decodes the scales of sub-blocks 2p+h, p = 0..3: the
+    // lane half is the block index of the two-block scale product and the k index of the minimum product.
+    static __device__ __forceinline__ void mma(float16_t &acc, const Tile &w, const A8Regs &a, const void *, int, int lane) {
+        const int h = lane >> 5;
+        const uint32_t y = w.hdr.y, z = w.hdr.z, x = w.hdr.w, hx = w.hdr.x;
+        half2_t dd;
+        __builtin_memcpy(&dd, &hx, 4);
+        const float d = (float)dd.x, dmin = (float)dd.y;
+        float dsc[4], ndm[4];
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            int sc, mn;
+            if (p < 2) { // sub-blocks 0..3
+                const int j8 = 8 * (2 * p);
+                const int sc0 = (y >> j8) & 63, sc1 = (y >> (j8 + 8)) & 63, m0 = (z >> j8) & 63, m1 = (z >> (j8 + 8)) & 63;
+                sc = h ? sc1 : sc0, mn = h ? m1 : m0;
+            } else { // sub-blocks 4..7
+                const int j8 = 8 * (2 * p - 4);
+                const int sc0 = ((x >> j8) & 15) | (((y >> (j8 + 6)) & 3) << 4), sc1 = ((x >> (j8 + 8)) & 15) | (((y >> (j8 + 14)) & 3) << 4);
+                const int m0 = ((x >> (j8 + 4)) & 15) | (((z >> (j8 + 6)) & 3) << 4), m1 = ((x >> (j8 + 12)) & 15) | (((z >> (j8 + 14)) & 3) << 4);
+                sc = h ? sc1 : sc0, mn = h ? m1 : m0;
+            }
+            dsc[p] = __fmul_rn(d, (float)sc);
+            ndm[p] = -__fmul_rn(dmin, (float)mn);
+        }
+        const f32x32_t zero32 = {0.f};
+        const i32x16_t zero16 = {0};
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            const f32x32_t s2 = __builtin_amdgcn_mfma_f32_32x32x1f32(a.as[p], dsc[p], zero32, 0, 0, 0);
+            const uint4_t raw = w.q[p];
+            uint4_t lo, hi;
+#pragma unroll
+            for (int i = 0; i < 4; i++) lo[i] = raw[i] & 0x0F0F0F0Fu, hi[i] = (raw[i] >> 4) & 0x0F0F0F0Fu;
+            const i32x16_t d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(as_i32x4(a.c[2 * p]), as_i32x4(lo), zero16, 0, 0, 0);
+            const i32x16_t d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(as_i32x4(a.c[2 * p + 1]), as_i32x4(hi), zero16, 0, 0, 0);
+            RD_FOLD16(acc, d0, s2, 0)
+            RD_FOLD16(acc, d1, s2, 16)
+        }
+#pragma unroll
+        for (int p = 0; p < 4; p++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.asum[p], ndm[p], acc, 0, 0, 0);
+    }
+    static __device__ __forceinline__ void finish(float16_t &, const void *, int, int) {}
+};
+
+// ---------------- W8A8: int8 codes, one f32 scale per row (goinfer WeightMat.Int8; backend/cuda/actgroup.cu:283-288,421-437) ----------------
+// Tile of 32 rows x 256 k, 8192 B: eight planes [64 lanes][16 B], plane g lane (row r, half h) = codes of elements 16h..16h+15 of
+// group g of the block. K is padded to a multiple of 256 with zero codes. facc += idot_g * aS_g; dst = facc * wScale[n].
+extern "C" __global__ __launch_bounds__(512) void rd_k_retile_w8a8_8(const uint8_t *__restrict__ raw, uint8_t *__restrict__ tiled, int N, int K) {
+    const int tile = blockIdx.x, kb = blockIdx.y, t = threadIdx.x; // 512 x 16 B
+    const int g = t >> 6, lane = t & 63, r = lane & 31, h = lane >> 5, k0 = kb * 256 + g * 32 + h * 16;
+    uint4_t v = {0u, 0u, 0u, 0u};
+    if (k0 < K) v = *(const uint4_t *)(raw + (size_t)(tile * 32 + r) * K + k0); // K % 32 == 0: a 16-byte run is inside K or past it
+    *(uint4_t *)(tiled + ((size_t)tile * gridDim.y + kb) * 8192 + (size_t)t * 16) = v;
+}
+
+struct W8Tile8 {
+    uint4_t q[8];
+};
+struct W8A8Traits8 {
+    typedef W8Tile8 Tile;
+    static constexpr int TILE_BYTES = 8192;
+    static __device__ __forceinline__ void load(Tile &w, rd_rsrc_t r, int off, int lane) {
+#pragma unroll
+        for (int g = 0; g < 8; g++) w.q[g] = buf_load16_nt(r, off + lane * 16 + (g >> 2) * 4096, (g & 3) * 1024);
+    }
+    static __device__ __forceinline__ void mma(float16_t &acc, const Tile &w, const A8Regs &a, const void *, int, int lane) {
+        const f32x32_t zero32 = {0.f};
+        const i32x16_t zero16 = {0};
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            // the activation scale of every (batch row, group) spread over the accumulator layout: a product with one
+            const f32x32_t s2 = __builtin_amdgcn_mfma_f32_32x32x1f32(a.as[p], 1.f, zero32, 0, 0, 0);
+            const i32x16_t d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(as_i32x4(a.c[2 * p]), as_i32x4(w.q[2 * p]), zero16, 0, 0, 0);
+            const i32x16_t d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(as_i32x4(a.c[2 * p + 1]), as_i32x4(w.q[2 * p + 1]), zero16, 0, 0, 0);
+            RD_FOLD16(acc, d0, s2, 0)
+            RD_FOLD16(acc, d1, s2, 16)
+        }
+    }
+    static __device__ __forceinline__ void finish(float16_t &acc, const void *aux, int tile, int lane) {
+        const float ws = ((const float *)aux)[tile * 32 + (lane & 31)];
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[r] = __fmul_rn(acc[r], ws);
+    }
+};
+
+// ---------------- W4A8: canonical int4 nibbles (value nib-8), binary16 scale per 32 (decoder/weightmat.go:160-178) ----------------
+// Tile of 32 rows x 256 k, 4608 B, the Q4_K tile's shape: 32 headers of 16 B (the row's eight group scales, f16), then four planes
+// [64 lanes][16 B]: plane p, lane (row r, half h), byte b = element 16h+b of group 2p in the low nibble and of group 2p+1 in the
+// high nibble (re-packed from the canonical order, element k in nibble k%2 of byte k/2, at upload). The dot runs on the stored
+// nibbles (0..15) and the -8 comes back as a term in the activation sums, exactly as Q4_K's minimum does:
+// sum_k (nib-8)*a = sum_k nib*a - 8*sum_k a, so  facc += ws_g*aS_g*idot_g;  facc += -(8*ws_g)*asum_g.  K padded to 256 with zeros.
+extern "C" __global__ __launch_bounds__(320) void rd_k_retile_w4a8_8(const uint8_t *__restrict__ nib, const uint16_t *__restrict__ s16,
+                                                                      uint8_t *__restrict__ tiled, int N, int K) {
+    const int tile = blockIdx.x, kb = blockIdx.y, t = threadIdx.x; // 288 x 16 B
+    if (t >= 288) return;
+    uint8_t *dst = tiled + ((size_t)tile * gridDim.y + kb) * 4608;
+    const int nG = K >> 5;
+    uint4_t v = {0u, 0u, 0u, 0u};
+    if (t < 32) {
+        uint16_t sc[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) sc[j] = kb * 8 + j < nG ? s16[(size_t)(tile * 32 + t) * nG + kb * 8 + j] : (uint16_t)0;
+        __builtin_memcpy(&v, sc, 16);
+    } else {
+        const int u = t - 32, p = u >> 6, lane = u & 63, r = lane & 31, h = lane >> 5;
+        const uint8_t *row = nib + (size_t)(tile * 32 + r) * (K >> 1);
+        uint8_t by[16];
+#pragma unroll
+        for (int b = 0; b < 16; b++) {
+            const int klo = kb * 256 + (2 * p) * 32 + h * 16 + b, khi = klo + 32;
+            const int lo = klo < K ? (row[klo >> 1] >> (4 * (klo & 1))) & 15 : 8, hi = khi < K ? (row[khi >> 1] >> (4 * (khi & 1))) & 15 : 8;
+            by[b] = (uint8_t)(lo | (hi << 4));
+        }
+        __builtin_memcpy(&v, by, 16);
+    }
+    *(uint4_t *)(dst + (size_t)t * 16) = v;
+}
+
+struct W4A8Traits8 {
+    typedef Q4K8Tile Tile;
+    static constexpr int TILE_BYTES = 4608;
+    static __device__ __forceinline__ void load(Tile &w, rd_rsrc_t r, int off, int lane) { Q4K8Traits::load(w, r, off, lane); }
+    static __device__ __forceinline__ void mma(float16_t &acc, const Tile &w, const A8Regs &a, const void *, int, int lane) {
+        const int h = lane >> 5;
+        float dsc[4], ndm[4];
+#pragma unroll
+        for (int p = 0; p < 4; p++) { // the scale of group 2p+h: half h of header word p
+            const uint32_t wd = w.hdr[p];
+            dsc[p] = f16_bits_to_f32((uint16_t)(h ? wd >> 16 : wd & 0xffffu));
+            ndm[p] = -8.f * dsc[p];
+        }
+        const f32x32_t zero32 = {0.f};
+        const i32x16_t zero16 = {0};
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            const f32x32_t s2 = __builtin_amdgcn_mfma_f32_32x32x1f32(a.as[p], dsc[p], zero32, 0, 0, 0);
+            const uint4_t raw = w.q[p];
+            uint4_t lo, hi;
+#pragma unroll
+            for (int i = 0; i < 4; i++) lo[i] = raw[i] & 0x0F0F0F0Fu, hi[i] = (raw[i] >> 4) & 0x0F0F0F0Fu;
+            const i32x16_t d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(as_i32x4(a.c[2 * p]), as_i32x4(lo), zero16, 0, 0, 0);
+            const i32x16_t d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(as_i32x4(a.c[2 * p + 1]), as_i32x4(hi), zero16, 0, 0, 0);
+            RD_FOLD16(acc, d0, s2, 0)
+            RD_FOLD16(acc, d1, s2, 16)
+        }
+#pragma unroll
+        for (int p = 0; p < 4; p++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.asum[p], ndm[p], acc, 0, 0, 0);
+    }
+    static __device__ __forceinline__ void finish(float16_t &, const void *, int, int) {}
+};
+
+// The K loop of one wave: two weight tiles and two activation blocks in registers, each refilled with the block two ahead as soon as
+// it has been multiplied. Loads are counted in issue order by the wave's wait counter, so a block's activations are asked for
+// before its weights: waiting for activations then never waits for younger weight tiles. The refills are unconditional (past
+// the end of the range the descriptor answers with zeros and touches no memory): only the second product of a round sits under
+// a branch, so the compiler's count of the loads in flight stays exact.
+template <class T>
+__device__ __forceinline__ void gemm8_wave_loop(float16_t &acc, const uint8_t *__restrict__ wb, const uint8_t *__restrict__ ab, int nk, const void *aux,
+                                                int tile, int lane) {
+#pragma unroll
+    for (int i = 0; i < 16; i++) acc[i] = 0.f;
+    if (nk <= 0) return;
+    constexpr int AB = RD_A8_BLOCK_BYTES;
+    const rd_rsrc_t wr = make_rsrc(wb, (uint32_t)nk * T::TILE_BYTES), ar = make_rsrc(ab, (uint32_t)nk * AB);
+    typename T::Tile w0, w1;
+    A8Regs a0, a1;
+    a8_load(a0, ar, lane * 16);
+    T::load(w0, wr, 0, lane);
+    a8_load(a1, ar, AB + lane * 16);
+    T::load(w1, wr, T::TILE_BYTES, lane);
+    for (int it = 0; it < nk; it += 2) {
+        T::mma(acc, w0, a0, aux, tile, lane);
+        a8_load(a0, ar, (it + 2) * AB + lane * 16);
+        T::load(w0, wr, (it + 2) * T::TILE_BYTES, lane);
+        if (it + 1 < nk) T::mma(acc, w1, a1, aux, tile, lane);
+        a8_load(a1, ar, (it + 3) * AB + lane * 16);
+        T::load(w1, wr, (it + 3) * T::TILE_BYTES, lane);
+    }
+}
+
+// Folds the KW waves' partial sums of each tile into the tile's first wave, ascending wave order, through LDS
+// (xch: TPB*(KW-1)*1024 floats). Every wave of the block calls it.
+template <int KW, int TPB>
+__device__ __forceinline__ void gemm8_fold_waves(float16_t &acc, float *xch) {
+    if constexpr (KW > 1) {
+        const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, t = wave / KW, kw = wave % KW;
+        float4_t *x4 = (float4_t *)xch;
+        if (kw > 0) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) x4[((t * (KW - 1) + kw - 1) * 4 + q) * 64 + lane] = (float4_t){acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]};
+        }
+        __syncthreads();
+        if (kw == 0) {
+#pragma unroll
+            for (int k2 = 1; k2 < KW; k2++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const float4_t v = x4[((t * (KW - 1) + k2 - 1) * 4 + q) * 64 + lane];
+                    acc[4 * q] += v.x, acc[4 * q + 1] += v.y, acc[4 * q + 2] += v.z, acc[4 * q + 3] += v.w;
+                }
+        }
+    }
+}
+
+// Grid (ceil(N/(32*TPB)), splits), block KW*TPB waves. P[split][32][ldP] receives the sums of K-blocks [split*kbPerSplit, +kbPerSplit).
+// resid != NULL (splits must be 1): the sums are added to resid[m][n] in place instead (the residual stream), nothing goes to P.
+template <class T, int KW, int TPB>
+__device__ __forceinline__ void gemm8_body(const uint8_t *__restrict__ Wt, const void *__restrict__ aux, const uint8_t *__restrict__ A8,
+                                           float *__restrict__ P, int N, int nKB, int kbPerSplit, int M, int ldP, float *__restrict__ resid, float *lds) {
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int tile = blockIdx.x * TPB + wave / KW, kw = wave % KW, split = blockIdx.y;
+    const int kb0 = split * kbPerSplit, kb1 = min(nKB, kb0 + kbPerSplit);
+    const int per = (max(kb1 - kb0, 0) + KW - 1) / KW;
+    const int s0 = kb0 + kw * per, nk = max(0, min(kb1, s0 + per) - s0);
+    const bool active = tile * 32 < N;
+    float16_t acc;
+    gemm8_wave_loop<T>(acc, Wt + ((size_t)(active ? tile : 0) * nKB + s0) * T::TILE_BYTES, A8 + (size_t)s0 * RD_A8_BLOCK_BYTES,
+                           active ? nk : 0, aux, tile, lane);
+    gemm8_fold_waves<KW, TPB>(acc, lds);
+    if (!active || kw != 0) return;
+    T::finish(acc, aux, tile, lane);
+    const int n = tile * 32 + (lane & 31);
+    if (resid) {
+        float old[16]; // all sixteen reads in flight before the first add
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int m = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+            old[r] = resid[(size_t)min(m, M - 1) * ldP + n];
+        }
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int m = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+            if (m < M) resid[(size_t)m * ldP + n] = __fadd_rn(old[r], acc[r]);
+        }
+        return;
+    }
+    float *out = P + (size_t)split * 32 * ldP + n;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const int m = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+        if (m < M) out[(size_t)m * ldP] = acc[r];
+    }
+}
+
+#define RD_GEMM8_KERNEL(NAME, TRAITS, KW, TPB)                                                                                                       \
+    extern "C" __global__ __launch_bounds__(64 * KW * TPB) void NAME(const uint8_t *__restrict__ Wt, const void *__restrict__ aux,                   \
+                                                                     const uint8_t *__restrict__ A8, float *__restrict__ P, int N, int nKB,         \
+                                                                     int kbPerSplit, int M, int ldP, float *__restrict__ resid) {                   \
+        __shared__ float lds[(KW > 1 ? TPB * (KW - 1) * 1024 : 1)];                                                                                  \
+        gemm8_body<TRAITS, KW, TPB>(Wt, aux, A8, P, N, nKB, kbPerSplit, M, ldP, resid, lds);                                                     \
+    }
+
+RD_GEMM8_KERNEL(rd_k_gemm8_q4k_kw2, Q4K8Traits, 2, 2)
+RD_GEMM8_KERNEL(rd_k_gemm8_q4k_kw4, Q4K8Traits, 4, 1)
+RD_GEMM8_KERNEL(rd_k_gemm8_q4k_kw8, Q4K8Traits, 8, 1)
+RD_GEMM8_KERNEL(rd_k_gemm8_w8a8_kw2, W8A8Traits8, 2, 2)
+RD_GEMM8_KERNEL(rd_k_gemm8_w8a8_kw4, W8A8Traits8, 4, 1)
+RD_GEMM8_KERNEL(rd_k_gemm8_w8a8_kw8, W8A8Traits8, 8, 1)
+RD_GEMM8_KERNEL(rd_k_gemm8_w4a8_kw2, W4A8Traits8, 2, 2)
+RD_GEMM8_KERNEL(rd_k_gemm8_w4a8_kw4, W4A8Traits8, 4, 1)
+RD_GEMM8_KERNEL(rd_k_gemm8_w4a8_kw8, W4A8Traits8, 8, 1)
+
+// ---------------- fused gate|up projection + SwiGLU + per-32 quantization ----------------
+// goinfer decoder/cpu_gateup_fused.go:83-148 in one launch. W holds [gate rows; up rows] (2*I rows). Grid (I/32), block 2*KW waves:
+// waves 0..KW-1 own gate tile t over K (each its own range), waves KW..2KW-1 the matching up tile. After the fold both finished
+// tiles meet in LDS in accumulator order, and every wave takes two of the sixteen accumulator registers: in that order a
+// half-wave holds the 32 columns of one batch row, which is exactly one activation group of the down projection, so
+// silu(gate)*up (silu in f64, decoder/rmsnorm.go:204-207) is quantized where it sits and written in the layout the down projection reads.
+// The K loop, its wave ranges and the fold are those of the plain kernel with the same KW: the sums are the same bits.
+template <class T, int KW>
+__device__ __forceinline__ void gemm8_gateup_body(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ A8, uint8_t *__restrict__ XpOut, int outKind,
+                                                  int I, int nKB, int M, float *lds) {
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int half = wave / KW, kw = wave % KW, t = blockIdx.x, nGate = I >> 5, tile = half * nGate + t;
+    const int per = (nKB + KW - 1) / KW, s0 = kw * per, nk = max(0, min(nKB, s0 + per) - s0);
+    float16_t acc;
+    gemm8_wave_loop<T>(acc, Wt + ((size_t)tile * nKB + s0) * T::TILE_BYTES, A8 + (size_t)s0 * RD_A8_BLOCK_BYTES, nk, nullptr, tile, lane);
+    gemm8_fold_waves<KW, 2>(acc, lds);
+    __syncthreads(); // the fold area is read; it now takes the two finished tiles as [gate | up][register][lane]
+    if (kw == 0) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) lds[(half * 16 + r) * 64 + lane] = acc[r];
+    }
+    __syncthreads();
+    constexpr int RPW = 16 / (2 * KW) > 0 ? 16 / (2 * KW) : 1; // accumulator registers per wave
+    const int n = t * 32 + (lane & 31);
+#pragma unroll
+    for (int j = 0; j < RPW; j++) {
+        const int r = wave * RPW + j;
+        if (r >= 16) break;
+        const int m = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+        const float a = __fmul_rn(silu_f64(lds[r * 64 + lane]), lds[(16 + r) * 64 + lane]);
+        const Quant1 q = quant_one(a);
+        if (m < M) panel_store(XpOut, outKind, m, n, q);
+    }
+}
+
+extern "C" __global__ __launch_bounds__(512) void rd_k_gemm8_q4k_gateup(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ A8,
+                                                                         uint8_t *__restrict__ XpOut, int outKind, int I, int nKB, int M) {
+    __shared__ float lds[2 * 3 * 1024];
+    gemm8_gateup_body<Q4K8Traits, 4>(Wt, A8, XpOut, outKind, I, nKB, M, lds);
+}

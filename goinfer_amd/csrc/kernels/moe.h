@@ -4,7 +4,7 @@
 // every expert's weights are streamed exactly once per step. rankOf[token][expert] (from rd_k_moe_route) is the map.
 #pragma once
 #include "act.h"
-#include "lin.h"
+#include "gemm8.h"
 
 // out[(token*k + rank)][N] = panels . W_e^T for the experts that have at least one token. Grid (ceil(N/128), nE), block 320 (four consumer waves and a panel producer).
 // xpStride: bytes between the experts' panel sets (0 = all experts read the same panels: the gate/up projections).
@@ -32,82 +32,86 @@ __device__ __forceinline__ int moe_block_expert(const unsigned *__restrict__ act
     return __syncthreads_or(mine) ? e : -1;
 }
 
-template <int TPB, int PF>
-__device__ __forceinline__ void moe_gemm_body(const uint8_t *__restrict__ Wt, size_t wStride, const uint8_t *__restrict__ Xp, size_t xpStride,
-                                              float *__restrict__ out, int N, int nKB, int T, int k, const signed char *__restrict__ rankOf, int nE,
-                                              const unsigned *__restrict__ activeBits, uint4_t *lds) {
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    // perExpertPanels: every expert reads panels of its own, so all blocks of an expert are placed on one XCD (blocks go to the
-    // eight XCDs round-robin in linear order) and its panels are pulled into one L2 instead of eight.
+// Per expert the weights are W4A8 tiles of the int8-MFMA kernels (gemm8.h: 4608 B per 32 rows x 256 k), the activations A8 blocks.
+// Block: TPB tiles x KW waves, every wave on its own K range, partial sums folded through LDS in wave order (as gemm8_body).
+template <int KW, int TPB>
+__device__ __forceinline__ void moe_gemm8_body(const uint8_t *__restrict__ Wt, size_t wStride, const uint8_t *__restrict__ A8, size_t a8Stride,
+                                               float *__restrict__ out, int N, int nKB, int T, int k, const signed char *__restrict__ rankOf, int nE,
+                                               const unsigned *__restrict__ activeBits, float *lds) {
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    // a8Stride != 0: every expert reads activations of its own, so all blocks of an expert are placed on one XCD (blocks go to the
+    // eight XCDs round-robin in linear order) and its activation blocks are pulled into one L2 instead of eight.
     int bx = blockIdx.x, row = blockIdx.y;
-    if (xpStride != 0 && (gridDim.y & 7) == 0) {
+    if (a8Stride != 0 && (gridDim.y & 7) == 0) {
         const int gx = gridDim.x, L = row * gx + bx, j = L >> 3;
         row = (j / gx) * 8 + (L & 7), bx = j % gx;
     }
     const int e = moe_block_expert(activeBits, rankOf, nE, T, row);
     if (e < 0) return;
-    const int tile = bx * TPB + (wave % TPB);
+    const int tile = bx * TPB + wave / KW, kw = wave % KW;
     const bool active = tile * 32 < N;
+    const int per = (nKB + KW - 1) / KW, s0 = kw * per, nk = max(0, min(nKB, s0 + per) - s0);
     float16_t acc;
-    const int ltile = active ? tile : (N >> 5) - 1;
-    gemm_mainloop_pc<W4MoeTraits, TPB, 1, PF>(acc, Wt + (size_t)e * wStride + (size_t)ltile * nKB * W4Traits::TILE_BYTES, Xp + (size_t)e * xpStride, 0,
-                                              nKB, lds);
-    if (!active || wave >= TPB) return;
+    gemm8_wave_loop<W4A8Traits8>(acc, Wt + (size_t)e * wStride + ((size_t)(active ? tile : 0) * nKB + s0) * W4A8Traits8::TILE_BYTES,
+                                 A8 + (size_t)e * a8Stride + (size_t)s0 * RD_A8_BLOCK_BYTES, active ? nk : 0, nullptr, tile, lane);
+    gemm8_fold_waves<KW, TPB>(acc, lds);
+    if (!active || kw != 0) return;
 #pragma unroll
     for (int r = 0; r < 16; r++) {
-        int m = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+        const int m = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
         if (m < T) {
-            int rank = rankOf[(size_t)m * nE + e];
+            const int rank = rankOf[(size_t)m * nE + e];
             if (rank >= 0) out[((size_t)m * k + rank) * N + tile * 32 + (lane & 31)] = acc[r];
         }
     }
 }
 
-extern "C" __global__ __launch_bounds__(320) __attribute__((amdgpu_waves_per_eu(7, 7))) void rd_k_gemm_w4a8_moe(const uint8_t *__restrict__ Wt, size_t wStride, const uint8_t *__restrict__ Xp,
-                                                                      size_t xpStride, float *__restrict__ out, int N, int nKB, int T, int k,
-                                                                      const signed char *__restrict__ rankOf, int nE,
-                                                                      const unsigned *__restrict__ activeBits) {
-    __shared__ uint4_t lds[2 * RD_LIN_PANEL_BYTES / 16];
-    moe_gemm_body<4, 3>(Wt, wStride, Xp, xpStride, out, N, nKB, T, k, rankOf, nE, activeBits, lds);
+// out[(token*k + rank)][N] = A8 . W_e^T for the experts that have at least one token. Grid (ceil(N/64), nE), block 256 (two tiles x two waves).
+// a8Stride: bytes between the experts' activation sets (0 = all experts read the same activations: the gate/up projections).
+extern "C" __global__ __launch_bounds__(256) void rd_k_gemm8_w4a8_moe(const uint8_t *__restrict__ Wt, size_t wStride, const uint8_t *__restrict__ A8,
+                                                                       size_t a8Stride, float *__restrict__ out, int N, int nKB, int T, int k,
+                                                                       const signed char *__restrict__ rankOf, int nE,
+                                                                       const unsigned *__restrict__ activeBits) {
+    __shared__ float lds[2 * 1024];
+    moe_gemm8_body<2, 2>(Wt, wStride, A8, a8Stride, out, N, nKB, T, k, rankOf, nE, activeBits, lds);
 }
-// The experts' gate|up projection with SwiGLU and the per-32 quantization in its epilogue (the expert twin of rd_k_gemm_q4k_gateup;
-// same values as rd_k_gemm_w4a8_moe followed by rd_k_moe_swiglu_quant, bit for bit). Wt per expert: [gate rows; up rows] (2*I rows).
-// Grid (I/64, nE), block 320: waves 0,1 own gate tiles 2x, 2x+1 of the block's expert, waves 2,3 the matching up tiles, over all
-// of K; the sums meet in LDS, and for every token routed to the expert one wave computes silu(gate)*up for the block's 64
-// columns (two activation groups), quantizes them and writes them into the expert's down-projection panels XpE. I % 64 == 0.
-extern "C" __global__ __launch_bounds__(320) void rd_k_gemm_w4a8_moe_gateup(const uint8_t *__restrict__ Wt, size_t wStride,
-                                                                             const uint8_t *__restrict__ Xp, uint8_t *__restrict__ XpE,
-                                                                             size_t xpeStride, int I, int nKB, int T,
-                                                                             const signed char *__restrict__ rankOf, int nE,
-                                                                             const unsigned *__restrict__ activeBits) {
-    __shared__ uint4_t lds[2 * RD_LIN_PANEL_BYTES / 16];
-    static_assert(2 * RD_LIN_PANEL_BYTES >= 4 * 32 * 32 * 4, "the four finished tiles are exchanged through the panel buffers");
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, wt = wave & 3;
+
+// The experts' gate|up projection with SwiGLU and the per-32 quantization in its epilogue (the expert twin of rd_k_gemm8_q4k_gateup;
+// same values as rd_k_gemm8_w4a8_moe followed by rd_k_moe_swiglu_quant, bit for bit: both cut K over two waves). Wt per expert:
+// [gate rows; up rows] (2*I rows). Grid (I/32, nE), block 256: waves 0,1 own gate tile x of the block's expert, waves 2,3 the
+// matching up tile; the finished tiles meet in LDS in accumulator order, every wave takes four accumulator registers, and the
+// rows routed to the expert are quantized (a half-wave holds the 32 columns of one row = one activation group) and written into
+// the expert's down-projection activations A8E.
+extern "C" __global__ __launch_bounds__(256) void rd_k_gemm8_w4a8_moe_gateup(const uint8_t *__restrict__ Wt, size_t wStride,
+                                                                              const uint8_t *__restrict__ A8, uint8_t *__restrict__ A8E,
+                                                                              size_t a8eStride, int I, int nKB, int T,
+                                                                              const signed char *__restrict__ rankOf, int nE,
+                                                                              const unsigned *__restrict__ activeBits) {
+    __shared__ float lds[2 * 1024];
+    constexpr int KW = 2;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int e = moe_block_expert(activeBits, rankOf, nE, T, blockIdx.y);
     if (e < 0) return;
-    const int nGate = I >> 5, tile = (wt >> 1) * nGate + blockIdx.x * 2 + (wt & 1);
+    const int half = wave / KW, kw = wave % KW, t = blockIdx.x, nGate = I >> 5, tile = half * nGate + t;
+    const int per = (nKB + KW - 1) / KW, s0 = kw * per, nk = max(0, min(nKB, s0 + per) - s0);
     float16_t acc;
-    gemm_mainloop_pc<W4MoeTraits, 4, 1, 3>(acc, Wt + (size_t)e * wStride + (size_t)tile * nKB * W4Traits::TILE_BYTES, Xp, 0, nKB, lds);
-    __syncthreads(); // every wave is done with the panels
-    float *xe = (float *)lds; // [tile wt][row m][column c]
-    if (wave < 4) {
+    gemm8_wave_loop<W4A8Traits8>(acc, Wt + (size_t)e * wStride + ((size_t)tile * nKB + s0) * W4A8Traits8::TILE_BYTES, A8 + (size_t)s0 * RD_A8_BLOCK_BYTES, nk,
+                                 nullptr, tile, lane);
+    gemm8_fold_waves<KW, 2>(acc, lds);
+    __syncthreads();
+    if (kw == 0) {
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int m = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-            xe[(wt * 32 + m) * 32 + (lane & 31)] = acc[r];
-        }
+        for (int r = 0; r < 16; r++) lds[(half * 16 + r) * 64 + lane] = acc[r];
     }
     __syncthreads();
-    if (wave >= 4) return;
-    unsigned long long routed = __ballot(lane < T && rankOf[(size_t)lane * nE + e] >= 0);
-    const int tl = lane >> 5, c = lane & 31;
-    for (int ord = 0; routed; ord++) {
-        const int m = __ffsll((long long)routed) - 1;
-        routed &= routed - 1;
-        if ((ord & 3) != wave) continue; // the routed rows go round the four waves
-        const float a = __fmul_rn(silu_f64(xe[(tl * 32 + m) * 32 + c]), xe[((2 + tl) * 32 + m) * 32 + c]);
-        float gs, xh = quant_g32(a, &gs); // a half-wave holds the 32 columns of one tile = one activation group
-        panel_store(XpE + (size_t)e * xpeStride, RD_PANEL_LIN4, m, (blockIdx.x * 2 + tl) * 32 + c, xh, gs);
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int r = wave * 4 + j, m = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+        const bool routed = m < T && rankOf[(size_t)m * nE + e] >= 0;
+        if (__ballot(routed) == 0) continue; // no row of this register is routed here: skip the f64 silu
+        const float a = __fmul_rn(silu_f64(lds[r * 64 + lane]), lds[(16 + r) * 64 + lane]);
+        const Quant1 q = quant_one(a);
+        if (routed) panel_store(A8E + (size_t)e * a8eStride, RD_PANEL_A8, m, t * 32 + (lane & 31), q);
     }
 }
 
@@ -121,8 +125,8 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_moe_swiglu_quant(const fl
         float g = gu[(size_t)row * 2 * I + n], u = gu[(size_t)row * 2 * I + I + n];
         a = __fmul_rn(silu_f64(g), u);
     }
-    float gs, xh = quant_g32(a, &gs);
-    if (n < I) panel_store(XpE + (size_t)e * xpStride, RD_PANEL_LIN4, t, n, xh, gs);
+    const Quant1 q = quant_one(a);
+    if (n < I) panel_store(XpE + (size_t)e * xpStride, RD_PANEL_A8, t, n, q);
 }
 
 // out[t][:] = sum over ranks, in rank order, of wgt[t][rank] * down[(t,rank)][:]  (decoder/mlp.go:100-103, addScaled: mul then add).

@@ -3,9 +3,9 @@
 // hipModuleGetFunction.
 #include "common.h"
 #include "q4k.h"
-#include "lin.h"
-#include "kquant.h"
 #include "act.h"
+#include "gemm8.h"
+#include "kquant.h"
 #include "attn.h"
 #include "misc.h"
 #include "moe.h"
@@ -20,7 +20,6 @@ extern "C" __global__ __launch_bounds__(512) void rd_k_attn_combine_quant(const 
     const int head = blockIdx.x, m = blockIdx.y;
     float v[4];
     if (!attn_combine_block(part, itemStart, partRows, nH, nKV, HD, m, head, lds, v)) return;
-    float x0, x1, x2, x3, gs;
-    quant_g32x4(v[0], v[1], v[2], v[3], &x0, &x1, &x2, &x3, &gs);
-    panel_store4(Xp + (size_t)(m >> 5) * xpStride, kind, m & 31, head * HD + threadIdx.x * 4, x0, x1, x2, x3, gs); // M-tile m/32, row m%32
+    const Quant4 q = quant_four(v[0], v[1], v[2], v[3]);
+    panel_store4(Xp + (size_t)(m >> 5) * xpStride, kind, m & 31, head * HD + threadIdx.x * 4, q); // M-tile m/32, row m%32
 }

@@ -90,6 +90,11 @@ int rd_dequant_q5k(rd_device *d, const void *blocks, int N, int K, float *out);
 int rd_dequant_q6k(rd_device *d, const void *blocks, int N, int K, float *out);
 int rd_gemm_q5k(rd_device *d, const void *W, int N, int K, const float *a, int M, float *dst);
 int rd_gemm_q6k(rd_device *d, const void *W, int N, int K, const float *a, int M, float *dst);
+/* The per-32 activation quantizer every int projection's input goes through (aikit QuantizeActQ group 32, call sites
+ * decoder/weightmat.go:845-862, cpu_gateup_fused.go:110-117; device twin backend/cuda/actgroup.cu:32-54 quantG32 — with the CPU
+ * path's round-half-away, not the twin's round-to-even): a host f32 [M][K] -> codes int8 [M][K], scales f32 [M][K/32]
+ * (maxabs/127, 0 for an all-zero group) and sums f32 [M][K/32] (scale * sum of the group's codes). K a multiple of 32. */
+int rd_quant_act(rd_device *d, const float *a, int M, int K, int8_t *codes, float *scales, float *sums);
 /* int8 per-row weights x per-32 int8 activations (backend/cuda/actgroup.cu:421-437 gemv_w8a8_g32). */
 int rd_gemm_w8a8(rd_device *d, const int8_t *q, const float *row_scale, int N, int K, const float *a, int M, float *dst);
 /* int4 group-32 weights with f16 scales x per-32 int8 activations (backend/cuda/actgroup.cu:243-275). */

@@ -34,7 +34,7 @@ def test_library_exports_every_declared_symbol():
 def test_code_object_is_built_for_gfx950():
     blob = open(capi.HSACO_PATH, "rb").read()
     assert (blob[:4] == b"\x7fELF" or blob.startswith(b"__CLANG_OFFLOAD_BUNDLE__")) and b"gfx950" in blob
-    for k in (b"rd_k_gemm_q4k", b"rd_k_attn_partial", b"rd_k_dequant_q4k", b"rd_k_moe_route", b"rd_k_gemm_q4k_gateup"):
+    for k in (b"rd_k_gemm8_q4k_kw4", b"rd_k_attn_partial", b"rd_k_dequant_q4k", b"rd_k_moe_route", b"rd_k_gemm8_q4k_gateup"):
         assert k in blob
 
 
