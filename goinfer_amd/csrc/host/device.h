@@ -70,8 +70,8 @@ struct DevBuf {
 };
 
 // block sizes that match the code object's launch bounds: the f16-MFMA k-quant GEMMs (4 consumer + 1 producer waves), the fused
-// gate|up kernel (two tiles x four waves), the expert kernels (two tiles x two waves)
-constexpr unsigned GEMM_THREADS = 320, GATEUP_THREADS = 512, MOE_THREADS = 256;
+// gate|up kernel (two tiles x two waves), the expert kernels (two tiles x two waves)
+constexpr unsigned GEMM_THREADS = 320, GATEUP_THREADS = 256, MOE_THREADS = 256;
 
 // How many 64-position KV blocks one attention work item covers for a sequence of nb blocks: every (sequence, kv head) is
 // cut into pieces. The cut depends on the sequence's own length only, never on what else is in the

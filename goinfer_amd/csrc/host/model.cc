@@ -621,11 +621,11 @@ static int launch_proj(rd_model *m, const DevWeight &w, const void *Xp, size_t x
     return RD_OK;
 }
 
-// Where the fused gate|up kernel can run it sums K over four waves per tile, folded in LDS. The unfused path — steps of more than
-// 32 rows, or the fused kernel switched off — is launched with the same four waves and one split, so both produce the same bits
+// Where the fused gate|up kernel can run it sums K over two waves per tile, folded in LDS. The unfused path — steps of more than
+// 32 rows, or the fused kernel switched off — is launched with the same two waves and one split, so both produce the same bits
 // and a row is the same row in a batch of any size.
 static bool gateup_fusable(const rd_model_desc &c, const DevWeight &w) { return w.kind == 0 && c.inter % 32 == 0; }
-constexpr int GATEUP_KW = 4; // waves per tile of the fused gate|up kernel
+constexpr int GATEUP_KW = 2; // waves per tile of the fused gate|up kernel
 
 constexpr int MOE_FOLD_FUSED_MAX = 8; // ranks rd_k_add_rmsnorm_quant folds in registers
 

@@ -374,7 +374,7 @@ RD_GEMM8_KERNEL(rd_k_gemm8_w4a8_kw8, W4A8Traits8, 8, 1)
 // ---------------- fused gate|up projection + SwiGLU + per-32 quantization ----------------
 // goinfer decoder/cpu_gateup_fused.go:83-148 in one launch. W holds [gate rows; up rows] (2*I rows). Grid (I/32), block 2*KW waves:
 // waves 0..KW-1 own gate tile t over K (each its own range), waves KW..2KW-1 the matching up tile. After the fold both finished
-// tiles meet in LDS in accumulator order, and every wave takes two of the sixteen accumulator registers: in that order a
+// tiles meet in LDS in accumulator order, and every wave takes its share of the sixteen accumulator registers: in that order a
 // half-wave holds the 32 columns of one batch row, which is exactly one activation group of the down projection, so
 // silu(gate)*up (silu in f64, decoder/rmsnorm.go:204-207) is quantized where it sits and written in the layout the down projection reads.
 // The K loop, its wave ranges and the fold are those of the plain kernel with the same KW: the sums are the same bits.
@@ -393,21 +393,27 @@ __device__ __forceinline__ void gemm8_gateup_body(const uint8_t *__restrict__ Wt
         for (int r = 0; r < 16; r++) lds[(half * 16 + r) * 64 + lane] = acc[r];
     }
     __syncthreads();
-    constexpr int RPW = 16 / (2 * KW) > 0 ? 16 / (2 * KW) : 1; // accumulator registers per wave
+    constexpr int RPW = 16 / (2 * KW); // accumulator registers per wave
     const int n = t * 32 + (lane & 31);
 #pragma unroll
     for (int j = 0; j < RPW; j++) {
         const int r = wave * RPW + j;
-        if (r >= 16) break;
         const int m = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
         const float a = __fmul_rn(silu_f64(lds[r * 64 + lane]), lds[(16 + r) * 64 + lane]);
         const Quant1 q = quant_one(a);
-        if (m < M) panel_store(XpOut, outKind, m, n, q);
+        if (outKind == RD_PANEL_A8) {
+            // four neighbouring lanes hold four consecutive elements of the row: their codes leave as one word
+            const int c = q.code & 255;
+            const uint32_t word = (uint32_t)dpp_i<0x00>(c) | ((uint32_t)dpp_i<0x55>(c) << 8) | ((uint32_t)dpp_i<0xAA>(c) << 16) | ((uint32_t)dpp_i<0xFF>(c) << 24);
+            if (m < M && (lane & 3) == 0) a8_store4(XpOut, m, n, word, q.sc, q.gsum);
+        } else if (m < M) {
+            panel_store(XpOut, outKind, m, n, q);
+        }
     }
 }
 
-extern "C" __global__ __launch_bounds__(512) void rd_k_gemm8_q4k_gateup(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ A8,
+extern "C" __global__ __launch_bounds__(256) void rd_k_gemm8_q4k_gateup(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ A8,
                                                                          uint8_t *__restrict__ XpOut, int outKind, int I, int nKB, int M) {
-    __shared__ float lds[2 * 3 * 1024];
-    gemm8_gateup_body<Q4K8Traits, 4>(Wt, A8, XpOut, outKind, I, nKB, M, lds);
+    __shared__ float lds[2 * 1024];
+    gemm8_gateup_body<Q4K8Traits, 2>(Wt, A8, XpOut, outKind, I, nKB, M, lds);
 }

@@ -299,8 +299,8 @@ def test_i8_kv_uploaded_prefix(dev):
 
 def test_wide_batch_rows_equal_solo_rows_deep_k(dev):
     """The same identity where K spans six super-blocks (hidden 1536): a one-row step runs the fused gate|up kernel, which sums K
-    over four waves per tile (two, two, one and one super-blocks), a step of more than 32 rows runs the plain GEMM and the SwiGLU
-    kernel — forced to those same four waves, so the bits agree. Switching the fused kernel off changes nothing either."""
+    over two waves per tile (three super-blocks each), a step of more than 32 rows runs the plain GEMM and the SwiGLU
+    kernel — forced to those same two waves, so the bits agree. Switching the fused kernel off changes nothing either."""
     import os
     cfg = dense_cfg(n_layers=2, hidden=1536, n_heads=12, n_kv=2, head_dim=128, inter=1536, vocab=512)
     B = 40
