@@ -94,6 +94,7 @@ static const KName kNames[] = {
     {"rd_k_kv_store", &Kernels::kv_store},
     {"rd_k_kv_read", &Kernels::kv_read},
     {"rd_k_qkv_rope_store", &Kernels::qkv_rope_store},
+    {"rd_k_rope_table", &Kernels::rope_table},
     {"rd_k_attn_partial", &Kernels::attn_partial},
     {"rd_k_kv_store_i8", &Kernels::kv_store_i8},
     {"rd_k_qkv_rope_store_i8", &Kernels::qkv_rope_store_i8},
@@ -158,10 +159,13 @@ static int open_common(int ordinal, const void *image, rd_device **out) {
     static const char *kindName[3] = {"q4k", "w8a8", "w4a8"};
     static const int kwOf[3] = {2, 4, 8};
     for (int kind = 0; kind < 3; kind++)
-        for (int i = 0; i < 3; i++) {
+        for (int i = 0; i < 6; i++) {
             char name[64];
-            snprintf(name, sizeof name, "rd_k_gemm8_%s_kw%d", kindName[kind], kwOf[i]);
-            if (hip->ModuleGetFunction(&d->k.gemm8[kind][i], d->module, name) != hipSuccess) {
+            if (i < 3)
+                snprintf(name, sizeof name, "rd_k_gemm8_%s_kw%d", kindName[kind], kwOf[i]);
+            else
+                snprintf(name, sizeof name, "rd_k_gemm8_%s_qkv_kw%d", kindName[kind], kwOf[i - 3]);
+            if (hip->ModuleGetFunction(i < 3 ? &d->k.gemm8[kind][i] : &d->k.gemm8_qkv[kind][i - 3], d->module, name) != hipSuccess) {
                 rd_set_error("code object lacks kernel %s", name);
                 (void)hip->ModuleUnload(d->module);
                 (void)hip->StreamDestroy(d->stream);

@@ -43,6 +43,7 @@ extern "C" int rd_model_create(rd_device *d, const rd_model_desc *desc, rd_model
         if (c.n_experts > 0) l.exp_have.assign((size_t)c.n_experts * 3, 0);
     int rc = d->alloc((void **)&m->inv_freq_dev, sizeof(double) * m->inv_freq.size());
     if (!rc) rc = d->h2d(m->inv_freq_dev, m->inv_freq.data(), sizeof(double) * m->inv_freq.size());
+    if (!rc) rc = d->alloc((void **)&m->rope_cs, sizeof(double) * 2 * (size_t)rd_model::ROWS_MAX * (c.head_dim / 2));
     if (!rc) rc = d->sync();
     if (rc) {
         delete m;
@@ -63,7 +64,7 @@ extern "C" void rd_model_destroy(rd_model *m) {
             d->release(p);
     }
     free_weight(d, &m->head);
-    for (void *p : {(void *)m->embed_q, (void *)m->embed_scale, (void *)m->inv_freq_dev, (void *)m->final_norm, (void *)m->tables, (void *)m->h, (void *)m->normed, (void *)m->P, (void *)m->qbuf,
+    for (void *p : {(void *)m->embed_q, (void *)m->embed_scale, (void *)m->inv_freq_dev, (void *)m->rope_cs, (void *)m->final_norm, (void *)m->tables, (void *)m->h, (void *)m->normed, (void *)m->P, (void *)m->qbuf,
                     (void *)m->part, (void *)m->cand_v, (void *)m->cand_i, (void *)m->logits, (void *)m->emb_dev, m->XpA, m->XpA2, m->XpB, (void *)m->ids, (void *)m->meta, (void *)m->router_logits, (void *)m->moe_wgt, (void *)m->moe_gu,
                     (void *)m->moe_dn, (void *)m->moe_out, (void *)m->moe_idx, (void *)m->moe_idx_all, (void *)m->moe_rank, (void *)m->moe_bits, (void *)m->topk_ids, (void *)m->topk_vals, (void *)m->topk_z, (void *)m->topk_scratch.ghist, (void *)m->topk_scratch.ccount, (void *)m->topk_scratch.gmax, (void *)m->topk_scratch.cand_i, (void *)m->topk_scratch.cand_v, (void *)m->topk_scratch.invT, (void *)m->topk_scratch.zpart, m->XpE})
         d->release(p);
@@ -166,6 +167,22 @@ static int fuse_and_upload(rd_device *d, PendingMat *parts, int n, DevWeight *w)
     return rc;
 }
 
+// The rows of a q, k or v projection reordered within each head so that a rotation pair (d, d + hd/2) lands in one 32-row GEMM
+// tile, sixteen rows apart: new row 32j + l of a head holds d = 16j + l for l < 16 and d = hd/2 + 16j + (l - 16) above
+// (qkv_col in the kernels is the inverse). The fused q|k|v kernel rotates the pair inside the tile that produced it.
+static void permute_head_rows(PendingMat *p, int hd) {
+    const size_t rowB = p->data.size() / (size_t)p->N, scB = p->scales.size() / (size_t)p->N;
+    std::vector<uint8_t> data(p->data.size()), scales(p->scales.size());
+    const int half = hd / 2;
+    for (int n = 0; n < p->N; n++) {
+        const int head = n / hd, c = n % hd, j = c >> 5, l = c & 31;
+        const int src = head * hd + (l < 16 ? 16 * j + l : half + 16 * j + (l - 16));
+        memcpy(&data[(size_t)n * rowB], &p->data[(size_t)src * rowB], rowB);
+        if (scB) memcpy(&scales[(size_t)n * scB], &p->scales[(size_t)src * scB], scB);
+    }
+    p->data.swap(data), p->scales.swap(scales);
+}
+
 static int accept(rd_model *m, int layer, int proj, PendingMat &&pm) {
     if (m->finalized) {
         rd_set_error("model already finalized");
@@ -187,6 +204,7 @@ static int accept(rd_model *m, int layer, int proj, PendingMat &&pm) {
     }
     l.pend[proj] = std::move(pm);
     if (proj <= RD_PROJ_V) {
+        permute_head_rows(&l.pend[proj], m->desc.head_dim);
         if (l.pend[RD_PROJ_Q].kind >= 0 && l.pend[RD_PROJ_K].kind >= 0 && l.pend[RD_PROJ_V].kind >= 0) {
             free_weight(d, &l.qkv);
             return fuse_and_upload(d, &l.pend[RD_PROJ_Q], 3, &l.qkv);
@@ -388,6 +406,11 @@ extern "C" int rd_model_finalize(rd_model *m) {
     RC(d->alloc(&m->XpA, m->xpAStride * tiles));
     RC(d->alloc(&m->XpA2, m->xpAStride * tiles));
     RC(d->alloc(&m->XpB, m->xpBStride * tiles));
+    // An A8 panel's last block is written only up to K: what lies past it (K not a multiple of 256) must hold finite scales and
+    // sums for good, since the GEMM multiplies them with the weights' zero padding.
+    HIPCHK(MemsetAsync(m->XpA, 0, m->xpAStride * tiles, d->stream));
+    HIPCHK(MemsetAsync(m->XpA2, 0, m->xpAStride * tiles, d->stream));
+    HIPCHK(MemsetAsync(m->XpB, 0, m->xpBStride * tiles, d->stream));
     RC(d->alloc((void **)&m->ids, sizeof(int) * R));
     RC(alloc_f32(d, &m->cand_v, R * ((c.vocab + 4095) / 4096)));
     RC(d->alloc((void **)&m->cand_i, sizeof(int) * R * (size_t)((c.vocab + 4095) / 4096)));
@@ -627,6 +650,12 @@ static int launch_proj(rd_model *m, const DevWeight &w, const void *Xp, size_t x
 static bool gateup_fusable(const rd_model_desc &c, const DevWeight &w) { return w.kind == 0 && c.inter % 32 == 0; }
 constexpr int GATEUP_KW = 2; // waves per tile of the fused gate|up kernel
 
+// The q|k|v GEMM can rotate and store its own output where nothing needs a whole head at once: no per-head q/k RMSNorm, the f16
+// cache (the int8 cache takes one scale per head), one weight of an int8-MFMA kind (not a group of kinds).
+static bool qkv_fusable(const rd_model *m, const LayerW &l) {
+    return is_gemm8_kind(l.qkv.kind) && !m->desc.qk_norm && m->kv_type == RD_KV_F16 && !getenv("ROCMDECODE_NO_FUSED_QKV");
+}
+
 constexpr int MOE_FOLD_FUSED_MAX = 8; // ranks rd_k_add_rmsnorm_quant folds in registers
 
 static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
@@ -788,26 +817,39 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
     // down-projection rows and their weights, folded by the kernel that adds them
     const float *resP = nullptr, *resW = nullptr;
     int resSplits = 0;
+    if (std::any_of(m->layers.begin(), m->layers.end(), [&](const LayerW &l) { return qkv_fusable(m, l); })) {
+        Scope s(m, KC_ROPE_STORE);
+        RC(d->launch(d->k.rope_table, (unsigned)B, 1, 1, (unsigned)(HD / 2), (const int *)m->rowPos, (const double *)m->inv_freq_dev, m->rope_cs, HD / 2));
+    }
     for (int li = 0; li < c.n_layers; li++) {
         LayerW &l = m->layers[(size_t)li];
         GemmPlan plan;
         RC(add_norm_quant(m, B, resP, resSplits, l.attn_norm, l.qkv, m->XpA, nullptr, resW));
-        {
-            Scope s(m, KC_GEMM_QKV);
-            RC(launch_proj(m, l.qkv, m->XpA, m->xpAStride, B, &plan));
-        }
-        {
+        if (qkv_fusable(m, l)) {
+            Scope s(m, KC_GEMM_QKV); // projection, bias, RoPE and the KV store in one launch per M-tile
+            const DevWeight &w = l.qkv;
+            const int nKB = kblocks_for(w), kw = plan_gemm(w.kind, w.N, nKB).kw; // the plain GEMM's waves per tile, in one split
+            for (int m0 = 0, mt = 0; m0 < B; m0 += 32, mt++)
+                RC(d->launch(d->k.gemm8_qkv[w.kind][kw == 8 ? 2 : (kw == 4 ? 1 : 0)], (unsigned)(w.N / 32), 1, 1, (unsigned)(64 * kw), (const void *)w.tiled, (const void *)w.scales,
+                             (const void *)((const char *)m->XpA + (size_t)mt * m->xpAStride), w.N, nKB, std::min(32, B - m0), m->qbuf, l.Kp, l.Vp,
+                             (const int *)m->tables, m->blocks_per_slot, (const int *)m->rowSlot, (const int *)m->rowPos, (const double *)m->rope_cs,
+                             (const float *)l.qkv_bias, nH, nKV, HD, m0));
+        } else {
+            {
+                Scope s(m, KC_GEMM_QKV);
+                RC(launch_proj(m, l.qkv, m->XpA, m->xpAStride, B, &plan));
+            }
             Scope s(m, KC_ROPE_STORE);
             if (m->kv_type == RD_KV_I8)
                 RC(d->launch(d->k.qkv_rope_store_i8, (unsigned)(nH + 2 * nKV), (unsigned)B, 1, (unsigned)(HD / 2), (const float *)m->P, plan.splits, m->qbuf,
                              (signed char *)l.Kp, (signed char *)l.Vp, l.Ksc, l.Vsc, (const int *)m->tables, m->blocks_per_slot, (const int *)m->rowSlot,
                              (const int *)m->rowPos, (const double *)m->inv_freq_dev, (const float *)l.q_norm, (const float *)l.k_norm, c.rms_eps, nH, nKV,
-                             HD, m->pStride, (const float *)l.qkv_bias));
+                             HD, m->pStride, (const float *)l.qkv_bias, 1));
             else
                 RC(d->launch(d->k.qkv_rope_store, (unsigned)(nH + 2 * nKV), (unsigned)B, 1, (unsigned)(HD / 2), (const float *)m->P, plan.splits, m->qbuf,
-                         l.Kp, l.Vp, (const int *)m->tables, m->blocks_per_slot, (const int *)m->rowSlot, (const int *)m->rowPos,
-                         (const double *)m->inv_freq_dev, (const float *)l.q_norm, (const float *)l.k_norm, c.rms_eps, nH, nKV, HD, m->pStride,
-                         (const float *)l.qkv_bias));
+                             l.Kp, l.Vp, (const int *)m->tables, m->blocks_per_slot, (const int *)m->rowSlot, (const int *)m->rowPos,
+                             (const double *)m->inv_freq_dev, (const float *)l.q_norm, (const float *)l.k_norm, c.rms_eps, nH, nKV, HD, m->pStride,
+                             (const float *)l.qkv_bias, 1));
         }
         {
             Scope s(m, KC_ATTN_PARTIAL);

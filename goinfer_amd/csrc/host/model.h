@@ -41,6 +41,7 @@ struct rd_model {
     rd_model_desc desc{};
     std::vector<double> inv_freq;
     double *inv_freq_dev = nullptr;
+    double *rope_cs = nullptr; // [max_rows][head_dim/2] (cos, sin) of the step's RoPE angles, written once per step
     std::vector<LayerW> layers;
     DevWeight head;
     PendingMat head_pend;

@@ -393,11 +393,11 @@ extern "C" int rd_qkv_rope_store(rd_device *d, int kv_type, int rows, const floa
     if (i8)
         RC(d->launch(d->k.qkv_rope_store_i8, (unsigned)(n_h + 2 * n_kv), (unsigned)rows, 1, (unsigned)(hd / 2), (const float *)X.p, 1, Q.as<float>(),
                      (signed char *)Kp.p, (signed char *)Vp.p, Ksc.as<float>(), Vsc.as<float>(), (const int *)T.p, bps, (const int *)S.p, (const int *)Pp.p,
-                     (const double *)F.p, (const float *)QN.p, (const float *)KN.p, eps, n_h, n_kv, hd, (size_t)0, (const float *)Bi.p));
+                     (const double *)F.p, (const float *)QN.p, (const float *)KN.p, eps, n_h, n_kv, hd, (size_t)0, (const float *)Bi.p, 0));
     else
         RC(d->launch(d->k.qkv_rope_store, (unsigned)(n_h + 2 * n_kv), (unsigned)rows, 1, (unsigned)(hd / 2), (const float *)X.p, 1, Q.as<float>(),
                      (uint16_t *)Kp.p, (uint16_t *)Vp.p, (const int *)T.p, bps, (const int *)S.p, (const int *)Pp.p, (const double *)F.p, (const float *)QN.p,
-                     (const float *)KN.p, eps, n_h, n_kv, hd, (size_t)0, (const float *)Bi.p));
+                     (const float *)KN.p, eps, n_h, n_kv, hd, (size_t)0, (const float *)Bi.p, 0));
     RC(d->d2h(q_out, Q.p, sizeof(float) * (size_t)rows * n_h * hd));
     for (int r = 0; r < rows; r++) {
         RC(d->launch(d->k.kv_read, 1u, (unsigned)n_kv, 1, (unsigned)hd, (const void *)Kp.p, (const void *)Vp.p, (const float *)Ksc.p, (const float *)Vsc.p,

@@ -114,31 +114,55 @@ extern "C" __global__ void rd_k_kv_read(const void *__restrict__ KpV, const void
     }
 }
 
+// NeoX rotation of the pair (x1, x2) = elements (d, d + HD/2) by the angle whose cosine and sine are c, s: products and sum
+// each rounded once in f64, then one rounding to f32 (decoder/rope.go:28-64 as amd64 computes it, without fused multiply-adds).
+__device__ __forceinline__ float rope_first(float x1, float x2, double c, double s) { return (float)__dsub_rn(__dmul_rn((double)x1, c), __dmul_rn((double)x2, s)); }
+__device__ __forceinline__ float rope_second(float x1, float x2, double c, double s) { return (float)__dadd_rn(__dmul_rn((double)x2, c), __dmul_rn((double)x1, s)); }
+
+// The resident model stores the rows of its q|k|v weight so that a rotation pair (d, d + HD/2) of a head falls into one 32-row
+// GEMM tile: tile j of a head holds d = 16j .. 16j+15 in its first sixteen rows and d + HD/2 in the other sixteen. Column of
+// element d of a head in that order:
+__device__ __forceinline__ int qkv_col(int d, int HD) {
+    const int half = HD >> 1, dd = d >= half ? d - half : d;
+    return ((dd >> 4) << 5) + (dd & 15) + (d >= half ? 16 : 0);
+}
+
+// cos and sin of every row's RoPE angles, once per step for all layers (the angle depends on the position and the pair only):
+// cs[row][t] = (cos, sin)(pos[row] * invFreq[t]) in f64. Grid (rows), block HD/2.
+extern "C" __global__ void rd_k_rope_table(const int *__restrict__ rowPos, const double *__restrict__ invFreq, double2 *__restrict__ cs, int half) {
+    const int m = blockIdx.x, t = threadIdx.x;
+    if (t >= half) return;
+    const double theta = __dmul_rn((double)rowPos[m], invFreq[t]);
+    cs[(size_t)m * half + t] = make_double2(cos(theta), sin(theta));
+}
+
 // After the q|k|v GEMM: reduce its split-K partials, optional q|k|v bias (Qwen2; decoder/attention.go:12-34 addBias, applied right
 // after the projections, program_cpu_n.go:470-476), optional per-head RMSNorm of q and k (Qwen3, decoder/program_cpu.go:351-364),
 // NeoX RoPE with f64 angles (decoder/rope.go:28-64), q -> f32 buffer, k,v -> this position of the row's sequence in the pool.
 // Grid (nH + 2*nKV, rows), block HD/2 threads... one thread per rotation pair.  P: [splits][32][(nH+2nKV)*HD].
+// permuted: the columns of a head in P are in the resident model's q|k|v row order (qkv_col).
 template <bool I8>
 __device__ __forceinline__ void qkv_rope_store_body(const float *__restrict__ P, int splits, float *__restrict__ q, void *__restrict__ KpV,
                                                void *__restrict__ VpV, float *__restrict__ Ksc, float *__restrict__ Vsc,
                                                const int *__restrict__ tables, int tabStride,
                                                const int *__restrict__ rowSlot, const int *__restrict__ rowPos, const double *__restrict__ invFreq,
                                                const float *__restrict__ qnorm, const float *__restrict__ knorm, float eps, int nH, int nKV, int HD,
-                                               size_t pStride, const float *__restrict__ bias) {
+                                               size_t pStride, const float *__restrict__ bias, int permuted) {
     int head = blockIdx.x, m = blockIdx.y, t = threadIdx.x, half = HD / 2; // one wave: half <= 64
+    const int c1 = permuted ? qkv_col(t, HD) : t, c2 = permuted ? qkv_col(t + half, HD) : t + half; // where the pair sits in the GEMM's output
     int Ntot = (nH + 2 * nKV) * HD, pos = rowPos[m];
     // everything this thread will need from memory is requested up front: one latency instead of a chain of them
     const int slotRow = rowSlot[m];
     const double invf = invFreq[t];
     const float *src = P + (size_t)(m >> 5) * pStride + (size_t)(m & 31) * Ntot + (size_t)head * HD; // M-tile m/32, row m%32
-    float x1 = src[t], x2 = src[t + half];
+    float x1 = src[c1], x2 = src[c2];
     float b1 = 0.f, b2 = 0.f;
     if (bias) b1 = bias[head * HD + t], b2 = bias[head * HD + t + half];
     for (int s0 = 1; s0 < splits; s0 += 8) { // ascending split order; eight splits' loads in flight together
         float a1[8], a2[8];
 #pragma unroll
         for (int j = 0; j < 8; j++)
-            if (s0 + j < splits) a1[j] = src[(size_t)(s0 + j) * 32 * Ntot + t], a2[j] = src[(size_t)(s0 + j) * 32 * Ntot + t + half];
+            if (s0 + j < splits) a1[j] = src[(size_t)(s0 + j) * 32 * Ntot + c1], a2[j] = src[(size_t)(s0 + j) * 32 * Ntot + c2];
 #pragma unroll
         for (int j = 0; j < 8; j++)
             if (s0 + j < splits) x1 = __fadd_rn(x1, a1[j]), x2 = __fadd_rn(x2, a2[j]);
@@ -156,10 +180,10 @@ __device__ __forceinline__ void qkv_rope_store_body(const float *__restrict__ P,
     }
     float o1 = x1, o2 = x2;
     if (isQ || isK) {
-        double theta = (double)pos * invf;
+        double theta = __dmul_rn((double)pos, invf);
         double c = cos(theta), s = sin(theta);
-        o1 = (float)((double)x1 * c - (double)x2 * s);
-        o2 = (float)((double)x2 * c + (double)x1 * s);
+        o1 = rope_first(x1, x2, c, s);
+        o2 = rope_second(x1, x2, c, s);
     }
     if (isQ) {
         float *dst = q + (size_t)m * nH * HD + (size_t)head * HD;
@@ -193,16 +217,17 @@ extern "C" __global__ void rd_k_qkv_rope_store(const float *__restrict__ P, int 
                                                uint16_t *__restrict__ Vp, const int *__restrict__ tables, int tabStride,
                                                const int *__restrict__ rowSlot, const int *__restrict__ rowPos, const double *__restrict__ invFreq,
                                                const float *__restrict__ qnorm, const float *__restrict__ knorm, float eps, int nH, int nKV, int HD,
-                                               size_t pStride, const float *__restrict__ bias) {
-    qkv_rope_store_body<false>(P, splits, q, Kp, Vp, nullptr, nullptr, tables, tabStride, rowSlot, rowPos, invFreq, qnorm, knorm, eps, nH, nKV, HD, pStride, bias);
+                                               size_t pStride, const float *__restrict__ bias, int permuted) {
+    qkv_rope_store_body<false>(P, splits, q, Kp, Vp, nullptr, nullptr, tables, tabStride, rowSlot, rowPos, invFreq, qnorm, knorm, eps, nH, nKV, HD, pStride, bias, permuted);
 }
 // The same into the int8 cache: the K or V head is quantized with its own scale after RoPE (backend/cuda/kv8_store.cu).
 extern "C" __global__ void rd_k_qkv_rope_store_i8(const float *__restrict__ P, int splits, float *__restrict__ q, signed char *__restrict__ Kp,
                                                   signed char *__restrict__ Vp, float *__restrict__ Ksc, float *__restrict__ Vsc,
                                                   const int *__restrict__ tables, int tabStride, const int *__restrict__ rowSlot,
                                                   const int *__restrict__ rowPos, const double *__restrict__ invFreq, const float *__restrict__ qnorm,
-                                                  const float *__restrict__ knorm, float eps, int nH, int nKV, int HD, size_t pStride, const float *__restrict__ bias) {
-    qkv_rope_store_body<true>(P, splits, q, Kp, Vp, Ksc, Vsc, tables, tabStride, rowSlot, rowPos, invFreq, qnorm, knorm, eps, nH, nKV, HD, pStride, bias);
+                                                  const float *__restrict__ knorm, float eps, int nH, int nKV, int HD, size_t pStride, const float *__restrict__ bias,
+                                                  int permuted) {
+    qkv_rope_store_body<true>(P, splits, q, Kp, Vp, Ksc, Vsc, tables, tabStride, rowSlot, rowPos, invFreq, qnorm, knorm, eps, nH, nKV, HD, pStride, bias, permuted);
 }
 
 typedef float float4v __attribute__((ext_vector_type(4)));

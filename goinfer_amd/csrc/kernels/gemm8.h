@@ -14,6 +14,7 @@
 // output's sum is fixed by (split, wave, super-block, group) and independent of M: a row in a batch is the row alone, bit for bit.
 #pragma once
 #include "act.h"
+#include "attn.h"
 
 typedef int i32x4_t __attribute__((ext_vector_type(4)));
 typedef int i32x16_t __attribute__((ext_vector_type(16)));
@@ -190,7 +191,7 @@ struct W8A8Traits8 {
     static __device__ __forceinline__ void finish(float16_t &acc, const void *aux, int tile, int lane) {
         const float ws = ((const float *)aux)[tile * 32 + (lane & 31)];
 #pragma unroll
-        for (int r = 0; r < 16; r++) acc[r] = __fmul_rn(acc[r], ws);
+        for (int r = 0; r < 16; r++) acc[r] = mul_rounded(acc[r], ws);
     }
 };
 
@@ -417,3 +418,91 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_gemm8_q4k_gateup(const ui
     __shared__ float lds[2 * 1024];
     gemm8_gateup_body<Q4K8Traits, 2>(Wt, A8, XpOut, outKind, I, nKB, M, lds);
 }
+
+// ---------------- q|k|v projection with bias, RoPE and the KV store in its epilogue ----------------
+// The plain kernel with one split and, instead of the store of the sums, what rd_k_qkv_rope_store does to them (same arithmetic,
+// same bits): the weight's rows are ordered so that a rotation pair sits in one tile, sixteen lanes apart (qkv_col), the angles'
+// cos and sin come from the step's table, q goes to the f32 buffer and k, v to the row's position in the f16 pool. For models
+// without QK-norm on the f16 cache. row0: first row of this M-tile among the step's rows. Grid (N/32), block KW waves.
+struct QkvEpilogue {
+    float *q;
+    uint16_t *Kp, *Vp;
+    const int *tables, *rowSlot, *rowPos;
+    const double2 *cs;
+    const float *bias;
+    int tabStride, nH, nKV, HD, row0;
+};
+template <class T, int KW>
+__device__ __forceinline__ void gemm8_qkv_body(const uint8_t *__restrict__ Wt, const void *__restrict__ aux, const uint8_t *__restrict__ A8, int N, int nKB,
+                                               int M, const QkvEpilogue &e, float *lds) {
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int tile = blockIdx.x, kw = wave;
+    const int per = (nKB + KW - 1) / KW, s0 = kw * per, nk = max(0, min(nKB, s0 + per) - s0);
+    float16_t acc;
+    gemm8_wave_loop<T>(acc, Wt + ((size_t)tile * nKB + s0) * T::TILE_BYTES, A8 + (size_t)s0 * RD_A8_BLOCK_BYTES, nk, aux, tile, lane);
+    const int HD = e.HD, half = HD >> 1, head = (tile * 32) / HD, j = ((tile * 32) % HD) >> 5, l = lane & 31, h = lane >> 5;
+    const int d = l < 16 ? 16 * j + l : half + 16 * j + (l - 16);
+    const bool isQ = head < e.nH, isK = !isQ && head < e.nH + e.nKV;
+    // The first wave's sixteen rows' positions, cache blocks and angles: each kind of load for all rows at once, the first two
+    // before the fold's barrier, so that the epilogue waits for memory three times and not three times per row.
+    int pos[16], blk[16];
+    if (kw == 0) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int m = e.row0 + min((r >> 2) * 8 + h * 4 + (r & 3), M - 1);
+            pos[r] = e.rowPos[m];
+            blk[r] = isQ ? 0 : e.rowSlot[m];
+        }
+    }
+    gemm8_fold_waves<KW, 1>(acc, lds);
+    if (kw != 0) return;
+    double2 cs[16];
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const int m = e.row0 + min((r >> 2) * 8 + h * 4 + (r & 3), M - 1);
+        if (!isQ) blk[r] = e.tables[(size_t)blk[r] * e.tabStride + (pos[r] >> 6)];
+        if (isQ || isK) cs[r] = e.cs[(size_t)m * half + (d < half ? d : d - half)];
+    }
+    T::finish(acc, aux, tile, lane);
+    const float b = e.bias ? e.bias[head * HD + d] : 0.f;
+    const int kvh = isK ? head - e.nH : head - e.nH - e.nKV;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const int mr = (r >> 2) * 8 + h * 4 + (r & 3), m = e.row0 + mr;
+        float x = acc[r];
+        if (e.bias) x = __fadd_rn(x, b);
+        const float other = swz_xor16_f(x); // the pair's other element, sixteen lanes away
+        float out = x;
+        if (isQ || isK) out = l < 16 ? rope_first(x, other, cs[r].x, cs[r].y) : rope_second(other, x, cs[r].x, cs[r].y);
+        if (mr >= M) continue;
+        if (isQ) {
+            e.q[(size_t)m * e.nH * HD + (size_t)head * HD + d] = out;
+        } else {
+            const int p = pos[r] & 63;
+            const size_t region = ((size_t)blk[r] * e.nKV + kvh) * 64 * HD;
+            if (isK)
+                e.Kp[region + (HD == 128 ? k_elem_index<128>(p, d) : k_elem_index<64>(p, d))] = f32_to_f16_half_up(out);
+            else
+                e.Vp[region + (HD == 128 ? v_elem_index<128>(p, d) : v_elem_index<64>(p, d))] = f32_to_f16_half_up(out);
+        }
+    }
+}
+
+#define RD_GEMM8_QKV_KERNEL(NAME, TRAITS, KW)                                                                                                          \
+    extern "C" __global__ __launch_bounds__(64 * KW) void NAME(                                                                                        \
+        const uint8_t *__restrict__ Wt, const void *__restrict__ aux, const uint8_t *__restrict__ A8, int N, int nKB, int M, float *__restrict__ q,     \
+        uint16_t *__restrict__ Kp, uint16_t *__restrict__ Vp, const int *__restrict__ tables, int tabStride, const int *__restrict__ rowSlot,           \
+        const int *__restrict__ rowPos, const double *__restrict__ cs, const float *__restrict__ bias, int nH, int nKV, int HD, int row0) {             \
+        __shared__ float lds[(KW - 1) * 1024];                                                                                                         \
+        QkvEpilogue e{q, Kp, Vp, tables, rowSlot, rowPos, (const double2 *)cs, bias, tabStride, nH, nKV, HD, row0};                                    \
+        gemm8_qkv_body<TRAITS, KW>(Wt, aux, A8, N, nKB, M, e, lds);                                                                                    \
+    }
+RD_GEMM8_QKV_KERNEL(rd_k_gemm8_q4k_qkv_kw2, Q4K8Traits, 2)
+RD_GEMM8_QKV_KERNEL(rd_k_gemm8_q4k_qkv_kw4, Q4K8Traits, 4)
+RD_GEMM8_QKV_KERNEL(rd_k_gemm8_q4k_qkv_kw8, Q4K8Traits, 8)
+RD_GEMM8_QKV_KERNEL(rd_k_gemm8_w8a8_qkv_kw2, W8A8Traits8, 2)
+RD_GEMM8_QKV_KERNEL(rd_k_gemm8_w8a8_qkv_kw4, W8A8Traits8, 4)
+RD_GEMM8_QKV_KERNEL(rd_k_gemm8_w8a8_qkv_kw8, W8A8Traits8, 8)
+RD_GEMM8_QKV_KERNEL(rd_k_gemm8_w4a8_qkv_kw2, W4A8Traits8, 2)
+RD_GEMM8_QKV_KERNEL(rd_k_gemm8_w4a8_qkv_kw4, W4A8Traits8, 4)
+RD_GEMM8_QKV_KERNEL(rd_k_gemm8_w4a8_qkv_kw8, W4A8Traits8, 8)

@@ -4,9 +4,9 @@
 #include "common.h"
 #include "q4k.h"
 #include "act.h"
+#include "attn.h"
 #include "gemm8.h"
 #include "kquant.h"
-#include "attn.h"
 #include "misc.h"
 #include "moe.h"
 #include "topk.h"

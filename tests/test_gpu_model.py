@@ -200,6 +200,41 @@ def test_moe_fused_expert_gateup_equals_two_launches(dev):
         pair.close()
 
 
+@pytest.mark.parametrize("shape", ["q4k_hd128", "w8a8_hd64_bias", "q4k_hd64_three_blocks"])
+def test_fused_qkv_equals_projection_then_rope_store(dev, shape):
+    """The q|k|v GEMM with bias, RoPE and the KV store in its epilogue against the same step run as GEMM + rope/store kernel:
+    identical logits and identical cache contents, bit for bit, for one M-tile and for rows spread over two."""
+    import os
+    if shape == "q4k_hd128":
+        cfg = dense_cfg(n_layers=2, hidden=512, n_heads=4, n_kv=2, head_dim=128, inter=512, vocab=512)
+    elif shape == "w8a8_hd64_bias":
+        cfg = dict(dense_cfg(n_layers=2, hidden=384, n_heads=6, n_kv=2, head_dim=64, inter=512, vocab=512, theta=1e6), qkv_bias=1)
+    else:
+        cfg = dense_cfg(n_layers=2, hidden=768, n_heads=12, n_kv=4, head_dim=64, inter=512, vocab=512)
+    nKV, hd = cfg["n_kv"], cfg["head_dim"]
+    for B in (5, 40):
+        pair = Pair(cfg, seed=91, dev=dev, slots=2 * B, ctx_cap=64)
+        try:
+            rng = np.random.default_rng(B)
+            for step in range(2):
+                emb = pair.emb[rng.integers(0, cfg["vocab"], B)]
+                fused, _ = pair.gpu.step_batch(list(range(B)), [step] * B, emb, capi.WANT_LOGITS)
+                os.environ["ROCMDECODE_NO_FUSED_QKV"] = "1"
+                try:
+                    plain, _ = pair.gpu.step_batch(list(range(B, 2 * B)), [step] * B, emb, capi.WANT_LOGITS)
+                finally:
+                    del os.environ["ROCMDECODE_NO_FUSED_QKV"]
+                assert np.array_equal(fused.view(np.uint32), plain.view(np.uint32)), (B, step)
+                for layer in range(cfg["n_layers"]):
+                    for b in (0, B - 1):
+                        kf, vf = pair.gpu.kv_download(b, layer, 0, step + 1)
+                        kp, vp = pair.gpu.kv_download(B + b, layer, 0, step + 1)
+                        assert np.array_equal(kf.view(np.uint32), kp.view(np.uint32)) and np.array_equal(vf.view(np.uint32), vp.view(np.uint32))
+                        assert np.abs(kf).max() > 0 and kf.shape[-1] == nKV * hd
+        finally:
+            pair.close()
+
+
 def test_step_errors(dev):
     pair = Pair(dense_cfg(n_layers=1), seed=6, dev=dev, slots=2, ctx_cap=64)
     e = pair.emb[:1]
