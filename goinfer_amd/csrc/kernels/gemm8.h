@@ -438,52 +438,58 @@ __device__ __forceinline__ void gemm8_qkv_body(const uint8_t *__restrict__ Wt, c
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int tile = blockIdx.x, kw = wave;
     const int per = (nKB + KW - 1) / KW, s0 = kw * per, nk = max(0, min(nKB, s0 + per) - s0);
-    float16_t acc;
-    gemm8_wave_loop<T>(acc, Wt + ((size_t)tile * nKB + s0) * T::TILE_BYTES, A8 + (size_t)s0 * RD_A8_BLOCK_BYTES, nk, aux, tile, lane);
-    const int HD = e.HD, half = HD >> 1, head = (tile * 32) / HD, j = ((tile * 32) % HD) >> 5, l = lane & 31, h = lane >> 5;
-    const int d = l < 16 ? 16 * j + l : half + 16 * j + (l - 16);
+    const int HD = e.HD, half = HD >> 1, head = (tile * 32) / HD, j = ((tile * 32) % HD) >> 5;
     const bool isQ = head < e.nH, isK = !isQ && head < e.nH + e.nKV;
-    // The first wave's sixteen rows' positions, cache blocks and angles: each kind of load for all rows at once, the first two
-    // before the fold's barrier, so that the epilogue waits for memory three times and not three times per row.
-    int pos[16], blk[16];
-    if (kw == 0) {
+    // The epilogue belongs to the whole block: the tile's 32 rows x 16 rotation pairs are dealt over its threads, PPT pairs each
+    // (thread t takes pair t & 15 of rows t >> 4, + 4*KW, ...), so no wave runs more than a few dozen instructions of it.
+    // What a thread needs from memory for its pairs is asked for ahead of time: the row's place in the cache (two dependent loads)
+    // before the K loop, the angle and the bias after it, ahead of the fold.
+    constexpr int PPT = 512 / (64 * KW);
+    const int pi = tid & 15, d1 = 16 * j + pi, d2 = half + d1; // this thread's pair: elements d1, d2 of the head, columns pi, pi + 16 of the tile
+    int where[PPT];                                            // block * 64 + position in the block
+    if (!isQ) {
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int m = e.row0 + min((r >> 2) * 8 + h * 4 + (r & 3), M - 1);
-            pos[r] = e.rowPos[m];
-            blk[r] = isQ ? 0 : e.rowSlot[m];
+        for (int i = 0; i < PPT; i++) {
+            const int m = e.row0 + min((tid >> 4) + 4 * KW * i, M - 1), pos = e.rowPos[m];
+            where[i] = e.tables[(size_t)e.rowSlot[m] * e.tabStride + (pos >> 6)] * 64 + (pos & 63);
         }
     }
-    gemm8_fold_waves<KW, 1>(acc, lds);
-    if (kw != 0) return;
-    double2 cs[16];
+    float16_t acc;
+    gemm8_wave_loop<T>(acc, Wt + ((size_t)tile * nKB + s0) * T::TILE_BYTES, A8 + (size_t)s0 * RD_A8_BLOCK_BYTES, nk, aux, tile, lane);
+    double2 cs[PPT];
+    float b1 = 0.f, b2 = 0.f;
+    if (isQ || isK) {
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-        const int m = e.row0 + min((r >> 2) * 8 + h * 4 + (r & 3), M - 1);
-        if (!isQ) blk[r] = e.tables[(size_t)blk[r] * e.tabStride + (pos[r] >> 6)];
-        if (isQ || isK) cs[r] = e.cs[(size_t)m * half + (d < half ? d : d - half)];
+        for (int i = 0; i < PPT; i++) cs[i] = e.cs[(size_t)(e.row0 + min((tid >> 4) + 4 * KW * i, M - 1)) * half + d1];
     }
-    T::finish(acc, aux, tile, lane);
-    const float b = e.bias ? e.bias[head * HD + d] : 0.f;
+    if (e.bias) b1 = e.bias[head * HD + d1], b2 = e.bias[head * HD + d2];
+    gemm8_fold_waves<KW, 1>(acc, lds);
+    float *sums = lds; // [32 rows][33]: the tile's sums, row stride 33 words against bank conflicts; the fold is done with this memory
+    if (kw == 0) {
+        T::finish(acc, aux, tile, lane);
+#pragma unroll
+        for (int r = 0; r < 16; r++) sums[((r >> 2) * 8 + (lane >> 5) * 4 + (r & 3)) * 33 + (lane & 31)] = acc[r];
+    }
+    __syncthreads();
     const int kvh = isK ? head - e.nH : head - e.nH - e.nKV;
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-        const int mr = (r >> 2) * 8 + h * 4 + (r & 3), m = e.row0 + mr;
-        float x = acc[r];
-        if (e.bias) x = __fadd_rn(x, b);
-        const float other = swz_xor16_f(x); // the pair's other element, sixteen lanes away
-        float out = x;
-        if (isQ || isK) out = l < 16 ? rope_first(x, other, cs[r].x, cs[r].y) : rope_second(other, x, cs[r].x, cs[r].y);
+    for (int i = 0; i < PPT; i++) {
+        const int mr = (tid >> 4) + 4 * KW * i, m = e.row0 + mr;
+        float x1 = sums[mr * 33 + pi], x2 = sums[mr * 33 + pi + 16];
         if (mr >= M) continue;
+        if (e.bias) x1 = __fadd_rn(x1, b1), x2 = __fadd_rn(x2, b2);
+        float o1 = x1, o2 = x2;
+        if (isQ || isK) o1 = rope_first(x1, x2, cs[i].x, cs[i].y), o2 = rope_second(x1, x2, cs[i].x, cs[i].y);
         if (isQ) {
-            e.q[(size_t)m * e.nH * HD + (size_t)head * HD + d] = out;
+            float *dst = e.q + (size_t)m * e.nH * HD + (size_t)head * HD;
+            dst[d1] = o1, dst[d2] = o2;
         } else {
-            const int p = pos[r] & 63;
-            const size_t region = ((size_t)blk[r] * e.nKV + kvh) * 64 * HD;
-            if (isK)
-                e.Kp[region + (HD == 128 ? k_elem_index<128>(p, d) : k_elem_index<64>(p, d))] = f32_to_f16_half_up(out);
-            else
-                e.Vp[region + (HD == 128 ? v_elem_index<128>(p, d) : v_elem_index<64>(p, d))] = f32_to_f16_half_up(out);
+            const int p = where[i] & 63;
+            const size_t region = ((size_t)(where[i] >> 6) * e.nKV + kvh) * 64 * HD;
+            uint16_t *dst = (isK ? e.Kp : e.Vp) + region;
+            const int i1 = isK ? (HD == 128 ? k_elem_index<128>(p, d1) : k_elem_index<64>(p, d1)) : (HD == 128 ? v_elem_index<128>(p, d1) : v_elem_index<64>(p, d1));
+            const int i2 = isK ? (HD == 128 ? k_elem_index<128>(p, d2) : k_elem_index<64>(p, d2)) : (HD == 128 ? v_elem_index<128>(p, d2) : v_elem_index<64>(p, d2));
+            dst[i1] = f32_to_f16_half_up(o1), dst[i2] = f32_to_f16_half_up(o2);
         }
     }
 }
@@ -493,7 +499,7 @@ __device__ __forceinline__ void gemm8_qkv_body(const uint8_t *__restrict__ Wt, c
         const uint8_t *__restrict__ Wt, const void *__restrict__ aux, const uint8_t *__restrict__ A8, int N, int nKB, int M, float *__restrict__ q,     \
         uint16_t *__restrict__ Kp, uint16_t *__restrict__ Vp, const int *__restrict__ tables, int tabStride, const int *__restrict__ rowSlot,           \
         const int *__restrict__ rowPos, const double *__restrict__ cs, const float *__restrict__ bias, int nH, int nKV, int HD, int row0) {             \
-        __shared__ float lds[(KW - 1) * 1024];                                                                                                         \
+        __shared__ float lds[KW > 2 ? (KW - 1) * 1024 : 32 * 33];                                                                                      \
         QkvEpilogue e{q, Kp, Vp, tables, rowSlot, rowPos, (const double2 *)cs, bias, tabStride, nH, nKV, HD, row0};                                    \
         gemm8_qkv_body<TRAITS, KW>(Wt, aux, A8, N, nKB, M, e, lds);                                                                                    \
     }
