@@ -22,6 +22,8 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+from bench_micro import counter_traffic, cpu_fields  # noqa: E402
+
 HBM_PEAK_GBS = 8000.0
 CPU_LAYERS = 8       # layers of the model the CPU baseline runs
 CPU_SECONDS = 12.0   # about this much timed CPU work
@@ -156,13 +158,13 @@ def run_c4(args):
     kv_launch = float((pos_prof + 2).sum()) * kv_pos_bytes / cfg["n_layers"]
     q_launch = B * cfg["n_heads"] * cfg["head_dim"] * 4
     achieved = (kv_launch + q_launch) / (avg_ms / 1e3) / 1e9
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "traffic.json")
-    if os.path.exists(tpath):
-        traffic = json.load(open(tpath)).get("%s/%s" % (kern, cfg["name"]))
+    traffic, t_ratio, t_src = counter_traffic("%s/%s/%s" % (kern, cfg["name"], args.kv), kv_launch + q_launch)
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "traffic": traffic if args.kv == "f16" else None, "kernel": "rd_k_attn_partial" if args.kv == "f16" else "rd_k_attn_partial_i8", "avg_launch_ms": round(avg_ms, 5),
-                "algorithmic_bytes_per_launch": int(kv_launch + q_launch)}
+                "traffic": traffic, "traffic_ratio": t_ratio, "traffic_source": t_src,
+                "kernel": "rd_k_attn_partial" if args.kv == "f16" else "rd_k_attn_partial_i8", "avg_launch_ms": round(avg_ms, 5),
+                "timing": "HIP events around every launch of the kernel in three extra steps after the timed ones (includes the launch gap; rocprofv3's kernel duration is 3-4 us shorter)",
+                "algorithmic_bytes_per_launch": int(kv_launch + q_launch),
+                "step_frac": round(step_gbs / HBM_PEAK_GBS, 4)}
     classes = {k: {"ms_per_step": round(v[0] / 3, 4), "launches_per_step": v[1] // 3} for k, v in prof.items()}
 
     # ---- a plain copy kernel of known size: the practical HBM rate, and the yardstick the traffic counters are scaled by ----
@@ -175,7 +177,7 @@ def run_c4(args):
         threads = min(16, len(os.sched_getaffinity(0)))
         log("CPU baseline on %d threads" % threads)
         v, sample = cpu_baseline(res, cfg, lens, kept_kv, threads, args.kv)
-        cpu = {"value": round(v, 3), "unit": "tok/s", "cores": threads, "kind": "port", "sample": sample}
+        cpu = dict({"value": round(v, 3), "unit": "tok/s"}, **cpu_fields(threads), kind="port", sample=sample)
     res.close()
     dev.close()
 
@@ -183,7 +185,7 @@ def run_c4(args):
         "metric": "batch-32 decode tok/s, Llama-3-8B-shape Q4_K; achieved HBM GB/s vs peak",
         "value": round(tok_s, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(float(ms.mean()), 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f16",
+        "dtype": "i8",
         "data": "synthetic: N(0,0.02) weights quantized to Q4_K (int8 head), N(0,1) KV, random token ids",
         "config": {"workload": "configs[3]: %s, %d layers, B=%d ragged, ctx U[%d,%d], greedy decode%s"
                                % (cfg["name"], cfg["n_layers"], B, args.ctx_min, args.ctx_max, "" if args.kv == "f16" else " (variant: int8 KV cache)"), "kv": args.kv,

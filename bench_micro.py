@@ -27,19 +27,57 @@ def emit(out):
     print(json.dumps(out, default=float))
 
 
-def base_line(metric, value, unit, steps, warmup, ms, workload, data, extra_cfg=None):
+def base_line(metric, value, unit, steps, warmup, ms, workload, data, extra_cfg=None, dtype="i8"):
     cfg = {"workload": workload}
     cfg.update(extra_cfg or {})
     return {"metric": metric, "value": round(value, 1), "unit": unit, "n_gpus": 1, "steps": steps, "warmup": warmup,
-            "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": data,
+            "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": data,
             "config": cfg}
 
 
 # ------------------------------------------------------------------------------------------------------------ C2
-def counter_traffic(key):
-    """HBM bytes per launch of a kernel on a workload as the rocprofv3 counter runs measured them (profiles/traffic.json), or None."""
+def host_cpu():
+    """(model name, physical cores) of this host from /proc/cpuinfo: distinct (physical id, core id) pairs, so SMT siblings
+    count once; (None, None) where the file does not say."""
+    model, cores, phys, core = None, set(), None, None
+    try:
+        for line in open("/proc/cpuinfo"):
+            k, _, v = line.partition(":")
+            k, v = k.strip(), v.strip()
+            if k == "model name" and model is None:
+                model = v
+            elif k == "physical id":
+                phys = v
+            elif k == "core id":
+                core = v
+            elif not k and phys is not None and core is not None:
+                cores.add((phys, core))
+                phys = core = None
+        if phys is not None and core is not None:
+            cores.add((phys, core))
+    except OSError:
+        pass
+    return model, (len(cores) or None)
+
+
+def counter_traffic(key, algorithmic_bytes):
+    """HBM bytes per launch of a kernel for THIS run: the run's algorithmic bytes times the ratio (counter traffic / algorithmic
+    bytes) that the rocprofv3 counter runs recorded for the kernel on this workload (profiles/traffic.json names the run each
+    ratio comes from). Returns (traffic, ratio, source) or (None, None, None)."""
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
-    return json.load(open(tpath)).get(key) if os.path.exists(tpath) else None
+    if not os.path.exists(tpath):
+        return None, None, None
+    e = json.load(open(tpath)).get(key)
+    if not e:
+        return None, None, None
+    return int(round(e["ratio"] * algorithmic_bytes)), e["ratio"], e["source"]
+
+
+def cpu_fields(n_threads):
+    """The fields of a cpu_baseline block that say what it ran on: threads used (`cores`, as the bench contract names them), the
+    host's CPU model and its physical core count."""
+    model, phys = host_cpu()
+    return {"cores": n_threads, "threads": n_threads, "physical_cores_on_host": phys, "cpu_model": model}
 
 
 def run_c2(args):
@@ -65,9 +103,9 @@ def run_c2(args):
                     head["us"] / 1e3, "configs[1]: Q4_K GEMM 14336x4096 / 4096x14336 / fused gate|up, M in {1,4,16,32,64}",
                     "synthetic: random Q4_K super-blocks with sane f16 scales, 8 weight copies used round-robin", {"cases": cases})
     out["roofline"] = {"bound": "hbm", "achieved": head["GBs"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(head["GBs"] / HBM_PEAK_GBS, 4),
-                       "traffic": counter_traffic("gemm_q4k_gateup/ffn-14336x4096-m32"), "kernel": "rd_k_gemm_q4k_gateup",
-                       "avg_launch_ms": round(head["us"] / 1e3, 5),
-                       "algorithmic_bytes_per_launch": head["bytes"]}
+                       "kernel": "rd_k_gemm8_q4k_gateup", "avg_launch_ms": round(head["us"] / 1e3, 5), "algorithmic_bytes_per_launch": head["bytes"]}
+    out["roofline"]["traffic"], out["roofline"]["traffic_ratio"], out["roofline"]["traffic_source"] = counter_traffic(
+        "gemm8_q4k_gateup/ffn-14336x4096-m32", head["bytes"])
     cpu = None
     if not args.no_cpu:
         from goinfer_amd import synth
@@ -83,7 +121,7 @@ def run_c2(args):
             ob.swiglu(ob.matmul(wg, a), ob.matmul(wu, a))
             t += time.time() - t0
             n += 1
-        cpu = {"value": round(head["bytes"] / (t / n) / 1e9, 2), "unit": "GB/s", "cores": threads(), "kind": "port",
+        cpu = {"value": round(head["bytes"] / (t / n) / 1e9, 2), "unit": "GB/s", **cpu_fields(threads()), "kind": "port",
                "sample": "oracle gate and up matmuls + SwiGLU at M=32, %d calls (%.1f s)" % (n, t)}
     out["cpu_baseline"] = cpu
     dev.close()
@@ -108,7 +146,7 @@ def run_kquant(args):
     head = next(c for c in cases if c["kernel"] == "rd_k_gemm_q6k" and c["N"] == 128256 and c["M"] == 32)
     out = base_line("Q6_K dequant-GEMM achieved HBM GB/s (head 128256x4096 at M=32; all cases listed)", head["GBs"], "GB/s", steps, warmup,
                     head["us"] / 1e3, "Q4_K / Q5_K / Q6_K GEMM at 14336x4096, 4096x14336, 128256x4096, M in {1,32}",
-                    "synthetic: random super-blocks with sane f16 scales, 4-8 weight copies used round-robin", {"cases": cases})
+                    "synthetic: random super-blocks with sane f16 scales, 4-8 weight copies used round-robin", {"cases": cases}, dtype="f16")
     out["roofline"] = {"bound": "hbm", "achieved": head["GBs"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(head["GBs"] / HBM_PEAK_GBS, 4),
                        "traffic": None, "kernel": "rd_k_gemm_q6k", "avg_launch_ms": round(head["us"] / 1e3, 5),
                        "algorithmic_bytes_per_launch": head["bytes"]}
@@ -127,7 +165,7 @@ def run_kquant(args):
             ob.matmul(w, a)
             t += time.time() - t0
             n += 1
-        cpu = {"value": round((N * (K // 256) * 210 + 4 * 32 * (K + N)) / (t / n) / 1e9, 2), "unit": "GB/s", "cores": threads(), "kind": "port",
+        cpu = {"value": round((N * (K // 256) * 210 + 4 * 32 * (K + N)) / (t / n) / 1e9, 2), "unit": "GB/s", **cpu_fields(threads()), "kind": "port",
                "sample": "oracle Q6_K matmul, %d x %d rows of the head at M=32, %d calls (%.1f s)" % (N, K, n, t)}
     out["cpu_baseline"] = cpu
     dev.close()
@@ -151,7 +189,7 @@ def run_topk(args):
     head = next(c for c in cases if c["rows"] == 32 and c["V"] == 128256 and c["k"] == 256 and c["values"] == "bell")
     out = base_line("device-side top-K of logits rows, achieved GB/s over one read of the rows (32 rows of 128256, K=256; all cases listed)",
                     head["GBs"], "GB/s", steps, warmup, head["us"] / 1e3, "top-K of logits rows (TopKRow): ids, logits and Z",
-                    "synthetic: sums of twelve uniforms (bell) or uniform values", {"cases": cases})
+                    "synthetic: sums of twelve uniforms (bell) or uniform values", {"cases": cases}, dtype="f32")
     out["roofline"] = {"bound": "hbm", "achieved": head["GBs"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(head["GBs"] / HBM_PEAK_GBS, 4),
                        "traffic": None, "kernel": "rd_k_topk_hist + rd_k_topk_pick + rd_k_topk_finish", "avg_launch_ms": round(head["us"] / 1e3, 5),
                        "algorithmic_bytes_per_launch": head["bytes"]}
@@ -168,7 +206,7 @@ def run_topk(args):
                 ob.softmax_z(x[r], 0.7)
             t += time.time() - t0
             n += 1
-        cpu = {"value": round(32 * 128256 * 4 / (t / n) / 1e9, 2), "unit": "GB/s", "cores": 1, "kind": "port",
+        cpu = {"value": round(32 * 128256 * 4 / (t / n) / 1e9, 2), "unit": "GB/s", **cpu_fields(1), "kind": "port",
                "sample": "oracle topKByLogit + Z over 32 rows of 128256, K=256, %d passes (%.1f s)" % (n, t)}
     out["cpu_baseline"] = cpu
     dev.close()
@@ -201,14 +239,15 @@ def run_c3(args):
                     "synthetic: uniform [-2,2) f16 KV (or random int8 codes and scales) in a paged pool with a scattered block table, f32 q",
                     {"kv": kv, "n_seq": nseq, "kv_positions": int(lens.sum()), "kv_len_min": int(lens.min()), "kv_len_max": int(lens.max()), "seed": args.seed,
                      "cases": [{"softcap": c, "call_us": round(v[0] * 1e3, 2), "call_GBs": round((kv_bytes + io_bytes) / v[0] / 1e6, 1),
-                                "partial_kernels_us": round(v[1] * 1e3, 2), "partial_kernels_GBs": round(kv_bytes / v[1] / 1e6, 1)} for c, v in res.items()]})
+                                "partial_kernels_us": round(v[1] * 1e3, 2), "partial_kernels_GBs": round(kv_bytes / v[1] / 1e6, 1)} for c, v in res.items()]}, dtype="f16")
     # the partial kernel is launched once per group of 32 rows: two launches per call here
     per_launch = (kv_bytes + nseq * nH * hd * 4) / 2
     out["roofline"] = {"bound": "hbm", "achieved": round(per_launch / (tp / 2) / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                        "frac": round(per_launch / (tp / 2) / 1e6 / HBM_PEAK_GBS, 4),
-                       "traffic": counter_traffic("attn_partial/64seq-u128-8192") if kv == "f16" and args.seed == 1234 else None,
                        "kernel": "rd_k_attn_partial" if kv == "f16" else "rd_k_attn_partial_i8",
                        "avg_launch_ms": round(tp / 2, 5), "algorithmic_bytes_per_launch": int(per_launch)}
+    out["roofline"]["traffic"], out["roofline"]["traffic_ratio"], out["roofline"]["traffic_source"] = counter_traffic(
+        "attn_partial/64seq-u128-8192/%s" % kv, per_launch)
     cpu = None
     if not args.no_cpu:
         from goinfer_amd import synth
@@ -229,7 +268,7 @@ def run_c3(args):
                 t_cpu += time.time() - t0
                 pos += n
             reps += 1
-        cpu = {"value": round(pos * 2 * kvd * 2 / t_cpu / 1e9, 3), "unit": "GB/s", "cores": threads(), "kind": "port",
+        cpu = {"value": round(pos * 2 * kvd * 2 / t_cpu / 1e9, 3), "unit": "GB/s", **cpu_fields(threads()), "kind": "port",
                "sample": "oracle attention (f64 accumulate, heads in parallel) on %d of the %d sequences, %d passes, %d positions (%.1f s)" % (
                    len(pick), nseq, reps, pos, t_cpu)}
     out["cpu_baseline"] = cpu
@@ -284,7 +323,7 @@ def run_c5(args):
     d2 = float(sum(len(set(idx2[:, l, :].ravel().tolist())) for l in range(layers)))
     g_ms = prof["moe_gemm_gateup"][0] / prof["moe_gemm_gateup"][1]
     per_launch = d2 * ebytes * (2.0 / 3.0) / layers
-    traffic = counter_traffic("gemm_w4a8_moe_gateup/%s" % cfg["name"])
+    traffic, t_ratio, t_src = counter_traffic("gemm8_w4a8_moe_gateup/%s" % cfg["name"], per_launch)
     out = base_line("batch-16 decode tok/s, Qwen3-MoE-30B-A3B shape (int4-g32 experts); achieved HBM GB/s vs peak", tok_s, "tok/s", steps, warmup,
                     float(ms.mean()), "configs[4]: %s, %d layers, B=%d ragged, ctx U[256,2048], greedy decode" % (cfg["name"], layers, B),
                     "synthetic: N(0,0.02) weights (Q4_K projections, int4-g32 experts, f32 router, int8 head), N(0,1) KV, random token ids",
@@ -293,7 +332,8 @@ def run_c5(args):
     out["step_hbm"] = {"algorithmic_bytes_per_step": int(step_bytes), "achieved_GBs": round(step_gbs, 1), "frac_of_peak": round(step_gbs / HBM_PEAK_GBS, 4),
                        "dense_weight_bytes": int(w_bytes), "expert_bytes": int(exp_bytes), "kv_read_bytes": int(kv_read)}
     out["roofline"] = {"bound": "hbm", "achieved": round(per_launch / (g_ms / 1e3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                       "frac": round(per_launch / (g_ms / 1e3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": traffic, "kernel": "rd_k_gemm_w4a8_moe_gateup",
+                       "frac": round(per_launch / (g_ms / 1e3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_ratio": t_ratio, "traffic_source": t_src,
+                       "kernel": "rd_k_moe_gemv_w4a8_gateup",
                        "avg_launch_ms": round(g_ms, 5), "algorithmic_bytes_per_launch": int(per_launch)}
     out["kernel_classes"] = classes
     cpu = None
@@ -351,7 +391,7 @@ def cpu_baseline_moe(res, cfg, lens, kept_kv):
         om.free_cache(cp)
     per_layer = max(t_step / n_steps - t_head, 1e-9) / nL
     full = per_layer * cfg["n_layers"] + t_head
-    return {"value": round(B / full, 3), "unit": "tok/s", "cores": threads(), "kind": "port",
+    return {"value": round(B / full, 3), "unit": "tok/s", **cpu_fields(threads()), "kind": "port",
             "sample": "oracle decodeMultiStep, %d of %d layers + int8 head, B=%d at the run's context lengths, %d greedy steps (%.1f s), "
                       "per-layer cost scaled to %d layers" % (nL, cfg["n_layers"], B, n_steps, t_step, cfg["n_layers"])}
 
@@ -442,6 +482,6 @@ def cpu_baseline_prefill(res, cfg, ids):
         n += 1
     om.free_cache(cp)
     per_layer = max(t / n - t_head, 1e-9) / nL
-    return {"value": round(1.0 / (per_layer * cfg["n_layers"]), 3), "unit": "tok/s", "cores": threads(), "kind": "port",
+    return {"value": round(1.0 / (per_layer * cfg["n_layers"]), 3), "unit": "tok/s", **cpu_fields(threads()), "kind": "port",
             "sample": "oracle, %d of %d layers, the prompt's first %d tokens one at a time (%.1f s), head time taken out, per-layer cost scaled to %d layers"
                       % (nL, cfg["n_layers"], n, t, cfg["n_layers"])}

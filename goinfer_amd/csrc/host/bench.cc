@@ -314,8 +314,8 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
         for (int i = 0; i < warmup + iters && !rc; i++) {
             const uint8_t *w = (const uint8_t *)W.p + (size_t)(i % copies) * wBytes;
             if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup)], d->stream);
-            rc = d->launch(d->k.gemm8_w4a8_moe, (unsigned)((N + 63) / 64), (unsigned)nE, 1, MOE_THREADS, (const void *)w, wStride, (const void *)Xp.p,
-                           perE ? xpStride : (size_t)0, O.as<float>(), N, nKB, T, 1, (const signed char *)R.p, nE,
+            rc = d->launch_lds(d->k.moe_gemv_w4a8, moe_gemv_grid(N, K), (unsigned)nE, 1, MOE_THREADS, moe_gemv_lds(K), (const void *)w, wStride, (const void *)Xp.p,
+                           perE ? xpStride : (size_t)0, O.as<float>(), N, K, T, 1, (const signed char *)R.p, nE,
                            (n_args >= 9 && args[8]) ? (const unsigned *)Bits.p : (const unsigned *)nullptr);
             if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup) + 1], d->stream);
         }

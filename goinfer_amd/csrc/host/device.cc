@@ -82,8 +82,9 @@ static const KName kNames[] = {
     {"rd_k_retile_w8a8_8", &Kernels::retile_w8a8_8},
     {"rd_k_retile_w4a8_8", &Kernels::retile_w4a8_8},
     {"rd_k_gemm8_q4k_gateup", &Kernels::gemm8_q4k_gateup},
-    {"rd_k_gemm8_w4a8_moe", &Kernels::gemm8_w4a8_moe},
-    {"rd_k_gemm8_w4a8_moe_gateup", &Kernels::gemm8_w4a8_moe_gateup},
+    {"rd_k_moe_gemv_w4a8", &Kernels::moe_gemv_w4a8},
+    {"rd_k_moe_gemv_w4a8_gateup", &Kernels::moe_gemv_w4a8_gateup},
+    {"rd_k_retile_w4a8_gv", &Kernels::retile_w4a8_gv},
     {"rd_k_retile_q4k8", &Kernels::retile_q4k8},
     {"rd_k_dequant_q5k", &Kernels::dequant_q5k},
     {"rd_k_retile_q5k", &Kernels::retile_q5k},
@@ -399,7 +400,7 @@ int upload_w8a8(rd_device *d, const int8_t *q, const float *row_scale, int N, in
     return RD_OK;
 }
 
-int upload_w4a8(rd_device *d, const uint8_t *nib, const uint16_t *s16, int N, int K, DevWeight *w) {
+int upload_w4a8(rd_device *d, const uint8_t *nib, const uint16_t *s16, int N, int K, DevWeight *w, bool expert) {
     if (N <= 0 || K <= 0 || K % 32 || N % 32) {
         rd_set_error("w4a8 upload: N=%d and K=%d must be multiples of 32", N, K);
         return RD_DECLINED;
@@ -411,7 +412,8 @@ int upload_w4a8(rd_device *d, const uint8_t *nib, const uint16_t *s16, int N, in
     if ((rc = raw.alloc(nb)) || (rc = rs.alloc(sb))) return rc;
     if ((rc = d->alloc(&w->tiled, (size_t)(N / 32) * nKB * 4608))) return rc;
     if ((rc = d->h2d(raw.p, nib, nb)) || (rc = d->h2d(rs.p, s16, sb))) return rc;
-    if ((rc = d->launch(d->k.retile_w4a8_8, N / 32, nKB, 1, 320, (const void *)raw.p, (const void *)rs.p, w->tiled, N, K))) return rc;
+    // an expert's weights take the tile order of the vector-ALU kernels (moe.h), a dense projection's that of the MFMA kernels
+    if ((rc = d->launch(expert ? d->k.retile_w4a8_gv : d->k.retile_w4a8_8, N / 32, nKB, 1, 320, (const void *)raw.p, (const void *)rs.p, w->tiled, N, K))) return rc;
     if ((rc = d->sync())) return rc;
     w->kind = 2, w->N = N, w->K = K;
     return RD_OK;

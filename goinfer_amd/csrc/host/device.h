@@ -21,14 +21,23 @@ constexpr size_t LIN_PANEL_BYTES = 8 * 64 * 16;
 constexpr size_t Q4K_TILE_BYTES = 4608;
 constexpr size_t A8_BLOCK_BYTES = 10240; // one A8 activation block: 256 elements x 32 rows (gemm8.h)
 inline size_t a8_bytes(int K) { return (size_t)((K + 255) / 256) * A8_BLOCK_BYTES; }
-enum { PANEL_Q4K = 0, PANEL_LIN = 1, PANEL_LIN4 = 2, PANEL_A8 = 3 };
+enum { PANEL_Q4K = 0, PANEL_LIN = 1, PANEL_LIN4 = 2, PANEL_A8 = 3, PANEL_ROW8 = 4 };
+// dynamic LDS of the experts' GEMM kernels: four rows of K elements (codes, scales, sums) + their exchange area
+inline unsigned moe_gemv_lds(int K) { return (unsigned)(4 * ((K + 255) / 256) * 320 + 1024); }
+constexpr int MOE_GEMV_MAX_K = 12288; // 4 rows x 48 blocks x 320 B + 1 KB = 61 KB of LDS
+// grid.x of rd_k_moe_gemv_w4a8 (moe.h): a wave streams about eight 256-element blocks, as whole tiles of 32 weight rows
+inline unsigned moe_gemv_grid(int N, int K) {
+    int per = std::max(1, 8 / ((K + 255) / 256));
+    if (const char *e = getenv("ROCMDECODE_MOE_TILES")) per = std::max(1, atoi(e));
+    return (unsigned)((N / 32 + 4 * per - 1) / (4 * per));
+}
 
 struct Kernels {
     hipFunction_t dequant_q4k, quant_act, reduce_splits, add_rmsnorm_quant, swiglu_quant;
     hipFunction_t unpack_act8, unpanel_a8, retile_q4k8, retile_w8a8_8, retile_w4a8_8;
     hipFunction_t gemm8[3][3]; // [weight kind 0 q4k, 1 w8a8, 2 w4a8][waves per tile 2, 4, 8]
     hipFunction_t gemm8_qkv[3][3]; // the q|k|v projection with RoPE and the KV store in its epilogue, indexed like gemm8
-    hipFunction_t gemm8_q4k_gateup, gemm8_w4a8_moe, gemm8_w4a8_moe_gateup, rope_table;
+    hipFunction_t gemm8_q4k_gateup, moe_gemv_w4a8, moe_gemv_w4a8_gateup, retile_w4a8_gv, rope_table;
     hipFunction_t dequant_q5k, retile_q5k, gemm_q5k, dequant_q6k, retile_q6k, gemm_q6k;
     hipFunction_t kv_store, kv_read, qkv_rope_store, attn_partial, attn_combine, attn_combine_quant;
     hipFunction_t kv_store_i8, qkv_rope_store_i8, attn_partial_i8, attn_partial_rows, attn_partial_rows_i8, attn_partial_deep, attn_partial_deep_i8, topk_rows, topk_hist, topk_pick, topk_finish;
@@ -43,6 +52,12 @@ struct rd_device {
     Kernels k{};
     std::vector<void *> owned; // device allocations freed at close
 
+    // the same with `lds` bytes of dynamic shared memory
+    template <typename... A> int launch_lds(hipFunction_t f, unsigned gx, unsigned gy, unsigned gz, unsigned bx, unsigned lds, A... a) {
+        void *args[] = {(void *)&a...};
+        hipError_t e = hip->ModuleLaunchKernel(f, gx, gy, gz, bx, 1, 1, lds, stream, args, nullptr);
+        return rd_hip_ok(hip, e, "hipModuleLaunchKernel") ? RD_OK : RD_ERR_HIP;
+    }
     template <typename... A> int launch(hipFunction_t f, unsigned gx, unsigned gy, unsigned gz, unsigned bx, A... a) {
         void *args[] = {(void *)&a...};
         hipError_t e = hip->ModuleLaunchKernel(f, gx, gy, gz, bx, 1, 1, 0, stream, args, nullptr);
@@ -143,7 +158,7 @@ int upload_q4k(rd_device *d, const void *blocks, int N, int K, DevWeight *w);
 int upload_q5k(rd_device *d, const void *blocks, int N, int K, DevWeight *w);
 int upload_q6k(rd_device *d, const void *blocks, int N, int K, DevWeight *w);
 int upload_w8a8(rd_device *d, const int8_t *q, const float *row_scale, int N, int K, DevWeight *w);
-int upload_w4a8(rd_device *d, const uint8_t *nib, const uint16_t *s16, int N, int K, DevWeight *w);
+int upload_w4a8(rd_device *d, const uint8_t *nib, const uint16_t *s16, int N, int K, DevWeight *w, bool expert = false);
 void free_weight(rd_device *d, DevWeight *w);
 // P[splits][32][N] = panels(Xp) . W^T ; returns the plan used
 // ldP: floats between rows of P (0 = w.N); splits > 0 forces the split count (trailing splits that get no K-block store zeros),

@@ -66,7 +66,7 @@ extern "C" void rd_model_destroy(rd_model *m) {
     free_weight(d, &m->head);
     for (void *p : {(void *)m->embed_q, (void *)m->embed_scale, (void *)m->inv_freq_dev, (void *)m->rope_cs, (void *)m->final_norm, (void *)m->tables, (void *)m->h, (void *)m->normed, (void *)m->P, (void *)m->qbuf,
                     (void *)m->part, (void *)m->cand_v, (void *)m->cand_i, (void *)m->logits, (void *)m->emb_dev, m->XpA, m->XpA2, m->XpB, (void *)m->ids, (void *)m->meta, (void *)m->router_logits, (void *)m->moe_wgt, (void *)m->moe_gu,
-                    (void *)m->moe_dn, (void *)m->moe_out, (void *)m->moe_idx, (void *)m->moe_idx_all, (void *)m->moe_rank, (void *)m->moe_bits, (void *)m->topk_ids, (void *)m->topk_vals, (void *)m->topk_z, (void *)m->topk_scratch.ghist, (void *)m->topk_scratch.ccount, (void *)m->topk_scratch.gmax, (void *)m->topk_scratch.cand_i, (void *)m->topk_scratch.cand_v, (void *)m->topk_scratch.invT, (void *)m->topk_scratch.zpart, m->XpE})
+                    (void *)m->moe_dn, (void *)m->moe_out, (void *)m->moe_idx, (void *)m->moe_idx_all, (void *)m->moe_rank, (void *)m->topk_ids, (void *)m->topk_vals, (void *)m->topk_z, (void *)m->topk_scratch.ghist, (void *)m->topk_scratch.ccount, (void *)m->topk_scratch.gmax, (void *)m->topk_scratch.cand_i, (void *)m->topk_scratch.cand_v, (void *)m->topk_scratch.invT, (void *)m->topk_scratch.zpart, m->XpE})
         d->release(p);
     if (m->host_stage) (void)d->hip->HostFree(m->host_stage);
     if (m->chain.host_ids) (void)d->hip->HostFree(m->chain.host_ids);
@@ -291,8 +291,12 @@ extern "C" int rd_model_upload_w4a8(rd_model *m, int layer, int proj, int expert
         RC(d->alloc(&l.exp_gateup, guBytes * c.n_experts));
         RC(d->alloc(&l.exp_down, dnBytes * c.n_experts));
     }
+    if (K > MOE_GEMV_MAX_K) {
+        rd_set_error("rocm resident declines: expert projection with K=%d (at most %d)", K, MOE_GEMV_MAX_K);
+        return RD_DECLINED;
+    }
     DevWeight tmp;
-    RC(upload_w4a8(d, nib, s16, N, K, &tmp));
+    RC(upload_w4a8(d, nib, s16, N, K, &tmp, true));
     size_t tb = (size_t)(N / 32) * ((K + 255) / 256) * 4608;
     uint8_t *dst = isDown ? (uint8_t *)l.exp_down + dnBytes * expert
                           : (uint8_t *)l.exp_gateup + guBytes * expert + (proj == RD_PROJ_UP ? guBytes / 2 : 0);
@@ -424,8 +428,6 @@ extern "C" int rd_model_finalize(rd_model *m) {
         RC(d->alloc((void **)&m->moe_idx, sizeof(int) * 32 * k));
         RC(d->alloc((void **)&m->moe_idx_all, sizeof(int) * (size_t)c.n_layers * 32 * k));
         RC(d->alloc((void **)&m->moe_rank, (size_t)32 * c.n_experts));
-        RC(d->alloc((void **)&m->moe_bits, sizeof(unsigned) * 8));
-        HIPCHK(MemsetAsync(m->moe_bits, 0, sizeof(unsigned) * 8, d->stream));
         RC(d->alloc(&m->XpE, (size_t)c.n_experts * a8_bytes(I)));
         HIPCHK(MemsetAsync(m->XpE, 0, (size_t)c.n_experts * a8_bytes(I), d->stream));
     }
@@ -500,6 +502,7 @@ extern "C" int rd_kv_configure_typed(rd_model *m, int slots, int ctx_cap, int kv
     RC(d->alloc((void **)&m->meta, sizeof(int) * m->meta_ints));
     constexpr int RM = rd_model::ROWS_MAX;
     m->rowSlot = m->meta, m->rowPos = m->meta + RM, m->rowLen = m->meta + 2 * RM, m->rowDraw = m->meta + 3 * RM;
+    m->moe_bits = (unsigned *)(m->meta + rd_model::META_HDR - 8);
     m->itemStart = m->meta + rd_model::META_HDR;
     m->items = (AttnItemH *)(m->meta + rd_model::META_HDR + rangeInts);
     // pinned staging, STAGE_SLOTS slots: the step's metadata block as on the device, then the embeddings
@@ -662,6 +665,7 @@ static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
     rd_device *d = m->d;
     const rd_model_desc &c = m->desc;
     int H = c.hidden, I = c.expert_inter, k = c.top_k, nE = c.n_experts;
+    unsigned *bits_dev = m->moe_bits;
     {
         Scope s(m, KC_MOE_ROUTER);
         int *trace = m->moe_idx_all + (size_t)layer * 32 * k;
@@ -675,12 +679,13 @@ static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
                 int e = m->replay_idx[(size_t)layer][(size_t)i];
                 bits[e >> 5] |= 1u << (e & 31);
             }
-            RC(d->h2d(m->moe_bits, bits, sizeof(bits)));
+            RC(d->h2d(bits_dev, bits, sizeof(bits)));
         } else {
+            // two launches: the logits over many blocks (one per token would leave the chip idle: measured twice as slow), then the routing
             RC(d->launch(d->k.matmul_f32, (unsigned)((nE + 3) / 4), (unsigned)B, 1, 256, (const float *)m->normed, (const float *)l.router,
-                         m->router_logits, B, H, nE, m->moe_bits));
+                         m->router_logits, B, H, nE, bits_dev));
             RC(d->launch(d->k.moe_route, (unsigned)B, 1, 1, 64, (const float *)m->router_logits, B, nE, k, c.norm_topk_prob, m->moe_idx, m->moe_wgt,
-                         m->moe_rank, trace, m->moe_bits));
+                         m->moe_rank, trace, bits_dev));
         }
     }
     const int nKBh = (H + 255) / 256, nKBi = (I + 255) / 256;
@@ -688,23 +693,23 @@ static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
     size_t xpStride = a8_bytes(I);
     if (I % 32 == 0 && !getenv("ROCMDECODE_NO_FUSED_MOE_GATEUP")) {
         Scope s(m, KC_MOE_GEMM); // gate|up of every touched expert + SwiGLU + quantization into the experts' down activations
-        RC(d->launch(d->k.gemm8_w4a8_moe_gateup, (unsigned)(I / 32), (unsigned)nE, 1, MOE_THREADS, (const void *)l.exp_gateup, guStride,
-                     (const void *)m->XpA, m->XpE, xpStride, I, nKBh, B, (const signed char *)m->moe_rank, nE, (const unsigned *)m->moe_bits));
+        RC(d->launch_lds(d->k.moe_gemv_w4a8_gateup, (unsigned)((I / 32 + 1) / 2), (unsigned)nE, 1, MOE_THREADS, moe_gemv_lds(H), (const void *)l.exp_gateup, guStride,
+                         (const void *)m->XpA, m->XpE, xpStride, I, H, B, (const signed char *)m->moe_rank, nE, (const unsigned *)bits_dev));
     } else {
         {
             Scope s(m, KC_MOE_GEMM);
-            RC(d->launch(d->k.gemm8_w4a8_moe, (unsigned)((2 * I + 63) / 64), (unsigned)nE, 1, MOE_THREADS, (const void *)l.exp_gateup, guStride,
-                         (const void *)m->XpA, (size_t)0, m->moe_gu, 2 * I, nKBh, B, k, (const signed char *)m->moe_rank, nE,
-                         (const unsigned *)m->moe_bits));
+            RC(d->launch_lds(d->k.moe_gemv_w4a8, moe_gemv_grid(2 * I, H), (unsigned)nE, 1, MOE_THREADS, moe_gemv_lds(H), (const void *)l.exp_gateup, guStride,
+                             (const void *)m->XpA, (size_t)0, m->moe_gu, 2 * I, H, B, k, (const signed char *)m->moe_rank, nE,
+                             (const unsigned *)bits_dev));
         }
         Scope s(m, KC_MOE_GLUE);
         RC(d->launch(d->k.moe_swiglu_quant, (unsigned)((I + 255) / 256), (unsigned)(B * k), 1, 256, (const float *)m->moe_gu, (const int *)m->moe_idx,
-                     I, k, m->XpE, xpStride));
+                     I, k, m->XpE, xpStride, (const signed char *)m->moe_rank, nE));
     }
     {
         Scope s(m, KC_MOE_GEMM_DOWN);
-        RC(d->launch(d->k.gemm8_w4a8_moe, (unsigned)((H + 63) / 64), (unsigned)nE, 1, MOE_THREADS, (const void *)l.exp_down, dnStride, (const void *)m->XpE,
-                     xpStride, m->moe_dn, H, nKBi, B, k, (const signed char *)m->moe_rank, nE, (const unsigned *)m->moe_bits));
+        RC(d->launch_lds(d->k.moe_gemv_w4a8, moe_gemv_grid(H, I), (unsigned)nE, 1, MOE_THREADS, moe_gemv_lds(I), (const void *)l.exp_down, dnStride,
+                         (const void *)m->XpE, xpStride, m->moe_dn, H, I, B, k, (const signed char *)m->moe_rank, nE, (const unsigned *)bits_dev));
     }
     if (k > MOE_FOLD_FUSED_MAX) { // else the next norm kernel folds the ranks itself as it adds them to the residual
         Scope s(m, KC_MOE_GLUE);
@@ -792,6 +797,7 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
             }
         }
         constexpr int HDR = rd_model::META_HDR;
+        memset(hm + HDR - 8, 0, sizeof(int) * 8);
         memcpy(hm + HDR, start.data(), sizeof(int) * start.size());
         memcpy(hm + HDR + rangeInts, items.data(), sizeof(AttnItemH) * items.size());
         RC(d->h2d(m->meta, hm, sizeof(int) * (HDR + rangeInts + items.size() * 4)));
@@ -898,7 +904,7 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
             {
                 Scope s(m, KC_ADD_NORM);
                 RC(d->launch(d->k.add_rmsnorm_quant, (unsigned)B, 1, 1, 1024, m->h, (const float *)m->P, plan.splits, (const float *)l.ffn_norm,
-                             c.rms_eps, H, m->XpA, (int)PANEL_A8, m->normed, (void *)nullptr, -1, m->pStride, m->xpAStride, m->xpAStride,
+                             c.rms_eps, H, m->XpA, (int)PANEL_ROW8, m->normed, (void *)nullptr, -1, m->pStride, m->xpAStride, m->xpAStride,
                              (const float *)nullptr));
             }
             RC(moe_ffn(m, B, li, l));

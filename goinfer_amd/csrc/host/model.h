@@ -74,7 +74,7 @@ struct rd_model {
     static constexpr int ROWS_MAX = 128;
     int max_rows = 32;
     size_t pStride = 0, xpAStride = 0, xpBStride = 0;
-    static constexpr int META_HDR = 3 * ROWS_MAX + ROWS_MAX * 6; // row slot, position, length and the rows' draw records (6 ints each)
+    static constexpr int META_HDR = 3 * ROWS_MAX + ROWS_MAX * 6 + 8; // row slot, position, length, the rows' draw records (6 ints each), the expert bitmap
     int *rowDraw = nullptr;               // inside meta
     const rd_draw *step_draws = nullptr;  // set by the entry point for the one step it runs; null = plain argmax for every row
     void *XpA = nullptr, *XpB = nullptr;
@@ -96,7 +96,7 @@ struct rd_model {
     float *topk_vals = nullptr;
     double *topk_z = nullptr;
     TopkScratch topk_scratch;
-    unsigned *moe_bits = nullptr;                    // bitmap of the experts the current layer's routing chose (8 words)
+    unsigned *moe_bits = nullptr;                    // inside meta: bitmap of the experts the current layer's routing chose (8 words)
     void *XpE = nullptr;                             // per-expert down panels
     // pinned host staging
     // STAGE_SLOTS slots used round-robin, so a caller that chains steps without reading anything back (the device greedy

@@ -59,3 +59,22 @@ __device__ __forceinline__ void a8_store4(uint8_t *__restrict__ A8, int m, int k
     }
 }
 
+// ROW8: the same quantized activations as plain rows, for the kernels that walk one row's groups in order (the experts' GEMMs,
+// which have a handful of rows each and run on the vector ALU): [32 rows][K] int8 codes, then [32][K/32] f32 scales, then
+// [32][K/32] f32 scaled code sums. K % 32 == 0; 40 bytes per element column, the size of the A8 blocks of the same K.
+__device__ __forceinline__ size_t row8_scales(int K) { return (size_t)32 * K; }
+__device__ __forceinline__ size_t row8_sums(int K) { return (size_t)32 * K + (size_t)32 * (K >> 5) * 4; }
+__device__ __forceinline__ void row8_store4(uint8_t *__restrict__ X, int K, int m, int k0, uint32_t codes, float sc, float gsum) {
+    *(uint32_t *)(X + (size_t)m * K + k0) = codes;
+    if ((k0 & 31) == 0) {
+        *(float *)(X + row8_scales(K) + ((size_t)m * (K >> 5) + (k0 >> 5)) * 4) = sc;
+        *(float *)(X + row8_sums(K) + ((size_t)m * (K >> 5) + (k0 >> 5)) * 4) = gsum;
+    }
+}
+__device__ __forceinline__ void row8_store1(uint8_t *__restrict__ X, int K, int m, int k, int code, float sc, float gsum) {
+    X[(size_t)m * K + k] = (uint8_t)code;
+    if ((k & 31) == 0) {
+        *(float *)(X + row8_scales(K) + ((size_t)m * (K >> 5) + (k >> 5)) * 4) = sc;
+        *(float *)(X + row8_sums(K) + ((size_t)m * (K >> 5) + (k >> 5)) * 4) = gsum;
+    }
+}

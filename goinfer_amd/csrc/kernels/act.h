@@ -4,7 +4,7 @@
 #include "a8.h"
 #include "common.h"
 
-enum { RD_PANEL_Q4K = 0, RD_PANEL_LIN = 1, RD_PANEL_LIN4 = 2, RD_PANEL_A8 = 3 };
+enum { RD_PANEL_Q4K = 0, RD_PANEL_LIN = 1, RD_PANEL_LIN4 = 2, RD_PANEL_A8 = 3, RD_PANEL_ROW8 = 4 };
 
 // One quantized element: its int8 code, the group's scale and scaled code sum, and the dequantized value code * scale that
 // the f16 panel kinds store.
@@ -31,9 +31,12 @@ __device__ __forceinline__ Quant4 quant_four(float v0, float v1, float v2, float
     return q;
 }
 
-// Store one quantized activation (element k of batch row m) in the layout the consuming GEMM reads.
-__device__ __forceinline__ void panel_store(uint8_t *__restrict__ Xp, int kind, int m, int k, const Quant1 &q) {
-    if (kind == RD_PANEL_A8) {
+// Store one quantized activation (element k of batch row m) in the layout the consuming GEMM reads. ldk: the row length, for
+// the one layout that needs it (RD_PANEL_ROW8).
+__device__ __forceinline__ void panel_store(uint8_t *__restrict__ Xp, int kind, int m, int k, const Quant1 &q, int ldk = 0) {
+    if (kind == RD_PANEL_ROW8) {
+        row8_store1(Xp, ldk, m, k, q.code, q.sc, q.gsum);
+    } else if (kind == RD_PANEL_A8) {
         Xp[a8_code_offset(m, k)] = (uint8_t)q.code;
         if ((k & 31) == 0) {
             uint8_t *p = Xp + a8_scale_offset(m, k >> 5);
@@ -54,8 +57,10 @@ __device__ __forceinline__ void panel_store(uint8_t *__restrict__ Xp, int kind, 
 
 // Four consecutive elements k0..k0+3 (k0 % 4 == 0) of batch row m. In a Q4_K panel they are the four bytes of one code
 // word and land in slots {0,1} and {4,5} (+2 for an odd sub-block) of one lane row: two 4-byte stores.
-__device__ __forceinline__ void panel_store4(uint8_t *__restrict__ Xp, int kind, int m, int k0, const Quant4 &q) {
-    if (kind == RD_PANEL_A8) {
+__device__ __forceinline__ void panel_store4(uint8_t *__restrict__ Xp, int kind, int m, int k0, const Quant4 &q, int ldk = 0) {
+    if (kind == RD_PANEL_ROW8) {
+        row8_store4(Xp, ldk, m, k0, q.codes, q.sc, q.gsum);
+    } else if (kind == RD_PANEL_A8) {
         a8_store4(Xp, m, k0, q.codes, q.sc, q.gsum);
     } else if (kind == RD_PANEL_Q4K) {
         half_t *base = (half_t *)(Xp + (size_t)(k0 >> 8) * RD_Q4K_PANEL_BYTES);
@@ -203,8 +208,8 @@ extern "C" __global__ __launch_bounds__(1024) void rd_k_add_rmsnorm_quant(float 
         float n2 = __fmul_rn(__fmul_rn(v[i].z, inv), wv[i].z), n3 = __fmul_rn(__fmul_rn(v[i].w, inv), wv[i].w);
         if (norm_out) *(float4_t *)(norm_out + (size_t)m * H + k0) = (float4_t){n0, n1, n2, n3};
         const Quant4 q = quant_four(n0, n1, n2, n3);
-        panel_store4(Xp, kind, mr, k0, q);
-        if (Xp2) panel_store4(Xp2, kind2, mr, k0, q); // a second consumer that reads another panel layout
+        panel_store4(Xp, kind, mr, k0, q, H);
+        if (Xp2) panel_store4(Xp2, kind2, mr, k0, q, H); // a second consumer that reads another panel layout
     }
 }
 

@@ -74,9 +74,12 @@ __device__ __forceinline__ i32x4_t as_i32x4(uint4_t v) {
     return r;
 }
 
-// acc += fold of one group's dots: a convert and an fma per output (the scale products come from the matrix core)
-#define RD_FOLD16(ACC, DOT, S, OFF)                                                    \
-    _Pragma("unroll") for (int r_ = 0; r_ < 16; r_++) ACC[r_] = __builtin_fmaf((float)DOT[r_], S[(OFF) + r_], ACC[r_]);
+// acc += fold of one group's dots: a convert and an fma per output (the scale products come from the matrix core). NR: how many
+// of the tile's sixteen accumulator registers hold batch rows in use: register r of lane half h is batch row (r>>2)*8 + h*4 + (r&3),
+// so a batch of at most 8 rows lives in registers 0..3 and the fold of the other twelve, three quarters of the kernel's
+// VALU work, is left out (their sums are never stored).
+#define RD_FOLD(ACC, DOT, S, OFF, NR)                                                  \
+    _Pragma("unroll") for (int r_ = 0; r_ < (NR); r_++) ACC[r_] = __builtin_fmaf((float)DOT[r_], S[(OFF) + r_], ACC[r_]);
 
 // ---------------- Q4_K ----------------
 // Tile of 32 rows x one super-block, 4608 B: the 32 headers (16 B: d, dmin, 12 scale bytes), then four planes [64 lanes][16 B]:
@@ -111,7 +114,7 @@ struct Q4K8Traits {
     }
     // acc[m][n] += sum over the super-block's 8 groups. Lane (n, h) decodes the scales of sub-blocks 2p+h, p = 0..3: the
     // lane half is the block index of the two-block scale product and the k index of the minimum product.
-    static __device__ __forceinline__ void mma(float16_t &acc, const Tile &w, const A8Regs &a, const void *, int, int lane) {
+    template <int NR> static __device__ __forceinline__ void mma(float16_t &acc, const Tile &w, const A8Regs &a, const void *, int, int lane) {
         const int h = lane >> 5;
         const uint32_t y = w.hdr.y, z = w.hdr.z, x = w.hdr.w, hx = w.hdr.x;
         half2_t dd;
@@ -145,8 +148,8 @@ struct Q4K8Traits {
             for (int i = 0; i < 4; i++) lo[i] = raw[i] & 0x0F0F0F0Fu, hi[i] = (raw[i] >> 4) & 0x0F0F0F0Fu;
             const i32x16_t d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(as_i32x4(a.c[2 * p]), as_i32x4(lo), zero16, 0, 0, 0);
             const i32x16_t d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(as_i32x4(a.c[2 * p + 1]), as_i32x4(hi), zero16, 0, 0, 0);
-            RD_FOLD16(acc, d0, s2, 0)
-            RD_FOLD16(acc, d1, s2, 16)
+            RD_FOLD(acc, d0, s2, 0, NR)
+            RD_FOLD(acc, d1, s2, 16, NR)
         }
 #pragma unroll
         for (int p = 0; p < 4; p++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.asum[p], ndm[p], acc, 0, 0, 0);
@@ -175,7 +178,7 @@ struct W8A8Traits8 {
 #pragma unroll
         for (int g = 0; g < 8; g++) w.q[g] = buf_load16_nt(r, off + lane * 16 + (g >> 2) * 4096, (g & 3) * 1024);
     }
-    static __device__ __forceinline__ void mma(float16_t &acc, const Tile &w, const A8Regs &a, const void *, int, int lane) {
+    template <int NR> static __device__ __forceinline__ void mma(float16_t &acc, const Tile &w, const A8Regs &a, const void *, int, int lane) {
         const f32x32_t zero32 = {0.f};
         const i32x16_t zero16 = {0};
 #pragma unroll
@@ -184,8 +187,8 @@ struct W8A8Traits8 {
             const f32x32_t s2 = __builtin_amdgcn_mfma_f32_32x32x1f32(a.as[p], 1.f, zero32, 0, 0, 0);
             const i32x16_t d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(as_i32x4(a.c[2 * p]), as_i32x4(w.q[2 * p]), zero16, 0, 0, 0);
             const i32x16_t d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(as_i32x4(a.c[2 * p + 1]), as_i32x4(w.q[2 * p + 1]), zero16, 0, 0, 0);
-            RD_FOLD16(acc, d0, s2, 0)
-            RD_FOLD16(acc, d1, s2, 16)
+            RD_FOLD(acc, d0, s2, 0, NR)
+            RD_FOLD(acc, d1, s2, 16, NR)
         }
     }
     static __device__ __forceinline__ void finish(float16_t &acc, const void *aux, int tile, int lane) {
@@ -232,7 +235,7 @@ struct W4A8Traits8 {
     typedef Q4K8Tile Tile;
     static constexpr int TILE_BYTES = 4608;
     static __device__ __forceinline__ void load(Tile &w, rd_rsrc_t r, int off, int lane) { Q4K8Traits::load(w, r, off, lane); }
-    static __device__ __forceinline__ void mma(float16_t &acc, const Tile &w, const A8Regs &a, const void *, int, int lane) {
+    template <int NR> static __device__ __forceinline__ void mma(float16_t &acc, const Tile &w, const A8Regs &a, const void *, int, int lane) {
         const int h = lane >> 5;
         float dsc[4], ndm[4];
 #pragma unroll
@@ -252,8 +255,8 @@ struct W4A8Traits8 {
             for (int i = 0; i < 4; i++) lo[i] = raw[i] & 0x0F0F0F0Fu, hi[i] = (raw[i] >> 4) & 0x0F0F0F0Fu;
             const i32x16_t d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(as_i32x4(a.c[2 * p]), as_i32x4(lo), zero16, 0, 0, 0);
             const i32x16_t d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(as_i32x4(a.c[2 * p + 1]), as_i32x4(hi), zero16, 0, 0, 0);
-            RD_FOLD16(acc, d0, s2, 0)
-            RD_FOLD16(acc, d1, s2, 16)
+            RD_FOLD(acc, d0, s2, 0, NR)
+            RD_FOLD(acc, d1, s2, 16, NR)
         }
 #pragma unroll
         for (int p = 0; p < 4; p++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.asum[p], ndm[p], acc, 0, 0, 0);
@@ -266,9 +269,12 @@ struct W4A8Traits8 {
 // before its weights: waiting for activations then never waits for younger weight tiles. The refills are unconditional (past
 // the end of the range the descriptor answers with zeros and touches no memory): only the second product of a round sits under
 // a branch, so the compiler's count of the loads in flight stays exact.
-template <class T>
+// NR: accumulator registers folded (RD_FOLD). aoff: the lane's byte offset inside an activation block, lane * 16 for batch row
+// lane & 31 (a caller that gathers rows passes the offset of another row, or one past every block for a row with no source:
+// the descriptor then answers zeros).
+template <class T, int NR = 16>
 __device__ __forceinline__ void gemm8_wave_loop(float16_t &acc, const uint8_t *__restrict__ wb, const uint8_t *__restrict__ ab, int nk, const void *aux,
-                                                int tile, int lane) {
+                                                int tile, int lane, int aoff) {
 #pragma unroll
     for (int i = 0; i < 16; i++) acc[i] = 0.f;
     if (nk <= 0) return;
@@ -276,16 +282,16 @@ __device__ __forceinline__ void gemm8_wave_loop(float16_t &acc, const uint8_t *_
     const rd_rsrc_t wr = make_rsrc(wb, (uint32_t)nk * T::TILE_BYTES), ar = make_rsrc(ab, (uint32_t)nk * AB);
     typename T::Tile w0, w1;
     A8Regs a0, a1;
-    a8_load(a0, ar, lane * 16);
+    a8_load(a0, ar, aoff);
     T::load(w0, wr, 0, lane);
-    a8_load(a1, ar, AB + lane * 16);
+    a8_load(a1, ar, AB + aoff);
     T::load(w1, wr, T::TILE_BYTES, lane);
     for (int it = 0; it < nk; it += 2) {
-        T::mma(acc, w0, a0, aux, tile, lane);
-        a8_load(a0, ar, (it + 2) * AB + lane * 16);
+        T::template mma<NR>(acc, w0, a0, aux, tile, lane);
+        a8_load(a0, ar, (it + 2) * AB + aoff);
         T::load(w0, wr, (it + 2) * T::TILE_BYTES, lane);
-        if (it + 1 < nk) T::mma(acc, w1, a1, aux, tile, lane);
-        a8_load(a1, ar, (it + 3) * AB + lane * 16);
+        if (it + 1 < nk) T::template mma<NR>(acc, w1, a1, aux, tile, lane);
+        a8_load(a1, ar, (it + 3) * AB + aoff);
         T::load(w1, wr, (it + 3) * T::TILE_BYTES, lane);
     }
 }
@@ -327,7 +333,7 @@ __device__ __forceinline__ void gemm8_body(const uint8_t *__restrict__ Wt, const
     const bool active = tile * 32 < N;
     float16_t acc;
     gemm8_wave_loop<T>(acc, Wt + ((size_t)(active ? tile : 0) * nKB + s0) * T::TILE_BYTES, A8 + (size_t)s0 * RD_A8_BLOCK_BYTES,
-                           active ? nk : 0, aux, tile, lane);
+                           active ? nk : 0, aux, tile, lane, lane * 16);
     gemm8_fold_waves<KW, TPB>(acc, lds);
     if (!active || kw != 0) return;
     T::finish(acc, aux, tile, lane);
@@ -386,7 +392,7 @@ __device__ __forceinline__ void gemm8_gateup_body(const uint8_t *__restrict__ Wt
     const int half = wave / KW, kw = wave % KW, t = blockIdx.x, nGate = I >> 5, tile = half * nGate + t;
     const int per = (nKB + KW - 1) / KW, s0 = kw * per, nk = max(0, min(nKB, s0 + per) - s0);
     float16_t acc;
-    gemm8_wave_loop<T>(acc, Wt + ((size_t)tile * nKB + s0) * T::TILE_BYTES, A8 + (size_t)s0 * RD_A8_BLOCK_BYTES, nk, nullptr, tile, lane);
+    gemm8_wave_loop<T>(acc, Wt + ((size_t)tile * nKB + s0) * T::TILE_BYTES, A8 + (size_t)s0 * RD_A8_BLOCK_BYTES, nk, nullptr, tile, lane, lane * 16);
     gemm8_fold_waves<KW, 2>(acc, lds);
     __syncthreads(); // the fold area is read; it now takes the two finished tiles as [gate | up][register][lane]
     if (kw == 0) {
@@ -455,7 +461,7 @@ __device__ __forceinline__ void gemm8_qkv_body(const uint8_t *__restrict__ Wt, c
         }
     }
     float16_t acc;
-    gemm8_wave_loop<T>(acc, Wt + ((size_t)tile * nKB + s0) * T::TILE_BYTES, A8 + (size_t)s0 * RD_A8_BLOCK_BYTES, nk, aux, tile, lane);
+    gemm8_wave_loop<T>(acc, Wt + ((size_t)tile * nKB + s0) * T::TILE_BYTES, A8 + (size_t)s0 * RD_A8_BLOCK_BYTES, nk, aux, tile, lane, lane * 16);
     double2 cs[PPT];
     float b1 = 0.f, b2 = 0.f;
     if (isQ || isK) {

@@ -1,17 +1,10 @@
 // moe.h — expert-major MoE FFN (goinfer decoder/mlp.go:630-726 moeMLPBatchWith; CUDA analogue backend/cuda/moe_rows.cu).
-// A decode batch has at most 32 tokens, so one 32-row MFMA tile covers every token: each expert's GEMM runs over all
-// token rows at once and stores only the rows routed to it — the ragged token-to-expert grouping costs no gather and
-// every expert's weights are streamed exactly once per step. rankOf[token][expert] (from rd_k_moe_route) is the map.
+// A step has at most 32 tokens. Every touched expert's weights are streamed once per GEMM for the rows routed to it (a second
+// time only past four rows); rankOf[token][expert] (from rd_k_moe_route) is the map from tokens to experts and ranks.
 #pragma once
 #include "act.h"
 #include "gemm8.h"
 
-// out[(token*k + rank)][N] = panels . W_e^T for the experts that have at least one token. Grid (ceil(N/128), nE), block 320 (four consumer waves and a panel producer).
-// xpStride: bytes between the experts' panel sets (0 = all experts read the same panels: the gate/up projections).
-// activeBits (may be NULL): the bitmap of experts with a token. Row y of the grid then works on the y-th expert whose bit is set,
-// and the rows past the last one exit: the blocks with work are the first in dispatch order, which spreads them evenly over
-// the XCDs and CUs (blocks are handed out round-robin; idle ones scattered among them skew that). Without the bitmap row y is
-// expert y, and exits when no token chose it.
 // The expert grid row `row` works on, or -1 (uniform over the block; every thread must call it).
 __device__ __forceinline__ int moe_block_expert(const unsigned *__restrict__ activeBits, const signed char *__restrict__ rankOf, int nE, int T, int row) {
     int e = row;
@@ -32,101 +25,285 @@ __device__ __forceinline__ int moe_block_expert(const unsigned *__restrict__ act
     return __syncthreads_or(mine) ? e : -1;
 }
 
-// Per expert the weights are W4A8 tiles of the int8-MFMA kernels (gemm8.h: 4608 B per 32 rows x 256 k), the activations A8 blocks.
-// Block: TPB tiles x KW waves, every wave on its own K range, partial sums folded through LDS in wave order (as gemm8_body).
-template <int KW, int TPB>
-__device__ __forceinline__ void moe_gemm8_body(const uint8_t *__restrict__ Wt, size_t wStride, const uint8_t *__restrict__ A8, size_t a8Stride,
-                                               float *__restrict__ out, int N, int nKB, int T, int k, const signed char *__restrict__ rankOf, int nE,
-                                               const unsigned *__restrict__ activeBits, float *lds) {
+// The experts' GEMMs run on the vector ALU, not on the matrix cores. A decode step gives an expert one to three rows (16 tokens x
+// top-8 over 128 experts), and a 32-row MFMA tile pays for all 32: the per-group fold alone (a convert and an fma per output and
+// group) costs more than the whole product does with v_dot4_i32_i8 over the rows that exist. Per wave: 32 weight rows x its share
+// of K; lane (row n, parity h) takes the groups 2p+h of every 256-element block, so one lane forms a group's whole int32 dot
+// (eight dot4) and folds it as the reference does (facc = fma(idot, aS*wS, facc); facc = fma(asum, -8*wS, facc)); the two
+// parities' sums are added at the end (even groups + odd groups), then the KW waves' in wave order. The expert's rows come four at
+// a time from LDS (codes, scales, sums; gathered by token); an expert with more than four rows takes another pass over its
+// weights. Arithmetic: exact int32 dot per group, f32 fold; the same for any number of rows in the step.
+//
+// Weight tile (rd_k_retile_w4a8_gv), 4608 B per 32 rows x 256 k like the MFMA kernels' tile: 32 headers of 16 B (the row's eight
+// group scales, f16), then four planes [64 lanes][16 B]: plane p, lane (row r, parity h), byte b = element b of group 2p+h in
+// the low nibble and element 16+b in the high nibble.
+extern "C" __global__ __launch_bounds__(320) void rd_k_retile_w4a8_gv(const uint8_t *__restrict__ nib, const uint16_t *__restrict__ s16,
+                                                                       uint8_t *__restrict__ tiled, int N, int K) {
+    const int tile = blockIdx.x, kb = blockIdx.y, t = threadIdx.x; // 288 x 16 B
+    if (t >= 288) return;
+    uint8_t *dst = tiled + ((size_t)tile * gridDim.y + kb) * 4608;
+    const int nG = K >> 5;
+    uint4_t v = {0u, 0u, 0u, 0u};
+    if (t < 32) {
+        uint16_t sc[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) sc[j] = kb * 8 + j < nG ? s16[(size_t)(tile * 32 + t) * nG + kb * 8 + j] : (uint16_t)0;
+        __builtin_memcpy(&v, sc, 16);
+    } else {
+        const int u = t - 32, p = u >> 6, lane = u & 63, r = lane & 31, h = lane >> 5;
+        const uint8_t *row = nib + (size_t)(tile * 32 + r) * (K >> 1);
+        uint8_t by[16];
+#pragma unroll
+        for (int b = 0; b < 16; b++) {
+            const int klo = kb * 256 + (2 * p + h) * 32 + b, khi = klo + 16;
+            const int lo = klo < K ? (row[klo >> 1] >> (4 * (klo & 1))) & 15 : 8, hi = khi < K ? (row[khi >> 1] >> (4 * (khi & 1))) & 15 : 8;
+            by[b] = (uint8_t)(lo | (hi << 4));
+        }
+        __builtin_memcpy(&v, by, 16);
+    }
+    *(uint4_t *)(dst + (size_t)t * 16) = v;
+}
+
+// The tokens of expert e in ascending order are its rows 0, 1, ...: *src = the token that is row (lane & 31), or -1 past the
+// last. Returns the number of rows. Every lane of the wave must call it.
+__device__ __forceinline__ int moe_expert_rows(const signed char *__restrict__ rankOf, int nE, int T, int e, int lane, int *src) {
+    const bool mine = lane < T && rankOf[(size_t)lane * nE + e] >= 0;
+    const uint32_t mk = (uint32_t)__ballot(mine);
+    uint32_t rest = mk;
+    for (int i = 0; i < (lane & 31); i++) rest &= rest - 1; // drop the lane & 31 lowest tokens
+    *src = rest ? __ffs((int)rest) - 1 : -1;
+    return __popc(mk);
+}
+
+constexpr int GV_ROWS = 4; // rows of an expert worked on per pass over its weights
+// LDS of a pass: the rows' codes [GV_ROWS][Kpad] (Kpad = K up to whole 256-blocks, zero-filled), then scales and sums [GV_ROWS][Kpad/32].
+__device__ __forceinline__ size_t gv_lds_bytes(int nKB) { return (size_t)GV_ROWS * nKB * (256 + 64); }
+
+// Stage the rows of a pass into LDS. X: ROW8 activations of K elements; row j of the pass is X's row rowOf[j] (>= 0) or all
+// zeros. All threads of the block call it with the same rowOf; the caller synchronizes.
+__device__ __forceinline__ void gv_stage(uint8_t *lds, const uint8_t *__restrict__ X, int K, int nKB, const int (&rowOf)[GV_ROWS]) {
+    const int Kpad = nKB * 256, nGp = nKB * 8, nG = K >> 5;
+    float *ldsS = (float *)(lds + (size_t)GV_ROWS * Kpad), *ldsU = ldsS + GV_ROWS * nGp;
+    for (int i = threadIdx.x; i < GV_ROWS * (Kpad >> 4); i += blockDim.x) {
+        const int j = i / (Kpad >> 4), c = i - j * (Kpad >> 4), row = j == 0 ? rowOf[0] : (j == 1 ? rowOf[1] : (j == 2 ? rowOf[2] : rowOf[3]));
+        uint4_t v = {0u, 0u, 0u, 0u};
+        if (row >= 0 && c * 16 < K) v = *(const uint4_t *)(X + (size_t)row * K + c * 16);
+        *(uint4_t *)(lds + (size_t)j * Kpad + c * 16) = v;
+    }
+    for (int i = threadIdx.x; i < GV_ROWS * nGp; i += blockDim.x) {
+        const int j = i / nGp, g = i - j * nGp, row = j == 0 ? rowOf[0] : (j == 1 ? rowOf[1] : (j == 2 ? rowOf[2] : rowOf[3]));
+        float sc = 0.f, su = 0.f;
+        if (row >= 0 && g < nG) sc = *(const float *)(X + row8_scales(K) + ((size_t)row * nG + g) * 4), su = *(const float *)(X + row8_sums(K) + ((size_t)row * nG + g) * 4);
+        ldsS[i] = sc, ldsU[i] = su;
+    }
+}
+
+// One 256-element block of the wave's tile against the R staged rows (R the same on every lane: the rows past it are skipped
+// by a scalar branch, one body of code for any R). kb: the block's index in K.
+__device__ __forceinline__ void gv_block(float (&facc)[GV_ROWS], const Q4K8Tile &w, const uint8_t *lds, int nKB, int kb, int h, int R) {
+    const int Kpad = nKB * 256, nGp = nKB * 8;
+    const float *ldsS = (const float *)(lds + (size_t)GV_ROWS * Kpad), *ldsU = ldsS + GV_ROWS * nGp;
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+        const uint32_t wd = w.hdr[p];
+        const float ws = f16_bits_to_f32((uint16_t)(h ? wd >> 16 : wd & 0xffffu)), nws = -8.f * ws;
+        const uint4_t raw = w.q[p];
+        uint32_t lo[4], hi[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) lo[i] = raw[i] & 0x0F0F0F0Fu, hi[i] = (raw[i] >> 4) & 0x0F0F0F0Fu;
+        const int g = kb * 8 + 2 * p + h;
+#pragma unroll
+        for (int j = 0; j < GV_ROWS; j++) {
+            if (j >= R) continue;
+            const uint4_t a0 = *(const uint4_t *)(lds + (size_t)j * Kpad + g * 32), a1 = *(const uint4_t *)(lds + (size_t)j * Kpad + g * 32 + 16);
+            int idot = 0;
+#pragma unroll
+            for (int i = 0; i < 4; i++) idot = __builtin_amdgcn_sdot4((int)lo[i], (int)a0[i], idot, false);
+#pragma unroll
+            for (int i = 0; i < 4; i++) idot = __builtin_amdgcn_sdot4((int)hi[i], (int)a1[i], idot, false);
+            facc[j] = __builtin_fmaf((float)idot, __fmul_rn(ldsS[j * nGp + g], ws), facc[j]);
+            facc[j] = __builtin_fmaf(ldsU[j * nGp + g], nws, facc[j]);
+        }
+    }
+}
+
+// A wave's stream of weight tiles for one pass: nTiles tiles of nKB 256-element blocks each, one after the other with three
+// blocks in flight the whole way (the next tile's first blocks are asked for while the current tile's last are worked on), so
+// the wave pays its start-up once. tileOff(q): byte offset of tile q's first block inside the descriptor; past the last tile
+// the loads go out of the descriptor's range and are answered with zeros. At the end of tile q: epi(q, facc), with facc[j] the
+// tile row's sum for staged row j on the lanes of both parities (parity 0's groups + parity 1's).
+struct GvTiles {
+    Q4K8Tile w[3];
+};
+template <class TileOff>
+__device__ __forceinline__ int gv_offset(int u, int nTiles, int nKB, TileOff tileOff) {
+    const int q = u / nKB;
+    return u < nTiles * nKB ? tileOff(q) + (u - q * nKB) * 4608 : 0x7ff00000;
+}
+// the stream's first three blocks, asked for before the pass's rows are staged so that the two waits overlap
+template <class TileOff>
+__device__ __forceinline__ void gv_first(GvTiles &t, rd_rsrc_t wr, int nTiles, TileOff tileOff, int nKB, int lane) {
+#pragma unroll
+    for (int i = 0; i < 3; i++) Q4K8Traits::load(t.w[i], wr, gv_offset(i, nTiles, nKB, tileOff), lane);
+}
+template <class TileOff, class Epi>
+__device__ __forceinline__ void gv_stream(GvTiles &t, rd_rsrc_t wr, int nTiles, TileOff tileOff, int nKB, const uint8_t *lds, int lane, int R, Epi epi) {
+    const int U = nTiles * nKB, h = lane >> 5;
+    auto off = [&](int u) { return gv_offset(u, nTiles, nKB, tileOff); };
+    float facc[GV_ROWS];
+#pragma unroll
+    for (int j = 0; j < GV_ROWS; j++) facc[j] = 0.f;
+    Q4K8Tile(&w)[3] = t.w;
+    int q = 0, kb = 0;
+    for (int u = 0; u < U; u += 3) {
+#pragma unroll
+        for (int i = 0; i < 3; i++) {
+            if (u + i < U) gv_block(facc, w[i], lds, nKB, kb, h, R);
+            Q4K8Traits::load(w[i], wr, off(u + i + 3), lane); // unconditional: the count of loads in flight stays exact
+            if (u + i < U && ++kb == nKB) {
+#pragma unroll
+                for (int j = 0; j < GV_ROWS; j++) {
+                    const float other = __shfl_xor(facc[j], 32, 64);
+                    facc[j] = h ? __fadd_rn(other, facc[j]) : __fadd_rn(facc[j], other);
+                }
+                epi(q, facc);
+#pragma unroll
+                for (int j = 0; j < GV_ROWS; j++) facc[j] = 0.f;
+                kb = 0, q++;
+            }
+        }
+    }
+}
+
+// out[(token*k + rank)][N] = X . W_e^T for the experts that have at least one token. Grid (gx, nE), block 256: four waves, each
+// streaming ceil(N / 32 / (4 gx)) consecutive tiles of 32 weight rows over the whole K (the launch picks gx: few tiles per wave
+// for a deep K, several for a shallow one, so that a wave has enough blocks to stream to pay for its start-up). X: ROW8 activations of K elements;
+// xStride: bytes between the experts' own activations, whose rows are the expert's tokens in ascending order (what
+// rd_k_moe_gemv_w4a8_gateup and rd_k_moe_swiglu_quant write), or 0: all experts read the step's rows (row = token) and gather theirs.
+// activeBits (may be NULL): the bitmap of experts with a token. Row y of the grid then works on the y-th expert whose bit is set,
+// and the rows past the last one exit: the blocks with work are the first in dispatch order, which spreads them evenly over
+// the XCDs and CUs (blocks are handed out round-robin; idle ones scattered among them skew that). Without the bitmap row y is
+// expert y, and exits when no token chose it. Dynamic LDS: gv_lds_bytes(nKB).
+extern "C" __global__ __launch_bounds__(256) void rd_k_moe_gemv_w4a8(const uint8_t *__restrict__ Wt, size_t wStride, const uint8_t *__restrict__ X,
+                                                                      size_t xStride, float *__restrict__ out, int N, int K, int T, int k,
+                                                                      const signed char *__restrict__ rankOf, int nE,
+                                                                      const unsigned *__restrict__ activeBits) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int nKB = (K + 255) >> 8;
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
-    // a8Stride != 0: every expert reads activations of its own, so all blocks of an expert are placed on one XCD (blocks go to the
-    // eight XCDs round-robin in linear order) and its activation blocks are pulled into one L2 instead of eight.
+    // xStride != 0: every expert reads activations of its own, so all blocks of an expert are placed on one XCD (blocks go to the
+    // eight XCDs round-robin in linear order) and its activations are pulled into one L2 instead of eight.
     int bx = blockIdx.x, row = blockIdx.y;
-    if (a8Stride != 0 && (gridDim.y & 7) == 0) {
+    if (xStride != 0 && (gridDim.y & 7) == 0) {
         const int gx = gridDim.x, L = row * gx + bx, j = L >> 3;
         row = (j / gx) * 8 + (L & 7), bx = j % gx;
     }
     const int e = moe_block_expert(activeBits, rankOf, nE, T, row);
     if (e < 0) return;
-    const int tile = bx * TPB + wave / KW, kw = wave % KW;
-    const bool active = tile * 32 < N;
-    const int per = (nKB + KW - 1) / KW, s0 = kw * per, nk = max(0, min(nKB, s0 + per) - s0);
-    float16_t acc;
-    gemm8_wave_loop<W4A8Traits8>(acc, Wt + (size_t)e * wStride + ((size_t)(active ? tile : 0) * nKB + s0) * W4A8Traits8::TILE_BYTES,
-                                 A8 + (size_t)e * a8Stride + (size_t)s0 * RD_A8_BLOCK_BYTES, active ? nk : 0, nullptr, tile, lane);
-    gemm8_fold_waves<KW, TPB>(acc, lds);
-    if (!active || kw != 0) return;
+    int src;
+    const int rows = moe_expert_rows(rankOf, nE, T, e, lane, &src);
+    Wt += (size_t)e * wStride, X += (size_t)e * xStride;
+    const int perWave = ((N >> 5) + 4 * (int)gridDim.x - 1) / (4 * (int)gridDim.x);
+    const int tile0 = (bx * 4 + wave) * perWave, nTiles = max(0, min(perWave, (N >> 5) - tile0));
+    const rd_rsrc_t wr = make_rsrc(Wt, (uint32_t)((N >> 5) * nKB * 4608));
+    for (int r0 = 0; r0 < rows; r0 += GV_ROWS) {
+        const int R = min(GV_ROWS, rows - r0);
+        int rowOf[GV_ROWS], tokOf[GV_ROWS]; // uniform: the pass's rows in X and their tokens (a lane is never asked for a token while it sits out a branch)
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-        const int m = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-        if (m < T) {
-            const int rank = rankOf[(size_t)m * nE + e];
-            if (rank >= 0) out[((size_t)m * k + rank) * N + tile * 32 + (lane & 31)] = acc[r];
+        for (int j = 0; j < GV_ROWS; j++) {
+            tokOf[j] = __builtin_amdgcn_readlane(src, min(r0 + j, 31));
+            rowOf[j] = r0 + j < rows ? (xStride == 0 ? tokOf[j] : r0 + j) : -1;
+        }
+        auto tileOff = [&](int q) { return (tile0 + q) * nKB * 4608; };
+        GvTiles wt;
+        gv_first(wt, wr, nTiles, tileOff, nKB, lane);
+        __syncthreads(); // the previous pass is done with the staged rows
+        gv_stage(lds, X, K, nKB, rowOf);
+        __syncthreads();
+        gv_stream(
+            wt, wr, nTiles, tileOff, nKB, lds, lane, R, [&](int q, const float(&facc)[GV_ROWS]) {
+                if (lane < 32) {
+#pragma unroll
+                    for (int j = 0; j < GV_ROWS; j++)
+                        if (j < R) out[((size_t)tokOf[j] * k + rankOf[(size_t)tokOf[j] * nE + e]) * N + (tile0 + q) * 32 + lane] = facc[j];
+                }
+            });
+    }
+}
+
+// The experts' gate|up projection with SwiGLU and the per-32 quantization in its epilogue (same values as rd_k_moe_gemv_w4a8
+// followed by rd_k_moe_swiglu_quant, bit for bit). Wt per expert: [gate rows; up rows] (2*I rows). Grid (ceil(I / 64), nE),
+// block 256: waves 0 and 2 stream gate tiles 2x and 2x+1 over the whole K, waves 1 and 3 the matching up tiles; a gate wave
+// leaves its sums in LDS and its up wave forms silu(gate) * up over the tile's 32 columns, which are one activation group,
+// quantizes it and writes it as row r0+j of the expert's own ROW8 activations XE (I elements a row). X: the step's rows, ROW8,
+// K elements. Dynamic LDS: gv_lds_bytes(nKB) + 1 KB.
+extern "C" __global__ __launch_bounds__(256) void rd_k_moe_gemv_w4a8_gateup(const uint8_t *__restrict__ Wt, size_t wStride,
+                                                                             const uint8_t *__restrict__ X, uint8_t *__restrict__ XE,
+                                                                             size_t xeStride, int I, int K, int T,
+                                                                             const signed char *__restrict__ rankOf, int nE,
+                                                                             const unsigned *__restrict__ activeBits) {
+    extern __shared__ __align__(16) uint8_t dyn[];
+    float *xch = (float *)dyn; // [2 pairs][GV_ROWS][32]: the gate waves' sums
+    uint8_t *lds = dyn + 1024;
+    const int nKB = (K + 255) >> 8;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int e = moe_block_expert(activeBits, rankOf, nE, T, blockIdx.y);
+    if (e < 0) return;
+    int src;
+    const int rows = moe_expert_rows(rankOf, nE, T, e, lane, &src);
+    Wt += (size_t)e * wStride, XE += (size_t)e * xeStride;
+    const int nGate = I >> 5, pair = wave >> 1, isUp = wave & 1, t = blockIdx.x * 2 + pair, nTiles = t < nGate ? 1 : 0;
+    const rd_rsrc_t wr = make_rsrc(Wt, (uint32_t)(2 * nGate * nKB * 4608));
+    auto tileOff = [&](int) { return (isUp * nGate + t) * nKB * 4608; };
+    for (int r0 = 0; r0 < rows; r0 += GV_ROWS) {
+        const int R = min(GV_ROWS, rows - r0);
+        int rowOf[GV_ROWS];
+#pragma unroll
+        for (int j = 0; j < GV_ROWS; j++) {
+            const int tok = __builtin_amdgcn_readlane(src, min(r0 + j, 31));
+            rowOf[j] = r0 + j < rows ? tok : -1;
+        }
+        GvTiles wt;
+        gv_first(wt, wr, nTiles, tileOff, nKB, lane);
+        __syncthreads(); // the previous pass is done with the staged rows and the exchanged sums
+        gv_stage(lds, X, K, nKB, rowOf);
+        __syncthreads();
+        float sum[GV_ROWS] = {0.f, 0.f, 0.f, 0.f};
+        gv_stream(wt, wr, nTiles, tileOff, nKB, lds, lane, R, [&](int, const float(&facc)[GV_ROWS]) {
+#pragma unroll
+            for (int j = 0; j < GV_ROWS; j++) sum[j] = facc[j];
+        });
+        if (!isUp && lane < 32) {
+#pragma unroll
+            for (int j = 0; j < GV_ROWS; j++) xch[(pair * GV_ROWS + j) * 32 + lane] = sum[j];
+        }
+        __syncthreads();
+        if (isUp && nTiles) {
+#pragma unroll
+            for (int j = 0; j < GV_ROWS; j++)
+                if (j < R) { // the same on every lane: both halves of the wave hold the row's 32 columns
+                    const Quant1 qv = quant_one(__fmul_rn(silu_f64(xch[(pair * GV_ROWS + j) * 32 + (lane & 31)]), sum[j]));
+                    if (lane < 32) panel_store(XE, RD_PANEL_ROW8, r0 + j, t * 32 + lane, qv, I);
+                }
         }
     }
 }
 
-// out[(token*k + rank)][N] = A8 . W_e^T for the experts that have at least one token. Grid (ceil(N/64), nE), block 256 (two tiles x two waves).
-// a8Stride: bytes between the experts' activation sets (0 = all experts read the same activations: the gate/up projections).
-extern "C" __global__ __launch_bounds__(256) void rd_k_gemm8_w4a8_moe(const uint8_t *__restrict__ Wt, size_t wStride, const uint8_t *__restrict__ A8,
-                                                                       size_t a8Stride, float *__restrict__ out, int N, int nKB, int T, int k,
-                                                                       const signed char *__restrict__ rankOf, int nE,
-                                                                       const unsigned *__restrict__ activeBits) {
-    __shared__ float lds[2 * 1024];
-    moe_gemm8_body<2, 2>(Wt, wStride, A8, a8Stride, out, N, nKB, T, k, rankOf, nE, activeBits, lds);
-}
-
-// The experts' gate|up projection with SwiGLU and the per-32 quantization in its epilogue (the expert twin of rd_k_gemm8_q4k_gateup;
-// same values as rd_k_gemm8_w4a8_moe followed by rd_k_moe_swiglu_quant, bit for bit: both cut K over two waves). Wt per expert:
-// [gate rows; up rows] (2*I rows). Grid (I/32, nE), block 256: waves 0,1 own gate tile x of the block's expert, waves 2,3 the
-// matching up tile; the finished tiles meet in LDS in accumulator order, every wave takes four accumulator registers, and the
-// rows routed to the expert are quantized (a half-wave holds the 32 columns of one row = one activation group) and written into
-// the expert's down-projection activations A8E.
-extern "C" __global__ __launch_bounds__(256) void rd_k_gemm8_w4a8_moe_gateup(const uint8_t *__restrict__ Wt, size_t wStride,
-                                                                              const uint8_t *__restrict__ A8, uint8_t *__restrict__ A8E,
-                                                                              size_t a8eStride, int I, int nKB, int T,
-                                                                              const signed char *__restrict__ rankOf, int nE,
-                                                                              const unsigned *__restrict__ activeBits) {
-    __shared__ float lds[2 * 1024];
-    constexpr int KW = 2;
-    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
-    const int e = moe_block_expert(activeBits, rankOf, nE, T, blockIdx.y);
-    if (e < 0) return;
-    const int half = wave / KW, kw = wave % KW, t = blockIdx.x, nGate = I >> 5, tile = half * nGate + t;
-    const int per = (nKB + KW - 1) / KW, s0 = kw * per, nk = max(0, min(nKB, s0 + per) - s0);
-    float16_t acc;
-    gemm8_wave_loop<W4A8Traits8>(acc, Wt + (size_t)e * wStride + ((size_t)tile * nKB + s0) * W4A8Traits8::TILE_BYTES, A8 + (size_t)s0 * RD_A8_BLOCK_BYTES, nk,
-                                 nullptr, tile, lane);
-    gemm8_fold_waves<KW, 2>(acc, lds);
-    __syncthreads();
-    if (kw == 0) {
-#pragma unroll
-        for (int r = 0; r < 16; r++) lds[(half * 16 + r) * 64 + lane] = acc[r];
-    }
-    __syncthreads();
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const int r = wave * 4 + j, m = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
-        const bool routed = m < T && rankOf[(size_t)m * nE + e] >= 0;
-        if (__ballot(routed) == 0) continue; // no row of this register is routed here: skip the f64 silu
-        const float a = __fmul_rn(silu_f64(lds[r * 64 + lane]), lds[(16 + r) * 64 + lane]);
-        const Quant1 q = quant_one(a);
-        if (routed) panel_store(A8E + (size_t)e * a8eStride, RD_PANEL_A8, m, t * 32 + (lane & 31), q);
-    }
-}
-
-// gate/up rows [(token,rank)][2I] -> silu(gate)*up -> per-32 quantization -> the down-projection panels of that row's expert.
-// Grid (ceil(I/256), T*k).
+// gate/up rows [(token,rank)][2I] -> silu(gate)*up -> per-32 quantization -> the down-projection activations of that row's expert,
+// at the token's place among the expert's tokens. Grid (ceil(I/256), T*k).
 extern "C" __global__ __launch_bounds__(256) void rd_k_moe_swiglu_quant(const float *__restrict__ gu, const int *__restrict__ idx, int I, int k,
-                                                                        uint8_t *__restrict__ XpE, size_t xpStride) {
-    int row = blockIdx.y, n = blockIdx.x * 256 + threadIdx.x, t = row / k, e = idx[row];
+                                                                        uint8_t *__restrict__ XpE, size_t xpStride, const signed char *__restrict__ rankOf,
+                                                                        int nE) {
+    int row = blockIdx.y, n = blockIdx.x * 256 + threadIdx.x, tok = row / k, e = idx[row];
+    int t = 0; // tokens before this one that chose the same expert
+    for (int i = 0; i < tok; i++) t += rankOf[(size_t)i * nE + e] >= 0;
     float a = 0.f;
     if (n < I) {
         float g = gu[(size_t)row * 2 * I + n], u = gu[(size_t)row * 2 * I + I + n];
         a = __fmul_rn(silu_f64(g), u);
     }
     const Quant1 q = quant_one(a);
-    if (n < I) panel_store(XpE + (size_t)e * xpStride, RD_PANEL_A8, t, n, q);
+    if (n < I) panel_store(XpE + (size_t)e * xpStride, RD_PANEL_ROW8, t, n, q, I);
 }
 
 // out[t][:] = sum over ranks, in rank order, of wgt[t][rank] * down[(t,rank)][:]  (decoder/mlp.go:100-103, addScaled: mul then add).
