@@ -280,9 +280,9 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
         for (void *p : {(void *)sc.ghist, (void *)sc.ccount, (void *)sc.gmax, (void *)sc.cand_i, (void *)sc.cand_v, (void *)sc.invT, (void *)sc.zpart})
             if (p) d->release(p);
     } else if (nm == "moe_gemm" && n_args >= 7) {
-        // args {N, K, nE, active, T, per_expert_panels, copies[, first[, bitmap]]}: the grouped expert GEMM over nE experts of which `active`
+        // args {N, K, nE, active, T, per_expert_panels, copies[, first[, bitmap[, rows]]]}: the grouped expert GEMM over nE experts of which `active`
         // have a token (spread evenly, or the first `active` ones when `first` is set: then every block with work precedes every
-        // block without in dispatch order; `bitmap`: the kernel gets the active-expert bitmap and orders the grid itself); int4 group-32 weights of arbitrary bits, `copies` weight sets used round-robin.
+        // block without in dispatch order; `bitmap`: the kernel gets the active-expert bitmap and orders the grid itself; `rows`: tokens per active expert, default 1); int4 group-32 weights of arbitrary bits, `copies` weight sets used round-robin.
         int N = (int)args[0], K = (int)args[1], nE = (int)args[2], active = (int)args[3], T = (int)args[4], perE = (int)args[5];
         int copies = (int)std::max<int64_t>(1, args[6]);
         if (N <= 0 || N % 32 || K <= 0 || K % 32 || nE < 1 || nE > 256 || active < 0 || active > nE || T < 1 || T > 32) {
@@ -296,13 +296,15 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
         if (!rc) rc = W.alloc(wBytes * copies);
         if (!rc) rc = Xp.alloc(xpStride * (perE ? nE : 1));
         if (!rc) rc = R.alloc((size_t)32 * nE);
-        if (!rc) rc = O.alloc(sizeof(float) * (size_t)T * N);
+        if (!rc) rc = O.alloc(sizeof(float) * (size_t)T * N * 8);
         if (!rc) rc = d->launch(d->k.fill_f16, 2048, 1, 1, 256, W.as<uint16_t>(), wBytes * copies / 2, 21u);
         if (!rc) rc = d->launch(d->k.fill_f16, 256, 1, 1, 256, Xp.as<uint16_t>(), xpStride * (perE ? nE : 1) / 2, 22u);
         if (!rc) {
             std::vector<signed char> rk((size_t)32 * nE, -1);
+            const int rowsPer = n_args >= 10 ? (int)std::min<int64_t>(T, std::max<int64_t>(1, args[9])) : 1;
             for (int e = 0; e < nE; e++)
-                if (n_args >= 8 && args[7] ? e < active : (long)(e + 1) * active / nE > (long)e * active / nE) rk[(size_t)(e % T) * nE + e] = 0;
+                if (n_args >= 8 && args[7] ? e < active : (long)(e + 1) * active / nE > (long)e * active / nE)
+                    for (int j = 0; j < rowsPer; j++) rk[(size_t)((e + j) % T) * nE + e] = 0;
             rc = d->h2d(R.p, rk.data(), rk.size());
             unsigned bits[8] = {0, 0, 0, 0, 0, 0, 0, 0};
             for (int e = 0; e < nE; e++)

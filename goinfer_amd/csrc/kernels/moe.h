@@ -29,14 +29,16 @@ __device__ __forceinline__ int moe_block_expert(const unsigned *__restrict__ act
 // top-8 over 128 experts), and a 32-row MFMA tile pays for all 32: the per-group fold alone (a convert and an fma per output and
 // group) costs more than the whole product does with v_dot4_i32_i8 over the rows that exist. Per wave: 32 weight rows x its share
 // of K; lane (row n, parity h) takes the groups 2p+h of every 256-element block, so one lane forms a group's whole int32 dot
-// (eight dot4) and folds it as the reference does (facc = fma(idot, aS*wS, facc); facc = fma(asum, -8*wS, facc)); the two
+// (eight dot4 over the signed values nib-8) and folds it as the reference does (facc = fma(idot, aS*wS, facc)); the two
 // parities' sums are added at the end (even groups + odd groups), then the KW waves' in wave order. The expert's rows come four at
 // a time from LDS (codes, scales, sums; gathered by token); an expert with more than four rows takes another pass over its
 // weights. Arithmetic: exact int32 dot per group, f32 fold; the same for any number of rows in the step.
 //
 // Weight tile (rd_k_retile_w4a8_gv), 4608 B per 32 rows x 256 k like the MFMA kernels' tile: 32 headers of 16 B (the row's eight
 // group scales, f16), then four planes [64 lanes][16 B]: plane p, lane (row r, parity h), byte b = element b of group 2p+h in
-// the low nibble and element 16+b in the high nibble.
+// the low nibble and element 16+b in the high nibble, each as the two's-complement nibble of its value nib-8 (= nib ^ 8): moved
+// to the top of a byte it is the int8 16*(nib-8), so a dot4 over such bytes is 16 times the group's signed dot, exactly, and
+// the 1/16 rides in the scale (a power of two).
 extern "C" __global__ __launch_bounds__(320) void rd_k_retile_w4a8_gv(const uint8_t *__restrict__ nib, const uint16_t *__restrict__ s16,
                                                                        uint8_t *__restrict__ tiled, int N, int K) {
     const int tile = blockIdx.x, kb = blockIdx.y, t = threadIdx.x; // 288 x 16 B
@@ -57,7 +59,7 @@ extern "C" __global__ __launch_bounds__(320) void rd_k_retile_w4a8_gv(const uint
         for (int b = 0; b < 16; b++) {
             const int klo = kb * 256 + (2 * p + h) * 32 + b, khi = klo + 16;
             const int lo = klo < K ? (row[klo >> 1] >> (4 * (klo & 1))) & 15 : 8, hi = khi < K ? (row[khi >> 1] >> (4 * (khi & 1))) & 15 : 8;
-            by[b] = (uint8_t)(lo | (hi << 4));
+            by[b] = (uint8_t)((lo ^ 8) | ((hi ^ 8) << 4));
         }
         __builtin_memcpy(&v, by, 16);
     }
@@ -76,14 +78,14 @@ __device__ __forceinline__ int moe_expert_rows(const signed char *__restrict__ r
 }
 
 constexpr int GV_ROWS = 4; // rows of an expert worked on per pass over its weights
-// LDS of a pass: the rows' codes [GV_ROWS][Kpad] (Kpad = K up to whole 256-blocks, zero-filled), then scales and sums [GV_ROWS][Kpad/32].
-__device__ __forceinline__ size_t gv_lds_bytes(int nKB) { return (size_t)GV_ROWS * nKB * (256 + 64); }
+// LDS of a pass: the rows' codes [GV_ROWS][Kpad] (Kpad = K up to whole 256-blocks, zero-filled), then their scales [GV_ROWS][Kpad/32].
+__device__ __forceinline__ size_t gv_lds_bytes(int nKB) { return (size_t)GV_ROWS * nKB * (256 + 32); }
 
 // Stage the rows of a pass into LDS. X: ROW8 activations of K elements; row j of the pass is X's row rowOf[j] (>= 0) or all
 // zeros. All threads of the block call it with the same rowOf; the caller synchronizes.
 __device__ __forceinline__ void gv_stage(uint8_t *lds, const uint8_t *__restrict__ X, int K, int nKB, const int (&rowOf)[GV_ROWS]) {
     const int Kpad = nKB * 256, nGp = nKB * 8, nG = K >> 5;
-    float *ldsS = (float *)(lds + (size_t)GV_ROWS * Kpad), *ldsU = ldsS + GV_ROWS * nGp;
+    float *ldsS = (float *)(lds + (size_t)GV_ROWS * Kpad);
     for (int i = threadIdx.x; i < GV_ROWS * (Kpad >> 4); i += blockDim.x) {
         const int j = i / (Kpad >> 4), c = i - j * (Kpad >> 4), row = j == 0 ? rowOf[0] : (j == 1 ? rowOf[1] : (j == 2 ? rowOf[2] : rowOf[3]));
         uint4_t v = {0u, 0u, 0u, 0u};
@@ -92,9 +94,7 @@ __device__ __forceinline__ void gv_stage(uint8_t *lds, const uint8_t *__restrict
     }
     for (int i = threadIdx.x; i < GV_ROWS * nGp; i += blockDim.x) {
         const int j = i / nGp, g = i - j * nGp, row = j == 0 ? rowOf[0] : (j == 1 ? rowOf[1] : (j == 2 ? rowOf[2] : rowOf[3]));
-        float sc = 0.f, su = 0.f;
-        if (row >= 0 && g < nG) sc = *(const float *)(X + row8_scales(K) + ((size_t)row * nG + g) * 4), su = *(const float *)(X + row8_sums(K) + ((size_t)row * nG + g) * 4);
-        ldsS[i] = sc, ldsU[i] = su;
+        ldsS[i] = row >= 0 && g < nG ? *(const float *)(X + row8_scales(K) + ((size_t)row * nG + g) * 4) : 0.f;
     }
 }
 
@@ -102,15 +102,15 @@ __device__ __forceinline__ void gv_stage(uint8_t *lds, const uint8_t *__restrict
 // by a scalar branch, one body of code for any R). kb: the block's index in K.
 __device__ __forceinline__ void gv_block(float (&facc)[GV_ROWS], const Q4K8Tile &w, const uint8_t *lds, int nKB, int kb, int h, int R) {
     const int Kpad = nKB * 256, nGp = nKB * 8;
-    const float *ldsS = (const float *)(lds + (size_t)GV_ROWS * Kpad), *ldsU = ldsS + GV_ROWS * nGp;
+    const float *ldsS = (const float *)(lds + (size_t)GV_ROWS * Kpad);
 #pragma unroll
     for (int p = 0; p < 4; p++) {
         const uint32_t wd = w.hdr[p];
-        const float ws = f16_bits_to_f32((uint16_t)(h ? wd >> 16 : wd & 0xffffu)), nws = -8.f * ws;
+        const float ws = f16_bits_to_f32((uint16_t)(h ? wd >> 16 : wd & 0xffffu));
         const uint4_t raw = w.q[p];
-        uint32_t lo[4], hi[4];
+        uint32_t lo[4], hi[4]; // bytes 16 * (nib - 8): elements 0..15 and 16..31 of the group
 #pragma unroll
-        for (int i = 0; i < 4; i++) lo[i] = raw[i] & 0x0F0F0F0Fu, hi[i] = (raw[i] >> 4) & 0x0F0F0F0Fu;
+        for (int i = 0; i < 4; i++) lo[i] = (raw[i] << 4) & 0xF0F0F0F0u, hi[i] = raw[i] & 0xF0F0F0F0u;
         const int g = kb * 8 + 2 * p + h;
 #pragma unroll
         for (int j = 0; j < GV_ROWS; j++) {
@@ -121,8 +121,8 @@ __device__ __forceinline__ void gv_block(float (&facc)[GV_ROWS], const Q4K8Tile 
             for (int i = 0; i < 4; i++) idot = __builtin_amdgcn_sdot4((int)lo[i], (int)a0[i], idot, false);
 #pragma unroll
             for (int i = 0; i < 4; i++) idot = __builtin_amdgcn_sdot4((int)hi[i], (int)a1[i], idot, false);
-            facc[j] = __builtin_fmaf((float)idot, __fmul_rn(ldsS[j * nGp + g], ws), facc[j]);
-            facc[j] = __builtin_fmaf(ldsU[j * nGp + g], nws, facc[j]);
+            // idot = 16 * sum (nib-8) * a, a multiple of 16: the shift is exact
+            facc[j] = __builtin_fmaf((float)(idot >> 4), __fmul_rn(ldsS[j * nGp + g], ws), facc[j]);
         }
     }
 }
@@ -200,12 +200,15 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_moe_gemv_w4a8(const uint8
     }
     const int e = moe_block_expert(activeBits, rankOf, nE, T, row);
     if (e < 0) return;
-    int src;
-    const int rows = moe_expert_rows(rankOf, nE, T, e, lane, &src);
     Wt += (size_t)e * wStride, X += (size_t)e * xStride;
     const int perWave = ((N >> 5) + 4 * (int)gridDim.x - 1) / (4 * (int)gridDim.x);
     const int tile0 = (bx * 4 + wave) * perWave, nTiles = max(0, min(perWave, (N >> 5) - tile0));
     const rd_rsrc_t wr = make_rsrc(Wt, (uint32_t)((N >> 5) * nKB * 4608));
+    auto tileOff = [&](int q) { return (tile0 + q) * nKB * 4608; };
+    GvTiles wt;
+    gv_first(wt, wr, nTiles, tileOff, nKB, lane); // the weights need only the expert: asked for before its rows are looked up
+    int src;
+    const int rows = moe_expert_rows(rankOf, nE, T, e, lane, &src);
     for (int r0 = 0; r0 < rows; r0 += GV_ROWS) {
         const int R = min(GV_ROWS, rows - r0);
         int rowOf[GV_ROWS], tokOf[GV_ROWS]; // uniform: the pass's rows in X and their tokens (a lane is never asked for a token while it sits out a branch)
@@ -214,9 +217,7 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_moe_gemv_w4a8(const uint8
             tokOf[j] = __builtin_amdgcn_readlane(src, min(r0 + j, 31));
             rowOf[j] = r0 + j < rows ? (xStride == 0 ? tokOf[j] : r0 + j) : -1;
         }
-        auto tileOff = [&](int q) { return (tile0 + q) * nKB * 4608; };
-        GvTiles wt;
-        gv_first(wt, wr, nTiles, tileOff, nKB, lane);
+        if (r0 > 0) gv_first(wt, wr, nTiles, tileOff, nKB, lane);
         __syncthreads(); // the previous pass is done with the staged rows
         gv_stage(lds, X, K, nKB, rowOf);
         __syncthreads();
@@ -249,12 +250,14 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_moe_gemv_w4a8_gateup(cons
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int e = moe_block_expert(activeBits, rankOf, nE, T, blockIdx.y);
     if (e < 0) return;
-    int src;
-    const int rows = moe_expert_rows(rankOf, nE, T, e, lane, &src);
     Wt += (size_t)e * wStride, XE += (size_t)e * xeStride;
     const int nGate = I >> 5, pair = wave >> 1, isUp = wave & 1, t = blockIdx.x * 2 + pair, nTiles = t < nGate ? 1 : 0;
     const rd_rsrc_t wr = make_rsrc(Wt, (uint32_t)(2 * nGate * nKB * 4608));
     auto tileOff = [&](int) { return (isUp * nGate + t) * nKB * 4608; };
+    GvTiles wt;
+    gv_first(wt, wr, nTiles, tileOff, nKB, lane); // the weights need only the expert: asked for before its rows are looked up
+    int src;
+    const int rows = moe_expert_rows(rankOf, nE, T, e, lane, &src);
     for (int r0 = 0; r0 < rows; r0 += GV_ROWS) {
         const int R = min(GV_ROWS, rows - r0);
         int rowOf[GV_ROWS];
@@ -263,8 +266,7 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_moe_gemv_w4a8_gateup(cons
             const int tok = __builtin_amdgcn_readlane(src, min(r0 + j, 31));
             rowOf[j] = r0 + j < rows ? tok : -1;
         }
-        GvTiles wt;
-        gv_first(wt, wr, nTiles, tileOff, nKB, lane);
+        if (r0 > 0) gv_first(wt, wr, nTiles, tileOff, nKB, lane);
         __syncthreads(); // the previous pass is done with the staged rows and the exchanged sums
         gv_stage(lds, X, K, nKB, rowOf);
         __syncthreads();
