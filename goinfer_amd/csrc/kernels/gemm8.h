@@ -322,7 +322,7 @@ __device__ __forceinline__ void gemm8_fold_waves(float16_t &acc, float *xch) {
 
 // Grid (ceil(N/(32*TPB)), splits), block KW*TPB waves. P[split][32][ldP] receives the sums of K-blocks [split*kbPerSplit, +kbPerSplit).
 // resid != NULL (splits must be 1): the sums are added to resid[m][n] in place instead (the residual stream), nothing goes to P.
-template <class T, int KW, int TPB>
+template <class T, int KW, int TPB, int NR = 16>
 __device__ __forceinline__ void gemm8_body(const uint8_t *__restrict__ Wt, const void *__restrict__ aux, const uint8_t *__restrict__ A8,
                                            float *__restrict__ P, int N, int nKB, int kbPerSplit, int M, int ldP, float *__restrict__ resid, float *lds) {
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
@@ -332,7 +332,7 @@ __device__ __forceinline__ void gemm8_body(const uint8_t *__restrict__ Wt, const
     const int s0 = kb0 + kw * per, nk = max(0, min(kb1, s0 + per) - s0);
     const bool active = tile * 32 < N;
     float16_t acc;
-    gemm8_wave_loop<T>(acc, Wt + ((size_t)(active ? tile : 0) * nKB + s0) * T::TILE_BYTES, A8 + (size_t)s0 * RD_A8_BLOCK_BYTES,
+    gemm8_wave_loop<T, NR>(acc, Wt + ((size_t)(active ? tile : 0) * nKB + s0) * T::TILE_BYTES, A8 + (size_t)s0 * RD_A8_BLOCK_BYTES,
                            active ? nk : 0, aux, tile, lane, lane * 16);
     gemm8_fold_waves<KW, TPB>(acc, lds);
     if (!active || kw != 0) return;
@@ -365,7 +365,13 @@ __device__ __forceinline__ void gemm8_body(const uint8_t *__restrict__ Wt, const
                                                                      const uint8_t *__restrict__ A8, float *__restrict__ P, int N, int nKB,         \
                                                                      int kbPerSplit, int M, int ldP, float *__restrict__ resid) {                   \
         __shared__ float lds[(KW > 1 ? TPB * (KW - 1) * 1024 : 1)];                                                                                  \
-        gemm8_body<TRAITS, KW, TPB>(Wt, aux, A8, P, N, nKB, kbPerSplit, M, ldP, resid, lds);                                                     \
+        /* up to 8 batch rows live in four accumulator registers, up to 16 in eight: the fold of the others is left out */                          \
+        if (M <= 8)                                                                                                                                  \
+            gemm8_body<TRAITS, KW, TPB, 4>(Wt, aux, A8, P, N, nKB, kbPerSplit, M, ldP, resid, lds);                                                  \
+        else if (M <= 16)                                                                                                                            \
+            gemm8_body<TRAITS, KW, TPB, 8>(Wt, aux, A8, P, N, nKB, kbPerSplit, M, ldP, resid, lds);                                                  \
+        else                                                                                                                                         \
+            gemm8_body<TRAITS, KW, TPB, 16>(Wt, aux, A8, P, N, nKB, kbPerSplit, M, ldP, resid, lds);                                                 \
     }
 
 RD_GEMM8_KERNEL(rd_k_gemm8_q4k_kw2, Q4K8Traits, 2, 2)
@@ -385,14 +391,14 @@ RD_GEMM8_KERNEL(rd_k_gemm8_w4a8_kw8, W4A8Traits8, 8, 1)
 // half-wave holds the 32 columns of one batch row, which is exactly one activation group of the down projection, so
 // silu(gate)*up (silu in f64, decoder/rmsnorm.go:204-207) is quantized where it sits and written in the layout the down projection reads.
 // The K loop, its wave ranges and the fold are those of the plain kernel with the same KW: the sums are the same bits.
-template <class T, int KW>
+template <class T, int KW, int NR = 16>
 __device__ __forceinline__ void gemm8_gateup_body(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ A8, uint8_t *__restrict__ XpOut, int outKind,
                                                   int I, int nKB, int M, float *lds) {
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int half = wave / KW, kw = wave % KW, t = blockIdx.x, nGate = I >> 5, tile = half * nGate + t;
     const int per = (nKB + KW - 1) / KW, s0 = kw * per, nk = max(0, min(nKB, s0 + per) - s0);
     float16_t acc;
-    gemm8_wave_loop<T>(acc, Wt + ((size_t)tile * nKB + s0) * T::TILE_BYTES, A8 + (size_t)s0 * RD_A8_BLOCK_BYTES, nk, nullptr, tile, lane, lane * 16);
+    gemm8_wave_loop<T, NR>(acc, Wt + ((size_t)tile * nKB + s0) * T::TILE_BYTES, A8 + (size_t)s0 * RD_A8_BLOCK_BYTES, nk, nullptr, tile, lane, lane * 16);
     gemm8_fold_waves<KW, 2>(acc, lds);
     __syncthreads(); // the fold area is read; it now takes the two finished tiles as [gate | up][register][lane]
     if (kw == 0) {
@@ -406,6 +412,7 @@ __device__ __forceinline__ void gemm8_gateup_body(const uint8_t *__restrict__ Wt
     for (int j = 0; j < RPW; j++) {
         const int r = wave * RPW + j;
         const int m = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+        if (r >= NR) continue; // batch rows past M: nothing folded, nothing to store
         const float a = __fmul_rn(silu_f64(lds[r * 64 + lane]), lds[(16 + r) * 64 + lane]);
         const Quant1 q = quant_one(a);
         if (outKind == RD_PANEL_A8) {
@@ -422,7 +429,12 @@ __device__ __forceinline__ void gemm8_gateup_body(const uint8_t *__restrict__ Wt
 extern "C" __global__ __launch_bounds__(256) void rd_k_gemm8_q4k_gateup(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ A8,
                                                                          uint8_t *__restrict__ XpOut, int outKind, int I, int nKB, int M) {
     __shared__ float lds[2 * 1024];
-    gemm8_gateup_body<Q4K8Traits, 2>(Wt, A8, XpOut, outKind, I, nKB, M, lds);
+    if (M <= 8)
+        gemm8_gateup_body<Q4K8Traits, 2, 4>(Wt, A8, XpOut, outKind, I, nKB, M, lds);
+    else if (M <= 16)
+        gemm8_gateup_body<Q4K8Traits, 2, 8>(Wt, A8, XpOut, outKind, I, nKB, M, lds);
+    else
+        gemm8_gateup_body<Q4K8Traits, 2, 16>(Wt, A8, XpOut, outKind, I, nKB, M, lds);
 }
 
 // ---------------- q|k|v projection with bias, RoPE and the KV store in its epilogue ----------------
@@ -438,7 +450,7 @@ struct QkvEpilogue {
     const float *bias;
     int tabStride, nH, nKV, HD, row0;
 };
-template <class T, int KW>
+template <class T, int KW, int NR = 16>
 __device__ __forceinline__ void gemm8_qkv_body(const uint8_t *__restrict__ Wt, const void *__restrict__ aux, const uint8_t *__restrict__ A8, int N, int nKB,
                                                int M, const QkvEpilogue &e, float *lds) {
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
@@ -461,7 +473,7 @@ __device__ __forceinline__ void gemm8_qkv_body(const uint8_t *__restrict__ Wt, c
         }
     }
     float16_t acc;
-    gemm8_wave_loop<T>(acc, Wt + ((size_t)tile * nKB + s0) * T::TILE_BYTES, A8 + (size_t)s0 * RD_A8_BLOCK_BYTES, nk, aux, tile, lane, lane * 16);
+    gemm8_wave_loop<T, NR>(acc, Wt + ((size_t)tile * nKB + s0) * T::TILE_BYTES, A8 + (size_t)s0 * RD_A8_BLOCK_BYTES, nk, aux, tile, lane, lane * 16);
     double2 cs[PPT];
     float b1 = 0.f, b2 = 0.f;
     if (isQ || isK) {
@@ -507,7 +519,12 @@ __device__ __forceinline__ void gemm8_qkv_body(const uint8_t *__restrict__ Wt, c
         const int *__restrict__ rowPos, const double *__restrict__ cs, const float *__restrict__ bias, int nH, int nKV, int HD, int row0) {             \
         __shared__ float lds[KW > 2 ? (KW - 1) * 1024 : 32 * 33];                                                                                      \
         QkvEpilogue e{q, Kp, Vp, tables, rowSlot, rowPos, (const double2 *)cs, bias, tabStride, nH, nKV, HD, row0};                                    \
-        gemm8_qkv_body<TRAITS, KW>(Wt, aux, A8, N, nKB, M, e, lds);                                                                                    \
+        if (M <= 8)                                                                                                                                    \
+            gemm8_qkv_body<TRAITS, KW, 4>(Wt, aux, A8, N, nKB, M, e, lds);                                                                             \
+        else if (M <= 16)                                                                                                                              \
+            gemm8_qkv_body<TRAITS, KW, 8>(Wt, aux, A8, N, nKB, M, e, lds);                                                                             \
+        else                                                                                                                                           \
+            gemm8_qkv_body<TRAITS, KW, 16>(Wt, aux, A8, N, nKB, M, e, lds);                                                                            \
     }
 RD_GEMM8_QKV_KERNEL(rd_k_gemm8_q4k_qkv_kw2, Q4K8Traits, 2)
 RD_GEMM8_QKV_KERNEL(rd_k_gemm8_q4k_qkv_kw4, Q4K8Traits, 4)
