@@ -152,7 +152,10 @@ def run_c4(args):
             a[0] += t
             a[1] += n
     kern = "attn_partial"
-    avg_ms = prof[kern][0] / prof[kern][1]
+    single_ms = prof[kern][0] / prof[kern][1]  # an event pair around every launch: carries the events' own 2-3 us
+    # the kernel's average launch duration proper: every layer's launch back to back between one pair of events (three steps' worth)
+    chain = [res.model.bench_attn_chain(slots, pos_prof + rep, ids0) for rep in range(3)]
+    avg_ms = float(np.mean([c[0] for c in chain]))
     # per launch (one layer): every sequence's K and V rows once (f16, or int8 and their scales), plus q in and partial results out
     G = cfg["n_heads"] // cfg["n_kv"]
     kv_launch = float((pos_prof + 2).sum()) * kv_pos_bytes / cfg["n_layers"]
@@ -162,7 +165,9 @@ def run_c4(args):
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": traffic, "traffic_ratio": t_ratio, "traffic_source": t_src,
                 "kernel": "rd_k_attn_partial" if args.kv == "f16" else "rd_k_attn_partial_i8", "avg_launch_ms": round(avg_ms, 5),
-                "timing": "HIP events around every launch of the kernel in three extra steps after the timed ones (includes the launch gap; rocprofv3's kernel duration is 3-4 us shorter)",
+                "avg_launch_ms_event_pair_per_launch": round(single_ms, 5),
+                "timing": "one pair of HIP events on the launch stream around the kernel's launches of all layers, back to back, at the context lengths right "
+                          "after the timed steps (3 x %d launches); an event pair around every single launch reads 2-3 us more (avg_launch_ms_event_pair_per_launch)" % chain[0][1],
                 "algorithmic_bytes_per_launch": int(kv_launch + q_launch),
                 "step_frac": round(step_gbs / HBM_PEAK_GBS, 4)}
     classes = {k: {"ms_per_step": round(v[0] / 3, 4), "launches_per_step": v[1] // 3} for k, v in prof.items()}

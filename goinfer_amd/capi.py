@@ -19,7 +19,7 @@ EXPORTS = [
     "rd_attn_ragged", "rd_moe_route", "rd_rmsnorm", "rd_rope", "rd_model_create", "rd_model_destroy",
     "rd_model_upload_q4k", "rd_model_upload_w8a8", "rd_model_upload_w4a8", "rd_model_upload_f32", "rd_model_finalize",
     "rd_kv_configure", "rd_kv_upload", "rd_kv_truncate", "rd_kv_reset", "rd_step_batch", "rd_forward",
-    "rd_last_moe_indices", "rd_model_upload_embedding", "rd_bench_steps", "rd_bench_profile", "rd_bench_prefill", "rd_bench_class_count",
+    "rd_last_moe_indices", "rd_model_upload_embedding", "rd_bench_steps", "rd_bench_profile", "rd_bench_attn_chain", "rd_bench_prefill", "rd_bench_class_count",
     "rd_bench_class_name", "rd_bench_kernel", "rd_gateup_q4k_quant", "rd_moe_replay", "rd_bench_attn", "rd_step_ragged", "rd_prefill_last",
     "rd_kv_configure_typed", "rd_attn_ragged_i8", "rd_attn_ragged_rows", "rd_plan_attention", "rd_plan_gemm", "rd_step_batch_topk", "rd_last_logits", "rd_topk_rows", "rd_bench_attn_i8", "rd_step_ragged_draw", "rd_forward_no_logits",
     "rd_step_batch_draw", "rd_sample_rows", "rd_greedy_chain_start", "rd_greedy_chain_next", "rd_sample_chain_start",
@@ -517,6 +517,15 @@ class Model:
         check(L.rd_bench_prefill(self.h, int(slot), len(ids), _p(ids), 1 if profile else 0, C.byref(total), _p(ms), _p(cnt)), "rd_bench_prefill")
         classes = {L.rd_bench_class_name(i).decode(): (float(ms[i]), int(cnt[i])) for i in range(n) if cnt[i]}
         return (float(total.value), classes) if profile else float(total.value)
+
+    def bench_attn_chain(self, slots, pos, ids0, reps=1):
+        """(ms per launch, launches) of the attention kernel launched back to back for every layer between one pair of events."""
+        slots = np.ascontiguousarray(slots, dtype=np.int32)
+        pos = np.ascontiguousarray(pos, dtype=np.int32)
+        ids0 = np.ascontiguousarray(ids0, dtype=np.int32)
+        ms, n = C.c_float(0), C.c_int(0)
+        check(lib().rd_bench_attn_chain(self.h, len(slots), _p(slots), _p(pos), _p(ids0), reps, C.byref(ms), C.byref(n)), "rd_bench_attn_chain")
+        return float(ms.value), int(n.value)
 
     def bench_profile(self, slots, pos, ids0):
         L = lib()

@@ -69,6 +69,32 @@ extern "C" int rd_bench_profile(rd_model *m, int B, const int *slot, const int *
     return rc ? rc : rc2;
 }
 
+// The attention kernel's average launch duration without an event pair around every launch: one step as in rd_bench_profile
+// (which leaves its work list, q rows and KV on the device), then the kernel of every layer launched back to back `reps` times
+// between ONE pair of events on the launch stream. *ms_per_launch = elapsed / (layers * reps); *launches = layers * reps.
+extern "C" int rd_bench_attn_chain(rd_model *m, int B, const int *slot, const int *pos, const int *ids0, int reps, float *ms_per_launch, int *launches) {
+    if (!m || !slot || !pos || !ids0 || !ms_per_launch || !launches || reps < 1) return RD_ERR_ARG;
+    rd_device *d = m->d;
+    RC(d->h2d(m->ids, ids0, sizeof(int) * (size_t)B));
+    RC(model_step(m, B, slot, pos, nullptr, nullptr, RD_WANT_ARGMAX, nullptr, nullptr));
+    RC(d->sync());
+    hipEvent_t a, b2;
+    (void)d->hip->EventCreate(&a), (void)d->hip->EventCreate(&b2);
+    int rc = RD_OK;
+    (void)d->hip->EventRecord(a, d->stream);
+    for (int r = 0; r < reps && !rc; r++)
+        for (auto &l : m->layers)
+            if ((rc = launch_attn_partial(m, l, m->last_items, m->last_grouped))) break;
+    (void)d->hip->EventRecord(b2, d->stream);
+    int rc2 = d->sync();
+    float ms = 0.f;
+    if (!rc && !rc2) (void)d->hip->EventElapsedTime(&ms, a, b2);
+    (void)d->hip->EventDestroy(a), (void)d->hip->EventDestroy(b2);
+    *launches = reps * (int)m->layers.size();
+    *ms_per_launch = ms / (float)*launches;
+    return rc ? rc : rc2;
+}
+
 // A prompt pass with every input on the device: rows 0..n-1 of `slot` from token ids through the embedding table, in the passes
 // rd_prefill_last makes (all rows but the last build only their K/V, as wide as the step goes; the last is a one-row step with
 // the head). ms_total: the whole prompt, HIP events on the launch stream. profile != 0: an event pair around every kernel class

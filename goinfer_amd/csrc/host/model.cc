@@ -719,6 +719,20 @@ static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
     return RD_OK;
 }
 
+// The attention kernel of one layer over the step's work list (nItems items already on the device).
+int launch_attn_partial(rd_model *m, const LayerW &l, size_t nItems, bool grouped) {
+    rd_device *d = m->d;
+    const rd_model_desc &c = m->desc;
+    const int nH = c.n_heads, nKV = c.n_kv_heads, HD = c.head_dim;
+    if (m->kv_type == RD_KV_I8)
+        return d->launch(attn_partial_kernel(d, true, grouped, nItems), (unsigned)nItems, 1, 1, 64, (const void *)m->items, (const int *)m->rowLen, (const int *)m->rowSlot,
+                         (const int *)m->tables, m->blocks_per_slot, (const signed char *)l.Kp, (const signed char *)l.Vp, (const float *)l.Ksc,
+                         (const float *)l.Vsc, (const float *)m->qbuf, m->part, nH, nKV, HD, c.attn_scale, c.attn_softcap);
+    return d->launch(attn_partial_kernel(d, false, grouped, nItems), (unsigned)nItems, 1, 1, 64, (const void *)m->items, (const int *)m->rowLen, (const int *)m->rowSlot,
+                     (const int *)m->tables, m->blocks_per_slot, (const uint16_t *)l.Kp, (const uint16_t *)l.Vp, (const float *)m->qbuf, m->part,
+                     nH, nKV, HD, c.attn_scale, c.attn_softcap);
+}
+
 // emb_host: [B][hidden] on the host, or emb_dev already on the device (benchmark loop). Logits/ids are host pointers.
 int model_step(rd_model *m, int B, const int *slot, const int *pos, const float *emb_host, const float *emb_dev, int want, float *logits,
                int *ids, bool multirow) {
@@ -765,6 +779,7 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
     bool grouped = false;
     RC(build_attn_items(m, B, slot, pos, items, start, &grouped));
     const int partRows = grouped ? ATTN_TILE_ROWS : nH / nKV;
+    m->last_items = items.size(), m->last_grouped = grouped;
     // Stage the step's metadata (and host embeddings) in pinned memory and upload it asynchronously. A slot is reused only
     // once the upload it last fed has completed, which its event tells.
     const unsigned stage_slot = m->stage_next++ % rd_model::STAGE_SLOTS;
@@ -859,14 +874,7 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
         }
         {
             Scope s(m, KC_ATTN_PARTIAL);
-            if (m->kv_type == RD_KV_I8)
-                RC(d->launch(attn_partial_kernel(d, true, grouped, items.size()), (unsigned)items.size(), 1, 1, 64, (const void *)m->items, (const int *)m->rowLen, (const int *)m->rowSlot,
-                             (const int *)m->tables, m->blocks_per_slot, (const signed char *)l.Kp, (const signed char *)l.Vp, (const float *)l.Ksc,
-                             (const float *)l.Vsc, (const float *)m->qbuf, m->part, nH, nKV, HD, c.attn_scale, c.attn_softcap));
-            else
-                RC(d->launch(attn_partial_kernel(d, false, grouped, items.size()), (unsigned)items.size(), 1, 1, 64, (const void *)m->items, (const int *)m->rowLen, (const int *)m->rowSlot,
-                         (const int *)m->tables, m->blocks_per_slot, (const uint16_t *)l.Kp, (const uint16_t *)l.Vp, (const float *)m->qbuf, m->part,
-                         nH, nKV, HD, c.attn_scale, c.attn_softcap));
+            RC(launch_attn_partial(m, l, items.size(), grouped));
         }
         {
             Scope s(m, KC_ATTN_COMBINE);

@@ -117,7 +117,10 @@ struct rd_model {
     std::vector<std::vector<signed char>> replay_rank;
 
     StepTimer timer;
+    size_t last_items = 0; // the last step's attention work list, still on the device (rd_bench_attn_chain replays it)
+    bool last_grouped = false;
 };
+int launch_attn_partial(rd_model *m, const LayerW &l, size_t nItems, bool grouped);
 
 // multirow: a slot may carry several rows at consecutive positions (ragged verify / prefill rows)
 int model_step(rd_model *m, int B, const int *slot, const int *pos, const float *emb_host, const float *emb_dev, int want, float *logits,

@@ -276,6 +276,10 @@ int rd_bench_steps(rd_model *m, int B, const int *slot, const int *pos0, const i
 /* One step with a HIP-event pair around every kernel class: class_ms[n] total milliseconds and class_n[n] launches,
  * n = rd_bench_class_count(); names from rd_bench_class_name. */
 int rd_bench_profile(rd_model *m, int B, const int *slot, const int *pos, const int *ids0, float *class_ms, int *class_n);
+/* The attention kernel's average launch duration: one step as above, then that kernel of every layer (its own KV, the step's
+ * work list) launched back to back `reps` times between one pair of HIP events on the launch stream, so no event sits between
+ * two launches. *ms_per_launch = elapsed / *launches, *launches = layers * reps. Measurement only. */
+int rd_bench_attn_chain(rd_model *m, int B, const int *slot, const int *pos, const int *ids0, int reps, float *ms_per_launch, int *launches);
 /* A whole prompt pass timed on the device: rows 0..n-1 of `slot` (reset first) from token ids through the embedding table, in
  * rd_prefill_last's passes. ms_total: milliseconds for the prompt; profile != 0 also fills class_ms / class_n as
  * rd_bench_profile does. */
