@@ -249,7 +249,7 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
             if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup)], d->stream);
             for (int m0 = 0; m0 < M && !rc; m0 += 32)
                 rc = d->launch(d->k.gemm8_q4k_gateup, (unsigned)(I / 32), 1, 1, GATEUP_THREADS, (const void *)w.tiled, (const void *)Xp.p, Xo.as<uint8_t>(),
-                               (int)PANEL_A8, I, K / 256, std::min(32, M - m0));
+                               (int)PANEL_A8, I, K / 256, std::min(32, M - m0), (size_t)0, (size_t)0);
             if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup) + 1], d->stream);
         }
         if (!rc) rc = d->sync();

@@ -426,8 +426,10 @@ void free_weight(rd_device *d, DevWeight *w) {
     *w = DevWeight();
 }
 
-int launch_gemm(rd_device *d, const DevWeight &w, const void *Xp, float *P, int M, GemmPlan *plan_out, int ldP, int splits, int kw, float *resid) {
-    if (M < 1 || M > 32) {
+int launch_gemm(rd_device *d, const DevWeight &w, const void *Xp, float *P, int M, GemmPlan *plan_out, int ldP, int splits, int kw, float *resid,
+                size_t xpStride, size_t pStride) {
+    const bool tiles_in_grid = is_gemm8_kind(w.kind) && M > 32; // the int8 kernels take further M-tiles as grid.z
+    if (M < 1 || (M > 32 && !tiles_in_grid) || M > GEMM_WIDE_ROWS) {
         rd_set_error("gemm: M=%d outside 1..32", M);
         return RD_ERR_ARG;
     }
@@ -441,8 +443,8 @@ int launch_gemm(rd_device *d, const DevWeight &w, const void *Xp, float *P, int 
     if (is_gemm8_kind(w.kind)) {
         const int tiles = w.N / 32, tpb = p.kw == 2 ? 2 : 1;
         hipFunction_t f = d->k.gemm8[w.kind][p.kw == 8 ? 2 : (p.kw == 4 ? 1 : 0)];
-        return d->launch(f, (unsigned)((tiles + tpb - 1) / tpb), (unsigned)p.splits, 1, (unsigned)(64 * p.kw * tpb), (const void *)w.tiled, (const void *)w.scales, Xp, P,
-                         w.N, nKB, p.kbPerSplit, M, ldP, resid);
+        return d->launch(f, (unsigned)((tiles + tpb - 1) / tpb), (unsigned)p.splits, (unsigned)((M + 31) / 32), (unsigned)(64 * p.kw * tpb), (const void *)w.tiled,
+                         (const void *)w.scales, Xp, P, w.N, nKB, p.kbPerSplit, M, ldP, resid, xpStride, pStride);
     }
     if (resid) {
         rd_set_error("gemm: weight kind %d has no residual epilogue", w.kind);
@@ -458,6 +460,7 @@ int launch_gemm_wide(rd_device *d, const DevWeight &w, const void *Xp, size_t xp
         rd_set_error("wide gemm: M=%d outside 1..%d", M, GEMM_WIDE_ROWS);
         return RD_ERR_ARG;
     }
+    if (is_gemm8_kind(w.kind)) return launch_gemm(d, w, Xp, P, M, plan_out, ldP, splits, kw, nullptr, xpStride, pStride); // all M-tiles in one launch
     for (int m0 = 0, mt = 0; m0 < M; m0 += 32, mt++) {
         int rc = launch_gemm(d, w, (const char *)Xp + (size_t)mt * xpStride, P + (size_t)mt * pStride, std::min(32, M - m0), plan_out, ldP, splits, kw);
         if (rc) return rc;

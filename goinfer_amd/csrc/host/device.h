@@ -166,11 +166,13 @@ void free_weight(rd_device *d, DevWeight *w);
 // Q4_K, int8 and int4-g32 weights go through the int8-MFMA kernels over A8 activation blocks (gemm8.h), Q5_K and Q6_K through
 // the f16-MFMA kernels over f16 panels (kquant.h). kw > 0 forces the waves per tile of the int8-MFMA kinds.
 // resid != NULL (int8-MFMA kinds, one split): the sums are added to resid[m][n] (row stride ldP) in place and nothing goes to P.
+// M > 32 (int8-MFMA kinds only): further M-tiles of 32 rows, xpStride bytes / pStride floats apart, ride in the same launch (grid.z).
 int launch_gemm(rd_device *d, const DevWeight &w, const void *Xp, float *P, int M, GemmPlan *plan, int ldP = 0, int splits = 0, int kw = 0,
-                float *resid = nullptr);
+                float *resid = nullptr, size_t xpStride = 0, size_t pStride = 0);
 inline bool is_gemm8_kind(int kind) { return kind >= 0 && kind <= 2; }
 // Up to 128 rows as M-tiles of 32: M-tile mt reads its panels at Xp + mt*xpStride (bytes) and writes its partial sums at
-// P + mt*pStride (floats), each laid out as launch_gemm's: one launch_gemm per M-tile, so a row is the same row whatever pass it rides in.
+// P + mt*pStride (floats), each laid out as launch_gemm's; the int8 kernels take the M-tiles as grid.z of one launch, the others one
+// launch per M-tile. Either way a row is the same row whatever pass it rides in.
 constexpr int GEMM_WIDE_ROWS = 128;
 int launch_gemm_wide(rd_device *d, const DevWeight &w, const void *Xp, size_t xpStride, float *P, size_t pStride, int M, GemmPlan *plan, int ldP = 0,
                      int splits = 0, int kw = 0);

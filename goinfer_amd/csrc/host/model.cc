@@ -847,14 +847,13 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
         GemmPlan plan;
         RC(add_norm_quant(m, B, resP, resSplits, l.attn_norm, l.qkv, m->XpA, nullptr, resW));
         if (qkv_fusable(m, l)) {
-            Scope s(m, KC_GEMM_QKV); // projection, bias, RoPE and the KV store in one launch per M-tile
+            Scope s(m, KC_GEMM_QKV); // projection, bias, RoPE and the KV store in one launch (M-tiles of 32 rows as grid.z)
             const DevWeight &w = l.qkv;
             const int nKB = kblocks_for(w), kw = plan_gemm(w.kind, w.N, nKB).kw; // the plain GEMM's waves per tile, in one split
-            for (int m0 = 0, mt = 0; m0 < B; m0 += 32, mt++)
-                RC(d->launch(d->k.gemm8_qkv[w.kind][kw == 8 ? 2 : (kw == 4 ? 1 : 0)], (unsigned)(w.N / 32), 1, 1, (unsigned)(64 * kw), (const void *)w.tiled, (const void *)w.scales,
-                             (const void *)((const char *)m->XpA + (size_t)mt * m->xpAStride), w.N, nKB, std::min(32, B - m0), m->qbuf, l.Kp, l.Vp,
-                             (const int *)m->tables, m->blocks_per_slot, (const int *)m->rowSlot, (const int *)m->rowPos, (const double *)m->rope_cs,
-                             (const float *)l.qkv_bias, nH, nKV, HD, m0));
+            RC(d->launch(d->k.gemm8_qkv[w.kind][kw == 8 ? 2 : (kw == 4 ? 1 : 0)], (unsigned)(w.N / 32), 1, (unsigned)((B + 31) / 32), (unsigned)(64 * kw),
+                         (const void *)w.tiled, (const void *)w.scales, (const void *)m->XpA, w.N, nKB, B, m->qbuf, l.Kp, l.Vp, (const int *)m->tables,
+                         m->blocks_per_slot, (const int *)m->rowSlot, (const int *)m->rowPos, (const double *)m->rope_cs, (const float *)l.qkv_bias, nH, nKV,
+                         HD, m->xpAStride));
         } else {
             {
                 Scope s(m, KC_GEMM_QKV);
@@ -887,10 +886,10 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
         }
         if (c.n_experts == 0) {
             RC(add_norm_quant(m, B, m->P, plan.splits, l.ffn_norm, l.gateup, m->XpA, nullptr));
-            if (B <= 32 && gateup_fusable(c, l.gateup) && !getenv("ROCMDECODE_NO_FUSED_GATEUP")) {
-                Scope s(m, KC_GEMM_GATEUP); // gate|up GEMM + SwiGLU + quantization in one launch
-                RC(d->launch(d->k.gemm8_q4k_gateup, (unsigned)(c.inter / 32), 1, 1, GATEUP_THREADS, (const void *)l.gateup.tiled, (const void *)m->XpA, m->XpB,
-                             panel_kind_for(l.down), c.inter, H / 256, B));
+            if (gateup_fusable(c, l.gateup) && !getenv("ROCMDECODE_NO_FUSED_GATEUP")) {
+                Scope s(m, KC_GEMM_GATEUP); // gate|up GEMM + SwiGLU + quantization in one launch (M-tiles of 32 rows as grid.z)
+                RC(d->launch(d->k.gemm8_q4k_gateup, (unsigned)(c.inter / 32), 1, (unsigned)((B + 31) / 32), GATEUP_THREADS, (const void *)l.gateup.tiled,
+                             (const void *)m->XpA, m->XpB, panel_kind_for(l.down), c.inter, H / 256, B, m->xpAStride, m->xpBStride));
             } else {
                 {
                     Scope s(m, KC_GEMM_GATEUP);

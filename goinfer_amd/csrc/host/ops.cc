@@ -128,7 +128,7 @@ extern "C" int rd_gateup_q4k_quant(rd_device *d, const void *Wg, const void *Wu,
             RC(d->h2d(A.p, a + (size_t)m0 * K, sizeof(float) * (size_t)mc * K));
             RC(quantize_rows(d, A.as<float>(), mc, K, PANEL_A8, 0, Xp.p));
             RC(d->launch(d->k.gemm8_q4k_gateup, (unsigned)(I / 32), 1, 1, GATEUP_THREADS, (const void *)w.tiled, (const void *)Xp.p, X2.as<uint8_t>(),
-                         (int)PANEL_A8, I, K / 256, mc));
+                         (int)PANEL_A8, I, K / 256, mc, (size_t)0, (size_t)0));
             RC(d->launch(d->k.unpanel_a8, (unsigned)(I / 256), (unsigned)mc, 1, 256, (const void *)X2.p, O.as<float>(), I));
             RC(d->d2h(dst + (size_t)m0 * I, O.p, sizeof(float) * (size_t)mc * I));
         }

@@ -360,11 +360,17 @@ __device__ __forceinline__ void gemm8_body(const uint8_t *__restrict__ Wt, const
     }
 }
 
+// Rows past 32 are further M-tiles of 32, one per grid.z: M-tile z reads its activations a8Stride bytes further on and writes its
+// sums pStride floats further on; the tiles of a launch are independent and a row's sums do not depend on how many there are.
 #define RD_GEMM8_KERNEL(NAME, TRAITS, KW, TPB)                                                                                                       \
     extern "C" __global__ __launch_bounds__(64 * KW * TPB) void NAME(const uint8_t *__restrict__ Wt, const void *__restrict__ aux,                   \
                                                                      const uint8_t *__restrict__ A8, float *__restrict__ P, int N, int nKB,         \
-                                                                     int kbPerSplit, int M, int ldP, float *__restrict__ resid) {                   \
+                                                                     int kbPerSplit, int M, int ldP, float *__restrict__ resid, size_t a8Stride,   \
+                                                                     size_t pStride) {                                                              \
         __shared__ float lds[(KW > 1 ? TPB * (KW - 1) * 1024 : 1)];                                                                                  \
+        const int z = blockIdx.z;                                                                                                                    \
+        A8 += (size_t)z * a8Stride, P += (size_t)z * pStride, M = min(32, M - 32 * z);                                                               \
+        if (resid) resid += (size_t)z * 32 * ldP;                                                                                                    \
         /* up to 8 batch rows live in four accumulator registers, up to 16 in eight: the fold of the others is left out */                          \
         if (M <= 8)                                                                                                                                  \
             gemm8_body<TRAITS, KW, TPB, 4>(Wt, aux, A8, P, N, nKB, kbPerSplit, M, ldP, resid, lds);                                                  \
@@ -426,9 +432,12 @@ __device__ __forceinline__ void gemm8_gateup_body(const uint8_t *__restrict__ Wt
     }
 }
 
+// grid.z: M-tiles of 32 rows, a8Stride / outStride bytes apart in the activations read and written.
 extern "C" __global__ __launch_bounds__(256) void rd_k_gemm8_q4k_gateup(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ A8,
-                                                                         uint8_t *__restrict__ XpOut, int outKind, int I, int nKB, int M) {
+                                                                         uint8_t *__restrict__ XpOut, int outKind, int I, int nKB, int M, size_t a8Stride,
+                                                                         size_t outStride) {
     __shared__ float lds[2 * 1024];
+    A8 += (size_t)blockIdx.z * a8Stride, XpOut += (size_t)blockIdx.z * outStride, M = min(32, M - 32 * (int)blockIdx.z);
     if (M <= 8)
         gemm8_gateup_body<Q4K8Traits, 2, 4>(Wt, A8, XpOut, outKind, I, nKB, M, lds);
     else if (M <= 16)
@@ -441,7 +450,7 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_gemm8_q4k_gateup(const ui
 // The plain kernel with one split and, instead of the store of the sums, what rd_k_qkv_rope_store does to them (same arithmetic,
 // same bits): the weight's rows are ordered so that a rotation pair sits in one tile, sixteen lanes apart (qkv_col), the angles'
 // cos and sin come from the step's table, q goes to the f32 buffer and k, v to the row's position in the f16 pool. For models
-// without QK-norm on the f16 cache. row0: first row of this M-tile among the step's rows. Grid (N/32), block KW waves.
+// without QK-norm on the f16 cache. Grid (N/32, 1, M-tiles of 32 rows), block KW waves; M: the step's rows.
 struct QkvEpilogue {
     float *q;
     uint16_t *Kp, *Vp;
@@ -516,8 +525,10 @@ __device__ __forceinline__ void gemm8_qkv_body(const uint8_t *__restrict__ Wt, c
     extern "C" __global__ __launch_bounds__(64 * KW) void NAME(                                                                                        \
         const uint8_t *__restrict__ Wt, const void *__restrict__ aux, const uint8_t *__restrict__ A8, int N, int nKB, int M, float *__restrict__ q,     \
         uint16_t *__restrict__ Kp, uint16_t *__restrict__ Vp, const int *__restrict__ tables, int tabStride, const int *__restrict__ rowSlot,           \
-        const int *__restrict__ rowPos, const double *__restrict__ cs, const float *__restrict__ bias, int nH, int nKV, int HD, int row0) {             \
+        const int *__restrict__ rowPos, const double *__restrict__ cs, const float *__restrict__ bias, int nH, int nKV, int HD, size_t a8Stride) {      \
         __shared__ float lds[KW > 2 ? (KW - 1) * 1024 : 32 * 33];                                                                                      \
+        const int row0 = 32 * (int)blockIdx.z; /* M-tile z: rows row0.. of the step, activations a8Stride bytes further on */                          \
+        A8 += (size_t)blockIdx.z * a8Stride, M = min(32, M - row0);                                                                                    \
         QkvEpilogue e{q, Kp, Vp, tables, rowSlot, rowPos, (const double2 *)cs, bias, tabStride, nH, nKV, HD, row0};                                    \
         if (M <= 8)                                                                                                                                    \
             gemm8_qkv_body<TRAITS, KW, 4>(Wt, aux, A8, N, nKB, M, e, lds);                                                                             \
