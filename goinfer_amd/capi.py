@@ -10,7 +10,7 @@ HSACO_PATH = os.path.join(HERE, "lib", "rocmdecode_gfx950.hsaco")
 
 RD_OK, RD_DECLINED = 0, 1
 PROJ = dict(q=0, k=1, v=2, o=3, gate=4, up=5, down=6, head=7)
-VEC = dict(attn_norm=0, ffn_norm=1, q_norm=2, k_norm=3, final_norm=4, router=5, qkv_bias=6)
+VEC = dict(attn_norm=0, ffn_norm=1, q_norm=2, k_norm=3, final_norm=4, router=5, qkv_bias=6, router_bias=7, attn_sinks=8)
 WANT_LOGITS, WANT_ARGMAX = 1, 2
 
 EXPORTS = [
@@ -19,7 +19,7 @@ EXPORTS = [
     "rd_attn_ragged", "rd_moe_route", "rd_rmsnorm", "rd_rope", "rd_model_create", "rd_model_destroy",
     "rd_model_upload_q4k", "rd_model_upload_w8a8", "rd_model_upload_w4a8", "rd_model_upload_f32", "rd_model_finalize",
     "rd_kv_configure", "rd_kv_upload", "rd_kv_truncate", "rd_kv_reset", "rd_step_batch", "rd_forward",
-    "rd_last_moe_indices", "rd_model_upload_embedding", "rd_bench_steps", "rd_bench_profile", "rd_bench_attn_chain", "rd_bench_prefill", "rd_bench_class_count",
+    "rd_last_moe_indices", "rd_model_upload_embedding", "rd_bench_steps", "rd_bench_profile", "rd_bench_attn_chain", "rd_moe_route_ex", "rd_attn_ragged_ex", "rd_model_set_router", "rd_model_set_window", "rd_bench_prefill", "rd_bench_class_count",
     "rd_bench_class_name", "rd_bench_kernel", "rd_gateup_q4k_quant", "rd_moe_replay", "rd_bench_attn", "rd_step_ragged", "rd_prefill_last",
     "rd_kv_configure_typed", "rd_attn_ragged_i8", "rd_attn_ragged_rows", "rd_plan_attention", "rd_plan_gemm", "rd_step_batch_topk", "rd_last_logits", "rd_topk_rows", "rd_bench_attn_i8", "rd_step_ragged_draw", "rd_forward_no_logits",
     "rd_step_batch_draw", "rd_sample_rows", "rd_greedy_chain_start", "rd_greedy_chain_next", "rd_sample_chain_start",
@@ -244,6 +244,20 @@ class Device:
                                         hd, C.c_float(scale), C.c_float(softcap), _p(out)), "rd_attn_ragged_rows")
         return out
 
+    def attn_ragged_ex(self, lens, k, v, q, n_h, n_kv, hd, scale, softcap=0.0, kv="f16", nq=None, window=0, sinks=None):
+        """rd_attn_ragged_rows (nq=None: one query row per sequence) with a sliding window and attention sinks."""
+        lens = np.ascontiguousarray(lens, dtype=np.int32)
+        off = np.zeros(len(lens), np.int64)
+        off[1:] = np.cumsum(lens[:-1])
+        k, v, q = _f32(k), _f32(v), _f32(q)
+        rows = len(lens) if nq is None else int(np.sum(nq))
+        nq_a = None if nq is None else np.ascontiguousarray(nq, dtype=np.int32)
+        sk = None if sinks is None else _f32(sinks)
+        out = np.empty((rows, n_h * hd), np.float32)
+        check(lib().rd_attn_ragged_ex(self.h, 0 if kv == "f16" else 1, len(lens), _p(lens), _p(nq_a), _p(off), _p(k), _p(v), _p(q), n_h, n_kv, hd,
+                                      C.c_float(scale), C.c_float(softcap), int(window), _p(sk), _p(out)), "rd_attn_ragged_ex")
+        return out
+
     def qkv_rope_store(self, x, pos, n_h, n_kv, hd, inv_freq, q_norm=None, k_norm=None, eps=1e-6, bias=None, kv="f16"):
         """The step's q|k|v epilogue on rows x [rows][(n_h+2n_kv)*hd]: (q, k as stored, v as stored)."""
         x = _f32(x)
@@ -270,12 +284,14 @@ class Device:
         check(lib().rd_quant_act(self.h, _p(a), M, K, _p(codes), _p(scales), _p(sums)), "rd_quant_act")
         return codes, scales, sums
 
-    def moe_route(self, logits, k, norm):
+    def moe_route(self, logits, k, norm, bias=None, sigmoid=False, scale=0.0, n_group=0, topk_group=0):
         logits = _f32(logits)
         T, nE = logits.shape
-        idx = np.empty((T, k), np.int32)
-        wgt = np.empty((T, k), np.float32)
-        check(lib().rd_moe_route(self.h, _p(logits), T, nE, k, int(norm), _p(idx), _p(wgt)), "rd_moe_route")
+        idx = np.full((T, k), -1, np.int32)
+        wgt = np.zeros((T, k), np.float32)
+        bs = None if bias is None else _f32(bias)
+        check(lib().rd_moe_route_ex(self.h, _p(logits), _p(bs), T, nE, k, int(sigmoid), int(norm), C.c_double(scale), int(n_group), int(topk_group),
+                                    _p(idx), _p(wgt)), "rd_moe_route_ex")
         return idx, wgt
 
     def rmsnorm(self, x, w, eps):
@@ -318,6 +334,12 @@ class Model:
                       _p(self._inv))
         self.h = C.c_void_p()
         check(lib().rd_model_create(dev.h, C.byref(d), C.byref(self.h)), "rd_model_create")
+        if cfg.get("router_sigmoid") or cfg.get("router_scale") or cfg.get("n_group"):  # the router's variant (mlp.go:130-228)
+            check(lib().rd_model_set_router(self.h, int(cfg.get("router_sigmoid", 0)), C.c_double(cfg.get("router_scale", 0.0)),
+                                            int(cfg.get("n_group", 0)), int(cfg.get("topk_group", 0))), "rd_model_set_router")
+
+    def set_window(self, layer, window):
+        check(lib().rd_model_set_window(self.h, layer, int(window)), "rd_model_set_window")
 
     def close(self):
         if self.h:

@@ -84,7 +84,7 @@ extern "C" int rd_bench_attn_chain(rd_model *m, int B, const int *slot, const in
     (void)d->hip->EventRecord(a, d->stream);
     for (int r = 0; r < reps && !rc; r++)
         for (auto &l : m->layers)
-            if ((rc = launch_attn_partial(m, l, m->last_items, m->last_grouped))) break;
+            if ((rc = launch_attn_partial(m, l))) break;
     (void)d->hip->EventRecord(b2, d->stream);
     int rc2 = d->sync();
     float ms = 0.f;
@@ -448,15 +448,15 @@ static int bench_attn_typed(rd_device *d, int kv_type, int n_seq, const int *len
             if (i8)
                 rc = d->launch(d->k.attn_partial_i8, (unsigned)g.nItems, 1, 1, 64, (const void *)g.I.p, (const int *)g.L.p, (const int *)g.S.p, (const int *)T.p,
                                maxBlocks, (const signed char *)Kp.p, (const signed char *)Vp.p, (const float *)Ksc.p, (const float *)Vsc.p,
-                               (const float *)((const float *)Q.p + (size_t)g.r0 * qd), g.P.as<float>(), n_h, n_kv, hd, scale, softcap);
+                               (const float *)((const float *)Q.p + (size_t)g.r0 * qd), g.P.as<float>(), n_h, n_kv, hd, scale, softcap, 0);
             else
                 rc = d->launch(d->k.attn_partial, (unsigned)g.nItems, 1, 1, 64, (const void *)g.I.p, (const int *)g.L.p, (const int *)g.S.p, (const int *)T.p, maxBlocks,
                                (const uint16_t *)Kp.p, (const uint16_t *)Vp.p, (const float *)((const float *)Q.p + (size_t)g.r0 * qd), g.P.as<float>(), n_h, n_kv, hd,
-                               scale, softcap);
+                               scale, softcap, 0);
             if (timed) (void)d->hip->EventRecord(evp[(t * nG + gi) * 2 + 1], d->stream);
             if (!rc)
                 rc = d->launch(d->k.attn_combine, (unsigned)n_h, (unsigned)g.rows, 1, (unsigned)(ATTN_PIECES * hd / 4), (const float *)g.P.p, (const int *)g.St.p, G,
-                               (float *)((float *)O.p + (size_t)g.r0 * qd), n_h, n_kv, hd);
+                               (float *)((float *)O.p + (size_t)g.r0 * qd), n_h, n_kv, hd, (const float *)nullptr);
         }
         if (timed) (void)d->hip->EventRecord(ev[2 * t + 1], d->stream);
     }

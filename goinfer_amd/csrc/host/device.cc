@@ -251,7 +251,9 @@ hipFunction_t attn_partial_kernel(const rd_device *d, bool i8, bool grouped, siz
     return i8 ? d->k.attn_partial_i8 : d->k.attn_partial;
 }
 
-bool build_attn_worklist(const int *len, const int *slot, int G, int rows, int n_kv, std::vector<AttnItemH> &items, std::vector<int> &ranges) {
+bool build_attn_worklist(const int *len, const int *slot, int G, int rows, int n_kv, std::vector<AttnItemH> &items, std::vector<int> &ranges,
+                         int window) {
+    auto first_block = [&](int r) { return window > 0 ? std::max(len[r] - window, 0) / 64 : 0; };
     static const bool no_groups = getenv("ROCMDECODE_NO_ATTN_GROUPS") != nullptr;
     const int maxGroup = (slot && !no_groups && G <= ATTN_TILE_ROWS) ? ATTN_TILE_ROWS / G : 1;
     struct Group {
@@ -260,7 +262,9 @@ bool build_attn_worklist(const int *len, const int *slot, int G, int rows, int n
     std::vector<Group> groups;
     for (int r = 0; r < rows;) {
         int n = 1;
-        while (n < maxGroup && r + n < rows && slot[r + n] == slot[r] && len[r + n] == len[r] + n && (len[r + n] + 63) / 64 == (len[r] + 63) / 64) n++;
+        while (n < maxGroup && r + n < rows && slot[r + n] == slot[r] && len[r + n] == len[r] + n && (len[r + n] + 63) / 64 == (len[r] + 63) / 64 &&
+               first_block(r + n) == first_block(r))
+            n++;
         groups.push_back({r, n});
         r += n;
     }
@@ -269,11 +273,11 @@ bool build_attn_worklist(const int *len, const int *slot, int G, int rows, int n
     ranges.assign((size_t)rows * n_kv * ATTN_RANGE_INTS, 0);
     bool grouped = false;
     for (const Group &g : groups) {
-        const int nb = (len[g.row] + 63) / 64, chunk = attn_chunk_blocks(nb);
+        const int nb = (len[g.row] + 63) / 64, fb = first_block(g.row), chunk = attn_chunk_blocks(nb - fb);
         grouped = grouped || g.n > 1;
         for (int h = 0; h < n_kv; h++) {
             const int first = (int)items.size();
-            for (int b0 = 0; b0 < nb; b0 += chunk) items.push_back({g.row, h | (g.n << 16), b0, std::min(nb, b0 + chunk)});
+            for (int b0 = fb; b0 < nb; b0 += chunk) items.push_back({g.row, h | (g.n << 16), b0, std::min(nb, b0 + chunk)});
             for (int j = 0; j < g.n; j++) {
                 int *rg = &ranges[((size_t)(g.row + j) * n_kv + h) * ATTN_RANGE_INTS];
                 rg[0] = first, rg[1] = (int)items.size(), rg[2] = j;

@@ -133,7 +133,10 @@ constexpr int ATTN_TILE_ROWS = 16; // head rows of the attention MFMA tile: an i
 // slot == nullptr: one position per item. Otherwise consecutive rows of one slot whose lengths ascend by one and need the same
 // number of blocks (so their cuts coincide) share items, up to 16/G of them; returns true if any item holds more than one
 // position, in which case the step runs the kernels that read the high bits of kvh and write 16 head rows per item.
-bool build_attn_worklist(const int *len, const int *slot, int G, int rows, int n_kv, std::vector<AttnItemH> &items, std::vector<int> &ranges);
+// window > 0: a sliding-window layer's list: a row's items cover only the blocks from position len-window on, and rows share
+// items only when those first blocks coincide as well.
+bool build_attn_worklist(const int *len, const int *slot, int G, int rows, int n_kv, std::vector<AttnItemH> &items, std::vector<int> &ranges,
+                         int window = 0);
 
 // split-K plan of one GEMM launch
 struct GemmPlan {

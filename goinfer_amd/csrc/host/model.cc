@@ -59,7 +59,7 @@ extern "C" void rd_model_destroy(rd_model *m) {
     (void)d->sync();
     for (auto &l : m->layers) {
         free_weight(d, &l.qkv), free_weight(d, &l.o), free_weight(d, &l.gateup), free_weight(d, &l.down);
-        for (void *p : {(void *)l.attn_norm, (void *)l.ffn_norm, (void *)l.q_norm, (void *)l.k_norm, (void *)l.qkv_bias, (void *)l.router, l.exp_gateup, l.exp_down,
+        for (void *p : {(void *)l.attn_norm, (void *)l.ffn_norm, (void *)l.q_norm, (void *)l.k_norm, (void *)l.qkv_bias, (void *)l.router, (void *)l.router_bias, (void *)l.sinks, l.exp_gateup, l.exp_down,
                         (void *)l.Kp, (void *)l.Vp, (void *)l.Ksc, (void *)l.Vsc})
             d->release(p);
     }
@@ -325,6 +325,8 @@ extern "C" int rd_model_upload_f32(rd_model *m, int layer, int which, const floa
         case RD_VEC_K_NORM: slot = &l.k_norm, want = (size_t)c.head_dim; break;
         case RD_VEC_QKV_BIAS: slot = &l.qkv_bias, want = (size_t)(c.n_heads + 2 * c.n_kv_heads) * c.head_dim; break;
         case RD_VEC_ROUTER: slot = &l.router, want = (size_t)c.n_experts * c.hidden; break;
+        case RD_VEC_ROUTER_BIAS: slot = &l.router_bias, want = (size_t)c.n_experts; break;
+        case RD_VEC_ATTN_SINKS: slot = &l.sinks, want = (size_t)c.n_heads; break;
         default: rd_set_error("unknown vector %d", which); return RD_ERR_ARG;
         }
     }
@@ -335,6 +337,38 @@ extern "C" int rd_model_upload_f32(rd_model *m, int layer, int which, const floa
     if (!*slot) RC(alloc_f32(d, slot, n));
     RC(d->h2d(*slot, v, sizeof(float) * n));
     return d->sync();
+}
+
+// The router's variant (decoder/mlp.go:130-228 routeExperts / groupLimit), before rd_model_finalize.
+extern "C" int rd_model_set_router(rd_model *m, int sigmoid, double scale, int n_group, int topk_group) {
+    if (!m) return RD_ERR_ARG;
+    if (m->finalized) {
+        rd_set_error("model already finalized");
+        return RD_ERR_STATE;
+    }
+    if (n_group > 32 || (n_group > 1 && (topk_group < 1 || topk_group > n_group || m->desc.n_experts % n_group))) {
+        rd_set_error("rocm resident declines: group-limited routing takes 2..32 groups that divide the experts, and 1..n_group of them");
+        return RD_DECLINED;
+    }
+    m->router_sigmoid = sigmoid ? 1 : 0, m->router_scale = (float)scale, m->n_group = n_group > 1 ? n_group : 0, m->topk_group = topk_group;
+    return RD_OK;
+}
+
+// A sliding-window layer (kvmgr.WindowNeedStart, internal/runtime/kvmgr/sequence.go:55-60): the layer's rows read the last
+// `window` positions only. Before rd_model_finalize; the windowed layers of a model share one window length.
+extern "C" int rd_model_set_window(rd_model *m, int layer, int window) {
+    if (!m || !layer_ok(m, layer, false) || window < 0) return RD_ERR_ARG;
+    if (m->finalized) {
+        rd_set_error("model already finalized");
+        return RD_ERR_STATE;
+    }
+    if (window > 0 && m->window > 0 && window != m->window) {
+        rd_set_error("rocm resident declines: sliding-window layers of different lengths (%d and %d)", m->window, window);
+        return RD_DECLINED;
+    }
+    m->layers[(size_t)layer].window = window;
+    if (window > 0) m->window = window;
+    return RD_OK;
 }
 
 // The int8 embedding table, resident so a greedy chain can run without the host (goinfer's GreedyChain*,
@@ -498,7 +532,8 @@ extern "C" int rd_kv_configure_typed(rd_model *m, int slots, int ctx_cap, int kv
     // The step's metadata lives in one device block so a step uploads it with one copy:
     // [row slot R][row position R][row length R][row draw records R x 6][item ranges max_rows*nKV*3][items max_items x 4] ints, R = ROWS_MAX
     const size_t rangeInts = (size_t)m->max_rows * c.n_kv_heads * ATTN_RANGE_INTS;
-    m->meta_ints = rd_model::META_HDR + rangeInts + (size_t)m->max_items * 4;
+    m->list_ints = rangeInts + (size_t)m->max_items * 4;
+    m->meta_ints = rd_model::META_HDR + m->list_ints * (m->window > 0 ? 2 : 1); // a second work list for the sliding-window layers
     RC(d->alloc((void **)&m->meta, sizeof(int) * m->meta_ints));
     constexpr int RM = rd_model::ROWS_MAX;
     m->rowSlot = m->meta, m->rowPos = m->meta + RM, m->rowLen = m->meta + 2 * RM, m->rowDraw = m->meta + 3 * RM;
@@ -596,10 +631,11 @@ struct Scope { // times one kernel class when the model's timer is on
 };
 
 // *grouped: some item covers several positions of one sequence (the step then runs the attention kernels for such items).
-static int build_attn_items(rd_model *m, int B, const int *slot, const int *pos, std::vector<AttnItemH> &items, std::vector<int> &ranges, bool *grouped) {
+static int build_attn_items(rd_model *m, int B, const int *slot, const int *pos, std::vector<AttnItemH> &items, std::vector<int> &ranges, bool *grouped,
+                            int window) {
     int len[rd_model::ROWS_MAX];
     for (int b = 0; b < B; b++) len[b] = pos[b] + 1;
-    *grouped = build_attn_worklist(len, slot, m->desc.n_heads / m->desc.n_kv_heads, B, m->desc.n_kv_heads, items, ranges);
+    *grouped = build_attn_worklist(len, slot, m->desc.n_heads / m->desc.n_kv_heads, B, m->desc.n_kv_heads, items, ranges, window);
     if ((int)items.size() > m->max_items) {
         rd_set_error("attention work list overflow (%zu items)", items.size());
         return RD_ERR_STATE;
@@ -685,7 +721,7 @@ static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
             RC(d->launch(d->k.matmul_f32, (unsigned)((nE + 3) / 4), (unsigned)B, 1, 256, (const float *)m->normed, (const float *)l.router,
                          m->router_logits, B, H, nE, bits_dev));
             RC(d->launch(d->k.moe_route, (unsigned)B, 1, 1, 64, (const float *)m->router_logits, B, nE, k, c.norm_topk_prob, m->moe_idx, m->moe_wgt,
-                         m->moe_rank, trace, bits_dev));
+                         m->moe_rank, trace, bits_dev, (const float *)l.router_bias, m->router_sigmoid, m->router_scale, m->n_group, m->topk_group));
         }
     }
     const int nKBh = (H + 255) / 256, nKBi = (I + 255) / 256;
@@ -719,18 +755,22 @@ static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
     return RD_OK;
 }
 
-// The attention kernel of one layer over the step's work list (nItems items already on the device).
-int launch_attn_partial(rd_model *m, const LayerW &l, size_t nItems, bool grouped) {
+// The attention kernel of one layer over the step's work list for it (already on the device): the whole-context list, or the
+// sliding-window list for a layer with a window.
+int launch_attn_partial(rd_model *m, const LayerW &l) {
     rd_device *d = m->d;
     const rd_model_desc &c = m->desc;
-    const int nH = c.n_heads, nKV = c.n_kv_heads, HD = c.head_dim;
+    const int nH = c.n_heads, nKV = c.n_kv_heads, HD = c.head_dim, li = l.window > 0 ? 1 : 0;
+    const size_t nItems = m->last_items[li];
+    const bool grouped = m->last_grouped[li];
+    const void *items = (const int *)m->items + (size_t)li * m->list_ints;
     if (m->kv_type == RD_KV_I8)
-        return d->launch(attn_partial_kernel(d, true, grouped, nItems), (unsigned)nItems, 1, 1, 64, (const void *)m->items, (const int *)m->rowLen, (const int *)m->rowSlot,
+        return d->launch(attn_partial_kernel(d, true, grouped, nItems), (unsigned)nItems, 1, 1, 64, items, (const int *)m->rowLen, (const int *)m->rowSlot,
                          (const int *)m->tables, m->blocks_per_slot, (const signed char *)l.Kp, (const signed char *)l.Vp, (const float *)l.Ksc,
-                         (const float *)l.Vsc, (const float *)m->qbuf, m->part, nH, nKV, HD, c.attn_scale, c.attn_softcap);
-    return d->launch(attn_partial_kernel(d, false, grouped, nItems), (unsigned)nItems, 1, 1, 64, (const void *)m->items, (const int *)m->rowLen, (const int *)m->rowSlot,
+                         (const float *)l.Vsc, (const float *)m->qbuf, m->part, nH, nKV, HD, c.attn_scale, c.attn_softcap, l.window);
+    return d->launch(attn_partial_kernel(d, false, grouped, nItems), (unsigned)nItems, 1, 1, 64, items, (const int *)m->rowLen, (const int *)m->rowSlot,
                      (const int *)m->tables, m->blocks_per_slot, (const uint16_t *)l.Kp, (const uint16_t *)l.Vp, (const float *)m->qbuf, m->part,
-                     nH, nKV, HD, c.attn_scale, c.attn_softcap);
+                     nH, nKV, HD, c.attn_scale, c.attn_softcap, l.window);
 }
 
 // emb_host: [B][hidden] on the host, or emb_dev already on the device (benchmark loop). Logits/ids are host pointers.
@@ -774,12 +814,14 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
         }
     }
     int H = c.hidden, nH = c.n_heads, nKV = c.n_kv_heads, HD = c.head_dim;
-    std::vector<AttnItemH> items;
-    std::vector<int> start;
-    bool grouped = false;
-    RC(build_attn_items(m, B, slot, pos, items, start, &grouped));
-    const int partRows = grouped ? ATTN_TILE_ROWS : nH / nKV;
-    m->last_items = items.size(), m->last_grouped = grouped;
+    const int nLists = m->window > 0 ? 2 : 1;
+    std::vector<AttnItemH> items[2];
+    std::vector<int> start[2];
+    for (int li = 0; li < nLists; li++) {
+        bool grouped = false;
+        RC(build_attn_items(m, B, slot, pos, items[li], start[li], &grouped, li ? m->window : 0));
+        m->last_items[li] = items[li].size(), m->last_grouped[li] = grouped;
+    }
     // Stage the step's metadata (and host embeddings) in pinned memory and upload it asynchronously. A slot is reused only
     // once the upload it last fed has completed, which its event tells.
     const unsigned stage_slot = m->stage_next++ % rd_model::STAGE_SLOTS;
@@ -813,9 +855,12 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
         }
         constexpr int HDR = rd_model::META_HDR;
         memset(hm + HDR - 8, 0, sizeof(int) * 8);
-        memcpy(hm + HDR, start.data(), sizeof(int) * start.size());
-        memcpy(hm + HDR + rangeInts, items.data(), sizeof(AttnItemH) * items.size());
-        RC(d->h2d(m->meta, hm, sizeof(int) * (HDR + rangeInts + items.size() * 4)));
+        for (int li = 0; li < nLists; li++) {
+            int *lst = hm + HDR + (size_t)li * m->list_ints;
+            memcpy(lst, start[li].data(), sizeof(int) * start[li].size());
+            memcpy(lst + rangeInts, items[li].data(), sizeof(AttnItemH) * items[li].size());
+        }
+        RC(d->h2d(m->meta, hm, sizeof(int) * (HDR + (size_t)(nLists - 1) * m->list_ints + rangeInts + items[nLists - 1].size() * 4)));
         if (emb_host) {
             memcpy(eh, emb_host, sizeof(float) * (size_t)B * H);
             RC(d->h2d(m->h, eh, sizeof(float) * (size_t)B * H));
@@ -873,12 +918,14 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
         }
         {
             Scope s(m, KC_ATTN_PARTIAL);
-            RC(launch_attn_partial(m, l, items.size(), grouped));
+            RC(launch_attn_partial(m, l));
         }
         {
             Scope s(m, KC_ATTN_COMBINE);
-            RC(d->launch(d->k.attn_combine_quant, (unsigned)nH, (unsigned)B, 1, (unsigned)(ATTN_PIECES * HD / 4), (const float *)m->part, (const int *)m->itemStart,
-                         partRows, m->XpB, panel_kind_for(l.o), nH, nKV, HD, m->xpBStride));
+            const int li = l.window > 0 ? 1 : 0;
+            RC(d->launch(d->k.attn_combine_quant, (unsigned)nH, (unsigned)B, 1, (unsigned)(ATTN_PIECES * HD / 4), (const float *)m->part,
+                         (const int *)m->itemStart + (size_t)li * m->list_ints, m->last_grouped[li] ? ATTN_TILE_ROWS : nH / nKV, m->XpB, panel_kind_for(l.o), nH, nKV,
+                         HD, m->xpBStride, (const float *)l.sinks));
         }
         {
             Scope s(m, KC_GEMM_O);

@@ -21,6 +21,9 @@ struct LayerW {
     PendingMat pend[RD_PROJ_COUNT];
     float *attn_norm = nullptr, *ffn_norm = nullptr, *q_norm = nullptr, *k_norm = nullptr;
     float *qkv_bias = nullptr; // optional: q bias, k bias, v bias end to end
+    float *router_bias = nullptr; // optional [nE]: e_score_correction_bias (selection only)
+    float *sinks = nullptr;       // optional [nH]: attention sinks
+    int window = 0;               // > 0: sliding-window layer
     // MoE
     float *router = nullptr;           // [nE][hidden] f32
     void *exp_gateup = nullptr;        // [nE] stacked tiled W4A8, each 2*expert_inter rows x hidden
@@ -49,6 +52,10 @@ struct rd_model {
     signed char *embed_q = nullptr; // optional device copy of the int8 embedding table (device-side greedy chain)
     float *embed_scale = nullptr;
     bool finalized = false;
+    // router variant (decoder/mlp.go:130-228): sigmoid scoring, routed scaling factor, group-limited selection
+    int router_sigmoid = 0, n_group = 0, topk_group = 0;
+    float router_scale = 0.f;
+    int window = 0; // the one window length the model's sliding-window layers share (0: none has one)
 
     // KV
     int slots = 0, ctx_cap = 0, blocks_per_slot = 0;
@@ -117,10 +124,13 @@ struct rd_model {
     std::vector<std::vector<signed char>> replay_rank;
 
     StepTimer timer;
-    size_t last_items = 0; // the last step's attention work list, still on the device (rd_bench_attn_chain replays it)
-    bool last_grouped = false;
+    // The step's attention work lists: [0] for the layers that read the whole context, [1] for the sliding-window layers (if any).
+    // list_ints: ints between the two lists' (ranges, items) blocks in the metadata. The last step's lists stay on the device
+    // (rd_bench_attn_chain replays them).
+    size_t list_ints = 0, last_items[2] = {0, 0};
+    bool last_grouped[2] = {false, false};
 };
-int launch_attn_partial(rd_model *m, const LayerW &l, size_t nItems, bool grouped);
+int launch_attn_partial(rd_model *m, const LayerW &l);
 
 // multirow: a slot may carry several rows at consecutive positions (ragged verify / prefill rows)
 int model_step(rd_model *m, int B, const int *slot, const int *pos, const float *emb_host, const float *emb_dev, int want, float *logits,

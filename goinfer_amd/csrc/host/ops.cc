@@ -314,20 +314,33 @@ extern "C" int rd_rope(rd_device *d, float *vec, int rows, int heads, int head_d
     return d->d2h(vec, V.p, sizeof(float) * n);
 }
 
-extern "C" int rd_moe_route(rd_device *d, const float *logits, int T, int nE, int k, int norm, int *idx, float *wgt) {
+extern "C" int rd_moe_route_ex(rd_device *d, const float *logits, const float *bias, int T, int nE, int k, int sigmoid, int norm, double scale,
+                               int n_group, int topk_group, int *idx, float *wgt) {
     if (!d || !logits || !idx || !wgt || T <= 0 || nE <= 0 || nE > 256 || k <= 0 || k > nE) {
         rd_set_error("rd_moe_route: bad arguments (nE <= 256)");
         return RD_ERR_ARG;
     }
-    DevBuf L(d), I(d), W(d);
+    if (n_group > 32 || (n_group > 1 && (topk_group < 1 || topk_group > n_group))) {
+        rd_set_error("rd_moe_route: group-limited routing takes 2..32 groups and 1..n_group of them");
+        return RD_ERR_ARG;
+    }
+    DevBuf L(d), I(d), W(d), Bi(d);
     RC(L.alloc(sizeof(float) * (size_t)T * nE));
     RC(I.alloc(sizeof(int) * (size_t)T * k));
     RC(W.alloc(sizeof(float) * (size_t)T * k));
     RC(d->h2d(L.p, logits, sizeof(float) * (size_t)T * nE));
+    RC(d->launch(d->k.fill_f32, 1, 1, 1, 64, I.as<float>(), (size_t)T * k, 0u)); // a row with fewer than k eligible experts leaves the rest as it finds it
+    if (bias) {
+        RC(Bi.alloc(sizeof(float) * (size_t)nE));
+        RC(d->h2d(Bi.p, bias, sizeof(float) * (size_t)nE));
+    }
     RC(d->launch(d->k.moe_route, (unsigned)T, 1, 1, 64, (const float *)L.p, T, nE, k, norm, I.as<int>(), W.as<float>(),
-                 (signed char *)nullptr, (int *)nullptr, (unsigned *)nullptr));
+                 (signed char *)nullptr, (int *)nullptr, (unsigned *)nullptr, (const float *)Bi.p, sigmoid, (float)scale, n_group, topk_group));
     RC(d->d2h(idx, I.p, sizeof(int) * (size_t)T * k));
     return d->d2h(wgt, W.p, sizeof(float) * (size_t)T * k);
+}
+extern "C" int rd_moe_route(rd_device *d, const float *logits, int T, int nE, int k, int norm, int *idx, float *wgt) {
+    return rd_moe_route_ex(d, logits, nullptr, T, nE, k, 0, norm, 0.0, 0, 0, idx, wgt);
 }
 
 // ---- the step's q|k|v epilogue on its own: bias, QK-norm, RoPE, and the K/V rows as the cache then holds them ----
@@ -411,7 +424,7 @@ extern "C" int rd_qkv_rope_store(rd_device *d, int kv_type, int rows, const floa
 // ---- ragged attention over a temporary paged pool (kernel-level entry point) ----
 // nq (optional): sequence i brings nq[i] query rows, its last nq[i] positions; row j of them sees keys 0..len[i]-nq[i]+j.
 static int attn_ragged_typed(rd_device *d, int kv_type, int n_seq, const int *len, const int *nq, const int64_t *off, const float *k, const float *v,
-                             const float *q, int n_h, int n_kv, int hd, float scale, float softcap, float *out) {
+                             const float *q, int n_h, int n_kv, int hd, float scale, float softcap, float *out, int window = 0, const float *sinks = nullptr) {
     if (!d || !len || !off || !k || !v || !q || !out || n_seq <= 0) return RD_ERR_ARG;
     if (n_kv <= 0 || n_h % n_kv || n_h / n_kv > 16 || (hd != 64 && hd != 128)) {
         rd_set_error("rd_attn_ragged declines: head_dim must be 64 or 128 and the GQA group <= 16");
@@ -484,9 +497,13 @@ static int attn_ragged_typed(rd_device *d, int kv_type, int n_seq, const int *le
         int rows = std::min(32, n_rows - r0);
         std::vector<AttnItemH> items;
         std::vector<int> start, slots(rowSeq.begin() + r0, rowSeq.begin() + r0 + rows), lens(rowLens.begin() + r0, rowLens.begin() + r0 + rows);
-        const bool grouped = build_attn_worklist(lens.data(), nq ? slots.data() : nullptr, G, rows, n_kv, items, start);
+        const bool grouped = build_attn_worklist(lens.data(), nq ? slots.data() : nullptr, G, rows, n_kv, items, start, window);
         const int partRows = grouped ? ATTN_TILE_ROWS : G;
-        DevBuf Q2(d), O2(d), L2(d), S2(d), I2(d), St2(d), P2(d);
+        DevBuf Q2(d), O2(d), L2(d), S2(d), I2(d), St2(d), P2(d), Sk(d);
+        if (sinks) {
+            RC(Sk.alloc(sizeof(float) * (size_t)n_h));
+            RC(d->h2d(Sk.p, sinks, sizeof(float) * (size_t)n_h));
+        }
         RC(Q2.alloc(sizeof(float) * (size_t)rows * qd));
         RC(O2.alloc(sizeof(float) * (size_t)rows * qd));
         RC(L2.alloc(sizeof(int) * (size_t)rows));
@@ -502,13 +519,13 @@ static int attn_ragged_typed(rd_device *d, int kv_type, int n_seq, const int *le
         if (i8)
             RC(d->launch(attn_partial_kernel(d, true, grouped, items.size()), (unsigned)items.size(), 1, 1, 64, (const void *)I2.p, (const int *)L2.p,
                          (const int *)S2.p, (const int *)T.p, maxBlocks, (const signed char *)Kp.p, (const signed char *)Vp.p, (const float *)Ksc.p,
-                         (const float *)Vsc.p, (const float *)Q2.p, P2.as<float>(), n_h, n_kv, hd, scale, softcap));
+                         (const float *)Vsc.p, (const float *)Q2.p, P2.as<float>(), n_h, n_kv, hd, scale, softcap, window));
         else
             RC(d->launch(attn_partial_kernel(d, false, grouped, items.size()), (unsigned)items.size(), 1, 1, 64, (const void *)I2.p, (const int *)L2.p,
                          (const int *)S2.p, (const int *)T.p, maxBlocks, (const uint16_t *)Kp.p, (const uint16_t *)Vp.p, (const float *)Q2.p, P2.as<float>(), n_h,
-                         n_kv, hd, scale, softcap));
+                         n_kv, hd, scale, softcap, window));
         RC(d->launch(d->k.attn_combine, (unsigned)n_h, (unsigned)rows, 1, (unsigned)(ATTN_PIECES * hd / 4), (const float *)P2.p, (const int *)St2.p, partRows,
-                     O2.as<float>(), n_h, n_kv, hd));
+                     O2.as<float>(), n_h, n_kv, hd, (const float *)Sk.p));
         RC(d->d2h(out + (size_t)r0 * qd, O2.p, sizeof(float) * (size_t)rows * qd));
     }
     return RD_OK;
@@ -525,6 +542,14 @@ extern "C" int rd_attn_ragged_rows(rd_device *d, int kv_type, int n_seq, const i
                                    const float *q, int n_h, int n_kv, int hd, float scale, float softcap, float *out) {
     if (!nq || (kv_type != RD_KV_F16 && kv_type != RD_KV_I8)) return RD_ERR_ARG;
     return attn_ragged_typed(d, kv_type, n_seq, len, nq, off, k, v, q, n_h, n_kv, hd, scale, softcap, out);
+}
+
+// The same with a sliding window (each row reads the last `window` positions of its sequence only; 0 = the whole sequence) and
+// attention sinks (sinks: host f32 [n_h] or NULL). nq may be NULL (one query row per sequence, the last position).
+extern "C" int rd_attn_ragged_ex(rd_device *d, int kv_type, int n_seq, const int *len, const int *nq, const int64_t *off, const float *k, const float *v,
+                                 const float *q, int n_h, int n_kv, int hd, float scale, float softcap, int window, const float *sinks, float *out) {
+    if ((kv_type != RD_KV_F16 && kv_type != RD_KV_I8) || window < 0) return RD_ERR_ARG;
+    return attn_ragged_typed(d, kv_type, n_seq, len, nq, off, k, v, q, n_h, n_kv, hd, scale, softcap, out, window, sinks);
 }
 
 // ---- top-K of logits rows (kernel-level entry point) ----

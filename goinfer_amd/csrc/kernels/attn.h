@@ -301,7 +301,7 @@ __device__ __forceinline__ half8_t kv8_to_half8(uint32_t w0, uint32_t w1) {
                 float s = S[t][r] * scale;                                                                                                             \
                 if constexpr (I8) s = S[t][r] * KS[t] * scale;                                                                                         \
                 if (softcap != 0.f) s = softcap * fast_tanh(s * rcap);                                                                                 \
-                if ((KEY0) + t * 16 + l16 >= lenr[r]) s = -INFINITY;                                                                                   \
+                if ((KEY0) + t * 16 + l16 >= lenr[r] || (KEY0) + t * 16 + l16 < startr[r]) s = -INFINITY;                                           \
                 S[t][r] = s;                                                                                                                           \
                 mx[r] = fmaxf(mx[r], s);                                                                                                               \
             }                                                                                                                                          \
@@ -311,14 +311,15 @@ __device__ __forceinline__ half8_t kv8_to_half8(uint32_t w0, uint32_t w1) {
         _Pragma("unroll")                                                                                                                              \
         for (int r = 0; r < 4; r++) {                                                                                                                  \
             float mn = fmaxf(mrun[r], mx[r]);                                                                                                          \
-            alpha[r] = __expf(mrun[r] - mn);                                                                                                           \
+            const bool none = mn == -INFINITY; /* no key of this row yet (all before its window): nothing moves */                                     \
+            alpha[r] = none ? 1.f : __expf(mrun[r] - mn);                                                                                              \
             mrun[r] = mn;                                                                                                                              \
             float ps = 0.f;                                                                                                                            \
         _Pragma("unroll")                                                                                                                              \
             for (int t = 0; t < 2; t++) {                                                                                                              \
-                float p = __expf(S[t][r] - mn);                                                                                                        \
+                float p = none ? 0.f : __expf(S[t][r] - mn);                                                                                           \
                 ps += p;                                                                                                                               \
-                if constexpr (I8) p = ((KEY0) + t * 16 + l16 < lenr[r]) ? p * VS[t] : 0.f;                                                             \
+                if constexpr (I8) p = ((KEY0) + t * 16 + l16 < lenr[r] && (KEY0) + t * 16 + l16 >= startr[r]) ? p * VS[t] : 0.f;                       \
                 half_t hi = (half_t)p;                                                                                                                 \
                 int idx = (4 * lg + r) * 32 + t * 16 + l16;                                                                                            \
                 pbuf[idx] = hi;                                                                                                                        \
@@ -357,7 +358,7 @@ __device__ __forceinline__ void attn_partial_body(const AttnItem *__restrict__ i
                                                   const int *__restrict__ tables, int tabStride, const void *__restrict__ KpV,
                                                   const void *__restrict__ VpV, const float *__restrict__ Ksc, const float *__restrict__ Vsc,
                                                   const float *__restrict__ q, float *__restrict__ part, int nH, int nKV, float scale,
-                                                  float softcap, half_t *pbuf) {
+                                                  float softcap, int window, half_t *pbuf) {
     constexpr int NC = HD / 32, NCT = HD / 16;
     constexpr int KL = I8 ? NC / 2 : NC, VL = I8 ? NCT / 2 : NCT; // 16-byte loads per key tile of K, per 32 keys of V
     constexpr int ELEM = I8 ? 1 : 2;
@@ -370,9 +371,13 @@ __device__ __forceinline__ void attn_partial_body(const AttnItem *__restrict__ i
     const int *tab = tables + (size_t)rowSlot[it.row] * tabStride;
     // head row a of the tile = (position a / G, head a % G); this lane loads Q for row l16 and owns score rows 4*lg + r
     const int qj = ROWS ? l16 / G : 0, qg = ROWS ? l16 - qj * G : l16;
-    int lenr[4];
+    // window > 0 (a sliding-window layer; kvmgr.WindowNeedStart): a row at position p = len-1 reads keys p-window+1 .. p only
+    int lenr[4], startr[4];
 #pragma unroll
-    for (int r = 0; r < 4; r++) lenr[r] = ROWS ? len0 + min((4 * lg + r) / G, nrows - 1) : len;
+    for (int r = 0; r < 4; r++) {
+        lenr[r] = ROWS ? len0 + min((4 * lg + r) / G, nrows - 1) : len;
+        startr[r] = window > 0 ? max(lenr[r] - window, 0) : 0;
+    }
 
     // Q fragments (A operand): lane (head row l16, d quarter lg)
     half8_t qhi[NC], qlo[NC];
@@ -480,12 +485,12 @@ extern "C" __global__ __launch_bounds__(64) void rd_k_attn_partial(const AttnIte
                                                                    const int *__restrict__ rowSlot, const int *__restrict__ tables, int tabStride,
                                                                    const uint16_t *__restrict__ Kp, const uint16_t *__restrict__ Vp,
                                                                    const float *__restrict__ q, float *__restrict__ part, int nH, int nKV, int HD,
-                                                                   float scale, float softcap) {
+                                                                   float scale, float softcap, int window) {
     __shared__ half_t pbuf[1024];
     if (HD == 128)
-        attn_partial_body<128, false>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, pbuf);
+        attn_partial_body<128, false>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, window, pbuf);
     else
-        attn_partial_body<64, false>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, pbuf);
+        attn_partial_body<64, false>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, window, pbuf);
 }
 
 // The same over the int8 cache: half the key/value bytes per launch.
@@ -494,12 +499,12 @@ extern "C" __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3
                                                                       const signed char *__restrict__ Kp, const signed char *__restrict__ Vp,
                                                                       const float *__restrict__ Ksc, const float *__restrict__ Vsc,
                                                                       const float *__restrict__ q, float *__restrict__ part, int nH, int nKV, int HD,
-                                                                      float scale, float softcap) {
+                                                                      float scale, float softcap, int window) {
     __shared__ half_t pbuf[1024];
     if (HD == 128)
-        attn_partial_body<128, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, Ksc, Vsc, q, part, nH, nKV, scale, softcap, pbuf);
+        attn_partial_body<128, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, Ksc, Vsc, q, part, nH, nKV, scale, softcap, window, pbuf);
     else
-        attn_partial_body<64, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, Ksc, Vsc, q, part, nH, nKV, scale, softcap, pbuf);
+        attn_partial_body<64, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, Ksc, Vsc, q, part, nH, nKV, scale, softcap, window, pbuf);
 }
 
 // The same two kernels with two units in flight per wave (see DEEP above), one wave per SIMD.
@@ -507,12 +512,12 @@ extern "C" __global__ __launch_bounds__(64) void rd_k_attn_partial_deep(const At
                                                                         const int *__restrict__ rowSlot, const int *__restrict__ tables, int tabStride,
                                                                         const uint16_t *__restrict__ Kp, const uint16_t *__restrict__ Vp,
                                                                         const float *__restrict__ q, float *__restrict__ part, int nH, int nKV, int HD,
-                                                                        float scale, float softcap) {
+                                                                        float scale, float softcap, int window) {
     __shared__ half_t pbuf[1024];
     if (HD == 128)
-        attn_partial_body<128, false, false, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, pbuf);
+        attn_partial_body<128, false, false, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, window, pbuf);
     else
-        attn_partial_body<64, false, false, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, pbuf);
+        attn_partial_body<64, false, false, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, window, pbuf);
 }
 
 extern "C" __global__ __launch_bounds__(64) void rd_k_attn_partial_deep_i8(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
@@ -520,12 +525,12 @@ extern "C" __global__ __launch_bounds__(64) void rd_k_attn_partial_deep_i8(const
                                                                       const signed char *__restrict__ Kp, const signed char *__restrict__ Vp,
                                                                       const float *__restrict__ Ksc, const float *__restrict__ Vsc,
                                                                       const float *__restrict__ q, float *__restrict__ part, int nH, int nKV, int HD,
-                                                                      float scale, float softcap) {
+                                                                      float scale, float softcap, int window) {
     __shared__ half_t pbuf[1024];
     if (HD == 128)
-        attn_partial_body<128, true, false, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, Ksc, Vsc, q, part, nH, nKV, scale, softcap, pbuf);
+        attn_partial_body<128, true, false, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, Ksc, Vsc, q, part, nH, nKV, scale, softcap, window, pbuf);
     else
-        attn_partial_body<64, true, false, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, Ksc, Vsc, q, part, nH, nKV, scale, softcap, pbuf);
+        attn_partial_body<64, true, false, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, Ksc, Vsc, q, part, nH, nKV, scale, softcap, window, pbuf);
 }
 
 // Items of several positions each (see ROWS above): steps that carry more than one row of a sequence — prompt passes, verification.
@@ -533,12 +538,12 @@ extern "C" __global__ __launch_bounds__(64) void rd_k_attn_partial_rows(const At
                                                                         const int *__restrict__ rowSlot, const int *__restrict__ tables, int tabStride,
                                                                         const uint16_t *__restrict__ Kp, const uint16_t *__restrict__ Vp,
                                                                         const float *__restrict__ q, float *__restrict__ part, int nH, int nKV, int HD,
-                                                                        float scale, float softcap) {
+                                                                        float scale, float softcap, int window) {
     __shared__ half_t pbuf[1024];
     if (HD == 128)
-        attn_partial_body<128, false, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, pbuf);
+        attn_partial_body<128, false, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, window, pbuf);
     else
-        attn_partial_body<64, false, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, pbuf);
+        attn_partial_body<64, false, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, window, pbuf);
 }
 
 extern "C" __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void rd_k_attn_partial_rows_i8(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
@@ -546,12 +551,12 @@ extern "C" __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3
                                                                       const signed char *__restrict__ Kp, const signed char *__restrict__ Vp,
                                                                       const float *__restrict__ Ksc, const float *__restrict__ Vsc,
                                                                       const float *__restrict__ q, float *__restrict__ part, int nH, int nKV, int HD,
-                                                                      float scale, float softcap) {
+                                                                      float scale, float softcap, int window) {
     __shared__ half_t pbuf[1024];
     if (HD == 128)
-        attn_partial_body<128, true, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, Ksc, Vsc, q, part, nH, nKV, scale, softcap, pbuf);
+        attn_partial_body<128, true, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, Ksc, Vsc, q, part, nH, nKV, scale, softcap, window, pbuf);
     else
-        attn_partial_body<64, true, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, Ksc, Vsc, q, part, nH, nKV, scale, softcap, pbuf);
+        attn_partial_body<64, true, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, Ksc, Vsc, q, part, nH, nKV, scale, softcap, window, pbuf);
 }
 
 // Merge the partials of one (row, query head) in ascending item order (deterministic):
@@ -561,8 +566,10 @@ extern "C" __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3
 // dq) brings four values of item i into LDS, so every item's load is in flight at once; the first HD/4 threads then fold
 // the items in order. lds: RD_ATTN_PIECES*(HD+2) floats. Returns true in the threads that hold a result (four consecutive d).
 #define RD_ATTN_PIECES 16
+// sinks (may be NULL): one learned logit per query head that joins the softmax's maximum and denominator and nothing else
+// (decoder/attention.go:305-322 sinkMax / sinkSum).
 __device__ __forceinline__ bool attn_combine_block(const float *__restrict__ part, const int *__restrict__ itemStart, int partRows, int nH, int nKV,
-                                                   int HD, int m, int head, float *lds, float *out) {
+                                                   int HD, int m, int head, float *lds, float *out, const float *__restrict__ sinks = nullptr) {
     const int Q = HD >> 2, ti = threadIdx.x / Q, dq = threadIdx.x - ti * Q;
     const int G = nH / nKV, kvh = head / G, g = head % G;
     const int *rg = itemStart + (m * nKV + kvh) * 3;
@@ -581,6 +588,7 @@ __device__ __forceinline__ bool attn_combine_block(const float *__restrict__ par
         __syncthreads();
         M = -INFINITY;
         for (int w = 0; w < (int)(blockDim.x >> 6); w++) M = fmaxf(M, mm[w]);
+        if (sinks) M = fmaxf(M, sinks[head]);
         __syncthreads(); // mm is reused by the rounds
     }
     float num[4] = {0.f, 0.f, 0.f, 0.f}, den = 0.f;
@@ -595,8 +603,10 @@ __device__ __forceinline__ bool attn_combine_block(const float *__restrict__ par
         }
         __syncthreads();
         if (ti == 0) {
-            if (n <= RD_ATTN_PIECES)
+            if (n <= RD_ATTN_PIECES) {
                 for (int i = 0; i < nb; i++) M = fmaxf(M, mm[i]);
+                if (sinks) M = fmaxf(M, sinks[head]);
+            }
             for (int i = 0; i < nb; i++) {
                 const float *v = vals + i * HD + dq * 4;
                 const float w = __expf(mm[i] - M);
@@ -607,6 +617,7 @@ __device__ __forceinline__ bool attn_combine_block(const float *__restrict__ par
         if (base + RD_ATTN_PIECES < n) __syncthreads(); // the next round overwrites what the folding threads read
     }
     if (ti != 0) return false;
+    if (sinks) den += __expf(sinks[head] - M);
 #pragma unroll
     for (int e = 0; e < 4; e++) out[e] = num[e] / den;
     return true;
@@ -614,11 +625,11 @@ __device__ __forceinline__ bool attn_combine_block(const float *__restrict__ par
 
 // Grid (nH, rows), block RD_ATTN_PIECES * HD/4.
 extern "C" __global__ __launch_bounds__(512) void rd_k_attn_combine(const float *__restrict__ part, const int *__restrict__ itemStart, int partRows,
-                                                                     float *__restrict__ out, int nH, int nKV, int HD) {
+                                                                     float *__restrict__ out, int nH, int nKV, int HD, const float *__restrict__ sinks) {
     __shared__ float lds[RD_ATTN_PIECES * (128 + 2)];
     const int head = blockIdx.x, m = blockIdx.y;
     float v[4];
-    if (attn_combine_block(part, itemStart, partRows, nH, nKV, HD, m, head, lds, v)) {
+    if (attn_combine_block(part, itemStart, partRows, nH, nKV, HD, m, head, lds, v, sinks)) {
         float *o = out + (size_t)m * nH * HD + (size_t)head * HD + threadIdx.x * 4;
         o[0] = v[0], o[1] = v[1], o[2] = v[2], o[3] = v[3];
     }

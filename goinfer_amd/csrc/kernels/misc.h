@@ -162,61 +162,124 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_matmul_f32(const float *_
     if (lane == 0) dst[(size_t)m * N + n] = (float)acc;
 }
 
-// decoder/mlp.go:130-184 routeExperts (softmax scoring, no bias, no group limit) + mlp.go:370-440 softmaxF32/topK:
-// f32 max; e = f32(exp(f64(x - max))); f64 sum in ascending expert order; scores *= f32(1/sum); k passes of strict '>'
-// (lowest index wins); weights = chosen scores, optionally divided by their f32 sum in rank order.
+// decoder/mlp.go:130-228 routeExperts / groupLimit + mlp.go:370-440 softmaxF32 / topK.
+// Scores: softmax (f32 max; e = f32(exp(f64(x - max))); f64 sum in ascending expert order; scores *= f32(1/sum)) or, for the
+// DeepSeek / GLM routers, each expert's own f32(1 / (1 + exp(-f64(x)))). Selection scores: scores + bias where the layer has an
+// e_score_correction_bias; with nGroup > 1 only the experts of the topkGroup best groups stay eligible (a group's score: the sum
+// of its two largest selection scores), the others become -inf and are never chosen. k passes of strict '>' (lowest index wins).
+// Weights: the chosen experts' unbiased scores, optionally divided by their f32 sum in rank order, then times scale when that
+// is neither 0 nor 1.
 // One wave per token (nE <= 256: up to four experts per lane). The f64 sum is taken by every lane over the same ascending
 // sequence (from LDS), so it is the reference's sum bit for bit. Also fills rankOf[token][expert] = rank or -1 for the
 // expert-major grouped GEMMs. Grid (T), block 64.
-// The routing of one token by one wave (see rd_k_moe_route); x: the token's nE logits (global or LDS).
+struct RouteOpts {
+    const float *bias; // [nE] or NULL
+    int sigmoid;
+    float scale; // 0 or 1: none
+    int nGroup, topkGroup; // nGroup <= 32
+};
+// a key that orders as the floats do (-0 and +0 alike), 0 for "nothing": -inf, which topK never picks, and lanes past nE
+__device__ __forceinline__ unsigned route_key(float v) {
+    if (!(v > -INFINITY)) return 0u;
+    if (v == 0.f) v = 0.f;
+    const unsigned u = __float_as_uint(v);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+// The routing of one token by one wave (see rd_k_moe_route); x: the token's nE logits (global or LDS). e64: 256 doubles of LDS.
 __device__ __forceinline__ void moe_route_wave(const float *x, int t, int nE, int k, int norm, int *__restrict__ idx, float *__restrict__ wgt,
                                                signed char *__restrict__ rankOf, double *e64, int *__restrict__ idx_copy,
-                                               unsigned *__restrict__ activeBits) {
+                                               unsigned *__restrict__ activeBits, const RouteOpts &ro) {
     const int lane = threadIdx.x & 63;
-    float xv[4], sc[4];
-    float mx = -INFINITY;
+    float xv[4], sc[4], sel[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         int i = lane + 64 * j;
         xv[j] = i < nE ? x[i] : -INFINITY;
-        mx = fmaxf(mx, xv[j]);
     }
-    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    if (ro.sigmoid) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) sc[j] = (float)(1.0 / (1.0 + exp(-(double)xv[j])));
+    } else {
+        float mx = fmaxf(fmaxf(xv[0], xv[1]), fmaxf(xv[2], xv[3]));
+        for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            int i = lane + 64 * j;
+            double e = i < nE ? exp((double)__fsub_rn(xv[j], mx)) : 0.0;
+            sc[j] = (float)e;
+            e64[i] = e; // all 256 entries: zeros past nE, which leave the sum as it is
+        }
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0): this wave's LDS writes have landed before its lanes read them back
+        double sum = 0;
+        for (int i = 0; i < nE; i += 8) { // eight reads in flight, then the adds in ascending order
+            double v[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) v[u] = e64[i + u];
+#pragma unroll
+            for (int u = 0; u < 8; u++) sum += v[u];
+        }
+        const float inv = (float)(1.0 / sum);
+#pragma unroll
+        for (int j = 0; j < 4; j++) sc[j] = mul_rounded(sc[j], inv); // rounded before a bias is added
+    }
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         int i = lane + 64 * j;
-        double e = i < nE ? exp((double)__fsub_rn(xv[j], mx)) : 0.0;
-        sc[j] = (float)e;
-        e64[i] = e; // all 256 entries: zeros past nE, which leave the sum as it is
-    }
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0): this wave's LDS writes have landed before its lanes read them back
-    double sum = 0;
-    for (int i = 0; i < nE; i += 8) { // eight reads in flight, then the adds in ascending order
-        double v[8];
-#pragma unroll
-        for (int u = 0; u < 8; u++) v[u] = e64[i + u];
-#pragma unroll
-        for (int u = 0; u < 8; u++) sum += v[u];
-    }
-    const float inv = (float)(1.0 / sum);
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        int i = lane + 64 * j;
-        sc[j] = i < nE ? __fmul_rn(sc[j], inv) : -INFINITY;
+        sel[j] = i < nE ? (ro.bias ? __fadd_rn(sc[j], ro.bias[i]) : sc[j]) : -INFINITY;
         if (rankOf && i < nE) rankOf[(size_t)t * nE + i] = -1;
+    }
+    if (ro.nGroup > 1) {
+        // group scores through LDS: the selection scores, then one lane per group, then every lane ranks the groups alike
+        float *selbuf = (float *)e64, *gs = selbuf + 256;
+        const int gsz = nE / ro.nGroup;
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int j = 0; j < 4; j++) selbuf[lane + 64 * j] = sel[j];
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        if (lane < ro.nGroup) {
+            float top1 = -INFINITY, top2 = -INFINITY;
+            for (int i = lane * gsz; i < (lane + 1) * gsz; i++) {
+                const float v = selbuf[i];
+                if (v > top1)
+                    top2 = top1, top1 = v;
+                else if (v > top2)
+                    top2 = v;
+            }
+            gs[lane] = __fadd_rn(top1, top2);
+        }
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        unsigned keep = 0u;
+        for (int r = 0; r < ro.topkGroup; r++) { // topK over the group scores: strict '>', lowest index wins, -inf never
+            float best = -INFINITY;
+            int bg = -1;
+            for (int g = 0; g < ro.nGroup; g++) {
+                const float v = gs[g];
+                if (!((keep >> g) & 1u) && v > best) best = v, bg = g;
+            }
+            if (bg < 0) break;
+            keep |= 1u << bg;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int i = lane + 64 * j, g = i / gsz;
+            if (g >= ro.nGroup || !((keep >> g) & 1u)) sel[j] = -INFINITY; // outside the kept groups, or past the last whole group
+        }
     }
     float s = 0.f, mine = 0.f; // lane j keeps the rank-j weight
     int n = 0;
     for (int r = 0; r < k; r++) {
-        // The pass's pick as the maximum of a 64-bit key per lane: (score bits + 1, ~index), 0 for nothing left. Scores are >= 0,
-        // so their bit patterns order as the values do; of equal scores the lower index has the larger key, which is the
-        // strict '>' scan's choice. The maximum over the wave: within rows of 16 lanes on the DPP path, across the rows by swizzle
-        // and one permute.
+        // The pass's pick as the maximum of a 64-bit key per lane: (order-preserving key of the selection score, ~index), 0 for
+        // nothing left. Of equal scores the lower index has the larger key, which is the strict '>' scan's choice. The maximum
+        // over the wave: within rows of 16 lanes on the DPP path, across the rows by swizzle and one permute.
         unsigned kh = 0u, kl = 0u;
 #pragma unroll
-        for (int j = 3; j >= 0; j--) // descending, '>=' on the score: the lowest index among this lane's equals survives
-            if (sc[j] >= 0.f && __float_as_uint(sc[j]) + 1u >= kh) kh = __float_as_uint(sc[j]) + 1u, kl = ~(unsigned)(lane + 64 * j);
+        for (int j = 3; j >= 0; j--) { // descending, '>=' on the key: the lowest index among this lane's equals survives
+            const unsigned kj = route_key(sel[j]);
+            if (kj != 0u && kj >= kh) kh = kj, kl = ~(unsigned)(lane + 64 * j);
+        }
         auto take = [&](unsigned oh, unsigned ol) {
             const bool gt = oh > kh || (oh == kh && ol > kl);
             kh = gt ? oh : kh, kl = gt ? ol : kl;
@@ -227,13 +290,15 @@ __device__ __forceinline__ void moe_route_wave(const float *x, int t, int nE, in
         take((unsigned)dpp_i<RD_DPP_ROW_MIRROR>((int)kh), (unsigned)dpp_i<RD_DPP_ROW_MIRROR>((int)kl));
         take((unsigned)swz_xor16_i((int)kh), (unsigned)swz_xor16_i((int)kl));
         take((unsigned)__shfl_xor((int)kh, 32, 64), (unsigned)__shfl_xor((int)kl, 32, 64));
-        if (kh == 0u) break; // nothing left (k > nE)
-        const int bi = (int)~kl;
-        const float best = __uint_as_float(kh - 1u);
+        if (kh == 0u) break; // nothing left (k > the eligible experts)
+        const int bi = (int)~kl, bj = bi >> 6;
+        // the weight is the chosen expert's unbiased score, which its own lane holds
+        const float mineSc = bj == 0 ? sc[0] : (bj == 1 ? sc[1] : (bj == 2 ? sc[2] : sc[3]));
+        const float best = __shfl(mineSc, bi & 63, 64);
 #pragma unroll
         for (int j = 0; j < 4; j++)
             if (bi == lane + 64 * j) {
-                sc[j] = -INFINITY; // used
+                sel[j] = -INFINITY; // used
                 if (rankOf) rankOf[(size_t)t * nE + bi] = (signed char)r;
             }
         if (lane == r) mine = best;
@@ -245,18 +310,25 @@ __device__ __forceinline__ void moe_route_wave(const float *x, int t, int nE, in
         s = __fadd_rn(s, best);
         n++;
     }
-    if (lane < n) wgt[(size_t)t * k + lane] = (norm && s > 0.f) ? mine / s : mine;
+    if (lane < n) {
+        float w = (norm && s > 0.f) ? mine / s : mine;
+        if (ro.scale != 0.f && ro.scale != 1.f) w = __fmul_rn(w, ro.scale);
+        wgt[(size_t)t * k + lane] = w;
+    }
 }
 
 // idx_copy (may be NULL) receives a second copy of the indices: the step's per-layer routing trace. activeBits (may be NULL):
 // a bitmap of nE bits, zero on entry, in which every chosen expert's bit is set.
+// bias (may be NULL), sigmoid, scale, nGroup, topkGroup: the router's variant (see above); all zero = softmax top-k.
 extern "C" __global__ __launch_bounds__(64) void rd_k_moe_route(const float *__restrict__ logits, int T, int nE, int k, int norm,
                                                                  int *__restrict__ idx, float *__restrict__ wgt, signed char *__restrict__ rankOf,
-                                                                 int *__restrict__ idx_copy, unsigned *__restrict__ activeBits) {
+                                                                 int *__restrict__ idx_copy, unsigned *__restrict__ activeBits,
+                                                                 const float *__restrict__ bias, int sigmoid, float scale, int nGroup, int topkGroup) {
     __shared__ double e64[256];
     const int t = blockIdx.x;
     if (t >= T) return;
-    moe_route_wave(logits + (size_t)t * nE, t, nE, k, norm, idx, wgt, rankOf, e64, idx_copy, activeBits);
+    const RouteOpts ro{bias, sigmoid, scale, nGroup, topkGroup};
+    moe_route_wave(logits + (size_t)t * nE, t, nE, k, norm, idx, wgt, rankOf, e64, idx_copy, activeBits, ro);
 }
 
 // Token embedding rows from an int8 table with one f32 scale per row (goinfer keeps the embedding table int8 in q4k mode,

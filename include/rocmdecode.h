@@ -39,7 +39,7 @@ typedef struct rd_model rd_model;
 enum { RD_PROJ_Q = 0, RD_PROJ_K, RD_PROJ_V, RD_PROJ_O, RD_PROJ_GATE, RD_PROJ_UP, RD_PROJ_DOWN, RD_PROJ_HEAD, RD_PROJ_COUNT };
 /* f32 vectors. RD_VEC_QKV_BIAS (optional): the q, k and v projection biases end to end, (n_heads + 2 n_kv_heads) * head_dim values,
  * added right after the projections (Qwen2; decoder/attention.go:12-34 addBias, program_cpu_n.go:470-476). */
-enum { RD_VEC_ATTN_NORM = 0, RD_VEC_FFN_NORM, RD_VEC_Q_NORM, RD_VEC_K_NORM, RD_VEC_FINAL_NORM, RD_VEC_ROUTER, RD_VEC_QKV_BIAS };
+enum { RD_VEC_ATTN_NORM = 0, RD_VEC_FFN_NORM, RD_VEC_Q_NORM, RD_VEC_K_NORM, RD_VEC_FINAL_NORM, RD_VEC_ROUTER, RD_VEC_QKV_BIAS, RD_VEC_ROUTER_BIAS, RD_VEC_ATTN_SINKS };
 /* rd_step_batch `want` */
 enum { RD_WANT_LOGITS = 1, RD_WANT_ARGMAX = 2 };
 
@@ -123,9 +123,21 @@ int rd_attn_ragged_i8(rd_device *d, int n_seq, const int *len, const int64_t *of
  * bit-identical to the row computed alone. */
 int rd_attn_ragged_rows(rd_device *d, int kv_type, int n_seq, const int *len, const int *nq, const int64_t *off, const float *k,
                         const float *v, const float *q, int n_h, int n_kv, int hd, float scale, float softcap, float *out);
+/* rd_attn_ragged_rows (nq may be NULL: one query row per sequence) with the two knobs of decoder/attention.go:57-143 /
+ * forwardn.go:379-500 that are not on every model: window > 0, each row reads only the last `window` positions up to its own
+ * (kvmgr.WindowNeedStart: start = max(pos - window + 1, 0)); sinks (host f32 [n_h] or NULL), one learned logit per query head
+ * that joins the softmax's maximum and denominator and nothing else (attention.go:305-322). */
+int rd_attn_ragged_ex(rd_device *d, int kv_type, int n_seq, const int *len, const int *nq, const int64_t *off, const float *k, const float *v,
+                      const float *q, int n_h, int n_kv, int hd, float scale, float softcap, int window, const float *sinks, float *out);
 /* MoE routing (decoder/mlp.go:130-184 routeExperts, softmax scoring; backend/cuda/moe.cu:49-104 moe_route):
  * logits host f32 [T][nE]; idx int32 [T][k], wgt f32 [T][k], rank order. */
 int rd_moe_route(rd_device *d, const float *logits, int T, int nE, int k, int norm, int *idx, float *wgt);
+/* The whole of routeExperts (decoder/mlp.go:130-228): sigmoid != 0 scores every expert by its own sigmoid instead of a softmax
+ * (DeepSeek / GLM); bias (host f32 [nE] or NULL, e_score_correction_bias) shifts the selection only, the weights stay the unbiased
+ * scores; n_group > 1 keeps only the experts of the topk_group best of n_group contiguous groups eligible (groupLimit; at most 32
+ * groups); scale (routed_scaling_factor) multiplies the weights when it is neither 0 nor 1. */
+int rd_moe_route_ex(rd_device *d, const float *logits, const float *bias, int T, int nE, int k, int sigmoid, int norm, double scale,
+                    int n_group, int topk_group, int *idx, float *wgt);
 /* RMSNorm rows (decoder/rmsnorm.go:29-92) and NeoX RoPE (decoder/rope.go:28-64), host pointers. */
 int rd_rmsnorm(rd_device *d, const float *x, const float *w, int rows, int dim, float eps, float *out);
 int rd_rope(rd_device *d, float *vec, int rows, int heads, int head_dim, const int *pos, const double *inv_freq);
@@ -145,8 +157,15 @@ int rd_model_upload_q6k(rd_model *m, int layer, int proj, const void *blocks, in
 int rd_model_upload_w8a8(rd_model *m, int layer, int proj, const int8_t *q, const float *row_scale, int N, int K);
 /* canonical int4 nibbles + binary16 group-32 scales (WeightMat.Int4F16, decoder/weightmat.go:904); expert < 0 = dense */
 int rd_model_upload_w4a8(rd_model *m, int layer, int proj, int expert, const uint8_t *nib, const uint16_t *s16, int N, int K);
-/* norms, router */
+/* norms, router; RD_VEC_ROUTER_BIAS: a layer's e_score_correction_bias [n_experts]; RD_VEC_ATTN_SINKS: its attention sinks [n_heads] */
 int rd_model_upload_f32(rd_model *m, int layer, int which, const float *v, size_t n);
+/* The router's variant, decoder/mlp.go:130-228 (routeExperts, groupLimit); before rd_model_finalize. sigmoid: per-expert sigmoid
+ * scores (DeepSeek / GLM) instead of a softmax; scale: routed_scaling_factor (0 or 1 = none); n_group > 1: group-limited
+ * selection among the topk_group best of n_group contiguous groups (at most 32 groups, which must divide the experts). */
+int rd_model_set_router(rd_model *m, int sigmoid, double scale, int n_group, int topk_group);
+/* A sliding-window layer (decoder/kvcache.go:1063-1068 WindowStart): its rows read the last `window` positions only. Before
+ * rd_model_finalize. The windowed layers of a model share one length (RD_DECLINED otherwise); the cache keeps every position. */
+int rd_model_set_window(rd_model *m, int layer, int window);
 /* after the last upload: checks every tensor the step needs is present */
 int rd_model_finalize(rd_model *m);
 

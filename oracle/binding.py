@@ -20,7 +20,8 @@ class Layer(C.Structure):
     _fields_ = [(n, Mat) for n in ("q", "k", "v", "o", "gate", "up", "down")] + [
         ("attn_norm", C.c_void_p), ("ffn_norm", C.c_void_p), ("q_norm", C.c_void_p), ("k_norm", C.c_void_p),
         ("q_bias", C.c_void_p), ("k_bias", C.c_void_p), ("v_bias", C.c_void_p),
-        ("router", Mat), ("exp_gate", C.POINTER(Mat)), ("exp_up", C.POINTER(Mat)), ("exp_down", C.POINTER(Mat))]
+        ("router", Mat), ("exp_gate", C.POINTER(Mat)), ("exp_up", C.POINTER(Mat)), ("exp_down", C.POINTER(Mat)),
+        ("router_bias", C.c_void_p), ("window", C.c_int), ("sinks", C.c_void_p)]
 
 
 class Model(C.Structure):
@@ -29,7 +30,8 @@ class Model(C.Structure):
                 ("eps", C.c_double), ("attn_scale", C.c_double), ("softcap", C.c_double),
                 ("inv_freq", C.c_void_p),
                 ("n_experts", C.c_int), ("top_k", C.c_int), ("norm_topk", C.c_int), ("exp_inter", C.c_int),
-                ("kv_f16", C.c_int), ("layers", C.POINTER(Layer)), ("final_norm", C.c_void_p), ("head", Mat)]
+                ("kv_f16", C.c_int), ("layers", C.POINTER(Layer)), ("final_norm", C.c_void_p), ("head", Mat),
+                ("router_sigmoid", C.c_int), ("router_scale", C.c_double), ("n_group", C.c_int), ("topk_group", C.c_int)]
 
 
 def f16_round_trip(x):
@@ -72,7 +74,7 @@ def lib():
 
 
 def _p(a):
-    return a.ctypes.data_as(C.c_void_p)
+    return a.ctypes.data_as(C.c_void_p) if a is not None else None
 
 
 def f32(a):
@@ -204,12 +206,21 @@ def swiglu(gate, up):
     return g
 
 
-def route_experts(logits, k, norm, scale=0.0):
+def route_experts(logits, k, norm, scale=0.0, bias=None, sigmoid=False, n_group=0, topk_group=0):
     lg = f32(logits)
     idx = np.empty(k, np.int32)
     wts = np.empty(k, np.float32)
-    n = lib().or_route_experts(_p(lg), lg.size, k, int(norm), C.c_double(scale), _p(idx), _p(wts))
+    bs = f32(bias) if bias is not None else None
+    n = lib().or_route_experts_ex(_p(lg), _p(bs), lg.size, k, int(sigmoid), int(norm), C.c_double(scale), int(n_group), int(topk_group),
+                                  _p(idx), _p(wts))
     return idx[:n], wts[:n]
+
+
+def group_limit(sel, n_group, topk_group):
+    sel = f32(sel)
+    out = np.empty_like(sel)
+    lib().or_group_limit(_p(sel), sel.size, int(n_group), int(topk_group), _p(out))
+    return out
 
 
 def topk_by_logit(x, k):
@@ -230,13 +241,14 @@ def argmax(x):
     return lib().or_argmax(_p(x), x.size)
 
 
-def attend(q, keys, vals, n_keys, nH, nKV, hd, scale, softcap=0.0, start=0):
+def attend(q, keys, vals, n_keys, nH, nKV, hd, scale, softcap=0.0, start=0, sinks=None):
     q = f32(q)
     keys = f32(keys)
     vals = f32(vals)
     ctx = np.empty(nH * hd, np.float32)
-    lib().or_attend(_p(q), _p(ctx), _p(keys), _p(vals), int(n_keys), int(start), nH, nKV, hd,
-                    C.c_double(scale), C.c_double(softcap))
+    sk = f32(sinks) if sinks is not None else None
+    lib().or_attend_sinks(_p(q), _p(ctx), _p(keys), _p(vals), int(n_keys), int(start), nH, nKV, hd,
+                          C.c_double(scale), C.c_double(softcap), _p(sk))
     return ctx
 
 
@@ -255,7 +267,8 @@ class OracleModel:
             for n in ("q", "k", "v", "o"):
                 setattr(L, n, lw[n].c())
             self._keep.append(lw)
-            for n in ("attn_norm", "ffn_norm", "q_norm", "k_norm", "q_bias", "k_bias", "v_bias"):
+            L.window = int(lw.get("window", 0))
+            for n in ("attn_norm", "ffn_norm", "q_norm", "k_norm", "q_bias", "k_bias", "v_bias", "router_bias", "sinks"):
                 if lw.get(n) is not None:
                     arr = f32(lw[n])
                     self._keep.append(arr)
@@ -275,7 +288,8 @@ class OracleModel:
         self.m = Model(nL, cfg["hidden"], cfg["n_heads"], cfg["n_kv"], cfg["head_dim"], cfg.get("inter", 0),
                        cfg["vocab"], cfg["eps"], cfg["attn_scale"], cfg.get("softcap", 0.0), _p(self._inv),
                        nE, cfg.get("top_k", 0), int(cfg.get("norm_topk", 0)), cfg.get("exp_inter", 0),
-                       int(cfg.get("kv_f16", 0)), self._layers, _p(self._fn), head.c())
+                       int(cfg.get("kv_f16", 0)), self._layers, _p(self._fn), head.c(),
+                       int(cfg.get("router_sigmoid", 0)), float(cfg.get("router_scale", 0.0)), int(cfg.get("n_group", 0)), int(cfg.get("topk_group", 0)))
 
     def new_cache(self, cap):
         return lib().or_cache_new(C.byref(self.m), cap)

@@ -343,12 +343,54 @@ int or_topk(const float *x, int n, int k, int *idx, float *val) {
     return cnt;
 }
 
-/* decoder/mlp.go:130-184 (routeExperts), softmax scoring without bias or group limit: weights are the
- * chosen scores, norm divides by their f32 sum taken in rank order, scale multiplies when not 0 or 1. */
-int or_route_experts(const float *logits, int nE, int k, int norm, double scale, int *idx, float *wts) {
-    float *scores = (float *)malloc(sizeof(float) * (size_t)nE);
-    or_softmax_f32(logits, nE, scores);
-    int n = or_topk(scores, nE, k, idx, NULL);
+/* decoder/mlp.go:186-228 (groupLimit): DeepSeek-V3 group-limited selection. The nE selection scores fall into nGroup contiguous
+ * groups of nE/nGroup; a group's score is the sum of its two largest entries; the topkGroup best groups (topK's rule) keep their
+ * scores, everything else, the experts past nGroup*(nE/nGroup) included, becomes -inf. out may not alias sel. */
+void or_group_limit(const float *sel, int nE, int nGroup, int topkGroup, float *out) {
+    int gsz = nE / nGroup;
+    float *gscore = (float *)malloc(sizeof(float) * (size_t)nGroup);
+    int *keepIdx = (int *)malloc(sizeof(int) * (size_t)(topkGroup > 0 ? topkGroup : 1));
+    for (int g = 0; g < nGroup; g++) {
+        float top1 = -INFINITY, top2 = -INFINITY;
+        for (int i = g * gsz; i < (g + 1) * gsz; i++) {
+            float v = sel[i];
+            if (v > top1) {
+                top2 = top1;
+                top1 = v;
+            } else if (v > top2) {
+                top2 = v;
+            }
+        }
+        gscore[g] = top1 + top2;
+    }
+    int nk = or_topk(gscore, nGroup, topkGroup, keepIdx, NULL);
+    for (int i = 0; i < nE; i++) out[i] = -INFINITY;
+    for (int j = 0; j < nk; j++)
+        for (int i = keepIdx[j] * gsz; i < (keepIdx[j] + 1) * gsz; i++) out[i] = sel[i];
+    free(gscore);
+    free(keepIdx);
+}
+
+/* decoder/mlp.go:130-184 (routeExperts). Scores: softmax over the experts, or (sigmoid) each expert's own
+ * float32(1/(1+exp(-float64(logit)))). Selection scores: scores + bias when there is a bias (e_score_correction_bias), masked by
+ * or_group_limit when nGroup > 1; the k best by topK's rule. Weights: the chosen experts' UNBIASED scores; norm divides them by
+ * their f32 sum taken in rank order (when it is > 0); scale multiplies them when it is neither 0 nor 1. */
+int or_route_experts_ex(const float *logits, const float *bias, int nE, int k, int sigmoid, int norm, double scale, int nGroup,
+                        int topkGroup, int *idx, float *wts) {
+    float *scores = (float *)malloc(sizeof(float) * (size_t)nE), *sel = scores, *lim = NULL;
+    if (sigmoid)
+        for (int i = 0; i < nE; i++) scores[i] = (float)(1.0 / (1.0 + exp(-(double)logits[i])));
+    else
+        or_softmax_f32(logits, nE, scores);
+    if (bias) {
+        sel = (float *)malloc(sizeof(float) * (size_t)nE);
+        for (int i = 0; i < nE; i++) sel[i] = scores[i] + bias[i];
+    }
+    if (nGroup > 1) {
+        lim = (float *)malloc(sizeof(float) * (size_t)nE);
+        or_group_limit(sel, nE, nGroup, topkGroup, lim);
+    }
+    int n = or_topk(lim ? lim : sel, nE, k, idx, NULL);
     for (int j = 0; j < n; j++) wts[j] = scores[idx[j]];
     if (norm) {
         float s = 0.f;
@@ -358,8 +400,13 @@ int or_route_experts(const float *logits, int nE, int k, int norm, double scale,
     }
     if (scale != 0 && scale != 1)
         for (int j = 0; j < n; j++) wts[j] *= (float)scale;
+    if (sel != scores) free(sel);
+    free(lim);
     free(scores);
     return n;
+}
+int or_route_experts(const float *logits, int nE, int k, int norm, double scale, int *idx, float *wts) {
+    return or_route_experts_ex(logits, NULL, nE, k, 0, norm, scale, 0, 0, idx, wts);
 }
 
 /* internal/runtime/sampling/sampler.go:485-520 (Argmax): strict '>' from index 0. */
@@ -769,8 +816,8 @@ static double softcap_score(double s, double c) { return c == 0 ? s : c * tanh(s
 /* decoder/forwardn.go:295-500 with useAcc64 and K=1 (the form program_cpu_n.go:497-515 calls), no sinks,
  * no tree mask: per query head, scores = f32(f64 dot) -> sc = softcap(f64(score)*scale) stored f32 ->
  * max -> e = exp(f64(sc_f32) - max) stored f32, f64 sum -> w = f32(f64(e_f32) * (1/sum)) -> AV in f64. */
-void or_attend(const float *q, float *ctx, const float *keys, const float *vals, int n_keys, int start,
-               int nH, int nKV, int hd, double scale, double softcap) {
+void or_attend_sinks(const float *q, float *ctx, const float *keys, const float *vals, int n_keys, int start,
+                     int nH, int nKV, int hd, double scale, double softcap, const float *sinks) {
     int kvDim = nKV * hd, group = nH / nKV;
 #pragma omp parallel for num_threads(g_threads) schedule(dynamic, 1)
     for (int qh = 0; qh < nH; qh++) {
@@ -785,12 +832,15 @@ void or_attend(const float *q, float *ctx, const float *keys, const float *vals,
                 scores[s] = (float)sc;
                 if (sc > maxS) maxS = sc;
             }
+            /* decoder/attention.go:305-322 sinkMax / sinkSum: the head's learned sink joins the max-shift and the denominator, nothing else */
+            if (sinks && (double)sinks[qh] > maxS) maxS = (double)sinks[qh];
             double sum = 0;
             for (int s = lo; s <= hi; s++) {
                 double e = exp((double)scores[s] - maxS);
                 scores[s] = (float)e;
                 sum += e;
             }
+            if (sinks) sum += exp((double)sinks[qh] - maxS);
             double inv = 1.0 / sum;
             for (int s = 0; s < lo; s++) scores[s] = 0.f;
             for (int s = lo; s <= hi; s++) scores[s] = (float)((double)scores[s] * inv);
@@ -800,6 +850,10 @@ void or_attend(const float *q, float *ctx, const float *keys, const float *vals,
         or_av_acc64(scores, vals, ctx + (size_t)qh * hd, 1, n_keys, hd, kvh * hd, kvDim);
         free(scores);
     }
+}
+void or_attend(const float *q, float *ctx, const float *keys, const float *vals, int n_keys, int start,
+               int nH, int nKV, int hd, double scale, double softcap) {
+    or_attend_sinks(q, ctx, keys, vals, n_keys, start, nH, nKV, hd, scale, softcap, NULL);
 }
 
 /* ------------------------------------------------------------------ model */
@@ -882,7 +936,7 @@ static void moe_mlp(const or_model *m, const or_layer *lw, const float *h, float
     float *g = (float *)malloc(sizeof(float) * (size_t)I), *u = (float *)malloc(sizeof(float) * (size_t)I);
     float *eo = (float *)malloc(sizeof(float) * (size_t)H);
     or_matmul(&lw->router, h, 1, logits);
-    int n = or_route_experts(logits, nE, k, m->norm_topk, 0, idx, wts);
+    int n = or_route_experts_ex(logits, lw->router_bias, nE, k, m->router_sigmoid, m->norm_topk, m->router_scale, m->n_group, m->topk_group, idx, wts);
     if (replay) { /* decoder/mlp.go:53-56: the recorded routing replaces this call's own */
         n = k;
         for (int j = 0; j < k; j++) idx[j] = idx_trace[j], wts[j] = wts_trace[j];
@@ -954,7 +1008,9 @@ int or_decode_multi_step_traced(const or_model *m, int B, const float *emb, or_c
             float *kr = c->k[l] + (size_t)c->pos * kvDim, *vr = c->v[l] + (size_t)c->pos * kvDim;
             kv_narrow_row(m, kb, kr); /* as the cache stores it: f32, binary16 or int8 per head */
             kv_narrow_row(m, vb, vr);
-            or_attend(qb, ctx + (size_t)b * qDim, c->k[l], c->v[l], c->pos + 1, 0, nH, nKV, hd, m->attn_scale, m->softcap);
+            /* kvmgr.WindowNeedStart (internal/runtime/kvmgr/sequence.go:55-60): a windowed layer reads keys pos-window+1 .. pos */
+            const int start = lw->window > 0 && c->pos - lw->window + 1 > 0 ? c->pos - lw->window + 1 : 0;
+            or_attend_sinks(qb, ctx + (size_t)b * qDim, c->k[l], c->v[l], c->pos + 1, start, nH, nKV, hd, m->attn_scale, m->softcap, lw->sinks);
         }
         or_matmul(&lw->o, ctx, B, att);
         for (size_t i = 0; i < (size_t)B * H; i++) h[i] += att[i];

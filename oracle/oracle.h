@@ -95,6 +95,10 @@ void or_swiglu(float *gate, const float *up, int n);
 void or_softmax_f32(const float *x, int n, float *out);
 int or_topk(const float *x, int n, int k, int *idx, float *val);
 int or_route_experts(const float *logits, int nE, int k, int norm, double scale, int *idx, float *wts);
+/* the whole of routeExperts: sigmoid scoring, selection bias, group-limited selection (decoder/mlp.go:130-228) */
+int or_route_experts_ex(const float *logits, const float *bias, int nE, int k, int sigmoid, int norm, double scale, int nGroup,
+                        int topkGroup, int *idx, float *wts);
+void or_group_limit(const float *sel, int nE, int nGroup, int topkGroup, float *out);
 int or_argmax(const float *x, int n); /* internal/runtime/sampling/sampler.go:485-520: first maximum wins */
 int or_topk_by_logit(const float *x, int n, int k, int *ids, float *vals); /* sampler.go:726-782 + the (logit desc, id asc) order of TopKRow */
 double or_softmax_z(const float *x, int n, double temperature);            /* the top-p denominator, f64 */
@@ -126,6 +130,9 @@ void or_set_threads(int n);
  * decoder/program_cpu_n.go:497-515 + forwardn.go:295-500 (useAcc64, K=1) + kvcache.go:21-40 (f16 narrowing) ---- */
 void or_attend(const float *q, float *ctx, const float *keys, const float *vals, int n_keys, int start,
                int nH, int nKV, int hd, double scale, double softcap);
+/* the same with attention sinks (decoder/attention.go:305-322): sinks[nH] or NULL */
+void or_attend_sinks(const float *q, float *ctx, const float *keys, const float *vals, int n_keys, int start,
+                     int nH, int nKV, int hd, double scale, double softcap, const float *sinks);
 
 /* ---- the model and decodeMultiStep: decoder/cpu_batch.go:166-197, program_cpu_n.go:406-563, mlp.go:36-120 ---- */
 typedef struct {
@@ -135,6 +142,9 @@ typedef struct {
     const float *q_bias, *k_bias, *v_bias; /* [nH*hd], [nKV*hd], [nKV*hd] or NULL (Qwen2 projection biases) */
     or_mat router;                     /* [nE, hidden] */
     or_mat *exp_gate, *exp_up, *exp_down; /* [nE] each */
+    const float *router_bias;          /* [nE] or NULL: e_score_correction_bias, shifts the selection only */
+    int window;                        /* > 0: this layer attends to the last `window` positions only (keys from pos-window+1) */
+    const float *sinks;                /* [nH] or NULL: a learned logit per query head that joins the softmax's max and denominator */
 } or_layer;
 
 typedef struct {
@@ -146,6 +156,9 @@ typedef struct {
     or_layer *layers;
     const float *final_norm;
     or_mat head;
+    int router_sigmoid;  /* 1: per-expert sigmoid scores instead of a softmax (DeepSeek / GLM) */
+    double router_scale; /* routed_scaling_factor; 0 or 1 = none */
+    int n_group, topk_group; /* > 1: group-limited selection */
 } or_model;
 
 typedef struct {

@@ -96,6 +96,14 @@ class Pair:
             lw["attn_norm"], lw["ffn_norm"] = vec(l, "attn_norm", H), vec(l, "ffn_norm", H)
             if cfg.get("qk_norm"):
                 lw["q_norm"], lw["k_norm"] = vec(l, "q_norm", hd), vec(l, "k_norm", hd)
+            if cfg.get("attn_sinks"):  # one learned logit per query head joining the softmax (decoder/attention.go:305-322)
+                lw["sinks"] = synth.normal(nxt(), nH, 2.0)
+                if self.gpu:
+                    self.gpu.upload_f32(l, "attn_sinks", lw["sinks"])
+            if cfg.get("window") and l % 2 == 0:  # sliding-window layers alternate with whole-context ones, as in Gemma-2
+                lw["window"] = int(cfg["window"])
+                if self.gpu:
+                    self.gpu.set_window(l, lw["window"])
             if cfg.get("qkv_bias"):  # Qwen2: biases on the q, k and v projections, sent to the GPU as one vector
                 b = synth.normal(nxt(), qd + 2 * kvd, 0.5)
                 lw["q_bias"], lw["k_bias"], lw["v_bias"] = b[:qd].copy(), b[qd:qd + kvd].copy(), b[qd + kvd:].copy()
@@ -109,6 +117,10 @@ class Pair:
                 if self.gpu:
                     self.gpu.upload_f32(l, "router", r)
                 lw["router"] = ob.WMat.from_f32(r)
+                if cfg.get("router_bias"):  # e_score_correction_bias: shifts the selection, not the weights
+                    lw["router_bias"] = synth.normal(nxt(), nE, 0.2)
+                    if self.gpu:
+                        self.gpu.upload_f32(l, "router_bias", lw["router_bias"])
                 lw["exp_gate"] = [mat(l, "gate", EI, H, e) for e in range(nE)]
                 lw["exp_up"] = [mat(l, "up", EI, H, e) for e in range(nE)]
                 lw["exp_down"] = [mat(l, "down", H, EI, e) for e in range(nE)]

@@ -1,0 +1,117 @@
+"""The knobs of the decode path that are not on the five benchmark configurations: router variants (sigmoid scoring, selection
+bias, group-limited selection, routed scaling factor; decoder/mlp.go:130-228), attention sinks and the sliding window
+(decoder/attention.go:57-143, 305-322; kvmgr.WindowNeedStart). Kernel level against the oracle (routing bit for bit, attention to
+the flash-decode bar of 1e-4), then whole models through the step."""
+import numpy as np
+import pytest
+
+from goinfer_amd import capi, synth
+from oracle import binding as ob
+from tests.models import Pair, dense_cfg, moe_cfg
+from tests.test_gpu_attention import i8_round_trip
+from tests.test_gpu_model import check
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    d = capi.Device(0)
+    yield d
+    d.close()
+
+
+@pytest.mark.parametrize("nE,k,sigmoid,use_bias,n_group,topk_group,scale,norm", [
+    (128, 8, True, True, 8, 4, 2.5, True),      # DeepSeek-V3 style: sigmoid + bias + groups + scale
+    (64, 6, True, True, 0, 0, 1.0, True),       # GLM: sigmoid + bias
+    (128, 8, False, True, 0, 0, 0.0, True),     # softmax with a selection bias
+    (160, 4, True, False, 4, 2, 16.0, False),   # groups without a bias
+    (30, 4, True, True, 4, 1, 0.0, True),       # experts past the last whole group are never eligible
+    (8, 6, True, True, 4, 1, 0.0, True),        # fewer eligible experts than k: the row comes back short
+    (256, 8, False, False, 0, 0, 0.0, True),    # the plain softmax router at the widest row
+])
+def test_route_variants_bit_exact(dev, nE, k, sigmoid, use_bias, n_group, topk_group, scale, norm):
+    rng = np.random.default_rng(nE * 7 + k)
+    T = 16
+    logits = (rng.standard_normal((T, nE)) * 2).astype(np.float32)
+    logits[3] = np.round(logits[3])          # ties
+    logits[4] = 0.0                          # all equal: the lowest indices win
+    bias = (rng.standard_normal(nE) * 0.3).astype(np.float32) if use_bias else None
+    idx, wgt = dev.moe_route(logits, k, norm, bias=bias, sigmoid=sigmoid, scale=scale, n_group=n_group, topk_group=topk_group)
+    for t in range(T):
+        wi, ww = ob.route_experts(logits[t], k, norm, scale, bias=bias, sigmoid=sigmoid, n_group=n_group, topk_group=topk_group)
+        n = len(wi)
+        assert np.array_equal(idx[t, :n], wi), (t, idx[t], wi)
+        assert np.array_equal(wgt[t, :n].view(np.uint32), ww.view(np.uint32)), (t, wgt[t], ww)
+
+
+@pytest.mark.parametrize("kv", ["f16", "i8"])
+@pytest.mark.parametrize("hd,nH,nKV", [(128, 8, 2), (64, 8, 8)])
+def test_attention_window_and_sinks(dev, kv, hd, nH, nKV):
+    """Rows over windowed contexts, with and without sinks and softcap, against the oracle's f64 attention over the rows as the
+    cache holds them; and a row in a ragged batch equals the row alone, bit for bit."""
+    lens = [1, 5, 63, 64, 65, 130, 700, 2000]
+    kvd = nKV * hd
+    ks = [synth.normal(100 + i, n * kvd).reshape(n, kvd) for i, n in enumerate(lens)]
+    vs = [synth.normal(200 + i, n * kvd).reshape(n, kvd) for i, n in enumerate(lens)]
+    q = synth.normal(9, len(lens) * nH * hd).reshape(len(lens), nH * hd)
+    sinks = synth.normal(11, nH, 2.0)
+    scale = hd ** -0.5
+    hold = (lambda x: ob.f16_round_trip(x)) if kv == "f16" else (lambda x: i8_round_trip(x, nKV, hd))
+    for window, sk, cap in ((0, sinks, 0.0), (48, None, 0.0), (100, sinks, 30.0), (1, sinks, 0.0), (4096, None, 0.0)):
+        got = dev.attn_ragged_ex(lens, np.concatenate(ks), np.concatenate(vs), q, nH, nKV, hd, scale, cap, kv=kv, window=window, sinks=sk)
+        for i, n in enumerate(lens):
+            start = max(n - window, 0) if window else 0
+            want = ob.attend(q[i], hold(ks[i]), hold(vs[i]), n, nH, nKV, hd, scale, cap, start=start, sinks=sk)
+            assert np.abs(got[i] - want).max() <= 1e-4 * max(1.0, np.abs(want).max()), (window, i, n)
+        solo = dev.attn_ragged_ex(lens[6:7], ks[6], vs[6], q[6:7], nH, nKV, hd, scale, cap, kv=kv, window=window, sinks=sk)
+        assert np.array_equal(solo[0].view(np.uint32), got[6].view(np.uint32))
+
+
+def test_attention_window_rows_of_one_sequence(dev):
+    """Several consecutive positions of a sequence in one call (a prompt pass), each row with its own window start: equal to the
+    rows computed one by one, bit for bit, and to the oracle."""
+    nH, nKV, hd, n, nq, window = 8, 2, 128, 300, 7, 70
+    kvd = nKV * hd
+    k, v = synth.normal(1, n * kvd).reshape(n, kvd), synth.normal(2, n * kvd).reshape(n, kvd)
+    q = synth.normal(3, nq * nH * hd).reshape(nq, nH * hd)
+    scale = hd ** -0.5
+    got = dev.attn_ragged_ex([n], k, v, q, nH, nKV, hd, scale, nq=[nq], window=window)
+    for j in range(nq):
+        ln = n - nq + 1 + j
+        one = dev.attn_ragged_ex([ln], k[:ln], v[:ln], q[j:j + 1], nH, nKV, hd, scale, window=window)
+        assert np.array_equal(one[0].view(np.uint32), got[j].view(np.uint32)), j
+        want = ob.attend(q[j], ob.f16_round_trip(k), ob.f16_round_trip(v), ln, nH, nKV, hd, scale, start=max(ln - window, 0))
+        assert np.abs(got[j] - want).max() <= 1e-4 * max(1.0, np.abs(want).max())
+
+
+def test_model_with_window_and_sinks(dev):
+    """A dense model whose even layers have a sliding window of 24 positions and whose every layer has attention sinks, through
+    ragged prompts that outgrow the window, then batched greedy steps, against the oracle."""
+    cfg = dict(dense_cfg(n_layers=4, hidden=256, n_heads=4, n_kv=2, head_dim=64, inter=512, vocab=512), window=24, attn_sinks=1)
+    rng = np.random.default_rng(21)
+    check(Pair(cfg, seed=31, dev=dev, slots=8), [list(rng.integers(0, 512, n)) for n in (3, 30, 70)], steps=4)
+    # and the window is not ignored: the same model without it answers differently once a context has outgrown it
+    a, b = Pair(cfg, seed=31, dev=dev, slots=2), Pair(dict(cfg, window=0), seed=31, dev=dev, slots=2)
+    try:
+        toks = list(rng.integers(0, 512, 40))
+        for p, t in enumerate(toks):
+            la, _ = a.gpu.step_batch([0], [p], a.emb[[t]])
+            lb, _ = b.gpu.step_batch([0], [p], b.emb[[t]])
+            if p < 24:
+                assert np.array_equal(la.view(np.uint32), lb.view(np.uint32)), p  # inside the window the two are one model
+        assert np.abs(la - lb).max() > 1e-3
+    finally:
+        a.close()
+        b.close()
+
+
+def test_moe_model_with_deepseek_style_router(dev):
+    """Sigmoid scores, a selection bias per layer, group-limited selection (4 groups, the best 2), weights renormalized and scaled
+    by 2.5, through the step against the oracle; rows are compared while their routing agrees with the oracle's."""
+    cfg = dict(moe_cfg(n_layers=2, hidden=256, n_heads=4, n_kv=2, head_dim=64, n_experts=16, top_k=4, exp_inter=128),
+               router_sigmoid=1, router_bias=1, n_group=4, topk_group=2, router_scale=2.5)
+    rng = np.random.default_rng(5)
+    _, _, (agree, total, diverged) = check(Pair(cfg, seed=41, dev=dev, slots=8), [list(rng.integers(0, 512, n)) for n in (2, 20)], steps=4)
+    assert agree >= 0.9 * total, (agree, total)
+    assert not all(diverged)
