@@ -21,7 +21,8 @@ class Layer(C.Structure):
         ("attn_norm", C.c_void_p), ("ffn_norm", C.c_void_p), ("q_norm", C.c_void_p), ("k_norm", C.c_void_p),
         ("q_bias", C.c_void_p), ("k_bias", C.c_void_p), ("v_bias", C.c_void_p),
         ("router", Mat), ("exp_gate", C.POINTER(Mat)), ("exp_up", C.POINTER(Mat)), ("exp_down", C.POINTER(Mat)),
-        ("router_bias", C.c_void_p), ("window", C.c_int), ("sinks", C.c_void_p)]
+        ("router_bias", C.c_void_p), ("window", C.c_int), ("sinks", C.c_void_p),
+        ("post_attn_norm", C.c_void_p), ("post_ffn_norm", C.c_void_p)]
 
 
 class Model(C.Structure):
@@ -31,7 +32,8 @@ class Model(C.Structure):
                 ("inv_freq", C.c_void_p),
                 ("n_experts", C.c_int), ("top_k", C.c_int), ("norm_topk", C.c_int), ("exp_inter", C.c_int),
                 ("kv_f16", C.c_int), ("layers", C.POINTER(Layer)), ("final_norm", C.c_void_p), ("head", Mat),
-                ("router_sigmoid", C.c_int), ("router_scale", C.c_double), ("n_group", C.c_int), ("topk_group", C.c_int)]
+                ("router_sigmoid", C.c_int), ("router_scale", C.c_double), ("n_group", C.c_int), ("topk_group", C.c_int),
+                ("norm_add_one", C.c_int), ("act_gelu_tanh", C.c_int), ("final_softcap", C.c_double)]
 
 
 def f16_round_trip(x):
@@ -60,6 +62,9 @@ def lib():
         L.or_f16_to_f32.argtypes = [C.c_uint16]
         L.or_silu.restype = C.c_float
         L.or_silu.argtypes = [C.c_float]
+        L.or_gelu_tanh.restype = C.c_float
+        L.or_gelu_tanh.argtypes = [C.c_float]
+        L.or_softcap_logits.argtypes = [C.c_void_p, C.c_size_t, C.c_float]
         L.or_quantize_row_int8.restype = C.c_float
         L.or_kprint_name.restype = C.c_char_p
         L.or_softmax_z.restype = C.c_double
@@ -206,6 +211,21 @@ def swiglu(gate, up):
     return g
 
 
+def geglu(gate, up):
+    """geluTanh(gate) * up, element by element."""
+    g = f32(gate).copy()
+    u = f32(up)
+    lib().or_geglu(_p(g), _p(u), g.size)
+    return g
+
+
+def softcap_logits(x, cap):
+    """cap * tanh(x / cap) as the final-logit softcap computes it."""
+    x = f32(x).copy()
+    lib().or_softcap_logits(_p(x), C.c_size_t(x.size), C.c_float(cap))
+    return x
+
+
 def route_experts(logits, k, norm, scale=0.0, bias=None, sigmoid=False, n_group=0, topk_group=0):
     lg = f32(logits)
     idx = np.empty(k, np.int32)
@@ -254,7 +274,8 @@ def attend(q, keys, vals, n_keys, nH, nKV, hd, scale, softcap=0.0, start=0, sink
 
 class OracleModel:
     """decodeMultiStep over numpy weights. layers: list of dicts with WMat entries q,k,v,o,(gate,up,down | router,
-    exp_gate[],exp_up[],exp_down[]) and f32 arrays attn_norm, ffn_norm, optional q_norm,k_norm and q_bias,k_bias,v_bias."""
+    exp_gate[],exp_up[],exp_down[]) and f32 arrays attn_norm, ffn_norm, optional q_norm,k_norm, q_bias,k_bias,v_bias,
+    router_bias, sinks, post_attn_norm, post_ffn_norm and an int window."""
 
     def __init__(self, cfg, layers, final_norm, head, inv_freq):
         self.cfg = cfg
@@ -268,7 +289,8 @@ class OracleModel:
                 setattr(L, n, lw[n].c())
             self._keep.append(lw)
             L.window = int(lw.get("window", 0))
-            for n in ("attn_norm", "ffn_norm", "q_norm", "k_norm", "q_bias", "k_bias", "v_bias", "router_bias", "sinks"):
+            for n in ("attn_norm", "ffn_norm", "q_norm", "k_norm", "q_bias", "k_bias", "v_bias", "router_bias", "sinks",
+                      "post_attn_norm", "post_ffn_norm"):
                 if lw.get(n) is not None:
                     arr = f32(lw[n])
                     self._keep.append(arr)
@@ -289,7 +311,8 @@ class OracleModel:
                        cfg["vocab"], cfg["eps"], cfg["attn_scale"], cfg.get("softcap", 0.0), _p(self._inv),
                        nE, cfg.get("top_k", 0), int(cfg.get("norm_topk", 0)), cfg.get("exp_inter", 0),
                        int(cfg.get("kv_f16", 0)), self._layers, _p(self._fn), head.c(),
-                       int(cfg.get("router_sigmoid", 0)), float(cfg.get("router_scale", 0.0)), int(cfg.get("n_group", 0)), int(cfg.get("topk_group", 0)))
+                       int(cfg.get("router_sigmoid", 0)), float(cfg.get("router_scale", 0.0)), int(cfg.get("n_group", 0)), int(cfg.get("topk_group", 0)),
+                       int(cfg.get("norm_add_one", 0)), int(cfg.get("act_gelu_tanh", 0)), float(cfg.get("final_softcap", 0.0)))
 
     def new_cache(self, cap):
         return lib().or_cache_new(C.byref(self.m), cap)

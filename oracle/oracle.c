@@ -305,6 +305,23 @@ void or_swiglu(float *gate, const float *up, int n) {
     for (int i = 0; i < n; i++) gate[i] = or_silu(gate[i]) * up[i];
 }
 
+/* decoder/rmsnorm.go:229-234 (geluTanh): 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))) in f64, narrowed once. */
+float or_gelu_tanh(float x) {
+    const double c = 0.7978845608028654;
+    double x64 = x;
+    double inner = c * (x64 + 0.044715 * x64 * x64 * x64);
+    return (float)(0.5 * x64 * (1 + tanh(inner)));
+}
+
+void or_geglu(float *gate, const float *up, int n) {
+    for (int i = 0; i < n; i++) gate[i] = or_gelu_tanh(gate[i]) * up[i];
+}
+
+/* decoder/model_forward.go:259-266 (softcapParallel): the division in f32, tanh in f64, the product in f32. */
+void or_softcap_logits(float *logits, size_t n, float cap) {
+    for (size_t i = 0; i < n; i++) logits[i] = cap * (float)tanh((double)(logits[i] / cap));
+}
+
 /* decoder/mlp.go:370-410 (softmaxF32): f32 max, e=exp(f64(x-max)) stored f32, f64 sum, out*=f32(1/sum). */
 void or_softmax_f32(const float *x, int n, float *out) {
     if (n == 0) return;
@@ -987,7 +1004,7 @@ int or_decode_multi_step_traced(const or_model *m, int B, const float *emb, or_c
     memcpy(h, emb, sizeof(float) * (size_t)B * H);
     for (int l = 0; l < m->n_layers; l++) {
         const or_layer *lw = &m->layers[l];
-        or_rmsnorm(norm, h, lw->attn_norm, B, H, m->eps, 0);
+        or_rmsnorm(norm, h, lw->attn_norm, B, H, m->eps, m->norm_add_one);
         or_matmul(&lw->q, norm, B, q);
         or_matmul(&lw->k, norm, B, k);
         or_matmul(&lw->v, norm, B, v);
@@ -1013,12 +1030,15 @@ int or_decode_multi_step_traced(const or_model *m, int B, const float *emb, or_c
             or_attend_sinks(qb, ctx + (size_t)b * qDim, c->k[l], c->v[l], c->pos + 1, start, nH, nKV, hd, m->attn_scale, m->softcap, lw->sinks);
         }
         or_matmul(&lw->o, ctx, B, att);
+        /* Gemma 2 (decoder/program_cpu.go:286-312, the PostAttn slot): the branch output is normed before the residual add */
+        if (lw->post_attn_norm) or_rmsnorm(att, att, lw->post_attn_norm, B, H, m->eps, m->norm_add_one);
         for (size_t i = 0; i < (size_t)B * H; i++) h[i] += att[i];
-        or_rmsnorm(norm, h, lw->ffn_norm, B, H, m->eps, 0);
+        or_rmsnorm(norm, h, lw->ffn_norm, B, H, m->eps, m->norm_add_one);
         if (m->n_experts == 0) {
             or_matmul(&lw->gate, norm, B, gate);
             or_matmul(&lw->up, norm, B, up);
-            or_swiglu(gate, up, B * I);
+            if (m->act_gelu_tanh) or_geglu(gate, up, B * I);
+            else or_swiglu(gate, up, B * I);
             or_matmul(&lw->down, gate, B, att);
         } else {
             for (int b = 0; b < B; b++)
@@ -1026,11 +1046,13 @@ int or_decode_multi_step_traced(const or_model *m, int B, const float *emb, or_c
                         moe_idx_trace ? moe_idx_trace + ((size_t)b * m->n_layers + l) * m->top_k : NULL,
                         moe_wts_trace ? moe_wts_trace + ((size_t)b * m->n_layers + l) * m->top_k : NULL, replay);
         }
+        if (lw->post_ffn_norm) or_rmsnorm(att, att, lw->post_ffn_norm, B, H, m->eps, m->norm_add_one);
         for (size_t i = 0; i < (size_t)B * H; i++) h[i] += att[i];
     }
     for (int b = 0; b < B; b++) caches[b]->pos++;
-    or_rmsnorm(h, h, m->final_norm, B, H, m->eps, 0);
+    or_rmsnorm(h, h, m->final_norm, B, H, m->eps, m->norm_add_one);
     or_matmul(&m->head, h, B, logits);
+    if (m->final_softcap > 0) or_softcap_logits(logits, (size_t)B * m->vocab, (float)m->final_softcap);
     free(h);
     free(norm);
     free(att);

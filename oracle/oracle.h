@@ -134,6 +134,11 @@ void or_attend(const float *q, float *ctx, const float *keys, const float *vals,
 void or_attend_sinks(const float *q, float *ctx, const float *keys, const float *vals, int n_keys, int start,
                      int nH, int nKV, int hd, double scale, double softcap, const float *sinks);
 
+/* decoder/rmsnorm.go:229-234 (geluTanh) and the GeGLU gate; decoder/model_forward.go:259-266 (softcapParallel) */
+float or_gelu_tanh(float x);
+void or_geglu(float *gate, const float *up, int n);
+void or_softcap_logits(float *logits, size_t n, float cap);
+
 /* ---- the model and decodeMultiStep: decoder/cpu_batch.go:166-197, program_cpu_n.go:406-563, mlp.go:36-120 ---- */
 typedef struct {
     or_mat q, k, v, o, gate, up, down; /* dense FFN when n_experts==0 */
@@ -145,6 +150,8 @@ typedef struct {
     const float *router_bias;          /* [nE] or NULL: e_score_correction_bias, shifts the selection only */
     int window;                        /* > 0: this layer attends to the last `window` positions only (keys from pos-window+1) */
     const float *sinks;                /* [nH] or NULL: a learned logit per query head that joins the softmax's max and denominator */
+    const float *post_attn_norm;       /* [hidden] or NULL: Gemma 2's norm of the attention output before it joins the residual */
+    const float *post_ffn_norm;        /* [hidden] or NULL: the same for the FFN output */
 } or_layer;
 
 typedef struct {
@@ -159,6 +166,9 @@ typedef struct {
     int router_sigmoid;  /* 1: per-expert sigmoid scores instead of a softmax (DeepSeek / GLM) */
     double router_scale; /* routed_scaling_factor; 0 or 1 = none */
     int n_group, topk_group; /* > 1: group-limited selection */
+    int norm_add_one;     /* 1: every RMSNorm scales by (1 + w) (Gemma stores weights as deviations from one) */
+    int act_gelu_tanh;    /* 1: the gated FFN is GeGLU with the tanh-approximate GELU instead of SwiGLU */
+    double final_softcap; /* > 0: logits become cap * tanh(logit / cap) */
 } or_model;
 
 typedef struct {

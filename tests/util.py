@@ -41,12 +41,20 @@ def tiny_model(name, wrap=ob.WMat.from_f32):
     hd = cfg.get("head_dim") or H // nH
     theta = cfg.get("rope_parameters", {}).get("rope_theta", cfg.get("rope_theta", 10000.0))
     nE = cfg.get("num_experts", cfg.get("num_local_experts", 0))
+    gemma2 = cfg["model_type"] == "gemma2"
     layers = []
     for l in range(cfg["num_hidden_layers"]):
         p = "model.layers.%d." % l
         lw = {n: wrap(t[p + "self_attn.%s_proj.weight" % n]) for n in ("q", "k", "v", "o")}
         lw["attn_norm"] = t[p + "input_layernorm.weight"]
-        lw["ffn_norm"] = t[p + "post_attention_layernorm.weight"]
+        if gemma2:  # four norm slots: before and after each branch
+            lw["post_attn_norm"] = t[p + "post_attention_layernorm.weight"]
+            lw["ffn_norm"] = t[p + "pre_feedforward_layernorm.weight"]
+            lw["post_ffn_norm"] = t[p + "post_feedforward_layernorm.weight"]
+            if cfg["layer_types"][l] == "sliding_attention":
+                lw["window"] = cfg["sliding_window"]
+        else:
+            lw["ffn_norm"] = t[p + "post_attention_layernorm.weight"]
         if p + "self_attn.q_norm.weight" in t:
             lw["q_norm"] = t[p + "self_attn.q_norm.weight"]
             lw["k_norm"] = t[p + "self_attn.k_norm.weight"]
@@ -70,5 +78,15 @@ def tiny_model(name, wrap=ob.WMat.from_f32):
              n_experts=nE, top_k=cfg.get("num_experts_per_tok", 0),
              norm_topk=1 if (cfg["model_type"] == "mixtral" or cfg.get("norm_topk_prob")) else 0,
              exp_inter=cfg.get("moe_intermediate_size", cfg.get("intermediate_size", 0)) if nE else 0)
-    m = ob.OracleModel(c, layers, t["model.norm.weight"], wrap(t["lm_head.weight"]), inv_freq(hd, theta))
-    return m, t["model.embed_tokens.weight"], cfg
+    emb = t["model.embed_tokens.weight"]
+    if gemma2:
+        # decoder/model_forward.go:41-53: embedding rows scaled by float32(sqrt(hidden)); tied head; (1+w) norms; GeGLU;
+        # attention scale query_pre_attn_scalar^-0.5; attention and final-logit softcaps
+        c.update(attn_scale=float(cfg["query_pre_attn_scalar"]) ** -0.5, softcap=cfg["attn_logit_softcapping"],
+                 final_softcap=cfg["final_logit_softcapping"], norm_add_one=1, act_gelu_tanh=1)
+        head = wrap(emb)
+        emb = emb * np.float32(np.sqrt(np.float64(H)))
+    else:
+        head = wrap(t["lm_head.weight"])
+    m = ob.OracleModel(c, layers, t["model.norm.weight"], head, inv_freq(hd, theta))
+    return m, emb, cfg
