@@ -10,7 +10,7 @@ HSACO_PATH = os.path.join(HERE, "lib", "rocmdecode_gfx950.hsaco")
 
 RD_OK, RD_DECLINED = 0, 1
 PROJ = dict(q=0, k=1, v=2, o=3, gate=4, up=5, down=6, head=7)
-VEC = dict(attn_norm=0, ffn_norm=1, q_norm=2, k_norm=3, final_norm=4, router=5, qkv_bias=6, router_bias=7, attn_sinks=8)
+VEC = dict(attn_norm=0, ffn_norm=1, q_norm=2, k_norm=3, final_norm=4, router=5, qkv_bias=6, router_bias=7, attn_sinks=8, post_attn_norm=9, post_ffn_norm=10)
 WANT_LOGITS, WANT_ARGMAX = 1, 2
 
 EXPORTS = [
@@ -19,7 +19,7 @@ EXPORTS = [
     "rd_attn_ragged", "rd_moe_route", "rd_rmsnorm", "rd_rope", "rd_model_create", "rd_model_destroy",
     "rd_model_upload_q4k", "rd_model_upload_w8a8", "rd_model_upload_w4a8", "rd_model_upload_f32", "rd_model_finalize",
     "rd_kv_configure", "rd_kv_upload", "rd_kv_truncate", "rd_kv_reset", "rd_step_batch", "rd_forward",
-    "rd_last_moe_indices", "rd_model_upload_embedding", "rd_bench_steps", "rd_bench_profile", "rd_bench_attn_chain", "rd_moe_route_ex", "rd_attn_ragged_ex", "rd_model_set_router", "rd_model_set_window", "rd_bench_prefill", "rd_bench_class_count",
+    "rd_last_moe_indices", "rd_model_upload_embedding", "rd_bench_steps", "rd_bench_profile", "rd_bench_attn_chain", "rd_moe_route_ex", "rd_attn_ragged_ex", "rd_model_set_router", "rd_model_set_window", "rd_model_set_block", "rd_bench_prefill", "rd_bench_class_count",
     "rd_bench_class_name", "rd_bench_kernel", "rd_gateup_q4k_quant", "rd_moe_replay", "rd_bench_attn", "rd_step_ragged", "rd_prefill_last",
     "rd_kv_configure_typed", "rd_attn_ragged_i8", "rd_attn_ragged_rows", "rd_plan_attention", "rd_plan_gemm", "rd_step_batch_topk", "rd_last_logits", "rd_topk_rows", "rd_bench_attn_i8", "rd_step_ragged_draw", "rd_forward_no_logits",
     "rd_step_batch_draw", "rd_sample_rows", "rd_greedy_chain_start", "rd_greedy_chain_next", "rd_sample_chain_start",
@@ -337,6 +337,10 @@ class Model:
         if cfg.get("router_sigmoid") or cfg.get("router_scale") or cfg.get("n_group"):  # the router's variant (mlp.go:130-228)
             check(lib().rd_model_set_router(self.h, int(cfg.get("router_sigmoid", 0)), C.c_double(cfg.get("router_scale", 0.0)),
                                             int(cfg.get("n_group", 0)), int(cfg.get("topk_group", 0))), "rd_model_set_router")
+
+        if cfg.get("norm_add_one") or cfg.get("act_gelu_tanh") or cfg.get("final_softcap"):  # Gemma's block (rmsnorm.go:10-13,229-234)
+            check(lib().rd_model_set_block(self.h, int(cfg.get("norm_add_one", 0)), int(cfg.get("act_gelu_tanh", 0)),
+                                           C.c_float(cfg.get("final_softcap", 0.0))), "rd_model_set_block")
 
     def set_window(self, layer, window):
         check(lib().rd_model_set_window(self.h, layer, int(window)), "rd_model_set_window")

@@ -82,6 +82,8 @@ static const KName kNames[] = {
     {"rd_k_retile_w8a8_8", &Kernels::retile_w8a8_8},
     {"rd_k_retile_w4a8_8", &Kernels::retile_w4a8_8},
     {"rd_k_gemm8_q4k_gateup", &Kernels::gemm8_q4k_gateup},
+    {"rd_k_gemm8_q4k_gateup_gelu", &Kernels::gemm8_q4k_gateup_gelu},
+    {"rd_k_add_one", &Kernels::add_one},
     {"rd_k_moe_gemv_w4a8", &Kernels::moe_gemv_w4a8},
     {"rd_k_moe_gemv_w4a8_gateup", &Kernels::moe_gemv_w4a8_gateup},
     {"rd_k_retile_w4a8_gv", &Kernels::retile_w4a8_gv},

@@ -59,7 +59,7 @@ extern "C" void rd_model_destroy(rd_model *m) {
     (void)d->sync();
     for (auto &l : m->layers) {
         free_weight(d, &l.qkv), free_weight(d, &l.o), free_weight(d, &l.gateup), free_weight(d, &l.down);
-        for (void *p : {(void *)l.attn_norm, (void *)l.ffn_norm, (void *)l.q_norm, (void *)l.k_norm, (void *)l.qkv_bias, (void *)l.router, (void *)l.router_bias, (void *)l.sinks, l.exp_gateup, l.exp_down,
+        for (void *p : {(void *)l.post_attn_norm, (void *)l.post_ffn_norm, (void *)l.attn_norm, (void *)l.ffn_norm, (void *)l.q_norm, (void *)l.k_norm, (void *)l.qkv_bias, (void *)l.router, (void *)l.router_bias, (void *)l.sinks, l.exp_gateup, l.exp_down,
                         (void *)l.Kp, (void *)l.Vp, (void *)l.Ksc, (void *)l.Vsc})
             d->release(p);
     }
@@ -327,12 +327,18 @@ extern "C" int rd_model_upload_f32(rd_model *m, int layer, int which, const floa
         case RD_VEC_ROUTER: slot = &l.router, want = (size_t)c.n_experts * c.hidden; break;
         case RD_VEC_ROUTER_BIAS: slot = &l.router_bias, want = (size_t)c.n_experts; break;
         case RD_VEC_ATTN_SINKS: slot = &l.sinks, want = (size_t)c.n_heads; break;
+        case RD_VEC_POST_ATTN_NORM: slot = &l.post_attn_norm, want = (size_t)c.hidden; break;
+        case RD_VEC_POST_FFN_NORM: slot = &l.post_ffn_norm, want = (size_t)c.hidden; break;
         default: rd_set_error("unknown vector %d", which); return RD_ERR_ARG;
         }
     }
     if (n != want) {
         rd_set_error("vector %d: got %zu values, want %zu", which, n, want);
         return RD_ERR_ARG;
+    }
+    if (m->finalized) { // the (1 + w) pass has run over the norm weights: a later upload would skip it
+        rd_set_error("model already finalized");
+        return RD_ERR_STATE;
     }
     if (!*slot) RC(alloc_f32(d, slot, n));
     RC(d->h2d(*slot, v, sizeof(float) * n));
@@ -351,6 +357,21 @@ extern "C" int rd_model_set_router(rd_model *m, int sigmoid, double scale, int n
         return RD_DECLINED;
     }
     m->router_sigmoid = sigmoid ? 1 : 0, m->router_scale = (float)scale, m->n_group = n_group > 1 ? n_group : 0, m->topk_group = topk_group;
+    return RD_OK;
+}
+
+// The block's family knobs (Gemma; backend/cuda/resident.go:549-565 finalSoftcap, act, addOneArg), before rd_model_finalize.
+extern "C" int rd_model_set_block(rd_model *m, int norm_add_one, int act, float final_softcap) {
+    if (!m || (act != RD_ACT_SILU && act != RD_ACT_GELU_TANH) || !(final_softcap >= 0.f)) return RD_ERR_ARG;
+    if (m->finalized) {
+        rd_set_error("model already finalized");
+        return RD_ERR_STATE;
+    }
+    if (act != RD_ACT_SILU && m->desc.n_experts > 0) {
+        rd_set_error("rocm resident declines: a GeGLU mixture-of-experts block");
+        return RD_DECLINED;
+    }
+    m->norm_add_one = norm_add_one ? 1 : 0, m->act = act, m->final_softcap = final_softcap;
     return RD_OK;
 }
 
@@ -419,6 +440,10 @@ extern "C" int rd_model_finalize(rd_model *m) {
             rd_set_error("layer %d is missing tensors", i);
             return RD_ERR_STATE;
         }
+        if (c.n_experts > 0 && (l.post_attn_norm || l.post_ffn_norm)) {
+            rd_set_error("rocm resident declines: post-branch norms around a mixture-of-experts block");
+            return RD_DECLINED;
+        }
         pf = std::max({pf, gemm_partial_floats(l.qkv), gemm_partial_floats(l.o), gemm_partial_floats(l.gateup), gemm_partial_floats(l.down)});
     }
     if (m->head.kind < 0 || !m->final_norm) {
@@ -470,6 +495,20 @@ extern "C" int rd_model_finalize(rd_model *m) {
     RC(topk_scratch_alloc(d, (int)R, c.vocab, &m->topk_scratch));
     RC(d->alloc((void **)&m->topk_z, sizeof(double) * R));
     for (auto &e : m->stage_ev) HIPCHK(EventCreate(&e));
+    if (m->norm_add_one && !m->ones_added) {
+        // Gemma stores every RMSNorm weight as its deviation from one; the norm scales by f32(1 + w) (decoder/rmsnorm.go:62-75),
+        // so the sum is formed once here and the kernels multiply by it as they do by a plain weight
+        auto bump = [&](float *w, int n) -> int {
+            return w ? d->launch(d->k.add_one, (unsigned)((n + 255) / 256), 1, 1, 256, w, n) : RD_OK;
+        };
+        for (LayerW &l : m->layers) {
+            for (float *w : {l.attn_norm, l.ffn_norm, l.post_attn_norm, l.post_ffn_norm}) RC(bump(w, H));
+            RC(bump(l.q_norm, c.head_dim));
+            RC(bump(l.k_norm, c.head_dim));
+        }
+        RC(bump(m->final_norm, H));
+        m->ones_added = true;
+    }
     m->finalized = true;
     return d->sync();
 }
@@ -656,14 +695,15 @@ static void panel_kinds_of(const DevWeight &w, int *kA, int *kB) {
 }
 
 // foldW: P holds an MoE layer's down-projection rows and foldW their weights (see the kernel); else split-K partial sums.
+// postW: the norm of the pending contribution itself (Gemma 2's post-attention / post-feed-forward norm), or null.
 static int add_norm_quant(rd_model *m, int B, const float *P, int splits, const float *w, const DevWeight &next, void *Xp, float *norm_out,
-                          const float *foldW = nullptr) {
+                          const float *foldW = nullptr, const float *postW = nullptr) {
     rd_device *d = m->d;
     Scope s(m, KC_ADD_NORM);
     int kA, kB;
     panel_kinds_of(next, &kA, &kB);
     return d->launch(d->k.add_rmsnorm_quant, (unsigned)B, 1, 1, 1024, m->h, P, splits, w, m->desc.rms_eps, m->desc.hidden, Xp, kA, norm_out,
-                     kB >= 0 ? m->XpA2 : (void *)nullptr, kB, m->pStride, m->xpAStride, m->xpAStride, foldW);
+                     kB >= 0 ? m->XpA2 : (void *)nullptr, kB, m->pStride, m->xpAStride, m->xpAStride, foldW, P ? postW : (const float *)nullptr);
 }
 
 // One GEMM, or for a group one GEMM per member into column ranges of the same P[split][32][N], all with the group's split
@@ -881,7 +921,7 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
     }
     // pending residual contribution: split-K partials of the previous block's last GEMM, or (resW set) an MoE layer's
     // down-projection rows and their weights, folded by the kernel that adds them
-    const float *resP = nullptr, *resW = nullptr;
+    const float *resP = nullptr, *resW = nullptr, *resPost = nullptr; // resPost: the pending contribution's own norm, if any
     int resSplits = 0;
     if (std::any_of(m->layers.begin(), m->layers.end(), [&](const LayerW &l) { return qkv_fusable(m, l); })) {
         Scope s(m, KC_ROPE_STORE);
@@ -890,7 +930,7 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
     for (int li = 0; li < c.n_layers; li++) {
         LayerW &l = m->layers[(size_t)li];
         GemmPlan plan;
-        RC(add_norm_quant(m, B, resP, resSplits, l.attn_norm, l.qkv, m->XpA, nullptr, resW));
+        RC(add_norm_quant(m, B, resP, resSplits, l.attn_norm, l.qkv, m->XpA, nullptr, resW, resPost));
         if (qkv_fusable(m, l)) {
             Scope s(m, KC_GEMM_QKV); // projection, bias, RoPE and the KV store in one launch (M-tiles of 32 rows as grid.z)
             const DevWeight &w = l.qkv;
@@ -932,10 +972,10 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
             RC(launch_gemm_wide(d, l.o, m->XpB, m->xpBStride, m->P, m->pStride, B, &plan));
         }
         if (c.n_experts == 0) {
-            RC(add_norm_quant(m, B, m->P, plan.splits, l.ffn_norm, l.gateup, m->XpA, nullptr));
+            RC(add_norm_quant(m, B, m->P, plan.splits, l.ffn_norm, l.gateup, m->XpA, nullptr, nullptr, l.post_attn_norm));
             if (gateup_fusable(c, l.gateup) && !getenv("ROCMDECODE_NO_FUSED_GATEUP")) {
                 Scope s(m, KC_GEMM_GATEUP); // gate|up GEMM + SwiGLU + quantization in one launch (M-tiles of 32 rows as grid.z)
-                RC(d->launch(d->k.gemm8_q4k_gateup, (unsigned)(c.inter / 32), 1, (unsigned)((B + 31) / 32), GATEUP_THREADS, (const void *)l.gateup.tiled,
+                RC(d->launch(m->act == RD_ACT_GELU_TANH ? d->k.gemm8_q4k_gateup_gelu : d->k.gemm8_q4k_gateup, (unsigned)(c.inter / 32), 1, (unsigned)((B + 31) / 32), GATEUP_THREADS, (const void *)l.gateup.tiled,
                              (const void *)m->XpA, m->XpB, panel_kind_for(l.down), c.inter, H / 256, B, m->xpAStride, m->xpBStride));
             } else {
                 {
@@ -947,30 +987,30 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
                 }
                 Scope s(m, KC_SWIGLU);
                 RC(d->launch(d->k.swiglu_quant, (unsigned)((c.inter + 1023) / 1024), (unsigned)B, 1, 256, (const float *)m->P, plan.splits, c.inter,
-                             m->XpB, panel_kind_for(l.down), (float *)nullptr, m->pStride, m->xpBStride));
+                             m->XpB, panel_kind_for(l.down), (float *)nullptr, m->pStride, m->xpBStride, m->act));
             }
             {
                 Scope s(m, KC_GEMM_DOWN);
                 RC(launch_gemm_wide(d, l.down, m->XpB, m->xpBStride, m->P, m->pStride, B, &plan));
             }
-            resP = m->P, resSplits = plan.splits, resW = nullptr;
+            resP = m->P, resSplits = plan.splits, resW = nullptr, resPost = l.post_ffn_norm;
         } else {
             {
                 Scope s(m, KC_ADD_NORM);
                 RC(d->launch(d->k.add_rmsnorm_quant, (unsigned)B, 1, 1, 1024, m->h, (const float *)m->P, plan.splits, (const float *)l.ffn_norm,
                              c.rms_eps, H, m->XpA, (int)PANEL_ROW8, m->normed, (void *)nullptr, -1, m->pStride, m->xpAStride, m->xpAStride,
-                             (const float *)nullptr));
+                             (const float *)nullptr, (const float *)nullptr));
             }
             RC(moe_ffn(m, B, li, l));
             if (c.top_k <= MOE_FOLD_FUSED_MAX)
-                resP = m->moe_dn, resSplits = c.top_k, resW = m->moe_wgt;
+                resP = m->moe_dn, resSplits = c.top_k, resW = m->moe_wgt, resPost = nullptr;
             else
-                resP = m->moe_out, resSplits = 1, resW = nullptr;
+                resP = m->moe_out, resSplits = 1, resW = nullptr, resPost = nullptr;
         }
     }
     if (want & (RD_WANT_LOGITS | RD_WANT_ARGMAX)) {
         GemmPlan plan;
-        RC(add_norm_quant(m, B, resP, resSplits, m->final_norm, m->head, m->XpA, nullptr, resW));
+        RC(add_norm_quant(m, B, resP, resSplits, m->final_norm, m->head, m->XpA, nullptr, resW, resPost));
         {
             Scope s(m, KC_GEMM_HEAD);
             RC(launch_gemm_wide(d, m->head, m->XpA, m->xpAStride, m->P, m->pStride, B, &plan));
@@ -979,7 +1019,8 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
             Scope s(m, KC_ARGMAX);
             int nChunks = (c.vocab + 4095) / 4096;
             RC(d->launch(d->k.argmax_rows, (unsigned)nChunks, (unsigned)B, 1, 256, (const float *)m->P, plan.splits, c.vocab, m->cand_v, m->cand_i,
-                         (want & RD_WANT_LOGITS) ? m->logits : (float *)nullptr, (const int *)(m->step_draws ? m->rowDraw : nullptr), m->pStride));
+                         (want & RD_WANT_LOGITS) ? m->logits : (float *)nullptr, (const int *)(m->step_draws ? m->rowDraw : nullptr), m->pStride,
+                         m->final_softcap));
             if (want & RD_WANT_ARGMAX) RC(d->launch(d->k.argmax_final, (unsigned)B, 1, 1, 64, (const float *)m->cand_v, (const int *)m->cand_i, nChunks, m->ids));
         }
     }

@@ -20,6 +20,7 @@ struct LayerW {
     DevWeight qkv, o, gateup, down;
     PendingMat pend[RD_PROJ_COUNT];
     float *attn_norm = nullptr, *ffn_norm = nullptr, *q_norm = nullptr, *k_norm = nullptr;
+    float *post_attn_norm = nullptr, *post_ffn_norm = nullptr; // optional: Gemma 2's norms of a branch's output before the residual add
     float *qkv_bias = nullptr; // optional: q bias, k bias, v bias end to end
     float *router_bias = nullptr; // optional [nE]: e_score_correction_bias (selection only)
     float *sinks = nullptr;       // optional [nH]: attention sinks
@@ -56,6 +57,9 @@ struct rd_model {
     int router_sigmoid = 0, n_group = 0, topk_group = 0;
     float router_scale = 0.f;
     int window = 0; // the one window length the model's sliding-window layers share (0: none has one)
+    int norm_add_one = 0, act = 0; // (1 + w) norm weights; the gated FFN's activation (RD_ACT_*)
+    float final_softcap = 0.f;     // > 0: logits become cap * tanh(logit / cap)
+    bool ones_added = false;       // the (1 + w) pass over the norm weights has run
 
     // KV
     int slots = 0, ctx_cap = 0, blocks_per_slot = 0;

@@ -110,12 +110,15 @@ extern "C" __global__ void rd_k_reduce_splits(const float *__restrict__ P, float
 // foldW != NULL: the pending contribution is an MoE layer's output instead, folded here from the experts' down-projection rows:
 // P is [(row*k + rank)][H] with k = splits (<= 8), foldW is [row][k], and the row's contribution is the sum over ranks, in rank
 // order from zero, of foldW * P (multiply, then add: decoder/mlp.go:100-103 addScaled).
+// postW != NULL (split-K contributions only): the summed contribution x is replaced by (x * invx) * postW, its own RMSNorm with
+// the same eps, before the add: Gemma 2's post-attention / post-feed-forward norm (decoder/program_cpu.go:286-312).
 extern "C" __global__ __launch_bounds__(1024) void rd_k_add_rmsnorm_quant(float *__restrict__ h, const float *__restrict__ P, int splits,
                                                                           const float *__restrict__ w, float eps, int H,
                                                                           uint8_t *__restrict__ Xp, int kind, float *__restrict__ norm_out,
                                                                           uint8_t *__restrict__ Xp2, int kind2, size_t pStride, size_t xpStride,
-                                                                          size_t xp2Stride, const float *__restrict__ foldW) {
-    __shared__ double red[16];
+                                                                          size_t xp2Stride, const float *__restrict__ foldW,
+                                                                          const float *__restrict__ postW) {
+    __shared__ double red[16], redPost[16];
     const int m = blockIdx.x, t = threadIdx.x, nv = H >> 2;
     // rows beyond 32 are further M-tiles: their partial sums and panels sit pStride floats / xpStride bytes further on
     const int mt = m >> 5, mr = m & 31;
@@ -183,6 +186,26 @@ extern "C" __global__ __launch_bounds__(1024) void rd_k_add_rmsnorm_quant(float 
                         a[i].z = __fadd_rn(a[i].z, b[i][j].z), a[i].w = __fadd_rn(a[i].w, b[i][j].w);
                     }
         }
+        if (postW) { // the branch output goes through its own RMSNorm before it joins the residual
+            double sp = 0;
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+                if (on[i]) sp += (double)a[i].x * a[i].x + (double)a[i].y * a[i].y + (double)a[i].z * a[i].z + (double)a[i].w * a[i].w;
+            sp = wave_sum64_d(sp);
+            if ((t & 63) == 0) redPost[t >> 6] = sp;
+            __syncthreads();
+            sp = 0;
+#pragma unroll
+            for (int i = 0; i < 16; i++) sp += redPost[i];
+            const float invP = (float)(1.0 / sqrt(sp / (double)H + (double)eps));
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+                if (on[i]) {
+                    const float4_t pw = *(const float4_t *)(postW + 4 * (t + i * 1024));
+                    a[i].x = __fmul_rn(__fmul_rn(a[i].x, invP), pw.x), a[i].y = __fmul_rn(__fmul_rn(a[i].y, invP), pw.y);
+                    a[i].z = __fmul_rn(__fmul_rn(a[i].z, invP), pw.z), a[i].w = __fmul_rn(__fmul_rn(a[i].w, invP), pw.w);
+                }
+        }
 #pragma unroll
         for (int i = 0; i < 2; i++)
             if (on[i]) {
@@ -214,9 +237,9 @@ extern "C" __global__ __launch_bounds__(1024) void rd_k_add_rmsnorm_quant(float 
 }
 
 // gate/up partials P[s][32][2I] -> act = silu(gate)*up (decoder/rmsnorm.go:204-207: silu in f64) -> per-32 quant -> panels.
-// Grid (ceil(I/1024), M), 256 threads, four consecutive columns per thread. I % 32 == 0.
+// Grid (ceil(I/1024), M), 256 threads, four consecutive columns per thread. I % 32 == 0. act 1: geluTanh(gate)*up (GeGLU).
 extern "C" __global__ __launch_bounds__(256) void rd_k_swiglu_quant(const float *__restrict__ P, int splits, int I, uint8_t *__restrict__ Xp,
-                                                                    int kind, float *__restrict__ act_out, size_t pStride, size_t xpStride) {
+                                                                    int kind, float *__restrict__ act_out, size_t pStride, size_t xpStride, int act) {
     const int row = blockIdx.y, m = row & 31, n0 = (blockIdx.x * 256 + threadIdx.x) * 4;
     P += (size_t)(row >> 5) * pStride; // M-tile of this row
     Xp += (size_t)(row >> 5) * xpStride;
@@ -232,7 +255,7 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_swiglu_quant(const float 
         }
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            a[i] = __fmul_rn(silu_f64(g[i]), u[i]);
+            a[i] = __fmul_rn(gate_act(g[i], act), u[i]);
         }
         if (act_out) *(float4_t *)(act_out + (size_t)row * I + n0) = (float4_t){a[0], a[1], a[2], a[3]};
     }

@@ -157,6 +157,18 @@ __device__ __forceinline__ float silu_f64(float g) {
     return (float)q;
 }
 
+// The tanh-approximate GELU of Gemma's GeGLU (decoder/rmsnorm.go:229-234 geluTanh): f32(0.5 x (1 + tanh(c (x + 0.044715 x^3)))),
+// every operation in f64 in goinfer's order, narrowed once. The products and sums are kept apart (no fused multiply-add): the
+// reference rounds each of them.
+__device__ __forceinline__ float gelu_tanh_f64(float g) {
+    const double x = (double)g;
+    const double cube = __dmul_rn(__dmul_rn(__dmul_rn(0.044715, x), x), x);
+    const double inner = __dmul_rn(0.7978845608028654, __dadd_rn(x, cube));
+    return (float)__dmul_rn(__dmul_rn(0.5, x), __dadd_rn(1.0, tanh(inner)));
+}
+// The gated FFN's activation: 0 = silu (SwiGLU), 1 = tanh-approximate GELU (GeGLU).
+__device__ __forceinline__ float gate_act(float g, int act) { return act ? gelu_tanh_f64(g) : silu_f64(g); }
+
 // Where element t (0..255) of a super-block goes inside a Q4_K activation panel, for batch row m.
 // Sub-block j=t/32 belongs to nibble pair p=j/2; lane half h=p/2 owns pairs 2h,2h+1; its 16 code words are the
 // 16 MFMA steps. Word s holds bytes e0..e0+3 (e0=4*(s%8)): the unpack yields

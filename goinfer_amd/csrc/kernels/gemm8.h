@@ -397,7 +397,7 @@ RD_GEMM8_KERNEL(rd_k_gemm8_w4a8_kw8, W4A8Traits8, 8, 1)
 // half-wave holds the 32 columns of one batch row, which is exactly one activation group of the down projection, so
 // silu(gate)*up (silu in f64, decoder/rmsnorm.go:204-207) is quantized where it sits and written in the layout the down projection reads.
 // The K loop, its wave ranges and the fold are those of the plain kernel with the same KW: the sums are the same bits.
-template <class T, int KW, int NR = 16>
+template <class T, int KW, int NR = 16, int ACT = 0>
 __device__ __forceinline__ void gemm8_gateup_body(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ A8, uint8_t *__restrict__ XpOut, int outKind,
                                                   int I, int nKB, int M, float *lds) {
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
@@ -419,7 +419,7 @@ __device__ __forceinline__ void gemm8_gateup_body(const uint8_t *__restrict__ Wt
         const int r = wave * RPW + j;
         const int m = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
         if (r >= NR) continue; // batch rows past M: nothing folded, nothing to store
-        const float a = __fmul_rn(silu_f64(lds[r * 64 + lane]), lds[(16 + r) * 64 + lane]);
+        const float a = __fmul_rn(gate_act(lds[r * 64 + lane], ACT), lds[(16 + r) * 64 + lane]);
         const Quant1 q = quant_one(a);
         if (outKind == RD_PANEL_A8) {
             // four neighbouring lanes hold four consecutive elements of the row: their codes leave as one word
@@ -432,19 +432,22 @@ __device__ __forceinline__ void gemm8_gateup_body(const uint8_t *__restrict__ Wt
     }
 }
 
-// grid.z: M-tiles of 32 rows, a8Stride / outStride bytes apart in the activations read and written.
-extern "C" __global__ __launch_bounds__(256) void rd_k_gemm8_q4k_gateup(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ A8,
-                                                                         uint8_t *__restrict__ XpOut, int outKind, int I, int nKB, int M, size_t a8Stride,
-                                                                         size_t outStride) {
-    __shared__ float lds[2 * 1024];
-    A8 += (size_t)blockIdx.z * a8Stride, XpOut += (size_t)blockIdx.z * outStride, M = min(32, M - 32 * (int)blockIdx.z);
-    if (M <= 8)
-        gemm8_gateup_body<Q4K8Traits, 2, 4>(Wt, A8, XpOut, outKind, I, nKB, M, lds);
-    else if (M <= 16)
-        gemm8_gateup_body<Q4K8Traits, 2, 8>(Wt, A8, XpOut, outKind, I, nKB, M, lds);
-    else
-        gemm8_gateup_body<Q4K8Traits, 2, 16>(Wt, A8, XpOut, outKind, I, nKB, M, lds);
-}
+// grid.z: M-tiles of 32 rows, a8Stride / outStride bytes apart in the activations read and written. The _gelu kernel is the
+// same with Gemma's geluTanh(gate)*up instead of silu(gate)*up.
+#define RD_GEMM8_GATEUP_KERNEL(NAME, ACT)                                                                                                         \
+    extern "C" __global__ __launch_bounds__(256) void NAME(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ A8, uint8_t *__restrict__ XpOut, \
+                                                           int outKind, int I, int nKB, int M, size_t a8Stride, size_t outStride) {            \
+        __shared__ float lds[2 * 1024];                                                                                                           \
+        A8 += (size_t)blockIdx.z * a8Stride, XpOut += (size_t)blockIdx.z * outStride, M = min(32, M - 32 * (int)blockIdx.z);                      \
+        if (M <= 8)                                                                                                                               \
+            gemm8_gateup_body<Q4K8Traits, 2, 4, ACT>(Wt, A8, XpOut, outKind, I, nKB, M, lds);                                                     \
+        else if (M <= 16)                                                                                                                         \
+            gemm8_gateup_body<Q4K8Traits, 2, 8, ACT>(Wt, A8, XpOut, outKind, I, nKB, M, lds);                                                     \
+        else                                                                                                                                      \
+            gemm8_gateup_body<Q4K8Traits, 2, 16, ACT>(Wt, A8, XpOut, outKind, I, nKB, M, lds);                                                    \
+    }
+RD_GEMM8_GATEUP_KERNEL(rd_k_gemm8_q4k_gateup, 0)
+RD_GEMM8_GATEUP_KERNEL(rd_k_gemm8_q4k_gateup_gelu, 1)
 
 // ---------------- q|k|v projection with bias, RoPE and the KV store in its epilogue ----------------
 // The plain kernel with one split and, instead of the store of the sums, what rd_k_qkv_rope_store does to them (same arithmetic,

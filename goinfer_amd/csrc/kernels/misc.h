@@ -60,7 +60,7 @@ __device__ __forceinline__ float gumbel_noise(uint32_t h) {
 // draw hi, 0), key seed), and a thread's four consecutive entries are exactly one Philox call.
 extern "C" __global__ __launch_bounds__(256) void rd_k_argmax_rows(const float *__restrict__ P, int splits, int N, float *__restrict__ cand_v,
                                                                    int *__restrict__ cand_i, float *__restrict__ logits_out,
-                                                                   const int *__restrict__ rowDraw, size_t pStride) {
+                                                                   const int *__restrict__ rowDraw, size_t pStride, float softcap) {
     __shared__ float bv[4];
     __shared__ int bi[4];
     const int m = blockIdx.y, t = threadIdx.x, nChunks = gridDim.x, mr = m & 31;
@@ -78,6 +78,10 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_argmax_rows(const float *
             for (int s = 1; s < splits; s++) {
                 float4_t b = *(const float4_t *)(P + ((size_t)s * 32 + mr) * N + n0);
                 a.x = __fadd_rn(a.x, b.x), a.y = __fadd_rn(a.y, b.y), a.z = __fadd_rn(a.z, b.z), a.w = __fadd_rn(a.w, b.w);
+            }
+            if (softcap > 0.f) { // decoder/model_forward.go:259-266: cap * f32(tanh(f64(logit / cap))), before anything reads the logits
+#pragma unroll
+                for (int e = 0; e < 4; e++) a[e] = mul_rounded(softcap, (float)tanh((double)__fdiv_rn(a[e], softcap)));
             }
             if (logits_out) *(float4_t *)(logits_out + (size_t)m * N + n0) = a;
             if (gumbel) {
@@ -104,6 +108,12 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_argmax_rows(const float *
         cand_v[m * nChunks + blockIdx.x] = best;
         cand_i[m * nChunks + blockIdx.x] = idx;
     }
+}
+
+// w[i] = 1 + w[i]: a norm weight stored as its deviation from one (Gemma; decoder/rmsnorm.go:62-75 scales by f32(1 + w)).
+extern "C" __global__ void rd_k_add_one(float *__restrict__ w, int n) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) w[i] = __fadd_rn(1.f, w[i]);
 }
 
 // Folds a row's chunk candidates. No comparable candidate (every key -Inf or NaN: a fully masked row) gives index 0, which

@@ -39,7 +39,8 @@ typedef struct rd_model rd_model;
 enum { RD_PROJ_Q = 0, RD_PROJ_K, RD_PROJ_V, RD_PROJ_O, RD_PROJ_GATE, RD_PROJ_UP, RD_PROJ_DOWN, RD_PROJ_HEAD, RD_PROJ_COUNT };
 /* f32 vectors. RD_VEC_QKV_BIAS (optional): the q, k and v projection biases end to end, (n_heads + 2 n_kv_heads) * head_dim values,
  * added right after the projections (Qwen2; decoder/attention.go:12-34 addBias, program_cpu_n.go:470-476). */
-enum { RD_VEC_ATTN_NORM = 0, RD_VEC_FFN_NORM, RD_VEC_Q_NORM, RD_VEC_K_NORM, RD_VEC_FINAL_NORM, RD_VEC_ROUTER, RD_VEC_QKV_BIAS, RD_VEC_ROUTER_BIAS, RD_VEC_ATTN_SINKS };
+enum { RD_VEC_ATTN_NORM = 0, RD_VEC_FFN_NORM, RD_VEC_Q_NORM, RD_VEC_K_NORM, RD_VEC_FINAL_NORM, RD_VEC_ROUTER, RD_VEC_QKV_BIAS, RD_VEC_ROUTER_BIAS, RD_VEC_ATTN_SINKS,
+       RD_VEC_POST_ATTN_NORM, RD_VEC_POST_FFN_NORM };
 /* rd_step_batch `want` */
 enum { RD_WANT_LOGITS = 1, RD_WANT_ARGMAX = 2 };
 
@@ -157,12 +158,22 @@ int rd_model_upload_q6k(rd_model *m, int layer, int proj, const void *blocks, in
 int rd_model_upload_w8a8(rd_model *m, int layer, int proj, const int8_t *q, const float *row_scale, int N, int K);
 /* canonical int4 nibbles + binary16 group-32 scales (WeightMat.Int4F16, decoder/weightmat.go:904); expert < 0 = dense */
 int rd_model_upload_w4a8(rd_model *m, int layer, int proj, int expert, const uint8_t *nib, const uint16_t *s16, int N, int K);
-/* norms, router; RD_VEC_ROUTER_BIAS: a layer's e_score_correction_bias [n_experts]; RD_VEC_ATTN_SINKS: its attention sinks [n_heads] */
+/* norms, router; RD_VEC_ROUTER_BIAS: a layer's e_score_correction_bias [n_experts]; RD_VEC_ATTN_SINKS: its attention sinks [n_heads];
+ * RD_VEC_POST_ATTN_NORM / RD_VEC_POST_FFN_NORM [hidden]: Gemma 2's norm of the attention / feed-forward output before it joins the
+ * residual (decoder/program_cpu.go:286-312, the PostAttn and PostMLP slots; backend/cuda/backend.go:86). Before rd_model_finalize. */
 int rd_model_upload_f32(rd_model *m, int layer, int which, const float *v, size_t n);
 /* The router's variant, decoder/mlp.go:130-228 (routeExperts, groupLimit); before rd_model_finalize. sigmoid: per-expert sigmoid
  * scores (DeepSeek / GLM) instead of a softmax; scale: routed_scaling_factor (0 or 1 = none); n_group > 1: group-limited
  * selection among the topk_group best of n_group contiguous groups (at most 32 groups, which must divide the experts). */
 int rd_model_set_router(rd_model *m, int sigmoid, double scale, int n_group, int topk_group);
+/* The block's family knobs, as backend/cuda/resident.go:549-565,2882-2886 holds them (addOneArg, act, finalSoftcap); before
+ * rd_model_finalize. norm_add_one: every RMSNorm weight is stored as its deviation from one and scales by f32(1 + w)
+ * (Architecture.RMSAddOne, decoder/rmsnorm.go:10-13,62-75; the sum is formed once at rd_model_finalize). act: the gated FFN's
+ * activation, RD_ACT_SILU (SwiGLU) or RD_ACT_GELU_TANH (Gemma's GeGLU, decoder/rmsnorm.go:229-234; dense FFN only). final_softcap
+ * > 0: logits become cap * tanh(logit / cap) (decoder/model_forward.go:259-266) before the argmax, the draws, the top-K and the
+ * copy to the host. */
+enum { RD_ACT_SILU = 0, RD_ACT_GELU_TANH = 1 };
+int rd_model_set_block(rd_model *m, int norm_add_one, int act, float final_softcap);
 /* A sliding-window layer (decoder/kvcache.go:1063-1068 WindowStart): its rows read the last `window` positions only. Before
  * rd_model_finalize. The windowed layers of a model share one length (RD_DECLINED otherwise); the cache keeps every position. */
 int rd_model_set_window(rd_model *m, int layer, int window);

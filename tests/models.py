@@ -85,7 +85,8 @@ class Pair:
             return ob.WMat(ob.OR_W8A8, N, K, q, sc, act_group=32)
 
         def vec(layer, which, n):
-            v = synth.normal(nxt(), n, 0.02, 1.0)
+            # norm weights around one; stored as the deviation from one where the model scales by (1 + w)
+            v = synth.normal(nxt(), n, 0.02, 0.0 if cfg.get("norm_add_one") else 1.0)
             if self.gpu:
                 self.gpu.upload_f32(layer, which, v)
             return v
@@ -94,6 +95,8 @@ class Pair:
         for l in range(cfg["n_layers"]):
             lw = dict(q=mat(l, "q", qd, H), k=mat(l, "k", kvd, H), v=mat(l, "v", kvd, H), o=mat(l, "o", H, qd))
             lw["attn_norm"], lw["ffn_norm"] = vec(l, "attn_norm", H), vec(l, "ffn_norm", H)
+            if cfg.get("post_norms"):  # Gemma 2: each branch's output is normed before it joins the residual
+                lw["post_attn_norm"], lw["post_ffn_norm"] = vec(l, "post_attn_norm", H), vec(l, "post_ffn_norm", H)
             if cfg.get("qk_norm"):
                 lw["q_norm"], lw["k_norm"] = vec(l, "q_norm", hd), vec(l, "k_norm", hd)
             if cfg.get("attn_sinks"):  # one learned logit per query head joining the softmax (decoder/attention.go:305-322)
@@ -125,7 +128,7 @@ class Pair:
                 lw["exp_up"] = [mat(l, "up", EI, H, e) for e in range(nE)]
                 lw["exp_down"] = [mat(l, "down", H, EI, e) for e in range(nE)]
             layers.append(lw)
-        fn = synth.normal(nxt(), H, 0.02, 1.0)
+        fn = synth.normal(nxt(), H, 0.02, 0.0 if cfg.get("norm_add_one") else 1.0)
         if self.gpu:
             self.gpu.upload_f32(-1, "final_norm", fn)
         head = mat(-1, "head", V, H)

@@ -115,3 +115,63 @@ def test_moe_model_with_deepseek_style_router(dev):
     _, _, (agree, total, diverged) = check(Pair(cfg, seed=41, dev=dev, slots=8), [list(rng.integers(0, 512, n)) for n in (2, 20)], steps=4)
     assert agree >= 0.9 * total, (agree, total)
     assert not all(diverged)
+
+
+GEMMA2 = dict(window=24, post_norms=1, norm_add_one=1, act_gelu_tanh=1, final_softcap=30.0)
+
+
+@pytest.mark.parametrize("hidden,heads", [(256, 4), (384, 6)])
+def test_gemma2_style_block(dev, hidden, heads):
+    """Gemma 2's block through the step against the oracle (which reproduces the reference's gemma2-tiny golden): (1 + w) norms
+    before and after both branches, GeGLU, attention softcap 50, a window on the even layers, final-logit softcap 30. hidden 256 runs
+    the fused gate|up kernel, hidden 384 the int8-row lane with the separate activation kernel."""
+    cfg = dict(dense_cfg(n_layers=4, hidden=hidden, n_heads=heads, n_kv=2, head_dim=64, inter=512, vocab=512, theta=1e4, eps=1e-6, softcap=50.0), **GEMMA2)
+    cfg["attn_scale"] = 144.0 ** -0.5  # query_pre_attn_scalar, not head_dim
+    rng = np.random.default_rng(61)
+    check(Pair(cfg, seed=71, dev=dev, slots=8), [list(rng.integers(0, 512, n)) for n in (3, 30, 70)], steps=4)
+
+
+def test_gemma2_knobs_are_not_ignored(dev):
+    """Each knob of the block changes the GPU's answer: the same weights without it give different logits. (The (1 + w) scale is
+    not in the list: the helper stores the same weights as deviations from one when it is on, so ignoring it on the GPU would
+    scale every norm by about 0.02 and fail the comparison with the oracle above.)"""
+    cfg = dict(dense_cfg(n_layers=2, hidden=256, n_heads=4, n_kv=2, head_dim=64, inter=512, vocab=512, softcap=50.0), **GEMMA2)
+    cfg["final_softcap"] = 2.0
+    toks = list(np.random.default_rng(62).integers(0, 512, 6))
+
+    def last_logits(c):
+        p = Pair(c, seed=72, dev=dev, slots=2)
+        try:
+            for pos, t in enumerate(toks):
+                lg, _ = p.gpu.step_batch([0], [pos], p.emb[[t]] * np.float32(16.0))
+            ref = p.oracle.new_cache(16)
+            for t in toks:
+                want = p.oracle.step(p.emb[[t]] * np.float32(16.0), [ref])
+            p.oracle.free_cache(ref)
+            assert np.abs(lg - want).max() <= 2e-2
+            return lg
+        finally:
+            p.close()
+
+    base = last_logits(cfg)
+    assert np.abs(base).max() < 2.0  # capped
+    for knob in ("post_norms", "act_gelu_tanh", "final_softcap"):
+        assert np.abs(last_logits(dict(cfg, **{knob: 0})) - base).max() > 1e-3, knob
+
+
+def test_gemma2_fused_gateup_equals_separate_kernels(dev, monkeypatch):
+    """The gate|up kernel with GeGLU in its epilogue against the plain GEMM followed by the activation kernel: the same bits."""
+    cfg = dict(dense_cfg(n_layers=2, hidden=256, n_heads=4, n_kv=2, head_dim=64, inter=512, vocab=512), **GEMMA2)
+    rng = np.random.default_rng(63)
+    toks = rng.integers(0, 512, (3, 40))
+    outs = []
+    for off in (False, True):
+        if off:
+            monkeypatch.setenv("ROCMDECODE_NO_FUSED_GATEUP", "1")
+        p = Pair(cfg, seed=73, dev=dev, slots=40)
+        try:
+            got = [p.gpu.step_batch(list(range(40)), [pos] * 40, p.emb[toks[pos]])[0] for pos in range(3)]
+            outs.append(np.stack(got))
+        finally:
+            p.close()
+    assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
