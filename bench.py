@@ -117,7 +117,7 @@ def run_c4(args):
     rng = np.random.default_rng(args.seed)
     lens = rng.integers(args.ctx_min, args.ctx_max + 1, B).astype(np.int64)  # context lengths uniform in [512, 4096] unless asked otherwise
     ids0 = rng.integers(0, cfg["vocab"], B).astype(np.int32)
-    cap = int(lens.max()) + args.steps + args.warmup + 8
+    cap = int(lens.max()) + args.steps + args.warmup + 48  # the timed steps, then the profiling and enqueue-cost steps after them
     dev = capi.Device(0)
     log("building %s, %d layers" % (cfg["name"], cfg["n_layers"]))
     res = workloads.Resident(dev, cfg, seed=args.seed, slots=B, ctx_cap=cap, keep_layers=0 if args.no_cpu else min(CPU_LAYERS, args.layers), progress=log, kv=args.kv)
@@ -172,6 +172,17 @@ def run_c4(args):
                 "step_frac": round(step_gbs / HBM_PEAK_GBS, 4)}
     classes = {k: {"ms_per_step": round(v[0] / 3, 4), "launches_per_step": v[1] // 3} for k, v in prof.items()}
 
+    # ---- the host's cost of enqueueing a step: the captured graph's one launch against the eager launches ----
+    host_us = {}
+    for i, (mode, on) in enumerate((("graph", True), ("eager", False))):
+        res.model.set_graph(on)
+        # each call takes 3 settling steps and 4 timed ones (the depth of the step's staging ring: a fifth would wait for the GPU)
+        # from where the previous call left the slots
+        runs = [res.model.bench_enqueue(slots, (pos_prof + 3 + 7 * (3 * i + j)).astype(np.int32), ids0, 4) for j in range(3)]
+        host_us[mode] = round(float(np.median(runs)), 1)
+    res.model.set_graph(True)
+    captures, replays = res.model.graph_stats()
+
     # ---- a plain copy kernel of known size: the practical HBM rate, and the yardstick the traffic counters are scaled by ----
     COPY_BYTES = 1 << 30
     cms = dev.bench_kernel("copy", [COPY_BYTES], 2, 6)
@@ -200,6 +211,8 @@ def run_c4(args):
         "roofline": roofline,
         "copy_kernel": {"bytes_read": COPY_BYTES, "bytes_written": COPY_BYTES, "GBs": round(copy_gbs, 1)},
         "kernel_classes": classes,
+        "host_enqueue_us_per_step": dict(host_us, note="wall clock of the host loop that enqueues a step, GPU not waited for; the timed steps above replay the graph"),
+        "graph": {"captures": captures, "steps_replayed": replays},
         "cpu_baseline": cpu,
     }
     print(json.dumps(out, default=float))

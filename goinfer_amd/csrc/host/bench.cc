@@ -2,6 +2,7 @@
 // already resident in HBM when the timed region starts.
 #include "model.h"
 #include <algorithm>
+#include <chrono>
 #include <memory>
 #include <numeric>
 #include <string.h>
@@ -44,6 +45,31 @@ extern "C" int rd_bench_steps(rd_model *m, int B, const int *slot, const int *po
     }
     for (auto &e : ev) (void)d->hip->EventDestroy(e);
     return rc;
+}
+
+// The host's own cost of a step: `steps` chained greedy steps are enqueued without waiting for the GPU and the wall clock of the
+// enqueue loop alone is taken (the stream is drained before and after). *host_us = microseconds of host time per step. With more
+// steps than the staging ring has slots (rd_model::STAGE_SLOTS) the loop waits for the GPU and measures that instead.
+extern "C" int rd_bench_enqueue(rd_model *m, int B, const int *slot, const int *pos0, const int *ids0, int steps, double *host_us) {
+    if (!m || !slot || !pos0 || !ids0 || !host_us || steps <= 0 || B < 1 || B > m->max_rows) return RD_ERR_ARG;
+    rd_device *d = m->d;
+    RC(d->h2d(m->ids, ids0, sizeof(int) * (size_t)B));
+    std::vector<int> pos((size_t)B);
+    int rc = RD_OK;
+    for (int i = 0; i < 3 && !rc; i++) { // settle: the third step with one key runs from the graph when graphs are on
+        for (int b = 0; b < B; b++) pos[(size_t)b] = pos0[b] + i;
+        rc = model_step(m, B, slot, pos.data(), nullptr, nullptr, RD_WANT_ARGMAX, nullptr, nullptr);
+    }
+    RC(d->sync());
+    const auto t0 = std::chrono::steady_clock::now();
+    for (int i = 3; i < 3 + steps && !rc; i++) {
+        for (int b = 0; b < B; b++) pos[(size_t)b] = pos0[b] + i;
+        rc = model_step(m, B, slot, pos.data(), nullptr, nullptr, RD_WANT_ARGMAX, nullptr, nullptr);
+    }
+    const auto t1 = std::chrono::steady_clock::now();
+    const int rc2 = d->sync();
+    *host_us = std::chrono::duration<double, std::micro>(t1 - t0).count() / steps;
+    return rc ? rc : rc2;
 }
 
 // One step with an event pair around every kernel class: class_ms[KC_COUNT] total milliseconds, class_n[KC_COUNT] launches.

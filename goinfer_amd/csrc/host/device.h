@@ -111,6 +111,8 @@ constexpr int ATTN_RANGE_INTS = 3; // per (row, kv head): first item, one past t
 // A work list of at most this many items (one per SIMD of the chip) runs the attention kernels that keep two units in flight
 // per wave: with so few waves nothing else hides a wave's memory latency. Same results bit for bit.
 constexpr int ATTN_DEEP_MAX_ITEMS = 1024;
+// A step's work list is launched padded to a multiple of this many items (one per compute unit) with items whose row is -1
+constexpr int ATTN_LIST_PAD = 256;
 hipFunction_t attn_partial_kernel(const struct rd_device *d, bool i8, bool grouped, size_t n_items);
 constexpr int TOPK_MAX = 1024; // = RD_TOPK_MAX of the top-K kernels
 constexpr int TOPK_CAP = 4096, TOPK_BINS = 2048, TOPK_CHUNK = 16384; // = RD_TOPK_CAP, RD_TOPK_BINS, RD_TOPK_CHUNK

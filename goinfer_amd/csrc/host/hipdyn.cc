@@ -42,6 +42,9 @@ static void load_once() {
            sym(h, "hipEventSynchronize", a.EventSynchronize) && sym(h, "hipEventElapsedTime", a.EventElapsedTime) &&
            sym(h, "hipModuleLoadData", a.ModuleLoadData) && sym(h, "hipModuleUnload", a.ModuleUnload) &&
            sym(h, "hipModuleGetFunction", a.ModuleGetFunction) && sym(h, "hipModuleLaunchKernel", a.ModuleLaunchKernel) &&
+           sym(h, "hipStreamBeginCapture", a.StreamBeginCapture) && sym(h, "hipStreamEndCapture", a.StreamEndCapture) &&
+           sym(h, "hipGraphInstantiate", a.GraphInstantiate) && sym(h, "hipGraphLaunch", a.GraphLaunch) &&
+           sym(h, "hipGraphDestroy", a.GraphDestroy) && sym(h, "hipGraphExecDestroy", a.GraphExecDestroy) &&
            sym(h, "hipGetErrorString", a.GetErrorString) && sym(h, "hipGetLastError", a.GetLastError);
 }
 

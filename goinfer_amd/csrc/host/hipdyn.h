@@ -33,6 +33,12 @@ struct HipApi {
     hipError_t (*ModuleGetFunction)(hipFunction_t *, hipModule_t, const char *);
     hipError_t (*ModuleLaunchKernel)(hipFunction_t, unsigned, unsigned, unsigned, unsigned, unsigned, unsigned, unsigned, hipStream_t,
                                      void **, void **);
+    hipError_t (*StreamBeginCapture)(hipStream_t, hipStreamCaptureMode);
+    hipError_t (*StreamEndCapture)(hipStream_t, hipGraph_t *);
+    hipError_t (*GraphInstantiate)(hipGraphExec_t *, hipGraph_t, hipGraphNode_t *, char *, size_t);
+    hipError_t (*GraphLaunch)(hipGraphExec_t, hipStream_t);
+    hipError_t (*GraphDestroy)(hipGraph_t);
+    hipError_t (*GraphExecDestroy)(hipGraphExec_t);
     const char *(*GetErrorString)(hipError_t);
     hipError_t (*GetLastError)();
 };

@@ -35,6 +35,7 @@ extern "C" int rd_model_create(rd_device *d, const rd_model_desc *desc, rd_model
     }
     rd_model *m = new rd_model();
     m->d = d;
+    m->graph.enabled = !getenv("ROCMDECODE_NO_GRAPH");
     m->desc = c;
     m->inv_freq.assign(c.rope_inv_freq, c.rope_inv_freq + c.head_dim / 2);
     m->desc.rope_inv_freq = nullptr;
@@ -57,6 +58,8 @@ extern "C" void rd_model_destroy(rd_model *m) {
     if (!m) return;
     rd_device *d = m->d;
     (void)d->sync();
+    if (m->graph.exec) (void)d->hip->GraphExecDestroy(m->graph.exec);
+    if (m->graph.graph) (void)d->hip->GraphDestroy(m->graph.graph);
     for (auto &l : m->layers) {
         free_weight(d, &l.qkv), free_weight(d, &l.o), free_weight(d, &l.gateup), free_weight(d, &l.down);
         for (void *p : {(void *)l.post_attn_norm, (void *)l.post_ffn_norm, (void *)l.attn_norm, (void *)l.ffn_norm, (void *)l.q_norm, (void *)l.k_norm, (void *)l.qkv_bias, (void *)l.router, (void *)l.router_bias, (void *)l.sinks, l.exp_gateup, l.exp_down,
@@ -567,6 +570,7 @@ extern "C" int rd_kv_configure_typed(rd_model *m, int slots, int ctx_cap, int kv
     m->slot_len.assign((size_t)slots, 0);
     // attention work list: every (row, kv head) of a step is cut into at most attn_max_pieces items
     m->max_items = m->max_rows * c.n_kv_heads * attn_max_pieces(m->blocks_per_slot);
+    m->max_items = (m->max_items + ATTN_LIST_PAD - 1) / ATTN_LIST_PAD * ATTN_LIST_PAD; // a step's list is padded to this grain
     RC(alloc_f32(d, &m->part, (size_t)m->max_items * ATTN_TILE_ROWS * (c.head_dim + 2)));
     // The step's metadata lives in one device block so a step uploads it with one copy:
     // [row slot R][row position R][row length R][row draw records R x 6][item ranges max_rows*nKV*3][items max_items x 4] ints, R = ROWS_MAX
@@ -813,112 +817,13 @@ int launch_attn_partial(rd_model *m, const LayerW &l) {
                      nH, nKV, HD, c.attn_scale, c.attn_softcap, l.window);
 }
 
-// emb_host: [B][hidden] on the host, or emb_dev already on the device (benchmark loop). Logits/ids are host pointers.
-int model_step(rd_model *m, int B, const int *slot, const int *pos, const float *emb_host, const float *emb_dev, int want, float *logits,
-               int *ids, bool multirow) {
+// Every launch of a step between the uploads (metadata, embeddings) and the copies back: the layers, the final norm, the head,
+// the argmax. What it launches depends on the model, B, `want`, and the state step_graph_key() lists, and on nothing else: the
+// per-step data (positions, tables, work lists, draw records) is read from device memory the uploads have already filled.
+static int step_launches(rd_model *m, int B, int want) {
     rd_device *d = m->d;
     const rd_model_desc &c = m->desc;
-    if (!m->finalized || !m->tables) {
-        rd_set_error("step before rd_model_finalize / rd_kv_configure");
-        return RD_ERR_STATE;
-    }
-    if (m->chain.open && !m->chain.in_call) {
-        rd_set_error("a chain is open: between its start and stop the resident takes no other step");
-        return RD_ERR_STATE;
-    }
-    if (B < 1 || B > m->max_rows) {
-        rd_set_error("rocm resident: batch %d outside the stepper range 1..%d", B, m->max_rows);
-        return RD_ERR_ARG;
-    }
-    RC(d->use());
-    // A slot may carry several rows in one step if they sit at consecutive positions (a ragged step's verify or prefill
-    // rows): all their K/V is written before any row attends, and row j reads keys [0, pos_j], so each row is the row its own
-    // single-token step would compute. Anything else naming a slot twice is refused before a byte is written.
-    for (int b = 0; b < B; b++) {
-        if (!slot_ok(m, slot[b])) return RD_ERR_ARG;
-        int prev = -1;
-        for (int a = 0; a < b; a++)
-            if (slot[a] == slot[b]) prev = a;
-        if (prev >= 0) {
-            if (!multirow || pos[b] != pos[prev] + 1) {
-                rd_set_error("slot %d appears twice in one step", slot[b]);
-                return RD_ERR_ARG;
-            }
-        } else if (pos[b] < 0 || pos[b] > m->slot_len[(size_t)slot[b]]) {
-            rd_set_error("row %d: position %d but slot %d holds %d rows", b, pos[b], slot[b], m->slot_len[(size_t)slot[b]]);
-            return RD_ERR_ARG;
-        }
-        if (pos[b] >= m->ctx_cap) { // ErrKVPoolFull: nothing has been written
-            rd_set_error("row %d: position %d reaches the context cap %d", b, pos[b], m->ctx_cap);
-            return RD_ERR_KV_FULL;
-        }
-    }
-    int H = c.hidden, nH = c.n_heads, nKV = c.n_kv_heads, HD = c.head_dim;
-    const int nLists = m->window > 0 ? 2 : 1;
-    std::vector<AttnItemH> items[2];
-    std::vector<int> start[2];
-    for (int li = 0; li < nLists; li++) {
-        bool grouped = false;
-        RC(build_attn_items(m, B, slot, pos, items[li], start[li], &grouped, li ? m->window : 0));
-        m->last_items[li] = items[li].size(), m->last_grouped[li] = grouped;
-    }
-    // Stage the step's metadata (and host embeddings) in pinned memory and upload it asynchronously. A slot is reused only
-    // once the upload it last fed has completed, which its event tells.
-    const unsigned stage_slot = m->stage_next++ % rd_model::STAGE_SLOTS;
-    if (m->stage_busy[stage_slot]) HIPCHK(EventSynchronize(m->stage_ev[stage_slot]));
-    {
-        char *st = (char *)m->host_stage + (size_t)stage_slot * m->host_stage_bytes;
-        int *hm = (int *)st; // the metadata block, laid out as on the device
-        const size_t rangeInts = (size_t)m->max_rows * nKV * ATTN_RANGE_INTS;
-        constexpr int RM = rd_model::ROWS_MAX;
-        float *eh = (float *)(st + m->stage_meta_bytes);
-        for (int b = 0; b < B; b++) hm[b] = slot[b], hm[RM + b] = pos[b], hm[2 * RM + b] = pos[b] + 1;
-        // Draw records (resident/forward.go:43-52 BatchDraw) with Sampler.gumbelDraw's guards applied here
-        // (internal/runtime/sampling/sampler_gumbel.go:80-88): a temperature <= 0 means 1, and one so small that 1/T
-        // overflows f32 is the plain argmax.
-        for (int b = 0; b < RM; b++) {
-            int *r = hm + 3 * RM + b * 6;
-            memset(r, 0, sizeof(int) * 6);
-            if (b >= B || !m->step_draws) continue;
-            const rd_draw &dw = m->step_draws[b];
-            r[0] = dw.mode;
-            if (dw.mode == RD_DRAW_GUMBEL) {
-                float invT = (float)(1.0 / (dw.temperature <= 0 ? 1.0 : dw.temperature));
-                if (std::isinf(invT)) {
-                    r[0] = RD_DRAW_GREEDY;
-                    continue;
-                }
-                memcpy(&r[1], &invT, 4);
-                r[2] = (int)(uint32_t)dw.seed, r[3] = (int)(uint32_t)(dw.seed >> 32);
-                r[4] = (int)(uint32_t)dw.draw, r[5] = (int)(uint32_t)(dw.draw >> 32);
-            }
-        }
-        constexpr int HDR = rd_model::META_HDR;
-        memset(hm + HDR - 8, 0, sizeof(int) * 8);
-        for (int li = 0; li < nLists; li++) {
-            int *lst = hm + HDR + (size_t)li * m->list_ints;
-            memcpy(lst, start[li].data(), sizeof(int) * start[li].size());
-            memcpy(lst + rangeInts, items[li].data(), sizeof(AttnItemH) * items[li].size());
-        }
-        RC(d->h2d(m->meta, hm, sizeof(int) * (HDR + (size_t)(nLists - 1) * m->list_ints + rangeInts + items[nLists - 1].size() * 4)));
-        if (emb_host) {
-            memcpy(eh, emb_host, sizeof(float) * (size_t)B * H);
-            RC(d->h2d(m->h, eh, sizeof(float) * (size_t)B * H));
-        }
-        HIPCHK(EventRecord(m->stage_ev[stage_slot], d->stream));
-        m->stage_busy[stage_slot] = true;
-        if (emb_host) {
-        } else if (emb_dev) {
-            HIPCHK(MemcpyAsync(m->h, emb_dev, sizeof(float) * (size_t)B * H, hipMemcpyDeviceToDevice, d->stream));
-        } else { // greedy chain: the previous step's argmax ids, still on the device
-            if (!m->embed_q) {
-                rd_set_error("greedy chain needs rd_model_upload_embedding");
-                return RD_ERR_STATE;
-            }
-            RC(d->launch(d->k.embed_rows, (unsigned)B, 1, 1, 256, (const signed char *)m->embed_q, (const float *)m->embed_scale, (const int *)m->ids,
-                         m->h, H));
-        }
-    }
+    const int H = c.hidden, nH = c.n_heads, nKV = c.n_kv_heads, HD = c.head_dim;
     // pending residual contribution: split-K partials of the previous block's last GEMM, or (resW set) an MoE layer's
     // down-projection rows and their weights, folded by the kernel that adds them
     const float *resP = nullptr, *resW = nullptr, *resPost = nullptr; // resPost: the pending contribution's own norm, if any
@@ -1024,6 +929,197 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
             if (want & RD_WANT_ARGMAX) RC(d->launch(d->k.argmax_final, (unsigned)B, 1, 1, 64, (const float *)m->cand_v, (const int *)m->cand_i, nChunks, m->ids));
         }
     }
+    return RD_OK;
+}
+
+// What step_launches() reads besides the model: two steps with equal keys issue the same launches with the same arguments, so
+// the second may replay the first one's captured graph. Empty: this step is not one to capture (timed, or replaying a routing).
+static std::vector<long> step_graph_key(rd_model *m, int B, int want) {
+    std::vector<long> k;
+    if (m->timer.on || m->replay_B != 0) return k;
+    k = {B, want, m->step_draws ? 1 : 0, (long)m->last_items[0], (long)m->last_items[1], m->last_grouped[0] ? 1 : 0, m->last_grouped[1] ? 1 : 0,
+         getenv("ROCMDECODE_NO_FUSED_GATEUP") ? 1 : 0, getenv("ROCMDECODE_NO_FUSED_QKV") ? 1 : 0, getenv("ROCMDECODE_NO_FUSED_MOE_GATEUP") ? 1 : 0,
+         getenv("ROCMDECODE_MOE_TILES") ? atol(getenv("ROCMDECODE_MOE_TILES")) : 0};
+    return k;
+}
+
+static void step_graph_drop(rd_model *m) {
+    rd_device *d = m->d;
+    if (m->graph.exec) (void)d->hip->GraphExecDestroy(m->graph.exec);
+    if (m->graph.graph) (void)d->hip->GraphDestroy(m->graph.graph);
+    m->graph.exec = nullptr, m->graph.graph = nullptr, m->graph.key.clear();
+}
+
+// The launches of a step, from a captured HIP graph when this step repeats the previous one's key (a decode loop whose work list
+// keeps its size: every step of a batch between two piece boundaries), eagerly otherwise. The second step in a row with one key
+// is captured (stream capture records the launches without running them) and the graph, once instantiated, runs that step too.
+// Any failure of the graph calls ends graph use for this model and the step is launched eagerly: the result is the same bits.
+static int step_run(rd_model *m, int B, int want) {
+    rd_device *d = m->d;
+    const HipApi *hip = d->hip;
+    std::vector<long> key;
+    if (m->graph.enabled) key = step_graph_key(m, B, want);
+    if (key.empty()) {
+        m->graph.prev_key.clear();
+        return step_launches(m, B, want);
+    }
+    if (m->graph.exec && key == m->graph.key) {
+        m->graph.replays++;
+        if (rd_hip_ok(hip, hip->GraphLaunch(m->graph.exec, d->stream), "hipGraphLaunch")) return RD_OK;
+        m->graph.enabled = false; // nothing of this step has run: fall through to the eager launches
+        step_graph_drop(m);
+        return step_launches(m, B, want);
+    }
+    const bool repeat = key == m->graph.prev_key;
+    m->graph.prev_key = key;
+    if (!repeat) return step_launches(m, B, want);
+    step_graph_drop(m);
+    if (!rd_hip_ok(hip, hip->StreamBeginCapture(d->stream, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture")) {
+        m->graph.enabled = false;
+        return step_launches(m, B, want);
+    }
+    const int rc = step_launches(m, B, want);
+    hipGraph_t g = nullptr;
+    const bool ended = rd_hip_ok(hip, hip->StreamEndCapture(d->stream, &g), "hipStreamEndCapture");
+    if (rc || !ended || !g || !rd_hip_ok(hip, hip->GraphInstantiate(&m->graph.exec, g, nullptr, nullptr, 0), "hipGraphInstantiate")) {
+        if (g) (void)hip->GraphDestroy(g);
+        m->graph.exec = nullptr, m->graph.enabled = false;
+        return rc ? rc : step_launches(m, B, want); // the capture ran nothing
+    }
+    m->graph.graph = g, m->graph.key = key, m->graph.captures++;
+    if (rd_hip_ok(hip, hip->GraphLaunch(m->graph.exec, d->stream), "hipGraphLaunch")) return RD_OK;
+    m->graph.enabled = false;
+    step_graph_drop(m);
+    return step_launches(m, B, want);
+}
+
+// Graph replay of the step's launches on or off (on at creation unless ROCMDECODE_NO_GRAPH is set), and how often it was used.
+extern "C" int rd_model_set_graph(rd_model *m, int on) {
+    if (!m) return RD_ERR_ARG;
+    RC(m->d->sync());
+    step_graph_drop(m);
+    m->graph.prev_key.clear();
+    m->graph.enabled = on != 0;
+    return RD_OK;
+}
+
+extern "C" int rd_model_graph_stats(rd_model *m, long long *captures, long long *replays) {
+    if (!m) return RD_ERR_ARG;
+    if (captures) *captures = m->graph.captures;
+    if (replays) *replays = m->graph.replays;
+    return RD_OK;
+}
+
+// emb_host: [B][hidden] on the host, or emb_dev already on the device (benchmark loop). Logits/ids are host pointers.
+int model_step(rd_model *m, int B, const int *slot, const int *pos, const float *emb_host, const float *emb_dev, int want, float *logits,
+               int *ids, bool multirow) {
+    rd_device *d = m->d;
+    const rd_model_desc &c = m->desc;
+    if (!m->finalized || !m->tables) {
+        rd_set_error("step before rd_model_finalize / rd_kv_configure");
+        return RD_ERR_STATE;
+    }
+    if (m->chain.open && !m->chain.in_call) {
+        rd_set_error("a chain is open: between its start and stop the resident takes no other step");
+        return RD_ERR_STATE;
+    }
+    if (B < 1 || B > m->max_rows) {
+        rd_set_error("rocm resident: batch %d outside the stepper range 1..%d", B, m->max_rows);
+        return RD_ERR_ARG;
+    }
+    RC(d->use());
+    // A slot may carry several rows in one step if they sit at consecutive positions (a ragged step's verify or prefill
+    // rows): all their K/V is written before any row attends, and row j reads keys [0, pos_j], so each row is the row its own
+    // single-token step would compute. Anything else naming a slot twice is refused before a byte is written.
+    for (int b = 0; b < B; b++) {
+        if (!slot_ok(m, slot[b])) return RD_ERR_ARG;
+        int prev = -1;
+        for (int a = 0; a < b; a++)
+            if (slot[a] == slot[b]) prev = a;
+        if (prev >= 0) {
+            if (!multirow || pos[b] != pos[prev] + 1) {
+                rd_set_error("slot %d appears twice in one step", slot[b]);
+                return RD_ERR_ARG;
+            }
+        } else if (pos[b] < 0 || pos[b] > m->slot_len[(size_t)slot[b]]) {
+            rd_set_error("row %d: position %d but slot %d holds %d rows", b, pos[b], slot[b], m->slot_len[(size_t)slot[b]]);
+            return RD_ERR_ARG;
+        }
+        if (pos[b] >= m->ctx_cap) { // ErrKVPoolFull: nothing has been written
+            rd_set_error("row %d: position %d reaches the context cap %d", b, pos[b], m->ctx_cap);
+            return RD_ERR_KV_FULL;
+        }
+    }
+    const int H = c.hidden, nKV = c.n_kv_heads;
+    const int nLists = m->window > 0 ? 2 : 1;
+    std::vector<AttnItemH> items[2];
+    std::vector<int> start[2];
+    for (int li = 0; li < nLists; li++) {
+        bool grouped = false;
+        RC(build_attn_items(m, B, slot, pos, items[li], start[li], &grouped, li ? m->window : 0));
+        // The list is launched padded to a multiple of ATTN_LIST_PAD with items that name no row (their waves leave at once):
+        // the launch then keeps its shape over many steps of a growing batch, which is what lets a captured graph be replayed.
+        items[li].resize((items[li].size() + ATTN_LIST_PAD - 1) / ATTN_LIST_PAD * ATTN_LIST_PAD, AttnItemH{-1, 0, 0, 0});
+        m->last_items[li] = items[li].size(), m->last_grouped[li] = grouped;
+    }
+    // Stage the step's metadata (and host embeddings) in pinned memory and upload it asynchronously. A slot is reused only
+    // once the upload it last fed has completed, which its event tells.
+    const unsigned stage_slot = m->stage_next++ % rd_model::STAGE_SLOTS;
+    if (m->stage_busy[stage_slot]) HIPCHK(EventSynchronize(m->stage_ev[stage_slot]));
+    {
+        char *st = (char *)m->host_stage + (size_t)stage_slot * m->host_stage_bytes;
+        int *hm = (int *)st; // the metadata block, laid out as on the device
+        const size_t rangeInts = (size_t)m->max_rows * nKV * ATTN_RANGE_INTS;
+        constexpr int RM = rd_model::ROWS_MAX;
+        float *eh = (float *)(st + m->stage_meta_bytes);
+        for (int b = 0; b < B; b++) hm[b] = slot[b], hm[RM + b] = pos[b], hm[2 * RM + b] = pos[b] + 1;
+        // Draw records (resident/forward.go:43-52 BatchDraw) with Sampler.gumbelDraw's guards applied here
+        // (internal/runtime/sampling/sampler_gumbel.go:80-88): a temperature <= 0 means 1, and one so small that 1/T
+        // overflows f32 is the plain argmax.
+        for (int b = 0; b < RM; b++) {
+            int *r = hm + 3 * RM + b * 6;
+            memset(r, 0, sizeof(int) * 6);
+            if (b >= B || !m->step_draws) continue;
+            const rd_draw &dw = m->step_draws[b];
+            r[0] = dw.mode;
+            if (dw.mode == RD_DRAW_GUMBEL) {
+                float invT = (float)(1.0 / (dw.temperature <= 0 ? 1.0 : dw.temperature));
+                if (std::isinf(invT)) {
+                    r[0] = RD_DRAW_GREEDY;
+                    continue;
+                }
+                memcpy(&r[1], &invT, 4);
+                r[2] = (int)(uint32_t)dw.seed, r[3] = (int)(uint32_t)(dw.seed >> 32);
+                r[4] = (int)(uint32_t)dw.draw, r[5] = (int)(uint32_t)(dw.draw >> 32);
+            }
+        }
+        constexpr int HDR = rd_model::META_HDR;
+        memset(hm + HDR - 8, 0, sizeof(int) * 8);
+        for (int li = 0; li < nLists; li++) {
+            int *lst = hm + HDR + (size_t)li * m->list_ints;
+            memcpy(lst, start[li].data(), sizeof(int) * start[li].size());
+            memcpy(lst + rangeInts, items[li].data(), sizeof(AttnItemH) * items[li].size());
+        }
+        RC(d->h2d(m->meta, hm, sizeof(int) * (HDR + (size_t)(nLists - 1) * m->list_ints + rangeInts + items[nLists - 1].size() * 4)));
+        if (emb_host) {
+            memcpy(eh, emb_host, sizeof(float) * (size_t)B * H);
+            RC(d->h2d(m->h, eh, sizeof(float) * (size_t)B * H));
+        }
+        HIPCHK(EventRecord(m->stage_ev[stage_slot], d->stream));
+        m->stage_busy[stage_slot] = true;
+        if (emb_host) {
+        } else if (emb_dev) {
+            HIPCHK(MemcpyAsync(m->h, emb_dev, sizeof(float) * (size_t)B * H, hipMemcpyDeviceToDevice, d->stream));
+        } else { // greedy chain: the previous step's argmax ids, still on the device
+            if (!m->embed_q) {
+                rd_set_error("greedy chain needs rd_model_upload_embedding");
+                return RD_ERR_STATE;
+            }
+            RC(d->launch(d->k.embed_rows, (unsigned)B, 1, 1, 256, (const signed char *)m->embed_q, (const float *)m->embed_scale, (const int *)m->ids,
+                         m->h, H));
+        }
+    }
+    RC(step_run(m, B, want));
     // else: no logits asked for (resident.Forward's ForwardNoLogits, decoder/resident/subsystems.go:68-77: a prompt token that only
     // builds its K/V): the final norm, the head GEMM and the argmax are skipped, and the last block's pending residual
     // contribution stays unadded, since nothing reads the hidden state after it.

@@ -60,6 +60,14 @@ struct rd_model {
     int norm_add_one = 0, act = 0; // (1 + w) norm weights; the gated FFN's activation (RD_ACT_*)
     float final_softcap = 0.f;     // > 0: logits become cap * tanh(logit / cap)
     bool ones_added = false;       // the (1 + w) pass over the norm weights has run
+    // The launches of a step as a captured HIP graph, replayed while steps keep one key (see step_run in model.cc)
+    struct StepGraph {
+        bool enabled = true;
+        hipGraph_t graph = nullptr;
+        hipGraphExec_t exec = nullptr;
+        std::vector<long> key, prev_key;
+        long captures = 0, replays = 0;
+    } graph;
 
     // KV
     int slots = 0, ctx_cap = 0, blocks_per_slot = 0;

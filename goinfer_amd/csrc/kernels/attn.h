@@ -363,6 +363,7 @@ __device__ __forceinline__ void attn_partial_body(const AttnItem *__restrict__ i
     constexpr int KL = I8 ? NC / 2 : NC, VL = I8 ? NCT / 2 : NCT; // 16-byte loads per key tile of K, per 32 keys of V
     constexpr int ELEM = I8 ? 1 : 2;
     AttnItem it = items[blockIdx.x];
+    if (it.row < 0) return; // padding of the work list: names no row
     const int nrows = ROWS ? it.kvh >> 16 : 1;
     it.kvh &= 0xffff;
     const int lane = threadIdx.x, l16 = lane & 15, lg = lane >> 4;

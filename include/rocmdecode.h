@@ -177,6 +177,14 @@ int rd_model_set_block(rd_model *m, int norm_add_one, int act, float final_softc
 /* A sliding-window layer (decoder/kvcache.go:1063-1068 WindowStart): its rows read the last `window` positions only. Before
  * rd_model_finalize. The windowed layers of a model share one length (RD_DECLINED otherwise); the cache keeps every position. */
 int rd_model_set_window(rd_model *m, int layer, int window);
+/* HIP-graph replay of a step's launches (the single-queue executor of backend/cuda/resident.go:2135 is the reference's answer to
+ * the same cost: a few hundred launches a step). Between the uploads of a step's metadata and the copies back, every launch
+ * depends only on the model, the batch size, what is asked for and the size of the attention work list; a step that repeats the
+ * previous step's values of those replays the graph captured from it, any other step is launched eagerly, and both give the same
+ * bits. On by default (ROCMDECODE_NO_GRAPH in the environment turns it off at rd_model_create); rd_model_graph_stats counts the
+ * graphs captured and the steps replayed. */
+int rd_model_set_graph(rd_model *m, int on);
+int rd_model_graph_stats(rd_model *m, long long *captures, long long *replays);
 /* after the last upload: checks every tensor the step needs is present */
 int rd_model_finalize(rd_model *m);
 
@@ -306,6 +314,9 @@ int rd_bench_steps(rd_model *m, int B, const int *slot, const int *pos0, const i
 /* One step with a HIP-event pair around every kernel class: class_ms[n] total milliseconds and class_n[n] launches,
  * n = rd_bench_class_count(); names from rd_bench_class_name. */
 int rd_bench_profile(rd_model *m, int B, const int *slot, const int *pos, const int *ids0, float *class_ms, int *class_n);
+/* The host's cost of a step: `steps` chained greedy steps enqueued without waiting for the GPU, wall clock of the enqueue loop
+ * alone, in microseconds per step (with and without graph replay: rd_model_set_graph). Measurement only. */
+int rd_bench_enqueue(rd_model *m, int B, const int *slot, const int *pos0, const int *ids0, int steps, double *host_us);
 /* The attention kernel's average launch duration: one step as above, then that kernel of every layer (its own KV, the step's
  * work list) launched back to back `reps` times between one pair of HIP events on the launch stream, so no event sits between
  * two launches. *ms_per_launch = elapsed / *launches, *launches = layers * reps. Measurement only. */
