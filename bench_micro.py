@@ -323,7 +323,7 @@ def run_c5(args):
     d2 = float(sum(len(set(idx2[:, l, :].ravel().tolist())) for l in range(layers)))
     g_ms = prof["moe_gemm_gateup"][0] / prof["moe_gemm_gateup"][1]
     per_launch = d2 * ebytes * (2.0 / 3.0) / layers
-    traffic, t_ratio, t_src = counter_traffic("gemm8_w4a8_moe_gateup/%s" % cfg["name"], per_launch)
+    traffic, t_ratio, t_src = counter_traffic("moe_gemv_w4a8_gateup/%s" % cfg["name"], per_launch)
     out = base_line("batch-16 decode tok/s, Qwen3-MoE-30B-A3B shape (int4-g32 experts); achieved HBM GB/s vs peak", tok_s, "tok/s", steps, warmup,
                     float(ms.mean()), "configs[4]: %s, %d layers, B=%d ragged, ctx U[256,2048], greedy decode" % (cfg["name"], layers, B),
                     "synthetic: N(0,0.02) weights (Q4_K projections, int4-g32 experts, f32 router, int8 head), N(0,1) KV, random token ids",

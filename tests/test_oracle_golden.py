@@ -48,7 +48,37 @@ def test_llama_tiny_text_parity(name, golden, reached):
     assert cont == g["continuation_ids"]
 
 
+def test_mistral_tiny_window_parity():
+    """decoder/mistral_tiny_window_test.go:66-95: a 3-layer Mistral with sliding_window 16 on every layer, a prompt longer than
+    the window, the reference's bars (argmax, cosine 0.9999, relative L2 1e-5, the greedy continuation); without the window the
+    restatement misses them."""
+    g = json.load(open(os.path.join(GOLDEN, "mistral_tiny_window_golden.json")))
+    assert len(g["prompt_ids"]) > g["window"]
+    m, emb, _ = tiny_model("mistral-tiny-window")
+    want = np.array(g["last_logits"], np.float64)
+
+    def rel_l2(logits):
+        got = logits.astype(np.float64)
+        return np.sqrt(((got - want) ** 2).sum() / (want ** 2).sum()), got @ want / np.linalg.norm(got) / np.linalg.norm(want)
+
+    logits, c = run_prompt(m, emb, g["prompt_ids"], cap=128)
+    rel, cos = rel_l2(logits)
+    assert ob.argmax(logits) == g["argmax"] and cos >= 0.9999 and rel <= 1e-5, (rel, cos)
+    cont, tok = [], ob.argmax(logits)
+    for _ in range(g["n_new"]):
+        cont.append(tok)
+        tok = ob.argmax(m.step(emb[tok][None, :], [c])[0])
+    m.free_cache(c)
+    assert cont == g["continuation_ids"]
+    for l in range(m.m.n_layers):
+        m._layers[l].window = 0
+    logits, c = run_prompt(m, emb, g["prompt_ids"], cap=128)
+    m.free_cache(c)
+    assert rel_l2(logits)[0] > 1e-3  # the whole context is another function
+
+
 @pytest.mark.parametrize("name,golden", [("qwen3moe-tiny", "qwen3moe_forward_golden.json"),
+                                         ("qwen3moe-tiny-k3", "qwen3moe_k3_forward_golden.json"),
                                          ("mixtral-tiny", "mixtral_forward_golden.json")])
 def test_moe_tiny_forward(name, golden):
     g = json.load(open(os.path.join(GOLDEN, golden)))

@@ -55,6 +55,8 @@ def tiny_model(name, wrap=ob.WMat.from_f32):
                 lw["window"] = cfg["sliding_window"]
         else:
             lw["ffn_norm"] = t[p + "post_attention_layernorm.weight"]
+            if cfg["model_type"] == "mistral" and cfg.get("sliding_window"):  # every layer slides
+                lw["window"] = cfg["sliding_window"]
         if p + "self_attn.q_norm.weight" in t:
             lw["q_norm"] = t[p + "self_attn.q_norm.weight"]
             lw["k_norm"] = t[p + "self_attn.k_norm.weight"]
