@@ -174,11 +174,16 @@ def run_c4(args):
 
     # ---- the host's cost of enqueueing a step: the captured graph's one launch against the eager launches ----
     host_us = {}
-    for i, (mode, on) in enumerate((("graph", True), ("eager", False))):
-        res.model.set_graph(on)
+    at = pos_prof + 3  # where the profiling passes left the slots
+    for mode, on in (("graph", True), ("eager", False)):
+        if not res.model.set_graph(on):  # declined under a profiler: the eager figure only
+            host_us[mode] = None
+            continue
         # each call takes 3 settling steps and 4 timed ones (the depth of the step's staging ring: a fifth would wait for the GPU)
-        # from where the previous call left the slots
-        runs = [res.model.bench_enqueue(slots, (pos_prof + 3 + 7 * (3 * i + j)).astype(np.int32), ids0, 4) for j in range(3)]
+        runs = []
+        for _ in range(3):
+            runs.append(res.model.bench_enqueue(slots, at.astype(np.int32), ids0, 4))
+            at = at + 7
         host_us[mode] = round(float(np.median(runs)), 1)
     res.model.set_graph(True)
     captures, replays = res.model.graph_stats()

@@ -352,7 +352,12 @@ class Model:
         return us.value
 
     def set_graph(self, on):
-        check(lib().rd_model_set_graph(self.h, 1 if on else 0), "rd_model_set_graph")
+        """Returns False when the library keeps graph replay off (a profiler tool library is attached)."""
+        rc = lib().rd_model_set_graph(self.h, 1 if on else 0)
+        if rc == 1:  # RD_DECLINED
+            return False
+        check(rc, "rd_model_set_graph")
+        return True
 
     def graph_stats(self):
         """(graphs captured, steps replayed from a graph)"""

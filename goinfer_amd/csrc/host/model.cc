@@ -15,6 +15,11 @@
 
 static int alloc_f32(rd_device *d, float **p, size_t n) { return d->alloc((void **)p, sizeof(float) * (n ? n : 1)); }
 
+static bool graph_allowed() {
+    if (getenv("ROCMDECODE_GRAPH")) return atoi(getenv("ROCMDECODE_GRAPH")) != 0;
+    return !getenv("ROCP_TOOL_LIBRARIES");
+}
+
 extern "C" int rd_model_create(rd_device *d, const rd_model_desc *desc, rd_model **out) {
     if (!d || !desc || !out) return RD_ERR_ARG;
     const rd_model_desc &c = *desc;
@@ -35,7 +40,10 @@ extern "C" int rd_model_create(rd_device *d, const rd_model_desc *desc, rd_model
     }
     rd_model *m = new rd_model();
     m->d = d;
-    m->graph.enabled = !getenv("ROCMDECODE_NO_GRAPH");
+    // Graph replay is on unless the environment says otherwise, or a rocprofiler tool library is attached (ROCP_TOOL_LIBRARIES, as
+    // rocprofv3 sets it): with kernel tracing on, replaying a captured graph ended in a segmentation fault inside the runtime on
+    // ROCm 7.2, while the same program runs clean without the tool. ROCMDECODE_GRAPH=1 keeps it on regardless.
+    m->graph.enabled = graph_allowed() && !getenv("ROCMDECODE_NO_GRAPH");
     m->desc = c;
     m->inv_freq.assign(c.rope_inv_freq, c.rope_inv_freq + c.head_dim / 2);
     m->desc.rope_inv_freq = nullptr;
@@ -999,6 +1007,11 @@ extern "C" int rd_model_set_graph(rd_model *m, int on) {
     RC(m->d->sync());
     step_graph_drop(m);
     m->graph.prev_key.clear();
+    m->graph.enabled = false;
+    if (on && !graph_allowed()) {
+        rd_set_error("graph replay stays off: a profiler tool library is attached (ROCP_TOOL_LIBRARIES); ROCMDECODE_GRAPH=1 overrides");
+        return RD_DECLINED;
+    }
     m->graph.enabled = on != 0;
     return RD_OK;
 }

@@ -181,8 +181,8 @@ int rd_model_set_window(rd_model *m, int layer, int window);
  * the same cost: a few hundred launches a step). Between the uploads of a step's metadata and the copies back, every launch
  * depends only on the model, the batch size, what is asked for and the size of the attention work list; a step that repeats the
  * previous step's values of those replays the graph captured from it, any other step is launched eagerly, and both give the same
- * bits. On by default (ROCMDECODE_NO_GRAPH in the environment turns it off at rd_model_create); rd_model_graph_stats counts the
- * graphs captured and the steps replayed. */
+ * bits. On by default; off at rd_model_create when ROCMDECODE_NO_GRAPH is set or a rocprofiler tool library is attached
+ * (ROCP_TOOL_LIBRARIES; ROCMDECODE_GRAPH=1 overrides; rd_model_set_graph(m, 1) then returns RD_DECLINED). rd_model_graph_stats counts the graphs captured and the steps replayed. */
 int rd_model_set_graph(rd_model *m, int on);
 int rd_model_graph_stats(rd_model *m, long long *captures, long long *replays);
 /* after the last upload: checks every tensor the step needs is present */

@@ -22,7 +22,19 @@
  *   or_qk_acc64 / or_av_acc64            pinned: linalg.MatmulQKAcc64, linalg.MatmulAVAcc64
  *   or_rmsnorm, or_rope, or_swiglu, or_softmax_f32, or_topk, or_route_experts, or_argmax
  *                                        plain Go in the reference, restated statement by statement;
- *                                        pinned by closed forms + the HF goldens (llama-tiny, qwen3moe-tiny, mixtral-tiny)
+ *                                        pinned by closed forms + the HF goldens (llama-tiny, internlm3-tiny, qwen3moe-tiny, mixtral-tiny)
+ *   or_route_experts_ex, or_group_limit  pinned: the known answers of the reference's decoder/moe_route_test.go (sigmoid scoring, the
+ *                                        selection bias, group-limited selection, the scaling factor), tests/test_oracle_routing.py;
+ *                                        top-3 routing also by the qwen3moe-tiny-k3 golden
+ *   the attention window (or_layer.window, `start` of or_attend)
+ *                                        pinned: the mistral-tiny-window golden (window 16 on every layer, the reference's bars
+ *                                        of decoder/mistral_tiny_window_test.go) and the gemma2-tiny golden (window 4 on alternate
+ *                                        layers); both fail with the window off
+ *   attention softcap, or_gelu_tanh / or_geglu, or_softcap_logits, (1 + w) norms, post-branch norms
+ *                                        pinned: the gemma2-tiny golden to 1e-5 (tests/test_oracle_golden.py shows each knob moves
+ *                                        the logits by > 1e-3 when switched off)
+ *   or_attend_sinks                      pinned by the closed form only (a softmax with one more logit per head, numpy f64):
+ *                                        the reference's fixture with sinks is a GGUF file with MXFP4 experts, outside this path
  *   or_topk_by_logit, or_softmax_z       pinned by what the definition fixes: the first K of the row sorted by (logit desc, id asc) is
  *                                        unique, so the heap restatement is checked against an independent full sort (numpy
  *                                        lexsort) on normal, heavily tied and signed-zero rows, K from 1 to the row (the shapes of
