@@ -446,6 +446,7 @@ static int bench_attn_typed(rd_device *d, int kv_type, int n_seq, const int *len
         std::vector<int> start, slots((size_t)g->rows), lens((size_t)g->rows);
         for (int i = 0; i < g->rows; i++) slots[(size_t)i] = r0 + i, lens[(size_t)i] = len[r0 + i];
         build_attn_worklist(lens.data(), nullptr, G, g->rows, n_kv, items, start);
+        attn_pad_items(items); // launched as the step launches it
         g->nItems = (int)items.size();
         RC(g->L.alloc(sizeof(int) * lens.size()));
         RC(g->S.alloc(sizeof(int) * slots.size()));
@@ -472,11 +473,11 @@ static int bench_attn_typed(rd_device *d, int kv_type, int n_seq, const int *len
             Group &g = *groups[gi];
             if (timed) (void)d->hip->EventRecord(evp[(t * nG + gi) * 2], d->stream);
             if (i8)
-                rc = d->launch(d->k.attn_partial_i8, (unsigned)g.nItems, 1, 1, 64, (const void *)g.I.p, (const int *)g.L.p, (const int *)g.S.p, (const int *)T.p,
+                rc = d->launch(d->k.attn_partial_i8, (unsigned)(g.nItems / ATTN_BLOCK_WAVES), 1, 1, 64 * ATTN_BLOCK_WAVES, (const void *)g.I.p, (const int *)g.L.p, (const int *)g.S.p, (const int *)T.p,
                                maxBlocks, (const signed char *)Kp.p, (const signed char *)Vp.p, (const float *)Ksc.p, (const float *)Vsc.p,
                                (const float *)((const float *)Q.p + (size_t)g.r0 * qd), g.P.as<float>(), n_h, n_kv, hd, scale, softcap, 0);
             else
-                rc = d->launch(d->k.attn_partial, (unsigned)g.nItems, 1, 1, 64, (const void *)g.I.p, (const int *)g.L.p, (const int *)g.S.p, (const int *)T.p, maxBlocks,
+                rc = d->launch(d->k.attn_partial, (unsigned)(g.nItems / ATTN_BLOCK_WAVES), 1, 1, 64 * ATTN_BLOCK_WAVES, (const void *)g.I.p, (const int *)g.L.p, (const int *)g.S.p, (const int *)T.p, maxBlocks,
                                (const uint16_t *)Kp.p, (const uint16_t *)Vp.p, (const float *)((const float *)Q.p + (size_t)g.r0 * qd), g.P.as<float>(), n_h, n_kv, hd,
                                scale, softcap, 0);
             if (timed) (void)d->hip->EventRecord(evp[(t * nG + gi) * 2 + 1], d->stream);

@@ -113,6 +113,14 @@ constexpr int ATTN_RANGE_INTS = 3; // per (row, kv head): first item, one past t
 constexpr int ATTN_DEEP_MAX_ITEMS = 1024;
 // A step's work list is launched padded to a multiple of this many items (one per compute unit) with items whose row is -1
 constexpr int ATTN_LIST_PAD = 256;
+// The step launches the attention kernels with this many waves a block, each on its own item (= RD_ATTN_BLOCK_WAVES of the
+// kernels; the kernel-level entry points launch their unpadded lists one wave a block)
+constexpr int ATTN_BLOCK_WAVES = 4;
+static_assert(ATTN_LIST_PAD % ATTN_BLOCK_WAVES == 0, "a padded list fills whole blocks");
+// Pads a work list for launching: grid = items / ATTN_BLOCK_WAVES blocks of 64 * ATTN_BLOCK_WAVES threads.
+inline void attn_pad_items(std::vector<AttnItemH> &items) {
+    items.resize((items.size() + ATTN_LIST_PAD - 1) / ATTN_LIST_PAD * ATTN_LIST_PAD, AttnItemH{-1, 0, 0, 0});
+}
 hipFunction_t attn_partial_kernel(const struct rd_device *d, bool i8, bool grouped, size_t n_items);
 constexpr int TOPK_MAX = 1024; // = RD_TOPK_MAX of the top-K kernels
 constexpr int TOPK_CAP = 4096, TOPK_BINS = 2048, TOPK_CHUNK = 16384; // = RD_TOPK_CAP, RD_TOPK_BINS, RD_TOPK_CHUNK

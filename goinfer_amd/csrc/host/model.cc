@@ -813,14 +813,14 @@ int launch_attn_partial(rd_model *m, const LayerW &l) {
     rd_device *d = m->d;
     const rd_model_desc &c = m->desc;
     const int nH = c.n_heads, nKV = c.n_kv_heads, HD = c.head_dim, li = l.window > 0 ? 1 : 0;
-    const size_t nItems = m->last_items[li];
+    const size_t nItems = m->last_items[li]; // padded to ATTN_LIST_PAD: a multiple of the waves a block runs
     const bool grouped = m->last_grouped[li];
     const void *items = (const int *)m->items + (size_t)li * m->list_ints;
     if (m->kv_type == RD_KV_I8)
-        return d->launch(attn_partial_kernel(d, true, grouped, nItems), (unsigned)nItems, 1, 1, 64, items, (const int *)m->rowLen, (const int *)m->rowSlot,
+        return d->launch(attn_partial_kernel(d, true, grouped, nItems), (unsigned)(nItems / ATTN_BLOCK_WAVES), 1, 1, 64 * ATTN_BLOCK_WAVES, items, (const int *)m->rowLen, (const int *)m->rowSlot,
                          (const int *)m->tables, m->blocks_per_slot, (const signed char *)l.Kp, (const signed char *)l.Vp, (const float *)l.Ksc,
                          (const float *)l.Vsc, (const float *)m->qbuf, m->part, nH, nKV, HD, c.attn_scale, c.attn_softcap, l.window);
-    return d->launch(attn_partial_kernel(d, false, grouped, nItems), (unsigned)nItems, 1, 1, 64, items, (const int *)m->rowLen, (const int *)m->rowSlot,
+    return d->launch(attn_partial_kernel(d, false, grouped, nItems), (unsigned)(nItems / ATTN_BLOCK_WAVES), 1, 1, 64 * ATTN_BLOCK_WAVES, items, (const int *)m->rowLen, (const int *)m->rowSlot,
                      (const int *)m->tables, m->blocks_per_slot, (const uint16_t *)l.Kp, (const uint16_t *)l.Vp, (const float *)m->qbuf, m->part,
                      nH, nKV, HD, c.attn_scale, c.attn_softcap, l.window);
 }
@@ -1072,7 +1072,7 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
         RC(build_attn_items(m, B, slot, pos, items[li], start[li], &grouped, li ? m->window : 0));
         // The list is launched padded to a multiple of ATTN_LIST_PAD with items that name no row (their waves leave at once):
         // the launch then keeps its shape over many steps of a growing batch, which is what lets a captured graph be replayed.
-        items[li].resize((items[li].size() + ATTN_LIST_PAD - 1) / ATTN_LIST_PAD * ATTN_LIST_PAD, AttnItemH{-1, 0, 0, 0});
+        attn_pad_items(items[li]);
         m->last_items[li] = items[li].size(), m->last_grouped[li] = grouped;
     }
     // Stage the step's metadata (and host embeddings) in pinned memory and upload it asynchronously. A slot is reused only

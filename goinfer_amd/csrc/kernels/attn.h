@@ -242,6 +242,8 @@ __device__ __forceinline__ float fast_tanh(float x) {
 
 __device__ __forceinline__ float ld_part(const float *p) { return *p; }
 
+// the attention kernels run with one wave a block or with this many, each wave on its own item
+#define RD_ATTN_BLOCK_WAVES 4
 struct AttnItem {
     int row, kvh, b0, b1; // first row, kv head (low 16 bits) and number of rows (high 16 bits), block range [b0,b1) of the sequence
 };
@@ -270,6 +272,16 @@ __device__ __forceinline__ half8_t kv8_to_half8(uint32_t w0, uint32_t w1) {
     v0 += off, v1 += off, v2 += off, v3 += off;
     return (half8_t){v0.x, v0.y, v1.x, v1.y, v2.x, v2.y, v3.x, v3.y};
 }
+
+// A wave's lanes exchange the probabilities through their own 2 KB of LDS: one wave's LDS operations complete in the order they
+// were issued, so ordering them for the compiler (and draining the wave's own LDS counter) is all the hand-off needs. A block-wide
+// barrier would be wrong here: the waves of a block work on different items with different trip counts.
+#define RD_WAVE_LDS_SYNC()                                       \
+    do {                                                         \
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   \
+        __builtin_amdgcn_wave_barrier();                         \
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");   \
+    } while (0)
 
 // The work on one unit of 32 keys whose K and V fragments (KF, VF) and int8 scales (KS, VS) are in registers: scores, online softmax
 // with a lazy rescale of the running output (only when some row's maximum moved: a factor of exactly 1 changes nothing; a key
@@ -333,14 +345,14 @@ __device__ __forceinline__ half8_t kv8_to_half8(uint32_t w0, uint32_t w1) {
         _Pragma("unroll")                                                                                                                              \
                 for (int r = 0; r < 4; r++) O[ct][r] *= alpha[r];                                                                                      \
         }                                                                                                                                              \
-        __syncthreads();                                                                                                                               \
+        RD_WAVE_LDS_SYNC();                                                                                                                                 \
         half8_t phi, plo;                                                                                                                              \
         {                                                                                                                                              \
             uint4_t a = *(const uint4_t *)(pbuf + l16 * 32 + lg * 8), bq = *(const uint4_t *)(pbuf + 512 + l16 * 32 + lg * 8);                         \
             __builtin_memcpy(&phi, &a, 16);                                                                                                            \
             __builtin_memcpy(&plo, &bq, 16);                                                                                                           \
         }                                                                                                                                              \
-        __syncthreads();                                                                                                                               \
+        RD_WAVE_LDS_SYNC();                                                                                                                                 \
         _Pragma("unroll")                                                                                                                              \
         for (int ct = 0; ct < NCT; ct++) {                                                                                                             \
             half8_t vb;                                                                                                                                \
@@ -362,11 +374,14 @@ __device__ __forceinline__ void attn_partial_body(const AttnItem *__restrict__ i
     constexpr int NC = HD / 32, NCT = HD / 16;
     constexpr int KL = I8 ? NC / 2 : NC, VL = I8 ? NCT / 2 : NCT; // 16-byte loads per key tile of K, per 32 keys of V
     constexpr int ELEM = I8 ? 1 : 2;
-    AttnItem it = items[blockIdx.x];
+    // a block is one wave, or several waves on consecutive items of the list (a step's padded list: fewer, fatter blocks to dispatch)
+    const int item = blockIdx.x * (int)(blockDim.x >> 6) + (int)(threadIdx.x >> 6);
+    pbuf += (threadIdx.x >> 6) * 1024;
+    AttnItem it = items[item];
     if (it.row < 0) return; // padding of the work list: names no row
     const int nrows = ROWS ? it.kvh >> 16 : 1;
     it.kvh &= 0xffff;
-    const int lane = threadIdx.x, l16 = lane & 15, lg = lane >> 4;
+    const int lane = threadIdx.x & 63, l16 = lane & 15, lg = lane >> 4;
     const int G = nH / nKV, len0 = rowLen[it.row];
     const int len = len0 + nrows - 1; // the longest row's: the unit loop runs to it
     const int *tab = tables + (size_t)rowSlot[it.row] * tabStride;
@@ -474,7 +489,7 @@ __device__ __forceinline__ void attn_partial_body(const AttnItem *__restrict__ i
         for (int o = 8; o > 0; o >>= 1) lrun[r] += __shfl_xor(lrun[r], o, 64);
         int g = 4 * lg + r;
         if (ROWS ? g < nrows * G : g < G) {
-            float *dst = part + ((size_t)blockIdx.x * (ROWS ? 16 : G) + g) * (HD + 2);
+            float *dst = part + ((size_t)item * (ROWS ? 16 : G) + g) * (HD + 2);
 #pragma unroll
             for (int ct = 0; ct < NCT; ct++) dst[ct * 16 + l16] = O[ct][r];
             if (l16 == 0) dst[HD] = mrun[r], dst[HD + 1] = lrun[r];
@@ -482,12 +497,12 @@ __device__ __forceinline__ void attn_partial_body(const AttnItem *__restrict__ i
     }
 }
 
-extern "C" __global__ __launch_bounds__(64) void rd_k_attn_partial(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
+extern "C" __global__ __launch_bounds__(64 * RD_ATTN_BLOCK_WAVES) void rd_k_attn_partial(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
                                                                    const int *__restrict__ rowSlot, const int *__restrict__ tables, int tabStride,
                                                                    const uint16_t *__restrict__ Kp, const uint16_t *__restrict__ Vp,
                                                                    const float *__restrict__ q, float *__restrict__ part, int nH, int nKV, int HD,
                                                                    float scale, float softcap, int window) {
-    __shared__ half_t pbuf[1024];
+    __shared__ half_t pbuf[RD_ATTN_BLOCK_WAVES * 1024];
     if (HD == 128)
         attn_partial_body<128, false>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, window, pbuf);
     else
@@ -495,13 +510,13 @@ extern "C" __global__ __launch_bounds__(64) void rd_k_attn_partial(const AttnIte
 }
 
 // The same over the int8 cache: half the key/value bytes per launch.
-extern "C" __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void rd_k_attn_partial_i8(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
+extern "C" __global__ __launch_bounds__(64 * RD_ATTN_BLOCK_WAVES) __attribute__((amdgpu_waves_per_eu(3, 3))) void rd_k_attn_partial_i8(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
                                                                       const int *__restrict__ rowSlot, const int *__restrict__ tables, int tabStride,
                                                                       const signed char *__restrict__ Kp, const signed char *__restrict__ Vp,
                                                                       const float *__restrict__ Ksc, const float *__restrict__ Vsc,
                                                                       const float *__restrict__ q, float *__restrict__ part, int nH, int nKV, int HD,
                                                                       float scale, float softcap, int window) {
-    __shared__ half_t pbuf[1024];
+    __shared__ half_t pbuf[RD_ATTN_BLOCK_WAVES * 1024];
     if (HD == 128)
         attn_partial_body<128, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, Ksc, Vsc, q, part, nH, nKV, scale, softcap, window, pbuf);
     else
@@ -509,25 +524,25 @@ extern "C" __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3
 }
 
 // The same two kernels with two units in flight per wave (see DEEP above), one wave per SIMD.
-extern "C" __global__ __launch_bounds__(64) void rd_k_attn_partial_deep(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
+extern "C" __global__ __launch_bounds__(64 * RD_ATTN_BLOCK_WAVES) void rd_k_attn_partial_deep(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
                                                                         const int *__restrict__ rowSlot, const int *__restrict__ tables, int tabStride,
                                                                         const uint16_t *__restrict__ Kp, const uint16_t *__restrict__ Vp,
                                                                         const float *__restrict__ q, float *__restrict__ part, int nH, int nKV, int HD,
                                                                         float scale, float softcap, int window) {
-    __shared__ half_t pbuf[1024];
+    __shared__ half_t pbuf[RD_ATTN_BLOCK_WAVES * 1024];
     if (HD == 128)
         attn_partial_body<128, false, false, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, window, pbuf);
     else
         attn_partial_body<64, false, false, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, window, pbuf);
 }
 
-extern "C" __global__ __launch_bounds__(64) void rd_k_attn_partial_deep_i8(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
+extern "C" __global__ __launch_bounds__(64 * RD_ATTN_BLOCK_WAVES) void rd_k_attn_partial_deep_i8(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
                                                                       const int *__restrict__ rowSlot, const int *__restrict__ tables, int tabStride,
                                                                       const signed char *__restrict__ Kp, const signed char *__restrict__ Vp,
                                                                       const float *__restrict__ Ksc, const float *__restrict__ Vsc,
                                                                       const float *__restrict__ q, float *__restrict__ part, int nH, int nKV, int HD,
                                                                       float scale, float softcap, int window) {
-    __shared__ half_t pbuf[1024];
+    __shared__ half_t pbuf[RD_ATTN_BLOCK_WAVES * 1024];
     if (HD == 128)
         attn_partial_body<128, true, false, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, Ksc, Vsc, q, part, nH, nKV, scale, softcap, window, pbuf);
     else
@@ -535,25 +550,25 @@ extern "C" __global__ __launch_bounds__(64) void rd_k_attn_partial_deep_i8(const
 }
 
 // Items of several positions each (see ROWS above): steps that carry more than one row of a sequence — prompt passes, verification.
-extern "C" __global__ __launch_bounds__(64) void rd_k_attn_partial_rows(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
+extern "C" __global__ __launch_bounds__(64 * RD_ATTN_BLOCK_WAVES) void rd_k_attn_partial_rows(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
                                                                         const int *__restrict__ rowSlot, const int *__restrict__ tables, int tabStride,
                                                                         const uint16_t *__restrict__ Kp, const uint16_t *__restrict__ Vp,
                                                                         const float *__restrict__ q, float *__restrict__ part, int nH, int nKV, int HD,
                                                                         float scale, float softcap, int window) {
-    __shared__ half_t pbuf[1024];
+    __shared__ half_t pbuf[RD_ATTN_BLOCK_WAVES * 1024];
     if (HD == 128)
         attn_partial_body<128, false, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, window, pbuf);
     else
         attn_partial_body<64, false, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, window, pbuf);
 }
 
-extern "C" __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void rd_k_attn_partial_rows_i8(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
+extern "C" __global__ __launch_bounds__(64 * RD_ATTN_BLOCK_WAVES) __attribute__((amdgpu_waves_per_eu(3, 3))) void rd_k_attn_partial_rows_i8(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
                                                                       const int *__restrict__ rowSlot, const int *__restrict__ tables, int tabStride,
                                                                       const signed char *__restrict__ Kp, const signed char *__restrict__ Vp,
                                                                       const float *__restrict__ Ksc, const float *__restrict__ Vsc,
                                                                       const float *__restrict__ q, float *__restrict__ part, int nH, int nKV, int HD,
                                                                       float scale, float softcap, int window) {
-    __shared__ half_t pbuf[1024];
+    __shared__ half_t pbuf[RD_ATTN_BLOCK_WAVES * 1024];
     if (HD == 128)
         attn_partial_body<128, true, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, Ksc, Vsc, q, part, nH, nKV, scale, softcap, window, pbuf);
     else
