@@ -473,13 +473,15 @@ static int bench_attn_typed(rd_device *d, int kv_type, int n_seq, const int *len
             Group &g = *groups[gi];
             if (timed) (void)d->hip->EventRecord(evp[(t * nG + gi) * 2], d->stream);
             if (i8)
-                rc = d->launch(d->k.attn_partial_i8, (unsigned)(g.nItems / ATTN_BLOCK_WAVES), 1, 1, 64 * ATTN_BLOCK_WAVES, (const void *)g.I.p, (const int *)g.L.p, (const int *)g.S.p, (const int *)T.p,
+                rc = d->launch(d->k.attn_partial_i8, (unsigned)g.nItems, 1, 1, 64, (const void *)g.I.p, (const int *)g.L.p, (const int *)g.S.p, (const int *)T.p,
                                maxBlocks, (const signed char *)Kp.p, (const signed char *)Vp.p, (const float *)Ksc.p, (const float *)Vsc.p,
                                (const float *)((const float *)Q.p + (size_t)g.r0 * qd), g.P.as<float>(), n_h, n_kv, hd, scale, softcap, 0);
-            else
-                rc = d->launch(d->k.attn_partial, (unsigned)(g.nItems / ATTN_BLOCK_WAVES), 1, 1, 64 * ATTN_BLOCK_WAVES, (const void *)g.I.p, (const int *)g.L.p, (const int *)g.S.p, (const int *)T.p, maxBlocks,
+            else {
+                const AttnLaunch al = attn_partial_kernel(d, false, false, (size_t)g.nItems);
+                rc = d->launch(al.f, (unsigned)g.nItems / al.waves, 1, 1, 64 * al.waves, (const void *)g.I.p, (const int *)g.L.p, (const int *)g.S.p, (const int *)T.p, maxBlocks,
                                (const uint16_t *)Kp.p, (const uint16_t *)Vp.p, (const float *)((const float *)Q.p + (size_t)g.r0 * qd), g.P.as<float>(), n_h, n_kv, hd,
                                scale, softcap, 0);
+            }
             if (timed) (void)d->hip->EventRecord(evp[(t * nG + gi) * 2 + 1], d->stream);
             if (!rc)
                 rc = d->launch(d->k.attn_combine, (unsigned)n_h, (unsigned)g.rows, 1, (unsigned)(ATTN_PIECES * hd / 4), (const float *)g.P.p, (const int *)g.St.p, G,

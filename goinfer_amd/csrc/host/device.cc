@@ -99,6 +99,7 @@ static const KName kNames[] = {
     {"rd_k_qkv_rope_store", &Kernels::qkv_rope_store},
     {"rd_k_rope_table", &Kernels::rope_table},
     {"rd_k_attn_partial", &Kernels::attn_partial},
+    {"rd_k_attn_partial_wide", &Kernels::attn_partial_wide},
     {"rd_k_kv_store_i8", &Kernels::kv_store_i8},
     {"rd_k_qkv_rope_store_i8", &Kernels::qkv_rope_store_i8},
     {"rd_k_attn_partial_i8", &Kernels::attn_partial_i8},
@@ -247,10 +248,13 @@ int launch_topk(rd_device *d, const float *logits, int rows, int V, int k, float
     return rc;
 }
 
-hipFunction_t attn_partial_kernel(const rd_device *d, bool i8, bool grouped, size_t n_items) {
-    if (grouped) return i8 ? d->k.attn_partial_rows_i8 : d->k.attn_partial_rows;
-    if (n_items <= (size_t)ATTN_DEEP_MAX_ITEMS && !getenv("ROCMDECODE_NO_DEEP_ATTN")) return i8 ? d->k.attn_partial_deep_i8 : d->k.attn_partial_deep;
-    return i8 ? d->k.attn_partial_i8 : d->k.attn_partial;
+AttnLaunch attn_partial_kernel(const rd_device *d, bool i8, bool grouped, size_t n_items) {
+    if (grouped) return {i8 ? d->k.attn_partial_rows_i8 : d->k.attn_partial_rows, 1u};
+    if (n_items <= (size_t)ATTN_DEEP_MAX_ITEMS && !getenv("ROCMDECODE_NO_DEEP_ATTN")) return {i8 ? d->k.attn_partial_deep_i8 : d->k.attn_partial_deep, 1u};
+    if (i8) return {d->k.attn_partial_i8, 1u};
+    if (n_items >= (size_t)ATTN_WIDE_MIN_ITEMS && n_items % ATTN_BLOCK_WAVES == 0 && !getenv("ROCMDECODE_NO_WIDE_ATTN"))
+        return {d->k.attn_partial_wide, (unsigned)ATTN_BLOCK_WAVES};
+    return {d->k.attn_partial, 1u};
 }
 
 bool build_attn_worklist(const int *len, const int *slot, int G, int rows, int n_kv, std::vector<AttnItemH> &items, std::vector<int> &ranges,

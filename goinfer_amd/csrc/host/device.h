@@ -39,7 +39,7 @@ struct Kernels {
     hipFunction_t gemm8_qkv[3][3]; // the q|k|v projection with RoPE and the KV store in its epilogue, indexed like gemm8
     hipFunction_t gemm8_q4k_gateup, gemm8_q4k_gateup_gelu, add_one, moe_gemv_w4a8, moe_gemv_w4a8_gateup, retile_w4a8_gv, rope_table;
     hipFunction_t dequant_q5k, retile_q5k, gemm_q5k, dequant_q6k, retile_q6k, gemm_q6k;
-    hipFunction_t kv_store, kv_read, qkv_rope_store, attn_partial, attn_combine, attn_combine_quant;
+    hipFunction_t kv_store, kv_read, qkv_rope_store, attn_partial, attn_partial_wide, attn_combine, attn_combine_quant;
     hipFunction_t kv_store_i8, qkv_rope_store_i8, attn_partial_i8, attn_partial_rows, attn_partial_rows_i8, attn_partial_deep, attn_partial_deep_i8, topk_rows, topk_hist, topk_pick, topk_finish;
     hipFunction_t rmsnorm, rope, argmax_rows, argmax_final, matmul_f32, moe_route, moe_swiglu_quant, moe_fold, embed_rows, copy16, unpanel_q4k, fill_f16, fill_f32;
 };
@@ -113,15 +113,20 @@ constexpr int ATTN_RANGE_INTS = 3; // per (row, kv head): first item, one past t
 constexpr int ATTN_DEEP_MAX_ITEMS = 1024;
 // A step's work list is launched padded to a multiple of this many items (one per compute unit) with items whose row is -1
 constexpr int ATTN_LIST_PAD = 256;
-// The step launches the attention kernels with this many waves a block, each on its own item (= RD_ATTN_BLOCK_WAVES of the
-// kernels; the kernel-level entry points launch their unpadded lists one wave a block)
-constexpr int ATTN_BLOCK_WAVES = 4;
+// Waves a block of rd_k_attn_partial_wide (= RD_ATTN_BLOCK_WAVES of the kernels), which takes the lists of at least
+// ATTN_WIDE_MIN_ITEMS items (two waves for every SIMD of the chip)
+constexpr int ATTN_BLOCK_WAVES = 4, ATTN_WIDE_MIN_ITEMS = 2048;
 static_assert(ATTN_LIST_PAD % ATTN_BLOCK_WAVES == 0, "a padded list fills whole blocks");
-// Pads a work list for launching: grid = items / ATTN_BLOCK_WAVES blocks of 64 * ATTN_BLOCK_WAVES threads.
+// Pads a work list for launching (whole blocks whatever kernel takes it).
 inline void attn_pad_items(std::vector<AttnItemH> &items) {
     items.resize((items.size() + ATTN_LIST_PAD - 1) / ATTN_LIST_PAD * ATTN_LIST_PAD, AttnItemH{-1, 0, 0, 0});
 }
-hipFunction_t attn_partial_kernel(const struct rd_device *d, bool i8, bool grouped, size_t n_items);
+// The attention kernel for a (padded) work list of n_items and the waves it runs a block: grid = n_items / waves, block = 64 * waves.
+struct AttnLaunch {
+    hipFunction_t f;
+    unsigned waves;
+};
+AttnLaunch attn_partial_kernel(const struct rd_device *d, bool i8, bool grouped, size_t n_items);
 constexpr int TOPK_MAX = 1024; // = RD_TOPK_MAX of the top-K kernels
 constexpr int TOPK_CAP = 4096, TOPK_BINS = 2048, TOPK_CHUNK = 16384; // = RD_TOPK_CAP, RD_TOPK_BINS, RD_TOPK_CHUNK
 // Scratch of the top-K over `rows` rows of width V (device memory the caller owns): per-chunk histograms and maxima, candidate

@@ -813,14 +813,15 @@ int launch_attn_partial(rd_model *m, const LayerW &l) {
     rd_device *d = m->d;
     const rd_model_desc &c = m->desc;
     const int nH = c.n_heads, nKV = c.n_kv_heads, HD = c.head_dim, li = l.window > 0 ? 1 : 0;
-    const size_t nItems = m->last_items[li]; // padded to ATTN_LIST_PAD: a multiple of the waves a block runs
+    const size_t nItems = m->last_items[li]; // padded to ATTN_LIST_PAD: whole blocks for any of the kernels
     const bool grouped = m->last_grouped[li];
     const void *items = (const int *)m->items + (size_t)li * m->list_ints;
+    const AttnLaunch al = attn_partial_kernel(d, m->kv_type == RD_KV_I8, grouped, nItems);
     if (m->kv_type == RD_KV_I8)
-        return d->launch(attn_partial_kernel(d, true, grouped, nItems), (unsigned)(nItems / ATTN_BLOCK_WAVES), 1, 1, 64 * ATTN_BLOCK_WAVES, items, (const int *)m->rowLen, (const int *)m->rowSlot,
+        return d->launch(al.f, (unsigned)(nItems / al.waves), 1, 1, 64 * al.waves, items, (const int *)m->rowLen, (const int *)m->rowSlot,
                          (const int *)m->tables, m->blocks_per_slot, (const signed char *)l.Kp, (const signed char *)l.Vp, (const float *)l.Ksc,
                          (const float *)l.Vsc, (const float *)m->qbuf, m->part, nH, nKV, HD, c.attn_scale, c.attn_softcap, l.window);
-    return d->launch(attn_partial_kernel(d, false, grouped, nItems), (unsigned)(nItems / ATTN_BLOCK_WAVES), 1, 1, 64 * ATTN_BLOCK_WAVES, items, (const int *)m->rowLen, (const int *)m->rowSlot,
+    return d->launch(al.f, (unsigned)(nItems / al.waves), 1, 1, 64 * al.waves, items, (const int *)m->rowLen, (const int *)m->rowSlot,
                      (const int *)m->tables, m->blocks_per_slot, (const uint16_t *)l.Kp, (const uint16_t *)l.Vp, (const float *)m->qbuf, m->part,
                      nH, nKV, HD, c.attn_scale, c.attn_softcap, l.window);
 }

@@ -517,12 +517,13 @@ static int attn_ragged_typed(rd_device *d, int kv_type, int n_seq, const int *le
         RC(d->h2d(S2.p, slots.data(), sizeof(int) * (size_t)rows));
         RC(d->h2d(I2.p, items.data(), sizeof(AttnItemH) * items.size()));
         RC(d->h2d(St2.p, start.data(), sizeof(int) * start.size()));
+        const AttnLaunch al = attn_partial_kernel(d, i8, grouped, items.size());
         if (i8)
-            RC(d->launch(attn_partial_kernel(d, true, grouped, items.size()), (unsigned)(items.size() / ATTN_BLOCK_WAVES), 1, 1, 64 * ATTN_BLOCK_WAVES, (const void *)I2.p, (const int *)L2.p,
+            RC(d->launch(al.f, (unsigned)(items.size() / al.waves), 1, 1, 64 * al.waves, (const void *)I2.p, (const int *)L2.p,
                          (const int *)S2.p, (const int *)T.p, maxBlocks, (const signed char *)Kp.p, (const signed char *)Vp.p, (const float *)Ksc.p,
                          (const float *)Vsc.p, (const float *)Q2.p, P2.as<float>(), n_h, n_kv, hd, scale, softcap, window));
         else
-            RC(d->launch(attn_partial_kernel(d, false, grouped, items.size()), (unsigned)(items.size() / ATTN_BLOCK_WAVES), 1, 1, 64 * ATTN_BLOCK_WAVES, (const void *)I2.p, (const int *)L2.p,
+            RC(d->launch(al.f, (unsigned)(items.size() / al.waves), 1, 1, 64 * al.waves, (const void *)I2.p, (const int *)L2.p,
                          (const int *)S2.p, (const int *)T.p, maxBlocks, (const uint16_t *)Kp.p, (const uint16_t *)Vp.p, (const float *)Q2.p, P2.as<float>(), n_h,
                          n_kv, hd, scale, softcap, window));
         RC(d->launch(d->k.attn_combine, (unsigned)n_h, (unsigned)rows, 1, (unsigned)(ATTN_PIECES * hd / 4), (const float *)P2.p, (const int *)St2.p, partRows,

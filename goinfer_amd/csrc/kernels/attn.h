@@ -242,7 +242,7 @@ __device__ __forceinline__ float fast_tanh(float x) {
 
 __device__ __forceinline__ float ld_part(const float *p) { return *p; }
 
-// the attention kernels run with one wave a block or with this many, each wave on its own item
+// rd_k_attn_partial_wide runs this many waves a block, each wave on its own item; the other attention kernels one
 #define RD_ATTN_BLOCK_WAVES 4
 struct AttnItem {
     int row, kvh, b0, b1; // first row, kv head (low 16 bits) and number of rows (high 16 bits), block range [b0,b1) of the sequence
@@ -497,7 +497,23 @@ __device__ __forceinline__ void attn_partial_body(const AttnItem *__restrict__ i
     }
 }
 
-extern "C" __global__ __launch_bounds__(64 * RD_ATTN_BLOCK_WAVES) void rd_k_attn_partial(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
+extern "C" __global__ __launch_bounds__(64) void rd_k_attn_partial(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
+                                                                   const int *__restrict__ rowSlot, const int *__restrict__ tables, int tabStride,
+                                                                   const uint16_t *__restrict__ Kp, const uint16_t *__restrict__ Vp,
+                                                                   const float *__restrict__ q, float *__restrict__ part, int nH, int nKV, int HD,
+                                                                   float scale, float softcap, int window) {
+    __shared__ half_t pbuf[1024];
+    if (HD == 128)
+        attn_partial_body<128, false>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, window, pbuf);
+    else
+        attn_partial_body<64, false>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, window, pbuf);
+}
+
+// The same with four waves a block, each on its own item (grid = items / 4; the list is padded to whole blocks): for work lists of
+// several waves per SIMD, where 4 096 one-wave blocks take the dispatcher longer than 1 024 fatter ones (61.0 against 62.2 us on one
+// machine at 32 sequences of 512 to 4 096 keys; no difference at 16 384 items). A short list wants its waves spread over the
+// compute units instead and keeps one wave a block.
+extern "C" __global__ __launch_bounds__(64 * RD_ATTN_BLOCK_WAVES) void rd_k_attn_partial_wide(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
                                                                    const int *__restrict__ rowSlot, const int *__restrict__ tables, int tabStride,
                                                                    const uint16_t *__restrict__ Kp, const uint16_t *__restrict__ Vp,
                                                                    const float *__restrict__ q, float *__restrict__ part, int nH, int nKV, int HD,
@@ -510,13 +526,13 @@ extern "C" __global__ __launch_bounds__(64 * RD_ATTN_BLOCK_WAVES) void rd_k_attn
 }
 
 // The same over the int8 cache: half the key/value bytes per launch.
-extern "C" __global__ __launch_bounds__(64 * RD_ATTN_BLOCK_WAVES) __attribute__((amdgpu_waves_per_eu(3, 3))) void rd_k_attn_partial_i8(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
+extern "C" __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void rd_k_attn_partial_i8(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
                                                                       const int *__restrict__ rowSlot, const int *__restrict__ tables, int tabStride,
                                                                       const signed char *__restrict__ Kp, const signed char *__restrict__ Vp,
                                                                       const float *__restrict__ Ksc, const float *__restrict__ Vsc,
                                                                       const float *__restrict__ q, float *__restrict__ part, int nH, int nKV, int HD,
                                                                       float scale, float softcap, int window) {
-    __shared__ half_t pbuf[RD_ATTN_BLOCK_WAVES * 1024];
+    __shared__ half_t pbuf[1024];
     if (HD == 128)
         attn_partial_body<128, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, Ksc, Vsc, q, part, nH, nKV, scale, softcap, window, pbuf);
     else
@@ -524,25 +540,25 @@ extern "C" __global__ __launch_bounds__(64 * RD_ATTN_BLOCK_WAVES) __attribute__(
 }
 
 // The same two kernels with two units in flight per wave (see DEEP above), one wave per SIMD.
-extern "C" __global__ __launch_bounds__(64 * RD_ATTN_BLOCK_WAVES) void rd_k_attn_partial_deep(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
+extern "C" __global__ __launch_bounds__(64) void rd_k_attn_partial_deep(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
                                                                         const int *__restrict__ rowSlot, const int *__restrict__ tables, int tabStride,
                                                                         const uint16_t *__restrict__ Kp, const uint16_t *__restrict__ Vp,
                                                                         const float *__restrict__ q, float *__restrict__ part, int nH, int nKV, int HD,
                                                                         float scale, float softcap, int window) {
-    __shared__ half_t pbuf[RD_ATTN_BLOCK_WAVES * 1024];
+    __shared__ half_t pbuf[1024];
     if (HD == 128)
         attn_partial_body<128, false, false, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, window, pbuf);
     else
         attn_partial_body<64, false, false, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, window, pbuf);
 }
 
-extern "C" __global__ __launch_bounds__(64 * RD_ATTN_BLOCK_WAVES) void rd_k_attn_partial_deep_i8(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
+extern "C" __global__ __launch_bounds__(64) void rd_k_attn_partial_deep_i8(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
                                                                       const int *__restrict__ rowSlot, const int *__restrict__ tables, int tabStride,
                                                                       const signed char *__restrict__ Kp, const signed char *__restrict__ Vp,
                                                                       const float *__restrict__ Ksc, const float *__restrict__ Vsc,
                                                                       const float *__restrict__ q, float *__restrict__ part, int nH, int nKV, int HD,
                                                                       float scale, float softcap, int window) {
-    __shared__ half_t pbuf[RD_ATTN_BLOCK_WAVES * 1024];
+    __shared__ half_t pbuf[1024];
     if (HD == 128)
         attn_partial_body<128, true, false, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, Ksc, Vsc, q, part, nH, nKV, scale, softcap, window, pbuf);
     else
@@ -550,25 +566,25 @@ extern "C" __global__ __launch_bounds__(64 * RD_ATTN_BLOCK_WAVES) void rd_k_attn
 }
 
 // Items of several positions each (see ROWS above): steps that carry more than one row of a sequence — prompt passes, verification.
-extern "C" __global__ __launch_bounds__(64 * RD_ATTN_BLOCK_WAVES) void rd_k_attn_partial_rows(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
+extern "C" __global__ __launch_bounds__(64) void rd_k_attn_partial_rows(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
                                                                         const int *__restrict__ rowSlot, const int *__restrict__ tables, int tabStride,
                                                                         const uint16_t *__restrict__ Kp, const uint16_t *__restrict__ Vp,
                                                                         const float *__restrict__ q, float *__restrict__ part, int nH, int nKV, int HD,
                                                                         float scale, float softcap, int window) {
-    __shared__ half_t pbuf[RD_ATTN_BLOCK_WAVES * 1024];
+    __shared__ half_t pbuf[1024];
     if (HD == 128)
         attn_partial_body<128, false, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, window, pbuf);
     else
         attn_partial_body<64, false, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, nullptr, nullptr, q, part, nH, nKV, scale, softcap, window, pbuf);
 }
 
-extern "C" __global__ __launch_bounds__(64 * RD_ATTN_BLOCK_WAVES) __attribute__((amdgpu_waves_per_eu(3, 3))) void rd_k_attn_partial_rows_i8(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
+extern "C" __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(3, 3))) void rd_k_attn_partial_rows_i8(const AttnItem *__restrict__ items, const int *__restrict__ rowLen,
                                                                       const int *__restrict__ rowSlot, const int *__restrict__ tables, int tabStride,
                                                                       const signed char *__restrict__ Kp, const signed char *__restrict__ Vp,
                                                                       const float *__restrict__ Ksc, const float *__restrict__ Vsc,
                                                                       const float *__restrict__ q, float *__restrict__ part, int nH, int nKV, int HD,
                                                                       float scale, float softcap, int window) {
-    __shared__ half_t pbuf[RD_ATTN_BLOCK_WAVES * 1024];
+    __shared__ half_t pbuf[1024];
     if (HD == 128)
         attn_partial_body<128, true, true>(items, rowLen, rowSlot, tables, tabStride, Kp, Vp, Ksc, Vsc, q, part, nH, nKV, scale, softcap, window, pbuf);
     else
