@@ -153,9 +153,13 @@ def run_c4(args):
             a[1] += n
     kern = "attn_partial"
     single_ms = prof[kern][0] / prof[kern][1]  # an event pair around every launch: carries the events' own 2-3 us
-    # the kernel's average launch duration proper: every layer's launch back to back between one pair of events (three steps' worth)
+    # every layer's launch back to back between one pair of events: the kernel with its work list, tables and q still in L2
     chain = [res.model.bench_attn_chain(slots, pos_prof + rep, ids0) for rep in range(3)]
-    avg_ms = float(np.mean([c[0] for c in chain]))
+    chain_ms = float(np.mean([c[0] for c in chain]))
+    # the kernel's average launch duration where it runs: whole steps against the same steps without their attention launches,
+    # each step between its own pair of events. This is the figure the profiler's kernel duration agrees with.
+    avg_ms, _ = res.model.bench_attn_in_step(slots, pos_prof + 2, ids0, 8)
+    kernel_name = res.model.attn_kernel_name()  # the variant this work list takes (wide blocks, two units in flight, int8 cache)
     # per launch (one layer): every sequence's K and V rows once (f16, or int8 and their scales), plus q in and partial results out
     G = cfg["n_heads"] // cfg["n_kv"]
     kv_launch = float((pos_prof + 2).sum()) * kv_pos_bytes / cfg["n_layers"]
@@ -164,10 +168,13 @@ def run_c4(args):
     traffic, t_ratio, t_src = counter_traffic("%s/%s/%s" % (kern, cfg["name"], args.kv), kv_launch + q_launch)
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": traffic, "traffic_ratio": t_ratio, "traffic_source": t_src,
-                "kernel": "rd_k_attn_partial" if args.kv == "f16" else "rd_k_attn_partial_i8", "avg_launch_ms": round(avg_ms, 5),
+                "kernel": kernel_name, "avg_launch_ms": round(avg_ms, 5),
                 "avg_launch_ms_event_pair_per_launch": round(single_ms, 5),
-                "timing": "one pair of HIP events on the launch stream around the kernel's launches of all layers, back to back, at the context lengths right "
-                          "after the timed steps (3 x %d launches); an event pair around every single launch reads 2-3 us more (avg_launch_ms_event_pair_per_launch)" % chain[0][1],
+                "avg_launch_ms_back_to_back": round(chain_ms, 5),
+                "timing": "HIP events on the launch stream around whole steps at the context lengths right after the timed ones: (a step - the same step "
+                          "without its attention launches) / layers, 8 pairs of steps; agrees with rocprofv3's kernel duration. The same kernel launched "
+                          "back to back for all layers between one pair of events (its work list, tables and q then stay in L2) reads about 2 us less "
+                          "(avg_launch_ms_back_to_back); an event pair around every single launch about 2 us more (avg_launch_ms_event_pair_per_launch)",
                 "algorithmic_bytes_per_launch": int(kv_launch + q_launch),
                 "step_frac": round(step_gbs / HBM_PEAK_GBS, 4)}
     classes = {k: {"ms_per_step": round(v[0] / 3, 4), "launches_per_step": v[1] // 3} for k, v in prof.items()}

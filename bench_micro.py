@@ -244,7 +244,7 @@ def run_c3(args):
     per_launch = (kv_bytes + nseq * nH * hd * 4) / 2
     out["roofline"] = {"bound": "hbm", "achieved": round(per_launch / (tp / 2) / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                        "frac": round(per_launch / (tp / 2) / 1e6 / HBM_PEAK_GBS, 4),
-                       "kernel": "rd_k_attn_partial" if kv == "f16" else "rd_k_attn_partial_i8",
+                       "kernel": "rd_k_attn_partial_wide" if kv == "f16" else "rd_k_attn_partial_i8",
                        "avg_launch_ms": round(tp / 2, 5), "algorithmic_bytes_per_launch": int(per_launch)}
     out["roofline"]["traffic"], out["roofline"]["traffic_ratio"], out["roofline"]["traffic_source"] = counter_traffic(
         "attn_partial/64seq-u128-8192/%s" % kv, per_launch)

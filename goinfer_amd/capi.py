@@ -19,7 +19,7 @@ EXPORTS = [
     "rd_attn_ragged", "rd_moe_route", "rd_rmsnorm", "rd_rope", "rd_model_create", "rd_model_destroy",
     "rd_model_upload_q4k", "rd_model_upload_w8a8", "rd_model_upload_w4a8", "rd_model_upload_f32", "rd_model_finalize",
     "rd_kv_configure", "rd_kv_upload", "rd_kv_truncate", "rd_kv_reset", "rd_step_batch", "rd_forward",
-    "rd_last_moe_indices", "rd_model_upload_embedding", "rd_bench_steps", "rd_bench_profile", "rd_bench_attn_chain", "rd_bench_enqueue", "rd_moe_route_ex", "rd_attn_ragged_ex", "rd_model_set_router", "rd_model_set_window", "rd_model_set_block", "rd_model_set_graph", "rd_model_graph_stats", "rd_bench_prefill", "rd_bench_class_count",
+    "rd_last_moe_indices", "rd_model_upload_embedding", "rd_bench_steps", "rd_bench_profile", "rd_bench_attn_chain", "rd_bench_enqueue", "rd_bench_attn_kernel_name", "rd_bench_attn_in_step", "rd_moe_route_ex", "rd_attn_ragged_ex", "rd_model_set_router", "rd_model_set_window", "rd_model_set_block", "rd_model_set_graph", "rd_model_graph_stats", "rd_bench_prefill", "rd_bench_class_count",
     "rd_bench_class_name", "rd_bench_kernel", "rd_gateup_q4k_quant", "rd_moe_replay", "rd_bench_attn", "rd_step_ragged", "rd_prefill_last",
     "rd_kv_configure_typed", "rd_attn_ragged_i8", "rd_attn_ragged_rows", "rd_plan_attention", "rd_plan_gemm", "rd_step_batch_topk", "rd_last_logits", "rd_topk_rows", "rd_bench_attn_i8", "rd_step_ragged_draw", "rd_forward_no_logits",
     "rd_step_batch_draw", "rd_sample_rows", "rd_greedy_chain_start", "rd_greedy_chain_next", "rd_sample_chain_start",
@@ -341,6 +341,21 @@ class Model:
         if cfg.get("norm_add_one") or cfg.get("act_gelu_tanh") or cfg.get("final_softcap"):  # Gemma's block (rmsnorm.go:10-13,229-234)
             check(lib().rd_model_set_block(self.h, int(cfg.get("norm_add_one", 0)), int(cfg.get("act_gelu_tanh", 0)),
                                            C.c_float(cfg.get("final_softcap", 0.0))), "rd_model_set_block")
+
+    def bench_attn_in_step(self, slots, pos, ids0, reps=8):
+        """(ms per attention launch inside the step, ms per whole step): whole steps against steps without their attention launches."""
+        slots = np.ascontiguousarray(slots, dtype=np.int32)
+        pos = np.ascontiguousarray(pos, dtype=np.int32)
+        ids0 = np.ascontiguousarray(ids0, dtype=np.int32)
+        a, b = C.c_float(0), C.c_float(0)
+        check(lib().rd_bench_attn_in_step(self.h, len(slots), _p(slots), _p(pos), _p(ids0), int(reps), C.byref(a), C.byref(b)), "rd_bench_attn_in_step")
+        return a.value, b.value
+
+    def attn_kernel_name(self):
+        """The attention kernel the last step launched for its whole-context work list."""
+        f = lib().rd_bench_attn_kernel_name
+        f.restype = C.c_char_p
+        return f(self.h).decode()
 
     def bench_enqueue(self, slots, pos0, ids0, steps):
         """Host microseconds per step to enqueue `steps` chained greedy steps (nothing waits for the GPU inside the loop)."""

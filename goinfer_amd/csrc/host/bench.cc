@@ -121,6 +121,49 @@ extern "C" int rd_bench_attn_chain(rd_model *m, int B, const int *slot, const in
     return rc ? rc : rc2;
 }
 
+// The attention kernel the model's last step launched for its whole-context work list (names the kernel a roofline is for).
+extern "C" const char *rd_bench_attn_kernel_name(rd_model *m) {
+    if (!m || !m->last_items[0]) return "";
+    return attn_partial_kernel_name(m->d, attn_partial_kernel(m->d, m->kv_type == RD_KV_I8, m->last_grouped[0], m->last_items[0]).f);
+}
+
+// The attention kernel's cost where it runs, inside the step: `reps` pairs of steps at the same positions, one whole and one with the
+// attention launches left out, each between its own pair of events; *ms_per_launch = (mean whole - mean without) / layers. Unlike
+// the back-to-back chain above, the kernel here starts as it does in service: behind the q|k|v projection, with the work list,
+// the tables and q not yet in any L2.
+extern "C" int rd_bench_attn_in_step(rd_model *m, int B, const int *slot, const int *pos, const int *ids0, int reps, float *ms_per_launch, float *ms_step) {
+    if (!m || !slot || !pos || !ids0 || !ms_per_launch || reps < 1) return RD_ERR_ARG;
+    rd_device *d = m->d;
+    RC(d->h2d(m->ids, ids0, sizeof(int) * (size_t)B));
+    RC(model_step(m, B, slot, pos, nullptr, nullptr, RD_WANT_ARGMAX, nullptr, nullptr)); // settle: the positions exist from here on
+    RC(d->sync());
+    std::vector<hipEvent_t> ev((size_t)reps * 4);
+    for (auto &e : ev) HIPCHK(EventCreate(&e));
+    int rc = RD_OK;
+    for (int r = 0; r < reps && !rc; r++)
+        for (int skip = 0; skip < 2 && !rc; skip++) {
+            m->bench_skip_attn = skip != 0;
+            (void)d->hip->EventRecord(ev[(size_t)r * 4 + 2 * skip], d->stream);
+            rc = model_step(m, B, slot, pos, nullptr, nullptr, RD_WANT_ARGMAX, nullptr, nullptr);
+            (void)d->hip->EventRecord(ev[(size_t)r * 4 + 2 * skip + 1], d->stream);
+        }
+    m->bench_skip_attn = false;
+    const int rc2 = d->sync();
+    double whole = 0, without = 0;
+    for (int r = 0; r < reps; r++) {
+        float a = 0.f, b = 0.f;
+        if (!rc && !rc2) {
+            (void)d->hip->EventElapsedTime(&a, ev[(size_t)r * 4], ev[(size_t)r * 4 + 1]);
+            (void)d->hip->EventElapsedTime(&b, ev[(size_t)r * 4 + 2], ev[(size_t)r * 4 + 3]);
+        }
+        whole += a, without += b;
+    }
+    for (auto &e : ev) (void)d->hip->EventDestroy(e);
+    *ms_per_launch = (float)((whole - without) / reps / (double)m->layers.size());
+    if (ms_step) *ms_step = (float)(whole / reps);
+    return rc ? rc : rc2;
+}
+
 // A prompt pass with every input on the device: rows 0..n-1 of `slot` from token ids through the embedding table, in the passes
 // rd_prefill_last makes (all rows but the last build only their K/V, as wide as the step goes; the last is a one-row step with
 // the head). ms_total: the whole prompt, HIP events on the launch stream. profile != 0: an event pair around every kernel class

@@ -257,6 +257,18 @@ AttnLaunch attn_partial_kernel(const rd_device *d, bool i8, bool grouped, size_t
     return {d->k.attn_partial, 1u};
 }
 
+const char *attn_partial_kernel_name(const rd_device *d, hipFunction_t f) {
+    const Kernels &k = d->k;
+    if (f == k.attn_partial_wide) return "rd_k_attn_partial_wide";
+    if (f == k.attn_partial) return "rd_k_attn_partial";
+    if (f == k.attn_partial_i8) return "rd_k_attn_partial_i8";
+    if (f == k.attn_partial_deep) return "rd_k_attn_partial_deep";
+    if (f == k.attn_partial_deep_i8) return "rd_k_attn_partial_deep_i8";
+    if (f == k.attn_partial_rows) return "rd_k_attn_partial_rows";
+    if (f == k.attn_partial_rows_i8) return "rd_k_attn_partial_rows_i8";
+    return "?";
+}
+
 bool build_attn_worklist(const int *len, const int *slot, int G, int rows, int n_kv, std::vector<AttnItemH> &items, std::vector<int> &ranges,
                          int window) {
     auto first_block = [&](int r) { return window > 0 ? std::max(len[r] - window, 0) / 64 : 0; };

@@ -127,6 +127,7 @@ struct AttnLaunch {
     unsigned waves;
 };
 AttnLaunch attn_partial_kernel(const struct rd_device *d, bool i8, bool grouped, size_t n_items);
+const char *attn_partial_kernel_name(const struct rd_device *d, hipFunction_t f);
 constexpr int TOPK_MAX = 1024; // = RD_TOPK_MAX of the top-K kernels
 constexpr int TOPK_CAP = 4096, TOPK_BINS = 2048, TOPK_CHUNK = 16384; // = RD_TOPK_CAP, RD_TOPK_BINS, RD_TOPK_CHUNK
 // Scratch of the top-K over `rows` rows of width V (device memory the caller owns): per-chunk histograms and maxima, candidate

@@ -872,7 +872,7 @@ static int step_launches(rd_model *m, int B, int want) {
         }
         {
             Scope s(m, KC_ATTN_PARTIAL);
-            RC(launch_attn_partial(m, l));
+            if (!m->bench_skip_attn) RC(launch_attn_partial(m, l));
         }
         {
             Scope s(m, KC_ATTN_COMBINE);
@@ -945,7 +945,7 @@ static int step_launches(rd_model *m, int B, int want) {
 // the second may replay the first one's captured graph. Empty: this step is not one to capture (timed, or replaying a routing).
 static std::vector<long> step_graph_key(rd_model *m, int B, int want) {
     std::vector<long> k;
-    if (m->timer.on || m->replay_B != 0) return k;
+    if (m->timer.on || m->replay_B != 0 || m->bench_skip_attn) return k;
     k = {B, want, m->step_draws ? 1 : 0, (long)m->last_items[0], (long)m->last_items[1], m->last_grouped[0] ? 1 : 0, m->last_grouped[1] ? 1 : 0,
          getenv("ROCMDECODE_NO_FUSED_GATEUP") ? 1 : 0, getenv("ROCMDECODE_NO_FUSED_QKV") ? 1 : 0, getenv("ROCMDECODE_NO_FUSED_MOE_GATEUP") ? 1 : 0,
          getenv("ROCMDECODE_MOE_TILES") ? atol(getenv("ROCMDECODE_MOE_TILES")) : 0};
