@@ -90,7 +90,7 @@ def run_c2(args):
     cases = []
     for name, kern, N, K, wbytes in (("up 14336x4096", "gemm_q4k", 14336, 4096, W), ("down 4096x14336", "gemm_q4k", 4096, 14336, W),
                                      ("fused gate|up 2x14336x4096 + SwiGLU", "gateup", 14336, 4096, 2 * W)):
-        for M in (1, 4, 16, 32, 64):
+        for M in ((args.m,) if getattr(args, "m", 0) else (1, 4, 16, 32, 64)):
             ms = dev.bench_kernel(kern, [N, K, M, 8], warmup, steps)  # 8 weight copies round-robin: nothing stays in the 256 MB cache
             t = float(np.median(ms))
             nbytes = wbytes + 4 * M * K + (4 * M * N if kern == "gemm_q4k" else 2 * M * N)  # weights + activations in + result out
@@ -98,7 +98,7 @@ def run_c2(args):
             cases.append({"case": name, "M": M, "us": round(t * 1e3, 2), "GBs": round(nbytes / t / 1e6, 1), "TFLOPs": round(flops / t / 1e9, 1),
                           "bytes": int(nbytes)})
             log("%s M=%d: %.1f us, %.0f GB/s" % (name, M, t * 1e3, nbytes / t / 1e6))
-    head = next(c for c in cases if c["case"].startswith("fused") and c["M"] == 32)
+    head = next(c for c in cases if c["case"].startswith("fused") and c["M"] == (getattr(args, "m", 0) or 32))
     out = base_line("Q4_K dequant-GEMM achieved HBM GB/s (fused gate|up SwiGLU at M=32; all cases listed)", head["GBs"], "GB/s", steps, warmup,
                     head["us"] / 1e3, "configs[1]: Q4_K GEMM 14336x4096 / 4096x14336 / fused gate|up, M in {1,4,16,32,64}",
                     "synthetic: random Q4_K super-blocks with sane f16 scales, 8 weight copies used round-robin", {"cases": cases})
