@@ -338,9 +338,10 @@ class Model:
             check(lib().rd_model_set_router(self.h, int(cfg.get("router_sigmoid", 0)), C.c_double(cfg.get("router_scale", 0.0)),
                                             int(cfg.get("n_group", 0)), int(cfg.get("topk_group", 0))), "rd_model_set_router")
 
-        if cfg.get("norm_add_one") or cfg.get("act_gelu_tanh") or cfg.get("final_softcap"):  # Gemma's block (rmsnorm.go:10-13,229-234)
+        if cfg.get("norm_add_one") or cfg.get("act_gelu_tanh") or cfg.get("final_softcap") or cfg.get("logit_scale"):
+            # Gemma's block (rmsnorm.go:10-13,229-234), Granite's logits_scaling (model_forward.go:304-320)
             check(lib().rd_model_set_block(self.h, int(cfg.get("norm_add_one", 0)), int(cfg.get("act_gelu_tanh", 0)),
-                                           C.c_float(cfg.get("final_softcap", 0.0))), "rd_model_set_block")
+                                           C.c_float(cfg.get("final_softcap", 0.0)), C.c_double(cfg.get("logit_scale", 0.0))), "rd_model_set_block")
 
     def bench_attn_in_step(self, slots, pos, ids0, reps=8):
         """(ms per attention launch inside the step, ms per whole step): whole steps against steps without their attention launches."""

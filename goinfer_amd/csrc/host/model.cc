@@ -372,8 +372,8 @@ extern "C" int rd_model_set_router(rd_model *m, int sigmoid, double scale, int n
 }
 
 // The block's family knobs (Gemma; backend/cuda/resident.go:549-565 finalSoftcap, act, addOneArg), before rd_model_finalize.
-extern "C" int rd_model_set_block(rd_model *m, int norm_add_one, int act, float final_softcap) {
-    if (!m || (act != RD_ACT_SILU && act != RD_ACT_GELU_TANH) || !(final_softcap >= 0.f)) return RD_ERR_ARG;
+extern "C" int rd_model_set_block(rd_model *m, int norm_add_one, int act, float final_softcap, double logit_scale) {
+    if (!m || (act != RD_ACT_SILU && act != RD_ACT_GELU_TANH) || !(final_softcap >= 0.f) || !(logit_scale >= 0.0)) return RD_ERR_ARG;
     if (m->finalized) {
         rd_set_error("model already finalized");
         return RD_ERR_STATE;
@@ -383,6 +383,7 @@ extern "C" int rd_model_set_block(rd_model *m, int norm_add_one, int act, float 
         return RD_DECLINED;
     }
     m->norm_add_one = norm_add_one ? 1 : 0, m->act = act, m->final_softcap = final_softcap;
+    m->logit_mul = (logit_scale != 0.0 && logit_scale != 1.0) ? (float)(1 / logit_scale) : 0.f;
     return RD_OK;
 }
 
@@ -934,7 +935,7 @@ static int step_launches(rd_model *m, int B, int want) {
             int nChunks = (c.vocab + 4095) / 4096;
             RC(d->launch(d->k.argmax_rows, (unsigned)nChunks, (unsigned)B, 1, 256, (const float *)m->P, plan.splits, c.vocab, m->cand_v, m->cand_i,
                          (want & RD_WANT_LOGITS) ? m->logits : (float *)nullptr, (const int *)(m->step_draws ? m->rowDraw : nullptr), m->pStride,
-                         m->final_softcap));
+                         m->final_softcap, m->logit_mul));
             if (want & RD_WANT_ARGMAX) RC(d->launch(d->k.argmax_final, (unsigned)B, 1, 1, 64, (const float *)m->cand_v, (const int *)m->cand_i, nChunks, m->ids));
         }
     }

@@ -59,6 +59,7 @@ struct rd_model {
     int window = 0; // the one window length the model's sliding-window layers share (0: none has one)
     int norm_add_one = 0, act = 0; // (1 + w) norm weights; the gated FFN's activation (RD_ACT_*)
     float final_softcap = 0.f;     // > 0: logits become cap * tanh(logit / cap)
+    float logit_mul = 0.f;         // not 0 or 1: logits are multiplied by it after the softcap (f32(1 / LogitScale))
     bool ones_added = false;       // the (1 + w) pass over the norm weights has run
     bool bench_skip_attn = false;  // measurement only: the step leaves out its attention launches (its results are then meaningless)
     // The launches of a step as a captured HIP graph, replayed while steps keep one key (see step_run in model.cc)

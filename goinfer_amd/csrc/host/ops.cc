@@ -268,7 +268,7 @@ extern "C" int rd_sample_rows(rd_device *d, const float *logits, int rows, int V
         RC(d->h2d(L.p, pad.data(), sizeof(float) * (size_t)nr * Vp));
         RC(d->h2d(rec.p, recs, sizeof(recs)));
         RC(d->launch(d->k.argmax_rows, (unsigned)nChunks, (unsigned)nr, 1, 256, (const float *)L.p, 1, Vp, cv.as<float>(), ci.as<int>(), (float *)nullptr,
-                     (const int *)rec.p, (size_t)0, 0.f));
+                     (const int *)rec.p, (size_t)0, 0.f, 0.f));
         RC(d->launch(d->k.argmax_final, (unsigned)nr, 1, 1, 64, (const float *)cv.p, (const int *)ci.p, nChunks, out.as<int>()));
         RC(d->d2h(ids + r0, out.p, sizeof(int) * (size_t)nr));
     }

@@ -60,7 +60,7 @@ __device__ __forceinline__ float gumbel_noise(uint32_t h) {
 // draw hi, 0), key seed), and a thread's four consecutive entries are exactly one Philox call.
 extern "C" __global__ __launch_bounds__(256) void rd_k_argmax_rows(const float *__restrict__ P, int splits, int N, float *__restrict__ cand_v,
                                                                    int *__restrict__ cand_i, float *__restrict__ logits_out,
-                                                                   const int *__restrict__ rowDraw, size_t pStride, float softcap) {
+                                                                   const int *__restrict__ rowDraw, size_t pStride, float softcap, float logitMul) {
     __shared__ float bv[4];
     __shared__ int bi[4];
     const int m = blockIdx.y, t = threadIdx.x, nChunks = gridDim.x, mr = m & 31;
@@ -82,6 +82,10 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_argmax_rows(const float *
             if (softcap > 0.f) { // decoder/model_forward.go:259-266: cap * f32(tanh(f64(logit / cap))), before anything reads the logits
 #pragma unroll
                 for (int e = 0; e < 4; e++) a[e] = mul_rounded(softcap, (float)tanh((double)__fdiv_rn(a[e], softcap)));
+            }
+            if (logitMul != 0.f && logitMul != 1.f) { // decoder/model_forward.go:304-320: logits *= f32(1 / LogitScale), after the softcap
+#pragma unroll
+                for (int e = 0; e < 4; e++) a[e] = mul_rounded(a[e], logitMul);
             }
             if (logits_out) *(float4_t *)(logits_out + (size_t)m * N + n0) = a;
             if (gumbel) {

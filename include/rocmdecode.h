@@ -170,10 +170,11 @@ int rd_model_set_router(rd_model *m, int sigmoid, double scale, int n_group, int
  * rd_model_finalize. norm_add_one: every RMSNorm weight is stored as its deviation from one and scales by f32(1 + w)
  * (Architecture.RMSAddOne, decoder/rmsnorm.go:10-13,62-75; the sum is formed once at rd_model_finalize). act: the gated FFN's
  * activation, RD_ACT_SILU (SwiGLU) or RD_ACT_GELU_TANH (Gemma's GeGLU, decoder/rmsnorm.go:229-234; dense FFN only). final_softcap
- * > 0: logits become cap * tanh(logit / cap) (decoder/model_forward.go:259-266) before the argmax, the draws, the top-K and the
- * copy to the host. */
+ * > 0: logits become cap * tanh(logit / cap) (decoder/model_forward.go:259-266); logit_scale not 0 or 1: they are then multiplied by
+ * f32(1 / logit_scale) (Architecture.LogitScale, Granite's logits_scaling; model_forward.go:304-320) — both before the argmax, the
+ * draws, the top-K and the copy to the host. */
 enum { RD_ACT_SILU = 0, RD_ACT_GELU_TANH = 1 };
-int rd_model_set_block(rd_model *m, int norm_add_one, int act, float final_softcap);
+int rd_model_set_block(rd_model *m, int norm_add_one, int act, float final_softcap, double logit_scale);
 /* A sliding-window layer (decoder/kvcache.go:1063-1068 WindowStart): its rows read the last `window` positions only. Before
  * rd_model_finalize. The windowed layers of a model share one length (RD_DECLINED otherwise); the cache keeps every position. */
 int rd_model_set_window(rd_model *m, int layer, int window);

@@ -33,7 +33,8 @@ class Model(C.Structure):
                 ("n_experts", C.c_int), ("top_k", C.c_int), ("norm_topk", C.c_int), ("exp_inter", C.c_int),
                 ("kv_f16", C.c_int), ("layers", C.POINTER(Layer)), ("final_norm", C.c_void_p), ("head", Mat),
                 ("router_sigmoid", C.c_int), ("router_scale", C.c_double), ("n_group", C.c_int), ("topk_group", C.c_int),
-                ("norm_add_one", C.c_int), ("act_gelu_tanh", C.c_int), ("final_softcap", C.c_double)]
+                ("norm_add_one", C.c_int), ("act_gelu_tanh", C.c_int), ("final_softcap", C.c_double),
+                ("logit_scale", C.c_double)]
 
 
 def f16_round_trip(x):
@@ -312,7 +313,8 @@ class OracleModel:
                        nE, cfg.get("top_k", 0), int(cfg.get("norm_topk", 0)), cfg.get("exp_inter", 0),
                        int(cfg.get("kv_f16", 0)), self._layers, _p(self._fn), head.c(),
                        int(cfg.get("router_sigmoid", 0)), float(cfg.get("router_scale", 0.0)), int(cfg.get("n_group", 0)), int(cfg.get("topk_group", 0)),
-                       int(cfg.get("norm_add_one", 0)), int(cfg.get("act_gelu_tanh", 0)), float(cfg.get("final_softcap", 0.0)))
+                       int(cfg.get("norm_add_one", 0)), int(cfg.get("act_gelu_tanh", 0)), float(cfg.get("final_softcap", 0.0)),
+                       float(cfg.get("logit_scale", 0.0)))
 
     def new_cache(self, cap):
         return lib().or_cache_new(C.byref(self.m), cap)

@@ -1053,6 +1053,10 @@ int or_decode_multi_step_traced(const or_model *m, int B, const float *emb, or_c
     or_rmsnorm(h, h, m->final_norm, B, H, m->eps, m->norm_add_one);
     or_matmul(&m->head, h, B, logits);
     if (m->final_softcap > 0) or_softcap_logits(logits, (size_t)B * m->vocab, (float)m->final_softcap);
+    if (m->logit_scale != 0 && m->logit_scale != 1) { /* decoder/model_forward.go:304-320, forwardn.go:823-831 */
+        const float inv = (float)(1 / m->logit_scale);
+        for (size_t i = 0; i < (size_t)B * m->vocab; i++) logits[i] *= inv;
+    }
     free(h);
     free(norm);
     free(att);

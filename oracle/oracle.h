@@ -33,6 +33,7 @@
  *   attention softcap, or_gelu_tanh / or_geglu, or_softcap_logits, (1 + w) norms, post-branch norms
  *                                        pinned: the gemma2-tiny golden to 1e-5 (tests/test_oracle_golden.py shows each knob moves
  *                                        the logits by > 1e-3 when switched off)
+ *   or_model.logit_scale                 pinned: the granite-dense-tiny golden (embedding x 12, attention scale 0.5, logits / 6)
  *   or_attend_sinks                      pinned by the closed form only (a softmax with one more logit per head, numpy f64):
  *                                        the reference's fixture with sinks is a GGUF file with MXFP4 experts, outside this path
  *   or_topk_by_logit, or_softmax_z       pinned by what the definition fixes: the first K of the row sorted by (logit desc, id asc) is
@@ -181,6 +182,7 @@ typedef struct {
     int norm_add_one;     /* 1: every RMSNorm scales by (1 + w) (Gemma stores weights as deviations from one) */
     int act_gelu_tanh;    /* 1: the gated FFN is GeGLU with the tanh-approximate GELU instead of SwiGLU */
     double final_softcap; /* > 0: logits become cap * tanh(logit / cap) */
+    double logit_scale;   /* not 0 or 1: logits are multiplied by f32(1 / logit_scale) after the softcap (Granite logits_scaling) */
 } or_model;
 
 typedef struct {

@@ -175,3 +175,21 @@ def test_gemma2_fused_gateup_equals_separate_kernels(dev, monkeypatch):
         finally:
             p.close()
     assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+
+
+def test_granite_style_multipliers(dev):
+    """Granite's block is a llama block with three multipliers (decoder/arch_granite.go:50-62): the embedding's arrives with the
+    rows, the attention scale is the model's, and the logits are divided by logits_scaling after the head."""
+    cfg = dict(dense_cfg(n_layers=2, hidden=256, n_heads=4, n_kv=2, head_dim=64, inter=512, vocab=512), logit_scale=6.0)
+    cfg["attn_scale"] = 0.0625
+    rng = np.random.default_rng(64)
+    check(Pair(cfg, seed=74, dev=dev, slots=4), [list(rng.integers(0, 512, n)) for n in (5, 40)], steps=3)
+    a, b = Pair(cfg, seed=74, dev=dev, slots=2), Pair(dict(cfg, logit_scale=0.0), seed=74, dev=dev, slots=2)
+    try:
+        e = a.emb[[7]]
+        la, _ = a.gpu.step_batch([0], [0], e)
+        lb, _ = b.gpu.step_batch([0], [0], e)
+        assert np.array_equal(la.view(np.uint32), (lb * np.float32(1.0 / 6.0)).view(np.uint32))  # one rounded multiply per logit
+    finally:
+        a.close()
+        b.close()

@@ -150,6 +150,27 @@ def test_gemma2_knobs_matter():
     assert run() <= 1e-5
 
 
+def test_granite_dense_tiny_forward():
+    """Granite's three multipliers on a llama block (cmd/gate/identity_assets.go, decoder/arch_granite.go:50-62): embedding x 12,
+    attention scale 0.5 in place of 1/sqrt(d), logits / 6; the reference's bars of decoder/forward_test.go:44-125."""
+    g = json.load(open(os.path.join(GOLDEN, "granite_dense_forward_golden.json")))
+    m, emb, _ = tiny_model("granite-dense-tiny")
+    logits, c = run_prompt(m, emb, g["ids"])
+    m.free_cache(c)
+    assert ob.argmax(logits) == g["argmax"]
+    for i, v in g["top_k"] + g["sample"]:
+        assert abs(float(logits[int(i)]) - v) <= 1e-5, (i, logits[int(i)], v)
+    l64 = logits.astype(np.float64)
+    st = g["stats"]
+    assert abs(l64.sum() - st["sum"]) <= 1e-3 * abs(st["sum"]) + 1e-6 and abs((l64 * l64).sum() - st["sum_sq"]) <= 1e-3 * st["sum_sq"]
+    keep = m.m.logit_scale
+    m.m.logit_scale = 0.0  # and the scale is not ignored
+    logits, c = run_prompt(m, emb, g["ids"])
+    m.free_cache(c)
+    m.m.logit_scale = keep
+    assert abs(float(logits[g["argmax"]]) - dict((int(i), v) for i, v in g["top_k"])[g["argmax"]]) > 1e-2
+
+
 def test_batched_rows_equal_single_rows():
     """decoder/cpu_batch_test.go:14-53: each row of a batched step is bit-identical to that sequence alone."""
     m, emb, _ = tiny_model("llama-tiny")

@@ -90,5 +90,9 @@ def tiny_model(name, wrap=ob.WMat.from_f32):
         emb = emb * np.float32(np.sqrt(np.float64(H)))
     else:
         head = wrap(t["lm_head.weight"])
+    if cfg["model_type"] == "granite":  # decoder/arch_granite.go:50-62: the three multipliers of a llama block (residual_multiplier is 1)
+        assert cfg["residual_multiplier"] == 1.0
+        c.update(attn_scale=float(cfg["attention_multiplier"]), logit_scale=float(cfg["logits_scaling"]))
+        emb = emb * np.float32(cfg["embedding_multiplier"])
     m = ob.OracleModel(c, layers, t["model.norm.weight"], head, inv_freq(hd, theta))
     return m, emb, cfg
