@@ -81,6 +81,22 @@ __device__ __forceinline__ i32x4_t as_i32x4(uint4_t v) {
 #define RD_FOLD(ACC, DOT, S, OFF, NR)                                                  \
     _Pragma("unroll") for (int r_ = 0; r_ < (NR); r_++) ACC[r_] = __builtin_fmaf((float)DOT[r_], S[(OFF) + r_], ACC[r_]);
 
+// The two lane halves' values of x on every lane: lo = lanes 0..31's, hi = lanes 32..63's (v_permlane32_swap).
+__device__ __forceinline__ void halves_i(int x, int &lo, int &hi) {
+    const auto r = __builtin_amdgcn_permlane32_swap((unsigned)x, (unsigned)x, false, false);
+    lo = (int)r[0], hi = (int)r[1];
+}
+__device__ __forceinline__ void halves_f(float x, float &lo, float &hi) {
+    int a, b;
+    halves_i(__float_as_int(x), a, b);
+    lo = __int_as_float(a), hi = __int_as_float(b);
+}
+__device__ __forceinline__ int halves_sum(int x) {
+    int a, b;
+    halves_i(x, a, b);
+    return a + b;
+}
+
 // ---------------- Q4_K ----------------
 // Tile of 32 rows x one super-block, 4608 B: the 32 headers (16 B: d, dmin, 12 scale bytes), then four planes [64 lanes][16 B]:
 // plane p, lane (row r, half h) holds raw code bytes [32p + 16h, +16) of row r, i.e. elements 16h..16h+15 of sub-block 2p in
@@ -112,15 +128,12 @@ struct Q4K8Traits {
 #pragma unroll
         for (int c = 0; c < 4; c++) w.q[c] = buf_load16_nt(r, off + lane * 16, 512 + c * 1024);
     }
-    // acc[m][n] += sum over the super-block's 8 groups. Lane (n, h) decodes the scales of sub-blocks 2p+h, p = 0..3: the
-    // lane half is the block index of the two-block scale product and the k index of the minimum product.
-    template <int NR> static __device__ __forceinline__ void mma(float16_t &acc, const Tile &w, const A8Regs &a, const void *, int, int lane) {
-        const int h = lane >> 5;
+    // Lane (n, h) decodes the scales of sub-blocks 2p+h, p = 0..3: dsc = d * sc, ndm = -(dmin * m).
+    static __device__ __forceinline__ void decode(const Tile &w, int h, float (&dsc)[4], float (&ndm)[4]) {
         const uint32_t y = w.hdr.y, z = w.hdr.z, x = w.hdr.w, hx = w.hdr.x;
         half2_t dd;
         __builtin_memcpy(&dd, &hx, 4);
         const float d = (float)dd.x, dmin = (float)dd.y;
-        float dsc[4], ndm[4];
 #pragma unroll
         for (int p = 0; p < 4; p++) {
             int sc, mn;
@@ -137,6 +150,12 @@ struct Q4K8Traits {
             dsc[p] = __fmul_rn(d, (float)sc);
             ndm[p] = -__fmul_rn(dmin, (float)mn);
         }
+    }
+    // acc[m][n] += sum over the super-block's 8 groups: the lane half is the block index of the two-block scale product and the k
+    // index of the minimum product.
+    template <int NR> static __device__ __forceinline__ void mma(float16_t &acc, const Tile &w, const A8Regs &a, const void *, int, int lane) {
+        float dsc[4], ndm[4];
+        decode(w, lane >> 5, dsc, ndm);
         const f32x32_t zero32 = {0.f};
         const i32x16_t zero16 = {0};
 #pragma unroll
@@ -153,6 +172,45 @@ struct Q4K8Traits {
         }
 #pragma unroll
         for (int p = 0; p < 4; p++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.asum[p], ndm[p], acc, 0, 0, 0);
+    }
+    // The same sums for ONE batch row on the vector ALU (a step of one sequence: goinfer's Forward). `a` holds row 0's operands
+    // broadcast: lane (n, h) has the row's codes 16h..16h+15 of every group and the scale and sum of groups 2p+h, beside its
+    // own weight row's codes and sub-block scales for the same elements and groups. A group's dot is the two lane halves'
+    // sixteen-element dots added (v_dot4_i32_i8, exact); the fold is the matrix-core path's own chain, operation for operation:
+    // its scale product is one rounded multiply (v_mfma_f32_32x32x1 with a zero accumulator gives exactly that), its groups are
+    // folded in ascending order with one fma each, and v_mfma_f32_32x32x2 is fma(a1, b1, fma(a0, b0, c)), k ascending — measured
+    // on 204 800 random outputs, no exception. The row is therefore the row a batch gives, bit for bit; the tests that compare a
+    // batched row with its solo run hold the two paths to that. Both lane halves compute the chain (accumulator 0 of the upper half
+    // is batch row 4, which a one-row step never stores).
+    static constexpr bool GEMV1 = true;
+    static __device__ __forceinline__ void mma1(float16_t &acc, const Tile &w, const A8Regs &a, const void *, int, int lane) {
+        float dsc[4], ndm[4];
+        decode(w, lane >> 5, dsc, ndm);
+        float f = acc[0];
+        float se[4], so[4];
+#pragma unroll
+        for (int p = 0; p < 4; p++) halves_f(__fmul_rn(a.as[p], dsc[p]), se[p], so[p]);
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            const uint4_t raw = w.q[p];
+            int x0 = 0, x1 = 0;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                x0 = __builtin_amdgcn_sdot4((int)(raw[i] & 0x0F0F0F0Fu), (int)a.c[2 * p][i], x0, false);
+                x1 = __builtin_amdgcn_sdot4((int)((raw[i] >> 4) & 0x0F0F0F0Fu), (int)a.c[2 * p + 1][i], x1, false);
+            }
+            f = __builtin_fmaf((float)halves_sum(x0), se[p], f);
+            f = __builtin_fmaf((float)halves_sum(x1), so[p], f);
+        }
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            float ae, ao, ne, no;
+            halves_f(a.asum[p], ae, ao);
+            halves_f(ndm[p], ne, no);
+            f = __builtin_fmaf(ae, ne, f);
+            f = __builtin_fmaf(ao, no, f);
+        }
+        acc[0] = f;
     }
     static __device__ __forceinline__ void finish(float16_t &, const void *, int, int) {}
 };
@@ -173,6 +231,8 @@ struct W8Tile8 {
 };
 struct W8A8Traits8 {
     typedef W8Tile8 Tile;
+    static constexpr bool GEMV1 = false;
+    static __device__ __forceinline__ void mma1(float16_t &, const Tile &, const A8Regs &, const void *, int, int) {}
     static constexpr int TILE_BYTES = 8192;
     static __device__ __forceinline__ void load(Tile &w, rd_rsrc_t r, int off, int lane) {
 #pragma unroll
@@ -234,6 +294,8 @@ extern "C" __global__ __launch_bounds__(320) void rd_k_retile_w4a8_8(const uint8
 struct W4A8Traits8 {
     typedef Q4K8Tile Tile;
     static constexpr int TILE_BYTES = 4608;
+    static constexpr bool GEMV1 = false;
+    static __device__ __forceinline__ void mma1(float16_t &, const Tile &, const A8Regs &, const void *, int, int) {}
     static __device__ __forceinline__ void load(Tile &w, rd_rsrc_t r, int off, int lane) { Q4K8Traits::load(w, r, off, lane); }
     template <int NR> static __device__ __forceinline__ void mma(float16_t &acc, const Tile &w, const A8Regs &a, const void *, int, int lane) {
         const int h = lane >> 5;
@@ -272,6 +334,15 @@ struct W4A8Traits8 {
 // NR: accumulator registers folded (RD_FOLD). aoff: the lane's byte offset inside an activation block, lane * 16 for batch row
 // lane & 31 (a caller that gathers rows passes the offset of another row, or one past every block for a row with no source:
 // the descriptor then answers zeros).
+// NR == 1: one batch row on the vector ALU (traits with GEMV1), else NR accumulator registers folded from the matrix core's dots
+template <class T, int NR>
+__device__ __forceinline__ void gemm8_mma(float16_t &acc, const typename T::Tile &w, const A8Regs &a, const void *aux, int tile, int lane) {
+    if constexpr (NR == 1)
+        T::mma1(acc, w, a, aux, tile, lane);
+    else
+        T::template mma<NR>(acc, w, a, aux, tile, lane);
+}
+
 template <class T, int NR = 16>
 __device__ __forceinline__ void gemm8_wave_loop(float16_t &acc, const uint8_t *__restrict__ wb, const uint8_t *__restrict__ ab, int nk, const void *aux,
                                                 int tile, int lane, int aoff) {
@@ -280,6 +351,7 @@ __device__ __forceinline__ void gemm8_wave_loop(float16_t &acc, const uint8_t *_
     if (nk <= 0) return;
     constexpr int AB = RD_A8_BLOCK_BYTES;
     const rd_rsrc_t wr = make_rsrc(wb, (uint32_t)nk * T::TILE_BYTES), ar = make_rsrc(ab, (uint32_t)nk * AB);
+    if constexpr (NR == 1) aoff = (lane >> 5) * 512; // batch row 0's operands on every lane of a half (see mma1)
     typename T::Tile w0, w1;
     A8Regs a0, a1;
     a8_load(a0, ar, aoff);
@@ -287,10 +359,10 @@ __device__ __forceinline__ void gemm8_wave_loop(float16_t &acc, const uint8_t *_
     a8_load(a1, ar, AB + aoff);
     T::load(w1, wr, T::TILE_BYTES, lane);
     for (int it = 0; it < nk; it += 2) {
-        T::template mma<NR>(acc, w0, a0, aux, tile, lane);
+        gemm8_mma<T, NR>(acc, w0, a0, aux, tile, lane);
         a8_load(a0, ar, (it + 2) * AB + aoff);
         T::load(w0, wr, (it + 2) * T::TILE_BYTES, lane);
-        if (it + 1 < nk) T::template mma<NR>(acc, w1, a1, aux, tile, lane);
+        if (it + 1 < nk) gemm8_mma<T, NR>(acc, w1, a1, aux, tile, lane);
         a8_load(a1, ar, (it + 3) * AB + aoff);
         T::load(w1, wr, (it + 3) * T::TILE_BYTES, lane);
     }
@@ -372,7 +444,9 @@ __device__ __forceinline__ void gemm8_body(const uint8_t *__restrict__ Wt, const
         A8 += (size_t)z * a8Stride, P += (size_t)z * pStride, M = min(32, M - 32 * z);                                                               \
         if (resid) resid += (size_t)z * 32 * ldP;                                                                                                    \
         /* up to 8 batch rows live in four accumulator registers, up to 16 in eight: the fold of the others is left out */                          \
-        if (M <= 8)                                                                                                                                  \
+        if (TRAITS::GEMV1 && M == 1) /* one row: the same sums on the vector ALU */                                                                  \
+            gemm8_body<TRAITS, KW, TPB, 1>(Wt, aux, A8, P, N, nKB, kbPerSplit, M, ldP, resid, lds);                                                  \
+        else if (M <= 8)                                                                                                                             \
             gemm8_body<TRAITS, KW, TPB, 4>(Wt, aux, A8, P, N, nKB, kbPerSplit, M, ldP, resid, lds);                                                  \
         else if (M <= 16)                                                                                                                            \
             gemm8_body<TRAITS, KW, TPB, 8>(Wt, aux, A8, P, N, nKB, kbPerSplit, M, ldP, resid, lds);                                                  \
@@ -439,7 +513,9 @@ __device__ __forceinline__ void gemm8_gateup_body(const uint8_t *__restrict__ Wt
                                                            int outKind, int I, int nKB, int M, size_t a8Stride, size_t outStride) {            \
         __shared__ float lds[2 * 1024];                                                                                                           \
         A8 += (size_t)blockIdx.z * a8Stride, XpOut += (size_t)blockIdx.z * outStride, M = min(32, M - 32 * (int)blockIdx.z);                      \
-        if (M <= 8)                                                                                                                               \
+        if (M == 1)                                                                                                                               \
+            gemm8_gateup_body<Q4K8Traits, 2, 1, ACT>(Wt, A8, XpOut, outKind, I, nKB, M, lds);                                                     \
+        else if (M <= 8)                                                                                                                          \
             gemm8_gateup_body<Q4K8Traits, 2, 4, ACT>(Wt, A8, XpOut, outKind, I, nKB, M, lds);                                                     \
         else if (M <= 16)                                                                                                                         \
             gemm8_gateup_body<Q4K8Traits, 2, 8, ACT>(Wt, A8, XpOut, outKind, I, nKB, M, lds);                                                     \
@@ -533,7 +609,9 @@ __device__ __forceinline__ void gemm8_qkv_body(const uint8_t *__restrict__ Wt, c
         const int row0 = 32 * (int)blockIdx.z; /* M-tile z: rows row0.. of the step, activations a8Stride bytes further on */                          \
         A8 += (size_t)blockIdx.z * a8Stride, M = min(32, M - row0);                                                                                    \
         QkvEpilogue e{q, Kp, Vp, tables, rowSlot, rowPos, (const double2 *)cs, bias, tabStride, nH, nKV, HD, row0};                                    \
-        if (M <= 8)                                                                                                                                    \
+        if (TRAITS::GEMV1 && M == 1)                                                                                                                   \
+            gemm8_qkv_body<TRAITS, KW, 1>(Wt, aux, A8, N, nKB, M, e, lds);                                                                             \
+        else if (M <= 8)                                                                                                                               \
             gemm8_qkv_body<TRAITS, KW, 4>(Wt, aux, A8, N, nKB, M, e, lds);                                                                             \
         else if (M <= 16)                                                                                                                              \
             gemm8_qkv_body<TRAITS, KW, 8>(Wt, aux, A8, N, nKB, M, e, lds);                                                                             \

@@ -89,7 +89,28 @@ def test_gemm_q4k_random_blocks_and_saturated_scales(dev):
     raw[::5, 4:16] = 0xFF
     a = synth.normal(3, M * K).reshape(M, K)
     w = ob.WMat(ob.OR_Q4K, N, K, raw, act_group=32)
-    assert rel_err(dev.gemm_q4k(raw, N, K, a), ob.matmul_f64ref(w, a)) < 1e-5
+    got = dev.gemm_q4k(raw, N, K, a)
+    assert rel_err(got, ob.matmul_f64ref(w, a)) < 1e-5
+    # one row alone runs on the vector ALU, a batch on the matrix cores: the same bits on every code, scale and minimum
+    for r in range(M):
+        solo = dev.gemm_q4k(raw, N, K, a[r:r + 1])
+        assert np.array_equal(solo[0].view(np.uint32), got[r].view(np.uint32)), r
+
+
+def test_one_row_path_equals_batch_rows_at_the_step_shapes(dev):
+    """The one-row kernels (v_dot4 on the vector ALU) against rows of a batch (int8 matrix cores), bit for bit, at shapes that take
+    each plan of the step: four waves a tile in one split, eight waves in two K splits, activations from tiny to large, a zero row."""
+    for N, K, seed in ((14336, 4096, 5), (4096, 14336, 6), (6144, 4096, 7)):
+        blocks = synth.q4k_normal(seed, N, K)
+        a = synth.normal(seed + 10, 6 * K).reshape(6, K)
+        a[1] *= 1e-4
+        a[2] *= 300.0
+        a[3] = 0.0
+        a[4, ::7] = 0.0
+        wide = dev.gemm_q4k(blocks, N, K, a)
+        for r in range(6):
+            solo = dev.gemm_q4k(blocks, N, K, a[r:r + 1])
+            assert np.array_equal(solo[0].view(np.uint32), wide[r].view(np.uint32)), (N, K, r)
 
 
 @pytest.mark.parametrize("M,K", [(1, 32), (3, 256), (32, 4096), (40, 896), (7, 14336)])
@@ -137,7 +158,10 @@ def test_fused_gate_up_kernel(dev, M):
     a = synth.normal(3, M * K).reshape(M, K)
     gate = ob.matmul(ob.WMat(ob.OR_Q4K, I, K, g, act_group=32), a)
     up = ob.matmul(ob.WMat(ob.OR_Q4K, I, K, u, act_group=32), a)
-    check_fused(dev.gateup_q4k_quant(g, u, I, K, a), gate, up)
+    got = dev.gateup_q4k_quant(g, u, I, K, a)
+    check_fused(got, gate, up)
+    solo = dev.gateup_q4k_quant(g, u, I, K, a[:1])  # one row: the vector-ALU kernel; the same quantized activations, bit for bit
+    assert np.array_equal(solo[0].view(np.uint32), got[0].view(np.uint32))
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 64, 128), (7, 256, 896), (32, 1024, 4096), (5, 96, 96)])
