@@ -186,6 +186,10 @@ struct Q4K8Traits {
     static __device__ __forceinline__ void mma1(float16_t &acc, const Tile &w, const A8Regs &a, const void *, int, int lane) {
         float dsc[4], ndm[4];
         decode(w, lane >> 5, dsc, ndm);
+        fold1(acc, w, a, dsc, ndm);
+    }
+    // dsc[p], ndm[p]: this lane's scale and negated minimum of group 2p + (lane half); codes 0..15 in the tile's nibbles
+    static __device__ __forceinline__ void fold1(float16_t &acc, const Tile &w, const A8Regs &a, const float (&dsc)[4], const float (&ndm)[4]) {
         float f = acc[0];
         float se[4], so[4];
 #pragma unroll
@@ -231,8 +235,25 @@ struct W8Tile8 {
 };
 struct W8A8Traits8 {
     typedef W8Tile8 Tile;
-    static constexpr bool GEMV1 = false;
-    static __device__ __forceinline__ void mma1(float16_t &, const Tile &, const A8Regs &, const void *, int, int) {}
+    // One batch row on the vector ALU (see Q4K8Traits::mma1): the scale "product with one" is the scale itself, the chain the same.
+    static constexpr bool GEMV1 = true;
+    static __device__ __forceinline__ void mma1(float16_t &acc, const Tile &w, const A8Regs &a, const void *, int, int) {
+        float f = acc[0];
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            float se, so;
+            halves_f(a.as[p], se, so);
+            int x0 = 0, x1 = 0;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                x0 = __builtin_amdgcn_sdot4((int)w.q[2 * p][i], (int)a.c[2 * p][i], x0, false);
+                x1 = __builtin_amdgcn_sdot4((int)w.q[2 * p + 1][i], (int)a.c[2 * p + 1][i], x1, false);
+            }
+            f = __builtin_fmaf((float)halves_sum(x0), se, f);
+            f = __builtin_fmaf((float)halves_sum(x1), so, f);
+        }
+        acc[0] = f;
+    }
     static constexpr int TILE_BYTES = 8192;
     static __device__ __forceinline__ void load(Tile &w, rd_rsrc_t r, int off, int lane) {
 #pragma unroll
@@ -294,8 +315,18 @@ extern "C" __global__ __launch_bounds__(320) void rd_k_retile_w4a8_8(const uint8
 struct W4A8Traits8 {
     typedef Q4K8Tile Tile;
     static constexpr int TILE_BYTES = 4608;
-    static constexpr bool GEMV1 = false;
-    static __device__ __forceinline__ void mma1(float16_t &, const Tile &, const A8Regs &, const void *, int, int) {}
+    static constexpr bool GEMV1 = true;
+    static __device__ __forceinline__ void mma1(float16_t &acc, const Tile &w, const A8Regs &a, const void *, int, int lane) {
+        const int h = lane >> 5;
+        float dsc[4], ndm[4];
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            const uint32_t wd = w.hdr[p];
+            dsc[p] = f16_bits_to_f32((uint16_t)(h ? wd >> 16 : wd & 0xffffu));
+            ndm[p] = -8.f * dsc[p];
+        }
+        Q4K8Traits::fold1(acc, w, a, dsc, ndm);
+    }
     static __device__ __forceinline__ void load(Tile &w, rd_rsrc_t r, int off, int lane) { Q4K8Traits::load(w, r, off, lane); }
     template <int NR> static __device__ __forceinline__ void mma(float16_t &acc, const Tile &w, const A8Regs &a, const void *, int, int lane) {
         const int h = lane >> 5;

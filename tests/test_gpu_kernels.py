@@ -170,7 +170,10 @@ def test_gemm_w8a8(dev, M, N, K):
     a = synth.normal(6, M * K).reshape(M, K)
     w = ob.WMat(ob.OR_W8A8, N, K, q, s, act_group=32)
     ref64 = ob.matmul_f64ref(w, a)
-    assert rel_err(dev.gemm_w8a8(q, s, a), ref64) < 1e-5
+    got = dev.gemm_w8a8(q, s, a)
+    assert rel_err(got, ref64) < 1e-5
+    for r in range(min(M, 3)):  # a row alone (the vector-ALU kernel) is the row of the batch, bit for bit
+        assert np.array_equal(dev.gemm_w8a8(q, s, a[r:r + 1])[0].view(np.uint32), got[r].view(np.uint32)), r
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 64, 128), (16, 768, 2048), (16, 2048, 768), (3, 64, 160)])
@@ -179,7 +182,10 @@ def test_gemm_w4a8(dev, M, N, K):
     a = synth.normal(9, M * K).reshape(M, K)
     w = ob.WMat(ob.OR_W4A8, N, K, nib, s16, act_group=32)
     ref64 = ob.matmul_f64ref(w, a)
-    assert rel_err(dev.gemm_w4a8(nib, s16, K, a), ref64) < 1e-5
+    got = dev.gemm_w4a8(nib, s16, K, a)
+    assert rel_err(got, ref64) < 1e-5
+    for r in range(min(M, 3)):  # a row alone (the vector-ALU kernel) is the row of the batch, bit for bit
+        assert np.array_equal(dev.gemm_w4a8(nib, s16, K, a[r:r + 1])[0].view(np.uint32), got[r].view(np.uint32)), r
 
 
 def test_rmsnorm_rope_route(dev):
