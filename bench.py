@@ -97,6 +97,8 @@ def parse_args():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--kv", default="f16", choices=["f16", "i8"],
                     help="KV cache element (c4 and c3): f16 as the metric is quoted, or goinfer's int8 cache (KVQuant i8), a variant of the workload")
+    ap.add_argument("--exp-act-group", type=int, default=0, choices=[0, 32],
+                    help="c5: the experts' activation quantization, 0 = one int8 scale per token row (the configuration as stated), 32 = per group of 32 (a variant)")
     ap.add_argument("--m", type=int, default=0, help="c2: only this batch width (for counter runs: one shape per kernel name)")
     ap.add_argument("--workload", default="c4", choices=["c4", "c2", "c3", "c5", "kquant", "topk", "prefill"],
                     help="c4 (default): the Llama-3-8B-shape step the metric is quoted on; c2: Q4_K GEMM microbench; c3: ragged "

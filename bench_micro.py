@@ -284,7 +284,8 @@ def run_c5(args):
     layers = args.layers if args.layers != 32 else 48
     B = args.batch if args.batch != 32 else 16
     steps, warmup = (args.steps if args.steps != 128 else 64), (args.warmup if args.warmup != 8 else 4)
-    cfg = workloads.qwen3_moe_cfg(layers)
+    cfg = workloads.qwen3_moe_cfg(layers, exp_act_group=getattr(args, "exp_act_group", 0))
+    row_act = cfg["exp_act_group"] == 0
     rng = np.random.default_rng(args.seed)
     lens = rng.integers(256, 2049, B).astype(np.int64)
     ids0 = rng.integers(0, cfg["vocab"], B).astype(np.int32)
@@ -323,9 +324,11 @@ def run_c5(args):
     d2 = float(sum(len(set(idx2[:, l, :].ravel().tolist())) for l in range(layers)))
     g_ms = prof["moe_gemm_gateup"][0] / prof["moe_gemm_gateup"][1]
     per_launch = d2 * ebytes * (2.0 / 3.0) / layers
-    traffic, t_ratio, t_src = counter_traffic("moe_gemv_w4a8_gateup/%s" % cfg["name"], per_launch)
+    gu_kernel = "rd_k_moe_gemv_w4a8r" if row_act else "rd_k_moe_gemv_w4a8_gateup"
+    traffic, t_ratio, t_src = counter_traffic("%s/%s" % (gu_kernel[5:], cfg["name"]), per_launch)
+    act_txt = "int8 activations per token row" if row_act else "int8 activations per group of 32 (a variant of the configuration)"
     out = base_line("batch-16 decode tok/s, Qwen3-MoE-30B-A3B shape (int4-g32 experts); achieved HBM GB/s vs peak", tok_s, "tok/s", steps, warmup,
-                    float(ms.mean()), "configs[4]: %s, %d layers, B=%d ragged, ctx U[256,2048], greedy decode" % (cfg["name"], layers, B),
+                    float(ms.mean()), "configs[4]: %s, %d layers, B=%d ragged, ctx U[256,2048], greedy decode, experts' %s" % (cfg["name"], layers, B, act_txt),
                     "synthetic: N(0,0.02) weights (Q4_K projections, int4-g32 experts, f32 router, int8 head), N(0,1) KV, random token ids",
                     {"batch": B, "ctx_min": int(lens.min()), "ctx_max": int(lens.max()), "ctx_mean": float(lens.mean()), "seed": args.seed,
                      "distinct_experts_per_layer_mean": round(float(np.mean(distinct)), 1)})
@@ -333,7 +336,7 @@ def run_c5(args):
                        "dense_weight_bytes": int(w_bytes), "expert_bytes": int(exp_bytes), "kv_read_bytes": int(kv_read)}
     out["roofline"] = {"bound": "hbm", "achieved": round(per_launch / (g_ms / 1e3) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                        "frac": round(per_launch / (g_ms / 1e3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_ratio": t_ratio, "traffic_source": t_src,
-                       "kernel": "rd_k_moe_gemv_w4a8_gateup",
+                       "kernel": gu_kernel,
                        "avg_launch_ms": round(g_ms, 5), "algorithmic_bytes_per_launch": int(per_launch)}
     out["kernel_classes"] = classes
     cpu = None
@@ -358,7 +361,8 @@ def cpu_baseline_moe(res, cfg, lens, kept_kv):
             lw[n] = kp[n]
         lw["router"] = ob.WMat.from_f32(kp["router"])
         for proj in ("gate", "up", "down"):
-            lw["exp_" + proj] = [ob.WMat(ob.OR_W4A8, ex[proj][2], ex[proj][3], ex[proj][0], ex[proj][1], act_group=32) for ex in kp["experts"]]
+            lw["exp_" + proj] = [ob.WMat(ob.OR_W4A8, ex[proj][2], ex[proj][3], ex[proj][0], ex[proj][1], act_group=cfg.get("exp_act_group", 32))
+                                 for ex in kp["experts"]]
         layers.append(lw)
     nL = len(layers)
     c = dict(cfg)

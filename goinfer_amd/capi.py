@@ -25,7 +25,7 @@ EXPORTS = [
     "rd_step_batch_draw", "rd_sample_rows", "rd_greedy_chain_start", "rd_greedy_chain_next", "rd_sample_chain_start",
     "rd_sample_chain_next", "rd_greedy_chain_stop",
     "rd_dequant_q5k", "rd_dequant_q6k", "rd_gemm_q5k", "rd_gemm_q6k", "rd_model_upload_q5k", "rd_model_upload_q6k",
-    "rd_kv_download", "rd_qkv_rope_store", "rd_topk_rows_static", "rd_quant_act",
+    "rd_kv_download", "rd_qkv_rope_store", "rd_topk_rows_static", "rd_quant_act", "rd_model_set_act_group",
 ]
 
 
@@ -191,22 +191,23 @@ class Device:
         check(lib().rd_gateup_q4k_quant(self.h, _p(gate), _p(up), I, K, _p(a), a.shape[0], _p(dst)), "rd_gateup_q4k_quant")
         return dst
 
-    def gemm_w8a8(self, q, scales, a):
+    def gemm_w8a8(self, q, scales, a, act_group=32):
+        """act_group 32: activations quantized per group of 32; 0: one scale per row (goinfer's ActQuantGroup)."""
         a = _f32(a)
         q = np.ascontiguousarray(q, dtype=np.int8)
         scales = _f32(scales)
         N, K = q.shape
         dst = np.empty((a.shape[0], N), np.float32)
-        check(lib().rd_gemm_w8a8(self.h, _p(q), _p(scales), N, K, _p(a), a.shape[0], _p(dst)), "rd_gemm_w8a8")
+        check(lib().rd_gemm_w8a8(self.h, _p(q), _p(scales), N, K, _p(a), a.shape[0], int(act_group), _p(dst)), "rd_gemm_w8a8")
         return dst
 
-    def gemm_w4a8(self, nib, s16, K, a):
+    def gemm_w4a8(self, nib, s16, K, a, act_group=32):
         a = _f32(a)
         nib = np.ascontiguousarray(nib, dtype=np.uint8)
         s16 = np.ascontiguousarray(s16, dtype=np.uint16)
         N = nib.shape[0]
         dst = np.empty((a.shape[0], N), np.float32)
-        check(lib().rd_gemm_w4a8(self.h, _p(nib), _p(s16), N, K, _p(a), a.shape[0], _p(dst)), "rd_gemm_w4a8")
+        check(lib().rd_gemm_w4a8(self.h, _p(nib), _p(s16), N, K, _p(a), a.shape[0], int(act_group), _p(dst)), "rd_gemm_w4a8")
         return dst
 
     def topk_rows(self, logits, k, temperature=1.0, want_z=True):
@@ -274,14 +275,15 @@ class Device:
                                       _p(bi), _p(q), _p(k), _p(v)), "rd_qkv_rope_store")
         return q, k, v
 
-    def quant_act(self, a):
-        """Per-32 int8 quantization of rows a [M][K]: (codes int8 [M][K], scales f32 [M][K/32], sums f32 [M][K/32])."""
+    def quant_act(self, a, act_group=32):
+        """int8 quantization of rows a [M][K]. act_group 32: (codes int8 [M][K], scales f32 [M][K/32], sums f32 [M][K/32]);
+        act_group 0, one scale per row: (codes, scales f32 [M], None)."""
         a = _f32(a)
         M, K = a.shape
         codes = np.empty((M, K), np.int8)
-        scales = np.empty((M, K // 32), np.float32)
-        sums = np.empty((M, K // 32), np.float32)
-        check(lib().rd_quant_act(self.h, _p(a), M, K, _p(codes), _p(scales), _p(sums)), "rd_quant_act")
+        scales = np.empty((M, K // 32) if act_group else (M,), np.float32)
+        sums = np.empty((M, K // 32), np.float32) if act_group else None
+        check(lib().rd_quant_act(self.h, _p(a), M, K, int(act_group), _p(codes), _p(scales), _p(sums)), "rd_quant_act")
         return codes, scales, sums
 
     def moe_route(self, logits, k, norm, bias=None, sigmoid=False, scale=0.0, n_group=0, topk_group=0):
@@ -409,6 +411,10 @@ class Model:
         s16 = np.ascontiguousarray(s16, dtype=np.uint16)
         check(lib().rd_model_upload_w4a8(self.h, layer, PROJ[proj], expert, _p(nib), _p(s16), nib.shape[0], K),
               "rd_model_upload_w4a8")
+
+    def set_act_group(self, act_group):
+        """goinfer's ActQuantGroup of the int8 / int4 tensors uploaded from here on: 32, or 0 = one activation scale per row."""
+        check(lib().rd_model_set_act_group(self.h, int(act_group)), "rd_model_set_act_group")
 
     def upload_f32(self, layer, which, v):
         v = _f32(v)

@@ -74,6 +74,10 @@ struct KName {
 static const KName kNames[] = {
     {"rd_k_dequant_q4k", &Kernels::dequant_q4k},
     {"rd_k_quant_act", &Kernels::quant_act},
+    {"rd_k_quant_act_row", &Kernels::quant_act_row},
+    {"rd_k_swiglu_quant_row", &Kernels::swiglu_quant_row},
+    {"rd_k_moe_gemv_w4a8r", &Kernels::moe_gemv_w4a8r},
+    {"rd_k_moe_swiglu_quant_row", &Kernels::moe_swiglu_quant_row},
     {"rd_k_reduce_splits", &Kernels::reduce_splits},
     {"rd_k_add_rmsnorm_quant", &Kernels::add_rmsnorm_quant},
     {"rd_k_swiglu_quant", &Kernels::swiglu_quant},
@@ -160,9 +164,9 @@ static int open_common(int ordinal, const void *image, rd_device **out) {
         }
         d->k.*(kn.slot) = f;
     }
-    static const char *kindName[3] = {"q4k", "w8a8", "w4a8"};
+    static const char *kindName[5] = {"q4k", "w8a8", "w4a8", "w8a8r", "w4a8r"};
     static const int kwOf[3] = {2, 4, 8};
-    for (int kind = 0; kind < 3; kind++)
+    for (int kind = 0; kind < 5; kind++)
         for (int i = 0; i < 6; i++) {
             char name[64];
             if (i < 3)
@@ -312,7 +316,7 @@ bool build_attn_worklist(const int *len, const int *slot, int G, int rows, int n
 // int8-MFMA kinds: enough waves to give every SIMD about two; K is cut inside the block first (KW waves per tile, their partial
 // sums folded in LDS, nothing through memory) and across blocks only when eight waves per tile still leave SIMDs idle.
 // The plan depends on the weight's shape only, never on the number of rows: a row is summed in the same order in any batch.
-GemmPlan plan_gemm(int kind, int N, int nKB) {
+GemmPlan plan_gemm(int kind, int N, int nKB, int act_group) {
     GemmPlan p;
     if (is_gemm8_kind(kind)) {
         const int tiles = (N + 31) / 32;
@@ -323,6 +327,7 @@ GemmPlan plan_gemm(int kind, int N, int nKB) {
         if (p.kw == 8) p.splits = std::max(1, std::min(want / 8, nKB / 8)); // every wave keeps at least one K-block
         if (const char *e = getenv("ROCMDECODE_GEMM8_KW")) p.kw = atoi(e) == 8 ? 8 : (atoi(e) == 2 ? 2 : 4);
         if (const char *e = getenv("ROCMDECODE_GEMM8_SPLITS")) p.splits = std::max(1, std::min(atoi(e), nKB));
+        if (act_group == 0) p.splits = 1;
         p.kbPerSplit = (nKB + p.splits - 1) / p.splits;
         p.splits = (nKB + p.kbPerSplit - 1) / p.kbPerSplit;
         return p;
@@ -345,6 +350,11 @@ size_t panel_bytes_for(const DevWeight &w) {
     return w.kind == 3 ? (size_t)(w.K / 256) * Q4K_PANEL_BYTES : (size_t)(w.K / 128) * LIN_PANEL_BYTES;
 }
 int panel_kind_for(const DevWeight &w) { return is_gemm8_kind(w.kind) ? PANEL_A8 : (w.kind == 3 ? PANEL_Q4K : PANEL_LIN); }
+int act_group_for(const DevWeight &w) { return w.kind == WKIND_GROUP ? (w.parts.empty() ? 32 : w.parts[0].act_group) : w.act_group; }
+int launch_quant_act(rd_device *d, const float *x, int M, int K, int kind, int act_group, void *Xp) {
+    if (act_group == 0) return d->launch(d->k.quant_act_row, (unsigned)M, 1, 1, 1024, x, Xp, K, kind);
+    return d->launch(d->k.quant_act, (unsigned)((K + 255) / 256), (unsigned)M, 1, 256, x, Xp, K, kind);
+}
 
 int upload_q4k(rd_device *d, const void *blocks, int N, int K, DevWeight *w) {
     if (N <= 0 || K <= 0 || K % 256 || N % 32) {
@@ -402,11 +412,18 @@ int upload_q6k(rd_device *d, const void *blocks, int N, int K, DevWeight *w) {
     return RD_OK;
 }
 
-int upload_w8a8(rd_device *d, const int8_t *q, const float *row_scale, int N, int K, DevWeight *w) {
+static bool act_group_ok(int g) {
+    if (g == 0 || g == 32) return true;
+    rd_set_error("rocm resident declines: activation quantization group %d (32 = per group of 32, 0 = one scale per row)", g);
+    return false;
+}
+
+int upload_w8a8(rd_device *d, const int8_t *q, const float *row_scale, int N, int K, DevWeight *w, int act_group) {
     if (N <= 0 || K <= 0 || K % 32 || N % 32) {
         rd_set_error("w8a8 upload: N=%d and K=%d must be multiples of 32", N, K);
         return RD_DECLINED;
     }
+    if (!act_group_ok(act_group)) return RD_DECLINED;
     size_t bytes = (size_t)N * K;
     const int nKB = (K + 255) / 256;
     DevBuf raw(d);
@@ -418,15 +435,16 @@ int upload_w8a8(rd_device *d, const int8_t *q, const float *row_scale, int N, in
     if ((rc = d->h2d(w->scales, row_scale, sizeof(float) * (size_t)N))) return rc;
     if ((rc = d->launch(d->k.retile_w8a8_8, N / 32, nKB, 1, 512, (const void *)raw.p, w->tiled, N, K))) return rc;
     if ((rc = d->sync())) return rc;
-    w->kind = 1, w->N = N, w->K = K;
+    w->kind = 1, w->N = N, w->K = K, w->act_group = act_group;
     return RD_OK;
 }
 
-int upload_w4a8(rd_device *d, const uint8_t *nib, const uint16_t *s16, int N, int K, DevWeight *w, bool expert) {
+int upload_w4a8(rd_device *d, const uint8_t *nib, const uint16_t *s16, int N, int K, DevWeight *w, bool expert, int act_group) {
     if (N <= 0 || K <= 0 || K % 32 || N % 32) {
         rd_set_error("w4a8 upload: N=%d and K=%d must be multiples of 32", N, K);
         return RD_DECLINED;
     }
+    if (!act_group_ok(act_group)) return RD_DECLINED;
     size_t nb = (size_t)N * K / 2, sb = (size_t)N * (K / 32) * 2;
     const int nKB = (K + 255) / 256;
     DevBuf raw(d), rs(d);
@@ -437,7 +455,7 @@ int upload_w4a8(rd_device *d, const uint8_t *nib, const uint16_t *s16, int N, in
     // an expert's weights take the tile order of the vector-ALU kernels (moe.h), a dense projection's that of the MFMA kernels
     if ((rc = d->launch(expert ? d->k.retile_w4a8_gv : d->k.retile_w4a8_8, N / 32, nKB, 1, 320, (const void *)raw.p, (const void *)rs.p, w->tiled, N, K))) return rc;
     if ((rc = d->sync())) return rc;
-    w->kind = 2, w->N = N, w->K = K;
+    w->kind = 2, w->N = N, w->K = K, w->act_group = act_group;
     return RD_OK;
 }
 
@@ -456,15 +474,19 @@ int launch_gemm(rd_device *d, const DevWeight &w, const void *Xp, float *P, int 
         return RD_ERR_ARG;
     }
     int nKB = kblocks_for(w);
-    GemmPlan p = plan_gemm(w.kind, w.N, nKB);
+    GemmPlan p = plan_gemm(w.kind, w.N, nKB, w.act_group);
     if (resid) splits = 1;
+    if (w.act_group == 0 && is_gemm8_kind(w.kind) && splits > 1) {
+        rd_set_error("gemm: a weight with per-row activation scales runs in one split (asked for %d)", splits);
+        return RD_ERR_STATE;
+    }
     if (splits > 0) p.kbPerSplit = (nKB + splits - 1) / splits, p.splits = splits;
     if (kw > 0) p.kw = kw;
     if (plan_out) *plan_out = p;
     if (ldP <= 0) ldP = w.N;
     if (is_gemm8_kind(w.kind)) {
         const int tiles = w.N / 32, tpb = p.kw == 2 ? 2 : 1;
-        hipFunction_t f = d->k.gemm8[w.kind][p.kw == 8 ? 2 : (p.kw == 4 ? 1 : 0)];
+        hipFunction_t f = d->k.gemm8[gemm8_lane(w)][p.kw == 8 ? 2 : (p.kw == 4 ? 1 : 0)];
         return d->launch(f, (unsigned)((tiles + tpb - 1) / tpb), (unsigned)p.splits, (unsigned)((M + 31) / 32), (unsigned)(64 * p.kw * tpb), (const void *)w.tiled,
                          (const void *)w.scales, Xp, P, w.N, nKB, p.kbPerSplit, M, ldP, resid, xpStride, pStride);
     }

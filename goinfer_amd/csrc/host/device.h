@@ -33,15 +33,16 @@ inline unsigned moe_gemv_grid(int N, int K) {
 }
 
 struct Kernels {
-    hipFunction_t dequant_q4k, quant_act, reduce_splits, add_rmsnorm_quant, swiglu_quant;
+    hipFunction_t dequant_q4k, quant_act, quant_act_row, reduce_splits, add_rmsnorm_quant, swiglu_quant, swiglu_quant_row;
     hipFunction_t unpack_act8, unpanel_a8, retile_q4k8, retile_w8a8_8, retile_w4a8_8;
-    hipFunction_t gemm8[3][3]; // [weight kind 0 q4k, 1 w8a8, 2 w4a8][waves per tile 2, 4, 8]
-    hipFunction_t gemm8_qkv[3][3]; // the q|k|v projection with RoPE and the KV store in its epilogue, indexed like gemm8
-    hipFunction_t gemm8_q4k_gateup, gemm8_q4k_gateup_gelu, add_one, moe_gemv_w4a8, moe_gemv_w4a8_gateup, retile_w4a8_gv, rope_table;
+    // [lane: 0 q4k, 1 w8a8, 2 w4a8 (per-32 activations), 3 w8a8, 4 w4a8 with one activation scale per row][waves per tile 2, 4, 8]
+    hipFunction_t gemm8[5][3];
+    hipFunction_t gemm8_qkv[5][3]; // the q|k|v projection with RoPE and the KV store in its epilogue, indexed like gemm8
+    hipFunction_t gemm8_q4k_gateup, gemm8_q4k_gateup_gelu, add_one, moe_gemv_w4a8, moe_gemv_w4a8r, moe_gemv_w4a8_gateup, retile_w4a8_gv, rope_table;
     hipFunction_t dequant_q5k, retile_q5k, gemm_q5k, dequant_q6k, retile_q6k, gemm_q6k;
     hipFunction_t kv_store, kv_read, qkv_rope_store, attn_partial, attn_partial_wide, attn_combine, attn_combine_quant;
     hipFunction_t kv_store_i8, qkv_rope_store_i8, attn_partial_i8, attn_partial_rows, attn_partial_rows_i8, attn_partial_deep, attn_partial_deep_i8, topk_rows, topk_hist, topk_pick, topk_finish;
-    hipFunction_t rmsnorm, rope, argmax_rows, argmax_final, matmul_f32, moe_route, moe_swiglu_quant, moe_fold, embed_rows, copy16, unpanel_q4k, fill_f16, fill_f32;
+    hipFunction_t rmsnorm, rope, argmax_rows, argmax_final, matmul_f32, moe_route, moe_swiglu_quant, moe_swiglu_quant_row, moe_fold, embed_rows, copy16, unpanel_q4k, fill_f16, fill_f32;
 };
 
 struct rd_device {
@@ -160,7 +161,8 @@ struct GemmPlan {
     int kbPerSplit; // K-blocks (blocks of 256, or 128 for Q6_K) per split
     int kw = 0;     // int8-MFMA kinds: waves per weight tile inside a block, each on its own K range (2, 4 or 8)
 };
-GemmPlan plan_gemm(int kind, int N, int nKB);
+// act_group 0 (one activation scale per row): one split, since the row's scale multiplies the finished sum inside the kernel
+GemmPlan plan_gemm(int kind, int N, int nKB, int act_group = 32);
 
 // Weight matrix resident on the device in its GEMM tiling.
 struct DevWeight {
@@ -168,6 +170,9 @@ struct DevWeight {
     int N = 0, K = 0;
     void *tiled = nullptr;  // re-tiled codes
     void *scales = nullptr; // w8a8: f32[N]
+    // goinfer's WeightMat.ActQuantGroup() for the int8 / int4 kinds: 32 = activations quantized per group of 32 (its q4k mode), 0 =
+    // one scale per row (its int8 / int4 modes; the only lane its staged QuantBackend hooks serve). K-quants are always 32.
+    int act_group = 32;
     std::vector<DevWeight> parts; // kind 5: the members, each of one kind, rows [col0[i], col0[i] + parts[i].N) of the group
     std::vector<int> col0;
 };
@@ -176,8 +181,14 @@ enum { WKIND_GROUP = 5 };
 int upload_q4k(rd_device *d, const void *blocks, int N, int K, DevWeight *w);
 int upload_q5k(rd_device *d, const void *blocks, int N, int K, DevWeight *w);
 int upload_q6k(rd_device *d, const void *blocks, int N, int K, DevWeight *w);
-int upload_w8a8(rd_device *d, const int8_t *q, const float *row_scale, int N, int K, DevWeight *w);
-int upload_w4a8(rd_device *d, const uint8_t *nib, const uint16_t *s16, int N, int K, DevWeight *w, bool expert = false);
+int upload_w8a8(rd_device *d, const int8_t *q, const float *row_scale, int N, int K, DevWeight *w, int act_group = 32);
+int upload_w4a8(rd_device *d, const uint8_t *nib, const uint16_t *s16, int N, int K, DevWeight *w, bool expert = false, int act_group = 32);
+// The activation quantizer a weight's GEMM expects of its producer: 32 or 0 (see DevWeight::act_group); a group's members agree.
+int act_group_for(const DevWeight &w);
+// index into Kernels::gemm8 / gemm8_qkv
+inline int gemm8_lane(const DevWeight &w) { return w.act_group == 0 && w.kind >= 1 ? w.kind + 2 : w.kind; }
+// x f32 [M][K] on the device -> the panels of `kind`, quantized per 32 (act_group 32) or per row (0). M <= 32.
+int launch_quant_act(rd_device *d, const float *x, int M, int K, int kind, int act_group, void *Xp);
 void free_weight(rd_device *d, DevWeight *w);
 // P[splits][32][N] = panels(Xp) . W^T ; returns the plan used
 // ldP: floats between rows of P (0 = w.N); splits > 0 forces the split count (trailing splits that get no K-block store zeros),

@@ -76,7 +76,7 @@ extern "C" void rd_model_destroy(rd_model *m) {
     }
     free_weight(d, &m->head);
     for (void *p : {(void *)m->embed_q, (void *)m->embed_scale, (void *)m->inv_freq_dev, (void *)m->rope_cs, (void *)m->final_norm, (void *)m->tables, (void *)m->h, (void *)m->normed, (void *)m->P, (void *)m->qbuf,
-                    (void *)m->part, (void *)m->cand_v, (void *)m->cand_i, (void *)m->logits, (void *)m->emb_dev, m->XpA, m->XpA2, m->XpB, (void *)m->ids, (void *)m->meta, (void *)m->router_logits, (void *)m->moe_wgt, (void *)m->moe_gu,
+                    (void *)m->part, (void *)m->attn_out, (void *)m->cand_v, (void *)m->cand_i, (void *)m->logits, (void *)m->emb_dev, m->XpA, m->XpA2, m->XpB, (void *)m->ids, (void *)m->meta, (void *)m->router_logits, (void *)m->moe_wgt, (void *)m->moe_gu,
                     (void *)m->moe_dn, (void *)m->moe_out, (void *)m->moe_idx, (void *)m->moe_idx_all, (void *)m->moe_rank, (void *)m->topk_ids, (void *)m->topk_vals, (void *)m->topk_z, (void *)m->topk_scratch.ghist, (void *)m->topk_scratch.ccount, (void *)m->topk_scratch.gmax, (void *)m->topk_scratch.cand_i, (void *)m->topk_scratch.cand_v, (void *)m->topk_scratch.invT, (void *)m->topk_scratch.zpart, m->XpE})
         d->release(p);
     if (m->host_stage) (void)d->hip->HostFree(m->host_stage);
@@ -125,24 +125,30 @@ static int upload_pending(rd_device *d, const PendingMat &p, DevWeight *w) {
     if (p.kind == 0) return upload_q4k(d, p.data.data(), p.N, p.K, w);
     if (p.kind == 3) return upload_q5k(d, p.data.data(), p.N, p.K, w);
     if (p.kind == 4) return upload_q6k(d, p.data.data(), p.N, p.K, w);
-    if (p.kind == 1) return upload_w8a8(d, (const int8_t *)p.data.data(), (const float *)p.scales.data(), p.N, p.K, w);
-    return upload_w4a8(d, p.data.data(), (const uint16_t *)p.scales.data(), p.N, p.K, w);
+    if (p.kind == 1) return upload_w8a8(d, (const int8_t *)p.data.data(), (const float *)p.scales.data(), p.N, p.K, w, p.act_group);
+    return upload_w4a8(d, p.data.data(), (const uint16_t *)p.scales.data(), p.N, p.K, w, false, p.act_group);
 }
 
 // Concatenate row-wise (all kinds are row-major with per-row side data) and upload as one weight. Members of different
 // kinds (a GGUF Q4_K_M file stores some attn_v as Q6_K, and goinfer's q4k mode turns those into int8 copies) become a group:
 // each run of one kind is its own weight, multiplied by its own kernel into the group's shared partial-sum buffer.
 static int fuse_and_upload(rd_device *d, PendingMat *parts, int n, DevWeight *w) {
-    for (int i = 1; i < n; i++)
+    auto group_of = [](const PendingMat &p) { return p.kind == 1 || p.kind == 2 ? p.act_group : 32; }; // K-quants are per-32 by kind
+    for (int i = 1; i < n; i++) {
         if (parts[i].K != parts[0].K) {
             rd_set_error("rocm resident declines: fused projections differ in K");
             return RD_DECLINED;
         }
+        if (group_of(parts[i]) != group_of(parts[0])) { // one quantizer feeds them all
+            rd_set_error("rocm resident declines: fused projections differ in activation quantization group (%d and %d)", group_of(parts[0]), group_of(parts[i]));
+            return RD_DECLINED;
+        }
+    }
     std::vector<PendingMat> runs;
     for (int i = 0; i < n; i++) {
         if (runs.empty() || runs.back().kind != parts[i].kind) {
             runs.emplace_back();
-            runs.back().kind = parts[i].kind, runs.back().K = parts[i].K, runs.back().N = 0;
+            runs.back().kind = parts[i].kind, runs.back().K = parts[i].K, runs.back().N = 0, runs.back().act_group = parts[i].act_group;
         }
         PendingMat &cat = runs.back();
         cat.N += parts[i].N;
@@ -266,7 +272,7 @@ extern "C" int rd_model_upload_w8a8(rd_model *m, int layer, int proj, const int8
     if (!layer_ok(m, layer, proj == RD_PROJ_HEAD)) return RD_ERR_ARG;
     RC(expect_shape(m, proj, N, K));
     PendingMat pm;
-    pm.kind = 1, pm.N = N, pm.K = K;
+    pm.kind = 1, pm.N = N, pm.K = K, pm.act_group = m->upload_act_group;
     pm.data.assign((const uint8_t *)q, (const uint8_t *)q + (size_t)N * K);
     pm.scales.assign((const uint8_t *)row_scale, (const uint8_t *)row_scale + sizeof(float) * (size_t)N);
     return accept(m, layer, proj, std::move(pm));
@@ -280,7 +286,7 @@ extern "C" int rd_model_upload_w4a8(rd_model *m, int layer, int proj, int expert
     if (expert < 0) {
         RC(expect_shape(m, proj, N, K));
         PendingMat pm;
-        pm.kind = 2, pm.N = N, pm.K = K;
+        pm.kind = 2, pm.N = N, pm.K = K, pm.act_group = m->upload_act_group;
         pm.data.assign(nib, nib + (size_t)N * K / 2);
         pm.scales.assign((const uint8_t *)s16, (const uint8_t *)s16 + 2 * (size_t)N * (K / 32));
         return accept(m, layer, proj, std::move(pm));
@@ -296,6 +302,15 @@ extern "C" int rd_model_upload_w4a8(rd_model *m, int layer, int proj, int expert
         rd_set_error("expert projection %d: got %dx%d", proj, N, K);
         return RD_ERR_ARG;
     }
+    if (m->exp_act_group >= 0 && m->exp_act_group != m->upload_act_group) {
+        rd_set_error("rocm resident declines: expert tensors differ in activation quantization group (%d and %d)", m->exp_act_group, m->upload_act_group);
+        return RD_DECLINED;
+    }
+    if (m->upload_act_group == 0 && I > 8192) {
+        rd_set_error("rocm resident declines: per-row expert activations with expert width %d (at most 8192)", I);
+        return RD_DECLINED;
+    }
+    m->exp_act_group = m->upload_act_group;
     LayerW &l = m->layers[(size_t)layer];
     size_t guBytes = (size_t)(2 * I / 32) * ((H + 255) / 256) * 4608, dnBytes = (size_t)(H / 32) * ((I + 255) / 256) * 4608;
     if (!l.exp_gateup) {
@@ -354,6 +369,23 @@ extern "C" int rd_model_upload_f32(rd_model *m, int layer, int which, const floa
     if (!*slot) RC(alloc_f32(d, slot, n));
     RC(d->h2d(*slot, v, sizeof(float) * n));
     return d->sync();
+}
+
+// WeightMat.ActQuantGroup() of the int8 / int4 tensors uploaded from here on (decoder/weightmat.go:837,909,936): 32 = activations
+// quantized per group of 32 (goinfer's q4k mode), 0 = one scale per row (its int8 / int4 modes, and the lane its staged
+// QuantBackend / QuantBackend4 hooks serve: decoder/backend.go:38-88).
+extern "C" int rd_model_set_act_group(rd_model *m, int act_group) {
+    if (!m) return RD_ERR_ARG;
+    if (m->finalized) {
+        rd_set_error("model already finalized");
+        return RD_ERR_STATE;
+    }
+    if (act_group != 0 && act_group != 32) {
+        rd_set_error("rocm resident declines: activation quantization group %d (32 = per group of 32, 0 = one scale per row)", act_group);
+        return RD_DECLINED;
+    }
+    m->upload_act_group = act_group;
+    return RD_OK;
 }
 
 // The router's variant (decoder/mlp.go:130-228 routeExperts / groupLimit), before rd_model_finalize.
@@ -423,7 +455,7 @@ extern "C" int rd_model_upload_embedding(rd_model *m, const int8_t *q, const flo
 // fewest any member's own plan asks for (no member then gets more splits than it has K-blocks).
 static GemmPlan group_plan(const DevWeight &w) {
     GemmPlan g{1 << 30, 0, 0};
-    for (const auto &p : w.parts) g.splits = std::min(g.splits, plan_gemm(p.kind, p.N, kblocks_for(p)).splits);
+    for (const auto &p : w.parts) g.splits = std::min(g.splits, plan_gemm(p.kind, p.N, kblocks_for(p), p.act_group).splits);
     return g;
 }
 
@@ -431,7 +463,7 @@ static size_t gemm_partial_floats(const DevWeight &w) {
     if (w.kind < 0) return 0;
     if (w.kind == WKIND_GROUP) return (size_t)group_plan(w).splits * 32 * w.N;
     int nKB = kblocks_for(w);
-    return (size_t)plan_gemm(w.kind, w.N, nKB).splits * 32 * w.N;
+    return (size_t)plan_gemm(w.kind, w.N, nKB, w.act_group).splits * 32 * w.N;
 }
 
 extern "C" int rd_model_finalize(rd_model *m) {
@@ -473,6 +505,7 @@ extern "C" int rd_model_finalize(rd_model *m) {
     RC(alloc_f32(d, &m->emb_dev, R * H));
     RC(alloc_f32(d, &m->normed, (size_t)32 * H));
     RC(alloc_f32(d, &m->qbuf, R * qd));
+    if (std::any_of(m->layers.begin(), m->layers.end(), [](const LayerW &l) { return act_group_for(l.o) == 0; })) RC(alloc_f32(d, &m->attn_out, R * qd));
     RC(alloc_f32(d, &m->logits, R * c.vocab));
     size_t kA = (size_t)H, kB = (size_t)std::max(qd, c.n_experts ? qd : c.inter);
     // room for either panel kind: 8 KB per 128 elements (int8/int4 consumers) or 17 KB per 256 (Q4_K consumers)
@@ -716,7 +749,8 @@ static int add_norm_quant(rd_model *m, int B, const float *P, int splits, const 
     int kA, kB;
     panel_kinds_of(next, &kA, &kB);
     return d->launch(d->k.add_rmsnorm_quant, (unsigned)B, 1, 1, 1024, m->h, P, splits, w, m->desc.rms_eps, m->desc.hidden, Xp, kA, norm_out,
-                     kB >= 0 ? m->XpA2 : (void *)nullptr, kB, m->pStride, m->xpAStride, m->xpAStride, foldW, P ? postW : (const float *)nullptr);
+                     kB >= 0 ? m->XpA2 : (void *)nullptr, kB, m->pStride, m->xpAStride, m->xpAStride, foldW, P ? postW : (const float *)nullptr,
+                     act_group_for(next));
 }
 
 // One GEMM, or for a group one GEMM per member into column ranges of the same P[split][32][N], all with the group's split
@@ -780,24 +814,30 @@ static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
     const int nKBh = (H + 255) / 256, nKBi = (I + 255) / 256;
     size_t guStride = (size_t)(2 * I / 32) * nKBh * 4608, dnStride = (size_t)(H / 32) * nKBi * 4608;
     size_t xpStride = a8_bytes(I);
-    if (I % 32 == 0 && !getenv("ROCMDECODE_NO_FUSED_MOE_GATEUP")) {
+    const bool rowAct = m->exp_act_group == 0; // one activation scale per row: SwiGLU's quantizer needs a whole row, so it is its own launch
+    hipFunction_t gemv = rowAct ? d->k.moe_gemv_w4a8r : d->k.moe_gemv_w4a8;
+    if (I % 32 == 0 && !rowAct && !getenv("ROCMDECODE_NO_FUSED_MOE_GATEUP")) {
         Scope s(m, KC_MOE_GEMM); // gate|up of every touched expert + SwiGLU + quantization into the experts' down activations
         RC(d->launch_lds(d->k.moe_gemv_w4a8_gateup, (unsigned)((I / 32 + 1) / 2), (unsigned)nE, 1, MOE_THREADS, moe_gemv_lds(H), (const void *)l.exp_gateup, guStride,
                          (const void *)m->XpA, m->XpE, xpStride, I, H, B, (const signed char *)m->moe_rank, nE, (const unsigned *)bits_dev));
     } else {
         {
             Scope s(m, KC_MOE_GEMM);
-            RC(d->launch_lds(d->k.moe_gemv_w4a8, moe_gemv_grid(2 * I, H), (unsigned)nE, 1, MOE_THREADS, moe_gemv_lds(H), (const void *)l.exp_gateup, guStride,
+            RC(d->launch_lds(gemv, moe_gemv_grid(2 * I, H), (unsigned)nE, 1, MOE_THREADS, moe_gemv_lds(H), (const void *)l.exp_gateup, guStride,
                              (const void *)m->XpA, (size_t)0, m->moe_gu, 2 * I, H, B, k, (const signed char *)m->moe_rank, nE,
                              (const unsigned *)bits_dev));
         }
         Scope s(m, KC_MOE_GLUE);
-        RC(d->launch(d->k.moe_swiglu_quant, (unsigned)((I + 255) / 256), (unsigned)(B * k), 1, 256, (const float *)m->moe_gu, (const int *)m->moe_idx,
-                     I, k, m->XpE, xpStride, (const signed char *)m->moe_rank, nE));
+        if (rowAct)
+            RC(d->launch(d->k.moe_swiglu_quant_row, (unsigned)(B * k), 1, 1, 256, (const float *)m->moe_gu, (const int *)m->moe_idx, I, k, m->XpE, xpStride,
+                         (const signed char *)m->moe_rank, nE));
+        else
+            RC(d->launch(d->k.moe_swiglu_quant, (unsigned)((I + 255) / 256), (unsigned)(B * k), 1, 256, (const float *)m->moe_gu, (const int *)m->moe_idx,
+                         I, k, m->XpE, xpStride, (const signed char *)m->moe_rank, nE));
     }
     {
         Scope s(m, KC_MOE_GEMM_DOWN);
-        RC(d->launch_lds(d->k.moe_gemv_w4a8, moe_gemv_grid(H, I), (unsigned)nE, 1, MOE_THREADS, moe_gemv_lds(I), (const void *)l.exp_down, dnStride,
+        RC(d->launch_lds(gemv, moe_gemv_grid(H, I), (unsigned)nE, 1, MOE_THREADS, moe_gemv_lds(I), (const void *)l.exp_down, dnStride,
                          (const void *)m->XpE, xpStride, m->moe_dn, H, I, B, k, (const signed char *)m->moe_rank, nE, (const unsigned *)bits_dev));
     }
     if (k > MOE_FOLD_FUSED_MAX) { // else the next norm kernel folds the ranks itself as it adds them to the residual
@@ -849,8 +889,8 @@ static int step_launches(rd_model *m, int B, int want) {
         if (qkv_fusable(m, l)) {
             Scope s(m, KC_GEMM_QKV); // projection, bias, RoPE and the KV store in one launch (M-tiles of 32 rows as grid.z)
             const DevWeight &w = l.qkv;
-            const int nKB = kblocks_for(w), kw = plan_gemm(w.kind, w.N, nKB).kw; // the plain GEMM's waves per tile, in one split
-            RC(d->launch(d->k.gemm8_qkv[w.kind][kw == 8 ? 2 : (kw == 4 ? 1 : 0)], (unsigned)(w.N / 32), 1, (unsigned)((B + 31) / 32), (unsigned)(64 * kw),
+            const int nKB = kblocks_for(w), kw = plan_gemm(w.kind, w.N, nKB, w.act_group).kw; // the plain GEMM's waves per tile, in one split
+            RC(d->launch(d->k.gemm8_qkv[gemm8_lane(w)][kw == 8 ? 2 : (kw == 4 ? 1 : 0)], (unsigned)(w.N / 32), 1, (unsigned)((B + 31) / 32), (unsigned)(64 * kw),
                          (const void *)w.tiled, (const void *)w.scales, (const void *)m->XpA, w.N, nKB, B, m->qbuf, l.Kp, l.Vp, (const int *)m->tables,
                          m->blocks_per_slot, (const int *)m->rowSlot, (const int *)m->rowPos, (const double *)m->rope_cs, (const float *)l.qkv_bias, nH, nKV,
                          HD, m->xpAStride));
@@ -875,7 +915,18 @@ static int step_launches(rd_model *m, int B, int want) {
             Scope s(m, KC_ATTN_PARTIAL);
             if (!m->bench_skip_attn) RC(launch_attn_partial(m, l));
         }
-        {
+        if (act_group_for(l.o) == 0) {
+            // the o projection takes one activation scale per row: the merged heads go out as f32 rows and the per-row quantizer
+            // (which needs the whole row's maximum) is its own launch
+            Scope s(m, KC_ATTN_COMBINE);
+            const int li = l.window > 0 ? 1 : 0;
+            RC(d->launch(d->k.attn_combine, (unsigned)nH, (unsigned)B, 1, (unsigned)(ATTN_PIECES * HD / 4), (const float *)m->part,
+                         (const int *)m->itemStart + (size_t)li * m->list_ints, m->last_grouped[li] ? ATTN_TILE_ROWS : nH / nKV, m->attn_out, nH, nKV, HD,
+                         (const float *)l.sinks));
+            for (int r0 = 0; r0 < B; r0 += 32)
+                RC(launch_quant_act(d, m->attn_out + (size_t)r0 * nH * HD, std::min(32, B - r0), nH * HD, panel_kind_for(l.o), 0,
+                                    (char *)m->XpB + (size_t)(r0 / 32) * m->xpBStride));
+        } else {
             Scope s(m, KC_ATTN_COMBINE);
             const int li = l.window > 0 ? 1 : 0;
             RC(d->launch(d->k.attn_combine_quant, (unsigned)nH, (unsigned)B, 1, (unsigned)(ATTN_PIECES * HD / 4), (const float *)m->part,
@@ -901,8 +952,12 @@ static int step_launches(rd_model *m, int B, int want) {
                         RC(launch_proj(m, l.gateup, m->XpA, m->xpAStride, B, &plan));
                 }
                 Scope s(m, KC_SWIGLU);
-                RC(d->launch(d->k.swiglu_quant, (unsigned)((c.inter + 1023) / 1024), (unsigned)B, 1, 256, (const float *)m->P, plan.splits, c.inter,
-                             m->XpB, panel_kind_for(l.down), (float *)nullptr, m->pStride, m->xpBStride, m->act));
+                if (act_group_for(l.down) == 0)
+                    RC(d->launch(d->k.swiglu_quant_row, (unsigned)B, 1, 1, 1024, (const float *)m->P, plan.splits, c.inter, m->XpB, panel_kind_for(l.down),
+                                 m->pStride, m->xpBStride, m->act));
+                else
+                    RC(d->launch(d->k.swiglu_quant, (unsigned)((c.inter + 1023) / 1024), (unsigned)B, 1, 256, (const float *)m->P, plan.splits, c.inter,
+                                 m->XpB, panel_kind_for(l.down), (float *)nullptr, m->pStride, m->xpBStride, m->act));
             }
             {
                 Scope s(m, KC_GEMM_DOWN);
@@ -914,7 +969,7 @@ static int step_launches(rd_model *m, int B, int want) {
                 Scope s(m, KC_ADD_NORM);
                 RC(d->launch(d->k.add_rmsnorm_quant, (unsigned)B, 1, 1, 1024, m->h, (const float *)m->P, plan.splits, (const float *)l.ffn_norm,
                              c.rms_eps, H, m->XpA, (int)PANEL_ROW8, m->normed, (void *)nullptr, -1, m->pStride, m->xpAStride, m->xpAStride,
-                             (const float *)nullptr, (const float *)nullptr));
+                             (const float *)nullptr, (const float *)nullptr, m->exp_act_group == 0 ? 0 : 32));
             }
             RC(moe_ffn(m, B, li, l));
             if (c.top_k <= MOE_FOLD_FUSED_MAX)

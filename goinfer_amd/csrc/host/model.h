@@ -12,6 +12,7 @@ enum {
 
 struct PendingMat { // a projection uploaded but not yet fused with its siblings (q|k|v, gate|up)
     int kind = -1, N = 0, K = 0;
+    int act_group = 32; // int8 / int4 kinds: WeightMat.ActQuantGroup() (32, or 0 = one activation scale per row)
     std::vector<uint8_t> data;
     std::vector<uint8_t> scales;
 };
@@ -57,6 +58,9 @@ struct rd_model {
     int router_sigmoid = 0, n_group = 0, topk_group = 0;
     float router_scale = 0.f;
     int window = 0; // the one window length the model's sliding-window layers share (0: none has one)
+    int upload_act_group = 32; // what rd_model_set_act_group last set: the ActQuantGroup of the int8 / int4 uploads that follow
+    int exp_act_group = -1;    // the experts' (one value for the model; -1 until the first expert tensor arrives)
+    float *attn_out = nullptr; // [max_rows][n_heads*head_dim] f32: the attention output ahead of a per-row quantizer (allocated when an o projection takes per-row activations)
     int norm_add_one = 0, act = 0; // (1 + w) norm weights; the gated FFN's activation (RD_ACT_*)
     float final_softcap = 0.f;     // > 0: logits become cap * tanh(logit / cap)
     float logit_mul = 0.f;         // not 0 or 1: logits are multiplied by it after the softcap (f32(1 / LogitScale))

@@ -28,10 +28,9 @@ extern "C" int rd_dequant_q4k(rd_device *d, const void *blocks, int N, int K, fl
     return d->d2h(out, o.p, nb * 256 * sizeof(float));
 }
 
-// a[M][K] host -> per-32 quantized f16 panels on the device, in chunks of 32 rows. Returns device buffers.
-static int quantize_rows(rd_device *d, const float *a_dev, int M, int K, int kind, size_t pbytes, void *Xp) {
-    (void)pbytes;
-    return d->launch(d->k.quant_act, (unsigned)((K + 255) / 256), (unsigned)M, 1, 256, a_dev, Xp, K, kind);
+// a[M][K] on the device (M <= 32) -> quantized panels of `kind`, per 32 or (act_group 0) per row.
+static int quantize_rows(rd_device *d, const float *a_dev, int M, int K, int kind, int act_group, void *Xp) {
+    return launch_quant_act(d, a_dev, M, K, kind, act_group, Xp);
 }
 
 static int gemm_host(rd_device *d, DevWeight &w, DevWeight *w2, const float *a, int M, float *dst) {
@@ -44,7 +43,7 @@ static int gemm_host(rd_device *d, DevWeight &w, DevWeight *w2, const float *a, 
     RC(Xp.alloc(pbytes * tiles));
     int nKB = kblocks_for(w);
     int Ntot = w2 ? 2 * N : N;
-    int maxSplits = plan_gemm(w.kind, Ntot, nKB).splits;
+    int maxSplits = plan_gemm(w.kind, Ntot, nKB, w.act_group).splits;
     const size_t pStride = (size_t)maxSplits * 32 * Ntot;
     RC(P.alloc(sizeof(float) * pStride * tiles));
     RC(O.alloc(sizeof(float) * (size_t)chunk * N));
@@ -52,7 +51,7 @@ static int gemm_host(rd_device *d, DevWeight &w, DevWeight *w2, const float *a, 
         int mc = std::min(chunk, M - m0);
         RC(d->h2d(A.p, a + (size_t)m0 * K, sizeof(float) * (size_t)mc * K));
         for (int t = 0; t * 32 < mc; t++)
-            RC(quantize_rows(d, A.as<float>() + (size_t)t * 32 * K, std::min(32, mc - t * 32), K, kind, pbytes, (char *)Xp.p + (size_t)t * pbytes));
+            RC(quantize_rows(d, A.as<float>() + (size_t)t * 32 * K, std::min(32, mc - t * 32), K, kind, w.act_group, (char *)Xp.p + (size_t)t * pbytes));
         GemmPlan plan;
         if (!w2) {
             RC(launch_gemm_wide(d, w, Xp.p, pbytes, P.as<float>(), pStride, mc, &plan));
@@ -126,7 +125,7 @@ extern "C" int rd_gateup_q4k_quant(rd_device *d, const void *Wg, const void *Wu,
         for (int m0 = 0; m0 < M; m0 += 32) {
             int mc = std::min(32, M - m0);
             RC(d->h2d(A.p, a + (size_t)m0 * K, sizeof(float) * (size_t)mc * K));
-            RC(quantize_rows(d, A.as<float>(), mc, K, PANEL_A8, 0, Xp.p));
+            RC(quantize_rows(d, A.as<float>(), mc, K, PANEL_A8, 32, Xp.p));
             RC(d->launch(d->k.gemm8_q4k_gateup, (unsigned)(I / 32), 1, 1, GATEUP_THREADS, (const void *)w.tiled, (const void *)Xp.p, X2.as<uint8_t>(),
                          (int)PANEL_A8, I, K / 256, mc, (size_t)0, (size_t)0));
             RC(d->launch(d->k.unpanel_a8, (unsigned)(I / 256), (unsigned)mc, 1, 256, (const void *)X2.p, O.as<float>(), I));
@@ -139,15 +138,17 @@ extern "C" int rd_gateup_q4k_quant(rd_device *d, const void *Wg, const void *Wu,
     return rc;
 }
 
-// The activation quantizer on its own (goinfer: aikit QuantizeActQ group 32, call sites decoder/weightmat.go:845-862;
-// backend/cuda/actgroup.cu:32-54 quantG32): a f32 [M][K] -> int8 codes [M][K], f32 scales and sums (scale * sum of codes) [M][K/32],
-// as the GEMMs consume them. K % 32 == 0.
-extern "C" int rd_quant_act(rd_device *d, const float *a, int M, int K, int8_t *codes, float *scales, float *sums) {
-    if (!d || !a || !codes || !scales || !sums || M <= 0 || K <= 0 || K % 32) {
-        rd_set_error("rd_quant_act: bad arguments (K must be a multiple of 32)");
+// The activation quantizer on its own (goinfer: aikit QuantizeActQ, call sites decoder/weightmat.go:845-862;
+// backend/cuda/actgroup.cu:32-54 quantG32, kv8_store.cu:27-35 for the per-row rule): a f32 [M][K] -> int8 codes [M][K] and,
+// act_group 32: f32 scales and sums (scale * sum of codes) [M][K/32]; act_group 0: one scale per row, scales [M] (sums untouched,
+// may be NULL). As the GEMMs consume them. K % 32 == 0.
+extern "C" int rd_quant_act(rd_device *d, const float *a, int M, int K, int act_group, int8_t *codes, float *scales, float *sums) {
+    if (!d || !a || !codes || !scales || (!sums && act_group != 0) || M <= 0 || K <= 0 || K % 32 || (act_group != 0 && act_group != 32)) {
+        rd_set_error("rd_quant_act: bad arguments (K must be a multiple of 32, act_group 32 or 0)");
         return RD_ERR_ARG;
     }
     const int nG = K / 32;
+    std::vector<float> rowS((size_t)32 * nG);
     DevBuf A(d), A8(d), C(d), S(d), U(d);
     RC(A.alloc(sizeof(float) * (size_t)32 * K));
     RC(A8.alloc(a8_bytes(K)));
@@ -157,9 +158,14 @@ extern "C" int rd_quant_act(rd_device *d, const float *a, int M, int K, int8_t *
     for (int m0 = 0; m0 < M; m0 += 32) {
         const int mc = std::min(32, M - m0);
         RC(d->h2d(A.p, a + (size_t)m0 * K, sizeof(float) * (size_t)mc * K));
-        RC(quantize_rows(d, A.as<float>(), mc, K, PANEL_A8, 0, A8.p));
+        RC(quantize_rows(d, A.as<float>(), mc, K, PANEL_A8, act_group, A8.p));
         RC(d->launch(d->k.unpack_act8, (unsigned)((K + 255) / 256), (unsigned)mc, 1, 256, (const void *)A8.p, (signed char *)C.p, S.as<float>(), U.as<float>(), K));
         RC(d->d2h(codes + (size_t)m0 * K, C.p, (size_t)mc * K));
+        if (act_group == 0) { // the row's scale sits in every group slot: the first is returned
+            RC(d->d2h(rowS.data(), S.p, sizeof(float) * (size_t)mc * nG));
+            for (int r = 0; r < mc; r++) scales[m0 + r] = rowS[(size_t)r * nG];
+            continue;
+        }
         RC(d->d2h(scales + (size_t)m0 * nG, S.p, sizeof(float) * (size_t)mc * nG));
         RC(d->d2h(sums + (size_t)m0 * nG, U.p, sizeof(float) * (size_t)mc * nG));
     }
@@ -211,20 +217,20 @@ extern "C" int rd_gemm_q6k(rd_device *d, const void *W, int N, int K, const floa
     return rc;
 }
 
-extern "C" int rd_gemm_w8a8(rd_device *d, const int8_t *q, const float *row_scale, int N, int K, const float *a, int M, float *dst) {
+extern "C" int rd_gemm_w8a8(rd_device *d, const int8_t *q, const float *row_scale, int N, int K, const float *a, int M, int act_group, float *dst) {
     if (!d || !q || !row_scale || !a || !dst || M <= 0) return RD_ERR_ARG;
     DevWeight w;
-    int rc = upload_w8a8(d, q, row_scale, N, K, &w);
+    int rc = upload_w8a8(d, q, row_scale, N, K, &w, act_group);
     if (rc) return rc;
     rc = gemm_host(d, w, nullptr, a, M, dst);
     free_weight(d, &w);
     return rc;
 }
 
-extern "C" int rd_gemm_w4a8(rd_device *d, const uint8_t *nib, const uint16_t *s16, int N, int K, const float *a, int M, float *dst) {
+extern "C" int rd_gemm_w4a8(rd_device *d, const uint8_t *nib, const uint16_t *s16, int N, int K, const float *a, int M, int act_group, float *dst) {
     if (!d || !nib || !s16 || !a || !dst || M <= 0) return RD_ERR_ARG;
     DevWeight w;
-    int rc = upload_w4a8(d, nib, s16, N, K, &w);
+    int rc = upload_w4a8(d, nib, s16, N, K, &w, false, act_group);
     if (rc) return rc;
     rc = gemm_host(d, w, nullptr, a, M, dst);
     free_weight(d, &w);

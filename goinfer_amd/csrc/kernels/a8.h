@@ -49,6 +49,17 @@ __device__ __forceinline__ uint32_t quant8_g32x4(float v0, float v1, float v2, f
     *gsum = __fmul_rn(s, (float)group_sum8_i(c0 + c1 + c2 + c3));
     return (uint32_t)(c0 & 255) | ((uint32_t)(c1 & 255) << 8) | ((uint32_t)(c2 & 255) << 16) | ((uint32_t)(c3 & 255) << 24);
 }
+// One scale for the whole row (goinfer's ActQuantGroup 0: linalg.QuantizeRowInt8, twin backend/cuda/kv8_store.cu:27-35): the
+// four consecutive elements of a lane against the row's scale s = maxabs/127 (1 for an all-zero row), codes round-half-away.
+// *gsum = s * sum of the codes of the lane's group of 32 (8 consecutive lanes), as the per-32 form stores it.
+__device__ __forceinline__ float row_scale_of(float maxabs) { return maxabs == 0.f ? 1.f : maxabs / 127.f; }
+__device__ __forceinline__ uint32_t quant8_rowx4(float v0, float v1, float v2, float v3, float s, float *gsum) {
+    const float inv = 1.f / s;
+    const int c0 = (int)fminf(127.f, fmaxf(-127.f, roundf(__fmul_rn(v0, inv)))), c1 = (int)fminf(127.f, fmaxf(-127.f, roundf(__fmul_rn(v1, inv))));
+    const int c2 = (int)fminf(127.f, fmaxf(-127.f, roundf(__fmul_rn(v2, inv)))), c3 = (int)fminf(127.f, fmaxf(-127.f, roundf(__fmul_rn(v3, inv))));
+    *gsum = __fmul_rn(s, (float)group_sum8_i(c0 + c1 + c2 + c3));
+    return (uint32_t)(c0 & 255) | ((uint32_t)(c1 & 255) << 8) | ((uint32_t)(c2 & 255) << 16) | ((uint32_t)(c3 & 255) << 24);
+}
 // Stores four consecutive elements k0..k0+3 (k0 % 4 == 0) of batch row m and, from the group's first lane, its scale and sum.
 __device__ __forceinline__ void a8_store4(uint8_t *__restrict__ A8, int m, int k0, uint32_t codes, float sc, float gsum) {
     *(uint32_t *)(A8 + a8_code_offset(m, k0)) = codes;

@@ -31,6 +31,26 @@ __device__ __forceinline__ Quant4 quant_four(float v0, float v1, float v2, float
     return q;
 }
 
+// The same against a scale that belongs to the whole row (ActQuantGroup 0).
+__device__ __forceinline__ Quant4 quant_four_row(float v0, float v1, float v2, float v3, float s) {
+    Quant4 q;
+    q.sc = s;
+    q.codes = quant8_rowx4(v0, v1, v2, v3, s, &q.gsum);
+#pragma unroll
+    for (int i = 0; i < 4; i++) q.x[i] = __fmul_rn((float)(int)(signed char)(q.codes >> (8 * i)), q.sc);
+    return q;
+}
+// The maximum of v over a block of up to 1024 threads, on every thread. red: 16 floats of LDS; every thread calls it.
+__device__ __forceinline__ float block_max(float v, float *red) {
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    __syncthreads(); // red may still be read from an earlier call
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float m = 0.f;
+    for (int i = 0; i < (int)((blockDim.x + 63) >> 6); i++) m = fmaxf(m, red[i]);
+    return m;
+}
+
 // Store one quantized activation (element k of batch row m) in the layout the consuming GEMM reads. ldk: the row length, for
 // the one layout that needs it (RD_PANEL_ROW8).
 __device__ __forceinline__ void panel_store(uint8_t *__restrict__ Xp, int kind, int m, int k, const Quant1 &q, int ldk = 0) {
@@ -92,6 +112,28 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_quant_act(const float *__
     if (k < K || kind == RD_PANEL_A8) panel_store(Xp, kind, m, k, q); // A8: the tail of the last block is written as zero groups
 }
 
+// The same with one scale per row (ActQuantGroup 0: linalg.QuantizeRowInt8; the scale lands in every group's slot of the row, the
+// sums stay per group of 32). Grid (M), 1024 threads, four consecutive elements per thread and round; K % 32 == 0. The row is
+// read twice: once for its maximum, once for its codes.
+extern "C" __global__ __launch_bounds__(1024) void rd_k_quant_act_row(const float *__restrict__ x, uint8_t *__restrict__ Xp, int K, int kind) {
+    __shared__ float red[16];
+    const int m = blockIdx.x, t = threadIdx.x, nv = K >> 2;
+    const int nvPad = kind == RD_PANEL_A8 ? ((K + 255) >> 8) << 6 : nv; // A8: the tail of the last block is written as zero codes
+    const float *row = x + (size_t)m * K;
+    float ma = 0.f;
+    for (int q = t; q < nv; q += 1024) {
+        const float4_t v = *(const float4_t *)(row + 4 * q);
+        ma = fmaxf(ma, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+    }
+    const float s = row_scale_of(block_max(ma, red));
+    for (int q = t; q < nvPad; q += 1024) { // groups of 8 lanes are inside K or past it together
+        float4_t v = {0.f, 0.f, 0.f, 0.f};
+        if (q < nv) v = *(const float4_t *)(row + 4 * q);
+        const Quant4 qq = quant_four_row(v.x, v.y, v.z, v.w, s);
+        panel_store4(Xp, kind, m, 4 * q, qq, K);
+    }
+}
+
 // out[m][n] = sum_s P[s][m][n] in ascending split order (deterministic).
 extern "C" __global__ void rd_k_reduce_splits(const float *__restrict__ P, float *__restrict__ out, int N, int splits) {
     int m = blockIdx.y, n = blockIdx.x * 256 + threadIdx.x;
@@ -117,8 +159,9 @@ extern "C" __global__ __launch_bounds__(1024) void rd_k_add_rmsnorm_quant(float 
                                                                           uint8_t *__restrict__ Xp, int kind, float *__restrict__ norm_out,
                                                                           uint8_t *__restrict__ Xp2, int kind2, size_t pStride, size_t xpStride,
                                                                           size_t xp2Stride, const float *__restrict__ foldW,
-                                                                          const float *__restrict__ postW) {
+                                                                          const float *__restrict__ postW, int actGroup) {
     __shared__ double red[16], redPost[16];
+    __shared__ float redMax[16];
     const int m = blockIdx.x, t = threadIdx.x, nv = H >> 2;
     // rows beyond 32 are further M-tiles: their partial sums and panels sit pStride floats / xpStride bytes further on
     const int mt = m >> 5, mr = m & 31;
@@ -223,14 +266,25 @@ extern "C" __global__ __launch_bounds__(1024) void rd_k_add_rmsnorm_quant(float 
 #pragma unroll
     for (int i = 0; i < 16; i++) ss += red[i];
     float inv = (float)(1.0 / sqrt(ss / (double)H + (double)eps));
+    float4_t nn[2];
+    float ma = 0.f;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        nn[i] = (float4_t){0.f, 0.f, 0.f, 0.f};
+        if (!on[i]) continue;
+        nn[i].x = __fmul_rn(__fmul_rn(v[i].x, inv), wv[i].x), nn[i].y = __fmul_rn(__fmul_rn(v[i].y, inv), wv[i].y);
+        nn[i].z = __fmul_rn(__fmul_rn(v[i].z, inv), wv[i].z), nn[i].w = __fmul_rn(__fmul_rn(v[i].w, inv), wv[i].w);
+        ma = fmaxf(ma, fmaxf(fmaxf(fabsf(nn[i].x), fabsf(nn[i].y)), fmaxf(fabsf(nn[i].z), fabsf(nn[i].w))));
+    }
+    // actGroup 0: the consuming projections take one activation scale per row (linalg.QuantizeRowInt8) instead of one per 32
+    const float rowS = actGroup == 0 ? row_scale_of(block_max(ma, redMax)) : 0.f;
 #pragma unroll
     for (int i = 0; i < 2; i++) {
         if (!on[i]) continue; // whole waves drop out together: nv is a multiple of 32
         int k0 = 4 * (t + i * 1024);
-        float n0 = __fmul_rn(__fmul_rn(v[i].x, inv), wv[i].x), n1 = __fmul_rn(__fmul_rn(v[i].y, inv), wv[i].y);
-        float n2 = __fmul_rn(__fmul_rn(v[i].z, inv), wv[i].z), n3 = __fmul_rn(__fmul_rn(v[i].w, inv), wv[i].w);
-        if (norm_out) *(float4_t *)(norm_out + (size_t)m * H + k0) = (float4_t){n0, n1, n2, n3};
-        const Quant4 q = quant_four(n0, n1, n2, n3);
+        const float n0 = nn[i].x, n1 = nn[i].y, n2 = nn[i].z, n3 = nn[i].w;
+        if (norm_out) *(float4_t *)(norm_out + (size_t)m * H + k0) = nn[i];
+        const Quant4 q = actGroup == 0 ? quant_four_row(n0, n1, n2, n3, rowS) : quant_four(n0, n1, n2, n3);
         panel_store4(Xp, kind, mr, k0, q, H);
         if (Xp2) panel_store4(Xp2, kind2, mr, k0, q, H); // a second consumer that reads another panel layout
     }
@@ -261,6 +315,42 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_swiglu_quant(const float 
     }
     const Quant4 q = quant_four(a[0], a[1], a[2], a[3]);
     if (on) panel_store4(Xp, kind, m, n0, q);
+}
+
+// The same with one scale per row of I (ActQuantGroup 0). Grid (M), 1024 threads: a thread keeps up to eight groups of four
+// columns (I <= 32768, I % 32 == 0) in registers between the row's maximum and its codes.
+extern "C" __global__ __launch_bounds__(1024) void rd_k_swiglu_quant_row(const float *__restrict__ P, int splits, int I, uint8_t *__restrict__ Xp,
+                                                                         int kind, size_t pStride, size_t xpStride, int act) {
+    __shared__ float red[16];
+    const int row = blockIdx.x, m = row & 31, t = threadIdx.x, nv = I >> 2, N2 = 2 * I;
+    P += (size_t)(row >> 5) * pStride;
+    Xp += (size_t)(row >> 5) * xpStride;
+    float4_t a[8];
+    float ma = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const int q = t + i * 1024;
+        a[i] = (float4_t){0.f, 0.f, 0.f, 0.f};
+        if (q >= nv) continue;
+        const int n0 = 4 * q;
+        float4_t g = *(const float4_t *)(P + (size_t)m * N2 + n0), u = *(const float4_t *)(P + (size_t)m * N2 + I + n0);
+        for (int s = 1; s < splits; s++) {
+            float4_t g2 = *(const float4_t *)(P + ((size_t)s * 32 + m) * N2 + n0), u2 = *(const float4_t *)(P + ((size_t)s * 32 + m) * N2 + I + n0);
+            g.x = __fadd_rn(g.x, g2.x), g.y = __fadd_rn(g.y, g2.y), g.z = __fadd_rn(g.z, g2.z), g.w = __fadd_rn(g.w, g2.w);
+            u.x = __fadd_rn(u.x, u2.x), u.y = __fadd_rn(u.y, u2.y), u.z = __fadd_rn(u.z, u2.z), u.w = __fadd_rn(u.w, u2.w);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; e++) a[i][e] = __fmul_rn(gate_act(g[e], act), u[e]);
+        ma = fmaxf(ma, fmaxf(fmaxf(fabsf(a[i].x), fabsf(a[i].y)), fmaxf(fabsf(a[i].z), fabsf(a[i].w))));
+    }
+    const float s = row_scale_of(block_max(ma, red));
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const int q = t + i * 1024;
+        if (q >= nv) continue; // groups of 8 lanes are on or off together
+        const Quant4 qq = quant_four_row(a[i].x, a[i].y, a[i].z, a[i].w, s);
+        panel_store4(Xp, kind, m, 4 * q, qq, I);
+    }
 }
 
 // A Q4_K-layout activation panel set back to rows: out[m][k] = the f16 value (code * scale) the GEMM reads for batch row m,

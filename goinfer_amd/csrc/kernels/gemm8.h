@@ -216,7 +216,8 @@ struct Q4K8Traits {
         }
         acc[0] = f;
     }
-    static __device__ __forceinline__ void finish(float16_t &, const void *, int, int) {}
+    static constexpr bool INT_ACC = false;
+    static __device__ __forceinline__ void finish(float16_t &, const void *, const uint8_t *, int, int) {}
 };
 
 // ---------------- W8A8: int8 codes, one f32 scale per row (goinfer WeightMat.Int8; backend/cuda/actgroup.cu:283-288,421-437) ----------------
@@ -272,10 +273,49 @@ struct W8A8Traits8 {
             RD_FOLD(acc, d1, s2, 16, NR)
         }
     }
-    static __device__ __forceinline__ void finish(float16_t &acc, const void *aux, int tile, int lane) {
+    static constexpr bool INT_ACC = false;
+    static __device__ __forceinline__ void finish(float16_t &acc, const void *aux, const uint8_t *, int tile, int lane) {
         const float ws = ((const float *)aux)[tile * 32 + (lane & 31)];
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[r] = mul_rounded(acc[r], ws);
+    }
+};
+
+// The scale of batch row m of an M-tile whose activations carry one scale per row (ActQuantGroup 0): the row's scale sits in
+// every group slot of its A8 blocks; the first block's first slot is read.
+__device__ __forceinline__ float a8_row_scale(const uint8_t *__restrict__ A8, int m) { return *(const float *)(A8 + a8_scale_offset(m, 0)); }
+
+// W8A8 with one activation scale per row (goinfer's ActQuantGroup 0, the lane its staged QuantBackend.MatmulW8A8 hook serves:
+// decoder/backend.go:38-46, weightmat.go:931-947; device twin internal/gpudev/gemv_quant.cu:99-112): the int32 dot runs over the
+// whole of K, exactly, on the matrix core's own accumulator (no fold in the loop at all), and the result is
+// dst = (f32(idot) * aS[m]) * wScale[n], two rounded multiplies: linalg.MatmulBTW8A8 bit for bit, whatever the order of the
+// partial dots. The sixteen accumulators are int32 values kept in the float registers' bits.
+struct W8A8RowTraits8 {
+    typedef W8Tile8 Tile;
+    static constexpr int TILE_BYTES = 8192;
+    static constexpr bool GEMV1 = true, INT_ACC = true;
+    static __device__ __forceinline__ void load(Tile &w, rd_rsrc_t r, int off, int lane) { W8A8Traits8::load(w, r, off, lane); }
+    template <int NR> static __device__ __forceinline__ void mma(float16_t &acc, const Tile &w, const A8Regs &a, const void *, int, int) {
+        i32x16_t d = __builtin_bit_cast(i32x16_t, acc);
+#pragma unroll
+        for (int g = 0; g < 8; g++) d = __builtin_amdgcn_mfma_i32_32x32x32_i8(as_i32x4(a.c[g]), as_i32x4(w.q[g]), d, 0, 0, 0);
+        acc = __builtin_bit_cast(float16_t, d);
+    }
+    static __device__ __forceinline__ void mma1(float16_t &acc, const Tile &w, const A8Regs &a, const void *, int, int) {
+        int x = 0;
+#pragma unroll
+        for (int g = 0; g < 8; g++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) x = __builtin_amdgcn_sdot4((int)w.q[g][i], (int)a.c[g][i], x, false);
+        acc[0] = __int_as_float(__float_as_int(acc[0]) + halves_sum(x));
+    }
+    static __device__ __forceinline__ void finish(float16_t &acc, const void *aux, const uint8_t *A8, int tile, int lane) {
+        const float ws = ((const float *)aux)[tile * 32 + (lane & 31)];
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int m = (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+            acc[r] = mul_rounded(mul_rounded((float)__float_as_int(acc[r]), a8_row_scale(A8, m)), ws);
+        }
     }
 };
 
@@ -354,7 +394,69 @@ struct W4A8Traits8 {
 #pragma unroll
         for (int p = 0; p < 4; p++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.asum[p], ndm[p], acc, 0, 0, 0);
     }
-    static __device__ __forceinline__ void finish(float16_t &, const void *, int, int) {}
+    static constexpr bool INT_ACC = false;
+    static __device__ __forceinline__ void finish(float16_t &, const void *, const uint8_t *, int, int) {}
+};
+
+// W4A8 with one activation scale per row (ActQuantGroup 0, the lane goinfer's staged QuantBackend4.MatmulW4A8 hook and its expert
+// kernels serve: decoder/backend.go:55-75, weightmat.go:904-912; device twins internal/gpudev/gemv_quant.cu:40-95,
+// backend/cuda/moe_rows.cu:24-106): per group of 32 facc = fma(f32(idot_g), ws_g, facc) with the signed dot of nib-8, and
+// dst = facc * aS[m] at the end. The stored nibble xor 8 is the two's-complement nibble of nib-8; at the top of a byte it is the
+// int8 16*(nib-8), so the matrix core's dot is 16 times the group's, exactly, and the 1/16 rides in the scale (a power of two:
+// the fma sees the same real product). The weight scale belongs to the lane (its column), so there is no scale outer product
+// and no sum term: eight int8 MFMAs a block and a convert and an fma per output and group.
+struct W4A8RowTraits8 {
+    typedef Q4K8Tile Tile;
+    static constexpr int TILE_BYTES = 4608;
+    static constexpr bool GEMV1 = true, INT_ACC = false;
+    static __device__ __forceinline__ void load(Tile &w, rd_rsrc_t r, int off, int lane) { Q4K8Traits::load(w, r, off, lane); }
+    static __device__ __forceinline__ void scales(const Tile &w, int p, float &s0, float &s1) { // groups 2p and 2p+1 of the lane's column, / 16
+        const uint32_t wd = w.hdr[p];
+        s0 = f16_bits_to_f32((uint16_t)(wd & 0xffffu)) * 0.0625f, s1 = f16_bits_to_f32((uint16_t)(wd >> 16)) * 0.0625f;
+    }
+    template <int NR> static __device__ __forceinline__ void mma(float16_t &acc, const Tile &w, const A8Regs &a, const void *, int, int) {
+        const i32x16_t zero16 = {0};
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            uint4_t lo, hi;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t x = w.q[p][i] ^ 0x88888888u;
+                lo[i] = (x << 4) & 0xF0F0F0F0u, hi[i] = x & 0xF0F0F0F0u;
+            }
+            float s0, s1;
+            scales(w, p, s0, s1);
+            const i32x16_t d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(as_i32x4(a.c[2 * p]), as_i32x4(lo), zero16, 0, 0, 0);
+            const i32x16_t d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(as_i32x4(a.c[2 * p + 1]), as_i32x4(hi), zero16, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < NR; r++) acc[r] = __builtin_fmaf((float)d0[r], s0, acc[r]);
+#pragma unroll
+            for (int r = 0; r < NR; r++) acc[r] = __builtin_fmaf((float)d1[r], s1, acc[r]);
+        }
+    }
+    // one batch row on the vector ALU: the same chain (group 2p, then 2p+1, one fma each), the dot from the two lane halves
+    static __device__ __forceinline__ void mma1(float16_t &acc, const Tile &w, const A8Regs &a, const void *, int, int) {
+        float f = acc[0];
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            int x0 = 0, x1 = 0;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t x = w.q[p][i] ^ 0x88888888u;
+                x0 = __builtin_amdgcn_sdot4((int)((x << 4) & 0xF0F0F0F0u), (int)a.c[2 * p][i], x0, false);
+                x1 = __builtin_amdgcn_sdot4((int)(x & 0xF0F0F0F0u), (int)a.c[2 * p + 1][i], x1, false);
+            }
+            float s0, s1;
+            scales(w, p, s0, s1);
+            f = __builtin_fmaf((float)halves_sum(x0), s0, f);
+            f = __builtin_fmaf((float)halves_sum(x1), s1, f);
+        }
+        acc[0] = f;
+    }
+    static __device__ __forceinline__ void finish(float16_t &acc, const void *, const uint8_t *A8, int, int lane) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[r] = mul_rounded(acc[r], a8_row_scale(A8, (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3)));
+    }
 };
 
 // The K loop of one wave: two weight tiles and two activation blocks in registers, each refilled with the block two ahead as soon as
@@ -401,7 +503,7 @@ __device__ __forceinline__ void gemm8_wave_loop(float16_t &acc, const uint8_t *_
 
 // Folds the KW waves' partial sums of each tile into the tile's first wave, ascending wave order, through LDS
 // (xch: TPB*(KW-1)*1024 floats). Every wave of the block calls it.
-template <int KW, int TPB>
+template <int KW, int TPB, bool INT_ACC = false>
 __device__ __forceinline__ void gemm8_fold_waves(float16_t &acc, float *xch) {
     if constexpr (KW > 1) {
         const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, t = wave / KW, kw = wave % KW;
@@ -417,7 +519,12 @@ __device__ __forceinline__ void gemm8_fold_waves(float16_t &acc, float *xch) {
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
                     const float4_t v = x4[((t * (KW - 1) + k2 - 1) * 4 + q) * 64 + lane];
-                    acc[4 * q] += v.x, acc[4 * q + 1] += v.y, acc[4 * q + 2] += v.z, acc[4 * q + 3] += v.w;
+                    if constexpr (INT_ACC) { // int32 partial dots in the registers' bits: exact in any order
+#pragma unroll
+                        for (int e = 0; e < 4; e++) acc[4 * q + e] = __int_as_float(__float_as_int(acc[4 * q + e]) + __float_as_int(v[e]));
+                    } else {
+                        acc[4 * q] += v.x, acc[4 * q + 1] += v.y, acc[4 * q + 2] += v.z, acc[4 * q + 3] += v.w;
+                    }
                 }
         }
     }
@@ -437,9 +544,9 @@ __device__ __forceinline__ void gemm8_body(const uint8_t *__restrict__ Wt, const
     float16_t acc;
     gemm8_wave_loop<T, NR>(acc, Wt + ((size_t)(active ? tile : 0) * nKB + s0) * T::TILE_BYTES, A8 + (size_t)s0 * RD_A8_BLOCK_BYTES,
                            active ? nk : 0, aux, tile, lane, lane * 16);
-    gemm8_fold_waves<KW, TPB>(acc, lds);
+    gemm8_fold_waves<KW, TPB, T::INT_ACC>(acc, lds);
     if (!active || kw != 0) return;
-    T::finish(acc, aux, tile, lane);
+    T::finish(acc, aux, A8, tile, lane);
     const int n = tile * 32 + (lane & 31);
     if (resid) {
         float old[16]; // all sixteen reads in flight before the first add
@@ -494,6 +601,13 @@ RD_GEMM8_KERNEL(rd_k_gemm8_w8a8_kw8, W8A8Traits8, 8, 1)
 RD_GEMM8_KERNEL(rd_k_gemm8_w4a8_kw2, W4A8Traits8, 2, 2)
 RD_GEMM8_KERNEL(rd_k_gemm8_w4a8_kw4, W4A8Traits8, 4, 1)
 RD_GEMM8_KERNEL(rd_k_gemm8_w4a8_kw8, W4A8Traits8, 8, 1)
+// one activation scale per row (ActQuantGroup 0); launched with one split: the row scale is applied to the finished sum
+RD_GEMM8_KERNEL(rd_k_gemm8_w8a8r_kw2, W8A8RowTraits8, 2, 2)
+RD_GEMM8_KERNEL(rd_k_gemm8_w8a8r_kw4, W8A8RowTraits8, 4, 1)
+RD_GEMM8_KERNEL(rd_k_gemm8_w8a8r_kw8, W8A8RowTraits8, 8, 1)
+RD_GEMM8_KERNEL(rd_k_gemm8_w4a8r_kw2, W4A8RowTraits8, 2, 2)
+RD_GEMM8_KERNEL(rd_k_gemm8_w4a8r_kw4, W4A8RowTraits8, 4, 1)
+RD_GEMM8_KERNEL(rd_k_gemm8_w4a8r_kw8, W4A8RowTraits8, 8, 1)
 
 // ---------------- fused gate|up projection + SwiGLU + per-32 quantization ----------------
 // goinfer decoder/cpu_gateup_fused.go:83-148 in one launch. W holds [gate rows; up rows] (2*I rows). Grid (I/32), block 2*KW waves:
@@ -600,10 +714,10 @@ __device__ __forceinline__ void gemm8_qkv_body(const uint8_t *__restrict__ Wt, c
         for (int i = 0; i < PPT; i++) cs[i] = e.cs[(size_t)(e.row0 + min((tid >> 4) + 4 * KW * i, M - 1)) * half + d1];
     }
     if (e.bias) b1 = e.bias[head * HD + d1], b2 = e.bias[head * HD + d2];
-    gemm8_fold_waves<KW, 1>(acc, lds);
+    gemm8_fold_waves<KW, 1, T::INT_ACC>(acc, lds);
     float *sums = lds; // [32 rows][33]: the tile's sums, row stride 33 words against bank conflicts; the fold is done with this memory
     if (kw == 0) {
-        T::finish(acc, aux, tile, lane);
+        T::finish(acc, aux, A8, tile, lane);
 #pragma unroll
         for (int r = 0; r < 16; r++) sums[((r >> 2) * 8 + (lane >> 5) * 4 + (r & 3)) * 33 + (lane & 31)] = acc[r];
     }
@@ -658,3 +772,9 @@ RD_GEMM8_QKV_KERNEL(rd_k_gemm8_w8a8_qkv_kw8, W8A8Traits8, 8)
 RD_GEMM8_QKV_KERNEL(rd_k_gemm8_w4a8_qkv_kw2, W4A8Traits8, 2)
 RD_GEMM8_QKV_KERNEL(rd_k_gemm8_w4a8_qkv_kw4, W4A8Traits8, 4)
 RD_GEMM8_QKV_KERNEL(rd_k_gemm8_w4a8_qkv_kw8, W4A8Traits8, 8)
+RD_GEMM8_QKV_KERNEL(rd_k_gemm8_w8a8r_qkv_kw2, W8A8RowTraits8, 2)
+RD_GEMM8_QKV_KERNEL(rd_k_gemm8_w8a8r_qkv_kw4, W8A8RowTraits8, 4)
+RD_GEMM8_QKV_KERNEL(rd_k_gemm8_w8a8r_qkv_kw8, W8A8RowTraits8, 8)
+RD_GEMM8_QKV_KERNEL(rd_k_gemm8_w4a8r_qkv_kw2, W4A8RowTraits8, 2)
+RD_GEMM8_QKV_KERNEL(rd_k_gemm8_w4a8r_qkv_kw4, W4A8RowTraits8, 4)
+RD_GEMM8_QKV_KERNEL(rd_k_gemm8_w4a8r_qkv_kw8, W4A8RowTraits8, 8)

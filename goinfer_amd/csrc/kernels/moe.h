@@ -100,6 +100,9 @@ __device__ __forceinline__ void gv_stage(uint8_t *lds, const uint8_t *__restrict
 
 // One 256-element block of the wave's tile against the R staged rows (R the same on every lane: the rows past it are skipped
 // by a scalar branch, one body of code for any R). kb: the block's index in K.
+// ROW: the rows carry one activation scale each (ActQuantGroup 0): the fold takes the weight's group scale alone, as the reference's
+// expert kernels do (backend/cuda/moe_rows.cu:60-75, moe.cu:116-173), and the caller multiplies the finished sum by the row's scale.
+template <bool ROW>
 __device__ __forceinline__ void gv_block(float (&facc)[GV_ROWS], const Q4K8Tile &w, const uint8_t *lds, int nKB, int kb, int h, int R) {
     const int Kpad = nKB * 256, nGp = nKB * 8;
     const float *ldsS = (const float *)(lds + (size_t)GV_ROWS * Kpad);
@@ -122,7 +125,7 @@ __device__ __forceinline__ void gv_block(float (&facc)[GV_ROWS], const Q4K8Tile 
 #pragma unroll
             for (int i = 0; i < 4; i++) idot = __builtin_amdgcn_sdot4((int)hi[i], (int)a1[i], idot, false);
             // idot = 16 * sum (nib-8) * a, a multiple of 16: the shift is exact
-            facc[j] = __builtin_fmaf((float)(idot >> 4), __fmul_rn(ldsS[j * nGp + g], ws), facc[j]);
+            facc[j] = __builtin_fmaf((float)(idot >> 4), ROW ? ws : __fmul_rn(ldsS[j * nGp + g], ws), facc[j]);
         }
     }
 }
@@ -146,7 +149,7 @@ __device__ __forceinline__ void gv_first(GvTiles &t, rd_rsrc_t wr, int nTiles, T
 #pragma unroll
     for (int i = 0; i < 3; i++) Q4K8Traits::load(t.w[i], wr, gv_offset(i, nTiles, nKB, tileOff), lane);
 }
-template <class TileOff, class Epi>
+template <bool ROW, class TileOff, class Epi>
 __device__ __forceinline__ void gv_stream(GvTiles &t, rd_rsrc_t wr, int nTiles, TileOff tileOff, int nKB, const uint8_t *lds, int lane, int R, Epi epi) {
     const int U = nTiles * nKB, h = lane >> 5;
     auto off = [&](int u) { return gv_offset(u, nTiles, nKB, tileOff); };
@@ -158,7 +161,7 @@ __device__ __forceinline__ void gv_stream(GvTiles &t, rd_rsrc_t wr, int nTiles, 
     for (int u = 0; u < U; u += 3) {
 #pragma unroll
         for (int i = 0; i < 3; i++) {
-            if (u + i < U) gv_block(facc, w[i], lds, nKB, kb, h, R);
+            if (u + i < U) gv_block<ROW>(facc, w[i], lds, nKB, kb, h, R);
             Q4K8Traits::load(w[i], wr, off(u + i + 3), lane); // unconditional: the count of loads in flight stays exact
             if (u + i < U && ++kb == nKB) {
 #pragma unroll
@@ -184,11 +187,10 @@ __device__ __forceinline__ void gv_stream(GvTiles &t, rd_rsrc_t wr, int nTiles, 
 // and the rows past the last one exit: the blocks with work are the first in dispatch order, which spreads them evenly over
 // the XCDs and CUs (blocks are handed out round-robin; idle ones scattered among them skew that). Without the bitmap row y is
 // expert y, and exits when no token chose it. Dynamic LDS: gv_lds_bytes(nKB).
-extern "C" __global__ __launch_bounds__(256) void rd_k_moe_gemv_w4a8(const uint8_t *__restrict__ Wt, size_t wStride, const uint8_t *__restrict__ X,
-                                                                      size_t xStride, float *__restrict__ out, int N, int K, int T, int k,
-                                                                      const signed char *__restrict__ rankOf, int nE,
-                                                                      const unsigned *__restrict__ activeBits) {
-    extern __shared__ __align__(16) uint8_t lds[];
+template <bool ROW>
+__device__ __forceinline__ void moe_gemv_body(const uint8_t *__restrict__ Wt, size_t wStride, const uint8_t *__restrict__ X, size_t xStride,
+                                              float *__restrict__ out, int N, int K, int T, int k, const signed char *__restrict__ rankOf, int nE,
+                                              const unsigned *__restrict__ activeBits, uint8_t *lds) {
     const int nKB = (K + 255) >> 8;
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     // xStride != 0: every expert reads activations of its own, so all blocks of an expert are placed on one XCD (blocks go to the
@@ -221,15 +223,35 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_moe_gemv_w4a8(const uint8
         __syncthreads(); // the previous pass is done with the staged rows
         gv_stage(lds, X, K, nKB, rowOf);
         __syncthreads();
-        gv_stream(
+        float rowS[GV_ROWS]; // ROW: the staged rows' scales (every group slot of a row holds it)
+#pragma unroll
+        for (int j = 0; j < GV_ROWS; j++) rowS[j] = ROW ? ((const float *)(lds + (size_t)GV_ROWS * nKB * 256))[j * nKB * 8] : 1.f;
+        gv_stream<ROW>(
             wt, wr, nTiles, tileOff, nKB, lds, lane, R, [&](int q, const float(&facc)[GV_ROWS]) {
                 if (lane < 32) {
 #pragma unroll
                     for (int j = 0; j < GV_ROWS; j++)
-                        if (j < R) out[((size_t)tokOf[j] * k + rankOf[(size_t)tokOf[j] * nE + e]) * N + (tile0 + q) * 32 + lane] = facc[j];
+                        if (j < R)
+                            out[((size_t)tokOf[j] * k + rankOf[(size_t)tokOf[j] * nE + e]) * N + (tile0 + q) * 32 + lane] =
+                                ROW ? mul_rounded(facc[j], rowS[j]) : facc[j];
                 }
             });
     }
+}
+extern "C" __global__ __launch_bounds__(256) void rd_k_moe_gemv_w4a8(const uint8_t *__restrict__ Wt, size_t wStride, const uint8_t *__restrict__ X,
+                                                                      size_t xStride, float *__restrict__ out, int N, int K, int T, int k,
+                                                                      const signed char *__restrict__ rankOf, int nE,
+                                                                      const unsigned *__restrict__ activeBits) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    moe_gemv_body<false>(Wt, wStride, X, xStride, out, N, K, T, k, rankOf, nE, activeBits, lds);
+}
+// The same over rows that carry one activation scale each (ActQuantGroup 0: BASELINE's "int8 per-token activations").
+extern "C" __global__ __launch_bounds__(256) void rd_k_moe_gemv_w4a8r(const uint8_t *__restrict__ Wt, size_t wStride, const uint8_t *__restrict__ X,
+                                                                       size_t xStride, float *__restrict__ out, int N, int K, int T, int k,
+                                                                       const signed char *__restrict__ rankOf, int nE,
+                                                                       const unsigned *__restrict__ activeBits) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    moe_gemv_body<true>(Wt, wStride, X, xStride, out, N, K, T, k, rankOf, nE, activeBits, lds);
 }
 
 // The experts' gate|up projection with SwiGLU and the per-32 quantization in its epilogue (same values as rd_k_moe_gemv_w4a8
@@ -271,7 +293,7 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_moe_gemv_w4a8_gateup(cons
         gv_stage(lds, X, K, nKB, rowOf);
         __syncthreads();
         float sum[GV_ROWS] = {0.f, 0.f, 0.f, 0.f};
-        gv_stream(wt, wr, nTiles, tileOff, nKB, lds, lane, R, [&](int, const float(&facc)[GV_ROWS]) {
+        gv_stream<false>(wt, wr, nTiles, tileOff, nKB, lds, lane, R, [&](int, const float(&facc)[GV_ROWS]) {
 #pragma unroll
             for (int j = 0; j < GV_ROWS; j++) sum[j] = facc[j];
         });
@@ -306,6 +328,38 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_moe_swiglu_quant(const fl
     }
     const Quant1 q = quant_one(a);
     if (n < I) panel_store(XpE + (size_t)e * xpStride, RD_PANEL_ROW8, t, n, q, I);
+}
+
+// The same with one scale per row of I (ActQuantGroup 0; backend/cuda/moe_rows.cu glu_quant_rows): one block of 256 threads per
+// (token, rank) row, four consecutive columns per thread and round, up to eight rounds (I <= 8192, I % 32 == 0) kept in registers
+// between the row's maximum and its codes. Grid (T*k).
+extern "C" __global__ __launch_bounds__(256) void rd_k_moe_swiglu_quant_row(const float *__restrict__ gu, const int *__restrict__ idx, int I, int k,
+                                                                            uint8_t *__restrict__ XpE, size_t xpStride,
+                                                                            const signed char *__restrict__ rankOf, int nE) {
+    __shared__ float red[16];
+    const int row = blockIdx.x, tok = row / k, e = idx[row], nv = I >> 2;
+    int t = 0; // tokens before this one that chose the same expert
+    for (int i = 0; i < tok; i++) t += rankOf[(size_t)i * nE + e] >= 0;
+    float4_t a[8];
+    float ma = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const int q = threadIdx.x + i * 256;
+        a[i] = (float4_t){0.f, 0.f, 0.f, 0.f};
+        if (q >= nv) continue;
+        const float4_t g = *(const float4_t *)(gu + (size_t)row * 2 * I + 4 * q), u = *(const float4_t *)(gu + (size_t)row * 2 * I + I + 4 * q);
+#pragma unroll
+        for (int c = 0; c < 4; c++) a[i][c] = __fmul_rn(silu_f64(g[c]), u[c]);
+        ma = fmaxf(ma, fmaxf(fmaxf(fabsf(a[i].x), fabsf(a[i].y)), fmaxf(fabsf(a[i].z), fabsf(a[i].w))));
+    }
+    const float s = row_scale_of(block_max(ma, red));
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const int q = threadIdx.x + i * 256;
+        if (q >= nv) continue; // groups of 8 lanes are on or off together
+        const Quant4 qq = quant_four_row(a[i].x, a[i].y, a[i].z, a[i].w, s);
+        panel_store4(XpE + (size_t)e * xpStride, RD_PANEL_ROW8, t, 4 * q, qq, I);
+    }
 }
 
 // out[t][:] = sum over ranks, in rank order, of wgt[t][rank] * down[(t,rank)][:]  (decoder/mlp.go:100-103, addScaled: mul then add).

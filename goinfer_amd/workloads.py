@@ -17,11 +17,13 @@ def llama3_8b_cfg(n_layers=32):
                 eps=1e-5, attn_scale=float(1.0 / np.sqrt(128)), softcap=0.0, theta=5e5)
 
 
-def qwen3_moe_cfg(n_layers=48):
-    """Qwen3-MoE-30B-A3B shape: 48 layers, hidden 2048, 32 Q / 4 KV heads, head_dim 128, 128 experts top-8, expert FFN 768."""
+def qwen3_moe_cfg(n_layers=48, exp_act_group=0):
+    """Qwen3-MoE-30B-A3B shape: 48 layers, hidden 2048, 32 Q / 4 KV heads, head_dim 128, 128 experts top-8, expert FFN 768.
+    The experts are int4-g32 with int8 activations quantized per token row (exp_act_group 0, goinfer's int4 mode); 32 gives the
+    variant whose expert activations are quantized per group of 32."""
     return dict(name="qwen3-moe-30b-a3b-shape", n_layers=n_layers, hidden=2048, n_heads=32, n_kv=4, head_dim=128, inter=0, vocab=151936,
                 eps=1e-6, attn_scale=float(1.0 / np.sqrt(128)), softcap=0.0, theta=1e6, n_experts=128, top_k=8, norm_topk=1,
-                exp_inter=768, qk_norm=1)
+                exp_inter=768, qk_norm=1, exp_act_group=exp_act_group)
 
 
 def inv_freq(head_dim, theta):
@@ -102,6 +104,7 @@ class Resident:
                 if keep is not None:
                     keep["router"] = r
                     keep["experts"] = []
+                m.set_act_group(cfg.get("exp_act_group", 32))
                 for e in range(nE):
                     ex = {}
                     for proj, N, K in (("gate", EI, H), ("up", EI, H), ("down", H, EI)):
@@ -116,6 +119,7 @@ class Resident:
                 progress("layer %d/%d uploaded" % (l + 1, cfg["n_layers"]))
         self.final_norm = synth.normal(nxt(), H, 0.02, 1.0)
         m.upload_f32(-1, "final_norm", self.final_norm)
+        m.set_act_group(cfg.get("act_group", 32))
         self.head = synth.w8a8_normal(nxt(), V, H, SIGMA)
         m.upload_w8a8(-1, "head", *self.head)
         self.embed = synth.w8a8_normal(nxt(), V, H, SIGMA)

@@ -91,15 +91,22 @@ int rd_dequant_q5k(rd_device *d, const void *blocks, int N, int K, float *out);
 int rd_dequant_q6k(rd_device *d, const void *blocks, int N, int K, float *out);
 int rd_gemm_q5k(rd_device *d, const void *W, int N, int K, const float *a, int M, float *dst);
 int rd_gemm_q6k(rd_device *d, const void *W, int N, int K, const float *a, int M, float *dst);
-/* The per-32 activation quantizer every int projection's input goes through (aikit QuantizeActQ group 32, call sites
- * decoder/weightmat.go:845-862, cpu_gateup_fused.go:110-117; device twin backend/cuda/actgroup.cu:32-54 quantG32 — with the CPU
- * path's round-half-away, not the twin's round-to-even): a host f32 [M][K] -> codes int8 [M][K], scales f32 [M][K/32]
- * (maxabs/127, 0 for an all-zero group) and sums f32 [M][K/32] (scale * sum of the group's codes). K a multiple of 32. */
-int rd_quant_act(rd_device *d, const float *a, int M, int K, int8_t *codes, float *scales, float *sums);
-/* int8 per-row weights x per-32 int8 activations (backend/cuda/actgroup.cu:421-437 gemv_w8a8_g32). */
-int rd_gemm_w8a8(rd_device *d, const int8_t *q, const float *row_scale, int N, int K, const float *a, int M, float *dst);
-/* int4 group-32 weights with f16 scales x per-32 int8 activations (backend/cuda/actgroup.cu:243-275). */
-int rd_gemm_w4a8(rd_device *d, const uint8_t *nib, const uint16_t *s16, int N, int K, const float *a, int M, float *dst);
+/* The activation quantizer every int projection's input goes through (aikit QuantizeActQ, call sites decoder/weightmat.go:845-862,
+ * cpu_gateup_fused.go:110-117; device twins backend/cuda/actgroup.cu:32-54 quantG32 and kv8_store.cu:27-35 — with the CPU path's
+ * round-half-away, not the twins' round-to-even): a host f32 [M][K] -> codes int8 [M][K] and
+ *   act_group 32: scales f32 [M][K/32] (maxabs/127, 1 for an all-zero group) and sums f32 [M][K/32] (scale * sum of the group's codes);
+ *   act_group 0 (linalg.QuantizeRowInt8, one scale per row): scales f32 [M]; sums is not written and may be NULL.
+ * K a multiple of 32. */
+int rd_quant_act(rd_device *d, const float *a, int M, int K, int act_group, int8_t *codes, float *scales, float *sums);
+/* act_group below is goinfer's WeightMat.ActQuantGroup(): 32 = activations quantized per group of 32 (the lanes its q4k mode runs
+ * on the CPU, decoder/weightmat.go:961-971), 0 = one scale per row, the only case in which goinfer consults a backend's staged
+ * QuantBackend.MatmulW8A8 / QuantBackend4.MatmulW4A8 hooks (decoder/backend.go:38-75, weightmat.go:909-912,936-938). */
+/* int8 per-row weights x int8 activations. act_group 32: backend/cuda/actgroup.cu:421-437 gemv_w8a8_g32. act_group 0:
+ * dst = (f32(int32 dot over K) * aScale[m]) * wScale[n], linalg.MatmulBTW8A8 bit for bit (internal/gpudev/gemv_quant.cu:99-112). */
+int rd_gemm_w8a8(rd_device *d, const int8_t *q, const float *row_scale, int N, int K, const float *a, int M, int act_group, float *dst);
+/* int4 group-32 weights with f16 scales x int8 activations. act_group 32: backend/cuda/actgroup.cu:243-275. act_group 0: per weight
+ * group facc = fma(f32(idot_g), ws_g, facc), dst = facc * aScale[m] (internal/gpudev/gemv_quant.cu:40-95, backend/cuda/moe_rows.cu:24-106). */
+int rd_gemm_w4a8(rd_device *d, const uint8_t *nib, const uint16_t *s16, int N, int K, const float *a, int M, int act_group, float *dst);
 /* The step's q|k|v epilogue on its own (backend/cuda/gemv_fwd.cu:51-101 rope_kv, prefill_batched.cu rope_kv_ragged; CPU:
  * decoder/attention.go:12-34 addBias, program_cpu.go:351-375 applyQKNorm / applyRope, kvcache.go:21-40,43-52 Append's narrowing):
  * x: host f32 [rows][(n_h+2*n_kv)*hd], the projections of `rows` (<= 32) sequences, row r at position pos[r] of its own cache.
@@ -158,6 +165,11 @@ int rd_model_upload_q6k(rd_model *m, int layer, int proj, const void *blocks, in
 int rd_model_upload_w8a8(rd_model *m, int layer, int proj, const int8_t *q, const float *row_scale, int N, int K);
 /* canonical int4 nibbles + binary16 group-32 scales (WeightMat.Int4F16, decoder/weightmat.go:904); expert < 0 = dense */
 int rd_model_upload_w4a8(rd_model *m, int layer, int proj, int expert, const uint8_t *nib, const uint16_t *s16, int N, int K);
+/* WeightMat.ActQuantGroup() of the int8 / int4 tensors (dense and expert) uploaded from here on: 32 (the default; goinfer's q4k
+ * mode) or 0 (one activation scale per row: its int8 / int4 modes, decoder/weightmat.go:837,909,936; the experts' kernels
+ * backend/cuda/moe_rows.cu:24-106, moe.cu:111-216). Projections that share a quantized input (q|k|v, gate|up) and all experts of a
+ * model must agree, RD_DECLINED otherwise; Q4_K / Q5_K / Q6_K tensors are per-32 by kind. Before rd_model_finalize. */
+int rd_model_set_act_group(rd_model *m, int act_group);
 /* norms, router; RD_VEC_ROUTER_BIAS: a layer's e_score_correction_bias [n_experts]; RD_VEC_ATTN_SINKS: its attention sinks [n_heads];
  * RD_VEC_POST_ATTN_NORM / RD_VEC_POST_FFN_NORM [hidden]: Gemma 2's norm of the attention / feed-forward output before it joins the
  * residual (decoder/program_cpu.go:286-312, the PostAttn and PostMLP slots; backend/cuda/backend.go:86). Before rd_model_finalize. */

@@ -11,9 +11,10 @@ def dense_cfg(n_layers=2, hidden=256, n_heads=4, n_kv=2, head_dim=64, inter=512,
                 eps=eps, attn_scale=float(1.0 / np.sqrt(head_dim)), softcap=softcap, theta=theta, kv_f16=1)
 
 
-def moe_cfg(n_layers=2, hidden=256, n_heads=4, n_kv=2, head_dim=64, n_experts=8, top_k=2, exp_inter=128, vocab=512):
+def moe_cfg(n_layers=2, hidden=256, n_heads=4, n_kv=2, head_dim=64, n_experts=8, top_k=2, exp_inter=128, vocab=512, exp_act_group=32):
+    """exp_act_group: the experts' ActQuantGroup, 32 (activations quantized per group of 32) or 0 (one scale per token row)."""
     c = dense_cfg(n_layers, hidden, n_heads, n_kv, head_dim, 0, vocab, theta=1e6, eps=1e-6)
-    c.update(n_experts=n_experts, top_k=top_k, norm_topk=1, exp_inter=exp_inter, qk_norm=1)
+    c.update(n_experts=n_experts, top_k=top_k, norm_topk=1, exp_inter=exp_inter, qk_norm=1, exp_act_group=exp_act_group)
     return c
 
 
@@ -36,7 +37,9 @@ class Pair:
     """The same synthetic model as an oracle model and (when dev is given) a resident GPU model."""
 
     def __init__(self, cfg, seed, dev=None, slots=8, ctx_cap=512, sigma=0.02, kinds=None, kv="f16"):
-        """kinds: optional {projection: 'q5k' | 'q6k' | 'w8a8'} for dense projections stored as those super-blocks or int8 rows."""
+        """kinds: optional {projection: 'q5k' | 'q6k' | 'w8a8' | 'w4a8'} for dense projections stored as those super-blocks, int8 rows
+        or int4-g32 rows. cfg["act_group"] / cfg["exp_act_group"] (default 32): goinfer's ActQuantGroup of the dense int8 / int4
+        tensors and of the experts, 0 = one activation scale per row."""
         if kv == "i8":  # the int8 KV cache on both sides
             cfg = dict(cfg, kv_f16=2)
         self.cfg = cfg
@@ -58,16 +61,25 @@ class Pair:
 
         def mat(layer, proj, N, K, expert=-1):
             """Q4_K when K is a multiple of 256, else int8 W8A8 (goinfer's q4k-mode policy, weightmat.go:33-38)."""
+            ag, eag = cfg.get("act_group", 32), cfg.get("exp_act_group", 32)
             if expert >= 0:
                 nib, s16 = synth.w4a8_normal(nxt(), N, K, sigma)
                 if self.gpu:
+                    self.gpu.set_act_group(eag)
                     self.gpu.upload_w4a8(layer, proj, expert, nib, s16, K)
-                return ob.WMat(ob.OR_W4A8, N, K, nib, s16, act_group=32)
+                return ob.WMat(ob.OR_W4A8, N, K, nib, s16, act_group=eag)
+            if self.gpu:
+                self.gpu.set_act_group(ag)
+            if kinds.get(proj) == "w4a8":
+                nib, s16 = synth.w4a8_normal(nxt(), N, K, sigma)
+                if self.gpu:
+                    self.gpu.upload_w4a8(layer, proj, -1, nib, s16, K)
+                return ob.WMat(ob.OR_W4A8, N, K, nib, s16, act_group=ag)
             if kinds.get(proj) == "w8a8":
                 q, sc = synth.w8a8_normal(nxt(), N, K, sigma)
                 if self.gpu:
                     self.gpu.upload_w8a8(layer, proj, q, sc)
-                return ob.WMat(ob.OR_W8A8, N, K, q, sc, act_group=32)
+                return ob.WMat(ob.OR_W8A8, N, K, q, sc, act_group=ag)
             if proj in kinds:
                 fmt = kinds[proj]
                 blocks = synth.kquant_normal(fmt, nxt(), N, K, sigma)
@@ -82,7 +94,7 @@ class Pair:
             q, sc = synth.w8a8_normal(nxt(), N, K, sigma)
             if self.gpu:
                 self.gpu.upload_w8a8(layer, proj, q, sc)
-            return ob.WMat(ob.OR_W8A8, N, K, q, sc, act_group=32)
+            return ob.WMat(ob.OR_W8A8, N, K, q, sc, act_group=ag)
 
         def vec(layer, which, n):
             # norm weights around one; stored as the deviation from one where the model scales by (1 + w)

@@ -188,6 +188,76 @@ def test_gemm_w4a8(dev, M, N, K):
         assert np.array_equal(dev.gemm_w4a8(nib, s16, K, a[r:r + 1])[0].view(np.uint32), got[r].view(np.uint32)), r
 
 
+@pytest.mark.parametrize("M,K", [(1, 32), (3, 256), (32, 4096), (40, 896), (7, 14336)])
+def test_activation_quantizer_per_row_bits(dev, M, K):
+    """rd_quant_act(act_group 0) against the oracle's QuantizeRowInt8 per row (fingerprint-pinned): codes and the row's one scale
+    bit for bit, on normal rows, an all-zero row (scale 1, codes 0), a row of exact half-way points (round half away from zero)
+    and a row with a saturating outlier."""
+    a = synth.normal(15 + M, M * K).reshape(M, K)
+    if M > 1:
+        a[1] = 0.0  # an all-zero row
+    g = a[M - 1]
+    c = np.random.default_rng(K).integers(-126, 126, K).astype(np.float32)
+    g[:] = (c + 0.5) * 0.125  # maxabs 127/8: x / scale is exact and (c + 0.5) * scale is a tie between c and c + 1
+    g[0], g[1] = 127 * 0.125, -127 * 0.125
+    if M > 2:
+        a[M // 2, K - 1] = 1e4  # an outlier: the row's other codes collapse to 0
+    codes, scales, _ = dev.quant_act(a, 0)
+    q, S = ob.quantize_act(a, 0)
+    assert np.array_equal(codes, q)
+    assert np.array_equal(scales.view(np.uint32), S[:, 0].view(np.uint32))
+    rne = np.clip(np.rint(g / 0.125), -127, 127)
+    assert (rne != q[M - 1]).sum() >= K // 4  # the tie row does tell half-away from round-to-even
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 64, 128), (7, 256, 896), (32, 1024, 4096), (5, 96, 96), (131, 160, 2048), (4, 4096, 14336)])
+def test_gemm_w8a8_per_row_bit_exact(dev, M, N, K):
+    """int8 weights x per-row int8 activations (ActQuantGroup 0, the lane goinfer's staged QuantBackend.MatmulW8A8 hook serves):
+    an exact int32 dot over the whole of K, then two rounded multiplies. The oracle's twin is digest-pinned to linalg.MatmulBTW8A8
+    on all three reference configurations; the GPU equals it bit for bit, in a batch (matrix cores), alone (vector ALU) and past
+    32 rows (further M-tiles)."""
+    q, s = synth.w8a8_normal(5, N, K)
+    a = synth.normal(6, M * K).reshape(M, K)
+    a[0, : K // 2] *= 30.0
+    want = ob.matmul(ob.WMat(ob.OR_W8A8, N, K, q, s, act_group=0), a)
+    got = dev.gemm_w8a8(q, s, a, act_group=0)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    solo = dev.gemm_w8a8(q, s, a[M - 1:M], act_group=0)
+    assert np.array_equal(solo[0].view(np.uint32), want[M - 1].view(np.uint32))
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 64, 128), (16, 768, 2048), (16, 2048, 768), (3, 64, 160), (40, 128, 4096)])
+def test_gemm_w4a8_per_row(dev, M, N, K):
+    """int4-g32 weights x per-row int8 activations (ActQuantGroup 0: BASELINE's "int8 per-token activations", the staged
+    QuantBackend4.MatmulW4A8 hook and the experts' kernels): within 1e-5 of the f64 sum like every other lane (the reference's
+    own kernel bar), the oracle too; a batched row is the row alone, bit for bit."""
+    nib, s16 = synth.w4a8_normal(8, N, K)
+    a = synth.normal(9, M * K).reshape(M, K)
+    a[0, : K // 2] *= 30.0  # groups of very different magnitude: the per-32 lane would give another answer
+    w = ob.WMat(ob.OR_W4A8, N, K, nib, s16, act_group=0)
+    ref64 = ob.matmul_f64ref(w, a)
+    got = dev.gemm_w4a8(nib, s16, K, a, act_group=0)
+    assert rel_err(ob.matmul(w, a), ref64) < 1e-5
+    assert rel_err(got, ref64) < 1e-5
+    assert rel_err(dev.gemm_w4a8(nib, s16, K, a, act_group=32), ref64) > 1e-4  # not the per-32 lane by another name
+    for r in range(min(M, 3)):
+        assert np.array_equal(dev.gemm_w4a8(nib, s16, K, a[r:r + 1], act_group=0)[0].view(np.uint32), got[r].view(np.uint32)), r
+
+
+def test_gemm_w4a8_per_row_random_nibbles(dev):
+    """Random bytes reach every nibble value (quantized normals stop at +-7) and a wide range of scales."""
+    N, K, M = 64, 1024, 5
+    rng = np.random.default_rng(5)
+    nib = rng.integers(0, 256, N * K // 2, dtype=np.uint8).reshape(N, K // 2)
+    s16 = ((rng.integers(1, 20, N * (K // 32)).astype(np.uint16) << 10) | rng.integers(0, 1024, N * (K // 32)).astype(np.uint16)).reshape(N, K // 32)
+    a = synth.normal(9, M * K).reshape(M, K)
+    w = ob.WMat(ob.OR_W4A8, N, K, nib, s16, act_group=0)
+    got = dev.gemm_w4a8(nib, s16, K, a, act_group=0)
+    assert rel_err(got, ob.matmul_f64ref(w, a)) < 1e-5
+    for r in range(M):
+        assert np.array_equal(dev.gemm_w4a8(nib, s16, K, a[r:r + 1], act_group=0)[0].view(np.uint32), got[r].view(np.uint32)), r
+
+
 def test_rmsnorm_rope_route(dev):
     x = synth.normal(1, 5 * 4096).reshape(5, 4096)
     w = synth.normal(2, 4096, 0.02, 1.0)

@@ -163,9 +163,39 @@ def test_softcap_model(dev):
     check(Pair(dense_cfg(softcap=50.0), seed=4, dev=dev, slots=4), [list(rng.integers(0, 512, n)) for n in (4, 70)], steps=3)
 
 
-def test_moe_ragged_batch(dev):
+@pytest.mark.parametrize("mode", ["int4", "int8"])
+def test_dense_per_row_activation_modes(dev, mode):
+    """goinfer's int4 and int8 modes: every projection int4-g32 (or int8) with ONE int8 activation scale per row (ActQuantGroup 0), the
+    head int8 likewise; the quantizers ahead of them (norm, attention combine, SwiGLU) then work on whole rows. The lanes goinfer's
+    staged MatmulW8A8 / MatmulW4A8 hooks serve (decoder/weightmat.go:909-912,936-938)."""
+    kind = "w4a8" if mode == "int4" else "w8a8"
+    cfg = dict(dense_cfg(n_layers=2, hidden=384, n_heads=6, n_kv=2, head_dim=64, inter=640, vocab=512, theta=1e6, eps=1e-6), act_group=0)
+    rng = np.random.default_rng(21)
+    kinds = {p: kind for p in ("q", "k", "v", "o", "gate", "up", "down")}
+    check(Pair(cfg, seed=23, dev=dev, slots=8, kinds=kinds), [list(rng.integers(0, 512, n)) for n in (3, 17, 70)], steps=5)
+
+
+def test_per_row_and_per_32_models_differ(dev):
+    """The activation group is not ignored: the same int4 weights with per-32 activations answer differently."""
+    cfg = dict(dense_cfg(n_layers=1, hidden=256, n_heads=4, n_kv=2, head_dim=64, inter=256, vocab=512), act_group=0)
+    kinds = {p: "w4a8" for p in ("q", "k", "v", "o", "gate", "up", "down")}
+    a, b = Pair(cfg, seed=24, dev=dev, slots=2, kinds=kinds), Pair(dict(cfg, act_group=32), seed=24, dev=dev, slots=2, kinds=kinds)
+    try:
+        e = a.emb[[7]]
+        ga, _ = a.gpu.step_batch([0], [0], e)
+        gb, _ = b.gpu.step_batch([0], [0], e)
+        oa, ob_ = a.oracle.step(e, [a.oracle.new_cache(8)]), b.oracle.step(e, [b.oracle.new_cache(8)])
+        assert np.abs(oa - ob_).max() > 1e-4 and np.abs(ga - gb).max() > 1e-4
+        assert np.abs(ga - oa).max() < np.abs(ga - ob_).max()
+    finally:
+        a.close()
+        b.close()
+
+
+@pytest.mark.parametrize("exp_act_group", [32, 0])
+def test_moe_ragged_batch(dev, exp_act_group):
     rng = np.random.default_rng(4)
-    _, _, (agree, total, diverged) = check(Pair(moe_cfg(), seed=5, dev=dev, slots=8),
+    _, _, (agree, total, diverged) = check(Pair(moe_cfg(exp_act_group=exp_act_group), seed=5, dev=dev, slots=8),
                                            [list(rng.integers(0, 512, n)) for n in (2, 33, 65)], steps=6)
     # Expert choice is discrete: once the hidden state carries the oracle's own noise floor, a router near-tie can flip,
     # and from then on that row computes a different function (goinfer's own tests replay the reference routing for this

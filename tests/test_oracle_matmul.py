@@ -120,3 +120,52 @@ def test_w8a8_per32_matmul_is_the_sum_of_pinned_pieces(M, N, K):
     rms = np.sqrt((want * want).mean())
     assert np.abs(ob.matmul(mat, a) - want).max() / rms < 1e-5
     assert np.abs(ob.matmul_f64ref(mat, a) - want).max() / rms < 1e-6
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 32, 128), (5, 96, 768), (16, 64, 2048), (3, 40, 96)])
+def test_w4a8_per_row_matmul_is_the_sum_of_pinned_pieces(M, N, K):
+    """The int4 lane with ONE activation scale per row (goinfer's ActQuantGroup 0: the experts' kernels and the staged MatmulW4A8
+    hook, decoder/weightmat.go:909-912, backend/cuda/moe_rows.cu:24-106), from the same pinned pieces: the activations are
+    quantize_act(group 0) = QuantizeRowInt8 per row. A per-group scale used where the row's belongs, or the row scale applied per
+    group, moves the result by per cent, not 1e-5."""
+    w = synth.normal(31 + N, N * K, 0.02).reshape(N, K)
+    nib, s16 = ob.quantize_int4(w)
+    a = synth.normal(7 + M, M * K).reshape(M, K)
+    a[0, : K // 2] *= 40.0  # a row whose groups differ widely in magnitude: per-row and per-32 scales then differ by far
+    mat = ob.WMat(ob.OR_W4A8, N, K, nib, s16, act_group=0)
+    q, S = ob.quantize_act(a, 0)
+    assert S.shape == (M, 1)
+    want = (q.astype(np.float64) * S.astype(np.float64)) @ int4_weights_f64(nib, s16, N, K).T
+    rms = np.sqrt((want * want).mean())
+    assert np.abs(ob.matmul(mat, a) - want).max() / rms < 1e-5
+    assert np.abs(ob.matmul_f64ref(mat, a) - want).max() / rms < 1e-6
+    per32 = ob.matmul(ob.WMat(ob.OR_W4A8, N, K, nib, s16, act_group=32), a)
+    assert np.abs(per32 - want).max() / rms > 1e-3  # the two lanes are different functions of the same inputs
+
+
+def test_w4a8_per_row_random_nibbles_and_scales():
+    N, K, M = 32, 512, 3
+    rng = np.random.default_rng(6)
+    nib = rng.integers(0, 256, N * K // 2, dtype=np.uint8).reshape(N, K // 2)
+    s16 = ((rng.integers(1, 20, N * (K // 32)).astype(np.uint16) << 10) | rng.integers(0, 1024, N * (K // 32)).astype(np.uint16)).reshape(N, K // 32)
+    a = synth.normal(9, M * K).reshape(M, K)
+    mat = ob.WMat(ob.OR_W4A8, N, K, nib, s16, act_group=0)
+    q, S = ob.quantize_act(a, 0)
+    want = (q.astype(np.float64) * S.astype(np.float64)) @ int4_weights_f64(nib, s16, N, K).T
+    rms = np.sqrt((want * want).mean())
+    assert np.abs(ob.matmul(mat, a) - want).max() / rms < 1e-5
+    assert np.abs(ob.matmul_f64ref(mat, a) - want).max() / rms < 1e-6
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 32, 128), (7, 64, 896), (32, 96, 4096)])
+def test_w8a8_per_row_matmul_is_exact_in_integers(M, N, K):
+    """The int8 lane with per-row activations is digest-pinned (linalg.MatmulBTW8A8, test_oracle_fingerprints.py). Independently:
+    its value is f32(f32(f32(idot) * aS) * wS) with an exact integer dot, which numpy restates in int64 and float32."""
+    w = synth.normal(41 + N, N * K, 0.02).reshape(N, K)
+    wq, ws = ob.quantize_rows_int8(w)
+    a = synth.normal(3 + M, M * K).reshape(M, K)
+    q, S = ob.quantize_act(a, 0)
+    idot = q.astype(np.int64) @ wq.astype(np.int64).T
+    want = (idot.astype(np.float32) * S.astype(np.float32)) * ws.astype(np.float32)[None, :]
+    got = ob.matmul(ob.WMat(ob.OR_W8A8, N, K, wq, ws, act_group=0), a)
+    assert np.array_equal(got.view(np.uint32), want.astype(np.float32).view(np.uint32))
