@@ -141,14 +141,14 @@ def run_kquant(args):
                 ms = dev.bench_kernel(kern, [N, K, M, 4 if N > 100000 else 8], warmup, steps)
                 t = float(np.median(ms))
                 nbytes = N * (K // 256) * bb + 4 * M * K + 4 * M * N
-                cases.append({"kernel": "rd_k_" + kern, "N": N, "K": K, "M": M, "us": round(t * 1e3, 2), "GBs": round(nbytes / t / 1e6, 1), "bytes": int(nbytes)})
+                cases.append({"kernel": "rd_k_gemm8_" + kern[5:], "N": N, "K": K, "M": M, "us": round(t * 1e3, 2), "GBs": round(nbytes / t / 1e6, 1), "bytes": int(nbytes)})
                 log("%s %dx%d M=%d: %.1f us, %.0f GB/s" % (kern, N, K, M, t * 1e3, nbytes / t / 1e6))
-    head = next(c for c in cases if c["kernel"] == "rd_k_gemm_q6k" and c["N"] == 128256 and c["M"] == 32)
+    head = next(c for c in cases if c["kernel"] == "rd_k_gemm8_q6k" and c["N"] == 128256 and c["M"] == 32)
     out = base_line("Q6_K dequant-GEMM achieved HBM GB/s (head 128256x4096 at M=32; all cases listed)", head["GBs"], "GB/s", steps, warmup,
                     head["us"] / 1e3, "Q4_K / Q5_K / Q6_K GEMM at 14336x4096, 4096x14336, 128256x4096, M in {1,32}",
-                    "synthetic: random super-blocks with sane f16 scales, 4-8 weight copies used round-robin", {"cases": cases}, dtype="f16")
+                    "synthetic: random super-blocks with sane f16 scales, 4-8 weight copies used round-robin", {"cases": cases}, dtype="i8")
     out["roofline"] = {"bound": "hbm", "achieved": head["GBs"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(head["GBs"] / HBM_PEAK_GBS, 4),
-                       "traffic": None, "kernel": "rd_k_gemm_q6k", "avg_launch_ms": round(head["us"] / 1e3, 5),
+                       "traffic": None, "kernel": "rd_k_gemm8_q6k_kw2", "avg_launch_ms": round(head["us"] / 1e3, 5),
                        "algorithmic_bytes_per_launch": head["bytes"]}
     cpu = None
     if not args.no_cpu:

@@ -271,8 +271,8 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
         for (auto &w : ws)
             if (!rc) rc = kind == 0 ? upload_q4k(d, raw.data(), N, K, &w) : (kind == 3 ? upload_q5k(d, raw.data(), N, K, &w) : upload_q6k(d, raw.data(), N, K, &w));
         DevBuf Xp(d), P(d), X(d);
-        const int pkind = kind == 0 ? PANEL_A8 : (kind == 3 ? PANEL_Q4K : PANEL_LIN);
-        size_t pb = kind == 0 ? a8_bytes(K) : (kind == 4 ? (size_t)(K / 128) * LIN_PANEL_BYTES : (size_t)(K / 256) * Q4K_PANEL_BYTES);
+        const int pkind = PANEL_A8;
+        size_t pb = a8_bytes(K);
         const int tiles = (M + 31) / 32; // rows beyond 32 are further M-tiles, each with its own panels and partial sums
         if (!rc) rc = Xp.alloc(pb * tiles);
         int nKB = K / kblock_of(kind);

@@ -94,10 +94,8 @@ static const KName kNames[] = {
     {"rd_k_retile_q4k8", &Kernels::retile_q4k8},
     {"rd_k_dequant_q5k", &Kernels::dequant_q5k},
     {"rd_k_retile_q5k", &Kernels::retile_q5k},
-    {"rd_k_gemm_q5k", &Kernels::gemm_q5k},
     {"rd_k_dequant_q6k", &Kernels::dequant_q6k},
     {"rd_k_retile_q6k", &Kernels::retile_q6k},
-    {"rd_k_gemm_q6k", &Kernels::gemm_q6k},
     {"rd_k_kv_store", &Kernels::kv_store},
     {"rd_k_kv_read", &Kernels::kv_read},
     {"rd_k_qkv_rope_store", &Kernels::qkv_rope_store},
@@ -127,7 +125,6 @@ static const KName kNames[] = {
     {"rd_k_moe_fold", &Kernels::moe_fold},
     {"rd_k_embed_rows", &Kernels::embed_rows},
     {"rd_k_copy16", &Kernels::copy16},
-    {"rd_k_unpanel_q4k", &Kernels::unpanel_q4k},
     {"rd_k_fill_f16", &Kernels::fill_f16},
     {"rd_k_fill_f32", &Kernels::fill_f32},
 };
@@ -164,9 +161,9 @@ static int open_common(int ordinal, const void *image, rd_device **out) {
         }
         d->k.*(kn.slot) = f;
     }
-    static const char *kindName[5] = {"q4k", "w8a8", "w4a8", "w8a8r", "w4a8r"};
+    static const char *kindName[7] = {"q4k", "w8a8", "w4a8", "w8a8r", "w4a8r", "q5k", "q6k"};
     static const int kwOf[3] = {2, 4, 8};
-    for (int kind = 0; kind < 5; kind++)
+    for (int kind = 0; kind < 7; kind++)
         for (int i = 0; i < 6; i++) {
             char name[64];
             if (i < 3)
@@ -332,24 +329,13 @@ GemmPlan plan_gemm(int kind, int N, int nKB, int act_group) {
         p.splits = (nKB + p.kbPerSplit - 1) / p.kbPerSplit;
         return p;
     }
-    int groups = (N + 127) / 128;
-    int target = 256;
-    if (const char *e = getenv("ROCMDECODE_GEMM_BLOCKS")) target = atoi(e) > 0 ? atoi(e) : target;
-    int want = target / groups; // rounded down: a few idle CUs cost less than another round of partial sums
-    int maxSplits = nKB >= 2 ? nKB / 2 : 1;
-    int splits = want < 1 ? 1 : (want > maxSplits ? maxSplits : want);
-    if (const char *e = getenv("ROCMDECODE_SPLITS")) splits = atoi(e) > 0 ? atoi(e) : splits;
-    if (splits > nKB) splits = nKB;
-    p.kbPerSplit = (nKB + splits - 1) / splits;
-    p.splits = (nKB + p.kbPerSplit - 1) / p.kbPerSplit;
+    rd_set_error("plan_gemm: unknown weight kind %d", kind);
+    p.splits = 1, p.kbPerSplit = nKB, p.kw = 2;
     return p;
 }
 
-size_t panel_bytes_for(const DevWeight &w) {
-    if (is_gemm8_kind(w.kind)) return a8_bytes(w.K);
-    return w.kind == 3 ? (size_t)(w.K / 256) * Q4K_PANEL_BYTES : (size_t)(w.K / 128) * LIN_PANEL_BYTES;
-}
-int panel_kind_for(const DevWeight &w) { return is_gemm8_kind(w.kind) ? PANEL_A8 : (w.kind == 3 ? PANEL_Q4K : PANEL_LIN); }
+size_t panel_bytes_for(const DevWeight &w) { return a8_bytes(w.K); }
+int panel_kind_for(const DevWeight &) { return PANEL_A8; }
 int act_group_for(const DevWeight &w) { return w.kind == WKIND_GROUP ? (w.parts.empty() ? 32 : w.parts[0].act_group) : w.act_group; }
 int launch_quant_act(rd_device *d, const float *x, int M, int K, int kind, int act_group, void *Xp) {
     if (act_group == 0) return d->launch(d->k.quant_act_row, (unsigned)M, 1, 1, 1024, x, Xp, K, kind);
@@ -374,8 +360,8 @@ int upload_q4k(rd_device *d, const void *blocks, int N, int K, DevWeight *w) {
     return RD_OK;
 }
 
-// Q5_K: 176 B super-blocks re-tiled to 5632 B per (32 rows, super-block). Q6_K: 210 B super-blocks re-tiled to two
-// 3456 B tiles per (32 rows, super-block), one per half; the tiled form is 6.75 bits per weight against 6.5625 raw.
+// Q5_K: 176 B super-blocks re-tiled to 5632 B per (32 rows, super-block), the file's own bits. Q6_K: 210 B super-blocks re-tiled
+// to 7168 B per (32 rows, super-block): the int8 scales and d per lane half, nibbles, high bit pairs; 7 bits per weight against 6.5625 raw.
 int upload_q5k(rd_device *d, const void *blocks, int N, int K, DevWeight *w) {
     if (N <= 0 || K <= 0 || K % 256 || N % 32) {
         rd_set_error("q5k upload: N=%d must be a multiple of 32 and K=%d of 256", N, K);
@@ -404,9 +390,9 @@ int upload_q6k(rd_device *d, const void *blocks, int N, int K, DevWeight *w) {
     DevBuf raw(d);
     int rc = raw.alloc(bytes);
     if (rc) return rc;
-    if ((rc = d->alloc(&w->tiled, (size_t)(N / 32) * nSB * 2 * 3456))) return rc;
+    if ((rc = d->alloc(&w->tiled, (size_t)(N / 32) * nSB * 7168))) return rc;
     if ((rc = d->h2d(raw.p, blocks, bytes))) return rc;
-    if ((rc = d->launch(d->k.retile_q6k, N / 32, 2 * nSB, 1, 256, (const void *)raw.p, w->tiled, N, nSB))) return rc;
+    if ((rc = d->launch(d->k.retile_q6k, N / 32, nSB, 1, 448, (const void *)raw.p, w->tiled, N, nSB))) return rc;
     if ((rc = d->sync())) return rc;
     w->kind = 4, w->N = N, w->K = K;
     return RD_OK;
@@ -468,8 +454,7 @@ void free_weight(rd_device *d, DevWeight *w) {
 
 int launch_gemm(rd_device *d, const DevWeight &w, const void *Xp, float *P, int M, GemmPlan *plan_out, int ldP, int splits, int kw, float *resid,
                 size_t xpStride, size_t pStride) {
-    const bool tiles_in_grid = is_gemm8_kind(w.kind) && M > 32; // the int8 kernels take further M-tiles as grid.z
-    if (M < 1 || (M > 32 && !tiles_in_grid) || M > GEMM_WIDE_ROWS) {
+    if (M < 1 || M > GEMM_WIDE_ROWS) { // rows past 32 are further M-tiles, grid.z of the launch
         rd_set_error("gemm: M=%d outside 1..32", M);
         return RD_ERR_ARG;
     }
@@ -490,12 +475,8 @@ int launch_gemm(rd_device *d, const DevWeight &w, const void *Xp, float *P, int 
         return d->launch(f, (unsigned)((tiles + tpb - 1) / tpb), (unsigned)p.splits, (unsigned)((M + 31) / 32), (unsigned)(64 * p.kw * tpb), (const void *)w.tiled,
                          (const void *)w.scales, Xp, P, w.N, nKB, p.kbPerSplit, M, ldP, resid, xpStride, pStride);
     }
-    if (resid) {
-        rd_set_error("gemm: weight kind %d has no residual epilogue", w.kind);
-        return RD_ERR_STATE;
-    }
-    unsigned gx = (unsigned)((w.N + 127) / 128);
-    return d->launch(w.kind == 3 ? d->k.gemm_q5k : d->k.gemm_q6k, gx, p.splits, 1, GEMM_THREADS, (const void *)w.tiled, Xp, P, w.N, nKB, p.kbPerSplit, M, ldP);
+    rd_set_error("gemm: unknown weight kind %d", w.kind);
+    return RD_ERR_STATE;
 }
 
 int launch_gemm_wide(rd_device *d, const DevWeight &w, const void *Xp, size_t xpStride, float *P, size_t pStride, int M, GemmPlan *plan_out, int ldP,
@@ -504,10 +485,5 @@ int launch_gemm_wide(rd_device *d, const DevWeight &w, const void *Xp, size_t xp
         rd_set_error("wide gemm: M=%d outside 1..%d", M, GEMM_WIDE_ROWS);
         return RD_ERR_ARG;
     }
-    if (is_gemm8_kind(w.kind)) return launch_gemm(d, w, Xp, P, M, plan_out, ldP, splits, kw, nullptr, xpStride, pStride); // all M-tiles in one launch
-    for (int m0 = 0, mt = 0; m0 < M; m0 += 32, mt++) {
-        int rc = launch_gemm(d, w, (const char *)Xp + (size_t)mt * xpStride, P + (size_t)mt * pStride, std::min(32, M - m0), plan_out, ldP, splits, kw);
-        if (rc) return rc;
-    }
-    return RD_OK;
+    return launch_gemm(d, w, Xp, P, M, plan_out, ldP, splits, kw, nullptr, xpStride, pStride); // all M-tiles in one launch
 }

@@ -16,12 +16,10 @@ bool rd_hip_ok(const HipApi *hip, hipError_t e, const char *what);
     } while (0)
 
 // sizes shared with the kernels (goinfer_amd/csrc/kernels/common.h)
-constexpr size_t Q4K_PANEL_BYTES = 17 * 64 * 16;
-constexpr size_t LIN_PANEL_BYTES = 8 * 64 * 16;
 constexpr size_t Q4K_TILE_BYTES = 4608;
 constexpr size_t A8_BLOCK_BYTES = 10240; // one A8 activation block: 256 elements x 32 rows (gemm8.h)
 inline size_t a8_bytes(int K) { return (size_t)((K + 255) / 256) * A8_BLOCK_BYTES; }
-enum { PANEL_Q4K = 0, PANEL_LIN = 1, PANEL_LIN4 = 2, PANEL_A8 = 3, PANEL_ROW8 = 4 };
+enum { PANEL_A8 = 3, PANEL_ROW8 = 4 }; // = RD_PANEL_* of the kernels
 // dynamic LDS of the experts' GEMM kernels: four rows of K elements (codes, scales, sums) + their exchange area
 inline unsigned moe_gemv_lds(int K) { return (unsigned)(4 * ((K + 255) / 256) * 320 + 1024); }
 constexpr int MOE_GEMV_MAX_K = 12288; // 4 rows x 48 blocks x 320 B + 1 KB = 61 KB of LDS
@@ -35,14 +33,14 @@ inline unsigned moe_gemv_grid(int N, int K) {
 struct Kernels {
     hipFunction_t dequant_q4k, quant_act, quant_act_row, reduce_splits, add_rmsnorm_quant, swiglu_quant, swiglu_quant_row;
     hipFunction_t unpack_act8, unpanel_a8, retile_q4k8, retile_w8a8_8, retile_w4a8_8;
-    // [lane: 0 q4k, 1 w8a8, 2 w4a8 (per-32 activations), 3 w8a8, 4 w4a8 with one activation scale per row][waves per tile 2, 4, 8]
-    hipFunction_t gemm8[5][3];
-    hipFunction_t gemm8_qkv[5][3]; // the q|k|v projection with RoPE and the KV store in its epilogue, indexed like gemm8
+    // [lane: 0 q4k, 1 w8a8, 2 w4a8 (per-32 activations), 3 w8a8, 4 w4a8 with one activation scale per row, 5 q5k, 6 q6k][waves per tile 2, 4, 8]
+    hipFunction_t gemm8[7][3];
+    hipFunction_t gemm8_qkv[7][3]; // the q|k|v projection with RoPE and the KV store in its epilogue, indexed like gemm8
     hipFunction_t gemm8_q4k_gateup, gemm8_q4k_gateup_gelu, add_one, moe_gemv_w4a8, moe_gemv_w4a8r, moe_gemv_w4a8_gateup, retile_w4a8_gv, rope_table;
-    hipFunction_t dequant_q5k, retile_q5k, gemm_q5k, dequant_q6k, retile_q6k, gemm_q6k;
+    hipFunction_t dequant_q5k, retile_q5k, dequant_q6k, retile_q6k;
     hipFunction_t kv_store, kv_read, qkv_rope_store, attn_partial, attn_partial_wide, attn_combine, attn_combine_quant;
     hipFunction_t kv_store_i8, qkv_rope_store_i8, attn_partial_i8, attn_partial_rows, attn_partial_rows_i8, attn_partial_deep, attn_partial_deep_i8, topk_rows, topk_hist, topk_pick, topk_finish;
-    hipFunction_t rmsnorm, rope, argmax_rows, argmax_final, matmul_f32, moe_route, moe_swiglu_quant, moe_swiglu_quant_row, moe_fold, embed_rows, copy16, unpanel_q4k, fill_f16, fill_f32;
+    hipFunction_t rmsnorm, rope, argmax_rows, argmax_final, matmul_f32, moe_route, moe_swiglu_quant, moe_swiglu_quant_row, moe_fold, embed_rows, copy16, fill_f16, fill_f32;
 };
 
 struct rd_device {
@@ -86,9 +84,9 @@ struct DevBuf {
     template <typename T> T *as() { return (T *)p; }
 };
 
-// block sizes that match the code object's launch bounds: the f16-MFMA k-quant GEMMs (4 consumer + 1 producer waves), the fused
-// gate|up kernel (two tiles x two waves), the expert kernels (two tiles x two waves)
-constexpr unsigned GEMM_THREADS = 320, GATEUP_THREADS = 256, MOE_THREADS = 256;
+// block sizes that match the code object's launch bounds: the fused gate|up kernel (two tiles x two waves), the expert kernels
+// (two tiles x two waves)
+constexpr unsigned GATEUP_THREADS = 256, MOE_THREADS = 256;
 
 // How many 64-position KV blocks one attention work item covers for a sequence of nb blocks: every (sequence, kv head) is
 // cut into pieces. The cut depends on the sequence's own length only, never on what else is in the
@@ -186,7 +184,7 @@ int upload_w4a8(rd_device *d, const uint8_t *nib, const uint16_t *s16, int N, in
 // The activation quantizer a weight's GEMM expects of its producer: 32 or 0 (see DevWeight::act_group); a group's members agree.
 int act_group_for(const DevWeight &w);
 // index into Kernels::gemm8 / gemm8_qkv
-inline int gemm8_lane(const DevWeight &w) { return w.act_group == 0 && w.kind >= 1 ? w.kind + 2 : w.kind; }
+inline int gemm8_lane(const DevWeight &w) { return w.kind >= 3 ? w.kind + 2 : (w.act_group == 0 && w.kind >= 1 ? w.kind + 2 : w.kind); }
 // x f32 [M][K] on the device -> the panels of `kind`, quantized per 32 (act_group 32) or per row (0). M <= 32.
 int launch_quant_act(rd_device *d, const float *x, int M, int K, int kind, int act_group, void *Xp);
 void free_weight(rd_device *d, DevWeight *w);
@@ -199,7 +197,7 @@ void free_weight(rd_device *d, DevWeight *w);
 // M > 32 (int8-MFMA kinds only): further M-tiles of 32 rows, xpStride bytes / pStride floats apart, ride in the same launch (grid.z).
 int launch_gemm(rd_device *d, const DevWeight &w, const void *Xp, float *P, int M, GemmPlan *plan, int ldP = 0, int splits = 0, int kw = 0,
                 float *resid = nullptr, size_t xpStride = 0, size_t pStride = 0);
-inline bool is_gemm8_kind(int kind) { return kind >= 0 && kind <= 2; }
+inline bool is_gemm8_kind(int kind) { return kind >= 0 && kind <= 4; } // every kind but a group: all run the int8-MFMA kernels
 // Up to 128 rows as M-tiles of 32: M-tile mt reads its panels at Xp + mt*xpStride (bytes) and writes its partial sums at
 // P + mt*pStride (floats), each laid out as launch_gemm's; the int8 kernels take the M-tiles as grid.z of one launch, the others one
 // launch per M-tile. Either way a row is the same row whatever pass it rides in.
@@ -209,5 +207,5 @@ int launch_gemm_wide(rd_device *d, const DevWeight &w, const void *Xp, size_t xp
 size_t panel_bytes_for(const DevWeight &w);
 int panel_kind_for(const DevWeight &w);
 // K-blocks of a weight: 256 elements (an A8 block, a Q5_K super-block), 128 for Q6_K's half super-blocks. The int8-MFMA kinds pad K up to whole blocks with zeros.
-inline int kblock_of(int kind) { return kind == 4 ? 128 : 256; }
+inline int kblock_of(int) { return 256; }
 inline int kblocks_for(const DevWeight &w) { return (w.K + kblock_of(w.kind) - 1) / kblock_of(w.kind); }

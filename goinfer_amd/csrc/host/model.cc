@@ -76,7 +76,7 @@ extern "C" void rd_model_destroy(rd_model *m) {
     }
     free_weight(d, &m->head);
     for (void *p : {(void *)m->embed_q, (void *)m->embed_scale, (void *)m->inv_freq_dev, (void *)m->rope_cs, (void *)m->final_norm, (void *)m->tables, (void *)m->h, (void *)m->normed, (void *)m->P, (void *)m->qbuf,
-                    (void *)m->part, (void *)m->attn_out, (void *)m->cand_v, (void *)m->cand_i, (void *)m->logits, (void *)m->emb_dev, m->XpA, m->XpA2, m->XpB, (void *)m->ids, (void *)m->meta, (void *)m->router_logits, (void *)m->moe_wgt, (void *)m->moe_gu,
+                    (void *)m->part, (void *)m->attn_out, (void *)m->cand_v, (void *)m->cand_i, (void *)m->logits, (void *)m->emb_dev, m->XpA, m->XpB, (void *)m->ids, (void *)m->meta, (void *)m->router_logits, (void *)m->moe_wgt, (void *)m->moe_gu,
                     (void *)m->moe_dn, (void *)m->moe_out, (void *)m->moe_idx, (void *)m->moe_idx_all, (void *)m->moe_rank, (void *)m->topk_ids, (void *)m->topk_vals, (void *)m->topk_z, (void *)m->topk_scratch.ghist, (void *)m->topk_scratch.ccount, (void *)m->topk_scratch.gmax, (void *)m->topk_scratch.cand_i, (void *)m->topk_scratch.cand_v, (void *)m->topk_scratch.invT, (void *)m->topk_scratch.zpart, m->XpE})
         d->release(p);
     if (m->host_stage) (void)d->hip->HostFree(m->host_stage);
@@ -159,7 +159,6 @@ static int fuse_and_upload(rd_device *d, PendingMat *parts, int n, DevWeight *w)
     if (runs.size() == 1) {
         rc = upload_pending(d, runs[0], w);
     } else {
-        std::vector<int> pk;
         DevWeight g;
         g.kind = WKIND_GROUP, g.K = parts[0].K, g.N = 0;
         for (auto &r : runs) {
@@ -167,12 +166,6 @@ static int fuse_and_upload(rd_device *d, PendingMat *parts, int n, DevWeight *w)
             g.col0.push_back(g.N);
             if ((rc = upload_pending(d, r, &g.parts.back()))) break;
             g.N += r.N;
-            int k = panel_kind_for(g.parts.back());
-            if (std::find(pk.begin(), pk.end(), k) == pk.end()) pk.push_back(k);
-        }
-        if (!rc && pk.size() > 2) {
-            rd_set_error("rocm resident declines: fused projections need more than two activation layouts");
-            rc = RD_DECLINED;
         }
         if (rc)
             free_weight(d, &g);
@@ -508,16 +501,13 @@ extern "C" int rd_model_finalize(rd_model *m) {
     if (std::any_of(m->layers.begin(), m->layers.end(), [](const LayerW &l) { return act_group_for(l.o) == 0; })) RC(alloc_f32(d, &m->attn_out, R * qd));
     RC(alloc_f32(d, &m->logits, R * c.vocab));
     size_t kA = (size_t)H, kB = (size_t)std::max(qd, c.n_experts ? qd : c.inter);
-    // room for either panel kind: 8 KB per 128 elements (int8/int4 consumers) or 17 KB per 256 (Q4_K consumers)
-    auto panel_room = [](size_t K) { return std::max({((K + 127) / 128) * (size_t)LIN_PANEL_BYTES, ((K + 255) / 256) * (size_t)Q4K_PANEL_BYTES, a8_bytes((int)K)}); };
+    auto panel_room = [](size_t K) { return a8_bytes((int)K); };
     m->xpAStride = panel_room(kA), m->xpBStride = panel_room(kB);
     RC(d->alloc(&m->XpA, m->xpAStride * tiles));
-    RC(d->alloc(&m->XpA2, m->xpAStride * tiles));
     RC(d->alloc(&m->XpB, m->xpBStride * tiles));
     // An A8 panel's last block is written only up to K: what lies past it (K not a multiple of 256) must hold finite scales and
     // sums for good, since the GEMM multiplies them with the weights' zero padding.
     HIPCHK(MemsetAsync(m->XpA, 0, m->xpAStride * tiles, d->stream));
-    HIPCHK(MemsetAsync(m->XpA2, 0, m->xpAStride * tiles, d->stream));
     HIPCHK(MemsetAsync(m->XpB, 0, m->xpBStride * tiles, d->stream));
     RC(d->alloc((void **)&m->ids, sizeof(int) * R));
     RC(alloc_f32(d, &m->cand_v, R * ((c.vocab + 4095) / 4096)));
@@ -728,29 +718,14 @@ static int build_attn_items(rd_model *m, int B, const int *slot, const int *pos,
     return RD_OK;
 }
 
-// The panel layouts a weight's GEMMs read: one, or two for a group whose members differ.
-static void panel_kinds_of(const DevWeight &w, int *kA, int *kB) {
-    *kB = -1;
-    if (w.kind != WKIND_GROUP) {
-        *kA = panel_kind_for(w);
-        return;
-    }
-    *kA = panel_kind_for(w.parts[0]);
-    for (const auto &p : w.parts)
-        if (panel_kind_for(p) != *kA) *kB = panel_kind_for(p);
-}
-
 // foldW: P holds an MoE layer's down-projection rows and foldW their weights (see the kernel); else split-K partial sums.
 // postW: the norm of the pending contribution itself (Gemma 2's post-attention / post-feed-forward norm), or null.
 static int add_norm_quant(rd_model *m, int B, const float *P, int splits, const float *w, const DevWeight &next, void *Xp, float *norm_out,
                           const float *foldW = nullptr, const float *postW = nullptr) {
     rd_device *d = m->d;
     Scope s(m, KC_ADD_NORM);
-    int kA, kB;
-    panel_kinds_of(next, &kA, &kB);
-    return d->launch(d->k.add_rmsnorm_quant, (unsigned)B, 1, 1, 1024, m->h, P, splits, w, m->desc.rms_eps, m->desc.hidden, Xp, kA, norm_out,
-                     kB >= 0 ? m->XpA2 : (void *)nullptr, kB, m->pStride, m->xpAStride, m->xpAStride, foldW, P ? postW : (const float *)nullptr,
-                     act_group_for(next));
+    return d->launch(d->k.add_rmsnorm_quant, (unsigned)B, 1, 1, 1024, m->h, P, splits, w, m->desc.rms_eps, m->desc.hidden, Xp, (int)PANEL_A8, norm_out,
+                     m->pStride, m->xpAStride, foldW, P ? postW : (const float *)nullptr, act_group_for(next));
 }
 
 // One GEMM, or for a group one GEMM per member into column ranges of the same P[split][32][N], all with the group's split
@@ -758,12 +733,10 @@ static int add_norm_quant(rd_model *m, int B, const float *P, int splits, const 
 static int launch_proj(rd_model *m, const DevWeight &w, const void *Xp, size_t xpStride, int B, GemmPlan *plan) {
     rd_device *d = m->d;
     if (w.kind != WKIND_GROUP) return launch_gemm_wide(d, w, Xp, xpStride, m->P, m->pStride, B, plan);
-    int kA, kB;
-    panel_kinds_of(w, &kA, &kB);
     GemmPlan g = group_plan(w);
     for (size_t i = 0; i < w.parts.size(); i++) {
         const DevWeight &p = w.parts[i];
-        RC(launch_gemm_wide(d, p, panel_kind_for(p) == kA ? Xp : m->XpA2, xpStride, m->P + w.col0[i], m->pStride, B, nullptr, w.N, g.splits));
+        RC(launch_gemm_wide(d, p, Xp, xpStride, m->P + w.col0[i], m->pStride, B, nullptr, w.N, g.splits));
     }
     g.kbPerSplit = 0;
     if (plan) *plan = g;
@@ -968,8 +941,8 @@ static int step_launches(rd_model *m, int B, int want) {
             {
                 Scope s(m, KC_ADD_NORM);
                 RC(d->launch(d->k.add_rmsnorm_quant, (unsigned)B, 1, 1, 1024, m->h, (const float *)m->P, plan.splits, (const float *)l.ffn_norm,
-                             c.rms_eps, H, m->XpA, (int)PANEL_ROW8, m->normed, (void *)nullptr, -1, m->pStride, m->xpAStride, m->xpAStride,
-                             (const float *)nullptr, (const float *)nullptr, m->exp_act_group == 0 ? 0 : 32));
+                             c.rms_eps, H, m->XpA, (int)PANEL_ROW8, m->normed, m->pStride, m->xpAStride, (const float *)nullptr,
+                             (const float *)nullptr, m->exp_act_group == 0 ? 0 : 32));
             }
             RC(moe_ffn(m, B, li, l));
             if (c.top_k <= MOE_FOLD_FUSED_MAX)

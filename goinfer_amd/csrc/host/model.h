@@ -103,7 +103,6 @@ struct rd_model {
     int *rowDraw = nullptr;               // inside meta
     const rd_draw *step_draws = nullptr;  // set by the entry point for the one step it runs; null = plain argmax for every row
     void *XpA = nullptr, *XpB = nullptr;
-    void *XpA2 = nullptr; // the normed row in a second panel layout, for a q|k|v or gate|up group whose members differ in kind
     size_t P_floats = 0;
     float *cand_v = nullptr;
     int *cand_i = nullptr;

@@ -1,10 +1,11 @@
-// act.h — the row-wise glue between GEMMs: split-K reduction, residual add, RMSNorm, SwiGLU, and the per-32 int8
-// activation quantization whose dequantized values are written as f16 MFMA panels for the next GEMM.
+// act.h — the row-wise glue between GEMMs: split-K reduction, residual add, RMSNorm, SwiGLU, and the int8 activation quantization
+// (per group of 32, or per row) written in the layout the next GEMM reads.
 #pragma once
 #include "a8.h"
 #include "common.h"
 
-enum { RD_PANEL_Q4K = 0, RD_PANEL_LIN = 1, RD_PANEL_LIN4 = 2, RD_PANEL_A8 = 3, RD_PANEL_ROW8 = 4 };
+// Activation layouts: A8 blocks for the int8-MFMA GEMMs (a8.h), ROW8 plain rows for the experts' vector-ALU kernels.
+enum { RD_PANEL_A8 = 3, RD_PANEL_ROW8 = 4 };
 
 // One quantized element: its int8 code, the group's scale and scaled code sum, and the dequantized value code * scale that
 // the f16 panel kinds store.
@@ -56,51 +57,22 @@ __device__ __forceinline__ float block_max(float v, float *red) {
 __device__ __forceinline__ void panel_store(uint8_t *__restrict__ Xp, int kind, int m, int k, const Quant1 &q, int ldk = 0) {
     if (kind == RD_PANEL_ROW8) {
         row8_store1(Xp, ldk, m, k, q.code, q.sc, q.gsum);
-    } else if (kind == RD_PANEL_A8) {
+    } else {
         Xp[a8_code_offset(m, k)] = (uint8_t)q.code;
         if ((k & 31) == 0) {
             uint8_t *p = Xp + a8_scale_offset(m, k >> 5);
             *(float *)p = q.sc;
             *(float *)(p + (RD_A8_SUMS - RD_A8_SCALES)) = q.gsum;
         }
-    } else if (kind == RD_PANEL_Q4K) {
-        half_t *base = (half_t *)(Xp + (size_t)(k >> 8) * RD_Q4K_PANEL_BYTES);
-        int t = k & 255, j = t >> 5;
-        base[q4k_panel_index(t, m)] = (half_t)q.xhat;
-        if ((t & 31) == 0) base[q4k_panel_sum_index(j, m)] = (half_t)q.gsum;
-        if ((t & 31) == 1) base[q4k_panel_sum_index(j, m) + 4] = (half_t)0.f;
-    } else {
-        half_t *base = (half_t *)(Xp + (size_t)(k >> 7) * RD_LIN_PANEL_BYTES);
-        base[kind == RD_PANEL_LIN ? lin_panel_index(k & 127, m) : lin4_panel_index(k & 127, m)] = (half_t)q.xhat;
     }
 }
 
-// Four consecutive elements k0..k0+3 (k0 % 4 == 0) of batch row m. In a Q4_K panel they are the four bytes of one code
-// word and land in slots {0,1} and {4,5} (+2 for an odd sub-block) of one lane row: two 4-byte stores.
+// Four consecutive elements k0..k0+3 (k0 % 4 == 0) of batch row m.
 __device__ __forceinline__ void panel_store4(uint8_t *__restrict__ Xp, int kind, int m, int k0, const Quant4 &q, int ldk = 0) {
     if (kind == RD_PANEL_ROW8) {
         row8_store4(Xp, ldk, m, k0, q.codes, q.sc, q.gsum);
-    } else if (kind == RD_PANEL_A8) {
-        a8_store4(Xp, m, k0, q.codes, q.sc, q.gsum);
-    } else if (kind == RD_PANEL_Q4K) {
-        half_t *base = (half_t *)(Xp + (size_t)(k0 >> 8) * RD_Q4K_PANEL_BYTES);
-        int t = k0 & 255, j = t >> 5;
-        half_t *row = base + q4k_panel_index(t, m); // slot of byte 0
-        *(half2_t *)row = (half2_t){(half_t)q.x[0], (half_t)q.x[2]};
-        *(half2_t *)(row + 4) = (half2_t){(half_t)q.x[1], (half_t)q.x[3]};
-        if ((t & 31) == 0) {
-            half_t *sp = base + q4k_panel_sum_index(j, m);
-            sp[0] = (half_t)q.gsum;
-            sp[4] = (half_t)0.f; // slots 4..7 of the sum step stay zero
-        }
-    } else if (kind == RD_PANEL_LIN) {
-        half_t *row = (half_t *)(Xp + (size_t)(k0 >> 7) * RD_LIN_PANEL_BYTES) + lin_panel_index(k0 & 127, m);
-        *(half2_t *)row = (half2_t){(half_t)q.x[0], (half_t)q.x[1]};
-        *(half2_t *)(row + 2) = (half2_t){(half_t)q.x[2], (half_t)q.x[3]};
     } else {
-        half_t *row = (half_t *)(Xp + (size_t)(k0 >> 7) * RD_LIN_PANEL_BYTES) + lin_panel_index((k0 & 127) & ~7, m);
-        int o = k0 & 4 ? 1 : 0; // offsets 0..3 -> slots 0,2,4,6; offsets 4..7 -> slots 1,3,5,7
-        row[o] = (half_t)q.x[0], row[o + 2] = (half_t)q.x[1], row[o + 4] = (half_t)q.x[2], row[o + 6] = (half_t)q.x[3];
+        a8_store4(Xp, m, k0, q.codes, q.sc, q.gsum);
     }
 }
 
@@ -147,8 +119,7 @@ extern "C" __global__ void rd_k_reduce_splits(const float *__restrict__ P, float
 //   h[m] (+)= sum_s P[s][m][:]   (residual add of a split-K GEMM result, when P != nullptr; ascending split order)
 //   normed = (h*inv)*w with inv = f32(1/sqrt(ss/H+eps)), ss summed in f64   (decoder/rmsnorm.go:29-92)
 //   panels <- per-32 quantization of normed                                  (weightmat.go:33-38)
-// Optionally writes normed f32 to norm_out (the MoE router reads the un-quantized row) and the same quantized values in a
-// second panel layout (Xp2, kind2) when the consuming projections differ in kind. H % 128 == 0, H <= 8192.
+// Optionally writes normed f32 to norm_out (the MoE router reads the un-quantized row). H % 128 == 0, H <= 8192.
 // foldW != NULL: the pending contribution is an MoE layer's output instead, folded here from the experts' down-projection rows:
 // P is [(row*k + rank)][H] with k = splits (<= 8), foldW is [row][k], and the row's contribution is the sum over ranks, in rank
 // order from zero, of foldW * P (multiply, then add: decoder/mlp.go:100-103 addScaled).
@@ -157,8 +128,7 @@ extern "C" __global__ void rd_k_reduce_splits(const float *__restrict__ P, float
 extern "C" __global__ __launch_bounds__(1024) void rd_k_add_rmsnorm_quant(float *__restrict__ h, const float *__restrict__ P, int splits,
                                                                           const float *__restrict__ w, float eps, int H,
                                                                           uint8_t *__restrict__ Xp, int kind, float *__restrict__ norm_out,
-                                                                          uint8_t *__restrict__ Xp2, int kind2, size_t pStride, size_t xpStride,
-                                                                          size_t xp2Stride, const float *__restrict__ foldW,
+                                                                          size_t pStride, size_t xpStride, const float *__restrict__ foldW,
                                                                           const float *__restrict__ postW, int actGroup) {
     __shared__ double red[16], redPost[16];
     __shared__ float redMax[16];
@@ -167,7 +137,6 @@ extern "C" __global__ __launch_bounds__(1024) void rd_k_add_rmsnorm_quant(float 
     const int mt = m >> 5, mr = m & 31;
     if (P) P += (size_t)mt * pStride;
     Xp += (size_t)mt * xpStride;
-    if (Xp2) Xp2 += (size_t)mt * xp2Stride;
     float4_t v[2];
     bool on[2];
     double ss = 0;
@@ -286,7 +255,6 @@ extern "C" __global__ __launch_bounds__(1024) void rd_k_add_rmsnorm_quant(float 
         if (norm_out) *(float4_t *)(norm_out + (size_t)m * H + k0) = nn[i];
         const Quant4 q = actGroup == 0 ? quant_four_row(n0, n1, n2, n3, rowS) : quant_four(n0, n1, n2, n3);
         panel_store4(Xp, kind, mr, k0, q, H);
-        if (Xp2) panel_store4(Xp2, kind2, mr, k0, q, H); // a second consumer that reads another panel layout
     }
 }
 
@@ -351,13 +319,4 @@ extern "C" __global__ __launch_bounds__(1024) void rd_k_swiglu_quant_row(const f
         const Quant4 qq = quant_four_row(a[i].x, a[i].y, a[i].z, a[i].w, s);
         panel_store4(Xp, kind, m, 4 * q, qq, I);
     }
-}
-
-// A Q4_K-layout activation panel set back to rows: out[m][k] = the f16 value (code * scale) the GEMM reads for batch row m,
-// element k. Grid (ceil(K/256), M), block 256. The inverse of panel_store, for checking what a fused producer wrote.
-extern "C" __global__ void rd_k_unpanel_q4k(const uint8_t *__restrict__ Xp, float *__restrict__ out, int K) {
-    const int kb = blockIdx.x, m = blockIdx.y, t = threadIdx.x, k = kb * 256 + t;
-    if (k >= K) return;
-    const half_t *base = (const half_t *)(Xp + (size_t)kb * RD_Q4K_PANEL_BYTES);
-    out[(size_t)m * K + k] = (float)base[q4k_panel_index(t, m)];
 }

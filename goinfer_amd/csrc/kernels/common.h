@@ -13,16 +13,6 @@ typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
 
 #define RD_WAVE 64
 
-// One activation "panel": the f16 operand of one K-block for all 32 batch rows, laid out exactly as the MFMA
-// A-operand fragments are read: [step][lane = half*32 + row][8 halves].
-//   Q4_K panels cover 256 k (one super-block): 16 data steps + 1 step holding the 8 group sums (for the -dmin*m term).
-//   Plain panels (int8 / int4-g32 weights) cover 128 k: 8 data steps in natural k order.
-#define RD_Q4K_PANEL_STEPS 17
-#define RD_Q4K_PANEL_BYTES (RD_Q4K_PANEL_STEPS * 64 * 16)
-#define RD_LIN_PANEL_STEPS 8
-#define RD_LIN_PANEL_BYTES (RD_LIN_PANEL_STEPS * 64 * 16)
-#define RD_Q4K_TILE_BYTES 4608 // 32 rows x 144 B, re-tiled: 512 B of headers + 4 x 1024 B of codes
-
 // Cross-lane exchanges on the VALU's data-parallel path (DPP) instead of the LDS crossbar: a few cycles each instead of
 // an LDS round trip. Each returns, for every lane, the value of its partner lane: XOR1/XOR2 inside a quad, then the
 // half-row and row mirrors (lane i <-> 7-i of its 8, lane i <-> 15-i of its 16) — partners in the other half, which is all
@@ -168,23 +158,3 @@ __device__ __forceinline__ float gelu_tanh_f64(float g) {
 }
 // The gated FFN's activation: 0 = silu (SwiGLU), 1 = tanh-approximate GELU (GeGLU).
 __device__ __forceinline__ float gate_act(float g, int act) { return act ? gelu_tanh_f64(g) : silu_f64(g); }
-
-// Where element t (0..255) of a super-block goes inside a Q4_K activation panel, for batch row m.
-// Sub-block j=t/32 belongs to nibble pair p=j/2; lane half h=p/2 owns pairs 2h,2h+1; its 16 code words are the
-// 16 MFMA steps. Word s holds bytes e0..e0+3 (e0=4*(s%8)): the unpack yields
-// [lo e0, lo e0+2, hi e0, hi e0+2, lo e0+1, lo e0+3, hi e0+1, hi e0+3] (lo = sub-block 2p, hi = 2p+1).
-__device__ __forceinline__ int q4k_panel_index(int t, int m) {
-    int j = t >> 5, e = t & 31, p = j >> 1, h = p >> 1, pp = p & 1;
-    int s = pp * 8 + (e >> 2), b = e & 3;
-    int slot = ((b & 1) << 2) + (b >> 1) + ((j & 1) << 1);
-    return ((s * 64 + h * 32 + m) << 3) + slot;
-}
-// Group sum of sub-block j for batch row m: step 16, lane half j/4, slot j%4.
-__device__ __forceinline__ int q4k_panel_sum_index(int j, int m) { return (((16 * 64) + (j >> 2) * 32 + m) << 3) + (j & 3); }
-// Plain panels: element t (0..127) of a 128-wide block, natural order: step t/16, half (t/8)&1, slot t%8.
-__device__ __forceinline__ int lin_panel_index(int t, int m) { return ((((t >> 4) * 64) + ((t >> 3) & 1) * 32 + m) << 3) + (t & 7); }
-// int4-g32 panels: as plain panels, but the 8 slots of a lane hold offsets [0,4,1,5,2,6,3,7] (the nibble unpack order).
-__device__ __forceinline__ int lin4_panel_index(int t, int m) {
-    int o = t & 7;
-    return ((((t >> 4) * 64) + ((t >> 3) & 1) * 32 + m) << 3) + (((o & 3) << 1) | (o >> 2));
-}
