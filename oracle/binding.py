@@ -101,6 +101,14 @@ def set_threads(n):
     lib().or_set_threads(int(n))
 
 
+FAULTS = dict(none=0, rope_pos=1, gqa_head=2, q4k_scale_index=3, no_softcap=4, q4k_no_min=5, causal_range=6, w4a8_scale_index=7)
+
+
+def set_fault(name):
+    """Turns the oracle into a deliberately wrong one (see oracle.h OR_FAULT_*): only for measuring what a parity test can see."""
+    lib().or_set_fault(FAULTS[name])
+
+
 def dequant_q4k(blocks):
     blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
     nb = blocks.size // 144

@@ -14,6 +14,11 @@
 static int g_threads = 1;
 void or_set_threads(int n) { g_threads = n < 1 ? 1 : n; }
 
+/* A deliberately WRONG oracle, for one purpose: to measure how large a mistake each parity test would catch
+ * (tests/test_oracle_mutants.py). 0 = the faithful restatement (the default and the only value any parity check runs with). */
+static int g_fault = 0;
+void or_set_fault(int f) { g_fault = f; }
+
 /* ------------------------------------------------------------------ f16 */
 /* internal/runtime/f16/f16.go:14-43 (Bits): round-half-up on the dropped mantissa bits. */
 uint16_t or_f32_to_f16(float f) {
@@ -597,8 +602,9 @@ static void matmul_q4k(const or_mat *w, const int8_t *aq, const float *aS, int M
                     int32_t idot = 0;
                     for (int l = 0; l < 32; l++) idot += (int32_t)qb[j * 32 + l] * (int32_t)a[j * 32 + l];
                     int g = b * 8 + j;
-                    facc = fmaf((float)idot, (d * (float)sc[j]) * aS[(size_t)m * nG + g], facc);
-                    facc = fmaf(-(dmin * (float)mn[j]), asum[(size_t)m * nG + g], facc);
+                    const int js = g_fault == OR_FAULT_Q4K_SCALE_INDEX ? (j + 1) & 7 : j; /* fault: the neighbouring sub-block's scale */
+                    facc = fmaf((float)idot, (d * (float)sc[js]) * aS[(size_t)m * nG + g], facc);
+                    if (g_fault != OR_FAULT_Q4K_NO_MIN) facc = fmaf(-(dmin * (float)mn[j]), asum[(size_t)m * nG + g], facc);
                 }
                 dst[(size_t)m * N + n] = facc;
             }
@@ -691,7 +697,7 @@ static void matmul_w4a8(const or_mat *w, const int8_t *aq, const float *aS, int 
                     int c = (int)((row[k >> 1] >> (4 * (k & 1))) & 15) - 8;
                     idot += c * (int32_t)a[k];
                 }
-                float ws = or_f16_to_f32(S16[(size_t)n * nG + g]);
+                float ws = or_f16_to_f32(S16[(size_t)n * nG + (g_fault == OR_FAULT_W4A8_SCALE_INDEX ? (g + 1) % nG : g)]);
                 if (ag > 0)
                     facc = fmaf((float)idot, ws * aS[(size_t)m * nG + g], facc);
                 else
@@ -836,12 +842,15 @@ static double softcap_score(double s, double c) { return c == 0 ? s : c * tanh(s
 void or_attend_sinks(const float *q, float *ctx, const float *keys, const float *vals, int n_keys, int start,
                      int nH, int nKV, int hd, double scale, double softcap, const float *sinks) {
     int kvDim = nKV * hd, group = nH / nKV;
+    if (g_fault == OR_FAULT_NO_SOFTCAP) softcap = 0;
 #pragma omp parallel for num_threads(g_threads) schedule(dynamic, 1)
     for (int qh = 0; qh < nH; qh++) {
         int kvh = qh / group;
+        if (g_fault == OR_FAULT_GQA_HEAD) kvh = (kvh + 1) % nKV; /* fault: the query head reads its neighbour's kv head */
         float *scores = (float *)malloc(sizeof(float) * (size_t)n_keys);
         or_qk_acc64(q + (size_t)qh * hd, keys, scores, 1, hd, n_keys, kvh * hd, kvDim);
         int lo = start < 0 ? 0 : start, hi = n_keys - 1;
+        if (g_fault == OR_FAULT_CAUSAL_RANGE && hi > lo) hi--; /* fault: the row does not see its own key */
         if (lo <= hi) {
             double maxS = -INFINITY;
             for (int s = lo; s <= hi; s++) {
@@ -1020,8 +1029,9 @@ int or_decode_multi_step_traced(const or_model *m, int B, const float *emb, or_c
                 qk_norm(qb, nH, hd, lw->q_norm, m->eps);
                 qk_norm(kb, nKV, hd, lw->k_norm, m->eps);
             }
-            or_rope(qb, nH, hd, c->pos, m->inv_freq, hd / 2, 1.0);
-            or_rope(kb, nKV, hd, c->pos, m->inv_freq, hd / 2, 1.0);
+            const int rpos = c->pos + (g_fault == OR_FAULT_ROPE_POS ? 1 : 0); /* fault: rotated for the next position */
+            or_rope(qb, nH, hd, rpos, m->inv_freq, hd / 2, 1.0);
+            or_rope(kb, nKV, hd, rpos, m->inv_freq, hd / 2, 1.0);
             float *kr = c->k[l] + (size_t)c->pos * kvDim, *vr = c->v[l] + (size_t)c->pos * kvDim;
             kv_narrow_row(m, kb, kr); /* as the cache stores it: f32, binary16 or int8 per head */
             kv_narrow_row(m, vb, vr);

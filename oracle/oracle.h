@@ -138,6 +138,10 @@ void or_matmul(const or_mat *w, const float *a, int M, float *dst);
 /* the same product with f64 accumulation over dequantized weights and dequantized activations */
 void or_matmul_f64ref(const or_mat *w, const float *a, int M, double *dst);
 void or_set_threads(int n);
+/* Mutations of the oracle, used only to measure what size of mistake a parity test catches (never by a parity check itself). */
+enum { OR_FAULT_NONE = 0, OR_FAULT_ROPE_POS = 1, OR_FAULT_GQA_HEAD = 2, OR_FAULT_Q4K_SCALE_INDEX = 3, OR_FAULT_NO_SOFTCAP = 4, OR_FAULT_Q4K_NO_MIN = 5,
+       OR_FAULT_CAUSAL_RANGE = 6, OR_FAULT_W4A8_SCALE_INDEX = 7 };
+void or_set_fault(int fault);
 
 /* ---- one sequence's decode attention over its own cache:
  * decoder/program_cpu_n.go:497-515 + forwardn.go:295-500 (useAcc64, K=1) + kvcache.go:21-40 (f16 narrowing) ---- */

@@ -194,6 +194,16 @@ def test_c4_llama3_8b_shape_step(dev):
     resident_steps(pair, lens, steps=3, seed=41)
 
 
+def test_c4_full_depth_full_contexts_greedy_steps(dev):
+    """All 32 layers at the configuration's own contexts, U[512,4096], for several greedy steps: 4 of the 32 sequences (the
+    oracle keeps f32 caches: 1 GB per sequence at this depth), drawn with the benchmark's seed. Teacher-forced on the oracle's
+    tokens; the row of slot 0 also equals its solo run bit for bit at every step."""
+    cfg = dict(workloads.llama3_8b_cfg(32), kv_f16=1)
+    lens = np.random.default_rng(1234).integers(512, 4097, 32)[[0, 9, 18, 27]]
+    pair = Pair(cfg, seed=33, dev=dev, slots=5, ctx_cap=int(lens.max()) + 8)
+    resident_steps(pair, lens, steps=4, seed=43)
+
+
 def test_c5_qwen3_moe_shape_step(dev):
     cfg = dict(workloads.qwen3_moe_cfg(2), kv_f16=1)
     lens = np.random.default_rng(4321).integers(256, 2049, 16)

@@ -159,8 +159,11 @@ def test_qwen2_projection_biases(dev):
 
 
 def test_softcap_model(dev):
+    """A cap small enough to bend this random-init model's scores (they are ~0.1): with Gemma's 50 a kernel that dropped the softcap
+    would pass (tests/test_oracle_mutants.py measures both)."""
+    from tests.test_oracle_mutants import SOFTCAP_THAT_BITES
     rng = np.random.default_rng(3)
-    check(Pair(dense_cfg(softcap=50.0), seed=4, dev=dev, slots=4), [list(rng.integers(0, 512, n)) for n in (4, 70)], steps=3)
+    check(Pair(dense_cfg(softcap=SOFTCAP_THAT_BITES), seed=4, dev=dev, slots=4), [list(rng.integers(0, 512, n)) for n in (4, 70)], steps=3)
 
 
 @pytest.mark.parametrize("mode", ["int4", "int8"])
@@ -192,18 +195,73 @@ def test_per_row_and_per_32_models_differ(dev):
         b.close()
 
 
+def run_moe_replayed(pair, prompts, steps):
+    """A MoE model against the oracle with the oracle's routing replayed at every position (goinfer's own way to compare MoE
+    forwards, decoder/mlp.go moeSelOverride: a flipped expert is a different function): prompts token by token, then batched
+    greedy steps, teacher-forced. No row is excused: every prompt's last logits and every row of every step is held to the bar,
+    and every batched row equals its solo twin bit for bit. The GPU's own routing runs first at each position and is only counted
+    (how often it is the oracle's); the replayed step then rewrites the same K/V rows. Returns (worst deviation, floor, agree, total)."""
+    B = len(prompts)
+    caches = [pair.oracle.new_cache(pair.ctx_cap) for _ in range(B)]
+    caches2 = [pair.oracle.new_cache(pair.ctx_cap) for _ in range(B)]  # the same run under a 1e-6 input change, same routing: the floor
+    floor, agree, total, pend = 0.0, 0, 0, []
+    last = []
+    for b, toks in enumerate(prompts):
+        for p, t in enumerate(toks):
+            e = pair.emb[[t]]
+            o, tr, wt = pair.oracle.step(e, [caches[b]], want_weights=True)
+            o2 = pair.oracle.step(perturbed(e, 1e-6, (b, p)), [caches2[b]], replay=(tr, wt))
+            floor = max(floor, float(np.abs(o - o2).max()))
+            pair.gpu.step_batch([b], [p], e, capi.WANT_ARGMAX)  # free-running: counted, then overwritten
+            agree += int((pair.gpu.last_moe_indices(1) == tr).sum())
+            total += tr.size
+            pair.gpu.moe_replay(tr, wt)
+            g, _ = pair.gpu.step_batch([b], [p], e)
+            pair.gpu.moe_replay(tr, wt)
+            pair.gpu.step_batch([B + b], [p], e)  # the twin slot, stepped alone below
+        pend.append((("prefill", b), g[0].copy(), o[0].copy()))
+        last.append(o[0].copy())
+    nxt = [ob.argmax(x) for x in last]
+    pos = [len(t) for t in prompts]
+    for s in range(steps):
+        emb = pair.emb[nxt]
+        o, tr, wt = pair.oracle.step(emb, caches, want_weights=True)
+        o2 = pair.oracle.step(perturbed(emb, 1e-6, (99, s)), caches2, replay=(tr, wt))
+        floor = max(floor, float(np.abs(o - o2).max()))
+        pair.gpu.step_batch(list(range(B)), pos, emb, capi.WANT_ARGMAX)
+        agree += int((pair.gpu.last_moe_indices(B) == tr).sum())
+        total += tr.size
+        pair.gpu.moe_replay(tr, wt)
+        g, ids = pair.gpu.step_batch(list(range(B)), pos, emb, capi.WANT_LOGITS | capi.WANT_ARGMAX)
+        for b in range(B):
+            pend.append((("step", s, b), g[b].copy(), o[b].copy()))
+            assert near_tie_ok(o[b], int(ids[b])), ("greedy token", s, b)
+            pair.gpu.moe_replay(tr[b:b + 1], wt[b:b + 1])
+            solo = pair.gpu.forward(B + b, pos[b], emb[b])
+            assert np.array_equal(solo.view(np.uint32), g[b].view(np.uint32)), ("batched row != solo row", s, b)
+        nxt = [ob.argmax(o[b]) for b in range(B)]
+        pos = [p + 1 for p in pos]
+    worst = 0.0
+    for what, g, o in pend:  # the floor is the whole run's: applied to every row once it is known
+        ok, d = logits_close(g, o, floor)
+        assert ok, (what, d, floor)
+        worst = max(worst, d)
+    for c in caches + caches2:
+        pair.oracle.free_cache(c)
+    pair.close()
+    return worst, floor, agree, total
+
+
 @pytest.mark.parametrize("exp_act_group", [32, 0])
 def test_moe_ragged_batch(dev, exp_act_group):
+    """exp_act_group 32: expert activations quantized per group of 32; 0: one int8 scale per token row (BASELINE's expert lane)."""
     rng = np.random.default_rng(4)
-    _, _, (agree, total, diverged) = check(Pair(moe_cfg(exp_act_group=exp_act_group), seed=5, dev=dev, slots=8),
-                                           [list(rng.integers(0, 512, n)) for n in (2, 33, 65)], steps=6)
-    # Expert choice is discrete: once the hidden state carries the oracle's own noise floor, a router near-tie can flip,
-    # and from then on that row computes a different function (goinfer's own tests replay the reference routing for this
-    # reason, decoder/mlp.go moeSelOverride). Rows are checked against the logit bar until their routing leaves the
-    # oracle's; bit-exact routing on identical logits is asserted at kernel level (test_gpu_kernels.py).
-    print("expert index agreement %d/%d, rows diverged %s" % (agree, total, diverged))
+    worst, floor, agree, total = run_moe_replayed(Pair(moe_cfg(exp_act_group=exp_act_group), seed=5, dev=dev, slots=8),
+                                                  [list(rng.integers(0, 512, n)) for n in (2, 33, 65)], steps=6)
+    # Expert choice is discrete: on the GPU's own routing a near-tie between two experts can flip under the oracle's noise floor;
+    # bit-exact routing on identical logits is asserted at kernel level (test_gpu_kernels.py). Here it is only counted.
+    print("worst logit deviation %.4f, oracle noise floor %.4f, free-running expert index agreement %d/%d" % (worst, floor, agree, total))
     assert agree >= 0.9 * total, (agree, total)
-    assert not all(diverged)
 
 
 def test_moe_fused_expert_gateup_equals_two_launches(dev):
