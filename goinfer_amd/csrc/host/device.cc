@@ -77,6 +77,8 @@ static const KName kNames[] = {
     {"rd_k_quant_act_row", &Kernels::quant_act_row},
     {"rd_k_swiglu_quant_row", &Kernels::swiglu_quant_row},
     {"rd_k_moe_gemv_w4a8r", &Kernels::moe_gemv_w4a8r},
+    {"rd_k_moe_gemv_w4a8r_f32in", &Kernels::moe_gemv_w4a8r_f32in},
+    {"rd_k_moe_gemv_w4a8r_gateup", &Kernels::moe_gemv_w4a8r_gateup},
     {"rd_k_moe_swiglu_quant_row", &Kernels::moe_swiglu_quant_row},
     {"rd_k_reduce_splits", &Kernels::reduce_splits},
     {"rd_k_add_rmsnorm_quant", &Kernels::add_rmsnorm_quant},

@@ -36,7 +36,7 @@ struct Kernels {
     // [lane: 0 q4k, 1 w8a8, 2 w4a8 (per-32 activations), 3 w8a8, 4 w4a8 with one activation scale per row, 5 q5k, 6 q6k][waves per tile 2, 4, 8]
     hipFunction_t gemm8[7][3];
     hipFunction_t gemm8_qkv[7][3]; // the q|k|v projection with RoPE and the KV store in its epilogue, indexed like gemm8
-    hipFunction_t gemm8_q4k_gateup, gemm8_q4k_gateup_gelu, add_one, moe_gemv_w4a8, moe_gemv_w4a8r, moe_gemv_w4a8_gateup, retile_w4a8_gv, rope_table;
+    hipFunction_t gemm8_q4k_gateup, gemm8_q4k_gateup_gelu, add_one, moe_gemv_w4a8, moe_gemv_w4a8r, moe_gemv_w4a8r_f32in, moe_gemv_w4a8_gateup, moe_gemv_w4a8r_gateup, retile_w4a8_gv, rope_table;
     hipFunction_t dequant_q5k, retile_q5k, dequant_q6k, retile_q6k;
     hipFunction_t kv_store, kv_read, qkv_rope_store, attn_partial, attn_partial_wide, attn_combine, attn_combine_quant;
     hipFunction_t kv_store_i8, qkv_rope_store_i8, attn_partial_i8, attn_partial_rows, attn_partial_rows_i8, attn_partial_deep, attn_partial_deep_i8, topk_rows, topk_hist, topk_pick, topk_finish;

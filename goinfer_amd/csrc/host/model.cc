@@ -77,7 +77,7 @@ extern "C" void rd_model_destroy(rd_model *m) {
     free_weight(d, &m->head);
     for (void *p : {(void *)m->embed_q, (void *)m->embed_scale, (void *)m->inv_freq_dev, (void *)m->rope_cs, (void *)m->final_norm, (void *)m->tables, (void *)m->h, (void *)m->normed, (void *)m->P, (void *)m->qbuf,
                     (void *)m->part, (void *)m->attn_out, (void *)m->cand_v, (void *)m->cand_i, (void *)m->logits, (void *)m->emb_dev, m->XpA, m->XpB, (void *)m->ids, (void *)m->meta, (void *)m->router_logits, (void *)m->moe_wgt, (void *)m->moe_gu,
-                    (void *)m->moe_dn, (void *)m->moe_out, (void *)m->moe_idx, (void *)m->moe_idx_all, (void *)m->moe_rank, (void *)m->topk_ids, (void *)m->topk_vals, (void *)m->topk_z, (void *)m->topk_scratch.ghist, (void *)m->topk_scratch.ccount, (void *)m->topk_scratch.gmax, (void *)m->topk_scratch.cand_i, (void *)m->topk_scratch.cand_v, (void *)m->topk_scratch.invT, (void *)m->topk_scratch.zpart, m->XpE})
+                    (void *)m->moe_dn, (void *)m->moe_out, (void *)m->moe_idx, (void *)m->moe_idx_all, (void *)m->moe_rank, (void *)m->topk_ids, (void *)m->topk_vals, (void *)m->topk_z, (void *)m->topk_scratch.ghist, (void *)m->topk_scratch.ccount, (void *)m->topk_scratch.gmax, (void *)m->topk_scratch.cand_i, (void *)m->topk_scratch.cand_v, (void *)m->topk_scratch.invT, (void *)m->topk_scratch.zpart, m->XpE, (void *)m->XEf, (void *)m->moe_rowmax})
         d->release(p);
     if (m->host_stage) (void)d->hip->HostFree(m->host_stage);
     if (m->chain.host_ids) (void)d->hip->HostFree(m->chain.host_ids);
@@ -524,6 +524,11 @@ extern "C" int rd_model_finalize(rd_model *m) {
         RC(d->alloc((void **)&m->moe_rank, (size_t)32 * c.n_experts));
         RC(d->alloc(&m->XpE, (size_t)c.n_experts * a8_bytes(I)));
         HIPCHK(MemsetAsync(m->XpE, 0, (size_t)c.n_experts * a8_bytes(I), d->stream));
+        if (m->exp_act_group == 0) {
+            RC(alloc_f32(d, &m->XEf, (size_t)c.n_experts * 32 * I));
+            RC(d->alloc((void **)&m->moe_rowmax, sizeof(unsigned) * (size_t)c.n_experts * 32));
+            HIPCHK(MemsetAsync(m->moe_rowmax, 0, sizeof(unsigned) * (size_t)c.n_experts * 32, d->stream));
+        }
     }
     RC(d->alloc((void **)&m->topk_ids, sizeof(int) * R * TOPK_MAX));
     RC(alloc_f32(d, &m->topk_vals, R * TOPK_MAX));
@@ -776,10 +781,11 @@ static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
                 bits[e >> 5] |= 1u << (e & 31);
             }
             RC(d->h2d(bits_dev, bits, sizeof(bits)));
+            if (m->moe_rowmax) HIPCHK(MemsetAsync(m->moe_rowmax, 0, sizeof(unsigned) * (size_t)nE * 32, d->stream)); // a replayed step is never captured in a graph
         } else {
             // two launches: the logits over many blocks (one per token would leave the chip idle: measured twice as slow), then the routing
             RC(d->launch(d->k.matmul_f32, (unsigned)((nE + 3) / 4), (unsigned)B, 1, 256, (const float *)m->normed, (const float *)l.router,
-                         m->router_logits, B, H, nE, bits_dev));
+                         m->router_logits, B, H, nE, bits_dev, m->moe_rowmax, m->moe_rowmax ? nE * 32 : 0));
             RC(d->launch(d->k.moe_route, (unsigned)B, 1, 1, 64, (const float *)m->router_logits, B, nE, k, c.norm_topk_prob, m->moe_idx, m->moe_wgt,
                          m->moe_rank, trace, bits_dev, (const float *)l.router_bias, m->router_sigmoid, m->router_scale, m->n_group, m->topk_group));
         }
@@ -787,9 +793,22 @@ static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
     const int nKBh = (H + 255) / 256, nKBi = (I + 255) / 256;
     size_t guStride = (size_t)(2 * I / 32) * nKBh * 4608, dnStride = (size_t)(H / 32) * nKBi * 4608;
     size_t xpStride = a8_bytes(I);
-    const bool rowAct = m->exp_act_group == 0; // one activation scale per row: SwiGLU's quantizer needs a whole row, so it is its own launch
+    const bool rowAct = m->exp_act_group == 0; // one activation scale per row
+    const bool fused = I % 32 == 0 && !getenv("ROCMDECODE_NO_FUSED_MOE_GATEUP");
     hipFunction_t gemv = rowAct ? d->k.moe_gemv_w4a8r : d->k.moe_gemv_w4a8;
-    if (I % 32 == 0 && !rowAct && !getenv("ROCMDECODE_NO_FUSED_MOE_GATEUP")) {
+    if (fused && rowAct) {
+        // gate|up + SwiGLU leave f32 rows and their maxima; the per-row quantizer, which needs a whole row, runs where the down projection
+        // stages its rows: two launches, as on the per-32 lane
+        {
+            Scope s(m, KC_MOE_GEMM);
+            RC(d->launch_lds(d->k.moe_gemv_w4a8r_gateup, (unsigned)((I / 32 + 1) / 2), (unsigned)nE, 1, MOE_THREADS, moe_gemv_lds(H), (const void *)l.exp_gateup, guStride,
+                             (const void *)m->XpA, m->XEf, m->moe_rowmax, I, H, B, (const signed char *)m->moe_rank, nE, (const unsigned *)bits_dev));
+        }
+        Scope s(m, KC_MOE_GEMM_DOWN);
+        RC(d->launch_lds(d->k.moe_gemv_w4a8r_f32in, moe_gemv_grid(H, I), (unsigned)nE, 1, MOE_THREADS, moe_gemv_lds(I), (const void *)l.exp_down, dnStride,
+                         (const float *)m->XEf, (const unsigned *)m->moe_rowmax, m->moe_dn, H, I, B, k, (const signed char *)m->moe_rank, nE,
+                         (const unsigned *)bits_dev));
+    } else if (fused) {
         Scope s(m, KC_MOE_GEMM); // gate|up of every touched expert + SwiGLU + quantization into the experts' down activations
         RC(d->launch_lds(d->k.moe_gemv_w4a8_gateup, (unsigned)((I / 32 + 1) / 2), (unsigned)nE, 1, MOE_THREADS, moe_gemv_lds(H), (const void *)l.exp_gateup, guStride,
                          (const void *)m->XpA, m->XpE, xpStride, I, H, B, (const signed char *)m->moe_rank, nE, (const unsigned *)bits_dev));
@@ -808,7 +827,7 @@ static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
             RC(d->launch(d->k.moe_swiglu_quant, (unsigned)((I + 255) / 256), (unsigned)(B * k), 1, 256, (const float *)m->moe_gu, (const int *)m->moe_idx,
                          I, k, m->XpE, xpStride, (const signed char *)m->moe_rank, nE));
     }
-    {
+    if (!(fused && rowAct)) {
         Scope s(m, KC_MOE_GEMM_DOWN);
         RC(d->launch_lds(gemv, moe_gemv_grid(H, I), (unsigned)nE, 1, MOE_THREADS, moe_gemv_lds(I), (const void *)l.exp_down, dnStride,
                          (const void *)m->XpE, xpStride, m->moe_dn, H, I, B, k, (const signed char *)m->moe_rank, nE, (const unsigned *)bits_dev));

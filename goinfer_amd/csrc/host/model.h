@@ -122,6 +122,8 @@ struct rd_model {
     TopkScratch topk_scratch;
     unsigned *moe_bits = nullptr;                    // inside meta: bitmap of the experts the current layer's routing chose (8 words)
     void *XpE = nullptr;                             // per-expert down panels
+    float *XEf = nullptr;                            // per-row expert activations: [nE][32][expert_inter] f32 rows ahead of the per-row quantizer
+    unsigned *moe_rowmax = nullptr;                  // [nE][32]: the bits of each such row's max |x| (cleared by the router's launch)
     // pinned host staging
     // STAGE_SLOTS slots used round-robin, so a caller that chains steps without reading anything back (the device greedy
     // chain) can enqueue several steps ahead of the GPU; a slot is rewritten only after its own upload has completed

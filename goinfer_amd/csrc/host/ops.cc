@@ -289,7 +289,7 @@ extern "C" int rd_matmul_bt(rd_device *d, const float *a, const float *b, float 
     RC(D.alloc(sizeof(float) * (size_t)M * N));
     RC(d->h2d(A.p, a, sizeof(float) * (size_t)M * K));
     RC(d->h2d(B.p, b, sizeof(float) * (size_t)N * K));
-    RC(d->launch(d->k.matmul_f32, (unsigned)((N + 3) / 4), (unsigned)M, 1, 256, (const float *)A.p, (const float *)B.p, D.as<float>(), M, K, N, (unsigned *)nullptr));
+    RC(d->launch(d->k.matmul_f32, (unsigned)((N + 3) / 4), (unsigned)M, 1, 256, (const float *)A.p, (const float *)B.p, D.as<float>(), M, K, N, (unsigned *)nullptr, (unsigned *)nullptr, 0));
     return d->d2h(dst, D.p, sizeof(float) * (size_t)M * N);
 }
 

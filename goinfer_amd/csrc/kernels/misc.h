@@ -145,10 +145,14 @@ extern "C" __global__ __launch_bounds__(64) void rd_k_argmax_final(const float *
 // 64 lane sums. Products of two f32 are exact in f64 and the sum carries ~29 spare bits, so the f32 result matches an
 // ascending-k f64 sum except when that sum falls within ~1e-15 (relative) of an f32 rounding boundary.
 // Grid (ceil(N/4), M), block 256. clear8 (may be NULL): eight words this launch sets to zero on the side — the router's launch
-// clears the active-expert bitmap that the routing kernel, next in the stream, fills.
+// clears the active-expert bitmap that the routing kernel, next in the stream, fills; clearN (may be NULL): nClear more words
+// (the experts' row maxima, which the gate|up kernel of the same layer accumulates with atomics).
 extern "C" __global__ __launch_bounds__(256) void rd_k_matmul_f32(const float *__restrict__ a, const float *__restrict__ b, float *__restrict__ dst,
-                                                                   int M, int K, int N, unsigned *__restrict__ clear8) {
+                                                                   int M, int K, int N, unsigned *__restrict__ clear8, unsigned *__restrict__ clearN,
+                                                                   int nClear) {
     if (clear8 && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x < 8) clear8[threadIdx.x] = 0u;
+    if (clearN && blockIdx.x == 0 && blockIdx.y == 0)
+        for (int i = threadIdx.x; i < nClear; i += 256) clearN[i] = 0u;
     const int lane = threadIdx.x & 63, n = blockIdx.x * 4 + (threadIdx.x >> 6), m = blockIdx.y;
     if (n >= N || m >= M) return;
     const float *ar = a + (size_t)m * K, *br = b + (size_t)n * K;

@@ -98,6 +98,31 @@ __device__ __forceinline__ void gv_stage(uint8_t *lds, const uint8_t *__restrict
     }
 }
 
+// The same from rows that are still f32 (an expert's silu(gate)*up rows, XF [32][K]) and their maxima (rowMax, the bits of max |x|
+// accumulated by the kernel that wrote them): the per-row quantizer (linalg.QuantizeRowInt8: scale maxabs/127, codes
+// round-half-away) runs as the rows are staged, so the rows never exist as codes in memory and SwiGLU needs no launch of its own.
+__device__ __forceinline__ void gv_stage_f32(uint8_t *lds, const float *__restrict__ XF, const unsigned *__restrict__ rowMax, int K, int nKB,
+                                             const int (&rowOf)[GV_ROWS]) {
+    const int Kpad = nKB * 256, nGp = nKB * 8;
+    float *ldsS = (float *)(lds + (size_t)GV_ROWS * Kpad);
+    for (int i = threadIdx.x; i < GV_ROWS * (Kpad >> 2); i += blockDim.x) {
+        const int j = i / (Kpad >> 2), c = i - j * (Kpad >> 2), row = j == 0 ? rowOf[0] : (j == 1 ? rowOf[1] : (j == 2 ? rowOf[2] : rowOf[3]));
+        uint32_t codes = 0u;
+        if (row >= 0 && c * 4 < K) {
+            const float inv = 1.f / row_scale_of(__uint_as_float(rowMax[row]));
+            const float4_t v = *(const float4_t *)(XF + (size_t)row * K + c * 4);
+            const int c0 = (int)fminf(127.f, fmaxf(-127.f, roundf(__fmul_rn(v.x, inv)))), c1 = (int)fminf(127.f, fmaxf(-127.f, roundf(__fmul_rn(v.y, inv))));
+            const int c2 = (int)fminf(127.f, fmaxf(-127.f, roundf(__fmul_rn(v.z, inv)))), c3 = (int)fminf(127.f, fmaxf(-127.f, roundf(__fmul_rn(v.w, inv))));
+            codes = (uint32_t)(c0 & 255) | ((uint32_t)(c1 & 255) << 8) | ((uint32_t)(c2 & 255) << 16) | ((uint32_t)(c3 & 255) << 24);
+        }
+        *(uint32_t *)(lds + (size_t)j * Kpad + c * 4) = codes;
+    }
+    for (int i = threadIdx.x; i < GV_ROWS * nGp; i += blockDim.x) {
+        const int j = i / nGp, row = j == 0 ? rowOf[0] : (j == 1 ? rowOf[1] : (j == 2 ? rowOf[2] : rowOf[3]));
+        ldsS[i] = row >= 0 ? row_scale_of(__uint_as_float(rowMax[row])) : 0.f;
+    }
+}
+
 // One 256-element block of the wave's tile against the R staged rows (R the same on every lane: the rows past it are skipped
 // by a scalar branch, one body of code for any R). kb: the block's index in K.
 // ROW: the rows carry one activation scale each (ActQuantGroup 0): the fold takes the weight's group scale alone, as the reference's
@@ -187,10 +212,11 @@ __device__ __forceinline__ void gv_stream(GvTiles &t, rd_rsrc_t wr, int nTiles, 
 // and the rows past the last one exit: the blocks with work are the first in dispatch order, which spreads them evenly over
 // the XCDs and CUs (blocks are handed out round-robin; idle ones scattered among them skew that). Without the bitmap row y is
 // expert y, and exits when no token chose it. Dynamic LDS: gv_lds_bytes(nKB).
-template <bool ROW>
+// F32IN (with ROW): X is the experts' f32 rows [expert][32][K] and rowMax their maxima [expert][32]; they are quantized per row as staged.
+template <bool ROW, bool F32IN = false>
 __device__ __forceinline__ void moe_gemv_body(const uint8_t *__restrict__ Wt, size_t wStride, const uint8_t *__restrict__ X, size_t xStride,
                                               float *__restrict__ out, int N, int K, int T, int k, const signed char *__restrict__ rankOf, int nE,
-                                              const unsigned *__restrict__ activeBits, uint8_t *lds) {
+                                              const unsigned *__restrict__ activeBits, uint8_t *lds, const unsigned *__restrict__ rowMax = nullptr) {
     const int nKB = (K + 255) >> 8;
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     // xStride != 0: every expert reads activations of its own, so all blocks of an expert are placed on one XCD (blocks go to the
@@ -221,7 +247,10 @@ __device__ __forceinline__ void moe_gemv_body(const uint8_t *__restrict__ Wt, si
         }
         if (r0 > 0) gv_first(wt, wr, nTiles, tileOff, nKB, lane);
         __syncthreads(); // the previous pass is done with the staged rows
-        gv_stage(lds, X, K, nKB, rowOf);
+        if constexpr (F32IN)
+            gv_stage_f32(lds, (const float *)X, rowMax + (size_t)e * 32, K, nKB, rowOf);
+        else
+            gv_stage(lds, X, K, nKB, rowOf);
         __syncthreads();
         float rowS[GV_ROWS]; // ROW: the staged rows' scales (every group slot of a row holds it)
 #pragma unroll
@@ -253,6 +282,16 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_moe_gemv_w4a8r(const uint
     extern __shared__ __align__(16) uint8_t lds[];
     moe_gemv_body<true>(Wt, wStride, X, xStride, out, N, K, T, k, rankOf, nE, activeBits, lds);
 }
+// The experts' down projection over rows still in f32 (what rd_k_moe_gemv_w4a8r_gateup leaves): XF [expert][32][K] f32 with the
+// expert's tokens in ascending order as rows 0, 1, ..., rowMax [expert][32] the bits of each row's max |x|. The same values as
+// rd_k_moe_swiglu_quant_row followed by rd_k_moe_gemv_w4a8r, bit for bit, in one launch less.
+extern "C" __global__ __launch_bounds__(256) void rd_k_moe_gemv_w4a8r_f32in(const uint8_t *__restrict__ Wt, size_t wStride, const float *__restrict__ XF,
+                                                                             const unsigned *__restrict__ rowMax, float *__restrict__ out, int N, int K,
+                                                                             int T, int k, const signed char *__restrict__ rankOf, int nE,
+                                                                             const unsigned *__restrict__ activeBits) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    moe_gemv_body<true, true>(Wt, wStride, (const uint8_t *)XF, (size_t)32 * K * sizeof(float), out, N, K, T, k, rankOf, nE, activeBits, lds, rowMax);
+}
 
 // The experts' gate|up projection with SwiGLU and the per-32 quantization in its epilogue (same values as rd_k_moe_gemv_w4a8
 // followed by rd_k_moe_swiglu_quant, bit for bit). Wt per expert: [gate rows; up rows] (2*I rows). Grid (ceil(I / 64), nE),
@@ -260,19 +299,22 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_moe_gemv_w4a8r(const uint
 // leaves its sums in LDS and its up wave forms silu(gate) * up over the tile's 32 columns, which are one activation group,
 // quantizes it and writes it as row r0+j of the expert's own ROW8 activations XE (I elements a row). X: the step's rows, ROW8,
 // K elements. Dynamic LDS: gv_lds_bytes(nKB) + 1 KB.
-extern "C" __global__ __launch_bounds__(256) void rd_k_moe_gemv_w4a8_gateup(const uint8_t *__restrict__ Wt, size_t wStride,
-                                                                             const uint8_t *__restrict__ X, uint8_t *__restrict__ XE,
-                                                                             size_t xeStride, int I, int K, int T,
-                                                                             const signed char *__restrict__ rankOf, int nE,
-                                                                             const unsigned *__restrict__ activeBits) {
-    extern __shared__ __align__(16) uint8_t dyn[];
+// ROW: the step's rows carry one activation scale each and the output stays f32 — XF [expert][32][I] with the expert's tokens as
+// rows 0, 1, ... and rowMax [expert][32] taking the bits of each row's max |silu(gate)*up| through atomicMax (zero on entry;
+// non-negative floats order as their bits): the per-row quantizer needs the whole row, which no block of this kernel has, so it
+// runs where the rows are staged next (rd_k_moe_gemv_w4a8r_f32in).
+template <bool ROW>
+__device__ __forceinline__ void moe_gateup_body(const uint8_t *__restrict__ Wt, size_t wStride, const uint8_t *__restrict__ X, uint8_t *__restrict__ XE,
+                                                size_t xeStride, float *__restrict__ XF, unsigned *__restrict__ rowMax, int I, int K, int T,
+                                                const signed char *__restrict__ rankOf, int nE, const unsigned *__restrict__ activeBits, uint8_t *dyn) {
     float *xch = (float *)dyn; // [2 pairs][GV_ROWS][32]: the gate waves' sums
     uint8_t *lds = dyn + 1024;
     const int nKB = (K + 255) >> 8;
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int e = moe_block_expert(activeBits, rankOf, nE, T, blockIdx.y);
     if (e < 0) return;
-    Wt += (size_t)e * wStride, XE += (size_t)e * xeStride;
+    Wt += (size_t)e * wStride;
+    if constexpr (!ROW) XE += (size_t)e * xeStride;
     const int nGate = I >> 5, pair = wave >> 1, isUp = wave & 1, t = blockIdx.x * 2 + pair, nTiles = t < nGate ? 1 : 0;
     const rd_rsrc_t wr = make_rsrc(Wt, (uint32_t)(2 * nGate * nKB * 4608));
     auto tileOff = [&](int) { return (isUp * nGate + t) * nKB * 4608; };
@@ -293,10 +335,14 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_moe_gemv_w4a8_gateup(cons
         gv_stage(lds, X, K, nKB, rowOf);
         __syncthreads();
         float sum[GV_ROWS] = {0.f, 0.f, 0.f, 0.f};
-        gv_stream<false>(wt, wr, nTiles, tileOff, nKB, lds, lane, R, [&](int, const float(&facc)[GV_ROWS]) {
+        gv_stream<ROW>(wt, wr, nTiles, tileOff, nKB, lds, lane, R, [&](int, const float(&facc)[GV_ROWS]) {
 #pragma unroll
             for (int j = 0; j < GV_ROWS; j++) sum[j] = facc[j];
         });
+        if constexpr (ROW) { // the row's scale multiplies the finished sum
+#pragma unroll
+            for (int j = 0; j < GV_ROWS; j++) sum[j] = mul_rounded(sum[j], ((const float *)(lds + (size_t)GV_ROWS * nKB * 256))[j * nKB * 8]);
+        }
         if (!isUp && lane < 32) {
 #pragma unroll
             for (int j = 0; j < GV_ROWS; j++) xch[(pair * GV_ROWS + j) * 32 + lane] = sum[j];
@@ -306,11 +352,35 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_moe_gemv_w4a8_gateup(cons
 #pragma unroll
             for (int j = 0; j < GV_ROWS; j++)
                 if (j < R) { // the same on every lane: both halves of the wave hold the row's 32 columns
-                    const Quant1 qv = quant_one(__fmul_rn(silu_f64(xch[(pair * GV_ROWS + j) * 32 + (lane & 31)]), sum[j]));
-                    if (lane < 32) panel_store(XE, RD_PANEL_ROW8, r0 + j, t * 32 + lane, qv, I);
+                    const float act = __fmul_rn(silu_f64(xch[(pair * GV_ROWS + j) * 32 + (lane & 31)]), sum[j]);
+                    if constexpr (ROW) {
+                        const size_t row = (size_t)e * 32 + r0 + j;
+                        if (lane < 32) XF[row * I + t * 32 + lane] = act;
+                        const float ma = wave_max32(fabsf(act));
+                        if (lane == 0) atomicMax(rowMax + row, __float_as_uint(ma));
+                    } else {
+                        const Quant1 qv = quant_one(act);
+                        if (lane < 32) panel_store(XE, RD_PANEL_ROW8, r0 + j, t * 32 + lane, qv, I);
+                    }
                 }
         }
     }
+}
+extern "C" __global__ __launch_bounds__(256) void rd_k_moe_gemv_w4a8_gateup(const uint8_t *__restrict__ Wt, size_t wStride,
+                                                                             const uint8_t *__restrict__ X, uint8_t *__restrict__ XE,
+                                                                             size_t xeStride, int I, int K, int T,
+                                                                             const signed char *__restrict__ rankOf, int nE,
+                                                                             const unsigned *__restrict__ activeBits) {
+    extern __shared__ __align__(16) uint8_t dyn[];
+    moe_gateup_body<false>(Wt, wStride, X, XE, xeStride, nullptr, nullptr, I, K, T, rankOf, nE, activeBits, dyn);
+}
+extern "C" __global__ __launch_bounds__(256) void rd_k_moe_gemv_w4a8r_gateup(const uint8_t *__restrict__ Wt, size_t wStride,
+                                                                              const uint8_t *__restrict__ X, float *__restrict__ XF,
+                                                                              unsigned *__restrict__ rowMax, int I, int K, int T,
+                                                                              const signed char *__restrict__ rankOf, int nE,
+                                                                              const unsigned *__restrict__ activeBits) {
+    extern __shared__ __align__(16) uint8_t dyn[];
+    moe_gateup_body<true>(Wt, wStride, X, nullptr, 0, XF, rowMax, I, K, T, rankOf, nE, activeBits, dyn);
 }
 
 // gate/up rows [(token,rank)][2I] -> silu(gate)*up -> per-32 quantization -> the down-projection activations of that row's expert,

@@ -264,11 +264,13 @@ def test_moe_ragged_batch(dev, exp_act_group):
     assert agree >= 0.9 * total, (agree, total)
 
 
-def test_moe_fused_expert_gateup_equals_two_launches(dev):
-    """The expert gate|up GEMM with SwiGLU and quantization in its epilogue against the same step run as GEMM + SwiGLU kernel:
-    identical logits and routing, bit for bit."""
+@pytest.mark.parametrize("exp_act_group", [32, 0])
+def test_moe_fused_expert_gateup_equals_two_launches(dev, exp_act_group):
+    """The expert gate|up GEMM with SwiGLU (and, per-32, the quantization) in its epilogue against the same step run as GEMM +
+    SwiGLU-and-quantize kernel: identical logits and routing, bit for bit. Per-row activations (group 0): the fused kernel leaves
+    f32 rows and their maxima and the down projection quantizes them as it stages them."""
     import os
-    cfg = moe_cfg(n_layers=2, hidden=512, n_heads=4, n_kv=2, head_dim=64, n_experts=16, top_k=4, exp_inter=256)
+    cfg = moe_cfg(n_layers=2, hidden=512, n_heads=4, n_kv=2, head_dim=64, n_experts=16, top_k=4, exp_inter=256, exp_act_group=exp_act_group)
     pair = Pair(cfg, seed=71, dev=dev, slots=12, ctx_cap=32)
     try:
         rng = np.random.default_rng(8)
