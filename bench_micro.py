@@ -406,7 +406,7 @@ MFMA_I8_PEAK_TOPS = 5000.0
 
 def run_prefill(args):
     """A prompt pass into the decode step's own paged KV (PrefillLast): Llama-3-8B shape, one sequence, 2048 prompt tokens from
-    position 0, in passes of 128 rows; token ids through the embedding table, so nothing crosses PCIe inside the timed region.
+    position 0, in passes of the model's widest step (512 rows); token ids through the embedding table, so nothing crosses PCIe inside the timed region.
     A step is one whole prompt."""
     from goinfer_amd import capi, workloads
     n_tok = 2048
@@ -427,8 +427,8 @@ def run_prefill(args):
     tok_s = n_tok / (float(ms.mean()) / 1e3)
     _, prof = res.model.bench_prefill(0, ids, profile=True)
     classes = {k: {"ms_per_step": round(v[0], 4), "launches_per_step": v[1]} for k, v in prof.items()}
-    # dominant kernel: the Q4_K GEMM over 128 rows (every weight tile read and dequantized once for four row tiles of 32); the
-    # four projections of a layer are one launch each per pass. Flops over all rows of the prompt, milliseconds over all four classes
+    # dominant kernels: the many-row Q4_K GEMMs (every weight tile decoded once for four row tiles of 32); the four projections of
+    # a layer are one launch each per pass. Flops over all rows of the prompt, milliseconds over all four classes
     # (the last row's one-row step rides in the same classes: 1 row of 2048).
     H, hd = cfg["hidden"], cfg["head_dim"]
     qd, kvd, I = cfg["n_heads"] * hd, cfg["n_kv"] * hd, cfg["inter"]
@@ -438,11 +438,11 @@ def run_prefill(args):
     g_n = sum(prof[k][1] for k in ("gemm_qkv", "gemm_o", "gemm_gateup", "gemm_down"))
     tfl = flops / (g_ms / 1e3) / 1e12
     out = base_line("prompt tok/s into the paged KV, Llama-3-8B-shape Q4_K, 2048-token prompt; achieved int8 MFMA TOP/s vs peak", tok_s, "tok/s", steps, warmup,
-                    float(ms.mean()), "prefill: %s, %d layers, one sequence, %d prompt tokens from position 0 (PrefillLast), passes of 128 rows"
-                    % (cfg["name"], args.layers, n_tok),
+                    float(ms.mean()), "prefill: %s, %d layers, one sequence, %d prompt tokens from position 0 (PrefillLast), passes of %d rows"
+                    % (cfg["name"], args.layers, n_tok, res.model.max_rows()),
                     "synthetic: N(0,0.02) weights quantized to Q4_K (int8 head and embedding), random token ids", {"prompt_tokens": n_tok, "seed": args.seed})
     out["roofline"] = {"bound": "mfma", "achieved": round(tfl, 1), "peak": MFMA_I8_PEAK_TOPS, "unit": "TOP/s", "frac": round(tfl / MFMA_I8_PEAK_TOPS, 4),
-                       "traffic": None, "kernel": "rd_k_gemm8_q4k_kw* (qkv with RoPE and KV store, o, gate|up, down)", "avg_launch_ms": round(g_ms / g_n, 5),
+                       "traffic": None, "kernel": "rd_k_gemm8_q4k_rows* (qkv with RoPE and KV store, o, gate|up with SwiGLU, down)", "avg_launch_ms": round(g_ms / g_n, 5),
                        "algorithmic_flops_per_launch": int(flops / g_n)}
     out["kernel_classes"] = classes
     cpu = None

@@ -18,7 +18,7 @@ EXPORTS = [
     "rd_device_mem_info", "rd_matmul_bt", "rd_dequant_q4k", "rd_gemm_q4k", "rd_gemm_w8a8", "rd_gemm_w4a8",
     "rd_attn_ragged", "rd_moe_route", "rd_rmsnorm", "rd_rope", "rd_model_create", "rd_model_destroy",
     "rd_model_upload_q4k", "rd_model_upload_w8a8", "rd_model_upload_w4a8", "rd_model_upload_f32", "rd_model_finalize",
-    "rd_kv_configure", "rd_kv_upload", "rd_kv_truncate", "rd_kv_reset", "rd_step_batch", "rd_forward",
+    "rd_kv_configure", "rd_kv_upload", "rd_kv_truncate", "rd_kv_reset", "rd_step_batch", "rd_model_max_rows", "rd_forward",
     "rd_last_moe_indices", "rd_model_upload_embedding", "rd_bench_steps", "rd_bench_profile", "rd_bench_attn_chain", "rd_bench_enqueue", "rd_bench_attn_kernel_name", "rd_bench_attn_in_step", "rd_moe_route_ex", "rd_attn_ragged_ex", "rd_model_set_router", "rd_model_set_window", "rd_model_set_block", "rd_model_set_graph", "rd_model_graph_stats", "rd_bench_prefill", "rd_bench_class_count",
     "rd_bench_class_name", "rd_bench_kernel", "rd_gateup_q4k_quant", "rd_moe_replay", "rd_bench_attn", "rd_step_ragged", "rd_prefill_last",
     "rd_kv_configure_typed", "rd_attn_ragged_i8", "rd_attn_ragged_rows", "rd_plan_attention", "rd_plan_gemm", "rd_step_batch_topk", "rd_last_logits", "rd_topk_rows", "rd_bench_attn_i8", "rd_step_ragged_draw", "rd_forward_no_logits",
@@ -445,6 +445,10 @@ class Model:
 
     def kv_truncate(self, slot, pos):
         check(lib().rd_kv_truncate(self.h, slot, pos), "rd_kv_truncate")
+
+    def max_rows(self):
+        """The widest step (BatchStepRange's hi) and the rows of a prompt pass."""
+        return int(lib().rd_model_max_rows(self.h))
 
     def step_batch(self, slots, pos, emb, want=WANT_LOGITS):
         emb = _f32(emb)

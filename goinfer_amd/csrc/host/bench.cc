@@ -235,7 +235,7 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
     if (!d || !name || !args || iters <= 0 || !ms_out) return RD_ERR_ARG;
     std::string nm(name);
     const bool isGemm = nm == "gemm_q4k" || nm == "gemm_q5k" || nm == "gemm_q6k";
-    if (isGemm && n_args >= 4 && (args[0] % 32 || args[1] % 256 || args[0] <= 0 || args[1] <= 0 || args[2] < 1 || args[2] > 128)) {
+    if (isGemm && n_args >= 4 && (args[0] % 32 || args[1] % 256 || args[0] <= 0 || args[1] <= 0 || args[2] < 1 || args[2] > GEMM_WIDE_ROWS)) {
         rd_set_error("%s bench: bad shape", name);
         return RD_ERR_ARG;
     }

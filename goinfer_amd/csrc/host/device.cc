@@ -87,6 +87,12 @@ static const KName kNames[] = {
     {"rd_k_unpanel_a8", &Kernels::unpanel_a8},
     {"rd_k_retile_w8a8_8", &Kernels::retile_w8a8_8},
     {"rd_k_retile_w4a8_8", &Kernels::retile_w4a8_8},
+    {"rd_k_gemm8_q4k_rows", &Kernels::gemm8_q4k_rows},
+    {"rd_k_gemm8_q4k_rows_g2", &Kernels::gemm8_q4k_rows_g2},
+    {"rd_k_gemm8_q4k_rows_gateup", &Kernels::gemm8_q4k_rows_gateup},
+    {"rd_k_gemm8_q4k_rows_gateup_gelu", &Kernels::gemm8_q4k_rows_gateup_gelu},
+    {"rd_k_gemm8_q4k_rows_qkv", &Kernels::gemm8_q4k_rows_qkv},
+    {"rd_k_gemm8_q4k_rows_qkv_g2", &Kernels::gemm8_q4k_rows_qkv_g2},
     {"rd_k_gemm8_q4k_gateup", &Kernels::gemm8_q4k_gateup},
     {"rd_k_gemm8_q4k_gateup_gelu", &Kernels::gemm8_q4k_gateup_gelu},
     {"rd_k_add_one", &Kernels::add_one},
@@ -454,6 +460,8 @@ void free_weight(rd_device *d, DevWeight *w) {
     *w = DevWeight();
 }
 
+bool rows_gemm_enabled() { return !getenv("ROCMDECODE_NO_ROWS_GEMM"); }
+
 int launch_gemm(rd_device *d, const DevWeight &w, const void *Xp, float *P, int M, GemmPlan *plan_out, int ldP, int splits, int kw, float *resid,
                 size_t xpStride, size_t pStride) {
     if (M < 1 || M > GEMM_WIDE_ROWS) { // rows past 32 are further M-tiles, grid.z of the launch
@@ -473,6 +481,13 @@ int launch_gemm(rd_device *d, const DevWeight &w, const void *Xp, float *P, int 
     if (ldP <= 0) ldP = w.N;
     if (is_gemm8_kind(w.kind)) {
         const int tiles = w.N / 32, tpb = p.kw == 2 ? 2 : 1;
+        // more than 32 rows of Q4_K: four M-tiles share each decoded weight tile (the same sums, row for row)
+        if (gemm8_lane(w) == 0 && M > 32 && rows_gemm_enabled()) {
+            const unsigned gz = (unsigned)((M + 127) / 128);
+            const bool two = rows_gemm_two_groups((size_t)tiles * p.splits * gz);
+            return d->launch(two ? d->k.gemm8_q4k_rows_g2 : d->k.gemm8_q4k_rows, (unsigned)tiles, (unsigned)p.splits, gz, two ? 512 : 256, (const void *)w.tiled, Xp,
+                             P, w.N, nKB, p.kbPerSplit, p.kw, M, ldP, resid, xpStride, pStride);
+        }
         hipFunction_t f = d->k.gemm8[gemm8_lane(w)][p.kw == 8 ? 2 : (p.kw == 4 ? 1 : 0)];
         return d->launch(f, (unsigned)((tiles + tpb - 1) / tpb), (unsigned)p.splits, (unsigned)((M + 31) / 32), (unsigned)(64 * p.kw * tpb), (const void *)w.tiled,
                          (const void *)w.scales, Xp, P, w.N, nKB, p.kbPerSplit, M, ldP, resid, xpStride, pStride);

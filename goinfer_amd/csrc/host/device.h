@@ -36,6 +36,9 @@ struct Kernels {
     // [lane: 0 q4k, 1 w8a8, 2 w4a8 (per-32 activations), 3 w8a8, 4 w4a8 with one activation scale per row, 5 q5k, 6 q6k][waves per tile 2, 4, 8]
     hipFunction_t gemm8[7][3];
     hipFunction_t gemm8_qkv[7][3]; // the q|k|v projection with RoPE and the KV store in its epilogue, indexed like gemm8
+    // Q4_K for passes of more than 32 rows: four M-tiles against each decoded weight tile (_g2: a second group of waves halves the K
+    // ranges, for grids of few weight tiles)
+    hipFunction_t gemm8_q4k_rows, gemm8_q4k_rows_g2, gemm8_q4k_rows_gateup, gemm8_q4k_rows_gateup_gelu, gemm8_q4k_rows_qkv, gemm8_q4k_rows_qkv_g2;
     hipFunction_t gemm8_q4k_gateup, gemm8_q4k_gateup_gelu, add_one, moe_gemv_w4a8, moe_gemv_w4a8r, moe_gemv_w4a8r_f32in, moe_gemv_w4a8_gateup, moe_gemv_w4a8r_gateup, retile_w4a8_gv, rope_table;
     hipFunction_t dequant_q5k, retile_q5k, dequant_q6k, retile_q6k;
     hipFunction_t kv_store, kv_read, qkv_rope_store, attn_partial, attn_partial_wide, attn_combine, attn_combine_quant;
@@ -201,7 +204,10 @@ inline bool is_gemm8_kind(int kind) { return kind >= 0 && kind <= 4; } // every 
 // Up to 128 rows as M-tiles of 32: M-tile mt reads its panels at Xp + mt*xpStride (bytes) and writes its partial sums at
 // P + mt*pStride (floats), each laid out as launch_gemm's; the int8 kernels take the M-tiles as grid.z of one launch, the others one
 // launch per M-tile. Either way a row is the same row whatever pass it rides in.
-constexpr int GEMM_WIDE_ROWS = 128;
+constexpr int GEMM_WIDE_ROWS = 512;
+// the many-row Q4_K kernels: whether a grid of `blocks` blocks of four waves takes the second group of waves (under two waves per SIMD otherwise)
+bool rows_gemm_enabled();
+inline bool rows_gemm_two_groups(size_t blocks) { return blocks < 2u * 256u; }
 int launch_gemm_wide(rd_device *d, const DevWeight &w, const void *Xp, size_t xpStride, float *P, size_t pStride, int M, GemmPlan *plan, int ldP = 0,
                      int splits = 0, int kw = 0);
 size_t panel_bytes_for(const DevWeight &w);

@@ -882,6 +882,13 @@ static int step_launches(rd_model *m, int B, int want) {
             Scope s(m, KC_GEMM_QKV); // projection, bias, RoPE and the KV store in one launch (M-tiles of 32 rows as grid.z)
             const DevWeight &w = l.qkv;
             const int nKB = kblocks_for(w), kw = plan_gemm(w.kind, w.N, nKB, w.act_group).kw; // the plain GEMM's waves per tile, in one split
+            if (gemm8_lane(w) == 0 && B > 32 && rows_gemm_enabled()) { // more than 32 rows: four M-tiles per decoded weight tile
+                const unsigned gz = (unsigned)((B + 127) / 128);
+                const bool two = rows_gemm_two_groups((size_t)(w.N / 32) * gz);
+                RC(d->launch(two ? d->k.gemm8_q4k_rows_qkv_g2 : d->k.gemm8_q4k_rows_qkv, (unsigned)(w.N / 32), 1, gz, two ? 512 : 256, (const void *)w.tiled,
+                             (const void *)m->XpA, w.N, nKB, kw, B, m->qbuf, l.Kp, l.Vp, (const int *)m->tables, m->blocks_per_slot, (const int *)m->rowSlot,
+                             (const int *)m->rowPos, (const double *)m->rope_cs, (const float *)l.qkv_bias, nH, nKV, HD, m->xpAStride));
+            } else
             RC(d->launch(d->k.gemm8_qkv[gemm8_lane(w)][kw == 8 ? 2 : (kw == 4 ? 1 : 0)], (unsigned)(w.N / 32), 1, (unsigned)((B + 31) / 32), (unsigned)(64 * kw),
                          (const void *)w.tiled, (const void *)w.scales, (const void *)m->XpA, w.N, nKB, B, m->qbuf, l.Kp, l.Vp, (const int *)m->tables,
                          m->blocks_per_slot, (const int *)m->rowSlot, (const int *)m->rowPos, (const double *)m->rope_cs, (const float *)l.qkv_bias, nH, nKV,
@@ -933,6 +940,11 @@ static int step_launches(rd_model *m, int B, int want) {
             RC(add_norm_quant(m, B, m->P, plan.splits, l.ffn_norm, l.gateup, m->XpA, nullptr, nullptr, l.post_attn_norm));
             if (gateup_fusable(c, l.gateup) && !getenv("ROCMDECODE_NO_FUSED_GATEUP")) {
                 Scope s(m, KC_GEMM_GATEUP); // gate|up GEMM + SwiGLU + quantization in one launch (M-tiles of 32 rows as grid.z)
+                if (B > 32 && rows_gemm_enabled()) // more than 32 rows: four M-tiles per decoded weight tile
+                    RC(d->launch(m->act == RD_ACT_GELU_TANH ? d->k.gemm8_q4k_rows_gateup_gelu : d->k.gemm8_q4k_rows_gateup, (unsigned)(c.inter / 32), 1,
+                                 (unsigned)((B + 127) / 128), 256, (const void *)l.gateup.tiled, (const void *)m->XpA, m->XpB, c.inter, H / 256, B, m->xpAStride,
+                                 m->xpBStride));
+                else
                 RC(d->launch(m->act == RD_ACT_GELU_TANH ? d->k.gemm8_q4k_gateup_gelu : d->k.gemm8_q4k_gateup, (unsigned)(c.inter / 32), 1, (unsigned)((B + 31) / 32), GATEUP_THREADS, (const void *)l.gateup.tiled,
                              (const void *)m->XpA, m->XpB, panel_kind_for(l.down), c.inter, H / 256, B, m->xpAStride, m->xpBStride));
             } else {
@@ -1195,6 +1207,8 @@ int model_step(rd_model *m, int B, const int *slot, const int *pos, const float 
     if ((want & RD_WANT_ARGMAX) && ids) RC(d->d2h(ids, m->ids, sizeof(int) * (size_t)B));
     return RD_OK;
 }
+
+extern "C" int rd_model_max_rows(const rd_model *m) { return m && m->finalized ? m->max_rows : 0; }
 
 extern "C" int rd_step_batch(rd_model *m, int B, const int *slot, const int *pos, const float *emb, int want, float *logits, int *ids) {
     if (!m || !slot || !pos || !emb) return RD_ERR_ARG;

@@ -96,7 +96,7 @@ struct rd_model {
     int kv_type = 0; // RD_KV_F16 or RD_KV_I8
     // Rows per step: up to ROWS_MAX as M-tiles of 32 (a dense model; MoE steps keep to one M-tile). The step's buffers hold
     // max_rows rows; partial sums and panels are per M-tile, pStride floats / xpStride bytes apart.
-    static constexpr int ROWS_MAX = 128;
+    static constexpr int ROWS_MAX = 512;
     int max_rows = 32;
     size_t pStride = 0, xpAStride = 0, xpBStride = 0;
     static constexpr int META_HDR = 3 * ROWS_MAX + ROWS_MAX * 6 + 8; // row slot, position, length, the rows' draw records (6 ints each), the expert bitmap

@@ -118,17 +118,27 @@ extern "C" int rd_gateup_q4k_quant(rd_device *d, const void *Wg, const void *Wu,
     if (rc) return rc;
     DevBuf A(d), Xp(d), X2(d), O(d);
     auto body = [&]() -> int {
-        RC(A.alloc(sizeof(float) * (size_t)32 * K));
-        RC(Xp.alloc(a8_bytes(K)));
-        RC(X2.alloc(a8_bytes(I)));
-        RC(O.alloc(sizeof(float) * (size_t)32 * I));
-        for (int m0 = 0; m0 < M; m0 += 32) {
-            int mc = std::min(32, M - m0);
+        // passes of up to GEMM_WIDE_ROWS rows as the step runs them: up to 32 rows in the decode kernel, more in the many-row kernel
+        const int chunk = std::min(M, GEMM_WIDE_ROWS), tiles = (chunk + 31) / 32;
+        const size_t xpStride = a8_bytes(K), x2Stride = a8_bytes(I);
+        RC(A.alloc(sizeof(float) * (size_t)chunk * K));
+        RC(Xp.alloc(xpStride * tiles));
+        RC(X2.alloc(x2Stride * tiles));
+        RC(O.alloc(sizeof(float) * (size_t)chunk * I));
+        for (int m0 = 0; m0 < M; m0 += chunk) {
+            int mc = std::min(chunk, M - m0);
             RC(d->h2d(A.p, a + (size_t)m0 * K, sizeof(float) * (size_t)mc * K));
-            RC(quantize_rows(d, A.as<float>(), mc, K, PANEL_A8, 32, Xp.p));
-            RC(d->launch(d->k.gemm8_q4k_gateup, (unsigned)(I / 32), 1, 1, GATEUP_THREADS, (const void *)w.tiled, (const void *)Xp.p, X2.as<uint8_t>(),
-                         (int)PANEL_A8, I, K / 256, mc, (size_t)0, (size_t)0));
-            RC(d->launch(d->k.unpanel_a8, (unsigned)(I / 256), (unsigned)mc, 1, 256, (const void *)X2.p, O.as<float>(), I));
+            for (int t = 0; t * 32 < mc; t++)
+                RC(quantize_rows(d, A.as<float>() + (size_t)t * 32 * K, std::min(32, mc - t * 32), K, PANEL_A8, 32, (char *)Xp.p + (size_t)t * xpStride));
+            if (mc > 32 && rows_gemm_enabled())
+                RC(d->launch(d->k.gemm8_q4k_rows_gateup, (unsigned)(I / 32), 1, (unsigned)((mc + 127) / 128), 256, (const void *)w.tiled, (const void *)Xp.p,
+                             X2.as<uint8_t>(), I, K / 256, mc, xpStride, x2Stride));
+            else
+                RC(d->launch(d->k.gemm8_q4k_gateup, (unsigned)(I / 32), 1, (unsigned)((mc + 31) / 32), GATEUP_THREADS, (const void *)w.tiled, (const void *)Xp.p,
+                             X2.as<uint8_t>(), (int)PANEL_A8, I, K / 256, mc, xpStride, x2Stride));
+            for (int t = 0; t * 32 < mc; t++)
+                RC(d->launch(d->k.unpanel_a8, (unsigned)(I / 256), (unsigned)std::min(32, mc - t * 32), 1, 256, (const void *)((char *)X2.p + (size_t)t * x2Stride),
+                             O.as<float>() + (size_t)t * 32 * I, I));
             RC(d->d2h(dst + (size_t)m0 * I, O.p, sizeof(float) * (size_t)mc * I));
         }
         return RD_OK;

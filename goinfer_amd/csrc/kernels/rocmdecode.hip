@@ -6,6 +6,7 @@
 #include "act.h"
 #include "attn.h"
 #include "gemm8.h"
+#include "gemm8_rows.h"
 #include "kquant.h"
 #include "misc.h"
 #include "moe.h"

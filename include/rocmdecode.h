@@ -224,6 +224,9 @@ int rd_kv_reset(rd_model *m, int slot);
 /* emb: host f32 [B][hidden] (embedding rows, already scaled: decoder/residency.go:1077-1123);
  * logits: host f32 [B][vocab] when want&RD_WANT_LOGITS; ids: int32 [B] when want&RD_WANT_ARGMAX (lowest index wins). */
 int rd_step_batch(rd_model *m, int B, const int *slot, const int *pos, const float *emb, int want, float *logits, int *ids);
+/* The widest step of a finalized model, the `hi` of resident/subsystems.go:111-116 BatchStepRange (lo is 1): 512 rows for a dense
+ * model (sixteen GEMM row tiles of 32), 32 for a MoE model; 0 before rd_model_finalize. Prompt passes run this many rows at once. */
+int rd_model_max_rows(const rd_model *m);
 /* A row's on-device draw: resident/forward.go:43-52 BatchDraw with the (seed, draw) of Sampler.NextDraw
  * (internal/runtime/sampling/sampler_gumbel.go:68-76). RD_DRAW_GUMBEL is the temperature-only draw
  * argmax_i(f32(l_i * 1/T) + G_i) with Philox4x32-10 noise, the function of sampler_gumbel.go:41-66,117-123 and

@@ -76,6 +76,24 @@ def test_gemm_q4k_rows_past_32_equal_solo_rows(dev):
         assert np.array_equal(solo[0].view(np.uint32), wide[r].view(np.uint32))
 
 
+@pytest.mark.parametrize("M,N,K", [(300, 160, 2048), (200, 256, 14336), (512, 4096, 768), (129, 6144, 4096)])
+def test_gemm_q4k_many_row_kernel_equals_the_32_row_kernel(dev, M, N, K):
+    """Past 32 rows four M-tiles share each decoded weight tile (one group of waves for a large grid, two for a small one, over
+    one K range or several, one split or two): every row comes out as the 32-row kernel and the one-row kernel give it, bit for
+    bit, and within 1e-5 of the f64 sum."""
+    blocks = synth.q4k_normal(31 + N, N, K)
+    a = synth.normal(32 + M, M * K).reshape(M, K)
+    wide = dev.gemm_q4k(blocks, N, K, a)
+    for r0 in (0, 96, M - 32):
+        part = dev.gemm_q4k(blocks, N, K, a[r0:r0 + 32])
+        assert np.array_equal(part.view(np.uint32), wide[r0:r0 + 32].view(np.uint32)), r0
+    solo = dev.gemm_q4k(blocks, N, K, a[M - 1:M])
+    assert np.array_equal(solo[0].view(np.uint32), wide[M - 1].view(np.uint32))
+    rows = [0, 33, M - 1]
+    w = ob.WMat(ob.OR_Q4K, N, K, blocks, act_group=32)
+    assert rel_err(wide[rows], ob.matmul_f64ref(w, a[rows])) < 1e-5
+
+
 def test_gemm_q4k_random_blocks_and_saturated_scales(dev):
     """Random bytes reach every code, scale and minimum (quantized normals do not), with every fifth block's 6-bit fields saturated:
     the shapes of the reference's own kernel test (actgroup_kernel_test.go:305-364, K = 3072, N = 200 rounded to whole tiles)."""
@@ -149,7 +167,7 @@ def test_gemm_q4k_fused_gate_up(dev):
     assert rel_err(got, want) < 1e-4  # silu(gate) * up of two GEMM outputs each within 1e-5
 
 
-@pytest.mark.parametrize("M", [1, 9, 32, 40])
+@pytest.mark.parametrize("M", [1, 9, 32, 40, 300])
 def test_fused_gate_up_kernel(dev, M):
     """The decode step's single-launch gate|up + SwiGLU + quantization kernel, on its own."""
     from tests.test_gpu_baseline_shapes import check_fused

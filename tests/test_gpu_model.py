@@ -448,25 +448,29 @@ def test_wide_batch_rows_equal_solo_rows_deep_k(dev):
         pair.close()
 
 
-@pytest.mark.parametrize("B", [70, 128])
-def test_wide_batch_rows_equal_solo_rows(dev, B):
-    """A dense model steps up to 128 rows at once (four GEMM row tiles): every row is still the row its own one-row step computes,
-    bit for bit, whatever tile it rides in; a batch past the range is refused."""
-    cfg = dense_cfg(n_layers=2)
+@pytest.mark.parametrize("B,wide", [(70, False), (128, False), (300, False), (300, True), (512, False)])
+def test_wide_batch_rows_equal_solo_rows(dev, B, wide):
+    """A dense model steps up to 512 rows at once (GEMM row tiles of 32, four to a weight tile in the many-row kernels): every row is
+    still the row its own one-row step computes, bit for bit, whatever tile it rides in; a batch past the range is refused.
+    wide: projections of several super-blocks, so the many-row kernels walk more than one K range per tile."""
+    cfg = dense_cfg(n_layers=2, hidden=1024, n_heads=8, n_kv=2, head_dim=128, inter=2560) if wide else dense_cfg(n_layers=2)
     pair = Pair(cfg, seed=61, dev=dev, slots=2 * B, ctx_cap=32)
     try:
+        assert pair.gpu.max_rows() == 512
         rng = np.random.default_rng(6)
         pos = [0] * B
         for step in range(3):
             toks = rng.integers(0, cfg["vocab"], B)
             emb = pair.emb[toks]
             got, ids = pair.gpu.step_batch(list(range(B)), pos, emb, capi.WANT_LOGITS | capi.WANT_ARGMAX)
-            for b in (0, 31, 32, 33, 63, 64, 69, B - 1):
+            for b in sorted({0, 31, 32, 33, 63, 64, 69, 127, 128, 129, 255, 256, 288, B - 1}):
+                if b >= B:
+                    continue
                 solo = pair.gpu.forward(B + b, pos[b], emb[b])
                 assert np.array_equal(solo.view(np.uint32), got[b].view(np.uint32)), (step, b)
                 assert ids[b] == int(np.argmax(got[b]))
             pos = [p + 1 for p in pos]  # the twin slots of the checked rows advance with them; the other twins are never read
         with pytest.raises(capi.RocmError, match="stepper range"):
-            pair.gpu.step_batch(list(range(129)), [0] * 129, pair.emb[:129])
+            pair.gpu.step_batch(list(range(513)), [0] * 513, np.zeros((513, cfg["hidden"]), np.float32))
     finally:
         pair.close()

@@ -151,13 +151,13 @@ def test_timed_prompt_pass_leaves_the_prefill_state(dev):
     device: the slot it fills continues with the same bits as a slot filled through rd_prefill_last from host rows."""
     from goinfer_amd import synth
     cfg = dense_cfg(n_layers=2, hidden=256, inter=512, vocab=4096)
-    pair = Pair(cfg, 47, dev, slots=2, ctx_cap=320)
+    pair = Pair(cfg, 47, dev, slots=2, ctx_cap=1152)
     try:
         q, sc = synth.w8a8_normal(78, cfg["vocab"], cfg["hidden"], 0.02)
         rows = q.astype(np.float32) * sc[:, None]
         pair.gpu.upload_embedding(q, sc)
         rng = np.random.default_rng(9)
-        toks = rng.integers(0, cfg["vocab"], 283)  # two full passes of 128, one of 26, the last row alone
+        toks = rng.integers(0, cfg["vocab"], 1100)  # two full passes of 512 rows, one of 75, the last row alone
         pair.gpu.prefill_last(0, 0, rows[toks])
         ms, classes = pair.gpu.bench_prefill(1, toks, profile=True)
         assert ms > 0 and classes["gemm_qkv"][1] == 4 * cfg["n_layers"]
