@@ -23,9 +23,10 @@ enum { PANEL_A8 = 3, PANEL_ROW8 = 4 }; // = RD_PANEL_* of the kernels
 // dynamic LDS of the experts' GEMM kernels: four rows of K elements (codes, scales, sums) + their exchange area
 inline unsigned moe_gemv_lds(int K) { return (unsigned)(4 * ((K + 255) / 256) * 320 + 1024); }
 constexpr int MOE_GEMV_MAX_K = 12288; // 4 rows x 48 blocks x 320 B + 1 KB = 61 KB of LDS
-// grid.x of rd_k_moe_gemv_w4a8 (moe.h): a wave streams about eight 256-element blocks, as whole tiles of 32 weight rows
+// grid.x of rd_k_moe_gemv_w4a8 (moe.h): a wave streams about four 256-element blocks, as whole tiles of 32 weight rows (measured on
+// the Qwen3-MoE down projection, K = 768: one tile a wave 27 us a launch, two tiles 30 us, four 41 us)
 inline unsigned moe_gemv_grid(int N, int K) {
-    int per = std::max(1, 8 / ((K + 255) / 256));
+    int per = std::max(1, 4 / ((K + 255) / 256));
     if (const char *e = getenv("ROCMDECODE_MOE_TILES")) per = std::max(1, atoi(e));
     return (unsigned)((N / 32 + 4 * per - 1) / (4 * per));
 }
