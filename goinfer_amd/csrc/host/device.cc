@@ -186,6 +186,7 @@ static int open_common(int ordinal, const void *image, rd_device **out) {
                 return RD_ERR_HIP;
             }
         }
+    topk_static_prepare_device(ordinal); // the allocation-free top-K's one-time set-up for this device, outside any capture
     *out = d;
     return RD_OK;
 }

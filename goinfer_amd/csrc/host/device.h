@@ -208,6 +208,7 @@ inline bool is_gemm8_kind(int kind) { return kind >= 0 && kind <= 4; } // every 
 constexpr int GEMM_WIDE_ROWS = 512;
 // the many-row Q4_K kernels: whether a grid of `blocks` blocks of four waves takes the second group of waves (under two waves per SIMD otherwise)
 bool rows_gemm_enabled();
+void topk_static_prepare_device(int ordinal); // ops.cc: opens the allocation-free top-K's library and looks its scratch up for this device
 inline bool rows_gemm_two_groups(size_t blocks) { return blocks < 2u * 256u; }
 int launch_gemm_wide(rd_device *d, const DevWeight &w, const void *Xp, size_t xpStride, float *P, size_t pStride, int M, GemmPlan *plan, int ldP = 0,
                      int splits = 0, int kw = 0);

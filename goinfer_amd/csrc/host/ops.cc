@@ -608,10 +608,15 @@ extern "C" int rd_topk_rows(rd_device *d, const float *logits, int rows, int V, 
 #include <dlfcn.h>
 #include <mutex>
 typedef int (*topk_static_fn)(int, void *, const float *, int, int, int, double, int, int *, float *, double *, char *, size_t);
-static topk_static_fn load_topk_static(std::string *why) {
+typedef int (*topk_static_prepare_fn)(int, char *, size_t);
+struct TopkStaticLib {
+    topk_static_fn run = nullptr;
+    topk_static_prepare_fn prepare = nullptr;
+    std::string err;
+};
+static const TopkStaticLib &load_topk_static() {
     static std::once_flag once;
-    static topk_static_fn fn = nullptr;
-    static std::string err;
+    static TopkStaticLib lib;
     std::call_once(once, [] {
         std::string path = "librocmdecode_static.so";
         Dl_info info;
@@ -623,26 +628,35 @@ static topk_static_fn load_topk_static(std::string *why) {
         if (const char *e = getenv("ROCMDECODE_STATIC_LIB")) path = e;
         void *h = dlopen(path.c_str(), RTLD_NOW | RTLD_LOCAL);
         if (!h) {
-            err = std::string("cannot load ") + path + ": " + dlerror();
+            lib.err = std::string("cannot load ") + path + ": " + dlerror();
             return;
         }
-        fn = (topk_static_fn)dlsym(h, "rd_topk_rows_static_impl");
-        if (!fn) err = path + " lacks rd_topk_rows_static_impl";
+        lib.run = (topk_static_fn)dlsym(h, "rd_topk_rows_static_impl");
+        lib.prepare = (topk_static_prepare_fn)dlsym(h, "rd_topk_static_prepare");
+        if (!lib.run || !lib.prepare) lib.run = nullptr, lib.err = path + " lacks rd_topk_rows_static_impl / rd_topk_static_prepare";
     });
-    if (!fn && why) *why = err;
-    return fn;
+    return lib;
+}
+
+// rd_device_open's part: the allocation-free library is opened and its scratch address looked up for this device now, so that a
+// later rd_topk_rows_static under stream capture has nothing left to set up. A missing library is not this call's error: the entry
+// point reports it when it is used.
+void topk_static_prepare_device(int ordinal) {
+    const TopkStaticLib &lib = load_topk_static();
+    if (!lib.run) return;
+    char msg[400] = "";
+    (void)lib.prepare(ordinal, msg, sizeof msg);
 }
 
 extern "C" int rd_topk_rows_static(int device, void *stream, const float *logits_dev, int rows, int V, int k, double temperature, int want_z,
                                    int *ids_dev, float *vals_dev, double *z_dev) {
-    std::string why;
-    topk_static_fn fn = load_topk_static(&why);
-    if (!fn) {
-        rd_set_error("rd_topk_rows_static: %s", why.c_str());
+    const TopkStaticLib &lib = load_topk_static();
+    if (!lib.run) {
+        rd_set_error("rd_topk_rows_static: %s", lib.err.c_str());
         return RD_ERR_STATE;
     }
     char msg[400] = "";
-    int rc = fn(device, stream, logits_dev, rows, V, k, temperature, want_z, ids_dev, vals_dev, z_dev, msg, sizeof msg);
+    int rc = lib.run(device, stream, logits_dev, rows, V, k, temperature, want_z, ids_dev, vals_dev, z_dev, msg, sizeof msg);
     if (rc) rd_set_error("%s", msg);
     return rc;
 }

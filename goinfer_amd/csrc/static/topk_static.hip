@@ -2,8 +2,9 @@
 // loops, harnesses that forbid hipMalloc. Same kernels as rd_topk_rows (../kernels/topk.h, compiled into this file's own code
 // object), same results; the scratch between the launches (per-chunk histograms and maxima, candidate lists and counts, the
 // chunks' shares of Z) lives in one file-scope device array instead of call-scoped allocations. Inputs and outputs are device
-// pointers the caller owns. This file is built by hipcc into librocmdecode_static.so, which librocmdecode.so opens on the first
-// call of rd_topk_rows_static; nothing here calls hipMalloc, hipFree or any allocating routine.
+// pointers the caller owns. This file is built by hipcc into librocmdecode_static.so, which librocmdecode.so opens when a device
+// is opened (rd_device_open looks the scratch address up for that device then, outside any capture) or, failing that, on the
+// first call of rd_topk_rows_static; nothing here calls hipMalloc, hipFree or any allocating routine.
 //
 // Every call on a GPU shares that GPU's array and finds the previous call's contents in it: the candidate counts, which must
 // start at zero, are cleared by a fill kernel at the head of every call (a kernel, not hipMemsetAsync: memset nodes captured
@@ -51,7 +52,33 @@ __global__ void rd_k_static_zero_counts(int *__restrict__ ccount, int n) {
     if (i < n) ccount[i] = 0;
 }
 
-// Return codes are rocmdecode.h's: 0 ok, -1 bad argument, -2 HIP error.
+// The device address of `device`'s copy of the scratch, looked up once (with that device current; the caller's current device is
+// put back). The lookup may load this file's code object onto the device, so it belongs outside stream capture: rd_device_open does it.
+static int scratch_base(int device, unsigned char **base, char *err, size_t err_len) {
+    std::lock_guard<std::mutex> lock(g_mu);
+    if (!g_scratch_ptr[device]) {
+        int prev = -1;
+        hipError_t e = hipGetDevice(&prev);
+        if (e != hipSuccess) return fail(err, err_len, -2, "hipGetDevice: %s", hipGetErrorString(e));
+        if (prev != device && (e = hipSetDevice(device)) != hipSuccess) return fail(err, err_len, -2, "hipSetDevice(%d): %s", device, hipGetErrorString(e));
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (prev != device) (void)hipSetDevice(prev);
+        if (e != hipSuccess || !p) return fail(err, err_len, -2, "hipGetSymbolAddress(scratch) on device %d: %s", device, hipGetErrorString(e));
+        g_scratch_ptr[device] = (unsigned char *)p;
+    }
+    *base = g_scratch_ptr[device];
+    return 0;
+}
+
+// Called by rd_device_open for the device it opens: the one-time lookup, done before anybody captures.
+extern "C" int rd_topk_static_prepare(int device, char *err, size_t err_len) {
+    if (device < 0 || device >= RD_STATIC_MAX_DEVICES) return fail(err, err_len, -1, "rd_topk_rows_static: device %d outside 0..%d", device, RD_STATIC_MAX_DEVICES - 1);
+    unsigned char *base;
+    return scratch_base(device, &base, err, err_len);
+}
+
+// Return codes are rocmdecode.h's: 0 ok, -1 bad argument, -2 HIP error. The caller's current device is the same on return.
 extern "C" int rd_topk_rows_static_impl(int device, void *stream_v, const float *logits, int rows, int V, int k, double temperature, int want_z, int *ids,
                                         float *vals, double *z, char *err, size_t err_len) {
     if (!logits || !ids || !vals || (want_z && !z)) return fail(err, err_len, -1, "rd_topk_rows_static: null pointer");
@@ -61,19 +88,14 @@ extern "C" int rd_topk_rows_static_impl(int device, void *stream_v, const float 
                     RD_STATIC_MAX_ROWS, RD_STATIC_MAX_V);
     if (k < 1 || k > RD_TOPK_MAX) return fail(err, err_len, -1, "rd_topk_rows_static: k=%d outside [1,%d]", k, RD_TOPK_MAX);
     if (k > V) k = V;
-    hipError_t e = hipSetDevice(device);
-    if (e != hipSuccess) return fail(err, err_len, -2, "hipSetDevice(%d): %s", device, hipGetErrorString(e));
     unsigned char *base;
-    {
-        std::lock_guard<std::mutex> lock(g_mu);
-        if (!g_scratch_ptr[device]) {
-            void *p = nullptr;
-            e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
-            if (e != hipSuccess || !p) return fail(err, err_len, -2, "hipGetSymbolAddress(scratch) on device %d: %s", device, hipGetErrorString(e));
-            g_scratch_ptr[device] = (unsigned char *)p;
-        }
-        base = g_scratch_ptr[device];
-    }
+    int rc = scratch_base(device, &base, err, err_len);
+    if (rc) return rc;
+    int prev = -1;
+    hipError_t e = hipGetDevice(&prev);
+    if (e != hipSuccess) return fail(err, err_len, -2, "hipGetDevice: %s", hipGetErrorString(e));
+    if (prev != device && (e = hipSetDevice(device)) != hipSuccess) return fail(err, err_len, -2, "hipSetDevice(%d): %s", device, hipGetErrorString(e));
+    (void)hipGetLastError(); // an error an earlier, unrelated call left behind is not this call's
     hipStream_t stream = (hipStream_t)stream_v;
     const float invT = temperature > 0 ? (float)(1.0 / temperature) : 1.f; // backend/cuda/topk.go:74-77
     double *zo = want_z ? z : nullptr;
@@ -93,6 +115,7 @@ extern "C" int rd_topk_rows_static_impl(int device, void *stream_v, const float 
                            (const int *)cand_i, ccount, (const double *)zpart, ids, vals, zo);
     }
     e = hipGetLastError();
+    if (prev != device) (void)hipSetDevice(prev);
     if (e != hipSuccess) return fail(err, err_len, -2, "rd_topk_rows_static: launch failed: %s", hipGetErrorString(e));
     return 0;
 }

@@ -262,10 +262,12 @@ int rd_topk_rows(rd_device *d, const float *logits, int rows, int V, int k, doub
  * hipMalloc). It has no counterpart in the reference. The same kernels and the same results, but nothing is allocated: the
  * scratch between the launches is a static 5.3 MB device array per GPU, and inputs and outputs are DEVICE pointers the caller
  * owns: logits_dev f32 [rows][V], ids_dev int32 and vals_dev f32 [rows][min(k,V)], z_dev f64 [rows] (may be NULL unless want_z).
- * The launches go to `stream` (a hipStream_t; NULL = the null stream) of GPU `device`, which the call makes current, and the
- * call returns without waiting for them. Limits: rows <= 32, V <= 262144, 1 <= k <= 1024; beyond them RD_ERR_ARG. Every call
- * on one GPU shares that GPU's scratch: calls that overlap on one GPU (two streams, two threads) race; calls in stream order
- * do not. Served by librocmdecode_static.so beside this library (opened on first use; RD_ERR_STATE if it is missing). */
+ * The launches go to `stream` (a hipStream_t; NULL = the null stream) of GPU `device` and the call returns without waiting for
+ * them; the caller's current device is the same on return. Limits: rows <= 32, V <= 262144, 1 <= k <= 1024; beyond them
+ * RD_ERR_ARG. Every call on one GPU shares that GPU's scratch: calls that overlap on one GPU (two streams, two threads) race;
+ * calls in stream order do not. Served by librocmdecode_static.so beside this library (RD_ERR_STATE if it is missing).
+ * Under stream capture: the one-time set-up for a GPU (opening that library, looking up the scratch's address there) happens in
+ * rd_device_open(device); a process that never opened the device makes one call outside capture first, which does the same. */
 int rd_topk_rows_static(int device, void *stream, const float *logits_dev, int rows, int V, int k, double temperature, int want_z, int *ids_dev,
                         float *vals_dev, double *z_dev);
 /* Decode chained on the device (decoder/resident/subsystems.go:78-100 GreedyChainStart / GreedyChainNext / GreedyChainStop and

@@ -99,3 +99,41 @@ def test_static_scratch_topk_rejects_what_exceeds_its_scratch():
     finally:
         hip.free_all()
         dev.close()
+
+
+def test_static_scratch_topk_under_stream_capture():
+    """What the entry point is for: captured on a caller-owned stream into a graph (the device was opened before, so nothing is left
+    to set up), replayed on fresh logits in the same buffers with ordinary work in between; every replay equals rd_topk_rows on the
+    same rows, bit for bit. An error left behind by an unrelated earlier call is not reported as this call's."""
+    dev = capi.Device(0)
+    hip = Hip()
+    L = hip.lib
+    try:
+        rows, V, k, T = 8, 151936, 256, 0.8
+        dl = hip.alloc(rows * V * 4)
+        di, dv, dz = hip.alloc(rows * k * 4), hip.alloc(rows * k * 4), hip.alloc(rows * 8)
+        stream, graph, gexec = C.c_void_p(), C.c_void_p(), C.c_void_p()
+        hip.check(L.hipStreamCreate(C.byref(stream)), "hipStreamCreate")
+        assert L.hipFree(C.c_void_p(16)) != 0  # leaves a sticky-until-read error behind
+        hip.check(L.hipStreamBeginCapture(stream, 1), "hipStreamBeginCapture")  # 1 = hipStreamCaptureModeThreadLocal
+        rc = capi.lib().rd_topk_rows_static(0, stream, dl, rows, V, k, C.c_double(T), 1, di, dv, dz)
+        end = L.hipStreamEndCapture(stream, C.byref(graph))
+        capi.check(rc, "rd_topk_rows_static under capture")
+        hip.check(end, "hipStreamEndCapture")
+        hip.check(L.hipGraphInstantiate(C.byref(gexec), graph, None, None, C.c_size_t(0)), "hipGraphInstantiate")
+        for rep in range(3):
+            x = bell_rows(rows, V, 100 + rep)
+            hip.check(L.hipMemcpy(dl, x.ctypes.data_as(C.c_void_p), C.c_size_t(x.nbytes), 1), "hipMemcpy H2D")
+            wi, wv, wz = dev.topk_rows(x, k, T)  # the program's own eager work between the replays
+            hip.check(L.hipGraphLaunch(gexec, stream), "hipGraphLaunch")
+            hip.check(L.hipStreamSynchronize(stream), "hipStreamSynchronize")
+            gi, gv, gz = hip.to_host(di, (rows, k), np.int32), hip.to_host(dv, (rows, k), np.float32), hip.to_host(dz, (rows,), np.float64)
+            assert np.array_equal(gi, wi), rep
+            assert np.array_equal(gv.view(np.uint32), wv.view(np.uint32)), rep
+            assert np.array_equal(gz, wz), rep
+        hip.check(L.hipGraphExecDestroy(gexec), "hipGraphExecDestroy")
+        hip.check(L.hipGraphDestroy(graph), "hipGraphDestroy")
+        hip.check(L.hipStreamDestroy(stream), "hipStreamDestroy")
+    finally:
+        hip.free_all()
+        dev.close()
