@@ -420,12 +420,16 @@ extern "C" int rd_model_set_window(rd_model *m, int layer, int window) {
         rd_set_error("model already finalized");
         return RD_ERR_STATE;
     }
+    // the model's window is what its layers hold now: a layer set back to 0 no longer counts
+    m->layers[(size_t)layer].window = 0;
+    m->window = 0;
+    for (const LayerW &l : m->layers) m->window = std::max(m->window, l.window);
     if (window > 0 && m->window > 0 && window != m->window) {
         rd_set_error("rocm resident declines: sliding-window layers of different lengths (%d and %d)", m->window, window);
         return RD_DECLINED;
     }
     m->layers[(size_t)layer].window = window;
-    if (window > 0) m->window = window;
+    m->window = std::max(m->window, window);
     return RD_OK;
 }
 
@@ -1006,9 +1010,14 @@ static int step_launches(rd_model *m, int B, int want) {
 static std::vector<long> step_graph_key(rd_model *m, int B, int want) {
     std::vector<long> k;
     if (m->timer.on || m->replay_B != 0 || m->bench_skip_attn) return k;
-    k = {B, want, m->step_draws ? 1 : 0, (long)m->last_items[0], (long)m->last_items[1], m->last_grouped[0] ? 1 : 0, m->last_grouped[1] ? 1 : 0,
-         getenv("ROCMDECODE_NO_FUSED_GATEUP") ? 1 : 0, getenv("ROCMDECODE_NO_FUSED_QKV") ? 1 : 0, getenv("ROCMDECODE_NO_FUSED_MOE_GATEUP") ? 1 : 0,
-         getenv("ROCMDECODE_MOE_TILES") ? atol(getenv("ROCMDECODE_MOE_TILES")) : 0};
+    k = {B, want, m->step_draws ? 1 : 0, (long)m->last_items[0], (long)m->last_items[1], m->last_grouped[0] ? 1 : 0, m->last_grouped[1] ? 1 : 0};
+    // every environment knob a launch consults, by value: a step after a change is launched (and captured) anew
+    for (const char *name : {"ROCMDECODE_NO_FUSED_GATEUP", "ROCMDECODE_NO_FUSED_QKV", "ROCMDECODE_NO_FUSED_MOE_GATEUP", "ROCMDECODE_MOE_TILES",
+                             "ROCMDECODE_GEMM8_KW", "ROCMDECODE_GEMM8_SPLITS", "ROCMDECODE_NO_DEEP_ATTN", "ROCMDECODE_NO_WIDE_ATTN",
+                             "ROCMDECODE_NO_ATTN_GROUPS", "ROCMDECODE_NO_ROWS_GEMM"}) {
+        const char *e = getenv(name);
+        k.push_back(e ? 1 + atol(e) : 0);
+    }
     return k;
 }
 
@@ -1033,8 +1042,10 @@ static int step_run(rd_model *m, int B, int want) {
         return step_launches(m, B, want);
     }
     if (m->graph.exec && key == m->graph.key) {
-        m->graph.replays++;
-        if (rd_hip_ok(hip, hip->GraphLaunch(m->graph.exec, d->stream), "hipGraphLaunch")) return RD_OK;
+        if (rd_hip_ok(hip, hip->GraphLaunch(m->graph.exec, d->stream), "hipGraphLaunch")) {
+            m->graph.replays++;
+            return RD_OK;
+        }
         m->graph.enabled = false; // nothing of this step has run: fall through to the eager launches
         step_graph_drop(m);
         return step_launches(m, B, want);

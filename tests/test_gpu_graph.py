@@ -131,3 +131,43 @@ def test_draw_steps_and_switching_the_graph_off(dev):
     finally:
         a.close()
         b.close()
+
+
+def test_a_changed_kernel_knob_is_never_served_by_an_older_graph(dev):
+    """The environment knobs that pick kernels (waves per GEMM tile, splits, attention kernel, fused epilogues) are part of what a
+    captured graph was recorded for: the step after a change is launched anew, not replayed, and equals the twin that never
+    uses a graph under the same knob; replays are counted only when the graph launch went through."""
+    import os
+    cfg = dense_cfg(n_layers=2, hidden=512, n_heads=4, n_kv=2, head_dim=128, inter=1024)
+    a, b = twins(cfg, 7, dev, slots=4, ctx_cap=64)
+    try:
+        rng = np.random.default_rng(3)
+        pos = 0
+
+        def step():
+            nonlocal pos
+            toks = rng.integers(0, cfg["vocab"], 4)
+            la = a.gpu.step_batch([0, 1, 2, 3], [pos] * 4, a.emb[toks])[0]
+            lb = b.gpu.step_batch([0, 1, 2, 3], [pos] * 4, b.emb[toks])[0]
+            pos += 1
+            assert same_bits(la, lb), pos
+
+        for _ in range(4):
+            step()
+        caps0, reps0 = a.gpu.graph_stats()
+        assert caps0 == 1 and reps0 == 2  # eager, captured (which runs the step), replayed, replayed
+        for knob, val in (("ROCMDECODE_GEMM8_KW", "2"), ("ROCMDECODE_GEMM8_SPLITS", "2"), ("ROCMDECODE_NO_DEEP_ATTN", "1"), ("ROCMDECODE_NO_ROWS_GEMM", "1")):
+            os.environ[knob] = val
+            try:
+                before = a.gpu.graph_stats()
+                step()  # a new key: launched eagerly
+                assert a.gpu.graph_stats() == before, knob
+                step()  # the second step under the knob is captured
+                step()
+                assert a.gpu.graph_stats() == (before[0] + 1, before[1] + 1), knob
+            finally:
+                del os.environ[knob]
+            step()  # and back: a new key again
+    finally:
+        a.close()
+        b.close()

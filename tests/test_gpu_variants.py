@@ -193,3 +193,22 @@ def test_granite_style_multipliers(dev):
     finally:
         a.close()
         b.close()
+
+
+def test_a_layer_set_back_to_no_window_no_longer_counts(dev):
+    """rd_model_set_window(layer, 0) takes the layer's window back: the model's window is what its layers hold, so another length
+    is then accepted, and two different lengths at once are still declined."""
+    cfg = dense_cfg(n_layers=3)
+    from tests.util import inv_freq
+    m = capi.Model(dev, cfg, inv_freq(cfg["head_dim"], cfg["theta"]))
+    try:
+        m.set_window(0, 16)
+        with pytest.raises(capi.RocmError, match="different lengths"):
+            m.set_window(1, 8)
+        m.set_window(0, 0)
+        m.set_window(1, 8)
+        m.set_window(2, 8)
+        with pytest.raises(capi.RocmError, match="different lengths"):
+            m.set_window(0, 16)
+    finally:
+        m.close()
