@@ -324,7 +324,7 @@ def run_c5(args):
     d2 = float(sum(len(set(idx2[:, l, :].ravel().tolist())) for l in range(layers)))
     g_ms = prof["moe_gemm_gateup"][0] / prof["moe_gemm_gateup"][1]
     per_launch = d2 * ebytes * (2.0 / 3.0) / layers
-    gu_kernel = "rd_k_moe_gemv_w4a8r" if row_act else "rd_k_moe_gemv_w4a8_gateup"
+    gu_kernel = "rd_k_moe_gemv_w4a8r_gateup" if row_act else "rd_k_moe_gemv_w4a8_gateup"
     traffic, t_ratio, t_src = counter_traffic("%s/%s" % (gu_kernel[5:], cfg["name"]), per_launch)
     act_txt = "int8 activations per token row" if row_act else "int8 activations per group of 32 (a variant of the configuration)"
     out = base_line("batch-16 decode tok/s, Qwen3-MoE-30B-A3B shape (int4-g32 experts); achieved HBM GB/s vs peak", tok_s, "tok/s", steps, warmup,
