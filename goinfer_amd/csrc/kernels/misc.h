@@ -204,28 +204,32 @@ __device__ __forceinline__ unsigned route_key(float v) {
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 // The routing of one token by one wave (see rd_k_moe_route); x: the token's nE logits (global or LDS). e64: 256 doubles of LDS.
+// NJ: experts per lane, nE <= 64 * NJ (the f64 exponentials are the wave's longest chain: a lane computes only those it holds).
+template <int NJ>
 __device__ __forceinline__ void moe_route_wave(const float *x, int t, int nE, int k, int norm, int *__restrict__ idx, float *__restrict__ wgt,
                                                signed char *__restrict__ rankOf, double *e64, int *__restrict__ idx_copy,
                                                unsigned *__restrict__ activeBits, const RouteOpts &ro) {
     const int lane = threadIdx.x & 63;
-    float xv[4], sc[4], sel[4];
+    float xv[NJ], sc[NJ], sel[NJ];
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
+    for (int j = 0; j < NJ; j++) {
         int i = lane + 64 * j;
         xv[j] = i < nE ? x[i] : -INFINITY;
     }
     if (ro.sigmoid) {
 #pragma unroll
-        for (int j = 0; j < 4; j++) sc[j] = (float)(1.0 / (1.0 + exp(-(double)xv[j])));
+        for (int j = 0; j < NJ; j++) sc[j] = (float)(1.0 / (1.0 + exp(-(double)xv[j])));
     } else {
-        float mx = fmaxf(fmaxf(xv[0], xv[1]), fmaxf(xv[2], xv[3]));
+        float mx = xv[0];
+#pragma unroll
+        for (int j = 1; j < NJ; j++) mx = fmaxf(mx, xv[j]);
         for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int j = 0; j < NJ; j++) {
             int i = lane + 64 * j;
             double e = i < nE ? exp((double)__fsub_rn(xv[j], mx)) : 0.0;
             sc[j] = (float)e;
-            e64[i] = e; // all 256 entries: zeros past nE, which leave the sum as it is
+            e64[i] = e; // all 64 * NJ entries: zeros past nE, which leave the sum as it is
         }
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0): this wave's LDS writes have landed before its lanes read them back
@@ -239,10 +243,10 @@ __device__ __forceinline__ void moe_route_wave(const float *x, int t, int nE, in
         }
         const float inv = (float)(1.0 / sum);
 #pragma unroll
-        for (int j = 0; j < 4; j++) sc[j] = mul_rounded(sc[j], inv); // rounded before a bias is added
+        for (int j = 0; j < NJ; j++) sc[j] = mul_rounded(sc[j], inv); // rounded before a bias is added
     }
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
+    for (int j = 0; j < NJ; j++) {
         int i = lane + 64 * j;
         sel[j] = i < nE ? (ro.bias ? __fadd_rn(sc[j], ro.bias[i]) : sc[j]) : -INFINITY;
         if (rankOf && i < nE) rankOf[(size_t)t * nE + i] = -1;
@@ -253,7 +257,7 @@ __device__ __forceinline__ void moe_route_wave(const float *x, int t, int nE, in
         const int gsz = nE / ro.nGroup;
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
-        for (int j = 0; j < 4; j++) selbuf[lane + 64 * j] = sel[j];
+        for (int j = 0; j < NJ; j++) selbuf[lane + 64 * j] = sel[j];
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_s_waitcnt(0xc07f);
         if (lane < ro.nGroup) {
@@ -281,7 +285,7 @@ __device__ __forceinline__ void moe_route_wave(const float *x, int t, int nE, in
             keep |= 1u << bg;
         }
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int j = 0; j < NJ; j++) {
             const int i = lane + 64 * j, g = i / gsz;
             if (g >= ro.nGroup || !((keep >> g) & 1u)) sel[j] = -INFINITY; // outside the kept groups, or past the last whole group
         }
@@ -294,7 +298,7 @@ __device__ __forceinline__ void moe_route_wave(const float *x, int t, int nE, in
         // over the wave: within rows of 16 lanes on the DPP path, across the rows by swizzle and one permute.
         unsigned kh = 0u, kl = 0u;
 #pragma unroll
-        for (int j = 3; j >= 0; j--) { // descending, '>=' on the key: the lowest index among this lane's equals survives
+        for (int j = NJ - 1; j >= 0; j--) { // descending, '>=' on the key: the lowest index among this lane's equals survives
             const unsigned kj = route_key(sel[j]);
             if (kj != 0u && kj >= kh) kh = kj, kl = ~(unsigned)(lane + 64 * j);
         }
@@ -311,10 +315,12 @@ __device__ __forceinline__ void moe_route_wave(const float *x, int t, int nE, in
         if (kh == 0u) break; // nothing left (k > the eligible experts)
         const int bi = (int)~kl, bj = bi >> 6;
         // the weight is the chosen expert's unbiased score, which its own lane holds
-        const float mineSc = bj == 0 ? sc[0] : (bj == 1 ? sc[1] : (bj == 2 ? sc[2] : sc[3]));
+        float mineSc = sc[0];
+#pragma unroll
+        for (int j = 1; j < NJ; j++) mineSc = bj == j ? sc[j] : mineSc;
         const float best = __shfl(mineSc, bi & 63, 64);
 #pragma unroll
-        for (int j = 0; j < 4; j++)
+        for (int j = 0; j < NJ; j++)
             if (bi == lane + 64 * j) {
                 sel[j] = -INFINITY; // used
                 if (rankOf) rankOf[(size_t)t * nE + bi] = (signed char)r;
@@ -346,7 +352,13 @@ extern "C" __global__ __launch_bounds__(64) void rd_k_moe_route(const float *__r
     const int t = blockIdx.x;
     if (t >= T) return;
     const RouteOpts ro{bias, sigmoid, scale, nGroup, topkGroup};
-    moe_route_wave(logits + (size_t)t * nE, t, nE, k, norm, idx, wgt, rankOf, e64, idx_copy, activeBits, ro);
+    const float *x = logits + (size_t)t * nE;
+    if (nE <= 64)
+        moe_route_wave<1>(x, t, nE, k, norm, idx, wgt, rankOf, e64, idx_copy, activeBits, ro);
+    else if (nE <= 128)
+        moe_route_wave<2>(x, t, nE, k, norm, idx, wgt, rankOf, e64, idx_copy, activeBits, ro);
+    else
+        moe_route_wave<4>(x, t, nE, k, norm, idx, wgt, rankOf, e64, idx_copy, activeBits, ro);
 }
 
 // Token embedding rows from an int8 table with one f32 scale per row (goinfer keeps the embedding table int8 in q4k mode,
