@@ -108,14 +108,12 @@ def test_c3_ragged_attention(dev, softcap):
     got = dev.attn_ragged(lens, k, v, q, nH, nKV, hd, scale, softcap)
     k16, v16 = ob.f16_round_trip(k), ob.f16_round_trip(v)
     off = np.concatenate([[0], np.cumsum(lens)])
-    # the oracle on every fourth sequence plus the shortest and the longest (f64 loops: the whole set would take minutes)
-    pick = sorted(set(range(0, nseq, 4)) | {int(np.argmin(lens)), int(np.argmax(lens))})
-    for i in pick:
+    for i in range(nseq):  # the oracle on every sequence of the call
         n = int(lens[i])
         want = ob.attend(q[i], k16[off[i]:off[i] + n], v16[off[i]:off[i] + n], n, nH, nKV, hd, scale, softcap)
         err = np.abs(got[i] - want).max() / np.abs(want).max()
         assert err <= 1e-4, (i, n, err)
-    # size-independent properties over all 64: a softmax-weighted mean of V lies inside V's range per dimension, and the
+    # size-independent properties as well: a softmax-weighted mean of V lies inside V's range per dimension, and the
     # result does not depend on which other sequences share the call
     for i in range(nseq):
         seg = v16[off[i]:off[i + 1]].reshape(-1, nKV, hd)

@@ -108,13 +108,15 @@ def test_model_with_window_and_sinks(dev):
 
 def test_moe_model_with_deepseek_style_router(dev):
     """Sigmoid scores, a selection bias per layer, group-limited selection (4 groups, the best 2), weights renormalized and scaled
-    by 2.5, through the step against the oracle; rows are compared while their routing agrees with the oracle's."""
-    cfg = dict(moe_cfg(n_layers=2, hidden=256, n_heads=4, n_kv=2, head_dim=64, n_experts=16, top_k=4, exp_inter=128),
+    by 2.5, through the step against the oracle on the oracle's replayed routing: every row of every step is held to the bar, none
+    excused; the GPU's own routing on its own hidden states is only counted."""
+    from tests.test_gpu_model import run_moe_replayed
+    cfg = dict(moe_cfg(n_layers=2, hidden=256, n_heads=4, n_kv=2, head_dim=64, n_experts=16, top_k=4, exp_inter=128, exp_act_group=0),
                router_sigmoid=1, router_bias=1, n_group=4, topk_group=2, router_scale=2.5)
     rng = np.random.default_rng(5)
-    _, _, (agree, total, diverged) = check(Pair(cfg, seed=41, dev=dev, slots=8), [list(rng.integers(0, 512, n)) for n in (2, 20)], steps=4)
+    worst, floor, agree, total = run_moe_replayed(Pair(cfg, seed=41, dev=dev, slots=8), [list(rng.integers(0, 512, n)) for n in (2, 20)], steps=4)
+    print("worst logit deviation %.4f, oracle noise floor %.4f, free-running expert index agreement %d/%d" % (worst, floor, agree, total))
     assert agree >= 0.9 * total, (agree, total)
-    assert not all(diverged)
 
 
 GEMMA2 = dict(window=24, post_norms=1, norm_add_one=1, act_gelu_tanh=1, final_softcap=30.0)
