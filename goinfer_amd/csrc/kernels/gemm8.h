@@ -128,24 +128,24 @@ struct Q4K8Traits {
 #pragma unroll
         for (int c = 0; c < 4; c++) w.q[c] = buf_load16_nt(r, off + lane * 16, 512 + c * 1024);
     }
-    // Lane (n, h) decodes the scales of sub-blocks 2p+h, p = 0..3: dsc = d * sc, ndm = -(dmin * m).
+    // Lane (n, h) decodes the scales of sub-blocks 2p+h, p = 0..3: dsc = d * sc, ndm = -(dmin * m). The 6-bit fields are cut out
+    // with the lane half folded into the bit offset (one v_bfe_u32 a field), not as both halves' values and a select.
     static __device__ __forceinline__ void decode(const Tile &w, int h, float (&dsc)[4], float (&ndm)[4]) {
         const uint32_t y = w.hdr.y, z = w.hdr.z, x = w.hdr.w, hx = w.hdr.x;
         half2_t dd;
         __builtin_memcpy(&dd, &hx, 4);
         const float d = (float)dd.x, dmin = (float)dd.y;
+        const uint32_t h8 = (uint32_t)h << 3;
 #pragma unroll
         for (int p = 0; p < 4; p++) {
-            int sc, mn;
-            if (p < 2) { // sub-blocks 0..3
-                const int j8 = 8 * (2 * p);
-                const int sc0 = (y >> j8) & 63, sc1 = (y >> (j8 + 8)) & 63, m0 = (z >> j8) & 63, m1 = (z >> (j8 + 8)) & 63;
-                sc = h ? sc1 : sc0, mn = h ? m1 : m0;
-            } else { // sub-blocks 4..7
-                const int j8 = 8 * (2 * p - 4);
-                const int sc0 = ((x >> j8) & 15) | (((y >> (j8 + 6)) & 3) << 4), sc1 = ((x >> (j8 + 8)) & 15) | (((y >> (j8 + 14)) & 3) << 4);
-                const int m0 = ((x >> (j8 + 4)) & 15) | (((z >> (j8 + 6)) & 3) << 4), m1 = ((x >> (j8 + 12)) & 15) | (((z >> (j8 + 14)) & 3) << 4);
-                sc = h ? sc1 : sc0, mn = h ? m1 : m0;
+            uint32_t sc, mn;
+            if (p < 2) { // sub-blocks 0..3: the low six bits of bytes 0..3 of the scale and the minimum word
+                const uint32_t j8 = 16u * p + h8;
+                sc = __builtin_amdgcn_ubfe(y, j8, 6u), mn = __builtin_amdgcn_ubfe(z, j8, 6u);
+            } else { // sub-blocks 4..7: a nibble of the third word and the top two bits of the matching byte
+                const uint32_t j8 = 16u * (p - 2) + h8;
+                sc = __builtin_amdgcn_ubfe(x, j8, 4u) | (__builtin_amdgcn_ubfe(y, j8 + 6u, 2u) << 4);
+                mn = __builtin_amdgcn_ubfe(x, j8 + 4u, 4u) | (__builtin_amdgcn_ubfe(z, j8 + 6u, 2u) << 4);
             }
             dsc[p] = __fmul_rn(d, (float)sc);
             ndm[p] = -__fmul_rn(dmin, (float)mn);
