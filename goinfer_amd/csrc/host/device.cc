@@ -483,7 +483,7 @@ int launch_gemm(rd_device *d, const DevWeight &w, const void *Xp, float *P, int 
     if (is_gemm8_kind(w.kind)) {
         const int tiles = w.N / 32, tpb = p.kw == 2 ? 2 : 1;
         // more than 32 rows of Q4_K: four M-tiles share each decoded weight tile (the same sums, row for row)
-        if (gemm8_lane(w) == 0 && M > 32 && rows_gemm_enabled()) {
+        if (gemm8_lane(w) == 0 && M >= ROWS_GEMM_MIN_ROWS && rows_gemm_enabled()) {
             const unsigned gz = (unsigned)((M + 127) / 128);
             const bool two = rows_gemm_two_groups((size_t)tiles * p.splits * gz);
             return d->launch(two ? d->k.gemm8_q4k_rows_g2 : d->k.gemm8_q4k_rows, (unsigned)tiles, (unsigned)p.splits, gz, two ? 512 : 256, (const void *)w.tiled, Xp,

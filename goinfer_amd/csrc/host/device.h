@@ -208,6 +208,9 @@ inline bool is_gemm8_kind(int kind) { return kind >= 0 && kind <= 4; } // every 
 constexpr int GEMM_WIDE_ROWS = 512;
 // the many-row Q4_K kernels: whether a grid of `blocks` blocks of four waves takes the second group of waves (under two waves per SIMD otherwise)
 bool rows_gemm_enabled();
+// rows from which a pass takes them: with one or two M-tiles half of a block's waves would idle, and the 32-row kernel over the
+// M-tiles is faster (9.3 against 7.9 ms a step at 64 rows of the Llama-3-8B shape; 14.0 against 14.7 at 128)
+constexpr int ROWS_GEMM_MIN_ROWS = 65;
 void topk_static_prepare_device(int ordinal); // ops.cc: opens the allocation-free top-K's library and looks its scratch up for this device
 inline bool rows_gemm_two_groups(size_t blocks) { return blocks < 2u * 256u; }
 int launch_gemm_wide(rd_device *d, const DevWeight &w, const void *Xp, size_t xpStride, float *P, size_t pStride, int M, GemmPlan *plan, int ldP = 0,

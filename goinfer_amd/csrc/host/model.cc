@@ -886,7 +886,7 @@ static int step_launches(rd_model *m, int B, int want) {
             Scope s(m, KC_GEMM_QKV); // projection, bias, RoPE and the KV store in one launch (M-tiles of 32 rows as grid.z)
             const DevWeight &w = l.qkv;
             const int nKB = kblocks_for(w), kw = plan_gemm(w.kind, w.N, nKB, w.act_group).kw; // the plain GEMM's waves per tile, in one split
-            if (gemm8_lane(w) == 0 && B > 32 && rows_gemm_enabled()) { // more than 32 rows: four M-tiles per decoded weight tile
+            if (gemm8_lane(w) == 0 && B >= ROWS_GEMM_MIN_ROWS && rows_gemm_enabled()) { // more than 32 rows: four M-tiles per decoded weight tile
                 const unsigned gz = (unsigned)((B + 127) / 128);
                 const bool two = rows_gemm_two_groups((size_t)(w.N / 32) * gz);
                 RC(d->launch(two ? d->k.gemm8_q4k_rows_qkv_g2 : d->k.gemm8_q4k_rows_qkv, (unsigned)(w.N / 32), 1, gz, two ? 512 : 256, (const void *)w.tiled,
@@ -944,7 +944,7 @@ static int step_launches(rd_model *m, int B, int want) {
             RC(add_norm_quant(m, B, m->P, plan.splits, l.ffn_norm, l.gateup, m->XpA, nullptr, nullptr, l.post_attn_norm));
             if (gateup_fusable(c, l.gateup) && !getenv("ROCMDECODE_NO_FUSED_GATEUP")) {
                 Scope s(m, KC_GEMM_GATEUP); // gate|up GEMM + SwiGLU + quantization in one launch (M-tiles of 32 rows as grid.z)
-                if (B > 32 && rows_gemm_enabled()) // more than 32 rows: four M-tiles per decoded weight tile
+                if (B >= ROWS_GEMM_MIN_ROWS && rows_gemm_enabled()) // more than 32 rows: four M-tiles per decoded weight tile
                     RC(d->launch(m->act == RD_ACT_GELU_TANH ? d->k.gemm8_q4k_rows_gateup_gelu : d->k.gemm8_q4k_rows_gateup, (unsigned)(c.inter / 32), 1,
                                  (unsigned)((B + 127) / 128), 256, (const void *)l.gateup.tiled, (const void *)m->XpA, m->XpB, c.inter, H / 256, B, m->xpAStride,
                                  m->xpBStride));

@@ -130,7 +130,7 @@ extern "C" int rd_gateup_q4k_quant(rd_device *d, const void *Wg, const void *Wu,
             RC(d->h2d(A.p, a + (size_t)m0 * K, sizeof(float) * (size_t)mc * K));
             for (int t = 0; t * 32 < mc; t++)
                 RC(quantize_rows(d, A.as<float>() + (size_t)t * 32 * K, std::min(32, mc - t * 32), K, PANEL_A8, 32, (char *)Xp.p + (size_t)t * xpStride));
-            if (mc > 32 && rows_gemm_enabled())
+            if (mc >= ROWS_GEMM_MIN_ROWS && rows_gemm_enabled())
                 RC(d->launch(d->k.gemm8_q4k_rows_gateup, (unsigned)(I / 32), 1, (unsigned)((mc + 127) / 128), 256, (const void *)w.tiled, (const void *)Xp.p,
                              X2.as<uint8_t>(), I, K / 256, mc, xpStride, x2Stride));
             else

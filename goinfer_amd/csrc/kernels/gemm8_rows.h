@@ -1,4 +1,5 @@
-// gemm8_rows.h — the Q4_K projections for passes of more than 32 rows (a prompt, or a ragged step with a prompt chunk riding):
+// gemm8_rows.h — the Q4_K projections for passes of more than two row tiles of 32 (65 to 512 rows: a prompt, a ragged step with a
+// prompt chunk riding, a wide decode batch):
 // goinfer's prompt-rate GEMM (backend/cuda/gemm_w4a8_mma.cu:57-188 keeps several row tiles of accumulators against one weight tile).
 //
 // A block owns one 32-row weight tile (and one K split) and four M-tiles of 32 batch rows, one per wave. Per super-block the four
@@ -109,7 +110,7 @@ __device__ __forceinline__ void rows_core(float16_t (&total)[NT], const uint8_t 
         rows_decode(bufs + ((s + 1) & 1) * RD_ROWS_BUF, plane, lane, h0, q0);
         h0 = h1, q0 = q1;
         raw_load(s + 3, h1, q1);
-        if (s < n) {
+        if (s < n && a8) { // (a wave whose M-tile lies past the pass's rows only decodes)
             const int kb = (NT > 1 && s >= nk) ? s - nk : s;
             rows_mma(cur, bufs + (s & 1) * RD_ROWS_BUF, lane, a);
             {
