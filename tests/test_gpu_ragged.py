@@ -58,7 +58,7 @@ def test_prefill_last_matches_token_by_token_and_oracle(dev):
     cfg = dense_cfg()
     pair = Pair(cfg, seed=52, dev=dev, slots=4, ctx_cap=256)
     rng = np.random.default_rng(6)
-    toks = list(rng.integers(0, cfg["vocab"], 97))  # four passes: 32 + 32 + 32 + 1
+    toks = list(rng.integers(0, cfg["vocab"], 97))  # one pass of 96 rows (three row tiles: the many-row kernels), then the last row alone
     got = pair.gpu.prefill_last(0, 0, pair.emb[toks])
     want = forward_tokens(pair, 1, toks)[-1]
     assert np.array_equal(bits(got), bits(want))
@@ -83,6 +83,38 @@ def test_prefill_last_matches_token_by_token_and_oracle(dev):
     ok, d = logits_close(g[0], o[0], max(floor, float(np.abs(o - o2).max())))
     assert ok, (d, floor)
     pair.close()
+
+
+VARIANTS = {
+    "wide": dense_cfg(n_layers=2, hidden=1024, n_heads=8, n_kv=2, head_dim=128, inter=2560),  # several K ranges a tile, head_dim 128
+    "qkv_bias": dict(dense_cfg(n_layers=2, hidden=512, n_heads=8, n_kv=2, head_dim=64, inter=1024, theta=1e6), qkv_bias=1),  # Qwen2: bias in the q|k|v epilogue
+    "geglu_post_norms": dict(dense_cfg(n_layers=2, hidden=512, n_heads=8, n_kv=2, head_dim=64, inter=1024, theta=1e4, eps=1e-6, softcap=50.0),
+                             window=24, post_norms=1, norm_add_one=1, act_gelu_tanh=1, final_softcap=30.0),  # Gemma 2's block
+}
+
+
+@pytest.mark.parametrize("variant", sorted(VARIANTS))
+@pytest.mark.parametrize("n", [70, 150, 300])
+def test_many_row_pass_equals_token_by_token(dev, variant, n):
+    """A prompt of 65 rows and more goes through the many-row projection kernels (plain, gate|up with SwiGLU or GeGLU, q|k|v with
+    bias and RoPE; one or two groups of waves by grid size): the last row's logits and the KV left behind are those of the
+    token-by-token path, bit for bit, whatever block variant rides on top."""
+    cfg = VARIANTS[variant]
+    pair = Pair(cfg, seed=58, dev=dev, slots=2, ctx_cap=n + 8)
+    try:
+        rng = np.random.default_rng(n)
+        toks = list(rng.integers(0, cfg["vocab"], n))
+        got = pair.gpu.prefill_last(0, 0, pair.emb[toks])
+        want = forward_tokens(pair, 1, toks)[-1]
+        assert np.array_equal(bits(got), bits(want))
+        for layer in range(cfg["n_layers"]):
+            ka, va = pair.gpu.kv_download(0, layer, 0, n)
+            kb, vb = pair.gpu.kv_download(1, layer, 0, n)
+            assert np.array_equal(bits(ka), bits(kb)) and np.array_equal(bits(va), bits(vb)), layer
+        nxt = pair.emb[int(rng.integers(0, cfg["vocab"]))]
+        assert np.array_equal(bits(pair.gpu.forward(0, n, nxt)), bits(pair.gpu.forward(1, n, nxt)))
+    finally:
+        pair.close()
 
 
 def test_ragged_refusals_write_nothing(dev):
