@@ -274,7 +274,7 @@ extern "C" __global__ __launch_bounds__(256) void rd_k_moe_gemv_w4a8(const uint8
     extern __shared__ __align__(16) uint8_t lds[];
     moe_gemv_body<false>(Wt, wStride, X, xStride, out, N, K, T, k, rankOf, nE, activeBits, lds);
 }
-// The same over rows that carry one activation scale each (ActQuantGroup 0: BASELINE's "int8 per-token activations").
+// The same over rows that carry one activation scale each (ActQuantGroup 0: the "int8 per-token activations" of the Qwen3-MoE benchmark configuration).
 extern "C" __global__ __launch_bounds__(256) void rd_k_moe_gemv_w4a8r(const uint8_t *__restrict__ Wt, size_t wStride, const uint8_t *__restrict__ X,
                                                                        size_t xStride, float *__restrict__ out, int N, int K, int T, int k,
                                                                        const signed char *__restrict__ rankOf, int nE,

@@ -246,7 +246,7 @@ def test_gemm_w8a8_per_row_bit_exact(dev, M, N, K):
 
 @pytest.mark.parametrize("M,N,K", [(1, 64, 128), (16, 768, 2048), (16, 2048, 768), (3, 64, 160), (40, 128, 4096)])
 def test_gemm_w4a8_per_row(dev, M, N, K):
-    """int4-g32 weights x per-row int8 activations (ActQuantGroup 0: BASELINE's "int8 per-token activations", the staged
+    """int4-g32 weights x per-row int8 activations (ActQuantGroup 0: the "int8 per-token activations" of the Qwen3-MoE benchmark configuration, the staged
     QuantBackend4.MatmulW4A8 hook and the experts' kernels): within 1e-5 of the f64 sum like every other lane (the reference's
     own kernel bar), the oracle too; a batched row is the row alone, bit for bit."""
     nib, s16 = synth.w4a8_normal(8, N, K)

@@ -236,7 +236,7 @@ def run_moe_replayed(pair, prompts, steps):
 
 @pytest.mark.parametrize("exp_act_group", [32, 0])
 def test_moe_ragged_batch(dev, exp_act_group):
-    """exp_act_group 32: expert activations quantized per group of 32; 0: one int8 scale per token row (BASELINE's expert lane)."""
+    """exp_act_group 32: expert activations quantized per group of 32; 0: one int8 scale per token row (the expert lane of the Qwen3-MoE benchmark configuration)."""
     rng = np.random.default_rng(4)
     worst, floor, agree, total = run_moe_replayed(Pair(moe_cfg(exp_act_group=exp_act_group), seed=5, dev=dev, slots=8),
                                                   [list(rng.integers(0, 512, n)) for n in (2, 33, 65)], steps=6)

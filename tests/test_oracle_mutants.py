@@ -6,8 +6,8 @@ Here the oracle is run against a deliberately wrong copy of itself (oracle.h OR_
 head reading its neighbour's kv head, a Q4_K sub-block scale taken from the neighbouring sub-block, the -dmin*m term dropped, the
 row not seeing its own key, the attention softcap dropped, an int4 group scale taken from the next group) on the same set-ups, with
 fewer rows so that it runs on a CPU in seconds, and the deviation is measured in bars. Every fault must land beyond one bar in every
-set-up the GPU tests use un-widened: then a GPU kernel with that fault fails there too. The measured factors are printed; DESIGN.md
-quotes them. The set-up with the late-layer residual stream (sigma 30) is the weakest by construction (the layer's own contribution
+set-up the GPU tests use un-widened: then a GPU kernel with that fault fails there too. The measured factors are printed.
+The set-up with the late-layer residual stream (sigma 30) is the weakest by construction (the layer's own contribution
 is a few per cent of the stream), which is why its numbers matter most."""
 import numpy as np
 import pytest
