@@ -161,7 +161,7 @@ def run_c4(args):
     chain_ms = float(np.mean([c[0] for c in chain]))
     # the kernel's average launch duration where it runs: whole steps against the same steps without their attention launches,
     # each step between its own pair of events. This is the figure the profiler's kernel duration agrees with.
-    avg_ms, _ = res.model.bench_attn_in_step(slots, pos_prof + 2, ids0, 8)
+    avg_ms, _ = res.model.bench_attn_in_step(slots, pos_prof + 2, ids0, 24)
     kernel_name = res.model.attn_kernel_name()  # the variant this work list takes (wide blocks, two units in flight, int8 cache)
     # per launch (one layer): every sequence's K and V rows once (f16, or int8 and their scales), plus q in and partial results out
     G = cfg["n_heads"] // cfg["n_kv"]
@@ -175,7 +175,7 @@ def run_c4(args):
                 "avg_launch_ms_event_pair_per_launch": round(single_ms, 5),
                 "avg_launch_ms_back_to_back": round(chain_ms, 5),
                 "timing": "HIP events on the launch stream around whole steps at the context lengths right after the timed ones: (a step - the same step "
-                          "without its attention launches) / layers, 8 pairs of steps; agrees with rocprofv3's kernel duration. The same kernel launched "
+                          "without its attention launches) / layers, the median of 24 pairs of steps; agrees with rocprofv3's kernel duration. The same kernel launched "
                           "back to back for all layers between one pair of events (its work list, tables and q then stay in L2) reads about 2 us less "
                           "(avg_launch_ms_back_to_back); an event pair around every single launch about 2 us more (avg_launch_ms_event_pair_per_launch)",
                 "algorithmic_bytes_per_launch": int(kv_launch + q_launch),

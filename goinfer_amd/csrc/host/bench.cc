@@ -149,18 +149,25 @@ extern "C" int rd_bench_attn_in_step(rd_model *m, int B, const int *slot, const 
         }
     m->bench_skip_attn = false;
     const int rc2 = d->sync();
-    double whole = 0, without = 0;
+    // the median over the pairs of (step - step without attention): a pair that caught a clock change or another process's burst
+    // does not move it
+    std::vector<double> diff((size_t)reps), whole((size_t)reps);
     for (int r = 0; r < reps; r++) {
         float a = 0.f, b = 0.f;
         if (!rc && !rc2) {
             (void)d->hip->EventElapsedTime(&a, ev[(size_t)r * 4], ev[(size_t)r * 4 + 1]);
             (void)d->hip->EventElapsedTime(&b, ev[(size_t)r * 4 + 2], ev[(size_t)r * 4 + 3]);
         }
-        whole += a, without += b;
+        diff[(size_t)r] = (double)a - (double)b, whole[(size_t)r] = a;
     }
     for (auto &e : ev) (void)d->hip->EventDestroy(e);
-    *ms_per_launch = (float)((whole - without) / reps / (double)m->layers.size());
-    if (ms_step) *ms_step = (float)(whole / reps);
+    auto median = [](std::vector<double> v) {
+        std::sort(v.begin(), v.end());
+        const size_t n = v.size();
+        return n % 2 ? v[n / 2] : 0.5 * (v[n / 2 - 1] + v[n / 2]);
+    };
+    *ms_per_launch = (float)(median(diff) / (double)m->layers.size());
+    if (ms_step) *ms_step = (float)median(whole);
     return rc ? rc : rc2;
 }
 

@@ -332,8 +332,8 @@ int rd_bench_steps(rd_model *m, int B, const int *slot, const int *pos0, const i
 /* One step with a HIP-event pair around every kernel class: class_ms[n] total milliseconds and class_n[n] launches,
  * n = rd_bench_class_count(); names from rd_bench_class_name. */
 int rd_bench_profile(rd_model *m, int B, const int *slot, const int *pos, const int *ids0, float *class_ms, int *class_n);
-/* The attention kernel's cost inside the step: (a whole step - the same step without its attention launches) / layers, over
- * `reps` pairs of steps at the same positions, each step between its own pair of events. Measurement only. */
+/* The attention kernel's cost inside the step: (a whole step - the same step without its attention launches) / layers, the median
+ * over `reps` pairs of steps at the same positions, each step between its own pair of events. Measurement only. */
 int rd_bench_attn_in_step(rd_model *m, int B, const int *slot, const int *pos, const int *ids0, int reps, float *ms_per_launch, float *ms_step);
 /* the name of the attention kernel the model's last step launched (measurement only) */
 const char *rd_bench_attn_kernel_name(rd_model *m);
