@@ -89,6 +89,10 @@ static const KName kNames[] = {
     {"rd_k_retile_w4a8_8", &Kernels::retile_w4a8_8},
     {"rd_k_gemm8_q4k_rows", &Kernels::gemm8_q4k_rows},
     {"rd_k_gemm8_q4k_rows_g2", &Kernels::gemm8_q4k_rows_g2},
+    {"rd_k_gemm8_q5k_rows", &Kernels::gemm8_q5k_rows},
+    {"rd_k_gemm8_q5k_rows_g2", &Kernels::gemm8_q5k_rows_g2},
+    {"rd_k_gemm8_q6k_rows", &Kernels::gemm8_q6k_rows},
+    {"rd_k_gemm8_q6k_rows_g2", &Kernels::gemm8_q6k_rows_g2},
     {"rd_k_gemm8_q4k_rows_gateup", &Kernels::gemm8_q4k_rows_gateup},
     {"rd_k_gemm8_q4k_rows_gateup_gelu", &Kernels::gemm8_q4k_rows_gateup_gelu},
     {"rd_k_gemm8_q4k_rows_qkv", &Kernels::gemm8_q4k_rows_qkv},
@@ -483,11 +487,14 @@ int launch_gemm(rd_device *d, const DevWeight &w, const void *Xp, float *P, int 
     if (is_gemm8_kind(w.kind)) {
         const int tiles = w.N / 32, tpb = p.kw == 2 ? 2 : 1;
         // more than 32 rows of Q4_K: four M-tiles share each decoded weight tile (the same sums, row for row)
-        if (gemm8_lane(w) == 0 && M >= ROWS_GEMM_MIN_ROWS && rows_gemm_enabled()) {
+        const int lane8 = gemm8_lane(w);
+        if ((lane8 == 0 || lane8 == 5 || lane8 == 6) && M >= ROWS_GEMM_MIN_ROWS && rows_gemm_enabled()) { // Q4_K, Q5_K, Q6_K
             const unsigned gz = (unsigned)((M + 127) / 128);
             const bool two = rows_gemm_two_groups((size_t)tiles * p.splits * gz);
-            return d->launch(two ? d->k.gemm8_q4k_rows_g2 : d->k.gemm8_q4k_rows, (unsigned)tiles, (unsigned)p.splits, gz, two ? 512 : 256, (const void *)w.tiled, Xp,
-                             P, w.N, nKB, p.kbPerSplit, p.kw, M, ldP, resid, xpStride, pStride);
+            hipFunction_t f = lane8 == 0 ? (two ? d->k.gemm8_q4k_rows_g2 : d->k.gemm8_q4k_rows)
+                                         : (lane8 == 5 ? (two ? d->k.gemm8_q5k_rows_g2 : d->k.gemm8_q5k_rows) : (two ? d->k.gemm8_q6k_rows_g2 : d->k.gemm8_q6k_rows));
+            return d->launch(f, (unsigned)tiles, (unsigned)p.splits, gz, two ? 512 : 256, (const void *)w.tiled, Xp, P, w.N, nKB, p.kbPerSplit, p.kw, M, ldP, resid,
+                             xpStride, pStride);
         }
         hipFunction_t f = d->k.gemm8[gemm8_lane(w)][p.kw == 8 ? 2 : (p.kw == 4 ? 1 : 0)];
         return d->launch(f, (unsigned)((tiles + tpb - 1) / tpb), (unsigned)p.splits, (unsigned)((M + 31) / 32), (unsigned)(64 * p.kw * tpb), (const void *)w.tiled,

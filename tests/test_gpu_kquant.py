@@ -75,6 +75,23 @@ def test_gemm(dev, fmt, M, N, K):
 
 
 @pytest.mark.parametrize("fmt", ["q5k", "q6k"])
+@pytest.mark.parametrize("M,N,K", [(70, 160, 2048), (300, 256, 14336), (512, 4096, 768), (129, 6144, 1024)])
+def test_gemm_many_rows_equal_the_32_row_kernel(dev, fmt, M, N, K):
+    """From 65 rows a pass runs the many-row kernel (four M-tiles against each tile decoded once; one or two groups of waves by the
+    size of the grid, one K range or several): every row is the row of the 32-row kernel, bit for bit, on random blocks (every code,
+    sign and scale value), and within 1e-5 of the f64 sum."""
+    raw = random_blocks(fmt, np.random.default_rng(7 + M), N * (K // 256))
+    a = synth.normal(32 + M, M * K).reshape(M, K)
+    wide = dev.gemm_kquant(fmt, raw, N, K, a)
+    for r0 in (0, 64, M - 32):
+        part = dev.gemm_kquant(fmt, raw, N, K, a[r0:r0 + 32])
+        assert np.array_equal(part.view(np.uint32), wide[r0:r0 + 32].view(np.uint32)), r0
+    rows = [0, 33, M - 1]
+    w = ob.WMat(FMT[fmt][1], N, K, raw, act_group=32)
+    assert rel_err(wide[rows], ob.matmul_f64ref(w, a[rows])) < 1e-5
+
+
+@pytest.mark.parametrize("fmt", ["q5k", "q6k"])
 def test_gemm_random_blocks(dev, fmt):
     """Every code, sign and scale value: random blocks rather than quantized normals."""
     N, K, M = 64, 512, 8
@@ -101,3 +118,22 @@ def test_model_mixed_kinds(dev, kinds):
     rng = np.random.default_rng(9)
     cfg = dense_cfg(n_layers=2, hidden=256, inter=512, vocab=512)
     check(Pair(cfg, seed=31, dev=dev, slots=8, kinds=kinds), [list(rng.integers(0, 512, n)) for n in (3, 40, 70)], steps=4)
+
+
+@pytest.mark.parametrize("kinds", [dict(v="q6k", down="q6k", head="q6k"), dict(q="q5k", k="q5k", v="q6k", up="q6k", o="q5k")], ids=["q4km", "q5km"])
+def test_mixed_kinds_prompt_pass_equals_token_by_token(dev, kinds):
+    """A 150-row prompt pass over a model whose projections mix Q4_K, Q5_K and Q6_K (each tensor through its own many-row kernel):
+    the last row's logits and the KV left behind are the token-by-token path's, bit for bit."""
+    cfg = dense_cfg(n_layers=2, hidden=512, n_heads=8, n_kv=2, head_dim=64, inter=1024, vocab=512)
+    pair = Pair(cfg, seed=33, dev=dev, slots=2, ctx_cap=160, kinds=kinds)
+    try:
+        toks = list(np.random.default_rng(3).integers(0, cfg["vocab"], 150))
+        got = pair.gpu.prefill_last(0, 0, pair.emb[toks])
+        want = np.stack([pair.gpu.forward(1, p, pair.emb[t]) for p, t in enumerate(toks)])[-1]
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+        for layer in range(cfg["n_layers"]):
+            ka, va = pair.gpu.kv_download(0, layer, 0, 150)
+            kb, vb = pair.gpu.kv_download(1, layer, 0, 150)
+            assert np.array_equal(ka.view(np.uint32), kb.view(np.uint32)) and np.array_equal(va.view(np.uint32), vb.view(np.uint32)), layer
+    finally:
+        pair.close()
