@@ -100,10 +100,11 @@ def parse_args():
     ap.add_argument("--exp-act-group", type=int, default=0, choices=[0, 32],
                     help="c5: the experts' activation quantization, 0 = one int8 scale per token row (the configuration as stated), 32 = per group of 32 (a variant)")
     ap.add_argument("--m", type=int, default=0, help="c2: only this batch width (for counter runs: one shape per kernel name)")
-    ap.add_argument("--workload", default="c4", choices=["c4", "c2", "c3", "c5", "kquant", "topk", "prefill"],
+    ap.add_argument("--workload", default="c4", choices=["c4", "c2", "c3", "c5", "kquant", "topk", "prefill", "issue"],
                     help="c4 (default): the Llama-3-8B-shape step the metric is quoted on; c2: Q4_K GEMM microbench; c3: ragged "
                          "attention microbench; c5: Qwen3-MoE-shape step; kquant: Q4_K / Q5_K / Q6_K GEMMs at the FFN and head shapes; topk: "
-                         "the device-side top-K of logits rows; prefill: a 2048-token prompt pass into the same paged KV")
+                         "the device-side top-K of logits rows; prefill: a 2048-token prompt pass into the same paged KV; issue: what a SIMD sustains "
+                         "of the int8 GEMMs' inner-loop instruction mix (no memory)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this backend is single-GPU (goinfer has no collective path); run with --gpus 1", file=sys.stderr)
@@ -242,4 +243,4 @@ if __name__ == "__main__":
         import bench_micro
         bench_micro.T0 = T0
         {"c2": bench_micro.run_c2, "c3": bench_micro.run_c3, "c5": bench_micro.run_c5, "kquant": bench_micro.run_kquant,
-         "topk": bench_micro.run_topk, "prefill": bench_micro.run_prefill}[_args.workload](_args)
+         "topk": bench_micro.run_topk, "prefill": bench_micro.run_prefill, "issue": bench_micro.run_issue}[_args.workload](_args)

@@ -213,6 +213,37 @@ def run_topk(args):
     emit(out)
 
 
+def run_issue(args):
+    """What one SIMD sustains of the int8 GEMMs' inner-loop instruction mix with no memory in the loop (rd_k_issue_*): the eight int8
+    MFMAs, the eight f32 MFMAs and the fold's 256 vector instructions of one (32 x 32 x 256) tile-block, each alone and all together,
+    at one and two waves a SIMD. `overlap` is the part of the shorter of (matrix core, vector ALU) that the mix hides:
+    0 = the times add, 1 = the shorter one is free. A step is one launch of `its` iterations on every SIMD."""
+    from goinfer_amd import capi
+    steps, warmup = (args.steps if args.steps != 128 else 7), (args.warmup if args.warmup != 8 else 2)
+    its = 20000
+    dev = capi.Device(0)
+    cases = []
+    for waves in (1, 2):
+        ns = {}
+        for mode, name in enumerate(("mfma_i8", "mfma_f32", "valu", "all")):
+            ms = dev.bench_kernel("issue", [mode, waves, its], warmup, steps)
+            ns[name] = float(np.median(ms)) * 1e6 / its / waves  # the SIMD's time per tile-block
+            log("%d wave(s) a SIMD, %s: %.1f ns per tile-block" % (waves, name, ns[name]))
+        mf = ns["mfma_i8"] + ns["mfma_f32"]
+        hidden = (mf + ns["valu"] - ns["all"]) / min(mf, ns["valu"])
+        cases.append({"waves_per_simd": waves, **{k + "_ns": round(v, 1) for k, v in ns.items()}, "sum_ns": round(mf + ns["valu"], 1), "overlap": round(hidden, 3)})
+    two = cases[-1]
+    tops = 2 * 8 * 32 * 32 * 32 / two["all_ns"] * 1024 / 1e3  # int8 multiply-adds x 2 of a tile-block, on 1024 SIMDs, TOP/s
+    out = base_line("int8 TOP/s of the Q4_K tile-block's instruction mix at two waves a SIMD, no memory in the loop", round(tops, 1), "TOP/s", steps, warmup,
+                    two["all_ns"] * its * 2 / 1e6, "issue-rate probe: 8 int8 MFMAs + 8 f32 MFMAs + 256 fold instructions a tile-block",
+                    "synthetic: registers only", {"cases": cases, "iterations": its}, dtype="i8")
+    out["roofline"] = {"bound": "mfma", "achieved": round(tops, 1), "peak": 5000.0, "unit": "TOP/s", "frac": round(tops / 5000.0, 4), "traffic": None,
+                       "kernel": "rd_k_issue_all", "avg_launch_ms": round(two["all_ns"] * its * 2 / 1e6, 4)}
+    out["cpu_baseline"] = None
+    dev.close()
+    emit(out)
+
+
 # ------------------------------------------------------------------------------------------------------------ C3
 def run_c3(args):
     """Ragged flash-decode attention: 64 sequences, KV lengths U[128,8192], 32 Q / 8 KV heads, head_dim 128, f16 KV; once without

@@ -237,6 +237,8 @@ extern "C" const char *rd_bench_class_name(int c) {
 //   "gateup"    args {I, K, M, copies}: the fused gate|up projection + SwiGLU + quantization kernel.
 //   "copy"      args {bytes}: a plain 16-byte-per-lane copy kernel over `bytes` (a multiple of 16), the yardstick for
 //               scaling hardware traffic counters and for the practical HBM rate.
+//   "issue"     args {mode, waves, iterations[, compute units = 256]}: the issue-rate probes (rd_k_issue_*: mode 0 int8 MFMAs, 1 f32 MFMAs, 2 the fold's
+//               vector instructions, 3 all of them) with `waves` (1..2) waves on every SIMD; no memory traffic in the loop.
 // ms_out[iters]: per-launch milliseconds (HIP events on the launch stream).
 extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *args, int n_args, int warmup, int iters, float *ms_out) {
     if (!d || !name || !args || iters <= 0 || !ms_out) return RD_ERR_ARG;
@@ -339,6 +341,24 @@ extern "C" int rd_bench_kernel(rd_device *d, const char *name, const int64_t *ar
         for (int i = 0; i < warmup + iters && !rc; i++) {
             if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup)], d->stream);
             rc = d->launch(d->k.copy16, 4096, 1, 1, 256, (const void *)A.p, Bf.p, (size_t)(bytes / 16));
+            if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup) + 1], d->stream);
+        }
+        if (!rc) rc = d->sync();
+    } else if (nm == "issue" && n_args >= 3) {
+        const int mode = (int)args[0], waves = (int)args[1], its = (int)args[2];
+        const int cus = n_args >= 4 ? (int)args[3] : 256; // the MI355X's compute units
+        if (mode < 0 || mode > 3 || waves < 1 || waves > 2 || its < 1 || its > 1000000 || cus < 1 || cus > 1024) {
+            rd_set_error("issue bench: mode 0..3, waves 1..2, iterations 1..1000000, compute units 1..1024");
+            rc = RD_ERR_ARG;
+        }
+        DevBuf In(d), Out(d);
+        if (!rc) rc = In.alloc(4096);
+        if (!rc) rc = Out.alloc(sizeof(float) * 256 * (size_t)cus * waves);
+        if (!rc) rc = d->launch(d->k.fill_f32, 4, 1, 1, 256, In.as<float>(), (size_t)1024, 3u); // any bits do: the loop reads them as ints
+        const hipFunction_t f = mode == 0 ? d->k.issue_mfma_i8 : (mode == 1 ? d->k.issue_mfma_f32 : (mode == 2 ? d->k.issue_valu : d->k.issue_all));
+        for (int i = 0; i < warmup + iters && !rc; i++) {
+            if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup)], d->stream);
+            rc = d->launch(f, (unsigned)(cus * waves), 1, 1, 256, its, (const int *)In.p, Out.as<float>());
             if (i >= warmup) (void)d->hip->EventRecord(ev[2 * (size_t)(i - warmup) + 1], d->stream);
         }
         if (!rc) rc = d->sync();

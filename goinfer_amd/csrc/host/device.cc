@@ -139,6 +139,10 @@ static const KName kNames[] = {
     {"rd_k_copy16", &Kernels::copy16},
     {"rd_k_fill_f16", &Kernels::fill_f16},
     {"rd_k_fill_f32", &Kernels::fill_f32},
+    {"rd_k_issue_mfma_i8", &Kernels::issue_mfma_i8},
+    {"rd_k_issue_mfma_f32", &Kernels::issue_mfma_f32},
+    {"rd_k_issue_valu", &Kernels::issue_valu},
+    {"rd_k_issue_all", &Kernels::issue_all},
 };
 
 static int open_common(int ordinal, const void *image, rd_device **out) {

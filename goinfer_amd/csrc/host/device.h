@@ -45,7 +45,7 @@ struct Kernels {
     hipFunction_t dequant_q5k, retile_q5k, dequant_q6k, retile_q6k;
     hipFunction_t kv_store, kv_read, qkv_rope_store, attn_partial, attn_partial_wide, attn_combine, attn_combine_quant;
     hipFunction_t kv_store_i8, qkv_rope_store_i8, attn_partial_i8, attn_partial_rows, attn_partial_rows_i8, attn_partial_deep, attn_partial_deep_i8, topk_rows, topk_hist, topk_pick, topk_finish;
-    hipFunction_t rmsnorm, rope, argmax_rows, argmax_final, matmul_f32, moe_route, moe_swiglu_quant, moe_swiglu_quant_row, moe_fold, embed_rows, copy16, fill_f16, fill_f32;
+    hipFunction_t rmsnorm, rope, argmax_rows, argmax_final, matmul_f32, moe_route, moe_swiglu_quant, moe_swiglu_quant_row, moe_fold, embed_rows, copy16, fill_f16, fill_f32, issue_mfma_i8, issue_mfma_f32, issue_valu, issue_all;
 };
 
 struct rd_device {

@@ -375,6 +375,63 @@ extern "C" __global__ void rd_k_copy16(const uint4 *__restrict__ src, uint4 *__r
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x) dst[i] = src[i];
 }
 
+// Issue-rate probes: what one SIMD sustains of the instruction mix of the int8 GEMMs' inner loop, with no memory in the loop. One
+// iteration is one (32 x 32 outputs, 256 deep) tile-block's worth: MODE 0 its eight int8 MFMAs, 1 its eight f32 MFMAs (four
+// 32x32x1 two-block scale products, four 32x32x2 minimum terms), 2 the fold's 256 vector instructions (128 converts, 128 fmas),
+// 3 all of them, none depending on another's result. Launched with (compute units x w) blocks of four waves, every SIMD holds w
+// waves; time per launch / iterations / w is the SIMD's time per tile-block. in: 1024 ints; out: one float per thread.
+typedef int rd_i32x4_t __attribute__((ext_vector_type(4)));
+typedef int rd_i32x16_t __attribute__((ext_vector_type(16)));
+typedef float rd_f32x32_t __attribute__((ext_vector_type(32)));
+template <int MODE> __device__ __forceinline__ void issue_probe(int iters, const int *__restrict__ in, float *__restrict__ out) {
+    const int lane = threadIdx.x & 63;
+    const rd_i32x4_t a = {in[lane], in[lane + 64], in[lane + 128], in[lane + 192]};
+    const rd_i32x4_t b = {in[lane + 1], in[lane + 65], in[lane + 129], in[lane + 193]};
+    const float sa = (float)in[lane + 2] * 1e-3f, sb = (float)in[lane + 3] * 1e-3f;
+    float16_t acc = {0.f}, facc = {0.f};
+    rd_i32x16_t d0 = {0}, d1 = {0}, p0, p1;
+    rd_f32x32_t s2 = {0.f}, ps;
+    for (int j = 0; j < 16; j++) p0[j] = in[lane + j], p1[j] = in[lane + j + 7];
+    for (int j = 0; j < 32; j++) ps[j] = (float)in[lane + j] * 1e-4f;
+    for (int it = 0; it < iters; it++) {
+        if (MODE == 0 || MODE == 3) {
+#pragma unroll
+            for (int p = 0; p < 4; p++) {
+                d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, d0, 0, 0, 0);
+                d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(b, a, d1, 0, 0, 0);
+            }
+        }
+        if (MODE == 1 || MODE == 3) {
+#pragma unroll
+            for (int p = 0; p < 4; p++) s2 = __builtin_amdgcn_mfma_f32_32x32x1f32(sa, sb, s2, 0, 0, 0);
+#pragma unroll
+            for (int p = 0; p < 4; p++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(sa, sb, acc, 0, 0, 0);
+        }
+        if (MODE == 2 || MODE == 3) {
+#pragma unroll
+            for (int p = 0; p < 4; p++) {
+#pragma unroll
+                for (int j = 0; j < 16; j++) {
+                    asm volatile("" : "+v"(p0[j])); // the compiler may not hoist the convert out of the loop
+                    facc[j] = __builtin_fmaf((float)p0[j], ps[j], facc[j]);
+                }
+#pragma unroll
+                for (int j = 0; j < 16; j++) {
+                    asm volatile("" : "+v"(p1[j]));
+                    facc[j] = __builtin_fmaf((float)p1[j], ps[16 + j], facc[j]);
+                }
+            }
+        }
+    }
+    float s = 0.f;
+    for (int j = 0; j < 16; j++) s += acc[j] + facc[j] + (float)d0[j] + (float)d1[j] + s2[j] + s2[j + 16];
+    out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+extern "C" __global__ __launch_bounds__(256) void rd_k_issue_mfma_i8(int iters, const int *in, float *out) { issue_probe<0>(iters, in, out); }
+extern "C" __global__ __launch_bounds__(256) void rd_k_issue_mfma_f32(int iters, const int *in, float *out) { issue_probe<1>(iters, in, out); }
+extern "C" __global__ __launch_bounds__(256) void rd_k_issue_valu(int iters, const int *in, float *out) { issue_probe<2>(iters, in, out); }
+extern "C" __global__ __launch_bounds__(256) void rd_k_issue_all(int iters, const int *in, float *out) { issue_probe<3>(iters, in, out); }
+
 // Synthetic operand fills for the micro-benchmarks: element i = uniform in [-2, 2) from a counter hash of (seed, i).
 __device__ __forceinline__ float fill_value(size_t i, unsigned seed) {
     unsigned long long z = (unsigned long long)i * 0x9E3779B97F4A7C15ull + (unsigned long long)seed * 0xBF58476D1CE4E5B9ull;
