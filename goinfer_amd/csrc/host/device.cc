@@ -99,6 +99,8 @@ static const KName kNames[] = {
     {"rd_k_gemm8_q4k_rows_qkv_g2", &Kernels::gemm8_q4k_rows_qkv_g2},
     {"rd_k_gemm8_q4k_gateup", &Kernels::gemm8_q4k_gateup},
     {"rd_k_gemm8_q4k_gateup_gelu", &Kernels::gemm8_q4k_gateup_gelu},
+    {"rd_k_gemm8_q4k_gateup_norm1", &Kernels::gemm8_q4k_gateup_norm1},
+    {"rd_k_gemm8_q4k_gateup_gelu_norm1", &Kernels::gemm8_q4k_gateup_gelu_norm1},
     {"rd_k_add_one", &Kernels::add_one},
     {"rd_k_moe_gemv_w4a8", &Kernels::moe_gemv_w4a8},
     {"rd_k_moe_gemv_w4a8_gateup", &Kernels::moe_gemv_w4a8_gateup},
@@ -194,6 +196,17 @@ static int open_common(int ordinal, const void *image, rd_device **out) {
                 return RD_ERR_HIP;
             }
         }
+    for (int i = 0; i < 3; i++) {
+        char name[64];
+        snprintf(name, sizeof name, "rd_k_gemm8_q4k_qkv_norm1_kw%d", 2 << i);
+        if (hip->ModuleGetFunction(&d->k.gemm8_q4k_qkv_norm1[i], d->module, name) != hipSuccess) {
+            rd_set_error("code object lacks kernel %s", name);
+            (void)hip->ModuleUnload(d->module);
+            (void)hip->StreamDestroy(d->stream);
+            delete d;
+            return RD_ERR_HIP;
+        }
+    }
     topk_static_prepare_device(ordinal); // the allocation-free top-K's one-time set-up for this device, outside any capture
     *out = d;
     return RD_OK;

@@ -41,6 +41,7 @@ struct Kernels {
     // ranges, for grids of few weight tiles)
     hipFunction_t gemm8_q4k_rows, gemm8_q4k_rows_g2, gemm8_q4k_rows_gateup, gemm8_q4k_rows_gateup_gelu, gemm8_q4k_rows_qkv, gemm8_q4k_rows_qkv_g2;
     hipFunction_t gemm8_q5k_rows, gemm8_q5k_rows_g2, gemm8_q6k_rows, gemm8_q6k_rows_g2; // the plain many-row kernel over Q5_K / Q6_K tiles
+    hipFunction_t gemm8_q4k_gateup_norm1, gemm8_q4k_gateup_gelu_norm1, gemm8_q4k_qkv_norm1[3]; // a one-row step's projections with the norm folded in
     hipFunction_t gemm8_q4k_gateup, gemm8_q4k_gateup_gelu, add_one, moe_gemv_w4a8, moe_gemv_w4a8r, moe_gemv_w4a8r_f32in, moe_gemv_w4a8_gateup, moe_gemv_w4a8r_gateup, retile_w4a8_gv, rope_table;
     hipFunction_t dequant_q5k, retile_q5k, dequant_q6k, retile_q6k;
     hipFunction_t kv_store, kv_read, qkv_rope_store, attn_partial, attn_partial_wide, attn_combine, attn_combine_quant;

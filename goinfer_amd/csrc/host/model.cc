@@ -75,7 +75,7 @@ extern "C" void rd_model_destroy(rd_model *m) {
             d->release(p);
     }
     free_weight(d, &m->head);
-    for (void *p : {(void *)m->embed_q, (void *)m->embed_scale, (void *)m->inv_freq_dev, (void *)m->rope_cs, (void *)m->final_norm, (void *)m->tables, (void *)m->h, (void *)m->normed, (void *)m->P, (void *)m->qbuf,
+    for (void *p : {(void *)m->embed_q, (void *)m->embed_scale, (void *)m->inv_freq_dev, (void *)m->rope_cs, (void *)m->final_norm, (void *)m->tables, (void *)m->h, (void *)m->h2, (void *)m->normed, (void *)m->P, (void *)m->qbuf,
                     (void *)m->part, (void *)m->attn_out, (void *)m->cand_v, (void *)m->cand_i, (void *)m->logits, (void *)m->emb_dev, m->XpA, m->XpB, (void *)m->ids, (void *)m->meta, (void *)m->router_logits, (void *)m->moe_wgt, (void *)m->moe_gu,
                     (void *)m->moe_dn, (void *)m->moe_out, (void *)m->moe_idx, (void *)m->moe_idx_all, (void *)m->moe_rank, (void *)m->topk_ids, (void *)m->topk_vals, (void *)m->topk_z, (void *)m->topk_scratch.ghist, (void *)m->topk_scratch.ccount, (void *)m->topk_scratch.gmax, (void *)m->topk_scratch.cand_i, (void *)m->topk_scratch.cand_v, (void *)m->topk_scratch.invT, (void *)m->topk_scratch.zpart, m->XpE, (void *)m->XEf, (void *)m->moe_rowmax})
         d->release(p);
@@ -499,6 +499,7 @@ extern "C" int rd_model_finalize(rd_model *m) {
     m->pStride = pf;
     RC(alloc_f32(d, &m->P, pf * tiles));
     RC(alloc_f32(d, &m->h, R * H));
+    RC(alloc_f32(d, &m->h2, (size_t)H));
     RC(alloc_f32(d, &m->emb_dev, R * H));
     RC(alloc_f32(d, &m->normed, (size_t)32 * H));
     RC(alloc_f32(d, &m->qbuf, R * qd));
@@ -729,11 +730,11 @@ static int build_attn_items(rd_model *m, int B, const int *slot, const int *pos,
 
 // foldW: P holds an MoE layer's down-projection rows and foldW their weights (see the kernel); else split-K partial sums.
 // postW: the norm of the pending contribution itself (Gemma 2's post-attention / post-feed-forward norm), or null.
-static int add_norm_quant(rd_model *m, int B, const float *P, int splits, const float *w, const DevWeight &next, void *Xp, float *norm_out,
+static int add_norm_quant(rd_model *m, float *h, int B, const float *P, int splits, const float *w, const DevWeight &next, void *Xp, float *norm_out,
                           const float *foldW = nullptr, const float *postW = nullptr) {
     rd_device *d = m->d;
     Scope s(m, KC_ADD_NORM);
-    return d->launch(d->k.add_rmsnorm_quant, (unsigned)B, 1, 1, 1024, m->h, P, splits, w, m->desc.rms_eps, m->desc.hidden, Xp, (int)PANEL_A8, norm_out,
+    return d->launch(d->k.add_rmsnorm_quant, (unsigned)B, 1, 1, 1024, h, P, splits, w, m->desc.rms_eps, m->desc.hidden, Xp, (int)PANEL_A8, norm_out,
                      m->pStride, m->xpAStride, foldW, P ? postW : (const float *)nullptr, act_group_for(next));
 }
 
@@ -863,6 +864,14 @@ int launch_attn_partial(rd_model *m, const LayerW &l) {
                      nH, nKV, HD, c.attn_scale, c.attn_softcap, l.window);
 }
 
+// A step of one row folds its norm-and-quantize launches into the projections that consume them (rd_k_gemm8_q4k_*_norm1: every
+// block forms the 16 KB row itself; the same bits, one launch less): where the pending contribution is plain split-K partials
+// (or none), the projection is one Q4_K weight quantized per group of 32, and the row fits the kernels' LDS image.
+static bool norm1_fusable(const rd_model *m, int B, const DevWeight &next, const float *foldW, const float *postW) {
+    const int H = m->desc.hidden;
+    return B == 1 && !foldW && !postW && next.kind == 0 && act_group_for(next) == 32 && H % 256 == 0 && H <= 4096 && !getenv("ROCMDECODE_NO_FUSED_NORM");
+}
+
 // Every launch of a step between the uploads (metadata, embeddings) and the copies back: the layers, the final norm, the head,
 // the argmax. What it launches depends on the model, B, `want`, and the state step_graph_key() lists, and on nothing else: the
 // per-step data (positions, tables, work lists, draw records) is read from device memory the uploads have already filled.
@@ -878,11 +887,23 @@ static int step_launches(rd_model *m, int B, int want) {
         Scope s(m, KC_ROPE_STORE);
         RC(d->launch(d->k.rope_table, (unsigned)B, 1, 1, (unsigned)(HD / 2), (const int *)m->rowPos, (const double *)m->inv_freq_dev, m->rope_cs, HD / 2));
     }
+    float *h = m->h; // the residual rows; a one-row step alternates between m->h and m->h2 (see norm1_fusable)
+    auto other = [&](float *p) { return p == m->h ? m->h2 : m->h; };
     for (int li = 0; li < c.n_layers; li++) {
         LayerW &l = m->layers[(size_t)li];
         GemmPlan plan;
-        RC(add_norm_quant(m, B, resP, resSplits, l.attn_norm, l.qkv, m->XpA, nullptr, resW, resPost));
-        if (qkv_fusable(m, l)) {
+        const bool qkvNorm1 = qkv_fusable(m, l) && gemm8_lane(l.qkv) == 0 && norm1_fusable(m, B, l.qkv, resW, resPost);
+        if (!qkvNorm1) RC(add_norm_quant(m, h, B, resP, resSplits, l.attn_norm, l.qkv, m->XpA, nullptr, resW, resPost));
+        if (qkvNorm1) {
+            Scope s(m, KC_GEMM_QKV); // one row: norm, quantization, projection, bias, RoPE and the KV store in one launch
+            const DevWeight &w = l.qkv;
+            const int nKB = kblocks_for(w), kw = plan_gemm(w.kind, w.N, nKB, w.act_group).kw;
+            RC(d->launch(d->k.gemm8_q4k_qkv_norm1[kw == 8 ? 2 : (kw == 4 ? 1 : 0)], (unsigned)(w.N / 32), 1, 1, (unsigned)(64 * kw), (const void *)w.tiled,
+                         (const void *)w.scales, w.N, nKB, m->qbuf, l.Kp, l.Vp, (const int *)m->tables, m->blocks_per_slot, (const int *)m->rowSlot,
+                         (const int *)m->rowPos, (const double *)m->rope_cs, (const float *)l.qkv_bias, nH, nKV, HD, (const float *)h, other(h), resP, resSplits,
+                         (const float *)l.attn_norm, c.rms_eps, H));
+            h = other(h);
+        } else if (qkv_fusable(m, l)) {
             Scope s(m, KC_GEMM_QKV); // projection, bias, RoPE and the KV store in one launch (M-tiles of 32 rows as grid.z)
             const DevWeight &w = l.qkv;
             const int nKB = kblocks_for(w), kw = plan_gemm(w.kind, w.N, nKB, w.act_group).kw; // the plain GEMM's waves per tile, in one split
@@ -941,8 +962,16 @@ static int step_launches(rd_model *m, int B, int want) {
             RC(launch_gemm_wide(d, l.o, m->XpB, m->xpBStride, m->P, m->pStride, B, &plan));
         }
         if (c.n_experts == 0) {
-            RC(add_norm_quant(m, B, m->P, plan.splits, l.ffn_norm, l.gateup, m->XpA, nullptr, nullptr, l.post_attn_norm));
-            if (gateup_fusable(c, l.gateup) && !getenv("ROCMDECODE_NO_FUSED_GATEUP")) {
+            const bool guFused = gateup_fusable(c, l.gateup) && !getenv("ROCMDECODE_NO_FUSED_GATEUP");
+            const bool guNorm1 = guFused && norm1_fusable(m, B, l.gateup, nullptr, l.post_attn_norm);
+            if (!guNorm1) RC(add_norm_quant(m, h, B, m->P, plan.splits, l.ffn_norm, l.gateup, m->XpA, nullptr, nullptr, l.post_attn_norm));
+            if (guNorm1) {
+                Scope s(m, KC_GEMM_GATEUP); // one row: norm, quantization, gate|up, SwiGLU and the down projection's quantization in one launch
+                RC(d->launch(m->act == RD_ACT_GELU_TANH ? d->k.gemm8_q4k_gateup_gelu_norm1 : d->k.gemm8_q4k_gateup_norm1, (unsigned)(c.inter / 32), 1, 1,
+                             GATEUP_THREADS, (const void *)l.gateup.tiled, m->XpB, panel_kind_for(l.down), c.inter, H / 256, (const float *)h, other(h),
+                             (const float *)m->P, plan.splits, (const float *)l.ffn_norm, c.rms_eps, H));
+                h = other(h);
+            } else if (guFused) {
                 Scope s(m, KC_GEMM_GATEUP); // gate|up GEMM + SwiGLU + quantization in one launch (M-tiles of 32 rows as grid.z)
                 if (B >= ROWS_GEMM_MIN_ROWS && rows_gemm_enabled()) // more than 32 rows: four M-tiles per decoded weight tile
                     RC(d->launch(m->act == RD_ACT_GELU_TANH ? d->k.gemm8_q4k_rows_gateup_gelu : d->k.gemm8_q4k_rows_gateup, (unsigned)(c.inter / 32), 1,
@@ -975,7 +1004,7 @@ static int step_launches(rd_model *m, int B, int want) {
         } else {
             {
                 Scope s(m, KC_ADD_NORM);
-                RC(d->launch(d->k.add_rmsnorm_quant, (unsigned)B, 1, 1, 1024, m->h, (const float *)m->P, plan.splits, (const float *)l.ffn_norm,
+                RC(d->launch(d->k.add_rmsnorm_quant, (unsigned)B, 1, 1, 1024, h, (const float *)m->P, plan.splits, (const float *)l.ffn_norm,
                              c.rms_eps, H, m->XpA, (int)PANEL_ROW8, m->normed, m->pStride, m->xpAStride, (const float *)nullptr,
                              (const float *)nullptr, m->exp_act_group == 0 ? 0 : 32));
             }
@@ -988,7 +1017,7 @@ static int step_launches(rd_model *m, int B, int want) {
     }
     if (want & (RD_WANT_LOGITS | RD_WANT_ARGMAX)) {
         GemmPlan plan;
-        RC(add_norm_quant(m, B, resP, resSplits, m->final_norm, m->head, m->XpA, nullptr, resW, resPost));
+        RC(add_norm_quant(m, h, B, resP, resSplits, m->final_norm, m->head, m->XpA, nullptr, resW, resPost));
         {
             Scope s(m, KC_GEMM_HEAD);
             RC(launch_gemm_wide(d, m->head, m->XpA, m->xpAStride, m->P, m->pStride, B, &plan));
@@ -1014,7 +1043,7 @@ static std::vector<long> step_graph_key(rd_model *m, int B, int want) {
     // every environment knob a launch consults, by value: a step after a change is launched (and captured) anew
     for (const char *name : {"ROCMDECODE_NO_FUSED_GATEUP", "ROCMDECODE_NO_FUSED_QKV", "ROCMDECODE_NO_FUSED_MOE_GATEUP", "ROCMDECODE_MOE_TILES",
                              "ROCMDECODE_GEMM8_KW", "ROCMDECODE_GEMM8_SPLITS", "ROCMDECODE_NO_DEEP_ATTN", "ROCMDECODE_NO_WIDE_ATTN",
-                             "ROCMDECODE_NO_ATTN_GROUPS", "ROCMDECODE_NO_ROWS_GEMM"}) {
+                             "ROCMDECODE_NO_ATTN_GROUPS", "ROCMDECODE_NO_ROWS_GEMM", "ROCMDECODE_NO_FUSED_NORM"}) {
         const char *e = getenv(name);
         k.push_back(e ? 1 + atol(e) : 0);
     }

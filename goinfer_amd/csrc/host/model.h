@@ -81,6 +81,7 @@ struct rd_model {
     std::vector<int> slot_len;
 
     // step scratch (device)
+    float *h2 = nullptr; // a one-row step's second residual row: the projections that fold the norm in read one and write the other
     float *h = nullptr, *normed = nullptr, *P = nullptr, *qbuf = nullptr, *part = nullptr, *logits = nullptr, *emb_dev = nullptr;
     // A device-chained decode (GreedyChain* / SampleChain*): forwards queued ahead of the host, one token id coming back per forward
     struct Chain {

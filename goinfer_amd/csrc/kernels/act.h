@@ -258,6 +258,76 @@ extern "C" __global__ __launch_bounds__(1024) void rd_k_add_rmsnorm_quant(float 
     }
 }
 
+// What rd_k_add_rmsnorm_quant leaves for ONE row (row 0 of a one-row step), recomputed by every block of the projection that
+// consumes it instead of being its own launch: a step of one sequence is bound by its launches, and the row is 16 KB. The plain
+// case only: split-K partials (or none), one scale per group of 32, no second norm, H % 256 == 0, H <= 4096. The block's BS
+// threads stand in for the standalone kernel's 1024: thread t is its threads t, t + BS, ... (same lane, so the wave sums and the
+// eight-lane quantization groups are the same lanes' — the same operations on the same values, bit for bit).
+//   hOut (every block holds the same values; the caller lets one block pass it): the residual row after the add
+//   img: the row's quantized form in LDS, RD_ROW0_KB_BYTES per 256 elements: codes [8 groups][32], then the groups' scales as
+//        [parity][4] floats and their scaled code sums alike — a lane half's sixteen codes of a group, and the scales and sums of
+//        its parity's four groups, are one 16-byte read each (a8_row0_from_lds)
+//   red: 16 doubles of LDS. Ends with a barrier: img is complete when it returns.
+constexpr int RD_ROW0_KB_BYTES = 320;
+template <int BS>
+__device__ __forceinline__ void norm_row0_to_lds(const float *__restrict__ hIn, float *__restrict__ hOut, const float *__restrict__ P, int splits,
+                                                 const float *__restrict__ w, float eps, int H, uint8_t *img, double *red) {
+    constexpr int NV = 1024 / BS;
+    const int t = threadIdx.x, nv = H >> 2;
+    float4_t v[NV], wv[NV], a[NV];
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        const int q = t + j * BS;
+        v[j] = (float4_t){0.f, 0.f, 0.f, 0.f};
+        if (q < nv) v[j] = *(const float4_t *)(hIn + 4 * q), wv[j] = *(const float4_t *)(w + 4 * q);
+        if (q < nv && P) a[j] = *(const float4_t *)(P + 4 * q);
+    }
+    if (P) {
+        for (int s = 1; s < splits; s++) // ascending split order
+#pragma unroll
+            for (int j = 0; j < NV; j++) {
+                const int q = t + j * BS;
+                if (q >= nv) continue;
+                const float4_t b = *(const float4_t *)(P + (size_t)s * 32 * H + 4 * q);
+                a[j].x = __fadd_rn(a[j].x, b.x), a[j].y = __fadd_rn(a[j].y, b.y), a[j].z = __fadd_rn(a[j].z, b.z), a[j].w = __fadd_rn(a[j].w, b.w);
+            }
+#pragma unroll
+        for (int j = 0; j < NV; j++)
+            if (t + j * BS < nv)
+                v[j].x = __fadd_rn(v[j].x, a[j].x), v[j].y = __fadd_rn(v[j].y, a[j].y), v[j].z = __fadd_rn(v[j].z, a[j].z), v[j].w = __fadd_rn(v[j].w, a[j].w);
+    }
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        const int q = t + j * BS;
+        if (hOut && q < nv) *(float4_t *)(hOut + 4 * q) = v[j];
+        double ss = 0;
+        ss += (double)v[j].x * v[j].x + (double)v[j].y * v[j].y + (double)v[j].z * v[j].z + (double)v[j].w * v[j].w;
+        ss = wave_sum64_d(ss);
+        if ((t & 63) == 0) red[q >> 6] = ss;
+    }
+    __syncthreads();
+    double ss = 0;
+#pragma unroll
+    for (int i = 0; i < 16; i++) ss += red[i];
+    const float inv = (float)(1.0 / sqrt(ss / (double)H + (double)eps));
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        const int q = t + j * BS;
+        if (q >= nv) continue; // whole waves drop out together: nv is a multiple of 64
+        const float n0 = __fmul_rn(__fmul_rn(v[j].x, inv), wv[j].x), n1 = __fmul_rn(__fmul_rn(v[j].y, inv), wv[j].y);
+        const float n2 = __fmul_rn(__fmul_rn(v[j].z, inv), wv[j].z), n3 = __fmul_rn(__fmul_rn(v[j].w, inv), wv[j].w);
+        const Quant4 qq = quant_four(n0, n1, n2, n3);
+        const int k0 = 4 * q, g = (k0 >> 5) & 7;
+        uint8_t *kb = img + (size_t)(k0 >> 8) * RD_ROW0_KB_BYTES;
+        *(uint32_t *)(kb + g * 32 + (k0 & 31)) = qq.codes;
+        if ((k0 & 31) == 0) {
+            *(float *)(kb + 256 + (g & 1) * 16 + (g >> 1) * 4) = qq.sc;
+            *(float *)(kb + 288 + (g & 1) * 16 + (g >> 1) * 4) = qq.gsum;
+        }
+    }
+    __syncthreads();
+}
+
 // gate/up partials P[s][32][2I] -> act = silu(gate)*up (decoder/rmsnorm.go:204-207: silu in f64) -> per-32 quant -> panels.
 // Grid (ceil(I/1024), M), 256 threads, four consecutive columns per thread. I % 32 == 0. act 1: geluTanh(gate)*up (GeGLU).
 extern "C" __global__ __launch_bounds__(256) void rd_k_swiglu_quant(const float *__restrict__ P, int splits, int I, uint8_t *__restrict__ Xp,

@@ -501,6 +501,53 @@ __device__ __forceinline__ void gemm8_wave_loop(float16_t &acc, const uint8_t *_
     }
 }
 
+// A one-row step whose norm-and-quantize kernel is folded into the projection (norm_row0_to_lds): the row's operands come from the
+// block's LDS image instead of the A8 panel. The registers get what a8_load gives a one-row wave (batch row 0's sixteen codes of
+// every group on each lane half, the scales and sums of the half's four groups), so mma1 forms the same sums from them.
+struct Row0Norm {
+    const float *hIn; // the residual row
+    float *hOut;      // the row after the pending add (another buffer: other blocks still read hIn)
+    const float *P;   // the pending split-K partials [splits][32][H] (row 0 of each), or null
+    const float *w;   // norm weights
+    int splits, H;
+    float eps;
+};
+__device__ __forceinline__ void a8_row0_from_lds(A8Regs &a, const uint8_t *img, int kb, int h) {
+    const uint8_t *p = img + (size_t)kb * RD_ROW0_KB_BYTES;
+#pragma unroll
+    for (int g = 0; g < 8; g++) a.c[g] = *(const uint4_t *)(p + g * 32 + h * 16);
+    a.as = *(const float4_t *)(p + 256 + h * 16);
+    a.asum = *(const float4_t *)(p + 288 + h * 16);
+}
+// w0, w1: the range's first two tiles, asked for by the caller before the row was formed. kb0: the range's first K-block.
+template <class T>
+__device__ __forceinline__ void gemm8_wave_loop_row0(float16_t &acc, typename T::Tile &w0, typename T::Tile &w1, rd_rsrc_t wr, const uint8_t *img, int kb0, int nk,
+                                                     const void *aux, int tile, int lane) {
+    const int h = lane >> 5;
+    A8Regs a0, a1;
+    for (int it = 0; it < nk; it += 2) {
+        a8_row0_from_lds(a0, img, kb0 + it, h);
+        if (it + 1 < nk) a8_row0_from_lds(a1, img, kb0 + it + 1, h);
+        T::mma1(acc, w0, a0, aux, tile, lane);
+        T::load(w0, wr, (it + 2) * T::TILE_BYTES, lane);
+        if (it + 1 < nk) T::mma1(acc, w1, a1, aux, tile, lane);
+        T::load(w1, wr, (it + 3) * T::TILE_BYTES, lane);
+    }
+}
+// The projection's K loop for a one-row step with the norm folded in: weights first, then the row, then the loop.
+template <class T, int BS>
+__device__ __forceinline__ void gemm8_row0_norm_loop(float16_t &acc, const uint8_t *__restrict__ wb, int kb0, int nk, const Row0Norm &rn, bool writesRow,
+                                                     uint8_t *img, double *red, const void *aux, int tile, int lane) {
+#pragma unroll
+    for (int i = 0; i < 16; i++) acc[i] = 0.f;
+    const rd_rsrc_t wr = make_rsrc(wb, (uint32_t)nk * T::TILE_BYTES);
+    typename T::Tile w0, w1;
+    T::load(w0, wr, 0, lane);
+    T::load(w1, wr, T::TILE_BYTES, lane);
+    norm_row0_to_lds<BS>(rn.hIn, writesRow ? rn.hOut : nullptr, rn.P, rn.splits, rn.w, rn.eps, rn.H, img, red);
+    gemm8_wave_loop_row0<T>(acc, w0, w1, wr, img, kb0, nk, aux, tile, lane);
+}
+
 // Folds the KW waves' partial sums of each tile into the tile's first wave, ascending wave order, through LDS
 // (xch: TPB*(KW-1)*1024 floats). Every wave of the block calls it.
 template <int KW, int TPB, bool INT_ACC = false>
@@ -616,14 +663,18 @@ RD_GEMM8_KERNEL(rd_k_gemm8_w4a8r_kw8, W4A8RowTraits8, 8, 1)
 // half-wave holds the 32 columns of one batch row, which is exactly one activation group of the down projection, so
 // silu(gate)*up (silu in f64, decoder/rmsnorm.go:204-207) is quantized where it sits and written in the layout the down projection reads.
 // The K loop, its wave ranges and the fold are those of the plain kernel with the same KW: the sums are the same bits.
-template <class T, int KW, int NR = 16, int ACT = 0>
+template <class T, int KW, int NR = 16, int ACT = 0, bool NORM = false>
 __device__ __forceinline__ void gemm8_gateup_body(const uint8_t *__restrict__ Wt, const uint8_t *__restrict__ A8, uint8_t *__restrict__ XpOut, int outKind,
-                                                  int I, int nKB, int M, float *lds) {
+                                                  int I, int nKB, int M, float *lds, const Row0Norm *rn = nullptr, uint8_t *img = nullptr,
+                                                  double *red = nullptr) {
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int half = wave / KW, kw = wave % KW, t = blockIdx.x, nGate = I >> 5, tile = half * nGate + t;
     const int per = (nKB + KW - 1) / KW, s0 = kw * per, nk = max(0, min(nKB, s0 + per) - s0);
     float16_t acc;
-    gemm8_wave_loop<T, NR>(acc, Wt + ((size_t)tile * nKB + s0) * T::TILE_BYTES, A8 + (size_t)s0 * RD_A8_BLOCK_BYTES, nk, nullptr, tile, lane, lane * 16);
+    if constexpr (NORM) // one row, its norm-and-quantize folded in (NR == 1)
+        gemm8_row0_norm_loop<T, 128 * KW>(acc, Wt + ((size_t)tile * nKB + s0) * T::TILE_BYTES, s0, nk, *rn, blockIdx.x == 0, img, red, nullptr, tile, lane);
+    else
+        gemm8_wave_loop<T, NR>(acc, Wt + ((size_t)tile * nKB + s0) * T::TILE_BYTES, A8 + (size_t)s0 * RD_A8_BLOCK_BYTES, nk, nullptr, tile, lane, lane * 16);
     gemm8_fold_waves<KW, 2>(acc, lds);
     __syncthreads(); // the fold area is read; it now takes the two finished tiles as [gate | up][register][lane]
     if (kw == 0) {
@@ -669,6 +720,22 @@ __device__ __forceinline__ void gemm8_gateup_body(const uint8_t *__restrict__ Wt
     }
 RD_GEMM8_GATEUP_KERNEL(rd_k_gemm8_q4k_gateup, 0)
 RD_GEMM8_GATEUP_KERNEL(rd_k_gemm8_q4k_gateup_gelu, 1)
+// A one-row step's gate|up projection with the norm-and-quantize kernel that feeds it folded in: every block forms the row
+// (hIn + the pending partials, RMSNorm, per-32 quantization; norm_row0_to_lds) while its first weight tiles are on their way,
+// block 0 writes the updated residual row to hOut, and the loop, the fold and the epilogue are the one-row kernel's own: the
+// same bits as rd_k_add_rmsnorm_quant followed by rd_k_gemm8_q4k_gateup, in one launch less. Grid (I/32), block 256.
+#define RD_GEMM8_GATEUP_NORM1_KERNEL(NAME, ACT)                                                                                                   \
+    extern "C" __global__ __launch_bounds__(256) void NAME(const uint8_t *__restrict__ Wt, uint8_t *__restrict__ XpOut, int outKind, int I, int nKB, \
+                                                           const float *__restrict__ hIn, float *__restrict__ hOut, const float *__restrict__ P,  \
+                                                           int splits, const float *__restrict__ w, float eps, int H) {                          \
+        __shared__ float lds[2 * 1024];                                                                                                           \
+        __shared__ __align__(16) uint8_t img[16 * RD_ROW0_KB_BYTES];                                                                              \
+        __shared__ double red[16];                                                                                                                \
+        const Row0Norm rn{hIn, hOut, P, w, splits, H, eps};                                                                                       \
+        gemm8_gateup_body<Q4K8Traits, 2, 1, ACT, true>(Wt, nullptr, XpOut, outKind, I, nKB, 1, lds, &rn, img, red);                               \
+    }
+RD_GEMM8_GATEUP_NORM1_KERNEL(rd_k_gemm8_q4k_gateup_norm1, 0)
+RD_GEMM8_GATEUP_NORM1_KERNEL(rd_k_gemm8_q4k_gateup_gelu_norm1, 1)
 
 // ---------------- q|k|v projection with bias, RoPE and the KV store in its epilogue ----------------
 // The plain kernel with one split and, instead of the store of the sums, what rd_k_qkv_rope_store does to them (same arithmetic,
@@ -683,9 +750,10 @@ struct QkvEpilogue {
     const float *bias;
     int tabStride, nH, nKV, HD, row0;
 };
-template <class T, int KW, int NR = 16>
+template <class T, int KW, int NR = 16, bool NORM = false>
 __device__ __forceinline__ void gemm8_qkv_body(const uint8_t *__restrict__ Wt, const void *__restrict__ aux, const uint8_t *__restrict__ A8, int N, int nKB,
-                                               int M, const QkvEpilogue &e, float *lds) {
+                                               int M, const QkvEpilogue &e, float *lds, const Row0Norm *rn = nullptr, uint8_t *img = nullptr,
+                                               double *red = nullptr) {
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int tile = blockIdx.x, kw = wave;
     const int per = (nKB + KW - 1) / KW, s0 = kw * per, nk = max(0, min(nKB, s0 + per) - s0);
@@ -706,7 +774,10 @@ __device__ __forceinline__ void gemm8_qkv_body(const uint8_t *__restrict__ Wt, c
         }
     }
     float16_t acc;
-    gemm8_wave_loop<T, NR>(acc, Wt + ((size_t)tile * nKB + s0) * T::TILE_BYTES, A8 + (size_t)s0 * RD_A8_BLOCK_BYTES, nk, aux, tile, lane, lane * 16);
+    if constexpr (NORM) // one row, its norm-and-quantize folded in (NR == 1)
+        gemm8_row0_norm_loop<T, 64 * KW>(acc, Wt + ((size_t)tile * nKB + s0) * T::TILE_BYTES, s0, nk, *rn, blockIdx.x == 0, img, red, aux, tile, lane);
+    else
+        gemm8_wave_loop<T, NR>(acc, Wt + ((size_t)tile * nKB + s0) * T::TILE_BYTES, A8 + (size_t)s0 * RD_A8_BLOCK_BYTES, nk, aux, tile, lane, lane * 16);
     double2 cs[PPT];
     float b1 = 0.f, b2 = 0.f;
     if (isQ || isK) {
@@ -763,6 +834,24 @@ __device__ __forceinline__ void gemm8_qkv_body(const uint8_t *__restrict__ Wt, c
         else                                                                                                                                           \
             gemm8_qkv_body<TRAITS, KW, 16>(Wt, aux, A8, N, nKB, M, e, lds);                                                                            \
     }
+// A one-row step's q|k|v projection with the norm-and-quantize kernel that feeds it folded in (see rd_k_gemm8_q4k_gateup_norm1):
+// the same bits as rd_k_add_rmsnorm_quant followed by the kernel above, in one launch less. Grid (N/32), block KW waves.
+#define RD_GEMM8_QKV_NORM1_KERNEL(NAME, TRAITS, KW)                                                                                                    \
+    extern "C" __global__ __launch_bounds__(64 * KW) void NAME(                                                                                        \
+        const uint8_t *__restrict__ Wt, const void *__restrict__ aux, int N, int nKB, float *__restrict__ q, uint16_t *__restrict__ Kp,                \
+        uint16_t *__restrict__ Vp, const int *__restrict__ tables, int tabStride, const int *__restrict__ rowSlot, const int *__restrict__ rowPos,      \
+        const double *__restrict__ cs, const float *__restrict__ bias, int nH, int nKV, int HD, const float *__restrict__ hIn, float *__restrict__ hOut, \
+        const float *__restrict__ P, int splits, const float *__restrict__ w, float eps, int H) {                                                      \
+        __shared__ float lds[KW > 2 ? (KW - 1) * 1024 : 32 * 33];                                                                                      \
+        __shared__ __align__(16) uint8_t img[16 * RD_ROW0_KB_BYTES];                                                                                   \
+        __shared__ double red[16];                                                                                                                     \
+        QkvEpilogue e{q, Kp, Vp, tables, rowSlot, rowPos, (const double2 *)cs, bias, tabStride, nH, nKV, HD, 0};                                       \
+        const Row0Norm rn{hIn, hOut, P, w, splits, H, eps};                                                                                            \
+        gemm8_qkv_body<TRAITS, KW, 1, true>(Wt, aux, nullptr, N, nKB, 1, e, lds, &rn, img, red);                                                       \
+    }
+RD_GEMM8_QKV_NORM1_KERNEL(rd_k_gemm8_q4k_qkv_norm1_kw2, Q4K8Traits, 2)
+RD_GEMM8_QKV_NORM1_KERNEL(rd_k_gemm8_q4k_qkv_norm1_kw4, Q4K8Traits, 4)
+RD_GEMM8_QKV_NORM1_KERNEL(rd_k_gemm8_q4k_qkv_norm1_kw8, Q4K8Traits, 8)
 RD_GEMM8_QKV_KERNEL(rd_k_gemm8_q4k_qkv_kw2, Q4K8Traits, 2)
 RD_GEMM8_QKV_KERNEL(rd_k_gemm8_q4k_qkv_kw4, Q4K8Traits, 4)
 RD_GEMM8_QKV_KERNEL(rd_k_gemm8_q4k_qkv_kw8, Q4K8Traits, 8)

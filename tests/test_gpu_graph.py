@@ -171,3 +171,34 @@ def test_a_changed_kernel_knob_is_never_served_by_an_older_graph(dev):
     finally:
         a.close()
         b.close()
+
+
+@pytest.mark.parametrize("name,cfg", [("hidden 256", dense_cfg(n_layers=3)), ("hidden 1024, biases", dict(dense_cfg(n_layers=2, hidden=1024, n_heads=8, n_kv=2, head_dim=128, inter=1536), qkv_bias=1)),
+                                      ("hidden 4096", dense_cfg(n_layers=2, hidden=4096, n_heads=8, n_kv=2, head_dim=128, inter=2048))])
+def test_one_row_steps_with_the_norm_folded_into_the_projections_equal_the_separate_kernels(dev, name, cfg):
+    """A step of one row forms the row's norm and quantization inside its q|k|v and gate|up projections (one launch less each); with
+    ROCMDECODE_NO_FUSED_NORM the norm kernel is launched on its own as in a batch. Both, eager and replayed from a graph, give the
+    same logits bit for bit, position after position (the residual row alternates between two buffers in the folded form), and the
+    row equals the same sequence's row in a batch of two."""
+    import os
+    a, b = twins(cfg, 11, dev, slots=4, ctx_cap=256)
+    c, d = Pair(cfg, seed=11, dev=dev, slots=4, ctx_cap=256), Pair(cfg, seed=11, dev=dev, slots=4, ctx_cap=256)
+    try:
+        rng = np.random.default_rng(5)
+        for p in range(70):  # crosses a 64-position block boundary
+            tok = rng.integers(0, cfg["vocab"], 2)
+            la = a.gpu.step_batch([0], [p], a.emb[tok[:1]])[0]  # folded, replayed from a graph after the second step
+            lb = b.gpu.step_batch([0], [p], b.emb[tok[:1]])[0]  # folded, eager
+            os.environ["ROCMDECODE_NO_FUSED_NORM"] = "1"
+            try:
+                lc = c.gpu.step_batch([0], [p], c.emb[tok[:1]])[0]  # the norm kernel on its own
+            finally:
+                del os.environ["ROCMDECODE_NO_FUSED_NORM"]
+            ld = d.gpu.step_batch([0, 1], [p, p], d.emb[tok])[0]  # the same sequence as row 0 of a batch of two
+            assert same_bits(la, lb), (name, p)
+            assert same_bits(la, lc), (name, p)
+            assert same_bits(la[0], ld[0]), (name, p)
+        assert a.gpu.graph_stats()[1] > 40
+    finally:
+        for m in (a, b, c, d):
+            m.close()
