@@ -519,33 +519,36 @@ __device__ __forceinline__ void a8_row0_from_lds(A8Regs &a, const uint8_t *img, 
     a.as = *(const float4_t *)(p + 256 + h * 16);
     a.asum = *(const float4_t *)(p + 288 + h * 16);
 }
-// w0, w1: the range's first two tiles, asked for by the caller before the row was formed. kb0: the range's first K-block.
-template <class T>
-__device__ __forceinline__ void gemm8_wave_loop_row0(float16_t &acc, typename T::Tile &w0, typename T::Tile &w1, rd_rsrc_t wr, const uint8_t *img, int kb0, int nk,
+// DEPTH weight tiles are in flight per wave (two: four were measured slower on the gate|up shape, 21.2 against 20.1 us a launch).
+// w[]: the range's first DEPTH tiles, asked for by the caller before the row was formed. kb0: the range's first K-block.
+template <class T, int DEPTH>
+__device__ __forceinline__ void gemm8_wave_loop_row0(float16_t &acc, typename T::Tile (&w)[DEPTH], rd_rsrc_t wr, const uint8_t *img, int kb0, int nk,
                                                      const void *aux, int tile, int lane) {
     const int h = lane >> 5;
-    A8Regs a0, a1;
-    for (int it = 0; it < nk; it += 2) {
-        a8_row0_from_lds(a0, img, kb0 + it, h);
-        if (it + 1 < nk) a8_row0_from_lds(a1, img, kb0 + it + 1, h);
-        T::mma1(acc, w0, a0, aux, tile, lane);
-        T::load(w0, wr, (it + 2) * T::TILE_BYTES, lane);
-        if (it + 1 < nk) T::mma1(acc, w1, a1, aux, tile, lane);
-        T::load(w1, wr, (it + 3) * T::TILE_BYTES, lane);
+    for (int it = 0; it < nk; it += DEPTH) {
+#pragma unroll
+        for (int i = 0; i < DEPTH; i++) {
+            if (it + i < nk) {
+                A8Regs a;
+                a8_row0_from_lds(a, img, kb0 + it + i, h);
+                T::mma1(acc, w[i], a, aux, tile, lane);
+            }
+            T::load(w[i], wr, (it + i + DEPTH) * T::TILE_BYTES, lane); // past the range: answered with zeros, never used
+        }
     }
 }
 // The projection's K loop for a one-row step with the norm folded in: weights first, then the row, then the loop.
-template <class T, int BS>
+template <class T, int BS, int DEPTH>
 __device__ __forceinline__ void gemm8_row0_norm_loop(float16_t &acc, const uint8_t *__restrict__ wb, int kb0, int nk, const Row0Norm &rn, bool writesRow,
                                                      uint8_t *img, double *red, const void *aux, int tile, int lane) {
 #pragma unroll
     for (int i = 0; i < 16; i++) acc[i] = 0.f;
     const rd_rsrc_t wr = make_rsrc(wb, (uint32_t)nk * T::TILE_BYTES);
-    typename T::Tile w0, w1;
-    T::load(w0, wr, 0, lane);
-    T::load(w1, wr, T::TILE_BYTES, lane);
+    typename T::Tile w[DEPTH];
+#pragma unroll
+    for (int i = 0; i < DEPTH; i++) T::load(w[i], wr, i * T::TILE_BYTES, lane);
     norm_row0_to_lds<BS>(rn.hIn, writesRow ? rn.hOut : nullptr, rn.P, rn.splits, rn.w, rn.eps, rn.H, img, red);
-    gemm8_wave_loop_row0<T>(acc, w0, w1, wr, img, kb0, nk, aux, tile, lane);
+    gemm8_wave_loop_row0<T, DEPTH>(acc, w, wr, img, kb0, nk, aux, tile, lane);
 }
 
 // Folds the KW waves' partial sums of each tile into the tile's first wave, ascending wave order, through LDS
@@ -672,7 +675,7 @@ __device__ __forceinline__ void gemm8_gateup_body(const uint8_t *__restrict__ Wt
     const int per = (nKB + KW - 1) / KW, s0 = kw * per, nk = max(0, min(nKB, s0 + per) - s0);
     float16_t acc;
     if constexpr (NORM) // one row, its norm-and-quantize folded in (NR == 1)
-        gemm8_row0_norm_loop<T, 128 * KW>(acc, Wt + ((size_t)tile * nKB + s0) * T::TILE_BYTES, s0, nk, *rn, blockIdx.x == 0, img, red, nullptr, tile, lane);
+        gemm8_row0_norm_loop<T, 128 * KW, 2>(acc, Wt + ((size_t)tile * nKB + s0) * T::TILE_BYTES, s0, nk, *rn, blockIdx.x == 0, img, red, nullptr, tile, lane);
     else
         gemm8_wave_loop<T, NR>(acc, Wt + ((size_t)tile * nKB + s0) * T::TILE_BYTES, A8 + (size_t)s0 * RD_A8_BLOCK_BYTES, nk, nullptr, tile, lane, lane * 16);
     gemm8_fold_waves<KW, 2>(acc, lds);
@@ -775,7 +778,7 @@ __device__ __forceinline__ void gemm8_qkv_body(const uint8_t *__restrict__ Wt, c
     }
     float16_t acc;
     if constexpr (NORM) // one row, its norm-and-quantize folded in (NR == 1)
-        gemm8_row0_norm_loop<T, 64 * KW>(acc, Wt + ((size_t)tile * nKB + s0) * T::TILE_BYTES, s0, nk, *rn, blockIdx.x == 0, img, red, aux, tile, lane);
+        gemm8_row0_norm_loop<T, 64 * KW, 2>(acc, Wt + ((size_t)tile * nKB + s0) * T::TILE_BYTES, s0, nk, *rn, blockIdx.x == 0, img, red, aux, tile, lane);
     else
         gemm8_wave_loop<T, NR>(acc, Wt + ((size_t)tile * nKB + s0) * T::TILE_BYTES, A8 + (size_t)s0 * RD_A8_BLOCK_BYTES, nk, aux, tile, lane, lane * 16);
     double2 cs[PPT];
