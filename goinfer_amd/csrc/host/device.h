@@ -93,6 +93,14 @@ struct DevBuf {
 // block sizes that match the code object's launch bounds: the fused gate|up kernel (two tiles x two waves), the expert kernels
 // (two tiles x two waves)
 constexpr unsigned GATEUP_THREADS = 256, MOE_THREADS = 256;
+// grid.z of the experts' gate|up kernels: an expert's passes of four rows run side by side in this many layers of blocks (one
+// layer while no expert can have a fifth row; ROCMDECODE_MOE_PASS_LAYERS overrides, for measurement). Measured on the
+// Qwen3-MoE-shape step of 16 rows: two layers take the gate|up launches from 1.86 to 1.77 ms a step; the down projection's
+// launches, whose blocks are fewer and longer, lose by it (1.32 to 1.36 ms) and keep one layer.
+inline unsigned moe_pass_layers(int T) {
+    if (const char *e = getenv("ROCMDECODE_MOE_PASS_LAYERS")) return (unsigned)std::max(1, std::min(8, atoi(e)));
+    return T > 4 ? 2u : 1u;
+}
 
 // How many 64-position KV blocks one attention work item covers for a sequence of nb blocks: every (sequence, kv head) is
 // cut into pieces. The cut depends on the sequence's own length only, never on what else is in the

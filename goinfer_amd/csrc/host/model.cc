@@ -806,7 +806,7 @@ static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
         // stages its rows: two launches, as on the per-32 lane
         {
             Scope s(m, KC_MOE_GEMM);
-            RC(d->launch_lds(d->k.moe_gemv_w4a8r_gateup, (unsigned)((I / 32 + 1) / 2), (unsigned)nE, 1, MOE_THREADS, moe_gemv_lds(H), (const void *)l.exp_gateup, guStride,
+            RC(d->launch_lds(d->k.moe_gemv_w4a8r_gateup, (unsigned)((I / 32 + 1) / 2), (unsigned)nE, moe_pass_layers(B), MOE_THREADS, moe_gemv_lds(H), (const void *)l.exp_gateup, guStride,
                              (const void *)m->XpA, m->XEf, m->moe_rowmax, I, H, B, (const signed char *)m->moe_rank, nE, (const unsigned *)bits_dev));
         }
         Scope s(m, KC_MOE_GEMM_DOWN);
@@ -815,12 +815,12 @@ static int moe_ffn(rd_model *m, int B, int layer, LayerW &l) {
                          (const unsigned *)bits_dev));
     } else if (fused) {
         Scope s(m, KC_MOE_GEMM); // gate|up of every touched expert + SwiGLU + quantization into the experts' down activations
-        RC(d->launch_lds(d->k.moe_gemv_w4a8_gateup, (unsigned)((I / 32 + 1) / 2), (unsigned)nE, 1, MOE_THREADS, moe_gemv_lds(H), (const void *)l.exp_gateup, guStride,
+        RC(d->launch_lds(d->k.moe_gemv_w4a8_gateup, (unsigned)((I / 32 + 1) / 2), (unsigned)nE, moe_pass_layers(B), MOE_THREADS, moe_gemv_lds(H), (const void *)l.exp_gateup, guStride,
                          (const void *)m->XpA, m->XpE, xpStride, I, H, B, (const signed char *)m->moe_rank, nE, (const unsigned *)bits_dev));
     } else {
         {
             Scope s(m, KC_MOE_GEMM);
-            RC(d->launch_lds(gemv, moe_gemv_grid(2 * I, H), (unsigned)nE, 1, MOE_THREADS, moe_gemv_lds(H), (const void *)l.exp_gateup, guStride,
+            RC(d->launch_lds(gemv, moe_gemv_grid(2 * I, H), (unsigned)nE, moe_pass_layers(B), MOE_THREADS, moe_gemv_lds(H), (const void *)l.exp_gateup, guStride,
                              (const void *)m->XpA, (size_t)0, m->moe_gu, 2 * I, H, B, k, (const signed char *)m->moe_rank, nE,
                              (const unsigned *)bits_dev));
         }
@@ -1043,7 +1043,7 @@ static std::vector<long> step_graph_key(rd_model *m, int B, int want) {
     // every environment knob a launch consults, by value: a step after a change is launched (and captured) anew
     for (const char *name : {"ROCMDECODE_NO_FUSED_GATEUP", "ROCMDECODE_NO_FUSED_QKV", "ROCMDECODE_NO_FUSED_MOE_GATEUP", "ROCMDECODE_MOE_TILES",
                              "ROCMDECODE_GEMM8_KW", "ROCMDECODE_GEMM8_SPLITS", "ROCMDECODE_NO_DEEP_ATTN", "ROCMDECODE_NO_WIDE_ATTN",
-                             "ROCMDECODE_NO_ATTN_GROUPS", "ROCMDECODE_NO_ROWS_GEMM", "ROCMDECODE_NO_FUSED_NORM"}) {
+                             "ROCMDECODE_NO_ATTN_GROUPS", "ROCMDECODE_NO_ROWS_GEMM", "ROCMDECODE_NO_FUSED_NORM", "ROCMDECODE_MOE_PASS_LAYERS"}) {
         const char *e = getenv(name);
         k.push_back(e ? 1 + atol(e) : 0);
     }

@@ -234,10 +234,13 @@ __device__ __forceinline__ void moe_gemv_body(const uint8_t *__restrict__ Wt, si
     const rd_rsrc_t wr = make_rsrc(Wt, (uint32_t)((N >> 5) * nKB * 4608));
     auto tileOff = [&](int q) { return (tile0 + q) * nKB * 4608; };
     GvTiles wt;
-    gv_first(wt, wr, nTiles, tileOff, nKB, lane); // the weights need only the expert: asked for before its rows are looked up
+    // The passes of an expert with more than GV_ROWS rows are dealt over grid.z (pass p to layer p % gridDim.z) and run side by
+    // side instead of one after the other; the layers past an expert's passes find nothing to do and leave.
+    bool primed = blockIdx.z == 0;
+    if (primed) gv_first(wt, wr, nTiles, tileOff, nKB, lane); // the weights need only the expert: asked for before its rows are looked up
     int src;
     const int rows = moe_expert_rows(rankOf, nE, T, e, lane, &src);
-    for (int r0 = 0; r0 < rows; r0 += GV_ROWS) {
+    for (int r0 = (int)blockIdx.z * GV_ROWS; r0 < rows; r0 += (int)gridDim.z * GV_ROWS) {
         const int R = min(GV_ROWS, rows - r0);
         int rowOf[GV_ROWS], tokOf[GV_ROWS]; // uniform: the pass's rows in X and their tokens (a lane is never asked for a token while it sits out a branch)
 #pragma unroll
@@ -245,7 +248,8 @@ __device__ __forceinline__ void moe_gemv_body(const uint8_t *__restrict__ Wt, si
             tokOf[j] = __builtin_amdgcn_readlane(src, min(r0 + j, 31));
             rowOf[j] = r0 + j < rows ? (xStride == 0 ? tokOf[j] : r0 + j) : -1;
         }
-        if (r0 > 0) gv_first(wt, wr, nTiles, tileOff, nKB, lane);
+        if (!primed) gv_first(wt, wr, nTiles, tileOff, nKB, lane);
+        primed = false;
         __syncthreads(); // the previous pass is done with the staged rows
         if constexpr (F32IN)
             gv_stage_f32(lds, (const float *)X, rowMax + (size_t)e * 32, K, nKB, rowOf);
@@ -319,10 +323,11 @@ __device__ __forceinline__ void moe_gateup_body(const uint8_t *__restrict__ Wt, 
     const rd_rsrc_t wr = make_rsrc(Wt, (uint32_t)(2 * nGate * nKB * 4608));
     auto tileOff = [&](int) { return (isUp * nGate + t) * nKB * 4608; };
     GvTiles wt;
-    gv_first(wt, wr, nTiles, tileOff, nKB, lane); // the weights need only the expert: asked for before its rows are looked up
+    bool primed = blockIdx.z == 0; // passes over grid.z as in moe_gemv_body
+    if (primed) gv_first(wt, wr, nTiles, tileOff, nKB, lane); // the weights need only the expert: asked for before its rows are looked up
     int src;
     const int rows = moe_expert_rows(rankOf, nE, T, e, lane, &src);
-    for (int r0 = 0; r0 < rows; r0 += GV_ROWS) {
+    for (int r0 = (int)blockIdx.z * GV_ROWS; r0 < rows; r0 += (int)gridDim.z * GV_ROWS) {
         const int R = min(GV_ROWS, rows - r0);
         int rowOf[GV_ROWS];
 #pragma unroll
@@ -330,7 +335,8 @@ __device__ __forceinline__ void moe_gateup_body(const uint8_t *__restrict__ Wt, 
             const int tok = __builtin_amdgcn_readlane(src, min(r0 + j, 31));
             rowOf[j] = r0 + j < rows ? tok : -1;
         }
-        if (r0 > 0) gv_first(wt, wr, nTiles, tileOff, nKB, lane);
+        if (!primed) gv_first(wt, wr, nTiles, tileOff, nKB, lane);
+        primed = false;
         __syncthreads(); // the previous pass is done with the staged rows and the exchanged sums
         gv_stage(lds, X, K, nKB, rowOf);
         __syncthreads();
