@@ -77,7 +77,7 @@ __device__ __forceinline__ int moe_expert_rows(const signed char *__restrict__ r
     return __popc(mk);
 }
 
-constexpr int GV_ROWS = 4; // rows of an expert worked on per pass over its weights
+constexpr int GV_ROWS = 4; // rows of an expert worked on per pass over its weights (two: 6.32 against 5.91 ms a Qwen3-MoE-shape step)
 // LDS of a pass: the rows' codes [GV_ROWS][Kpad] (Kpad = K up to whole 256-blocks, zero-filled), then their scales [GV_ROWS][Kpad/32].
 __device__ __forceinline__ size_t gv_lds_bytes(int nKB) { return (size_t)GV_ROWS * nKB * (256 + 32); }
 
@@ -340,7 +340,7 @@ __device__ __forceinline__ void moe_gateup_body(const uint8_t *__restrict__ Wt, 
         __syncthreads(); // the previous pass is done with the staged rows and the exchanged sums
         gv_stage(lds, X, K, nKB, rowOf);
         __syncthreads();
-        float sum[GV_ROWS] = {0.f, 0.f, 0.f, 0.f};
+        float sum[GV_ROWS] = {};
         gv_stream<ROW>(wt, wr, nTiles, tileOff, nKB, lds, lane, R, [&](int, const float(&facc)[GV_ROWS]) {
 #pragma unroll
             for (int j = 0; j < GV_ROWS; j++) sum[j] = facc[j];
