@@ -350,7 +350,9 @@ int rd_bench_attn_chain(rd_model *m, int B, const int *slot, const int *pos, con
 int rd_bench_prefill(rd_model *m, int slot, int n, const int *ids, int profile, float *ms_total, float *class_ms, int *class_n);
 int rd_bench_class_count(void);
 const char *rd_bench_class_name(int c);
-/* Times `iters` launches of one kernel over resident synthetic operands: "gemm_q4k" args {N,K,M,copies}; "copy" args {bytes}. */
+/* Times `iters` launches of one kernel over resident synthetic operands: "gemm_q4k" / "gemm_q5k" / "gemm_q6k" args {N,K,M,copies};
+ * "gateup" args {I,K,M,copies}; "moe_gemm"; "topk" args {rows,V,k}; "copy" args {bytes}; "issue" args {mode,waves,iterations}: the
+ * issue-rate probes (the int8 GEMMs' inner-loop instruction mix with every operand in registers). ms_out[iters]: per launch. */
 int rd_bench_kernel(rd_device *d, const char *name, const int64_t *args, int n_args, int warmup, int iters, float *ms_out);
 /* The ragged attention of one layer over a synthetic paged f16 pool built on the device (the attention micro-benchmark):
  * n_seq sequences of len[i] keys, rows in groups of 32. ms_total[iters]: partial + combine kernels of every group;
