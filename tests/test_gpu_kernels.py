@@ -296,3 +296,14 @@ def test_rmsnorm_rope_route(dev):
         wi, ww = ob.route_experts(logits[t], 8, True)
         assert np.array_equal(idx[t], wi)
         assert np.array_equal(wgt[t].view(np.uint32), ww.view(np.uint32))
+
+
+def test_issue_probes_run_and_decline_bad_arguments(dev):
+    """The issue-rate probes (the int8 GEMMs' inner-loop instruction mix with every operand in registers) launch and time; the mix
+    of all three parts takes at least as long as its longest part. Bad arguments are declined, not launched."""
+    t = [float(np.median(dev.bench_kernel("issue", [mode, 2, 400], 1, 3))) for mode in range(4)]
+    assert all(np.isfinite(x) and x > 0 for x in t), t
+    assert t[3] > 0.9 * max(t[:3]), t
+    for bad in ([4, 1, 100], [0, 3, 100], [0, 1, 0], [0, 1, 100, 5000]):
+        with pytest.raises(capi.RocmError):
+            dev.bench_kernel("issue", bad, 0, 1)
